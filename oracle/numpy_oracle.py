@@ -1,0 +1,138 @@
+"""Float64 NumPy restatement of one PhysicsAttention layer / Transolver block, written from the formulas.
+
+TEST INFRASTRUCTURE ONLY (see oracle/torch_oracle.py for the rule on who may import oracle/).
+
+This file deliberately shares no code with ``torch_oracle.py``: it uses index-explicit einsum / loops in
+float64 so that a transposed operand, a wrong head split or a dropped term in either restatement makes the
+two disagree.  Each step cites the reference lines (relative to the reference checkout) it follows.
+Inputs are plain ``dict[str, np.ndarray]`` keyed like the reference ``state_dict``.
+"""
+
+from __future__ import annotations
+
+import math
+
+import numpy as np
+
+_erf = np.vectorize(math.erf, otypes=[np.float64])
+
+
+def _f64(a):
+    return np.asarray(a, dtype=np.float64)
+
+
+def linear_projection(x, weight, bias):
+    """y[b,n,o] = sum_c x[b,n,c] W[o,c] + bias[o]  (nn.Linear; physics_attention.py:625-627)."""
+    return np.einsum("bnc,oc->bno", _f64(x), _f64(weight)) + _f64(bias)
+
+
+def conv2d_projection(x, weight, bias, grid_h, grid_w):
+    """Zero-padded stride-1 cross-correlation on tokens n = i*grid_w + j (physics_attention.py:740,772-783).
+
+    y[b, i*W+j, o] = bias[o] + sum_{c,u,v} W[o,c,u,v] * x[b, (i+u-p)*W + (j+v-p), c], p = k//2, out-of-grid terms are 0.
+    Direct loops over the k*k taps.
+    """
+    x = _f64(x)
+    weight = _f64(weight)
+    b, n, c = x.shape
+    o, c2, k, k2 = weight.shape
+    assert n == grid_h * grid_w and c == c2 and k == k2
+    p = k // 2
+    img = x.reshape(b, grid_h, grid_w, c)
+    out = np.zeros((b, grid_h, grid_w, o))
+    for u in range(k):
+        for v in range(k):
+            di, dj = u - p, v - p
+            i0, i1 = max(0, -di), min(grid_h, grid_h - di)
+            j0, j1 = max(0, -dj), min(grid_w, grid_w - dj)
+            if i0 >= i1 or j0 >= j1:
+                continue
+            src = img[:, i0 + di:i1 + di, j0 + dj:j1 + dj, :]
+            out[:, i0:i1, j0:j1, :] += np.einsum("bijc,oc->bijo", src, weight[:, :, u, v])
+    return out.reshape(b, n, o) + _f64(bias)
+
+
+def layer_forward(p, x, heads, dim_head, variant="irregular", spatial_shape=None):
+    """All intermediates of one layer in float64 (steps 1-9 below follow physics_attention.py:529-558).
+
+    p: in_project_x.{weight,bias}, in_project_fx.{weight,bias}, in_project_slice.{weight,bias},
+       temperature, qkv_project.weight, out_linear.{weight,bias}
+    """
+    x = _f64(x)
+    B, N, C = x.shape
+    H, D = heads, dim_head
+    # 1. projections, channel c = h*D + d (:114-117, :652-660 / :768-783)
+    if variant == "irregular":
+        xm = linear_projection(x, p["in_project_x.weight"], p["in_project_x.bias"])
+        fm = linear_projection(x, p["in_project_fx.weight"], p["in_project_fx.bias"])
+    else:
+        gh, gw = spatial_shape
+        xm = conv2d_projection(x, p["in_project_x.weight"], p["in_project_x.bias"], gh, gw)
+        fm = conv2d_projection(x, p["in_project_fx.weight"], p["in_project_fx.bias"], gh, gw)
+    xm = xm.reshape(B, N, H, D)
+    fm = fm.reshape(B, N, H, D)
+    # 2. slice logits, one (S, D) weight shared by all heads (:537)
+    ws, bs = _f64(p["in_project_slice.weight"]), _f64(p["in_project_slice.bias"])
+    S = ws.shape[0]
+    logits = np.einsum("bnhd,sd->bnhs", xm, ws) + bs
+    # 3. clamp temperature to [0.5, 5], softmax over S (:173-178)
+    t = np.clip(_f64(p["temperature"]).reshape(H), 0.5, 5.0)
+    z = logits / t[None, None, :, None]
+    z = z - z.max(axis=-1, keepdims=True)
+    e = np.exp(z)
+    w = e / e.sum(axis=-1, keepdims=True)
+    # 4. norm over points + 1e-2 (:185)
+    norm = w.sum(axis=1) + 1e-2  # (B, H, S)
+    # 5. slice tokens = sum_n (w / norm) fx_mid (:188-203)
+    tok = np.einsum("bnhs,bnhd->bhsd", w / norm[:, None, :, :], fm)
+    # 6. qkv = tok Wqkv^T (no bias, :309,:448); q | k | v split in that order (:450,:458)
+    wqkv = _f64(p["qkv_project.weight"])
+    q = np.einsum("bhsd,ed->bhse", tok, wqkv[0:D])
+    k = np.einsum("bhsd,ed->bhse", tok, wqkv[D:2 * D])
+    v = np.einsum("bhsd,ed->bhse", tok, wqkv[2 * D:3 * D])
+    # 7. softmax(q k^T / sqrt(D)) v (:461-463, default SDPA scale)
+    sc = np.einsum("bhse,bhte->bhst", q, k) / math.sqrt(D)
+    sc = sc - sc.max(axis=-1, keepdims=True)
+    a = np.exp(sc)
+    a = a / a.sum(axis=-1, keepdims=True)
+    tok_out = np.einsum("bhst,bhte->bhse", a, v)
+    # 8. deslice with the un-normalised w, merge heads (:492-495)
+    o = np.einsum("bnhs,bhsd->bnhd", w, tok_out).reshape(B, N, H * D)
+    # 9. output projection (:498)
+    y = np.einsum("bnk,ok->bno", o, _f64(p["out_linear.weight"])) + _f64(p["out_linear.bias"])
+    return dict(x_mid=xm, fx_mid=fm, logits=logits, w=w, norm=norm, tok=tok, tok_out=tok_out, y=y)
+
+
+def layer_norm(x, gamma, beta, eps=1e-5):
+    """Biased-variance LayerNorm over the last axis (torch.nn.LayerNorm default eps; transolver.py:210)."""
+    x = _f64(x)
+    mu = x.mean(axis=-1, keepdims=True)
+    var = ((x - mu) ** 2).mean(axis=-1, keepdims=True)
+    return (x - mu) / np.sqrt(var + eps) * _f64(gamma) + _f64(beta)
+
+
+def gelu_erf(x):
+    """Exact GELU: 0.5 x (1 + erf(x / sqrt 2)) (activations.py:198 'gelu' -> nn.GELU())."""
+    x = _f64(x)
+    return 0.5 * x * (1.0 + _erf(x / math.sqrt(2.0)))
+
+
+def mlp(p, prefix, x):
+    """Linear -> GELU -> Linear with keys layers.0 / layers.2 (mlp_layers.py:139-156)."""
+    h = np.einsum("bnc,oc->bno", _f64(x), _f64(p[prefix + "layers.0.weight"])) + _f64(p[prefix + "layers.0.bias"])
+    h = gelu_erf(h)
+    return np.einsum("bnc,oc->bno", h, _f64(p[prefix + "layers.2.weight"])) + _f64(p[prefix + "layers.2.bias"])
+
+
+def block_forward(p, fx, heads, dim_head, last_layer, variant="irregular", spatial_shape=None):
+    """One Transolver block (transolver.py:300-309); p holds the block's state_dict (keys 'ln_1.weight', 'Attn.*', ...)."""
+    fx = _f64(fx)
+    attn_p = {k[len("Attn."):]: v for k, v in p.items() if k.startswith("Attn.")}
+    h1 = layer_norm(fx, p["ln_1.weight"], p["ln_1.bias"])
+    fx = layer_forward(attn_p, h1, heads, dim_head, variant, spatial_shape)["y"] + fx
+    h2 = layer_norm(fx, p["ln_mlp1.0.weight"], p["ln_mlp1.0.bias"])
+    fx = mlp(p, "ln_mlp1.1.", h2) + fx
+    if last_layer:
+        h3 = layer_norm(fx, p["ln_mlp2.0.weight"], p["ln_mlp2.0.bias"])
+        return np.einsum("bnc,oc->bno", h3, _f64(p["ln_mlp2.1.weight"])) + _f64(p["ln_mlp2.1.bias"])
+    return fx

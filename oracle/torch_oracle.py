@@ -1,0 +1,328 @@
+"""CPU restatement of the reference's Transolver PhysicsAttention path (PyTorch ATen ops).
+
+TEST INFRASTRUCTURE ONLY.  Nothing in the shipped package may import this file;
+only tests/, __graft_entry__.smoke() and bench.py's cpu_baseline leg use it, and
+only as the checker / the timed CPU baseline.
+
+It issues the same ATen op sequence as the reference's ``use_te=False`` path so that
+(a) it can be timed as the reference's CPU path and (b) module construction consumes
+the global RNG in the same order as the reference (needed to reproduce the reference's
+golden output files).  Each function cites the reference lines it follows; paths are
+relative to the reference checkout.
+
+Pinning status (what checks this file, see tests/test_oracle_*.py):
+  * every stage against the independent float64 NumPy restatement in
+    ``oracle/numpy_oracle.py`` (different code, loops / einsum in float64);
+  * closed forms and invariants (softmax rows, clamp special cases, norm sum,
+    N=1 eps case, zero slice weight => hand-computable layer output, k=1 conv == linear);
+  * the reference's own golden outputs ``tests/golden/transolver2d_output.pth`` and
+    ``transolver_irregular_output.pth`` (whole model, rtol 1e-3 / atol 2e-3 and 1e-3).
+"""
+
+from __future__ import annotations
+
+import math
+
+import numpy as np
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+SLICE_NORM_EPS = 1e-2  # physicsnemo/nn/module/physics_attention.py:185
+TEMP_MIN, TEMP_MAX = 0.5, 5.0  # physics_attention.py:173
+
+
+# --------------------------------------------------------------------------- stages
+def split_heads(t: torch.Tensor, heads: int, dim_head: int) -> torch.Tensor:
+    """(B, N, H*D) -> (B, N, H, D), channel c = h*D + d (physics_attention.py:114, pattern :658)."""
+    b, n, _ = t.shape
+    return t.reshape(b, n, heads, dim_head)
+
+
+def project_linear(x, wx, bx, wfx, bfx, heads, dim_head):
+    """Irregular-mesh projections (physics_attention.py:652-660 -> :114-117)."""
+    x_mid = split_heads(F.linear(x, wx, bx), heads, dim_head)
+    fx_mid = split_heads(F.linear(x, wfx, bfx), heads, dim_head)
+    return x_mid, fx_mid
+
+
+def project_conv2d(x, wx, bx, wfx, bfx, heads, dim_head, grid_h, grid_w):
+    """Structured-2D projections (physics_attention.py:768-783).
+
+    x is (B, N, C) with N = grid_h*grid_w, token n = i*grid_w + j; the reference views it
+    as NHWC, permutes to NCHW, applies a stride-1 zero-padded k x k cross-correlation
+    (padding k//2) and flattens back with "B (H D) h w -> B (h w) H D".
+    """
+    b, n, c = x.shape
+    k = wx.shape[-1]
+    img = x.view(b, grid_h, grid_w, c).permute(0, 3, 1, 2)
+
+    def one(w, bias):
+        y = F.conv2d(img, w, bias, stride=1, padding=k // 2)  # (B, H*D, h, w)
+        y = y.flatten(2).transpose(1, 2)  # (B, h*w, H*D)
+        return split_heads(y, heads, dim_head)
+
+    return one(wx, bx), one(wfx, bfx)
+
+
+def slice_logits(x_mid, w_slice, b_slice):
+    """in_project_slice on the head-split tensor (physics_attention.py:537): one (S, D) weight for all heads."""
+    return F.linear(x_mid, w_slice, b_slice)
+
+
+def slice_weights_and_tokens(logits, fx_mid, temperature):
+    """Temperature softmax + normalised aggregation (physics_attention.py:172-206, plus=False branch).
+
+    Returns (w, slice_token, slice_norm): w is the UN-normalised softmax (B, N, H, S); slice_token
+    (B, H, S, D) = sum_n (w / (sum_n w + 1e-2)) * fx_mid.
+    """
+    temp = torch.clamp(temperature, min=TEMP_MIN, max=TEMP_MAX).to(logits.dtype)
+    w = F.softmax(logits / temp, dim=-1)
+    w = w.to(logits.dtype)
+    norm = w.sum(1) + SLICE_NORM_EPS  # (B, H, S)
+    normed = w / norm[:, None, :, :]
+    tok = torch.matmul(normed.permute(0, 2, 3, 1), fx_mid.permute(0, 2, 1, 3))
+    return w, tok, norm
+
+
+def slice_attention(tok, w_qkv, dim_head):
+    """Self-attention among the S slice tokens of each (batch, head) (physics_attention.py:448-463).
+
+    qkv columns are [q | k | v]; SDPA default scale 1/sqrt(D), no mask.
+    """
+    qkv = F.linear(tok, w_qkv)  # (B, H, S, 3D), no bias (:309)
+    b, h, s, _ = qkv.shape
+    qkv = qkv.reshape(b, h, s, 3, dim_head)
+    q, k, v = qkv.unbind(3)
+    return F.scaled_dot_product_attention(q, k, v, is_causal=False)
+
+
+def deslice_and_project(w, tok_out, w_out, b_out):
+    """Scatter slice tokens back to points, merge heads, output projection (physics_attention.py:492-499)."""
+    o = torch.einsum("bths,bhsd->bthd", w, tok_out)
+    o = o.reshape(o.shape[0], o.shape[1], -1)
+    return F.linear(o, w_out, b_out)
+
+
+# --------------------------------------------------------------------------- modules
+class _AttentionCore(nn.Module):
+    """Parameter container + forward shared by both variants.
+
+    Sub-module registration order equals the reference base class
+    (physics_attention.py:281-327) so that ``state_dict`` order and RNG draws match:
+    softmax, dropout, in_project_slice (+orthogonal_), qkv_project, out_linear, out_dropout.
+    """
+
+    def __init__(self, dim, heads, dim_head, dropout, slice_num):
+        super().__init__()
+        self.dim, self.heads, self.dim_head, self.slice_num = dim, heads, dim_head, slice_num
+        self.softmax = nn.Softmax(dim=-1)
+        self.dropout = nn.Dropout(dropout)
+        self.temperature = nn.Parameter(torch.full((1, 1, heads, 1), 0.5))
+        self.in_project_slice = nn.Linear(dim_head, slice_num)
+        nn.init.orthogonal_(self.in_project_slice.weight)
+        self.qkv_project = nn.Linear(dim_head, 3 * dim_head, bias=False)
+        self.out_linear = nn.Linear(heads * dim_head, dim)
+        self.out_dropout = nn.Dropout(dropout)
+
+    def _project(self, x):  # pragma: no cover - abstract
+        raise NotImplementedError
+
+    def stages(self, x):
+        """Forward returning every intermediate (used by the parity tests)."""
+        x_mid, fx_mid = self._project(x)
+        logits = slice_logits(x_mid, self.in_project_slice.weight, self.in_project_slice.bias)
+        w, tok, norm = slice_weights_and_tokens(logits, fx_mid, self.temperature)
+        tok_out = slice_attention(tok, self.qkv_project.weight, self.dim_head)
+        y = deslice_and_project(w, tok_out, self.out_linear.weight, self.out_linear.bias)
+        return dict(x_mid=x_mid, fx_mid=fx_mid, logits=logits, w=w, tok=tok, norm=norm,
+                    tok_out=tok_out, y=self.out_dropout(y))
+
+    def forward(self, x):
+        # Validation and messages: physics_attention.py:516-526
+        if x.ndim != 3:
+            raise ValueError(
+                f"Expected 3D input tensor (B, N, C), got {x.ndim}D tensor with shape {tuple(x.shape)}"
+            )
+        if x.shape[-1] != self.dim:
+            raise ValueError(f"Expected input feature dimension {self.dim}, got {x.shape[-1]}")
+        return self.stages(x)["y"]
+
+
+class OraclePhysicsAttentionIrregularMesh(_AttentionCore):
+    """physics_attention.py:561-660 with use_te=False, plus=False."""
+
+    def __init__(self, dim, heads=8, dim_head=64, dropout=0.0, slice_num=64):
+        super().__init__(dim, heads, dim_head, dropout, slice_num)
+        self.in_project_x = nn.Linear(dim, heads * dim_head)
+        self.in_project_fx = nn.Linear(dim, heads * dim_head)
+
+    def _project(self, x):
+        return project_linear(x, self.in_project_x.weight, self.in_project_x.bias,
+                              self.in_project_fx.weight, self.in_project_fx.bias,
+                              self.heads, self.dim_head)
+
+
+class OraclePhysicsAttentionStructuredMesh2D(_AttentionCore):
+    """physics_attention.py:663-783 with use_te=False, plus=False."""
+
+    def __init__(self, dim, spatial_shape, heads=8, dim_head=64, dropout=0.0, slice_num=64, kernel=3):
+        super().__init__(dim, heads, dim_head, dropout, slice_num)
+        self.H, self.W = spatial_shape[0], spatial_shape[1]
+        inner = heads * dim_head
+        self.in_project_x = nn.Conv2d(dim, inner, kernel, 1, kernel // 2)
+        self.in_project_fx = nn.Conv2d(dim, inner, kernel, 1, kernel // 2)
+
+    def _project(self, x):
+        return project_conv2d(x, self.in_project_x.weight, self.in_project_x.bias,
+                              self.in_project_fx.weight, self.in_project_fx.bias,
+                              self.heads, self.dim_head, self.H, self.W)
+
+
+class OracleMlp(nn.Module):
+    """Linear -> GELU(erf) -> Linear, keys ``layers.0`` / ``layers.2``
+    (physicsnemo/nn/module/mlp_layers.py:139-173 with one hidden width; activations.py:198 'gelu' -> nn.GELU())."""
+
+    def __init__(self, in_features, hidden_features, out_features):
+        super().__init__()
+        self.layers = nn.Sequential(
+            nn.Linear(in_features, hidden_features), nn.GELU(), nn.Linear(hidden_features, out_features)
+        )
+
+    def forward(self, x):
+        return self.layers(x)
+
+
+class OracleTransolverBlock(nn.Module):
+    """physicsnemo/models/transolver/transolver.py:182-309 (use_te=False). Order: ln_1, Attn, ln_mlp1, [ln_mlp2]."""
+
+    def __init__(self, num_heads, hidden_dim, dropout=0.0, mlp_ratio=4, last_layer=False, out_dim=1,
+                 slice_num=32, spatial_shape=None):
+        super().__init__()
+        self.last_layer = last_layer
+        self.ln_1 = nn.LayerNorm(hidden_dim)
+        if spatial_shape is None:
+            self.Attn = OraclePhysicsAttentionIrregularMesh(
+                hidden_dim, heads=num_heads, dim_head=hidden_dim // num_heads, dropout=dropout, slice_num=slice_num)
+        elif len(spatial_shape) == 2:
+            self.Attn = OraclePhysicsAttentionStructuredMesh2D(
+                hidden_dim, spatial_shape=spatial_shape, heads=num_heads, dim_head=hidden_dim // num_heads,
+                dropout=dropout, slice_num=slice_num)
+        else:
+            raise ValueError("oracle covers irregular and structured-2D variants only")
+        self.ln_mlp1 = nn.Sequential(nn.LayerNorm(hidden_dim),
+                                     OracleMlp(hidden_dim, hidden_dim * mlp_ratio, hidden_dim))
+        if last_layer:
+            self.ln_mlp2 = nn.Sequential(nn.LayerNorm(hidden_dim), nn.Linear(hidden_dim, out_dim))
+
+    def forward(self, fx):
+        fx = self.Attn(self.ln_1(fx)) + fx  # transolver.py:300
+        fx = self.ln_mlp1(fx) + fx  # :303
+        return self.ln_mlp2(fx) if self.last_layer else fx  # :306-309
+
+
+def unified_pos_grid(structured_shape, ref):
+    """Distance of every grid point (i/(h-1), j/(w-1)) to a ref x ref lattice on [0,1]^2
+    (transolver.py:617-645), shape (1, h*w, ref*ref), float32."""
+    h, w = structured_shape
+    gx = torch.tensor(np.linspace(0, 1, h), dtype=torch.float)
+    gy = torch.tensor(np.linspace(0, 1, w), dtype=torch.float)
+    grid = torch.stack(torch.meshgrid(gx, gy, indexing="ij"), dim=-1)  # (h, w, 2)
+    rx = torch.tensor(np.linspace(0, 1, ref), dtype=torch.float)
+    lattice = torch.stack(torch.meshgrid(rx, rx, indexing="ij"), dim=-1)  # (ref, ref, 2)
+    diff = grid[:, :, None, None, :] - lattice[None, None, :, :, :]
+    return torch.sqrt((diff ** 2).sum(-1)).reshape(1, h * w, ref * ref).contiguous()
+
+
+def _trunc_normal_by_rejection_(t: torch.Tensor, std: float, a: float = -2.0, b: float = 2.0):
+    """trunc_normal_ as torch >= 2.12 draws it: ``normal_()`` then redraw values outside [a, b].
+
+    The reference's golden files are locked to that algorithm (test/common/fwdaccuracy.py:116-125).
+    With std = 0.02 and bounds +-2 the rejection branch is unreachable in practice (100 sigma).
+    """
+    with torch.no_grad():
+        t.normal_(0.0, std)
+        bad = (t < a) | (t > b)
+        while bool(bad.any()):
+            t[bad] = torch.empty(int(bad.sum())).normal_(0.0, std)
+            bad = (t < a) | (t > b)
+    return t
+
+
+class OracleTransolver(nn.Module):
+    """transolver.py:447-736 (use_te=False, time_input=False, plus=False).
+
+    ``init="rejection"`` draws trunc_normal_ the torch>=2.12 way (see above); ``init="native"`` calls
+    this interpreter's ``nn.init.trunc_normal_``.
+    """
+
+    def __init__(self, functional_dim, out_dim, embedding_dim=None, n_layers=4, n_hidden=256, dropout=0.0,
+                 n_head=8, mlp_ratio=4, slice_num=32, unified_pos=False, ref=8, structured_shape=None,
+                 init="native"):
+        super().__init__()
+        if n_hidden % n_head != 0:
+            raise ValueError(f"Transolver requires n_hidden % n_head == 0, but got n_hidden={n_hidden}, n_head={n_head}")
+        if structured_shape is None and unified_pos:
+            raise ValueError("Transolver requires structured_shape when using unified_pos=True")
+        self.structured_shape, self.unified_pos = structured_shape, unified_pos
+        if unified_pos:
+            self.register_buffer("embedding", unified_pos_grid(structured_shape, ref))
+            self.embedding_dim = ref * ref
+        else:
+            if embedding_dim is None:
+                raise ValueError("Transolver requires embedding_dim when unified_pos=False")
+            self.embedding_dim = embedding_dim
+        self.preprocess = OracleMlp(functional_dim + self.embedding_dim, n_hidden * 2, n_hidden)
+        self.n_hidden = n_hidden
+        self.blocks = nn.ModuleList([
+            OracleTransolverBlock(n_head, n_hidden, dropout, mlp_ratio=mlp_ratio, out_dim=out_dim,
+                                  slice_num=slice_num, spatial_shape=structured_shape,
+                                  last_layer=(i == n_layers - 1))
+            for i in range(n_layers)
+        ])
+        self._init_kind = init
+        self.apply(self._init_weights)  # transolver.py:566-593: post-order, every nn.Linear, LayerNorm -> (1, 0)
+
+    def _init_weights(self, m):
+        if isinstance(m, nn.Linear):
+            if self._init_kind == "rejection":
+                _trunc_normal_by_rejection_(m.weight, std=0.02)
+            else:
+                nn.init.trunc_normal_(m.weight, std=0.02)
+            if m.bias is not None:
+                nn.init.constant_(m.bias, 0)
+        if isinstance(m, nn.LayerNorm):
+            nn.init.constant_(m.bias, 0)
+            nn.init.constant_(m.weight, 1.0)
+
+    def forward(self, fx, embedding=None):
+        if fx.ndim < 2:
+            raise ValueError(f"Expected input tensor with at least 2 dimensions, got {fx.ndim}D tensor with shape {tuple(fx.shape)}")
+        if not self.unified_pos and embedding is None:
+            raise ValueError("Embedding is required when unified_pos=False")
+        unflatten = False
+        if self.unified_pos:
+            embedding = self.embedding.repeat(fx.shape[0], 1, 1)  # :690-693
+        if self.structured_shape is not None:
+            if fx.ndim != 3:
+                unflatten = True
+                fx = fx.reshape(fx.shape[0], -1, fx.shape[-1])
+            if embedding is not None and embedding.ndim != 3:
+                embedding = embedding.reshape(embedding.shape[0], -1, embedding.shape[-1])
+        fx = torch.cat((embedding, fx), -1)  # embedding FIRST (:716)
+        fx = self.preprocess(fx)
+        for blk in self.blocks:
+            fx = blk(fx)
+        if unflatten:
+            fx = fx.reshape(fx.shape[0], *self.structured_shape, -1)
+        return fx
+
+
+def rel_l2(a: torch.Tensor, b: torch.Tensor) -> float:
+    """||a - b||_2 / ||b||_2 in float64."""
+    a64, b64 = a.double().flatten(), b.double().flatten()
+    return float((a64 - b64).norm() / b64.norm().clamp_min(1e-300))
+
+
+def sdpa_scale(dim_head: int) -> float:
+    return 1.0 / math.sqrt(dim_head)
