@@ -1,0 +1,141 @@
+/*
+ * physattn.h -- C ABI of libphysattn.so: the forward pass of Transolver's PhysicsAttention layer on
+ * AMD MI355X (gfx950), hand-written HIP kernels.
+ *
+ * The reference implementation is pure Python (PyTorch ATen ops) and has no native interface; every
+ * entry point below cites the reference code it replaces (paths relative to the reference checkout,
+ * physicsnemo/nn/module/physics_attention.py is abbreviated PA.py, physicsnemo/models/transolver/
+ * transolver.py is abbreviated TR.py).
+ *
+ * Conventions
+ *   - Plain pointers and sizes only.  All tensor pointers are DEVICE pointers, 16-byte aligned,
+ *     contiguous row-major (last index fastest) in the shapes stated.
+ *   - Symbols: B batch, N points per batch, C = layer width `dim`, H heads, D dim_head, S slice_num.
+ *   - `dtype` selects the ACTIVATION element type (x, intermediates, y) and the element type of the
+ *     three large weights (in_project_x, in_project_fx, out_linear): PA_F32 or PA_BF16.
+ *     Small parameters are ALWAYS float32: every bias, temperature (H), in_project_slice weight (S,D)
+ *     and bias (S), qkv_project weight (3D,D), LayerNorm gamma/beta.
+ *     Slice tokens, slice norms and reduction partials are ALWAYS float32.
+ *   - Ownership: the caller allocates every input, output and workspace.  The library never
+ *     allocates, frees or keeps a pointer after the call returns.
+ *   - Every call only enqueues work on `stream` (a hipStream_t passed as void*; NULL = the default
+ *     stream); it never synchronises the host.  Calls are re-entrant.
+ *   - Return value: 0 = success; negative = argument error (see PA_ERR_*), nothing was enqueued;
+ *     positive = hipError_t reported by a launch.  Nothing throws or aborts across this boundary.
+ */
+#ifndef PHYSATTN_H
+#define PHYSATTN_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define PA_F32 0
+#define PA_BF16 1
+
+#define PA_OK 0
+#define PA_ERR_NULL (-1)        /* a required pointer is NULL */
+#define PA_ERR_DIMS (-2)        /* a dimension is <= 0 or inconsistent */
+#define PA_ERR_UNSUPPORTED (-3) /* shape/dtype outside what the kernels serve */
+#define PA_ERR_ALIGN (-4)       /* a pointer is not 16-byte aligned */
+#define PA_ERR_WORKSPACE (-5)   /* workspace too small */
+
+/* Limits of the general kernels (PA_ERR_UNSUPPORTED beyond them). */
+#define PA_MAX_D 128
+#define PA_MAX_S 256
+
+/* Library version (major*10000 + minor*100 + patch). No reference counterpart. */
+int pa_version(void);
+
+/* Static text for a PA_ERR_* code (or "hip error" for positive codes). No reference counterpart. */
+const char *pa_status_string(int code);
+
+/* Dimensions of one layer call.  `conv_k` = 0 selects the irregular-mesh variant (nn.Linear
+ * projections, PA.py:625-627); conv_k = k > 0 selects the structured-2D variant (k x k Conv2d,
+ * stride 1, zero padding k/2, PA.py:740-742) and then N must equal grid_h*grid_w with token
+ * n = i*grid_w + j (PA.py:772-783). */
+typedef struct pa_shape {
+  int64_t B, N, C, H, D, S;
+  int64_t grid_h, grid_w, conv_k;
+} pa_shape;
+
+/* Parameters of one layer, named as the reference state_dict keys (PA.py:285-327, :625-627, :740-742). */
+typedef struct pa_params {
+  const void *in_project_x_weight;   /* dtype, (H*D, C) or (H*D, C, k, k) */
+  const float *in_project_x_bias;    /* (H*D) */
+  const void *in_project_fx_weight;  /* dtype, same shape */
+  const float *in_project_fx_bias;   /* (H*D) */
+  const float *in_project_slice_weight; /* (S, D), shared by all heads (PA.py:301,537) */
+  const float *in_project_slice_bias;   /* (S) */
+  const float *temperature;          /* (H); clamped to [0.5, 5] inside (PA.py:173) */
+  const float *qkv_project_weight;   /* (3D, D), rows [q | k | v], no bias (PA.py:309,450) */
+  const void *out_linear_weight;     /* dtype, (C, H*D) */
+  const float *out_linear_bias;      /* (C) */
+} pa_params;
+
+/* Optional fused tail of the caller TransolverBlock.forward (TR.py:300-303):
+ *   fx_new = y + residual;  ln_out = LayerNorm(fx_new; gamma, beta, eps)
+ * All-NULL / zero = plain layer output. */
+typedef struct pa_block_tail {
+  const void *residual; /* dtype, (B, N, C) or NULL */
+  const float *ln_gamma; /* (C) or NULL */
+  const float *ln_beta;  /* (C) or NULL */
+  float ln_eps;          /* torch default 1e-5 */
+  void *ln_out;          /* dtype, (B, N, C) or NULL */
+} pa_block_tail;
+
+/* Bytes of caller-provided workspace pa_layer_forward needs for this shape. Negative = error code. */
+int64_t pa_workspace_bytes(int dtype, const pa_shape *shape);
+
+/* Which kernel family serves this shape: 0 = general kernels (fp32 FMA), 1 = bf16 MFMA kernels.
+ * Negative = error code.  No reference counterpart. */
+int pa_query_path(int dtype, const pa_shape *shape);
+
+/* ---- stage-level entry points (natural layouts; general kernels) ------------------------------ */
+
+/* Stage (a1): input projections, replaces project_input_onto_slices (PA.py:629-660 irregular,
+ * :744-783 structured 2D) -> x_mid, fx_mid as (B, N, H*D) with channel c = h*D + d. */
+int pa_project_inputs(int dtype, const pa_shape *shape, const pa_params *p, const void *x,
+                      void *x_mid, void *fx_mid, void *stream);
+
+/* Stage (a2): slice logits + temperature softmax, replaces in_project_slice (PA.py:537) and the
+ * softmax half of _compute_slices_from_projections (PA.py:172-181): w (B, N, H, S), rows sum to 1. */
+int pa_slice_softmax(int dtype, const pa_shape *shape, const pa_params *p, const void *x_mid, void *w,
+                     void *stream);
+
+/* Stage (b): slice-token aggregation, replaces PA.py:185-203.
+ *   partials: float32 scratch of pa_reduce_partial_count(shape) * B*H*S*(D+1) elements
+ *   slice_token (B,H,S,D) = (sum_n w fx_mid) / (sum_n w + 1e-2);  slice_norm (B,H,S) = sum_n w + 1e-2.
+ * Two passes: per-chunk partial sums, then a fixed-order combine (bit-reproducible, no atomics). */
+int64_t pa_reduce_partial_count(const pa_shape *shape);
+int pa_slice_reduce(int dtype, const pa_shape *shape, const void *w, const void *fx_mid, float *partials,
+                    float *slice_token, float *slice_norm, void *stream);
+
+/* Stage (c): self-attention among the S slice tokens of each (batch, head), replaces
+ * _compute_slice_attention_sdpa (PA.py:429-465): softmax(q k^T / sqrt(D)) v, float32, LDS resident. */
+int pa_slice_attention(const pa_shape *shape, const pa_params *p, const float *slice_token,
+                       float *out_slice_token, void *stream);
+
+/* Stage (d): deslice + out_linear (+ optional residual / LayerNorm tail), replaces
+ * _project_attention_outputs (PA.py:467-499) and TR.py:300-303.
+ *   scratch: dtype, (B, N, H*D) caller-provided. tail may be NULL. */
+int pa_deslice_project(int dtype, const pa_shape *shape, const pa_params *p, const void *w,
+                       const float *out_slice_token, void *scratch, void *y, const pa_block_tail *tail,
+                       void *stream);
+
+/* ---- whole layer ------------------------------------------------------------------------------ */
+
+/* Replaces PhysicsAttentionBase.forward (PA.py:501-558), plus=False, use_te=False, dropout off.
+ *   x (B,N,C) -> y (B,N,C) [= out_linear output; with a tail: y = fx_new, tail->ln_out = LN(fx_new)].
+ *   slice_token_out: optional float32 (B,H,S,D) copy of the aggregated slice tokens (may be NULL).
+ * Dispatches to the bf16 MFMA kernels when pa_query_path() == 1, else to the general kernels. */
+int pa_layer_forward(int dtype, const pa_shape *shape, const pa_params *p, const void *x, void *y,
+                     const pa_block_tail *tail, float *slice_token_out, void *workspace,
+                     int64_t workspace_bytes, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PHYSATTN_H */

@@ -1,0 +1,9 @@
+"""MI355X-native forward path of Transolver's PhysicsAttention layer (hand-written HIP kernels behind a C ABI)."""
+from .physics_attention import (  # noqa: F401
+    PhysicsAttentionBase,
+    PhysicsAttentionIrregularMesh,
+    PhysicsAttentionStructuredMesh2D,
+)
+from .transolver import Mlp, Transolver, TransolverBlock  # noqa: F401
+
+__version__ = "0.1.0"

@@ -1,0 +1,101 @@
+"""ctypes binding of libphysattn.so (see include/physattn.h for the contract of every symbol).
+
+PyTorch is used for device memory and streams only.  There is no fallback: if the library is not
+built, or a call returns an error code, a RuntimeError is raised.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from ctypes import POINTER, Structure, c_char_p, c_float, c_int, c_int64, c_void_p
+
+import torch  # noqa: F401  (must be imported first: its HIP runtime is the one the library binds to)
+
+LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libphysattn.so")
+
+PA_F32, PA_BF16 = 0, 1
+
+EXPORTED = [
+    "pa_version", "pa_status_string", "pa_workspace_bytes", "pa_query_path", "pa_project_inputs",
+    "pa_slice_softmax", "pa_reduce_partial_count", "pa_slice_reduce", "pa_slice_attention",
+    "pa_deslice_project", "pa_layer_forward",
+]
+
+
+class PaShape(Structure):
+    _fields_ = [(n, c_int64) for n in ("B", "N", "C", "H", "D", "S", "grid_h", "grid_w", "conv_k")]
+
+
+class PaParams(Structure):
+    _fields_ = [(n, c_void_p) for n in (
+        "in_project_x_weight", "in_project_x_bias", "in_project_fx_weight", "in_project_fx_bias",
+        "in_project_slice_weight", "in_project_slice_bias", "temperature", "qkv_project_weight",
+        "out_linear_weight", "out_linear_bias")]
+
+
+class PaBlockTail(Structure):
+    _fields_ = [("residual", c_void_p), ("ln_gamma", c_void_p), ("ln_beta", c_void_p), ("ln_eps", c_float),
+                ("ln_out", c_void_p)]
+
+
+_lib = None
+
+
+def load() -> ctypes.CDLL:
+    """Load the shared library once; raise if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            f"{LIB_PATH} is missing: build it with `python -m physicsnemo_amd.build` "
+            "(hipcc, gfx950). There is no fallback path.")
+    lib = ctypes.CDLL(LIB_PATH)
+    ps, pp, pt = POINTER(PaShape), POINTER(PaParams), POINTER(PaBlockTail)
+    lib.pa_version.restype = c_int
+    lib.pa_version.argtypes = []
+    lib.pa_status_string.restype = c_char_p
+    lib.pa_status_string.argtypes = [c_int]
+    lib.pa_workspace_bytes.restype = c_int64
+    lib.pa_workspace_bytes.argtypes = [c_int, ps]
+    lib.pa_query_path.restype = c_int
+    lib.pa_query_path.argtypes = [c_int, ps]
+    lib.pa_project_inputs.restype = c_int
+    lib.pa_project_inputs.argtypes = [c_int, ps, pp, c_void_p, c_void_p, c_void_p, c_void_p]
+    lib.pa_slice_softmax.restype = c_int
+    lib.pa_slice_softmax.argtypes = [c_int, ps, pp, c_void_p, c_void_p, c_void_p]
+    lib.pa_reduce_partial_count.restype = c_int64
+    lib.pa_reduce_partial_count.argtypes = [ps]
+    lib.pa_slice_reduce.restype = c_int
+    lib.pa_slice_reduce.argtypes = [c_int, ps, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]
+    lib.pa_slice_attention.restype = c_int
+    lib.pa_slice_attention.argtypes = [ps, pp, c_void_p, c_void_p, c_void_p]
+    lib.pa_deslice_project.restype = c_int
+    lib.pa_deslice_project.argtypes = [c_int, ps, pp, c_void_p, c_void_p, c_void_p, c_void_p, pt, c_void_p]
+    lib.pa_layer_forward.restype = c_int
+    lib.pa_layer_forward.argtypes = [c_int, ps, pp, c_void_p, c_void_p, pt, c_void_p, c_void_p, c_int64, c_void_p]
+    _lib = lib
+    return lib
+
+
+def check(code: int, what: str) -> None:
+    """Turn a non-zero return code into a RuntimeError."""
+    if code != 0:
+        msg = load().pa_status_string(int(code)).decode()
+        raise RuntimeError(f"{what} failed: {msg} (code {code})")
+
+
+def dtype_code(dtype: torch.dtype) -> int:
+    if dtype == torch.float32:
+        return PA_F32
+    if dtype == torch.bfloat16:
+        return PA_BF16
+    raise TypeError(f"physicsnemo_amd kernels take float32 or bfloat16 activations, got {dtype}")
+
+
+def current_stream_ptr(device: torch.device) -> int:
+    return int(torch.cuda.current_stream(device).cuda_stream)
+
+
+def ptr(t) -> int | None:
+    return None if t is None else int(t.data_ptr())

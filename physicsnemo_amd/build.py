@@ -1,0 +1,40 @@
+"""Build libphysattn.so for gfx950 with hipcc (in-tree, next to the sources)."""
+from __future__ import annotations
+
+import os
+import subprocess
+import sys
+
+PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(PKG_DIR, "csrc")
+LIB_PATH = os.path.join(PKG_DIR, "libphysattn.so")
+SOURCES = ["pa_api.hip", "pa_general.hip", "pa_mfma.hip"]
+
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+    # packed-FP32 VALU forms are kept off for every kernel in this library
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wall", "-Wno-unused-function",
+]
+
+
+def build(verbose: bool = True) -> str:
+    """Compile every HIP source into one shared library; returns its path. Raises on failure."""
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    srcs = [os.path.join(CSRC, s) for s in SOURCES if os.path.exists(os.path.join(CSRC, s))]
+    cmd = [hipcc, *HIPCC_FLAGS, *srcs, "-o", LIB_PATH + ".tmp"]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    out = "\n".join(l for l in proc.stdout.splitlines() if "packed-fp32-ops" not in l)
+    if proc.returncode != 0:
+        raise RuntimeError(f"hipcc failed ({proc.returncode}):\n{out}")
+    if verbose and out.strip():
+        print(out)
+    os.replace(LIB_PATH + ".tmp", LIB_PATH)
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    build()
+    sys.exit(0)

@@ -1,0 +1,205 @@
+// C ABI of libphysattn.so: argument validation, workspace carving and dispatch.  No kernels here.
+#include "pa_common.h"
+#include "pa_host.h"
+
+namespace {
+
+using pa::aligned16;
+
+int check_shape(int dtype, const pa_shape *s) {
+  if (!s) return PA_ERR_NULL;
+  if (dtype != PA_F32 && dtype != PA_BF16) return PA_ERR_UNSUPPORTED;
+  if (s->B <= 0 || s->N <= 0 || s->C <= 0 || s->H <= 0 || s->D <= 0 || s->S <= 0) return PA_ERR_DIMS;
+  if (s->conv_k < 0) return PA_ERR_DIMS;
+  if (s->conv_k > 0) {
+    if (s->grid_h <= 0 || s->grid_w <= 0 || s->grid_h * s->grid_w != s->N) return PA_ERR_DIMS;
+    if (s->conv_k % 2 == 0) return PA_ERR_UNSUPPORTED;  // even kernels change the output size in the reference
+  }
+  if (s->D > PA_MAX_D || s->S > PA_MAX_S) return PA_ERR_UNSUPPORTED;
+  if (s->C > (1 << 16) || s->H > 1024) return PA_ERR_UNSUPPORTED;
+  if (s->N > (int64_t)1 << 31 || s->B > (1 << 20)) return PA_ERR_UNSUPPORTED;
+  if (s->B * s->H > 65535) return PA_ERR_UNSUPPORTED;  // grid.y of the reduction
+  if (pa::general::combine_attn_lds_bytes(*s) > pa::kMaxLdsBytes) return PA_ERR_UNSUPPORTED;
+  return PA_OK;
+}
+
+int64_t round_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
+
+int64_t elem_bytes(int dtype) { return dtype == PA_F32 ? 4 : 2; }
+
+// Workspace plan of the general path.
+struct GeneralPlan {
+  int64_t off_x_mid, off_fx_mid, off_w, off_partials, off_tok, off_norm, off_tok_out, total;
+  int64_t G;
+};
+
+GeneralPlan plan_general(int dtype, const pa_shape &s) {
+  GeneralPlan p{};
+  const int64_t e = elem_bytes(dtype), M = s.B * s.N, HD = s.H * s.D;
+  p.G = pa::general::partial_count(s);
+  int64_t off = 0;
+  p.off_x_mid = off;  // reused for out_x once the slice weights exist
+  off += round_up(M * HD * e, 256);
+  p.off_fx_mid = off;
+  off += round_up(M * HD * e, 256);
+  p.off_w = off;
+  off += round_up(M * s.H * s.S * e, 256);
+  p.off_partials = off;
+  off += round_up(p.G * s.B * s.H * s.S * (s.D + 1) * 4, 256);
+  p.off_tok = off;
+  off += round_up(s.B * s.H * s.S * s.D * 4, 256);
+  p.off_norm = off;
+  off += round_up(s.B * s.H * s.S * 4, 256);
+  p.off_tok_out = off;
+  off += round_up(s.B * s.H * s.S * s.D * 4, 256);
+  p.total = off;
+  return p;
+}
+
+int check_params(const pa_params *p) {
+  if (!p) return PA_ERR_NULL;
+  if (!p->in_project_x_weight || !p->in_project_x_bias || !p->in_project_fx_weight || !p->in_project_fx_bias ||
+      !p->in_project_slice_weight || !p->in_project_slice_bias || !p->temperature || !p->qkv_project_weight ||
+      !p->out_linear_weight || !p->out_linear_bias)
+    return PA_ERR_NULL;
+  if (!aligned16(p->in_project_x_weight) || !aligned16(p->in_project_fx_weight) || !aligned16(p->out_linear_weight))
+    return PA_ERR_ALIGN;
+  return PA_OK;
+}
+
+int check_tail(const pa_block_tail *t) {
+  if (!t) return PA_OK;
+  if (t->ln_out && (!t->ln_gamma || !t->ln_beta)) return PA_ERR_NULL;
+  if (!aligned16(t->residual) || !aligned16(t->ln_out)) return PA_ERR_ALIGN;
+  return PA_OK;
+}
+
+bool tail_active(const pa_block_tail *t) { return t && (t->residual || t->ln_out); }
+
+}  // namespace
+
+extern "C" {
+
+int pa_version(void) { return 100; }
+
+const char *pa_status_string(int code) {
+  switch (code) {
+    case PA_OK: return "ok";
+    case PA_ERR_NULL: return "a required pointer is NULL";
+    case PA_ERR_DIMS: return "a dimension is non-positive or inconsistent";
+    case PA_ERR_UNSUPPORTED: return "shape or dtype outside the supported range";
+    case PA_ERR_ALIGN: return "a pointer is not 16-byte aligned";
+    case PA_ERR_WORKSPACE: return "workspace too small";
+    default: return code > 0 ? "hip error" : "unknown error";
+  }
+}
+
+int pa_query_path(int dtype, const pa_shape *shape) {
+  int rc = check_shape(dtype, shape);
+  if (rc) return rc;
+  return 0;
+}
+
+int64_t pa_workspace_bytes(int dtype, const pa_shape *shape) {
+  int rc = check_shape(dtype, shape);
+  if (rc) return rc;
+  return plan_general(dtype, *shape).total;
+}
+
+int pa_project_inputs(int dtype, const pa_shape *shape, const pa_params *p, const void *x, void *x_mid, void *fx_mid,
+                      void *stream) {
+  int rc = check_shape(dtype, shape);
+  if (rc) return rc;
+  if ((rc = check_params(p))) return rc;
+  if (!x || !x_mid || !fx_mid) return PA_ERR_NULL;
+  if (!aligned16(x) || !aligned16(x_mid) || !aligned16(fx_mid)) return PA_ERR_ALIGN;
+  return pa::general::project_inputs(dtype, *shape, *p, x, x_mid, fx_mid, static_cast<hipStream_t>(stream));
+}
+
+int pa_slice_softmax(int dtype, const pa_shape *shape, const pa_params *p, const void *x_mid, void *w, void *stream) {
+  int rc = check_shape(dtype, shape);
+  if (rc) return rc;
+  if (!p || !p->in_project_slice_weight || !p->in_project_slice_bias || !p->temperature || !x_mid || !w) return PA_ERR_NULL;
+  if (!aligned16(x_mid) || !aligned16(w)) return PA_ERR_ALIGN;
+  return pa::general::slice_softmax(dtype, *shape, *p, x_mid, w, static_cast<hipStream_t>(stream));
+}
+
+int64_t pa_reduce_partial_count(const pa_shape *shape) {
+  int rc = check_shape(PA_F32, shape);
+  if (rc) return rc;
+  return pa::general::partial_count(*shape);
+}
+
+int pa_slice_reduce(int dtype, const pa_shape *shape, const void *w, const void *fx_mid, float *partials,
+                    float *slice_token, float *slice_norm, void *stream) {
+  int rc = check_shape(dtype, shape);
+  if (rc) return rc;
+  if (!w || !fx_mid || !partials || !slice_token || !slice_norm) return PA_ERR_NULL;
+  if (!aligned16(w) || !aligned16(fx_mid) || !aligned16(partials)) return PA_ERR_ALIGN;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  rc = pa::general::slice_partial(dtype, *shape, w, fx_mid, partials, st);
+  if (rc) return rc;
+  // the combine kernel also runs the slice attention; here only its token/norm outputs are wanted
+  pa_params none{};
+  return pa::general::combine_attention(*shape, none, partials, pa::general::partial_count(*shape), slice_token,
+                                        slice_norm, nullptr, st);
+}
+
+int pa_slice_attention(const pa_shape *shape, const pa_params *p, const float *slice_token, float *out_slice_token,
+                       void *stream) {
+  int rc = check_shape(PA_F32, shape);
+  if (rc) return rc;
+  if (!p || !p->qkv_project_weight || !slice_token || !out_slice_token) return PA_ERR_NULL;
+  // tokens enter as a single already-normalised "partial": the numerators with a zero count column
+  // are not available here, so this entry point uses the dedicated token-input mode (G = 0).
+  return pa::general::combine_attention(*shape, *p, slice_token, 0, nullptr, nullptr, out_slice_token,
+                                        static_cast<hipStream_t>(stream));
+}
+
+int pa_deslice_project(int dtype, const pa_shape *shape, const pa_params *p, const void *w, const float *out_slice_token,
+                       void *scratch, void *y, const pa_block_tail *tail, void *stream) {
+  int rc = check_shape(dtype, shape);
+  if (rc) return rc;
+  if (!p || !p->out_linear_weight || !p->out_linear_bias || !w || !out_slice_token || !scratch || !y) return PA_ERR_NULL;
+  if (!aligned16(w) || !aligned16(scratch) || !aligned16(y) || !aligned16(p->out_linear_weight)) return PA_ERR_ALIGN;
+  if ((rc = check_tail(tail))) return rc;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if ((rc = pa::general::deslice(dtype, *shape, w, out_slice_token, scratch, st))) return rc;
+  if ((rc = pa::general::out_linear(dtype, *shape, *p, scratch, y, st))) return rc;
+  if (tail_active(tail)) rc = pa::general::residual_ln(dtype, *shape, y, *tail, st);
+  return rc;
+}
+
+int pa_layer_forward(int dtype, const pa_shape *shape, const pa_params *p, const void *x, void *y,
+                     const pa_block_tail *tail, float *slice_token_out, void *workspace, int64_t workspace_bytes,
+                     void *stream) {
+  int rc = check_shape(dtype, shape);
+  if (rc) return rc;
+  if ((rc = check_params(p))) return rc;
+  if (!x || !y || !workspace) return PA_ERR_NULL;
+  if (!aligned16(x) || !aligned16(y) || !aligned16(workspace)) return PA_ERR_ALIGN;
+  if ((rc = check_tail(tail))) return rc;
+  const pa_shape &s = *shape;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+
+  const GeneralPlan plan = plan_general(dtype, s);
+  if (workspace_bytes < plan.total) return PA_ERR_WORKSPACE;
+  char *ws = static_cast<char *>(workspace);
+  void *x_mid = ws + plan.off_x_mid, *fx_mid = ws + plan.off_fx_mid, *w = ws + plan.off_w;
+  float *partials = reinterpret_cast<float *>(ws + plan.off_partials);
+  float *tok = slice_token_out ? slice_token_out : reinterpret_cast<float *>(ws + plan.off_tok);
+  float *norm = reinterpret_cast<float *>(ws + plan.off_norm);
+  float *tok_out = reinterpret_cast<float *>(ws + plan.off_tok_out);
+
+  if ((rc = pa::general::project_inputs(dtype, s, *p, x, x_mid, fx_mid, st))) return rc;
+  if ((rc = pa::general::slice_softmax(dtype, s, *p, x_mid, w, st))) return rc;
+  if ((rc = pa::general::slice_partial(dtype, s, w, fx_mid, partials, st))) return rc;
+  if ((rc = pa::general::combine_attention(s, *p, partials, plan.G, tok, norm, tok_out, st))) return rc;
+  void *out_x = x_mid;
+  if ((rc = pa::general::deslice(dtype, s, w, tok_out, out_x, st))) return rc;
+  if ((rc = pa::general::out_linear(dtype, s, *p, out_x, y, st))) return rc;
+  if (tail_active(tail)) rc = pa::general::residual_ln(dtype, s, y, *tail, st);
+  return rc;
+}
+
+}  // extern "C"

@@ -1,0 +1,55 @@
+// Shared device helpers for the PhysicsAttention kernels (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/physattn.h"
+
+namespace pa {
+
+constexpr float kSliceNormEps = 1e-2f;  // PA.py:185
+constexpr float kTempMin = 0.5f;        // PA.py:173
+constexpr float kTempMax = 5.0f;
+constexpr float kLog2e = 1.4426950408889634f;
+
+// bf16 stored as raw 16 bits; conversions are round-to-nearest-even like torch's.
+struct bf16 {
+  uint16_t bits;
+};
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint16_t b) { return __uint_as_float(((uint32_t)b) << 16); }
+
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);  // quiet NaN
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+
+__device__ __forceinline__ float load_as_f32(const float *p) { return *p; }
+__device__ __forceinline__ float load_as_f32(const bf16 *p) { return bf16_bits_to_f32(p->bits); }
+__device__ __forceinline__ void store_from_f32(float *p, float v) { *p = v; }
+__device__ __forceinline__ void store_from_f32(bf16 *p, float v) { p->bits = f32_to_bf16_bits(v); }
+
+// value after a round trip through the storage type (what a later kernel will read back)
+__device__ __forceinline__ float round_to(const float *, float v) { return v; }
+__device__ __forceinline__ float round_to(const bf16 *, float v) { return bf16_bits_to_f32(f32_to_bf16_bits(v)); }
+
+__device__ __forceinline__ float clamp_temperature(float t) { return fminf(fmaxf(t, kTempMin), kTempMax); }
+
+// wave64 butterfly reductions
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+  return v;
+}
+
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+}  // namespace pa

@@ -1,0 +1,560 @@
+// General PhysicsAttention kernels: any (C, H, D, S) within the library limits, fp32 or bf16 storage,
+// fp32 arithmetic on the vector ALUs, natural tensor layouts.  They serve fp32 runs (rtol 1e-4 class),
+// the structured-2D (Conv2d) projections and every shape the MFMA kernels do not cover.
+//
+// Stage map (reference lines in include/physattn.h):
+//   rows_gemm_kernel          in_project_x / in_project_fx (Linear or k x k Conv2d as implicit GEMM), out_linear
+//   slice_softmax_kernel      in_project_slice + clamp(temperature) + softmax over S
+//   slice_partial_kernel      per-chunk sums  sum_n w[n,s] * [fx_mid[n,:], 1]
+//   slice_combine_attn_kernel fixed-order combine, / (norm + 1e-2), qkv, softmax(q k^T / sqrt D) v   (LDS resident)
+//   deslice_kernel            out_x[n,h,:] = sum_s w[n,h,s] * tok'[h,s,:]
+//   residual_ln_kernel        fx_new = y + residual; ln_out = LayerNorm(fx_new)
+#include "pa_common.h"
+#include "pa_host.h"
+
+namespace pa {
+namespace general {
+
+// ------------------------------------------------------------------------------------------------
+// rows_gemm_kernel: out[m, o] = bias[o] + sum_k A(m, k) * W[o, k]
+//   linear: A(m, k) = in[m*K + k]
+//   conv  : K = ks*ks*C, k = tap*C + c, tap = u*ks + v; A(m,k) = in[b, (i+u-p)*gw + (j+v-p), c] or 0 outside
+//           the grid; the PyTorch weight element is W[o, c, u, v] = W[o*K + c*ks*ks + tap].
+// 64x64 output tile per 256-thread workgroup, 4x4 outputs per thread, K staged 16 at a time through LDS.
+// blockIdx.z selects one of two (W, bias, out) sets that share the same input (x_mid and fx_mid).
+// ------------------------------------------------------------------------------------------------
+struct GemmArgs {
+  const void *in;
+  const void *w[2];
+  const float *bias[2];
+  void *out[2];
+  int64_t M;   // rows = B*N
+  int K, O;    // reduction length, output columns
+  int C, N, gh, gw, ks;  // conv geometry (ks = 0: linear)
+};
+
+template <typename TA, typename TW>
+__global__ __launch_bounds__(256) void rows_gemm_kernel(GemmArgs a) {
+  __shared__ float As[16][64 + 4];
+  __shared__ float Ws[16][64 + 4];
+  const int z = blockIdx.z;
+  const TA *in = static_cast<const TA *>(a.in);
+  const TW *W = static_cast<const TW *>(a.w[z]);
+  const float *bias = a.bias[z];
+  TA *out = static_cast<TA *>(a.out[z]);
+  const int t = threadIdx.x;
+  const int tx = t & 15, ty = t >> 4;
+  const int64_t m0 = (int64_t)blockIdx.x * 64;
+  const int o0 = blockIdx.y * 64;
+  const int lr = t >> 2;         // tile row / tile out column this thread stages
+  const int lk = (t & 3) * 4;    // first of 4 consecutive k it stages
+  const int pad = a.ks / 2;
+  const int taps = a.ks * a.ks;
+
+  // decode the staged row once
+  const int64_t m_ld = m0 + lr;
+  const bool m_ok = m_ld < a.M;
+  int64_t b_ld = 0;
+  int i_ld = 0, j_ld = 0;
+  if (a.ks > 0 && m_ok) {
+    b_ld = m_ld / a.N;
+    int n = (int)(m_ld - b_ld * a.N);
+    i_ld = n / a.gw;
+    j_ld = n - i_ld * a.gw;
+  }
+  const int o_ld = o0 + lr;
+
+  float acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+
+  for (int k0 = 0; k0 < a.K; k0 += 16) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int k = k0 + lk + q;
+      float av = 0.f, wv = 0.f;
+      if (k < a.K) {
+        if (a.ks == 0) {
+          if (m_ok) av = load_as_f32(in + m_ld * a.K + k);
+          if (o_ld < a.O) wv = load_as_f32(W + (int64_t)o_ld * a.K + k);
+        } else {
+          const int tap = k / a.C, c = k - tap * a.C;
+          const int u = tap / a.ks, v = tap - u * a.ks;
+          const int ii = i_ld + u - pad, jj = j_ld + v - pad;
+          if (m_ok && ii >= 0 && ii < a.gh && jj >= 0 && jj < a.gw)
+            av = load_as_f32(in + ((b_ld * a.N + (int64_t)ii * a.gw + jj) * a.C + c));
+          if (o_ld < a.O) wv = load_as_f32(W + (int64_t)o_ld * a.K + (int64_t)c * taps + tap);
+        }
+      }
+      As[lk + q][lr] = av;
+      Ws[lk + q][lr] = wv;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < 16; ++kk) {
+      float av[4], wv[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) av[i] = As[kk][ty * 4 + i];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) wv[j] = Ws[kk][tx * 4 + j];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(av[i], wv[j], acc[i][j]);
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int64_t m = m0 + ty * 4 + i;
+    if (m >= a.M) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int o = o0 + tx * 4 + j;
+      if (o < a.O) store_from_f32(out + m * a.O + o, acc[i][j] + (bias ? bias[o] : 0.f));
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// slice_softmax_kernel: R consecutive rows (points) per workgroup.
+//   logits[r,h,s] = bias[s] + sum_d x_mid[r, h*D+d] * Wslice[s, d];  w = softmax_s(logits / clamp(T_h, .5, 5))
+// LDS: x rows (head stride D+1), Wslice, logits/weights (row stride S+1).  The finished block of
+// R*H*S weights is contiguous in global memory and is written with unit stride.
+// ------------------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void slice_softmax_kernel(const T *__restrict__ x_mid, const float *__restrict__ w_slice,
+                                                            const float *__restrict__ b_slice,
+                                                            const float *__restrict__ temperature, T *__restrict__ w_out,
+                                                            int64_t M, int H, int D, int S, int R) {
+  extern __shared__ float lds[];
+  float *xs = lds;                       // R * H * (D+1)
+  float *wsl = xs + R * H * (D + 1);     // S * D
+  float *bsl = wsl + S * D;              // S
+  float *lg = bsl + S;                   // R * H * (S+1)
+  const int t = threadIdx.x;
+  const int64_t m0 = (int64_t)blockIdx.x * R;
+  const int rows = (int)min((int64_t)R, M - m0);
+  const int HD = H * D;
+  for (int i = t; i < rows * HD; i += 256) {
+    const int r = i / HD, c = i - r * HD;
+    const int h = c / D, d = c - h * D;
+    xs[(r * H + h) * (D + 1) + d] = load_as_f32(x_mid + (m0 + r) * HD + c);
+  }
+  for (int i = t; i < S * D; i += 256) wsl[i] = w_slice[i];
+  for (int i = t; i < S; i += 256) bsl[i] = b_slice[i];
+  __syncthreads();
+  for (int pair = t; pair < rows * H; pair += 256) {
+    const int h = pair % H;
+    const float temp = clamp_temperature(temperature[h]);
+    const float *xr = xs + pair * (D + 1);
+    float *lrow = lg + pair * (S + 1);
+    float mx = -INFINITY;
+    for (int s = 0; s < S; ++s) {
+      float acc = 0.f;
+      const float *wr = wsl + s * D;
+      for (int d = 0; d < D; ++d) acc = fmaf(xr[d], wr[d], acc);
+      // the Linear output is materialised in the storage type before the division (PA.py:537,177)
+      const float z = round_to(w_out, acc + bsl[s]) / temp;
+      lrow[s] = z;
+      mx = fmaxf(mx, z);
+    }
+    float sum = 0.f;
+    for (int s = 0; s < S; ++s) {
+      const float e = expf(lrow[s] - mx);
+      lrow[s] = e;
+      sum += e;
+    }
+    const float inv = 1.f / sum;
+    for (int s = 0; s < S; ++s) lrow[s] *= inv;
+  }
+  __syncthreads();
+  const int HS = H * S;
+  for (int i = t; i < rows * HS; i += 256) {
+    const int pair = i / S, s = i - pair * S;
+    store_from_f32(w_out + m0 * HS + i, lg[pair * (S + 1) + s]);
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// slice_partial_kernel: grid (G chunks, B*H, output slabs).  For its chunk of points of one (b, h):
+//   partial[s, d] = sum_n w[n, s] * fx_mid[n, d]   (d < D),   partial[s, D] = sum_n w[n, s]
+// Each thread owns up to 16 outputs of a 4096-output slab and walks the chunk 32 points at a time
+// through LDS.  Sums run in a fixed order, so the result is bit-reproducible.
+// ------------------------------------------------------------------------------------------------
+constexpr int kSlab = 4096;
+constexpr int kPartialTile = 32;
+
+template <typename T>
+__global__ __launch_bounds__(256) void slice_partial_kernel(const T *__restrict__ w, const T *__restrict__ fx_mid,
+                                                            float *__restrict__ partials, int B, int64_t N, int H, int D,
+                                                            int S, int64_t chunk) {
+  extern __shared__ float lds[];
+  float *wl = lds;                       // 32 * S
+  float *fl = wl + kPartialTile * S;     // 32 * (D+1)
+  const int t = threadIdx.x;
+  const int g = blockIdx.x;
+  const int b = blockIdx.y / H, h = blockIdx.y % H;
+  const int D1 = D + 1;
+  const int n_out = S * D1;
+  const int slab0 = blockIdx.z * kSlab;
+  int os[16], od[16];
+  float acc[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int o = slab0 + t + 256 * i;
+    const bool ok = o < n_out;
+    os[i] = ok ? o / D1 : 0;
+    od[i] = ok ? o % D1 : 0;
+    acc[i] = 0.f;
+  }
+  const int64_t n_begin = (int64_t)g * chunk;
+  const int64_t n_end = min(N, n_begin + chunk);
+  const int HS = H * S, HD = H * D;
+  for (int64_t n0 = n_begin; n0 < n_end; n0 += kPartialTile) {
+    const int pts = (int)min((int64_t)kPartialTile, n_end - n0);
+    for (int i = t; i < kPartialTile * S; i += 256) {
+      const int p = i / S, s = i - p * S;
+      wl[i] = p < pts ? load_as_f32(w + ((int64_t)b * N + n0 + p) * HS + h * S + s) : 0.f;
+    }
+    for (int i = t; i < kPartialTile * D1; i += 256) {
+      const int p = i / D1, d = i - p * D1;
+      float v = 0.f;
+      if (p < pts) v = d < D ? load_as_f32(fx_mid + ((int64_t)b * N + n0 + p) * HD + h * D + d) : 1.f;
+      fl[i] = v;
+    }
+    __syncthreads();
+    for (int p = 0; p < kPartialTile; ++p) {
+      const float *wp = wl + p * S;
+      const float *fp = fl + p * D1;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[i] = fmaf(wp[os[i]], fp[od[i]], acc[i]);
+    }
+    __syncthreads();
+  }
+  float *dst = partials + (((int64_t)g * B + b) * H + h) * n_out;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int o = slab0 + t + 256 * i;
+    if (o < n_out) dst[o] = acc[i];
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// slice_combine_attn_kernel: one workgroup per (b, h), everything after the load stays in LDS.
+//   1. num[s, :], cnt[s] = sum over the G partials in index order
+//   2. tok = num / (cnt + 1e-2)            -> slice_token, slice_norm (optional outputs)
+//   3. q|k|v = tok Wqkv^T                  (rows of Wqkv: [0,D) q, [D,2D) k, [2D,3D) v)
+//   4. out[s, :] = softmax_t(q[s].k[t] / sqrt(D)) v[t, :], one wave per query row
+// `partial_stride` = elements between consecutive partials of the same (b, h).  G == 0: `partials` holds
+// finished tokens (steps 1-2 skipped); out_token == nullptr: stop after step 2.
+// ------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void slice_combine_attn_kernel(const float *__restrict__ partials, int G,
+                                                                 int64_t partial_stride, const float *__restrict__ w_qkv,
+                                                                 float *__restrict__ slice_token,
+                                                                 float *__restrict__ slice_norm,
+                                                                 float *__restrict__ out_token, int D, int S) {
+  extern __shared__ float lds[];
+  const int D1 = D + 1;
+  float *tok = lds;              // S * D1 (column D holds the count, then the norm)
+  float *q = tok + S * D1;       // S * D1
+  float *k = q + S * D1;
+  float *v = k + S * D1;
+  float *prow = v + S * D1;      // 4 waves * S
+  const int t = threadIdx.x;
+  const int bh = blockIdx.x;
+  const int n_out = S * D1;
+  if (G > 0) {
+    const float *src = partials + (int64_t)bh * n_out;
+    for (int o = t; o < n_out; o += 256) {
+      float acc = 0.f;
+      for (int g = 0; g < G; ++g) acc += src[(int64_t)g * partial_stride + o];
+      tok[o] = acc;
+    }
+    __syncthreads();
+    for (int s = t; s < S; s += 256) tok[s * D1 + D] += kSliceNormEps;
+    __syncthreads();
+    for (int i = t; i < S * D; i += 256) {
+      const int s = i / D, d = i - s * D;
+      const float val = tok[s * D1 + d] / tok[s * D1 + D];
+      tok[s * D1 + d] = val;
+      if (slice_token) slice_token[(int64_t)bh * S * D + i] = val;
+    }
+    if (slice_norm)
+      for (int s = t; s < S; s += 256) slice_norm[(int64_t)bh * S + s] = tok[s * D1 + D];
+  } else {
+    // G == 0: `partials` already holds finished slice tokens (B, H, S, D)
+    for (int i = t; i < S * D; i += 256) tok[(i / D) * D1 + (i % D)] = partials[(int64_t)bh * S * D + i];
+  }
+  if (!out_token) return;  // reduction-only call (uniform across the workgroup)
+  __syncthreads();
+  for (int i = t; i < S * 3 * D; i += 256) {
+    const int s = i / (3 * D), e = i - s * 3 * D;
+    const float *wr = w_qkv + (int64_t)e * D;
+    const float *tr = tok + s * D1;
+    float acc = 0.f;
+    for (int d = 0; d < D; ++d) acc = fmaf(tr[d], wr[d], acc);
+    float *dst = e < D ? q : (e < 2 * D ? k : v);
+    dst[s * D1 + (e % D)] = acc;
+  }
+  __syncthreads();
+  const int wave = t >> 6, lane = t & 63;
+  const float scale = rsqrtf((float)D);
+  float *pr = prow + wave * S;
+  for (int s = wave; s < S; s += 4) {
+    const float *qs = q + s * D1;
+    float mx = -INFINITY;
+    for (int u = lane; u < S; u += 64) {
+      const float *ku = k + u * D1;
+      float acc = 0.f;
+      for (int e = 0; e < D; ++e) acc = fmaf(qs[e], ku[e], acc);
+      acc *= scale;
+      pr[u] = acc;
+      mx = fmaxf(mx, acc);
+    }
+    mx = wave_max(mx);
+    float sum = 0.f;
+    for (int u = lane; u < S; u += 64) {
+      const float e = expf(pr[u] - mx);
+      pr[u] = e;
+      sum += e;
+    }
+    sum = wave_sum(sum);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    const float inv = 1.f / sum;
+    for (int e = lane; e < D; e += 64) {
+      float acc = 0.f;
+      for (int u = 0; u < S; ++u) acc = fmaf(pr[u], v[u * D1 + e], acc);
+      out_token[((int64_t)bh * S + s) * D + e] = acc * inv;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// deslice_kernel: grid (row tiles of R, B-independent; H).  out_x[m, h*D + d] = sum_s w[m, h, s] * tok'[b, h, s, d]
+// A row tile never straddles two batches (the host picks tiles per batch).
+// ------------------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void deslice_kernel(const T *__restrict__ w, const float *__restrict__ out_token,
+                                                      T *__restrict__ out_x, int64_t N, int H, int D, int S, int R,
+                                                      int tiles_per_batch) {
+  extern __shared__ float lds[];
+  float *tk = lds;            // S * D
+  float *wl = tk + S * D;     // R * (S+1)
+  const int t = threadIdx.x;
+  const int h = blockIdx.y;
+  const int b = blockIdx.x / tiles_per_batch;
+  const int64_t n0 = (int64_t)(blockIdx.x % tiles_per_batch) * R;
+  const int rows = (int)min((int64_t)R, N - n0);
+  const int64_t m0 = (int64_t)b * N + n0;
+  for (int i = t; i < S * D; i += 256) tk[i] = out_token[((int64_t)b * H + h) * S * D + i];
+  for (int i = t; i < rows * S; i += 256) {
+    const int r = i / S, s = i - r * S;
+    wl[r * (S + 1) + s] = load_as_f32(w + (m0 + r) * H * S + h * S + s);
+  }
+  __syncthreads();
+  for (int i = t; i < rows * D; i += 256) {
+    const int r = i / D, d = i - r * D;
+    const float *wr = wl + r * (S + 1);
+    float acc = 0.f;
+    for (int s = 0; s < S; ++s) acc = fmaf(wr[s], tk[s * D + d], acc);
+    store_from_f32(out_x + (m0 + r) * H * D + h * D + d, acc);
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// residual_ln_kernel: one wave per row.  y <- y + residual (rounded to the storage type);
+// ln_out = (y - mean) / sqrt(var + eps) * gamma + beta with the biased variance, all statistics in fp32.
+// ------------------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void residual_ln_kernel(T *__restrict__ y, const T *__restrict__ residual,
+                                                          const float *__restrict__ gamma, const float *__restrict__ beta,
+                                                          float eps, T *__restrict__ ln_out, int64_t M, int C) {
+  const int lane = threadIdx.x & 63;
+  const int64_t m = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (m >= M) return;
+  T *yr = y + m * C;
+  float sum = 0.f;
+  for (int c = lane; c < C; c += 64) {
+    float v = load_as_f32(yr + c);
+    if (residual) {
+      v = round_to(yr, v + load_as_f32(residual + m * C + c));
+      store_from_f32(yr + c, v);
+    }
+    sum += v;
+  }
+  if (!ln_out) return;
+  const float mean = wave_sum(sum) / (float)C;
+  float sq = 0.f;
+  for (int c = lane; c < C; c += 64) {
+    const float dlt = load_as_f32(yr + c) - mean;
+    sq = fmaf(dlt, dlt, sq);
+  }
+  const float rstd = rsqrtf(wave_sum(sq) / (float)C + eps);
+  for (int c = lane; c < C; c += 64) {
+    const float v = (load_as_f32(yr + c) - mean) * rstd;
+    store_from_f32(ln_out + m * C + c, v * gamma[c] + beta[c]);
+  }
+}
+
+// ================================================================================================
+// host launchers
+// ================================================================================================
+static int launch_status() {
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? PA_OK : (int)e;
+}
+
+template <typename F>
+static int allow_dynamic_lds(F kernel, size_t bytes) {
+  if (bytes > kMaxLdsBytes) return PA_ERR_UNSUPPORTED;
+  if (bytes > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+    if (e != hipSuccess) return (int)e;
+  }
+  return PA_OK;
+}
+
+template <typename TA, typename TW>
+static int launch_gemm(const GemmArgs &a, int nsets, hipStream_t st) {
+  dim3 grid((unsigned)((a.M + 63) / 64), (unsigned)((a.O + 63) / 64), (unsigned)nsets);
+  hipLaunchKernelGGL((rows_gemm_kernel<TA, TW>), grid, dim3(256), 0, st, a);
+  return launch_status();
+}
+
+int project_inputs(int dtype, const pa_shape &s, const pa_params &p, const void *x, void *x_mid, void *fx_mid,
+                   hipStream_t st) {
+  GemmArgs a{};
+  a.in = x;
+  a.w[0] = p.in_project_x_weight;
+  a.w[1] = p.in_project_fx_weight;
+  a.bias[0] = p.in_project_x_bias;
+  a.bias[1] = p.in_project_fx_bias;
+  a.out[0] = x_mid;
+  a.out[1] = fx_mid;
+  a.M = s.B * s.N;
+  a.O = (int)(s.H * s.D);
+  a.C = (int)s.C;
+  a.N = (int)s.N;
+  a.gh = (int)s.grid_h;
+  a.gw = (int)s.grid_w;
+  a.ks = (int)s.conv_k;
+  a.K = s.conv_k > 0 ? (int)(s.conv_k * s.conv_k * s.C) : (int)s.C;
+  return dtype == PA_F32 ? launch_gemm<float, float>(a, 2, st) : launch_gemm<bf16, bf16>(a, 2, st);
+}
+
+int out_linear(int dtype, const pa_shape &s, const pa_params &p, const void *out_x, void *y, hipStream_t st) {
+  GemmArgs a{};
+  a.in = out_x;
+  a.w[0] = p.out_linear_weight;
+  a.bias[0] = p.out_linear_bias;
+  a.out[0] = y;
+  a.M = s.B * s.N;
+  a.K = (int)(s.H * s.D);
+  a.O = (int)s.C;
+  a.ks = 0;
+  return dtype == PA_F32 ? launch_gemm<float, float>(a, 1, st) : launch_gemm<bf16, bf16>(a, 1, st);
+}
+
+template <typename T>
+static int slice_softmax_t(const pa_shape &s, const pa_params &p, const void *x_mid, void *w, hipStream_t st) {
+  const int H = (int)s.H, D = (int)s.D, S = (int)s.S;
+  const size_t fixed = (size_t)(S * D + S) * 4;
+  const size_t per_row = (size_t)(H * (D + 1) + H * (S + 1)) * 4;
+  if (fixed + per_row > 60 * 1024) return PA_ERR_UNSUPPORTED;
+  int R = (int)((60 * 1024 - fixed) / per_row);
+  if (R > 8) R = 8;
+  const size_t lds = fixed + per_row * R;
+  int rc = allow_dynamic_lds(slice_softmax_kernel<T>, lds);
+  if (rc) return rc;
+  const int64_t M = s.B * s.N;
+  hipLaunchKernelGGL((slice_softmax_kernel<T>), dim3((unsigned)((M + R - 1) / R)), dim3(256), lds, st,
+                     static_cast<const T *>(x_mid), p.in_project_slice_weight, p.in_project_slice_bias, p.temperature,
+                     static_cast<T *>(w), M, H, D, S, R);
+  return launch_status();
+}
+
+int slice_softmax(int dtype, const pa_shape &s, const pa_params &p, const void *x_mid, void *w, hipStream_t st) {
+  return dtype == PA_F32 ? slice_softmax_t<float>(s, p, x_mid, w, st) : slice_softmax_t<bf16>(s, p, x_mid, w, st);
+}
+
+// Number of point chunks of the first reduction pass: enough workgroups to fill 256 CUs several times
+// over, at least 256 points per chunk.  Depends on the shape only, so results are reproducible.
+int64_t partial_count(const pa_shape &s) {
+  int64_t by_size = (s.N + 255) / 256;
+  int64_t by_grid = (4096 + s.B * s.H - 1) / (s.B * s.H);
+  int64_t g = by_size < by_grid ? by_size : by_grid;
+  return g < 1 ? 1 : g;
+}
+
+size_t combine_attn_lds_bytes(const pa_shape &s) { return (size_t)(4 * s.S * (s.D + 1) + 4 * s.S) * 4; }
+
+template <typename T>
+static int slice_partial_t(const pa_shape &s, const void *w, const void *fx_mid, float *partials, hipStream_t st) {
+  const int64_t G = partial_count(s);
+  const int64_t chunk = (s.N + G - 1) / G;
+  const int n_out = (int)(s.S * (s.D + 1));
+  const size_t lds = (size_t)(kPartialTile * s.S + kPartialTile * (s.D + 1)) * 4;
+  int rc = allow_dynamic_lds(slice_partial_kernel<T>, lds);
+  if (rc) return rc;
+  dim3 grid((unsigned)G, (unsigned)(s.B * s.H), (unsigned)((n_out + kSlab - 1) / kSlab));
+  hipLaunchKernelGGL((slice_partial_kernel<T>), grid, dim3(256), lds, st, static_cast<const T *>(w),
+                     static_cast<const T *>(fx_mid), partials, (int)s.B, s.N, (int)s.H, (int)s.D, (int)s.S, chunk);
+  return launch_status();
+}
+
+int combine_attention(const pa_shape &s, const pa_params &p, const float *partials, int64_t G, float *slice_token,
+                      float *slice_norm, float *out_token, hipStream_t st) {
+  const size_t lds = combine_attn_lds_bytes(s);
+  int rc = allow_dynamic_lds(slice_combine_attn_kernel, lds);
+  if (rc) return rc;
+  const int64_t stride = s.B * s.H * s.S * (s.D + 1);
+  hipLaunchKernelGGL(slice_combine_attn_kernel, dim3((unsigned)(s.B * s.H)), dim3(256), lds, st, partials, (int)G, stride,
+                     p.qkv_project_weight, slice_token, slice_norm, out_token, (int)s.D, (int)s.S);
+  return launch_status();
+}
+
+int slice_partial(int dtype, const pa_shape &s, const void *w, const void *fx_mid, float *partials, hipStream_t st) {
+  return dtype == PA_F32 ? slice_partial_t<float>(s, w, fx_mid, partials, st)
+                         : slice_partial_t<bf16>(s, w, fx_mid, partials, st);
+}
+
+template <typename T>
+static int deslice_t(const pa_shape &s, const void *w, const float *out_token, void *out_x, hipStream_t st) {
+  int R = 32;
+  size_t lds = (size_t)(s.S * s.D + R * (s.S + 1)) * 4;
+  int rc = allow_dynamic_lds(deslice_kernel<T>, lds);
+  if (rc) return rc;
+  const int tiles = (int)((s.N + R - 1) / R);
+  dim3 grid((unsigned)(tiles * s.B), (unsigned)s.H);
+  hipLaunchKernelGGL((deslice_kernel<T>), grid, dim3(256), lds, st, static_cast<const T *>(w), out_token,
+                     static_cast<T *>(out_x), s.N, (int)s.H, (int)s.D, (int)s.S, R, tiles);
+  return launch_status();
+}
+
+int deslice(int dtype, const pa_shape &s, const void *w, const float *out_token, void *out_x, hipStream_t st) {
+  return dtype == PA_F32 ? deslice_t<float>(s, w, out_token, out_x, st) : deslice_t<bf16>(s, w, out_token, out_x, st);
+}
+
+int residual_ln(int dtype, const pa_shape &s, void *y, const pa_block_tail &tail, hipStream_t st) {
+  const int64_t M = s.B * s.N;
+  dim3 grid((unsigned)((M + 3) / 4));
+  if (dtype == PA_F32)
+    hipLaunchKernelGGL((residual_ln_kernel<float>), grid, dim3(256), 0, st, static_cast<float *>(y),
+                       static_cast<const float *>(tail.residual), tail.ln_gamma, tail.ln_beta, tail.ln_eps,
+                       static_cast<float *>(tail.ln_out), M, (int)s.C);
+  else
+    hipLaunchKernelGGL((residual_ln_kernel<bf16>), grid, dim3(256), 0, st, static_cast<bf16 *>(y),
+                       static_cast<const bf16 *>(tail.residual), tail.ln_gamma, tail.ln_beta, tail.ln_eps,
+                       static_cast<bf16 *>(tail.ln_out), M, (int)s.C);
+  return launch_status();
+}
+
+}  // namespace general
+}  // namespace pa

@@ -1,0 +1,28 @@
+// Host-side declarations shared by the kernel translation units and the C ABI.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include "../../include/physattn.h"
+
+namespace pa {
+
+constexpr size_t kMaxLdsBytes = 160 * 1024;  // LDS per workgroup on gfx950
+
+namespace general {
+int project_inputs(int dtype, const pa_shape &s, const pa_params &p, const void *x, void *x_mid, void *fx_mid,
+                   hipStream_t st);
+int out_linear(int dtype, const pa_shape &s, const pa_params &p, const void *out_x, void *y, hipStream_t st);
+int slice_softmax(int dtype, const pa_shape &s, const pa_params &p, const void *x_mid, void *w, hipStream_t st);
+int64_t partial_count(const pa_shape &s);
+size_t combine_attn_lds_bytes(const pa_shape &s);
+int slice_partial(int dtype, const pa_shape &s, const void *w, const void *fx_mid, float *partials, hipStream_t st);
+int combine_attention(const pa_shape &s, const pa_params &p, const float *partials, int64_t G, float *slice_token,
+                      float *slice_norm, float *out_token, hipStream_t st);
+int deslice(int dtype, const pa_shape &s, const void *w, const float *out_token, void *out_x, hipStream_t st);
+int residual_ln(int dtype, const pa_shape &s, void *y, const pa_block_tail &tail, hipStream_t st);
+}  // namespace general
+
+}  // namespace pa

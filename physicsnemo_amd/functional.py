@@ -1,0 +1,139 @@
+"""Tensor-level wrappers over the C ABI: one function per entry point of include/physattn.h.
+
+Every function takes CUDA (ROCm) tensors, allocates outputs/workspace with torch and enqueues the HIP
+kernels on torch's current stream.  `params` is the dict produced by
+`physicsnemo_amd.physics_attention.PhysicsAttentionBase.kernel_params`.
+"""
+from __future__ import annotations
+
+from ctypes import byref
+from typing import NamedTuple
+
+import torch
+
+from . import _lib
+
+
+class LayerDims(NamedTuple):
+    B: int
+    N: int
+    C: int
+    H: int
+    D: int
+    S: int
+    grid_h: int = 0
+    grid_w: int = 0
+    conv_k: int = 0
+
+    def c(self) -> _lib.PaShape:
+        return _lib.PaShape(*self)
+
+
+_PARAM_FIELDS = [f for f, _ in _lib.PaParams._fields_]
+
+
+def _c_params(params: dict) -> _lib.PaParams:
+    return _lib.PaParams(*[_lib.ptr(params.get(k)) for k in _PARAM_FIELDS])
+
+
+def _need_cuda(*tensors):
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError("physicsnemo_amd runs on GPU tensors only (there is no CPU path)")
+        if t is not None and not t.is_contiguous():
+            raise RuntimeError("physicsnemo_amd kernels need contiguous tensors")
+
+
+def query_path(dtype: torch.dtype, dims: LayerDims) -> int:
+    """0 = general kernels, 1 = bf16 MFMA kernels."""
+    rc = _lib.load().pa_query_path(_lib.dtype_code(dtype), byref(dims.c()))
+    if rc < 0:
+        _lib.check(rc, "pa_query_path")
+    return rc
+
+
+def project_inputs(x, params, dims: LayerDims):
+    _need_cuda(x)
+    lib = _lib.load()
+    x_mid = torch.empty(dims.B, dims.N, dims.H * dims.D, dtype=x.dtype, device=x.device)
+    fx_mid = torch.empty_like(x_mid)
+    _lib.check(lib.pa_project_inputs(_lib.dtype_code(x.dtype), byref(dims.c()), byref(_c_params(params)),
+                                     x.data_ptr(), x_mid.data_ptr(), fx_mid.data_ptr(),
+                                     _lib.current_stream_ptr(x.device)), "pa_project_inputs")
+    return x_mid, fx_mid
+
+
+def slice_softmax(x_mid, params, dims: LayerDims):
+    _need_cuda(x_mid)
+    lib = _lib.load()
+    w = torch.empty(dims.B, dims.N, dims.H, dims.S, dtype=x_mid.dtype, device=x_mid.device)
+    _lib.check(lib.pa_slice_softmax(_lib.dtype_code(x_mid.dtype), byref(dims.c()), byref(_c_params(params)),
+                                    x_mid.data_ptr(), w.data_ptr(), _lib.current_stream_ptr(x_mid.device)),
+               "pa_slice_softmax")
+    return w
+
+
+def slice_reduce(w, fx_mid, dims: LayerDims):
+    _need_cuda(w, fx_mid)
+    lib = _lib.load()
+    shape = dims.c()
+    g = lib.pa_reduce_partial_count(byref(shape))
+    if g < 0:
+        _lib.check(int(g), "pa_reduce_partial_count")
+    partials = torch.empty(g * dims.B * dims.H * dims.S * (dims.D + 1), dtype=torch.float32, device=w.device)
+    tok = torch.empty(dims.B, dims.H, dims.S, dims.D, dtype=torch.float32, device=w.device)
+    norm = torch.empty(dims.B, dims.H, dims.S, dtype=torch.float32, device=w.device)
+    _lib.check(lib.pa_slice_reduce(_lib.dtype_code(w.dtype), byref(shape), w.data_ptr(), fx_mid.data_ptr(),
+                                   partials.data_ptr(), tok.data_ptr(), norm.data_ptr(),
+                                   _lib.current_stream_ptr(w.device)), "pa_slice_reduce")
+    return tok, norm
+
+
+def slice_attention(tok, params, dims: LayerDims):
+    _need_cuda(tok)
+    lib = _lib.load()
+    out = torch.empty_like(tok)
+    _lib.check(lib.pa_slice_attention(byref(dims.c()), byref(_c_params(params)), tok.data_ptr(), out.data_ptr(),
+                                      _lib.current_stream_ptr(tok.device)), "pa_slice_attention")
+    return out
+
+
+def _c_tail(residual, ln_weight, ln_bias, ln_eps, ln_out):
+    return _lib.PaBlockTail(_lib.ptr(residual), _lib.ptr(ln_weight), _lib.ptr(ln_bias), float(ln_eps), _lib.ptr(ln_out))
+
+
+def deslice_project(w, tok_out, params, dims: LayerDims, residual=None, ln_weight=None, ln_bias=None, ln_eps=1e-5):
+    """Returns y, or (fx_new, ln_out) when a residual / LayerNorm tail is requested."""
+    _need_cuda(w, tok_out, residual)
+    lib = _lib.load()
+    y = torch.empty(dims.B, dims.N, dims.C, dtype=w.dtype, device=w.device)
+    scratch = torch.empty(dims.B, dims.N, dims.H * dims.D, dtype=w.dtype, device=w.device)
+    ln_out = torch.empty_like(y) if ln_weight is not None else None
+    tail = _c_tail(residual, ln_weight, ln_bias, ln_eps, ln_out)
+    _lib.check(lib.pa_deslice_project(_lib.dtype_code(w.dtype), byref(dims.c()), byref(_c_params(params)),
+                                      w.data_ptr(), tok_out.data_ptr(), scratch.data_ptr(), y.data_ptr(),
+                                      byref(tail), _lib.current_stream_ptr(w.device)), "pa_deslice_project")
+    return y if (residual is None and ln_out is None) else (y, ln_out)
+
+
+def layer_forward(x, params, dims: LayerDims, residual=None, ln_weight=None, ln_bias=None, ln_eps=1e-5,
+                  return_slice_tokens=False):
+    """Whole PhysicsAttention layer.  Returns y, or (fx_new, ln_out) with a tail; slice tokens appended on request."""
+    _need_cuda(x, residual)
+    lib = _lib.load()
+    code = _lib.dtype_code(x.dtype)
+    shape = dims.c()
+    nbytes = lib.pa_workspace_bytes(code, byref(shape))
+    if nbytes < 0:
+        _lib.check(int(nbytes), "pa_workspace_bytes")
+    workspace = torch.empty(int(nbytes), dtype=torch.uint8, device=x.device)
+    y = torch.empty(dims.B, dims.N, dims.C, dtype=x.dtype, device=x.device)
+    ln_out = torch.empty_like(y) if ln_weight is not None else None
+    tok = (torch.empty(dims.B, dims.H, dims.S, dims.D, dtype=torch.float32, device=x.device)
+           if return_slice_tokens else None)
+    tail = _c_tail(residual, ln_weight, ln_bias, ln_eps, ln_out)
+    _lib.check(lib.pa_layer_forward(code, byref(shape), byref(_c_params(params)), x.data_ptr(), y.data_ptr(),
+                                    byref(tail), _lib.ptr(tok), workspace.data_ptr(), int(nbytes),
+                                    _lib.current_stream_ptr(x.device)), "pa_layer_forward")
+    out = y if (residual is None and ln_out is None) else (y, ln_out)
+    return (out, tok) if return_slice_tokens else out

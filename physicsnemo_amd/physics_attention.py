@@ -1,0 +1,181 @@
+"""Drop-in PhysicsAttention modules whose forward runs hand-written HIP kernels (libphysattn.so).
+
+Mirrors the constructor signatures, parameter names / registration order and input validation of the
+reference classes in physicsnemo/nn/module/physics_attention.py:
+  PhysicsAttentionBase            :209-558
+  PhysicsAttentionIrregularMesh   :561-660
+  PhysicsAttentionStructuredMesh2D:663-783
+so that a reference ``state_dict`` loads unchanged and seeded construction consumes the RNG identically.
+
+Scope: forward only, ``plus=False``.  ``use_te`` is accepted for signature compatibility and ignored: the
+HIP kernels are the only backend.  There is no CPU path and no autograd: calling with gradients enabled on
+tensors that require grad raises.
+"""
+from __future__ import annotations
+
+import torch
+import torch.nn as nn
+
+from . import functional as PF
+
+__all__ = ["PhysicsAttentionBase", "PhysicsAttentionIrregularMesh", "PhysicsAttentionStructuredMesh2D"]
+
+
+class PhysicsAttentionBase(nn.Module):
+    """Parameters shared by the variants plus the HIP forward (reference base class: :262-327, :501-558)."""
+
+    def __init__(self, dim: int, heads: int, dim_head: int, dropout: float, slice_num: int, use_te: bool, plus: bool):
+        super().__init__()
+        if plus:
+            raise NotImplementedError("Transolver++ (plus=True) is not served by the HIP kernels")
+        self.dim = dim
+        self.dim_head = dim_head
+        self.heads = heads
+        self.slice_num = slice_num
+        self.plus = plus
+        self.scale = dim_head ** -0.5
+        self.use_te = use_te
+
+        # registration order follows the reference so state_dict order and RNG draws agree
+        self.softmax = nn.Softmax(dim=-1)
+        self.dropout = nn.Dropout(dropout)
+        self.temperature = nn.Parameter(torch.ones([1, 1, heads, 1]) * 0.5)
+        self.in_project_slice = nn.Linear(dim_head, slice_num)
+        torch.nn.init.orthogonal_(self.in_project_slice.weight)
+        self.qkv_project = nn.Linear(dim_head, 3 * dim_head, bias=False)
+        self.out_linear = nn.Linear(dim_head * heads, dim)
+        self.out_dropout = nn.Dropout(dropout)
+        self._kernel_param_cache: dict = {}
+
+    # ---------------------------------------------------------------- parameters in kernel form
+    def _conv_geometry(self):
+        return 0, 0, 0
+
+    def layer_dims(self, x: torch.Tensor) -> PF.LayerDims:
+        gh, gw, k = self._conv_geometry()
+        return PF.LayerDims(x.shape[0], x.shape[1], self.dim, self.heads, self.dim_head, self.slice_num, gh, gw, k)
+
+    def kernel_params(self, dtype: torch.dtype, device: torch.device) -> dict:
+        """Parameters as the C ABI wants them: the three large weights in ``dtype``, everything else float32,
+        contiguous.  Cached until a parameter is modified in place, replaced or moved."""
+        named = [
+            ("in_project_x_weight", self.in_project_x.weight, True),
+            ("in_project_x_bias", self.in_project_x.bias, False),
+            ("in_project_fx_weight", self.in_project_fx.weight, True),
+            ("in_project_fx_bias", self.in_project_fx.bias, False),
+            ("in_project_slice_weight", self.in_project_slice.weight, False),
+            ("in_project_slice_bias", self.in_project_slice.bias, False),
+            ("temperature", self.temperature, False),
+            ("qkv_project_weight", self.qkv_project.weight, False),
+            ("out_linear_weight", self.out_linear.weight, True),
+            ("out_linear_bias", self.out_linear.bias, False),
+        ]
+        stamp = (dtype, device) + tuple((p.data_ptr(), p._version, p.dtype) for _, p, _ in named)
+        hit = self._kernel_param_cache.get("stamp")
+        if hit == stamp:
+            return self._kernel_param_cache["params"]
+        with torch.no_grad():
+            params = {
+                name: p.detach().to(device=device, dtype=dtype if big else torch.float32).contiguous().reshape(-1).clone()
+                for name, p, big in named
+            }
+        self._kernel_param_cache = {"stamp": stamp, "params": params}
+        return params
+
+    # ---------------------------------------------------------------- forward
+    def _validate(self, x: torch.Tensor) -> None:
+        # same checks and messages as the reference forward (:516-526)
+        if x.ndim != 3:
+            raise ValueError(
+                f"Expected 3D input tensor (B, N, C), got {x.ndim}D tensor with shape {tuple(x.shape)}")
+        if x.shape[-1] != self.dim:
+            raise ValueError(f"Expected input feature dimension {self.dim}, got {x.shape[-1]}")
+
+    def _check_spatial(self, x: torch.Tensor) -> None:
+        pass
+
+    def _prepare_input(self, x: torch.Tensor) -> torch.Tensor:
+        if not x.is_cuda:
+            raise RuntimeError("physicsnemo_amd PhysicsAttention runs on GPU tensors only (no CPU fallback)")
+        if torch.is_grad_enabled() and (x.requires_grad or any(p.requires_grad for p in self.parameters())):
+            raise RuntimeError(
+                "physicsnemo_amd PhysicsAttention implements the forward pass only; call it under "
+                "torch.no_grad() / torch.inference_mode()")
+        if self.training and self.out_dropout.p > 0:
+            raise RuntimeError("dropout > 0 in training mode is not served by the HIP kernels")
+        if torch.is_autocast_enabled("cuda"):
+            ac = torch.get_autocast_dtype("cuda")
+            if ac != torch.bfloat16:
+                raise TypeError(f"autocast dtype {ac} is not supported (bfloat16 only)")
+            x = x.to(torch.bfloat16)
+        if x.dtype not in (torch.float32, torch.bfloat16):
+            raise TypeError(f"expected float32 or bfloat16 input, got {x.dtype}")
+        self._check_spatial(x)
+        return x.contiguous()
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        """(B, N, C) -> (B, N, C); replaces reference forward :501-558."""
+        self._validate(x)
+        x = self._prepare_input(x)
+        return PF.layer_forward(x, self.kernel_params(x.dtype, x.device), self.layer_dims(x))
+
+    def forward_block(self, x: torch.Tensor, residual: torch.Tensor, ln: nn.LayerNorm):
+        """Layer + the caller block's ``+ residual`` and following LayerNorm in one pass
+        (physicsnemo/models/transolver/transolver.py:300-303).  Returns (fx_new, LayerNorm(fx_new))."""
+        self._validate(x)
+        x = self._prepare_input(x)
+        residual = residual.to(x.dtype).contiguous()
+        return PF.layer_forward(
+            x, self.kernel_params(x.dtype, x.device), self.layer_dims(x), residual=residual,
+            ln_weight=ln.weight.detach().float().contiguous(), ln_bias=ln.bias.detach().float().contiguous(),
+            ln_eps=ln.eps)
+
+    def forward_stages(self, x: torch.Tensor) -> dict:
+        """Stage-by-stage forward through the natural-layout entry points; returns every intermediate."""
+        self._validate(x)
+        x = self._prepare_input(x)
+        dims = self.layer_dims(x)
+        p = self.kernel_params(x.dtype, x.device)
+        x_mid, fx_mid = PF.project_inputs(x, p, dims)
+        w = PF.slice_softmax(x_mid, p, dims)
+        tok, norm = PF.slice_reduce(w, fx_mid, dims)
+        tok_out = PF.slice_attention(tok, p, dims)
+        y = PF.deslice_project(w, tok_out, p, dims)
+        H, D = self.heads, self.dim_head
+        return dict(x_mid=x_mid.view(dims.B, dims.N, H, D), fx_mid=fx_mid.view(dims.B, dims.N, H, D), w=w, tok=tok,
+                    norm=norm, tok_out=tok_out, y=y)
+
+
+class PhysicsAttentionIrregularMesh(PhysicsAttentionBase):
+    """Unstructured point clouds: nn.Linear projections (reference :606-627)."""
+
+    def __init__(self, dim: int, heads: int = 8, dim_head: int = 64, dropout: float = 0.0, slice_num: int = 64,
+                 use_te: bool = True, plus: bool = False):
+        super().__init__(dim, heads, dim_head, dropout, slice_num, use_te, plus)
+        inner_dim = dim_head * heads
+        self.in_project_x = nn.Linear(dim, inner_dim)
+        self.in_project_fx = nn.Linear(dim, inner_dim)
+
+
+class PhysicsAttentionStructuredMesh2D(PhysicsAttentionBase):
+    """Row-major 2D grids: k x k Conv2d projections, stride 1, zero padding k//2 (reference :721-742).
+
+    ``forward`` takes the flattened ``(B, H_s*W_s, C)`` tensor with token n = i*W_s + j (:768-783).
+    """
+
+    def __init__(self, dim: int, spatial_shape: tuple[int, int], heads: int = 8, dim_head: int = 64,
+                 dropout: float = 0.0, slice_num: int = 64, kernel: int = 3, use_te: bool = True, plus: bool = False):
+        super().__init__(dim, heads, dim_head, dropout, slice_num, use_te, plus)
+        inner_dim = dim_head * heads
+        self.H = spatial_shape[0]
+        self.W = spatial_shape[1]
+        self.kernel = kernel
+        self.in_project_x = nn.Conv2d(dim, inner_dim, kernel, 1, kernel // 2)
+        self.in_project_fx = nn.Conv2d(dim, inner_dim, kernel, 1, kernel // 2)
+
+    def _conv_geometry(self):
+        return self.H, self.W, self.kernel
+
+    def _check_spatial(self, x: torch.Tensor) -> None:
+        # the reference reshapes with x.view(B, H, W, C) (:772): same failure for a wrong token count
+        x.view(x.shape[0], self.H, self.W, x.shape[-1])

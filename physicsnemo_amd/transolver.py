@@ -1,0 +1,175 @@
+"""Host-side mirror of the caller of the hot path: TransolverBlock and Transolver
+(physicsnemo/models/transolver/transolver.py:137-309 and :447-736, use_te=False, time_input=False, plus=False).
+
+The PhysicsAttention layer, its residual add and the LayerNorm that follows it run in the HIP library; the
+remaining glue (LayerNorm before the layer, the two MLPs, the output head) uses PyTorch-ROCm tensor ops.
+Module names, registration order and state_dict keys match the reference so its checkpoints load unchanged,
+including the legacy ``linear_pre`` / ``linear_post`` MLP keys (:92-97).
+"""
+from __future__ import annotations
+
+import numpy as np
+import torch
+import torch.nn as nn
+
+from .physics_attention import PhysicsAttentionIrregularMesh, PhysicsAttentionStructuredMesh2D
+
+__all__ = ["Mlp", "TransolverBlock", "Transolver"]
+
+_LEGACY_MLP_KEYS = {
+    "linear_pre.weight": "layers.0.weight",
+    "linear_pre.bias": "layers.0.bias",
+    "linear_post.weight": "layers.2.weight",
+    "linear_post.bias": "layers.2.bias",
+}
+
+_ACTIVATIONS = {"gelu": nn.GELU, "relu": nn.ReLU, "silu": nn.SiLU, "tanh": nn.Tanh, "sigmoid": nn.Sigmoid}
+
+
+class Mlp(nn.Module):
+    """Linear -> activation -> Linear under ``layers.{0,2}`` (physicsnemo/nn/module/mlp_layers.py:139-173)."""
+
+    def __init__(self, in_features: int, hidden_features: int, out_features: int, act_layer: str = "gelu"):
+        super().__init__()
+        try:
+            act = _ACTIVATIONS[act_layer.lower()]()
+        except KeyError:
+            raise KeyError(f"Activation function {act_layer} not found. Available options are: {list(_ACTIVATIONS)}")
+        self.layers = nn.Sequential(nn.Linear(in_features, hidden_features), act, nn.Linear(hidden_features, out_features))
+
+    def _load_from_state_dict(self, state_dict, prefix, *args, **kwargs):
+        for old, new in _LEGACY_MLP_KEYS.items():
+            if prefix + old in state_dict and prefix + new not in state_dict:
+                state_dict[prefix + new] = state_dict.pop(prefix + old)
+        return super()._load_from_state_dict(state_dict, prefix, *args, **kwargs)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return self.layers(x)
+
+
+class TransolverBlock(nn.Module):
+    """LayerNorm -> PhysicsAttention -> +residual -> LayerNorm -> MLP -> +residual [-> LayerNorm -> Linear]."""
+
+    def __init__(self, num_heads: int, hidden_dim: int, dropout: float, act: str = "gelu", mlp_ratio: int = 4,
+                 last_layer: bool = False, out_dim: int = 1, slice_num: int = 32,
+                 spatial_shape: tuple[int, ...] | None = None, use_te: bool = True, plus: bool = False):
+        super().__init__()
+        self.last_layer = last_layer
+        self.ln_1 = nn.LayerNorm(hidden_dim)
+        common = dict(heads=num_heads, dim_head=hidden_dim // num_heads, dropout=dropout, slice_num=slice_num,
+                      use_te=use_te, plus=plus)
+        if spatial_shape is None:
+            self.Attn = PhysicsAttentionIrregularMesh(hidden_dim, **common)
+        elif len(spatial_shape) == 2:
+            self.Attn = PhysicsAttentionStructuredMesh2D(hidden_dim, spatial_shape=spatial_shape, **common)
+        elif len(spatial_shape) == 3:
+            raise NotImplementedError("the structured-3D (Conv3d) variant is not built")
+        else:
+            raise ValueError(
+                f"Unexpected length of spatial shape encountered in Transolver_block: {len(spatial_shape)}. Expected 2 or 3.")
+        self.ln_mlp1 = nn.Sequential(nn.LayerNorm(hidden_dim), Mlp(hidden_dim, hidden_dim * mlp_ratio, hidden_dim, act))
+        if last_layer:
+            self.ln_mlp2 = nn.Sequential(nn.LayerNorm(hidden_dim), nn.Linear(hidden_dim, out_dim))
+
+    def forward(self, fx: torch.Tensor) -> torch.Tensor:
+        # fx1 = Attn(ln_1(fx)) + fx and LayerNorm(fx1) come out of one fused library call (reference :300, :303)
+        fx1, normed = self.Attn.forward_block(self.ln_1(fx), fx, self.ln_mlp1[0])
+        fx2 = self.ln_mlp1[1](normed) + fx1
+        return self.ln_mlp2(fx2) if self.last_layer else fx2
+
+
+class Transolver(nn.Module):
+    """Transolver model (reference :447-736) built on the HIP PhysicsAttention layer; forward only."""
+
+    def __init__(self, functional_dim: int, out_dim: int, embedding_dim: int | None = None, n_layers: int = 4,
+                 n_hidden: int = 256, dropout: float = 0.0, n_head: int = 8, act: str = "gelu", mlp_ratio: int = 4,
+                 slice_num: int = 32, unified_pos: bool = False, ref: int = 8,
+                 structured_shape: None | tuple[int, ...] = None, use_te: bool = True, time_input: bool = False,
+                 plus: bool = False) -> None:
+        super().__init__()
+        if time_input:
+            raise NotImplementedError("time_input=True is not built")
+        self.use_te = use_te
+        if not n_hidden % n_head == 0:
+            raise ValueError(
+                f"Transolver requires n_hidden % n_head == 0, but got n_hidden={n_hidden}, n_head={n_head} "
+                f"(remainder={n_hidden % n_head})")
+        if structured_shape is not None:
+            if len(structured_shape) not in [2, 3]:
+                raise ValueError(
+                    f"Transolver only supports 2D or 3D structured data, got shape with {len(structured_shape)} dimensions")
+            if not all([s > 0 and s == int(s) for s in structured_shape]):
+                raise ValueError(f"Transolver requires positive integer shapes, got {structured_shape}")
+        elif unified_pos:
+            raise ValueError("Transolver requires structured_shape when using unified_pos=True")
+        self.structured_shape = structured_shape
+        self.unified_pos = unified_pos
+        if unified_pos:
+            self.register_buffer("embedding", self.get_grid(ref))
+            self.embedding_dim = ref * ref
+        else:
+            if embedding_dim is None:
+                raise ValueError("Transolver requires embedding_dim when unified_pos=False")
+            self.embedding_dim = embedding_dim
+        self.preprocess = Mlp(functional_dim + self.embedding_dim, n_hidden * 2, n_hidden, act)
+        self.time_input = time_input
+        self.n_hidden = n_hidden
+        self.blocks = nn.ModuleList([
+            TransolverBlock(num_heads=n_head, hidden_dim=n_hidden, dropout=dropout, act=act, mlp_ratio=mlp_ratio,
+                            out_dim=out_dim, slice_num=slice_num, spatial_shape=structured_shape,
+                            last_layer=(i == n_layers - 1), use_te=use_te, plus=plus)
+            for i in range(n_layers)
+        ])
+        self.initialize_weights()
+
+    def initialize_weights(self) -> None:
+        self.apply(self._init_weights)
+
+    def _init_weights(self, m: nn.Module) -> None:
+        # every nn.Linear (the slice projection included) is redrawn; Conv2d keeps its default init (:579-593)
+        if isinstance(m, nn.Linear):
+            nn.init.trunc_normal_(m.weight, std=0.02)
+            if m.bias is not None:
+                nn.init.constant_(m.bias, 0)
+        if isinstance(m, (nn.LayerNorm, nn.BatchNorm1d)):
+            nn.init.constant_(m.bias, 0)
+            nn.init.constant_(m.weight, 1.0)
+
+    def get_grid(self, ref: int, batchsize: int = 1) -> torch.Tensor:
+        """Distances from every grid point to a ref x ref lattice on the unit square, (B, H*W, ref*ref) (:595-645)."""
+        if self.structured_shape is None:
+            raise ValueError("Cannot generate positional encoding grid: structured_shape is None. "
+                             "This method requires structured_shape to be set.")
+        size_x, size_y = self.structured_shape
+        px = torch.tensor(np.linspace(0, 1, size_x), dtype=torch.float)
+        py = torch.tensor(np.linspace(0, 1, size_y), dtype=torch.float)
+        pts = torch.stack(torch.meshgrid(px, py, indexing="ij"), dim=-1).reshape(-1, 1, 2)
+        lr = torch.tensor(np.linspace(0, 1, ref), dtype=torch.float)
+        lattice = torch.stack(torch.meshgrid(lr, lr, indexing="ij"), dim=-1).reshape(1, -1, 2)
+        pos = torch.sqrt(((pts - lattice) ** 2).sum(-1))
+        return pos.unsqueeze(0).repeat(batchsize, 1, 1).contiguous()
+
+    def forward(self, fx: torch.Tensor, embedding: torch.Tensor | None = None, time: torch.Tensor | None = None):
+        if fx.ndim < 2:
+            raise ValueError(
+                f"Expected input tensor with at least 2 dimensions, got {fx.ndim}D tensor with shape {tuple(fx.shape)}")
+        if not self.unified_pos and embedding is None:
+            raise ValueError("Embedding is required when unified_pos=False")
+        if time is not None:
+            raise NotImplementedError("time input is not built")
+        unflatten_output = False
+        if self.unified_pos:
+            embedding = self.embedding.repeat(fx.shape[0], 1, 1)
+        if self.structured_shape is not None:
+            if fx.ndim != 3:
+                unflatten_output = True
+                fx = fx.reshape(fx.shape[0], -1, fx.shape[-1])
+            if embedding is not None and embedding.ndim != 3:
+                embedding = embedding.reshape(embedding.shape[0], -1, embedding.shape[-1])
+        fx = torch.cat((embedding.to(fx.dtype), fx), -1)  # embedding first, then the functional input (:716)
+        fx = self.preprocess(fx)
+        for block in self.blocks:
+            fx = block(fx)
+        if unflatten_output:
+            fx = fx.reshape(fx.shape[0], *self.structured_shape, -1)
+        return fx

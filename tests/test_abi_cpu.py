@@ -1,0 +1,128 @@
+"""CPU-side checks of the C-ABI library and the host modules (no kernel is launched)."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+import physicsnemo_amd as pn
+from physicsnemo_amd import _lib
+from physicsnemo_amd import functional as PF
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_loads_and_exports_every_declared_symbol():
+    lib = _lib.load()
+    header = open(os.path.join(ROOT, "include", "physattn.h")).read()
+    declared = set(re.findall(r"\b(pa_[a-z_0-9]+)\s*\(", header))
+    assert declared, "no declarations parsed"
+    assert declared == set(_lib.EXPORTED)
+    for name in declared:
+        assert hasattr(lib, name), name
+    assert lib.pa_version() >= 100
+    assert lib.pa_status_string(0) == b"ok"
+
+
+def _shape(**kw):
+    base = dict(B=1, N=64, C=64, H=2, D=32, S=16, grid_h=0, grid_w=0, conv_k=0)
+    base.update(kw)
+    return _lib.PaShape(**base)
+
+
+def test_argument_errors_are_codes_not_crashes():
+    lib = _lib.load()
+    assert lib.pa_workspace_bytes(0, None) == -1
+    assert lib.pa_workspace_bytes(0, ctypes.byref(_shape(N=0))) == -2
+    assert lib.pa_workspace_bytes(7, ctypes.byref(_shape())) == -3
+    assert lib.pa_workspace_bytes(0, ctypes.byref(_shape(D=4096))) == -3
+    assert lib.pa_workspace_bytes(0, ctypes.byref(_shape(conv_k=3, grid_h=8, grid_w=9))) == -2  # 72 != 64
+    assert lib.pa_workspace_bytes(0, ctypes.byref(_shape(conv_k=2, grid_h=8, grid_w=8))) == -3
+    assert lib.pa_workspace_bytes(0, ctypes.byref(_shape())) > 0
+    # null tensors / params are rejected before anything touches a device
+    s = _shape()
+    assert lib.pa_layer_forward(0, ctypes.byref(s), None, None, None, None, None, None, 0, None) == -1
+    p = _lib.PaParams(*([256] * 10))
+    assert lib.pa_layer_forward(0, ctypes.byref(s), ctypes.byref(p), None, None, None, None, None, 0, None) == -1
+    assert lib.pa_layer_forward(0, ctypes.byref(s), ctypes.byref(p), 256, 256, None, None, 256, 1, None) == -5
+    assert lib.pa_layer_forward(0, ctypes.byref(s), ctypes.byref(p), 260, 256, None, None, 256, 1 << 40, None) == -4
+    assert lib.pa_status_string(-5) == b"workspace too small"
+
+
+def test_module_signatures_state_dict_and_seeded_init_match_oracle():
+    from oracle import torch_oracle as to
+    torch.manual_seed(7)
+    a = pn.PhysicsAttentionIrregularMesh(64, heads=4, dim_head=16, slice_num=8, use_te=False)
+    torch.manual_seed(7)
+    b = to.OraclePhysicsAttentionIrregularMesh(64, heads=4, dim_head=16, slice_num=8)
+    sa, sb = a.state_dict(), b.state_dict()
+    assert list(sa) == list(sb)
+    for k in sa:
+        assert torch.equal(sa[k], sb[k]), k
+    torch.manual_seed(7)
+    a2 = pn.PhysicsAttentionStructuredMesh2D(32, (5, 6), heads=2, dim_head=16, slice_num=8, kernel=3, use_te=False)
+    torch.manual_seed(7)
+    b2 = to.OraclePhysicsAttentionStructuredMesh2D(32, (5, 6), heads=2, dim_head=16, slice_num=8, kernel=3)
+    assert list(a2.state_dict()) == list(b2.state_dict())
+    assert all(torch.equal(a2.state_dict()[k], b2.state_dict()[k]) for k in a2.state_dict())
+    assert (a2.H, a2.W) == (5, 6)
+    # reference defaults: heads=8, dim_head=64, slice_num=64, use_te=True accepted
+    d = pn.PhysicsAttentionIrregularMesh(128)
+    assert (d.heads, d.dim_head, d.in_project_slice.out_features) == (8, 64, 64)
+    assert isinstance(d.temperature, torch.nn.Parameter) and tuple(d.temperature.shape) == (1, 1, 8, 1)
+    assert torch.all(d.temperature == 0.5)
+    # orthogonal slice projection: rows of a (16, 32) weight are orthonormal (reference test_physics_attention.py:667-685)
+    o = pn.PhysicsAttentionIrregularMesh(64, heads=2, dim_head=32, slice_num=16)
+    wwt = o.in_project_slice.weight @ o.in_project_slice.weight.T
+    assert torch.allclose(wwt, torch.eye(16), atol=1e-5)
+
+
+def test_model_state_dict_matches_oracle_and_loads_legacy_keys():
+    from oracle import torch_oracle as to
+    kw = dict(functional_dim=2, out_dim=3, embedding_dim=3, n_layers=2, n_hidden=32, n_head=4, slice_num=8, mlp_ratio=2)
+    torch.manual_seed(1)
+    m = pn.Transolver(use_te=False, **kw)
+    torch.manual_seed(1)
+    o = to.OracleTransolver(**kw)
+    assert list(m.state_dict()) == list(o.state_dict())
+    assert all(torch.equal(m.state_dict()[k], o.state_dict()[k]) for k in m.state_dict())
+    sd = {k.replace("layers.0", "linear_pre").replace("layers.2", "linear_post"): v for k, v in o.state_dict().items()}
+    assert any("linear_pre" in k for k in sd)
+    m.load_state_dict(sd)  # legacy MLP key names (reference transolver.py:92-97)
+    s2 = pn.Transolver(functional_dim=1, out_dim=1, n_layers=1, n_hidden=16, n_head=2, structured_shape=(4, 5),
+                       unified_pos=True, ref=2, use_te=False)
+    assert tuple(s2.embedding.shape) == (1, 20, 4)
+    assert torch.equal(s2.embedding, to.unified_pos_grid((4, 5), 2))
+
+
+def test_validation_messages_and_no_cpu_fallback():
+    m = pn.PhysicsAttentionIrregularMesh(8, heads=2, dim_head=4, slice_num=3, use_te=False)
+    with pytest.raises(ValueError, match="Expected 3D input"):
+        m(torch.randn(4, 8))
+    with pytest.raises(ValueError, match="Expected input feature dimension 8, got 6"):
+        m(torch.randn(1, 4, 6))
+    with torch.no_grad(), pytest.raises(RuntimeError, match="GPU tensors only"):
+        m(torch.randn(1, 4, 8))
+    with pytest.raises(NotImplementedError):
+        pn.PhysicsAttentionIrregularMesh(8, heads=2, dim_head=4, plus=True)
+    with pytest.raises(ValueError, match="n_hidden % n_head"):
+        pn.Transolver(functional_dim=1, out_dim=1, embedding_dim=1, n_hidden=30, n_head=4)
+    with pytest.raises(ValueError, match="structured_shape when using unified_pos"):
+        pn.Transolver(functional_dim=1, out_dim=1, unified_pos=True)
+
+
+def test_missing_library_fails_loudly(monkeypatch):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/libphysattn.so")
+    with pytest.raises(RuntimeError, match="no fallback"):
+        _lib.load()
+
+
+def test_product_package_never_imports_the_oracle():
+    pkg = os.path.join(ROOT, "physicsnemo_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h", ".cpp")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert "oracle" not in text.lower(), f

@@ -1,0 +1,172 @@
+"""GPU parity: the HIP path (through the C ABI) against the CPU oracle on the same seeded inputs and weights.
+
+Bars: fp32 within rtol 1e-4 (atol = 1e-4 * max|ref|); bf16 within relative L2 error 1e-2 of the fp32 oracle.
+"""
+import os
+
+import pytest
+import torch
+
+from oracle import torch_oracle as to
+import physicsnemo_amd as pn
+from gpu_util import announce, assert_fp32_close, assert_rel_l2, make_pair
+
+pytestmark = pytest.mark.gpu
+GOLD = os.path.join(os.path.dirname(__file__), "golden")
+STAGES = ("x_mid", "fx_mid", "w", "tok", "norm", "tok_out", "y")
+
+
+@pytest.mark.parametrize("B,N,dim,heads,dim_head,S", [
+    (1, 100, 64, 4, 16, 4), (2, 500, 128, 8, 16, 16), (4, 1000, 256, 8, 32, 64), (2, 333, 96, 3, 32, 32),
+    (1, 257, 64, 2, 64, 16), (2, 129, 128, 4, 16, 32),  # inner_dim != dim, as the reference layer tests allow
+    (1, 1, 32, 2, 16, 8),  # single point: exposes the 1e-2 epsilon
+])
+def test_fp32_irregular_stages_and_layer(B, N, dim, heads, dim_head, S):
+    announce("fp32 irregular", B, N, dim, heads, dim_head, S)
+    ref, hip = make_pair("irregular", dim, heads, dim_head, S, sharpen=2.0,
+                         temps=[0.3 + 5.7 * i / max(1, heads - 1) for i in range(heads)])
+    x = torch.randn(B, N, dim)
+    with torch.no_grad():
+        want = ref.stages(x)
+        got = hip.forward_stages(x.cuda())
+        y = hip(x.cuda())
+    for k in STAGES:
+        assert_fp32_close(got[k], want[k], k)
+    assert_fp32_close(y, want["y"], "layer y")
+    assert y.shape == (B, N, dim) and y.dtype == torch.float32
+
+
+@pytest.mark.parametrize("kernel,grid", [(1, (8, 8)), (3, (16, 16)), (3, (9, 14)), (5, (12, 7)), (7, (10, 10))])
+def test_fp32_structured2d_stages_and_layer(kernel, grid):
+    announce("fp32 structured2d", kernel, grid)
+    B, dim, heads, dim_head, S = 2, 32, 4, 8, 16
+    ref, hip = make_pair("structured2d", dim, heads, dim_head, S, spatial=grid, kernel=kernel, sharpen=2.0)
+    x = torch.randn(B, grid[0] * grid[1], dim)
+    with torch.no_grad():
+        want = ref.stages(x)
+        got = hip.forward_stages(x.cuda())
+        y = hip(x.cuda())
+    for k in STAGES:
+        assert_fp32_close(got[k], want[k], k)
+    assert_fp32_close(y, want["y"], "layer y")
+
+
+def test_fp32_block_tail_residual_and_layernorm():
+    announce("fp32 block tail")
+    B, N, dim, heads, S = 2, 300, 128, 8, 32
+    ref, hip = make_pair("irregular", dim, heads, dim // heads, S)
+    ln = torch.nn.LayerNorm(dim)
+    with torch.no_grad():
+        ln.weight.add_(0.2 * torch.randn(dim))
+        ln.bias.add_(0.2 * torch.randn(dim))
+    x, res = torch.randn(B, N, dim), torch.randn(B, N, dim)
+    with torch.no_grad():
+        want_fx = ref(x) + res
+        want_ln = ln(want_fx)
+        fx, normed = hip.forward_block(x.cuda(), res.cuda(), ln.cuda())
+    assert_fp32_close(fx, want_fx, "fx_new")
+    assert_fp32_close(normed, want_ln, "LayerNorm(fx_new)")
+
+
+def test_fp32_closed_form_zero_slice_projection():
+    # w = 1/S everywhere -> every point gets Wout tile_H(Wv sum_n fx_mid / (N + 0.01 S)) + bout
+    announce("fp32 closed form")
+    B, N, C, H, D, S = 2, 77, 64, 4, 16, 8
+    ref, hip = make_pair("irregular", C, H, D, S)
+    with torch.no_grad():
+        for m in (ref, hip):
+            m.in_project_slice.weight.zero_()
+            m.in_project_slice.bias.zero_()
+    x = torch.randn(B, N, C)
+    sd = {k: v.double() for k, v in ref.state_dict().items()}
+    fm = x.double() @ sd["in_project_fx.weight"].T + sd["in_project_fx.bias"]
+    tok = (fm.sum(1) / (N + 0.01 * S)).reshape(B, H, D)
+    o = torch.einsum("bhd,ed->bhe", tok, sd["qkv_project.weight"][2 * D:]).reshape(B, H * D)
+    want = (o @ sd["out_linear.weight"].T + sd["out_linear.bias"])[:, None, :].expand(B, N, C)
+    with torch.no_grad():
+        y = hip(x.cuda())
+    assert_fp32_close(y, want.float(), "closed form")
+
+
+def test_bf16_layer_against_fp32_oracle():
+    announce("bf16 general shapes")
+    for (B, N, dim, heads, dim_head, S) in [(2, 1000, 128, 8, 16, 32), (1, 515, 64, 2, 32, 4)]:
+        ref, hip = make_pair("irregular", dim, heads, dim_head, S)
+        x = torch.randn(B, N, dim)
+        with torch.no_grad():
+            want = ref(x)
+            y = hip(x.cuda().bfloat16())
+        assert y.dtype == torch.bfloat16
+        assert_rel_l2(y, want, f"bf16 y {B, N, dim, heads, dim_head, S}")
+
+
+def test_autocast_bf16_and_errors_on_gpu():
+    announce("autocast + error paths")
+    ref, hip = make_pair("irregular", 64, 4, 16, 8)
+    x = torch.randn(2, 200, 64)
+    with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
+        y = hip(x.cuda())
+    assert y.dtype == torch.bfloat16
+    with torch.no_grad():
+        assert_rel_l2(y, ref(x), "autocast y")
+    with pytest.raises(RuntimeError, match="forward pass only"):
+        hip(x.cuda())  # grad enabled, parameters require grad
+    with torch.no_grad(), pytest.raises(ValueError, match="Expected 3D input"):
+        hip(x.cuda()[0])
+    _, hip2 = make_pair("structured2d", 16, 2, 8, 4, spatial=(4, 4))
+    with torch.no_grad(), pytest.raises(RuntimeError):
+        hip2(torch.randn(1, 15, 16).cuda())  # 15 tokens cannot be viewed as a 4 x 4 grid
+
+
+def test_run_to_run_determinism():
+    announce("determinism")
+    ref, hip = make_pair("irregular", 128, 8, 16, 32)
+    x = torch.randn(2, 5000, 128).cuda()
+    with torch.no_grad():
+        a = hip(x)
+        for _ in range(5):
+            assert torch.equal(hip(x), a)
+
+
+def _golden_model(kind):
+    torch.manual_seed(0)
+    if kind == "2d":
+        kw = dict(structured_shape=(85, 85), n_layers=8, n_hidden=64, n_head=4, mlp_ratio=1, functional_dim=1,
+                  out_dim=1, slice_num=32, ref=1, unified_pos=True)
+        ref = to.OracleTransolver(init="rejection", **kw)
+        args = (torch.randn(4, 85 * 85, 1), torch.randn(4, 85, 85))
+        gold, atol = "transolver2d_output.pth", 2e-3
+    else:
+        kw = dict(structured_shape=None, n_layers=8, n_hidden=64, n_head=4, mlp_ratio=1, functional_dim=2,
+                  embedding_dim=3, out_dim=1, slice_num=32, unified_pos=False)
+        ref = to.OracleTransolver(init="rejection", **kw)
+        args = (torch.randn(4, 12345, 3), torch.randn(4, 12345, 2))
+        gold, atol = "transolver_irregular_output.pth", 1e-3
+    hip = pn.Transolver(use_te=False, **kw)
+    hip.load_state_dict(ref.state_dict())
+    return hip.cuda().eval(), args, torch.load(os.path.join(GOLD, gold), weights_only=True)[0], atol
+
+
+@pytest.mark.parametrize("kind", ["2d", "irregular"])
+def test_full_model_reproduces_reference_golden_output(kind):
+    # the reference's own non-regression vectors (test/models/transolver/test_transolver.py:97-169), its tolerances
+    announce("golden", kind)
+    hip, args, gold, atol = _golden_model(kind)
+    with torch.no_grad():
+        out = hip(*[a.cuda() for a in args]).cpu()
+    assert out.shape == gold.shape
+    assert torch.allclose(out, gold, rtol=1e-3, atol=atol), float((out - gold).abs().max())
+    assert float((out - gold).abs().max()) < 1e-4
+
+
+def test_model_flatten_equivalence_on_gpu():
+    announce("flatten equivalence")
+    torch.manual_seed(0)
+    m = pn.Transolver(functional_dim=3, out_dim=2, embedding_dim=4, structured_shape=(16, 16), n_layers=2,
+                      n_hidden=32, n_head=4, slice_num=8, use_te=False).cuda().eval()
+    fx, emb = torch.randn(2, 16, 16, 3).cuda(), torch.randn(2, 16, 16, 4).cuda()
+    with torch.no_grad():
+        a = m(fx, embedding=emb)
+        b = m(fx.reshape(2, -1, 3), embedding=emb.reshape(2, -1, 4))
+    assert a.shape == (2, 16, 16, 2)
+    assert torch.allclose(a.reshape(2, -1, 2), b, atol=1e-6)
