@@ -125,6 +125,34 @@ int pa_deslice_project(int dtype, const pa_shape *shape, const pa_params *p, con
                        const float *out_slice_token, void *scratch, void *y, const pa_block_tail *tail,
                        void *stream);
 
+/* ---- stage-level entry points of the bf16 MFMA kernels (shapes with pa_query_path() == 1) ------
+ * Intermediates use an internal register-order ("packed") layout; buffers are opaque to the caller and
+ * sized by pa_mfma_buffer_bytes(shape, which):
+ *   PA_BUF_BLOB     repacked parameters        PA_BUF_FX_PACK  fx_mid        PA_BUF_W_PACK  slice weights
+ *   PA_BUF_PARTIALS float32 reduction partials PA_BUF_TOKP     attended slice tokens as bf16 MFMA operands
+ * They replace the same reference lines as the natural-layout stages above. */
+#define PA_BUF_BLOB 0
+#define PA_BUF_FX_PACK 1
+#define PA_BUF_W_PACK 2
+#define PA_BUF_PARTIALS 3
+#define PA_BUF_TOKP 4
+int64_t pa_mfma_buffer_bytes(const pa_shape *shape, int which);
+/* Repack the layer parameters (bf16 large weights) for the MFMA kernels; run once per parameter set. */
+int pa_mfma_pack_params(const pa_shape *shape, const pa_params *p, void *blob, void *stream);
+/* Kernel (a): projections + slice logits + temperature softmax (PA.py:529-537, :172-181). x is bf16 (B,N,C). */
+int pa_mfma_project_softmax(const pa_shape *shape, const void *blob, const void *x, void *fx_pack, void *w_pack,
+                            void *stream);
+/* Kernel (b): first pass of the slice aggregation (PA.py:185-203) -> partials. */
+int pa_mfma_slice_reduce(const pa_shape *shape, const void *w_pack, const void *fx_pack, float *partials,
+                         void *stream);
+/* Second pass + kernel (c): fixed-order combine, normalisation, slice attention (PA.py:185-203, :429-465).
+ * slice_token / slice_norm may be NULL. Writes out_slice_token (B,H,S,D) float32 and its packed copy tokp. */
+int pa_mfma_combine_attention(const pa_shape *shape, const pa_params *p, const float *partials, float *slice_token,
+                              float *slice_norm, float *out_slice_token, void *tokp, void *stream);
+/* Kernel (d): deslice + out_linear + optional residual / LayerNorm tail (PA.py:467-499, TR.py:300-303). */
+int pa_mfma_deslice_project(const pa_shape *shape, const void *blob, const void *w_pack, const void *tokp, void *y,
+                            const pa_block_tail *tail, void *stream);
+
 /* ---- whole layer ------------------------------------------------------------------------------ */
 
 /* Replaces PhysicsAttentionBase.forward (PA.py:501-558), plus=False, use_te=False, dropout off.

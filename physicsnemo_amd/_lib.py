@@ -18,8 +18,11 @@ PA_F32, PA_BF16 = 0, 1
 EXPORTED = [
     "pa_version", "pa_status_string", "pa_workspace_bytes", "pa_query_path", "pa_project_inputs",
     "pa_slice_softmax", "pa_reduce_partial_count", "pa_slice_reduce", "pa_slice_attention",
-    "pa_deslice_project", "pa_layer_forward",
+    "pa_deslice_project", "pa_layer_forward", "pa_mfma_buffer_bytes", "pa_mfma_pack_params",
+    "pa_mfma_project_softmax", "pa_mfma_slice_reduce", "pa_mfma_combine_attention", "pa_mfma_deslice_project",
 ]
+
+PA_BUF_BLOB, PA_BUF_FX_PACK, PA_BUF_W_PACK, PA_BUF_PARTIALS, PA_BUF_TOKP = range(5)
 
 
 class PaShape(Structure):
@@ -74,6 +77,18 @@ def load() -> ctypes.CDLL:
     lib.pa_deslice_project.argtypes = [c_int, ps, pp, c_void_p, c_void_p, c_void_p, c_void_p, pt, c_void_p]
     lib.pa_layer_forward.restype = c_int
     lib.pa_layer_forward.argtypes = [c_int, ps, pp, c_void_p, c_void_p, pt, c_void_p, c_void_p, c_int64, c_void_p]
+    lib.pa_mfma_buffer_bytes.restype = c_int64
+    lib.pa_mfma_buffer_bytes.argtypes = [ps, c_int]
+    lib.pa_mfma_pack_params.restype = c_int
+    lib.pa_mfma_pack_params.argtypes = [ps, pp, c_void_p, c_void_p]
+    lib.pa_mfma_project_softmax.restype = c_int
+    lib.pa_mfma_project_softmax.argtypes = [ps, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]
+    lib.pa_mfma_slice_reduce.restype = c_int
+    lib.pa_mfma_slice_reduce.argtypes = [ps, c_void_p, c_void_p, c_void_p, c_void_p]
+    lib.pa_mfma_combine_attention.restype = c_int
+    lib.pa_mfma_combine_attention.argtypes = [ps, pp, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]
+    lib.pa_mfma_deslice_project.restype = c_int
+    lib.pa_mfma_deslice_project.argtypes = [ps, c_void_p, c_void_p, c_void_p, c_void_p, pt, c_void_p]
     _lib = lib
     return lib
 

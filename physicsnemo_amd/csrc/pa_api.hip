@@ -56,6 +56,47 @@ GeneralPlan plan_general(int dtype, const pa_shape &s) {
   return p;
 }
 
+// Workspace plan of the MFMA path.
+struct MfmaPlan {
+  int64_t off_blob, off_fx, off_w, off_partials, off_tok, off_norm, off_tok_out, off_tokp, total;
+  int64_t G;
+};
+
+int64_t mfma_partials_bytes(const pa_shape &s) {
+  return pa::mfma::reduce_groups(s) * s.B * s.H * s.S * (s.D + 1) * 4;
+}
+
+MfmaPlan plan_mfma(const pa_shape &s) {
+  MfmaPlan p{};
+  p.G = pa::mfma::reduce_groups(s);
+  int64_t off = 0;
+  p.off_blob = off;
+  off += round_up(pa::mfma::blob_bytes(s), 256);
+  p.off_fx = off;
+  off += round_up(pa::mfma::fx_pack_bytes(s), 256);
+  p.off_w = off;
+  off += round_up(pa::mfma::w_pack_bytes(s), 256);
+  p.off_partials = off;
+  off += round_up(mfma_partials_bytes(s), 256);
+  p.off_tok = off;
+  off += round_up(s.B * s.H * s.S * s.D * 4, 256);
+  p.off_norm = off;
+  off += round_up(s.B * s.H * s.S * 4, 256);
+  p.off_tok_out = off;
+  off += round_up(s.B * s.H * s.S * s.D * 4, 256);
+  p.off_tokp = off;
+  off += round_up(pa::mfma::tokp_bytes(s), 256);
+  p.total = off;
+  return p;
+}
+
+int compute_units() {
+  int dev = 0, n = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return 256;
+  if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) return 256;
+  return n;
+}
+
 int check_params(const pa_params *p) {
   if (!p) return PA_ERR_NULL;
   if (!p->in_project_x_weight || !p->in_project_x_bias || !p->in_project_fx_weight || !p->in_project_fx_bias ||
@@ -97,12 +138,13 @@ const char *pa_status_string(int code) {
 int pa_query_path(int dtype, const pa_shape *shape) {
   int rc = check_shape(dtype, shape);
   if (rc) return rc;
-  return 0;
+  return pa::mfma::supported(dtype, *shape) ? 1 : 0;
 }
 
 int64_t pa_workspace_bytes(int dtype, const pa_shape *shape) {
   int rc = check_shape(dtype, shape);
   if (rc) return rc;
+  if (pa::mfma::supported(dtype, *shape)) return plan_mfma(*shape).total;
   return plan_general(dtype, *shape).total;
 }
 
@@ -170,6 +212,76 @@ int pa_deslice_project(int dtype, const pa_shape *shape, const pa_params *p, con
   return rc;
 }
 
+int64_t pa_mfma_buffer_bytes(const pa_shape *shape, int which) {
+  int rc = check_shape(PA_BF16, shape);
+  if (rc) return rc;
+  if (!pa::mfma::supported(PA_BF16, *shape)) return PA_ERR_UNSUPPORTED;
+  switch (which) {
+    case PA_BUF_BLOB: return pa::mfma::blob_bytes(*shape);
+    case PA_BUF_FX_PACK: return pa::mfma::fx_pack_bytes(*shape);
+    case PA_BUF_W_PACK: return pa::mfma::w_pack_bytes(*shape);
+    case PA_BUF_PARTIALS: return mfma_partials_bytes(*shape);
+    case PA_BUF_TOKP: return pa::mfma::tokp_bytes(*shape);
+    default: return PA_ERR_DIMS;
+  }
+}
+
+static int check_mfma(const pa_shape *shape) {
+  int rc = check_shape(PA_BF16, shape);
+  if (rc) return rc;
+  return pa::mfma::supported(PA_BF16, *shape) ? PA_OK : PA_ERR_UNSUPPORTED;
+}
+
+int pa_mfma_pack_params(const pa_shape *shape, const pa_params *p, void *blob, void *stream) {
+  int rc = check_mfma(shape);
+  if (rc) return rc;
+  if ((rc = check_params(p))) return rc;
+  if (!blob) return PA_ERR_NULL;
+  if (!aligned16(blob)) return PA_ERR_ALIGN;
+  return pa::mfma::pack_params(*shape, *p, blob, static_cast<hipStream_t>(stream));
+}
+
+int pa_mfma_project_softmax(const pa_shape *shape, const void *blob, const void *x, void *fx_pack, void *w_pack,
+                            void *stream) {
+  int rc = check_mfma(shape);
+  if (rc) return rc;
+  if (!blob || !x || !fx_pack || !w_pack) return PA_ERR_NULL;
+  if (!aligned16(blob) || !aligned16(x) || !aligned16(fx_pack) || !aligned16(w_pack)) return PA_ERR_ALIGN;
+  return pa::mfma::project_softmax(*shape, blob, x, fx_pack, w_pack, static_cast<hipStream_t>(stream));
+}
+
+int pa_mfma_slice_reduce(const pa_shape *shape, const void *w_pack, const void *fx_pack, float *partials, void *stream) {
+  int rc = check_mfma(shape);
+  if (rc) return rc;
+  if (!w_pack || !fx_pack || !partials) return PA_ERR_NULL;
+  if (!aligned16(w_pack) || !aligned16(fx_pack) || !aligned16(partials)) return PA_ERR_ALIGN;
+  return pa::mfma::slice_reduce(*shape, w_pack, fx_pack, partials, static_cast<hipStream_t>(stream));
+}
+
+int pa_mfma_combine_attention(const pa_shape *shape, const pa_params *p, const float *partials, float *slice_token,
+                              float *slice_norm, float *out_slice_token, void *tokp, void *stream) {
+  int rc = check_mfma(shape);
+  if (rc) return rc;
+  if (!p || !p->qkv_project_weight || !partials || !out_slice_token || !tokp) return PA_ERR_NULL;
+  if (!aligned16(partials) || !aligned16(tokp)) return PA_ERR_ALIGN;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  rc = pa::general::combine_attention(*shape, *p, partials, pa::mfma::reduce_groups(*shape), slice_token, slice_norm,
+                                      out_slice_token, st);
+  if (rc) return rc;
+  return pa::mfma::pack_tokens(*shape, out_slice_token, tokp, st);
+}
+
+int pa_mfma_deslice_project(const pa_shape *shape, const void *blob, const void *w_pack, const void *tokp, void *y,
+                            const pa_block_tail *tail, void *stream) {
+  int rc = check_mfma(shape);
+  if (rc) return rc;
+  if (!blob || !w_pack || !tokp || !y) return PA_ERR_NULL;
+  if (!aligned16(blob) || !aligned16(w_pack) || !aligned16(tokp) || !aligned16(y)) return PA_ERR_ALIGN;
+  if ((rc = check_tail(tail))) return rc;
+  return pa::mfma::deslice_project(*shape, blob, w_pack, tokp, y, tail_active(tail) ? tail : nullptr, compute_units(),
+                                   static_cast<hipStream_t>(stream));
+}
+
 int pa_layer_forward(int dtype, const pa_shape *shape, const pa_params *p, const void *x, void *y,
                      const pa_block_tail *tail, float *slice_token_out, void *workspace, int64_t workspace_bytes,
                      void *stream) {
@@ -182,9 +294,24 @@ int pa_layer_forward(int dtype, const pa_shape *shape, const pa_params *p, const
   const pa_shape &s = *shape;
   hipStream_t st = static_cast<hipStream_t>(stream);
 
+  char *ws = static_cast<char *>(workspace);
+  if (pa::mfma::supported(dtype, s)) {
+    const MfmaPlan mp = plan_mfma(s);
+    if (workspace_bytes < mp.total) return PA_ERR_WORKSPACE;
+    void *blob = ws + mp.off_blob, *fxp = ws + mp.off_fx, *wp = ws + mp.off_w, *tokp = ws + mp.off_tokp;
+    float *partials = reinterpret_cast<float *>(ws + mp.off_partials);
+    float *tok = slice_token_out ? slice_token_out : reinterpret_cast<float *>(ws + mp.off_tok);
+    float *norm = reinterpret_cast<float *>(ws + mp.off_norm);
+    float *tok_out = reinterpret_cast<float *>(ws + mp.off_tok_out);
+    if ((rc = pa::mfma::pack_params(s, *p, blob, st))) return rc;
+    if ((rc = pa::mfma::project_softmax(s, blob, x, fxp, wp, st))) return rc;
+    if ((rc = pa::mfma::slice_reduce(s, wp, fxp, partials, st))) return rc;
+    if ((rc = pa::general::combine_attention(s, *p, partials, mp.G, tok, norm, tok_out, st))) return rc;
+    if ((rc = pa::mfma::pack_tokens(s, tok_out, tokp, st))) return rc;
+    return pa::mfma::deslice_project(s, blob, wp, tokp, y, tail_active(tail) ? tail : nullptr, compute_units(), st);
+  }
   const GeneralPlan plan = plan_general(dtype, s);
   if (workspace_bytes < plan.total) return PA_ERR_WORKSPACE;
-  char *ws = static_cast<char *>(workspace);
   void *x_mid = ws + plan.off_x_mid, *fx_mid = ws + plan.off_fx_mid, *w = ws + plan.off_w;
   float *partials = reinterpret_cast<float *>(ws + plan.off_partials);
   float *tok = slice_token_out ? slice_token_out : reinterpret_cast<float *>(ws + plan.off_tok);

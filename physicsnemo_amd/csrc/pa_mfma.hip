@@ -1,0 +1,635 @@
+// bf16 MFMA kernels for the irregular-mesh PhysicsAttention layer on gfx950 (D = 32, C = H*32 in {128, 256},
+// S in {16, 32, 64, 128}).  v_mfma_f32_32x32x16_bf16 everywhere, fp32 accumulation.
+//
+// Work unit: a TILE of 32 consecutive points of one batch, owned by one wavefront.
+//
+// MFMA register layouts used below (lane = 32*g + i, i = lane % 32, g = lane / 32):
+//   A operand (32 x 16): lane holds row i, k = 8g + j, j = 0..7.      B operand (16 x 32): column i, k = 8g + j.
+//   C/D (32 x 32): lane holds column i; register r = 0..15 is row  rowmap(r, g) = 8*(r/4) + 4*g + r%4.
+// A C/D tile converted to bf16 is therefore directly a pair of A (or B) operands of a following MFMA whose
+// reduction index is the C/D ROW index, taken in the order
+//   kperm(kk, g, j) = 16*kk + 8*(j/4) + 4*g + j%4          (kk = 0, 1 selects registers 8kk .. 8kk+7)
+// provided the other operand is loaded with the same permutation.  All chained products below rely on this;
+// no shuffles or LDS transposes are needed between the GEMMs of one kernel.
+//
+// Intermediates between kernels are stored in that register order ("packed"), 16 bytes per lane, 1 KiB per wave
+// store, so every global access of the three big kernels is a full-width coalesced transaction:
+//   w_pack [tile][h][cq][lane][8]  slice weights, chunk cq = 16 slices: element j <-> slice 16cq + 8(j/4) + 4g + j%4
+//                                  of point i of the tile                       (B operand of the deslice product)
+//   fx_pack[tile][h][kk][lane][8]  fx_mid, lane i <-> channel d = i of head h, element j <-> point kperm(kk, g, j)
+//                                                                                (A operand of the aggregation)
+#include "pa_common.h"
+#include "pa_host.h"
+
+namespace pa {
+namespace mfma {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ f32x16 mma(u32x4 a, u32x4 b, f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+}
+
+__device__ __forceinline__ int rowmap(int r, int g) { return 8 * (r >> 2) + 4 * g + (r & 3); }
+__device__ __forceinline__ int kperm(int kk, int g, int j) { return 16 * kk + 8 * (j >> 2) + 4 * g + (j & 3); }
+
+// registers 8*HALF .. 8*HALF+7 of an accumulator, scaled, as 8 bf16 (round to nearest even)
+template <int HALF>
+__device__ __forceinline__ u32x4 pack_half(const f32x16 &v, float scale = 1.f) {
+  bf16x8 o;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) o[j] = (__bf16)(v[8 * HALF + j] * scale);
+  return __builtin_bit_cast(u32x4, o);
+}
+
+__device__ __forceinline__ uint16_t to_bf16_bits(float f) { return __builtin_bit_cast(uint16_t, (__bf16)f); }
+
+// ------------------------------------------------------------------------------------------------
+// Packed parameter blob (built once per call by pack_params_kernel).  Offsets in 16-byte units.
+//   win [h][m][ks][lane]  m = 0: in_project_x, 1: in_project_fx; W_m[h*32 + i][16ks + 8g + j]
+//   wsl [st][kk][lane]    in_project_slice[32st + i][kperm(kk, g, j)]   (0 beyond S)
+//   wout[ct][h][kk][lane] out_linear[i*CT + ct][h*32 + kperm(kk, g, j)],  CT = C/32
+//   then float vectors: bias_x[C], bias_fx[C], bias_slice[ST*32] (-1e30 beyond S), bias_out[C], tscale[H]
+// ------------------------------------------------------------------------------------------------
+struct BlobPlan {
+  int64_t win, wsl, wout, fvec, total_units;  // 16-byte units
+};
+
+__host__ __device__ inline BlobPlan blob_plan(int C, int S) {
+  const int H = C / 32, KS = C / 16, ST = (S + 31) / 32, CT = C / 32;
+  BlobPlan p;
+  p.win = 0;
+  p.wsl = p.win + (int64_t)H * 2 * KS * 64;
+  p.wout = p.wsl + (int64_t)ST * 2 * 64;
+  p.fvec = p.wout + (int64_t)CT * H * 2 * 64;
+  const int64_t nfloat = 3 * C + ST * 32 + H;
+  p.total_units = p.fvec + (nfloat + 3) / 4;
+  return p;
+}
+
+__global__ __launch_bounds__(256) void pack_params_kernel(pa_params p, u32x4 *__restrict__ blob, int C, int S) {
+  const int H = C / 32, KS = C / 16, ST = (S + 31) / 32, CT = C / 32;
+  const BlobPlan bp = blob_plan(C, S);
+  const uint16_t *wx = static_cast<const uint16_t *>(p.in_project_x_weight);
+  const uint16_t *wfx = static_cast<const uint16_t *>(p.in_project_fx_weight);
+  const uint16_t *wo = static_cast<const uint16_t *>(p.out_linear_weight);
+  const int64_t n_units = bp.fvec;
+  for (int64_t u = (int64_t)blockIdx.x * 256 + threadIdx.x; u < n_units; u += (int64_t)gridDim.x * 256) {
+    const int lane = (int)(u & 63), i = lane & 31, g = lane >> 5;
+    uint16_t e[8];
+    if (u < bp.wsl) {
+      int64_t q = u >> 6;
+      const int ks = (int)(q % KS);
+      q /= KS;
+      const int m = (int)(q & 1), h = (int)(q >> 1);
+      const uint16_t *src = (m ? wfx : wx) + (int64_t)(h * 32 + i) * C + 16 * ks + 8 * g;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) e[j] = src[j];
+    } else if (u < bp.wout) {
+      const int q = (int)((u - bp.wsl) >> 6);
+      const int kk = q & 1, st = q >> 1;
+      const int s = 32 * st + i;
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        e[j] = s < S ? to_bf16_bits(p.in_project_slice_weight[(int64_t)s * 32 + kperm(kk, g, j)]) : (uint16_t)0;
+    } else {
+      int q = (int)((u - bp.wout) >> 6);
+      const int kk = q & 1;
+      q >>= 1;
+      const int h = q % H, ct = q / H;
+      const uint16_t *src = wo + (int64_t)(i * CT + ct) * C + h * 32;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) e[j] = src[kperm(kk, g, j)];
+    }
+    u32x4 v;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) v[j] = (uint32_t)e[2 * j] | ((uint32_t)e[2 * j + 1] << 16);
+    blob[u] = v;
+  }
+  float *fv = reinterpret_cast<float *>(blob + bp.fvec);
+  const int nfloat = 3 * C + ST * 32 + H;
+  for (int k = blockIdx.x * 256 + threadIdx.x; k < nfloat; k += gridDim.x * 256) {
+    float v;
+    if (k < C) v = p.in_project_x_bias[k];
+    else if (k < 2 * C) v = p.in_project_fx_bias[k - C];
+    else if (k < 2 * C + ST * 32) v = (k - 2 * C) < S ? p.in_project_slice_bias[k - 2 * C] : -1e30f;
+    else if (k < 3 * C + ST * 32) v = p.out_linear_bias[k - 2 * C - ST * 32];
+    else v = kLog2e / clamp_temperature(p.temperature[k - 3 * C - ST * 32]);
+    fv[k] = v;
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Kernel (a): projections + slice logits + temperature softmax.   512 threads = 8 waves = 8 tiles.
+//   x_mid^T (32 ch x 32 pts) = Wx_h . x^T          A = Wx_h frags (LDS), B = x frags (registers, loaded once)
+//   fx_mid  (32 pts x 32 d)  = x . Wfx_h^T         A = x frags,          B = Wfx_h frags (LDS)   -> fx_pack
+//   logits^T(32 s x 32 pts)  = Wslice . x_mid^T    A = Wslice frags (LDS), B = bf16(x_mid^T) straight from registers
+//   softmax over s: in-lane over the accumulator registers plus one exchange with lane^32          -> w_pack
+// Per-head weights (Wx_h | Wfx_h, 2*KS KiB) are double-buffered in LDS: the next head's 64 bytes per thread
+// are fetched into registers before the current head's products and stored to LDS after them.
+// ------------------------------------------------------------------------------------------------
+template <int C, int S>
+__global__ __launch_bounds__(512) void project_softmax_kernel(const u32x4 *__restrict__ blob, const uint16_t *__restrict__ x,
+                                                              u32x4 *__restrict__ fx_pack, u32x4 *__restrict__ w_pack,
+                                                              int64_t N, int tpb, int64_t total_tiles) {
+  constexpr int H = C / 32, KS = C / 16, ST = (S + 31) / 32, NCH = S / 16;
+  constexpr int HEAD_UNITS = 2 * KS * 64;  // 16-byte units of one head's weights
+  constexpr int PER_THREAD = HEAD_UNITS / 512;
+  static_assert(HEAD_UNITS % 512 == 0, "head weights must split evenly over the workgroup");
+  extern __shared__ u32x4 smem[];
+  u32x4 *wbuf = smem;                       // 2 * HEAD_UNITS
+  u32x4 *wsl = wbuf + 2 * HEAD_UNITS;       // ST * 2 * 64
+  float *fvec = reinterpret_cast<float *>(wsl + ST * 2 * 64);
+  float *bias_x = fvec, *bias_f = fvec + C, *bias_s = fvec + 2 * C, *tscale = fvec + 3 * C + ST * 32;
+  const BlobPlan bp = blob_plan(C, S);
+
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, i = lane & 31, g = lane >> 5;
+  const int64_t tile = (int64_t)blockIdx.x * 8 + wave;
+  const bool tile_ok = tile < total_tiles;
+  const int64_t b = tile_ok ? tile / tpb : 0;
+  const int64_t n = tile_ok ? (tile - b * tpb) * 32 + i : 0;
+  const bool valid = tile_ok && n < N;
+
+  // x fragments of this wave's 32 points (zero rows beyond N)
+  u32x4 xf[KS];
+  {
+    const u32x4 *xr = reinterpret_cast<const u32x4 *>(x + ((int64_t)b * N + n) * C) + g;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) xf[ks] = valid ? xr[2 * ks] : u32x4{0, 0, 0, 0};
+  }
+  // small parameters and the first head's weights
+  for (int u = tid; u < ST * 2 * 64; u += 512) wsl[u] = blob[bp.wsl + u];
+  {
+    const float *src = reinterpret_cast<const float *>(blob + bp.fvec);
+    for (int k = tid; k < 3 * C + ST * 32 + H; k += 512) fvec[k] = src[k];
+  }
+#pragma unroll
+  for (int q = 0; q < PER_THREAD; ++q) wbuf[q * 512 + tid] = blob[bp.win + q * 512 + tid];
+  __syncthreads();
+
+  for (int h = 0; h < H; ++h) {
+    u32x4 nxt[PER_THREAD];
+    if (h + 1 < H) {
+#pragma unroll
+      for (int q = 0; q < PER_THREAD; ++q) nxt[q] = blob[bp.win + (int64_t)(h + 1) * HEAD_UNITS + q * 512 + tid];
+    }
+    if (tile_ok) {
+      const u32x4 *wb = wbuf + (h & 1) * HEAD_UNITS;
+      f32x16 ax, af;
+      {
+        const float bf = bias_f[h * 32 + i];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          ax[r] = bias_x[h * 32 + rowmap(r, g)];
+          af[r] = bf;
+        }
+      }
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const u32x4 a = wb[ks * 64 + lane];
+        const u32x4 bw = wb[(KS + ks) * 64 + lane];
+        ax = mma(a, xf[ks], ax);
+        af = mma(xf[ks], bw, af);
+      }
+      u32x4 *fdst = fx_pack + ((tile * H + h) * 2) * 64 + lane;
+      fdst[0] = pack_half<0>(af);
+      fdst[64] = pack_half<1>(af);
+
+      const u32x4 xb0 = pack_half<0>(ax), xb1 = pack_half<1>(ax);
+      f32x16 lg[ST];
+      float mx = -INFINITY;
+#pragma unroll
+      for (int st = 0; st < ST; ++st) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) lg[st][r] = bias_s[32 * st + rowmap(r, g)];
+        lg[st] = mma(wsl[(st * 2 + 0) * 64 + lane], xb0, lg[st]);
+        lg[st] = mma(wsl[(st * 2 + 1) * 64 + lane], xb1, lg[st]);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) mx = fmaxf(mx, lg[st][r]);
+      }
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      const float sc = tscale[h];
+      const float off = mx * sc;
+      float sum = 0.f;
+#pragma unroll
+      for (int st = 0; st < ST; ++st)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const float e = __builtin_amdgcn_exp2f(fmaf(lg[st][r], sc, -off));
+          lg[st][r] = e;
+          sum += e;
+        }
+      sum += __shfl_xor(sum, 32, 64);
+      const float inv = valid ? __builtin_amdgcn_rcpf(sum) : 0.f;
+      u32x4 *wdst = w_pack + ((tile * H + h) * NCH) * 64 + lane;
+#pragma unroll
+      for (int st = 0; st < ST; ++st) {
+        if (2 * st < NCH) wdst[(2 * st) * 64] = pack_half<0>(lg[st], inv);
+        if (2 * st + 1 < NCH) wdst[(2 * st + 1) * 64] = pack_half<1>(lg[st], inv);
+      }
+    }
+    if (h + 1 < H) {
+      u32x4 *dst = wbuf + ((h + 1) & 1) * HEAD_UNITS;
+#pragma unroll
+      for (int q = 0; q < PER_THREAD; ++q) dst[q * 512 + tid] = nxt[q];
+    }
+    __syncthreads();
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Kernel (b): slice-token aggregation, streaming over the packed w / fx_mid.  grid (G groups, B*H), 4 waves.
+// Each wave walks every 4th tile of its group's tile range for one (batch, head):
+//   w^T (32 pts x 32 s, C/D layout: lane <-> slice, registers <-> points) = w_chunk . SEL     (an exact MFMA
+//       "transpose": A = stored chunk (rows = points), B = 0/1 selection matrix)
+//   norm[s]  += sum of those registers                       (fp32, in lane)
+//   tok^T (32 d x 32 s) += fx_chunk (A, rows = d, k = points) . bf16(w^T) (B, k = points)
+// The 4 waves' accumulators are summed through LDS in wave order and written as one partial
+//   partials[g][b][h][s][0..D-1] = sum_n w fx,   [..][D] = sum_n w          (layout of the general combine kernel)
+// ------------------------------------------------------------------------------------------------
+template <int S>
+__global__ __launch_bounds__(256) void slice_reduce_kernel(const u32x4 *__restrict__ w_pack, const u32x4 *__restrict__ fx_pack,
+                                                           float *__restrict__ partials, int B, int H, int tpb,
+                                                           int tiles_per_group) {
+  constexpr int ST = (S + 31) / 32, NCH = S / 16, D = 32, D1 = D + 1;
+  extern __shared__ float red[];  // [4 waves][ST][17][64]
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, i = lane & 31, g = lane >> 5;
+  const int bh = blockIdx.y, b = bh / H, h = bh - b * H;
+  u32x4 sel[2];
+#pragma unroll
+  for (int par = 0; par < 2; ++par) {
+    bf16x8 s8;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) s8[j] = (__bf16)((i == kperm(par, g, j)) ? 1.f : 0.f);
+    sel[par] = __builtin_bit_cast(u32x4, s8);
+  }
+  f32x16 tok[ST];
+  float nrm[ST];
+#pragma unroll
+  for (int st = 0; st < ST; ++st) {
+    nrm[st] = 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) tok[st][r] = 0.f;
+  }
+  const int t_begin = blockIdx.x * tiles_per_group;
+  const int t_end = min(tpb, t_begin + tiles_per_group);
+  for (int t = t_begin + wave; t < t_end; t += 4) {
+    const int64_t gt = (int64_t)b * tpb + t;
+    const u32x4 *wsrc = w_pack + ((gt * H + h) * NCH) * 64 + lane;
+    const u32x4 *fsrc = fx_pack + ((gt * H + h) * 2) * 64 + lane;
+    u32x4 wf[NCH];
+#pragma unroll
+    for (int cq = 0; cq < NCH; ++cq) wf[cq] = wsrc[cq * 64];
+    const u32x4 f0 = fsrc[0], f1 = fsrc[64];
+#pragma unroll
+    for (int st = 0; st < ST; ++st) {
+      f32x16 tr;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) tr[r] = 0.f;
+      tr = mma(wf[2 * st], sel[0], tr);
+      if (2 * st + 1 < NCH) tr = mma(wf[2 * st + 1 < NCH ? 2 * st + 1 : 0], sel[1], tr);
+      float s16 = 0.f;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) s16 += tr[r];
+      nrm[st] += s16;
+      tok[st] = mma(f0, pack_half<0>(tr), tok[st]);
+      tok[st] = mma(f1, pack_half<1>(tr), tok[st]);
+    }
+  }
+  float *mine = red + (size_t)wave * ST * 17 * 64;
+#pragma unroll
+  for (int st = 0; st < ST; ++st) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) mine[(st * 17 + r) * 64 + lane] = tok[st][r];
+    mine[(st * 17 + 16) * 64 + lane] = nrm[st];
+  }
+  __syncthreads();
+  float *dst = partials + (((int64_t)blockIdx.x * B + b) * H + h) * (S * D1);
+  for (int e = tid; e < ST * 17 * 64; e += 256) {
+    const int l = e & 63, r = (e >> 6) % 17, st = (e >> 6) / 17;
+    const int s = 32 * st + (l & 31);
+    if (s >= S) continue;
+    if (r < 16) {
+      float acc = 0.f;
+#pragma unroll
+      for (int w4 = 0; w4 < 4; ++w4) acc += red[(size_t)w4 * ST * 17 * 64 + e];
+      dst[s * D1 + rowmap(r, l >> 5)] = acc;
+    } else if (l < 32) {
+      float acc = 0.f;
+#pragma unroll
+      for (int w4 = 0; w4 < 4; ++w4) {
+        acc += red[(size_t)w4 * ST * 17 * 64 + e];
+        acc += red[(size_t)w4 * ST * 17 * 64 + e + 32];
+      }
+      dst[s * D1 + D] = acc;
+    }
+  }
+}
+
+// tok' (B, H, S, 32) fp32 -> bf16 A operands of the deslice product: tokp[b][h][cq][lane][j] = tok'[b][h][16cq + kperm-slice][i]
+__global__ __launch_bounds__(256) void pack_tokens_kernel(const float *__restrict__ tok, u32x4 *__restrict__ tokp, int64_t units,
+                                                          int S) {
+  const int NCH = S / 16;
+  for (int64_t u = (int64_t)blockIdx.x * 256 + threadIdx.x; u < units; u += (int64_t)gridDim.x * 256) {
+    const int lane = (int)(u & 63), i = lane & 31, g = lane >> 5;
+    const int64_t q = u >> 6;
+    const int cq = (int)(q % NCH);
+    const int64_t bh = q / NCH;
+    bf16x8 o;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) o[j] = (__bf16)tok[(bh * S + 16 * cq + kperm(0, g, j)) * 32 + i];
+    tokp[u] = __builtin_bit_cast(u32x4, o);
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Kernel (d): deslice + out_linear (+ residual, + LayerNorm).  Persistent: the whole packed out_linear weight
+// (C*C*2 bytes) sits in LDS, so one 4-wave workgroup per CU (one wave per SIMD, up to 512 registers each)
+// loops over tiles; each wave owns a tile at a time.
+//   out_x^T (32 d x 32 pts) = tok'^T_h . w^T_h       A = tokp frags (global, L2 resident), B = w_pack chunks
+//   y (32 pts x C)          = out_x . Wout^T         A = bf16(out_x^T) from registers, B = Wout frags (LDS)
+// Output columns are interleaved over the C/32 accumulator tiles (column of tile ct, lane i = i*CT + ct) so each
+// lane ends up with CT consecutive channels of a row: one 16-byte store per row and lane (C = 256).
+// ------------------------------------------------------------------------------------------------
+template <int C, int S>
+__global__ __launch_bounds__(256) void deslice_project_kernel(const u32x4 *__restrict__ blob, const u32x4 *__restrict__ w_pack,
+                                                              const u32x4 *__restrict__ tokp, uint16_t *__restrict__ y,
+                                                              const uint16_t *__restrict__ residual,
+                                                              const float *__restrict__ ln_gamma,
+                                                              const float *__restrict__ ln_beta, float ln_eps,
+                                                              uint16_t *__restrict__ ln_out, int64_t N, int tpb,
+                                                              int64_t total_tiles) {
+  constexpr int H = C / 32, CT = C / 32, ST = (S + 31) / 32, NCH = S / 16;
+  constexpr int WOUT_UNITS = CT * H * 2 * 64;
+  extern __shared__ u32x4 smem[];
+  u32x4 *wo = smem;  // WOUT_UNITS
+  const BlobPlan bp = blob_plan(C, S);
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, i = lane & 31, g = lane >> 5;
+  for (int u = tid; u < WOUT_UNITS; u += 256) wo[u] = blob[bp.wout + u];
+  float bout[CT], gam[CT], bet[CT];
+  {
+    const float *fv = reinterpret_cast<const float *>(blob + bp.fvec) + 2 * C + ST * 32;
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+      bout[ct] = fv[i * CT + ct];
+      gam[ct] = ln_out ? ln_gamma[i * CT + ct] : 1.f;
+      bet[ct] = ln_out ? ln_beta[i * CT + ct] : 0.f;
+    }
+  }
+  __syncthreads();
+
+  for (int64_t tile = (int64_t)blockIdx.x * 4 + wave; tile < total_tiles; tile += (int64_t)gridDim.x * 4) {
+    const int64_t b = tile / tpb;
+    const int64_t n0 = (tile - b * tpb) * 32;
+    // deslice every head; keep bf16(out_x^T) as A operands of the projection
+    u32x4 oxf[H][2];
+#pragma unroll
+    for (int h = 0; h < H; ++h) {
+      const u32x4 *wsrc = w_pack + ((tile * H + h) * NCH) * 64 + lane;
+      const u32x4 *tsrc = tokp + (((int64_t)b * H + h) * NCH) * 64 + lane;
+      f32x16 ox;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) ox[r] = 0.f;
+#pragma unroll
+      for (int cq = 0; cq < NCH; ++cq) ox = mma(tsrc[cq * 64], wsrc[cq * 64], ox);
+      oxf[h][0] = pack_half<0>(ox);
+      oxf[h][1] = pack_half<1>(ox);
+    }
+    f32x16 acc[CT];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[ct][r] = bout[ct];
+#pragma unroll
+      for (int h = 0; h < H; ++h) {
+        acc[ct] = mma(oxf[h][0], wo[((ct * H + h) * 2 + 0) * 64 + lane], acc[ct]);
+        acc[ct] = mma(oxf[h][1], wo[((ct * H + h) * 2 + 1) * 64 + lane], acc[ct]);
+      }
+    }
+    // epilogue: row = point, this lane holds channels i*CT .. i*CT+CT-1
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int64_t n = n0 + rowmap(r, g);
+      const bool ok = n < N;
+      const int64_t off = ((int64_t)b * N + n) * C + i * CT;
+      float v[CT];
+#pragma unroll
+      for (int ct = 0; ct < CT; ++ct) v[ct] = acc[ct][r];
+      if (residual) {
+        // y is rounded to bf16 before the residual is added, and the sum rounded again (two tensor ops upstream)
+        uint16_t rs[CT];
+        if (ok) {
+          if constexpr (CT == 8) {
+            const u32x4 q = *reinterpret_cast<const u32x4 *>(residual + off);
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+              rs[2 * k] = (uint16_t)(q[k] & 0xffffu);
+              rs[2 * k + 1] = (uint16_t)(q[k] >> 16);
+            }
+          } else {
+            const u32x2 q = *reinterpret_cast<const u32x2 *>(residual + off);
+#pragma unroll
+            for (int k = 0; k < 2; ++k) {
+              rs[2 * k] = (uint16_t)(q[k] & 0xffffu);
+              rs[2 * k + 1] = (uint16_t)(q[k] >> 16);
+            }
+          }
+        } else {
+#pragma unroll
+          for (int ct = 0; ct < CT; ++ct) rs[ct] = 0;
+        }
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) v[ct] = (float)(__bf16)v[ct] + bf16_bits_to_f32(rs[ct]);
+      }
+      uint16_t ob[CT];
+#pragma unroll
+      for (int ct = 0; ct < CT; ++ct) {
+        ob[ct] = to_bf16_bits(v[ct]);
+        v[ct] = bf16_bits_to_f32(ob[ct]);
+      }
+      if (ok) {
+        if constexpr (CT == 8) {
+          u32x4 q;
+#pragma unroll
+          for (int k = 0; k < 4; ++k) q[k] = (uint32_t)ob[2 * k] | ((uint32_t)ob[2 * k + 1] << 16);
+          *reinterpret_cast<u32x4 *>(y + off) = q;
+        } else {
+          u32x2 q;
+#pragma unroll
+          for (int k = 0; k < 2; ++k) q[k] = (uint32_t)ob[2 * k] | ((uint32_t)ob[2 * k + 1] << 16);
+          *reinterpret_cast<u32x2 *>(y + off) = q;
+        }
+      }
+      if (ln_out) {
+        float s1 = 0.f;
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) s1 += v[ct];
+#pragma unroll
+        for (int o = 16; o > 0; o >>= 1) s1 += __shfl_xor(s1, o, 64);
+        const float mean = s1 * (1.f / C);
+        float s2 = 0.f;
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) {
+          const float dl = v[ct] - mean;
+          s2 = fmaf(dl, dl, s2);
+        }
+#pragma unroll
+        for (int o = 16; o > 0; o >>= 1) s2 += __shfl_xor(s2, o, 64);
+        const float rstd = rsqrtf(s2 * (1.f / C) + ln_eps);
+        uint16_t lb[CT];
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) lb[ct] = to_bf16_bits((v[ct] - mean) * rstd * gam[ct] + bet[ct]);
+        if (ok) {
+          if constexpr (CT == 8) {
+            u32x4 q;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) q[k] = (uint32_t)lb[2 * k] | ((uint32_t)lb[2 * k + 1] << 16);
+            *reinterpret_cast<u32x4 *>(ln_out + off) = q;
+          } else {
+            u32x2 q;
+#pragma unroll
+            for (int k = 0; k < 2; ++k) q[k] = (uint32_t)lb[2 * k] | ((uint32_t)lb[2 * k + 1] << 16);
+            *reinterpret_cast<u32x2 *>(ln_out + off) = q;
+          }
+        }
+      }
+    }
+  }
+}
+
+// ================================================================================================
+// host side
+// ================================================================================================
+static int launch_status() {
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? PA_OK : (int)e;
+}
+
+template <typename F>
+static int allow_dynamic_lds(F kernel, size_t bytes) {
+  if (bytes > kMaxLdsBytes) return PA_ERR_UNSUPPORTED;
+  if (bytes > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+    if (e != hipSuccess) return (int)e;
+  }
+  return PA_OK;
+}
+
+bool supported(int dtype, const pa_shape &s) {
+  if (dtype != PA_BF16 || s.conv_k != 0 || s.D != 32 || s.C != s.H * 32) return false;
+  if (s.C != 128 && s.C != 256) return false;
+  if (s.S != 16 && s.S != 32 && s.S != 64 && s.S != 128) return false;
+  if ((s.N + 31) / 32 * s.B > ((int64_t)1 << 31) / 8) return false;
+  return true;
+}
+
+int64_t tiles_per_batch(const pa_shape &s) { return (s.N + 31) / 32; }
+
+int64_t reduce_groups(const pa_shape &s) {
+  const int64_t tpb = tiles_per_batch(s);
+  int64_t g = (1024 + s.B * s.H - 1) / (s.B * s.H);
+  const int64_t cap = (tpb + 7) / 8;
+  if (g > cap) g = cap;
+  return g < 1 ? 1 : g;
+}
+
+int64_t blob_bytes(const pa_shape &s) { return blob_plan((int)s.C, (int)s.S).total_units * 16; }
+int64_t fx_pack_bytes(const pa_shape &s) { return s.B * tiles_per_batch(s) * s.H * 2 * 1024; }
+int64_t w_pack_bytes(const pa_shape &s) { return s.B * tiles_per_batch(s) * s.H * (s.S / 16) * 1024; }
+int64_t tokp_bytes(const pa_shape &s) { return s.B * s.H * (s.S / 16) * 1024; }
+
+int pack_params(const pa_shape &s, const pa_params &p, void *blob, hipStream_t st) {
+  hipLaunchKernelGGL(pack_params_kernel, dim3(64), dim3(256), 0, st, p, static_cast<u32x4 *>(blob), (int)s.C, (int)s.S);
+  return launch_status();
+}
+
+template <int C, int S>
+static int project_softmax_cs(const pa_shape &s, const void *blob, const void *x, void *fx_pack, void *w_pack,
+                              hipStream_t st) {
+  constexpr int KS = C / 16, ST = (S + 31) / 32, H = C / 32;
+  const size_t lds = (size_t)(2 * 2 * KS * 64 + ST * 2 * 64) * 16 + (size_t)(3 * C + ST * 32 + H) * 4;
+  int rc = allow_dynamic_lds(project_softmax_kernel<C, S>, lds);
+  if (rc) return rc;
+  const int64_t tpb = tiles_per_batch(s), total = tpb * s.B;
+  hipLaunchKernelGGL((project_softmax_kernel<C, S>), dim3((unsigned)((total + 7) / 8)), dim3(512), lds, st,
+                     static_cast<const u32x4 *>(blob), static_cast<const uint16_t *>(x), static_cast<u32x4 *>(fx_pack),
+                     static_cast<u32x4 *>(w_pack), s.N, (int)tpb, total);
+  return launch_status();
+}
+
+template <int S>
+static int slice_reduce_s(const pa_shape &s, const void *w_pack, const void *fx_pack, float *partials, hipStream_t st) {
+  constexpr int ST = (S + 31) / 32;
+  const size_t lds = (size_t)4 * ST * 17 * 64 * 4;
+  int rc = allow_dynamic_lds(slice_reduce_kernel<S>, lds);
+  if (rc) return rc;
+  const int64_t tpb = tiles_per_batch(s), G = reduce_groups(s);
+  const int tiles_per_group = (int)((tpb + G - 1) / G);
+  hipLaunchKernelGGL((slice_reduce_kernel<S>), dim3((unsigned)G, (unsigned)(s.B * s.H)), dim3(256), lds, st,
+                     static_cast<const u32x4 *>(w_pack), static_cast<const u32x4 *>(fx_pack), partials, (int)s.B, (int)s.H,
+                     (int)tpb, tiles_per_group);
+  return launch_status();
+}
+
+template <int C, int S>
+static int deslice_project_cs(const pa_shape &s, const void *blob, const void *w_pack, const void *tokp, void *y,
+                              const pa_block_tail *tail, int num_cu, hipStream_t st) {
+  constexpr int H = C / 32, CT = C / 32;
+  const size_t lds = (size_t)CT * H * 2 * 64 * 16;
+  int rc = allow_dynamic_lds(deslice_project_kernel<C, S>, lds);
+  if (rc) return rc;
+  const int64_t tpb = tiles_per_batch(s), total = tpb * s.B;
+  int64_t grid = (total + 3) / 4;
+  if (grid > num_cu) grid = num_cu;
+  hipLaunchKernelGGL((deslice_project_kernel<C, S>), dim3((unsigned)grid), dim3(256), lds, st,
+                     static_cast<const u32x4 *>(blob), static_cast<const u32x4 *>(w_pack),
+                     static_cast<const u32x4 *>(tokp), static_cast<uint16_t *>(y),
+                     static_cast<const uint16_t *>(tail ? tail->residual : nullptr), tail ? tail->ln_gamma : nullptr,
+                     tail ? tail->ln_beta : nullptr, tail ? tail->ln_eps : 0.f,
+                     static_cast<uint16_t *>(tail ? tail->ln_out : nullptr), s.N, (int)tpb, total);
+  return launch_status();
+}
+
+#define PA_DISPATCH_CS(FN, ...)                                     \
+  do {                                                              \
+    if (s.C == 256) {                                               \
+      if (s.S == 16) return FN<256, 16>(__VA_ARGS__);               \
+      if (s.S == 32) return FN<256, 32>(__VA_ARGS__);               \
+      if (s.S == 64) return FN<256, 64>(__VA_ARGS__);               \
+      return FN<256, 128>(__VA_ARGS__);                             \
+    }                                                               \
+    if (s.S == 16) return FN<128, 16>(__VA_ARGS__);                 \
+    if (s.S == 32) return FN<128, 32>(__VA_ARGS__);                 \
+    if (s.S == 64) return FN<128, 64>(__VA_ARGS__);                 \
+    return FN<128, 128>(__VA_ARGS__);                               \
+  } while (0)
+
+int project_softmax(const pa_shape &s, const void *blob, const void *x, void *fx_pack, void *w_pack, hipStream_t st) {
+  PA_DISPATCH_CS(project_softmax_cs, s, blob, x, fx_pack, w_pack, st);
+}
+
+int slice_reduce(const pa_shape &s, const void *w_pack, const void *fx_pack, float *partials, hipStream_t st) {
+  if (s.S == 16) return slice_reduce_s<16>(s, w_pack, fx_pack, partials, st);
+  if (s.S == 32) return slice_reduce_s<32>(s, w_pack, fx_pack, partials, st);
+  if (s.S == 64) return slice_reduce_s<64>(s, w_pack, fx_pack, partials, st);
+  return slice_reduce_s<128>(s, w_pack, fx_pack, partials, st);
+}
+
+int pack_tokens(const pa_shape &s, const float *tok_out, void *tokp, hipStream_t st) {
+  const int64_t units = s.B * s.H * (s.S / 16) * 64;
+  hipLaunchKernelGGL(pack_tokens_kernel, dim3((unsigned)((units + 255) / 256)), dim3(256), 0, st, tok_out,
+                     static_cast<u32x4 *>(tokp), units, (int)s.S);
+  return launch_status();
+}
+
+int deslice_project(const pa_shape &s, const void *blob, const void *w_pack, const void *tokp, void *y,
+                    const pa_block_tail *tail, int num_cu, hipStream_t st) {
+  PA_DISPATCH_CS(deslice_project_cs, s, blob, w_pack, tokp, y, tail, num_cu, st);
+}
+
+}  // namespace mfma
+}  // namespace pa

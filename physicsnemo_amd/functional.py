@@ -137,3 +137,58 @@ def layer_forward(x, params, dims: LayerDims, residual=None, ln_weight=None, ln_
                                     _lib.current_stream_ptr(x.device)), "pa_layer_forward")
     out = y if (residual is None and ln_out is None) else (y, ln_out)
     return (out, tok) if return_slice_tokens else out
+
+
+class MfmaStages:
+    """The bf16 MFMA kernels one by one (pa_mfma_* entry points) with their opaque buffers held as torch tensors.
+
+    Used for per-kernel timing and for checking the MFMA path's slice tokens; `layer_forward` runs the same
+    kernels in one library call.
+    """
+
+    def __init__(self, params: dict, dims: LayerDims, device):
+        lib = _lib.load()
+        self.lib, self.params, self.dims, self.device = lib, params, dims, device
+        self.shape = dims.c()
+        self.cparams = _c_params(params)
+
+        def buf(which):
+            n = lib.pa_mfma_buffer_bytes(byref(self.shape), which)
+            if n < 0:
+                _lib.check(int(n), "pa_mfma_buffer_bytes")
+            return torch.empty(int(n), dtype=torch.uint8, device=device)
+
+        self.blob, self.fx_pack, self.w_pack = buf(_lib.PA_BUF_BLOB), buf(_lib.PA_BUF_FX_PACK), buf(_lib.PA_BUF_W_PACK)
+        self.partials, self.tokp = buf(_lib.PA_BUF_PARTIALS), buf(_lib.PA_BUF_TOKP)
+        f32 = dict(dtype=torch.float32, device=device)
+        self.tok = torch.empty(dims.B, dims.H, dims.S, dims.D, **f32)
+        self.norm = torch.empty(dims.B, dims.H, dims.S, **f32)
+        self.tok_out = torch.empty(dims.B, dims.H, dims.S, dims.D, **f32)
+
+    def _stream(self):
+        return _lib.current_stream_ptr(self.device)
+
+    def pack_params(self):
+        _lib.check(self.lib.pa_mfma_pack_params(byref(self.shape), byref(self.cparams), self.blob.data_ptr(),
+                                                self._stream()), "pa_mfma_pack_params")
+
+    def project_softmax(self, x):
+        _need_cuda(x)
+        _lib.check(self.lib.pa_mfma_project_softmax(byref(self.shape), self.blob.data_ptr(), x.data_ptr(),
+                                                    self.fx_pack.data_ptr(), self.w_pack.data_ptr(), self._stream()),
+                   "pa_mfma_project_softmax")
+
+    def slice_reduce(self):
+        _lib.check(self.lib.pa_mfma_slice_reduce(byref(self.shape), self.w_pack.data_ptr(), self.fx_pack.data_ptr(),
+                                                 self.partials.data_ptr(), self._stream()), "pa_mfma_slice_reduce")
+
+    def combine_attention(self):
+        _lib.check(self.lib.pa_mfma_combine_attention(byref(self.shape), byref(self.cparams), self.partials.data_ptr(),
+                                                      self.tok.data_ptr(), self.norm.data_ptr(), self.tok_out.data_ptr(),
+                                                      self.tokp.data_ptr(), self._stream()), "pa_mfma_combine_attention")
+
+    def deslice_project(self, y, residual=None, ln_weight=None, ln_bias=None, ln_eps=1e-5, ln_out=None):
+        tail = _c_tail(residual, ln_weight, ln_bias, ln_eps, ln_out)
+        _lib.check(self.lib.pa_mfma_deslice_project(byref(self.shape), self.blob.data_ptr(), self.w_pack.data_ptr(),
+                                                    self.tokp.data_ptr(), y.data_ptr(), byref(tail), self._stream()),
+                   "pa_mfma_deslice_project")

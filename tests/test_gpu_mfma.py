@@ -1,0 +1,131 @@
+"""GPU parity of the bf16 MFMA kernels (through the C ABI) against the fp32 CPU oracle.
+
+Bar for bf16: relative L2 error <= 1e-2 against the fp32 oracle (outputs and slice tokens).
+"""
+import pytest
+import torch
+
+from oracle import torch_oracle as to
+import physicsnemo_amd as pn
+from physicsnemo_amd import functional as PF
+from gpu_util import announce, assert_rel_l2, make_pair
+
+pytestmark = pytest.mark.gpu
+
+
+def _run(B, N, C, S, seed=0, sharpen=1.0, temps=None):
+    H = C // 32
+    ref, hip = make_pair("irregular", C, H, 32, S, seed=seed, sharpen=sharpen, temps=temps)
+    x = torch.randn(B, N, C)
+    xb = x.cuda().bfloat16()
+    dims = hip.layer_dims(xb)
+    assert PF.query_path(torch.bfloat16, dims) == 1, "shape must be served by the MFMA kernels"
+    with torch.no_grad():
+        want = ref.stages(xb.float().cpu())  # same bf16-rounded input, fp32 arithmetic
+        y, tok = PF.layer_forward(xb, hip.kernel_params(torch.bfloat16, xb.device), dims, return_slice_tokens=True)
+    return ref, hip, xb, want, y, tok
+
+
+@pytest.mark.parametrize("B,N,C,S", [
+    (1, 4096, 256, 64), (2, 1000, 256, 64), (1, 2048, 256, 16), (1, 2048, 256, 32), (1, 1500, 256, 128),
+    (3, 777, 128, 32), (1, 31, 128, 16), (1, 33, 256, 64), (2, 2048, 128, 128), (1, 4096, 128, 64),
+])
+def test_mfma_layer_matches_fp32_oracle(B, N, C, S):
+    announce("mfma layer", B, N, C, S)
+    _, _, _, want, y, tok = _run(B, N, C, S)
+    assert y.dtype == torch.bfloat16 and y.shape == (B, N, C)
+    assert torch.isfinite(y.float()).all()
+    assert_rel_l2(tok, want["tok"], "slice tokens")
+    assert_rel_l2(y, want["y"], "layer output")
+
+
+def test_mfma_sharp_softmax_and_clamped_temperatures():
+    announce("mfma sharp softmax")
+    temps = [0.1, 0.5, 1.0, 2.0, 5.0, 10.0, 0.7, 3.0]  # 0.1 and 10 exercise both clamps
+    _, _, _, want, y, tok = _run(2, 3000, 256, 64, seed=3, sharpen=4.0, temps=temps)
+    assert_rel_l2(tok, want["tok"], "slice tokens")
+    assert_rel_l2(y, want["y"], "layer output")
+
+
+def test_mfma_stage_entry_points_agree_with_layer_call():
+    announce("mfma stages == layer")
+    B, N, C, S = 2, 1234, 256, 64
+    ref, hip, xb, want, y, tok = _run(B, N, C, S)
+    st = PF.MfmaStages(hip.kernel_params(torch.bfloat16, xb.device), hip.layer_dims(xb), xb.device)
+    y2 = torch.empty_like(y)
+    st.pack_params()
+    st.project_softmax(xb)
+    st.slice_reduce()
+    st.combine_attention()
+    st.deslice_project(y2)
+    assert torch.equal(y2, y)
+    assert torch.equal(st.tok, tok)
+    # norm invariant: sum_s (norm - 0.01) = number of points, up to bf16 rounding of the weights
+    total = (st.norm - 0.01).sum(-1)
+    assert torch.allclose(total, torch.full_like(total, float(N)), rtol=2e-3)
+    assert_rel_l2(st.norm, want["norm"], "slice norm", tol=5e-3)
+    assert_rel_l2(st.tok_out, want["tok_out"], "attended tokens")
+
+
+def test_mfma_block_tail_residual_layernorm():
+    announce("mfma block tail")
+    B, N, C, S = 2, 999, 256, 32
+    ref, hip = make_pair("irregular", C, C // 32, 32, S)
+    ln = torch.nn.LayerNorm(C)
+    with torch.no_grad():
+        ln.weight.add_(0.2 * torch.randn(C))
+        ln.bias.add_(0.2 * torch.randn(C))
+    x, res = torch.randn(B, N, C), torch.randn(B, N, C)
+    xb, rb = x.cuda().bfloat16(), res.cuda().bfloat16()
+    with torch.no_grad():
+        want_fx = ref(xb.float().cpu()) + rb.float().cpu()
+        want_ln = ln(want_fx)
+        fx, normed = hip.forward_block(xb, rb, ln.cuda())
+    assert_rel_l2(fx, want_fx, "fx_new")
+    assert_rel_l2(normed, want_ln, "LayerNorm(fx_new)")
+
+
+def test_mfma_determinism_and_point_permutation():
+    announce("mfma determinism / permutation")
+    B, N, C, S = 1, 8192, 256, 64
+    ref, hip, xb, want, y, tok = _run(B, N, C, S)
+    p = hip.kernel_params(torch.bfloat16, xb.device)
+    dims = hip.layer_dims(xb)
+    with torch.no_grad():
+        for _ in range(3):
+            y2, tok2 = PF.layer_forward(xb, p, dims, return_slice_tokens=True)
+            assert torch.equal(y2, y) and torch.equal(tok2, tok)
+        perm = torch.randperm(N, device=xb.device)
+        y3, tok3 = PF.layer_forward(xb[:, perm].contiguous(), p, dims, return_slice_tokens=True)
+    # slice tokens do not depend on the order of the points (only the summation order changes)
+    assert_rel_l2(tok3, tok, "tokens under a point permutation", tol=1e-4)
+    assert_rel_l2(y3, y[:, perm], "outputs follow the permutation", tol=2e-3)
+
+
+def test_mfma_full_size_properties():
+    # headline shape (1,048,576 points, C=256, S=64): size-independent properties instead of an oracle run
+    announce("mfma full size")
+    B, N, C, S = 1, 1 << 20, 256, 64
+    H = C // 32
+    torch.manual_seed(0)
+    hip = pn.PhysicsAttentionIrregularMesh(C, heads=H, dim_head=32, slice_num=S, use_te=False).eval().cuda()
+    g = torch.Generator().manual_seed(1234)
+    xb = torch.randn(B, N, C, generator=g).bfloat16().cuda()
+    p = hip.kernel_params(torch.bfloat16, xb.device)
+    dims = hip.layer_dims(xb)
+    st = PF.MfmaStages(p, dims, xb.device)
+    y = torch.empty_like(xb)
+    st.pack_params(); st.project_softmax(xb); st.slice_reduce(); st.combine_attention(); st.deslice_project(y)
+    total = (st.norm - 0.01).sum(-1)
+    assert torch.allclose(total, torch.full_like(total, float(N)), rtol=2e-3)
+    assert torch.isfinite(y.float()).all()
+    # a 4096-point prefix run through the oracle with the full run's slice tokens: y = deslice(w, tok') for those points
+    sub = xb[:, :4096].float().cpu()
+    ref = to.OraclePhysicsAttentionIrregularMesh(C, heads=H, dim_head=32, slice_num=S).eval()
+    ref.load_state_dict({k: v.cpu() for k, v in hip.state_dict().items()})
+    with torch.no_grad():
+        xm, _ = ref._project(sub)
+        w, _, _ = to.slice_weights_and_tokens(to.slice_logits(xm, ref.in_project_slice.weight, ref.in_project_slice.bias),
+                                              torch.zeros(1, 4096, H, 32), ref.temperature)
+        want = to.deslice_and_project(w, st.tok_out.cpu(), ref.out_linear.weight, ref.out_linear.bias)
+    assert_rel_l2(y[:, :4096], want, "prefix of the full-size output")
