@@ -1,0 +1,208 @@
+#!/usr/bin/env python3
+"""Benchmark of the PhysicsAttention forward path on one MI355X.
+
+Default workload (the configuration the headline metric is quoted on): one PhysicsAttentionIrregularMesh layer,
+bf16, B=1, N=1,048,576 points, C=256, 8 heads (D=32), slice_num=64, synthetic N(0,1) input (seed 1234),
+seeded random weights (seed 0, orthogonal slice projection).  A "step" is one full layer forward through
+the C ABI (parameter repack + kernels a, b, combine/attention, d), inputs resident in HBM.
+
+Prints ONE JSON line: whole-layer Mpoints/s, the roofline of the dominant kernel (measured live with events on
+the launch stream), per-kernel figures, and the CPU baseline (the oracle's ATen op sequence timed on the host
+cores on a bounded sample of the same workload).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0       # MI355X HBM3E, published
+MFMA_BF16_PEAK_TF = 2500.0  # MI355X dense bf16, published
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--points", type=int, default=1 << 20)
+    ap.add_argument("--batch", type=int, default=1)
+    ap.add_argument("--hidden", type=int, default=256)
+    ap.add_argument("--slices", type=int, default=64)
+    ap.add_argument("--kernel-reps", type=int, default=20, help="launches per kernel for the per-kernel timing")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain 1 GiB device copy (known traffic) so FETCH_SIZE / WRITE_SIZE can be scaled")
+    ap.add_argument("--cpu-seconds", type=float, default=15.0, help="target CPU time of the baseline leg")
+    return ap.parse_args()
+
+
+def algorithmic_bytes_per_point(C, H, S, b=2):
+    """Bytes each kernel must move per point when every tensor is read / written once (bf16)."""
+    return {
+        "project_softmax": (C + C + H * S) * b,   # read x; write fx_mid, w
+        "slice_reduce": (H * S + C) * b,          # read w, fx_mid
+        "deslice_project": (H * S + C) * b,       # read w; write y   (+C*b per extra residual / LayerNorm tensor)
+    }
+
+
+def mfma_flops_per_point(C, S):
+    return {
+        "project_softmax": 4 * C * C + 2 * C * S,  # two projections + slice logits
+        "slice_reduce": 2 * C * S,                 # aggregation
+        "deslice_project": 2 * C * S + 2 * C * C,  # deslice + out_linear
+    }
+
+
+def time_kernel(fn, reps):
+    import torch
+
+    fn()
+    torch.cuda.synchronize()
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    start.record()  # recorded on torch's current stream, the stream the library launches on
+    for _ in range(reps):
+        fn()
+    stop.record()
+    stop.synchronize()
+    return start.elapsed_time(stop) / reps  # ms per launch
+
+
+def cpu_baseline(state_dict, x_cpu_f32, C, H, S, target_seconds):
+    """The oracle (the reference's ATen op sequence) on the host cores, fp32, on a prefix of the same points."""
+    import torch
+
+    from oracle import torch_oracle as to
+
+    ref = to.OraclePhysicsAttentionIrregularMesh(C, heads=H, dim_head=C // H, slice_num=S).eval()
+    ref.load_state_dict(state_dict)
+    threads = torch.get_num_threads()
+    n_total = x_cpu_f32.shape[1]
+    probe = min(16384, n_total)
+    with torch.no_grad():
+        ref(x_cpu_f32[:, :probe])
+        t0 = time.perf_counter()
+        ref(x_cpu_f32[:, :probe])
+        per_point = (time.perf_counter() - t0) / probe
+        # 2 warm-ups + 5 timed runs within the budget
+        n = int(min(n_total, max(probe, target_seconds / 7.0 / per_point)))
+        n = min(n, 262144)
+        xs = x_cpu_f32[:, :n].contiguous()
+        for _ in range(2):
+            ref(xs)
+        times = []
+        for _ in range(5):
+            t0 = time.perf_counter()
+            ref(xs)
+            times.append(time.perf_counter() - t0)
+    med = statistics.median(times)
+    return {
+        "value": round(xs.shape[0] * n / med / 1e6, 4), "unit": "Mpoints/s", "cores": threads, "kind": "port",
+        "sample": f"first {n} of {n_total} points of the same input, fp32, median of 5 runs after 2 warm-ups, "
+                  f"torch {torch.__version__} CPU ATen ops, {threads} threads",
+    }
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU only (got --gpus {args.gpus}): this build has no multi-GPU path; "
+              "run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+    import torch
+
+    import physicsnemo_amd as pn
+    from physicsnemo_amd import functional as PF
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (no CPU path exists for the product)", file=sys.stderr)
+        sys.exit(2)
+    dev = torch.device("cuda:0")
+    B, N, C, S = args.batch, args.points, args.hidden, args.slices
+    H = C // 32
+    torch.manual_seed(0)
+    layer = pn.PhysicsAttentionIrregularMesh(C, heads=H, dim_head=32, slice_num=S, use_te=False).eval()
+    state = {k: v.clone() for k, v in layer.state_dict().items()}
+    layer = layer.to(dev)
+    gen = torch.Generator().manual_seed(1234)
+    x_cpu = torch.randn(B, N, C, generator=gen)
+    x = x_cpu.to(dev).bfloat16().contiguous()
+    dims = layer.layer_dims(x)
+    path = PF.query_path(torch.bfloat16, dims)
+
+    with torch.no_grad():
+        for _ in range(args.warmup):
+            y = layer(x)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            y = layer(x)
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed / args.steps * 1e3
+    mpoints = B * N / (ms_per_step * 1e-3) / 1e6
+    assert torch.isfinite(y[:, :1024].float()).all()
+
+    if args.calibrate_copy:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+
+    kernels = {}
+    roofline = None
+    if path == 1:
+        params = layer.kernel_params(torch.bfloat16, dev)
+        st = PF.MfmaStages(params, dims, dev)
+        yk = torch.empty_like(x)
+        st.pack_params()
+        stage_fns = {
+            "project_softmax": lambda: st.project_softmax(x),
+            "slice_reduce": st.slice_reduce,
+            "combine_attention": st.combine_attention,
+            "deslice_project": lambda: st.deslice_project(yk),
+            "pack_params": st.pack_params,
+        }
+        bytes_pp = algorithmic_bytes_per_point(C, H, S)
+        flops_pp = mfma_flops_per_point(C, S)
+        for name, fn in stage_fns.items():
+            ms = time_kernel(fn, args.kernel_reps)
+            entry = {"ms": round(ms, 4)}
+            if name in bytes_pp:
+                gbs = bytes_pp[name] * B * N / (ms * 1e-3) / 1e9
+                tf = flops_pp[name] * B * N / (ms * 1e-3) / 1e12
+                entry.update({"algorithmic_bytes": bytes_pp[name] * B * N, "hbm_gbs": round(gbs, 1),
+                              "hbm_frac": round(gbs / HBM_PEAK_GBS, 4), "mfma_tflops": round(tf, 1),
+                              "mfma_frac": round(tf / MFMA_BF16_PEAK_TF, 4)})
+            kernels[name] = entry
+        dominant = max(bytes_pp, key=lambda k: kernels[k]["ms"])
+        roofline = {"kernel": dominant, "bound": "hbm", "achieved": kernels[dominant]["hbm_gbs"], "peak": HBM_PEAK_GBS,
+                    "unit": "GB/s", "frac": kernels[dominant]["hbm_frac"], "traffic": None}
+
+    out = {
+        "metric": "Mpoints/s per PhysicsAttention layer at 1M pts bf16; % HBM/MFMA roofline",
+        "value": round(mpoints, 2), "unit": "Mpoints/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "cfg3: single PhysicsAttentionIrregularMesh layer forward", "batch": B, "points": N,
+                   "hidden": C, "heads": H, "dim_head": 32, "slice_num": S,
+                   "kernel_path": "mfma" if path == 1 else "general"},
+        "roofline": roofline, "kernels": kernels,
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(state, x_cpu, C, H, S, args.cpu_seconds)
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -106,7 +106,8 @@ int pa_slice_softmax(int dtype, const pa_shape *shape, const pa_params *p, const
                      void *stream);
 
 /* Stage (b): slice-token aggregation, replaces PA.py:185-203.
- *   partials: float32 scratch of pa_reduce_partial_count(shape) * B*H*S*(D+1) elements
+ *   partials: float32 scratch of pa_reduce_partial_count(shape) * B*H*S*(D+1) elements (per-chunk sums
+ *             plus one slot for their total)
  *   slice_token (B,H,S,D) = (sum_n w fx_mid) / (sum_n w + 1e-2);  slice_norm (B,H,S) = sum_n w + 1e-2.
  * Two passes: per-chunk partial sums, then a fixed-order combine (bit-reproducible, no atomics). */
 int64_t pa_reduce_partial_count(const pa_shape *shape);

@@ -45,7 +45,7 @@ GeneralPlan plan_general(int dtype, const pa_shape &s) {
   p.off_w = off;
   off += round_up(M * s.H * s.S * e, 256);
   p.off_partials = off;
-  off += round_up(p.G * s.B * s.H * s.S * (s.D + 1) * 4, 256);
+  off += round_up((p.G + 1) * s.B * s.H * s.S * (s.D + 1) * 4, 256);  // G partials + their total
   p.off_tok = off;
   off += round_up(s.B * s.H * s.S * s.D * 4, 256);
   p.off_norm = off;
@@ -63,7 +63,7 @@ struct MfmaPlan {
 };
 
 int64_t mfma_partials_bytes(const pa_shape &s) {
-  return pa::mfma::reduce_groups(s) * s.B * s.H * s.S * (s.D + 1) * 4;
+  return (pa::mfma::reduce_groups(s) + 1) * s.B * s.H * s.S * (s.D + 1) * 4;  // G partials + their total
 }
 
 MfmaPlan plan_mfma(const pa_shape &s) {
@@ -169,7 +169,7 @@ int pa_slice_softmax(int dtype, const pa_shape *shape, const pa_params *p, const
 int64_t pa_reduce_partial_count(const pa_shape *shape) {
   int rc = check_shape(PA_F32, shape);
   if (rc) return rc;
-  return pa::general::partial_count(*shape);
+  return pa::general::partial_count(*shape) + 1;  // G partial sums + one slot for their total
 }
 
 int pa_slice_reduce(int dtype, const pa_shape *shape, const void *w, const void *fx_mid, float *partials,

@@ -184,6 +184,7 @@ __global__ __launch_bounds__(256) void slice_softmax_kernel(const T *__restrict_
 // Each thread owns up to 16 outputs of a 4096-output slab and walks the chunk 32 points at a time
 // through LDS.  Sums run in a fixed order, so the result is bit-reproducible.
 // ------------------------------------------------------------------------------------------------
+constexpr int kAttnThreads = 1024;  // slice_combine_attn_kernel: 16 waves, one query row per wave at a time
 constexpr int kSlab = 4096;
 constexpr int kPartialTile = 32;
 
@@ -243,6 +244,31 @@ __global__ __launch_bounds__(256) void slice_partial_kernel(const T *__restrict_
 }
 
 // ------------------------------------------------------------------------------------------------
+// combine_partials_kernel: second pass of the reduction, parallel over outputs.  grid (ceil(n_out/64), B*H);
+// 64 outputs x 4 quarter-ranges of the G partials per workgroup; each thread adds its quarter in index order,
+// the four quarter sums are then added in a fixed order ((q0 + q1) + q2) + q3: bit-reproducible, no atomics.
+// ------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void combine_partials_kernel(const float *__restrict__ partials, int G,
+                                                               int64_t partial_stride, float *__restrict__ combined,
+                                                               int n_out) {
+  __shared__ float quarter[4][64];
+  const int t = threadIdx.x, q = t >> 6, l = t & 63;
+  const int o = blockIdx.x * 64 + l;
+  const int bh = blockIdx.y;
+  const int per = (G + 3) / 4;
+  const int g0 = q * per, g1 = min(G, g0 + per);
+  float acc = 0.f;
+  if (o < n_out) {
+    const float *src = partials + (int64_t)bh * n_out + o;
+    for (int g = g0; g < g1; ++g) acc += src[(int64_t)g * partial_stride];
+  }
+  quarter[q][l] = acc;
+  __syncthreads();
+  if (q == 0 && o < n_out)
+    combined[(int64_t)bh * n_out + o] = ((quarter[0][l] + quarter[1][l]) + quarter[2][l]) + quarter[3][l];
+}
+
+// ------------------------------------------------------------------------------------------------
 // slice_combine_attn_kernel: one workgroup per (b, h), everything after the load stays in LDS.
 //   1. num[s, :], cnt[s] = sum over the G partials in index order
 //   2. tok = num / (cnt + 1e-2)            -> slice_token, slice_norm (optional outputs)
@@ -251,50 +277,55 @@ __global__ __launch_bounds__(256) void slice_partial_kernel(const T *__restrict_
 // `partial_stride` = elements between consecutive partials of the same (b, h).  G == 0: `partials` holds
 // finished tokens (steps 1-2 skipped); out_token == nullptr: stop after step 2.
 // ------------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void slice_combine_attn_kernel(const float *__restrict__ partials, int G,
+__global__ __launch_bounds__(kAttnThreads) void slice_combine_attn_kernel(const float *__restrict__ partials, int G,
                                                                  int64_t partial_stride, const float *__restrict__ w_qkv,
                                                                  float *__restrict__ slice_token,
                                                                  float *__restrict__ slice_norm,
-                                                                 float *__restrict__ out_token, int D, int S) {
+                                                                 float *__restrict__ out_token, int D, int S,
+                                                                 int stage_w) {
   extern __shared__ float lds[];
   const int D1 = D + 1;
   float *tok = lds;              // S * D1 (column D holds the count, then the norm)
   float *q = tok + S * D1;       // S * D1
   float *k = q + S * D1;
   float *v = k + S * D1;
-  float *prow = v + S * D1;      // 4 waves * S
+  float *prow = v + S * D1;      // one row of S per wave
+  float *wq = prow + (kAttnThreads / 64) * S;      // 3D * D1 (only when stage_w)
   const int t = threadIdx.x;
   const int bh = blockIdx.x;
   const int n_out = S * D1;
   if (G > 0) {
     const float *src = partials + (int64_t)bh * n_out;
-    for (int o = t; o < n_out; o += 256) {
+    for (int o = t; o < n_out; o += kAttnThreads) {
       float acc = 0.f;
       for (int g = 0; g < G; ++g) acc += src[(int64_t)g * partial_stride + o];
       tok[o] = acc;
     }
     __syncthreads();
-    for (int s = t; s < S; s += 256) tok[s * D1 + D] += kSliceNormEps;
+    for (int s = t; s < S; s += kAttnThreads) tok[s * D1 + D] += kSliceNormEps;
     __syncthreads();
-    for (int i = t; i < S * D; i += 256) {
+    for (int i = t; i < S * D; i += kAttnThreads) {
       const int s = i / D, d = i - s * D;
       const float val = tok[s * D1 + d] / tok[s * D1 + D];
       tok[s * D1 + d] = val;
       if (slice_token) slice_token[(int64_t)bh * S * D + i] = val;
     }
     if (slice_norm)
-      for (int s = t; s < S; s += 256) slice_norm[(int64_t)bh * S + s] = tok[s * D1 + D];
+      for (int s = t; s < S; s += kAttnThreads) slice_norm[(int64_t)bh * S + s] = tok[s * D1 + D];
   } else {
     // G == 0: `partials` already holds finished slice tokens (B, H, S, D)
-    for (int i = t; i < S * D; i += 256) tok[(i / D) * D1 + (i % D)] = partials[(int64_t)bh * S * D + i];
+    for (int i = t; i < S * D; i += kAttnThreads) tok[(i / D) * D1 + (i % D)] = partials[(int64_t)bh * S * D + i];
   }
   if (!out_token) return;  // reduction-only call (uniform across the workgroup)
+  if (stage_w)
+    for (int i = t; i < 3 * D * D; i += kAttnThreads) wq[(i / D) * D1 + (i % D)] = w_qkv[i];
   __syncthreads();
-  for (int i = t; i < S * 3 * D; i += 256) {
+  for (int i = t; i < S * 3 * D; i += kAttnThreads) {
     const int s = i / (3 * D), e = i - s * 3 * D;
-    const float *wr = w_qkv + (int64_t)e * D;
+    const float *wr = stage_w ? wq + e * D1 : w_qkv + (int64_t)e * D;
     const float *tr = tok + s * D1;
     float acc = 0.f;
+#pragma unroll 8
     for (int d = 0; d < D; ++d) acc = fmaf(tr[d], wr[d], acc);
     float *dst = e < D ? q : (e < 2 * D ? k : v);
     dst[s * D1 + (e % D)] = acc;
@@ -303,12 +334,13 @@ __global__ __launch_bounds__(256) void slice_combine_attn_kernel(const float *__
   const int wave = t >> 6, lane = t & 63;
   const float scale = rsqrtf((float)D);
   float *pr = prow + wave * S;
-  for (int s = wave; s < S; s += 4) {
+  for (int s = wave; s < S; s += kAttnThreads / 64) {
     const float *qs = q + s * D1;
     float mx = -INFINITY;
     for (int u = lane; u < S; u += 64) {
       const float *ku = k + u * D1;
       float acc = 0.f;
+#pragma unroll 8
       for (int e = 0; e < D; ++e) acc = fmaf(qs[e], ku[e], acc);
       acc *= scale;
       pr[u] = acc;
@@ -327,6 +359,7 @@ __global__ __launch_bounds__(256) void slice_combine_attn_kernel(const float *__
     const float inv = 1.f / sum;
     for (int e = lane; e < D; e += 64) {
       float acc = 0.f;
+#pragma unroll 8
       for (int u = 0; u < S; ++u) acc = fmaf(pr[u], v[u * D1 + e], acc);
       out_token[((int64_t)bh * S + s) * D + e] = acc * inv;
     }
@@ -493,7 +526,9 @@ int64_t partial_count(const pa_shape &s) {
   return g < 1 ? 1 : g;
 }
 
-size_t combine_attn_lds_bytes(const pa_shape &s) { return (size_t)(4 * s.S * (s.D + 1) + 4 * s.S) * 4; }
+size_t combine_attn_lds_bytes(const pa_shape &s) {
+  return (size_t)(4 * s.S * (s.D + 1) + (kAttnThreads / 64) * s.S) * 4;
+}
 
 template <typename T>
 static int slice_partial_t(const pa_shape &s, const void *w, const void *fx_mid, float *partials, hipStream_t st) {
@@ -509,14 +544,30 @@ static int slice_partial_t(const pa_shape &s, const void *w, const void *fx_mid,
   return launch_status();
 }
 
+// `partials` holds G partial sums followed by one spare slot (index G) that receives their fixed-order total.
+// G == 0: `partials` holds finished slice tokens (attention only).
 int combine_attention(const pa_shape &s, const pa_params &p, const float *partials, int64_t G, float *slice_token,
                       float *slice_norm, float *out_token, hipStream_t st) {
-  const size_t lds = combine_attn_lds_bytes(s);
+  size_t lds = combine_attn_lds_bytes(s);
+  const size_t wq_bytes = (size_t)3 * s.D * (s.D + 1) * 4;
+  const int stage_w = lds + wq_bytes <= 96 * 1024 ? 1 : 0;  // qkv weight rows in LDS when they fit comfortably
+  if (stage_w) lds += wq_bytes;
   int rc = allow_dynamic_lds(slice_combine_attn_kernel, lds);
   if (rc) return rc;
   const int64_t stride = s.B * s.H * s.S * (s.D + 1);
-  hipLaunchKernelGGL(slice_combine_attn_kernel, dim3((unsigned)(s.B * s.H)), dim3(256), lds, st, partials, (int)G, stride,
-                     p.qkv_project_weight, slice_token, slice_norm, out_token, (int)s.D, (int)s.S);
+  const float *src = partials;
+  int g_attn = (int)G;
+  if (G > 1) {
+    float *combined = const_cast<float *>(partials) + G * stride;
+    const int n_out = (int)(s.S * (s.D + 1));
+    hipLaunchKernelGGL(combine_partials_kernel, dim3((unsigned)((n_out + 63) / 64), (unsigned)(s.B * s.H)), dim3(256), 0,
+                       st, partials, (int)G, stride, combined, n_out);
+    if ((rc = launch_status())) return rc;
+    src = combined;
+    g_attn = 1;
+  }
+  hipLaunchKernelGGL(slice_combine_attn_kernel, dim3((unsigned)(s.B * s.H)), dim3(kAttnThreads), lds, st, src, g_attn, stride,
+                     p.qkv_project_weight, slice_token, slice_norm, out_token, (int)s.D, (int)s.S, stage_w);
   return launch_status();
 }
 

@@ -18,6 +18,8 @@
 //                                  of point i of the tile                       (B operand of the deslice product)
 //   fx_pack[tile][h][kk][lane][8]  fx_mid, lane i <-> channel d = i of head h, element j <-> point kperm(kk, g, j)
 //                                                                                (A operand of the aggregation)
+#include <stdlib.h>
+
 #include "pa_common.h"
 #include "pa_host.h"
 
@@ -51,7 +53,7 @@ __device__ __forceinline__ uint16_t to_bf16_bits(float f) { return __builtin_bit
 // Packed parameter blob (built once per call by pack_params_kernel).  Offsets in 16-byte units.
 //   win [h][m][ks][lane]  m = 0: in_project_x, 1: in_project_fx; W_m[h*32 + i][16ks + 8g + j]
 //   wsl [st][kk][lane]    in_project_slice[32st + i][kperm(kk, g, j)]   (0 beyond S)
-//   wout[ct][h][kk][lane] out_linear[i*CT + ct][h*32 + kperm(kk, g, j)],  CT = C/32
+//   wout[ct][h][kk][lane] out_linear[32ct + i][h*32 + kperm(kk, g, j)],  ct < C/32
 //   then float vectors: bias_x[C], bias_fx[C], bias_slice[ST*32] (-1e30 beyond S), bias_out[C], tscale[H]
 // ------------------------------------------------------------------------------------------------
 struct BlobPlan {
@@ -71,7 +73,7 @@ __host__ __device__ inline BlobPlan blob_plan(int C, int S) {
 }
 
 __global__ __launch_bounds__(256) void pack_params_kernel(pa_params p, u32x4 *__restrict__ blob, int C, int S) {
-  const int H = C / 32, KS = C / 16, ST = (S + 31) / 32, CT = C / 32;
+  const int H = C / 32, KS = C / 16, ST = (S + 31) / 32;
   const BlobPlan bp = blob_plan(C, S);
   const uint16_t *wx = static_cast<const uint16_t *>(p.in_project_x_weight);
   const uint16_t *wfx = static_cast<const uint16_t *>(p.in_project_fx_weight);
@@ -100,7 +102,7 @@ __global__ __launch_bounds__(256) void pack_params_kernel(pa_params p, u32x4 *__
       const int kk = q & 1;
       q >>= 1;
       const int h = q % H, ct = q / H;
-      const uint16_t *src = wo + (int64_t)(i * CT + ct) * C + h * 32;
+      const uint16_t *src = wo + (int64_t)(ct * 32 + i) * C + h * 32;
 #pragma unroll
       for (int j = 0; j < 8; ++j) e[j] = src[kperm(kk, g, j)];
     }
@@ -131,14 +133,15 @@ __global__ __launch_bounds__(256) void pack_params_kernel(pa_params p, u32x4 *__
 // Per-head weights (Wx_h | Wfx_h, 2*KS KiB) are double-buffered in LDS: the next head's 64 bytes per thread
 // are fetched into registers before the current head's products and stored to LDS after them.
 // ------------------------------------------------------------------------------------------------
-template <int C, int S>
-__global__ __launch_bounds__(512) void project_softmax_kernel(const u32x4 *__restrict__ blob, const uint16_t *__restrict__ x,
+template <int C, int S, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void project_softmax_kernel(const u32x4 *__restrict__ blob, const uint16_t *__restrict__ x,
                                                               u32x4 *__restrict__ fx_pack, u32x4 *__restrict__ w_pack,
                                                               int64_t N, int tpb, int64_t total_tiles) {
   constexpr int H = C / 32, KS = C / 16, ST = (S + 31) / 32, NCH = S / 16;
   constexpr int HEAD_UNITS = 2 * KS * 64;  // 16-byte units of one head's weights
-  constexpr int PER_THREAD = HEAD_UNITS / 512;
-  static_assert(HEAD_UNITS % 512 == 0, "head weights must split evenly over the workgroup");
+  constexpr int NT = WAVES * 64;
+  constexpr int PER_THREAD = HEAD_UNITS / NT;
+  static_assert(HEAD_UNITS % NT == 0, "head weights must split evenly over the workgroup");
   extern __shared__ u32x4 smem[];
   u32x4 *wbuf = smem;                       // 2 * HEAD_UNITS
   u32x4 *wsl = wbuf + 2 * HEAD_UNITS;       // ST * 2 * 64
@@ -147,94 +150,136 @@ __global__ __launch_bounds__(512) void project_softmax_kernel(const u32x4 *__res
   const BlobPlan bp = blob_plan(C, S);
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, i = lane & 31, g = lane >> 5;
-  const int64_t tile = (int64_t)blockIdx.x * 8 + wave;
-  const bool tile_ok = tile < total_tiles;
-  const int64_t b = tile_ok ? tile / tpb : 0;
-  const int64_t n = tile_ok ? (tile - b * tpb) * 32 + i : 0;
-  const bool valid = tile_ok && n < N;
+  const int64_t tile_raw = (int64_t)blockIdx.x * WAVES + wave;
+  const bool tile_ok = tile_raw < total_tiles;
+  // waves past the end recompute the last tile (no divergent control flow in the loop) and store nothing
+  const int64_t tile = tile_ok ? tile_raw : total_tiles - 1;
+  const int64_t b = tile / tpb;
+  const int64_t n = (tile - b * tpb) * 32 + i;
+  const bool valid = n < N;
 
   // x fragments of this wave's 32 points (zero rows beyond N)
   u32x4 xf[KS];
   {
-    const u32x4 *xr = reinterpret_cast<const u32x4 *>(x + ((int64_t)b * N + n) * C) + g;
+    const u32x4 *xr = reinterpret_cast<const u32x4 *>(x + ((int64_t)b * N + (valid ? n : 0)) * C) + g;
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) xf[ks] = valid ? xr[2 * ks] : u32x4{0, 0, 0, 0};
+    for (int ks = 0; ks < KS; ++ks) {
+      const u32x4 v = xr[2 * ks];
+      xf[ks] = valid ? v : u32x4{0, 0, 0, 0};
+    }
   }
   // small parameters and the first head's weights
-  for (int u = tid; u < ST * 2 * 64; u += 512) wsl[u] = blob[bp.wsl + u];
+  for (int u = tid; u < ST * 2 * 64; u += NT) wsl[u] = blob[bp.wsl + u];
   {
     const float *src = reinterpret_cast<const float *>(blob + bp.fvec);
-    for (int k = tid; k < 3 * C + ST * 32 + H; k += 512) fvec[k] = src[k];
+    for (int k = tid; k < 3 * C + ST * 32 + H; k += NT) fvec[k] = src[k];
   }
 #pragma unroll
-  for (int q = 0; q < PER_THREAD; ++q) wbuf[q * 512 + tid] = blob[bp.win + q * 512 + tid];
+  for (int q = 0; q < PER_THREAD; ++q) wbuf[q * NT + tid] = blob[bp.win + q * NT + tid];
   __syncthreads();
+  u32x4 wsf[ST][2];  // in_project_slice fragments: the same for every head
+#pragma unroll
+  for (int st = 0; st < ST; ++st) {
+    wsf[st][0] = wsl[(st * 2 + 0) * 64 + lane];
+    wsf[st][1] = wsl[(st * 2 + 1) * 64 + lane];
+  }
 
+  // Order inside one head period (it keeps every vector-memory wait exact):
+  //   issue next head's weight loads -> products + softmax (results held in registers)
+  //   -> next head's weights into the other LDS buffer (waits for those loads only: nothing younger is in flight)
+  //   -> this head's global stores -> barrier
   for (int h = 0; h < H; ++h) {
+    const int hn = h + 1 < H ? h + 1 : h;  // the last period re-fetches its own weights (discarded)
     u32x4 nxt[PER_THREAD];
-    if (h + 1 < H) {
 #pragma unroll
-      for (int q = 0; q < PER_THREAD; ++q) nxt[q] = blob[bp.win + (int64_t)(h + 1) * HEAD_UNITS + q * 512 + tid];
-    }
-    if (tile_ok) {
-      const u32x4 *wb = wbuf + (h & 1) * HEAD_UNITS;
-      f32x16 ax, af;
-      {
-        const float bf = bias_f[h * 32 + i];
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          ax[r] = bias_x[h * 32 + rowmap(r, g)];
-          af[r] = bf;
-        }
-      }
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        const u32x4 a = wb[ks * 64 + lane];
-        const u32x4 bw = wb[(KS + ks) * 64 + lane];
-        ax = mma(a, xf[ks], ax);
-        af = mma(xf[ks], bw, af);
-      }
-      u32x4 *fdst = fx_pack + ((tile * H + h) * 2) * 64 + lane;
-      fdst[0] = pack_half<0>(af);
-      fdst[64] = pack_half<1>(af);
+    for (int q = 0; q < PER_THREAD; ++q) nxt[q] = blob[bp.win + (int64_t)hn * HEAD_UNITS + q * NT + tid];
 
-      const u32x4 xb0 = pack_half<0>(ax), xb1 = pack_half<1>(ax);
-      f32x16 lg[ST];
-      float mx = -INFINITY;
+    const u32x4 *wb = wbuf + (h & 1) * HEAD_UNITS;
+    f32x16 ax, af;
+    {
+      const float bf = bias_f[h * 32 + i];
 #pragma unroll
-      for (int st = 0; st < ST; ++st) {
-#pragma unroll
-        for (int r = 0; r < 16; ++r) lg[st][r] = bias_s[32 * st + rowmap(r, g)];
-        lg[st] = mma(wsl[(st * 2 + 0) * 64 + lane], xb0, lg[st]);
-        lg[st] = mma(wsl[(st * 2 + 1) * 64 + lane], xb1, lg[st]);
-#pragma unroll
-        for (int r = 0; r < 16; ++r) mx = fmaxf(mx, lg[st][r]);
-      }
-      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-      const float sc = tscale[h];
-      const float off = mx * sc;
-      float sum = 0.f;
-#pragma unroll
-      for (int st = 0; st < ST; ++st)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const float e = __builtin_amdgcn_exp2f(fmaf(lg[st][r], sc, -off));
-          lg[st][r] = e;
-          sum += e;
-        }
-      sum += __shfl_xor(sum, 32, 64);
-      const float inv = valid ? __builtin_amdgcn_rcpf(sum) : 0.f;
-      u32x4 *wdst = w_pack + ((tile * H + h) * NCH) * 64 + lane;
-#pragma unroll
-      for (int st = 0; st < ST; ++st) {
-        if (2 * st < NCH) wdst[(2 * st) * 64] = pack_half<0>(lg[st], inv);
-        if (2 * st + 1 < NCH) wdst[(2 * st + 1) * 64] = pack_half<1>(lg[st], inv);
+      for (int r = 0; r < 16; ++r) {
+        ax[r] = bias_x[h * 32 + rowmap(r, g)];
+        af[r] = bf;
       }
     }
-    if (h + 1 < H) {
+    // fragment reads run one group of GRP k-steps ahead of the products that use them
+    constexpr int GRP = 4, NG = KS / GRP;
+    static_assert(KS % GRP == 0, "k-steps must split into groups");
+    u32x4 fa[2][GRP], fb[2][GRP];
+#pragma unroll
+    for (int q = 0; q < GRP; ++q) {
+      fa[0][q] = wb[q * 64 + lane];
+      fb[0][q] = wb[(KS + q) * 64 + lane];
+    }
+    // the scheduling barriers keep the compiler from sinking the reads back next to their uses
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int grp = 0; grp < NG; ++grp) {
+      const int cur = grp & 1;
+      if (grp + 1 < NG) {
+#pragma unroll
+        for (int q = 0; q < GRP; ++q) {
+          fa[cur ^ 1][q] = wb[((grp + 1) * GRP + q) * 64 + lane];
+          fb[cur ^ 1][q] = wb[(KS + (grp + 1) * GRP + q) * 64 + lane];
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int q = 0; q < GRP; ++q) {
+        ax = mma(fa[cur][q], xf[grp * GRP + q], ax);
+        af = mma(xf[grp * GRP + q], fb[cur][q], af);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    const u32x4 fxp0 = pack_half<0>(af), fxp1 = pack_half<1>(af);
+
+    const u32x4 xb0 = pack_half<0>(ax), xb1 = pack_half<1>(ax);
+    f32x16 lg[ST];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int st = 0; st < ST; ++st) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) lg[st][r] = bias_s[32 * st + rowmap(r, g)];
+      lg[st] = mma(wsf[st][0], xb0, lg[st]);
+      lg[st] = mma(wsf[st][1], xb1, lg[st]);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) mx = fmaxf(mx, lg[st][r]);
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float sc = tscale[h];
+    const float off = mx * sc;
+    float sum = 0.f;
+#pragma unroll
+    for (int st = 0; st < ST; ++st)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const float e = __builtin_amdgcn_exp2f(fmaf(lg[st][r], sc, -off));
+        lg[st][r] = e;
+        sum += e;
+      }
+    sum += __shfl_xor(sum, 32, 64);
+    const float inv = valid ? __builtin_amdgcn_rcpf(sum) : 0.f;
+    u32x4 wp[NCH];
+#pragma unroll
+    for (int st = 0; st < ST; ++st) {
+      if (2 * st < NCH) wp[2 * st < NCH ? 2 * st : 0] = pack_half<0>(lg[st], inv);
+      if (2 * st + 1 < NCH) wp[2 * st + 1 < NCH ? 2 * st + 1 : 0] = pack_half<1>(lg[st], inv);
+    }
+
+    {
       u32x4 *dst = wbuf + ((h + 1) & 1) * HEAD_UNITS;
 #pragma unroll
-      for (int q = 0; q < PER_THREAD; ++q) dst[q * 512 + tid] = nxt[q];
+      for (int q = 0; q < PER_THREAD; ++q) dst[q * NT + tid] = nxt[q];
+    }
+    if (tile_ok) {
+      u32x4 *fdst = fx_pack + ((tile * H + h) * 2) * 64 + lane;
+      fdst[0] = fxp0;
+      fdst[64] = fxp1;
+      u32x4 *wdst = w_pack + ((tile * H + h) * NCH) * 64 + lane;
+#pragma unroll
+      for (int cq = 0; cq < NCH; ++cq) wdst[cq * 64] = wp[cq];
     }
     __syncthreads();
   }
@@ -346,156 +391,201 @@ __global__ __launch_bounds__(256) void pack_tokens_kernel(const float *__restric
 }
 
 // ------------------------------------------------------------------------------------------------
-// Kernel (d): deslice + out_linear (+ residual, + LayerNorm).  Persistent: the whole packed out_linear weight
-// (C*C*2 bytes) sits in LDS, so one 4-wave workgroup per CU (one wave per SIMD, up to 512 registers each)
-// loops over tiles; each wave owns a tile at a time.
-//   out_x^T (32 d x 32 pts) = tok'^T_h . w^T_h       A = tokp frags (global, L2 resident), B = w_pack chunks
-//   y (32 pts x C)          = out_x . Wout^T         A = bf16(out_x^T) from registers, B = Wout frags (LDS)
-// Output columns are interleaved over the C/32 accumulator tiles (column of tile ct, lane i = i*CT + ct) so each
-// lane ends up with CT consecutive channels of a row: one 16-byte store per row and lane (C = 256).
+// Kernel (d): deslice + out_linear (+ residual, + LayerNorm).  Persistent workgroups of H waves; one 32-point
+// tile per iteration, worked on by the whole workgroup:
+//   wave h   : out_x^T_h (32 d x 32 pts) = tok'^T_h . w^T_h   A = tokp frags (LDS, per batch), B = w_pack chunks
+//              (global, fetched one tile ahead into registers)  -> bf16 A operands into LDS
+//   wave ct  : y[:, 32ct .. 32ct+31] (32 pts x 32 ch) = out_x . Wout^T    A = out_x frags (LDS), B = its slice of
+//              out_linear, register resident for the whole kernel        -> fp32 tile into LDS
+//   wave r   : rows 32/H*r ..: + residual, rounding, LayerNorm statistics over the full row by a wave reduction,
+//              full-row coalesced stores (C*2 bytes per store instruction).
+// TAIL (compile time): 0 plain, 1 residual + LayerNorm, 2 residual only, 3 LayerNorm only.
+// MASKED = false: the steady-state kernel, full tiles only; its loop body has no branch around a memory
+// operation and issues the next tile's loads right after the last use of the current ones, so every wait
+// counts exactly the younger operations.  MASKED = true: the ragged last tile of each batch (one per workgroup).
 // ------------------------------------------------------------------------------------------------
-template <int C, int S>
-__global__ __launch_bounds__(256) void deslice_project_kernel(const u32x4 *__restrict__ blob, const u32x4 *__restrict__ w_pack,
-                                                              const u32x4 *__restrict__ tokp, uint16_t *__restrict__ y,
-                                                              const uint16_t *__restrict__ residual,
-                                                              const float *__restrict__ ln_gamma,
-                                                              const float *__restrict__ ln_beta, float ln_eps,
-                                                              uint16_t *__restrict__ ln_out, int64_t N, int tpb,
-                                                              int64_t total_tiles) {
-  constexpr int H = C / 32, CT = C / 32, ST = (S + 31) / 32, NCH = S / 16;
-  constexpr int WOUT_UNITS = CT * H * 2 * 64;
-  extern __shared__ u32x4 smem[];
-  u32x4 *wo = smem;  // WOUT_UNITS
+template <int C, int S, int TAIL, bool MASKED>
+__global__ __launch_bounds__(C * 2) void deslice_project_kernel(const u32x4 *__restrict__ blob, const u32x4 *__restrict__ w_pack,
+                                                                const u32x4 *__restrict__ tokp, uint16_t *__restrict__ y,
+                                                                const uint16_t *__restrict__ residual,
+                                                                const float *__restrict__ ln_gamma,
+                                                                const float *__restrict__ ln_beta, float ln_eps,
+                                                                uint16_t *__restrict__ ln_out, int64_t N, int tpb,
+                                                                int nfull, int64_t total_items) {
+  constexpr bool HAS_RES = TAIL == 1 || TAIL == 2, HAS_LN = TAIL == 1 || TAIL == 3;
+  constexpr int H = C / 32, ST = (S + 31) / 32, NCH = S / 16, NT = C * 2;
+  constexpr int ROWS = 32 / H;        // rows of the tile finished by each wave
+  constexpr int CPL = C / 64;         // consecutive channels per lane in the epilogue
+  constexpr int YS = C + 8;           // row stride (floats): rows 4 apart land 32 banks apart
+  typedef uint32_t rowvec __attribute__((ext_vector_type(CPL / 2)));  // CPL bf16
+  __shared__ u32x4 oxs[H * 2 * 64];
+  __shared__ u32x4 tps[H * NCH * 64];
+  __shared__ float ys[32 * YS];
   const BlobPlan bp = blob_plan(C, S);
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, i = lane & 31, g = lane >> 5;
-  for (int u = tid; u < WOUT_UNITS; u += 256) wo[u] = blob[bp.wout + u];
-  float bout[CT], gam[CT], bet[CT];
-  {
-    const float *fv = reinterpret_cast<const float *>(blob + bp.fvec) + 2 * C + ST * 32;
+
+  u32x4 wout[H][2];
 #pragma unroll
-    for (int ct = 0; ct < CT; ++ct) {
-      bout[ct] = fv[i * CT + ct];
-      gam[ct] = ln_out ? ln_gamma[i * CT + ct] : 1.f;
-      bet[ct] = ln_out ? ln_beta[i * CT + ct] : 0.f;
+  for (int h = 0; h < H; ++h) {
+    wout[h][0] = blob[bp.wout + ((wave * H + h) * 2 + 0) * 64 + lane];
+    wout[h][1] = blob[bp.wout + ((wave * H + h) * 2 + 1) * 64 + lane];
+  }
+  const float *fv = reinterpret_cast<const float *>(blob + bp.fvec) + 2 * C + ST * 32;
+  const float bias = fv[wave * 32 + i];
+  float gam[CPL], bet[CPL];
+#pragma unroll
+  for (int k = 0; k < CPL; ++k) {
+    gam[k] = HAS_LN ? ln_gamma[lane * CPL + k] : 1.f;
+    bet[k] = HAS_LN ? ln_beta[lane * CPL + k] : 0.f;
+  }
+
+  // item -> (batch, tile-in-batch): full tiles for the steady-state kernel, the last (ragged) tile otherwise
+  int64_t item = blockIdx.x;
+  int64_t b = MASKED ? item : item / nfull;
+  int64_t t = MASKED ? (int64_t)tpb - 1 : item - b * nfull;
+  u32x4 wcur[NCH];
+  rowvec rcur[ROWS];
+  {
+    const u32x4 *wsrc = w_pack + (((b * tpb + t) * H + wave) * NCH) * 64 + lane;
+#pragma unroll
+    for (int cq = 0; cq < NCH; ++cq) wcur[cq] = wsrc[cq * 64];
+    if constexpr (HAS_RES) {
+#pragma unroll
+      for (int rr = 0; rr < ROWS; ++rr) {
+        int64_t n = t * 32 + wave * ROWS + rr;
+        if (MASKED && n >= N) n = N - 1;
+        rcur[rr] = *reinterpret_cast<const rowvec *>(residual + (b * N + n) * C + lane * CPL);
+      }
     }
   }
-  __syncthreads();
-
-  for (int64_t tile = (int64_t)blockIdx.x * 4 + wave; tile < total_tiles; tile += (int64_t)gridDim.x * 4) {
-    const int64_t b = tile / tpb;
-    const int64_t n0 = (tile - b * tpb) * 32;
-    // deslice every head; keep bf16(out_x^T) as A operands of the projection
-    u32x4 oxf[H][2];
+  if constexpr (!MASKED) {
+    // Placeholder stores to this wave's first output rows (overwritten by the real results below).  They put the
+    // loop entry in the same state as the loop back-edge -- prefetch loads followed by one epilogue's worth of
+    // stores -- so the wait before the first use of wcur allows exactly those younger stores to stay in flight
+    // instead of draining the memory pipeline every iteration.
+    rowvec zero;
 #pragma unroll
-    for (int h = 0; h < H; ++h) {
-      const u32x4 *wsrc = w_pack + ((tile * H + h) * NCH) * 64 + lane;
-      const u32x4 *tsrc = tokp + (((int64_t)b * H + h) * NCH) * 64 + lane;
-      f32x16 ox;
+    for (int k = 0; k < CPL / 2; ++k) zero[k] = 0u;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) ox[r] = 0.f;
-#pragma unroll
-      for (int cq = 0; cq < NCH; ++cq) ox = mma(tsrc[cq * 64], wsrc[cq * 64], ox);
-      oxf[h][0] = pack_half<0>(ox);
-      oxf[h][1] = pack_half<1>(ox);
+    for (int rr = 0; rr < ROWS; ++rr) {
+      const int64_t off = (b * N + t * 32 + wave * ROWS + rr) * C + lane * CPL;
+      *reinterpret_cast<rowvec *>(y + off) = zero;
+      if constexpr (HAS_LN) *reinterpret_cast<rowvec *>(ln_out + off) = zero;
     }
-    f32x16 acc[CT];
+  }
+  int64_t b_loaded = -1;
+  while (true) {
+    if (b != b_loaded) {  // workgroup-uniform: (re)load this batch's attended tokens
+      __syncthreads();
+      for (int u = tid; u < H * NCH * 64; u += NT) tps[u] = tokp[b * (H * NCH * 64) + u];
+      __syncthreads();
+      b_loaded = b;
+    }
+    const int64_t n0 = t * 32;
+    // deslice this wave's head (last use of wcur)
+    f32x16 ox;
 #pragma unroll
-    for (int ct = 0; ct < CT; ++ct) {
+    for (int r = 0; r < 16; ++r) ox[r] = 0.f;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) acc[ct][r] = bout[ct];
+    for (int cq = 0; cq < NCH; ++cq) ox = mma(tps[(wave * NCH + cq) * 64 + lane], wcur[cq], ox);
+    // fetch the next item's slice weights and residual rows (the last iteration re-fetches its own)
+    const int64_t item_next = item + gridDim.x;
+    const bool more = !MASKED && item_next < total_items;
+    const int64_t itn = more ? item_next : item;
+    const int64_t bn = MASKED ? b : itn / nfull;
+    const int64_t tn = MASKED ? t : itn - bn * nfull;
+    u32x4 wnext[NCH];
+    rowvec rnext[ROWS];
+    {
+      const u32x4 *wsrc = w_pack + (((bn * tpb + tn) * H + wave) * NCH) * 64 + lane;
 #pragma unroll
-      for (int h = 0; h < H; ++h) {
-        acc[ct] = mma(oxf[h][0], wo[((ct * H + h) * 2 + 0) * 64 + lane], acc[ct]);
-        acc[ct] = mma(oxf[h][1], wo[((ct * H + h) * 2 + 1) * 64 + lane], acc[ct]);
+      for (int cq = 0; cq < NCH; ++cq) wnext[cq] = wsrc[cq * 64];
+      if constexpr (HAS_RES && !MASKED) {
+#pragma unroll
+        for (int rr = 0; rr < ROWS; ++rr)
+          rnext[rr] = *reinterpret_cast<const rowvec *>(residual + (bn * N + tn * 32 + wave * ROWS + rr) * C + lane * CPL);
       }
     }
-    // epilogue: row = point, this lane holds channels i*CT .. i*CT+CT-1
+    oxs[(wave * 2 + 0) * 64 + lane] = pack_half<0>(ox);
+    oxs[(wave * 2 + 1) * 64 + lane] = pack_half<1>(ox);
+    __syncthreads();
+    // this wave's 32 output channels
+    f32x16 acc;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int64_t n = n0 + rowmap(r, g);
-      const bool ok = n < N;
-      const int64_t off = ((int64_t)b * N + n) * C + i * CT;
-      float v[CT];
+    for (int r = 0; r < 16; ++r) acc[r] = bias;
 #pragma unroll
-      for (int ct = 0; ct < CT; ++ct) v[ct] = acc[ct][r];
-      if (residual) {
-        // y is rounded to bf16 before the residual is added, and the sum rounded again (two tensor ops upstream)
-        uint16_t rs[CT];
-        if (ok) {
-          if constexpr (CT == 8) {
-            const u32x4 q = *reinterpret_cast<const u32x4 *>(residual + off);
+    for (int hh = 0; hh < H; hh += 4) {
+      u32x4 of[4][2];
 #pragma unroll
-            for (int k = 0; k < 4; ++k) {
-              rs[2 * k] = (uint16_t)(q[k] & 0xffffu);
-              rs[2 * k + 1] = (uint16_t)(q[k] >> 16);
-            }
-          } else {
-            const u32x2 q = *reinterpret_cast<const u32x2 *>(residual + off);
+      for (int q = 0; q < 4; ++q) {
+        of[q][0] = oxs[((hh + q) * 2 + 0) * 64 + lane];
+        of[q][1] = oxs[((hh + q) * 2 + 1) * 64 + lane];
+      }
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int k = 0; k < 2; ++k) {
-              rs[2 * k] = (uint16_t)(q[k] & 0xffffu);
-              rs[2 * k + 1] = (uint16_t)(q[k] >> 16);
-            }
-          }
-        } else {
+      for (int q = 0; q < 4; ++q) {
+        acc = mma(of[q][0], wout[hh + q][0], acc);
+        acc = mma(of[q][1], wout[hh + q][1], acc);
+      }
+    }
 #pragma unroll
-          for (int ct = 0; ct < CT; ++ct) rs[ct] = 0;
+    for (int r = 0; r < 16; ++r) ys[rowmap(r, g) * YS + wave * 32 + i] = acc[r];
+    __syncthreads();
+    // finish ROWS full rows per wave
+#pragma unroll
+    for (int rr = 0; rr < ROWS; ++rr) {
+      const int row = wave * ROWS + rr;
+      const int64_t n = n0 + row;
+      const bool ok = !MASKED || n < N;
+      const int64_t off = (b * N + n) * C + lane * CPL;
+      float v[CPL];
+      rowvec ob;
+#pragma unroll
+      for (int k = 0; k < CPL; k += 2) {
+        float t0 = ys[row * YS + lane * CPL + k], t1 = ys[row * YS + lane * CPL + k + 1];
+        if constexpr (HAS_RES) {
+          // y is rounded to bf16 first, then the sum is rounded (two tensor ops upstream)
+          const uint32_t rv = rcur[rr][k / 2];
+          t0 = (float)(__bf16)t0 + bf16_bits_to_f32((uint16_t)(rv & 0xffffu));
+          t1 = (float)(__bf16)t1 + bf16_bits_to_f32((uint16_t)(rv >> 16));
         }
-#pragma unroll
-        for (int ct = 0; ct < CT; ++ct) v[ct] = (float)(__bf16)v[ct] + bf16_bits_to_f32(rs[ct]);
+        const uint16_t o0 = to_bf16_bits(t0), o1 = to_bf16_bits(t1);
+        v[k] = bf16_bits_to_f32(o0);
+        v[k + 1] = bf16_bits_to_f32(o1);
+        ob[k / 2] = (uint32_t)o0 | ((uint32_t)o1 << 16);
       }
-      uint16_t ob[CT];
-#pragma unroll
-      for (int ct = 0; ct < CT; ++ct) {
-        ob[ct] = to_bf16_bits(v[ct]);
-        v[ct] = bf16_bits_to_f32(ob[ct]);
-      }
-      if (ok) {
-        if constexpr (CT == 8) {
-          u32x4 q;
-#pragma unroll
-          for (int k = 0; k < 4; ++k) q[k] = (uint32_t)ob[2 * k] | ((uint32_t)ob[2 * k + 1] << 16);
-          *reinterpret_cast<u32x4 *>(y + off) = q;
-        } else {
-          u32x2 q;
-#pragma unroll
-          for (int k = 0; k < 2; ++k) q[k] = (uint32_t)ob[2 * k] | ((uint32_t)ob[2 * k + 1] << 16);
-          *reinterpret_cast<u32x2 *>(y + off) = q;
-        }
-      }
-      if (ln_out) {
+      if (ok) *reinterpret_cast<rowvec *>(y + off) = ob;
+      if constexpr (HAS_LN) {
         float s1 = 0.f;
 #pragma unroll
-        for (int ct = 0; ct < CT; ++ct) s1 += v[ct];
-#pragma unroll
-        for (int o = 16; o > 0; o >>= 1) s1 += __shfl_xor(s1, o, 64);
-        const float mean = s1 * (1.f / C);
+        for (int k = 0; k < CPL; ++k) s1 += v[k];
+        const float mean = wave_sum(s1) * (1.f / C);
         float s2 = 0.f;
 #pragma unroll
-        for (int ct = 0; ct < CT; ++ct) {
-          const float dl = v[ct] - mean;
+        for (int k = 0; k < CPL; ++k) {
+          const float dl = v[k] - mean;
           s2 = fmaf(dl, dl, s2);
         }
+        const float rstd = rsqrtf(wave_sum(s2) * (1.f / C) + ln_eps);
+        rowvec lb;
 #pragma unroll
-        for (int o = 16; o > 0; o >>= 1) s2 += __shfl_xor(s2, o, 64);
-        const float rstd = rsqrtf(s2 * (1.f / C) + ln_eps);
-        uint16_t lb[CT];
-#pragma unroll
-        for (int ct = 0; ct < CT; ++ct) lb[ct] = to_bf16_bits((v[ct] - mean) * rstd * gam[ct] + bet[ct]);
-        if (ok) {
-          if constexpr (CT == 8) {
-            u32x4 q;
-#pragma unroll
-            for (int k = 0; k < 4; ++k) q[k] = (uint32_t)lb[2 * k] | ((uint32_t)lb[2 * k + 1] << 16);
-            *reinterpret_cast<u32x4 *>(ln_out + off) = q;
-          } else {
-            u32x2 q;
-#pragma unroll
-            for (int k = 0; k < 2; ++k) q[k] = (uint32_t)lb[2 * k] | ((uint32_t)lb[2 * k + 1] << 16);
-            *reinterpret_cast<u32x2 *>(ln_out + off) = q;
-          }
+        for (int k = 0; k < CPL; k += 2) {
+          const uint16_t l0 = to_bf16_bits((v[k] - mean) * rstd * gam[k] + bet[k]);
+          const uint16_t l1 = to_bf16_bits((v[k + 1] - mean) * rstd * gam[k + 1] + bet[k + 1]);
+          lb[k / 2] = (uint32_t)l0 | ((uint32_t)l1 << 16);
         }
+        if (ok) *reinterpret_cast<rowvec *>(ln_out + off) = lb;
       }
+    }
+    if (!more) break;
+    item = itn;
+    b = bn;
+    t = tn;
+#pragma unroll
+    for (int cq = 0; cq < NCH; ++cq) wcur[cq] = wnext[cq];
+    if constexpr (HAS_RES) {
+#pragma unroll
+      for (int rr = 0; rr < ROWS; ++rr) rcur[rr] = rnext[rr];
     }
   }
 }
@@ -547,18 +637,29 @@ int pack_params(const pa_shape &s, const pa_params &p, void *blob, hipStream_t s
   return launch_status();
 }
 
+template <int C, int S, int WAVES>
+static int project_softmax_w(const pa_shape &s, const void *blob, const void *x, void *fx_pack, void *w_pack,
+                             hipStream_t st) {
+  constexpr int KS = C / 16, ST = (S + 31) / 32, H = C / 32;
+  const size_t lds = (size_t)(2 * 2 * KS * 64 + ST * 2 * 64) * 16 + (size_t)(3 * C + ST * 32 + H) * 4;
+  int rc = allow_dynamic_lds(project_softmax_kernel<C, S, WAVES>, lds);
+  if (rc) return rc;
+  const int64_t tpb = tiles_per_batch(s), total = tpb * s.B;
+  hipLaunchKernelGGL((project_softmax_kernel<C, S, WAVES>), dim3((unsigned)((total + WAVES - 1) / WAVES)), dim3(WAVES * 64),
+                     lds, st, static_cast<const u32x4 *>(blob), static_cast<const uint16_t *>(x),
+                     static_cast<u32x4 *>(fx_pack), static_cast<u32x4 *>(w_pack), s.N, (int)tpb, total);
+  return launch_status();
+}
+
 template <int C, int S>
 static int project_softmax_cs(const pa_shape &s, const void *blob, const void *x, void *fx_pack, void *w_pack,
                               hipStream_t st) {
-  constexpr int KS = C / 16, ST = (S + 31) / 32, H = C / 32;
-  const size_t lds = (size_t)(2 * 2 * KS * 64 + ST * 2 * 64) * 16 + (size_t)(3 * C + ST * 32 + H) * 4;
-  int rc = allow_dynamic_lds(project_softmax_kernel<C, S>, lds);
-  if (rc) return rc;
-  const int64_t tpb = tiles_per_batch(s), total = tpb * s.B;
-  hipLaunchKernelGGL((project_softmax_kernel<C, S>), dim3((unsigned)((total + 7) / 8)), dim3(512), lds, st,
-                     static_cast<const u32x4 *>(blob), static_cast<const uint16_t *>(x), static_cast<u32x4 *>(fx_pack),
-                     static_cast<u32x4 *>(w_pack), s.N, (int)tpb, total);
-  return launch_status();
+  static const int waves = [] {
+    const char *e = getenv("PA_KA_WAVES");
+    return e ? atoi(e) : 8;
+  }();
+  if (waves == 4) return project_softmax_w<C, S, 4>(s, blob, x, fx_pack, w_pack, st);
+  return project_softmax_w<C, S, 8>(s, blob, x, fx_pack, w_pack, st);
 }
 
 template <int S>
@@ -575,23 +676,51 @@ static int slice_reduce_s(const pa_shape &s, const void *w_pack, const void *fx_
   return launch_status();
 }
 
+template <int C, int S, int TAIL>
+static int deslice_project_t(const pa_shape &s, const void *blob, const void *w_pack, const void *tokp, void *y,
+                             const pa_block_tail *tail, int num_cu, hipStream_t st) {
+  const int64_t tpb = tiles_per_batch(s);
+  const int nfull = (int)(s.N / 32);
+  const u32x4 *bl = static_cast<const u32x4 *>(blob), *wp = static_cast<const u32x4 *>(w_pack),
+              *tp = static_cast<const u32x4 *>(tokp);
+  uint16_t *yo = static_cast<uint16_t *>(y);
+  const uint16_t *res = static_cast<const uint16_t *>(tail ? tail->residual : nullptr);
+  const float *gm = tail ? tail->ln_gamma : nullptr, *bt = tail ? tail->ln_beta : nullptr;
+  const float eps = tail ? tail->ln_eps : 0.f;
+  uint16_t *lo = static_cast<uint16_t *>(tail ? tail->ln_out : nullptr);
+  if (nfull > 0) {
+    static int per_cu = 0;  // resident workgroups per CU for this instantiation
+    if (per_cu == 0) {
+      int nb = 0;
+      if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, deslice_project_kernel<C, S, TAIL, false>, C * 2, 0) !=
+              hipSuccess || nb < 1)
+        nb = 1;
+      per_cu = nb;
+    }
+    const int64_t total = (int64_t)nfull * s.B;
+    int64_t grid = (int64_t)num_cu * per_cu;
+    if (grid > total) grid = total;
+    hipLaunchKernelGGL((deslice_project_kernel<C, S, TAIL, false>), dim3((unsigned)grid), dim3(C * 2), 0, st, bl, wp, tp,
+                       yo, res, gm, bt, eps, lo, s.N, (int)tpb, nfull, total);
+    int rc = launch_status();
+    if (rc) return rc;
+  }
+  if (s.N % 32 != 0) {
+    hipLaunchKernelGGL((deslice_project_kernel<C, S, TAIL, true>), dim3((unsigned)s.B), dim3(C * 2), 0, st, bl, wp, tp, yo,
+                       res, gm, bt, eps, lo, s.N, (int)tpb, nfull, s.B);
+    return launch_status();
+  }
+  return PA_OK;
+}
+
 template <int C, int S>
 static int deslice_project_cs(const pa_shape &s, const void *blob, const void *w_pack, const void *tokp, void *y,
                               const pa_block_tail *tail, int num_cu, hipStream_t st) {
-  constexpr int H = C / 32, CT = C / 32;
-  const size_t lds = (size_t)CT * H * 2 * 64 * 16;
-  int rc = allow_dynamic_lds(deslice_project_kernel<C, S>, lds);
-  if (rc) return rc;
-  const int64_t tpb = tiles_per_batch(s), total = tpb * s.B;
-  int64_t grid = (total + 3) / 4;
-  if (grid > num_cu) grid = num_cu;
-  hipLaunchKernelGGL((deslice_project_kernel<C, S>), dim3((unsigned)grid), dim3(256), lds, st,
-                     static_cast<const u32x4 *>(blob), static_cast<const u32x4 *>(w_pack),
-                     static_cast<const u32x4 *>(tokp), static_cast<uint16_t *>(y),
-                     static_cast<const uint16_t *>(tail ? tail->residual : nullptr), tail ? tail->ln_gamma : nullptr,
-                     tail ? tail->ln_beta : nullptr, tail ? tail->ln_eps : 0.f,
-                     static_cast<uint16_t *>(tail ? tail->ln_out : nullptr), s.N, (int)tpb, total);
-  return launch_status();
+  const bool has_res = tail && tail->residual, has_ln = tail && tail->ln_out;
+  if (has_res && has_ln) return deslice_project_t<C, S, 1>(s, blob, w_pack, tokp, y, tail, num_cu, st);
+  if (has_res) return deslice_project_t<C, S, 2>(s, blob, w_pack, tokp, y, tail, num_cu, st);
+  if (has_ln) return deslice_project_t<C, S, 3>(s, blob, w_pack, tokp, y, tail, num_cu, st);
+  return deslice_project_t<C, S, 0>(s, blob, w_pack, tokp, y, tail, num_cu, st);
 }
 
 #define PA_DISPATCH_CS(FN, ...)                                     \
