@@ -130,8 +130,8 @@ __global__ __launch_bounds__(256) void pack_params_kernel(pa_params p, u32x4 *__
 //   fx_mid  (32 pts x 32 d)  = x . Wfx_h^T         A = x frags,          B = Wfx_h frags (LDS)   -> fx_pack
 //   logits^T(32 s x 32 pts)  = Wslice . x_mid^T    A = Wslice frags (LDS), B = bf16(x_mid^T) straight from registers
 //   softmax over s: in-lane over the accumulator registers plus one exchange with lane^32          -> w_pack
-// Per-head weights (Wx_h | Wfx_h, 2*KS KiB) are double-buffered in LDS: the next head's 64 bytes per thread
-// are fetched into registers before the current head's products and stored to LDS after them.
+// Per-head weights (Wx_h | Wfx_h, 2*KS KiB) are double-buffered in LDS: the next head's bytes are fetched into
+// registers before the current head's work and stored to LDS after it.
 // ------------------------------------------------------------------------------------------------
 template <int C, int S, int WAVES>
 __global__ __launch_bounds__(WAVES * 64) void project_softmax_kernel(const u32x4 *__restrict__ blob, const uint16_t *__restrict__ x,
@@ -184,16 +184,9 @@ __global__ __launch_bounds__(WAVES * 64) void project_softmax_kernel(const u32x4
     wsf[st][1] = wsl[(st * 2 + 1) * 64 + lane];
   }
 
-  // Order inside one head period (it keeps every vector-memory wait exact):
-  //   issue next head's weight loads -> products + softmax (results held in registers)
-  //   -> next head's weights into the other LDS buffer (waits for those loads only: nothing younger is in flight)
-  //   -> this head's global stores -> barrier
-  for (int h = 0; h < H; ++h) {
-    const int hn = h + 1 < H ? h + 1 : h;  // the last period re-fetches its own weights (discarded)
-    u32x4 nxt[PER_THREAD];
-#pragma unroll
-    for (int q = 0; q < PER_THREAD; ++q) nxt[q] = blob[bp.win + (int64_t)hn * HEAD_UNITS + q * NT + tid];
-
+  // ---- the two halves of one head's work -------------------------------------------------------------------
+  // products(h): both projections and the slice logits (MFMA bound)
+  auto products = [&](int h, u32x4 &fxp0, u32x4 &fxp1, f32x16(&lg)[ST]) {
     const u32x4 *wb = wbuf + (h & 1) * HEAD_UNITS;
     f32x16 ax, af;
     {
@@ -205,7 +198,7 @@ __global__ __launch_bounds__(WAVES * 64) void project_softmax_kernel(const u32x4
       }
     }
     // fragment reads run one group of GRP k-steps ahead of the products that use them
-    constexpr int GRP = 4, NG = KS / GRP;
+    constexpr int GRP = 2, NG = KS / GRP;
     static_assert(KS % GRP == 0, "k-steps must split into groups");
     u32x4 fa[2][GRP], fb[2][GRP];
 #pragma unroll
@@ -233,20 +226,24 @@ __global__ __launch_bounds__(WAVES * 64) void project_softmax_kernel(const u32x4
       }
       __builtin_amdgcn_sched_barrier(0);
     }
-    const u32x4 fxp0 = pack_half<0>(af), fxp1 = pack_half<1>(af);
-
+    fxp0 = pack_half<0>(af);
+    fxp1 = pack_half<1>(af);
     const u32x4 xb0 = pack_half<0>(ax), xb1 = pack_half<1>(ax);
-    f32x16 lg[ST];
-    float mx = -INFINITY;
 #pragma unroll
     for (int st = 0; st < ST; ++st) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) lg[st][r] = bias_s[32 * st + rowmap(r, g)];
       lg[st] = mma(wsf[st][0], xb0, lg[st]);
       lg[st] = mma(wsf[st][1], xb1, lg[st]);
+    }
+  };
+  // softmax(h): temperature softmax over the slices of each point (VALU bound); packs the weights
+  auto softmax = [&](int h, f32x16(&lg)[ST], u32x4(&wp)[NCH]) {
+    float mx = -INFINITY;
+#pragma unroll
+    for (int st = 0; st < ST; ++st)
 #pragma unroll
       for (int r = 0; r < 16; ++r) mx = fmaxf(mx, lg[st][r]);
-    }
     mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
     const float sc = tscale[h];
     const float off = mx * sc;
@@ -261,27 +258,75 @@ __global__ __launch_bounds__(WAVES * 64) void project_softmax_kernel(const u32x4
       }
     sum += __shfl_xor(sum, 32, 64);
     const float inv = valid ? __builtin_amdgcn_rcpf(sum) : 0.f;
-    u32x4 wp[NCH];
 #pragma unroll
     for (int st = 0; st < ST; ++st) {
       if (2 * st < NCH) wp[2 * st < NCH ? 2 * st : 0] = pack_half<0>(lg[st], inv);
       if (2 * st + 1 < NCH) wp[2 * st + 1 < NCH ? 2 * st + 1 : 0] = pack_half<1>(lg[st], inv);
     }
+  };
 
+  // ---- H + 1 periods, one barrier each ----------------------------------------------------------------------
+  // The lower half of the waves runs products(p) then softmax(p); the upper half runs softmax(p-1) then products(p).
+  //
+  // Memory-operation order (vector-memory waits complete in issue order, so this order is what keeps the waits
+  // short): the weights of head p+1 are loaded into registers during period p-1, BEFORE that period's global
+  // stores; in period p they are copied to the free LDS buffer.  The wait in front of that copy therefore only
+  // covers loads that are older than every store still in flight, and the stores of w / fx_mid drain in the
+  // background.  Two register sets alternate, so the loop advances two periods per trip.  Every store is issued
+  // unconditionally (periods without a new result re-store the previous one; waves past the end re-store the last
+  // tile with identical values), which keeps the loop body free of branches around memory operations.
+  const bool late = wave >= WAVES / 2;
+  f32x16 lg[ST];
+  u32x4 fxp0 = {0, 0, 0, 0}, fxp1 = {0, 0, 0, 0}, wp[NCH];
+#pragma unroll
+  for (int cq = 0; cq < NCH; ++cq) wp[cq] = u32x4{0, 0, 0, 0};
+  u32x4 nA[PER_THREAD], nB[PER_THREAD];
+  {
+    const int h1 = H > 1 ? 1 : 0;
+#pragma unroll
+    for (int q = 0; q < PER_THREAD; ++q) nA[q] = blob[bp.win + (int64_t)h1 * HEAD_UNITS + q * NT + tid];
+    // placeholder stores (overwritten by period 0 / 1): give the loop entry the same pending-store state as the
+    // loop back-edge so that the first wait of the loop is as short as all the others
+    u32x4 *fdst = fx_pack + ((tile * H + 0) * 2) * 64 + lane;
+    fdst[0] = fxp0;
+    fdst[64] = fxp1;
+    u32x4 *wdst = w_pack + ((tile * H + 0) * NCH) * 64 + lane;
+#pragma unroll
+    for (int cq = 0; cq < NCH; ++cq) wdst[cq * 64] = wp[cq];
+  }
+  auto period = [&](int p, u32x4(&n_ready)[PER_THREAD], u32x4(&n_load)[PER_THREAD]) {
+    int h_w;
+    if (!late) {
+      if (p < H) {
+        products(p, fxp0, fxp1, lg);
+        softmax(p, lg, wp);
+      }
+      h_w = p < H ? p : H - 1;
+    } else {
+      if (p > 0) softmax(p - 1, lg, wp);
+      if (p < H) products(p, fxp0, fxp1, lg);
+      h_w = p > 0 ? p - 1 : 0;
+    }
+    const int h_f = p < H ? p : H - 1;
     {
-      u32x4 *dst = wbuf + ((h + 1) & 1) * HEAD_UNITS;
+      u32x4 *dst = wbuf + ((p + 1) & 1) * HEAD_UNITS;
 #pragma unroll
-      for (int q = 0; q < PER_THREAD; ++q) dst[q * NT + tid] = nxt[q];
+      for (int q = 0; q < PER_THREAD; ++q) dst[q * NT + tid] = n_ready[q];
     }
-    if (tile_ok) {
-      u32x4 *fdst = fx_pack + ((tile * H + h) * 2) * 64 + lane;
-      fdst[0] = fxp0;
-      fdst[64] = fxp1;
-      u32x4 *wdst = w_pack + ((tile * H + h) * NCH) * 64 + lane;
+    const int h2 = p + 2 < H ? p + 2 : H - 1;
 #pragma unroll
-      for (int cq = 0; cq < NCH; ++cq) wdst[cq * 64] = wp[cq];
-    }
+    for (int q = 0; q < PER_THREAD; ++q) n_load[q] = blob[bp.win + (int64_t)h2 * HEAD_UNITS + q * NT + tid];
+    u32x4 *fdst = fx_pack + ((tile * H + h_f) * 2) * 64 + lane;
+    fdst[0] = fxp0;
+    fdst[64] = fxp1;
+    u32x4 *wdst = w_pack + ((tile * H + h_w) * NCH) * 64 + lane;
+#pragma unroll
+    for (int cq = 0; cq < NCH; ++cq) wdst[cq * 64] = wp[cq];
     __syncthreads();
+  };
+  for (int p = 0; p <= H; p += 2) {
+    period(p, nA, nB);
+    if (p + 1 <= H) period(p + 1, nB, nA);
   }
 }
 
