@@ -247,7 +247,7 @@ int pa_mfma_project_softmax(const pa_shape *shape, const void *blob, const void 
   if (rc) return rc;
   if (!blob || !x || !fx_pack || !w_pack) return PA_ERR_NULL;
   if (!aligned16(blob) || !aligned16(x) || !aligned16(fx_pack) || !aligned16(w_pack)) return PA_ERR_ALIGN;
-  return pa::mfma::project_softmax(*shape, blob, x, fx_pack, w_pack, static_cast<hipStream_t>(stream));
+  return pa::mfma::project_softmax(*shape, blob, x, fx_pack, w_pack, compute_units(), static_cast<hipStream_t>(stream));
 }
 
 int pa_mfma_slice_reduce(const pa_shape *shape, const void *w_pack, const void *fx_pack, float *partials, void *stream) {
@@ -304,7 +304,7 @@ int pa_layer_forward(int dtype, const pa_shape *shape, const pa_params *p, const
     float *norm = reinterpret_cast<float *>(ws + mp.off_norm);
     float *tok_out = reinterpret_cast<float *>(ws + mp.off_tok_out);
     if ((rc = pa::mfma::pack_params(s, *p, blob, st))) return rc;
-    if ((rc = pa::mfma::project_softmax(s, blob, x, fxp, wp, st))) return rc;
+    if ((rc = pa::mfma::project_softmax(s, blob, x, fxp, wp, compute_units(), st))) return rc;
     if ((rc = pa::mfma::slice_reduce(s, wp, fxp, partials, st))) return rc;
     if ((rc = pa::general::combine_attention(s, *p, partials, mp.G, tok, norm, tok_out, st))) return rc;
     if ((rc = pa::mfma::pack_tokens(s, tok_out, tokp, st))) return rc;

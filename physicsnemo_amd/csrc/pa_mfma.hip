@@ -125,7 +125,7 @@ __global__ __launch_bounds__(256) void pack_params_kernel(pa_params p, u32x4 *__
 }
 
 // ------------------------------------------------------------------------------------------------
-// Kernel (a): projections + slice logits + temperature softmax.   512 threads = 8 waves = 8 tiles.
+// Kernel (a): projections + slice logits + temperature softmax.   Persistent, 8 waves = 8 tiles per set.
 //   x_mid^T (32 ch x 32 pts) = Wx_h . x^T          A = Wx_h frags (LDS), B = x frags (registers, loaded once)
 //   fx_mid  (32 pts x 32 d)  = x . Wfx_h^T         A = x frags,          B = Wfx_h frags (LDS)   -> fx_pack
 //   logits^T(32 s x 32 pts)  = Wslice . x_mid^T    A = Wslice frags (LDS), B = bf16(x_mid^T) straight from registers
@@ -150,24 +150,28 @@ __global__ __launch_bounds__(WAVES * 64) void project_softmax_kernel(const u32x4
   const BlobPlan bp = blob_plan(C, S);
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, i = lane & 31, g = lane >> 5;
-  const int64_t tile_raw = (int64_t)blockIdx.x * WAVES + wave;
-  const bool tile_ok = tile_raw < total_tiles;
-  // waves past the end recompute the last tile (no divergent control flow in the loop) and store nothing
-  const int64_t tile = tile_ok ? tile_raw : total_tiles - 1;
-  const int64_t b = tile / tpb;
-  const int64_t n = (tile - b * tpb) * 32 + i;
-  const bool valid = n < N;
-
-  // x fragments of this wave's 32 points (zero rows beyond N)
+  // Persistent workgroup: tile sets blockIdx.x, blockIdx.x + gridDim.x, ...; a set is WAVES consecutive tiles.
+  // Waves past the last tile recompute it (identical values, identical stores): no divergent control flow.
+  const int64_t nsets = (total_tiles + WAVES - 1) / WAVES;
+  const int64_t nloc = (nsets - blockIdx.x + gridDim.x - 1) / gridDim.x;  // sets of this workgroup (>= 1)
+  int64_t set_cur = blockIdx.x, tile = 0, tile_nxt;
+  bool valid = false, valid_nxt;
   u32x4 xf[KS];
-  {
-    const u32x4 *xr = reinterpret_cast<const u32x4 *>(x + ((int64_t)b * N + (valid ? n : 0)) * C) + g;
+  // x fragments of the wave's 32 points of tile set `set` (zero rows beyond N) -> xf, tile_nxt, valid_nxt
+  auto load_x = [&](int64_t set) {
+    const int64_t traw = set * WAVES + wave;
+    tile_nxt = traw < total_tiles ? traw : total_tiles - 1;
+    const int64_t b = tile_nxt / tpb;
+    const int64_t n = (tile_nxt - b * tpb) * 32 + i;
+    valid_nxt = n < N;
+    const u32x4 *xr = reinterpret_cast<const u32x4 *>(x + ((int64_t)b * N + (valid_nxt ? n : 0)) * C) + g;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       const u32x4 v = xr[2 * ks];
-      xf[ks] = valid ? v : u32x4{0, 0, 0, 0};
+      xf[ks] = valid_nxt ? v : u32x4{0, 0, 0, 0};
     }
-  }
+  };
+  load_x(set_cur);
   // small parameters and the first head's weights
   for (int u = tid; u < ST * 2 * 64; u += NT) wsl[u] = blob[bp.wsl + u];
   {
@@ -186,8 +190,8 @@ __global__ __launch_bounds__(WAVES * 64) void project_softmax_kernel(const u32x4
 
   // ---- the two halves of one head's work -------------------------------------------------------------------
   // products(h): both projections and the slice logits (MFMA bound)
-  auto products = [&](int h, u32x4 &fxp0, u32x4 &fxp1, f32x16(&lg)[ST]) {
-    const u32x4 *wb = wbuf + (h & 1) * HEAD_UNITS;
+  auto products = [&](int buf, int h, u32x4 &fxp0, u32x4 &fxp1, f32x16(&lg)[ST]) {
+    const u32x4 *wb = wbuf + buf * HEAD_UNITS;
     f32x16 ax, af;
     {
       const float bf = bias_f[h * 32 + i];
@@ -265,16 +269,18 @@ __global__ __launch_bounds__(WAVES * 64) void project_softmax_kernel(const u32x4
     }
   };
 
-  // ---- H + 1 periods, one barrier each ----------------------------------------------------------------------
+  // ---- H + 1 periods per tile set, one barrier each ------------------------------------------------------------
   // The lower half of the waves runs products(p) then softmax(p); the upper half runs softmax(p-1) then products(p).
   //
   // Memory-operation order (vector-memory waits complete in issue order, so this order is what keeps the waits
-  // short): the weights of head p+1 are loaded into registers during period p-1, BEFORE that period's global
-  // stores; in period p they are copied to the free LDS buffer.  The wait in front of that copy therefore only
-  // covers loads that are older than every store still in flight, and the stores of w / fx_mid drain in the
-  // background.  Two register sets alternate, so the loop advances two periods per trip.  Every store is issued
-  // unconditionally (periods without a new result re-store the previous one; waves past the end re-store the last
-  // tile with identical values), which keeps the loop body free of branches around memory operations.
+  // short): the weights of the head needed two periods later are loaded into registers AFTER the copy of the
+  // previously loaded set into the free LDS buffer and BEFORE this period's global stores.  The wait in front of
+  // that copy therefore never covers the stores of the period before, and the stores of w / fx_mid drain in the
+  // background.  Two register sets alternate, so the loop advances two periods per trip.  The x fragments of the
+  // next tile set are fetched in period H-1, right after their last use, and land during period H.  Every store
+  // is issued unconditionally (periods without a new result re-store the previous one), which keeps the loop
+  // body free of branches around stores.
+  constexpr int P = H + 1;
   const bool late = wave >= WAVES / 2;
   f32x16 lg[ST];
   u32x4 fxp0 = {0, 0, 0, 0}, fxp1 = {0, 0, 0, 0}, wp[NCH];
@@ -285,48 +291,64 @@ __global__ __launch_bounds__(WAVES * 64) void project_softmax_kernel(const u32x4
     const int h1 = H > 1 ? 1 : 0;
 #pragma unroll
     for (int q = 0; q < PER_THREAD; ++q) nA[q] = blob[bp.win + (int64_t)h1 * HEAD_UNITS + q * NT + tid];
-    // placeholder stores (overwritten by period 0 / 1): give the loop entry the same pending-store state as the
+    // placeholder stores (overwritten by periods 0 / 1): give the loop entry the same pending-store state as the
     // loop back-edge so that the first wait of the loop is as short as all the others
-    u32x4 *fdst = fx_pack + ((tile * H + 0) * 2) * 64 + lane;
+    u32x4 *fdst = fx_pack + ((tile_nxt * H + 0) * 2) * 64 + lane;
     fdst[0] = fxp0;
     fdst[64] = fxp1;
-    u32x4 *wdst = w_pack + ((tile * H + 0) * NCH) * 64 + lane;
+    u32x4 *wdst = w_pack + ((tile_nxt * H + 0) * NCH) * 64 + lane;
 #pragma unroll
     for (int cq = 0; cq < NCH; ++cq) wdst[cq * 64] = wp[cq];
   }
-  auto period = [&](int p, u32x4(&n_ready)[PER_THREAD], u32x4(&n_load)[PER_THREAD]) {
+  // head whose weights period q needs (period H of a set has no products; it keeps the last head's)
+  auto head_of = [&](int64_t q) {
+    const int p = (int)(q % P);
+    return p < H ? p : H - 1;
+  };
+  auto period = [&](int64_t q, u32x4(&n_ready)[PER_THREAD], u32x4(&n_load)[PER_THREAD]) {
+    const int p = (int)(q % P);
+    if (p == 0) {  // a new tile set starts: its x fragments were issued in period H-1 of the previous one
+      tile = tile_nxt;
+      valid = valid_nxt;
+    }
     int h_w;
     if (!late) {
       if (p < H) {
-        products(p, fxp0, fxp1, lg);
+        products((int)(q & 1), p, fxp0, fxp1, lg);
         softmax(p, lg, wp);
       }
       h_w = p < H ? p : H - 1;
     } else {
       if (p > 0) softmax(p - 1, lg, wp);
-      if (p < H) products(p, fxp0, fxp1, lg);
+      if (p < H) products((int)(q & 1), p, fxp0, fxp1, lg);
       h_w = p > 0 ? p - 1 : 0;
     }
     const int h_f = p < H ? p : H - 1;
     {
-      u32x4 *dst = wbuf + ((p + 1) & 1) * HEAD_UNITS;
+      u32x4 *dst = wbuf + ((q + 1) & 1) * HEAD_UNITS;
 #pragma unroll
-      for (int q = 0; q < PER_THREAD; ++q) dst[q * NT + tid] = n_ready[q];
+      for (int k = 0; k < PER_THREAD; ++k) dst[k * NT + tid] = n_ready[k];
     }
-    const int h2 = p + 2 < H ? p + 2 : H - 1;
+    const int h2 = head_of(q + 2);
 #pragma unroll
-    for (int q = 0; q < PER_THREAD; ++q) n_load[q] = blob[bp.win + (int64_t)h2 * HEAD_UNITS + q * NT + tid];
+    for (int k = 0; k < PER_THREAD; ++k) n_load[k] = blob[bp.win + (int64_t)h2 * HEAD_UNITS + k * NT + tid];
     u32x4 *fdst = fx_pack + ((tile * H + h_f) * 2) * 64 + lane;
     fdst[0] = fxp0;
     fdst[64] = fxp1;
     u32x4 *wdst = w_pack + ((tile * H + h_w) * NCH) * 64 + lane;
 #pragma unroll
     for (int cq = 0; cq < NCH; ++cq) wdst[cq * 64] = wp[cq];
+    if (p == H - 1) {  // last use of xf is behind us: fetch the next set's (the last set re-fetches its own)
+      const int64_t set_next = set_cur + gridDim.x < nsets ? set_cur + gridDim.x : set_cur;
+      load_x(set_next);
+      set_cur = set_next;
+    }
     __syncthreads();
   };
-  for (int p = 0; p <= H; p += 2) {
-    period(p, nA, nB);
-    if (p + 1 <= H) period(p + 1, nB, nA);
+  const int64_t Q = nloc * P;
+  for (int64_t q = 0; q < Q; q += 2) {
+    period(q, nA, nB);
+    if (q + 1 < Q) period(q + 1, nB, nA);
   }
 }
 
@@ -684,13 +706,15 @@ int pack_params(const pa_shape &s, const pa_params &p, void *blob, hipStream_t s
 
 template <int C, int S, int WAVES>
 static int project_softmax_w(const pa_shape &s, const void *blob, const void *x, void *fx_pack, void *w_pack,
-                             hipStream_t st) {
+                             int num_cu, hipStream_t st) {
   constexpr int KS = C / 16, ST = (S + 31) / 32, H = C / 32;
   const size_t lds = (size_t)(2 * 2 * KS * 64 + ST * 2 * 64) * 16 + (size_t)(3 * C + ST * 32 + H) * 4;
   int rc = allow_dynamic_lds(project_softmax_kernel<C, S, WAVES>, lds);
   if (rc) return rc;
   const int64_t tpb = tiles_per_batch(s), total = tpb * s.B;
-  hipLaunchKernelGGL((project_softmax_kernel<C, S, WAVES>), dim3((unsigned)((total + WAVES - 1) / WAVES)), dim3(WAVES * 64),
+  int64_t grid = (total + WAVES - 1) / WAVES;
+  if (grid > num_cu) grid = num_cu;  // one persistent workgroup per CU
+  hipLaunchKernelGGL((project_softmax_kernel<C, S, WAVES>), dim3((unsigned)grid), dim3(WAVES * 64),
                      lds, st, static_cast<const u32x4 *>(blob), static_cast<const uint16_t *>(x),
                      static_cast<u32x4 *>(fx_pack), static_cast<u32x4 *>(w_pack), s.N, (int)tpb, total);
   return launch_status();
@@ -698,13 +722,8 @@ static int project_softmax_w(const pa_shape &s, const void *blob, const void *x,
 
 template <int C, int S>
 static int project_softmax_cs(const pa_shape &s, const void *blob, const void *x, void *fx_pack, void *w_pack,
-                              hipStream_t st) {
-  static const int waves = [] {
-    const char *e = getenv("PA_KA_WAVES");
-    return e ? atoi(e) : 8;
-  }();
-  if (waves == 4) return project_softmax_w<C, S, 4>(s, blob, x, fx_pack, w_pack, st);
-  return project_softmax_w<C, S, 8>(s, blob, x, fx_pack, w_pack, st);
+                              int num_cu, hipStream_t st) {
+  return project_softmax_w<C, S, 8>(s, blob, x, fx_pack, w_pack, num_cu, st);
 }
 
 template <int S>
@@ -782,8 +801,9 @@ static int deslice_project_cs(const pa_shape &s, const void *blob, const void *w
     return FN<128, 128>(__VA_ARGS__);                               \
   } while (0)
 
-int project_softmax(const pa_shape &s, const void *blob, const void *x, void *fx_pack, void *w_pack, hipStream_t st) {
-  PA_DISPATCH_CS(project_softmax_cs, s, blob, x, fx_pack, w_pack, st);
+int project_softmax(const pa_shape &s, const void *blob, const void *x, void *fx_pack, void *w_pack, int num_cu,
+                    hipStream_t st) {
+  PA_DISPATCH_CS(project_softmax_cs, s, blob, x, fx_pack, w_pack, num_cu, st);
 }
 
 int slice_reduce(const pa_shape &s, const void *w_pack, const void *fx_pack, float *partials, hipStream_t st) {
