@@ -38,6 +38,7 @@ def parse_args():
     ap.add_argument("--slices", type=int, default=64)
     ap.add_argument("--kernel-reps", type=int, default=20, help="launches per kernel for the per-kernel timing")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-models", action="store_true", help="skip the per-full-model throughput lines")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy (known traffic) so FETCH_SIZE / WRITE_SIZE can be scaled")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="target CPU time of the baseline leg")
@@ -109,6 +110,38 @@ def cpu_baseline(state_dict, x_cpu_f32, C, H, S, target_seconds):
         "sample": f"first {n} of {n_total} points of the same input, fp32, median of 5 runs after 2 warm-ups, "
                   f"torch {torch.__version__} CPU ATen ops, {threads} threads",
     }
+
+
+def time_full_model(name, B, N, functional_dim, embedding_dim, slice_num, n_layers, steps=5, warmup=2):
+    """Forward of a whole Transolver (bf16 autocast, random-init weights, synthetic N(0,1) inputs) -> Mpoints/s.
+
+    The PhysicsAttention layers, their residual adds and the LayerNorms that follow run in the HIP library; the
+    remaining glue (first LayerNorm, MLPs, output head) is PyTorch-ROCm.
+    """
+    import torch
+
+    import physicsnemo_amd as pn
+
+    torch.manual_seed(0)
+    model = pn.Transolver(functional_dim=functional_dim, embedding_dim=embedding_dim, out_dim=4, n_layers=n_layers,
+                          n_hidden=256, n_head=8, slice_num=slice_num, use_te=False).eval().cuda()
+    g = torch.Generator().manual_seed(1234)
+    fx = torch.randn(B, N, functional_dim, generator=g).cuda()
+    emb = torch.randn(B, N, embedding_dim, generator=g).cuda()
+    with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
+        for _ in range(warmup):
+            out = model(fx, emb)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            out = model(fx, emb)
+        torch.cuda.synchronize()
+        dt = (time.perf_counter() - t0) / steps
+    assert torch.isfinite(out.float()).all()
+    del model, fx, emb, out
+    torch.cuda.empty_cache()
+    return {"workload": name, "batch": B, "points": N, "layers": n_layers, "slice_num": slice_num,
+            "ms_per_forward": round(dt * 1e3, 3), "mpoints_per_s": round(B * N / dt / 1e6, 2)}
 
 
 def main():
@@ -205,6 +238,11 @@ def main():
                    "kernel_path": "mfma" if path == 1 else "general"},
         "roofline": roofline, "kernels": kernels,
     }
+    if not args.no_models:
+        out["full_model"] = [
+            time_full_model("cfg2: Transolver irregular 2D, 8 layers", 8, 32768, 3, 2, 64, 8),
+            time_full_model("cfg4: Transolver 3D surface cloud, 8 layers", 1, 1000000, 1, 6, 32, 8),
+        ]
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(state, x_cpu, C, H, S, args.cpu_seconds)
     print(json.dumps(out), flush=True)

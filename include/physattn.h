@@ -12,7 +12,8 @@
  *     contiguous row-major (last index fastest) in the shapes stated.
  *   - Symbols: B batch, N points per batch, C = layer width `dim`, H heads, D dim_head, S slice_num.
  *   - `dtype` selects the ACTIVATION element type (x, intermediates, y) and the element type of the
- *     three large weights (in_project_x, in_project_fx, out_linear): PA_F32 or PA_BF16.
+ *     three large weights (in_project_x, in_project_fx, out_linear): PA_F32 or PA_BF16; PA_BF16_W8 = bf16
+ *     activations with fp8-e4m3 large weights (see below).
  *     Small parameters are ALWAYS float32: every bias, temperature (H), in_project_slice weight (S,D)
  *     and bias (S), qkv_project weight (3D,D), LayerNorm gamma/beta.
  *     Slice tokens, slice norms and reduction partials are ALWAYS float32.
@@ -34,6 +35,10 @@ extern "C" {
 
 #define PA_F32 0
 #define PA_BF16 1
+/* bf16 activations; the three large weights are fp8 e4m3 (OCP "fn": bias 7, no infinities, 0x7f/0xff = NaN) bytes
+ * with one float32 scale per OUTPUT channel: W[o, :] = scale[o] * decode(byte[o, :]).  Irregular variant only.
+ * No reference counterpart (the reference's only fp8 is Transformer Engine delayed scaling). */
+#define PA_BF16_W8 2
 
 #define PA_OK 0
 #define PA_ERR_NULL (-1)        /* a required pointer is NULL */
@@ -73,6 +78,10 @@ typedef struct pa_params {
   const float *qkv_project_weight;   /* (3D, D), rows [q | k | v], no bias (PA.py:309,450) */
   const void *out_linear_weight;     /* dtype, (C, H*D) */
   const float *out_linear_bias;      /* (C) */
+  /* PA_BF16_W8 only (NULL otherwise): per-output-channel scales of the fp8 weights */
+  const float *in_project_x_scale;   /* (H*D) */
+  const float *in_project_fx_scale;  /* (H*D) */
+  const float *out_linear_scale;     /* (C) */
 } pa_params;
 
 /* Optional fused tail of the caller TransolverBlock.forward (TR.py:300-303):

@@ -13,7 +13,7 @@ import torch  # noqa: F401  (must be imported first: its HIP runtime is the one 
 
 LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libphysattn.so")
 
-PA_F32, PA_BF16 = 0, 1
+PA_F32, PA_BF16, PA_BF16_W8 = 0, 1, 2
 
 EXPORTED = [
     "pa_version", "pa_status_string", "pa_workspace_bytes", "pa_query_path", "pa_project_inputs",
@@ -33,7 +33,7 @@ class PaParams(Structure):
     _fields_ = [(n, c_void_p) for n in (
         "in_project_x_weight", "in_project_x_bias", "in_project_fx_weight", "in_project_fx_bias",
         "in_project_slice_weight", "in_project_slice_bias", "temperature", "qkv_project_weight",
-        "out_linear_weight", "out_linear_bias")]
+        "out_linear_weight", "out_linear_bias", "in_project_x_scale", "in_project_fx_scale", "out_linear_scale")]
 
 
 class PaBlockTail(Structure):

@@ -8,7 +8,8 @@ using pa::aligned16;
 
 int check_shape(int dtype, const pa_shape *s) {
   if (!s) return PA_ERR_NULL;
-  if (dtype != PA_F32 && dtype != PA_BF16) return PA_ERR_UNSUPPORTED;
+  if (dtype != PA_F32 && dtype != PA_BF16 && dtype != PA_BF16_W8) return PA_ERR_UNSUPPORTED;
+  if (dtype == PA_BF16_W8 && s->conv_k != 0) return PA_ERR_UNSUPPORTED;
   if (s->B <= 0 || s->N <= 0 || s->C <= 0 || s->H <= 0 || s->D <= 0 || s->S <= 0) return PA_ERR_DIMS;
   if (s->conv_k < 0) return PA_ERR_DIMS;
   if (s->conv_k > 0) {
@@ -26,6 +27,11 @@ int check_shape(int dtype, const pa_shape *s) {
 int64_t round_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
 
 int64_t elem_bytes(int dtype) { return dtype == PA_F32 ? 4 : 2; }
+
+// bf16 copies of the three fp8 weights (PA_BF16_W8), placed at the end of the workspace
+int64_t dequant_bytes(int dtype, const pa_shape &s) {
+  return dtype == PA_BF16_W8 ? 3 * round_up(s.H * s.D * s.C * 2, 256) : 0;
+}
 
 // Workspace plan of the general path.
 struct GeneralPlan {
@@ -138,20 +144,23 @@ const char *pa_status_string(int code) {
 int pa_query_path(int dtype, const pa_shape *shape) {
   int rc = check_shape(dtype, shape);
   if (rc) return rc;
-  return pa::mfma::supported(dtype, *shape) ? 1 : 0;
+  return pa::mfma::supported(dtype == PA_BF16_W8 ? PA_BF16 : dtype, *shape) ? 1 : 0;
 }
 
 int64_t pa_workspace_bytes(int dtype, const pa_shape *shape) {
   int rc = check_shape(dtype, shape);
   if (rc) return rc;
-  if (pa::mfma::supported(dtype, *shape)) return plan_mfma(*shape).total;
-  return plan_general(dtype, *shape).total;
+  const int act = dtype == PA_BF16_W8 ? PA_BF16 : dtype;
+  const int64_t extra = dequant_bytes(dtype, *shape);
+  if (pa::mfma::supported(act, *shape)) return plan_mfma(*shape).total + extra;
+  return plan_general(act, *shape).total + extra;
 }
 
 int pa_project_inputs(int dtype, const pa_shape *shape, const pa_params *p, const void *x, void *x_mid, void *fx_mid,
                       void *stream) {
   int rc = check_shape(dtype, shape);
   if (rc) return rc;
+  if (dtype == PA_BF16_W8) return PA_ERR_UNSUPPORTED;  // fp8 weights: whole-layer entry point only
   if ((rc = check_params(p))) return rc;
   if (!x || !x_mid || !fx_mid) return PA_ERR_NULL;
   if (!aligned16(x) || !aligned16(x_mid) || !aligned16(fx_mid)) return PA_ERR_ALIGN;
@@ -161,6 +170,7 @@ int pa_project_inputs(int dtype, const pa_shape *shape, const pa_params *p, cons
 int pa_slice_softmax(int dtype, const pa_shape *shape, const pa_params *p, const void *x_mid, void *w, void *stream) {
   int rc = check_shape(dtype, shape);
   if (rc) return rc;
+  if (dtype == PA_BF16_W8) return PA_ERR_UNSUPPORTED;  // fp8 weights: whole-layer entry point only
   if (!p || !p->in_project_slice_weight || !p->in_project_slice_bias || !p->temperature || !x_mid || !w) return PA_ERR_NULL;
   if (!aligned16(x_mid) || !aligned16(w)) return PA_ERR_ALIGN;
   return pa::general::slice_softmax(dtype, *shape, *p, x_mid, w, static_cast<hipStream_t>(stream));
@@ -176,6 +186,7 @@ int pa_slice_reduce(int dtype, const pa_shape *shape, const void *w, const void 
                     float *slice_token, float *slice_norm, void *stream) {
   int rc = check_shape(dtype, shape);
   if (rc) return rc;
+  if (dtype == PA_BF16_W8) return PA_ERR_UNSUPPORTED;  // fp8 weights: whole-layer entry point only
   if (!w || !fx_mid || !partials || !slice_token || !slice_norm) return PA_ERR_NULL;
   if (!aligned16(w) || !aligned16(fx_mid) || !aligned16(partials)) return PA_ERR_ALIGN;
   hipStream_t st = static_cast<hipStream_t>(stream);
@@ -202,6 +213,7 @@ int pa_deslice_project(int dtype, const pa_shape *shape, const pa_params *p, con
                        void *scratch, void *y, const pa_block_tail *tail, void *stream) {
   int rc = check_shape(dtype, shape);
   if (rc) return rc;
+  if (dtype == PA_BF16_W8) return PA_ERR_UNSUPPORTED;  // fp8 weights: whole-layer entry point only
   if (!p || !p->out_linear_weight || !p->out_linear_bias || !w || !out_slice_token || !scratch || !y) return PA_ERR_NULL;
   if (!aligned16(w) || !aligned16(scratch) || !aligned16(y) || !aligned16(p->out_linear_weight)) return PA_ERR_ALIGN;
   if ((rc = check_tail(tail))) return rc;
@@ -295,6 +307,25 @@ int pa_layer_forward(int dtype, const pa_shape *shape, const pa_params *p, const
   hipStream_t st = static_cast<hipStream_t>(stream);
 
   char *ws = static_cast<char *>(workspace);
+  pa_params deq;  // PA_BF16_W8: parameters with the fp8 weights expanded to bf16 in the workspace tail
+  if (dtype == PA_BF16_W8) {
+    if (!p->in_project_x_scale || !p->in_project_fx_scale || !p->out_linear_scale) return PA_ERR_NULL;
+    const int64_t body = pa::mfma::supported(PA_BF16, s) ? plan_mfma(s).total : plan_general(PA_BF16, s).total;
+    const int64_t one = round_up(s.H * s.D * s.C * 2, 256);
+    if (workspace_bytes < body + 3 * one) return PA_ERR_WORKSPACE;
+    char *w0 = ws + body;
+    deq = *p;
+    if ((rc = pa::general::dequant_e4m3(p->in_project_x_weight, p->in_project_x_scale, w0, s.H * s.D, s.C, st))) return rc;
+    if ((rc = pa::general::dequant_e4m3(p->in_project_fx_weight, p->in_project_fx_scale, w0 + one, s.H * s.D, s.C, st)))
+      return rc;
+    if ((rc = pa::general::dequant_e4m3(p->out_linear_weight, p->out_linear_scale, w0 + 2 * one, s.C, s.H * s.D, st)))
+      return rc;
+    deq.in_project_x_weight = w0;
+    deq.in_project_fx_weight = w0 + one;
+    deq.out_linear_weight = w0 + 2 * one;
+    p = &deq;
+    dtype = PA_BF16;
+  }
   if (pa::mfma::supported(dtype, s)) {
     const MfmaPlan mp = plan_mfma(s);
     if (workspace_bytes < mp.total) return PA_ERR_WORKSPACE;

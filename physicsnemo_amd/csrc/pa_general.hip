@@ -435,6 +435,26 @@ __global__ __launch_bounds__(256) void residual_ln_kernel(T *__restrict__ y, con
   }
 }
 
+// ------------------------------------------------------------------------------------------------
+// dequant_e4m3_kernel: out[o, k] = bf16(scale[o] * decode_e4m3fn(in[o, k])).  e4m3fn: 1 sign, 4 exponent (bias 7),
+// 3 mantissa bits; exponent 0 is subnormal (2^-6 * m/8); 0x7f / 0xff are NaN; there are no infinities.
+// ------------------------------------------------------------------------------------------------
+__device__ __forceinline__ float decode_e4m3fn(uint8_t v) {
+  const int e = (v >> 3) & 15, m = v & 7;
+  float mag;
+  if (e == 15 && m == 7) mag = __uint_as_float(0x7fc00000u);
+  else if (e == 0) mag = (float)m * 0.001953125f;                      // m/8 * 2^-6
+  else mag = __uint_as_float((uint32_t)(e + 120) << 23 | (uint32_t)m << 20);  // 2^(e-7) * (1 + m/8)
+  return (v & 0x80) ? -mag : mag;
+}
+
+__global__ __launch_bounds__(256) void dequant_e4m3_kernel(const uint8_t *__restrict__ in, const float *__restrict__ scale,
+                                                           bf16 *__restrict__ out, int64_t rows, int64_t cols) {
+  const int64_t n = rows * cols;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256)
+    store_from_f32(out + i, scale[i / cols] * decode_e4m3fn(in[i]));
+}
+
 // ================================================================================================
 // host launchers
 // ================================================================================================
@@ -458,6 +478,14 @@ template <typename TA, typename TW>
 static int launch_gemm(const GemmArgs &a, int nsets, hipStream_t st) {
   dim3 grid((unsigned)((a.M + 63) / 64), (unsigned)((a.O + 63) / 64), (unsigned)nsets);
   hipLaunchKernelGGL((rows_gemm_kernel<TA, TW>), grid, dim3(256), 0, st, a);
+  return launch_status();
+}
+
+int dequant_e4m3(const void *in, const float *scale, void *out, int64_t rows, int64_t cols, hipStream_t st) {
+  int64_t blocks = (rows * cols + 255) / 256;
+  if (blocks > 1024) blocks = 1024;
+  hipLaunchKernelGGL(dequant_e4m3_kernel, dim3((unsigned)blocks), dim3(256), 0, st, static_cast<const uint8_t *>(in),
+                     scale, static_cast<bf16 *>(out), rows, cols);
   return launch_status();
 }
 

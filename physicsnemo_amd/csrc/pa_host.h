@@ -12,6 +12,7 @@ namespace pa {
 constexpr size_t kMaxLdsBytes = 160 * 1024;  // LDS per workgroup on gfx950
 
 namespace general {
+int dequant_e4m3(const void *in, const float *scale, void *out, int64_t rows, int64_t cols, hipStream_t st);
 int project_inputs(int dtype, const pa_shape &s, const pa_params &p, const void *x, void *x_mid, void *fx_mid,
                    hipStream_t st);
 int out_linear(int dtype, const pa_shape &s, const pa_params &p, const void *out_x, void *y, hipStream_t st);

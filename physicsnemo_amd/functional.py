@@ -116,12 +116,30 @@ def deslice_project(w, tok_out, params, dims: LayerDims, residual=None, ln_weigh
     return y if (residual is None and ln_out is None) else (y, ln_out)
 
 
+def quantize_e4m3_per_channel(weight: torch.Tensor):
+    """(out, in) weight -> (uint8 e4m3fn bytes, float32 scale per output channel), scale = max|row| / 448."""
+    w = weight.detach().float()
+    scale = w.abs().amax(dim=1).clamp_min(1e-12) / 448.0
+    q = (w / scale[:, None]).to(torch.float8_e4m3fn)
+    return q.view(torch.uint8).contiguous(), scale.contiguous()
+
+
+def dequantize_e4m3_per_channel(q: torch.Tensor, scale: torch.Tensor) -> torch.Tensor:
+    return q.view(torch.float8_e4m3fn).float() * scale[:, None]
+
+
 def layer_forward(x, params, dims: LayerDims, residual=None, ln_weight=None, ln_bias=None, ln_eps=1e-5,
                   return_slice_tokens=False):
-    """Whole PhysicsAttention layer.  Returns y, or (fx_new, ln_out) with a tail; slice tokens appended on request."""
+    """Whole PhysicsAttention layer.  Returns y, or (fx_new, ln_out) with a tail; slice tokens appended on request.
+
+    If `params` carries `in_project_x_scale` the three large weights are fp8-e4m3 bytes (PA_BF16_W8)."""
     _need_cuda(x, residual)
     lib = _lib.load()
     code = _lib.dtype_code(x.dtype)
+    if params.get("in_project_x_scale") is not None:
+        if x.dtype != torch.bfloat16:
+            raise TypeError("fp8-e4m3 weights need bfloat16 activations")
+        code = _lib.PA_BF16_W8
     shape = dims.c()
     nbytes = lib.pa_workspace_bytes(code, byref(shape))
     if nbytes < 0:

@@ -46,6 +46,17 @@ class PhysicsAttentionBase(nn.Module):
         self.out_linear = nn.Linear(dim_head * heads, dim)
         self.out_dropout = nn.Dropout(dropout)
         self._kernel_param_cache: dict = {}
+        self.fp8_weights = False  # see use_fp8_weights()
+
+    def use_fp8_weights(self, enabled: bool = True):
+        """Serve bf16 inputs with the three large weights quantised to fp8-e4m3, one scale per output channel
+        (scale = max|row| / 448).  The kernels expand them to bf16 MFMA operands; activations stay bf16.
+        Irregular-mesh variant only.  No counterpart in the reference."""
+        if enabled and self._conv_geometry()[2] != 0:
+            raise NotImplementedError("fp8 weights are served for the irregular-mesh variant only")
+        self.fp8_weights = bool(enabled)
+        self._kernel_param_cache = {}
+        return self
 
     # ---------------------------------------------------------------- parameters in kernel form
     def _conv_geometry(self):
@@ -70,7 +81,8 @@ class PhysicsAttentionBase(nn.Module):
             ("out_linear_weight", self.out_linear.weight, True),
             ("out_linear_bias", self.out_linear.bias, False),
         ]
-        stamp = (dtype, device) + tuple((p.data_ptr(), p._version, p.dtype) for _, p, _ in named)
+        fp8 = self.fp8_weights and dtype == torch.bfloat16
+        stamp = (dtype, device, fp8) + tuple((p.data_ptr(), p._version, p.dtype) for _, p, _ in named)
         hit = self._kernel_param_cache.get("stamp")
         if hit == stamp:
             return self._kernel_param_cache["params"]
@@ -79,6 +91,12 @@ class PhysicsAttentionBase(nn.Module):
                 name: p.detach().to(device=device, dtype=dtype if big else torch.float32).contiguous().reshape(-1).clone()
                 for name, p, big in named
             }
+            if fp8:
+                for name, p, big in named:
+                    if big:
+                        q, scale = PF.quantize_e4m3_per_channel(p.detach().reshape(p.shape[0], -1))
+                        params[name] = q.to(device).reshape(-1)
+                        params[name.replace("_weight", "_scale")] = scale.to(device)
         self._kernel_param_cache = {"stamp": stamp, "params": params}
         return params
 

@@ -129,3 +129,33 @@ def test_mfma_full_size_properties():
                                               torch.zeros(1, 4096, H, 32), ref.temperature)
         want = to.deslice_and_project(w, st.tok_out.cpu(), ref.out_linear.weight, ref.out_linear.bias)
     assert_rel_l2(y[:, :4096], want, "prefix of the full-size output")
+
+
+@pytest.mark.parametrize("B,N,C,S", [(2, 3000, 256, 64), (1, 2000, 128, 32), (1, 700, 512, 128)])
+def test_fp8_e4m3_weight_variant(B, N, C, S):
+    # bf16 activations, fp8-e4m3 per-output-channel-scaled projection weights.  The reference for the 1e-2 bar is
+    # the fp32 oracle holding the SAME (dequantised) weights; the error against the unquantised weights is printed.
+    announce("fp8 weights", B, N, C, S)
+    H = C // 32
+    ref, hip = make_pair("irregular", C, H, 32, S)
+    x = torch.randn(B, N, C)
+    xb = x.cuda().bfloat16()
+    with torch.no_grad():
+        want_full = ref(xb.float().cpu())
+        deq = {}
+        for name in ("in_project_x", "in_project_fx", "out_linear"):
+            w = getattr(ref, name).weight
+            q, s = PF.quantize_e4m3_per_channel(w)
+            deq[name] = PF.dequantize_e4m3_per_channel(q, s)
+            getattr(ref, name).weight.copy_(deq[name])
+        want_q = ref(xb.float().cpu())
+        y8 = hip.use_fp8_weights(True)(xb)
+        # the same dequantised weights served as ordinary bf16 weights must give the identical result
+        hip.use_fp8_weights(False)
+        for name in deq:
+            getattr(hip, name).weight.copy_(deq[name].cuda())
+        y16 = hip(xb)
+    assert y8.dtype == torch.bfloat16
+    assert_rel_l2(y8, want_q, "fp8-weight layer vs fp32 oracle with the dequantised weights")
+    assert torch.equal(y8, y16)
+    print("rel-L2 against the unquantised fp32 layer:", to.rel_l2(y8.float().cpu(), want_full), flush=True)

@@ -1,0 +1,76 @@
+"""Full-model GPU parity at the BASELINE configurations (HIP layer inside the Transolver glue) against the CPU oracle."""
+import math
+
+import pytest
+import torch
+
+from oracle import torch_oracle as to
+import physicsnemo_amd as pn
+from gpu_util import announce, assert_fp32_close, assert_rel_l2
+
+pytestmark = pytest.mark.gpu
+
+
+def _pair(**kw):
+    torch.manual_seed(0)
+    ref = to.OracleTransolver(**kw).eval()
+    hip = pn.Transolver(use_te=False, **kw).eval()
+    hip.load_state_dict(ref.state_dict())
+    return ref, hip.cuda()
+
+
+def test_cfg1_structured2d_fp32_full_size():
+    # cfg1: grid 85 x 85 (N = 7225), batch 4, n_hidden 128, 8 heads (D = 16), 32 slices, 4 layers, mlp_ratio 1, fp32
+    announce("cfg1 structured 2D fp32")
+    ref, hip = _pair(functional_dim=1, embedding_dim=2, out_dim=1, n_layers=4, n_hidden=128, n_head=8, mlp_ratio=1,
+                     slice_num=32, structured_shape=(85, 85), unified_pos=False)
+    g = torch.Generator().manual_seed(1234)
+    lin = torch.linspace(0, 1, 85)
+    pos = torch.stack(torch.meshgrid(lin, lin, indexing="ij"), -1).reshape(1, 7225, 2).repeat(4, 1, 1)
+    fx = torch.randn(4, 7225, 1, generator=g)
+    with torch.no_grad():
+        want = ref(fx, pos)
+        got = hip(fx.cuda(), pos.cuda())
+    assert got.shape == (4, 7225, 1)
+    assert_fp32_close(got, want, "cfg1 model output")
+
+
+def test_cfg2_irregular_bf16_autocast():
+    # cfg2: 32768 annulus points, n_hidden 256, 8 heads, 64 slices, 8 layers (batch 2 of the 8 to bound CPU time)
+    announce("cfg2 irregular bf16")
+    ref, hip = _pair(functional_dim=3, embedding_dim=2, out_dim=4, n_layers=8, n_hidden=256, n_head=8, slice_num=64)
+    g = torch.Generator().manual_seed(1234)
+    B, N = 2, 32768
+    r = torch.sqrt(torch.empty(B, N).uniform_(0.25, 1.0, generator=g))
+    th = torch.empty(B, N).uniform_(0, 2 * math.pi, generator=g)
+    pos = torch.stack((r * torch.cos(th), r * torch.sin(th)), -1)
+    fx = torch.randn(B, N, 3, generator=g)
+    with torch.no_grad():
+        want = ref(fx, pos)
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            got = hip(fx.cuda(), pos.cuda())
+    assert got.shape == (B, N, 4)
+    # eight bf16 layers deep: the north-star bar (rel-L2 1e-2 vs fp32) is stated per layer; the model gets 2e-2
+    assert_rel_l2(got, want, "cfg2 model output", tol=2e-2)
+
+
+def test_cfg4_surface_bf16_layer_stack_reduced():
+    # cfg4 shape class: 3 coords + 3 normals + 1 field, n_hidden 256, 8 heads, 32 slices, 8 layers; 20000 points
+    # (not a multiple of 32: exercises the ragged tile) on an ellipsoid perturbed by low-order harmonics
+    announce("cfg4 surface bf16")
+    ref, hip = _pair(functional_dim=1, embedding_dim=6, out_dim=4, n_layers=8, n_hidden=256, n_head=8, slice_num=32)
+    g = torch.Generator().manual_seed(1234)
+    N = 20000
+    th = torch.acos(torch.empty(N).uniform_(-1, 1, generator=g))
+    ph = torch.empty(N).uniform_(0, 2 * math.pi, generator=g)
+    rad = 1 + 0.1 * (3 * torch.cos(th) ** 2 - 1) / 2 + 0.05 * torch.sin(th) ** 2 * torch.cos(th) * torch.cos(2 * ph)
+    xyz = torch.stack((1.0 * rad * torch.sin(th) * torch.cos(ph), 0.6 * rad * torch.sin(th) * torch.sin(ph),
+                       0.4 * rad * torch.cos(th)), -1)
+    nrm = torch.nn.functional.normalize(xyz / torch.tensor([1.0, 0.36, 0.16]), dim=-1)
+    emb = torch.cat((xyz, nrm), -1)[None]
+    fx = torch.randn(1, N, 1, generator=g)
+    with torch.no_grad():
+        want = ref(fx, emb)
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            got = hip(fx.cuda(), emb.cuda())
+    assert_rel_l2(got, want, "cfg4-class model output", tol=2e-2)
