@@ -353,6 +353,192 @@ __global__ __launch_bounds__(WAVES * 64) void project_softmax_kernel(const u32x4
 }
 
 // ------------------------------------------------------------------------------------------------
+// Kernel (a), weights-stationary form.  One persistent workgroup per CU, H/2 waves (one per SIMD for C = 256), each
+// wave owns TWO heads and keeps their Wx | Wfx fragments (2 * 2 * KS * 4 VGPRs) in registers for the whole kernel:
+// no weight traffic at all after the prologue.  The x rows of a SET of TS tiles (TS * 32 points) are staged in LDS
+// by the whole workgroup with full-row coalesced loads; unit u (16 bytes) of row r is stored at r*UPR + (u ^ (r&7)),
+// which makes both the row-wise writes and the fragment reads (row i, unit 2ks+g) bank-conflict free.  One x
+// fragment read (1 KiB) feeds 2 MFMAs of a head, i.e. 0.5 KiB of LDS per MFMA (the tile-stationary form needs 1).
+// The set buffers are double buffered; the next set is fetched one tile at a time into 4 registers per thread at
+// the start of a tile and written to LDS at its end; one barrier per set.
+//
+// Inside a wave the work is a chain of head-steps  (tile t, head hh):  products(t, hh) [MFMA]  overlapped with
+// softmax + stores of the previous head-step [VALU, VMEM]; both are straight-line code in one scheduling region.
+// The loop over sets is the only loop; its body has no branch around a memory operation (waves past the last
+// tile recompute it and re-store identical values; the very first softmax runs on zero logits and is overwritten).
+// ------------------------------------------------------------------------------------------------
+template <int C, int S>
+__global__ __launch_bounds__((C / 64) * 64) void project_softmax_ws_kernel(const u32x4 *__restrict__ blob,
+                                                                           const uint16_t *__restrict__ x,
+                                                                           u32x4 *__restrict__ fx_pack,
+                                                                           u32x4 *__restrict__ w_pack, int64_t N, int tpb,
+                                                                           int64_t total_tiles) {
+  constexpr int H = C / 32, KS = C / 16, ST = (S + 31) / 32, NCH = S / 16;
+  constexpr int WAVES = H / 2, NT = WAVES * 64;
+  constexpr int TS = 4;                 // tiles per set
+  constexpr int UPR = C / 8;            // 16-byte units per row
+  constexpr int SET_UNITS = TS * 32 * UPR;
+  constexpr int CHUNK = 32 * UPR / NT;  // units per thread and tile when staging
+  static_assert((32 * UPR) % NT == 0, "a tile must split evenly over the workgroup");
+  extern __shared__ u32x4 smem[];
+  u32x4 *xs = smem;                     // 2 * SET_UNITS
+  u32x4 *wsl = xs + 2 * SET_UNITS;      // ST * 2 * 64
+  float *fvec = reinterpret_cast<float *>(wsl + ST * 2 * 64);
+  float *bias_x = fvec, *bias_f = fvec + C, *bias_s = fvec + 2 * C, *tscale = fvec + 3 * C + ST * 32;
+  const BlobPlan bp = blob_plan(C, S);
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, i = lane & 31, g = lane >> 5;
+
+  // this wave's two heads: Wx (A operand of x_mid^T) and Wfx (B operand of fx_mid), register resident
+  u32x4 wx[2][KS], wf[2][KS];
+#pragma unroll
+  for (int hh = 0; hh < 2; ++hh)
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int64_t base = bp.win + ((int64_t)(2 * wave + hh) * 2) * KS * 64;
+      wx[hh][ks] = blob[base + ks * 64 + lane];
+      wf[hh][ks] = blob[base + (KS + ks) * 64 + lane];
+    }
+  for (int u = tid; u < ST * 2 * 64; u += NT) wsl[u] = blob[bp.wsl + u];
+  {
+    const float *src = reinterpret_cast<const float *>(blob + bp.fvec);
+    for (int k = tid; k < 3 * C + ST * 32 + H; k += NT) fvec[k] = src[k];
+  }
+
+  const int64_t nsets = (total_tiles + TS - 1) / TS;
+  const int64_t nloc = (nsets - blockIdx.x + gridDim.x - 1) / gridDim.x;
+  auto tile_of = [&](int64_t set, int t) {
+    const int64_t tr = set * TS + t;
+    return tr < total_tiles ? tr : total_tiles - 1;
+  };
+  // staging: this thread's CHUNK units of tile (set, t): unit k*NT + tid -> row rc, position pos
+  auto stage_load = [&](int64_t set, int t, u32x4(&st)[CHUNK]) {
+    const int64_t tile = tile_of(set, t);
+    const int64_t b = tile / tpb;
+    const int64_t n0 = (tile - b * tpb) * 32;
+#pragma unroll
+    for (int k = 0; k < CHUNK; ++k) {
+      const int idx = k * NT + tid, rc = idx / UPR, pos = idx - rc * UPR;
+      const bool ok = n0 + rc < N;
+      const u32x4 v = *reinterpret_cast<const u32x4 *>(x + ((int64_t)b * N + (ok ? n0 + rc : 0)) * C + pos * 8);
+      st[k] = ok ? v : u32x4{0, 0, 0, 0};
+    }
+  };
+  auto stage_store = [&](int buf, int t, const u32x4(&st)[CHUNK]) {
+#pragma unroll
+    for (int k = 0; k < CHUNK; ++k) {
+      const int idx = k * NT + tid, rc = idx / UPR, pos = idx - rc * UPR;
+      xs[buf * SET_UNITS + (t * 32 + rc) * UPR + (pos ^ (rc & 7))] = st[k];
+    }
+  };
+  {  // first set
+    int64_t set0 = blockIdx.x;
+#pragma unroll
+    for (int t = 0; t < TS; ++t) {
+      u32x4 st[CHUNK];
+      stage_load(set0, t, st);
+      stage_store(0, t, st);
+    }
+  }
+  __syncthreads();
+
+  // state of the previous head-step (its logits still need the softmax)
+  f32x16 lg[ST];
+#pragma unroll
+  for (int st = 0; st < ST; ++st)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) lg[st][r] = 0.f;
+  int64_t tile_prev = tile_of(blockIdx.x, 0);
+  int h_prev = 2 * wave;
+  bool valid_prev = false;
+
+  auto softmax_store = [&]() {
+    float mx = -INFINITY;
+#pragma unroll
+    for (int st = 0; st < ST; ++st)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) mx = fmaxf(mx, lg[st][r]);
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float sc = tscale[h_prev];
+    const float off = mx * sc;
+    float sum = 0.f;
+#pragma unroll
+    for (int st = 0; st < ST; ++st)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const float e = __builtin_amdgcn_exp2f(fmaf(lg[st][r], sc, -off));
+        lg[st][r] = e;
+        sum += e;
+      }
+    sum += __shfl_xor(sum, 32, 64);
+    const float inv = valid_prev ? __builtin_amdgcn_rcpf(sum) : 0.f;
+    u32x4 *wdst = w_pack + ((tile_prev * H + h_prev) * NCH) * 64 + lane;
+#pragma unroll
+    for (int st = 0; st < ST; ++st) {
+      if (2 * st < NCH) wdst[(2 * st) * 64] = pack_half<0>(lg[st], inv);
+      if (2 * st + 1 < NCH) wdst[(2 * st + 1) * 64] = pack_half<1>(lg[st], inv);
+    }
+  };
+
+  // products of (tile at slot t of buffer buf, head 2*wave + hh); leaves the logits in lg and stores fx_mid
+  auto products = [&](int buf, int t, int hh, int64_t tile) {
+    const int h = 2 * wave + hh;
+    const u32x4 *xb = xs + buf * SET_UNITS + (t * 32 + i) * UPR;
+    f32x16 ax, af;
+    {
+      const float bf = bias_f[h * 32 + i];
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        ax[r] = bias_x[h * 32 + rowmap(r, g)];
+        af[r] = bf;
+      }
+    }
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const u32x4 xf = xb[(2 * ks + g) ^ (i & 7)];
+      ax = mma(wx[hh][ks], xf, ax);
+      af = mma(xf, wf[hh][ks], af);
+    }
+    u32x4 *fdst = fx_pack + ((tile * H + h) * 2) * 64 + lane;
+    fdst[0] = pack_half<0>(af);
+    fdst[64] = pack_half<1>(af);
+    const u32x4 xb0 = pack_half<0>(ax), xb1 = pack_half<1>(ax);
+#pragma unroll
+    for (int st = 0; st < ST; ++st) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) lg[st][r] = bias_s[32 * st + rowmap(r, g)];
+      lg[st] = mma(wsl[(st * 2 + 0) * 64 + lane], xb0, lg[st]);
+      lg[st] = mma(wsl[(st * 2 + 1) * 64 + lane], xb1, lg[st]);
+    }
+  };
+
+  int64_t set = blockIdx.x;
+  for (int64_t sl = 0; sl < nloc; ++sl) {
+    const int buf = (int)(sl & 1);
+    const int64_t set_next = set + gridDim.x < nsets ? set + gridDim.x : set;  // the last set re-fetches itself
+#pragma unroll
+    for (int t = 0; t < TS; ++t) {
+      u32x4 stg[CHUNK];
+      stage_load(set_next, t, stg);
+      const int64_t tile = tile_of(set, t);
+      const int64_t b = tile / tpb;
+      const bool valid = (tile - b * tpb) * 32 + i < N;
+#pragma unroll
+      for (int hh = 0; hh < 2; ++hh) {
+        softmax_store();  // previous head-step (VALU / stores), independent of the products below (MFMA)
+        products(buf, t, hh, tile);
+        tile_prev = tile;
+        h_prev = 2 * wave + hh;
+        valid_prev = valid;
+      }
+      stage_store(buf ^ 1, t, stg);
+    }
+    set = set_next;
+    __syncthreads();
+  }
+  softmax_store();  // the last head-step
+}
+
+// ------------------------------------------------------------------------------------------------
 // Kernel (b): slice-token aggregation, streaming over the packed w / fx_mid.  grid (G groups, B*H), 4 waves.
 // Each wave walks every 4th tile of its group's tile range for one (batch, head):
 //   w^T (32 pts x 32 s, C/D layout: lane <-> slice, registers <-> points) = w_chunk . SEL     (an exact MFMA
@@ -721,8 +907,37 @@ static int project_softmax_w(const pa_shape &s, const void *blob, const void *x,
 }
 
 template <int C, int S>
+static int project_softmax_ws(const pa_shape &s, const void *blob, const void *x, void *fx_pack, void *w_pack,
+                              int num_cu, hipStream_t st) {
+  constexpr int ST = (S + 31) / 32, H = C / 32, TS = 4, UPR = C / 8, WAVES = H / 2;
+  const size_t lds = (size_t)(2 * TS * 32 * UPR + ST * 2 * 64) * 16 + (size_t)(3 * C + ST * 32 + H) * 4;
+  int rc = allow_dynamic_lds(project_softmax_ws_kernel<C, S>, lds);
+  if (rc) return rc;
+  const int64_t tpb = tiles_per_batch(s), total = tpb * s.B;
+  static int per_cu = 0;  // resident workgroups per CU for this instantiation
+  if (per_cu == 0) {
+    int nb = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, project_softmax_ws_kernel<C, S>, WAVES * 64, lds) != hipSuccess ||
+        nb < 1)
+      nb = 1;
+    per_cu = nb;
+  }
+  int64_t grid = (total + TS - 1) / TS;
+  if (grid > (int64_t)num_cu * per_cu) grid = (int64_t)num_cu * per_cu;
+  hipLaunchKernelGGL((project_softmax_ws_kernel<C, S>), dim3((unsigned)grid), dim3(WAVES * 64), lds, st,
+                     static_cast<const u32x4 *>(blob), static_cast<const uint16_t *>(x), static_cast<u32x4 *>(fx_pack),
+                     static_cast<u32x4 *>(w_pack), s.N, (int)tpb, total);
+  return launch_status();
+}
+
+template <int C, int S>
 static int project_softmax_cs(const pa_shape &s, const void *blob, const void *x, void *fx_pack, void *w_pack,
                               int num_cu, hipStream_t st) {
+  static const int form = [] {
+    const char *e = getenv("PA_KA_FORM");
+    return e ? atoi(e) : 1;
+  }();
+  if (form == 1) return project_softmax_ws<C, S>(s, blob, x, fx_pack, w_pack, num_cu, st);
   return project_softmax_w<C, S, 8>(s, blob, x, fx_pack, w_pack, num_cu, st);
 }
 
