@@ -353,28 +353,28 @@ __global__ __launch_bounds__(WAVES * 64) void project_softmax_kernel(const u32x4
 }
 
 // ------------------------------------------------------------------------------------------------
-// Kernel (a), weights-stationary form.  One persistent workgroup per CU, H/2 waves (one per SIMD for C = 256), each
-// wave owns TWO heads and keeps their Wx | Wfx fragments (2 * 2 * KS * 4 VGPRs) in registers for the whole kernel:
-// no weight traffic at all after the prologue.  The x rows of a SET of TS tiles (TS * 32 points) are staged in LDS
+// Kernel (a), weights-stationary form.  One persistent workgroup per CU, H waves (two per SIMD for C = 256), each
+// wave owns ONE head and keeps its Wx | Wfx fragments (2 * KS * 4 = 128 VGPRs for C = 256) in registers for the
+// whole kernel: no weight traffic at all after the prologue.  The x rows of a SET of TS tiles (TS * 32 points) are staged in LDS
 // by the whole workgroup with full-row coalesced loads; unit u (16 bytes) of row r is stored at r*UPR + (u ^ (r&7)),
 // which makes both the row-wise writes and the fragment reads (row i, unit 2ks+g) bank-conflict free.  One x
 // fragment read (1 KiB) feeds 2 MFMAs of a head, i.e. 0.5 KiB of LDS per MFMA (the tile-stationary form needs 1).
 // The set buffers are double buffered; the next set is fetched one tile at a time into 4 registers per thread at
 // the start of a tile and written to LDS at its end; one barrier per set.
 //
-// Inside a wave the work is a chain of head-steps  (tile t, head hh):  products(t, hh) [MFMA]  overlapped with
-// softmax + stores of the previous head-step [VALU, VMEM]; both are straight-line code in one scheduling region.
+// Inside a wave the work is a chain of head-steps, one per tile:  products(t) [MFMA]  interleaved with the
+// softmax + stores of the previous head-step [VALU, VMEM].
 // The loop over sets is the only loop; its body has no branch around a memory operation (waves past the last
 // tile recompute it and re-store identical values; the very first softmax runs on zero logits and is overwritten).
 // ------------------------------------------------------------------------------------------------
-template <int C, int S>
-__global__ __launch_bounds__((C / 64) * 64) void project_softmax_ws_kernel(const u32x4 *__restrict__ blob,
+template <int C, int S, int HPW>
+__global__ __launch_bounds__((C / 32 / HPW) * 64) void project_softmax_ws_kernel(const u32x4 *__restrict__ blob,
                                                                            const uint16_t *__restrict__ x,
                                                                            u32x4 *__restrict__ fx_pack,
                                                                            u32x4 *__restrict__ w_pack, int64_t N, int tpb,
                                                                            int64_t total_tiles) {
   constexpr int H = C / 32, KS = C / 16, ST = (S + 31) / 32, NCH = S / 16;
-  constexpr int WAVES = H / 2, NT = WAVES * 64;
+  constexpr int WAVES = H / HPW, NT = WAVES * 64;
   constexpr int TS = 4;                 // tiles per set
   constexpr int UPR = C / 8;            // 16-byte units per row
   constexpr int SET_UNITS = TS * 32 * UPR;
@@ -388,13 +388,13 @@ __global__ __launch_bounds__((C / 64) * 64) void project_softmax_ws_kernel(const
   const BlobPlan bp = blob_plan(C, S);
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, i = lane & 31, g = lane >> 5;
 
-  // this wave's two heads: Wx (A operand of x_mid^T) and Wfx (B operand of fx_mid), register resident
-  u32x4 wx[2][KS], wf[2][KS];
+  // this wave's head: Wx (A operand of x_mid^T) and Wfx (B operand of fx_mid), register resident
+  u32x4 wx[HPW][KS], wf[HPW][KS];
 #pragma unroll
-  for (int hh = 0; hh < 2; ++hh)
+  for (int hh = 0; hh < HPW; ++hh)
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      const int64_t base = bp.win + ((int64_t)(2 * wave + hh) * 2) * KS * 64;
+      const int64_t base = bp.win + ((int64_t)(HPW * wave + hh) * 2) * KS * 64;
       wx[hh][ks] = blob[base + ks * 64 + lane];
       wf[hh][ks] = blob[base + (KS + ks) * 64 + lane];
     }
@@ -406,20 +406,23 @@ __global__ __launch_bounds__((C / 64) * 64) void project_softmax_ws_kernel(const
 
   const int64_t nsets = (total_tiles + TS - 1) / TS;
   const int64_t nloc = (nsets - blockIdx.x + gridDim.x - 1) / gridDim.x;
+  const int ntiles = (int)total_tiles;  // < 2^28 (checked on the host)
   auto tile_of = [&](int64_t set, int t) {
-    const int64_t tr = set * TS + t;
-    return tr < total_tiles ? tr : total_tiles - 1;
+    const int tr = (int)set * TS + t;
+    return tr < ntiles ? tr : ntiles - 1;
   };
   // staging: this thread's CHUNK units of tile (set, t): unit k*NT + tid -> row rc, position pos
   auto stage_load = [&](int64_t set, int t, u32x4(&st)[CHUNK]) {
-    const int64_t tile = tile_of(set, t);
-    const int64_t b = tile / tpb;
-    const int64_t n0 = (tile - b * tpb) * 32;
+    const int tile = tile_of(set, t);
+    const int b = tile / tpb;
+    const int n0 = (tile - b * tpb) * 32;
+    const uint16_t *xbase = x + ((int64_t)b * N + n0) * C;
+    const int rows_ok = (int)min((int64_t)32, N - n0);
 #pragma unroll
     for (int k = 0; k < CHUNK; ++k) {
       const int idx = k * NT + tid, rc = idx / UPR, pos = idx - rc * UPR;
-      const bool ok = n0 + rc < N;
-      const u32x4 v = *reinterpret_cast<const u32x4 *>(x + ((int64_t)b * N + (ok ? n0 + rc : 0)) * C + pos * 8);
+      const bool ok = rc < rows_ok;
+      const u32x4 v = *reinterpret_cast<const u32x4 *>(xbase + (ok ? rc : 0) * C + pos * 8);
       st[k] = ok ? v : u32x4{0, 0, 0, 0};
     }
   };
@@ -441,14 +444,15 @@ __global__ __launch_bounds__((C / 64) * 64) void project_softmax_ws_kernel(const
   }
   __syncthreads();
 
+
   // state of the previous head-step (its logits still need the softmax)
   f32x16 lg[ST];
 #pragma unroll
   for (int st = 0; st < ST; ++st)
 #pragma unroll
     for (int r = 0; r < 16; ++r) lg[st][r] = 0.f;
-  int64_t tile_prev = tile_of(blockIdx.x, 0);
-  int h_prev = 2 * wave;
+  int tile_prev = tile_of(blockIdx.x, 0);
+  int h_prev = HPW * wave;
   bool valid_prev = false;
 
   auto softmax_store = [&]() {
@@ -471,7 +475,7 @@ __global__ __launch_bounds__((C / 64) * 64) void project_softmax_ws_kernel(const
       }
     sum += __shfl_xor(sum, 32, 64);
     const float inv = valid_prev ? __builtin_amdgcn_rcpf(sum) : 0.f;
-    u32x4 *wdst = w_pack + ((tile_prev * H + h_prev) * NCH) * 64 + lane;
+    u32x4 *wdst = w_pack + (((int64_t)tile_prev * H + h_prev) * NCH) * 64 + lane;
 #pragma unroll
     for (int st = 0; st < ST; ++st) {
       if (2 * st < NCH) wdst[(2 * st) * 64] = pack_half<0>(lg[st], inv);
@@ -479,9 +483,20 @@ __global__ __launch_bounds__((C / 64) * 64) void project_softmax_ws_kernel(const
     }
   };
 
-  // products of (tile at slot t of buffer buf, head 2*wave + hh); leaves the logits in lg and stores fx_mid
-  auto products = [&](int buf, int t, int hh, int64_t tile) {
-    const int h = 2 * wave + hh;
+  // One head-step: products of the tile at slot t of buffer buf (this wave's head) interleaved, MFMA by MFMA, with the
+  // softmax + stores of the PREVIOUS head-step (whose logits are in lg).  The 2*KS projection MFMAs form 2*KS units;
+  // each unit is one MFMA plus a slice of the softmax small enough to run in its shadow, and a scheduling barrier
+  // closes the unit so the compiler keeps this mix:
+  //   units [0, UA)        running maximum over the logits         (then one exchange with lane^32)
+  //   units [UA, UA+UB)    exp2 and running sum                    (then one exchange, reciprocal)
+  //   units [UA+UB, 2*KS)  scale, convert to bf16, store each finished 16-slice chunk
+  // Afterwards lg is free and receives this step's logits.
+  auto head_step = [&](int buf, int t, int hh, int tile) {
+    const int h = HPW * wave + hh;
+    constexpr int U = 2 * KS, R = ST * 16;           // units, logit registers per lane
+    constexpr int UA = U / 4, UB = U / 2, UC = U - UA - UB;
+    constexpr int RA = (R + UA - 1) / UA, RB = (R + UB - 1) / UB, RC = (R + UC - 1) / UC;
+    constexpr int RING = 3, AHEAD = 2;               // x fragments are read AHEAD k-steps early
     const u32x4 *xb = xs + buf * SET_UNITS + (t * 32 + i) * UPR;
     f32x16 ax, af;
     {
@@ -492,13 +507,62 @@ __global__ __launch_bounds__((C / 64) * 64) void project_softmax_ws_kernel(const
         af[r] = bf;
       }
     }
+    u32x4 xf[RING];
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      const u32x4 xf = xb[(2 * ks + g) ^ (i & 7)];
-      ax = mma(wx[hh][ks], xf, ax);
-      af = mma(xf, wf[hh][ks], af);
+    for (int q = 0; q < AHEAD; ++q) xf[q] = xb[(2 * q + g) ^ (i & 7)];
+    const float sc = tscale[h_prev];
+    float mx = -INFINITY, off = 0.f, sum = 0.f, inv = 0.f;
+    u32x4 *wdst = w_pack + (((int64_t)tile_prev * H + h_prev) * NCH) * 64 + lane;
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int ks = u >> 1;
+      if ((u & 1) == 0) {
+        if (ks + AHEAD < KS) xf[(ks + AHEAD) % RING] = xb[(2 * (ks + AHEAD) + g) ^ (i & 7)];
+        ax = mma(wx[hh][ks], xf[ks % RING], ax);
+      } else {
+        af = mma(xf[ks % RING], wf[hh][ks], af);
+      }
+      if (u < UA) {
+#pragma unroll
+        for (int k = 0; k < RA; ++k) {
+          const int r = u * RA + k;
+          if (r < R) mx = fmaxf(mx, lg[r >> 4][r & 15]);
+        }
+        if (u == UA - 1) {
+          mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+          off = mx * sc;
+        }
+      } else if (u < UA + UB) {
+#pragma unroll
+        for (int k = 0; k < RB; ++k) {
+          const int r = (u - UA) * RB + k;
+          if (r < R) {
+            const float e = __builtin_amdgcn_exp2f(fmaf(lg[r >> 4][r & 15], sc, -off));
+            lg[r >> 4][r & 15] = e;
+            sum += e;
+          }
+        }
+        if (u == UA + UB - 1) {
+          sum += __shfl_xor(sum, 32, 64);
+          inv = valid_prev ? __builtin_amdgcn_rcpf(sum) : 0.f;
+        }
+      } else {
+#pragma unroll
+        for (int k = 0; k < RC; ++k) {
+          const int r = (u - UA - UB) * RC + k;
+          if (r < R) {
+            lg[r >> 4][r & 15] *= inv;
+            if ((r & 7) == 7 && (r >> 3) < NCH) {  // chunk r/8 complete
+              if (((r >> 3) & 1) == 0) wdst[(r >> 3) * 64] = pack_half<0>(lg[r >> 4]);
+              else wdst[(r >> 3) * 64] = pack_half<1>(lg[r >> 4]);
+            }
+          }
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
     }
-    u32x4 *fdst = fx_pack + ((tile * H + h) * 2) * 64 + lane;
+    u32x4 *fdst = fx_pack + (((int64_t)tile * H + h) * 2) * 64 + lane;
     fdst[0] = pack_half<0>(af);
     fdst[64] = pack_half<1>(af);
     const u32x4 xb0 = pack_half<0>(ax), xb1 = pack_half<1>(ax);
@@ -517,20 +581,24 @@ __global__ __launch_bounds__((C / 64) * 64) void project_softmax_ws_kernel(const
     const int64_t set_next = set + gridDim.x < nsets ? set + gridDim.x : set;  // the last set re-fetches itself
 #pragma unroll
     for (int t = 0; t < TS; ++t) {
+      __builtin_amdgcn_sched_barrier(0);  // keep each tile's work (and its register live ranges) to itself
       u32x4 stg[CHUNK];
       stage_load(set_next, t, stg);
-      const int64_t tile = tile_of(set, t);
-      const int64_t b = tile / tpb;
-      const bool valid = (tile - b * tpb) * 32 + i < N;
+      __builtin_amdgcn_sched_barrier(0);
+      const int tile = tile_of(set, t);
+      const int b = tile / tpb;
+      const bool valid = (int64_t)(tile - b * tpb) * 32 + i < N;
 #pragma unroll
-      for (int hh = 0; hh < 2; ++hh) {
-        softmax_store();  // previous head-step (VALU / stores), independent of the products below (MFMA)
-        products(buf, t, hh, tile);
+      for (int hh = 0; hh < HPW; ++hh) {
+        head_step(buf, t, hh, tile);
         tile_prev = tile;
-        h_prev = 2 * wave + hh;
+        h_prev = HPW * wave + hh;
         valid_prev = valid;
+        __builtin_amdgcn_sched_barrier(0);
       }
+      __builtin_amdgcn_sched_barrier(0);
       stage_store(buf ^ 1, t, stg);
+      __builtin_amdgcn_sched_barrier(0);
     }
     set = set_next;
     __syncthreads();
@@ -906,25 +974,25 @@ static int project_softmax_w(const pa_shape &s, const void *blob, const void *x,
   return launch_status();
 }
 
-template <int C, int S>
+template <int C, int S, int HPW>
 static int project_softmax_ws(const pa_shape &s, const void *blob, const void *x, void *fx_pack, void *w_pack,
                               int num_cu, hipStream_t st) {
-  constexpr int ST = (S + 31) / 32, H = C / 32, TS = 4, UPR = C / 8, WAVES = H / 2;
+  constexpr int ST = (S + 31) / 32, H = C / 32, TS = 4, UPR = C / 8, WAVES = H / HPW;
   const size_t lds = (size_t)(2 * TS * 32 * UPR + ST * 2 * 64) * 16 + (size_t)(3 * C + ST * 32 + H) * 4;
-  int rc = allow_dynamic_lds(project_softmax_ws_kernel<C, S>, lds);
+  int rc = allow_dynamic_lds(project_softmax_ws_kernel<C, S, HPW>, lds);
   if (rc) return rc;
   const int64_t tpb = tiles_per_batch(s), total = tpb * s.B;
   static int per_cu = 0;  // resident workgroups per CU for this instantiation
   if (per_cu == 0) {
     int nb = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, project_softmax_ws_kernel<C, S>, WAVES * 64, lds) != hipSuccess ||
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, project_softmax_ws_kernel<C, S, HPW>, WAVES * 64, lds) != hipSuccess ||
         nb < 1)
       nb = 1;
     per_cu = nb;
   }
   int64_t grid = (total + TS - 1) / TS;
   if (grid > (int64_t)num_cu * per_cu) grid = (int64_t)num_cu * per_cu;
-  hipLaunchKernelGGL((project_softmax_ws_kernel<C, S>), dim3((unsigned)grid), dim3(WAVES * 64), lds, st,
+  hipLaunchKernelGGL((project_softmax_ws_kernel<C, S, HPW>), dim3((unsigned)grid), dim3(WAVES * 64), lds, st,
                      static_cast<const u32x4 *>(blob), static_cast<const uint16_t *>(x), static_cast<u32x4 *>(fx_pack),
                      static_cast<u32x4 *>(w_pack), s.N, (int)tpb, total);
   return launch_status();
@@ -937,7 +1005,8 @@ static int project_softmax_cs(const pa_shape &s, const void *blob, const void *x
     const char *e = getenv("PA_KA_FORM");
     return e ? atoi(e) : 1;
   }();
-  if (form == 1) return project_softmax_ws<C, S>(s, blob, x, fx_pack, w_pack, num_cu, st);
+  if (form == 1) return project_softmax_ws<C, S, 2>(s, blob, x, fx_pack, w_pack, num_cu, st);
+  if (form == 2) return project_softmax_ws<C, S, 1>(s, blob, x, fx_pack, w_pack, num_cu, st);
   return project_softmax_w<C, S, 8>(s, blob, x, fx_pack, w_pack, num_cu, st);
 }
 
