@@ -579,26 +579,26 @@ __global__ __launch_bounds__((C / 32 / HPW) * 64) void project_softmax_ws_kernel
   for (int64_t sl = 0; sl < nloc; ++sl) {
     const int buf = (int)(sl & 1);
     const int64_t set_next = set + gridDim.x < nsets ? set + gridDim.x : set;  // the last set re-fetches itself
+    // head-major order inside a set: a head's weights are used for TS consecutive head-steps
 #pragma unroll
-    for (int t = 0; t < TS; ++t) {
-      __builtin_amdgcn_sched_barrier(0);  // keep each tile's work (and its register live ranges) to itself
-      u32x4 stg[CHUNK];
-      stage_load(set_next, t, stg);
-      __builtin_amdgcn_sched_barrier(0);
-      const int tile = tile_of(set, t);
-      const int b = tile / tpb;
-      const bool valid = (int64_t)(tile - b * tpb) * 32 + i < N;
+    for (int hh = 0; hh < HPW; ++hh) {
 #pragma unroll
-      for (int hh = 0; hh < HPW; ++hh) {
+      for (int t = 0; t < TS; ++t) {
+        __builtin_amdgcn_sched_barrier(0);  // keep each head-step's work (and its register live ranges) to itself
+        u32x4 stg[CHUNK];
+        if (hh == HPW - 1) stage_load(set_next, t, stg);
+        __builtin_amdgcn_sched_barrier(0);
+        const int tile = tile_of(set, t);
+        const int b = tile / tpb;
+        const bool valid = (int64_t)(tile - b * tpb) * 32 + i < N;
         head_step(buf, t, hh, tile);
         tile_prev = tile;
         h_prev = HPW * wave + hh;
         valid_prev = valid;
         __builtin_amdgcn_sched_barrier(0);
+        if (hh == HPW - 1) stage_store(buf ^ 1, t, stg);
+        __builtin_amdgcn_sched_barrier(0);
       }
-      __builtin_amdgcn_sched_barrier(0);
-      stage_store(buf ^ 1, t, stg);
-      __builtin_amdgcn_sched_barrier(0);
     }
     set = set_next;
     __syncthreads();
