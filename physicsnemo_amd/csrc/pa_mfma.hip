@@ -18,8 +18,6 @@
 //                                  of point i of the tile                       (B operand of the deslice product)
 //   fx_pack[tile][h][kk][lane][8]  fx_mid, lane i <-> channel d = i of head h, element j <-> point kperm(kk, g, j)
 //                                                                                (A operand of the aggregation)
-#include <stdlib.h>
-
 #include "pa_common.h"
 #include "pa_host.h"
 
@@ -125,256 +123,30 @@ __global__ __launch_bounds__(256) void pack_params_kernel(pa_params p, u32x4 *__
 }
 
 // ------------------------------------------------------------------------------------------------
-// Kernel (a): projections + slice logits + temperature softmax.   Persistent, 8 waves = 8 tiles per set.
-//   x_mid^T (32 ch x 32 pts) = Wx_h . x^T          A = Wx_h frags (LDS), B = x frags (registers, loaded once)
-//   fx_mid  (32 pts x 32 d)  = x . Wfx_h^T         A = x frags,          B = Wfx_h frags (LDS)   -> fx_pack
+// Kernel (a): projections + slice logits + temperature softmax, weights-stationary.
+//   x_mid^T (32 ch x 32 pts) = Wx_h . x^T          A = Wx_h frags (registers), B = x frags (LDS)
+//   fx_mid  (32 pts x 32 d)  = x . Wfx_h^T         A = x frags (LDS),          B = Wfx_h frags (registers)  -> fx_pack
 //   logits^T(32 s x 32 pts)  = Wslice . x_mid^T    A = Wslice frags (LDS), B = bf16(x_mid^T) straight from registers
-//   softmax over s: in-lane over the accumulator registers plus one exchange with lane^32          -> w_pack
-// Per-head weights (Wx_h | Wfx_h, 2*KS KiB) are double-buffered in LDS: the next head's bytes are fetched into
-// registers before the current head's work and stored to LDS after it.
+//   softmax over s: in-lane over the accumulator registers plus one exchange with lane^32               -> w_pack
+// One persistent workgroup per CU with H waves (two per SIMD for C = 256).  Wave h owns head h and keeps its
+// Wx | Wfx fragments (2 * KS * 4 = 128 registers for C = 256) in registers for the whole kernel: after the
+// prologue there is no weight traffic at all.  The x rows of a SET of TS tiles (TS * 32 points) are staged in LDS by
+// the whole workgroup with full-row coalesced loads; unit u (16 bytes) of row r is stored at r*UPR + (u ^ (r & 7)),
+// which makes both the row-wise writes and the fragment reads (row i, unit 2ks+g) bank-conflict free.  One fragment
+// read (1 KiB) feeds two MFMAs.  The set buffers are double buffered; the next set is fetched one tile at a time
+// into registers at the start of a tile and written to LDS at its end; one barrier per set.
+// The loop over sets is the only loop; its body has no branch around a memory operation (waves past the last tile
+// recompute it and re-store identical values).  The two waves of a SIMD drift apart, so one wave's MFMA phase
+// overlaps the other's softmax (VALU) phase.
 // ------------------------------------------------------------------------------------------------
-template <int C, int S, int WAVES>
-__global__ __launch_bounds__(WAVES * 64) void project_softmax_kernel(const u32x4 *__restrict__ blob, const uint16_t *__restrict__ x,
-                                                              u32x4 *__restrict__ fx_pack, u32x4 *__restrict__ w_pack,
-                                                              int64_t N, int tpb, int64_t total_tiles) {
+template <int C, int S>
+__global__ __launch_bounds__((C / 32) * 64) void project_softmax_kernel(const u32x4 *__restrict__ blob,
+                                                                        const uint16_t *__restrict__ x,
+                                                                        u32x4 *__restrict__ fx_pack,
+                                                                        u32x4 *__restrict__ w_pack, int64_t N, int tpb,
+                                                                        int64_t total_tiles) {
   constexpr int H = C / 32, KS = C / 16, ST = (S + 31) / 32, NCH = S / 16;
-  constexpr int HEAD_UNITS = 2 * KS * 64;  // 16-byte units of one head's weights
-  constexpr int NT = WAVES * 64;
-  constexpr int PER_THREAD = HEAD_UNITS / NT;
-  static_assert(HEAD_UNITS % NT == 0, "head weights must split evenly over the workgroup");
-  extern __shared__ u32x4 smem[];
-  u32x4 *wbuf = smem;                       // 2 * HEAD_UNITS
-  u32x4 *wsl = wbuf + 2 * HEAD_UNITS;       // ST * 2 * 64
-  float *fvec = reinterpret_cast<float *>(wsl + ST * 2 * 64);
-  float *bias_x = fvec, *bias_f = fvec + C, *bias_s = fvec + 2 * C, *tscale = fvec + 3 * C + ST * 32;
-  const BlobPlan bp = blob_plan(C, S);
-
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, i = lane & 31, g = lane >> 5;
-  // Persistent workgroup: tile sets blockIdx.x, blockIdx.x + gridDim.x, ...; a set is WAVES consecutive tiles.
-  // Waves past the last tile recompute it (identical values, identical stores): no divergent control flow.
-  const int64_t nsets = (total_tiles + WAVES - 1) / WAVES;
-  const int64_t nloc = (nsets - blockIdx.x + gridDim.x - 1) / gridDim.x;  // sets of this workgroup (>= 1)
-  int64_t set_cur = blockIdx.x, tile = 0, tile_nxt;
-  bool valid = false, valid_nxt;
-  u32x4 xf[KS];
-  // x fragments of the wave's 32 points of tile set `set` (zero rows beyond N) -> xf, tile_nxt, valid_nxt
-  auto load_x = [&](int64_t set) {
-    const int64_t traw = set * WAVES + wave;
-    tile_nxt = traw < total_tiles ? traw : total_tiles - 1;
-    const int64_t b = tile_nxt / tpb;
-    const int64_t n = (tile_nxt - b * tpb) * 32 + i;
-    valid_nxt = n < N;
-    const u32x4 *xr = reinterpret_cast<const u32x4 *>(x + ((int64_t)b * N + (valid_nxt ? n : 0)) * C) + g;
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      const u32x4 v = xr[2 * ks];
-      xf[ks] = valid_nxt ? v : u32x4{0, 0, 0, 0};
-    }
-  };
-  load_x(set_cur);
-  // small parameters and the first head's weights
-  for (int u = tid; u < ST * 2 * 64; u += NT) wsl[u] = blob[bp.wsl + u];
-  {
-    const float *src = reinterpret_cast<const float *>(blob + bp.fvec);
-    for (int k = tid; k < 3 * C + ST * 32 + H; k += NT) fvec[k] = src[k];
-  }
-#pragma unroll
-  for (int q = 0; q < PER_THREAD; ++q) wbuf[q * NT + tid] = blob[bp.win + q * NT + tid];
-  __syncthreads();
-  u32x4 wsf[ST][2];  // in_project_slice fragments: the same for every head
-#pragma unroll
-  for (int st = 0; st < ST; ++st) {
-    wsf[st][0] = wsl[(st * 2 + 0) * 64 + lane];
-    wsf[st][1] = wsl[(st * 2 + 1) * 64 + lane];
-  }
-
-  // ---- the two halves of one head's work -------------------------------------------------------------------
-  // products(h): both projections and the slice logits (MFMA bound)
-  auto products = [&](int buf, int h, u32x4 &fxp0, u32x4 &fxp1, f32x16(&lg)[ST]) {
-    const u32x4 *wb = wbuf + buf * HEAD_UNITS;
-    f32x16 ax, af;
-    {
-      const float bf = bias_f[h * 32 + i];
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        ax[r] = bias_x[h * 32 + rowmap(r, g)];
-        af[r] = bf;
-      }
-    }
-    // fragment reads run one group of GRP k-steps ahead of the products that use them
-    constexpr int GRP = 2, NG = KS / GRP;
-    static_assert(KS % GRP == 0, "k-steps must split into groups");
-    u32x4 fa[2][GRP], fb[2][GRP];
-#pragma unroll
-    for (int q = 0; q < GRP; ++q) {
-      fa[0][q] = wb[q * 64 + lane];
-      fb[0][q] = wb[(KS + q) * 64 + lane];
-    }
-    // the scheduling barriers keep the compiler from sinking the reads back next to their uses
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int grp = 0; grp < NG; ++grp) {
-      const int cur = grp & 1;
-      if (grp + 1 < NG) {
-#pragma unroll
-        for (int q = 0; q < GRP; ++q) {
-          fa[cur ^ 1][q] = wb[((grp + 1) * GRP + q) * 64 + lane];
-          fb[cur ^ 1][q] = wb[(KS + (grp + 1) * GRP + q) * 64 + lane];
-        }
-      }
-      __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int q = 0; q < GRP; ++q) {
-        ax = mma(fa[cur][q], xf[grp * GRP + q], ax);
-        af = mma(xf[grp * GRP + q], fb[cur][q], af);
-      }
-      __builtin_amdgcn_sched_barrier(0);
-    }
-    fxp0 = pack_half<0>(af);
-    fxp1 = pack_half<1>(af);
-    const u32x4 xb0 = pack_half<0>(ax), xb1 = pack_half<1>(ax);
-#pragma unroll
-    for (int st = 0; st < ST; ++st) {
-#pragma unroll
-      for (int r = 0; r < 16; ++r) lg[st][r] = bias_s[32 * st + rowmap(r, g)];
-      lg[st] = mma(wsf[st][0], xb0, lg[st]);
-      lg[st] = mma(wsf[st][1], xb1, lg[st]);
-    }
-  };
-  // softmax(h): temperature softmax over the slices of each point (VALU bound); packs the weights
-  auto softmax = [&](int h, f32x16(&lg)[ST], u32x4(&wp)[NCH]) {
-    float mx = -INFINITY;
-#pragma unroll
-    for (int st = 0; st < ST; ++st)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) mx = fmaxf(mx, lg[st][r]);
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-    const float sc = tscale[h];
-    const float off = mx * sc;
-    float sum = 0.f;
-#pragma unroll
-    for (int st = 0; st < ST; ++st)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const float e = __builtin_amdgcn_exp2f(fmaf(lg[st][r], sc, -off));
-        lg[st][r] = e;
-        sum += e;
-      }
-    sum += __shfl_xor(sum, 32, 64);
-    const float inv = valid ? __builtin_amdgcn_rcpf(sum) : 0.f;
-#pragma unroll
-    for (int st = 0; st < ST; ++st) {
-      if (2 * st < NCH) wp[2 * st < NCH ? 2 * st : 0] = pack_half<0>(lg[st], inv);
-      if (2 * st + 1 < NCH) wp[2 * st + 1 < NCH ? 2 * st + 1 : 0] = pack_half<1>(lg[st], inv);
-    }
-  };
-
-  // ---- H + 1 periods per tile set, one barrier each ------------------------------------------------------------
-  // The lower half of the waves runs products(p) then softmax(p); the upper half runs softmax(p-1) then products(p).
-  //
-  // Memory-operation order (vector-memory waits complete in issue order, so this order is what keeps the waits
-  // short): the weights of the head needed two periods later are loaded into registers AFTER the copy of the
-  // previously loaded set into the free LDS buffer and BEFORE this period's global stores.  The wait in front of
-  // that copy therefore never covers the stores of the period before, and the stores of w / fx_mid drain in the
-  // background.  Two register sets alternate, so the loop advances two periods per trip.  The x fragments of the
-  // next tile set are fetched in period H-1, right after their last use, and land during period H.  Every store
-  // is issued unconditionally (periods without a new result re-store the previous one), which keeps the loop
-  // body free of branches around stores.
-  constexpr int P = H + 1;
-  const bool late = wave >= WAVES / 2;
-  f32x16 lg[ST];
-  u32x4 fxp0 = {0, 0, 0, 0}, fxp1 = {0, 0, 0, 0}, wp[NCH];
-#pragma unroll
-  for (int cq = 0; cq < NCH; ++cq) wp[cq] = u32x4{0, 0, 0, 0};
-  u32x4 nA[PER_THREAD], nB[PER_THREAD];
-  {
-    const int h1 = H > 1 ? 1 : 0;
-#pragma unroll
-    for (int q = 0; q < PER_THREAD; ++q) nA[q] = blob[bp.win + (int64_t)h1 * HEAD_UNITS + q * NT + tid];
-    // placeholder stores (overwritten by periods 0 / 1): give the loop entry the same pending-store state as the
-    // loop back-edge so that the first wait of the loop is as short as all the others
-    u32x4 *fdst = fx_pack + ((tile_nxt * H + 0) * 2) * 64 + lane;
-    fdst[0] = fxp0;
-    fdst[64] = fxp1;
-    u32x4 *wdst = w_pack + ((tile_nxt * H + 0) * NCH) * 64 + lane;
-#pragma unroll
-    for (int cq = 0; cq < NCH; ++cq) wdst[cq * 64] = wp[cq];
-  }
-  // head whose weights period q needs (period H of a set has no products; it keeps the last head's)
-  auto head_of = [&](int64_t q) {
-    const int p = (int)(q % P);
-    return p < H ? p : H - 1;
-  };
-  auto period = [&](int64_t q, u32x4(&n_ready)[PER_THREAD], u32x4(&n_load)[PER_THREAD]) {
-    const int p = (int)(q % P);
-    if (p == 0) {  // a new tile set starts: its x fragments were issued in period H-1 of the previous one
-      tile = tile_nxt;
-      valid = valid_nxt;
-    }
-    int h_w;
-    if (!late) {
-      if (p < H) {
-        products((int)(q & 1), p, fxp0, fxp1, lg);
-        softmax(p, lg, wp);
-      }
-      h_w = p < H ? p : H - 1;
-    } else {
-      if (p > 0) softmax(p - 1, lg, wp);
-      if (p < H) products((int)(q & 1), p, fxp0, fxp1, lg);
-      h_w = p > 0 ? p - 1 : 0;
-    }
-    const int h_f = p < H ? p : H - 1;
-    {
-      u32x4 *dst = wbuf + ((q + 1) & 1) * HEAD_UNITS;
-#pragma unroll
-      for (int k = 0; k < PER_THREAD; ++k) dst[k * NT + tid] = n_ready[k];
-    }
-    const int h2 = head_of(q + 2);
-#pragma unroll
-    for (int k = 0; k < PER_THREAD; ++k) n_load[k] = blob[bp.win + (int64_t)h2 * HEAD_UNITS + k * NT + tid];
-    u32x4 *fdst = fx_pack + ((tile * H + h_f) * 2) * 64 + lane;
-    fdst[0] = fxp0;
-    fdst[64] = fxp1;
-    u32x4 *wdst = w_pack + ((tile * H + h_w) * NCH) * 64 + lane;
-#pragma unroll
-    for (int cq = 0; cq < NCH; ++cq) wdst[cq * 64] = wp[cq];
-    if (p == H - 1) {  // last use of xf is behind us: fetch the next set's (the last set re-fetches its own)
-      const int64_t set_next = set_cur + gridDim.x < nsets ? set_cur + gridDim.x : set_cur;
-      load_x(set_next);
-      set_cur = set_next;
-    }
-    __syncthreads();
-  };
-  const int64_t Q = nloc * P;
-  for (int64_t q = 0; q < Q; q += 2) {
-    period(q, nA, nB);
-    if (q + 1 < Q) period(q + 1, nB, nA);
-  }
-}
-
-// ------------------------------------------------------------------------------------------------
-// Kernel (a), weights-stationary form.  One persistent workgroup per CU, H waves (two per SIMD for C = 256), each
-// wave owns ONE head and keeps its Wx | Wfx fragments (2 * KS * 4 = 128 VGPRs for C = 256) in registers for the
-// whole kernel: no weight traffic at all after the prologue.  The x rows of a SET of TS tiles (TS * 32 points) are staged in LDS
-// by the whole workgroup with full-row coalesced loads; unit u (16 bytes) of row r is stored at r*UPR + (u ^ (r&7)),
-// which makes both the row-wise writes and the fragment reads (row i, unit 2ks+g) bank-conflict free.  One x
-// fragment read (1 KiB) feeds 2 MFMAs of a head, i.e. 0.5 KiB of LDS per MFMA (the tile-stationary form needs 1).
-// The set buffers are double buffered; the next set is fetched one tile at a time into 4 registers per thread at
-// the start of a tile and written to LDS at its end; one barrier per set.
-//
-// Inside a wave the work is a chain of head-steps, one per tile:  products(t) [MFMA]  interleaved with the
-// softmax + stores of the previous head-step [VALU, VMEM].
-// The loop over sets is the only loop; its body has no branch around a memory operation (waves past the last
-// tile recompute it and re-store identical values; the very first softmax runs on zero logits and is overwritten).
-// ------------------------------------------------------------------------------------------------
-template <int C, int S, int HPW>
-__global__ __launch_bounds__((C / 32 / HPW) * 64) void project_softmax_ws_kernel(const u32x4 *__restrict__ blob,
-                                                                           const uint16_t *__restrict__ x,
-                                                                           u32x4 *__restrict__ fx_pack,
-                                                                           u32x4 *__restrict__ w_pack, int64_t N, int tpb,
-                                                                           int64_t total_tiles) {
-  constexpr int H = C / 32, KS = C / 16, ST = (S + 31) / 32, NCH = S / 16;
-  constexpr int WAVES = H / HPW, NT = WAVES * 64;
+  constexpr int WAVES = H, NT = WAVES * 64;
   constexpr int TS = 4;                 // tiles per set
   constexpr int UPR = C / 8;            // 16-byte units per row
   constexpr int SET_UNITS = TS * 32 * UPR;
@@ -387,31 +159,29 @@ __global__ __launch_bounds__((C / 32 / HPW) * 64) void project_softmax_ws_kernel
   float *bias_x = fvec, *bias_f = fvec + C, *bias_s = fvec + 2 * C, *tscale = fvec + 3 * C + ST * 32;
   const BlobPlan bp = blob_plan(C, S);
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, i = lane & 31, g = lane >> 5;
+  const int h = wave;
 
-  // this wave's head: Wx (A operand of x_mid^T) and Wfx (B operand of fx_mid), register resident
-  u32x4 wx[HPW][KS], wf[HPW][KS];
+  u32x4 wx[KS], wf[KS];
 #pragma unroll
-  for (int hh = 0; hh < HPW; ++hh)
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      const int64_t base = bp.win + ((int64_t)(HPW * wave + hh) * 2) * KS * 64;
-      wx[hh][ks] = blob[base + ks * 64 + lane];
-      wf[hh][ks] = blob[base + (KS + ks) * 64 + lane];
-    }
+  for (int ks = 0; ks < KS; ++ks) {
+    const int64_t base = bp.win + ((int64_t)h * 2) * KS * 64;
+    wx[ks] = blob[base + ks * 64 + lane];
+    wf[ks] = blob[base + (KS + ks) * 64 + lane];
+  }
   for (int u = tid; u < ST * 2 * 64; u += NT) wsl[u] = blob[bp.wsl + u];
   {
     const float *src = reinterpret_cast<const float *>(blob + bp.fvec);
     for (int k = tid; k < 3 * C + ST * 32 + H; k += NT) fvec[k] = src[k];
   }
 
+  const int ntiles = (int)total_tiles;  // < 2^28 (checked on the host)
   const int64_t nsets = (total_tiles + TS - 1) / TS;
   const int64_t nloc = (nsets - blockIdx.x + gridDim.x - 1) / gridDim.x;
-  const int ntiles = (int)total_tiles;  // < 2^28 (checked on the host)
   auto tile_of = [&](int64_t set, int t) {
     const int tr = (int)set * TS + t;
     return tr < ntiles ? tr : ntiles - 1;
   };
-  // staging: this thread's CHUNK units of tile (set, t): unit k*NT + tid -> row rc, position pos
+  // staging: this thread's CHUNK units of tile (set, t): unit k*NT + tid -> row rc, position pos (zero rows beyond N)
   auto stage_load = [&](int64_t set, int t, u32x4(&st)[CHUNK]) {
     const int tile = tile_of(set, t);
     const int b = tile / tpb;
@@ -433,177 +203,97 @@ __global__ __launch_bounds__((C / 32 / HPW) * 64) void project_softmax_ws_kernel
       xs[buf * SET_UNITS + (t * 32 + rc) * UPR + (pos ^ (rc & 7))] = st[k];
     }
   };
-  {  // first set
-    int64_t set0 = blockIdx.x;
 #pragma unroll
-    for (int t = 0; t < TS; ++t) {
-      u32x4 st[CHUNK];
-      stage_load(set0, t, st);
-      stage_store(0, t, st);
-    }
+  for (int t = 0; t < TS; ++t) {  // first set
+    u32x4 st[CHUNK];
+    stage_load(blockIdx.x, t, st);
+    stage_store(0, t, st);
   }
   __syncthreads();
-
-
-  // state of the previous head-step (its logits still need the softmax)
-  f32x16 lg[ST];
-#pragma unroll
-  for (int st = 0; st < ST; ++st)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) lg[st][r] = 0.f;
-  int tile_prev = tile_of(blockIdx.x, 0);
-  int h_prev = HPW * wave;
-  bool valid_prev = false;
-
-  auto softmax_store = [&]() {
-    float mx = -INFINITY;
-#pragma unroll
-    for (int st = 0; st < ST; ++st)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) mx = fmaxf(mx, lg[st][r]);
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-    const float sc = tscale[h_prev];
-    const float off = mx * sc;
-    float sum = 0.f;
-#pragma unroll
-    for (int st = 0; st < ST; ++st)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const float e = __builtin_amdgcn_exp2f(fmaf(lg[st][r], sc, -off));
-        lg[st][r] = e;
-        sum += e;
-      }
-    sum += __shfl_xor(sum, 32, 64);
-    const float inv = valid_prev ? __builtin_amdgcn_rcpf(sum) : 0.f;
-    u32x4 *wdst = w_pack + (((int64_t)tile_prev * H + h_prev) * NCH) * 64 + lane;
-#pragma unroll
-    for (int st = 0; st < ST; ++st) {
-      if (2 * st < NCH) wdst[(2 * st) * 64] = pack_half<0>(lg[st], inv);
-      if (2 * st + 1 < NCH) wdst[(2 * st + 1) * 64] = pack_half<1>(lg[st], inv);
-    }
-  };
-
-  // One head-step: products of the tile at slot t of buffer buf (this wave's head) interleaved, MFMA by MFMA, with the
-  // softmax + stores of the PREVIOUS head-step (whose logits are in lg).  The 2*KS projection MFMAs form 2*KS units;
-  // each unit is one MFMA plus a slice of the softmax small enough to run in its shadow, and a scheduling barrier
-  // closes the unit so the compiler keeps this mix:
-  //   units [0, UA)        running maximum over the logits         (then one exchange with lane^32)
-  //   units [UA, UA+UB)    exp2 and running sum                    (then one exchange, reciprocal)
-  //   units [UA+UB, 2*KS)  scale, convert to bf16, store each finished 16-slice chunk
-  // Afterwards lg is free and receives this step's logits.
-  auto head_step = [&](int buf, int t, int hh, int tile) {
-    const int h = HPW * wave + hh;
-    constexpr int U = 2 * KS, R = ST * 16;           // units, logit registers per lane
-    constexpr int UA = U / 4, UB = U / 2, UC = U - UA - UB;
-    constexpr int RA = (R + UA - 1) / UA, RB = (R + UB - 1) / UB, RC = (R + UC - 1) / UC;
-    constexpr int RING = 3, AHEAD = 2;               // x fragments are read AHEAD k-steps early
-    const u32x4 *xb = xs + buf * SET_UNITS + (t * 32 + i) * UPR;
-    f32x16 ax, af;
-    {
-      const float bf = bias_f[h * 32 + i];
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        ax[r] = bias_x[h * 32 + rowmap(r, g)];
-        af[r] = bf;
-      }
-    }
-    u32x4 xf[RING];
-#pragma unroll
-    for (int q = 0; q < AHEAD; ++q) xf[q] = xb[(2 * q + g) ^ (i & 7)];
-    const float sc = tscale[h_prev];
-    float mx = -INFINITY, off = 0.f, sum = 0.f, inv = 0.f;
-    u32x4 *wdst = w_pack + (((int64_t)tile_prev * H + h_prev) * NCH) * 64 + lane;
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int ks = u >> 1;
-      if ((u & 1) == 0) {
-        if (ks + AHEAD < KS) xf[(ks + AHEAD) % RING] = xb[(2 * (ks + AHEAD) + g) ^ (i & 7)];
-        ax = mma(wx[hh][ks], xf[ks % RING], ax);
-      } else {
-        af = mma(xf[ks % RING], wf[hh][ks], af);
-      }
-      if (u < UA) {
-#pragma unroll
-        for (int k = 0; k < RA; ++k) {
-          const int r = u * RA + k;
-          if (r < R) mx = fmaxf(mx, lg[r >> 4][r & 15]);
-        }
-        if (u == UA - 1) {
-          mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-          off = mx * sc;
-        }
-      } else if (u < UA + UB) {
-#pragma unroll
-        for (int k = 0; k < RB; ++k) {
-          const int r = (u - UA) * RB + k;
-          if (r < R) {
-            const float e = __builtin_amdgcn_exp2f(fmaf(lg[r >> 4][r & 15], sc, -off));
-            lg[r >> 4][r & 15] = e;
-            sum += e;
-          }
-        }
-        if (u == UA + UB - 1) {
-          sum += __shfl_xor(sum, 32, 64);
-          inv = valid_prev ? __builtin_amdgcn_rcpf(sum) : 0.f;
-        }
-      } else {
-#pragma unroll
-        for (int k = 0; k < RC; ++k) {
-          const int r = (u - UA - UB) * RC + k;
-          if (r < R) {
-            lg[r >> 4][r & 15] *= inv;
-            if ((r & 7) == 7 && (r >> 3) < NCH) {  // chunk r/8 complete
-              if (((r >> 3) & 1) == 0) wdst[(r >> 3) * 64] = pack_half<0>(lg[r >> 4]);
-              else wdst[(r >> 3) * 64] = pack_half<1>(lg[r >> 4]);
-            }
-          }
-        }
-      }
-      __builtin_amdgcn_sched_barrier(0);
-    }
-    u32x4 *fdst = fx_pack + (((int64_t)tile * H + h) * 2) * 64 + lane;
-    fdst[0] = pack_half<0>(af);
-    fdst[64] = pack_half<1>(af);
-    const u32x4 xb0 = pack_half<0>(ax), xb1 = pack_half<1>(ax);
-#pragma unroll
-    for (int st = 0; st < ST; ++st) {
-#pragma unroll
-      for (int r = 0; r < 16; ++r) lg[st][r] = bias_s[32 * st + rowmap(r, g)];
-      lg[st] = mma(wsl[(st * 2 + 0) * 64 + lane], xb0, lg[st]);
-      lg[st] = mma(wsl[(st * 2 + 1) * 64 + lane], xb1, lg[st]);
-    }
-  };
 
   int64_t set = blockIdx.x;
   for (int64_t sl = 0; sl < nloc; ++sl) {
     const int buf = (int)(sl & 1);
     const int64_t set_next = set + gridDim.x < nsets ? set + gridDim.x : set;  // the last set re-fetches itself
-    // head-major order inside a set: a head's weights are used for TS consecutive head-steps
 #pragma unroll
-    for (int hh = 0; hh < HPW; ++hh) {
+    for (int t = 0; t < TS; ++t) {
+      __builtin_amdgcn_sched_barrier(0);  // keep each tile's work (and its register live ranges) to itself
+      u32x4 stg[CHUNK];
+      stage_load(set_next, t, stg);
+      __builtin_amdgcn_sched_barrier(0);
+      const int tile = tile_of(set, t);
+      const int b = tile / tpb;
+      const bool valid = (int64_t)(tile - b * tpb) * 32 + i < N;
+
+      // ---- products ----
+      const u32x4 *xb = xs + buf * SET_UNITS + (t * 32 + i) * UPR;
+      f32x16 ax, af;
+      {
+        const float bf = bias_f[h * 32 + i];
 #pragma unroll
-      for (int t = 0; t < TS; ++t) {
-        __builtin_amdgcn_sched_barrier(0);  // keep each head-step's work (and its register live ranges) to itself
-        u32x4 stg[CHUNK];
-        if (hh == HPW - 1) stage_load(set_next, t, stg);
-        __builtin_amdgcn_sched_barrier(0);
-        const int tile = tile_of(set, t);
-        const int b = tile / tpb;
-        const bool valid = (int64_t)(tile - b * tpb) * 32 + i < N;
-        head_step(buf, t, hh, tile);
-        tile_prev = tile;
-        h_prev = HPW * wave + hh;
-        valid_prev = valid;
-        __builtin_amdgcn_sched_barrier(0);
-        if (hh == HPW - 1) stage_store(buf ^ 1, t, stg);
-        __builtin_amdgcn_sched_barrier(0);
+        for (int r = 0; r < 16; ++r) {
+          ax[r] = bias_x[h * 32 + rowmap(r, g)];
+          af[r] = bf;
+        }
       }
+      constexpr int RING = 3, AHEAD = 2;  // x fragments are read AHEAD k-steps before the MFMAs that use them
+      u32x4 xf[RING];
+#pragma unroll
+      for (int q = 0; q < AHEAD; ++q) xf[q] = xb[(2 * q + g) ^ (i & 7)];
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        if (ks + AHEAD < KS) xf[(ks + AHEAD) % RING] = xb[(2 * (ks + AHEAD) + g) ^ (i & 7)];
+        ax = mma(wx[ks], xf[ks % RING], ax);
+        af = mma(xf[ks % RING], wf[ks], af);
+        __builtin_amdgcn_sched_barrier(0);  // keeps the compiler from sinking the reads back next to their uses
+      }
+      u32x4 *fdst = fx_pack + (((int64_t)tile * H + h) * 2) * 64 + lane;
+      fdst[0] = pack_half<0>(af);
+      fdst[64] = pack_half<1>(af);
+      const u32x4 xb0 = pack_half<0>(ax), xb1 = pack_half<1>(ax);
+      f32x16 lg[ST];
+#pragma unroll
+      for (int st = 0; st < ST; ++st) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) lg[st][r] = bias_s[32 * st + rowmap(r, g)];
+        lg[st] = mma(wsl[(st * 2 + 0) * 64 + lane], xb0, lg[st]);
+        lg[st] = mma(wsl[(st * 2 + 1) * 64 + lane], xb1, lg[st]);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+
+      // ---- softmax over the slices of each point, in the base-2 domain: w = exp2((l - max) * log2e / T) / sum ----
+      float mx = -INFINITY;
+#pragma unroll
+      for (int st = 0; st < ST; ++st)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) mx = fmaxf(mx, lg[st][r]);
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      const float sc = tscale[h];
+      const float off = mx * sc;
+      float sum = 0.f;
+#pragma unroll
+      for (int st = 0; st < ST; ++st)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const float e = __builtin_amdgcn_exp2f(fmaf(lg[st][r], sc, -off));
+          lg[st][r] = e;
+          sum += e;
+        }
+      sum += __shfl_xor(sum, 32, 64);
+      const float inv = valid ? __builtin_amdgcn_rcpf(sum) : 0.f;  // rows beyond N get zero weight
+      u32x4 *wdst = w_pack + (((int64_t)tile * H + h) * NCH) * 64 + lane;
+#pragma unroll
+      for (int st = 0; st < ST; ++st) {
+        if (2 * st < NCH) wdst[(2 * st) * 64] = pack_half<0>(lg[st], inv);
+        if (2 * st + 1 < NCH) wdst[(2 * st + 1) * 64] = pack_half<1>(lg[st], inv);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      stage_store(buf ^ 1, t, stg);
+      __builtin_amdgcn_sched_barrier(0);
     }
     set = set_next;
     __syncthreads();
   }
-  softmax_store();  // the last head-step
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -958,56 +648,28 @@ int pack_params(const pa_shape &s, const pa_params &p, void *blob, hipStream_t s
   return launch_status();
 }
 
-template <int C, int S, int WAVES>
-static int project_softmax_w(const pa_shape &s, const void *blob, const void *x, void *fx_pack, void *w_pack,
-                             int num_cu, hipStream_t st) {
-  constexpr int KS = C / 16, ST = (S + 31) / 32, H = C / 32;
-  const size_t lds = (size_t)(2 * 2 * KS * 64 + ST * 2 * 64) * 16 + (size_t)(3 * C + ST * 32 + H) * 4;
-  int rc = allow_dynamic_lds(project_softmax_kernel<C, S, WAVES>, lds);
-  if (rc) return rc;
-  const int64_t tpb = tiles_per_batch(s), total = tpb * s.B;
-  int64_t grid = (total + WAVES - 1) / WAVES;
-  if (grid > num_cu) grid = num_cu;  // one persistent workgroup per CU
-  hipLaunchKernelGGL((project_softmax_kernel<C, S, WAVES>), dim3((unsigned)grid), dim3(WAVES * 64),
-                     lds, st, static_cast<const u32x4 *>(blob), static_cast<const uint16_t *>(x),
-                     static_cast<u32x4 *>(fx_pack), static_cast<u32x4 *>(w_pack), s.N, (int)tpb, total);
-  return launch_status();
-}
-
-template <int C, int S, int HPW>
-static int project_softmax_ws(const pa_shape &s, const void *blob, const void *x, void *fx_pack, void *w_pack,
+template <int C, int S>
+static int project_softmax_cs(const pa_shape &s, const void *blob, const void *x, void *fx_pack, void *w_pack,
                               int num_cu, hipStream_t st) {
-  constexpr int ST = (S + 31) / 32, H = C / 32, TS = 4, UPR = C / 8, WAVES = H / HPW;
+  constexpr int ST = (S + 31) / 32, H = C / 32, TS = 4, UPR = C / 8, WAVES = H;
   const size_t lds = (size_t)(2 * TS * 32 * UPR + ST * 2 * 64) * 16 + (size_t)(3 * C + ST * 32 + H) * 4;
-  int rc = allow_dynamic_lds(project_softmax_ws_kernel<C, S, HPW>, lds);
+  int rc = allow_dynamic_lds(project_softmax_kernel<C, S>, lds);
   if (rc) return rc;
   const int64_t tpb = tiles_per_batch(s), total = tpb * s.B;
   static int per_cu = 0;  // resident workgroups per CU for this instantiation
   if (per_cu == 0) {
     int nb = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, project_softmax_ws_kernel<C, S, HPW>, WAVES * 64, lds) != hipSuccess ||
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, project_softmax_kernel<C, S>, WAVES * 64, lds) != hipSuccess ||
         nb < 1)
       nb = 1;
     per_cu = nb;
   }
   int64_t grid = (total + TS - 1) / TS;
   if (grid > (int64_t)num_cu * per_cu) grid = (int64_t)num_cu * per_cu;
-  hipLaunchKernelGGL((project_softmax_ws_kernel<C, S, HPW>), dim3((unsigned)grid), dim3(WAVES * 64), lds, st,
+  hipLaunchKernelGGL((project_softmax_kernel<C, S>), dim3((unsigned)grid), dim3(WAVES * 64), lds, st,
                      static_cast<const u32x4 *>(blob), static_cast<const uint16_t *>(x), static_cast<u32x4 *>(fx_pack),
                      static_cast<u32x4 *>(w_pack), s.N, (int)tpb, total);
   return launch_status();
-}
-
-template <int C, int S>
-static int project_softmax_cs(const pa_shape &s, const void *blob, const void *x, void *fx_pack, void *w_pack,
-                              int num_cu, hipStream_t st) {
-  static const int form = [] {
-    const char *e = getenv("PA_KA_FORM");
-    return e ? atoi(e) : 1;
-  }();
-  if (form == 1) return project_softmax_ws<C, S, 2>(s, blob, x, fx_pack, w_pack, num_cu, st);
-  if (form == 2) return project_softmax_ws<C, S, 1>(s, blob, x, fx_pack, w_pack, num_cu, st);
-  return project_softmax_w<C, S, 8>(s, blob, x, fx_pack, w_pack, num_cu, st);
 }
 
 template <int S>
