@@ -181,33 +181,34 @@ __global__ __launch_bounds__((C / 32) * 64) void project_softmax_kernel(const u3
     const int tr = (int)set * TS + t;
     return tr < ntiles ? tr : ntiles - 1;
   };
-  // staging: this thread's CHUNK units of tile (set, t): unit k*NT + tid -> row rc, position pos (zero rows beyond N)
-  auto stage_load = [&](int64_t set, int t, u32x4(&st)[CHUNK]) {
+  // staging: this thread's CHUNK units of tile (set, t): unit k*NT + tid -> row rc, position pos.  The load only
+  // issues (rows beyond N re-read row 0 of the tile); the values are first touched in stage_store, a whole tile of
+  // work later, where rows beyond N are replaced by zeros.
+  auto stage_load = [&](int64_t set, int t, u32x4(&st)[CHUNK], int &rows_ok) {
     const int tile = tile_of(set, t);
     const int b = tile / tpb;
     const int n0 = (tile - b * tpb) * 32;
     const uint16_t *xbase = x + ((int64_t)b * N + n0) * C;
-    const int rows_ok = (int)min((int64_t)32, N - n0);
+    rows_ok = (int)min((int64_t)32, N - n0);
 #pragma unroll
     for (int k = 0; k < CHUNK; ++k) {
       const int idx = k * NT + tid, rc = idx / UPR, pos = idx - rc * UPR;
-      const bool ok = rc < rows_ok;
-      const u32x4 v = *reinterpret_cast<const u32x4 *>(xbase + (ok ? rc : 0) * C + pos * 8);
-      st[k] = ok ? v : u32x4{0, 0, 0, 0};
+      st[k] = *reinterpret_cast<const u32x4 *>(xbase + (rc < rows_ok ? rc : 0) * C + pos * 8);
     }
   };
-  auto stage_store = [&](int buf, int t, const u32x4(&st)[CHUNK]) {
+  auto stage_store = [&](int buf, int t, const u32x4(&st)[CHUNK], int rows_ok) {
 #pragma unroll
     for (int k = 0; k < CHUNK; ++k) {
       const int idx = k * NT + tid, rc = idx / UPR, pos = idx - rc * UPR;
-      xs[buf * SET_UNITS + (t * 32 + rc) * UPR + (pos ^ (rc & 7))] = st[k];
+      xs[buf * SET_UNITS + (t * 32 + rc) * UPR + (pos ^ (rc & 7))] = rc < rows_ok ? st[k] : u32x4{0, 0, 0, 0};
     }
   };
 #pragma unroll
   for (int t = 0; t < TS; ++t) {  // first set
     u32x4 st[CHUNK];
-    stage_load(blockIdx.x, t, st);
-    stage_store(0, t, st);
+    int rows_ok;
+    stage_load(blockIdx.x, t, st, rows_ok);
+    stage_store(0, t, st, rows_ok);
   }
   __syncthreads();
 
@@ -219,7 +220,8 @@ __global__ __launch_bounds__((C / 32) * 64) void project_softmax_kernel(const u3
     for (int t = 0; t < TS; ++t) {
       __builtin_amdgcn_sched_barrier(0);  // keep each tile's work (and its register live ranges) to itself
       u32x4 stg[CHUNK];
-      stage_load(set_next, t, stg);
+      int stg_rows;
+      stage_load(set_next, t, stg, stg_rows);
       __builtin_amdgcn_sched_barrier(0);
       const int tile = tile_of(set, t);
       const int b = tile / tpb;
@@ -288,7 +290,7 @@ __global__ __launch_bounds__((C / 32) * 64) void project_softmax_kernel(const u3
         if (2 * st + 1 < NCH) wdst[(2 * st + 1) * 64] = pack_half<1>(lg[st], inv);
       }
       __builtin_amdgcn_sched_barrier(0);
-      stage_store(buf ^ 1, t, stg);
+      stage_store(buf ^ 1, t, stg, stg_rows);
       __builtin_amdgcn_sched_barrier(0);
     }
     set = set_next;
