@@ -4,7 +4,7 @@
 Default workload (the configuration the headline metric is quoted on): one PhysicsAttentionIrregularMesh layer,
 bf16, B=1, N=1,048,576 points, C=256, 8 heads (D=32), slice_num=64, synthetic N(0,1) input (seed 1234),
 seeded random weights (seed 0, orthogonal slice projection).  A "step" is one full layer forward through
-the C ABI (parameter repack + kernels a, b, combine/attention, d), inputs resident in HBM.
+the C ABI (parameter repack + kernels a+b fused, combine/attention, d), inputs resident in HBM.
 
 Prints ONE JSON line: whole-layer Mpoints/s, the roofline of the dominant kernel (measured live with events on
 the launch stream), per-kernel figures, and the CPU baseline (the oracle's ATen op sequence timed on the host
@@ -48,6 +48,7 @@ def parse_args():
 def algorithmic_bytes_per_point(C, H, S, b=2):
     """Bytes each kernel must move per point when every tensor is read / written once (bf16)."""
     return {
+        "project_softmax_reduce": (C + H * S) * b,  # read x; write w (fx_mid stays on chip)
         "project_softmax": (C + C + H * S) * b,   # read x; write fx_mid, w
         "slice_reduce": (H * S + C) * b,          # read w, fx_mid
         "deslice_project": (H * S + C) * b,       # read w; write y   (+C*b per extra residual / LayerNorm tensor)
@@ -56,6 +57,7 @@ def algorithmic_bytes_per_point(C, H, S, b=2):
 
 def mfma_flops_per_point(C, S):
     return {
+        "project_softmax_reduce": 4 * C * C + 4 * C * S,  # two projections + slice logits + aggregation
         "project_softmax": 4 * C * C + 2 * C * S,  # two projections + slice logits
         "slice_reduce": 2 * C * S,                 # aggregation
         "deslice_project": 2 * C * S + 2 * C * C,  # deslice + out_linear
@@ -199,13 +201,22 @@ def main():
         st = PF.MfmaStages(params, dims, dev)
         yk = torch.empty_like(x)
         st.pack_params()
-        stage_fns = {
-            "project_softmax": lambda: st.project_softmax(x),
-            "slice_reduce": st.slice_reduce,
+        fused = st.fused_groups > 0  # the layer call runs kernels (a)+(b) as one launch
+        stage_fns = {}
+        if fused:  # the separate kernels first, so that the later stages time on the layer path's partials
+            stage_fns["project_softmax"] = lambda: st.project_softmax(x)
+            stage_fns["slice_reduce"] = st.slice_reduce
+            stage_fns["project_softmax_reduce"] = lambda: st.project_softmax_reduce(x)
+        else:
+            stage_fns["project_softmax"] = lambda: st.project_softmax(x)
+            stage_fns["slice_reduce"] = st.slice_reduce
+        stage_fns.update({
             "combine_attention": st.combine_attention,
             "deslice_project": lambda: st.deslice_project(yk),
             "pack_params": st.pack_params,
-        }
+        })
+        on_path = ({"project_softmax_reduce", "deslice_project"} if fused else
+                   {"project_softmax", "slice_reduce", "deslice_project"})
         bytes_pp = algorithmic_bytes_per_point(C, H, S)
         flops_pp = mfma_flops_per_point(C, S)
         for name, fn in stage_fns.items():
@@ -217,11 +228,12 @@ def main():
                 entry.update({"algorithmic_bytes": bytes_pp[name] * B * N, "hbm_gbs": round(gbs, 1),
                               "hbm_frac": round(gbs / HBM_PEAK_GBS, 4), "mfma_tflops": round(tf, 1),
                               "mfma_frac": round(tf / MFMA_BF16_PEAK_TF, 4)})
+            entry["on_layer_path"] = name in on_path or name in ("combine_attention", "pack_params")
             kernels[name] = entry
-        dominant = max(bytes_pp, key=lambda k: kernels[k]["ms"])
+        dominant = max(on_path, key=lambda k: kernels[k]["ms"])
         # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a 1 GiB copy (x2.0 / x1.0);
         # measured for the default workload only (profiles/layer_cfg3_s64_hbm_traffic.md)
-        measured_traffic = {"project_softmax": (549 + 1536) << 20, "slice_reduce": (1536 + 8) << 20,
+        measured_traffic = {"project_softmax_reduce": None, "project_softmax": (549 + 1536) << 20, "slice_reduce": (1536 + 8) << 20,
                             "deslice_project": (1025 + 512) << 20}
         default_workload = (B, N, C, S) == (1, 1 << 20, 256, 64)
         roofline = {"kernel": dominant, "bound": "hbm", "achieved": kernels[dominant]["hbm_gbs"], "peak": HBM_PEAK_GBS,

@@ -155,10 +155,19 @@ int pa_mfma_project_softmax(const pa_shape *shape, const void *blob, const void 
 /* Kernel (b): first pass of the slice aggregation (PA.py:185-203) -> partials. */
 int pa_mfma_slice_reduce(const pa_shape *shape, const void *w_pack, const void *fx_pack, float *partials,
                          void *stream);
+/* Kernels (a)+(b) in one launch (S <= 64): projections, slice softmax and the first pass of the slice aggregation
+ * (PA.py:529-537, :172-181, :185-203); fx_mid never leaves the chip. Writes w_pack and partials. This is what
+ * pa_layer_forward runs when it applies; PA_ERR_UNSUPPORTED otherwise. */
+int pa_mfma_project_softmax_reduce(const pa_shape *shape, const void *blob, const void *x, void *w_pack,
+                                   float *partials, void *stream);
+/* Number of partial sums a first pass leaves in `partials`: fused = 1 for pa_mfma_project_softmax_reduce (or
+ * PA_ERR_UNSUPPORTED where it does not apply), 0 for pa_mfma_slice_reduce. Pass it to pa_mfma_combine_attention. */
+int64_t pa_mfma_partial_groups(const pa_shape *shape, int fused);
 /* Second pass + kernel (c): fixed-order combine, normalisation, slice attention (PA.py:185-203, :429-465).
- * slice_token / slice_norm may be NULL. Writes out_slice_token (B,H,S,D) float32 and its packed copy tokp. */
-int pa_mfma_combine_attention(const pa_shape *shape, const pa_params *p, const float *partials, float *slice_token,
-                              float *slice_norm, float *out_slice_token, void *tokp, void *stream);
+ * groups = pa_mfma_partial_groups() of the producer. slice_token / slice_norm may be NULL. Writes out_slice_token (B,H,S,D) float32 and its packed copy tokp. */
+int pa_mfma_combine_attention(const pa_shape *shape, const pa_params *p, const float *partials, int64_t groups,
+                              float *slice_token, float *slice_norm, float *out_slice_token, void *tokp,
+                              void *stream);
 /* Kernel (d): deslice + out_linear + optional residual / LayerNorm tail (PA.py:467-499, TR.py:300-303). */
 int pa_mfma_deslice_project(const pa_shape *shape, const void *blob, const void *w_pack, const void *tokp, void *y,
                             const pa_block_tail *tail, void *stream);

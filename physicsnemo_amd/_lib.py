@@ -19,7 +19,8 @@ EXPORTED = [
     "pa_version", "pa_status_string", "pa_workspace_bytes", "pa_query_path", "pa_project_inputs",
     "pa_slice_softmax", "pa_reduce_partial_count", "pa_slice_reduce", "pa_slice_attention",
     "pa_deslice_project", "pa_layer_forward", "pa_mfma_buffer_bytes", "pa_mfma_pack_params",
-    "pa_mfma_project_softmax", "pa_mfma_slice_reduce", "pa_mfma_combine_attention", "pa_mfma_deslice_project",
+    "pa_mfma_project_softmax", "pa_mfma_slice_reduce", "pa_mfma_project_softmax_reduce", "pa_mfma_partial_groups",
+     "pa_mfma_combine_attention", "pa_mfma_deslice_project",
 ]
 
 PA_BUF_BLOB, PA_BUF_FX_PACK, PA_BUF_W_PACK, PA_BUF_PARTIALS, PA_BUF_TOKP = range(5)
@@ -86,7 +87,11 @@ def load() -> ctypes.CDLL:
     lib.pa_mfma_slice_reduce.restype = c_int
     lib.pa_mfma_slice_reduce.argtypes = [ps, c_void_p, c_void_p, c_void_p, c_void_p]
     lib.pa_mfma_combine_attention.restype = c_int
-    lib.pa_mfma_combine_attention.argtypes = [ps, pp, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]
+    lib.pa_mfma_combine_attention.argtypes = [ps, pp, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]
+    lib.pa_mfma_project_softmax_reduce.restype = c_int
+    lib.pa_mfma_project_softmax_reduce.argtypes = [ps, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]
+    lib.pa_mfma_partial_groups.restype = c_int64
+    lib.pa_mfma_partial_groups.argtypes = [ps, c_int]
     lib.pa_mfma_deslice_project.restype = c_int
     lib.pa_mfma_deslice_project.argtypes = [ps, c_void_p, c_void_p, c_void_p, c_void_p, pt, c_void_p]
     _lib = lib

@@ -68,13 +68,23 @@ struct MfmaPlan {
   int64_t G;
 };
 
+int compute_units();
+
+// partial slice-token sums the first reduction pass leaves: one per workgroup of the fused kernel (a), or one per
+// point group of kernel (b)
+int64_t mfma_groups(const pa_shape &s, bool fused) {
+  return fused ? pa::mfma::project_groups(s, compute_units(), true) : pa::mfma::reduce_groups(s);
+}
+
 int64_t mfma_partials_bytes(const pa_shape &s) {
-  return (pa::mfma::reduce_groups(s) + 1) * s.B * s.H * s.S * (s.D + 1) * 4;  // G partials + their total
+  int64_t g = mfma_groups(s, false);
+  if (pa::mfma::fuse_reduce(s)) g = std::max(g, mfma_groups(s, true));
+  return (g + 1) * s.B * s.H * s.S * (s.D + 1) * 4;  // G partials + their total
 }
 
 MfmaPlan plan_mfma(const pa_shape &s) {
   MfmaPlan p{};
-  p.G = pa::mfma::reduce_groups(s);
+  p.G = mfma_groups(s, pa::mfma::fuse_reduce(s));
   int64_t off = 0;
   p.off_blob = off;
   off += round_up(pa::mfma::blob_bytes(s), 256);
@@ -259,7 +269,26 @@ int pa_mfma_project_softmax(const pa_shape *shape, const void *blob, const void 
   if (rc) return rc;
   if (!blob || !x || !fx_pack || !w_pack) return PA_ERR_NULL;
   if (!aligned16(blob) || !aligned16(x) || !aligned16(fx_pack) || !aligned16(w_pack)) return PA_ERR_ALIGN;
-  return pa::mfma::project_softmax(*shape, blob, x, fx_pack, w_pack, compute_units(), static_cast<hipStream_t>(stream));
+  return pa::mfma::project_softmax(*shape, blob, x, fx_pack, w_pack, nullptr, compute_units(),
+                                   static_cast<hipStream_t>(stream));
+}
+
+int64_t pa_mfma_partial_groups(const pa_shape *shape, int fused) {
+  int rc = check_mfma(shape);
+  if (rc) return rc;
+  if (fused && !pa::mfma::fuse_reduce(*shape)) return PA_ERR_UNSUPPORTED;
+  return mfma_groups(*shape, fused != 0);
+}
+
+int pa_mfma_project_softmax_reduce(const pa_shape *shape, const void *blob, const void *x, void *w_pack, float *partials,
+                                   void *stream) {
+  int rc = check_mfma(shape);
+  if (rc) return rc;
+  if (!pa::mfma::fuse_reduce(*shape)) return PA_ERR_UNSUPPORTED;
+  if (!blob || !x || !w_pack || !partials) return PA_ERR_NULL;
+  if (!aligned16(blob) || !aligned16(x) || !aligned16(w_pack) || !aligned16(partials)) return PA_ERR_ALIGN;
+  return pa::mfma::project_softmax(*shape, blob, x, nullptr, w_pack, partials, compute_units(),
+                                   static_cast<hipStream_t>(stream));
 }
 
 int pa_mfma_slice_reduce(const pa_shape *shape, const void *w_pack, const void *fx_pack, float *partials, void *stream) {
@@ -270,14 +299,16 @@ int pa_mfma_slice_reduce(const pa_shape *shape, const void *w_pack, const void *
   return pa::mfma::slice_reduce(*shape, w_pack, fx_pack, partials, static_cast<hipStream_t>(stream));
 }
 
-int pa_mfma_combine_attention(const pa_shape *shape, const pa_params *p, const float *partials, float *slice_token,
-                              float *slice_norm, float *out_slice_token, void *tokp, void *stream) {
+int pa_mfma_combine_attention(const pa_shape *shape, const pa_params *p, const float *partials, int64_t groups,
+                              float *slice_token, float *slice_norm, float *out_slice_token, void *tokp, void *stream) {
   int rc = check_mfma(shape);
   if (rc) return rc;
+  if (groups < 1 || (groups + 1) * shape->B * shape->H * shape->S * (shape->D + 1) * 4 > mfma_partials_bytes(*shape))
+    return PA_ERR_DIMS;
   if (!p || !p->qkv_project_weight || !partials || !out_slice_token || !tokp) return PA_ERR_NULL;
   if (!aligned16(partials) || !aligned16(tokp)) return PA_ERR_ALIGN;
   hipStream_t st = static_cast<hipStream_t>(stream);
-  rc = pa::general::combine_attention(*shape, *p, partials, pa::mfma::reduce_groups(*shape), slice_token, slice_norm,
+  rc = pa::general::combine_attention(*shape, *p, partials, groups, slice_token, slice_norm,
                                       out_slice_token, st);
   if (rc) return rc;
   return pa::mfma::pack_tokens(*shape, out_slice_token, tokp, st);
@@ -335,8 +366,12 @@ int pa_layer_forward(int dtype, const pa_shape *shape, const pa_params *p, const
     float *norm = reinterpret_cast<float *>(ws + mp.off_norm);
     float *tok_out = reinterpret_cast<float *>(ws + mp.off_tok_out);
     if ((rc = pa::mfma::pack_params(s, *p, blob, st))) return rc;
-    if ((rc = pa::mfma::project_softmax(s, blob, x, fxp, wp, compute_units(), st))) return rc;
-    if ((rc = pa::mfma::slice_reduce(s, wp, fxp, partials, st))) return rc;
+    if (pa::mfma::fuse_reduce(s)) {  // kernel (a) also leaves the partial slice-token sums
+      if ((rc = pa::mfma::project_softmax(s, blob, x, nullptr, wp, partials, compute_units(), st))) return rc;
+    } else {
+      if ((rc = pa::mfma::project_softmax(s, blob, x, fxp, wp, nullptr, compute_units(), st))) return rc;
+      if ((rc = pa::mfma::slice_reduce(s, wp, fxp, partials, st))) return rc;
+    }
     if ((rc = pa::general::combine_attention(s, *p, partials, mp.G, tok, norm, tok_out, st))) return rc;
     if ((rc = pa::mfma::pack_tokens(s, tok_out, tokp, st))) return rc;
     return pa::mfma::deslice_project(s, blob, wp, tokp, y, tail_active(tail) ? tail : nullptr, compute_units(), st);

@@ -35,8 +35,10 @@ int64_t fx_pack_bytes(const pa_shape &s);
 int64_t w_pack_bytes(const pa_shape &s);
 int64_t tokp_bytes(const pa_shape &s);
 int pack_params(const pa_shape &s, const pa_params &p, void *blob, hipStream_t st);
-int project_softmax(const pa_shape &s, const void *blob, const void *x, void *fx_pack, void *w_pack, int num_cu,
-                    hipStream_t st);
+int64_t project_groups(const pa_shape &s, int num_cu, bool fused);
+bool fuse_reduce(const pa_shape &s);
+int project_softmax(const pa_shape &s, const void *blob, const void *x, void *fx_pack, void *w_pack, float *partials,
+                    int num_cu, hipStream_t st);
 int slice_reduce(const pa_shape &s, const void *w_pack, const void *fx_pack, float *partials, hipStream_t st);
 int pack_tokens(const pa_shape &s, const float *tok_out, void *tokp, hipStream_t st);
 int deslice_project(const pa_shape &s, const void *blob, const void *w_pack, const void *tokp, void *y,

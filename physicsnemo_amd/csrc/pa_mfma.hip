@@ -123,43 +123,52 @@ __global__ __launch_bounds__(256) void pack_params_kernel(pa_params p, u32x4 *__
 }
 
 // ------------------------------------------------------------------------------------------------
-// Kernel (a): projections + slice logits + temperature softmax, weights-stationary.
+// Kernel (a): projections + slice logits + temperature softmax, weights-stationary; optionally fused with the
+// first pass of the slice-token aggregation (FUSED).
 //   x_mid^T (32 ch x 32 pts) = Wx_h . x^T          A = Wx_h frags (registers), B = x frags (LDS)
-//   fx_mid  (32 pts x 32 d)  = x . Wfx_h^T         A = x frags (LDS),          B = Wfx_h frags (registers)  -> fx_pack
+//   fx_mid  (32 pts x 32 d)  = x . Wfx_h^T         A = x frags (LDS),          B = Wfx_h frags (registers)
 //   logits^T(32 s x 32 pts)  = Wslice . x_mid^T    A = Wslice frags (LDS), B = bf16(x_mid^T) straight from registers
 //   softmax over s: in-lane over the accumulator registers plus one exchange with lane^32               -> w_pack
-// One persistent workgroup per CU with H waves (two per SIMD for C = 256).  Wave h owns head h and keeps its
-// Wx | Wfx fragments (2 * KS * 4 = 128 registers for C = 256) in registers for the whole kernel: after the
-// prologue there is no weight traffic at all.  The x rows of a SET of TS tiles (TS * 32 points) are staged in LDS by
-// the whole workgroup with full-row coalesced loads; unit u (16 bytes) of row r is stored at r*UPR + (u ^ (r & 7)),
-// which makes both the row-wise writes and the fragment reads (row i, unit 2ks+g) bank-conflict free.  One fragment
-// read (1 KiB) feeds two MFMAs.  The set buffers are double buffered; the next set is fetched one tile at a time
-// into registers at the start of a tile and written to LDS at its end; one barrier per set.
-// The loop over sets is the only loop; its body has no branch around a memory operation (waves past the last tile
-// recompute it and re-store identical values).  The two waves of a SIMD drift apart, so one wave's MFMA phase
-// overlaps the other's softmax (VALU) phase.
+//   !FUSED: fx_mid -> fx_pack (kernel (b) aggregates later)
+//    FUSED: w^T (lanes <-> slices, registers <-> points) = w_chunk . SEL  (an exact MFMA "transpose"),
+//           tok^T_h (32 d x S) += bf16(fx_mid)^T . w^T, norm_h += sum_n w; accumulators live in LDS between tiles
+//           (a wave owns its head, so there is no cross-wave reduction) and leave as one partial per workgroup:
+//           partials[g][b][h][s][0..D-1] = sum_n w fx_mid, [..][D] = sum_n w   (layout of the combine kernel).
+// Grid (G workgroups per batch, B); workgroup (g, b) walks the tile sets g, g+G, ... of batch b, H waves (two per
+// SIMD for C = 256).  Wave h owns head h and keeps its Wx | Wfx fragments (2 * KS * 4 = 128 registers for C = 256)
+// in registers for the whole kernel: after the prologue there is no weight traffic at all.  The x rows of a SET of
+// TS tiles are staged in LDS by the whole workgroup with full-row coalesced loads; unit u (16 bytes) of row r is
+// stored at r*UPR + (u ^ (r & 7)), which makes both the row-wise writes and the fragment reads (row i, unit 2ks+g)
+// bank-conflict free.  One fragment read (1 KiB) feeds two MFMAs.  The set buffers are double buffered; the next
+// set is fetched one tile at a time into registers at the start of a tile and written to LDS at its end; one
+// barrier per set.  The loop over sets is the only loop; its body has no branch around a global memory operation
+// (slots past the last tile of the batch recompute it and re-store identical values; they skip the aggregation).
 // ------------------------------------------------------------------------------------------------
-template <int C, int S>
+template <int C, int S, bool FUSED>
 __global__ __launch_bounds__((C / 32) * 64) void project_softmax_kernel(const u32x4 *__restrict__ blob,
                                                                         const uint16_t *__restrict__ x,
                                                                         u32x4 *__restrict__ fx_pack,
-                                                                        u32x4 *__restrict__ w_pack, int64_t N, int tpb,
-                                                                        int64_t total_tiles) {
-  constexpr int H = C / 32, KS = C / 16, ST = (S + 31) / 32, NCH = S / 16;
+                                                                        u32x4 *__restrict__ w_pack,
+                                                                        float *__restrict__ partials, int64_t N, int tpb) {
+  constexpr int H = C / 32, KS = C / 16, ST = (S + 31) / 32, NCH = S / 16, D1 = 33;
   constexpr int WAVES = H, NT = WAVES * 64;
-  constexpr int TS = 4;                 // tiles per set
+  constexpr int TS = FUSED ? 2 : 4;     // tiles per set (the fused form needs LDS for the accumulators)
   constexpr int UPR = C / 8;            // 16-byte units per row
   constexpr int SET_UNITS = TS * 32 * UPR;
   constexpr int CHUNK = 32 * UPR / NT;  // units per thread and tile when staging
+  constexpr int ACC_UNITS = ST * 4 * 64 + ST * 16;  // per head: tok^T accumulator (16-byte units) + norm row
   static_assert((32 * UPR) % NT == 0, "a tile must split evenly over the workgroup");
   extern __shared__ u32x4 smem[];
   u32x4 *xs = smem;                     // 2 * SET_UNITS
   u32x4 *wsl = xs + 2 * SET_UNITS;      // ST * 2 * 64
-  float *fvec = reinterpret_cast<float *>(wsl + ST * 2 * 64);
+  u32x4 *sel = wsl + ST * 2 * 64;       // 2 * 64: the 0/1 selection matrices of the MFMA transpose
+  u32x4 *accs = sel + 2 * 64;           // FUSED: H * ACC_UNITS
+  float *fvec = reinterpret_cast<float *>(accs + (FUSED ? H * ACC_UNITS : 0));
   float *bias_x = fvec, *bias_f = fvec + C, *bias_s = fvec + 2 * C, *tscale = fvec + 3 * C + ST * 32;
   const BlobPlan bp = blob_plan(C, S);
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, i = lane & 31, g = lane >> 5;
   const int h = wave;
+  const int b = blockIdx.y;
 
   u32x4 wx[KS], wf[KS];
 #pragma unroll
@@ -173,23 +182,29 @@ __global__ __launch_bounds__((C / 32) * 64) void project_softmax_kernel(const u3
     const float *src = reinterpret_cast<const float *>(blob + bp.fvec);
     for (int k = tid; k < 3 * C + ST * 32 + H; k += NT) fvec[k] = src[k];
   }
+  u32x4 *acc_tok = accs + h * ACC_UNITS;                                        // [st][q][lane]: registers 4q..4q+3
+  float *acc_nrm = reinterpret_cast<float *>(accs + h * ACC_UNITS + ST * 4 * 64);  // [st][lane]
+  if constexpr (FUSED) {
+    if (tid < 128) {
+      const int par = tid >> 6;
+      bf16x8 s8;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) s8[j] = (__bf16)((i == kperm(par, g, j)) ? 1.f : 0.f);
+      sel[tid] = __builtin_bit_cast(u32x4, s8);
+    }
+    for (int u = lane; u < ACC_UNITS; u += 64) acc_tok[u] = u32x4{0, 0, 0, 0};
+  }
 
-  const int ntiles = (int)total_tiles;  // < 2^28 (checked on the host)
-  const int64_t nsets = (total_tiles + TS - 1) / TS;
-  const int64_t nloc = (nsets - blockIdx.x + gridDim.x - 1) / gridDim.x;
-  auto tile_of = [&](int64_t set, int t) {
-    const int tr = (int)set * TS + t;
-    return tr < ntiles ? tr : ntiles - 1;
-  };
-  // staging: this thread's CHUNK units of tile (set, t): unit k*NT + tid -> row rc, position pos.  The load only
-  // issues (rows beyond N re-read row 0 of the tile); the values are first touched in stage_store, a whole tile of
-  // work later, where rows beyond N are replaced by zeros.
-  auto stage_load = [&](int64_t set, int t, u32x4(&st)[CHUNK], int &rows_ok) {
-    const int tile = tile_of(set, t);
-    const int b = tile / tpb;
-    const int n0 = (tile - b * tpb) * 32;
-    const uint16_t *xbase = x + ((int64_t)b * N + n0) * C;
-    rows_ok = (int)min((int64_t)32, N - n0);
+  const int nsets = (tpb + TS - 1) / TS;  // per batch
+  const int nloc = (nsets - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x;
+  const uint16_t *xbatch = x + (int64_t)b * N * C;
+  // staging: this thread's CHUNK units of tile `tile` of the batch: unit k*NT + tid -> row rc, position pos.  The
+  // load only issues (rows beyond N re-read row 0 of the tile); the values are first touched in stage_store, a whole
+  // tile of work later, where rows beyond N are replaced by zeros.
+  auto stage_load = [&](int tile, u32x4(&st)[CHUNK], int &rows_ok) {
+    const int t = tile < tpb ? tile : tpb - 1;
+    const uint16_t *xbase = xbatch + (int64_t)t * 32 * C;
+    rows_ok = (int)min((int64_t)32, N - (int64_t)t * 32);
 #pragma unroll
     for (int k = 0; k < CHUNK; ++k) {
       const int idx = k * NT + tid, rc = idx / UPR, pos = idx - rc * UPR;
@@ -207,25 +222,27 @@ __global__ __launch_bounds__((C / 32) * 64) void project_softmax_kernel(const u3
   for (int t = 0; t < TS; ++t) {  // first set
     u32x4 st[CHUNK];
     int rows_ok;
-    stage_load(blockIdx.x, t, st, rows_ok);
+    stage_load((int)blockIdx.x * TS + t, st, rows_ok);
     stage_store(0, t, st, rows_ok);
   }
   __syncthreads();
 
-  int64_t set = blockIdx.x;
-  for (int64_t sl = 0; sl < nloc; ++sl) {
-    const int buf = (int)(sl & 1);
-    const int64_t set_next = set + gridDim.x < nsets ? set + gridDim.x : set;  // the last set re-fetches itself
+  int set = blockIdx.x;
+  for (int sl = 0; sl < nloc; ++sl) {
+    const int buf = sl & 1;
+    const int set_next = set + (int)gridDim.x < nsets ? set + (int)gridDim.x : set;  // the last set re-fetches itself
 #pragma unroll
     for (int t = 0; t < TS; ++t) {
       __builtin_amdgcn_sched_barrier(0);  // keep each tile's work (and its register live ranges) to itself
       u32x4 stg[CHUNK];
       int stg_rows;
-      stage_load(set_next, t, stg, stg_rows);
+      stage_load(set_next * TS + t, stg, stg_rows);
       __builtin_amdgcn_sched_barrier(0);
-      const int tile = tile_of(set, t);
-      const int b = tile / tpb;
-      const bool valid = (int64_t)(tile - b * tpb) * 32 + i < N;
+      const int slot = set * TS + t;
+      const bool dup = slot >= tpb;  // past the batch's last tile: recompute it, contribute nothing
+      const int tb = dup ? tpb - 1 : slot;
+      const int64_t tile = (int64_t)b * tpb + tb;
+      const bool valid = (int64_t)tb * 32 + i < N;
 
       // ---- products ----
       const u32x4 *xb = xs + buf * SET_UNITS + (t * 32 + i) * UPR;
@@ -249,9 +266,12 @@ __global__ __launch_bounds__((C / 32) * 64) void project_softmax_kernel(const u3
         af = mma(xf[ks % RING], wf[ks], af);
         __builtin_amdgcn_sched_barrier(0);  // keeps the compiler from sinking the reads back next to their uses
       }
-      u32x4 *fdst = fx_pack + (((int64_t)tile * H + h) * 2) * 64 + lane;
-      fdst[0] = pack_half<0>(af);
-      fdst[64] = pack_half<1>(af);
+      const u32x4 fxp0 = pack_half<0>(af), fxp1 = pack_half<1>(af);
+      if constexpr (!FUSED) {
+        u32x4 *fdst = fx_pack + ((tile * H + h) * 2) * 64 + lane;
+        fdst[0] = fxp0;
+        fdst[64] = fxp1;
+      }
       const u32x4 xb0 = pack_half<0>(ax), xb1 = pack_half<1>(ax);
       f32x16 lg[ST];
 #pragma unroll
@@ -283,18 +303,70 @@ __global__ __launch_bounds__((C / 32) * 64) void project_softmax_kernel(const u3
         }
       sum += __shfl_xor(sum, 32, 64);
       const float inv = valid ? __builtin_amdgcn_rcpf(sum) : 0.f;  // rows beyond N get zero weight
-      u32x4 *wdst = w_pack + (((int64_t)tile * H + h) * NCH) * 64 + lane;
+      u32x4 wp[2 * ST];
 #pragma unroll
       for (int st = 0; st < ST; ++st) {
-        if (2 * st < NCH) wdst[(2 * st) * 64] = pack_half<0>(lg[st], inv);
-        if (2 * st + 1 < NCH) wdst[(2 * st + 1) * 64] = pack_half<1>(lg[st], inv);
+        wp[2 * st] = pack_half<0>(lg[st], inv);
+        wp[2 * st + 1] = pack_half<1>(lg[st], inv);
       }
+      u32x4 *wdst = w_pack + ((tile * H + h) * NCH) * 64 + lane;
+#pragma unroll
+      for (int cq = 0; cq < NCH; ++cq) wdst[cq * 64] = wp[cq];
       __builtin_amdgcn_sched_barrier(0);
+
+      // ---- aggregation of this tile into the head's LDS accumulators ----
+      if constexpr (FUSED) {
+        if (!dup) {
+#pragma unroll
+          for (int st = 0; st < ST; ++st) {
+            f32x16 tr;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) tr[r] = 0.f;
+            tr = mma(wp[2 * st], sel[lane], tr);
+            if (2 * st + 1 < NCH) tr = mma(wp[2 * st + 1], sel[64 + lane], tr);
+            float s16 = 0.f;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) s16 += tr[r];
+            acc_nrm[st * 64 + lane] += s16;
+            f32x16 tok;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              const u32x4 v = acc_tok[(st * 4 + q) * 64 + lane];
+#pragma unroll
+              for (int k = 0; k < 4; ++k) tok[4 * q + k] = __uint_as_float(v[k]);
+            }
+            tok = mma(fxp0, pack_half<0>(tr), tok);
+            tok = mma(fxp1, pack_half<1>(tr), tok);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              u32x4 v;
+#pragma unroll
+              for (int k = 0; k < 4; ++k) v[k] = __float_as_uint(tok[4 * q + k]);
+              acc_tok[(st * 4 + q) * 64 + lane] = v;
+            }
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
       stage_store(buf ^ 1, t, stg, stg_rows);
       __builtin_amdgcn_sched_barrier(0);
     }
     set = set_next;
     __syncthreads();
+  }
+  if constexpr (FUSED) {
+    // this wave's head: accumulators -> partials[g][b][h][s][d], [..][D] = count
+    float *dst = partials + (((int64_t)blockIdx.x * gridDim.y + b) * H + h) * (S * D1);
+    const float *tokf = reinterpret_cast<const float *>(acc_tok);
+#pragma unroll
+    for (int st = 0; st < ST; ++st) {
+      const int s = 32 * st + i;
+      if (s < S) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) dst[s * D1 + rowmap(r, g)] = tokf[((st * 4 + (r >> 2)) * 64 + lane) * 4 + (r & 3)];
+        if (g == 0) dst[s * D1 + 32] = acc_nrm[st * 64 + lane] + acc_nrm[st * 64 + lane + 32];
+      }
+    }
   }
 }
 
@@ -626,7 +698,7 @@ bool supported(int dtype, const pa_shape &s) {
   if (dtype != PA_BF16 || s.conv_k != 0 || s.D != 32 || s.C != s.H * 32) return false;
   if (s.C != 128 && s.C != 256) return false;
   if (s.S != 16 && s.S != 32 && s.S != 64 && s.S != 128) return false;
-  if ((s.N + 31) / 32 * s.B > ((int64_t)1 << 31) / 8) return false;
+  if ((s.N + 31) / 32 * s.B > ((int64_t)1 << 31) / 8 || s.B > 65535) return false;
   return true;
 }
 
@@ -650,28 +722,42 @@ int pack_params(const pa_shape &s, const pa_params &p, void *blob, hipStream_t s
   return launch_status();
 }
 
+// workgroups per batch of kernel (a): about one resident workgroup per CU in total
+int64_t project_groups(const pa_shape &s, int num_cu, bool fused) {
+  const int64_t ts = fused ? 2 : 4;
+  const int64_t nsets = (tiles_per_batch(s) + ts - 1) / ts;
+  int64_t g = num_cu / s.B;
+  if (g < 1) g = 1;
+  if (g > nsets) g = nsets;
+  return g;
+}
+
+bool fuse_reduce(const pa_shape &s) { return s.S <= 64; }  // the LDS accumulators of the fused form fit up to S = 64
+
+template <int C, int S, bool FUSED>
+static int project_softmax_f(const pa_shape &s, const void *blob, const void *x, void *fx_pack, void *w_pack,
+                             float *partials, int num_cu, hipStream_t st) {
+  constexpr int ST = (S + 31) / 32, H = C / 32, TS = FUSED ? 2 : 4, UPR = C / 8, WAVES = H;
+  constexpr int ACC_UNITS = ST * 4 * 64 + ST * 16;
+  const size_t lds = (size_t)(2 * TS * 32 * UPR + ST * 2 * 64 + 2 * 64 + (FUSED ? H * ACC_UNITS : 0)) * 16 +
+                     (size_t)(3 * C + ST * 32 + H) * 4;
+  int rc = allow_dynamic_lds(project_softmax_kernel<C, S, FUSED>, lds);
+  if (rc) return rc;
+  const int64_t tpb = tiles_per_batch(s);
+  const int64_t G = project_groups(s, num_cu, FUSED);
+  hipLaunchKernelGGL((project_softmax_kernel<C, S, FUSED>), dim3((unsigned)G, (unsigned)s.B), dim3(WAVES * 64), lds, st,
+                     static_cast<const u32x4 *>(blob), static_cast<const uint16_t *>(x), static_cast<u32x4 *>(fx_pack),
+                     static_cast<u32x4 *>(w_pack), partials, s.N, (int)tpb);
+  return launch_status();
+}
+
 template <int C, int S>
 static int project_softmax_cs(const pa_shape &s, const void *blob, const void *x, void *fx_pack, void *w_pack,
-                              int num_cu, hipStream_t st) {
-  constexpr int ST = (S + 31) / 32, H = C / 32, TS = 4, UPR = C / 8, WAVES = H;
-  const size_t lds = (size_t)(2 * TS * 32 * UPR + ST * 2 * 64) * 16 + (size_t)(3 * C + ST * 32 + H) * 4;
-  int rc = allow_dynamic_lds(project_softmax_kernel<C, S>, lds);
-  if (rc) return rc;
-  const int64_t tpb = tiles_per_batch(s), total = tpb * s.B;
-  static int per_cu = 0;  // resident workgroups per CU for this instantiation
-  if (per_cu == 0) {
-    int nb = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, project_softmax_kernel<C, S>, WAVES * 64, lds) != hipSuccess ||
-        nb < 1)
-      nb = 1;
-    per_cu = nb;
+                              float *partials, int num_cu, hipStream_t st) {
+  if constexpr (S <= 64) {
+    if (partials) return project_softmax_f<C, S, true>(s, blob, x, fx_pack, w_pack, partials, num_cu, st);
   }
-  int64_t grid = (total + TS - 1) / TS;
-  if (grid > (int64_t)num_cu * per_cu) grid = (int64_t)num_cu * per_cu;
-  hipLaunchKernelGGL((project_softmax_kernel<C, S>), dim3((unsigned)grid), dim3(WAVES * 64), lds, st,
-                     static_cast<const u32x4 *>(blob), static_cast<const uint16_t *>(x), static_cast<u32x4 *>(fx_pack),
-                     static_cast<u32x4 *>(w_pack), s.N, (int)tpb, total);
-  return launch_status();
+  return project_softmax_f<C, S, false>(s, blob, x, fx_pack, w_pack, nullptr, num_cu, st);
 }
 
 template <int S>
@@ -749,9 +835,10 @@ static int deslice_project_cs(const pa_shape &s, const void *blob, const void *w
     return FN<128, 128>(__VA_ARGS__);                               \
   } while (0)
 
-int project_softmax(const pa_shape &s, const void *blob, const void *x, void *fx_pack, void *w_pack, int num_cu,
-                    hipStream_t st) {
-  PA_DISPATCH_CS(project_softmax_cs, s, blob, x, fx_pack, w_pack, num_cu, st);
+// partials != nullptr (and S <= 64): fused with the first reduction pass; fx_pack is then not written
+int project_softmax(const pa_shape &s, const void *blob, const void *x, void *fx_pack, void *w_pack, float *partials,
+                    int num_cu, hipStream_t st) {
+  PA_DISPATCH_CS(project_softmax_cs, s, blob, x, fx_pack, w_pack, partials, num_cu, st);
 }
 
 int slice_reduce(const pa_shape &s, const void *w_pack, const void *fx_pack, float *partials, hipStream_t st) {

@@ -182,6 +182,8 @@ class MfmaStages:
         self.tok = torch.empty(dims.B, dims.H, dims.S, dims.D, **f32)
         self.norm = torch.empty(dims.B, dims.H, dims.S, **f32)
         self.tok_out = torch.empty(dims.B, dims.H, dims.S, dims.D, **f32)
+        self.groups = int(lib.pa_mfma_partial_groups(byref(self.shape), 0))   # producer of `partials`: kernel (b)
+        self.fused_groups = int(lib.pa_mfma_partial_groups(byref(self.shape), 1))  # < 0: fused form not available
 
     def _stream(self):
         return _lib.current_stream_ptr(self.device)
@@ -199,10 +201,19 @@ class MfmaStages:
     def slice_reduce(self):
         _lib.check(self.lib.pa_mfma_slice_reduce(byref(self.shape), self.w_pack.data_ptr(), self.fx_pack.data_ptr(),
                                                  self.partials.data_ptr(), self._stream()), "pa_mfma_slice_reduce")
+        self._producer_groups = self.groups
+
+    def project_softmax_reduce(self, x):
+        """Kernels (a)+(b) in one launch (what `layer_forward` runs when slice_num <= 64)."""
+        _need_cuda(x)
+        _lib.check(self.lib.pa_mfma_project_softmax_reduce(byref(self.shape), self.blob.data_ptr(), x.data_ptr(),
+                                                           self.w_pack.data_ptr(), self.partials.data_ptr(),
+                                                           self._stream()), "pa_mfma_project_softmax_reduce")
+        self._producer_groups = self.fused_groups
 
     def combine_attention(self):
         _lib.check(self.lib.pa_mfma_combine_attention(byref(self.shape), byref(self.cparams), self.partials.data_ptr(),
-                                                      self.tok.data_ptr(), self.norm.data_ptr(), self.tok_out.data_ptr(),
+                                                      self._producer_groups, self.tok.data_ptr(), self.norm.data_ptr(), self.tok_out.data_ptr(),
                                                       self.tokp.data_ptr(), self._stream()), "pa_mfma_combine_attention")
 
     def deslice_project(self, y, residual=None, ln_weight=None, ln_bias=None, ln_eps=1e-5, ln_out=None):

@@ -29,6 +29,7 @@ def _run(B, N, C, S, seed=0, sharpen=1.0, temps=None):
 @pytest.mark.parametrize("B,N,C,S", [
     (1, 4096, 256, 64), (2, 1000, 256, 64), (1, 2048, 256, 16), (1, 2048, 256, 32), (1, 1500, 256, 128),
     (3, 777, 128, 32), (1, 31, 128, 16), (1, 33, 256, 64), (2, 2048, 128, 128), (1, 4096, 128, 64),
+    (5, 97, 256, 64), (2, 40000, 256, 32), (300, 64, 128, 16),
 ])
 def test_mfma_layer_matches_fp32_oracle(B, N, C, S):
     announce("mfma layer", B, N, C, S)
@@ -47,19 +48,39 @@ def test_mfma_sharp_softmax_and_clamped_temperatures():
     assert_rel_l2(y, want["y"], "layer output")
 
 
-def test_mfma_stage_entry_points_agree_with_layer_call():
-    announce("mfma stages == layer")
-    B, N, C, S = 2, 1234, 256, 64
+@pytest.mark.parametrize("B,N,C,S", [(2, 1234, 256, 64), (3, 500, 128, 32), (1, 4000, 256, 16), (2, 900, 256, 128)])
+def test_mfma_stage_entry_points_agree_with_layer_call(B, N, C, S):
+    announce("mfma stages == layer", B, N, C, S)
     ref, hip, xb, want, y, tok = _run(B, N, C, S)
     st = PF.MfmaStages(hip.kernel_params(torch.bfloat16, xb.device), hip.layer_dims(xb), xb.device)
-    y2 = torch.empty_like(y)
+    fused = st.fused_groups > 0
+    assert fused == (S <= 64)
     st.pack_params()
+    # the separate kernels (a) and (b)
+    y_ab = torch.empty_like(y)
     st.project_softmax(xb)
+    w_pack_a = st.w_pack.clone()
     st.slice_reduce()
     st.combine_attention()
-    st.deslice_project(y2)
-    assert torch.equal(y2, y)
-    assert torch.equal(st.tok, tok)
+    st.deslice_project(y_ab)
+    tok_ab, norm_ab = st.tok.clone(), st.norm.clone()
+    if fused:
+        # one launch for (a)+(b): this is what the layer call runs -> bit-identical to it; against the separate
+        # kernels only the order of the fp32 partial sums differs (same bf16 operands)
+        st.w_pack.zero_()
+        y_f = torch.empty_like(y)
+        st.project_softmax_reduce(xb)
+        assert torch.equal(st.w_pack, w_pack_a)
+        st.combine_attention()
+        st.deslice_project(y_f)
+        assert torch.equal(y_f, y)
+        assert torch.equal(st.tok, tok)
+        assert_rel_l2(st.tok, tok_ab, "fused vs separate slice tokens", tol=1e-5)
+        assert_rel_l2(st.norm, norm_ab, "fused vs separate slice norm", tol=1e-5)
+        assert_rel_l2(y_f, y_ab, "fused vs separate output", tol=2e-3)
+    else:
+        assert torch.equal(y_ab, y)
+        assert torch.equal(tok_ab, tok)
     # norm invariant: sum_s (norm - 0.01) = number of points, up to bf16 rounding of the weights
     total = (st.norm - 0.01).sum(-1)
     assert torch.allclose(total, torch.full_like(total, float(N)), rtol=2e-3)
