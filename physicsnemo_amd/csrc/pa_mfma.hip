@@ -122,6 +122,17 @@ __global__ __launch_bounds__(256) void pack_params_kernel(pa_params p, u32x4 *__
   }
 }
 
+// value of lane l combined with the value of lane l ^ 32, without a trip through LDS: v_permlane32_swap hands every
+// lane the lower-half and the upper-half value of its column
+__device__ __forceinline__ float half_max(float v) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float half_sum(float v) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
 // ------------------------------------------------------------------------------------------------
 // Kernel (a): projections + slice logits + temperature softmax, weights-stationary; optionally fused with the
 // first pass of the slice-token aggregation (FUSED).
@@ -138,8 +149,9 @@ __global__ __launch_bounds__(256) void pack_params_kernel(pa_params p, u32x4 *__
 // SIMD for C = 256).  Wave h owns head h and keeps its Wx | Wfx fragments (2 * KS * 4 = 128 registers for C = 256)
 // in registers for the whole kernel: after the prologue there is no weight traffic at all.  The x rows of a SET of
 // TS tiles are staged in LDS by the whole workgroup with full-row coalesced loads; unit u (16 bytes) of row r is
-// stored at r*UPR + (u ^ (r & 7)), which makes both the row-wise writes and the fragment reads (row i, unit 2ks+g)
-// bank-conflict free.  One fragment read (1 KiB) feeds two MFMAs.  The set buffers are double buffered; the next
+// stored at r*(UPR+1) + u: the one-unit stagger per row makes the 16 lanes of a 128-bit access (rows i..i+15, same
+// unit) cover all 64 banks, so both the row-wise writes and the fragment reads (row i, unit 2ks+g) are free of bank
+// conflicts, and every fragment address is one base register plus an immediate offset.  One fragment read (1 KiB) feeds two MFMAs.  The set buffers are double buffered; the next
 // set is fetched one tile at a time into registers at the start of a tile and written to LDS at its end; one
 // barrier per set.  The loop over sets is the only loop; its body has no branch around a global memory operation
 // (slots past the last tile of the batch recompute it and re-store identical values; they skip the aggregation).
@@ -154,7 +166,8 @@ __global__ __launch_bounds__((C / 32) * 64) void project_softmax_kernel(const u3
   constexpr int WAVES = H, NT = WAVES * 64;
   constexpr int TS = FUSED ? 2 : 4;     // tiles per set (the fused form needs LDS for the accumulators)
   constexpr int UPR = C / 8;            // 16-byte units per row
-  constexpr int SET_UNITS = TS * 32 * UPR;
+  constexpr int ROWU = UPR + 1;         // LDS row stride in units: one unit of stagger per row (see above)
+  constexpr int SET_UNITS = TS * 32 * ROWU;
   constexpr int CHUNK = 32 * UPR / NT;  // units per thread and tile when staging
   constexpr int ACC_UNITS = ST * 4 * 64 + ST * 16;  // per head: tok^T accumulator (16-byte units) + norm row
   static_assert((32 * UPR) % NT == 0, "a tile must split evenly over the workgroup");
@@ -215,7 +228,7 @@ __global__ __launch_bounds__((C / 32) * 64) void project_softmax_kernel(const u3
 #pragma unroll
     for (int k = 0; k < CHUNK; ++k) {
       const int idx = k * NT + tid, rc = idx / UPR, pos = idx - rc * UPR;
-      xs[buf * SET_UNITS + (t * 32 + rc) * UPR + (pos ^ (rc & 7))] = rc < rows_ok ? st[k] : u32x4{0, 0, 0, 0};
+      xs[buf * SET_UNITS + (t * 32 + rc) * ROWU + pos] = rc < rows_ok ? st[k] : u32x4{0, 0, 0, 0};
     }
   };
 #pragma unroll
@@ -245,7 +258,7 @@ __global__ __launch_bounds__((C / 32) * 64) void project_softmax_kernel(const u3
       const bool valid = (int64_t)tb * 32 + i < N;
 
       // ---- products ----
-      const u32x4 *xb = xs + buf * SET_UNITS + (t * 32 + i) * UPR;
+      const u32x4 *xb = xs + buf * SET_UNITS + (t * 32 + i) * ROWU + g;
       f32x16 ax, af;
       {
         const float bf = bias_f[h * 32 + i];
@@ -255,13 +268,14 @@ __global__ __launch_bounds__((C / 32) * 64) void project_softmax_kernel(const u3
           af[r] = bf;
         }
       }
-      constexpr int RING = 3, AHEAD = 2;  // x fragments are read AHEAD k-steps before the MFMAs that use them
+      // x fragments are read AHEAD k-steps before the MFMAs that use them (S = 128 has no registers to spare)
+      constexpr int RING = ST > 2 ? 2 : 3, AHEAD = RING - 1;
       u32x4 xf[RING];
 #pragma unroll
-      for (int q = 0; q < AHEAD; ++q) xf[q] = xb[(2 * q + g) ^ (i & 7)];
+      for (int q = 0; q < AHEAD; ++q) xf[q] = xb[2 * q];
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
-        if (ks + AHEAD < KS) xf[(ks + AHEAD) % RING] = xb[(2 * (ks + AHEAD) + g) ^ (i & 7)];
+        if (ks + AHEAD < KS) xf[(ks + AHEAD) % RING] = xb[2 * (ks + AHEAD)];
         ax = mma(wx[ks], xf[ks % RING], ax);
         af = mma(xf[ks % RING], wf[ks], af);
         __builtin_amdgcn_sched_barrier(0);  // keeps the compiler from sinking the reads back next to their uses
@@ -289,7 +303,7 @@ __global__ __launch_bounds__((C / 32) * 64) void project_softmax_kernel(const u3
       for (int st = 0; st < ST; ++st)
 #pragma unroll
         for (int r = 0; r < 16; ++r) mx = fmaxf(mx, lg[st][r]);
-      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      mx = half_max(mx);
       const float sc = tscale[h];
       const float off = mx * sc;
       float sum = 0.f;
@@ -301,7 +315,7 @@ __global__ __launch_bounds__((C / 32) * 64) void project_softmax_kernel(const u3
           lg[st][r] = e;
           sum += e;
         }
-      sum += __shfl_xor(sum, 32, 64);
+      sum = half_sum(sum);
       const float inv = valid ? __builtin_amdgcn_rcpf(sum) : 0.f;  // rows beyond N get zero weight
       u32x4 wp[2 * ST];
 #pragma unroll
@@ -739,7 +753,7 @@ static int project_softmax_f(const pa_shape &s, const void *blob, const void *x,
                              float *partials, int num_cu, hipStream_t st) {
   constexpr int ST = (S + 31) / 32, H = C / 32, TS = FUSED ? 2 : 4, UPR = C / 8, WAVES = H;
   constexpr int ACC_UNITS = ST * 4 * 64 + ST * 16;
-  const size_t lds = (size_t)(2 * TS * 32 * UPR + ST * 2 * 64 + 2 * 64 + (FUSED ? H * ACC_UNITS : 0)) * 16 +
+  const size_t lds = (size_t)(2 * TS * 32 * (UPR + 1) + ST * 2 * 64 + 2 * 64 + (FUSED ? H * ACC_UNITS : 0)) * 16 +
                      (size_t)(3 * C + ST * 32 + H) * 4;
   int rc = allow_dynamic_lds(project_softmax_kernel<C, S, FUSED>, lds);
   if (rc) return rc;
