@@ -233,7 +233,7 @@ def main():
         dominant = max(on_path, key=lambda k: kernels[k]["ms"])
         # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a 1 GiB copy (x2.0 / x1.0);
         # measured for the default workload only (profiles/layer_cfg3_s64_hbm_traffic.md)
-        measured_traffic = {"project_softmax_reduce": None, "project_softmax": (549 + 1536) << 20, "slice_reduce": (1536 + 8) << 20,
+        measured_traffic = {"project_softmax_reduce": (517 + 1041) << 20, "project_softmax": (542 + 1536) << 20, "slice_reduce": (1536 + 8) << 20,
                             "deslice_project": (1025 + 512) << 20}
         default_workload = (B, N, C, S) == (1, 1 << 20, 256, 64)
         roofline = {"kernel": dominant, "bound": "hbm", "achieved": kernels[dominant]["hbm_gbs"], "peak": HBM_PEAK_GBS,
