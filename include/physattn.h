@@ -172,6 +172,27 @@ int pa_mfma_combine_attention(const pa_shape *shape, const pa_params *p, const f
 int pa_mfma_deslice_project(const pa_shape *shape, const void *blob, const void *w_pack, const void *tokp, void *y,
                             const pa_block_tail *tail, void *stream);
 
+/* ---- block MLP ---------------------------------------------------------------------------------- */
+
+/* Parameters of Mlp(C -> F -> C) with GELU (physicsnemo/nn/module/mlp_layers.py:139-173): torch layouts,
+ * w1 (F,C) and w2 (C,F) in the activation dtype, biases float32. */
+typedef struct pa_mlp_params {
+  const void *w1;
+  const float *b1;
+  const void *w2;
+  const float *b2;
+} pa_mlp_params;
+
+/* 1 if pa_mlp_forward serves (dtype, rows, C, F) [bf16, C in {128, 256}, F a multiple of 64], else 0. */
+int pa_mlp_query(int dtype, int64_t rows, int64_t C, int64_t F);
+/* Bytes of workspace pa_mlp_forward needs (the repacked weights), or a negative error code. */
+int64_t pa_mlp_workspace_bytes(int dtype, int64_t rows, int64_t C, int64_t F);
+/* y = w2 . gelu_erf(w1 . u + b1) + b2 for `rows` rows of u (rows, C); with a tail: y = that + tail->residual and
+ * tail->ln_out = LayerNorm(y). Replaces `self.ln_mlp1[1](ln) + fx` of TransolverBlock.forward (TR.py:301-303) and
+ * produces the LayerNorm the next consumer starts with (TR.py:300 of the next block, or :305-307). */
+int pa_mlp_forward(int dtype, int64_t rows, int64_t C, int64_t F, const pa_mlp_params *p, const void *u, void *y,
+                   const pa_block_tail *tail, void *workspace, int64_t workspace_bytes, void *stream);
+
 /* ---- whole layer ------------------------------------------------------------------------------ */
 
 /* Replaces PhysicsAttentionBase.forward (PA.py:501-558), plus=False, use_te=False, dropout off.

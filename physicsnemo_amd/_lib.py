@@ -20,7 +20,7 @@ EXPORTED = [
     "pa_slice_softmax", "pa_reduce_partial_count", "pa_slice_reduce", "pa_slice_attention",
     "pa_deslice_project", "pa_layer_forward", "pa_mfma_buffer_bytes", "pa_mfma_pack_params",
     "pa_mfma_project_softmax", "pa_mfma_slice_reduce", "pa_mfma_project_softmax_reduce", "pa_mfma_partial_groups",
-     "pa_mfma_combine_attention", "pa_mfma_deslice_project",
+     "pa_mfma_combine_attention", "pa_mfma_deslice_project", "pa_mlp_query", "pa_mlp_workspace_bytes", "pa_mlp_forward",
 ]
 
 PA_BUF_BLOB, PA_BUF_FX_PACK, PA_BUF_W_PACK, PA_BUF_PARTIALS, PA_BUF_TOKP = range(5)
@@ -35,6 +35,10 @@ class PaParams(Structure):
         "in_project_x_weight", "in_project_x_bias", "in_project_fx_weight", "in_project_fx_bias",
         "in_project_slice_weight", "in_project_slice_bias", "temperature", "qkv_project_weight",
         "out_linear_weight", "out_linear_bias", "in_project_x_scale", "in_project_fx_scale", "out_linear_scale")]
+
+
+class PaMlpParams(Structure):
+    _fields_ = [(n, c_void_p) for n in ("w1", "b1", "w2", "b2")]
 
 
 class PaBlockTail(Structure):
@@ -94,6 +98,13 @@ def load() -> ctypes.CDLL:
     lib.pa_mfma_partial_groups.argtypes = [ps, c_int]
     lib.pa_mfma_deslice_project.restype = c_int
     lib.pa_mfma_deslice_project.argtypes = [ps, c_void_p, c_void_p, c_void_p, c_void_p, pt, c_void_p]
+    lib.pa_mlp_query.restype = c_int
+    lib.pa_mlp_query.argtypes = [c_int, c_int64, c_int64, c_int64]
+    lib.pa_mlp_workspace_bytes.restype = c_int64
+    lib.pa_mlp_workspace_bytes.argtypes = [c_int, c_int64, c_int64, c_int64]
+    lib.pa_mlp_forward.restype = c_int
+    lib.pa_mlp_forward.argtypes = [c_int, c_int64, c_int64, c_int64, POINTER(PaMlpParams), c_void_p, c_void_p, pt, c_void_p,
+                                   c_int64, c_void_p]
     _lib = lib
     return lib
 

@@ -325,6 +325,30 @@ int pa_mfma_deslice_project(const pa_shape *shape, const void *blob, const void 
                                    static_cast<hipStream_t>(stream));
 }
 
+int pa_mlp_query(int dtype, int64_t rows, int64_t C, int64_t F) { return pa::mlp::supported(dtype, rows, C, F) ? 1 : 0; }
+
+int64_t pa_mlp_workspace_bytes(int dtype, int64_t rows, int64_t C, int64_t F) {
+  if (rows <= 0 || C <= 0 || F <= 0) return PA_ERR_DIMS;
+  if (!pa::mlp::supported(dtype, rows, C, F)) return PA_ERR_UNSUPPORTED;
+  return round_up(pa::mlp::blob_bytes(C, F), 256);
+}
+
+int pa_mlp_forward(int dtype, int64_t rows, int64_t C, int64_t F, const pa_mlp_params *p, const void *u, void *y,
+                   const pa_block_tail *tail, void *workspace, int64_t workspace_bytes, void *stream) {
+  if (rows <= 0 || C <= 0 || F <= 0) return PA_ERR_DIMS;
+  if (!pa::mlp::supported(dtype, rows, C, F)) return PA_ERR_UNSUPPORTED;
+  if (!p || !p->w1 || !p->b1 || !p->w2 || !p->b2 || !u || !y || !workspace) return PA_ERR_NULL;
+  if (!aligned16(p->w1) || !aligned16(p->w2) || !aligned16(u) || !aligned16(y) || !aligned16(workspace))
+    return PA_ERR_ALIGN;
+  int rc = check_tail(tail);
+  if (rc) return rc;
+  if (workspace_bytes < pa::mlp::blob_bytes(C, F)) return PA_ERR_WORKSPACE;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if ((rc = pa::mlp::pack(C, F, p->w1, p->w2, workspace, st))) return rc;
+  return pa::mlp::forward(rows, C, F, workspace, p->b1, p->b2, u, y, tail_active(tail) ? tail : nullptr, compute_units(),
+                          st);
+}
+
 int pa_layer_forward(int dtype, const pa_shape *shape, const pa_params *p, const void *x, void *y,
                      const pa_block_tail *tail, float *slice_token_out, void *workspace, int64_t workspace_bytes,
                      void *stream) {

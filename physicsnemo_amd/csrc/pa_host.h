@@ -45,4 +45,12 @@ int deslice_project(const pa_shape &s, const void *blob, const void *w_pack, con
                     const pa_block_tail *tail, int num_cu, hipStream_t st);
 }  // namespace mfma
 
+namespace mlp {
+bool supported(int dtype, int64_t rows, int64_t C, int64_t F);
+int64_t blob_bytes(int64_t C, int64_t F);
+int pack(int64_t C, int64_t F, const void *w1, const void *w2, void *blob, hipStream_t st);
+int forward(int64_t rows, int64_t C, int64_t F, const void *blob, const float *b1, const float *b2, const void *u,
+            void *y, const pa_block_tail *tail, int num_cu, hipStream_t st);
+}  // namespace mlp
+
 }  // namespace pa

@@ -20,32 +20,10 @@
 //                                                                                (A operand of the aggregation)
 #include "pa_common.h"
 #include "pa_host.h"
+#include "pa_mfma_ops.h"
 
 namespace pa {
 namespace mfma {
-
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef float f32x16 __attribute__((ext_vector_type(16)));
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
-
-__device__ __forceinline__ f32x16 mma(u32x4 a, u32x4 b, f32x16 c) {
-  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
-}
-
-__device__ __forceinline__ int rowmap(int r, int g) { return 8 * (r >> 2) + 4 * g + (r & 3); }
-__device__ __forceinline__ int kperm(int kk, int g, int j) { return 16 * kk + 8 * (j >> 2) + 4 * g + (j & 3); }
-
-// registers 8*HALF .. 8*HALF+7 of an accumulator, scaled, as 8 bf16 (round to nearest even)
-template <int HALF>
-__device__ __forceinline__ u32x4 pack_half(const f32x16 &v, float scale = 1.f) {
-  bf16x8 o;
-#pragma unroll
-  for (int j = 0; j < 8; ++j) o[j] = (__bf16)(v[8 * HALF + j] * scale);
-  return __builtin_bit_cast(u32x4, o);
-}
-
-__device__ __forceinline__ uint16_t to_bf16_bits(float f) { return __builtin_bit_cast(uint16_t, (__bf16)f); }
 
 // ------------------------------------------------------------------------------------------------
 // Packed parameter blob (built once per call by pack_params_kernel).  Offsets in 16-byte units.
@@ -120,17 +98,6 @@ __global__ __launch_bounds__(256) void pack_params_kernel(pa_params p, u32x4 *__
     else v = kLog2e / clamp_temperature(p.temperature[k - 3 * C - ST * 32]);
     fv[k] = v;
   }
-}
-
-// value of lane l combined with the value of lane l ^ 32, without a trip through LDS: v_permlane32_swap hands every
-// lane the lower-half and the upper-half value of its column
-__device__ __forceinline__ float half_max(float v) {
-  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
-}
-__device__ __forceinline__ float half_sum(float v) {
-  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
 // ------------------------------------------------------------------------------------------------

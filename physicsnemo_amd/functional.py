@@ -157,6 +157,36 @@ def layer_forward(x, params, dims: LayerDims, residual=None, ln_weight=None, ln_
     return (out, tok) if return_slice_tokens else out
 
 
+def mlp_supported(dtype: torch.dtype, rows: int, C: int, F: int) -> bool:
+    """True if `mlp_forward` serves this shape with the MFMA kernel (bf16, C in {128, 256}, F a multiple of 64)."""
+    if dtype != torch.bfloat16:
+        return False
+    return bool(_lib.load().pa_mlp_query(_lib.PA_BF16, rows, C, F))
+
+
+def mlp_forward(u, w1, b1, w2, b2, residual=None, ln_weight=None, ln_bias=None, ln_eps=1e-5):
+    """y = w2 . gelu(w1 . u + b1) + b2 [+ residual]; returns y, or (y, LayerNorm(y)) when ln_weight is given.
+
+    u (..., C) bfloat16; w1 (F, C), w2 (C, F) bfloat16; b1, b2, ln_weight, ln_bias float32."""
+    _need_cuda(u, w1, b1, w2, b2, residual, ln_weight, ln_bias)
+    lib = _lib.load()
+    C, F = w1.shape[1], w1.shape[0]
+    rows = u.numel() // C
+    code = _lib.dtype_code(u.dtype)
+    nbytes = lib.pa_mlp_workspace_bytes(code, rows, C, F)
+    if nbytes < 0:
+        _lib.check(int(nbytes), "pa_mlp_workspace_bytes")
+    workspace = torch.empty(int(nbytes), dtype=torch.uint8, device=u.device)
+    y = torch.empty_like(u)
+    ln_out = torch.empty_like(u) if ln_weight is not None else None
+    params = _lib.PaMlpParams(_lib.ptr(w1), _lib.ptr(b1), _lib.ptr(w2), _lib.ptr(b2))
+    tail = _c_tail(residual, ln_weight, ln_bias, ln_eps, ln_out)
+    _lib.check(lib.pa_mlp_forward(code, rows, C, F, byref(params), u.data_ptr(), y.data_ptr(), byref(tail),
+                                  workspace.data_ptr(), int(nbytes), _lib.current_stream_ptr(u.device)),
+               "pa_mlp_forward")
+    return y if ln_out is None else (y, ln_out)
+
+
 class MfmaStages:
     """The bf16 MFMA kernels one by one (pa_mfma_* entry points) with their opaque buffers held as torch tensors.
 

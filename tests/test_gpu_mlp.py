@@ -1,0 +1,82 @@
+"""GPU parity of the fused block MLP (pa_mlp_forward, through the C ABI) against the fp32 CPU oracle.
+
+Bar for bf16: relative L2 error <= 1e-2 against the fp32 oracle evaluated on the same bf16-rounded inputs/weights.
+"""
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import torch_oracle as to
+from physicsnemo_amd import functional as PF
+from gpu_util import announce, assert_rel_l2
+
+pytestmark = pytest.mark.gpu
+
+
+def _case(rows_shape, C, Fh, seed=0, scale=1.0):
+    torch.manual_seed(seed)
+    ref = to.OracleMlp(C, Fh, C).eval()
+    with torch.no_grad():
+        for p in ref.parameters():  # bf16-representable weights: both sides compute with the same numbers
+            p.mul_(scale)
+        ref.layers[0].weight.copy_(ref.layers[0].weight.bfloat16().float())
+        ref.layers[2].weight.copy_(ref.layers[2].weight.bfloat16().float())
+    u = torch.randn(*rows_shape, C).bfloat16()
+    res = torch.randn(*rows_shape, C).bfloat16()
+    gamma, beta = torch.rand(C) + 0.5, torch.randn(C) * 0.1
+    dev = torch.device("cuda:0")
+    args = dict(
+        u=u.to(dev), w1=ref.layers[0].weight.detach().bfloat16().to(dev).contiguous(),
+        b1=ref.layers[0].bias.detach().float().to(dev), w2=ref.layers[2].weight.detach().bfloat16().to(dev).contiguous(),
+        b2=ref.layers[2].bias.detach().float().to(dev))
+    return ref, u, res, gamma, beta, args
+
+
+@pytest.mark.parametrize("rows_shape,C,Fh", [
+    ((1, 4096), 256, 1024), ((2, 1000), 256, 1024), ((1, 257), 256, 256), ((3, 77), 128, 512), ((1, 1), 256, 1024),
+    ((1, 5000), 128, 128), ((1, 20000), 256, 512),
+])
+def test_mlp_matches_fp32_oracle(rows_shape, C, Fh):
+    announce("mlp", rows_shape, C, Fh)
+    ref, u, res, gamma, beta, args = _case(rows_shape, C, Fh)
+    assert PF.mlp_supported(torch.bfloat16, u.numel() // C, C, Fh)
+    dev = args["u"].device
+    with torch.no_grad():
+        want = ref(u.float())
+        want_sum = want + res.float()
+        want_ln = F.layer_norm(want_sum, (C,), gamma, beta, 1e-5)
+        y = PF.mlp_forward(**args)
+        y2, ln2 = PF.mlp_forward(**args, residual=res.to(dev), ln_weight=gamma.to(dev), ln_bias=beta.to(dev))
+        y3 = PF.mlp_forward(**args, residual=res.to(dev))
+        y4, ln4 = PF.mlp_forward(**args, ln_weight=gamma.to(dev), ln_bias=beta.to(dev))
+    assert y.dtype == torch.bfloat16 and y.shape == u.shape
+    assert torch.isfinite(y.float()).all()
+    assert_rel_l2(y, want, "mlp output")
+    assert_rel_l2(y2, want_sum, "mlp + residual")
+    assert_rel_l2(ln2, want_ln, "LayerNorm(mlp + residual)")
+    assert torch.equal(y3, y2)
+    assert torch.equal(y4, y)
+    assert_rel_l2(ln4, F.layer_norm(want, (C,), gamma, beta, 1e-5), "LayerNorm(mlp)")
+
+
+def test_mlp_gelu_tails_and_determinism():
+    announce("mlp large activations / determinism")
+    # large pre-activations exercise both saturated ends of the erf and the sign handling
+    ref, u, res, gamma, beta, args = _case((1, 3000), 256, 1024, seed=3, scale=6.0)
+    with torch.no_grad():
+        want = ref(u.float())
+        y = PF.mlp_forward(**args)
+        y_again = PF.mlp_forward(**args)
+    assert_rel_l2(y, want, "mlp output, large activations")
+    assert torch.equal(y, y_again)
+    # rows are independent: a prefix gives the same bits
+    args_prefix = dict(args, u=args["u"][:, :777].contiguous())
+    with torch.no_grad():
+        y_prefix = PF.mlp_forward(**args_prefix)
+    assert torch.equal(y_prefix, y[:, :777])
+
+
+def test_mlp_rejects_unsupported():
+    assert not PF.mlp_supported(torch.float32, 100, 256, 1024)
+    assert not PF.mlp_supported(torch.bfloat16, 100, 512, 2048)
+    assert not PF.mlp_supported(torch.bfloat16, 100, 256, 1000)
