@@ -1,55 +1,64 @@
 // Fused block MLP on gfx950 MFMA:  y = W2 . gelu(W1 . u + b1) + b2  [+ residual]  [-> LayerNorm(y)]
 // for bf16 rows u (M x C), hidden width F, C in {128, 256}, F a multiple of 64.
 // Replaces the reference's `ln_mlp1[1](ln) + fx` (physicsnemo/models/transolver/transolver.py:301-303; Mlp:
-// physicsnemo/nn/module/mlp_layers.py:139-173, GELU = exact erf form, activations.py:188-243) and hands the
+// physicsnemo/nn/module/mlp_layers.py:139-173, GELU = erf form, activations.py:188-243) and hands the
 // LayerNorm of the result to the next consumer (next block's ln_1 or the output head's LayerNorm).
 //
-// One workgroup of 4 waves per CU, one wave per SIMD (512 registers per lane); wave w owns 64 rows of a block of
-// 256 rows:
-//   * its rows of u stay in registers as B operands for the whole block (lane <-> row, k <-> channel);
-//   * the weights stream through LDS in chunks of 64 hidden units, fetched with direct global -> LDS loads one chunk
-//     ahead (two buffers, one barrier per chunk); every weight fragment read from LDS feeds two MFMAs (the wave's two
-//     32-row halves), which keeps LDS at half its bandwidth;
-//   * h^T (64 hidden x rows) = W1_chunk . u^T comes out with lanes <-> rows and registers <-> hidden units, so
-//     gelu(h) rounded to bf16 is directly the B operand of  y^T (C x rows) += W2_chunk . gelu(h)^T;
-//   * the y^T accumulators of all C channels (2 * C/32 * 16 = 256 registers for C = 256) live in the accumulation
-//     registers for the whole block;
-//   * epilogue: y^T -> bf16 -> this wave's share of the idle weight buffer (granule-swizzled transpose) -> row-major
-//     rows: + residual, LayerNorm statistics by DPP reductions, full-row coalesced stores.
+// One workgroup of 4 waves per CU, one wave per SIMD (256 vector + 256 accumulation registers per lane).  A block
+// of 128 rows is shared by two pairs of waves; the waves (rg, p = 0 / 1) of a pair own the same 64 rows:
+//   * the rows of u stay in registers as B operands for the whole block (lane <-> row, k <-> channel);
+//   * the weights stream through LDS in slots of 64 hidden units, fetched with direct global -> LDS loads one slot
+//     ahead (two buffers); every weight fragment read from LDS feeds two MFMAs (the two 32-row halves), which
+//     keeps LDS at half its bandwidth;
+//   * wave p computes hidden tile p (32 units) of the slot: h^T = W1_tile . u^T comes out with lanes <-> rows and
+//     registers <-> hidden units, so gelu(h) rounded to bf16 is directly a B operand of the second product; the
+//     partner's tile comes through LDS;
+//   * wave p accumulates y^T (C/2 channels x 64 rows) += W2[channel half p, slot] . gelu(h)^T in accumulation
+//     registers for the whole block.  The second product runs one slot behind the first, so the VALU work of the
+//     activation of slot c is issued behind the MFMAs of the second product of slot c-1 (slot c of the packed
+//     weights therefore holds W1 of hidden chunk c and W2 of hidden chunk c-1);
+//   * epilogue: y^T -> bf16 -> the idle weight buffer (granule-swizzled transpose, both waves of a pair) ->
+//     row-major rows: + residual, LayerNorm statistics by DPP reductions, full-row coalesced stores.
 #include "pa_common.h"
 #include "pa_host.h"
 #include "pa_mfma_ops.h"
 
 #include <type_traits>
+#include <utility>
 
 namespace pa {
 namespace mlp {
 
 using namespace pa::mfma;
 
-constexpr int kRowsPerBlock = 256;  // 4 waves x 64 rows
+constexpr int kRowsPerBlock = 128;  // 2 pairs of waves x 64 rows
 
-// 16-byte units of one weight chunk: W1 fragments [n 2][ks C/16][lane], then W2 fragments [ct C/32][k4 4][lane]
-__host__ __device__ constexpr int chunk_units(int C) { return (2 * (C / 16) + (C / 32) * 4) * 64; }
+// 16-byte units of one weight slot: W1 fragments [n 2][ks C/16][lane], then W2 fragments [ct C/32][k4 4][lane]
+__host__ __device__ constexpr int slot_units(int C) { return (2 * (C / 16) + (C / 32) * 4) * 64; }
 
-// W1 (F x C) and W2 (C x F), bf16 row-major -> fragment order, chunk after chunk.
+// W1 (F x C) and W2 (C x F), bf16 row-major -> fragment order, F/64 + 1 slots: slot c holds W1 of hidden chunk c
+// (zeros in the last slot) and W2 of hidden chunk c - 1 (zeros in the first).
 //   W1 fragment (n, ks): lane (i, g) holds W1[64c + 32n + i][16ks + 8g + j]
-//   W2 fragment (ct, k4 = 2n + kk): lane (i, g) holds W2[32ct + i][64c + 32n + kperm(kk, g, j)]
+//   W2 fragment (ct, k4 = 2n + kk): lane (i, g) holds W2[32ct + i][64(c-1) + 32n + kperm(kk, g, j)]
 __global__ __launch_bounds__(256) void pack_kernel(const uint16_t *__restrict__ w1, const uint16_t *__restrict__ w2,
                                                    u32x4 *__restrict__ blob, int C, int F) {
-  const int KS = C / 16, NF1 = 2 * KS, CU = chunk_units(C);
-  const int64_t total = (int64_t)(F / 64) * CU;
+  const int KS = C / 16, NF1 = 2 * KS, SU = slot_units(C), NC = F / 64;
+  const int64_t total = (int64_t)(NC + 1) * SU;
   for (int64_t u = (int64_t)blockIdx.x * 256 + threadIdx.x; u < total; u += (int64_t)gridDim.x * 256) {
-    const int c = (int)(u / CU), r = (int)(u - (int64_t)c * CU), frag = r >> 6, lane = r & 63, i = lane & 31, g = lane >> 5;
+    const int c = (int)(u / SU), r = (int)(u - (int64_t)c * SU), frag = r >> 6, lane = r & 63, i = lane & 31, g = lane >> 5;
     uint16_t e[8];
-    if (frag < NF1) {
-      const int n = frag / KS, ks = frag - n * KS;
-      const uint16_t *src = w1 + (int64_t)(64 * c + 32 * n + i) * C + 16 * ks + 8 * g;
 #pragma unroll
-      for (int j = 0; j < 8; ++j) e[j] = src[j];
-    } else {
+    for (int j = 0; j < 8; ++j) e[j] = 0;
+    if (frag < NF1) {
+      if (c < NC) {
+        const int n = frag / KS, ks = frag - n * KS;
+        const uint16_t *src = w1 + (int64_t)(64 * c + 32 * n + i) * C + 16 * ks + 8 * g;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) e[j] = src[j];
+      }
+    } else if (c > 0) {
       const int q = frag - NF1, ct = q >> 2, k4 = q & 3, n = k4 >> 1, kk = k4 & 1;
-      const uint16_t *src = w2 + (int64_t)(32 * ct + i) * F + 64 * c + 32 * n;
+      const uint16_t *src = w2 + (int64_t)(32 * ct + i) * F + 64 * (c - 1) + 32 * n;
 #pragma unroll
       for (int j = 0; j < 8; ++j) e[j] = src[kperm(kk, g, j)];
     }
@@ -60,26 +69,49 @@ __global__ __launch_bounds__(256) void pack_kernel(const uint16_t *__restrict__ 
   }
 }
 
-// 64 x 16 bytes, one per lane, from global memory straight into LDS at lds_wave_base + lane (no registers).
-// The load is asynchronous and counted by vmcnt; its data must not be read before a wait and a barrier.
-__device__ __forceinline__ void load_to_lds(const u32x4 *gsrc_lane, u32x4 *lds_wave_base) {
-  const unsigned lds = __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)lds_wave_base);
-  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds), "v"(gsrc_lane) : "memory");
+// Four direct global -> LDS loads of 64 x 16 bytes each (no registers): the wave's lanes read sbase + voff + k KiB
+// (voff = 16 * lane) and the data land at LDS byte address lds + k KiB + 16 * lane, k = 0..3 (the instruction offset
+// applies to the global and to the LDS address alike).  sbase and lds are wave-uniform.  The loads are asynchronous
+// and counted by vmcnt; their data must not be read before a wait and a barrier.
+__device__ __forceinline__ void load4_to_lds(const void *sbase, unsigned voff, unsigned lds) {
+  asm volatile(
+      "s_mov_b32 m0, %2\n\t"
+      "s_nop 0\n\t"
+      "global_load_lds_dwordx4 %1, %0\n\t"
+      "global_load_lds_dwordx4 %1, %0 offset:1024\n\t"
+      "global_load_lds_dwordx4 %1, %0 offset:2048\n\t"
+      "global_load_lds_dwordx4 %1, %0 offset:3072" ::"s"(sbase),
+      "v"(voff), "s"(lds)
+      : "memory");
 }
 
-// exact-erf GELU; erf by Abramowitz-Stegun 7.1.26 (|error| < 2e-7 in fp32)
-__device__ __forceinline__ float gelu_erf(float x) {
-  const float z = x * 0.70710678118654752f, a = fabsf(z);
-  const float t = __builtin_amdgcn_rcpf(fmaf(0.3275911f, a, 1.f));
-  float p = fmaf(1.061405429f, t, -1.453152027f);
-  p = fmaf(p, t, 1.421413741f);
-  p = fmaf(p, t, -0.284496736f);
-  p = fmaf(p, t, 0.254829592f);
-  p *= t;
-  const float e = __builtin_amdgcn_exp2f(a * a * -kLog2e);
-  const float er = copysignf(fmaf(-p, e, 1.f), z);
-  const float hx = 0.5f * x;
-  return fmaf(hx, er, hx);
+// f(integral_constant<int, 0>{}), ..., f(integral_constant<int, N - 1>{}): a loop whose index is a constant expression
+template <class F, int... I>
+__device__ __forceinline__ void static_for_impl(F &&f, std::integer_sequence<int, I...>) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void static_for(F &&f) {
+  static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+
+// GELU(x) = x * Phi(x), Phi in the logistic form 1 / (1 + exp(-2 x P(x^2))) with P fitted to the exact erf form:
+// max |error| 2.6e-5 over all x (the plain tanh form has 4.7e-4); |x| is clamped where Phi is 0 or 1 in fp32.
+__device__ __forceinline__ float gelu(float x) {
+  const float x2 = fminf(x * x, 81.f);  // beyond |x| = 9 Phi is 0 or 1 in fp32; keeps x P(x^2) monotone
+  // -2 * log2(e) * (c0 + c1 x^2 + c2 x^4)
+  float p = fmaf(-3.51902394e-04f * -2.f * kLog2e, x2, 3.70080200e-02f * -2.f * kLog2e);
+  p = fmaf(p, x2, 7.97505275e-01f * -2.f * kLog2e);
+  const float e = __builtin_amdgcn_exp2f(x * p);
+  return x * __builtin_amdgcn_rcpf(1.f + e);
+}
+
+// 8 floats -> 8 bf16 (round to nearest even)
+__device__ __forceinline__ u32x4 pack8(const float (&v)[8]) {
+  bf16x8 o;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) o[j] = (__bf16)v[j];
+  return __builtin_bit_cast(u32x4, o);
 }
 
 // sum over the 64 lanes, returned in every lane: DPP steps inside each row of 16, then the four row totals
@@ -103,17 +135,20 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     const float *__restrict__ ln_gamma, const float *__restrict__ ln_beta, float ln_eps, uint16_t *__restrict__ ln_out,
     int64_t M, int F, int64_t nblocks) {
   constexpr bool HAS_RES = TAIL == 1 || TAIL == 2, HAS_LN = TAIL == 1 || TAIL == 3;
-  constexpr int KS = C / 16, CT = C / 32, NF1 = 2 * KS, CU = chunk_units(C);
-  constexpr int WU = CU / 4;     // units of a chunk fetched by each wave = its staging share in the epilogue
-  constexpr int NDMA = WU / 64;  // direct-to-LDS loads per wave and chunk
+  constexpr int KS = C / 16, CT = C / 32, CTH = CT / 2, NF1 = 2 * KS, SU = slot_units(C);
+  constexpr int WU = SU / 4;     // units of a slot fetched by each wave
+  constexpr int NDMA = WU / 64;  // direct-to-LDS loads per wave and slot
   constexpr int CPL = C / 64;    // consecutive channels per lane in the row-major epilogue
   constexpr int G4 = C / 4;      // 8-byte granules (4 channels) per staged row
-  static_assert(WU * 16 == 32 * C * 2, "a wave's share of a chunk buffer must hold 32 bf16 rows");
+  static_assert(SU * 16 == 128 * C * 2, "a slot buffer must hold the 128 bf16 rows of a block in the epilogue");
   extern __shared__ u32x4 smem[];
-  u32x4 *wbuf = smem;  // 2 * CU
-  float *b1s = reinterpret_cast<float *>(smem + 2 * CU);
+  u32x4 *wbuf = smem;            // 2 * SU
+  u32x4 *xch = wbuf + 2 * SU;    // [wave 4][m 2][kk 2][lane]: gelu(h) tiles handed to the partner wave
+  float *b1s = reinterpret_cast<float *>(xch + 4 * 4 * 64);
   float *b2s = b1s + F;
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, i = lane & 31, g = lane >> 5;
+  const int tid = threadIdx.x, lane = tid & 63, i = lane & 31, g = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: addresses derived from it stay scalar
+  const int rg = wave >> 1, p = wave & 1;
   const int NC = F / 64;
 
   for (int k = tid; k < F; k += 256) b1s[k] = b1[k];
@@ -125,18 +160,19 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     bet[k] = HAS_LN ? ln_beta[lane * CPL + k] : 0.f;
   }
 
-  auto fetch_chunk = [&](int64_t gc, int c) {  // this wave's share of chunk c into buffer gc & 1
-    const u32x4 *src = blob + (int64_t)c * CU + wave * WU + lane;
-    u32x4 *dst = wbuf + (gc & 1) * CU + wave * WU;
+  static_assert(NDMA % 4 == 0, "a wave fetches its share of a slot four loads at a time");
+  auto fetch_slot = [&](int64_t gs, int c) {  // this wave's share of slot c into buffer gs & 1
+    const u32x4 *src = blob + (int64_t)c * SU + wave * WU;
+    const unsigned dst = (unsigned)(uintptr_t)(wbuf + (gs & 1) * SU + wave * WU);
 #pragma unroll
-    for (int q = 0; q < NDMA; ++q) load_to_lds(src + q * 64, dst + q * 64);
+    for (int q = 0; q < NDMA; q += 4) load4_to_lds(src + q * 64, lane * 16, dst + q * 1024);
   };
 
-  int64_t gc = 0;  // chunks processed so far by this workgroup (buffer parity)
-  if ((int64_t)blockIdx.x < nblocks) fetch_chunk(0, 0);
+  int64_t gs = 0;  // slots processed so far by this workgroup (buffer parity)
+  if ((int64_t)blockIdx.x < nblocks) fetch_slot(0, 0);
   for (int64_t mb = blockIdx.x; mb < nblocks; mb += gridDim.x) {
-    // this wave's rows as B operands: lane (i, g) holds row 32m + i, channels 16ks + 8g .. + 7
-    const int64_t row0 = mb * kRowsPerBlock + wave * 64;
+    // the pair's rows as B operands: lane (i, g) holds row 32m + i, channels 16ks + 8g .. + 7
+    const int64_t row0 = mb * kRowsPerBlock + rg * 64;
     u32x4 ub[2][KS];
 #pragma unroll
     for (int m = 0; m < 2; ++m) {
@@ -146,144 +182,188 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) ub[m][ks] = *reinterpret_cast<const u32x4 *>(src + 16 * ks);
     }
-    f32x16 yacc[2][CT];
+    f32x16 yacc[2][CTH];  // channels 32 * (CTH * p + ct) + rowmap(r, g)
 #pragma unroll
     for (int m = 0; m < 2; ++m)
 #pragma unroll
-      for (int ct = 0; ct < CT; ++ct)
+      for (int ct = 0; ct < CTH; ++ct)
 #pragma unroll
         for (int r = 0; r < 16; ++r) yacc[m][ct][r] = 0.f;
+    // gelu(h) of hidden chunk c-1 as B operands [m][kk]: this wave's tile and the partner's
+    u32x4 hown[2][2], hpar[2][2];
+    float hrest[2][8];  // second half (registers 8..15) of this wave's h tile of chunk c-1, before the activation
+#pragma unroll
+    for (int m = 0; m < 2; ++m) {
+      hown[m][0] = u32x4{0, 0, 0, 0};
+#pragma unroll
+      for (int j = 0; j < 8; ++j) hrest[m][j] = 0.f;
+    }
 
-    for (int c = 0; c < NC; ++c, ++gc) {
-      // chunk gc has landed (every wave waits for its own share, then all meet); the other buffer is free
+    for (int c = 0; c <= NC; ++c, ++gs) {
+      // slot gs has landed (every wave waits for its own share, then all meet) and the other buffer is free
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       __syncthreads();
-      if (c + 1 < NC) fetch_chunk(gc + 1, c + 1);
-      else if (mb + gridDim.x < nblocks) fetch_chunk(gc + 1, 0);
-      const u32x4 *wb = wbuf + (gc & 1) * CU + lane;
+      if (c < NC) fetch_slot(gs + 1, c + 1);
+      else if (mb + gridDim.x < nblocks) fetch_slot(gs + 1, 0);
+      const u32x4 *wb = wbuf + (gs & 1) * SU + lane;
+      // this wave's fragments of the slot: W1 of hidden tile p; W2 of its channel half, hidden tile p ("own") first
+      const u32x4 *w1f = wb + p * KS * 64;
+      const u32x4 *w2own = wb + (NF1 + p * CTH * 4 + 2 * p) * 64, *w2par = wb + (NF1 + p * CTH * 4 + 2 * (1 - p)) * 64;
 
-      // h^T = W1_chunk . u^T + b1: two tiles of 32 hidden units for each of the two row halves
-      f32x16 hacc[2][2];
+      // One slot = 2 phases of KS resp. 4 * CTH steps; a step = one weight fragment (read from LDS AHEAD steps
+      // early), two MFMAs and, behind them, one or two gelu evaluations:
+      //   phase 1   h^T tile p of hidden chunk c += W1 fragment . u^T (both row halves);
+      //             gelu of the second half of the tile of chunk c-1 -> the tile is complete, goes to the partner
+      //   phase 2   y^T += W2 fragment(ct, k4) of hidden chunk c-1 . gelu(h)^T (own tile, then the partner's);
+      //             gelu of the first half of the tile of chunk c
+      constexpr int RING = 4, AHEAD = 3;
+      f32x16 hacc[2];
 #pragma unroll
-      for (int n = 0; n < 2; ++n)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) hacc[0][n][r] = hacc[1][n][r] = b1s[64 * c + 32 * n + rowmap(r, g)];
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks)
-#pragma unroll
-        for (int n = 0; n < 2; ++n) {
-          const u32x4 a = wb[(n * KS + ks) * 64];
-          hacc[0][n] = mma(a, ub[0][ks], hacc[0][n]);
-          hacc[1][n] = mma(a, ub[1][ks], hacc[1][n]);
-        }
-      // gelu, rounded to bf16: B operands of the second product (k4 = 2n + kk)
-      u32x4 hb[2][4];
+      for (int r = 0; r < 16; ++r) hacc[0][r] = hacc[1][r] = b1s[(c < NC ? 64 * c : 0) + 32 * p + rowmap(r, g)];
+      {
+        constexpr int EV = 16 / KS > 0 ? 16 / KS : 1;  // evaluations per step (16 over KS steps)
+        static_assert(KS * EV == 16 || KS == 16, "phase 1 must cover 16 evaluations");
+        u32x4 fr[RING];
+        static_for<AHEAD>([&](auto q) { fr[decltype(q)::value] = w1f[decltype(q)::value * 64]; });
+        static_for<KS>([&](auto st) {
+          constexpr int step = decltype(st)::value;
+          if constexpr (step + AHEAD < KS) fr[(step + AHEAD) % RING] = w1f[(step + AHEAD) * 64];
+          const u32x4 a = fr[step % RING];
+          hacc[0] = mma(a, ub[0][step], hacc[0]);
+          hacc[1] = mma(a, ub[1][step], hacc[1]);
+          static_for<(KS == 16 ? 1 : 16 / KS)>([&](auto q) {
+            constexpr int E = step * (KS == 16 ? 1 : 16 / KS) + decltype(q)::value, m = E / 8, j = E % 8;
+            hrest[m][j] = gelu(hrest[m][j]);
+            if constexpr (j == 7) hown[m][1] = pack8(hrest[m]);
+          });
+          __builtin_amdgcn_sched_barrier(0);  // keeps the issue order as written
+        });
+      }
+      // the tile of chunk c-1 is complete: hand it to the partner, take the partner's
 #pragma unroll
       for (int m = 0; m < 2; ++m)
 #pragma unroll
-        for (int n = 0; n < 2; ++n) {
+        for (int kk = 0; kk < 2; ++kk) xch[((wave * 2 + m) * 2 + kk) * 64 + lane] = hown[m][kk];
+      __syncthreads();
 #pragma unroll
-          for (int r = 0; r < 16; ++r) hacc[m][n][r] = gelu_erf(hacc[m][n][r]);
-          hb[m][2 * n] = pack_half<0>(hacc[m][n]);
-          hb[m][2 * n + 1] = pack_half<1>(hacc[m][n]);
+      for (int m = 0; m < 2; ++m)
+#pragma unroll
+        for (int kk = 0; kk < 2; ++kk) hpar[m][kk] = xch[(((wave ^ 1) * 2 + m) * 2 + kk) * 64 + lane];
+      {
+        constexpr int NS2 = 4 * CTH, EV = 16 / NS2 > 0 ? 16 / NS2 : 1;
+        static_assert(NS2 * EV == 16, "phase 2 must cover 16 evaluations");
+        float fl[2][8];
+        u32x4 hfirst[2];
+        auto frag2 = [&](auto st) {  // step -> (k4' = step / CTH, ct = step % CTH); k4' < 2: own tile, kk = k4' % 2
+          constexpr int t = decltype(st)::value, k4 = t / CTH, ct = t % CTH;
+          return (k4 < 2 ? w2own : w2par)[(ct * 4 + (k4 & 1)) * 64];
+        };
+        u32x4 fr[RING];
+        static_for<AHEAD>([&](auto q) { fr[decltype(q)::value] = frag2(q); });
+        static_for<NS2>([&](auto st) {
+          constexpr int t = decltype(st)::value, k4 = t / CTH, ct = t % CTH, kk = k4 & 1;
+          if constexpr (t + AHEAD < NS2) fr[(t + AHEAD) % RING] = frag2(std::integral_constant<int, t + AHEAD>{});
+          const u32x4 a = fr[t % RING];
+          yacc[0][ct] = mma(a, k4 < 2 ? hown[0][kk] : hpar[0][kk], yacc[0][ct]);
+          yacc[1][ct] = mma(a, k4 < 2 ? hown[1][kk] : hpar[1][kk], yacc[1][ct]);
+          static_for<EV>([&](auto q) {
+            constexpr int E = t * EV + decltype(q)::value, m = E / 8, j = E % 8;
+            fl[m][j] = gelu(hacc[m][j]);
+            if constexpr (j == 7) hfirst[m] = pack8(fl[m]);
+          });
+          __builtin_amdgcn_sched_barrier(0);
+        });
+#pragma unroll
+        for (int m = 0; m < 2; ++m) {
+          hown[m][0] = hfirst[m];
+#pragma unroll
+          for (int j = 0; j < 8; ++j) hrest[m][j] = hacc[m][8 + j];
         }
-      // y^T += W2_chunk . gelu(h)^T
-#pragma unroll
-      for (int k4 = 0; k4 < 4; ++k4)
-#pragma unroll
-        for (int ct = 0; ct < CT; ++ct) {
-          const u32x4 a = wb[(NF1 + ct * 4 + k4) * 64];
-          yacc[0][ct] = mma(a, hb[0][k4], yacc[0][ct]);
-          yacc[1][ct] = mma(a, hb[1][k4], yacc[1][ct]);
-        }
+      }
     }
 
-    // ---- epilogue: the buffer of the last chunk is idle once every wave is past its last MFMA ----
+    // ---- epilogue: the buffer of the last slot is idle once every wave is past its last MFMA ----
     __syncthreads();
-    uint32_t *stg = reinterpret_cast<uint32_t *>(wbuf + ((gc - 1) & 1) * CU + wave * WU);  // [32 rows][C/2 words]
+    uint32_t *stg = reinterpret_cast<uint32_t *>(wbuf + ((gs - 1) & 1) * SU) + rg * 64 * (C / 2);  // [64 rows][C/2 words]
+    // y^T + b2 -> bf16 -> staged rows; granule gr (4 channels) of row rw sits at gr ^ ((2 rw) % G4)
 #pragma unroll
-    for (int m = 0; m < 2; ++m) {
-      // y^T + b2 -> bf16 -> staged rows; granule gr (4 channels) of row i sits at gr ^ ((2i) % G4)
+    for (int m = 0; m < 2; ++m)
 #pragma unroll
-      for (int ct = 0; ct < CT; ++ct)
+      for (int ct = 0; ct < CTH; ++ct)
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-          const int ch = 32 * ct + 8 * q + 4 * g;
+          const int ch = 32 * (CTH * p + ct) + 8 * q + 4 * g, rw = 32 * m + i;
           const float v0 = yacc[m][ct][4 * q + 0] + b2s[ch + 0], v1 = yacc[m][ct][4 * q + 1] + b2s[ch + 1];
           const float v2 = yacc[m][ct][4 * q + 2] + b2s[ch + 2], v3 = yacc[m][ct][4 * q + 3] + b2s[ch + 3];
-          const int gr = (ch >> 2) ^ ((2 * i) & (G4 - 1));
+          const int gr = (ch >> 2) ^ ((2 * rw) & (G4 - 1));
           u32x2 pk;
           pk[0] = (uint32_t)to_bf16_bits(v0) | ((uint32_t)to_bf16_bits(v1) << 16);
           pk[1] = (uint32_t)to_bf16_bits(v2) | ((uint32_t)to_bf16_bits(v3) << 16);
-          *reinterpret_cast<u32x2 *>(stg + i * (C / 2) + gr * 2) = pk;
+          *reinterpret_cast<u32x2 *>(stg + rw * (C / 2) + gr * 2) = pk;
         }
-      __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "workgroup");  // staged rows are read back by other lanes of this wave
-      __builtin_amdgcn_wave_barrier();
-      // rows, 8 at a time: lane holds CPL consecutive channels
-      constexpr int RB = 8;
+    __syncthreads();  // both waves of a pair have staged their channel halves
+    // wave p finishes rows 32p .. 32p+31 of the pair, 8 at a time: lane holds CPL consecutive channels
+    constexpr int RB = 8;
 #pragma unroll 1
-      for (int rb = 0; rb < 32; rb += RB) {
-        uint32_t rsd[RB][CPL / 2];
-        if constexpr (HAS_RES) {
-#pragma unroll
-          for (int rr = 0; rr < RB; ++rr) {
-            int64_t r = row0 + 32 * m + rb + rr;
-            if (r >= M) r = M - 1;
-#pragma unroll
-            for (int w = 0; w < CPL / 2; ++w)
-              rsd[rr][w] = *reinterpret_cast<const uint32_t *>(residual + r * C + lane * CPL + 2 * w);
-          }
-        }
+    for (int rb = 0; rb < 32; rb += RB) {
+      uint32_t rsd[RB][CPL / 2];
+      if constexpr (HAS_RES) {
 #pragma unroll
         for (int rr = 0; rr < RB; ++rr) {
-          const int row = rb + rr;
-          const int64_t r = row0 + 32 * m + row;
-          const bool ok = r < M;
-          float v[CPL];
-          uint32_t ob[CPL / 2];
+          int64_t r = row0 + 32 * p + rb + rr;
+          if (r >= M) r = M - 1;
 #pragma unroll
-          for (int w = 0; w < CPL / 2; ++w) {
-            const int word = lane * (CPL / 2) + w;  // word of the row; granule = word / 2
-            const uint32_t sv = stg[row * (C / 2) + ((((word >> 1) ^ ((2 * row) & (G4 - 1))) << 1) | (word & 1))];
-            float t0 = bf16_bits_to_f32((uint16_t)(sv & 0xffffu)), t1 = bf16_bits_to_f32((uint16_t)(sv >> 16));
-            if constexpr (HAS_RES) {  // the MLP output is a bf16 tensor; the sum is rounded again
-              t0 += bf16_bits_to_f32((uint16_t)(rsd[rr][w] & 0xffffu));
-              t1 += bf16_bits_to_f32((uint16_t)(rsd[rr][w] >> 16));
-            }
-            const uint16_t o0 = to_bf16_bits(t0), o1 = to_bf16_bits(t1);
-            v[2 * w] = bf16_bits_to_f32(o0);
-            v[2 * w + 1] = bf16_bits_to_f32(o1);
-            ob[w] = (uint32_t)o0 | ((uint32_t)o1 << 16);
+          for (int w = 0; w < CPL / 2; ++w)
+            rsd[rr][w] = *reinterpret_cast<const uint32_t *>(residual + r * C + lane * CPL + 2 * w);
+        }
+      }
+#pragma unroll
+      for (int rr = 0; rr < RB; ++rr) {
+        const int rw = 32 * p + rb + rr;
+        const int64_t r = row0 + rw;
+        const bool ok = r < M;
+        float v[CPL];
+        uint32_t ob[CPL / 2];
+#pragma unroll
+        for (int w = 0; w < CPL / 2; ++w) {
+          const int word = lane * (CPL / 2) + w;  // word of the row; granule = word / 2
+          const uint32_t sv = stg[rw * (C / 2) + ((((word >> 1) ^ ((2 * rw) & (G4 - 1))) << 1) | (word & 1))];
+          float t0 = bf16_bits_to_f32((uint16_t)(sv & 0xffffu)), t1 = bf16_bits_to_f32((uint16_t)(sv >> 16));
+          if constexpr (HAS_RES) {  // the MLP output is a bf16 tensor; the sum is rounded again
+            t0 += bf16_bits_to_f32((uint16_t)(rsd[rr][w] & 0xffffu));
+            t1 += bf16_bits_to_f32((uint16_t)(rsd[rr][w] >> 16));
           }
+          const uint16_t o0 = to_bf16_bits(t0), o1 = to_bf16_bits(t1);
+          v[2 * w] = bf16_bits_to_f32(o0);
+          v[2 * w + 1] = bf16_bits_to_f32(o1);
+          ob[w] = (uint32_t)o0 | ((uint32_t)o1 << 16);
+        }
+        if (ok) {
+#pragma unroll
+          for (int w = 0; w < CPL / 2; ++w) *reinterpret_cast<uint32_t *>(y + r * C + lane * CPL + 2 * w) = ob[w];
+        }
+        if constexpr (HAS_LN) {
+          float s1 = 0.f;
+#pragma unroll
+          for (int k = 0; k < CPL; ++k) s1 += v[k];
+          const float mean = wave_sum_dpp(s1) * (1.f / C);
+          float s2 = 0.f;
+#pragma unroll
+          for (int k = 0; k < CPL; ++k) {
+            const float dl = v[k] - mean;
+            s2 = fmaf(dl, dl, s2);
+          }
+          const float rstd = rsqrtf(wave_sum_dpp(s2) * (1.f / C) + ln_eps);
           if (ok) {
 #pragma unroll
-            for (int w = 0; w < CPL / 2; ++w) *reinterpret_cast<uint32_t *>(y + r * C + lane * CPL + 2 * w) = ob[w];
-          }
-          if constexpr (HAS_LN) {
-            float s1 = 0.f;
-#pragma unroll
-            for (int k = 0; k < CPL; ++k) s1 += v[k];
-            const float mean = wave_sum_dpp(s1) * (1.f / C);
-            float s2 = 0.f;
-#pragma unroll
-            for (int k = 0; k < CPL; ++k) {
-              const float dl = v[k] - mean;
-              s2 = fmaf(dl, dl, s2);
-            }
-            const float rstd = rsqrtf(wave_sum_dpp(s2) * (1.f / C) + ln_eps);
-            if (ok) {
-#pragma unroll
-              for (int w = 0; w < CPL / 2; ++w) {
-                const uint16_t l0 = to_bf16_bits((v[2 * w] - mean) * rstd * gam[2 * w] + bet[2 * w]);
-                const uint16_t l1 = to_bf16_bits((v[2 * w + 1] - mean) * rstd * gam[2 * w + 1] + bet[2 * w + 1]);
-                *reinterpret_cast<uint32_t *>(ln_out + r * C + lane * CPL + 2 * w) = (uint32_t)l0 | ((uint32_t)l1 << 16);
-              }
+            for (int w = 0; w < CPL / 2; ++w) {
+              const uint16_t l0 = to_bf16_bits((v[2 * w] - mean) * rstd * gam[2 * w] + bet[2 * w]);
+              const uint16_t l1 = to_bf16_bits((v[2 * w + 1] - mean) * rstd * gam[2 * w + 1] + bet[2 * w + 1]);
+              *reinterpret_cast<uint32_t *>(ln_out + r * C + lane * CPL + 2 * w) = (uint32_t)l0 | ((uint32_t)l1 << 16);
             }
           }
         }
       }
-      __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "workgroup");  // rows read before the other half overwrites the stage
-      __builtin_amdgcn_wave_barrier();
     }
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // nothing may still be landing in LDS when the workgroup ends
@@ -294,12 +374,12 @@ bool supported(int dtype, int64_t rows, int64_t C, int64_t F) {
   return dtype == PA_BF16 && rows > 0 && (C == 128 || C == 256) && F >= 64 && F % 64 == 0 && F <= 8192;
 }
 
-int64_t blob_bytes(int64_t C, int64_t F) { return (F / 64) * (int64_t)chunk_units((int)C) * 16; }
+int64_t blob_bytes(int64_t C, int64_t F) { return (F / 64 + 1) * (int64_t)slot_units((int)C) * 16; }
 
-static size_t lds_bytes(int C, int F) { return (size_t)2 * chunk_units(C) * 16 + (size_t)(F + C) * 4; }
+static size_t lds_bytes(int C, int F) { return (size_t)(2 * slot_units(C) + 4 * 4 * 64) * 16 + (size_t)(F + C) * 4; }
 
 int pack(int64_t C, int64_t F, const void *w1, const void *w2, void *blob, hipStream_t st) {
-  const int64_t total = (F / 64) * (int64_t)chunk_units((int)C);
+  const int64_t total = (F / 64 + 1) * (int64_t)slot_units((int)C);
   const int grid = (int)((total + 255) / 256 < 1024 ? (total + 255) / 256 : 1024);
   hipLaunchKernelGGL(pack_kernel, dim3(grid), dim3(256), 0, st, static_cast<const uint16_t *>(w1),
                      static_cast<const uint16_t *>(w2), static_cast<u32x4 *>(blob), (int)C, (int)F);
