@@ -69,18 +69,14 @@ __global__ __launch_bounds__(256) void pack_kernel(const uint16_t *__restrict__ 
   }
 }
 
-// Four direct global -> LDS loads of 64 x 16 bytes each (no registers): the wave's lanes read sbase + voff + k KiB
-// (voff = 16 * lane) and the data land at LDS byte address lds + k KiB + 16 * lane, k = 0..3 (the instruction offset
-// applies to the global and to the LDS address alike).  sbase and lds are wave-uniform.  The loads are asynchronous
-// and counted by vmcnt; their data must not be read before a wait and a barrier.
-__device__ __forceinline__ void load4_to_lds(const void *sbase, unsigned voff, unsigned lds) {
+// One direct global -> LDS load of 64 x 16 bytes (no registers): the wave's lanes read sbase + voff (voff = 16 * lane)
+// and the data land at LDS byte address lds + 16 * lane.  sbase and lds are wave-uniform.  The load is asynchronous
+// and counted by vmcnt; its data must not be read before a wait and a barrier.
+__device__ __forceinline__ void load_to_lds(const void *sbase, unsigned voff, unsigned lds) {
   asm volatile(
       "s_mov_b32 m0, %2\n\t"
       "s_nop 0\n\t"
-      "global_load_lds_dwordx4 %1, %0\n\t"
-      "global_load_lds_dwordx4 %1, %0 offset:1024\n\t"
-      "global_load_lds_dwordx4 %1, %0 offset:2048\n\t"
-      "global_load_lds_dwordx4 %1, %0 offset:3072" ::"s"(sbase),
+      "global_load_lds_dwordx4 %1, %0" ::"s"(sbase),
       "v"(voff), "s"(lds)
       : "memory");
 }
@@ -160,20 +156,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     bet[k] = HAS_LN ? ln_beta[lane * CPL + k] : 0.f;
   }
 
-  static_assert(NDMA % 4 == 0, "a wave fetches its share of a slot four loads at a time");
-  auto fetch_slot = [&](int64_t gs, int c) {  // this wave's share of slot c into buffer gs & 1
-    const u32x4 *src = blob + (int64_t)c * SU + wave * WU;
-    const unsigned dst = (unsigned)(uintptr_t)(wbuf + (gs & 1) * SU + wave * WU);
-#pragma unroll
-    for (int q = 0; q < NDMA; q += 4) load4_to_lds(src + q * 64, lane * 16, dst + q * 1024);
+  static_assert(NDMA == KS, "one direct-to-LDS load per step of the first phase");
+  // piece q of this wave's share of slot c into buffer gs & 1
+  auto fetch_piece = [&](int64_t gs, int c, int q) {
+    const u32x4 *src = blob + (int64_t)c * SU + wave * WU + q * 64;
+    const unsigned dst = (unsigned)(uintptr_t)(wbuf + (gs & 1) * SU + wave * WU + q * 64);
+    load_to_lds(src, lane * 16, dst);
   };
-
-  int64_t gs = 0;  // slots processed so far by this workgroup (buffer parity)
-  if ((int64_t)blockIdx.x < nblocks) fetch_slot(0, 0);
-  for (int64_t mb = blockIdx.x; mb < nblocks; mb += gridDim.x) {
-    // the pair's rows as B operands: lane (i, g) holds row 32m + i, channels 16ks + 8g .. + 7
+  auto load_rows = [&](int64_t mb, u32x4(&ub)[2][KS]) {  // the pair's rows of block mb as B operands
     const int64_t row0 = mb * kRowsPerBlock + rg * 64;
-    u32x4 ub[2][KS];
 #pragma unroll
     for (int m = 0; m < 2; ++m) {
       int64_t r = row0 + 32 * m + i;
@@ -182,6 +173,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) ub[m][ks] = *reinterpret_cast<const u32x4 *>(src + 16 * ks);
     }
+  };
+
+  int64_t gs = 0;  // slots processed so far by this workgroup (buffer parity)
+  if ((int64_t)blockIdx.x < nblocks) {
+#pragma unroll
+    for (int q = 0; q < NDMA; ++q) fetch_piece(0, 0, q);
+  }
+  // lane (i, g) holds row 32m + i, channels 16ks + 8g .. + 7
+  u32x4 ub[2][KS];
+  if ((int64_t)blockIdx.x < nblocks) load_rows(blockIdx.x, ub);
+  for (int64_t mb = blockIdx.x; mb < nblocks; mb += gridDim.x) {
+    const int64_t row0 = mb * kRowsPerBlock + rg * 64;
     f32x16 yacc[2][CTH];  // channels 32 * (CTH * p + ct) + rowmap(r, g)
 #pragma unroll
     for (int m = 0; m < 2; ++m)
@@ -203,8 +206,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
       // slot gs has landed (every wave waits for its own share, then all meet) and the other buffer is free
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       __syncthreads();
-      if (c < NC) fetch_slot(gs + 1, c + 1);
-      else if (mb + gridDim.x < nblocks) fetch_slot(gs + 1, 0);
+      // the next slot is fetched piece by piece behind the steps of phase 1 (its buffer was last read in phase 2 of
+      // the slot before this one)
+      const bool has_next = c < NC || mb + gridDim.x < nblocks;
+      const int c_next = c < NC ? c + 1 : 0;
+      if (has_next) {
+#pragma unroll
+        for (int q = 0; q < NDMA; ++q) fetch_piece(gs + 1, c_next, q);
+      }
       const u32x4 *wb = wbuf + (gs & 1) * SU + lane;
       // this wave's fragments of the slot: W1 of hidden tile p; W2 of its channel half, hidden tile p ("own") first
       const u32x4 *w1f = wb + p * KS * 64;
@@ -244,11 +253,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
       for (int m = 0; m < 2; ++m)
 #pragma unroll
         for (int kk = 0; kk < 2; ++kk) xch[((wave * 2 + m) * 2 + kk) * 64 + lane] = hown[m][kk];
-      __syncthreads();
-#pragma unroll
-      for (int m = 0; m < 2; ++m)
-#pragma unroll
-        for (int kk = 0; kk < 2; ++kk) hpar[m][kk] = xch[(((wave ^ 1) * 2 + m) * 2 + kk) * 64 + lane];
       {
         constexpr int NS2 = 4 * CTH, EV = 16 / NS2 > 0 ? 16 / NS2 : 1;
         static_assert(NS2 * EV == 16, "phase 2 must cover 16 evaluations");
@@ -262,6 +266,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         static_for<AHEAD>([&](auto q) { fr[decltype(q)::value] = frag2(q); });
         static_for<NS2>([&](auto st) {
           constexpr int t = decltype(st)::value, k4 = t / CTH, ct = t % CTH, kk = k4 & 1;
+          if constexpr (t == 2 * CTH) {  // the own tile is used up: now the partner's (written before phase 2)
+            __syncthreads();
+#pragma unroll
+            for (int m = 0; m < 2; ++m)
+#pragma unroll
+              for (int k = 0; k < 2; ++k) hpar[m][k] = xch[(((wave ^ 1) * 2 + m) * 2 + k) * 64 + lane];
+          }
           if constexpr (t + AHEAD < NS2) fr[(t + AHEAD) % RING] = frag2(std::integral_constant<int, t + AHEAD>{});
           const u32x4 a = fr[t % RING];
           yacc[0][ct] = mma(a, k4 < 2 ? hown[0][kk] : hpar[0][kk], yacc[0][ct]);
@@ -284,6 +295,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 
     // ---- epilogue: the buffer of the last slot is idle once every wave is past its last MFMA ----
     __syncthreads();
+    // the rows of this workgroup's next block travel while the epilogue runs (past the end: this block again)
+    load_rows(mb + gridDim.x < nblocks ? mb + gridDim.x : mb, ub);
     uint32_t *stg = reinterpret_cast<uint32_t *>(wbuf + ((gs - 1) & 1) * SU) + rg * 64 * (C / 2);  // [64 rows][C/2 words]
     // y^T + b2 -> bf16 -> staged rows; granule gr (4 channels) of row rw sits at gr ^ ((2 rw) % G4)
 #pragma unroll
@@ -303,7 +316,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         }
     __syncthreads();  // both waves of a pair have staged their channel halves
     // wave p finishes rows 32p .. 32p+31 of the pair, 8 at a time: lane holds CPL consecutive channels
-    constexpr int RB = 8;
+    constexpr int RB = 32;
 #pragma unroll 1
     for (int rb = 0; rb < 32; rb += RB) {
       uint32_t rsd[RB][CPL / 2];

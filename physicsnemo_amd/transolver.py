@@ -1,8 +1,10 @@
 """Host-side mirror of the caller of the hot path: TransolverBlock and Transolver
 (physicsnemo/models/transolver/transolver.py:137-309 and :447-736, use_te=False, time_input=False, plus=False).
 
-The PhysicsAttention layer, its residual add and the LayerNorm that follows it run in the HIP library; the
-remaining glue (LayerNorm before the layer, the two MLPs, the output head) uses PyTorch-ROCm tensor ops.
+The PhysicsAttention layer, its residual add and the LayerNorm that follows it run in the HIP library, and so does
+the block MLP with its residual add and the LayerNorm the next block starts with whenever the fused kernel serves
+the shape (bf16, hidden 128 / 256, GELU); the remaining glue (preprocess MLP, the first LayerNorm, the output
+Linear, and every MLP the kernel does not serve) uses PyTorch-ROCm tensor ops.
 Module names, registration order and state_dict keys match the reference so its checkpoints load unchanged,
 including the legacy ``linear_pre`` / ``linear_post`` MLP keys (:92-97).
 """
@@ -12,6 +14,7 @@ import numpy as np
 import torch
 import torch.nn as nn
 
+from . import functional as PF
 from .physics_attention import PhysicsAttentionIrregularMesh, PhysicsAttentionStructuredMesh2D
 
 __all__ = ["Mlp", "TransolverBlock", "Transolver"]
@@ -70,12 +73,51 @@ class TransolverBlock(nn.Module):
         self.ln_mlp1 = nn.Sequential(nn.LayerNorm(hidden_dim), Mlp(hidden_dim, hidden_dim * mlp_ratio, hidden_dim, act))
         if last_layer:
             self.ln_mlp2 = nn.Sequential(nn.LayerNorm(hidden_dim), nn.Linear(hidden_dim, out_dim))
+        self._mlp_cache: dict = {}
+
+    # ---------------------------------------------------------------- fused MLP (pa_mlp_forward)
+    def _mlp_kernel_params(self, device):
+        """bf16 weights / fp32 biases of ln_mlp1's Mlp for the fused kernel; cached until a parameter changes."""
+        lin1, lin2 = self.ln_mlp1[1].layers[0], self.ln_mlp1[1].layers[2]
+        named = (lin1.weight, lin1.bias, lin2.weight, lin2.bias)
+        stamp = (device,) + tuple((t.data_ptr(), t._version, t.dtype) for t in named)
+        if self._mlp_cache.get("stamp") != stamp:
+            with torch.no_grad():
+                params = (lin1.weight.detach().to(device=device, dtype=torch.bfloat16).contiguous().clone(),
+                          lin1.bias.detach().to(device=device, dtype=torch.float32).contiguous().clone(),
+                          lin2.weight.detach().to(device=device, dtype=torch.bfloat16).contiguous().clone(),
+                          lin2.bias.detach().to(device=device, dtype=torch.float32).contiguous().clone())
+            self._mlp_cache = {"stamp": stamp, "params": params}
+        return self._mlp_cache["params"]
+
+    def _mlp_kernel_serves(self, normed: torch.Tensor) -> bool:
+        mlp = self.ln_mlp1[1]
+        if not (normed.is_cuda and normed.dtype == torch.bfloat16 and isinstance(mlp.layers[1], nn.GELU)
+                and mlp.layers[1].approximate == "none"):
+            return False
+        hidden = mlp.layers[0].out_features
+        return PF.mlp_supported(normed.dtype, normed.numel() // normed.shape[-1], normed.shape[-1], hidden)
+
+    def forward_chain(self, fx: torch.Tensor, normed_in: torch.Tensor | None, next_ln: nn.LayerNorm | None):
+        """One block inside a chain of blocks: takes LayerNorm_1(fx) if the previous stage already produced it and
+        returns (fx_out, next_ln(fx_out) or None).  Same arithmetic as `forward` (reference :300-303)."""
+        x_in = normed_in if normed_in is not None else self.ln_1(fx)
+        # fx1 = Attn(ln_1(fx)) + fx and LayerNorm(fx1) come out of one fused library call (reference :300, :303)
+        fx1, normed = self.Attn.forward_block(x_in, fx, self.ln_mlp1[0])
+        if self._mlp_kernel_serves(normed):
+            w1, b1, w2, b2 = self._mlp_kernel_params(normed.device)
+            if next_ln is None:
+                return PF.mlp_forward(normed, w1, b1, w2, b2, residual=fx1), None
+            return PF.mlp_forward(normed, w1, b1, w2, b2, residual=fx1,
+                                  ln_weight=next_ln.weight.detach().float().contiguous(),
+                                  ln_bias=next_ln.bias.detach().float().contiguous(), ln_eps=next_ln.eps)
+        return self.ln_mlp1[1](normed) + fx1, None
 
     def forward(self, fx: torch.Tensor) -> torch.Tensor:
-        # fx1 = Attn(ln_1(fx)) + fx and LayerNorm(fx1) come out of one fused library call (reference :300, :303)
-        fx1, normed = self.Attn.forward_block(self.ln_1(fx), fx, self.ln_mlp1[0])
-        fx2 = self.ln_mlp1[1](normed) + fx1
-        return self.ln_mlp2(fx2) if self.last_layer else fx2
+        if self.last_layer:
+            fx2, normed = self.forward_chain(fx, None, self.ln_mlp2[0])
+            return self.ln_mlp2[1](normed) if normed is not None else self.ln_mlp2(fx2)
+        return self.forward_chain(fx, None, None)[0]
 
 
 class Transolver(nn.Module):
@@ -168,8 +210,14 @@ class Transolver(nn.Module):
                 embedding = embedding.reshape(embedding.shape[0], -1, embedding.shape[-1])
         fx = torch.cat((embedding.to(fx.dtype), fx), -1)  # embedding first, then the functional input (:716)
         fx = self.preprocess(fx)
-        for block in self.blocks:
-            fx = block(fx)
+        # each block hands the next one its residual stream and, when the fused MLP kernel ran, LayerNorm_1 of it
+        normed = None
+        for k, block in enumerate(self.blocks):
+            if block.last_layer:
+                fx, normed = block.forward_chain(fx, normed, block.ln_mlp2[0])
+                fx = block.ln_mlp2[1](normed) if normed is not None else block.ln_mlp2(fx)
+            else:
+                fx, normed = block.forward_chain(fx, normed, self.blocks[k + 1].ln_1)
         if unflatten_output:
             fx = fx.reshape(fx.shape[0], *self.structured_shape, -1)
         return fx
