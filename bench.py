@@ -114,11 +114,34 @@ def cpu_baseline(state_dict, x_cpu_f32, C, H, S, target_seconds):
     }
 
 
+def time_block_mlp(rows, C, hidden, reps=10):
+    """The fused block MLP kernel alone (LN'd rows -> Linear -> GELU -> Linear -> + residual -> LayerNorm), bf16."""
+    import torch
+
+    from physicsnemo_amd import functional as PF
+
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(4321)
+    u = torch.randn(1, rows, C, generator=g).to(dev).bfloat16()
+    res = torch.randn(1, rows, C, generator=g).to(dev).bfloat16()
+    w1 = (torch.randn(hidden, C, generator=g) * C ** -0.5).to(dev).bfloat16()
+    w2 = (torch.randn(C, hidden, generator=g) * hidden ** -0.5).to(dev).bfloat16()
+    b1, b2 = torch.zeros(hidden, device=dev), torch.zeros(C, device=dev)
+    gam, bet = torch.ones(C, device=dev), torch.zeros(C, device=dev)
+    ms = time_kernel(lambda: PF.mlp_forward(u, w1, b1, w2, b2, residual=res, ln_weight=gam, ln_bias=bet), reps)
+    flops = 4.0 * C * hidden * rows
+    return {"rows": rows, "hidden": C, "mlp_hidden": hidden, "ms": round(ms, 4),
+            "mfma_tflops": round(flops / (ms * 1e-3) / 1e12, 1),
+            "mfma_frac": round(flops / (ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TF, 4),
+            "algorithmic_bytes": 4 * rows * C * 2,  # read rows and residual, write the sum and its LayerNorm
+            "hbm_frac": round(4 * rows * C * 2 / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+
+
 def time_full_model(name, B, N, functional_dim, embedding_dim, slice_num, n_layers, steps=5, warmup=2):
     """Forward of a whole Transolver (bf16 autocast, random-init weights, synthetic N(0,1) inputs) -> Mpoints/s.
 
-    The PhysicsAttention layers, their residual adds and the LayerNorms that follow run in the HIP library; the
-    remaining glue (first LayerNorm, MLPs, output head) is PyTorch-ROCm.
+    The PhysicsAttention layers, the block MLPs, their residual adds and the LayerNorms between them run in the HIP
+    library; the remaining glue (preprocess MLP, first LayerNorm, output Linear) is PyTorch-ROCm.
     """
     import torch
 
@@ -251,6 +274,7 @@ def main():
         "roofline": roofline, "kernels": kernels,
     }
     if not args.no_models:
+        out["block_mlp"] = time_block_mlp(1 << 20, 256, 1024)
         out["full_model"] = [
             time_full_model("cfg2: Transolver irregular 2D, 8 layers", 8, 32768, 3, 2, 64, 8),
             time_full_model("cfg4: Transolver 3D surface cloud, 8 layers", 1, 1000000, 1, 6, 32, 8),

@@ -110,8 +110,9 @@ __device__ __forceinline__ u32x4 pack8(const float (&v)[8]) {
   return __builtin_bit_cast(u32x4, o);
 }
 
-// sum over the 64 lanes, returned in every lane: DPP steps inside each row of 16, then the four row totals
-__device__ __forceinline__ float wave_sum_dpp(float v) {
+// sum over the 32 lanes of this lane's half of the wave, returned in every lane of the half: DPP steps inside each
+// row of 16 lanes, then v_permlane16_swap pairs the two rows of the half
+__device__ __forceinline__ float half_wave_sum(float v) {
   auto step = [](float x, auto ctrl) {
     constexpr int c = decltype(ctrl)::value;
     return x + __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(x), c, 0xf, 0xf, true));
@@ -120,8 +121,8 @@ __device__ __forceinline__ float wave_sum_dpp(float v) {
   v = step(v, std::integral_constant<int, 0x4E>{});   // quad_perm [2,3,0,1]
   v = step(v, std::integral_constant<int, 0x141>{});  // row_half_mirror
   v = step(v, std::integral_constant<int, 0x140>{});  // row_mirror
-  auto row_total = [&](int l) { return __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(v), l)); };
-  return (row_total(0) + row_total(16)) + (row_total(32) + row_total(48));
+  const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
 template <int C, int TAIL>
@@ -134,7 +135,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   constexpr int KS = C / 16, CT = C / 32, CTH = CT / 2, NF1 = 2 * KS, SU = slot_units(C);
   constexpr int WU = SU / 4;     // units of a slot fetched by each wave
   constexpr int NDMA = WU / 64;  // direct-to-LDS loads per wave and slot
-  constexpr int CPL = C / 64;    // consecutive channels per lane in the row-major epilogue
+  constexpr int CPH = C / 32;    // consecutive channels per lane in the row-major epilogue (half a wave per row)
+  constexpr int WPH = CPH / 2;   // 32-bit words per lane and row
   constexpr int G4 = C / 4;      // 8-byte granules (4 channels) per staged row
   static_assert(SU * 16 == 128 * C * 2, "a slot buffer must hold the 128 bf16 rows of a block in the epilogue");
   extern __shared__ u32x4 smem[];
@@ -149,11 +151,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 
   for (int k = tid; k < F; k += 256) b1s[k] = b1[k];
   for (int k = tid; k < C; k += 256) b2s[k] = b2[k];
-  float gam[CPL], bet[CPL];
+  const int half = lane >> 5;  // in the epilogue each half of the wave finishes one row per step
+  float gam[CPH], bet[CPH];
 #pragma unroll
-  for (int k = 0; k < CPL; ++k) {
-    gam[k] = HAS_LN ? ln_gamma[lane * CPL + k] : 1.f;
-    bet[k] = HAS_LN ? ln_beta[lane * CPL + k] : 0.f;
+  for (int k = 0; k < CPH; ++k) {
+    gam[k] = HAS_LN ? ln_gamma[i * CPH + k] : 1.f;
+    bet[k] = HAS_LN ? ln_beta[i * CPH + k] : 0.f;
   }
 
   static_assert(NDMA == KS, "one direct-to-LDS load per step of the first phase");
@@ -315,67 +318,61 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
           *reinterpret_cast<u32x2 *>(stg + rw * (C / 2) + gr * 2) = pk;
         }
     __syncthreads();  // both waves of a pair have staged their channel halves
-    // wave p finishes rows 32p .. 32p+31 of the pair, 8 at a time: lane holds CPL consecutive channels
-    constexpr int RB = 32;
-#pragma unroll 1
-    for (int rb = 0; rb < 32; rb += RB) {
-      uint32_t rsd[RB][CPL / 2];
-      if constexpr (HAS_RES) {
+    // wave p finishes rows 32p .. 32p+31 of the pair, two per step: lanes 0-31 one row, lanes 32-63 the next, CPH
+    // consecutive channels per lane (16-byte accesses for C = 256)
+    typedef uint32_t rowv __attribute__((ext_vector_type(WPH)));
+    constexpr int NRS = 16;
+    rowv rsd[NRS];
+    if constexpr (HAS_RES) {
 #pragma unroll
-        for (int rr = 0; rr < RB; ++rr) {
-          int64_t r = row0 + 32 * p + rb + rr;
-          if (r >= M) r = M - 1;
-#pragma unroll
-          for (int w = 0; w < CPL / 2; ++w)
-            rsd[rr][w] = *reinterpret_cast<const uint32_t *>(residual + r * C + lane * CPL + 2 * w);
-        }
+      for (int rr = 0; rr < NRS; ++rr) {
+        int64_t r = row0 + 32 * p + 2 * rr + half;
+        if (r >= M) r = M - 1;
+        rsd[rr] = *reinterpret_cast<const rowv *>(residual + r * C + i * CPH);
       }
+    }
 #pragma unroll
-      for (int rr = 0; rr < RB; ++rr) {
-        const int rw = 32 * p + rb + rr;
-        const int64_t r = row0 + rw;
-        const bool ok = r < M;
-        float v[CPL];
-        uint32_t ob[CPL / 2];
+    for (int rr = 0; rr < NRS; ++rr) {
+      const int rw = 32 * p + 2 * rr + half;
+      const int64_t r = row0 + rw;
+      const bool ok = r < M;
+      // granules (4 channels) i*CPH/4 .. of row rw; the swizzle flips an even number, so they stay adjacent
+      const rowv sv = *reinterpret_cast<const rowv *>(stg + rw * (C / 2) + (((i * CPH / 4) ^ ((2 * rw) & (G4 - 1))) << 1));
+      float v[CPH];
+      rowv ob;
 #pragma unroll
-        for (int w = 0; w < CPL / 2; ++w) {
-          const int word = lane * (CPL / 2) + w;  // word of the row; granule = word / 2
-          const uint32_t sv = stg[rw * (C / 2) + ((((word >> 1) ^ ((2 * rw) & (G4 - 1))) << 1) | (word & 1))];
-          float t0 = bf16_bits_to_f32((uint16_t)(sv & 0xffffu)), t1 = bf16_bits_to_f32((uint16_t)(sv >> 16));
-          if constexpr (HAS_RES) {  // the MLP output is a bf16 tensor; the sum is rounded again
-            t0 += bf16_bits_to_f32((uint16_t)(rsd[rr][w] & 0xffffu));
-            t1 += bf16_bits_to_f32((uint16_t)(rsd[rr][w] >> 16));
-          }
-          const uint16_t o0 = to_bf16_bits(t0), o1 = to_bf16_bits(t1);
-          v[2 * w] = bf16_bits_to_f32(o0);
-          v[2 * w + 1] = bf16_bits_to_f32(o1);
-          ob[w] = (uint32_t)o0 | ((uint32_t)o1 << 16);
+      for (int w = 0; w < WPH; ++w) {
+        float t0 = bf16_bits_to_f32((uint16_t)(sv[w] & 0xffffu)), t1 = bf16_bits_to_f32((uint16_t)(sv[w] >> 16));
+        if constexpr (HAS_RES) {  // the MLP output is a bf16 tensor; the sum is rounded again
+          t0 += bf16_bits_to_f32((uint16_t)(rsd[rr][w] & 0xffffu));
+          t1 += bf16_bits_to_f32((uint16_t)(rsd[rr][w] >> 16));
         }
-        if (ok) {
+        const uint16_t o0 = to_bf16_bits(t0), o1 = to_bf16_bits(t1);
+        v[2 * w] = bf16_bits_to_f32(o0);
+        v[2 * w + 1] = bf16_bits_to_f32(o1);
+        ob[w] = (uint32_t)o0 | ((uint32_t)o1 << 16);
+      }
+      if (ok) *reinterpret_cast<rowv *>(y + r * C + i * CPH) = ob;
+      if constexpr (HAS_LN) {
+        float s1 = 0.f;
 #pragma unroll
-          for (int w = 0; w < CPL / 2; ++w) *reinterpret_cast<uint32_t *>(y + r * C + lane * CPL + 2 * w) = ob[w];
+        for (int k = 0; k < CPH; ++k) s1 += v[k];
+        const float mean = half_wave_sum(s1) * (1.f / C);
+        float s2 = 0.f;
+#pragma unroll
+        for (int k = 0; k < CPH; ++k) {
+          const float dl = v[k] - mean;
+          s2 = fmaf(dl, dl, s2);
         }
-        if constexpr (HAS_LN) {
-          float s1 = 0.f;
+        const float rstd = rsqrtf(half_wave_sum(s2) * (1.f / C) + ln_eps);
+        rowv lb;
 #pragma unroll
-          for (int k = 0; k < CPL; ++k) s1 += v[k];
-          const float mean = wave_sum_dpp(s1) * (1.f / C);
-          float s2 = 0.f;
-#pragma unroll
-          for (int k = 0; k < CPL; ++k) {
-            const float dl = v[k] - mean;
-            s2 = fmaf(dl, dl, s2);
-          }
-          const float rstd = rsqrtf(wave_sum_dpp(s2) * (1.f / C) + ln_eps);
-          if (ok) {
-#pragma unroll
-            for (int w = 0; w < CPL / 2; ++w) {
-              const uint16_t l0 = to_bf16_bits((v[2 * w] - mean) * rstd * gam[2 * w] + bet[2 * w]);
-              const uint16_t l1 = to_bf16_bits((v[2 * w + 1] - mean) * rstd * gam[2 * w + 1] + bet[2 * w + 1]);
-              *reinterpret_cast<uint32_t *>(ln_out + r * C + lane * CPL + 2 * w) = (uint32_t)l0 | ((uint32_t)l1 << 16);
-            }
-          }
+        for (int w = 0; w < WPH; ++w) {
+          const uint16_t l0 = to_bf16_bits((v[2 * w] - mean) * rstd * gam[2 * w] + bet[2 * w]);
+          const uint16_t l1 = to_bf16_bits((v[2 * w + 1] - mean) * rstd * gam[2 * w + 1] + bet[2 * w + 1]);
+          lb[w] = (uint32_t)l0 | ((uint32_t)l1 << 16);
         }
+        if (ok) *reinterpret_cast<rowv *>(ln_out + r * C + i * CPH) = lb;
       }
     }
   }
