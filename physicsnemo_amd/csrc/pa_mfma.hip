@@ -146,7 +146,8 @@ __global__ __launch_bounds__((C / 32) * 64) void project_softmax_kernel(const u3
   float *fvec = reinterpret_cast<float *>(accs + (FUSED ? H * ACC_UNITS : 0));
   float *bias_x = fvec, *bias_f = fvec + C, *bias_s = fvec + 2 * C, *tscale = fvec + 3 * C + ST * 32;
   const BlobPlan bp = blob_plan(C, S);
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, i = lane & 31, g = lane >> 5;
+  const int tid = threadIdx.x, lane = tid & 63, i = lane & 31, g = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: addresses derived from it stay scalar
   const int h = wave;
   const int b = blockIdx.y;
 
@@ -367,7 +368,8 @@ __global__ __launch_bounds__(256) void slice_reduce_kernel(const u32x4 *__restri
                                                            int tiles_per_group) {
   constexpr int ST = (S + 31) / 32, NCH = S / 16, D = 32, D1 = D + 1;
   extern __shared__ float red[];  // [4 waves][ST][17][64]
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, i = lane & 31, g = lane >> 5;
+  const int tid = threadIdx.x, lane = tid & 63, i = lane & 31, g = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: addresses derived from it stay scalar
   const int bh = blockIdx.y, b = bh / H, h = bh - b * H;
   u32x4 sel[2];
 #pragma unroll
@@ -488,7 +490,8 @@ __global__ __launch_bounds__(C * 2) void deslice_project_kernel(const u32x4 *__r
   __shared__ u32x4 tps[H * NCH * 64];
   __shared__ float ys[32 * YS];
   const BlobPlan bp = blob_plan(C, S);
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, i = lane & 31, g = lane >> 5;
+  const int tid = threadIdx.x, lane = tid & 63, i = lane & 31, g = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: addresses derived from it stay scalar
 
   u32x4 wout[H][2];
 #pragma unroll
