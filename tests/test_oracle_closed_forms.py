@@ -253,3 +253,33 @@ def test_state_dict_keys_and_shapes_match_reference_contract():
         "temperature", "in_project_slice.weight", "in_project_slice.bias", "qkv_project.weight",
         "out_linear.weight", "out_linear.bias", "in_project_x.weight", "in_project_x.bias",
         "in_project_fx.weight", "in_project_fx.bias"]
+
+
+def test_mlp_kernel_gelu_constants_against_exact_erf():
+    """The fused MLP kernel evaluates GELU as x / (1 + exp2(x * P(min(x^2, 81)))) with the three constants found in
+    physicsnemo_amd/csrc/pa_mlp.hip.  Evaluate that form (float32, constants parsed from the source) against the
+    exact erf form on a dense grid: a wrong or mistyped constant moves the error far above the bound."""
+    import math
+    import os
+    import re
+
+    import numpy as np
+
+    src = open(os.path.join(os.path.dirname(__file__), "..", "physicsnemo_amd", "csrc", "pa_mlp.hip")).read()
+    body = src[src.index("__device__ __forceinline__ float gelu(float x)"):]
+    body = body[:body.index("}")]
+    consts = [float(c) for c in re.findall(r"(-?\d\.\d+e-?\d+)f \* -2\.f \* kLog2e", body)]
+    assert len(consts) == 3, consts
+    c2, c1, c0 = consts  # order of appearance: x^4, x^2, constant term
+    clamp = float(re.search(r"fminf\(x \* x, (\d+)\.f\)", body).group(1))
+    x = np.linspace(-30, 30, 1200001, dtype=np.float32)
+    x2 = np.minimum(x * x, np.float32(clamp))
+    k = np.float32(-2.0 * 1.4426950408889634)
+    p = (np.float32(c2) * k * x2 + np.float32(c1) * k) * x2 + np.float32(c0) * k
+    with np.errstate(over="ignore"):
+        got = x / (np.float32(1) + np.exp2(x * p, dtype=np.float32))
+    want = np.array([0.5 * v * (1.0 + math.erf(v / math.sqrt(2.0))) for v in x[::40].astype(np.float64)])
+    err = np.abs(got[::40].astype(np.float64) - want)
+    assert err.max() < 3e-5, err.max()
+    # saturation ends: exactly x for large x, exactly 0 (up to sign) for large negative x
+    assert got[-1] == x[-1] and abs(got[0]) == 0.0
