@@ -169,6 +169,35 @@ def time_full_model(name, B, N, functional_dim, embedding_dim, slice_num, n_laye
             "ms_per_forward": round(dt * 1e3, 3), "mpoints_per_s": round(B * N / dt / 1e6, 2)}
 
 
+def time_structured_model(steps=5, warmup=2):
+    """cfg1: Transolver on a structured 85 x 85 grid (Conv2d k = 3 projections), fp32, 4 layers, hidden 128, 8 heads,
+    32 slices, mlp_ratio 1, batch 4 -> Mpoints/s.  Served by the general (fp32) kernels."""
+    import torch
+
+    import physicsnemo_amd as pn
+
+    torch.manual_seed(0)
+    model = pn.Transolver(functional_dim=1, embedding_dim=2, out_dim=1, n_layers=4, n_hidden=128, n_head=8, mlp_ratio=1,
+                          slice_num=32, structured_shape=(85, 85), unified_pos=False, use_te=False).eval().cuda()
+    g = torch.Generator().manual_seed(1234)
+    lin = torch.linspace(0, 1, 85)
+    pos = torch.stack(torch.meshgrid(lin, lin, indexing="ij"), -1).reshape(1, 7225, 2).repeat(4, 1, 1).cuda()
+    fx = torch.randn(4, 7225, 1, generator=g).cuda()
+    with torch.no_grad():
+        for _ in range(warmup):
+            out = model(fx, pos)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            out = model(fx, pos)
+        torch.cuda.synchronize()
+        dt = (time.perf_counter() - t0) / steps
+    assert torch.isfinite(out).all()
+    return {"workload": "cfg1: Transolver structured 2D 85x85 (conv k=3), fp32, 4 layers", "batch": 4, "points": 7225,
+            "layers": 4, "slice_num": 32, "ms_per_forward": round(dt * 1e3, 3),
+            "mpoints_per_s": round(4 * 7225 / dt / 1e6, 2)}
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -276,6 +305,7 @@ def main():
     if not args.no_models:
         out["block_mlp"] = time_block_mlp(1 << 20, 256, 1024)
         out["full_model"] = [
+            time_structured_model(),
             time_full_model("cfg2: Transolver irregular 2D, 8 layers", 8, 32768, 3, 2, 64, 8),
             time_full_model("cfg4: Transolver 3D surface cloud, 8 layers", 1, 1000000, 1, 6, 32, 8),
         ]

@@ -206,8 +206,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     }
 
     for (int c = 0; c <= NC; ++c, ++gs) {
-      // slot gs has landed (every wave waits for its own share, then all meet) and the other buffer is free
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      // slot gs has landed (every wave waits for its own share, then all meet) and the other buffer is free.  The
+      // first slot of a later block was waited for before the epilogue of the block before it, whose stores may
+      // still be in flight here.
+      if (c > 0 || gs == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       __syncthreads();
       // the next slot is fetched piece by piece behind the steps of phase 1 (its buffer was last read in phase 2 of
       // the slot before this one)
@@ -297,6 +299,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     }
 
     // ---- epilogue: the buffer of the last slot is idle once every wave is past its last MFMA ----
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's share of the next block's first slot has landed
     __syncthreads();
     // the rows of this workgroup's next block travel while the epilogue runs (past the end: this block again)
     load_rows(mb + gridDim.x < nblocks ? mb + gridDim.x : mb, ub);
