@@ -211,14 +211,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
       // still be in flight here.
       if (c > 0 || gs == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       __syncthreads();
-      // the next slot is fetched piece by piece behind the steps of phase 1 (its buffer was last read in phase 2 of
-      // the slot before this one)
       const bool has_next = c < NC || mb + gridDim.x < nblocks;
       const int c_next = c < NC ? c + 1 : 0;
-      if (has_next) {
-#pragma unroll
-        for (int q = 0; q < NDMA; ++q) fetch_piece(gs + 1, c_next, q);
-      }
       const u32x4 *wb = wbuf + (gs & 1) * SU + lane;
       // this wave's fragments of the slot: W1 of hidden tile p; W2 of its channel half, hidden tile p ("own") first
       const u32x4 *w1f = wb + p * KS * 64;
@@ -239,6 +233,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         static_assert(KS * EV == 16 || KS == 16, "phase 1 must cover 16 evaluations");
         u32x4 fr[RING];
         static_for<AHEAD>([&](auto q) { fr[decltype(q)::value] = w1f[decltype(q)::value * 64]; });
+        // the first fragments and the bias are on their way: now the next slot's fetch, whose issue keeps the wave
+        // busy for a while (its buffer was last read in phase 2 of the slot before this one)
+        if (has_next) {
+#pragma unroll
+          for (int q = 0; q < NDMA; ++q) fetch_piece(gs + 1, c_next, q);
+        }
         static_for<KS>([&](auto st) {
           constexpr int step = decltype(st)::value;
           if constexpr (step + AHEAD < KS) fr[(step + AHEAD) % RING] = w1f[(step + AHEAD) * 64];
@@ -271,7 +271,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         static_for<AHEAD>([&](auto q) { fr[decltype(q)::value] = frag2(q); });
         static_for<NS2>([&](auto st) {
           constexpr int t = decltype(st)::value, k4 = t / CTH, ct = t % CTH, kk = k4 & 1;
-          if constexpr (t == 2 * CTH) {  // the own tile is used up: now the partner's (written before phase 2)
+          if constexpr (t == 2 * CTH - 2) {  // two steps before the partner's tile (written before phase 2) is needed
             __syncthreads();
 #pragma unroll
             for (int m = 0; m < 2; ++m)
