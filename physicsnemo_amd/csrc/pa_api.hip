@@ -308,10 +308,7 @@ int pa_mfma_combine_attention(const pa_shape *shape, const pa_params *p, const f
   if (!p || !p->qkv_project_weight || !partials || !out_slice_token || !tokp) return PA_ERR_NULL;
   if (!aligned16(partials) || !aligned16(tokp)) return PA_ERR_ALIGN;
   hipStream_t st = static_cast<hipStream_t>(stream);
-  rc = pa::general::combine_attention(*shape, *p, partials, groups, slice_token, slice_norm,
-                                      out_slice_token, st);
-  if (rc) return rc;
-  return pa::mfma::pack_tokens(*shape, out_slice_token, tokp, st);
+  return pa::mfma::combine_attention(*shape, *p, partials, groups, slice_token, slice_norm, out_slice_token, tokp, st);
 }
 
 int pa_mfma_deslice_project(const pa_shape *shape, const void *blob, const void *w_pack, const void *tokp, void *y,
@@ -396,8 +393,7 @@ int pa_layer_forward(int dtype, const pa_shape *shape, const pa_params *p, const
       if ((rc = pa::mfma::project_softmax(s, blob, x, fxp, wp, nullptr, compute_units(), st))) return rc;
       if ((rc = pa::mfma::slice_reduce(s, wp, fxp, partials, st))) return rc;
     }
-    if ((rc = pa::general::combine_attention(s, *p, partials, mp.G, tok, norm, tok_out, st))) return rc;
-    if ((rc = pa::mfma::pack_tokens(s, tok_out, tokp, st))) return rc;
+    if ((rc = pa::mfma::combine_attention(s, *p, partials, mp.G, tok, norm, tok_out, tokp, st))) return rc;
     return pa::mfma::deslice_project(s, blob, wp, tokp, y, tail_active(tail) ? tail : nullptr, compute_units(), st);
   }
   const GeneralPlan plan = plan_general(dtype, s);

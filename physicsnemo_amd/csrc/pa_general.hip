@@ -574,6 +574,20 @@ static int slice_partial_t(const pa_shape &s, const void *w, const void *fx_mid,
 
 // `partials` holds G partial sums followed by one spare slot (index G) that receives their fixed-order total.
 // G == 0: `partials` holds finished slice tokens (attention only).
+// Fixed-order total of the G partial sums [G][B][H][S][D+1]; the total goes to slot G of the same buffer.  Returns
+// where the totals are (the partials themselves when G == 1).
+int combine_partials(const pa_shape &s, const float *partials, int64_t G, const float **combined, hipStream_t st) {
+  const int64_t stride = s.B * s.H * s.S * (s.D + 1);
+  *combined = partials;
+  if (G <= 1) return PA_OK;
+  float *total = const_cast<float *>(partials) + G * stride;
+  const int n_out = (int)(s.S * (s.D + 1));
+  hipLaunchKernelGGL(combine_partials_kernel, dim3((unsigned)((n_out + 63) / 64), (unsigned)(s.B * s.H)), dim3(256), 0, st,
+                     partials, (int)G, stride, total, n_out);
+  *combined = total;
+  return launch_status();
+}
+
 int combine_attention(const pa_shape &s, const pa_params &p, const float *partials, int64_t G, float *slice_token,
                       float *slice_norm, float *out_token, hipStream_t st) {
   size_t lds = combine_attn_lds_bytes(s);
@@ -584,17 +598,8 @@ int combine_attention(const pa_shape &s, const pa_params &p, const float *partia
   if (rc) return rc;
   const int64_t stride = s.B * s.H * s.S * (s.D + 1);
   const float *src = partials;
-  int g_attn = (int)G;
-  if (G > 1) {
-    float *combined = const_cast<float *>(partials) + G * stride;
-    const int n_out = (int)(s.S * (s.D + 1));
-    hipLaunchKernelGGL(combine_partials_kernel, dim3((unsigned)((n_out + 63) / 64), (unsigned)(s.B * s.H)), dim3(256), 0,
-                       st, partials, (int)G, stride, combined, n_out);
-    if ((rc = launch_status())) return rc;
-    src = combined;
-    g_attn = 1;
-  }
-  hipLaunchKernelGGL(slice_combine_attn_kernel, dim3((unsigned)(s.B * s.H)), dim3(kAttnThreads), lds, st, src, g_attn, stride,
+  if ((rc = combine_partials(s, partials, G, &src, st))) return rc;
+  hipLaunchKernelGGL(slice_combine_attn_kernel, dim3((unsigned)(s.B * s.H)), dim3(kAttnThreads), lds, st, src, G == 0 ? 0 : 1, stride,
                      p.qkv_project_weight, slice_token, slice_norm, out_token, (int)s.D, (int)s.S, stage_w);
   return launch_status();
 }

@@ -20,6 +20,7 @@ int slice_softmax(int dtype, const pa_shape &s, const pa_params &p, const void *
 int64_t partial_count(const pa_shape &s);
 size_t combine_attn_lds_bytes(const pa_shape &s);
 int slice_partial(int dtype, const pa_shape &s, const void *w, const void *fx_mid, float *partials, hipStream_t st);
+int combine_partials(const pa_shape &s, const float *partials, int64_t G, const float **combined, hipStream_t st);
 int combine_attention(const pa_shape &s, const pa_params &p, const float *partials, int64_t G, float *slice_token,
                       float *slice_norm, float *out_token, hipStream_t st);
 int deslice(int dtype, const pa_shape &s, const void *w, const float *out_token, void *out_x, hipStream_t st);
@@ -41,6 +42,8 @@ int project_softmax(const pa_shape &s, const void *blob, const void *x, void *fx
                     int num_cu, hipStream_t st);
 int slice_reduce(const pa_shape &s, const void *w_pack, const void *fx_pack, float *partials, hipStream_t st);
 int pack_tokens(const pa_shape &s, const float *tok_out, void *tokp, hipStream_t st);
+int combine_attention(const pa_shape &s, const pa_params &p, const float *partials, int64_t G, float *slice_token,
+                      float *slice_norm, float *out_token, void *tokp, hipStream_t st);
 int deslice_project(const pa_shape &s, const void *blob, const void *w_pack, const void *tokp, void *y,
                     const pa_block_tail *tail, int num_cu, hipStream_t st);
 }  // namespace mfma

@@ -459,6 +459,120 @@ __global__ __launch_bounds__(256) void pack_tokens_kernel(const float *__restric
 }
 
 // ------------------------------------------------------------------------------------------------
+// Kernel (c): normalisation of the combined sums and the per-head slice self-attention, fp32 MFMA
+// (v_mfma_f32_32x32x2_f32: A lane (i, g) holds A[i][k = g], B lane (i, g) holds B[k = g][i], C/D as above).
+// One workgroup per (b, h), one wave per tile of 32 slices; lane (i, g) of wave w owns slice s = 32w + i.
+//   tok[s][:]  = num[s][:] / (cnt[s] + 1e-2)                                    -> slice_token, slice_norm
+//   q^T, k^T, v^T (32 e x 32 s) = Wq|k|v (A) . tok^T (B: lane <-> s, k <-> d)    registers <-> e = rowmap(r, g)
+//   k, v -> LDS; scores^T (keys x queries) = k (A, from LDS) . q^T: register r of q^T is directly the B operand of
+//   the step whose reduction pair is d = rowmap(r, 0 / 1)
+//   softmax over the keys: in-lane over registers and key tiles + one exchange with lane ^ 32
+//   out^T (32 d x 32 s) = v^T (A, from LDS) . P^T: register r of P^T is directly the B operand of the step whose
+//   key pair is rowmap(r, 0 / 1)                                                -> out_token (fp32), tokp (bf16,
+//   A-operand order of the deslice product: tokp[b][h][cq][lane'][j] = tok'[16cq + kperm(0, g', j)][d], lane' = 32g' + d)
+// ------------------------------------------------------------------------------------------------
+__device__ __forceinline__ f32x16 mma32(float a, float b, f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
+}
+
+template <int S>
+__global__ __launch_bounds__(64 * ((S + 31) / 32)) void slice_attention_kernel(const float *__restrict__ combined,
+                                                                               const float *__restrict__ w_qkv,
+                                                                               float *__restrict__ slice_token,
+                                                                               float *__restrict__ slice_norm,
+                                                                               float *__restrict__ out_token,
+                                                                               uint16_t *__restrict__ tokp) {
+  constexpr int NTILE = (S + 31) / 32, D = 32, D1 = 33, NCH = S / 16;
+  __shared__ float ks[NTILE * 32 * D1], vs[NTILE * 32 * D1];
+  const int bh = blockIdx.x, tid = threadIdx.x, lane = tid & 63, i = lane & 31, g = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int s = 32 * wave + i;
+  const bool live = s < S;
+
+  const float *src = combined + ((int64_t)bh * S + (live ? s : 0)) * D1;
+  const float cnt = src[D] + kSliceNormEps;
+  float tk[16];  // tok[s][2kk + g]
+#pragma unroll
+  for (int kk = 0; kk < 16; ++kk) tk[kk] = live ? src[2 * kk + g] / cnt : 0.f;
+  if (live) {
+    if (slice_token) {
+#pragma unroll
+      for (int kk = 0; kk < 16; ++kk) slice_token[((int64_t)bh * S + s) * D + 2 * kk + g] = tk[kk];
+    }
+    if (slice_norm && g == 0) slice_norm[(int64_t)bh * S + s] = cnt;
+  }
+
+  f32x16 qT, kT, vT;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) qT[r] = kT[r] = vT[r] = 0.f;
+#pragma unroll
+  for (int kk = 0; kk < 16; ++kk) {
+    const float *wr = w_qkv + i * D + 2 * kk + g;  // row e = 32m + i of Wqkv, column d = 2kk + g
+    qT = mma32(wr[0], tk[kk], qT);
+    kT = mma32(wr[32 * D], tk[kk], kT);
+    vT = mma32(wr[64 * D], tk[kk], vT);
+  }
+  // q scaled for a base-2 softmax: exp(x / sqrt(D)) = exp2(x * log2e / sqrt(D))
+  const float qscale = kLog2e * 0.17677669529663687f;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    qT[r] *= qscale;
+    ks[s * D1 + rowmap(r, g)] = kT[r];
+    vs[s * D1 + rowmap(r, g)] = vT[r];
+  }
+  __syncthreads();
+
+  f32x16 sc[NTILE];  // scores^T: lane <-> my query, register r <-> key 32tt + rowmap(r, g)
+#pragma unroll
+  for (int tt = 0; tt < NTILE; ++tt) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) sc[tt][r] = 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) sc[tt] = mma32(ks[(32 * tt + i) * D1 + rowmap(r, g)], qT[r], sc[tt]);
+  }
+  float mx = -INFINITY;
+#pragma unroll
+  for (int tt = 0; tt < NTILE; ++tt)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      if constexpr (S % 32 != 0) {
+        if (32 * tt + rowmap(r, g) >= S) sc[tt][r] = -INFINITY;  // keys beyond S
+      }
+      mx = fmaxf(mx, sc[tt][r]);
+    }
+  mx = half_max(mx);
+  float sum = 0.f;
+#pragma unroll
+  for (int tt = 0; tt < NTILE; ++tt)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      sc[tt][r] = __builtin_amdgcn_exp2f(sc[tt][r] - mx);
+      sum += sc[tt][r];
+    }
+  sum = half_sum(sum);
+
+  f32x16 oT;  // out^T: lane <-> my query, register r <-> d = rowmap(r, g)
+#pragma unroll
+  for (int r = 0; r < 16; ++r) oT[r] = 0.f;
+#pragma unroll
+  for (int tt = 0; tt < NTILE; ++tt)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) oT = mma32(vs[(32 * tt + rowmap(r, g)) * D1 + i], sc[tt][r], oT);
+  const float inv = 1.f / sum;
+  if (live) {
+    float *dst = out_token + ((int64_t)bh * S + s) * D;
+    const int cq = s >> 4, ss = s & 15, gp = (ss >> 2) & 1, j = 4 * (ss >> 3) + (ss & 3);
+    uint16_t *pk = tokp + (((int64_t)bh * NCH + cq) * 64 + 32 * gp) * 8 + j;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const float o = oT[r] * inv;
+      dst[rowmap(r, g)] = o;
+      pk[rowmap(r, g) * 8] = to_bf16_bits(o);
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
 // Kernel (d): deslice + out_linear (+ residual, + LayerNorm).  Persistent workgroups of H waves; one 32-point
 // tile per iteration, worked on by the whole workgroup:
 //   wave h   : out_x^T_h (32 d x 32 pts) = tok'^T_h . w^T_h   A = tokp frags (LDS, per batch), B = w_pack chunks
@@ -830,6 +944,29 @@ int slice_reduce(const pa_shape &s, const void *w_pack, const void *fx_pack, flo
   if (s.S == 32) return slice_reduce_s<32>(s, w_pack, fx_pack, partials, st);
   if (s.S == 64) return slice_reduce_s<64>(s, w_pack, fx_pack, partials, st);
   return slice_reduce_s<128>(s, w_pack, fx_pack, partials, st);
+}
+
+template <int S>
+static int slice_attention_s(const pa_shape &s, const float *combined, const float *w_qkv, float *slice_token,
+                             float *slice_norm, float *out_token, void *tokp, hipStream_t st) {
+  hipLaunchKernelGGL((slice_attention_kernel<S>), dim3((unsigned)(s.B * s.H)), dim3(64 * ((S + 31) / 32)), 0, st, combined,
+                     w_qkv, slice_token, slice_norm, out_token, static_cast<uint16_t *>(tokp));
+  return launch_status();
+}
+
+// second pass of the reduction + kernel (c); also leaves the attended tokens as bf16 operands of kernel (d)
+int combine_attention(const pa_shape &s, const pa_params &p, const float *partials, int64_t G, float *slice_token,
+                      float *slice_norm, float *out_token, void *tokp, hipStream_t st) {
+  const float *combined = nullptr;
+  int rc = pa::general::combine_partials(s, partials, G, &combined, st);
+  if (rc) return rc;
+  switch (s.S) {
+    case 16: return slice_attention_s<16>(s, combined, p.qkv_project_weight, slice_token, slice_norm, out_token, tokp, st);
+    case 32: return slice_attention_s<32>(s, combined, p.qkv_project_weight, slice_token, slice_norm, out_token, tokp, st);
+    case 64: return slice_attention_s<64>(s, combined, p.qkv_project_weight, slice_token, slice_norm, out_token, tokp, st);
+    case 128: return slice_attention_s<128>(s, combined, p.qkv_project_weight, slice_token, slice_norm, out_token, tokp, st);
+    default: return PA_ERR_UNSUPPORTED;
+  }
 }
 
 int pack_tokens(const pa_shape &s, const float *tok_out, void *tokp, hipStream_t st) {
