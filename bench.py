@@ -153,20 +153,31 @@ def time_full_model(name, B, N, functional_dim, embedding_dim, slice_num, n_laye
     g = torch.Generator().manual_seed(1234)
     fx = torch.randn(B, N, functional_dim, generator=g).cuda()
     emb = torch.randn(B, N, embedding_dim, generator=g).cuda()
-    with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
+    def fwd(a, b):
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            return model(a, b)
+
+    def timed(fn):
         for _ in range(warmup):
-            out = model(fx, emb)
+            o = fn(fx, emb)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for _ in range(steps):
-            out = model(fx, emb)
+            o = fn(fx, emb)
         torch.cuda.synchronize()
-        dt = (time.perf_counter() - t0) / steps
-    assert torch.isfinite(out.float()).all()
+        return (time.perf_counter() - t0) / steps, o
+
+    with torch.no_grad():
+        dt, out = timed(fwd)
+        assert torch.isfinite(out.float()).all()
+        graphed = pn.GraphedForward(fwd, fx, emb)  # the same forward replayed from a HIP graph
+        dt_graph, out = timed(lambda a, b: graphed.replay())
+        assert torch.isfinite(out.float()).all()
     del model, fx, emb, out
     torch.cuda.empty_cache()
     return {"workload": name, "batch": B, "points": N, "layers": n_layers, "slice_num": slice_num,
-            "ms_per_forward": round(dt * 1e3, 3), "mpoints_per_s": round(B * N / dt / 1e6, 2)}
+            "ms_per_forward": round(dt * 1e3, 3), "mpoints_per_s": round(B * N / dt / 1e6, 2),
+            "ms_per_forward_graph": round(dt_graph * 1e3, 3), "mpoints_per_s_graph": round(B * N / dt_graph / 1e6, 2)}
 
 
 def time_structured_model(steps=5, warmup=2):
@@ -238,6 +249,18 @@ def main():
     mpoints = B * N / (ms_per_step * 1e-3) / 1e6
     assert torch.isfinite(y[:, :1024].float()).all()
 
+    # the same call recorded once into a HIP graph and replayed (same kernels, one submission per step)
+    graphed = pn.GraphedForward(layer, x)  # its static input holds a copy of x
+    for _ in range(args.warmup):
+        graphed.replay()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        graphed.replay()
+    torch.cuda.synchronize()
+    ms_graph = (time.perf_counter() - t0) / args.steps * 1e3
+    del graphed
+
     if args.calibrate_copy:
         src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
         dst = torch.empty_like(src)
@@ -301,6 +324,7 @@ def main():
                    "hidden": C, "heads": H, "dim_head": 32, "slice_num": S,
                    "kernel_path": "mfma" if path == 1 else "general"},
         "roofline": roofline, "kernels": kernels,
+        "graph_replay": {"ms_per_step": round(ms_graph, 4), "mpoints_per_s": round(B * N / (ms_graph * 1e-3) / 1e6, 2)},
     }
     if not args.no_models:
         out["block_mlp"] = time_block_mlp(1 << 20, 256, 1024)

@@ -4,6 +4,7 @@ from .physics_attention import (  # noqa: F401
     PhysicsAttentionIrregularMesh,
     PhysicsAttentionStructuredMesh2D,
 )
+from .graphs import GraphedForward  # noqa: F401
 from .transolver import Mlp, Transolver, TransolverBlock  # noqa: F401
 
 __version__ = "0.1.0"

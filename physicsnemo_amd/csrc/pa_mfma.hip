@@ -442,22 +442,6 @@ __global__ __launch_bounds__(256) void slice_reduce_kernel(const u32x4 *__restri
   }
 }
 
-// tok' (B, H, S, 32) fp32 -> bf16 A operands of the deslice product: tokp[b][h][cq][lane][j] = tok'[b][h][16cq + kperm-slice][i]
-__global__ __launch_bounds__(256) void pack_tokens_kernel(const float *__restrict__ tok, u32x4 *__restrict__ tokp, int64_t units,
-                                                          int S) {
-  const int NCH = S / 16;
-  for (int64_t u = (int64_t)blockIdx.x * 256 + threadIdx.x; u < units; u += (int64_t)gridDim.x * 256) {
-    const int lane = (int)(u & 63), i = lane & 31, g = lane >> 5;
-    const int64_t q = u >> 6;
-    const int cq = (int)(q % NCH);
-    const int64_t bh = q / NCH;
-    bf16x8 o;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) o[j] = (__bf16)tok[(bh * S + 16 * cq + kperm(0, g, j)) * 32 + i];
-    tokp[u] = __builtin_bit_cast(u32x4, o);
-  }
-}
-
 // ------------------------------------------------------------------------------------------------
 // Kernel (c): normalisation of the combined sums and the per-head slice self-attention, fp32 MFMA
 // (v_mfma_f32_32x32x2_f32: A lane (i, g) holds A[i][k = g], B lane (i, g) holds B[k = g][i], C/D as above).
@@ -967,13 +951,6 @@ int combine_attention(const pa_shape &s, const pa_params &p, const float *partia
     case 128: return slice_attention_s<128>(s, combined, p.qkv_project_weight, slice_token, slice_norm, out_token, tokp, st);
     default: return PA_ERR_UNSUPPORTED;
   }
-}
-
-int pack_tokens(const pa_shape &s, const float *tok_out, void *tokp, hipStream_t st) {
-  const int64_t units = s.B * s.H * (s.S / 16) * 64;
-  hipLaunchKernelGGL(pack_tokens_kernel, dim3((unsigned)((units + 255) / 256)), dim3(256), 0, st, tok_out,
-                     static_cast<u32x4 *>(tokp), units, (int)s.S);
-  return launch_status();
 }
 
 int deslice_project(const pa_shape &s, const void *blob, const void *w_pack, const void *tokp, void *y,
