@@ -224,7 +224,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
       //             gelu of the second half of the tile of chunk c-1 -> the tile is complete, goes to the partner
       //   phase 2   y^T += W2 fragment(ct, k4) of hidden chunk c-1 . gelu(h)^T (own tile, then the partner's);
       //             gelu of the first half of the tile of chunk c
-      constexpr int RING = 4, AHEAD = 3;
+      constexpr int RING = 6, AHEAD = 5;
       f32x16 hacc[2];
 #pragma unroll
       for (int r = 0; r < 16; ++r) hacc[0][r] = hacc[1][r] = b1s[(c < NC ? 64 * c : 0) + 32 * p + rowmap(r, g)];
