@@ -58,17 +58,19 @@ int pa_version(void);
 const char *pa_status_string(int code);
 
 /* Dimensions of one layer call.  `conv_k` = 0 selects the irregular-mesh variant (nn.Linear
- * projections, PA.py:625-627); conv_k = k > 0 selects the structured-2D variant (k x k Conv2d,
- * stride 1, zero padding k/2, PA.py:740-742) and then N must equal grid_h*grid_w with token
- * n = i*grid_w + j (PA.py:772-783). */
+ * projections, PA.py:625-627); conv_k = k > 0 selects a structured variant (k x k Conv2d or k x k x k Conv3d,
+ * stride 1, zero padding k/2, PA.py:740-742, :865-867): grid_d = 0 is the 2-D grid, N = grid_h*grid_w, token
+ * n = i*grid_w + j (PA.py:772-783); grid_d > 0 the 3-D grid, N = grid_h*grid_w*grid_d, token
+ * n = (i*grid_w + j)*grid_d + l (PA.py:896-907). */
 typedef struct pa_shape {
   int64_t B, N, C, H, D, S;
   int64_t grid_h, grid_w, conv_k;
+  int64_t grid_d;
 } pa_shape;
 
 /* Parameters of one layer, named as the reference state_dict keys (PA.py:285-327, :625-627, :740-742). */
 typedef struct pa_params {
-  const void *in_project_x_weight;   /* dtype, (H*D, C) or (H*D, C, k, k) */
+  const void *in_project_x_weight;   /* dtype, (H*D, C), (H*D, C, k, k) or (H*D, C, k, k, k) */
   const float *in_project_x_bias;    /* (H*D) */
   const void *in_project_fx_weight;  /* dtype, same shape */
   const float *in_project_fx_bias;   /* (H*D) */

@@ -52,6 +52,34 @@ def conv2d_projection(x, weight, bias, grid_h, grid_w):
     return out.reshape(b, n, o) + _f64(bias)
 
 
+def conv3d_projection(x, weight, bias, grid_h, grid_w, grid_d):
+    """Zero-padded stride-1 cross-correlation on tokens n = (i*W + j)*Dg + l (physics_attention.py:865-867,892-907).
+
+    y[b, n(i,j,l), o] = bias[o] + sum_{c,u,v,z} W[o,c,u,v,z] * x[b, n(i+u-p, j+v-p, l+z-p), c], p = k//2,
+    out-of-grid terms are 0.  Direct loops over the k^3 taps.
+    """
+    x = _f64(x)
+    weight = _f64(weight)
+    b, n, c = x.shape
+    o, c2, k, k2, k3 = weight.shape
+    assert n == grid_h * grid_w * grid_d and c == c2 and k == k2 == k3
+    p = k // 2
+    vol = x.reshape(b, grid_h, grid_w, grid_d, c)
+    out = np.zeros((b, grid_h, grid_w, grid_d, o))
+    for u in range(k):
+        for v in range(k):
+            for z in range(k):
+                di, dj, dl = u - p, v - p, z - p
+                i0, i1 = max(0, -di), min(grid_h, grid_h - di)
+                j0, j1 = max(0, -dj), min(grid_w, grid_w - dj)
+                l0, l1 = max(0, -dl), min(grid_d, grid_d - dl)
+                if i0 >= i1 or j0 >= j1 or l0 >= l1:
+                    continue
+                src = vol[:, i0 + di:i1 + di, j0 + dj:j1 + dj, l0 + dl:l1 + dl, :]
+                out[:, i0:i1, j0:j1, l0:l1, :] += np.einsum("bijlc,oc->bijlo", src, weight[:, :, u, v, z])
+    return out.reshape(b, n, o) + _f64(bias)
+
+
 def layer_forward(p, x, heads, dim_head, variant="irregular", spatial_shape=None):
     """All intermediates of one layer in float64 (steps 1-9 below follow physics_attention.py:529-558).
 
@@ -65,6 +93,10 @@ def layer_forward(p, x, heads, dim_head, variant="irregular", spatial_shape=None
     if variant == "irregular":
         xm = linear_projection(x, p["in_project_x.weight"], p["in_project_x.bias"])
         fm = linear_projection(x, p["in_project_fx.weight"], p["in_project_fx.bias"])
+    elif len(spatial_shape) == 3:
+        gh, gw, gd = spatial_shape
+        xm = conv3d_projection(x, p["in_project_x.weight"], p["in_project_x.bias"], gh, gw, gd)
+        fm = conv3d_projection(x, p["in_project_fx.weight"], p["in_project_fx.bias"], gh, gw, gd)
     else:
         gh, gw = spatial_shape
         xm = conv2d_projection(x, p["in_project_x.weight"], p["in_project_x.bias"], gh, gw)

@@ -65,6 +65,25 @@ def project_conv2d(x, wx, bx, wfx, bfx, heads, dim_head, grid_h, grid_w):
     return one(wx, bx), one(wfx, bfx)
 
 
+def project_conv3d(x, wx, bx, wfx, bfx, heads, dim_head, grid_h, grid_w, grid_d):
+    """Structured-3D projections (physics_attention.py:892-907).
+
+    x is (B, N, C) with N = grid_h*grid_w*grid_d, token n = (i*grid_w + j)*grid_d + l; the reference views it
+    as (B, h, w, d, C), permutes to (B, C, h, w, d), applies a stride-1 zero-padded k^3 cross-correlation
+    (padding k//2) and flattens back with "B (H D) h w d -> B (h w d) H D".
+    """
+    b, n, c = x.shape
+    k = wx.shape[-1]
+    vol = x.view(b, grid_h, grid_w, grid_d, c).permute(0, 4, 1, 2, 3)
+
+    def one(w, bias):
+        y = F.conv3d(vol, w, bias, stride=1, padding=k // 2)  # (B, H*D, h, w, d)
+        y = y.flatten(2).transpose(1, 2)  # (B, h*w*d, H*D)
+        return split_heads(y, heads, dim_head)
+
+    return one(wx, bx), one(wfx, bfx)
+
+
 def slice_logits(x_mid, w_slice, b_slice):
     """in_project_slice on the head-split tensor (physics_attention.py:537): one (S, D) weight for all heads."""
     return F.linear(x_mid, w_slice, b_slice)
@@ -179,6 +198,22 @@ class OraclePhysicsAttentionStructuredMesh2D(_AttentionCore):
                               self.heads, self.dim_head, self.H, self.W)
 
 
+class OraclePhysicsAttentionStructuredMesh3D(_AttentionCore):
+    """physics_attention.py:786-907 with use_te=False, plus=False."""
+
+    def __init__(self, dim, spatial_shape, heads=8, dim_head=64, dropout=0.0, slice_num=32, kernel=3):
+        super().__init__(dim, heads, dim_head, dropout, slice_num)
+        self.H, self.W, self.D = spatial_shape[0], spatial_shape[1], spatial_shape[2]
+        inner = heads * dim_head
+        self.in_project_x = nn.Conv3d(dim, inner, kernel, 1, kernel // 2)
+        self.in_project_fx = nn.Conv3d(dim, inner, kernel, 1, kernel // 2)
+
+    def _project(self, x):
+        return project_conv3d(x, self.in_project_x.weight, self.in_project_x.bias,
+                              self.in_project_fx.weight, self.in_project_fx.bias,
+                              self.heads, self.dim_head, self.H, self.W, self.D)
+
+
 class OracleMlp(nn.Module):
     """Linear -> GELU(erf) -> Linear, keys ``layers.0`` / ``layers.2``
     (physicsnemo/nn/module/mlp_layers.py:139-173 with one hidden width; activations.py:198 'gelu' -> nn.GELU())."""
@@ -208,8 +243,12 @@ class OracleTransolverBlock(nn.Module):
             self.Attn = OraclePhysicsAttentionStructuredMesh2D(
                 hidden_dim, spatial_shape=spatial_shape, heads=num_heads, dim_head=hidden_dim // num_heads,
                 dropout=dropout, slice_num=slice_num)
+        elif len(spatial_shape) == 3:
+            self.Attn = OraclePhysicsAttentionStructuredMesh3D(
+                hidden_dim, spatial_shape=spatial_shape, heads=num_heads, dim_head=hidden_dim // num_heads,
+                dropout=dropout, slice_num=slice_num)
         else:
-            raise ValueError("oracle covers irregular and structured-2D variants only")
+            raise ValueError("oracle covers the irregular, structured-2D and structured-3D variants only")
         self.ln_mlp1 = nn.Sequential(nn.LayerNorm(hidden_dim),
                                      OracleMlp(hidden_dim, hidden_dim * mlp_ratio, hidden_dim))
         if last_layer:

@@ -3,6 +3,7 @@ from .physics_attention import (  # noqa: F401
     PhysicsAttentionBase,
     PhysicsAttentionIrregularMesh,
     PhysicsAttentionStructuredMesh2D,
+    PhysicsAttentionStructuredMesh3D,
 )
 from .graphs import GraphedForward  # noqa: F401
 from .transolver import Mlp, Transolver, TransolverBlock  # noqa: F401

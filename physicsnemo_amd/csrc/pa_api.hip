@@ -11,9 +11,12 @@ int check_shape(int dtype, const pa_shape *s) {
   if (dtype != PA_F32 && dtype != PA_BF16 && dtype != PA_BF16_W8) return PA_ERR_UNSUPPORTED;
   if (dtype == PA_BF16_W8 && s->conv_k != 0) return PA_ERR_UNSUPPORTED;
   if (s->B <= 0 || s->N <= 0 || s->C <= 0 || s->H <= 0 || s->D <= 0 || s->S <= 0) return PA_ERR_DIMS;
-  if (s->conv_k < 0) return PA_ERR_DIMS;
+  if (s->conv_k < 0 || (s->conv_k == 0 && s->grid_d != 0)) return PA_ERR_DIMS;
   if (s->conv_k > 0) {
-    if (s->grid_h <= 0 || s->grid_w <= 0 || s->grid_h * s->grid_w != s->N) return PA_ERR_DIMS;
+    if (s->grid_h <= 0 || s->grid_w <= 0 || s->grid_d < 0) return PA_ERR_DIMS;
+    if (s->grid_h * s->grid_w * (s->grid_d > 0 ? s->grid_d : 1) != s->N) return PA_ERR_DIMS;
+    const int64_t taps = s->conv_k * s->conv_k * (s->grid_d > 0 ? s->conv_k : 1);
+    if (taps * s->C > (int64_t)1 << 30) return PA_ERR_UNSUPPORTED;
     if (s->conv_k % 2 == 0) return PA_ERR_UNSUPPORTED;  // even kernels change the output size in the reference
   }
   if (s->D > PA_MAX_D || s->S > PA_MAX_S) return PA_ERR_UNSUPPORTED;

@@ -18,8 +18,9 @@ namespace general {
 // ------------------------------------------------------------------------------------------------
 // rows_gemm_kernel: out[m, o] = bias[o] + sum_k A(m, k) * W[o, k]
 //   linear: A(m, k) = in[m*K + k]
-//   conv  : K = ks*ks*C, k = tap*C + c, tap = u*ks + v; A(m,k) = in[b, (i+u-p)*gw + (j+v-p), c] or 0 outside
-//           the grid; the PyTorch weight element is W[o, c, u, v] = W[o*K + c*ks*ks + tap].
+//   conv  : K = taps*C, k = tap*C + c; 2-D: taps = ks^2, tap = u*ks + v, A(m,k) = in[b, (i+u-p)*gw + (j+v-p), c];
+//           3-D: taps = ks^3, tap = (u*ks + v)*ks + z, A(m,k) = in[b, ((i+u-p)*gw + (j+v-p))*gd + (l+z-p), c];
+//           0 outside the grid; the PyTorch weight element is W[o, c, u, v(, z)] = W[o*K + c*taps + tap].
 // 64x64 output tile per 256-thread workgroup, 4x4 outputs per thread, K staged 16 at a time through LDS.
 // blockIdx.z selects one of two (W, bias, out) sets that share the same input (x_mid and fx_mid).
 // ------------------------------------------------------------------------------------------------
@@ -31,6 +32,7 @@ struct GemmArgs {
   int64_t M;   // rows = B*N
   int K, O;    // reduction length, output columns
   int C, N, gh, gw, ks;  // conv geometry (ks = 0: linear)
+  int gd;                // depth of a 3-D grid (0: 2-D)
 };
 
 template <typename TA, typename TW>
@@ -49,16 +51,20 @@ __global__ __launch_bounds__(256) void rows_gemm_kernel(GemmArgs a) {
   const int lr = t >> 2;         // tile row / tile out column this thread stages
   const int lk = (t & 3) * 4;    // first of 4 consecutive k it stages
   const int pad = a.ks / 2;
-  const int taps = a.ks * a.ks;
+  const int gd = a.gd > 0 ? a.gd : 1;          // a 2-D grid is a 3-D grid of depth 1 with a single depth tap
+  const int ksd = a.gd > 0 ? a.ks : 1;
+  const int taps = a.ks * a.ks * ksd;
 
   // decode the staged row once
   const int64_t m_ld = m0 + lr;
   const bool m_ok = m_ld < a.M;
   int64_t b_ld = 0;
-  int i_ld = 0, j_ld = 0;
+  int i_ld = 0, j_ld = 0, l_ld = 0;
   if (a.ks > 0 && m_ok) {
     b_ld = m_ld / a.N;
     int n = (int)(m_ld - b_ld * a.N);
+    l_ld = n % gd;
+    n /= gd;
     i_ld = n / a.gw;
     j_ld = n - i_ld * a.gw;
   }
@@ -81,10 +87,11 @@ __global__ __launch_bounds__(256) void rows_gemm_kernel(GemmArgs a) {
           if (o_ld < a.O) wv = load_as_f32(W + (int64_t)o_ld * a.K + k);
         } else {
           const int tap = k / a.C, c = k - tap * a.C;
-          const int u = tap / a.ks, v = tap - u * a.ks;
-          const int ii = i_ld + u - pad, jj = j_ld + v - pad;
-          if (m_ok && ii >= 0 && ii < a.gh && jj >= 0 && jj < a.gw)
-            av = load_as_f32(in + ((b_ld * a.N + (int64_t)ii * a.gw + jj) * a.C + c));
+          const int uv = tap / ksd, z = tap - uv * ksd;
+          const int u = uv / a.ks, v = uv - u * a.ks;
+          const int ii = i_ld + u - pad, jj = j_ld + v - pad, ll = l_ld + (a.gd > 0 ? z - pad : 0);
+          if (m_ok && ii >= 0 && ii < a.gh && jj >= 0 && jj < a.gw && ll >= 0 && ll < gd)
+            av = load_as_f32(in + ((b_ld * a.N + ((int64_t)ii * a.gw + jj) * gd + ll) * a.C + c));
           if (o_ld < a.O) wv = load_as_f32(W + (int64_t)o_ld * a.K + (int64_t)c * taps + tap);
         }
       }
@@ -506,7 +513,8 @@ int project_inputs(int dtype, const pa_shape &s, const pa_params &p, const void 
   a.gh = (int)s.grid_h;
   a.gw = (int)s.grid_w;
   a.ks = (int)s.conv_k;
-  a.K = s.conv_k > 0 ? (int)(s.conv_k * s.conv_k * s.C) : (int)s.C;
+  a.gd = (int)s.grid_d;
+  a.K = s.conv_k > 0 ? (int)(s.conv_k * s.conv_k * (s.grid_d > 0 ? s.conv_k : 1) * s.C) : (int)s.C;
   return dtype == PA_F32 ? launch_gemm<float, float>(a, 2, st) : launch_gemm<bf16, bf16>(a, 2, st);
 }
 

@@ -24,6 +24,7 @@ class LayerDims(NamedTuple):
     grid_h: int = 0
     grid_w: int = 0
     conv_k: int = 0
+    grid_d: int = 0
 
     def c(self) -> _lib.PaShape:
         return _lib.PaShape(*self)

@@ -5,6 +5,7 @@ reference classes in physicsnemo/nn/module/physics_attention.py:
   PhysicsAttentionBase            :209-558
   PhysicsAttentionIrregularMesh   :561-660
   PhysicsAttentionStructuredMesh2D:663-783
+  PhysicsAttentionStructuredMesh3D:786-907
 so that a reference ``state_dict`` loads unchanged and seeded construction consumes the RNG identically.
 
 Scope: forward only, ``plus=False``.  ``use_te`` is accepted for signature compatibility and ignored: the
@@ -18,7 +19,8 @@ import torch.nn as nn
 
 from . import functional as PF
 
-__all__ = ["PhysicsAttentionBase", "PhysicsAttentionIrregularMesh", "PhysicsAttentionStructuredMesh2D"]
+__all__ = ["PhysicsAttentionBase", "PhysicsAttentionIrregularMesh", "PhysicsAttentionStructuredMesh2D",
+           "PhysicsAttentionStructuredMesh3D"]
 
 
 class PhysicsAttentionBase(nn.Module):
@@ -60,11 +62,12 @@ class PhysicsAttentionBase(nn.Module):
 
     # ---------------------------------------------------------------- parameters in kernel form
     def _conv_geometry(self):
-        return 0, 0, 0
+        """(grid_h, grid_w, kernel, grid_d): all zero for the irregular variant, grid_d = 0 for a 2-D grid."""
+        return 0, 0, 0, 0
 
     def layer_dims(self, x: torch.Tensor) -> PF.LayerDims:
-        gh, gw, k = self._conv_geometry()
-        return PF.LayerDims(x.shape[0], x.shape[1], self.dim, self.heads, self.dim_head, self.slice_num, gh, gw, k)
+        gh, gw, k, gd = self._conv_geometry()
+        return PF.LayerDims(x.shape[0], x.shape[1], self.dim, self.heads, self.dim_head, self.slice_num, gh, gw, k, gd)
 
     def kernel_params(self, dtype: torch.dtype, device: torch.device) -> dict:
         """Parameters as the C ABI wants them: the three large weights in ``dtype``, everything else float32,
@@ -192,8 +195,33 @@ class PhysicsAttentionStructuredMesh2D(PhysicsAttentionBase):
         self.in_project_fx = nn.Conv2d(dim, inner_dim, kernel, 1, kernel // 2)
 
     def _conv_geometry(self):
-        return self.H, self.W, self.kernel
+        return self.H, self.W, self.kernel, 0
 
     def _check_spatial(self, x: torch.Tensor) -> None:
         # the reference reshapes with x.view(B, H, W, C) (:772): same failure for a wrong token count
         x.view(x.shape[0], self.H, self.W, x.shape[-1])
+
+
+class PhysicsAttentionStructuredMesh3D(PhysicsAttentionBase):
+    """Row-major 3D grids: k x k x k Conv3d projections, stride 1, zero padding k//2 (reference :857-867).
+
+    ``forward`` takes the flattened ``(B, H_s*W_s*D_s, C)`` tensor with token n = (i*W_s + j)*D_s + l (:896-907).
+    """
+
+    def __init__(self, dim: int, spatial_shape: tuple[int, int, int], heads: int = 8, dim_head: int = 64,
+                 dropout: float = 0.0, slice_num: int = 32, kernel: int = 3, use_te: bool = True, plus: bool = False):
+        super().__init__(dim, heads, dim_head, dropout, slice_num, use_te, plus)
+        inner_dim = dim_head * heads
+        self.H = spatial_shape[0]
+        self.W = spatial_shape[1]
+        self.D = spatial_shape[2]
+        self.kernel = kernel
+        self.in_project_x = nn.Conv3d(dim, inner_dim, kernel, 1, kernel // 2)
+        self.in_project_fx = nn.Conv3d(dim, inner_dim, kernel, 1, kernel // 2)
+
+    def _conv_geometry(self):
+        return self.H, self.W, self.kernel, self.D
+
+    def _check_spatial(self, x: torch.Tensor) -> None:
+        # the reference reshapes with x.view(B, H, W, D, C) (:896): same failure for a wrong token count
+        x.view(x.shape[0], self.H, self.W, self.D, x.shape[-1])

@@ -15,7 +15,8 @@ import torch
 import torch.nn as nn
 
 from . import functional as PF
-from .physics_attention import PhysicsAttentionIrregularMesh, PhysicsAttentionStructuredMesh2D
+from .physics_attention import (PhysicsAttentionIrregularMesh, PhysicsAttentionStructuredMesh2D,
+                                PhysicsAttentionStructuredMesh3D)
 
 __all__ = ["Mlp", "TransolverBlock", "Transolver"]
 
@@ -66,7 +67,7 @@ class TransolverBlock(nn.Module):
         elif len(spatial_shape) == 2:
             self.Attn = PhysicsAttentionStructuredMesh2D(hidden_dim, spatial_shape=spatial_shape, **common)
         elif len(spatial_shape) == 3:
-            raise NotImplementedError("the structured-3D (Conv3d) variant is not built")
+            self.Attn = PhysicsAttentionStructuredMesh3D(hidden_dim, spatial_shape=spatial_shape, **common)
         else:
             raise ValueError(
                 f"Unexpected length of spatial shape encountered in Transolver_block: {len(spatial_shape)}. Expected 2 or 3.")

@@ -18,6 +18,11 @@ def make_pair(variant, dim, heads, dim_head, slice_num, spatial=None, kernel=3, 
     if variant == "irregular":
         ref = to.OraclePhysicsAttentionIrregularMesh(dim, heads=heads, dim_head=dim_head, slice_num=slice_num)
         hip = pn.PhysicsAttentionIrregularMesh(dim, heads=heads, dim_head=dim_head, slice_num=slice_num, use_te=False)
+    elif variant == "structured3d":
+        ref = to.OraclePhysicsAttentionStructuredMesh3D(dim, spatial, heads=heads, dim_head=dim_head,
+                                                        slice_num=slice_num, kernel=kernel)
+        hip = pn.PhysicsAttentionStructuredMesh3D(dim, spatial, heads=heads, dim_head=dim_head, slice_num=slice_num,
+                                                  kernel=kernel, use_te=False)
     else:
         ref = to.OraclePhysicsAttentionStructuredMesh2D(dim, spatial, heads=heads, dim_head=dim_head,
                                                         slice_num=slice_num, kernel=kernel)

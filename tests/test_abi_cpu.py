@@ -39,6 +39,8 @@ def test_argument_errors_are_codes_not_crashes():
     assert lib.pa_workspace_bytes(0, ctypes.byref(_shape(D=4096))) == -3
     assert lib.pa_workspace_bytes(0, ctypes.byref(_shape(conv_k=3, grid_h=8, grid_w=9))) == -2  # 72 != 64
     assert lib.pa_workspace_bytes(0, ctypes.byref(_shape(conv_k=2, grid_h=8, grid_w=8))) == -3
+    assert lib.pa_workspace_bytes(0, ctypes.byref(_shape(conv_k=3, grid_h=4, grid_w=4, grid_d=4))) > 0  # 64 points
+    assert lib.pa_workspace_bytes(0, ctypes.byref(_shape(conv_k=3, grid_h=4, grid_w=4, grid_d=5))) == -2
     assert lib.pa_workspace_bytes(0, ctypes.byref(_shape())) > 0
     # null tensors / params are rejected before anything touches a device
     s = _shape()
@@ -67,6 +69,13 @@ def test_module_signatures_state_dict_and_seeded_init_match_oracle():
     assert list(a2.state_dict()) == list(b2.state_dict())
     assert all(torch.equal(a2.state_dict()[k], b2.state_dict()[k]) for k in a2.state_dict())
     assert (a2.H, a2.W) == (5, 6)
+    torch.manual_seed(7)
+    a3 = pn.PhysicsAttentionStructuredMesh3D(32, (3, 4, 5), heads=2, dim_head=16, slice_num=8, kernel=3, use_te=False)
+    torch.manual_seed(7)
+    b3 = to.OraclePhysicsAttentionStructuredMesh3D(32, (3, 4, 5), heads=2, dim_head=16, slice_num=8, kernel=3)
+    assert list(a3.state_dict()) == list(b3.state_dict())
+    assert all(torch.equal(a3.state_dict()[k], b3.state_dict()[k]) for k in a3.state_dict())
+    assert (a3.H, a3.W, a3.D) == (3, 4, 5) and tuple(a3.in_project_x.weight.shape) == (32, 32, 3, 3, 3)
     # reference defaults: heads=8, dim_head=64, slice_num=64, use_te=True accepted
     d = pn.PhysicsAttentionIrregularMesh(128)
     assert (d.heads, d.dim_head, d.in_project_slice.out_features) == (8, 64, 64)

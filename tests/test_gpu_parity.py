@@ -51,6 +51,44 @@ def test_fp32_structured2d_stages_and_layer(kernel, grid):
     assert_fp32_close(y, want["y"], "layer y")
 
 
+@pytest.mark.parametrize("kernel,grid", [(3, (4, 4, 4)), (3, (8, 8, 8)), (5, (8, 8, 8)), (3, (3, 5, 7)), (1, (4, 6, 5))])
+def test_fp32_structured3d_stages_and_layer(kernel, grid):
+    announce("fp32 structured3d", kernel, grid)
+    B, dim, heads, dim_head, S = 2, 32, 4, 8, 8
+    ref, hip = make_pair("structured3d", dim, heads, dim_head, S, spatial=grid, kernel=kernel, sharpen=2.0)
+    x = torch.randn(B, grid[0] * grid[1] * grid[2], dim)
+    with torch.no_grad():
+        want = ref.stages(x)
+        got = hip.forward_stages(x.cuda())
+        y = hip(x.cuda())
+        yb = hip(x.cuda().bfloat16())
+    for k in STAGES:
+        assert_fp32_close(got[k], want[k], k)
+    assert_fp32_close(y, want["y"], "layer y")
+    assert_rel_l2(yb, want["y"], "bf16 layer y", tol=2e-2)
+    with pytest.raises(RuntimeError):
+        hip(x.cuda()[:, :-1])  # the token count must match the grid, as in the reference's view()
+
+
+def test_structured3d_model_flatten_equivalence():
+    announce("structured3d model: (B, H, W, D, C) input == flattened input")
+    torch.manual_seed(0)
+    grid = (6, 5, 4)
+    m = pn.Transolver(functional_dim=2, out_dim=3, embedding_dim=3, structured_shape=grid, n_layers=2, n_hidden=32,
+                      n_head=4, slice_num=8, mlp_ratio=2, use_te=False).eval().cuda()
+    ref = to.OracleTransolver(functional_dim=2, out_dim=3, embedding_dim=3, structured_shape=grid, n_layers=2, n_hidden=32,
+                              n_head=4, slice_num=8, mlp_ratio=2).eval()
+    ref.load_state_dict(m.state_dict())
+    fx, emb = torch.randn(2, *grid, 2), torch.randn(2, *grid, 3)
+    with torch.no_grad():
+        out5 = m(fx.cuda(), emb.cuda())
+        outf = m(fx.reshape(2, -1, 2).cuda(), emb.reshape(2, -1, 3).cuda())
+        want = ref(fx, emb)
+    assert out5.shape == (2, *grid, 3)
+    assert torch.equal(out5.reshape(2, -1, 3), outf)
+    assert_fp32_close(out5, want, "structured3d model")
+
+
 def test_fp32_block_tail_residual_and_layernorm():
     announce("fp32 block tail")
     B, N, dim, heads, S = 2, 300, 128, 8, 32

@@ -86,6 +86,54 @@ def test_conv_token_order_and_zero_padding():
     np.testing.assert_allclose(no.conv2d_projection(x.numpy(), w2.numpy(), zero.numpy(), gh, gw).reshape(gh, gw), got2.numpy())
 
 
+@pytest.mark.parametrize("kernel", [1, 3])
+def test_torch_oracle_equals_numpy_oracle_structured3d(kernel):
+    B, grid, C, H, D, S = 2, (3, 4, 5), 6, 2, 4, 5
+    m = to.OraclePhysicsAttentionStructuredMesh3D(C, grid, heads=H, dim_head=D, slice_num=S, kernel=kernel).double()
+    x = torch.randn(B, grid[0] * grid[1] * grid[2], C, dtype=torch.float64)
+    with torch.no_grad():
+        st = m.stages(x)
+    ref = no.layer_forward(_sd_np(m), x.numpy(), H, D, variant="structured3d", spatial_shape=grid)
+    for key in ("x_mid", "fx_mid", "w", "tok", "tok_out", "y"):
+        np.testing.assert_allclose(st[key].numpy(), ref[key], rtol=1e-10, atol=1e-12, err_msg=key)
+
+
+def test_conv3d_special_cases_pin_token_order_and_orientation():
+    gh, gw, gd = 3, 4, 5
+    zero = torch.zeros(1, dtype=torch.float64)
+    # (a) a grid of depth 1 with weights confined to the central depth tap is the 2-D variant
+    x2 = torch.randn(2, gh * gw, 3, dtype=torch.float64)
+    w2 = torch.randn(4, 3, 3, 3, dtype=torch.float64)
+    b2 = torch.randn(4, dtype=torch.float64)
+    w3 = torch.zeros(4, 3, 3, 3, 3, dtype=torch.float64)
+    w3[:, :, :, :, 1] = w2
+    a, _ = to.project_conv2d(x2, w2, b2, w2, b2, 1, 4, gh, gw)
+    c, _ = to.project_conv3d(x2, w3, b2, w3, b2, 1, 4, gh, gw, 1)
+    assert torch.allclose(a, c, rtol=1e-12, atol=1e-13)
+    # (b) k = 1 is the per-point linear map
+    xl = torch.randn(2, gh * gw * gd, 3, dtype=torch.float64)
+    w1 = torch.randn(4, 3, 1, 1, 1, dtype=torch.float64)
+    c1, _ = to.project_conv3d(xl, w1, b2, w1, b2, 1, 4, gh, gw, gd)
+    l1, _ = to.project_linear(xl, w1[:, :, 0, 0, 0], b2, w1[:, :, 0, 0, 0], b2, 1, 4)
+    assert torch.allclose(c1, l1, rtol=1e-12, atol=1e-13)
+    # (c) token order n = (i*W + j)*Dg + l and cross-correlation orientation: tap (u, v, z) reads x[i+u-1, j+v-1, l+z-1]
+    x = torch.zeros(1, gh * gw * gd, 1, dtype=torch.float64)
+    i0, j0, l0 = 1, 3, 4
+    x[0, (i0 * gw + j0) * gd + l0, 0] = 1.0
+    w = torch.zeros(1, 1, 3, 3, 3, dtype=torch.float64)
+    w[0, 0, 0, 2, 1] = 1.0  # reads one step back in i, one step forward in j, same l
+    out, _ = to.project_conv3d(x, w, zero, w, zero, 1, 1, gh, gw, gd)
+    vol = out.reshape(gh, gw, gd)
+    assert vol[i0 + 1, j0 - 1, l0] == 1.0 and vol.sum() == 1.0
+    ones = torch.ones(1, 1, 3, 3, 3, dtype=torch.float64)
+    full, _ = to.project_conv3d(x, ones, zero, ones, zero, 1, 1, gh, gw, gd)
+    want = torch.zeros(gh, gw, gd, dtype=torch.float64)
+    want[0:3, 2:4, 3:5] = 1.0  # the 3x3x3 neighbourhood clipped at the faces (zero padding)
+    assert torch.equal(full.reshape(gh, gw, gd), want)
+    np.testing.assert_allclose(
+        no.conv3d_projection(x.numpy(), w.numpy(), zero.numpy(), gh, gw, gd).reshape(gh, gw, gd), vol.numpy())
+
+
 def test_softmax_rows_and_temperature_clamp():
     B, N, H, D, S = 2, 11, 3, 4, 5
     logits = torch.randn(B, N, H, S, dtype=torch.float64) * 4
