@@ -137,6 +137,54 @@ int pa_deslice_project(int dtype, const pa_shape *shape, const pa_params *p, con
                        const float *out_slice_token, void *scratch, void *y, const pa_block_tail *tail,
                        void *stream);
 
+/* ---- backward pass (general kernels; fp32 arithmetic, fp32 or bf16 storage) -------------------------
+ * The reference has no backward code of its own: gradients come from autograd over PA.py:501-558
+ * (exercised by test/nn/module/test_physics_attention.py:185-226, :364-387).  The entry points below are the
+ * layer-specific parts of that gradient; the weight gradients, which are plain GEMMs over the point axis
+ * (d W = d out^T . in), are left to the caller's GEMM library.  With g = d out_x (B,N,H*D):
+ *   1. pa_rows_gemm            g = d y . W_out                  (and, last, d x = [d x_mid | d fx_mid] . [W_x ; W_fx])
+ *   2. pa_slice_weighted_sum   d tok'[s,:] = sum_n w[n,s] g[n,:]                      (adjoint of PA.py:480-481)
+ *   3. pa_slice_attention_backward   d tok' -> gradients of the un-normalised slice sums  (PA.py:429-465, :185-203)
+ *   4. pa_slice_softmax_backward     per point: d x_mid, d fx_mid, d z (slice logits before the temperature),
+ *                                    d temperature                                    (PA.py:172-203, :480-481, :537)
+ */
+
+/* out[m, o] = bias[o] + sum_k A(m, k) weight[o, k] over the B*N rows of `in` (B, N, c_in); bias may be NULL.
+ * grid->conv_k == 0: A(m, k) = in[m, k], weight (c_out, c_in).  conv_k = k > 0: the stride-1 zero-padded
+ * convolution over the point grid (grid_h, grid_w[, grid_d]) with weight (c_out, c_in, k, k[, k]) as torch lays
+ * it out.  Only B, N, grid_* and conv_k of `grid` are read.  `weight` has the activation dtype. */
+int pa_rows_gemm(int dtype, const pa_shape *grid, int64_t c_in, int64_t c_out, const void *in, const void *weight,
+                 const float *bias, void *out, void *stream);
+
+/* sums[b,h,s,d] = sum_n w[b,n,h,s] v[b,n,h*D+d] for d < D, sums[b,h,s,D] = sum_n w[b,n,h,s]; float32
+ * (B,H,S,D+1).  `partials` as for pa_slice_reduce.  Two passes, fixed order. */
+int pa_slice_weighted_sum(int dtype, const pa_shape *shape, const void *w, const void *v, float *partials,
+                          float *sums, void *stream);
+
+/* 1 if the backward entry points serve this shape (their LDS footprints fit), 0 if not, negative = error. */
+int pa_backward_query(int dtype, const pa_shape *shape);
+
+/* Backward of the slice attention and of the normalisation tok = num / nrm (nrm = slice_norm = sum_n w + 1e-2).
+ *   d_out_slice_token (B,H,S,D): gradient w.r.t. the attended tokens.
+ *   scratch: float32, B*H*2*S*S elements.
+ *   d_num (B,H,S,D), d_norm (B,H,S): gradients w.r.t. num and nrm.  slice_norm == NULL: d_num receives the
+ *   gradient w.r.t. slice_token itself and d_norm is not written (plain backward of pa_slice_attention).
+ *   d_qkv_partials (B*H, 3D, D): each (b,h)'s share of d qkv_project_weight; the caller adds them up. */
+int pa_slice_attention_backward(const pa_shape *shape, const pa_params *p, const float *slice_token,
+                                const float *slice_norm, const float *d_out_slice_token, float *scratch,
+                                float *d_num, float *d_norm, float *d_qkv_partials, void *stream);
+
+/* Per-point part of the backward pass.  Inputs as saved by the forward stages (x_mid, fx_mid (B,N,H*D), w (B,N,H,S),
+ * out_slice_token (B,H,S,D)), d_out_x (B,N,H*D) and the d_num / d_norm of pa_slice_attention_backward.  Outputs:
+ *   d_proj (B,N,2*H*D) = [d x_mid | d fx_mid];  d_z (B,N,H,S) = gradient of the in_project_slice output;
+ *   d_temperature_partials: float32, pa_backward_point_tiles(shape) * H elements; d clamp(temperature)[h] is the
+ *   sum over the first index (the caller masks it with 0.5 <= temperature <= 5, the clamp's own gradient). */
+int64_t pa_backward_point_tiles(const pa_shape *shape);
+int pa_slice_softmax_backward(int dtype, const pa_shape *shape, const pa_params *p, const void *x_mid,
+                              const void *fx_mid, const void *w, const void *d_out_x, const float *out_slice_token,
+                              const float *d_num, const float *d_norm, void *d_proj, void *d_z,
+                              float *d_temperature_partials, void *stream);
+
 /* ---- stage-level entry points of the bf16 MFMA kernels (shapes with pa_query_path() == 1) ------
  * Intermediates use an internal register-order ("packed") layout; buffers are opaque to the caller and
  * sized by pa_mfma_buffer_bytes(shape, which):

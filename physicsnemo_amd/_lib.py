@@ -21,6 +21,8 @@ EXPORTED = [
     "pa_deslice_project", "pa_layer_forward", "pa_mfma_buffer_bytes", "pa_mfma_pack_params",
     "pa_mfma_project_softmax", "pa_mfma_slice_reduce", "pa_mfma_project_softmax_reduce", "pa_mfma_partial_groups",
      "pa_mfma_combine_attention", "pa_mfma_deslice_project", "pa_mlp_query", "pa_mlp_workspace_bytes", "pa_mlp_forward",
+    "pa_rows_gemm", "pa_slice_weighted_sum", "pa_backward_query", "pa_backward_point_tiles",
+    "pa_slice_attention_backward", "pa_slice_softmax_backward",
 ]
 
 PA_BUF_BLOB, PA_BUF_FX_PACK, PA_BUF_W_PACK, PA_BUF_PARTIALS, PA_BUF_TOKP = range(5)
@@ -105,6 +107,18 @@ def load() -> ctypes.CDLL:
     lib.pa_mlp_forward.restype = c_int
     lib.pa_mlp_forward.argtypes = [c_int, c_int64, c_int64, c_int64, POINTER(PaMlpParams), c_void_p, c_void_p, pt, c_void_p,
                                    c_int64, c_void_p]
+    lib.pa_rows_gemm.restype = c_int
+    lib.pa_rows_gemm.argtypes = [c_int, ps, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]
+    lib.pa_slice_weighted_sum.restype = c_int
+    lib.pa_slice_weighted_sum.argtypes = [c_int, ps, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]
+    lib.pa_backward_query.restype = c_int
+    lib.pa_backward_query.argtypes = [c_int, ps]
+    lib.pa_backward_point_tiles.restype = c_int64
+    lib.pa_backward_point_tiles.argtypes = [ps]
+    lib.pa_slice_attention_backward.restype = c_int
+    lib.pa_slice_attention_backward.argtypes = [ps, pp] + [c_void_p] * 8
+    lib.pa_slice_softmax_backward.restype = c_int
+    lib.pa_slice_softmax_backward.argtypes = [c_int, ps, pp] + [c_void_p] * 11
     _lib = lib
     return lib
 

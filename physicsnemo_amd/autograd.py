@@ -1,0 +1,104 @@
+"""Training path of the PhysicsAttention layer: a torch.autograd.Function whose forward runs the stage-level HIP
+kernels and keeps their intermediates, and whose backward runs the backward kernels of libphysattn.so.
+
+The reference has no backward code of its own (autograd differentiates physics_attention.py:501-558 op by op);
+this is the same gradient, assembled from
+  * hand-written kernels for everything specific to the layer (slice softmax, slice sums, slice attention,
+    deslice and their adjoints, the input-gradient GEMMs / transposed convolutions), and
+  * the GEMM library behind ``torch.matmul`` for the weight gradients, which are plain ``d out^T . in`` products
+    over the point axis.
+"""
+from __future__ import annotations
+
+import itertools
+
+import torch
+
+from . import functional as PF
+
+
+def _rows(t: torch.Tensor) -> torch.Tensor:
+    return t.reshape(-1, t.shape[-1])
+
+
+def _conv_weight_grad(d_out: torch.Tensor, x: torch.Tensor, grid: tuple, k: int) -> torch.Tensor:
+    """d W[o, c, taps...] = sum over grid points of d_out[p, o] * x[p + tap - k//2, c] (zero outside the grid).
+
+    d_out (B, N, O), x (B, N, C) channels-last over `grid`; returns (O, C, k, ..., k) in d_out's dtype."""
+    B, O, C, nd, pad = x.shape[0], d_out.shape[-1], x.shape[-1], len(grid), k // 2
+    dg, xg = d_out.reshape(B, *grid, O), x.reshape(B, *grid, C)
+    dW = torch.zeros((O, C) + (k,) * nd, dtype=d_out.dtype, device=x.device)
+    for tap in itertools.product(range(k), repeat=nd):
+        lo = [max(0, pad - u) for u in tap]
+        hi = [min(g, g + pad - u) for g, u in zip(grid, tap)]
+        if any(a >= b for a, b in zip(lo, hi)):
+            continue
+        out_sl = (slice(None),) + tuple(slice(a, b) for a, b in zip(lo, hi))
+        in_sl = (slice(None),) + tuple(slice(a + u - pad, b + u - pad) for a, b, u in zip(lo, hi, tap))
+        dW[(slice(None), slice(None)) + tap] = dg[out_sl].reshape(-1, O).t() @ xg[in_sl].reshape(-1, C)
+    return dW
+
+
+class PhysicsAttentionFunction(torch.autograd.Function):
+    """y = PhysicsAttention(x); differentiable w.r.t. x and the ten parameters."""
+
+    @staticmethod
+    def forward(ctx, x, dims, kparams, wx, bx, wf, bf, ws, bs, temperature, wqkv, wo, bo):
+        x_mid, fx_mid = PF.project_inputs(x, kparams, dims)
+        w = PF.slice_softmax(x_mid, kparams, dims)
+        tok, norm = PF.slice_reduce(w, fx_mid, dims)
+        tok_out = PF.slice_attention(tok, kparams, dims)
+        y, out_x = PF.deslice_project(w, tok_out, kparams, dims, return_out_x=True)
+        ctx.save_for_backward(x, x_mid, fx_mid, w, tok, norm, tok_out, out_x, temperature)
+        ctx.dims, ctx.kparams = dims, kparams
+        ctx.param_like = (wx, bx, wf, bf, ws, bs, temperature, wqkv, wo, bo)
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, x_mid, fx_mid, w, tok, norm, tok_out, out_x, temperature = ctx.saved_tensors
+        dims, kp = ctx.dims, ctx.kparams
+        B, N, C, H, D, S = dims.B, dims.N, dims.C, dims.H, dims.D, dims.S
+        HD = H * D
+        dy = dy.to(x.dtype).contiguous()
+        linear = PF.LayerDims(B, N, C, H, D, S)
+
+        # out_linear: g = d out_x, d W_out, d b_out
+        wo = kp["out_linear_weight"].view(C, HD)
+        g = PF.rows_gemm(dy, wo.t().contiguous(), None, linear, C, HD)
+        d_wo = _rows(dy).t() @ _rows(out_x)
+        d_bo = _rows(dy).sum(0, dtype=torch.float32)
+
+        # adjoint of the deslice w.r.t. the attended tokens, then the slice attention and the normalisation
+        d_tok_out = PF.slice_weighted_sum(w, g, dims)[..., :D].contiguous()
+        d_num, d_norm, d_wqkv = PF.slice_attention_backward(tok, norm, d_tok_out, kp, dims)
+
+        # per point: slice softmax, aggregation and deslice adjoints
+        d_proj, d_z, d_temp = PF.slice_softmax_backward(x_mid, fx_mid, w, g, tok_out, d_num, d_norm, kp, dims)
+        d_ws = d_z.reshape(-1, S).t() @ x_mid.reshape(-1, D)
+        d_bs = d_z.reshape(-1, S).sum(0, dtype=torch.float32)
+        t = temperature.reshape(-1)
+        d_temp = d_temp * ((t >= 0.5) & (t <= 5.0)).to(d_temp.dtype)
+
+        # input projections: d x and the weight / bias gradients
+        k = dims.conv_k
+        wx, wf = kp["in_project_x_weight"], kp["in_project_fx_weight"]
+        if k == 0:
+            w_cat = torch.cat([wx.view(HD, C).t(), wf.view(HD, C).t()], dim=1).contiguous()  # (C, 2HD)
+            dx = PF.rows_gemm(d_proj, w_cat, None, linear, 2 * HD, C)
+            d_w_in = _rows(d_proj).t() @ _rows(x)  # (2HD, C)
+        else:
+            grid = (dims.grid_h, dims.grid_w) + ((dims.grid_d,) if dims.grid_d > 0 else ())
+            taps = (k,) * len(grid)
+            w_both = torch.cat([wx.view(HD, C, *taps), wf.view(HD, C, *taps)], dim=0)  # (2HD, C, k, ...)
+            # transposed convolution = the same gather with flipped taps and swapped channel roles
+            w_t = w_both.flip(dims=tuple(range(2, 2 + len(grid)))).transpose(0, 1).contiguous()
+            dx = PF.rows_gemm(d_proj, w_t, None, dims, 2 * HD, C)
+            d_w_in = _conv_weight_grad(d_proj, x, grid, k)
+        d_b_in = _rows(d_proj).sum(0, dtype=torch.float32)
+
+        like = ctx.param_like
+        grads = (d_w_in[:HD], d_b_in[:HD], d_w_in[HD:], d_b_in[HD:], d_ws, d_bs, d_temp, d_wqkv, d_wo, d_bo)
+        grads = tuple(gr.reshape(p.shape).to(p.dtype) if ctx.needs_input_grad[3 + i] else None
+                      for i, (gr, p) in enumerate(zip(grads, like)))
+        return (dx if ctx.needs_input_grad[0] else None, None, None) + grads

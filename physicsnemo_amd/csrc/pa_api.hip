@@ -237,6 +237,91 @@ int pa_deslice_project(int dtype, const pa_shape *shape, const pa_params *p, con
   return rc;
 }
 
+int pa_rows_gemm(int dtype, const pa_shape *grid, int64_t c_in, int64_t c_out, const void *in, const void *weight,
+                 const float *bias, void *out, void *stream) {
+  if (!grid) return PA_ERR_NULL;
+  if (dtype != PA_F32 && dtype != PA_BF16) return PA_ERR_UNSUPPORTED;
+  if (grid->B <= 0 || grid->N <= 0 || c_in <= 0 || c_out <= 0 || grid->conv_k < 0) return PA_ERR_DIMS;
+  if (c_in > (1 << 16) || c_out > (1 << 16) || grid->N > (int64_t)1 << 31) return PA_ERR_UNSUPPORTED;
+  if (grid->conv_k > 0) {
+    if (grid->grid_h <= 0 || grid->grid_w <= 0 || grid->grid_d < 0) return PA_ERR_DIMS;
+    if (grid->grid_h * grid->grid_w * (grid->grid_d > 0 ? grid->grid_d : 1) != grid->N) return PA_ERR_DIMS;
+    if (grid->conv_k % 2 == 0) return PA_ERR_UNSUPPORTED;
+    const int64_t taps = grid->conv_k * grid->conv_k * (grid->grid_d > 0 ? grid->conv_k : 1);
+    if (taps * c_in > (int64_t)1 << 30) return PA_ERR_UNSUPPORTED;
+  } else if (grid->grid_d != 0) {
+    return PA_ERR_DIMS;
+  }
+  if (!in || !weight || !out) return PA_ERR_NULL;
+  if (!aligned16(in) || !aligned16(weight) || !aligned16(out)) return PA_ERR_ALIGN;
+  return pa::general::rows_gemm(dtype, *grid, c_in, c_out, in, weight, bias, out, static_cast<hipStream_t>(stream));
+}
+
+int pa_slice_weighted_sum(int dtype, const pa_shape *shape, const void *w, const void *v, float *partials, float *sums,
+                          void *stream) {
+  int rc = check_shape(dtype, shape);
+  if (rc) return rc;
+  if (dtype == PA_BF16_W8) return PA_ERR_UNSUPPORTED;
+  if (!w || !v || !partials || !sums) return PA_ERR_NULL;
+  if (!aligned16(w) || !aligned16(v) || !aligned16(partials) || !aligned16(sums)) return PA_ERR_ALIGN;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if ((rc = pa::general::slice_partial(dtype, *shape, w, v, partials, st))) return rc;
+  const float *total = nullptr;
+  if ((rc = pa::general::combine_partials(*shape, partials, pa::general::partial_count(*shape), &total, st))) return rc;
+  const size_t bytes = (size_t)(shape->B * shape->H * shape->S * (shape->D + 1)) * 4;
+  hipError_t e = hipMemcpyAsync(sums, total, bytes, hipMemcpyDeviceToDevice, st);
+  return e == hipSuccess ? PA_OK : (int)e;
+}
+
+static int check_backward_shape(int dtype, const pa_shape *shape) {
+  int rc = check_shape(dtype, shape);
+  if (rc) return rc;
+  if (dtype == PA_BF16_W8) return PA_ERR_UNSUPPORTED;
+  if (pa::backward::attention_lds_bytes(*shape) > pa::kMaxLdsBytes) return PA_ERR_UNSUPPORTED;
+  if (pa::backward::point_tile_rows(*shape) == 0) return PA_ERR_UNSUPPORTED;
+  return PA_OK;
+}
+
+int pa_backward_query(int dtype, const pa_shape *shape) {
+  int rc = check_backward_shape(dtype, shape);
+  return rc == PA_OK ? 1 : (rc == PA_ERR_UNSUPPORTED ? 0 : rc);
+}
+
+int64_t pa_backward_point_tiles(const pa_shape *shape) {
+  int rc = check_backward_shape(PA_F32, shape);
+  if (rc) return rc;
+  return pa::backward::point_tiles(*shape);
+}
+
+int pa_slice_attention_backward(const pa_shape *shape, const pa_params *p, const float *slice_token,
+                                const float *slice_norm, const float *d_out_slice_token, float *scratch,
+                                float *d_num, float *d_norm, float *d_qkv_partials, void *stream) {
+  int rc = check_backward_shape(PA_F32, shape);
+  if (rc) return rc;
+  if (!p || !p->qkv_project_weight || !slice_token || !d_out_slice_token || !scratch || !d_num || !d_qkv_partials)
+    return PA_ERR_NULL;
+  if (slice_norm && !d_norm) return PA_ERR_NULL;
+  return pa::backward::slice_attention(*shape, *p, slice_token, slice_norm, d_out_slice_token, scratch, d_num, d_norm,
+                                       d_qkv_partials, static_cast<hipStream_t>(stream));
+}
+
+int pa_slice_softmax_backward(int dtype, const pa_shape *shape, const pa_params *p, const void *x_mid,
+                              const void *fx_mid, const void *w, const void *d_out_x, const float *out_slice_token,
+                              const float *d_num, const float *d_norm, void *d_proj, void *d_z,
+                              float *d_temperature_partials, void *stream) {
+  int rc = check_backward_shape(dtype, shape);
+  if (rc) return rc;
+  if (!p || !p->in_project_slice_weight || !p->in_project_slice_bias || !p->temperature) return PA_ERR_NULL;
+  if (!x_mid || !fx_mid || !w || !d_out_x || !out_slice_token || !d_num || !d_norm || !d_proj || !d_z ||
+      !d_temperature_partials)
+    return PA_ERR_NULL;
+  if (!aligned16(x_mid) || !aligned16(fx_mid) || !aligned16(w) || !aligned16(d_out_x) || !aligned16(d_proj) ||
+      !aligned16(d_z))
+    return PA_ERR_ALIGN;
+  return pa::backward::slice_softmax(dtype, *shape, *p, x_mid, fx_mid, w, d_out_x, out_slice_token, d_num, d_norm,
+                                     d_proj, d_z, d_temperature_partials, static_cast<hipStream_t>(stream));
+}
+
 int64_t pa_mfma_buffer_bytes(const pa_shape *shape, int which) {
   int rc = check_shape(PA_BF16, shape);
   if (rc) return rc;

@@ -1,0 +1,361 @@
+// Backward pass of the PhysicsAttention layer: the per-point and per-slice kernels (fp32 arithmetic on the
+// vector ALUs, fp32 or bf16 storage, natural layouts).  Gradients that are plain GEMMs over the point axis
+// (the weight gradients) are left to the caller's GEMM library; everything that is specific to the layer
+// is here.
+//
+// Forward (PA.py:501-558), per batch b and head h, with T = clamp(temperature_h, .5, 5):
+//   z[n,s]   = x_mid[n,:] . Ws[s,:] + bs[s];  w[n,:] = softmax_s(z[n,:] / T)
+//   num[s,:] = sum_n w[n,s] fx_mid[n,:];  nrm[s] = sum_n w[n,s] + 1e-2;  tok = num / nrm
+//   tok'     = softmax(q k^T / sqrt D) v with q|k|v = tok Wqkv^T
+//   out_x[n,:] = sum_s w[n,s] tok'[s,:]
+// Backward, given g = d out_x:
+//   d tok'[s,:] = sum_n w[n,s] g[n,:]                    (slice_partial_kernel + combine, same as the forward sum)
+//   d tok       = attention backward                      (slice_attention_backward_kernel)
+//   d num = d tok / nrm;  d nrm[s] = -(d tok[s,:] . tok[s,:]) / nrm[s]
+//   d w[n,s]  = g[n,:] . tok'[s,:] + fx_mid[n,:] . d num[s,:] + d nrm[s]      (slice_softmax_backward_kernel)
+//   d fx_mid[n,:] = sum_s w[n,s] d num[s,:]
+//   d l[n,s]  = w[n,s] (d w[n,s] - sum_s' w[n,s'] d w[n,s']);  d z = d l / T;  d T = -sum_{n,s} d l (z/T) / T
+//   d x_mid[n,:] = sum_s d z[n,s] Ws[s,:]
+#include "pa_common.h"
+#include "pa_host.h"
+
+namespace pa {
+namespace backward {
+
+constexpr int kAttnBwdThreads = 512;
+
+// ------------------------------------------------------------------------------------------------
+// slice_attention_backward_kernel: one workgroup per (b, h).  Recomputes q, k, v and the S x S attention
+// matrix P from the saved slice tokens, then
+//   dP = dO v^T;  dSc = P * (dP - rowsum(P * dP)) / sqrt(D);  dq = dSc k;  dk = dSc^T q;  dv = P^T dO
+//   d tok = dq Wq + dk Wk + dv Wv;   dWq = dq^T tok, dWk = dk^T tok, dWv = dv^T tok   (this (b, h)'s share)
+// P and dSc live in a caller-provided scratch of 2*S*S floats per (b, h) (cache resident); the S x D operands in LDS.
+// `slice_norm` != nullptr: the outputs are d num = d tok / nrm and d nrm (gradients of the un-normalised sums);
+// nullptr: d_num receives d tok itself and d_norm is not written.
+// ------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(kAttnBwdThreads) void slice_attention_backward_kernel(
+    const float *__restrict__ slice_token, const float *__restrict__ slice_norm, const float *__restrict__ w_qkv,
+    const float *__restrict__ d_out_token, float *__restrict__ scratch, float *__restrict__ d_num,
+    float *__restrict__ d_norm, float *__restrict__ d_wqkv_part, int D, int S) {
+  extern __shared__ float lds[];
+  const int D1 = D + 1;
+  float *tok = lds;             // S * D1
+  float *q = tok + S * D1;      // later: d tok
+  float *k = q + S * D1;
+  float *v = k + S * D1;
+  float *dq = v + S * D1;
+  float *dk = dq + S * D1;
+  float *dv = dk + S * D1;
+  float *rows = dv + S * D1;    // per wave: p[S], ds[S]
+  const int t = threadIdx.x;
+  const int bh = blockIdx.x;
+  const int wave = t >> 6, lane = t & 63;
+  constexpr int kWaves = kAttnBwdThreads / 64;
+  const float *tk = slice_token + (int64_t)bh * S * D;
+  const float *dO = d_out_token + (int64_t)bh * S * D;
+  float *P = scratch + (int64_t)bh * 2 * S * S;
+  float *dSc = P + (int64_t)S * S;
+
+  for (int i = t; i < S * D; i += kAttnBwdThreads) tok[(i / D) * D1 + (i % D)] = tk[i];
+  __syncthreads();
+  for (int i = t; i < S * 3 * D; i += kAttnBwdThreads) {
+    const int s = i / (3 * D), e = i - s * 3 * D;
+    const float *wr = w_qkv + (int64_t)e * D;
+    const float *tr = tok + s * D1;
+    float acc = 0.f;
+    for (int d = 0; d < D; ++d) acc = fmaf(tr[d], wr[d], acc);
+    float *dst = e < D ? q : (e < 2 * D ? k : v);
+    dst[s * D1 + (e % D)] = acc;
+  }
+  __syncthreads();
+
+  const float scale = rsqrtf((float)D);
+  float *pr = rows + wave * 2 * S;
+  float *dr = pr + S;
+  for (int s = wave; s < S; s += kWaves) {
+    const float *qs = q + s * D1;
+    const float *dos = dO + (int64_t)s * D;
+    float mx = -INFINITY;
+    for (int u = lane; u < S; u += 64) {
+      const float *ku = k + u * D1;
+      const float *vu = v + u * D1;
+      float acc = 0.f, dp = 0.f;
+      for (int e = 0; e < D; ++e) {
+        acc = fmaf(qs[e], ku[e], acc);
+        dp = fmaf(dos[e], vu[e], dp);
+      }
+      acc *= scale;
+      pr[u] = acc;
+      dr[u] = dp;
+      mx = fmaxf(mx, acc);
+    }
+    mx = wave_max(mx);
+    float sum = 0.f;
+    for (int u = lane; u < S; u += 64) {
+      const float e = expf(pr[u] - mx);
+      pr[u] = e;
+      sum += e;
+    }
+    sum = wave_sum(sum);
+    const float inv = 1.f / sum;
+    float delta = 0.f;
+    for (int u = lane; u < S; u += 64) {
+      const float p = pr[u] * inv;
+      pr[u] = p;
+      delta = fmaf(p, dr[u], delta);
+    }
+    delta = wave_sum(delta);
+    for (int u = lane; u < S; u += 64) {
+      const float ds = pr[u] * (dr[u] - delta) * scale;
+      dr[u] = ds;
+      P[(int64_t)s * S + u] = pr[u];
+      dSc[(int64_t)s * S + u] = ds;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    for (int e = lane; e < D; e += 64) {
+      float acc = 0.f;
+      for (int u = 0; u < S; ++u) acc = fmaf(dr[u], k[u * D1 + e], acc);
+      dq[s * D1 + e] = acc;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+  }
+  __syncthreads();  // P, dSc (global, this workgroup's own) and dq are complete
+
+  for (int i = t; i < S * D; i += kAttnBwdThreads) {
+    const int u = i / D, e = i - u * D;
+    float ak = 0.f, av = 0.f;
+    for (int s = 0; s < S; ++s) {
+      ak = fmaf(dSc[(int64_t)s * S + u], q[s * D1 + e], ak);
+      av = fmaf(P[(int64_t)s * S + u], dO[(int64_t)s * D + e], av);
+    }
+    dk[u * D1 + e] = ak;
+    dv[u * D1 + e] = av;
+  }
+  __syncthreads();
+
+  float *dtok = q;  // q is no longer needed
+  for (int i = t; i < S * D; i += kAttnBwdThreads) {
+    const int s = i / D, d = i - s * D;
+    const float *wq = w_qkv + d, *wk = wq + (int64_t)D * D, *wv = wk + (int64_t)D * D;
+    float acc = 0.f;
+    for (int e = 0; e < D; ++e) {
+      acc = fmaf(dq[s * D1 + e], wq[(int64_t)e * D], acc);
+      acc = fmaf(dk[s * D1 + e], wk[(int64_t)e * D], acc);
+      acc = fmaf(dv[s * D1 + e], wv[(int64_t)e * D], acc);
+    }
+    dtok[s * D1 + d] = acc;
+    const float scale_out = slice_norm ? 1.f / slice_norm[(int64_t)bh * S + s] : 1.f;
+    d_num[(int64_t)bh * S * D + i] = acc * scale_out;
+  }
+  for (int i = t; i < 3 * D * D; i += kAttnBwdThreads) {
+    const int which = i / (D * D), rem = i - which * D * D;
+    const int e = rem / D, d = rem - e * D;
+    const float *src = which == 0 ? dq : (which == 1 ? dk : dv);
+    float acc = 0.f;
+    for (int s = 0; s < S; ++s) acc = fmaf(src[s * D1 + e], tok[s * D1 + d], acc);
+    d_wqkv_part[(int64_t)bh * 3 * D * D + i] = acc;
+  }
+  if (!slice_norm) return;
+  __syncthreads();
+  for (int s = t; s < S; s += kAttnBwdThreads) {
+    float acc = 0.f;
+    for (int d = 0; d < D; ++d) acc = fmaf(dtok[s * D1 + d], tok[s * D1 + d], acc);
+    d_norm[(int64_t)bh * S + s] = -acc / slice_norm[(int64_t)bh * S + s];
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// slice_softmax_backward_kernel: grid (row tiles of R points per batch, H).  See the file header for the formulas.
+// LDS: the head's tables tok', d num, Ws (row stride D+1), d nrm, bs; the tile's rows of x_mid, fx_mid, g (row stride
+// D+1) and three R x (S+1) arrays (w, d w -> d z, logits).  R is a power of two <= 32, 256 / R threads share a row
+// in the row reductions.
+// Outputs: d_proj (B, N, 2*H*D) = [d x_mid | d fx_mid], d_z (B, N, H, S), dT_part[tile, h] (summed by the caller).
+// ------------------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void slice_softmax_backward_kernel(
+    const T *__restrict__ x_mid, const T *__restrict__ fx_mid, const T *__restrict__ w, const T *__restrict__ d_out_x,
+    const float *__restrict__ out_token, const float *__restrict__ d_num, const float *__restrict__ d_norm,
+    const float *__restrict__ w_slice, const float *__restrict__ b_slice, const float *__restrict__ temperature,
+    T *__restrict__ d_proj, T *__restrict__ d_z, float *__restrict__ dT_part, int64_t N, int H, int D, int S, int R,
+    int tiles_per_batch) {
+  extern __shared__ float lds[];
+  const int D1 = D + 1, S1 = S + 1;
+  float *to = lds;               // S * D1
+  float *dn = to + S * D1;       // S * D1
+  float *ws = dn + S * D1;       // S * D1
+  float *dnr = ws + S * D1;      // S
+  float *bs = dnr + S;           // S
+  float *xm = bs + S;            // R * D1
+  float *fm = xm + R * D1;       // R * D1
+  float *go = fm + R * D1;       // R * D1
+  float *wl = go + R * D1;       // R * S1
+  float *dwl = wl + R * S1;      // R * S1
+  float *lgl = dwl + R * S1;     // R * S1
+  __shared__ float red[4];
+  const int t = threadIdx.x;
+  const int h = blockIdx.y;
+  const int b = blockIdx.x / tiles_per_batch;
+  const int64_t n0 = (int64_t)(blockIdx.x % tiles_per_batch) * R;
+  const int rows = (int)min((int64_t)R, N - n0);
+  const int64_t m0 = (int64_t)b * N + n0;
+  const int HD = H * D, HS = H * S;
+  const float temp = clamp_temperature(temperature[h]);
+  const float inv_temp = 1.f / temp;
+
+  const int64_t bh = (int64_t)b * H + h;
+  for (int i = t; i < S * D; i += 256) {
+    const int s = i / D, d = i - s * D;
+    to[s * D1 + d] = out_token[bh * S * D + i];
+    dn[s * D1 + d] = d_num[bh * S * D + i];
+    ws[s * D1 + d] = w_slice[i];
+  }
+  for (int i = t; i < S; i += 256) {
+    dnr[i] = d_norm[bh * S + i];
+    bs[i] = b_slice[i];
+  }
+  for (int i = t; i < R * D; i += 256) {
+    const int r = i / D, d = i - r * D;
+    const bool ok = r < rows;
+    const int64_t off = (m0 + r) * HD + h * D + d;
+    xm[r * D1 + d] = ok ? load_as_f32(x_mid + off) : 0.f;
+    fm[r * D1 + d] = ok ? load_as_f32(fx_mid + off) : 0.f;
+    go[r * D1 + d] = ok ? load_as_f32(d_out_x + off) : 0.f;
+  }
+  for (int i = t; i < R * S; i += 256) {
+    const int r = i / S, s = i - r * S;
+    wl[r * S1 + s] = r < rows ? load_as_f32(w + (m0 + r) * HS + h * S + s) : 0.f;
+  }
+  __syncthreads();
+
+  // d w and the logits
+  for (int i = t; i < R * S; i += 256) {
+    const int r = i / S, s = i - r * S;
+    const float *xr = xm + r * D1, *fr = fm + r * D1, *gr = go + r * D1;
+    const float *tr = to + s * D1, *nr = dn + s * D1, *wr = ws + s * D1;
+    float z = 0.f, dw = 0.f;
+    for (int d = 0; d < D; ++d) {
+      z = fmaf(xr[d], wr[d], z);
+      dw = fmaf(gr[d], tr[d], dw);
+      dw = fmaf(fr[d], nr[d], dw);
+    }
+    lgl[r * S1 + s] = round_to(x_mid, z + bs[s]) * inv_temp;  // the forward divides the stored Linear output
+    dwl[r * S1 + s] = dw + dnr[s];
+  }
+  __syncthreads();
+
+  // softmax backward per row; 256 / R threads per row
+  const int tpr = 256 / R;
+  const int r_own = t / tpr, j_own = t - r_own * tpr;
+  float dot = 0.f;
+  for (int s = j_own; s < S; s += tpr) dot = fmaf(wl[r_own * S1 + s], dwl[r_own * S1 + s], dot);
+  for (int off = tpr >> 1; off > 0; off >>= 1) dot += __shfl_xor(dot, off, 64);
+  float tsum = 0.f;
+  for (int s = j_own; s < S; s += tpr) {
+    const float dl = wl[r_own * S1 + s] * (dwl[r_own * S1 + s] - dot);
+    tsum = fmaf(dl, lgl[r_own * S1 + s], tsum);
+    dwl[r_own * S1 + s] = dl * inv_temp;
+  }
+  tsum = wave_sum(tsum);
+  if ((t & 63) == 0) red[t >> 6] = tsum;
+  __syncthreads();
+  if (t == 0) dT_part[(int64_t)blockIdx.x * H + h] = -(((red[0] + red[1]) + red[2]) + red[3]) * inv_temp;
+
+  for (int i = t; i < rows * S; i += 256) {
+    const int r = i / S, s = i - r * S;
+    store_from_f32(d_z + (m0 + r) * HS + h * S + s, dwl[r * S1 + s]);
+  }
+  for (int i = t; i < rows * D; i += 256) {
+    const int r = i / D, d = i - r * D;
+    const float *wr = wl + r * S1, *zr = dwl + r * S1;
+    float dx = 0.f, df = 0.f;
+    for (int s = 0; s < S; ++s) {
+      dx = fmaf(zr[s], ws[s * D1 + d], dx);
+      df = fmaf(wr[s], dn[s * D1 + d], df);
+    }
+    store_from_f32(d_proj + (m0 + r) * 2 * HD + h * D + d, dx);
+    store_from_f32(d_proj + (m0 + r) * 2 * HD + HD + h * D + d, df);
+  }
+}
+
+// ================================================================================================
+// host launchers
+// ================================================================================================
+static int launch_status() {
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? PA_OK : (int)e;
+}
+
+template <typename F>
+static int allow_dynamic_lds(F kernel, size_t bytes) {
+  if (bytes > kMaxLdsBytes) return PA_ERR_UNSUPPORTED;
+  if (bytes > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+    if (e != hipSuccess) return (int)e;
+  }
+  return PA_OK;
+}
+
+size_t attention_lds_bytes(const pa_shape &s) {
+  return (size_t)(7 * s.S * (s.D + 1) + (kAttnBwdThreads / 64) * 2 * s.S) * 4;
+}
+
+int slice_attention(const pa_shape &s, const pa_params &p, const float *slice_token, const float *slice_norm,
+                    const float *d_out_token, float *scratch, float *d_num, float *d_norm, float *d_wqkv_part,
+                    hipStream_t st) {
+  const size_t lds = attention_lds_bytes(s);
+  int rc = allow_dynamic_lds(slice_attention_backward_kernel, lds);
+  if (rc) return rc;
+  hipLaunchKernelGGL(slice_attention_backward_kernel, dim3((unsigned)(s.B * s.H)), dim3(kAttnBwdThreads), lds, st,
+                     slice_token, slice_norm, p.qkv_project_weight, d_out_token, scratch, d_num, d_norm, d_wqkv_part,
+                     (int)s.D, (int)s.S);
+  return launch_status();
+}
+
+// Rows per tile of slice_softmax_backward_kernel: the largest power of two <= 32 whose LDS footprint fits; 0 = none.
+int point_tile_rows(const pa_shape &s) {
+  const size_t fixed = (size_t)(3 * s.S * (s.D + 1) + 2 * s.S) * 4;
+  for (int R = 32; R >= 4; R >>= 1) {
+    const size_t per = (size_t)R * (3 * (s.D + 1) + 3 * (s.S + 1)) * 4;
+    if (fixed + per <= 120 * 1024) return R;
+  }
+  return 0;
+}
+
+int64_t point_tiles(const pa_shape &s) {
+  const int R = point_tile_rows(s);
+  return R == 0 ? 0 : s.B * ((s.N + R - 1) / R);
+}
+
+template <typename T>
+static int slice_softmax_t(const pa_shape &s, const pa_params &p, const void *x_mid, const void *fx_mid, const void *w,
+                           const void *d_out_x, const float *out_token, const float *d_num, const float *d_norm,
+                           void *d_proj, void *d_z, float *dT_part, hipStream_t st) {
+  const int R = point_tile_rows(s);
+  if (R == 0) return PA_ERR_UNSUPPORTED;
+  const size_t lds =
+      (size_t)(3 * s.S * (s.D + 1) + 2 * s.S + (size_t)R * (3 * (s.D + 1) + 3 * (s.S + 1))) * 4;
+  int rc = allow_dynamic_lds(slice_softmax_backward_kernel<T>, lds);
+  if (rc) return rc;
+  const int tiles = (int)((s.N + R - 1) / R);
+  dim3 grid((unsigned)(tiles * s.B), (unsigned)s.H);
+  hipLaunchKernelGGL((slice_softmax_backward_kernel<T>), grid, dim3(256), lds, st, static_cast<const T *>(x_mid),
+                     static_cast<const T *>(fx_mid), static_cast<const T *>(w), static_cast<const T *>(d_out_x),
+                     out_token, d_num, d_norm, p.in_project_slice_weight, p.in_project_slice_bias, p.temperature,
+                     static_cast<T *>(d_proj), static_cast<T *>(d_z), dT_part, s.N, (int)s.H, (int)s.D, (int)s.S, R,
+                     tiles);
+  return launch_status();
+}
+
+int slice_softmax(int dtype, const pa_shape &s, const pa_params &p, const void *x_mid, const void *fx_mid,
+                  const void *w, const void *d_out_x, const float *out_token, const float *d_num, const float *d_norm,
+                  void *d_proj, void *d_z, float *dT_part, hipStream_t st) {
+  return dtype == PA_F32
+             ? slice_softmax_t<float>(s, p, x_mid, fx_mid, w, d_out_x, out_token, d_num, d_norm, d_proj, d_z, dT_part, st)
+             : slice_softmax_t<bf16>(s, p, x_mid, fx_mid, w, d_out_x, out_token, d_num, d_norm, d_proj, d_z, dT_part, st);
+}
+
+}  // namespace backward
+}  // namespace pa

@@ -518,6 +518,27 @@ int project_inputs(int dtype, const pa_shape &s, const pa_params &p, const void 
   return dtype == PA_F32 ? launch_gemm<float, float>(a, 2, st) : launch_gemm<bf16, bf16>(a, 2, st);
 }
 
+// out[m, o] = bias[o] + sum_k A(m, k) weight[o, k] for any (c_in, c_out): a Linear over the rows when grid.conv_k == 0,
+// else the k x k (x k) convolution over grid's point grid with weight (c_out, c_in, k, k(, k)).
+int rows_gemm(int dtype, const pa_shape &grid, int64_t c_in, int64_t c_out, const void *in, const void *weight,
+              const float *bias, void *out, hipStream_t st) {
+  GemmArgs a{};
+  a.in = in;
+  a.w[0] = weight;
+  a.bias[0] = bias;
+  a.out[0] = out;
+  a.M = grid.B * grid.N;
+  a.O = (int)c_out;
+  a.C = (int)c_in;
+  a.N = (int)grid.N;
+  a.gh = (int)grid.grid_h;
+  a.gw = (int)grid.grid_w;
+  a.ks = (int)grid.conv_k;
+  a.gd = (int)grid.grid_d;
+  a.K = grid.conv_k > 0 ? (int)(grid.conv_k * grid.conv_k * (grid.grid_d > 0 ? grid.conv_k : 1) * c_in) : (int)c_in;
+  return dtype == PA_F32 ? launch_gemm<float, float>(a, 1, st) : launch_gemm<bf16, bf16>(a, 1, st);
+}
+
 int out_linear(int dtype, const pa_shape &s, const pa_params &p, const void *out_x, void *y, hipStream_t st) {
   GemmArgs a{};
   a.in = out_x;

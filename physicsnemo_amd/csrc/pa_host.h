@@ -16,6 +16,8 @@ int dequant_e4m3(const void *in, const float *scale, void *out, int64_t rows, in
 int project_inputs(int dtype, const pa_shape &s, const pa_params &p, const void *x, void *x_mid, void *fx_mid,
                    hipStream_t st);
 int out_linear(int dtype, const pa_shape &s, const pa_params &p, const void *out_x, void *y, hipStream_t st);
+int rows_gemm(int dtype, const pa_shape &grid, int64_t c_in, int64_t c_out, const void *in, const void *weight,
+              const float *bias, void *out, hipStream_t st);
 int slice_softmax(int dtype, const pa_shape &s, const pa_params &p, const void *x_mid, void *w, hipStream_t st);
 int64_t partial_count(const pa_shape &s);
 size_t combine_attn_lds_bytes(const pa_shape &s);
@@ -26,6 +28,18 @@ int combine_attention(const pa_shape &s, const pa_params &p, const float *partia
 int deslice(int dtype, const pa_shape &s, const void *w, const float *out_token, void *out_x, hipStream_t st);
 int residual_ln(int dtype, const pa_shape &s, void *y, const pa_block_tail &tail, hipStream_t st);
 }  // namespace general
+
+namespace backward {
+size_t attention_lds_bytes(const pa_shape &s);
+int slice_attention(const pa_shape &s, const pa_params &p, const float *slice_token, const float *slice_norm,
+                    const float *d_out_token, float *scratch, float *d_num, float *d_norm, float *d_wqkv_part,
+                    hipStream_t st);
+int point_tile_rows(const pa_shape &s);
+int64_t point_tiles(const pa_shape &s);
+int slice_softmax(int dtype, const pa_shape &s, const pa_params &p, const void *x_mid, const void *fx_mid,
+                  const void *w, const void *d_out_x, const float *out_token, const float *d_num, const float *d_norm,
+                  void *d_proj, void *d_z, float *dT_part, hipStream_t st);
+}  // namespace backward
 
 namespace mfma {
 bool supported(int dtype, const pa_shape &s);

@@ -103,8 +103,10 @@ def _c_tail(residual, ln_weight, ln_bias, ln_eps, ln_out):
     return _lib.PaBlockTail(_lib.ptr(residual), _lib.ptr(ln_weight), _lib.ptr(ln_bias), float(ln_eps), _lib.ptr(ln_out))
 
 
-def deslice_project(w, tok_out, params, dims: LayerDims, residual=None, ln_weight=None, ln_bias=None, ln_eps=1e-5):
-    """Returns y, or (fx_new, ln_out) when a residual / LayerNorm tail is requested."""
+def deslice_project(w, tok_out, params, dims: LayerDims, residual=None, ln_weight=None, ln_bias=None, ln_eps=1e-5,
+                    return_out_x=False):
+    """Returns y, or (fx_new, ln_out) when a residual / LayerNorm tail is requested; with `return_out_x` the
+    desliced (B, N, H*D) input of out_linear is appended."""
     _need_cuda(w, tok_out, residual)
     lib = _lib.load()
     y = torch.empty(dims.B, dims.N, dims.C, dtype=w.dtype, device=w.device)
@@ -114,7 +116,8 @@ def deslice_project(w, tok_out, params, dims: LayerDims, residual=None, ln_weigh
     _lib.check(lib.pa_deslice_project(_lib.dtype_code(w.dtype), byref(dims.c()), byref(_c_params(params)),
                                       w.data_ptr(), tok_out.data_ptr(), scratch.data_ptr(), y.data_ptr(),
                                       byref(tail), _lib.current_stream_ptr(w.device)), "pa_deslice_project")
-    return y if (residual is None and ln_out is None) else (y, ln_out)
+    out = y if (residual is None and ln_out is None) else (y, ln_out)
+    return (out, scratch) if return_out_x else out
 
 
 def quantize_e4m3_per_channel(weight: torch.Tensor):
@@ -252,3 +255,75 @@ class MfmaStages:
         _lib.check(self.lib.pa_mfma_deslice_project(byref(self.shape), self.blob.data_ptr(), self.w_pack.data_ptr(),
                                                     self.tokp.data_ptr(), y.data_ptr(), byref(tail), self._stream()),
                    "pa_mfma_deslice_project")
+
+
+# ---------------------------------------------------------------------------------------------------
+# backward-pass entry points
+# ---------------------------------------------------------------------------------------------------
+def backward_supported(dtype: torch.dtype, dims: LayerDims) -> bool:
+    rc = _lib.load().pa_backward_query(_lib.dtype_code(dtype), byref(dims.c()))
+    if rc < 0:
+        _lib.check(rc, "pa_backward_query")
+    return bool(rc)
+
+
+def rows_gemm(inp, weight, bias, dims: LayerDims, c_in: int, c_out: int):
+    """out (B, N, c_out) = Linear or grid convolution of inp (B, N, c_in); `dims` supplies B, N and the grid."""
+    _need_cuda(inp, weight, bias)
+    out = torch.empty(dims.B, dims.N, c_out, dtype=inp.dtype, device=inp.device)
+    _lib.check(_lib.load().pa_rows_gemm(_lib.dtype_code(inp.dtype), byref(dims.c()), c_in, c_out, inp.data_ptr(),
+                                        weight.data_ptr(), _lib.ptr(bias), out.data_ptr(),
+                                        _lib.current_stream_ptr(inp.device)), "pa_rows_gemm")
+    return out
+
+
+def slice_weighted_sum(w, v, dims: LayerDims):
+    """(B, H, S, D+1) float32: sum_n w[n,s] * [v[n,:], 1]."""
+    _need_cuda(w, v)
+    lib = _lib.load()
+    shape = dims.c()
+    g = lib.pa_reduce_partial_count(byref(shape))
+    if g < 0:
+        _lib.check(int(g), "pa_reduce_partial_count")
+    partials = torch.empty(g * dims.B * dims.H * dims.S * (dims.D + 1), dtype=torch.float32, device=w.device)
+    sums = torch.empty(dims.B, dims.H, dims.S, dims.D + 1, dtype=torch.float32, device=w.device)
+    _lib.check(lib.pa_slice_weighted_sum(_lib.dtype_code(w.dtype), byref(shape), w.data_ptr(), v.data_ptr(),
+                                         partials.data_ptr(), sums.data_ptr(), _lib.current_stream_ptr(w.device)),
+               "pa_slice_weighted_sum")
+    return sums
+
+
+def slice_attention_backward(tok, norm, d_tok_out, params, dims: LayerDims):
+    """Returns (d_num, d_norm, d_qkv_weight); with norm=None: (d_tok, None, d_qkv_weight)."""
+    _need_cuda(tok, norm, d_tok_out)
+    f32 = dict(dtype=torch.float32, device=tok.device)
+    BH = dims.B * dims.H
+    scratch = torch.empty(BH * 2 * dims.S * dims.S, **f32)
+    d_num = torch.empty(dims.B, dims.H, dims.S, dims.D, **f32)
+    d_norm = torch.empty(dims.B, dims.H, dims.S, **f32) if norm is not None else None
+    parts = torch.empty(BH, 3 * dims.D, dims.D, **f32)
+    _lib.check(_lib.load().pa_slice_attention_backward(byref(dims.c()), byref(_c_params(params)), tok.data_ptr(),
+                                                       _lib.ptr(norm), d_tok_out.data_ptr(), scratch.data_ptr(),
+                                                       d_num.data_ptr(), _lib.ptr(d_norm), parts.data_ptr(),
+                                                       _lib.current_stream_ptr(tok.device)),
+               "pa_slice_attention_backward")
+    return d_num, d_norm, parts.sum(0)
+
+
+def slice_softmax_backward(x_mid, fx_mid, w, d_out_x, tok_out, d_num, d_norm, params, dims: LayerDims):
+    """Returns (d_proj (B,N,2HD) = [d x_mid | d fx_mid], d_z (B,N,H,S), d clamp(temperature) (H) float32)."""
+    _need_cuda(x_mid, fx_mid, w, d_out_x, tok_out, d_num, d_norm)
+    lib = _lib.load()
+    shape = dims.c()
+    tiles = lib.pa_backward_point_tiles(byref(shape))
+    if tiles < 0:
+        _lib.check(int(tiles), "pa_backward_point_tiles")
+    d_proj = torch.empty(dims.B, dims.N, 2 * dims.H * dims.D, dtype=w.dtype, device=w.device)
+    d_z = torch.empty(dims.B, dims.N, dims.H, dims.S, dtype=w.dtype, device=w.device)
+    dT = torch.empty(int(tiles), dims.H, dtype=torch.float32, device=w.device)
+    _lib.check(lib.pa_slice_softmax_backward(_lib.dtype_code(w.dtype), byref(shape), byref(_c_params(params)),
+                                             x_mid.data_ptr(), fx_mid.data_ptr(), w.data_ptr(), d_out_x.data_ptr(),
+                                             tok_out.data_ptr(), d_num.data_ptr(), d_norm.data_ptr(),
+                                             d_proj.data_ptr(), d_z.data_ptr(), dT.data_ptr(),
+                                             _lib.current_stream_ptr(w.device)), "pa_slice_softmax_backward")
+    return d_proj, d_z, dT.sum(0)

@@ -8,9 +8,10 @@ reference classes in physicsnemo/nn/module/physics_attention.py:
   PhysicsAttentionStructuredMesh3D:786-907
 so that a reference ``state_dict`` loads unchanged and seeded construction consumes the RNG identically.
 
-Scope: forward only, ``plus=False``.  ``use_te`` is accepted for signature compatibility and ignored: the
-HIP kernels are the only backend.  There is no CPU path and no autograd: calling with gradients enabled on
-tensors that require grad raises.
+Scope: ``plus=False``.  ``use_te`` is accepted for signature compatibility and ignored: the HIP kernels are the
+only backend and there is no CPU path.  Under ``torch.no_grad()`` the fused inference kernels run; with gradients
+enabled on tensors that require them the stage-level kernels run and the backward pass is served by the library's
+backward kernels (see ``autograd.py``).
 """
 from __future__ import annotations
 
@@ -18,6 +19,7 @@ import torch
 import torch.nn as nn
 
 from . import functional as PF
+from .autograd import PhysicsAttentionFunction
 
 __all__ = ["PhysicsAttentionBase", "PhysicsAttentionIrregularMesh", "PhysicsAttentionStructuredMesh2D",
            "PhysicsAttentionStructuredMesh3D"]
@@ -115,13 +117,12 @@ class PhysicsAttentionBase(nn.Module):
     def _check_spatial(self, x: torch.Tensor) -> None:
         pass
 
+    def _needs_grad(self, x: torch.Tensor) -> bool:
+        return torch.is_grad_enabled() and (x.requires_grad or any(p.requires_grad for p in self.parameters()))
+
     def _prepare_input(self, x: torch.Tensor) -> torch.Tensor:
         if not x.is_cuda:
             raise RuntimeError("physicsnemo_amd PhysicsAttention runs on GPU tensors only (no CPU fallback)")
-        if torch.is_grad_enabled() and (x.requires_grad or any(p.requires_grad for p in self.parameters())):
-            raise RuntimeError(
-                "physicsnemo_amd PhysicsAttention implements the forward pass only; call it under "
-                "torch.no_grad() / torch.inference_mode()")
         if self.training and self.out_dropout.p > 0:
             raise RuntimeError("dropout > 0 in training mode is not served by the HIP kernels")
         if torch.is_autocast_enabled("cuda"):
@@ -134,10 +135,27 @@ class PhysicsAttentionBase(nn.Module):
         self._check_spatial(x)
         return x.contiguous()
 
+    def _forward_with_grad(self, x: torch.Tensor) -> torch.Tensor:
+        """Training path: stage-level kernels forward, backward kernels in `autograd.PhysicsAttentionFunction`."""
+        if self.fp8_weights:
+            raise RuntimeError("fp8 weights are an inference format: no gradients flow through them")
+        dims = self.layer_dims(x)
+        if not PF.backward_supported(x.dtype, dims):
+            raise RuntimeError(f"the backward kernels do not serve this shape: {dims}")
+        return PhysicsAttentionFunction.apply(
+            x, dims, self.kernel_params(x.dtype, x.device), self.in_project_x.weight, self.in_project_x.bias,
+            self.in_project_fx.weight, self.in_project_fx.bias, self.in_project_slice.weight,
+            self.in_project_slice.bias, self.temperature, self.qkv_project.weight, self.out_linear.weight,
+            self.out_linear.bias)
+
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        """(B, N, C) -> (B, N, C); replaces reference forward :501-558."""
+        """(B, N, C) -> (B, N, C); replaces reference forward :501-558.  With gradients enabled on tensors that
+        require them the differentiable path runs (stage-level kernels + backward kernels)."""
         self._validate(x)
+        needs_grad = self._needs_grad(x)
         x = self._prepare_input(x)
+        if needs_grad:
+            return self._forward_with_grad(x)
         return PF.layer_forward(x, self.kernel_params(x.dtype, x.device), self.layer_dims(x))
 
     def forward_block(self, x: torch.Tensor, residual: torch.Tensor, ln: nn.LayerNorm):

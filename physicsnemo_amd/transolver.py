@@ -1,12 +1,15 @@
 """Host-side mirror of the caller of the hot path: TransolverBlock and Transolver
 (physicsnemo/models/transolver/transolver.py:137-309 and :447-736, use_te=False, time_input=False, plus=False).
 
-The PhysicsAttention layer, its residual add and the LayerNorm that follows it run in the HIP library, and so does
+Inference (no gradients required): the PhysicsAttention layer, its residual add and the LayerNorm that follows it
+run in the HIP library, and so does
 the block MLP with its residual add and the LayerNorm the next block starts with whenever the fused kernel serves
 the shape (bf16, hidden 128 / 256, GELU); the remaining glue (preprocess MLP, the first LayerNorm, the output
 Linear, and every MLP the kernel does not serve) uses PyTorch-ROCm tensor ops.
 Module names, registration order and state_dict keys match the reference so its checkpoints load unchanged,
 including the legacy ``linear_pre`` / ``linear_post`` MLP keys (:92-97).
+Training (gradients required): the layer runs its differentiable path (stage-level kernels forward, the library's
+backward kernels backward); LayerNorms, MLPs and residual adds are differentiable PyTorch-ROCm tensor ops.
 """
 from __future__ import annotations
 
@@ -99,9 +102,17 @@ class TransolverBlock(nn.Module):
         hidden = mlp.layers[0].out_features
         return PF.mlp_supported(normed.dtype, normed.numel() // normed.shape[-1], normed.shape[-1], hidden)
 
+    def _needs_grad(self, fx: torch.Tensor) -> bool:
+        return torch.is_grad_enabled() and (fx.requires_grad or any(p.requires_grad for p in self.parameters()))
+
     def forward_chain(self, fx: torch.Tensor, normed_in: torch.Tensor | None, next_ln: nn.LayerNorm | None):
         """One block inside a chain of blocks: takes LayerNorm_1(fx) if the previous stage already produced it and
         returns (fx_out, next_ln(fx_out) or None).  Same arithmetic as `forward` (reference :300-303)."""
+        if self._needs_grad(fx):
+            # training: the layer's autograd path, LayerNorms / MLP as differentiable tensor ops (reference :300-303)
+            x_in = normed_in if normed_in is not None else self.ln_1(fx)
+            fx1 = self.Attn(x_in) + fx
+            return self.ln_mlp1(fx1) + fx1, None
         x_in = normed_in if normed_in is not None else self.ln_1(fx)
         # fx1 = Attn(ln_1(fx)) + fx and LayerNorm(fx1) come out of one fused library call (reference :300, :303)
         fx1, normed = self.Attn.forward_block(x_in, fx, self.ln_mlp1[0])
@@ -122,7 +133,7 @@ class TransolverBlock(nn.Module):
 
 
 class Transolver(nn.Module):
-    """Transolver model (reference :447-736) built on the HIP PhysicsAttention layer; forward only."""
+    """Transolver model (reference :447-736) built on the HIP PhysicsAttention layer."""
 
     def __init__(self, functional_dim: int, out_dim: int, embedding_dim: int | None = None, n_layers: int = 4,
                  n_hidden: int = 256, dropout: float = 0.0, n_head: int = 8, act: str = "gelu", mlp_ratio: int = 4,

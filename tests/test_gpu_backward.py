@@ -1,0 +1,134 @@
+"""Backward pass of the HIP layer against autograd over the fp32 oracle (the oracle's own gradient is pinned by
+finite differences in test_oracle_closed_forms.py).  Bars: fp32 gradients rtol 1e-4 with atol = 1e-4 * max|ref|
+per tensor; bf16 gradients rel-L2 <= 3e-2 against the fp32 reference gradients."""
+import pytest
+import torch
+
+from oracle import torch_oracle as to
+import physicsnemo_amd as pn
+from physicsnemo_amd import functional as PF
+from gpu_util import announce, assert_fp32_close, assert_rel_l2, make_pair
+
+pytestmark = pytest.mark.gpu
+
+
+def _grads(module, x, probe):
+    """Gradients of sum(module(x) * probe) w.r.t. x and every parameter."""
+    module.zero_grad(set_to_none=True)
+    x = x.clone().requires_grad_(True)
+    y = module(x)
+    (y.float() * probe.to(y.device)).sum().backward()
+    out = {"x": x.grad}
+    out.update({name: p.grad for name, p in module.named_parameters()})
+    return y, out
+
+
+CASES = [
+    ("irregular", dict(dim=32, heads=4, dim_head=8, slice_num=8), 2, 300, None, 3),
+    ("irregular", dict(dim=64, heads=2, dim_head=32, slice_num=64), 1, 1000, None, 3),
+    ("irregular", dict(dim=48, heads=3, dim_head=16, slice_num=20), 3, 77, None, 3),
+    ("structured2d", dict(dim=32, heads=4, dim_head=8, slice_num=8), 2, 63, (7, 9), 3),
+    ("structured2d", dict(dim=16, heads=2, dim_head=8, slice_num=8), 1, 30, (5, 6), 5),
+    ("structured3d", dict(dim=16, heads=2, dim_head=8, slice_num=8), 2, 60, (3, 4, 5), 3),
+]
+
+
+@pytest.mark.parametrize("variant,kw,B,N,grid,kernel", CASES)
+def test_fp32_layer_gradients(variant, kw, B, N, grid, kernel):
+    announce("fp32 backward", variant, kw, B, N, grid, kernel)
+    heads = kw["heads"]
+    temps = [0.3, 1.0, 2.5, 7.0][:heads] if heads <= 4 else None  # heads outside [0.5, 5] get zero temperature grad
+    ref, hip = make_pair(variant, kw["dim"], heads, kw["dim_head"], kw["slice_num"], spatial=grid, kernel=kernel,
+                         sharpen=2.0, temps=temps)
+    ref.train(), hip.train()
+    x = torch.randn(B, N, kw["dim"])
+    probe = torch.randn(B, N, kw["dim"])
+    y_ref, want = _grads(ref, x, probe)
+    y_hip, got = _grads(hip, x.cuda(), probe)
+    assert_fp32_close(y_hip, y_ref, "forward y (training path)")
+    assert set(got) == set(want)
+    for name in want:
+        assert got[name] is not None and got[name].shape == want[name].shape, name
+        assert_fp32_close(got[name], want[name], f"grad {name}", rtol=2e-4)
+    if temps is not None:
+        t = got["temperature"].flatten().cpu()
+        assert t[0] == 0.0 and (heads < 4 or t[3] == 0.0)
+        assert t[1] != 0.0
+
+
+def test_slice_attention_backward_stage():
+    announce("slice attention backward stage")
+    B, H, S, D = 2, 3, 24, 16
+    torch.manual_seed(3)
+    tok = torch.randn(B, H, S, D)
+    wqkv = torch.randn(3 * D, D) / D ** 0.5
+    d_out = torch.randn(B, H, S, D)
+    tok_r, w_r = tok.clone().requires_grad_(True), wqkv.clone().requires_grad_(True)
+    q, k, v = (tok_r @ w_r.t()).chunk(3, dim=-1)
+    out = torch.softmax(q @ k.transpose(-1, -2) / D ** 0.5, dim=-1) @ v
+    (out * d_out).sum().backward()
+    dims = PF.LayerDims(B, 100, H * D, H, D, S)
+    params = {"qkv_project_weight": wqkv.cuda().contiguous()}
+    d_tok, d_norm, d_w = PF.slice_attention_backward(tok.cuda(), None, d_out.cuda(), params, dims)
+    assert d_norm is None
+    assert_fp32_close(d_tok, tok_r.grad, "d slice_token")
+    assert_fp32_close(d_w, w_r.grad, "d qkv weight")
+
+
+def test_bf16_layer_gradients():
+    announce("bf16 backward (autocast)")
+    ref, hip = make_pair("irregular", 256, 8, 32, 64, sharpen=2.0)
+    ref.train(), hip.train()
+    torch.manual_seed(5)
+    x = torch.randn(2, 2048, 256)
+    probe = torch.randn(2, 2048, 256)
+    _, want = _grads(ref, x, probe)
+    hip.zero_grad(set_to_none=True)
+    xc = x.cuda().requires_grad_(True)
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        y = hip(xc)
+    assert y.dtype == torch.bfloat16
+    (y.float() * probe.cuda()).sum().backward()
+    got = {"x": xc.grad}
+    got.update({name: p.grad for name, p in hip.named_parameters()})
+    for name in want:
+        assert got[name].dtype == torch.float32 and torch.isfinite(got[name]).all(), name
+        assert_rel_l2(got[name], want[name], f"bf16 grad {name}", tol=3e-2)
+
+
+def test_model_training_step_matches_oracle():
+    announce("Transolver training step fp32")
+    torch.manual_seed(0)
+    kw = dict(functional_dim=2, out_dim=3, embedding_dim=3, n_layers=2, n_hidden=32, n_head=4, slice_num=8, mlp_ratio=2)
+    m = pn.Transolver(use_te=False, **kw).cuda().train()
+    ref = to.OracleTransolver(**kw).train()
+    ref.load_state_dict(m.state_dict())
+    fx, emb, target = torch.randn(2, 200, 2), torch.randn(2, 200, 3), torch.randn(2, 200, 3)
+    loss_ref = ((ref(fx, emb) - target) ** 2).mean()
+    loss_ref.backward()
+    loss = ((m(fx.cuda(), emb.cuda()) - target.cuda()) ** 2).mean()
+    loss.backward()
+    assert abs(float(loss.detach()) - float(loss_ref.detach())) <= 1e-4 * abs(float(loss_ref.detach()))
+    want = dict(ref.named_parameters())
+    for name, p in m.named_parameters():
+        assert p.grad is not None, name
+        assert_fp32_close(p.grad, want[name].grad, f"grad {name}", rtol=5e-4)
+    # the same optimiser step on both sides leads to the same new loss
+    torch.optim.SGD(m.parameters(), lr=0.01).step()
+    torch.optim.SGD(ref.parameters(), lr=0.01).step()
+    with torch.no_grad():
+        loss2 = float(((m(fx.cuda(), emb.cuda()) - target.cuda()) ** 2).mean())
+        loss2_ref = float(((ref(fx, emb) - target) ** 2).mean())
+    assert abs(loss2 - loss2_ref) <= 1e-4 * abs(loss2_ref)
+    assert loss2_ref >= float(loss_ref) or loss2 < float(loss.detach())
+
+
+def test_gradients_reach_the_input_only_when_asked():
+    announce("needs_input_grad handling")
+    _, hip = make_pair("irregular", 32, 4, 8, 8)
+    for p in hip.parameters():
+        p.requires_grad_(False)
+    x = torch.randn(1, 50, 32, device="cuda", requires_grad=True)
+    hip(x).sum().backward()
+    assert x.grad is not None and torch.isfinite(x.grad).all()
+    assert all(p.grad is None for p in hip.parameters())

@@ -134,6 +134,29 @@ def test_conv3d_special_cases_pin_token_order_and_orientation():
         no.conv3d_projection(x.numpy(), w.numpy(), zero.numpy(), gh, gw, gd).reshape(gh, gw, gd), vol.numpy())
 
 
+@pytest.mark.parametrize("variant", ["irregular", "structured2d"])
+def test_oracle_gradient_matches_finite_differences(variant):
+    """The GPU backward tests compare against autograd over the torch oracle; here that gradient is pinned by
+    central finite differences in float64 (torch.autograd.gradcheck), w.r.t. the input and every parameter."""
+    torch.manual_seed(11)
+    if variant == "irregular":
+        m = to.OraclePhysicsAttentionIrregularMesh(6, heads=2, dim_head=3, slice_num=4).double()
+        n = 7
+    else:
+        m = to.OraclePhysicsAttentionStructuredMesh2D(6, (3, 4), heads=2, dim_head=3, slice_num=4, kernel=3).double()
+        n = 12
+    with torch.no_grad():
+        m.temperature.copy_(torch.tensor([0.8, 2.0], dtype=torch.float64).view(1, 1, 2, 1))
+    names = [k for k, _ in m.named_parameters()]
+    params = [p.detach().clone().requires_grad_(True) for _, p in m.named_parameters()]
+    x = torch.randn(2, n, 6, dtype=torch.float64, requires_grad=True)
+
+    def fn(x, *ps):
+        return torch.func.functional_call(m, dict(zip(names, ps)), (x,))
+
+    assert torch.autograd.gradcheck(fn, (x, *params), eps=1e-6, atol=1e-6, rtol=1e-5)
+
+
 def test_softmax_rows_and_temperature_clamp():
     B, N, H, D, S = 2, 11, 3, 4, 5
     logits = torch.randn(B, N, H, S, dtype=torch.float64) * 4
