@@ -137,6 +137,39 @@ def time_block_mlp(rows, C, hidden, reps=10):
             "hbm_frac": round(4 * rows * C * 2 / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
 
 
+def time_training_step(points, C, S, reps=3):
+    """Forward + backward of one layer under bf16 autocast at the layer workload's size: the differentiable path
+    (stage-level kernels forward, backward kernels + GEMM-library weight gradients backward)."""
+    import torch
+
+    import physicsnemo_amd as pn
+
+    torch.manual_seed(0)
+    layer = pn.PhysicsAttentionIrregularMesh(C, heads=C // 32, dim_head=32, slice_num=S, use_te=False).cuda().train()
+    x = torch.randn(1, points, C, device="cuda").bfloat16().requires_grad_(True)
+    dy = torch.ones(1, points, C, device="cuda", dtype=torch.bfloat16)
+
+    def step():
+        layer.zero_grad(set_to_none=True)
+        x.grad = None
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            y = layer(x)
+        y.backward(dy)
+
+    for _ in range(2):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / reps * 1e3
+    assert torch.isfinite(x.grad[:, :1024].float()).all()
+    return {"workload": f"layer forward + backward, {points} points, C={C}, S={S}, bf16 autocast",
+            "ms_per_step": round(ms, 3), "mpoints_per_s": round(points / (ms * 1e-3) / 1e6, 2),
+            "kernels": "general (fp32 FMA) stage and backward kernels; weight gradients via the GEMM library"}
+
+
 def time_full_model(name, B, N, functional_dim, embedding_dim, slice_num, n_layers, steps=5, warmup=2):
     """Forward of a whole Transolver (bf16 autocast, random-init weights, synthetic N(0,1) inputs) -> Mpoints/s.
 
@@ -328,6 +361,7 @@ def main():
     }
     if not args.no_models:
         out["block_mlp"] = time_block_mlp(1 << 20, 256, 1024)
+        out["training_step"] = time_training_step(N, C, S)
         out["full_model"] = [
             time_structured_model(),
             time_full_model("cfg2: Transolver irregular 2D, 8 layers", 8, 32768, 3, 2, 64, 8),

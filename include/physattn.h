@@ -107,7 +107,8 @@ int pa_query_path(int dtype, const pa_shape *shape);
 /* ---- stage-level entry points (natural layouts; general kernels) ------------------------------ */
 
 /* Stage (a1): input projections, replaces project_input_onto_slices (PA.py:629-660 irregular,
- * :744-783 structured 2D) -> x_mid, fx_mid as (B, N, H*D) with channel c = h*D + d. */
+ * :744-783 structured 2D) -> x_mid, fx_mid as (B, N, H*D) with channel c = h*D + d.  fx_mid == NULL: only x_mid is
+ * computed and in_project_fx_* are not read (the single projection of plus=True, PA.py:652). */
 int pa_project_inputs(int dtype, const pa_shape *shape, const pa_params *p, const void *x,
                       void *x_mid, void *fx_mid, void *stream);
 
@@ -115,6 +116,24 @@ int pa_project_inputs(int dtype, const pa_shape *shape, const pa_params *p, cons
  * softmax half of _compute_slices_from_projections (PA.py:172-181): w (B, N, H, S), rows sum to 1. */
 int pa_slice_softmax(int dtype, const pa_shape *shape, const pa_params *p, const void *x_mid, void *w,
                      void *stream);
+
+/* Transolver++ (plus=True, PA.py:166-170, :287-295, :530-532): one projection (fx_mid = x_mid: call
+ * pa_project_inputs with in_project_fx_* and fx_mid NULL and pass x_mid as fx_mid to the later stages), a learned
+ * per-point temperature  max(temperature[h] + proj_temperature(x_mid[n,h,:]), 0.01)  with
+ * proj_temperature = Linear(D,S) -> GELU -> Linear(S,1) -> GELU, and Gumbel noise added to the slice logits before
+ * the division (physicsnemo/nn/module/gumbel_softmax.py:49-57).  All four tensors float32. */
+typedef struct pa_plus_params {
+  const float *proj_temperature_0_weight; /* (S, D) */
+  const float *proj_temperature_0_bias;   /* (S) */
+  const float *proj_temperature_2_weight; /* (1, S) */
+  const float *proj_temperature_2_bias;   /* (1) */
+} pa_plus_params;
+
+/* Stage (a2) of Transolver++: replaces in_project_slice (PA.py:537) and the plus branch of
+ * _compute_slices_from_projections (PA.py:166-170).  `uniform` (B,N,H,S), activation dtype: the U[0,1) samples the
+ * reference draws with torch.rand_like(logits); the kernel forms the noise -log(-log(u + 1e-8) + 1e-8) itself. */
+int pa_slice_softmax_plus(int dtype, const pa_shape *shape, const pa_params *p, const pa_plus_params *plus,
+                          const void *x_mid, const void *uniform, void *w, void *stream);
 
 /* Stage (b): slice-token aggregation, replaces PA.py:185-203.
  *   partials: float32 scratch of pa_reduce_partial_count(shape) * B*H*S*(D+1) elements (per-chunk sums

@@ -80,12 +80,19 @@ def conv3d_projection(x, weight, bias, grid_h, grid_w, grid_d):
     return out.reshape(b, n, o) + _f64(bias)
 
 
-def layer_forward(p, x, heads, dim_head, variant="irregular", spatial_shape=None):
+def layer_forward(p, x, heads, dim_head, variant="irregular", spatial_shape=None, noise_u=None):
     """All intermediates of one layer in float64 (steps 1-9 below follow physics_attention.py:529-558).
 
     p: in_project_x.{weight,bias}, in_project_fx.{weight,bias}, in_project_slice.{weight,bias},
        temperature, qkv_project.weight, out_linear.{weight,bias}
+    Transolver++ (plus=True) is selected by the absence of in_project_fx.weight: then fx_mid = x_mid (:530-532),
+    p also holds proj_temperature.{0,2}.{weight,bias} and noise_u (B, N, H, S) holds the uniform samples behind
+    the Gumbel noise (gumbel_softmax.py:50).
     """
+    plus = "in_project_fx.weight" not in p
+    if plus:
+        p = dict(p)
+        p["in_project_fx.weight"], p["in_project_fx.bias"] = p["in_project_x.weight"], p["in_project_x.bias"]
     x = _f64(x)
     B, N, C = x.shape
     H, D = heads, dim_head
@@ -108,8 +115,19 @@ def layer_forward(p, x, heads, dim_head, variant="irregular", spatial_shape=None
     S = ws.shape[0]
     logits = np.einsum("bnhd,sd->bnhs", xm, ws) + bs
     # 3. clamp temperature to [0.5, 5], softmax over S (:173-178)
-    t = np.clip(_f64(p["temperature"]).reshape(H), 0.5, 5.0)
-    z = logits / t[None, None, :, None]
+    if plus:
+        # per-point temperature, clamped from below only (:168-169); noise added before the division
+        # (gumbel_softmax.py:50-55)
+        h1 = gelu_erf(np.einsum("bnhd,sd->bnhs", xm, _f64(p["proj_temperature.0.weight"]))
+                      + _f64(p["proj_temperature.0.bias"]))
+        h2 = gelu_erf(np.einsum("bnhs,os->bnho", h1, _f64(p["proj_temperature.2.weight"]))
+                      + _f64(p["proj_temperature.2.bias"]))
+        t = np.maximum(_f64(p["temperature"]).reshape(1, 1, H, 1) + h2, 0.01)
+        u = _f64(noise_u)
+        z = (logits + -np.log(-np.log(u + 1e-8) + 1e-8)) / t
+    else:
+        t = np.clip(_f64(p["temperature"]).reshape(H), 0.5, 5.0)
+        z = logits / t[None, None, :, None]
     z = z - z.max(axis=-1, keepdims=True)
     e = np.exp(z)
     w = e / e.sum(axis=-1, keepdims=True)

@@ -104,6 +104,29 @@ def slice_weights_and_tokens(logits, fx_mid, temperature):
     return w, tok, norm
 
 
+def gumbel_from_uniform(u):
+    """Gumbel(0, 1) noise from uniform samples as the reference forms it
+    (physicsnemo/nn/module/gumbel_softmax.py:50-51): -log(-log(u + 1e-8) + 1e-8)."""
+    return -torch.log(-torch.log(u + 1e-8) + 1e-8)
+
+
+def slice_weights_and_tokens_plus(logits, x_mid, temperature, proj_temperature, u):
+    """Transolver++ branch (physics_attention.py:166-170 + gumbel_softmax.py:49-57): per-point temperature
+    temperature_h + proj_temperature(x_mid[n, h, :]) clamped from below at 0.01, Gumbel noise added to the logits
+    BEFORE the division, then softmax; aggregation as in the plain branch (:185-206) with fx_mid = x_mid (:530-532).
+
+    ``u`` holds the uniform samples the reference would draw with ``torch.rand_like(logits)``.
+    """
+    temp = temperature + proj_temperature(x_mid)  # (1,1,H,1) + (B,N,H,1)
+    temp = torch.clamp(temp, min=0.01).to(logits.dtype)
+    w = F.softmax((logits + gumbel_from_uniform(u)) / temp, dim=-1)
+    w = w.to(logits.dtype)
+    norm = w.sum(1) + SLICE_NORM_EPS
+    normed = w / norm[:, None, :, :]
+    tok = torch.matmul(normed.permute(0, 2, 3, 1), x_mid.permute(0, 2, 1, 3))
+    return w, tok, norm, temp
+
+
 def slice_attention(tok, w_qkv, dim_head):
     """Self-attention among the S slice tokens of each (batch, head) (physics_attention.py:448-463).
 
@@ -132,12 +155,16 @@ class _AttentionCore(nn.Module):
     softmax, dropout, in_project_slice (+orthogonal_), qkv_project, out_linear, out_dropout.
     """
 
-    def __init__(self, dim, heads, dim_head, dropout, slice_num):
+    def __init__(self, dim, heads, dim_head, dropout, slice_num, plus=False):
         super().__init__()
         self.dim, self.heads, self.dim_head, self.slice_num = dim, heads, dim_head, slice_num
+        self.plus = plus
         self.softmax = nn.Softmax(dim=-1)
         self.dropout = nn.Dropout(dropout)
         self.temperature = nn.Parameter(torch.full((1, 1, heads, 1), 0.5))
+        if plus:  # physics_attention.py:287-295
+            self.proj_temperature = nn.Sequential(nn.Linear(dim_head, slice_num), nn.GELU(),
+                                                  nn.Linear(slice_num, 1), nn.GELU())
         self.in_project_slice = nn.Linear(dim_head, slice_num)
         nn.init.orthogonal_(self.in_project_slice.weight)
         self.qkv_project = nn.Linear(dim_head, 3 * dim_head, bias=False)
@@ -147,11 +174,16 @@ class _AttentionCore(nn.Module):
     def _project(self, x):  # pragma: no cover - abstract
         raise NotImplementedError
 
-    def stages(self, x):
-        """Forward returning every intermediate (used by the parity tests)."""
+    def stages(self, x, noise_u=None):
+        """Forward returning every intermediate (used by the parity tests).  ``noise_u`` (plus=True only): the
+        uniform samples behind the Gumbel noise; drawn with ``torch.rand_like`` when not given, as the reference does."""
         x_mid, fx_mid = self._project(x)
         logits = slice_logits(x_mid, self.in_project_slice.weight, self.in_project_slice.bias)
-        w, tok, norm = slice_weights_and_tokens(logits, fx_mid, self.temperature)
+        if self.plus:
+            u = torch.rand_like(logits) if noise_u is None else noise_u
+            w, tok, norm, _ = slice_weights_and_tokens_plus(logits, x_mid, self.temperature, self.proj_temperature, u)
+        else:
+            w, tok, norm = slice_weights_and_tokens(logits, fx_mid, self.temperature)
         tok_out = slice_attention(tok, self.qkv_project.weight, self.dim_head)
         y = deslice_and_project(w, tok_out, self.out_linear.weight, self.out_linear.bias)
         return dict(x_mid=x_mid, fx_mid=fx_mid, logits=logits, w=w, tok=tok, norm=norm,
@@ -167,32 +199,44 @@ class _AttentionCore(nn.Module):
             raise ValueError(f"Expected input feature dimension {self.dim}, got {x.shape[-1]}")
         return self.stages(x)["y"]
 
+    def forward_with_noise(self, x, noise_u):
+        return self.stages(x, noise_u)["y"]
+
 
 class OraclePhysicsAttentionIrregularMesh(_AttentionCore):
-    """physics_attention.py:561-660 with use_te=False, plus=False."""
+    """physics_attention.py:561-660 with use_te=False; plus=True drops in_project_fx (:622-627)."""
 
-    def __init__(self, dim, heads=8, dim_head=64, dropout=0.0, slice_num=64):
-        super().__init__(dim, heads, dim_head, dropout, slice_num)
+    def __init__(self, dim, heads=8, dim_head=64, dropout=0.0, slice_num=64, plus=False):
+        super().__init__(dim, heads, dim_head, dropout, slice_num, plus)
         self.in_project_x = nn.Linear(dim, heads * dim_head)
-        self.in_project_fx = nn.Linear(dim, heads * dim_head)
+        if not plus:
+            self.in_project_fx = nn.Linear(dim, heads * dim_head)
 
     def _project(self, x):
+        if self.plus:
+            x_mid = split_heads(F.linear(x, self.in_project_x.weight, self.in_project_x.bias), self.heads, self.dim_head)
+            return x_mid, x_mid
         return project_linear(x, self.in_project_x.weight, self.in_project_x.bias,
                               self.in_project_fx.weight, self.in_project_fx.bias,
                               self.heads, self.dim_head)
 
 
 class OraclePhysicsAttentionStructuredMesh2D(_AttentionCore):
-    """physics_attention.py:663-783 with use_te=False, plus=False."""
+    """physics_attention.py:663-783 with use_te=False; plus=True drops in_project_fx (:741-742)."""
 
-    def __init__(self, dim, spatial_shape, heads=8, dim_head=64, dropout=0.0, slice_num=64, kernel=3):
-        super().__init__(dim, heads, dim_head, dropout, slice_num)
+    def __init__(self, dim, spatial_shape, heads=8, dim_head=64, dropout=0.0, slice_num=64, kernel=3, plus=False):
+        super().__init__(dim, heads, dim_head, dropout, slice_num, plus)
         self.H, self.W = spatial_shape[0], spatial_shape[1]
         inner = heads * dim_head
         self.in_project_x = nn.Conv2d(dim, inner, kernel, 1, kernel // 2)
-        self.in_project_fx = nn.Conv2d(dim, inner, kernel, 1, kernel // 2)
+        if not plus:
+            self.in_project_fx = nn.Conv2d(dim, inner, kernel, 1, kernel // 2)
 
     def _project(self, x):
+        if self.plus:
+            x_mid, _ = project_conv2d(x, self.in_project_x.weight, self.in_project_x.bias, self.in_project_x.weight,
+                                      self.in_project_x.bias, self.heads, self.dim_head, self.H, self.W)
+            return x_mid, x_mid
         return project_conv2d(x, self.in_project_x.weight, self.in_project_x.bias,
                               self.in_project_fx.weight, self.in_project_fx.bias,
                               self.heads, self.dim_head, self.H, self.W)

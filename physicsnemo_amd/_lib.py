@@ -22,7 +22,7 @@ EXPORTED = [
     "pa_mfma_project_softmax", "pa_mfma_slice_reduce", "pa_mfma_project_softmax_reduce", "pa_mfma_partial_groups",
      "pa_mfma_combine_attention", "pa_mfma_deslice_project", "pa_mlp_query", "pa_mlp_workspace_bytes", "pa_mlp_forward",
     "pa_rows_gemm", "pa_slice_weighted_sum", "pa_backward_query", "pa_backward_point_tiles",
-    "pa_slice_attention_backward", "pa_slice_softmax_backward",
+    "pa_slice_attention_backward", "pa_slice_softmax_backward", "pa_slice_softmax_plus",
 ]
 
 PA_BUF_BLOB, PA_BUF_FX_PACK, PA_BUF_W_PACK, PA_BUF_PARTIALS, PA_BUF_TOKP = range(5)
@@ -41,6 +41,11 @@ class PaParams(Structure):
 
 class PaMlpParams(Structure):
     _fields_ = [(n, c_void_p) for n in ("w1", "b1", "w2", "b2")]
+
+
+class PaPlusParams(Structure):
+    _fields_ = [(n, c_void_p) for n in ("proj_temperature_0_weight", "proj_temperature_0_bias",
+                                        "proj_temperature_2_weight", "proj_temperature_2_bias")]
 
 
 class PaBlockTail(Structure):
@@ -119,6 +124,8 @@ def load() -> ctypes.CDLL:
     lib.pa_slice_attention_backward.argtypes = [ps, pp] + [c_void_p] * 8
     lib.pa_slice_softmax_backward.restype = c_int
     lib.pa_slice_softmax_backward.argtypes = [c_int, ps, pp] + [c_void_p] * 11
+    lib.pa_slice_softmax_plus.restype = c_int
+    lib.pa_slice_softmax_plus.argtypes = [c_int, ps, pp, POINTER(PaPlusParams)] + [c_void_p] * 4
     _lib = lib
     return lib
 

@@ -174,10 +174,27 @@ int pa_project_inputs(int dtype, const pa_shape *shape, const pa_params *p, cons
   int rc = check_shape(dtype, shape);
   if (rc) return rc;
   if (dtype == PA_BF16_W8) return PA_ERR_UNSUPPORTED;  // fp8 weights: whole-layer entry point only
-  if ((rc = check_params(p))) return rc;
-  if (!x || !x_mid || !fx_mid) return PA_ERR_NULL;
-  if (!aligned16(x) || !aligned16(x_mid) || !aligned16(fx_mid)) return PA_ERR_ALIGN;
+  if (!p || !p->in_project_x_weight || !p->in_project_x_bias) return PA_ERR_NULL;
+  if (fx_mid && (!p->in_project_fx_weight || !p->in_project_fx_bias)) return PA_ERR_NULL;
+  if (!x || !x_mid) return PA_ERR_NULL;
+  if (!aligned16(x) || !aligned16(x_mid) || !aligned16(fx_mid) || !aligned16(p->in_project_x_weight) ||
+      !aligned16(p->in_project_fx_weight))
+    return PA_ERR_ALIGN;
   return pa::general::project_inputs(dtype, *shape, *p, x, x_mid, fx_mid, static_cast<hipStream_t>(stream));
+}
+
+int pa_slice_softmax_plus(int dtype, const pa_shape *shape, const pa_params *p, const pa_plus_params *plus,
+                          const void *x_mid, const void *uniform, void *w, void *stream) {
+  int rc = check_shape(dtype, shape);
+  if (rc) return rc;
+  if (dtype == PA_BF16_W8) return PA_ERR_UNSUPPORTED;
+  if (!p || !p->in_project_slice_weight || !p->in_project_slice_bias || !p->temperature) return PA_ERR_NULL;
+  if (!plus || !plus->proj_temperature_0_weight || !plus->proj_temperature_0_bias || !plus->proj_temperature_2_weight ||
+      !plus->proj_temperature_2_bias)
+    return PA_ERR_NULL;
+  if (!x_mid || !uniform || !w) return PA_ERR_NULL;
+  if (!aligned16(x_mid) || !aligned16(uniform) || !aligned16(w)) return PA_ERR_ALIGN;
+  return pa::general::slice_softmax_plus(dtype, *shape, *p, *plus, x_mid, uniform, w, static_cast<hipStream_t>(stream));
 }
 
 int pa_slice_softmax(int dtype, const pa_shape *shape, const pa_params *p, const void *x_mid, void *w, void *stream) {

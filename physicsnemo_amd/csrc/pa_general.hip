@@ -186,6 +186,89 @@ __global__ __launch_bounds__(256) void slice_softmax_kernel(const T *__restrict_
 }
 
 // ------------------------------------------------------------------------------------------------
+// slice_softmax_plus_kernel: the Transolver++ form of slice_softmax_kernel (PA.py:166-170, gumbel_softmax.py:49-57).
+//   temp[r,h]  = max(temperature[h] + gelu(b2 + sum_s w2[s] gelu(b1[s] + x_mid[r,h,:] . w1[s,:])), 0.01)
+//   w[r,h,:]   = softmax_s((logits[r,h,s] - log(-log(u[r,h,s] + 1e-8) + 1e-8)) / temp[r,h])
+// `uniform` holds the caller's U[0,1) samples in the activation type (what torch.rand_like(logits) draws).
+// ------------------------------------------------------------------------------------------------
+__device__ __forceinline__ float gelu_erf(float v) { return 0.5f * v * (1.f + erff(v * 0.70710678118654752f)); }
+
+template <typename T>
+__global__ __launch_bounds__(256) void slice_softmax_plus_kernel(
+    const T *__restrict__ x_mid, const T *__restrict__ uniform, const float *__restrict__ w_slice,
+    const float *__restrict__ b_slice, const float *__restrict__ temperature, const float *__restrict__ pt_w1,
+    const float *__restrict__ pt_b1, const float *__restrict__ pt_w2, const float *__restrict__ pt_b2,
+    T *__restrict__ w_out, int64_t M, int H, int D, int S, int R) {
+  extern __shared__ float lds[];
+  float *xs = lds;                       // R * H * (D+1)
+  float *wsl = xs + R * H * (D + 1);     // S * D
+  float *bsl = wsl + S * D;              // S
+  float *w1 = bsl + S;                   // S * D
+  float *b1 = w1 + S * D;                // S
+  float *w2 = b1 + S;                    // S
+  float *lg = w2 + S;                    // R * H * (S+1)
+  const int t = threadIdx.x;
+  const int64_t m0 = (int64_t)blockIdx.x * R;
+  const int rows = (int)min((int64_t)R, M - m0);
+  const int HD = H * D, HS = H * S;
+  for (int i = t; i < rows * HD; i += 256) {
+    const int r = i / HD, c = i - r * HD;
+    const int h = c / D, d = c - h * D;
+    xs[(r * H + h) * (D + 1) + d] = load_as_f32(x_mid + (m0 + r) * HD + c);
+  }
+  for (int i = t; i < S * D; i += 256) {
+    wsl[i] = w_slice[i];
+    w1[i] = pt_w1[i];
+  }
+  for (int i = t; i < S; i += 256) {
+    bsl[i] = b_slice[i];
+    b1[i] = pt_b1[i];
+    w2[i] = pt_w2[i];
+  }
+  for (int i = t; i < rows * HS; i += 256) {
+    const int pair = i / S, s = i - pair * S;
+    lg[pair * (S + 1) + s] = load_as_f32(uniform + m0 * HS + i);
+  }
+  __syncthreads();
+  for (int pair = t; pair < rows * H; pair += 256) {
+    const int h = pair % H;
+    const float *xr = xs + pair * (D + 1);
+    float *lrow = lg + pair * (S + 1);
+    float tacc = pt_b2[0];
+    for (int s = 0; s < S; ++s) {
+      float acc = b1[s];
+      const float *wr = w1 + s * D;
+      for (int d = 0; d < D; ++d) acc = fmaf(xr[d], wr[d], acc);
+      tacc = fmaf(w2[s], gelu_erf(acc), tacc);
+    }
+    const float temp = round_to(w_out, fmaxf(temperature[h] + gelu_erf(tacc), 0.01f));
+    float mx = -INFINITY;
+    for (int s = 0; s < S; ++s) {
+      float acc = 0.f;
+      const float *wr = wsl + s * D;
+      for (int d = 0; d < D; ++d) acc = fmaf(xr[d], wr[d], acc);
+      const float noise = -logf(-logf(lrow[s] + 1e-8f) + 1e-8f);
+      const float z = (round_to(w_out, acc + bsl[s]) + noise) / temp;
+      lrow[s] = z;
+      mx = fmaxf(mx, z);
+    }
+    float sum = 0.f;
+    for (int s = 0; s < S; ++s) {
+      const float e = expf(lrow[s] - mx);
+      lrow[s] = e;
+      sum += e;
+    }
+    const float inv = 1.f / sum;
+    for (int s = 0; s < S; ++s) lrow[s] *= inv;
+  }
+  __syncthreads();
+  for (int i = t; i < rows * HS; i += 256) {
+    const int pair = i / S, s = i - pair * S;
+    store_from_f32(w_out + m0 * HS + i, lg[pair * (S + 1) + s]);
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
 // slice_partial_kernel: grid (G chunks, B*H, output slabs).  For its chunk of points of one (b, h):
 //   partial[s, d] = sum_n w[n, s] * fx_mid[n, d]   (d < D),   partial[s, D] = sum_n w[n, s]
 // Each thread owns up to 16 outputs of a 4096-output slab and walks the chunk 32 points at a time
@@ -515,7 +598,8 @@ int project_inputs(int dtype, const pa_shape &s, const pa_params &p, const void 
   a.ks = (int)s.conv_k;
   a.gd = (int)s.grid_d;
   a.K = s.conv_k > 0 ? (int)(s.conv_k * s.conv_k * (s.grid_d > 0 ? s.conv_k : 1) * s.C) : (int)s.C;
-  return dtype == PA_F32 ? launch_gemm<float, float>(a, 2, st) : launch_gemm<bf16, bf16>(a, 2, st);
+  const int nsets = fx_mid ? 2 : 1;  // Transolver++ has a single projection
+  return dtype == PA_F32 ? launch_gemm<float, float>(a, nsets, st) : launch_gemm<bf16, bf16>(a, nsets, st);
 }
 
 // out[m, o] = bias[o] + sum_k A(m, k) weight[o, k] for any (c_in, c_out): a Linear over the rows when grid.conv_k == 0,
@@ -572,6 +656,32 @@ static int slice_softmax_t(const pa_shape &s, const pa_params &p, const void *x_
 
 int slice_softmax(int dtype, const pa_shape &s, const pa_params &p, const void *x_mid, void *w, hipStream_t st) {
   return dtype == PA_F32 ? slice_softmax_t<float>(s, p, x_mid, w, st) : slice_softmax_t<bf16>(s, p, x_mid, w, st);
+}
+
+template <typename T>
+static int slice_softmax_plus_t(const pa_shape &s, const pa_params &p, const pa_plus_params &pp, const void *x_mid,
+                                const void *uniform, void *w, hipStream_t st) {
+  const int H = (int)s.H, D = (int)s.D, S = (int)s.S;
+  const size_t fixed = (size_t)(2 * S * D + 3 * S) * 4;
+  const size_t per_row = (size_t)(H * (D + 1) + H * (S + 1)) * 4;
+  if (fixed + per_row > 60 * 1024) return PA_ERR_UNSUPPORTED;
+  int R = (int)((60 * 1024 - fixed) / per_row);
+  if (R > 8) R = 8;
+  const size_t lds = fixed + per_row * R;
+  int rc = allow_dynamic_lds(slice_softmax_plus_kernel<T>, lds);
+  if (rc) return rc;
+  const int64_t M = s.B * s.N;
+  hipLaunchKernelGGL((slice_softmax_plus_kernel<T>), dim3((unsigned)((M + R - 1) / R)), dim3(256), lds, st,
+                     static_cast<const T *>(x_mid), static_cast<const T *>(uniform), p.in_project_slice_weight,
+                     p.in_project_slice_bias, p.temperature, pp.proj_temperature_0_weight, pp.proj_temperature_0_bias,
+                     pp.proj_temperature_2_weight, pp.proj_temperature_2_bias, static_cast<T *>(w), M, H, D, S, R);
+  return launch_status();
+}
+
+int slice_softmax_plus(int dtype, const pa_shape &s, const pa_params &p, const pa_plus_params &pp, const void *x_mid,
+                       const void *uniform, void *w, hipStream_t st) {
+  return dtype == PA_F32 ? slice_softmax_plus_t<float>(s, p, pp, x_mid, uniform, w, st)
+                         : slice_softmax_plus_t<bf16>(s, p, pp, x_mid, uniform, w, st);
 }
 
 // Number of point chunks of the first reduction pass: enough workgroups to fill 256 CUs several times

@@ -19,6 +19,8 @@ int out_linear(int dtype, const pa_shape &s, const pa_params &p, const void *out
 int rows_gemm(int dtype, const pa_shape &grid, int64_t c_in, int64_t c_out, const void *in, const void *weight,
               const float *bias, void *out, hipStream_t st);
 int slice_softmax(int dtype, const pa_shape &s, const pa_params &p, const void *x_mid, void *w, hipStream_t st);
+int slice_softmax_plus(int dtype, const pa_shape &s, const pa_params &p, const pa_plus_params &pp, const void *x_mid,
+                       const void *uniform, void *w, hipStream_t st);
 int64_t partial_count(const pa_shape &s);
 size_t combine_attn_lds_bytes(const pa_shape &s);
 int slice_partial(int dtype, const pa_shape &s, const void *w, const void *fx_mid, float *partials, hipStream_t st);

@@ -54,14 +54,29 @@ def query_path(dtype: torch.dtype, dims: LayerDims) -> int:
 
 
 def project_inputs(x, params, dims: LayerDims):
+    """(x_mid, fx_mid); Transolver++ parameter sets (no in_project_fx) share one projection: fx_mid is x_mid."""
     _need_cuda(x)
     lib = _lib.load()
     x_mid = torch.empty(dims.B, dims.N, dims.H * dims.D, dtype=x.dtype, device=x.device)
-    fx_mid = torch.empty_like(x_mid)
+    fx_mid = torch.empty_like(x_mid) if params.get("in_project_fx_weight") is not None else None
     _lib.check(lib.pa_project_inputs(_lib.dtype_code(x.dtype), byref(dims.c()), byref(_c_params(params)),
-                                     x.data_ptr(), x_mid.data_ptr(), fx_mid.data_ptr(),
+                                     x.data_ptr(), x_mid.data_ptr(), _lib.ptr(fx_mid),
                                      _lib.current_stream_ptr(x.device)), "pa_project_inputs")
-    return x_mid, fx_mid
+    return x_mid, (x_mid if fx_mid is None else fx_mid)
+
+
+def slice_softmax_plus(x_mid, uniform, params, dims: LayerDims):
+    """Transolver++ slice weights: learned per-point temperature and Gumbel noise from the uniform samples given."""
+    _need_cuda(x_mid, uniform)
+    if uniform.dtype != x_mid.dtype or uniform.shape != (dims.B, dims.N, dims.H, dims.S):
+        raise ValueError("uniform samples must have the activation dtype and shape (B, N, H, S)")
+    w = torch.empty(dims.B, dims.N, dims.H, dims.S, dtype=x_mid.dtype, device=x_mid.device)
+    plus = _lib.PaPlusParams(*[_lib.ptr(params[k]) for k, _ in _lib.PaPlusParams._fields_])
+    _lib.check(_lib.load().pa_slice_softmax_plus(_lib.dtype_code(x_mid.dtype), byref(dims.c()),
+                                                 byref(_c_params(params)), byref(plus), x_mid.data_ptr(),
+                                                 uniform.data_ptr(), w.data_ptr(),
+                                                 _lib.current_stream_ptr(x_mid.device)), "pa_slice_softmax_plus")
+    return w
 
 
 def slice_softmax(x_mid, params, dims: LayerDims):

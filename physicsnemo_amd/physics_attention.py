@@ -8,7 +8,7 @@ reference classes in physicsnemo/nn/module/physics_attention.py:
   PhysicsAttentionStructuredMesh3D:786-907
 so that a reference ``state_dict`` loads unchanged and seeded construction consumes the RNG identically.
 
-Scope: ``plus=False``.  ``use_te`` is accepted for signature compatibility and ignored: the HIP kernels are the
+``plus=True`` (Transolver++) runs through the stage-level kernels, forward only.  ``use_te`` is accepted for signature compatibility and ignored: the HIP kernels are the
 only backend and there is no CPU path.  Under ``torch.no_grad()`` the fused inference kernels run; with gradients
 enabled on tensors that require them the stage-level kernels run and the backward pass is served by the library's
 backward kernels (see ``autograd.py``).
@@ -30,8 +30,6 @@ class PhysicsAttentionBase(nn.Module):
 
     def __init__(self, dim: int, heads: int, dim_head: int, dropout: float, slice_num: int, use_te: bool, plus: bool):
         super().__init__()
-        if plus:
-            raise NotImplementedError("Transolver++ (plus=True) is not served by the HIP kernels")
         self.dim = dim
         self.dim_head = dim_head
         self.heads = heads
@@ -44,6 +42,9 @@ class PhysicsAttentionBase(nn.Module):
         self.softmax = nn.Softmax(dim=-1)
         self.dropout = nn.Dropout(dropout)
         self.temperature = nn.Parameter(torch.ones([1, 1, heads, 1]) * 0.5)
+        if plus:  # Transolver++: learned per-point temperature offset (reference :287-295)
+            self.proj_temperature = nn.Sequential(nn.Linear(dim_head, slice_num), nn.GELU(),
+                                                  nn.Linear(slice_num, 1), nn.GELU())
         self.in_project_slice = nn.Linear(dim_head, slice_num)
         torch.nn.init.orthogonal_(self.in_project_slice.weight)
         self.qkv_project = nn.Linear(dim_head, 3 * dim_head, bias=False)
@@ -56,8 +57,8 @@ class PhysicsAttentionBase(nn.Module):
         """Serve bf16 inputs with the three large weights quantised to fp8-e4m3, one scale per output channel
         (scale = max|row| / 448).  The kernels expand them to bf16 MFMA operands; activations stay bf16.
         Irregular-mesh variant only.  No counterpart in the reference."""
-        if enabled and self._conv_geometry()[2] != 0:
-            raise NotImplementedError("fp8 weights are served for the irregular-mesh variant only")
+        if enabled and (self._conv_geometry()[2] != 0 or self.plus):
+            raise NotImplementedError("fp8 weights are served for the irregular-mesh variant with plus=False only")
         self.fp8_weights = bool(enabled)
         self._kernel_param_cache = {}
         return self
@@ -77,8 +78,16 @@ class PhysicsAttentionBase(nn.Module):
         named = [
             ("in_project_x_weight", self.in_project_x.weight, True),
             ("in_project_x_bias", self.in_project_x.bias, False),
-            ("in_project_fx_weight", self.in_project_fx.weight, True),
-            ("in_project_fx_bias", self.in_project_fx.bias, False),
+        ]
+        if self.plus:
+            named += [("proj_temperature_0_weight", self.proj_temperature[0].weight, False),
+                      ("proj_temperature_0_bias", self.proj_temperature[0].bias, False),
+                      ("proj_temperature_2_weight", self.proj_temperature[2].weight, False),
+                      ("proj_temperature_2_bias", self.proj_temperature[2].bias, False)]
+        else:
+            named += [("in_project_fx_weight", self.in_project_fx.weight, True),
+                      ("in_project_fx_bias", self.in_project_fx.bias, False)]
+        named += [
             ("in_project_slice_weight", self.in_project_slice.weight, False),
             ("in_project_slice_bias", self.in_project_slice.bias, False),
             ("temperature", self.temperature, False),
@@ -139,6 +148,8 @@ class PhysicsAttentionBase(nn.Module):
         """Training path: stage-level kernels forward, backward kernels in `autograd.PhysicsAttentionFunction`."""
         if self.fp8_weights:
             raise RuntimeError("fp8 weights are an inference format: no gradients flow through them")
+        if self.plus:
+            raise NotImplementedError("the backward kernels do not cover Transolver++ (plus=True)")
         dims = self.layer_dims(x)
         if not PF.backward_supported(x.dtype, dims):
             raise RuntimeError(f"the backward kernels do not serve this shape: {dims}")
@@ -156,12 +167,43 @@ class PhysicsAttentionBase(nn.Module):
         x = self._prepare_input(x)
         if needs_grad:
             return self._forward_with_grad(x)
+        if self.plus:
+            return self.forward_with_noise(x, None)
         return PF.layer_forward(x, self.kernel_params(x.dtype, x.device), self.layer_dims(x))
+
+    def forward_with_noise(self, x: torch.Tensor, noise_u: torch.Tensor | None, stages: bool = False):
+        """Transolver++ forward (reference :166-170, :530-532) through the stage-level kernels.  ``noise_u``
+        (B, N, H, S): the uniform samples behind the Gumbel noise; ``None`` draws them from torch's generator of the
+        input's device exactly as the reference's ``torch.rand_like(slice_projections)`` does."""
+        if not self.plus:
+            raise RuntimeError("forward_with_noise is the plus=True path")
+        self._validate(x)
+        if self._needs_grad(x):
+            raise NotImplementedError("the backward kernels do not cover Transolver++ (plus=True)")
+        x = self._prepare_input(x)
+        dims = self.layer_dims(x)
+        p = self.kernel_params(x.dtype, x.device)
+        x_mid, fx_mid = PF.project_inputs(x, p, dims)
+        if noise_u is None:
+            noise_u = torch.rand((dims.B, dims.N, dims.H, dims.S), dtype=x.dtype, device=x.device)
+        w = PF.slice_softmax_plus(x_mid, noise_u.to(x.dtype).contiguous(), p, dims)
+        tok, norm = PF.slice_reduce(w, fx_mid, dims)
+        tok_out = PF.slice_attention(tok, p, dims)
+        y = PF.deslice_project(w, tok_out, p, dims)
+        if stages:
+            H, D = self.heads, self.dim_head
+            return dict(x_mid=x_mid.view(dims.B, dims.N, H, D), w=w, tok=tok, norm=norm, tok_out=tok_out, y=y)
+        return y
 
     def forward_block(self, x: torch.Tensor, residual: torch.Tensor, ln: nn.LayerNorm):
         """Layer + the caller block's ``+ residual`` and following LayerNorm in one pass
         (physicsnemo/models/transolver/transolver.py:300-303).  Returns (fx_new, LayerNorm(fx_new))."""
         self._validate(x)
+        if self.plus:
+            y = self.forward_with_noise(x, None)
+            fx_new = y + residual.to(y.dtype)
+            normed = torch.nn.functional.layer_norm(fx_new.float(), ln.normalized_shape, ln.weight, ln.bias, ln.eps)
+            return fx_new, normed.to(y.dtype)
         x = self._prepare_input(x)
         residual = residual.to(x.dtype).contiguous()
         return PF.layer_forward(
@@ -193,7 +235,8 @@ class PhysicsAttentionIrregularMesh(PhysicsAttentionBase):
         super().__init__(dim, heads, dim_head, dropout, slice_num, use_te, plus)
         inner_dim = dim_head * heads
         self.in_project_x = nn.Linear(dim, inner_dim)
-        self.in_project_fx = nn.Linear(dim, inner_dim)
+        if not plus:
+            self.in_project_fx = nn.Linear(dim, inner_dim)
 
 
 class PhysicsAttentionStructuredMesh2D(PhysicsAttentionBase):
@@ -210,7 +253,8 @@ class PhysicsAttentionStructuredMesh2D(PhysicsAttentionBase):
         self.W = spatial_shape[1]
         self.kernel = kernel
         self.in_project_x = nn.Conv2d(dim, inner_dim, kernel, 1, kernel // 2)
-        self.in_project_fx = nn.Conv2d(dim, inner_dim, kernel, 1, kernel // 2)
+        if not plus:
+            self.in_project_fx = nn.Conv2d(dim, inner_dim, kernel, 1, kernel // 2)
 
     def _conv_geometry(self):
         return self.H, self.W, self.kernel, 0
@@ -235,7 +279,8 @@ class PhysicsAttentionStructuredMesh3D(PhysicsAttentionBase):
         self.D = spatial_shape[2]
         self.kernel = kernel
         self.in_project_x = nn.Conv3d(dim, inner_dim, kernel, 1, kernel // 2)
-        self.in_project_fx = nn.Conv3d(dim, inner_dim, kernel, 1, kernel // 2)
+        if not plus:
+            self.in_project_fx = nn.Conv3d(dim, inner_dim, kernel, 1, kernel // 2)
 
     def _conv_geometry(self):
         return self.H, self.W, self.kernel, self.D

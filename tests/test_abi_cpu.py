@@ -106,6 +106,7 @@ def test_model_state_dict_matches_oracle_and_loads_legacy_keys():
 
 
 def test_validation_messages_and_no_cpu_fallback():
+    from oracle import torch_oracle as to
     m = pn.PhysicsAttentionIrregularMesh(8, heads=2, dim_head=4, slice_num=3, use_te=False)
     with pytest.raises(ValueError, match="Expected 3D input"):
         m(torch.randn(4, 8))
@@ -113,8 +114,16 @@ def test_validation_messages_and_no_cpu_fallback():
         m(torch.randn(1, 4, 6))
     with torch.no_grad(), pytest.raises(RuntimeError, match="GPU tensors only"):
         m(torch.randn(1, 4, 8))
-    with pytest.raises(NotImplementedError):
-        pn.PhysicsAttentionIrregularMesh(8, heads=2, dim_head=4, plus=True)
+    with pytest.raises(RuntimeError, match="GPU tensors only"):
+        m(torch.randn(1, 4, 8))  # gradients enabled: still no CPU path
+    # Transolver++: no in_project_fx, proj_temperature registered right after temperature (reference :285-295, :622-627)
+    torch.manual_seed(3)
+    mp = pn.PhysicsAttentionIrregularMesh(8, heads=2, dim_head=4, slice_num=3, plus=True, use_te=False)
+    torch.manual_seed(3)
+    op = to.OraclePhysicsAttentionIrregularMesh(8, heads=2, dim_head=4, slice_num=3, plus=True)
+    assert list(mp.state_dict()) == list(op.state_dict())
+    assert all(torch.equal(mp.state_dict()[k], op.state_dict()[k]) for k in mp.state_dict())
+    assert "in_project_fx.weight" not in mp.state_dict()
     with pytest.raises(ValueError, match="n_hidden % n_head"):
         pn.Transolver(functional_dim=1, out_dim=1, embedding_dim=1, n_hidden=30, n_head=4)
     with pytest.raises(ValueError, match="structured_shape when using unified_pos"):

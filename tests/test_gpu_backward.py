@@ -120,7 +120,7 @@ def test_model_training_step_matches_oracle():
         loss2 = float(((m(fx.cuda(), emb.cuda()) - target.cuda()) ** 2).mean())
         loss2_ref = float(((ref(fx, emb) - target) ** 2).mean())
     assert abs(loss2 - loss2_ref) <= 1e-4 * abs(loss2_ref)
-    assert loss2_ref >= float(loss_ref) or loss2 < float(loss.detach())
+    assert loss2_ref >= float(loss_ref.detach()) or loss2 < float(loss.detach())
 
 
 def test_gradients_reach_the_input_only_when_asked():

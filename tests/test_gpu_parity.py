@@ -147,8 +147,13 @@ def test_autocast_bf16_and_errors_on_gpu():
     assert y.dtype == torch.bfloat16
     with torch.no_grad():
         assert_rel_l2(y, ref(x), "autocast y")
-    with pytest.raises(RuntimeError, match="forward pass only"):
-        hip(x.cuda())  # grad enabled, parameters require grad
+    y_grad = hip(x.cuda())  # grad enabled, parameters require grad: the differentiable path
+    assert y_grad.requires_grad and y_grad.grad_fn is not None
+    assert_fp32_close(y_grad, ref(x), "differentiable-path y")
+    hip.use_fp8_weights(True)
+    with pytest.raises(RuntimeError, match="no gradients"):
+        hip(x.cuda().bfloat16())
+    hip.use_fp8_weights(False)
     with torch.no_grad(), pytest.raises(ValueError, match="Expected 3D input"):
         hip(x.cuda()[0])
     _, hip2 = make_pair("structured2d", 16, 2, 8, 4, spatial=(4, 4))

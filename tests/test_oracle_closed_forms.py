@@ -157,6 +157,47 @@ def test_oracle_gradient_matches_finite_differences(variant):
     assert torch.autograd.gradcheck(fn, (x, *params), eps=1e-6, atol=1e-6, rtol=1e-5)
 
 
+def test_plus_branch_numpy_vs_torch_and_special_cases():
+    torch.manual_seed(21)
+    B, N, C, H, D, S = 2, 9, 6, 2, 4, 5
+    m = to.OraclePhysicsAttentionIrregularMesh(C, heads=H, dim_head=D, slice_num=S, plus=True).double()
+    assert "in_project_fx.weight" not in m.state_dict()
+    assert list(m.state_dict())[:5] == ["temperature", "proj_temperature.0.weight", "proj_temperature.0.bias",
+                                        "proj_temperature.2.weight", "proj_temperature.2.bias"]
+    x = torch.randn(B, N, C, dtype=torch.float64)
+    u = torch.rand(B, N, H, S, dtype=torch.float64)
+    with torch.no_grad():
+        st = m.stages(x, u)
+    ref = no.layer_forward(_sd_np(m), x.numpy(), H, D, noise_u=u.numpy())
+    for key in ("x_mid", "w", "tok", "tok_out", "y"):
+        np.testing.assert_allclose(st[key].numpy(), ref[key], rtol=1e-10, atol=1e-12, err_msg=key)
+    # noise that is the same for every slice of a point cancels in the softmax, and a proj_temperature whose last
+    # Linear is zero adds GELU(0) = 0: the layer is then the plain one with in_project_fx := in_project_x
+    # (temperatures inside [0.5, 5], where both clamps are inactive)
+    plain = to.OraclePhysicsAttentionIrregularMesh(C, heads=H, dim_head=D, slice_num=S).double()
+    sd = {k: v for k, v in m.state_dict().items() if not k.startswith("proj_temperature")}
+    sd["in_project_fx.weight"], sd["in_project_fx.bias"] = sd["in_project_x.weight"], sd["in_project_x.bias"]
+    plain.load_state_dict(sd)
+    with torch.no_grad():
+        m.proj_temperature[2].weight.zero_()
+        m.proj_temperature[2].bias.zero_()
+        m.temperature.copy_(torch.tensor([0.7, 3.0], dtype=torch.float64).view(1, 1, 2, 1))
+        plain.temperature.copy_(m.temperature)
+        u_const = torch.rand(B, N, H, 1, dtype=torch.float64).expand(B, N, H, S)
+        assert torch.allclose(m.forward_with_noise(x, u_const), plain(x), rtol=1e-11, atol=1e-12)
+        # below the plain clamp's floor the plus branch keeps the small temperature (floor 0.01, not 0.5)
+        m.temperature.fill_(0.1)
+        w_small = m.stages(x, u_const)["w"]
+        want = torch.softmax(m.stages(x, u_const)["logits"] / 0.1, dim=-1)
+        assert torch.allclose(w_small, want, rtol=1e-10, atol=1e-12)
+        m.temperature.fill_(-3.0)  # clamps to 0.01
+        want = torch.softmax(m.stages(x, u_const)["logits"] / 0.01, dim=-1)
+        assert torch.allclose(m.stages(x, u_const)["w"], want, rtol=1e-10, atol=1e-12)
+    # the noise is Gumbel(0, 1): mean = Euler-Mascheroni, variance = pi^2 / 6
+    g = to.gumbel_from_uniform(torch.rand(400000, dtype=torch.float64))
+    assert abs(float(g.mean()) - 0.5772156649) < 0.01 and abs(float(g.var()) - math.pi ** 2 / 6) < 0.03
+
+
 def test_softmax_rows_and_temperature_clamp():
     B, N, H, D, S = 2, 11, 3, 4, 5
     logits = torch.randn(B, N, H, S, dtype=torch.float64) * 4
