@@ -24,17 +24,6 @@ namespace general {
 // 64x64 output tile per 256-thread workgroup, 4x4 outputs per thread, K staged 16 at a time through LDS.
 // blockIdx.z selects one of two (W, bias, out) sets that share the same input (x_mid and fx_mid).
 // ------------------------------------------------------------------------------------------------
-struct GemmArgs {
-  const void *in;
-  const void *w[2];
-  const float *bias[2];
-  void *out[2];
-  int64_t M;   // rows = B*N
-  int K, O;    // reduction length, output columns
-  int C, N, gh, gw, ks;  // conv geometry (ks = 0: linear)
-  int gd;                // depth of a 3-D grid (0: 2-D)
-};
-
 template <typename TA, typename TW>
 __global__ __launch_bounds__(256) void rows_gemm_kernel(GemmArgs a) {
   __shared__ float As[16][64 + 4];
@@ -566,6 +555,7 @@ static int allow_dynamic_lds(F kernel, size_t bytes) {
 
 template <typename TA, typename TW>
 static int launch_gemm(const GemmArgs &a, int nsets, hipStream_t st) {
+  if (gemm::serves(a, nsets, sizeof(TA))) return gemm::launch(a, nsets, sizeof(TA) == 4 ? PA_F32 : PA_BF16, st);
   dim3 grid((unsigned)((a.M + 63) / 64), (unsigned)((a.O + 63) / 64), (unsigned)nsets);
   hipLaunchKernelGGL((rows_gemm_kernel<TA, TW>), grid, dim3(256), 0, st, a);
   return launch_status();

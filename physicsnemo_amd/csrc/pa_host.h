@@ -11,6 +11,30 @@ namespace pa {
 
 constexpr size_t kMaxLdsBytes = 160 * 1024;  // LDS per workgroup on gfx950
 
+// Arguments of the row GEMMs: out[m, o] = bias[o] + sum_k A(m, k) * W[o, k]
+//   linear: A(m, k) = in[m*K + k]
+//   conv  : K = taps*C, k = tap*C + c; 2-D: taps = ks^2, tap = u*ks + v, A(m,k) = in[b, (i+u-p)*gw + (j+v-p), c];
+//           3-D: taps = ks^3, tap = (u*ks + v)*ks + z, A(m,k) = in[b, ((i+u-p)*gw + (j+v-p))*gd + (l+z-p), c];
+//           0 outside the grid; the PyTorch weight element is W[o, c, u, v(, z)] = W[o*K + c*taps + tap].
+// Up to two (W, bias, out) sets share the same input (x_mid and fx_mid), selected by blockIdx.z.
+struct GemmArgs {
+  const void *in;
+  const void *w[2];
+  const float *bias[2];
+  void *out[2];
+  int64_t M;   // rows = B*N
+  int K, O;    // reduction length, output columns
+  int C, N, gh, gw, ks;  // conv geometry (ks = 0: linear)
+  int gd;                // depth of a 3-D grid (0: 2-D)
+};
+
+namespace gemm {
+// MFMA row GEMM (fp32: v_mfma_f32_32x32x2_f32, bf16: v_mfma_f32_32x32x16_bf16); `serves` tells whether the shape and
+// the pointers meet its 16-byte granularity, otherwise the scalar kernel of the general family runs.
+bool serves(const GemmArgs &a, int nsets, size_t elem_bytes);
+int launch(const GemmArgs &a, int nsets, int dtype, hipStream_t st);
+}  // namespace gemm
+
 namespace general {
 int dequant_e4m3(const void *in, const float *scale, void *out, int64_t rows, int64_t cols, hipStream_t st);
 int project_inputs(int dtype, const pa_shape &s, const pa_params &p, const void *x, void *x_mid, void *fx_mid,
