@@ -241,6 +241,30 @@ int pa_mfma_combine_attention(const pa_shape *shape, const pa_params *p, const f
 int pa_mfma_deslice_project(const pa_shape *shape, const void *blob, const void *w_pack, const void *tokp, void *y,
                             const pa_block_tail *tail, void *stream);
 
+/* ---- backward pass on the bf16 MFMA kernels (pa_mfma_backward_query() == 1: MFMA shapes with S <= 64) -------
+ * Same gradient as the general backward entry points above, for callers that ran the forward through the pa_mfma_*
+ * stages and kept w_pack, the slice tokens and tokp.  No reference counterpart beyond autograd over PA.py:501-558. */
+int pa_mfma_backward_query(const pa_shape *shape);
+/* bf16 Linear over the rows of `in` (B, N, c_in) -> H*32 columns, weight (H*32, c_in) bf16, bias float32 or NULL:
+ * `out` natural (B, N, H*32) and/or `out_pack` in the packed layout of PA_BUF_FX_PACK (either may be NULL). */
+int pa_rows_gemm_packed(const pa_shape *shape, int64_t c_in, const void *in, const void *weight, const float *bias,
+                        void *out, void *out_pack, void *stream);
+/* sums (B,H,S,D+1) float32 = sum_n w[n,s] [v[n,:], 1] from the packed operands (adjoint of the deslice when v = d out_x);
+ * `partials` sized as PA_BUF_PARTIALS. */
+int pa_mfma_slice_weighted_sum(const pa_shape *shape, const void *w_pack, const void *v_pack, float *partials,
+                               float *sums, void *stream);
+/* out_x (B, N, H*32) bf16 = deslice of the attended tokens (PA.py:492-495), the input of d W_out = dy^T out_x. */
+int pa_mfma_deslice(const pa_shape *shape, const void *w_pack, const void *tokp, void *out_x, void *stream);
+/* Per-point part of the backward pass, as pa_slice_softmax_backward but with the slice weights taken from w_pack.
+ * tables: scratch of pa_mfma_backward_tables_bytes(shape) bytes; d_temperature_partials: float32,
+ * pa_mfma_backward_groups(shape) * H elements (sum over the first index). */
+int64_t pa_mfma_backward_tables_bytes(const pa_shape *shape);
+int64_t pa_mfma_backward_groups(const pa_shape *shape);
+int pa_mfma_slice_softmax_backward(const pa_shape *shape, const pa_params *p, const void *x_mid, const void *fx_mid,
+                                   const void *d_out_x, const void *w_pack, const float *out_slice_token,
+                                   const float *d_num, const float *d_norm, void *tables, void *d_proj, void *d_z,
+                                   float *d_temperature_partials, void *stream);
+
 /* ---- block MLP ---------------------------------------------------------------------------------- */
 
 /* Parameters of Mlp(C -> F -> C) with GELU (physicsnemo/nn/module/mlp_layers.py:139-173): torch layouts,

@@ -23,6 +23,8 @@ EXPORTED = [
      "pa_mfma_combine_attention", "pa_mfma_deslice_project", "pa_mlp_query", "pa_mlp_workspace_bytes", "pa_mlp_forward",
     "pa_rows_gemm", "pa_slice_weighted_sum", "pa_backward_query", "pa_backward_point_tiles",
     "pa_slice_attention_backward", "pa_slice_softmax_backward", "pa_slice_softmax_plus",
+    "pa_mfma_backward_query", "pa_rows_gemm_packed", "pa_mfma_slice_weighted_sum", "pa_mfma_deslice",
+    "pa_mfma_backward_tables_bytes", "pa_mfma_backward_groups", "pa_mfma_slice_softmax_backward",
 ]
 
 PA_BUF_BLOB, PA_BUF_FX_PACK, PA_BUF_W_PACK, PA_BUF_PARTIALS, PA_BUF_TOKP = range(5)
@@ -126,6 +128,20 @@ def load() -> ctypes.CDLL:
     lib.pa_slice_softmax_backward.argtypes = [c_int, ps, pp] + [c_void_p] * 11
     lib.pa_slice_softmax_plus.restype = c_int
     lib.pa_slice_softmax_plus.argtypes = [c_int, ps, pp, POINTER(PaPlusParams)] + [c_void_p] * 4
+    lib.pa_mfma_backward_query.restype = c_int
+    lib.pa_mfma_backward_query.argtypes = [ps]
+    lib.pa_rows_gemm_packed.restype = c_int
+    lib.pa_rows_gemm_packed.argtypes = [ps, c_int64] + [c_void_p] * 6
+    lib.pa_mfma_slice_weighted_sum.restype = c_int
+    lib.pa_mfma_slice_weighted_sum.argtypes = [ps] + [c_void_p] * 5
+    lib.pa_mfma_deslice.restype = c_int
+    lib.pa_mfma_deslice.argtypes = [ps] + [c_void_p] * 4
+    lib.pa_mfma_backward_tables_bytes.restype = c_int64
+    lib.pa_mfma_backward_tables_bytes.argtypes = [ps]
+    lib.pa_mfma_backward_groups.restype = c_int64
+    lib.pa_mfma_backward_groups.argtypes = [ps]
+    lib.pa_mfma_slice_softmax_backward.restype = c_int
+    lib.pa_mfma_slice_softmax_backward.argtypes = [ps, pp] + [c_void_p] * 12
     _lib = lib
     return lib
 

@@ -39,8 +39,45 @@ def _conv_weight_grad(d_out: torch.Tensor, x: torch.Tensor, grid: tuple, k: int)
     return dW
 
 
+def _finish_backward(ctx, x, dy, out_x, d_wqkv, d_proj, d_z, d_temp, x_mid, temperature):
+    """Everything after the layer-specific kernels: d x (input-gradient GEMM / transposed convolution) and the weight
+    and bias gradients, which are plain GEMMs / column sums over the point axis."""
+    dims, kp = ctx.dims, ctx.kparams
+    B, N, C, H, D, S = dims.B, dims.N, dims.C, dims.H, dims.D, dims.S
+    HD = H * D
+    linear = PF.LayerDims(B, N, C, H, D, S)
+    d_wo = _rows(dy).t() @ _rows(out_x)
+    d_bo = _rows(dy).sum(0, dtype=torch.float32)
+    d_ws = d_z.reshape(-1, S).t() @ x_mid.reshape(-1, D)
+    d_bs = d_z.reshape(-1, S).sum(0, dtype=torch.float32)
+    t = temperature.reshape(-1)
+    d_temp = d_temp * ((t >= 0.5) & (t <= 5.0)).to(d_temp.dtype)
+
+    k = dims.conv_k
+    wx, wf = kp["in_project_x_weight"], kp["in_project_fx_weight"]
+    if k == 0:
+        w_cat = torch.cat([wx.view(HD, C).t(), wf.view(HD, C).t()], dim=1).contiguous()  # (C, 2HD)
+        dx = PF.rows_gemm(d_proj, w_cat, None, linear, 2 * HD, C) if ctx.needs_input_grad[0] else None
+        d_w_in = _rows(d_proj).t() @ _rows(x)  # (2HD, C)
+    else:
+        grid = (dims.grid_h, dims.grid_w) + ((dims.grid_d,) if dims.grid_d > 0 else ())
+        taps = (k,) * len(grid)
+        w_both = torch.cat([wx.view(HD, C, *taps), wf.view(HD, C, *taps)], dim=0)  # (2HD, C, k, ...)
+        # transposed convolution = the same gather with flipped taps and swapped channel roles
+        w_t = w_both.flip(dims=tuple(range(2, 2 + len(grid)))).transpose(0, 1).contiguous()
+        dx = PF.rows_gemm(d_proj, w_t, None, dims, 2 * HD, C) if ctx.needs_input_grad[0] else None
+        d_w_in = _conv_weight_grad(d_proj, x, grid, k)
+    d_b_in = _rows(d_proj).sum(0, dtype=torch.float32)
+
+    grads = (d_w_in[:HD], d_b_in[:HD], d_w_in[HD:], d_b_in[HD:], d_ws, d_bs, d_temp, d_wqkv, d_wo, d_bo)
+    grads = tuple(gr.reshape(p.shape).to(p.dtype) if ctx.needs_input_grad[3 + i] else None
+                  for i, (gr, p) in enumerate(zip(grads, ctx.param_like)))
+    return (dx, None, None) + grads
+
+
 class PhysicsAttentionFunction(torch.autograd.Function):
-    """y = PhysicsAttention(x); differentiable w.r.t. x and the ten parameters."""
+    """y = PhysicsAttention(x); differentiable w.r.t. x and the ten parameters.  General kernels (any shape, fp32 or
+    bf16 storage): the forward keeps x_mid, fx_mid, the slice weights, the slice tokens and out_x."""
 
     @staticmethod
     def forward(ctx, x, dims, kparams, wx, bx, wf, bf, ws, bs, temperature, wqkv, wo, bo):
@@ -58,47 +95,53 @@ class PhysicsAttentionFunction(torch.autograd.Function):
     def backward(ctx, dy):
         x, x_mid, fx_mid, w, tok, norm, tok_out, out_x, temperature = ctx.saved_tensors
         dims, kp = ctx.dims, ctx.kparams
-        B, N, C, H, D, S = dims.B, dims.N, dims.C, dims.H, dims.D, dims.S
-        HD = H * D
+        C, HD, D = dims.C, dims.H * dims.D, dims.D
         dy = dy.to(x.dtype).contiguous()
-        linear = PF.LayerDims(B, N, C, H, D, S)
-
-        # out_linear: g = d out_x, d W_out, d b_out
-        wo = kp["out_linear_weight"].view(C, HD)
-        g = PF.rows_gemm(dy, wo.t().contiguous(), None, linear, C, HD)
-        d_wo = _rows(dy).t() @ _rows(out_x)
-        d_bo = _rows(dy).sum(0, dtype=torch.float32)
-
+        linear = PF.LayerDims(dims.B, dims.N, C, dims.H, D, dims.S)
+        # out_linear: g = d out_x
+        g = PF.rows_gemm(dy, kp["out_linear_weight"].view(C, HD).t().contiguous(), None, linear, C, HD)
         # adjoint of the deslice w.r.t. the attended tokens, then the slice attention and the normalisation
         d_tok_out = PF.slice_weighted_sum(w, g, dims)[..., :D].contiguous()
         d_num, d_norm, d_wqkv = PF.slice_attention_backward(tok, norm, d_tok_out, kp, dims)
-
         # per point: slice softmax, aggregation and deslice adjoints
         d_proj, d_z, d_temp = PF.slice_softmax_backward(x_mid, fx_mid, w, g, tok_out, d_num, d_norm, kp, dims)
-        d_ws = d_z.reshape(-1, S).t() @ x_mid.reshape(-1, D)
-        d_bs = d_z.reshape(-1, S).sum(0, dtype=torch.float32)
-        t = temperature.reshape(-1)
-        d_temp = d_temp * ((t >= 0.5) & (t <= 5.0)).to(d_temp.dtype)
+        return _finish_backward(ctx, x, dy, out_x, d_wqkv, d_proj, d_z, d_temp, x_mid, temperature)
 
-        # input projections: d x and the weight / bias gradients
-        k = dims.conv_k
-        wx, wf = kp["in_project_x_weight"], kp["in_project_fx_weight"]
-        if k == 0:
-            w_cat = torch.cat([wx.view(HD, C).t(), wf.view(HD, C).t()], dim=1).contiguous()  # (C, 2HD)
-            dx = PF.rows_gemm(d_proj, w_cat, None, linear, 2 * HD, C)
-            d_w_in = _rows(d_proj).t() @ _rows(x)  # (2HD, C)
+
+class PhysicsAttentionMfmaFunction(torch.autograd.Function):
+    """The same gradient on the bf16 MFMA kernels (irregular variant, D = 32, C in {128, 256}, S <= 64).
+
+    The forward is the inference path (fused projection / softmax / aggregation kernel, slice attention, deslice +
+    out_linear) with its packed slice weights kept; the backward recomputes x_mid / fx_mid with one MFMA GEMM and reads
+    the slice weights in their packed form."""
+
+    @staticmethod
+    def forward(ctx, x, dims, kparams, wx, bx, wf, bf, ws, bs, temperature, wqkv, wo, bo):
+        st = PF.MfmaStages(kparams, dims, x.device)
+        st.pack_params()
+        if st.fused_groups > 0:
+            st.project_softmax_reduce(x)
         else:
-            grid = (dims.grid_h, dims.grid_w) + ((dims.grid_d,) if dims.grid_d > 0 else ())
-            taps = (k,) * len(grid)
-            w_both = torch.cat([wx.view(HD, C, *taps), wf.view(HD, C, *taps)], dim=0)  # (2HD, C, k, ...)
-            # transposed convolution = the same gather with flipped taps and swapped channel roles
-            w_t = w_both.flip(dims=tuple(range(2, 2 + len(grid)))).transpose(0, 1).contiguous()
-            dx = PF.rows_gemm(d_proj, w_t, None, dims, 2 * HD, C)
-            d_w_in = _conv_weight_grad(d_proj, x, grid, k)
-        d_b_in = _rows(d_proj).sum(0, dtype=torch.float32)
+            st.project_softmax(x)
+            st.slice_reduce()
+        st.combine_attention()
+        y = torch.empty_like(x)
+        st.deslice_project(y)
+        ctx.save_for_backward(x, temperature)
+        ctx.stages, ctx.dims, ctx.kparams = st, dims, kparams
+        ctx.param_like = (wx, bx, wf, bf, ws, bs, temperature, wqkv, wo, bo)
+        return y
 
-        like = ctx.param_like
-        grads = (d_w_in[:HD], d_b_in[:HD], d_w_in[HD:], d_b_in[HD:], d_ws, d_bs, d_temp, d_wqkv, d_wo, d_bo)
-        grads = tuple(gr.reshape(p.shape).to(p.dtype) if ctx.needs_input_grad[3 + i] else None
-                      for i, (gr, p) in enumerate(zip(grads, like)))
-        return (dx if ctx.needs_input_grad[0] else None, None, None) + grads
+    @staticmethod
+    def backward(ctx, dy):
+        x, temperature = ctx.saved_tensors
+        st, dims, kp = ctx.stages, ctx.dims, ctx.kparams
+        C, HD, D = dims.C, dims.H * dims.D, dims.D
+        dy = dy.to(x.dtype).contiguous()
+        g, g_pack = st.rows_gemm_packed(dy, kp["out_linear_weight"].view(C, HD).t().contiguous(), None)
+        x_mid, fx_mid = PF.project_inputs(x, kp, dims)
+        d_tok_out = st.slice_weighted_sum(g_pack)[..., :D].contiguous()
+        d_num, d_norm, d_wqkv = PF.slice_attention_backward(st.tok, st.norm, d_tok_out, kp, dims)
+        out_x = st.deslice()
+        d_proj, d_z, d_temp = st.slice_softmax_backward(x_mid, fx_mid, g, d_num, d_norm)
+        return _finish_backward(ctx, x, dy, out_x, d_wqkv, d_proj, d_z, d_temp, x_mid, temperature)

@@ -339,6 +339,81 @@ int pa_slice_softmax_backward(int dtype, const pa_shape *shape, const pa_params 
                                      d_proj, d_z, d_temperature_partials, static_cast<hipStream_t>(stream));
 }
 
+int pa_mfma_backward_query(const pa_shape *shape) {
+  int rc = check_shape(PA_BF16, shape);
+  if (rc) return rc;
+  return pa::mfma::backward_supported(*shape) && check_backward_shape(PA_BF16, shape) == PA_OK ? 1 : 0;
+}
+
+int64_t pa_mfma_backward_tables_bytes(const pa_shape *shape) {
+  int rc = check_shape(PA_BF16, shape);
+  if (rc) return rc;
+  if (!pa::mfma::backward_supported(*shape)) return PA_ERR_UNSUPPORTED;
+  return pa::mfma::backward_tables_bytes(*shape);
+}
+
+int64_t pa_mfma_backward_groups(const pa_shape *shape) {
+  int rc = check_shape(PA_BF16, shape);
+  if (rc) return rc;
+  if (!pa::mfma::backward_supported(*shape)) return PA_ERR_UNSUPPORTED;
+  return pa::mfma::backward_groups(*shape, compute_units()) * shape->B;
+}
+
+int pa_rows_gemm_packed(const pa_shape *shape, int64_t c_in, const void *in, const void *weight, const float *bias,
+                        void *out, void *out_pack, void *stream) {
+  int rc = check_shape(PA_BF16, shape);
+  if (rc) return rc;
+  if (!pa::mfma::supported(PA_BF16, *shape)) return PA_ERR_UNSUPPORTED;
+  if (c_in <= 0 || c_in > (1 << 16)) return PA_ERR_DIMS;
+  if (!in || !weight || (!out && !out_pack)) return PA_ERR_NULL;
+  if (!aligned16(in) || !aligned16(weight) || !aligned16(out) || !aligned16(out_pack)) return PA_ERR_ALIGN;
+  return pa::general::rows_gemm_packed(*shape, c_in, in, weight, bias, out, out_pack, static_cast<hipStream_t>(stream));
+}
+
+int pa_mfma_slice_weighted_sum(const pa_shape *shape, const void *w_pack, const void *v_pack, float *partials, float *sums,
+                               void *stream) {
+  int rc = check_shape(PA_BF16, shape);
+  if (rc) return rc;
+  if (!pa::mfma::supported(PA_BF16, *shape)) return PA_ERR_UNSUPPORTED;
+  if (!w_pack || !v_pack || !partials || !sums) return PA_ERR_NULL;
+  if (!aligned16(w_pack) || !aligned16(v_pack) || !aligned16(partials) || !aligned16(sums)) return PA_ERR_ALIGN;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if ((rc = pa::mfma::slice_reduce(*shape, w_pack, v_pack, partials, st))) return rc;
+  const float *total = nullptr;
+  if ((rc = pa::general::combine_partials(*shape, partials, mfma_groups(*shape, false), &total, st))) return rc;
+  const size_t bytes = (size_t)(shape->B * shape->H * shape->S * (shape->D + 1)) * 4;
+  hipError_t e = hipMemcpyAsync(sums, total, bytes, hipMemcpyDeviceToDevice, st);
+  return e == hipSuccess ? PA_OK : (int)e;
+}
+
+int pa_mfma_deslice(const pa_shape *shape, const void *w_pack, const void *tokp, void *out_x, void *stream) {
+  int rc = check_shape(PA_BF16, shape);
+  if (rc) return rc;
+  if (!pa::mfma::supported(PA_BF16, *shape)) return PA_ERR_UNSUPPORTED;
+  if (!w_pack || !tokp || !out_x) return PA_ERR_NULL;
+  if (!aligned16(w_pack) || !aligned16(tokp) || !aligned16(out_x)) return PA_ERR_ALIGN;
+  return pa::mfma::deslice_natural(*shape, w_pack, tokp, out_x, compute_units(), static_cast<hipStream_t>(stream));
+}
+
+int pa_mfma_slice_softmax_backward(const pa_shape *shape, const pa_params *p, const void *x_mid, const void *fx_mid,
+                                   const void *d_out_x, const void *w_pack, const float *out_slice_token,
+                                   const float *d_num, const float *d_norm, void *tables, void *d_proj, void *d_z,
+                                   float *d_temperature_partials, void *stream) {
+  int rc = check_shape(PA_BF16, shape);
+  if (rc) return rc;
+  if (!pa::mfma::backward_supported(*shape)) return PA_ERR_UNSUPPORTED;
+  if (!p || !p->in_project_slice_weight || !p->in_project_slice_bias || !p->temperature) return PA_ERR_NULL;
+  if (!x_mid || !fx_mid || !d_out_x || !w_pack || !out_slice_token || !d_num || !d_norm || !tables || !d_proj || !d_z ||
+      !d_temperature_partials)
+    return PA_ERR_NULL;
+  if (!aligned16(x_mid) || !aligned16(fx_mid) || !aligned16(d_out_x) || !aligned16(w_pack) || !aligned16(tables) ||
+      !aligned16(d_proj) || !aligned16(d_z))
+    return PA_ERR_ALIGN;
+  return pa::mfma::slice_softmax_backward(*shape, *p, x_mid, fx_mid, d_out_x, w_pack, out_slice_token, d_num, d_norm, tables,
+                                          d_proj, d_z, d_temperature_partials, compute_units(),
+                                          static_cast<hipStream_t>(stream));
+}
+
 int64_t pa_mfma_buffer_bytes(const pa_shape *shape, int which) {
   int rc = check_shape(PA_BF16, shape);
   if (rc) return rc;

@@ -65,15 +65,24 @@ __global__ __launch_bounds__(256) void rows_gemm_mfma_kernel(GemmArgs a) {
   const int taps = a.ks * a.ks * ksd;
   const int pad = a.ks / 2;
 
+  // Row numbering: the rows of `in` in order, or (pack_tpb > 0) batch by batch with every batch padded to whole
+  // 32-point tiles, so that a wave's 32 rows are one tile of one batch.
+  const int64_t padded = (int64_t)a.pack_tpb * 32;  // rows per batch in the padded numbering
+  auto real_row = [&](int64_t vm) -> int64_t {
+    if (a.pack_tpb == 0) return vm < a.M ? vm : -1;
+    const int64_t b = vm / padded, n = vm - b * padded;
+    return (n < a.N && b * a.N + n < a.M) ? b * a.N + n : -1;
+  };
+
   // the 4 input rows this thread stages: global row, and for a convolution its batch offset and grid coordinates
   int64_t arow[4];
   int ci[4], cj[4], cl[4];
 #pragma unroll
   for (int p = 0; p < 4; ++p) {
     const int64_t m = m0 + r0 + 32 * p;
-    arow[p] = m < a.M ? m : -1;
+    arow[p] = real_row(m);
     ci[p] = cj[p] = cl[p] = 0;
-    if (a.ks > 0 && m < a.M) {
+    if (a.ks > 0 && m < a.M) {  // convolutions never use the padded numbering
       const int64_t b = m / a.N;
       int n = (int)(m - b * a.N);
       cl[p] = n % gd;
@@ -151,15 +160,28 @@ __global__ __launch_bounds__(256) void rows_gemm_mfma_kernel(GemmArgs a) {
     __syncthreads();
   }
 
+  const int64_t tile = (int64_t)blockIdx.x * 4 + wave;  // this wave's 32 rows (one (batch, tile) when packing)
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) {
     const int o = o0 + nt * 32 + i;
     if (o >= a.O) continue;
     const float bv = bias ? bias[o] : 0.f;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int64_t m = m0 + wave * 32 + mfma::rowmap(r, g);
-      if (m < a.M) store_from_f32(out + m * a.O + o, acc[nt][r] + bv);
+    for (int r = 0; r < 16; ++r) acc[nt][r] += bv;
+    if (out) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int64_t m = real_row(tile * 32 + mfma::rowmap(r, g));
+        if (m >= 0) store_from_f32(out + m * a.O + o, acc[nt][r]);
+      }
+    }
+    if constexpr (sizeof(T) == 2) {
+      u32x4 *pk = static_cast<u32x4 *>(a.out_pack[z]);
+      const int head = (o0 >> 5) + nt;
+      if (a.pack_tpb > 0 && pk && tile * 32 < (a.M / a.N) * padded) {
+        pk[((tile * a.pack_heads + head) * 2 + 0) * 64 + lane] = mfma::pack_half<0>(acc[nt]);
+        pk[((tile * a.pack_heads + head) * 2 + 1) * 64 + lane] = mfma::pack_half<1>(acc[nt]);
+      }
     }
   }
 }
@@ -170,13 +192,14 @@ bool serves(const GemmArgs &a, int nsets, size_t elem_bytes) {
   if (a.ks > 0 && a.C % ue != 0) return false;          // a unit must not straddle two taps
   if (!aligned16(a.in)) return false;
   for (int z = 0; z < nsets; ++z)
-    if (!aligned16(a.w[z]) || !a.out[z]) return false;
+    if (!aligned16(a.w[z]) || (!a.out[z] && !a.out_pack[z])) return false;
   return true;
 }
 
 template <typename T, int NT>
 static int launch_t(const GemmArgs &a, int nsets, hipStream_t st) {
-  dim3 grid((unsigned)((a.M + kRows - 1) / kRows), (unsigned)((a.O + 32 * NT - 1) / (32 * NT)), (unsigned)nsets);
+  const int64_t rows = a.pack_tpb > 0 ? (a.M / a.N) * a.pack_tpb * 32 : a.M;
+  dim3 grid((unsigned)((rows + kRows - 1) / kRows), (unsigned)((a.O + 32 * NT - 1) / (32 * NT)), (unsigned)nsets);
   hipLaunchKernelGGL((rows_gemm_mfma_kernel<T, NT>), grid, dim3(256), 0, st, a);
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? PA_OK : (int)e;

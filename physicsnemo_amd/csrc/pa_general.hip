@@ -613,6 +613,27 @@ int rows_gemm(int dtype, const pa_shape &grid, int64_t c_in, int64_t c_out, cons
   return dtype == PA_F32 ? launch_gemm<float, float>(a, 1, st) : launch_gemm<bf16, bf16>(a, 1, st);
 }
 
+// bf16 Linear over the rows with the result in natural layout (`out`, may be NULL) and in the packed operand layout of
+// the MFMA slice kernels (`out_pack`, (B * tiles * H * 2) KiB as fx_pack); c_out = H * 32.
+int rows_gemm_packed(const pa_shape &s, int64_t c_in, const void *in, const void *weight, const float *bias, void *out,
+                     void *out_pack, hipStream_t st) {
+  GemmArgs a{};
+  a.in = in;
+  a.w[0] = weight;
+  a.bias[0] = bias;
+  a.out[0] = out;
+  a.out_pack[0] = out_pack;
+  a.M = s.B * s.N;
+  a.N = (int)s.N;
+  a.K = (int)c_in;
+  a.O = (int)(s.H * 32);
+  a.C = (int)c_in;
+  a.pack_tpb = (int)((s.N + 31) / 32);
+  a.pack_heads = (int)s.H;
+  if (c_in % 8 != 0 || !gemm::serves(a, 1, 2)) return PA_ERR_UNSUPPORTED;
+  return gemm::launch(a, 1, PA_BF16, st);
+}
+
 int out_linear(int dtype, const pa_shape &s, const pa_params &p, const void *out_x, void *y, hipStream_t st) {
   GemmArgs a{};
   a.in = out_x;

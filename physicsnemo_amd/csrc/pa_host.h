@@ -26,6 +26,11 @@ struct GemmArgs {
   int K, O;    // reduction length, output columns
   int C, N, gh, gw, ks;  // conv geometry (ks = 0: linear)
   int gd;                // depth of a 3-D grid (0: 2-D)
+  // MFMA kernel only, bf16, Linear, O = 32 * pack_heads: pack_tpb > 0 walks the rows batch by batch in tiles of 32
+  // points (pack_tpb tiles per batch, the last one padded) and also writes each (tile, head) block of the result in
+  // the packed operand layout of the MFMA slice kernels (fx_pack).  out[z] may then be NULL.
+  void *out_pack[2];
+  int pack_tpb, pack_heads;
 };
 
 namespace gemm {
@@ -42,6 +47,8 @@ int project_inputs(int dtype, const pa_shape &s, const pa_params &p, const void 
 int out_linear(int dtype, const pa_shape &s, const pa_params &p, const void *out_x, void *y, hipStream_t st);
 int rows_gemm(int dtype, const pa_shape &grid, int64_t c_in, int64_t c_out, const void *in, const void *weight,
               const float *bias, void *out, hipStream_t st);
+int rows_gemm_packed(const pa_shape &s, int64_t c_in, const void *in, const void *weight, const float *bias, void *out,
+                     void *out_pack, hipStream_t st);
 int slice_softmax(int dtype, const pa_shape &s, const pa_params &p, const void *x_mid, void *w, hipStream_t st);
 int slice_softmax_plus(int dtype, const pa_shape &s, const pa_params &p, const pa_plus_params &pp, const void *x_mid,
                        const void *uniform, void *w, hipStream_t st);
@@ -68,6 +75,14 @@ int slice_softmax(int dtype, const pa_shape &s, const pa_params &p, const void *
 }  // namespace backward
 
 namespace mfma {
+bool backward_supported(const pa_shape &s);
+int64_t backward_groups(const pa_shape &s, int num_cu);
+int64_t backward_tables_bytes(const pa_shape &s);
+int deslice_natural(const pa_shape &s, const void *w_pack, const void *tokp, void *out_x, int num_cu, hipStream_t st);
+int slice_softmax_backward(const pa_shape &s, const pa_params &p, const void *x_mid, const void *fx_mid,
+                           const void *d_out_x, const void *w_pack, const float *out_token, const float *d_num,
+                           const float *d_norm, void *tables, void *d_proj, void *d_z, float *dT_part, int num_cu,
+                           hipStream_t st);
 bool supported(int dtype, const pa_shape &s);
 int64_t tiles_per_batch(const pa_shape &s);
 int64_t reduce_groups(const pa_shape &s);

@@ -265,6 +265,53 @@ class MfmaStages:
                                                       self._producer_groups, self.tok.data_ptr(), self.norm.data_ptr(), self.tok_out.data_ptr(),
                                                       self.tokp.data_ptr(), self._stream()), "pa_mfma_combine_attention")
 
+    # ---- backward-pass stages (pa_mfma_backward_query() == 1) ----
+    def rows_gemm_packed(self, inp, weight, bias, natural=True, packed=True):
+        """bf16 Linear (B, N, c_in) -> H*32 columns; returns (natural (B, N, H*32) or None, packed buffer or None)."""
+        _need_cuda(inp, weight, bias)
+        d = self.dims
+        out = torch.empty(d.B, d.N, d.H * 32, dtype=torch.bfloat16, device=self.device) if natural else None
+        pack = torch.empty_like(self.fx_pack) if packed else None
+        _lib.check(self.lib.pa_rows_gemm_packed(byref(self.shape), inp.shape[-1], inp.data_ptr(), weight.data_ptr(),
+                                                _lib.ptr(bias), _lib.ptr(out), _lib.ptr(pack), self._stream()),
+                   "pa_rows_gemm_packed")
+        return out, pack
+
+    def slice_weighted_sum(self, v_pack):
+        """(B, H, S, D+1) float32: sum_n w[n,s] [v[n,:], 1] with w from w_pack and v in the packed layout."""
+        d = self.dims
+        sums = torch.empty(d.B, d.H, d.S, d.D + 1, dtype=torch.float32, device=self.device)
+        _lib.check(self.lib.pa_mfma_slice_weighted_sum(byref(self.shape), self.w_pack.data_ptr(), v_pack.data_ptr(),
+                                                       self.partials.data_ptr(), sums.data_ptr(), self._stream()),
+                   "pa_mfma_slice_weighted_sum")
+        return sums
+
+    def deslice(self):
+        """out_x (B, N, H*32) bf16 from w_pack and the attended tokens."""
+        d = self.dims
+        out_x = torch.empty(d.B, d.N, d.H * 32, dtype=torch.bfloat16, device=self.device)
+        _lib.check(self.lib.pa_mfma_deslice(byref(self.shape), self.w_pack.data_ptr(), self.tokp.data_ptr(),
+                                            out_x.data_ptr(), self._stream()), "pa_mfma_deslice")
+        return out_x
+
+    def slice_softmax_backward(self, x_mid, fx_mid, d_out_x, d_num, d_norm):
+        """Returns (d_proj (B,N,2HD) = [d x_mid | d fx_mid], d_z (B,N,H,S), d clamp(temperature) (H) float32)."""
+        _need_cuda(x_mid, fx_mid, d_out_x, d_num, d_norm)
+        d = self.dims
+        nbytes = self.lib.pa_mfma_backward_tables_bytes(byref(self.shape))
+        groups = self.lib.pa_mfma_backward_groups(byref(self.shape))
+        if nbytes < 0 or groups < 0:
+            _lib.check(int(min(nbytes, groups)), "pa_mfma_backward_tables_bytes")
+        tables = torch.empty(int(nbytes), dtype=torch.uint8, device=self.device)
+        d_proj = torch.empty(d.B, d.N, 2 * d.H * 32, dtype=torch.bfloat16, device=self.device)
+        d_z = torch.empty(d.B, d.N, d.H, d.S, dtype=torch.bfloat16, device=self.device)
+        dT = torch.empty(int(groups), d.H, dtype=torch.float32, device=self.device)
+        _lib.check(self.lib.pa_mfma_slice_softmax_backward(
+            byref(self.shape), byref(self.cparams), x_mid.data_ptr(), fx_mid.data_ptr(), d_out_x.data_ptr(),
+            self.w_pack.data_ptr(), self.tok_out.data_ptr(), d_num.data_ptr(), d_norm.data_ptr(), tables.data_ptr(),
+            d_proj.data_ptr(), d_z.data_ptr(), dT.data_ptr(), self._stream()), "pa_mfma_slice_softmax_backward")
+        return d_proj, d_z, dT.sum(0)
+
     def deslice_project(self, y, residual=None, ln_weight=None, ln_bias=None, ln_eps=1e-5, ln_out=None):
         tail = _c_tail(residual, ln_weight, ln_bias, ln_eps, ln_out)
         _lib.check(self.lib.pa_mfma_deslice_project(byref(self.shape), self.blob.data_ptr(), self.w_pack.data_ptr(),
@@ -279,6 +326,16 @@ def backward_supported(dtype: torch.dtype, dims: LayerDims) -> bool:
     rc = _lib.load().pa_backward_query(_lib.dtype_code(dtype), byref(dims.c()))
     if rc < 0:
         _lib.check(rc, "pa_backward_query")
+    return bool(rc)
+
+
+def mfma_backward_supported(dtype: torch.dtype, dims: LayerDims) -> bool:
+    """True if the bf16 MFMA backward kernels serve this shape (MFMA forward shapes with slice_num <= 64)."""
+    if dtype != torch.bfloat16:
+        return False
+    rc = _lib.load().pa_mfma_backward_query(byref(dims.c()))
+    if rc < 0:
+        _lib.check(rc, "pa_mfma_backward_query")
     return bool(rc)
 
 

@@ -19,7 +19,7 @@ import torch
 import torch.nn as nn
 
 from . import functional as PF
-from .autograd import PhysicsAttentionFunction
+from .autograd import PhysicsAttentionFunction, PhysicsAttentionMfmaFunction
 
 __all__ = ["PhysicsAttentionBase", "PhysicsAttentionIrregularMesh", "PhysicsAttentionStructuredMesh2D",
            "PhysicsAttentionStructuredMesh3D"]
@@ -153,7 +153,8 @@ class PhysicsAttentionBase(nn.Module):
         dims = self.layer_dims(x)
         if not PF.backward_supported(x.dtype, dims):
             raise RuntimeError(f"the backward kernels do not serve this shape: {dims}")
-        return PhysicsAttentionFunction.apply(
+        fn = PhysicsAttentionMfmaFunction if PF.mfma_backward_supported(x.dtype, dims) else PhysicsAttentionFunction
+        return fn.apply(
             x, dims, self.kernel_params(x.dtype, x.device), self.in_project_x.weight, self.in_project_x.bias,
             self.in_project_fx.weight, self.in_project_fx.bias, self.in_project_slice.weight,
             self.in_project_slice.bias, self.temperature, self.qkv_project.weight, self.out_linear.weight,
