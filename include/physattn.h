@@ -245,6 +245,14 @@ int pa_mfma_deslice_project(const pa_shape *shape, const void *blob, const void 
  * Same gradient as the general backward entry points above, for callers that ran the forward through the pa_mfma_*
  * stages and kept w_pack, the slice tokens and tokp.  No reference counterpart beyond autograd over PA.py:501-558. */
 int pa_mfma_backward_query(const pa_shape *shape);
+/* Weight-gradient product over the row axis (d W = d out^T . in, the adjoint of a Linear): for bf16 matrices a
+ * (rows, lda) and b (rows, ldb) in natural layout,  P[i][j] = sum_m a[m][i] * b[m][j]  for i < cols_a, j < cols_b.
+ * cols_a, cols_b multiples of 32 (cols_b in {32, 64, 128, 256}; cols_a <= 256 or a multiple of 256); lda, ldb multiples
+ * of 8.  The kernel leaves pa_cols_gemm_chunks(rows) partial results, partials (chunks, cols_a, cols_b) float32; the
+ * caller adds them up over the first index (fixed order: deterministic). */
+int64_t pa_cols_gemm_chunks(int64_t rows);
+int pa_cols_gemm(int64_t rows, const void *a, int64_t lda, int64_t cols_a, const void *b, int64_t ldb, int64_t cols_b,
+                 float *partials, void *stream);
 /* bf16 Linear over the rows of `in` (B, N, c_in) -> H*32 columns, weight (H*32, c_in) bf16, bias float32 or NULL:
  * `out` natural (B, N, H*32) and/or `out_pack` in the packed layout of PA_BUF_FX_PACK (either may be NULL). */
 int pa_rows_gemm_packed(const pa_shape *shape, int64_t c_in, const void *in, const void *weight, const float *bias,

@@ -25,6 +25,7 @@ EXPORTED = [
     "pa_slice_attention_backward", "pa_slice_softmax_backward", "pa_slice_softmax_plus",
     "pa_mfma_backward_query", "pa_rows_gemm_packed", "pa_mfma_slice_weighted_sum", "pa_mfma_deslice",
     "pa_mfma_backward_tables_bytes", "pa_mfma_backward_groups", "pa_mfma_slice_softmax_backward",
+    "pa_cols_gemm_chunks", "pa_cols_gemm",
 ]
 
 PA_BUF_BLOB, PA_BUF_FX_PACK, PA_BUF_W_PACK, PA_BUF_PARTIALS, PA_BUF_TOKP = range(5)
@@ -142,6 +143,10 @@ def load() -> ctypes.CDLL:
     lib.pa_mfma_backward_groups.argtypes = [ps]
     lib.pa_mfma_slice_softmax_backward.restype = c_int
     lib.pa_mfma_slice_softmax_backward.argtypes = [ps, pp] + [c_void_p] * 12
+    lib.pa_cols_gemm_chunks.restype = c_int64
+    lib.pa_cols_gemm_chunks.argtypes = [c_int64]
+    lib.pa_cols_gemm.restype = c_int
+    lib.pa_cols_gemm.argtypes = [c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_void_p]
     _lib = lib
     return lib
 

@@ -5,8 +5,8 @@ The reference has no backward code of its own (autograd differentiates physics_a
 this is the same gradient, assembled from
   * hand-written kernels for everything specific to the layer (slice softmax, slice sums, slice attention,
     deslice and their adjoints, the input-gradient GEMMs / transposed convolutions), and
-  * the GEMM library behind ``torch.matmul`` for the weight gradients, which are plain ``d out^T . in`` products
-    over the point axis.
+  * the weight gradients ``d out^T . in`` (products over the point axis) on the library's own MFMA kernel for bf16
+    shapes it serves, and on the GEMM library behind ``torch.matmul`` otherwise (fp32, convolutions, odd widths).
 """
 from __future__ import annotations
 
@@ -19,6 +19,13 @@ from . import functional as PF
 
 def _rows(t: torch.Tensor) -> torch.Tensor:
     return t.reshape(-1, t.shape[-1])
+
+
+def _wgrad(d_out: torch.Tensor, inp: torch.Tensor) -> torch.Tensor:
+    """d W = d out^T . in over all rows: the library's MFMA kernel where it serves the shape, else the GEMM library."""
+    if PF.cols_gemm_supported(d_out, inp):
+        return PF.cols_gemm(d_out, inp)
+    return _rows(d_out).t() @ _rows(inp)
 
 
 def _conv_weight_grad(d_out: torch.Tensor, x: torch.Tensor, grid: tuple, k: int) -> torch.Tensor:
@@ -46,9 +53,9 @@ def _finish_backward(ctx, x, dy, out_x, d_wqkv, d_proj, d_z, d_temp, x_mid, temp
     B, N, C, H, D, S = dims.B, dims.N, dims.C, dims.H, dims.D, dims.S
     HD = H * D
     linear = PF.LayerDims(B, N, C, H, D, S)
-    d_wo = _rows(dy).t() @ _rows(out_x)
+    d_wo = _wgrad(dy, out_x)
     d_bo = _rows(dy).sum(0, dtype=torch.float32)
-    d_ws = d_z.reshape(-1, S).t() @ x_mid.reshape(-1, D)
+    d_ws = _wgrad(d_z.reshape(-1, S), x_mid.reshape(-1, D))
     d_bs = d_z.reshape(-1, S).sum(0, dtype=torch.float32)
     t = temperature.reshape(-1)
     d_temp = d_temp * ((t >= 0.5) & (t <= 5.0)).to(d_temp.dtype)
@@ -58,7 +65,7 @@ def _finish_backward(ctx, x, dy, out_x, d_wqkv, d_proj, d_z, d_temp, x_mid, temp
     if k == 0:
         w_cat = torch.cat([wx.view(HD, C).t(), wf.view(HD, C).t()], dim=1).contiguous()  # (C, 2HD)
         dx = PF.rows_gemm(d_proj, w_cat, None, linear, 2 * HD, C) if ctx.needs_input_grad[0] else None
-        d_w_in = _rows(d_proj).t() @ _rows(x)  # (2HD, C)
+        d_w_in = _wgrad(d_proj, x)  # (2HD, C)
     else:
         grid = (dims.grid_h, dims.grid_w) + ((dims.grid_d,) if dims.grid_d > 0 else ())
         taps = (k,) * len(grid)

@@ -186,6 +186,265 @@ __global__ __launch_bounds__(256) void rows_gemm_mfma_kernel(GemmArgs a) {
   }
 }
 
+// ------------------------------------------------------------------------------------------------
+// rows_linear_kernel: the bf16 Linear over very many rows, weights stationary.  out = in . W^T + bias with
+// K = 16 * KS in {128, 256, 512} and up to 256 output columns per workgroup (grid.y walks wider outputs, grid.z the
+// second (W, bias, out) set).  One wave per 32 output columns keeps its W rows in registers (KS operand fragments) for
+// the whole kernel; the workgroup walks the 32-row tiles g, g + G, ... of its batch range; a tile's rows are staged in
+// LDS by the whole workgroup with full-row coalesced loads ([row][unit] with one unit of stagger per row, see above)
+// and read back as operand fragments by every wave; the next tile is fetched into registers while the current one is
+// multiplied.  The product is formed as out^T (channels x rows: lanes <-> rows, registers <-> channels) so that a
+// row's 32 channels leave as 16-byte stores; with packing on, the un-transposed tile (lanes <-> channels) is formed
+// as well and written in the packed operand layout of the slice kernels.
+// Rows are numbered as in rows_gemm_mfma_kernel (padded per batch when pack_tpb > 0).
+// ------------------------------------------------------------------------------------------------
+template <int KS>
+__global__ __launch_bounds__(512) void rows_linear_kernel(GemmArgs a) {
+  constexpr int K = 16 * KS, UPR = K / 8, ROWU = UPR + 1;
+  extern __shared__ u32x4 xs_all[];
+  u32x4(*xs)[32 * ROWU] = reinterpret_cast<u32x4(*)[32 * ROWU]>(xs_all);  // two tile buffers
+  const int z = blockIdx.z;
+  const uint16_t *in = static_cast<const uint16_t *>(a.in);
+  const uint16_t *W = static_cast<const uint16_t *>(a.w[z]);
+  uint16_t *out = static_cast<uint16_t *>(a.out[z]);
+  u32x4 *pk = static_cast<u32x4 *>(a.out_pack[z]);
+  const int tid = threadIdx.x, lane = tid & 63, i = lane & 31, g = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int NT = blockDim.x;
+  const int o0 = blockIdx.y * 256 + wave * 32;  // this wave's output columns
+
+  u32x4 wf[KS];  // W[o0 + i][16 ks + 8 g + j]: the A operand of out^T and the B operand of the un-transposed tile
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks)
+    wf[ks] = *reinterpret_cast<const u32x4 *>(W + (int64_t)(o0 + i) * K + 16 * ks + 8 * g);
+  float bias_t[16];  // bias of channel rowmap(r, g) (out^T: registers <-> channels)
+#pragma unroll
+  for (int r = 0; r < 16; ++r) bias_t[r] = a.bias[z] ? a.bias[z][o0 + mfma::rowmap(r, g)] : 0.f;
+  const float bias_n = a.bias[z] ? a.bias[z][o0 + i] : 0.f;
+
+  const int64_t padded = (int64_t)a.pack_tpb * 32;
+  const int64_t ntiles = a.pack_tpb > 0 ? (a.M / a.N) * a.pack_tpb : (a.M + 31) / 32;
+  auto real_row = [&](int64_t vm) -> int64_t {
+    if (a.pack_tpb == 0) return vm < a.M ? vm : -1;
+    const int64_t b = vm / padded, n = vm - b * padded;
+    return (n < a.N && b * a.N + n < a.M) ? b * a.N + n : -1;
+  };
+  // staging: unit idx = k * NT + tid of the tile -> row idx / UPR, position idx % UPR; 32 * UPR units per tile
+  const int per_thread = (32 * UPR + NT - 1) / NT;
+  u32x4 stg[4];  // per_thread <= 4 for every supported (K, workgroup size) pair
+  auto stage_load = [&](int64_t tile) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int idx = k * NT + tid;
+      stg[k] = u32x4{0, 0, 0, 0};
+      if (k < per_thread && idx < 32 * UPR) {
+        const int rc = idx / UPR, pos = idx - rc * UPR;
+        const int64_t m = real_row(tile * 32 + rc);
+        if (m >= 0) stg[k] = *reinterpret_cast<const u32x4 *>(in + m * K + pos * 8);
+      }
+    }
+  };
+  auto stage_store = [&](int buf) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int idx = k * NT + tid;
+      if (k < per_thread && idx < 32 * UPR) {
+        const int rc = idx / UPR, pos = idx - rc * UPR;
+        xs[buf][rc * ROWU + pos] = stg[k];
+      }
+    }
+  };
+
+  int64_t tile = blockIdx.x;
+  if (tile < ntiles) {
+    stage_load(tile);
+    stage_store(0);
+  }
+  __syncthreads();
+  int buf = 0;
+  for (; tile < ntiles; tile += gridDim.x, buf ^= 1) {
+    const int64_t next = tile + gridDim.x < ntiles ? tile + gridDim.x : tile;  // the last tile re-fetches itself
+    stage_load(next);
+    const u32x4 *xb = &xs[buf][i * ROWU + g];
+    f32x16 acc_t, acc_n;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      acc_t[r] = bias_t[r];
+      acc_n[r] = bias_n;
+    }
+    if (pk) {
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const u32x4 xf = xb[2 * ks];
+        acc_t = mfma::mma(wf[ks], xf, acc_t);
+        acc_n = mfma::mma(xf, wf[ks], acc_n);
+      }
+    } else {
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) acc_t = mfma::mma(wf[ks], xb[2 * ks], acc_t);
+    }
+    if (out) {
+      const int64_t m = real_row(tile * 32 + i);
+      mfma::store_tile_natural(acc_t, out + (m >= 0 ? m : 0) * a.O + o0, g, m >= 0);
+    }
+    if (pk) {
+      const int head = o0 >> 5;
+      pk[((tile * a.pack_heads + head) * 2 + 0) * 64 + lane] = mfma::pack_half<0>(acc_n);
+      pk[((tile * a.pack_heads + head) * 2 + 1) * 64 + lane] = mfma::pack_half<1>(acc_n);
+    }
+    stage_store(buf ^ 1);
+    __syncthreads();
+  }
+}
+
+bool linear_serves(const GemmArgs &a, int nsets, size_t elem_bytes) {
+  if (elem_bytes != 2 || a.ks != 0) return false;
+  if (a.K != 128 && a.K != 256 && a.K != 512) return false;
+  if (a.O % 32 != 0 || (a.O > 256 && a.O % 256 != 0)) return false;
+  if (a.M < 4096) return false;  // small problems: the tiled kernel has less fixed cost
+  if ((a.O < 256 ? a.O : 256) * 2 < a.K) return false;  // staging: at most 4 units per thread and tile
+  if (!aligned16(a.in)) return false;
+  for (int z = 0; z < nsets; ++z)
+    if (!aligned16(a.w[z]) || !aligned16(a.out[z]) || (!a.out[z] && !a.out_pack[z])) return false;
+  return true;
+}
+
+int linear_launch(const GemmArgs &a, int nsets, int num_cu, hipStream_t st) {
+  const int64_t ntiles = a.pack_tpb > 0 ? (a.M / a.N) * a.pack_tpb : (a.M + 31) / 32;
+  const int waves = (a.O < 256 ? a.O : 256) / 32;
+  // resident workgroups: the register-held weights leave room for one 8-wave workgroup per CU (two for K = 128)
+  int64_t gx = (a.K == 128 ? 2 : 1) * (int64_t)num_cu / (((a.O + 255) / 256) * nsets);
+  if (gx < 1) gx = 1;
+  if (gx > ntiles) gx = ntiles;
+  const dim3 grid((unsigned)gx, (unsigned)((a.O + 255) / 256), (unsigned)nsets), block((unsigned)(waves * 64));
+  const size_t lds = (size_t)2 * 32 * (a.K / 8 + 1) * 16;
+  if (lds > 48 * 1024 &&
+      hipFuncSetAttribute(reinterpret_cast<const void *>(rows_linear_kernel<32>),
+                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+    return PA_ERR_UNSUPPORTED;
+  switch (a.K) {
+    case 128: hipLaunchKernelGGL((rows_linear_kernel<8>), grid, block, lds, st, a); break;
+    case 256: hipLaunchKernelGGL((rows_linear_kernel<16>), grid, block, lds, st, a); break;
+    case 512: hipLaunchKernelGGL((rows_linear_kernel<32>), grid, block, lds, st, a); break;
+    default: return PA_ERR_UNSUPPORTED;
+  }
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? PA_OK : (int)e;
+}
+
+// ------------------------------------------------------------------------------------------------
+// cols_gemm_kernel: weight-gradient products  P[oa][ob] = sum_m A[m][oa] * B[m][ob]  over a huge row count m (bf16
+// rows in natural layout, fp32 result).  grid (G row chunks, OA / 256); workgroup = one wave per 32 columns of A (up to
+// 8); wave w owns output rows 32w..32w+31 and all NB = OB / 32 column groups.  Both operands have the reduction index m
+// as their slow index in memory, so each 32-row block is transposed on the matrix cores first: the natural 16-byte
+// loads are MFMA A operands (lane <-> row m, k <-> channel); multiplied by 0/1 selection matrices they give an exact copy
+// of the block with lanes <-> channels and registers <-> rows, which, converted back to bf16, is an operand whose
+// reduction index is m.  Every wave transposes its own A group; the B groups are transposed once per workgroup and
+// shared through LDS (double buffered, one barrier per block).  Each chunk leaves one partial result
+// partials[g][oa][ob]; the caller adds the G partials up in index order.
+// ------------------------------------------------------------------------------------------------
+template <int NB>
+__global__ __launch_bounds__(512) void cols_gemm_kernel(const uint16_t *__restrict__ A, int lda, int OA,
+                                                        const uint16_t *__restrict__ B, int ldb, int64_t M,
+                                                        int64_t blocks_per_chunk, float *__restrict__ partials) {
+  constexpr int OB = 32 * NB;
+  __shared__ u32x4 bts[2][NB * 2 * 64];
+  const int tid = threadIdx.x, lane = tid & 63, i = lane & 31, g = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int nwaves = blockDim.x >> 6;
+  const int a0 = blockIdx.y * 256 + wave * 32;  // first A column of this wave
+
+  u32x4 sel[2];  // sel[kk]: column i receives the k element whose channel is 16kk + 8g + j
+#pragma unroll
+  for (int kk = 0; kk < 2; ++kk) {
+    mfma::bf16x8 s8;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) s8[j] = (__bf16)((i == 16 * kk + 8 * g + j) ? 1.f : 0.f);
+    sel[kk] = __builtin_bit_cast(u32x4, s8);
+  }
+  // a 32 x 32 block (rows m0.., columns c0..) of a natural-layout matrix -> two operands whose k index runs over m
+  auto transposed = [&](const uint16_t *base, int ld, int64_t m0, int c0, u32x4 &t0, u32x4 &t1) {
+    const int64_t m = m0 + i;
+    u32x4 f0 = u32x4{0, 0, 0, 0}, f1 = f0;
+    if (m < M) {
+      const uint16_t *row = base + m * ld + c0 + 8 * g;
+      f0 = *reinterpret_cast<const u32x4 *>(row);
+      f1 = *reinterpret_cast<const u32x4 *>(row + 16);
+    }
+    f32x16 t;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) t[r] = 0.f;
+    t = mfma::mma(f0, sel[0], t);
+    t = mfma::mma(f1, sel[1], t);
+    t0 = mfma::pack_half<0>(t);
+    t1 = mfma::pack_half<1>(t);
+  };
+
+  f32x16 acc[NB];
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[nb][r] = 0.f;
+
+  const int64_t blk0 = (int64_t)blockIdx.x * blocks_per_chunk;
+  const int64_t nblk = (M + 31) / 32;
+  int64_t blk_end = blk0 + blocks_per_chunk;
+  if (blk_end > nblk) blk_end = nblk;
+  int buf = 0;
+  for (int64_t blk = blk0; blk < blk_end; ++blk, buf ^= 1) {
+    const int64_t m0 = blk * 32;
+    u32x4 at0, at1;
+    transposed(A, lda, m0, a0, at0, at1);
+    for (int nb = wave; nb < NB; nb += nwaves) {
+      u32x4 b0, b1;
+      transposed(B, ldb, m0, 32 * nb, b0, b1);
+      bts[buf][(nb * 2 + 0) * 64 + lane] = b0;
+      bts[buf][(nb * 2 + 1) * 64 + lane] = b1;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+      acc[nb] = mfma::mma(at0, bts[buf][(nb * 2 + 0) * 64 + lane], acc[nb]);
+      acc[nb] = mfma::mma(at1, bts[buf][(nb * 2 + 1) * 64 + lane], acc[nb]);
+    }
+  }
+  float *dst = partials + ((int64_t)blockIdx.x * OA + a0) * OB;
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) dst[(int64_t)mfma::rowmap(r, g) * OB + 32 * nb + i] = acc[nb][r];
+}
+
+int64_t cols_gemm_chunks(int64_t M, int num_cu) {
+  const int64_t nblk = (M + 31) / 32;
+  int64_t g = 2 * (int64_t)num_cu;
+  if (g > nblk) g = nblk;
+  return g < 1 ? 1 : g;
+}
+
+int cols_gemm(const void *A, int64_t lda, int64_t OA, const void *B, int64_t ldb, int64_t OB, int64_t M,
+              float *partials, int num_cu, hipStream_t st) {
+  if (OA % 32 != 0 || OB % 32 != 0 || OA <= 0 || OB <= 0 || lda % 8 != 0 || ldb % 8 != 0) return PA_ERR_UNSUPPORTED;
+  if (OA > 256 && OA % 256 != 0) return PA_ERR_UNSUPPORTED;
+  const int64_t G = cols_gemm_chunks(M, num_cu);
+  const int64_t nblk = (M + 31) / 32;
+  const int64_t per = (nblk + G - 1) / G;
+  const dim3 grid((unsigned)G, (unsigned)((OA + 255) / 256)), block((unsigned)((OA < 256 ? OA : 256) * 2));
+  const uint16_t *a = static_cast<const uint16_t *>(A), *b = static_cast<const uint16_t *>(B);
+#define PA_COLS(NBV) \
+  hipLaunchKernelGGL((cols_gemm_kernel<NBV>), grid, block, 0, st, a, (int)lda, (int)OA, b, (int)ldb, M, per, partials)
+  switch (OB / 32) {
+    case 1: PA_COLS(1); break;
+    case 2: PA_COLS(2); break;
+    case 4: PA_COLS(4); break;
+    case 8: PA_COLS(8); break;
+    default: return PA_ERR_UNSUPPORTED;
+  }
+#undef PA_COLS
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? PA_OK : (int)e;
+}
+
 bool serves(const GemmArgs &a, int nsets, size_t elem_bytes) {
   const int ue = (int)(16 / elem_bytes);
   if (a.K % ue != 0) return false;                      // rows must be whole 16-byte units
@@ -213,6 +472,13 @@ static int launch_n(const GemmArgs &a, int nsets, hipStream_t st) {
 }
 
 int launch(const GemmArgs &a, int nsets, int dtype, hipStream_t st) {
+  if (dtype == PA_BF16 && linear_serves(a, nsets, 2)) {
+    int dev = 0, cus = 256;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+      cus = 256;
+    return linear_launch(a, nsets, cus, st);
+  }
   return dtype == PA_F32 ? launch_n<float>(a, nsets, st) : launch_n<bf16>(a, nsets, st);
 }
 

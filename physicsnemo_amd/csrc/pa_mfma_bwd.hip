@@ -17,34 +17,6 @@
 namespace pa {
 namespace mfma {
 
-// A 32 x 32 accumulator tile (lane (i, g) <-> point i, register r <-> channel rowmap(r, g)) to bf16 rows in natural
-// layout: `row` points at channel 0 of this lane's point.  Registers 4q..4q+3 hold channels 8q + 4g .. + 3; swapping
-// halves with lane ^ 32 gives each lane 8 consecutive channels (g = 0: 0-7 and 8-15, g = 1: 16-23 and 24-31), so a
-// point's 64 bytes leave as four 16-byte stores.  `nch` = valid channels (32, or 16: the lower half only).
-__device__ __forceinline__ void store_tile_natural(const f32x16 &v, uint16_t *row, int g, bool ok, int nch = 32) {
-  uint32_t p[4][2];
-#pragma unroll
-  for (int q = 0; q < 4; ++q)
-#pragma unroll
-    for (int w = 0; w < 2; ++w)
-      p[q][w] = (uint32_t)to_bf16_bits(v[4 * q + 2 * w]) | ((uint32_t)to_bf16_bits(v[4 * q + 2 * w + 1]) << 16);
-  u32x4 s0, s1;
-#pragma unroll
-  for (int w = 0; w < 2; ++w) {
-    // lower half-wave: (own piece 0, partner's piece 0); upper half-wave: (partner's piece 2, own piece 2)
-    const auto a = __builtin_amdgcn_permlane32_swap(p[0][w], p[2][w], false, false);
-    s0[w] = a[0];
-    s0[2 + w] = a[1];
-    const auto b = __builtin_amdgcn_permlane32_swap(p[1][w], p[3][w], false, false);
-    s1[w] = b[0];
-    s1[2 + w] = b[1];
-  }
-  if (ok && (g == 0 || nch > 16)) {
-    *reinterpret_cast<u32x4 *>(row + 16 * g) = s0;
-    *reinterpret_cast<u32x4 *>(row + 16 * g + 8) = s1;
-  }
-}
-
 // ------------------------------------------------------------------------------------------------
 // deslice_natural_kernel: grid (G, B), H waves; wave h walks the batch's tiles g, g + G, ...
 //   out_x^T_h (32 d x 32 pts) = tok'^T_h (A: tokp fragments, registers) . w_h (B: w_pack chunks)

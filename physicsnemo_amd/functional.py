@@ -339,6 +339,29 @@ def mfma_backward_supported(dtype: torch.dtype, dims: LayerDims) -> bool:
     return bool(rc)
 
 
+def cols_gemm_supported(a: torch.Tensor, b: torch.Tensor) -> bool:
+    ca, cb = a.shape[-1], b.shape[-1]
+    return (a.dtype == torch.bfloat16 and b.dtype == torch.bfloat16 and a.is_cuda and ca % 32 == 0
+            and (ca <= 256 or ca % 256 == 0) and cb in (32, 64, 128, 256))
+
+
+def cols_gemm(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    """a^T . b over the leading (row) axes: bf16 (..., ca) and (..., cb) with equal row counts -> float32 (ca, cb).
+
+    The weight-gradient product d W = d out^T . in on the MFMA kernel `cols_gemm_kernel`."""
+    _need_cuda(a, b)
+    lib = _lib.load()
+    ca, cb = a.shape[-1], b.shape[-1]
+    rows = a.numel() // ca
+    if b.numel() // cb != rows:
+        raise ValueError("cols_gemm needs the same number of rows on both sides")
+    chunks = lib.pa_cols_gemm_chunks(rows)
+    partials = torch.empty(int(chunks), ca, cb, dtype=torch.float32, device=a.device)
+    _lib.check(lib.pa_cols_gemm(rows, a.data_ptr(), ca, ca, b.data_ptr(), cb, cb, partials.data_ptr(),
+                                _lib.current_stream_ptr(a.device)), "pa_cols_gemm")
+    return partials.sum(0)
+
+
 def rows_gemm(inp, weight, bias, dims: LayerDims, c_in: int, c_out: int):
     """out (B, N, c_out) = Linear or grid convolution of inp (B, N, c_in); `dims` supplies B, N and the grid."""
     _need_cuda(inp, weight, bias)

@@ -199,3 +199,17 @@ def test_mfma_deslice_natural_layout():
         want_sums = torch.einsum("bnhs,bnhd->bhsd", stages["w"], (x @ w.float().cpu().t()).reshape(2, 500, 8, 32))
         assert_rel_l2(sums[..., :32], want_sums, "slice sums of the packed GEMM output")
         assert_rel_l2(sums[..., 32], stages["w"].sum(1), "slice counts")
+
+
+@pytest.mark.parametrize("rows,ca,cb", [(5000, 64, 32), (1000, 256, 256), (333, 512, 256), (31, 32, 32), (70000, 256, 128)])
+def test_cols_gemm_weight_gradient_product(rows, ca, cb):
+    announce("cols_gemm", rows, ca, cb)
+    torch.manual_seed(rows)
+    a = torch.randn(rows, ca, device="cuda").bfloat16()
+    b = torch.randn(rows, cb, device="cuda").bfloat16()
+    assert PF.cols_gemm_supported(a, b)
+    got = PF.cols_gemm(a, b)
+    want = a.double().t() @ b.double()  # exact products of the bf16 inputs; the kernel accumulates them in fp32
+    assert got.shape == (ca, cb) and got.dtype == torch.float32
+    assert_fp32_close(got, want.float(), "a^T b", rtol=1e-4)
+    assert torch.equal(got, PF.cols_gemm(a, b))  # fixed summation order
