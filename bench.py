@@ -138,8 +138,8 @@ def time_block_mlp(rows, C, hidden, reps=10):
 
 
 def time_training_step(points, C, S, reps=3):
-    """Forward + backward of one layer under bf16 autocast at the layer workload's size: the differentiable path
-    (stage-level kernels forward, backward kernels + GEMM-library weight gradients backward)."""
+    """Forward + backward of one layer under bf16 autocast at the layer workload's size (gradients w.r.t. the input
+    and all ten parameters)."""
     import torch
 
     import physicsnemo_amd as pn
@@ -167,7 +167,8 @@ def time_training_step(points, C, S, reps=3):
     assert torch.isfinite(x.grad[:, :1024].float()).all()
     return {"workload": f"layer forward + backward, {points} points, C={C}, S={S}, bf16 autocast",
             "ms_per_step": round(ms, 3), "mpoints_per_s": round(points / (ms * 1e-3) / 1e6, 2),
-            "kernels": "general (fp32 FMA) stage and backward kernels; weight gradients via the GEMM library"}
+            "kernels": "MFMA forward kernels; backward: weights-stationary row GEMMs, packed slice sum, per-point MFMA "
+                       "backward kernel, split-row MFMA weight-gradient kernel"}
 
 
 def time_full_model(name, B, N, functional_dim, embedding_dim, slice_num, n_layers, steps=5, warmup=2):

@@ -249,10 +249,11 @@ int pa_mfma_backward_query(const pa_shape *shape);
  * (rows, lda) and b (rows, ldb) in natural layout,  P[i][j] = sum_m a[m][i] * b[m][j]  for i < cols_a, j < cols_b.
  * cols_a, cols_b multiples of 32 (cols_b in {32, 64, 128, 256}; cols_a <= 256 or a multiple of 256); lda, ldb multiples
  * of 8.  The kernel leaves pa_cols_gemm_chunks(rows) partial results, partials (chunks, cols_a, cols_b) float32; the
- * caller adds them up over the first index (fixed order: deterministic). */
+ * caller adds them up over the first index (fixed order: deterministic).  col_sum_partials (chunks, cols_a) float32,
+ * optional (NULL to skip): the column sums of a, i.e. the bias gradient that goes with the weight gradient. */
 int64_t pa_cols_gemm_chunks(int64_t rows);
 int pa_cols_gemm(int64_t rows, const void *a, int64_t lda, int64_t cols_a, const void *b, int64_t ldb, int64_t cols_b,
-                 float *partials, void *stream);
+                 float *partials, float *col_sum_partials, void *stream);
 /* bf16 Linear over the rows of `in` (B, N, c_in) -> H*32 columns, weight (H*32, c_in) bf16, bias float32 or NULL:
  * `out` natural (B, N, H*32) and/or `out_pack` in the packed layout of PA_BUF_FX_PACK (either may be NULL). */
 int pa_rows_gemm_packed(const pa_shape *shape, int64_t c_in, const void *in, const void *weight, const float *bias,

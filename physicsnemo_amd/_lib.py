@@ -146,7 +146,7 @@ def load() -> ctypes.CDLL:
     lib.pa_cols_gemm_chunks.restype = c_int64
     lib.pa_cols_gemm_chunks.argtypes = [c_int64]
     lib.pa_cols_gemm.restype = c_int
-    lib.pa_cols_gemm.argtypes = [c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_void_p]
+    lib.pa_cols_gemm.argtypes = [c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_void_p]
     _lib = lib
     return lib
 

@@ -21,11 +21,12 @@ def _rows(t: torch.Tensor) -> torch.Tensor:
     return t.reshape(-1, t.shape[-1])
 
 
-def _wgrad(d_out: torch.Tensor, inp: torch.Tensor) -> torch.Tensor:
-    """d W = d out^T . in over all rows: the library's MFMA kernel where it serves the shape, else the GEMM library."""
+def _wgrad(d_out: torch.Tensor, inp: torch.Tensor):
+    """(d W, d b) = (d out^T . in, column sums of d out) over all rows: one pass of the library's MFMA kernel where it
+    serves the shape, else the GEMM library and a reduction."""
     if PF.cols_gemm_supported(d_out, inp):
-        return PF.cols_gemm(d_out, inp)
-    return _rows(d_out).t() @ _rows(inp)
+        return PF.cols_gemm(d_out, inp, col_sums=True)
+    return _rows(d_out).t() @ _rows(inp), _rows(d_out).sum(0, dtype=torch.float32)
 
 
 def _conv_weight_grad(d_out: torch.Tensor, x: torch.Tensor, grid: tuple, k: int) -> torch.Tensor:
@@ -53,10 +54,8 @@ def _finish_backward(ctx, x, dy, out_x, d_wqkv, d_proj, d_z, d_temp, x_mid, temp
     B, N, C, H, D, S = dims.B, dims.N, dims.C, dims.H, dims.D, dims.S
     HD = H * D
     linear = PF.LayerDims(B, N, C, H, D, S)
-    d_wo = _wgrad(dy, out_x)
-    d_bo = _rows(dy).sum(0, dtype=torch.float32)
-    d_ws = _wgrad(d_z.reshape(-1, S), x_mid.reshape(-1, D))
-    d_bs = d_z.reshape(-1, S).sum(0, dtype=torch.float32)
+    d_wo, d_bo = _wgrad(dy, out_x)
+    d_ws, d_bs = _wgrad(d_z.reshape(-1, S), x_mid.reshape(-1, D))
     t = temperature.reshape(-1)
     d_temp = d_temp * ((t >= 0.5) & (t <= 5.0)).to(d_temp.dtype)
 
@@ -65,7 +64,7 @@ def _finish_backward(ctx, x, dy, out_x, d_wqkv, d_proj, d_z, d_temp, x_mid, temp
     if k == 0:
         w_cat = torch.cat([wx.view(HD, C).t(), wf.view(HD, C).t()], dim=1).contiguous()  # (C, 2HD)
         dx = PF.rows_gemm(d_proj, w_cat, None, linear, 2 * HD, C) if ctx.needs_input_grad[0] else None
-        d_w_in = _wgrad(d_proj, x)  # (2HD, C)
+        d_w_in, d_b_in = _wgrad(d_proj, x)  # (2HD, C), (2HD)
     else:
         grid = (dims.grid_h, dims.grid_w) + ((dims.grid_d,) if dims.grid_d > 0 else ())
         taps = (k,) * len(grid)
@@ -74,7 +73,7 @@ def _finish_backward(ctx, x, dy, out_x, d_wqkv, d_proj, d_z, d_temp, x_mid, temp
         w_t = w_both.flip(dims=tuple(range(2, 2 + len(grid)))).transpose(0, 1).contiguous()
         dx = PF.rows_gemm(d_proj, w_t, None, dims, 2 * HD, C) if ctx.needs_input_grad[0] else None
         d_w_in = _conv_weight_grad(d_proj, x, grid, k)
-    d_b_in = _rows(d_proj).sum(0, dtype=torch.float32)
+        d_b_in = _rows(d_proj).sum(0, dtype=torch.float32)
 
     grads = (d_w_in[:HD], d_b_in[:HD], d_w_in[HD:], d_b_in[HD:], d_ws, d_bs, d_temp, d_wqkv, d_wo, d_bo)
     grads = tuple(gr.reshape(p.shape).to(p.dtype) if ctx.needs_input_grad[3 + i] else None

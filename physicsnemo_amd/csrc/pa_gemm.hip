@@ -346,7 +346,8 @@ int linear_launch(const GemmArgs &a, int nsets, int num_cu, hipStream_t st) {
 template <int NB>
 __global__ __launch_bounds__(512) void cols_gemm_kernel(const uint16_t *__restrict__ A, int lda, int OA,
                                                         const uint16_t *__restrict__ B, int ldb, int64_t M,
-                                                        int64_t blocks_per_chunk, float *__restrict__ partials) {
+                                                        int64_t blocks_per_chunk, float *__restrict__ partials,
+                                                        float *__restrict__ col_sums) {
   constexpr int OB = 32 * NB;
   __shared__ u32x4 bts[2][NB * 2 * 64];
   const int tid = threadIdx.x, lane = tid & 63, i = lane & 31, g = lane >> 5;
@@ -380,11 +381,14 @@ __global__ __launch_bounds__(512) void cols_gemm_kernel(const uint16_t *__restri
     t1 = mfma::pack_half<1>(t);
   };
 
-  f32x16 acc[NB];
+  f32x16 acc[NB], acc_s;  // acc_s: A^T . 1 (every column the same): the column sums of A
+#pragma unroll
+  for (int r = 0; r < 16; ++r) acc_s[r] = 0.f;
 #pragma unroll
   for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[nb][r] = 0.f;
+  const u32x4 ones = u32x4{0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u};  // 8 x bf16(1.0)
 
   const int64_t blk0 = (int64_t)blockIdx.x * blocks_per_chunk;
   const int64_t nblk = (M + 31) / 32;
@@ -395,6 +399,10 @@ __global__ __launch_bounds__(512) void cols_gemm_kernel(const uint16_t *__restri
     const int64_t m0 = blk * 32;
     u32x4 at0, at1;
     transposed(A, lda, m0, a0, at0, at1);
+    if (col_sums) {
+      acc_s = mfma::mma(at0, ones, acc_s);
+      acc_s = mfma::mma(at1, ones, acc_s);
+    }
     for (int nb = wave; nb < NB; nb += nwaves) {
       u32x4 b0, b1;
       transposed(B, ldb, m0, 32 * nb, b0, b1);
@@ -413,6 +421,10 @@ __global__ __launch_bounds__(512) void cols_gemm_kernel(const uint16_t *__restri
   for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
     for (int r = 0; r < 16; ++r) dst[(int64_t)mfma::rowmap(r, g) * OB + 32 * nb + i] = acc[nb][r];
+  if (col_sums && i == 0) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) col_sums[(int64_t)blockIdx.x * OA + a0 + mfma::rowmap(r, g)] = acc_s[r];
+  }
 }
 
 int64_t cols_gemm_chunks(int64_t M, int num_cu) {
@@ -423,7 +435,7 @@ int64_t cols_gemm_chunks(int64_t M, int num_cu) {
 }
 
 int cols_gemm(const void *A, int64_t lda, int64_t OA, const void *B, int64_t ldb, int64_t OB, int64_t M,
-              float *partials, int num_cu, hipStream_t st) {
+              float *partials, float *col_sums, int num_cu, hipStream_t st) {
   if (OA % 32 != 0 || OB % 32 != 0 || OA <= 0 || OB <= 0 || lda % 8 != 0 || ldb % 8 != 0) return PA_ERR_UNSUPPORTED;
   if (OA > 256 && OA % 256 != 0) return PA_ERR_UNSUPPORTED;
   const int64_t G = cols_gemm_chunks(M, num_cu);
@@ -432,7 +444,7 @@ int cols_gemm(const void *A, int64_t lda, int64_t OA, const void *B, int64_t ldb
   const dim3 grid((unsigned)G, (unsigned)((OA + 255) / 256)), block((unsigned)((OA < 256 ? OA : 256) * 2));
   const uint16_t *a = static_cast<const uint16_t *>(A), *b = static_cast<const uint16_t *>(B);
 #define PA_COLS(NBV) \
-  hipLaunchKernelGGL((cols_gemm_kernel<NBV>), grid, block, 0, st, a, (int)lda, (int)OA, b, (int)ldb, M, per, partials)
+  hipLaunchKernelGGL((cols_gemm_kernel<NBV>), grid, block, 0, st, a, (int)lda, (int)OA, b, (int)ldb, M, per, partials, col_sums)
   switch (OB / 32) {
     case 1: PA_COLS(1); break;
     case 2: PA_COLS(2); break;

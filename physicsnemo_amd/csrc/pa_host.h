@@ -41,7 +41,7 @@ int launch(const GemmArgs &a, int nsets, int dtype, hipStream_t st);
 // weight-gradient products over the row axis: partials[g][oa][ob] = sum over chunk g of A[m][oa] * B[m][ob] (bf16 in)
 int64_t cols_gemm_chunks(int64_t M, int num_cu);
 int cols_gemm(const void *A, int64_t lda, int64_t OA, const void *B, int64_t ldb, int64_t OB, int64_t M,
-              float *partials, int num_cu, hipStream_t st);
+              float *partials, float *col_sums, int num_cu, hipStream_t st);
 }  // namespace gemm
 
 namespace general {

@@ -345,10 +345,11 @@ def cols_gemm_supported(a: torch.Tensor, b: torch.Tensor) -> bool:
             and (ca <= 256 or ca % 256 == 0) and cb in (32, 64, 128, 256))
 
 
-def cols_gemm(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+def cols_gemm(a: torch.Tensor, b: torch.Tensor, col_sums: bool = False):
     """a^T . b over the leading (row) axes: bf16 (..., ca) and (..., cb) with equal row counts -> float32 (ca, cb).
 
-    The weight-gradient product d W = d out^T . in on the MFMA kernel `cols_gemm_kernel`."""
+    The weight-gradient product d W = d out^T . in on the MFMA kernel `cols_gemm_kernel`; with `col_sums` the column
+    sums of a (the matching bias gradient) come back as well, from the same pass."""
     _need_cuda(a, b)
     lib = _lib.load()
     ca, cb = a.shape[-1], b.shape[-1]
@@ -357,9 +358,10 @@ def cols_gemm(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
         raise ValueError("cols_gemm needs the same number of rows on both sides")
     chunks = lib.pa_cols_gemm_chunks(rows)
     partials = torch.empty(int(chunks), ca, cb, dtype=torch.float32, device=a.device)
-    _lib.check(lib.pa_cols_gemm(rows, a.data_ptr(), ca, ca, b.data_ptr(), cb, cb, partials.data_ptr(),
+    sums = torch.empty(int(chunks), ca, dtype=torch.float32, device=a.device) if col_sums else None
+    _lib.check(lib.pa_cols_gemm(rows, a.data_ptr(), ca, ca, b.data_ptr(), cb, cb, partials.data_ptr(), _lib.ptr(sums),
                                 _lib.current_stream_ptr(a.device)), "pa_cols_gemm")
-    return partials.sum(0)
+    return (partials.sum(0), sums.sum(0)) if col_sums else partials.sum(0)
 
 
 def rows_gemm(inp, weight, bias, dims: LayerDims, c_in: int, c_out: int):

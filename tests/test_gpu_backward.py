@@ -208,7 +208,8 @@ def test_cols_gemm_weight_gradient_product(rows, ca, cb):
     a = torch.randn(rows, ca, device="cuda").bfloat16()
     b = torch.randn(rows, cb, device="cuda").bfloat16()
     assert PF.cols_gemm_supported(a, b)
-    got = PF.cols_gemm(a, b)
+    got, sums = PF.cols_gemm(a, b, col_sums=True)
+    assert_fp32_close(sums, a.double().sum(0).float(), "column sums of a", rtol=1e-4)
     want = a.double().t() @ b.double()  # exact products of the bf16 inputs; the kernel accumulates them in fp32
     assert got.shape == (ca, cb) and got.dtype == torch.float32
     assert_fp32_close(got, want.float(), "a^T b", rtol=1e-4)
