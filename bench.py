@@ -356,7 +356,7 @@ def main():
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "cfg3: single PhysicsAttentionIrregularMesh layer forward", "batch": B, "points": N,
                    "hidden": C, "heads": H, "dim_head": 32, "slice_num": S,
-                   "kernel_path": "mfma" if path == 1 else "general"},
+                   "kernel_path": {0: "general", 1: "mfma", 2: "mfma-staged"}[path]},
         "roofline": roofline, "kernels": kernels,
         "graph_replay": {"ms_per_step": round(ms_graph, 4), "mpoints_per_s": round(B * N / (ms_graph * 1e-3) / 1e6, 2)},
     }

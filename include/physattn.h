@@ -100,8 +100,10 @@ typedef struct pa_block_tail {
 /* Bytes of caller-provided workspace pa_layer_forward needs for this shape. Negative = error code. */
 int64_t pa_workspace_bytes(int dtype, const pa_shape *shape);
 
-/* Which kernel family serves this shape: 0 = general kernels (fp32 FMA), 1 = bf16 MFMA kernels.
- * Negative = error code.  No reference counterpart. */
+/* Which kernel family pa_layer_forward runs for this shape: 0 = general kernels, 1 = fused bf16 MFMA kernels
+ * (C in {128, 256}), 2 = staged bf16 MFMA kernels (the same arithmetic as separate launches; adds C = 512, needs
+ * B*N >= 4096).  The pa_mfma_* stage entry points serve the shapes with answer 1.  Negative = error code.
+ * No reference counterpart. */
 int pa_query_path(int dtype, const pa_shape *shape);
 
 /* ---- stage-level entry points (natural layouts; general kernels) ------------------------------ */

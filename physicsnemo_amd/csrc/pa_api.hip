@@ -109,6 +109,52 @@ MfmaPlan plan_mfma(const pa_shape &s) {
   return p;
 }
 
+// Workspace plan of the staged MFMA path.
+struct StagedPlan {
+  int64_t off_x_mid, off_fx, off_w, off_partials, off_tok, off_norm, off_tok_out, off_tokp, total;
+  int64_t G;
+};
+
+StagedPlan plan_staged(const pa_shape &s) {
+  StagedPlan p{};
+  p.G = mfma_groups(s, false);
+  const int64_t tiles = s.B * pa::mfma::tiles_per_batch(s);
+  int64_t off = 0;
+  p.off_x_mid = off;  // natural (B, N, H*32); reused for out_x once the slice weights exist
+  off += round_up(s.B * s.N * s.H * 32 * 2, 256);
+  p.off_fx = off;
+  off += round_up(tiles * s.H * 2 * 1024, 256);
+  p.off_w = off;
+  off += round_up(tiles * s.H * (s.S / 16) * 1024, 256);
+  p.off_partials = off;
+  off += round_up((p.G + 1) * s.B * s.H * s.S * (s.D + 1) * 4, 256);
+  p.off_tok = off;
+  off += round_up(s.B * s.H * s.S * s.D * 4, 256);
+  p.off_norm = off;
+  off += round_up(s.B * s.H * s.S * 4, 256);
+  p.off_tok_out = off;
+  off += round_up(s.B * s.H * s.S * s.D * 4, 256);
+  p.off_tokp = off;
+  off += round_up(s.B * s.H * (s.S / 16) * 1024, 256);
+  p.total = off;
+  return p;
+}
+
+// 0 general kernels, 1 fused MFMA kernels, 2 staged MFMA kernels
+int kernel_path(int dtype, const pa_shape &s) {
+  if (pa::mfma::supported(dtype, s)) return 1;
+  if (pa::mfma::staged_supported(dtype, s)) return 2;
+  return 0;
+}
+
+int64_t body_bytes(int dtype, const pa_shape &s) {
+  switch (kernel_path(dtype, s)) {
+    case 1: return plan_mfma(s).total;
+    case 2: return plan_staged(s).total;
+    default: return plan_general(dtype, s).total;
+  }
+}
+
 int compute_units() {
   int dev = 0, n = 0;
   if (hipGetDevice(&dev) != hipSuccess) return 256;
@@ -157,16 +203,14 @@ const char *pa_status_string(int code) {
 int pa_query_path(int dtype, const pa_shape *shape) {
   int rc = check_shape(dtype, shape);
   if (rc) return rc;
-  return pa::mfma::supported(dtype == PA_BF16_W8 ? PA_BF16 : dtype, *shape) ? 1 : 0;
+  return kernel_path(dtype == PA_BF16_W8 ? PA_BF16 : dtype, *shape);
 }
 
 int64_t pa_workspace_bytes(int dtype, const pa_shape *shape) {
   int rc = check_shape(dtype, shape);
   if (rc) return rc;
   const int act = dtype == PA_BF16_W8 ? PA_BF16 : dtype;
-  const int64_t extra = dequant_bytes(dtype, *shape);
-  if (pa::mfma::supported(act, *shape)) return plan_mfma(*shape).total + extra;
-  return plan_general(act, *shape).total + extra;
+  return body_bytes(act, *shape) + dequant_bytes(dtype, *shape);
 }
 
 int pa_project_inputs(int dtype, const pa_shape *shape, const pa_params *p, const void *x, void *x_mid, void *fx_mid,
@@ -556,7 +600,7 @@ int pa_layer_forward(int dtype, const pa_shape *shape, const pa_params *p, const
   pa_params deq;  // PA_BF16_W8: parameters with the fp8 weights expanded to bf16 in the workspace tail
   if (dtype == PA_BF16_W8) {
     if (!p->in_project_x_scale || !p->in_project_fx_scale || !p->out_linear_scale) return PA_ERR_NULL;
-    const int64_t body = pa::mfma::supported(PA_BF16, s) ? plan_mfma(s).total : plan_general(PA_BF16, s).total;
+    const int64_t body = body_bytes(PA_BF16, s);
     const int64_t one = round_up(s.H * s.D * s.C * 2, 256);
     if (workspace_bytes < body + 3 * one) return PA_ERR_WORKSPACE;
     char *w0 = ws + body;
@@ -589,6 +633,39 @@ int pa_layer_forward(int dtype, const pa_shape *shape, const pa_params *p, const
     }
     if ((rc = pa::mfma::combine_attention(s, *p, partials, mp.G, tok, norm, tok_out, tokp, st))) return rc;
     return pa::mfma::deslice_project(s, blob, wp, tokp, y, tail_active(tail) ? tail : nullptr, compute_units(), st);
+  }
+  if (pa::mfma::staged_supported(dtype, s)) {
+    const StagedPlan sp = plan_staged(s);
+    if (workspace_bytes < sp.total) return PA_ERR_WORKSPACE;
+    void *x_mid = ws + sp.off_x_mid, *fxp = ws + sp.off_fx, *wp = ws + sp.off_w, *tokp = ws + sp.off_tokp;
+    float *partials = reinterpret_cast<float *>(ws + sp.off_partials);
+    float *tok = slice_token_out ? slice_token_out : reinterpret_cast<float *>(ws + sp.off_tok);
+    float *norm = reinterpret_cast<float *>(ws + sp.off_norm);
+    float *tok_out = reinterpret_cast<float *>(ws + sp.off_tok_out);
+    pa::GemmArgs a{};  // x -> x_mid (natural) and fx_mid (packed): two weight sets over the same rows
+    a.in = x;
+    a.w[0] = p->in_project_x_weight;
+    a.w[1] = p->in_project_fx_weight;
+    a.bias[0] = p->in_project_x_bias;
+    a.bias[1] = p->in_project_fx_bias;
+    a.out[0] = x_mid;
+    a.out_pack[1] = fxp;
+    a.M = s.B * s.N;
+    a.N = (int)s.N;
+    a.K = a.C = (int)s.C;
+    a.O = (int)(s.H * 32);
+    a.pack_tpb = (int)pa::mfma::tiles_per_batch(s);
+    a.pack_heads = (int)s.H;
+    if (!pa::gemm::serves(a, 2, 2)) return PA_ERR_UNSUPPORTED;
+    if ((rc = pa::gemm::launch(a, 2, PA_BF16, st))) return rc;
+    if ((rc = pa::mfma::slice_softmax_pack(s, *p, x_mid, wp, compute_units(), st))) return rc;
+    if ((rc = pa::mfma::slice_reduce(s, wp, fxp, partials, st))) return rc;
+    if ((rc = pa::mfma::combine_attention(s, *p, partials, sp.G, tok, norm, tok_out, tokp, st))) return rc;
+    void *out_x = x_mid;
+    if ((rc = pa::mfma::deslice_natural(s, wp, tokp, out_x, compute_units(), st))) return rc;
+    if ((rc = pa::general::out_linear(dtype, s, *p, out_x, y, st))) return rc;
+    if (tail_active(tail)) rc = pa::general::residual_ln(dtype, s, y, *tail, st);
+    return rc;
   }
   const GeneralPlan plan = plan_general(dtype, s);
   if (workspace_bytes < plan.total) return PA_ERR_WORKSPACE;

@@ -79,6 +79,9 @@ int slice_softmax(int dtype, const pa_shape &s, const pa_params &p, const void *
 }  // namespace backward
 
 namespace mfma {
+bool staged_supported(int dtype, const pa_shape &s);
+int slice_softmax_pack(const pa_shape &s, const pa_params &p, const void *x_mid, void *w_pack, int num_cu,
+                       hipStream_t st);
 bool backward_supported(const pa_shape &s);
 int64_t backward_groups(const pa_shape &s, int num_cu);
 int64_t backward_tables_bytes(const pa_shape &s);

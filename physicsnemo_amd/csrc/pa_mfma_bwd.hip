@@ -18,7 +18,8 @@ namespace pa {
 namespace mfma {
 
 // ------------------------------------------------------------------------------------------------
-// deslice_natural_kernel: grid (G, B), H waves; wave h walks the batch's tiles g, g + G, ...
+// deslice_natural_kernel: grid (G, B, head groups), one wave per head of the group; wave h walks the batch's tiles
+// g, g + G, ...
 //   out_x^T_h (32 d x 32 pts) = tok'^T_h (A: tokp fragments, registers) . w_h (B: w_pack chunks)
 // ------------------------------------------------------------------------------------------------
 template <int S>
@@ -27,7 +28,7 @@ __global__ __launch_bounds__(512) void deslice_natural_kernel(const u32x4 *__res
                                                               uint16_t *__restrict__ out_x, int64_t N, int tpb, int H) {
   constexpr int NCH = S / 16;
   const int tid = threadIdx.x, lane = tid & 63, i = lane & 31, g = lane >> 5;
-  const int h = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int h = blockIdx.z * (blockDim.x >> 6) + __builtin_amdgcn_readfirstlane(tid >> 6);
   const int b = blockIdx.y;
   u32x4 tp[NCH];
 #pragma unroll
@@ -275,7 +276,12 @@ int64_t backward_tables_bytes(const pa_shape &s) {
 }
 
 int deslice_natural(const pa_shape &s, const void *w_pack, const void *tokp, void *out_x, int num_cu, hipStream_t st) {
-  const dim3 grid((unsigned)backward_groups(s, num_cu), (unsigned)s.B), block((unsigned)(s.H * 64));
+  const int waves = (int)(s.H < 8 ? s.H : 8);
+  if (s.H % waves != 0) return PA_ERR_UNSUPPORTED;
+  const int groups = (int)(s.H / waves);
+  int64_t gx = backward_groups(s, num_cu) / groups;
+  if (gx < 1) gx = 1;
+  const dim3 grid((unsigned)gx, (unsigned)s.B, (unsigned)groups), block((unsigned)(waves * 64));
   const u32x4 *wp = static_cast<const u32x4 *>(w_pack), *tp = static_cast<const u32x4 *>(tokp);
   uint16_t *ox = static_cast<uint16_t *>(out_x);
   const int tpb = (int)tiles_per_batch(s);

@@ -46,7 +46,7 @@ def _need_cuda(*tensors):
 
 
 def query_path(dtype: torch.dtype, dims: LayerDims) -> int:
-    """0 = general kernels, 1 = bf16 MFMA kernels."""
+    """0 = general kernels, 1 = fused bf16 MFMA kernels, 2 = staged bf16 MFMA kernels (512-wide layers)."""
     rc = _lib.load().pa_query_path(_lib.dtype_code(dtype), byref(dims.c()))
     if rc < 0:
         _lib.check(rc, "pa_query_path")

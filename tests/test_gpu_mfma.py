@@ -13,13 +13,13 @@ from gpu_util import announce, assert_rel_l2, make_pair
 pytestmark = pytest.mark.gpu
 
 
-def _run(B, N, C, S, seed=0, sharpen=1.0, temps=None):
+def _run(B, N, C, S, seed=0, sharpen=1.0, temps=None, path=1):
     H = C // 32
     ref, hip = make_pair("irregular", C, H, 32, S, seed=seed, sharpen=sharpen, temps=temps)
     x = torch.randn(B, N, C)
     xb = x.cuda().bfloat16()
     dims = hip.layer_dims(xb)
-    assert PF.query_path(torch.bfloat16, dims) == 1, "shape must be served by the MFMA kernels"
+    assert PF.query_path(torch.bfloat16, dims) == path, "shape must be served by the expected kernel family"
     with torch.no_grad():
         want = ref.stages(xb.float().cpu())  # same bf16-rounded input, fp32 arithmetic
         y, tok = PF.layer_forward(xb, hip.kernel_params(torch.bfloat16, xb.device), dims, return_slice_tokens=True)
@@ -38,6 +38,29 @@ def test_mfma_layer_matches_fp32_oracle(B, N, C, S):
     assert torch.isfinite(y.float()).all()
     assert_rel_l2(tok, want["tok"], "slice tokens")
     assert_rel_l2(y, want["y"], "layer output")
+
+
+@pytest.mark.parametrize("B,N,C,S", [(1, 5000, 512, 128), (2, 3001, 512, 64), (3, 2048, 512, 32), (1, 4096, 512, 16)])
+def test_staged_mfma_layer_for_512_wide_layers(B, N, C, S):
+    # 16 heads: projections, slice softmax, slice sums, slice attention, deslice and out_linear as separate MFMA kernels
+    announce("staged mfma layer", B, N, C, S)
+    ref, hip, xb, want, y, tok = _run(B, N, C, S, sharpen=2.0, path=2)
+    assert y.dtype == torch.bfloat16 and y.shape == (B, N, C)
+    assert_rel_l2(tok, want["tok"], "slice tokens")
+    assert_rel_l2(y, want["y"], "layer output")
+    # the block tail (residual + LayerNorm) of the staged path
+    ln = torch.nn.LayerNorm(C)
+    with torch.no_grad():
+        ln.weight.uniform_(0.5, 1.5)
+        ln.bias.uniform_(-0.5, 0.5)
+        res = torch.randn(B, N, C)
+        fx_new, normed = hip.forward_block(xb, res.cuda().bfloat16(), ln.cuda())
+        want_fx = want["y"] + res.bfloat16().float()
+        assert_rel_l2(fx_new, want_fx, "fx_new")
+        assert_rel_l2(normed, ln.cpu()(want_fx), "LayerNorm(fx_new)", tol=1.5e-2)
+    # small inputs of the same layer stay on the general kernels and agree with the staged kernels' arithmetic class
+    xs = xb[:, :100].contiguous()
+    assert PF.query_path(torch.bfloat16, hip.layer_dims(xs)) == 0
 
 
 def test_mfma_sharp_softmax_and_clamped_temperatures():
@@ -152,7 +175,7 @@ def test_mfma_full_size_properties():
     assert_rel_l2(y[:, :4096], want, "prefix of the full-size output")
 
 
-@pytest.mark.parametrize("B,N,C,S", [(2, 3000, 256, 64), (1, 2000, 128, 32), (1, 700, 512, 128)])
+@pytest.mark.parametrize("B,N,C,S", [(2, 3000, 256, 64), (1, 2000, 128, 32), (1, 700, 512, 128), (1, 6000, 512, 128)])
 def test_fp8_e4m3_weight_variant(B, N, C, S):
     # bf16 activations, fp8-e4m3 per-output-channel-scaled projection weights.  The reference for the 1e-2 bar is
     # the fp32 oracle holding the SAME (dequantised) weights; the error against the unquantised weights is printed.
