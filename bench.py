@@ -171,7 +171,8 @@ def time_training_step(points, C, S, reps=3):
                        "backward kernel, split-row MFMA weight-gradient kernel"}
 
 
-def time_full_model(name, B, N, functional_dim, embedding_dim, slice_num, n_layers, steps=5, warmup=2):
+def time_full_model(name, B, N, functional_dim, embedding_dim, slice_num, n_layers, steps=5, warmup=2, n_hidden=256,
+                    fp8_weights=False, graph=True):
     """Forward of a whole Transolver (bf16 autocast, random-init weights, synthetic N(0,1) inputs) -> Mpoints/s.
 
     The PhysicsAttention layers, the block MLPs, their residual adds and the LayerNorms between them run in the HIP
@@ -183,7 +184,10 @@ def time_full_model(name, B, N, functional_dim, embedding_dim, slice_num, n_laye
 
     torch.manual_seed(0)
     model = pn.Transolver(functional_dim=functional_dim, embedding_dim=embedding_dim, out_dim=4, n_layers=n_layers,
-                          n_hidden=256, n_head=8, slice_num=slice_num, use_te=False).eval().cuda()
+                          n_hidden=n_hidden, n_head=n_hidden // 32, slice_num=slice_num, use_te=False).eval().cuda()
+    if fp8_weights:  # the layers' three large weights as fp8-e4m3 bytes with per-output-channel scales
+        for blk in model.blocks:
+            blk.Attn.use_fp8_weights(True)
     g = torch.Generator().manual_seed(1234)
     fx = torch.randn(B, N, functional_dim, generator=g).cuda()
     emb = torch.randn(B, N, embedding_dim, generator=g).cuda()
@@ -204,14 +208,18 @@ def time_full_model(name, B, N, functional_dim, embedding_dim, slice_num, n_laye
     with torch.no_grad():
         dt, out = timed(fwd)
         assert torch.isfinite(out.float()).all()
-        graphed = pn.GraphedForward(fwd, fx, emb)  # the same forward replayed from a HIP graph
-        dt_graph, out = timed(lambda a, b: graphed.replay())
-        assert torch.isfinite(out.float()).all()
+        res = {"workload": name, "batch": B, "points": N, "layers": n_layers, "hidden": n_hidden, "slice_num": slice_num,
+               "ms_per_forward": round(dt * 1e3, 3), "mpoints_per_s": round(B * N / dt / 1e6, 2)}
+        if graph:
+            graphed = pn.GraphedForward(fwd, fx, emb)  # the same forward replayed from a HIP graph
+            dt_graph, out = timed(lambda a, b: graphed.replay())
+            assert torch.isfinite(out.float()).all()
+            res.update({"ms_per_forward_graph": round(dt_graph * 1e3, 3),
+                        "mpoints_per_s_graph": round(B * N / dt_graph / 1e6, 2)})
+            del graphed
     del model, fx, emb, out
     torch.cuda.empty_cache()
-    return {"workload": name, "batch": B, "points": N, "layers": n_layers, "slice_num": slice_num,
-            "ms_per_forward": round(dt * 1e3, 3), "mpoints_per_s": round(B * N / dt / 1e6, 2),
-            "ms_per_forward_graph": round(dt_graph * 1e3, 3), "mpoints_per_s_graph": round(B * N / dt_graph / 1e6, 2)}
+    return res
 
 
 def time_structured_model(steps=5, warmup=2):
@@ -367,6 +375,8 @@ def main():
             time_structured_model(),
             time_full_model("cfg2: Transolver irregular 2D, 8 layers", 8, 32768, 3, 2, 64, 8),
             time_full_model("cfg4: Transolver 3D surface cloud, 8 layers", 1, 1000000, 1, 6, 32, 8),
+            time_full_model("cfg5: Transolver 3D volume, 12 layers, hidden 512, fp8-e4m3 projection weights", 1, 4194304,
+                            4, 3, 128, 12, steps=2, warmup=1, n_hidden=512, fp8_weights=True, graph=False),
         ]
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(state, x_cpu, C, H, S, args.cpu_seconds)

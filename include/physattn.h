@@ -297,6 +297,10 @@ int64_t pa_mlp_workspace_bytes(int dtype, int64_t rows, int64_t C, int64_t F);
 int pa_mlp_forward(int dtype, int64_t rows, int64_t C, int64_t F, const pa_mlp_params *p, const void *u, void *y,
                    const pa_block_tail *tail, void *workspace, int64_t workspace_bytes, void *stream);
 
+/* The block tail on its own (TR.py:300-303, :305-307): y (rows, C) <- y + tail->residual (if given), then
+ * tail->ln_out = LayerNorm(y) (if given).  For callers whose producer of y is not one of the fused kernels. */
+int pa_residual_layernorm(int dtype, int64_t rows, int64_t C, void *y, const pa_block_tail *tail, void *stream);
+
 /* ---- whole layer ------------------------------------------------------------------------------ */
 
 /* Replaces PhysicsAttentionBase.forward (PA.py:501-558), plus=False, use_te=False, dropout off.

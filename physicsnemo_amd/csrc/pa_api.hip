@@ -383,6 +383,19 @@ int pa_slice_softmax_backward(int dtype, const pa_shape *shape, const pa_params 
                                      d_proj, d_z, d_temperature_partials, static_cast<hipStream_t>(stream));
 }
 
+int pa_residual_layernorm(int dtype, int64_t rows, int64_t C, void *y, const pa_block_tail *tail, void *stream) {
+  if (dtype != PA_F32 && dtype != PA_BF16) return PA_ERR_UNSUPPORTED;
+  if (rows <= 0 || C <= 0 || C > (1 << 16)) return PA_ERR_DIMS;
+  if (!y || !tail || (!tail->residual && !tail->ln_out)) return PA_ERR_NULL;
+  int rc = check_tail(tail);
+  if (rc) return rc;
+  pa_shape s{};
+  s.B = 1;
+  s.N = rows;
+  s.C = C;
+  return pa::general::residual_ln(dtype, s, y, *tail, static_cast<hipStream_t>(stream));
+}
+
 int64_t pa_cols_gemm_chunks(int64_t rows) {
   if (rows <= 0) return PA_ERR_DIMS;
   return pa::gemm::cols_gemm_chunks(rows, compute_units());

@@ -514,6 +514,82 @@ __global__ __launch_bounds__(256) void residual_ln_kernel(T *__restrict__ y, con
   }
 }
 
+// residual_ln_vec_kernel: the same with 16-byte accesses for rows that are whole 16-byte units (C % UE == 0,
+// C <= 64 * UPL * UE): lane l owns units l, l + 64, ... of its row and keeps them in registers between the passes.
+template <typename T, int UPL>
+__global__ __launch_bounds__(256) void residual_ln_vec_kernel(T *__restrict__ y, const T *__restrict__ residual,
+                                                              const float *__restrict__ gamma,
+                                                              const float *__restrict__ beta, float eps,
+                                                              T *__restrict__ ln_out, int64_t M, int C) {
+  constexpr int UE = 16 / sizeof(T);
+  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+  const int lane = threadIdx.x & 63;
+  const int units = C / UE;
+  float gam[UPL][UE], bet[UPL][UE];  // this lane's LayerNorm parameters stay in registers across its rows
+#pragma unroll
+  for (int k = 0; k < UPL; ++k)
+#pragma unroll
+    for (int e = 0; e < UE; ++e) {
+      const int c = (lane + 64 * k) * UE + e;
+      gam[k][e] = (ln_out && c < C) ? gamma[c] : 1.f;
+      bet[k][e] = (ln_out && c < C) ? beta[c] : 0.f;
+    }
+  // one wave per row at a time; the grid is sized to the machine and every wave walks rows a grid apart
+  for (int64_t m = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6); m < M; m += (int64_t)gridDim.x * 4) {
+  T *yr = y + m * C;
+  float v[UPL][UE];
+  float sum = 0.f;
+#pragma unroll
+  for (int k = 0; k < UPL; ++k) {
+    const int u = lane + 64 * k;
+    if (u < units) {
+      u32x4 a = *reinterpret_cast<const u32x4 *>(yr + u * UE);
+      const T *ae = reinterpret_cast<const T *>(&a);
+      if (residual) {
+        u32x4 r = *reinterpret_cast<const u32x4 *>(residual + m * C + u * UE);
+        const T *re = reinterpret_cast<const T *>(&r);
+        alignas(16) T o[UE];
+#pragma unroll
+        for (int e = 0; e < UE; ++e) {
+          v[k][e] = round_to(yr, load_as_f32(ae + e) + load_as_f32(re + e));
+          store_from_f32(o + e, v[k][e]);
+        }
+        *reinterpret_cast<u32x4 *>(yr + u * UE) = *reinterpret_cast<const u32x4 *>(o);
+      } else {
+#pragma unroll
+        for (int e = 0; e < UE; ++e) v[k][e] = load_as_f32(ae + e);
+      }
+#pragma unroll
+      for (int e = 0; e < UE; ++e) sum += v[k][e];
+    }
+  }
+  if (!ln_out) continue;
+  const float mean = wave_sum(sum) / (float)C;
+  float sq = 0.f;
+#pragma unroll
+  for (int k = 0; k < UPL; ++k)
+    if (lane + 64 * k < units) {
+#pragma unroll
+      for (int e = 0; e < UE; ++e) {
+        const float d = v[k][e] - mean;
+        sq = fmaf(d, d, sq);
+      }
+    }
+  const float rstd = rsqrtf(wave_sum(sq) / (float)C + eps);
+#pragma unroll
+  for (int k = 0; k < UPL; ++k) {
+    const int u = lane + 64 * k;
+    if (u < units) {
+      alignas(16) T o[UE];
+#pragma unroll
+      for (int e = 0; e < UE; ++e)
+        store_from_f32(o + e, (v[k][e] - mean) * rstd * gam[k][e] + bet[k][e]);
+      *reinterpret_cast<u32x4 *>(ln_out + m * C + u * UE) = *reinterpret_cast<const u32x4 *>(o);
+    }
+  }
+  }
+}
+
 // ------------------------------------------------------------------------------------------------
 // dequant_e4m3_kernel: out[o, k] = bf16(scale[o] * decode_e4m3fn(in[o, k])).  e4m3fn: 1 sign, 4 exponent (bias 7),
 // 3 mantissa bits; exponent 0 is subnormal (2^-6 * m/8); 0x7f / 0xff are NaN; there are no infinities.
@@ -776,18 +852,34 @@ int deslice(int dtype, const pa_shape &s, const void *w, const float *out_token,
   return dtype == PA_F32 ? deslice_t<float>(s, w, out_token, out_x, st) : deslice_t<bf16>(s, w, out_token, out_x, st);
 }
 
-int residual_ln(int dtype, const pa_shape &s, void *y, const pa_block_tail &tail, hipStream_t st) {
+template <typename T>
+static int residual_ln_t(const pa_shape &s, void *y, const pa_block_tail &tail, hipStream_t st) {
   const int64_t M = s.B * s.N;
+  const int C = (int)s.C;
+  constexpr int UE = 16 / sizeof(T);
   dim3 grid((unsigned)((M + 3) / 4));
-  if (dtype == PA_F32)
-    hipLaunchKernelGGL((residual_ln_kernel<float>), grid, dim3(256), 0, st, static_cast<float *>(y),
-                       static_cast<const float *>(tail.residual), tail.ln_gamma, tail.ln_beta, tail.ln_eps,
-                       static_cast<float *>(tail.ln_out), M, (int)s.C);
+  const dim3 vgrid((unsigned)std::min<int64_t>((M + 3) / 4, 256 * 16));  // the vector kernel's waves walk the rows
+  T *yp = static_cast<T *>(y), *lo = static_cast<T *>(tail.ln_out);
+  const T *res = static_cast<const T *>(tail.residual);
+  const bool vec = C % UE == 0 && aligned16(y) && aligned16(tail.residual) && aligned16(tail.ln_out);
+  const int upl = (C / UE + 63) / 64;
+  if (vec && upl <= 1)
+    hipLaunchKernelGGL((residual_ln_vec_kernel<T, 1>), vgrid, dim3(256), 0, st, yp, res, tail.ln_gamma, tail.ln_beta,
+                       tail.ln_eps, lo, M, C);
+  else if (vec && upl <= 2)
+    hipLaunchKernelGGL((residual_ln_vec_kernel<T, 2>), vgrid, dim3(256), 0, st, yp, res, tail.ln_gamma, tail.ln_beta,
+                       tail.ln_eps, lo, M, C);
+  else if (vec && upl <= 4)
+    hipLaunchKernelGGL((residual_ln_vec_kernel<T, 4>), vgrid, dim3(256), 0, st, yp, res, tail.ln_gamma, tail.ln_beta,
+                       tail.ln_eps, lo, M, C);
   else
-    hipLaunchKernelGGL((residual_ln_kernel<bf16>), grid, dim3(256), 0, st, static_cast<bf16 *>(y),
-                       static_cast<const bf16 *>(tail.residual), tail.ln_gamma, tail.ln_beta, tail.ln_eps,
-                       static_cast<bf16 *>(tail.ln_out), M, (int)s.C);
+    hipLaunchKernelGGL((residual_ln_kernel<T>), grid, dim3(256), 0, st, yp, res, tail.ln_gamma, tail.ln_beta,
+                       tail.ln_eps, lo, M, C);
   return launch_status();
+}
+
+int residual_ln(int dtype, const pa_shape &s, void *y, const pa_block_tail &tail, hipStream_t st) {
+  return dtype == PA_F32 ? residual_ln_t<float>(s, y, tail, st) : residual_ln_t<bf16>(s, y, tail, st);
 }
 
 }  // namespace general

@@ -176,6 +176,17 @@ def layer_forward(x, params, dims: LayerDims, residual=None, ln_weight=None, ln_
     return (out, tok) if return_slice_tokens else out
 
 
+def residual_layernorm(y, residual=None, ln_weight=None, ln_bias=None, ln_eps=1e-5):
+    """In place y <- y + residual (if given); returns (y, LayerNorm(y)) when ln_weight is given, else y."""
+    _need_cuda(y, residual, ln_weight, ln_bias)
+    C = y.shape[-1]
+    ln_out = torch.empty_like(y) if ln_weight is not None else None
+    tail = _c_tail(residual, ln_weight, ln_bias, ln_eps, ln_out)
+    _lib.check(_lib.load().pa_residual_layernorm(_lib.dtype_code(y.dtype), y.numel() // C, C, y.data_ptr(), byref(tail),
+                                                 _lib.current_stream_ptr(y.device)), "pa_residual_layernorm")
+    return y if ln_out is None else (y, ln_out)
+
+
 def mlp_supported(dtype: torch.dtype, rows: int, C: int, F: int) -> bool:
     """True if `mlp_forward` serves this shape with the MFMA kernel (bf16, C in {128, 256}, F a multiple of 64)."""
     if dtype != torch.bfloat16:

@@ -123,7 +123,16 @@ class TransolverBlock(nn.Module):
             return PF.mlp_forward(normed, w1, b1, w2, b2, residual=fx1,
                                   ln_weight=next_ln.weight.detach().float().contiguous(),
                                   ln_bias=next_ln.bias.detach().float().contiguous(), ln_eps=next_ln.eps)
-        return self.ln_mlp1[1](normed) + fx1, None
+        # MLP shapes the fused kernel does not serve: tensor-op MLP, then residual add (+ the next LayerNorm) in one pass
+        h = self.ln_mlp1[1](normed)
+        if h.is_cuda and h.dtype == fx1.dtype and h.dtype in (torch.float32, torch.bfloat16):
+            h = h.contiguous()
+            if next_ln is None:
+                return PF.residual_layernorm(h, residual=fx1.contiguous()), None
+            return PF.residual_layernorm(h, residual=fx1.contiguous(),
+                                         ln_weight=next_ln.weight.detach().float().contiguous(),
+                                         ln_bias=next_ln.bias.detach().float().contiguous(), ln_eps=next_ln.eps)
+        return h + fx1, None
 
     def forward(self, fx: torch.Tensor) -> torch.Tensor:
         if self.last_layer:
