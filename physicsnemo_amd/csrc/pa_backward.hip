@@ -1,7 +1,7 @@
 // Backward pass of the PhysicsAttention layer: the per-point and per-slice kernels (fp32 arithmetic on the
-// vector ALUs, fp32 or bf16 storage, natural layouts).  Gradients that are plain GEMMs over the point axis
-// (the weight gradients) are left to the caller's GEMM library; everything that is specific to the layer
-// is here.
+// vector ALUs, fp32 or bf16 storage, natural layouts) of the general kernel family.  The weight gradients, plain
+// d out^T . in products over the point axis, are computed by cols_gemm_kernel (pa_gemm.hip) or the caller's GEMM
+// library; the bf16 MFMA versions of these kernels are in pa_mfma_bwd.hip.
 //
 // Forward (PA.py:501-558), per batch b and head h, with T = clamp(temperature_h, .5, 5):
 //   z[n,s]   = x_mid[n,:] . Ws[s,:] + bs[s];  w[n,:] = softmax_s(z[n,:] / T)
@@ -282,22 +282,6 @@ __global__ __launch_bounds__(256) void slice_softmax_backward_kernel(
 // ================================================================================================
 // host launchers
 // ================================================================================================
-static int launch_status() {
-  hipError_t e = hipGetLastError();
-  return e == hipSuccess ? PA_OK : (int)e;
-}
-
-template <typename F>
-static int allow_dynamic_lds(F kernel, size_t bytes) {
-  if (bytes > kMaxLdsBytes) return PA_ERR_UNSUPPORTED;
-  if (bytes > 48 * 1024) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
-    if (e != hipSuccess) return (int)e;
-  }
-  return PA_OK;
-}
-
 size_t attention_lds_bytes(const pa_shape &s) {
   return (size_t)(7 * s.S * (s.D + 1) + (kAttnBwdThreads / 64) * 2 * s.S) * 4;
 }

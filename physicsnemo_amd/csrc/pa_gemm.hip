@@ -317,19 +317,15 @@ int linear_launch(const GemmArgs &a, int nsets, int num_cu, hipStream_t st) {
   if (gx < 1) gx = 1;
   if (gx > ntiles) gx = ntiles;
   const dim3 grid((unsigned)gx, (unsigned)((a.O + 255) / 256), (unsigned)nsets), block((unsigned)(waves * 64));
-  const size_t lds = (size_t)2 * 32 * (a.K / 8 + 1) * 16;
-  if (lds > 48 * 1024 &&
-      hipFuncSetAttribute(reinterpret_cast<const void *>(rows_linear_kernel<32>),
-                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
-    return PA_ERR_UNSUPPORTED;
+  const size_t lds = (size_t)2 * 32 * (a.K / 8 + 1) * 16;  // only K = 512 exceeds the default limit
+  if (int rc = allow_dynamic_lds(rows_linear_kernel<32>, a.K == 512 ? lds : 0)) return rc;
   switch (a.K) {
     case 128: hipLaunchKernelGGL((rows_linear_kernel<8>), grid, block, lds, st, a); break;
     case 256: hipLaunchKernelGGL((rows_linear_kernel<16>), grid, block, lds, st, a); break;
     case 512: hipLaunchKernelGGL((rows_linear_kernel<32>), grid, block, lds, st, a); break;
     default: return PA_ERR_UNSUPPORTED;
   }
-  hipError_t e = hipGetLastError();
-  return e == hipSuccess ? PA_OK : (int)e;
+  return launch_status();
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -453,8 +449,7 @@ int cols_gemm(const void *A, int64_t lda, int64_t OA, const void *B, int64_t ldb
     default: return PA_ERR_UNSUPPORTED;
   }
 #undef PA_COLS
-  hipError_t e = hipGetLastError();
-  return e == hipSuccess ? PA_OK : (int)e;
+  return launch_status();
 }
 
 bool serves(const GemmArgs &a, int nsets, size_t elem_bytes) {
@@ -472,8 +467,7 @@ static int launch_t(const GemmArgs &a, int nsets, hipStream_t st) {
   const int64_t rows = a.pack_tpb > 0 ? (a.M / a.N) * a.pack_tpb * 32 : a.M;
   dim3 grid((unsigned)((rows + kRows - 1) / kRows), (unsigned)((a.O + 32 * NT - 1) / (32 * NT)), (unsigned)nsets);
   hipLaunchKernelGGL((rows_gemm_mfma_kernel<T, NT>), grid, dim3(256), 0, st, a);
-  hipError_t e = hipGetLastError();
-  return e == hipSuccess ? PA_OK : (int)e;
+  return launch_status();
 }
 
 template <typename T>

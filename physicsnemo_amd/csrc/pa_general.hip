@@ -613,22 +613,6 @@ __global__ __launch_bounds__(256) void dequant_e4m3_kernel(const uint8_t *__rest
 // ================================================================================================
 // host launchers
 // ================================================================================================
-static int launch_status() {
-  hipError_t e = hipGetLastError();
-  return e == hipSuccess ? PA_OK : (int)e;
-}
-
-template <typename F>
-static int allow_dynamic_lds(F kernel, size_t bytes) {
-  if (bytes > kMaxLdsBytes) return PA_ERR_UNSUPPORTED;
-  if (bytes > 48 * 1024) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
-    if (e != hipSuccess) return (int)e;
-  }
-  return PA_OK;
-}
-
 template <typename TA, typename TW>
 static int launch_gemm(const GemmArgs &a, int nsets, hipStream_t st) {
   if (gemm::serves(a, nsets, sizeof(TA))) return gemm::launch(a, nsets, sizeof(TA) == 4 ? PA_F32 : PA_BF16, st);

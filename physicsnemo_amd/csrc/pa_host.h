@@ -11,6 +11,24 @@ namespace pa {
 
 constexpr size_t kMaxLdsBytes = 160 * 1024;  // LDS per workgroup on gfx950
 
+// result of the launch just enqueued, as a C-ABI return code
+inline int launch_status() {
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? PA_OK : (int)e;
+}
+
+// opt a kernel in to more than the default 48 KiB of dynamic LDS
+template <typename F>
+inline int allow_dynamic_lds(F kernel, size_t bytes) {
+  if (bytes > kMaxLdsBytes) return PA_ERR_UNSUPPORTED;
+  if (bytes > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+    if (e != hipSuccess) return (int)e;
+  }
+  return PA_OK;
+}
+
 // Arguments of the row GEMMs: out[m, o] = bias[o] + sum_k A(m, k) * W[o, k]
 //   linear: A(m, k) = in[m*K + k]
 //   conv  : K = taps*C, k = tap*C + c; 2-D: taps = ks^2, tap = u*ks + v, A(m,k) = in[b, (i+u-p)*gw + (j+v-p), c];

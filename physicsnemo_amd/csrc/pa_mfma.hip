@@ -760,22 +760,6 @@ __global__ __launch_bounds__(C * 2) void deslice_project_kernel(const u32x4 *__r
 // ================================================================================================
 // host side
 // ================================================================================================
-static int launch_status() {
-  hipError_t e = hipGetLastError();
-  return e == hipSuccess ? PA_OK : (int)e;
-}
-
-template <typename F>
-static int allow_dynamic_lds(F kernel, size_t bytes) {
-  if (bytes > kMaxLdsBytes) return PA_ERR_UNSUPPORTED;
-  if (bytes > 48 * 1024) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
-    if (e != hipSuccess) return (int)e;
-  }
-  return PA_OK;
-}
-
 bool supported(int dtype, const pa_shape &s) {
   if (dtype != PA_BF16 || s.conv_k != 0 || s.D != 32 || s.C != s.H * 32) return false;
   if (s.C != 128 && s.C != 256) return false;

@@ -256,11 +256,6 @@ __global__ __launch_bounds__(512) void slice_softmax_backward_mfma_kernel(
 // ================================================================================================
 // host side
 // ================================================================================================
-static int launch_status() {
-  hipError_t e = hipGetLastError();
-  return e == hipSuccess ? PA_OK : (int)e;
-}
-
 bool backward_supported(const pa_shape &s) { return supported(PA_BF16, s) && s.S <= 64; }
 
 int64_t backward_groups(const pa_shape &s, int num_cu) {

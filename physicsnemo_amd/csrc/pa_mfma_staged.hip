@@ -84,11 +84,6 @@ __global__ __launch_bounds__(512) void slice_softmax_pack_kernel(const uint16_t 
   }
 }
 
-static int launch_status() {
-  hipError_t e = hipGetLastError();
-  return e == hipSuccess ? PA_OK : (int)e;
-}
-
 // shapes of the staged path: what the fused kernels serve plus C = 512, large enough for the row kernels to pay off
 bool staged_supported(int dtype, const pa_shape &s) {
   if (dtype != PA_BF16 || s.conv_k != 0 || s.D != 32 || s.C != s.H * 32) return false;

@@ -213,3 +213,58 @@ def test_model_flatten_equivalence_on_gpu():
         b = m(fx.reshape(2, -1, 3), embedding=emb.reshape(2, -1, 4))
     assert a.shape == (2, 16, 16, 2)
     assert torch.allclose(a.reshape(2, -1, 2), b, atol=1e-6)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rows,C", [(1000, 512), (37, 48), (5000, 256), (300, 1024), (64, 36)])
+def test_residual_layernorm_entry_point(dtype, rows, C):
+    announce("pa_residual_layernorm", dtype, rows, C)
+    from physicsnemo_amd import functional as PF
+    torch.manual_seed(rows + C)
+    y, res = torch.randn(rows, C), torch.randn(rows, C)
+    gamma, beta = torch.rand(C) + 0.5, torch.randn(C)
+    yq, rq = y.to(dtype), res.to(dtype)
+    want_sum = (yq.float() + rq.float()).to(dtype).float()  # the sum is stored in the activation type first
+    want_ln = torch.nn.functional.layer_norm(want_sum, (C,), gamma, beta, 1e-5)
+    got_sum, got_ln = PF.residual_layernorm(yq.cuda().clone(), residual=rq.cuda(), ln_weight=gamma.cuda(),
+                                            ln_bias=beta.cuda(), ln_eps=1e-5)
+    assert torch.equal(got_sum.float().cpu(), want_sum)
+    if dtype == torch.float32:
+        assert_fp32_close(got_ln, want_ln, "LayerNorm(y + residual)")
+    else:
+        assert_rel_l2(got_ln, want_ln, "LayerNorm(y + residual)", tol=5e-3)
+    only_ln = PF.residual_layernorm(yq.cuda().clone(), ln_weight=gamma.cuda(), ln_bias=beta.cuda())[1]
+    want = torch.nn.functional.layer_norm(yq.float(), (C,), gamma, beta, 1e-5)
+    (assert_fp32_close if dtype == torch.float32 else assert_rel_l2)(only_ln, want, "LayerNorm(y)")
+    only_sum = PF.residual_layernorm(yq.cuda().clone(), residual=rq.cuda())
+    assert torch.equal(only_sum.float().cpu(), want_sum)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("B,N,cin,cout,grid,k", [
+    (2, 300, 64, 96, None, 0), (1, 5000, 256, 256, None, 0), (1, 6000, 512, 256, None, 0), (3, 50, 20, 7, None, 0),
+    (2, 63, 32, 48, (7, 9), 3), (1, 60, 16, 40, (3, 4, 5), 3), (1, 30, 12, 8, (5, 6), 5),
+])
+def test_rows_gemm_entry_point(dtype, B, N, cin, cout, grid, k):
+    # every kernel behind pa_rows_gemm: scalar FMA (odd widths), fp32 / bf16 MFMA tiles, weights-stationary bf16 Linear
+    announce("pa_rows_gemm", dtype, B, N, cin, cout, grid, k)
+    from physicsnemo_amd import functional as PF
+    torch.manual_seed(N + cin)
+    x = torch.randn(B, N, cin).to(dtype)
+    bias = torch.randn(cout)
+    if grid is None:
+        w = (torch.randn(cout, cin) / cin ** 0.5).to(dtype)
+        want = x.float() @ w.float().t() + bias
+        dims = PF.LayerDims(B, N, cin, 1, 1, 1)
+    else:
+        w = (torch.randn(cout, cin, *([k] * len(grid))) / (cin * k ** len(grid)) ** 0.5).to(dtype)
+        img = x.float().reshape(B, *grid, cin).movedim(-1, 1)
+        conv = torch.nn.functional.conv2d if len(grid) == 2 else torch.nn.functional.conv3d
+        want = conv(img, w.float(), bias, padding=k // 2).flatten(2).transpose(1, 2)
+        dims = PF.LayerDims(B, N, cin, 1, 1, 1, grid[0], grid[1], k, grid[2] if len(grid) == 3 else 0)
+    got = PF.rows_gemm(x.cuda(), w.cuda().contiguous(), bias.cuda(), dims, cin, cout)
+    assert got.shape == (B, N, cout) and got.dtype == dtype
+    if dtype == torch.float32:
+        assert_fp32_close(got, want, "rows gemm")
+    else:
+        assert_rel_l2(got, want, "rows gemm", tol=5e-3)
