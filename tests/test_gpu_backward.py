@@ -214,3 +214,23 @@ def test_cols_gemm_weight_gradient_product(rows, ca, cb):
     assert got.shape == (ca, cb) and got.dtype == torch.float32
     assert_fp32_close(got, want.float(), "a^T b", rtol=1e-4)
     assert torch.equal(got, PF.cols_gemm(a, b))  # fixed summation order
+
+
+def test_bf16_model_training_step_runs_the_mfma_backward():
+    announce("Transolver training step, bf16 autocast, MFMA backward inside the blocks")
+    torch.manual_seed(1)
+    kw = dict(functional_dim=3, out_dim=2, embedding_dim=2, n_layers=2, n_hidden=128, n_head=4, slice_num=32, mlp_ratio=2)
+    m = pn.Transolver(use_te=False, **kw).cuda().train()
+    ref = to.OracleTransolver(**kw).train()
+    ref.load_state_dict(m.state_dict())
+    fx, emb, target = torch.randn(2, 700, 3), torch.randn(2, 700, 2), torch.randn(2, 700, 2)
+    ((ref(fx, emb) - target) ** 2).mean().backward()
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        out = m(fx.cuda(), emb.cuda())
+    ((out.float() - target.cuda()) ** 2).mean().backward()
+    want = dict(ref.named_parameters())
+    for name, p in m.named_parameters():
+        assert p.grad is not None and torch.isfinite(p.grad).all(), name
+        if "temperature" in name or want[name].grad.abs().max() < 1e-6:
+            continue
+        assert_rel_l2(p.grad, want[name].grad, f"bf16 model grad {name}", tol=8e-2)
