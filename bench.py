@@ -345,7 +345,8 @@ def main():
                 entry.update({"algorithmic_bytes": bytes_pp[name] * B * N, "hbm_gbs": round(gbs, 1),
                               "hbm_frac": round(gbs / HBM_PEAK_GBS, 4), "mfma_tflops": round(tf, 1),
                               "mfma_frac": round(tf / MFMA_BF16_PEAK_TF, 4)})
-            entry["on_layer_path"] = name in on_path or name in ("combine_attention", "pack_params")
+            # the parameter repack runs once per parameter set (the module keeps the packed copy), not per layer call
+            entry["on_layer_path"] = name in on_path or name == "combine_attention"
             kernels[name] = entry
         dominant = max(on_path, key=lambda k: kernels[k]["ms"])
         # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a 1 GiB copy (x2.0 / x1.0);

@@ -311,6 +311,14 @@ int pa_layer_forward(int dtype, const pa_shape *shape, const pa_params *p, const
                      const pa_block_tail *tail, float *slice_token_out, void *workspace,
                      int64_t workspace_bytes, void *stream);
 
+/* pa_layer_forward for the fused MFMA shapes (pa_query_path() == 1, bf16 weights) with the parameters already
+ * repacked by pa_mfma_pack_params into `blob` (PA_BUF_BLOB bytes): callers that run many forwards with unchanged
+ * weights keep the blob and skip the repack.  Of `p` only qkv_project_weight is read.  Workspace as for
+ * pa_layer_forward.  No reference counterpart. */
+int pa_mfma_layer_forward(const pa_shape *shape, const pa_params *p, const void *blob, const void *x, void *y,
+                          const pa_block_tail *tail, float *slice_token_out, void *workspace,
+                          int64_t workspace_bytes, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

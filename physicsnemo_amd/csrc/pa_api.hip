@@ -182,6 +182,25 @@ int check_tail(const pa_block_tail *t) {
 
 bool tail_active(const pa_block_tail *t) { return t && (t->residual || t->ln_out); }
 
+// the fused MFMA kernels of one layer call, parameters already repacked into `blob`
+int mfma_layer(const pa_shape &s, const pa_params &p, const void *blob, const void *x, void *y, const pa_block_tail *tail,
+               float *slice_token_out, char *ws, const MfmaPlan &mp, hipStream_t st) {
+  void *fxp = ws + mp.off_fx, *wp = ws + mp.off_w, *tokp = ws + mp.off_tokp;
+  float *partials = reinterpret_cast<float *>(ws + mp.off_partials);
+  float *tok = slice_token_out ? slice_token_out : reinterpret_cast<float *>(ws + mp.off_tok);
+  float *norm = reinterpret_cast<float *>(ws + mp.off_norm);
+  float *tok_out = reinterpret_cast<float *>(ws + mp.off_tok_out);
+  int rc;
+  if (pa::mfma::fuse_reduce(s)) {  // kernel (a) also leaves the partial slice-token sums
+    if ((rc = pa::mfma::project_softmax(s, blob, x, nullptr, wp, partials, compute_units(), st))) return rc;
+  } else {
+    if ((rc = pa::mfma::project_softmax(s, blob, x, fxp, wp, nullptr, compute_units(), st))) return rc;
+    if ((rc = pa::mfma::slice_reduce(s, wp, fxp, partials, st))) return rc;
+  }
+  if ((rc = pa::mfma::combine_attention(s, p, partials, mp.G, tok, norm, tok_out, tokp, st))) return rc;
+  return pa::mfma::deslice_project(s, blob, wp, tokp, y, tail_active(tail) ? tail : nullptr, compute_units(), st);
+}
+
 }  // namespace
 
 extern "C" {
@@ -597,6 +616,20 @@ int pa_mlp_forward(int dtype, int64_t rows, int64_t C, int64_t F, const pa_mlp_p
                           st);
 }
 
+int pa_mfma_layer_forward(const pa_shape *shape, const pa_params *p, const void *blob, const void *x, void *y,
+                          const pa_block_tail *tail, float *slice_token_out, void *workspace, int64_t workspace_bytes,
+                          void *stream) {
+  int rc = check_mfma(shape);
+  if (rc) return rc;
+  if (!p || !p->qkv_project_weight || !blob || !x || !y || !workspace) return PA_ERR_NULL;
+  if (!aligned16(blob) || !aligned16(x) || !aligned16(y) || !aligned16(workspace)) return PA_ERR_ALIGN;
+  if ((rc = check_tail(tail))) return rc;
+  const MfmaPlan mp = plan_mfma(*shape);
+  if (workspace_bytes < mp.total) return PA_ERR_WORKSPACE;
+  return mfma_layer(*shape, *p, blob, x, y, tail, slice_token_out, static_cast<char *>(workspace), mp,
+                    static_cast<hipStream_t>(stream));
+}
+
 int pa_layer_forward(int dtype, const pa_shape *shape, const pa_params *p, const void *x, void *y,
                      const pa_block_tail *tail, float *slice_token_out, void *workspace, int64_t workspace_bytes,
                      void *stream) {
@@ -632,20 +665,9 @@ int pa_layer_forward(int dtype, const pa_shape *shape, const pa_params *p, const
   if (pa::mfma::supported(dtype, s)) {
     const MfmaPlan mp = plan_mfma(s);
     if (workspace_bytes < mp.total) return PA_ERR_WORKSPACE;
-    void *blob = ws + mp.off_blob, *fxp = ws + mp.off_fx, *wp = ws + mp.off_w, *tokp = ws + mp.off_tokp;
-    float *partials = reinterpret_cast<float *>(ws + mp.off_partials);
-    float *tok = slice_token_out ? slice_token_out : reinterpret_cast<float *>(ws + mp.off_tok);
-    float *norm = reinterpret_cast<float *>(ws + mp.off_norm);
-    float *tok_out = reinterpret_cast<float *>(ws + mp.off_tok_out);
+    void *blob = ws + mp.off_blob;
     if ((rc = pa::mfma::pack_params(s, *p, blob, st))) return rc;
-    if (pa::mfma::fuse_reduce(s)) {  // kernel (a) also leaves the partial slice-token sums
-      if ((rc = pa::mfma::project_softmax(s, blob, x, nullptr, wp, partials, compute_units(), st))) return rc;
-    } else {
-      if ((rc = pa::mfma::project_softmax(s, blob, x, fxp, wp, nullptr, compute_units(), st))) return rc;
-      if ((rc = pa::mfma::slice_reduce(s, wp, fxp, partials, st))) return rc;
-    }
-    if ((rc = pa::mfma::combine_attention(s, *p, partials, mp.G, tok, norm, tok_out, tokp, st))) return rc;
-    return pa::mfma::deslice_project(s, blob, wp, tokp, y, tail_active(tail) ? tail : nullptr, compute_units(), st);
+    return mfma_layer(s, *p, blob, x, y, tail, slice_token_out, ws, mp, st);
   }
   if (pa::mfma::staged_supported(dtype, s)) {
     const StagedPlan sp = plan_staged(s);

@@ -169,9 +169,24 @@ def layer_forward(x, params, dims: LayerDims, residual=None, ln_weight=None, ln_
     tok = (torch.empty(dims.B, dims.H, dims.S, dims.D, dtype=torch.float32, device=x.device)
            if return_slice_tokens else None)
     tail = _c_tail(residual, ln_weight, ln_bias, ln_eps, ln_out)
-    _lib.check(lib.pa_layer_forward(code, byref(shape), byref(_c_params(params)), x.data_ptr(), y.data_ptr(),
-                                    byref(tail), _lib.ptr(tok), workspace.data_ptr(), int(nbytes),
-                                    _lib.current_stream_ptr(x.device)), "pa_layer_forward")
+    blob = None
+    if code == _lib.PA_BF16 and lib.pa_query_path(code, byref(shape)) == 1:
+        # fused MFMA path: the repacked parameters are kept with the parameter set and reused until it changes
+        blob = params.get("_mfma_blob")
+        if blob is None:
+            n = lib.pa_mfma_buffer_bytes(byref(shape), _lib.PA_BUF_BLOB)
+            blob = torch.empty(int(n), dtype=torch.uint8, device=x.device)
+            _lib.check(lib.pa_mfma_pack_params(byref(shape), byref(_c_params(params)), blob.data_ptr(),
+                                               _lib.current_stream_ptr(x.device)), "pa_mfma_pack_params")
+            params["_mfma_blob"] = blob
+    if blob is not None:
+        _lib.check(lib.pa_mfma_layer_forward(byref(shape), byref(_c_params(params)), blob.data_ptr(), x.data_ptr(),
+                                             y.data_ptr(), byref(tail), _lib.ptr(tok), workspace.data_ptr(), int(nbytes),
+                                             _lib.current_stream_ptr(x.device)), "pa_mfma_layer_forward")
+    else:
+        _lib.check(lib.pa_layer_forward(code, byref(shape), byref(_c_params(params)), x.data_ptr(), y.data_ptr(),
+                                        byref(tail), _lib.ptr(tok), workspace.data_ptr(), int(nbytes),
+                                        _lib.current_stream_ptr(x.device)), "pa_layer_forward")
     out = y if (residual is None and ln_out is None) else (y, ln_out)
     return (out, tok) if return_slice_tokens else out
 
