@@ -176,6 +176,11 @@ int pa_deslice_project(int dtype, const pa_shape *shape, const pa_params *p, con
  * it out.  Only B, N, grid_* and conv_k of `grid` are read.  `weight` has the activation dtype. */
 int pa_rows_gemm(int dtype, const pa_shape *grid, int64_t c_in, int64_t c_out, const void *in, const void *weight,
                  const float *bias, void *out, void *stream);
+/* The same followed by an activation: act = 0 none, 1 = GELU in its erf form.  With act = 1 and a second call this is
+ * the preprocess Mlp of the model, Linear -> GELU -> Linear (TR.py:519-525, mlp_layers.py:139-173); with act = 0 and
+ * c_out = out_dim the output head ln_mlp2[1] (TR.py:305-307). */
+int pa_rows_gemm_act(int dtype, const pa_shape *grid, int64_t c_in, int64_t c_out, const void *in, const void *weight,
+                     const float *bias, int act, void *out, void *stream);
 
 /* sums[b,h,s,d] = sum_n w[b,n,h,s] v[b,n,h*D+d] for d < D, sums[b,h,s,D] = sum_n w[b,n,h,s]; float32
  * (B,H,S,D+1).  `partials` as for pa_slice_reduce.  Two passes, fixed order. */

@@ -319,7 +319,13 @@ int pa_deslice_project(int dtype, const pa_shape *shape, const pa_params *p, con
 
 int pa_rows_gemm(int dtype, const pa_shape *grid, int64_t c_in, int64_t c_out, const void *in, const void *weight,
                  const float *bias, void *out, void *stream) {
+  return pa_rows_gemm_act(dtype, grid, c_in, c_out, in, weight, bias, 0, out, stream);
+}
+
+int pa_rows_gemm_act(int dtype, const pa_shape *grid, int64_t c_in, int64_t c_out, const void *in, const void *weight,
+                     const float *bias, int act, void *out, void *stream) {
   if (!grid) return PA_ERR_NULL;
+  if (act != 0 && act != 1) return PA_ERR_UNSUPPORTED;
   if (dtype != PA_F32 && dtype != PA_BF16) return PA_ERR_UNSUPPORTED;
   if (grid->B <= 0 || grid->N <= 0 || c_in <= 0 || c_out <= 0 || grid->conv_k < 0) return PA_ERR_DIMS;
   if (c_in > (1 << 16) || c_out > (1 << 16) || grid->N > (int64_t)1 << 31) return PA_ERR_UNSUPPORTED;
@@ -334,7 +340,7 @@ int pa_rows_gemm(int dtype, const pa_shape *grid, int64_t c_in, int64_t c_out, c
   }
   if (!in || !weight || !out) return PA_ERR_NULL;
   if (!aligned16(in) || !aligned16(weight) || !aligned16(out)) return PA_ERR_ALIGN;
-  return pa::general::rows_gemm(dtype, *grid, c_in, c_out, in, weight, bias, out, static_cast<hipStream_t>(stream));
+  return pa::general::rows_gemm(dtype, *grid, c_in, c_out, in, weight, bias, act, out, static_cast<hipStream_t>(stream));
 }
 
 int pa_slice_weighted_sum(int dtype, const pa_shape *shape, const void *w, const void *v, float *partials, float *sums,

@@ -36,6 +36,9 @@ __device__ __forceinline__ void store_from_f32(bf16 *p, float v) { p->bits = f32
 __device__ __forceinline__ float round_to(const float *, float v) { return v; }
 __device__ __forceinline__ float round_to(const bf16 *, float v) { return bf16_bits_to_f32(f32_to_bf16_bits(v)); }
 
+// GELU in its erf form (torch.nn.GELU default, activations.py:198)
+__device__ __forceinline__ float gelu_erf(float v) { return 0.5f * v * (1.f + erff(v * 0.70710678118654752f)); }
+
 __device__ __forceinline__ float clamp_temperature(float t) { return fminf(fmaxf(t, kTempMin), kTempMax); }
 
 // wave64 butterfly reductions

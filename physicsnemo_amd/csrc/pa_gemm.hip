@@ -168,6 +168,10 @@ __global__ __launch_bounds__(256) void rows_gemm_mfma_kernel(GemmArgs a) {
     const float bv = bias ? bias[o] : 0.f;
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[nt][r] += bv;
+    if (a.act == 1) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[nt][r] = gelu_erf(acc[nt][r]);
+    }
     if (out) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
@@ -298,7 +302,7 @@ __global__ __launch_bounds__(512) void rows_linear_kernel(GemmArgs a) {
 }
 
 bool linear_serves(const GemmArgs &a, int nsets, size_t elem_bytes) {
-  if (elem_bytes != 2 || a.ks != 0) return false;
+  if (elem_bytes != 2 || a.ks != 0 || a.act != 0) return false;  // activations: the tiled kernel
   if (a.K != 128 && a.K != 256 && a.K != 512) return false;
   if (a.O % 32 != 0 || (a.O > 256 && a.O % 256 != 0)) return false;
   if (a.M < 4096) return false;  // small problems: the tiled kernel has less fixed cost

@@ -109,7 +109,10 @@ __global__ __launch_bounds__(256) void rows_gemm_kernel(GemmArgs a) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int o = o0 + tx * 4 + j;
-      if (o < a.O) store_from_f32(out + m * a.O + o, acc[i][j] + (bias ? bias[o] : 0.f));
+      if (o < a.O) {
+        const float v = acc[i][j] + (bias ? bias[o] : 0.f);
+        store_from_f32(out + m * a.O + o, a.act == 1 ? gelu_erf(v) : v);
+      }
     }
   }
 }
@@ -180,8 +183,6 @@ __global__ __launch_bounds__(256) void slice_softmax_kernel(const T *__restrict_
 //   w[r,h,:]   = softmax_s((logits[r,h,s] - log(-log(u[r,h,s] + 1e-8) + 1e-8)) / temp[r,h])
 // `uniform` holds the caller's U[0,1) samples in the activation type (what torch.rand_like(logits) draws).
 // ------------------------------------------------------------------------------------------------
-__device__ __forceinline__ float gelu_erf(float v) { return 0.5f * v * (1.f + erff(v * 0.70710678118654752f)); }
-
 template <typename T>
 __global__ __launch_bounds__(256) void slice_softmax_plus_kernel(
     const T *__restrict__ x_mid, const T *__restrict__ uniform, const float *__restrict__ w_slice,
@@ -655,8 +656,9 @@ int project_inputs(int dtype, const pa_shape &s, const pa_params &p, const void 
 // out[m, o] = bias[o] + sum_k A(m, k) weight[o, k] for any (c_in, c_out): a Linear over the rows when grid.conv_k == 0,
 // else the k x k (x k) convolution over grid's point grid with weight (c_out, c_in, k, k(, k)).
 int rows_gemm(int dtype, const pa_shape &grid, int64_t c_in, int64_t c_out, const void *in, const void *weight,
-              const float *bias, void *out, hipStream_t st) {
+              const float *bias, int act, void *out, hipStream_t st) {
   GemmArgs a{};
+  a.act = act;
   a.in = in;
   a.w[0] = weight;
   a.bias[0] = bias;

@@ -49,6 +49,7 @@ struct GemmArgs {
   // the packed operand layout of the MFMA slice kernels (fx_pack).  out[z] may then be NULL.
   void *out_pack[2];
   int pack_tpb, pack_heads;
+  int act;  // applied to out (not to out_pack): 0 none, 1 GELU in its erf form (torch.nn.GELU default)
 };
 
 namespace gemm {
@@ -68,7 +69,7 @@ int project_inputs(int dtype, const pa_shape &s, const pa_params &p, const void 
                    hipStream_t st);
 int out_linear(int dtype, const pa_shape &s, const pa_params &p, const void *out_x, void *y, hipStream_t st);
 int rows_gemm(int dtype, const pa_shape &grid, int64_t c_in, int64_t c_out, const void *in, const void *weight,
-              const float *bias, void *out, hipStream_t st);
+              const float *bias, int act, void *out, hipStream_t st);
 int rows_gemm_packed(const pa_shape &s, int64_t c_in, const void *in, const void *weight, const float *bias, void *out,
                      void *out_pack, hipStream_t st);
 int slice_softmax(int dtype, const pa_shape &s, const pa_params &p, const void *x_mid, void *w, hipStream_t st);

@@ -390,14 +390,24 @@ def cols_gemm(a: torch.Tensor, b: torch.Tensor, col_sums: bool = False):
     return (partials.sum(0), sums.sum(0)) if col_sums else partials.sum(0)
 
 
-def rows_gemm(inp, weight, bias, dims: LayerDims, c_in: int, c_out: int):
-    """out (B, N, c_out) = Linear or grid convolution of inp (B, N, c_in); `dims` supplies B, N and the grid."""
+def rows_gemm(inp, weight, bias, dims: LayerDims, c_in: int, c_out: int, gelu: bool = False):
+    """out (B, N, c_out) = Linear or grid convolution of inp (B, N, c_in), optionally followed by GELU (erf form);
+    `dims` supplies B, N and the grid."""
     _need_cuda(inp, weight, bias)
     out = torch.empty(dims.B, dims.N, c_out, dtype=inp.dtype, device=inp.device)
-    _lib.check(_lib.load().pa_rows_gemm(_lib.dtype_code(inp.dtype), byref(dims.c()), c_in, c_out, inp.data_ptr(),
-                                        weight.data_ptr(), _lib.ptr(bias), out.data_ptr(),
-                                        _lib.current_stream_ptr(inp.device)), "pa_rows_gemm")
+    _lib.check(_lib.load().pa_rows_gemm_act(_lib.dtype_code(inp.dtype), byref(dims.c()), c_in, c_out, inp.data_ptr(),
+                                            weight.data_ptr(), _lib.ptr(bias), 1 if gelu else 0, out.data_ptr(),
+                                            _lib.current_stream_ptr(inp.device)), "pa_rows_gemm_act")
     return out
+
+
+def linear(inp, weight, bias, gelu: bool = False):
+    """torch.nn.functional.linear over the last axis (+ optional GELU) on the library's row GEMM kernels."""
+    lead = inp.shape[:-1]
+    rows = inp.numel() // inp.shape[-1]
+    out = rows_gemm(inp.reshape(1, rows, inp.shape[-1]).contiguous(), weight, bias,
+                    LayerDims(1, rows, inp.shape[-1], 1, 1, 1), inp.shape[-1], weight.shape[0], gelu)
+    return out.reshape(*lead, weight.shape[0])
 
 
 def slice_weighted_sum(w, v, dims: LayerDims):

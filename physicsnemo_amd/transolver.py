@@ -4,8 +4,9 @@
 Inference (no gradients required): the PhysicsAttention layer, its residual add and the LayerNorm that follows it
 run in the HIP library, and so does
 the block MLP with its residual add and the LayerNorm the next block starts with whenever the fused kernel serves
-the shape (bf16, hidden 128 / 256, GELU); the remaining glue (preprocess MLP, the first LayerNorm, the output
-Linear, and every MLP the kernel does not serve) uses PyTorch-ROCm tensor ops.
+the shape (bf16, hidden 128 / 256, GELU); the preprocess MLP, the first LayerNorm and the output Linear run on the
+library's row GEMM / LayerNorm kernels; what is left to PyTorch-ROCm tensor ops is the concatenation of the inputs
+and every block MLP the fused kernel does not serve.
 Module names, registration order and state_dict keys match the reference so its checkpoints load unchanged,
 including the legacy ``linear_pre`` / ``linear_post`` MLP keys (:92-97).
 Training (gradients required): the layer runs its differentiable path (stage-level kernels forward, the library's
@@ -185,6 +186,30 @@ class Transolver(nn.Module):
         ])
         self.initialize_weights()
 
+    # ---------------------------------------------------------------- glue layers on the library kernels
+    def _glue_on_library(self, fx: torch.Tensor) -> bool:
+        """Inference on a GPU with a GELU preprocess Mlp: the preprocess Mlp, the first LayerNorm and the output Linear
+        run on the library's row kernels; otherwise (training, other activations) they are PyTorch-ROCm tensor ops."""
+        if not fx.is_cuda or self.blocks[0]._needs_grad(fx) or any(p.requires_grad for p in self.preprocess.parameters()) \
+                and torch.is_grad_enabled():
+            return False
+        act = self.preprocess.layers[1]
+        if not (isinstance(act, nn.GELU) and act.approximate == "none"):
+            return False
+        dtype = torch.get_autocast_dtype("cuda") if torch.is_autocast_enabled("cuda") else fx.dtype
+        return dtype in (torch.float32, torch.bfloat16)
+
+    def _library_linear(self, x: torch.Tensor, lin: nn.Linear, gelu: bool = False) -> torch.Tensor:
+        cache = self.__dict__.setdefault("_linear_cache", {})
+        stamp = (x.dtype, x.device, lin.weight.data_ptr(), lin.weight._version, lin.bias.data_ptr(), lin.bias._version)
+        hit = cache.get(id(lin))
+        if hit is None or hit[0] != stamp:
+            with torch.no_grad():
+                hit = (stamp, lin.weight.detach().to(device=x.device, dtype=x.dtype).contiguous().clone(),
+                       lin.bias.detach().to(device=x.device, dtype=torch.float32).contiguous().clone())
+            cache[id(lin)] = hit
+        return PF.linear(x, hit[1], hit[2], gelu=gelu)
+
     def initialize_weights(self) -> None:
         self.apply(self._init_weights)
 
@@ -230,13 +255,30 @@ class Transolver(nn.Module):
             if embedding is not None and embedding.ndim != 3:
                 embedding = embedding.reshape(embedding.shape[0], -1, embedding.shape[-1])
         fx = torch.cat((embedding.to(fx.dtype), fx), -1)  # embedding first, then the functional input (:716)
-        fx = self.preprocess(fx)
-        # each block hands the next one its residual stream and, when the fused MLP kernel ran, LayerNorm_1 of it
+        on_library = self._glue_on_library(fx)
         normed = None
+        if on_library:
+            # preprocess Mlp (Linear -> GELU -> Linear, :519-525) and the first block's LayerNorm on the library kernels
+            if torch.is_autocast_enabled("cuda"):
+                fx = fx.to(torch.get_autocast_dtype("cuda"))
+            lin1, lin2 = self.preprocess.layers[0], self.preprocess.layers[2]
+            if lin2.in_features <= 512:  # the weights-stationary row kernel holds up to 512 input features
+                fx = self._library_linear(self._library_linear(fx.contiguous(), lin1, gelu=True), lin2)
+            else:
+                fx = self.preprocess(fx).contiguous()
+            ln = self.blocks[0].ln_1
+            fx, normed = PF.residual_layernorm(fx, ln_weight=ln.weight.detach().float().contiguous(),
+                                               ln_bias=ln.bias.detach().float().contiguous(), ln_eps=ln.eps)
+        else:
+            fx = self.preprocess(fx)
+        # each block hands the next one its residual stream and, when the fused MLP kernel ran, LayerNorm_1 of it
         for k, block in enumerate(self.blocks):
             if block.last_layer:
                 fx, normed = block.forward_chain(fx, normed, block.ln_mlp2[0])
-                fx = block.ln_mlp2[1](normed) if normed is not None else block.ln_mlp2(fx)
+                if normed is not None and on_library:
+                    fx = self._library_linear(normed, block.ln_mlp2[1])  # output head (:305-307)
+                else:
+                    fx = block.ln_mlp2[1](normed) if normed is not None else block.ln_mlp2(fx)
             else:
                 fx, normed = block.forward_chain(fx, normed, self.blocks[k + 1].ln_1)
         if unflatten_output:
