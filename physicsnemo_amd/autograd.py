@@ -26,6 +26,17 @@ def _wgrad(d_out: torch.Tensor, inp: torch.Tensor):
     serves the shape, else the GEMM library and a reduction."""
     if PF.cols_gemm_supported(d_out, inp):
         return PF.cols_gemm(d_out, inp, col_sums=True)
+    ca, cb = d_out.shape[-1], inp.shape[-1]
+    rows = d_out.numel() // ca
+    fold = 32 // ca if ca < 32 and 32 % ca == 0 else 0
+    if fold and rows % fold == 0 and d_out.is_contiguous() and inp.is_contiguous():
+        # narrow d out (slice_num 16): `fold` consecutive rows side by side make 32 columns; the wanted product is the
+        # sum of the diagonal blocks of the folded one
+        a2, b2 = d_out.reshape(rows // fold, 32), inp.reshape(rows // fold, cb * fold)
+        if PF.cols_gemm_supported(a2, b2):
+            p2, s2 = PF.cols_gemm(a2, b2, col_sums=True)
+            dw = sum(p2[k * ca:(k + 1) * ca, k * cb:(k + 1) * cb] for k in range(fold))
+            return dw, s2.reshape(fold, ca).sum(0)
     return _rows(d_out).t() @ _rows(inp), _rows(d_out).sum(0, dtype=torch.float32)
 
 

@@ -1,4 +1,4 @@
-// bf16 MFMA kernels of the backward pass (shapes of the MFMA forward path with S <= 64).  They consume the packed
+// bf16 MFMA kernels of the backward pass (the shapes of the fused MFMA forward path).  They consume the packed
 // slice weights the forward kernels leave behind (w_pack) and natural-layout (B, N, H*32) activations / gradients:
 //
 //   deslice_natural_kernel        out_x[n, h, :] = sum_s w[n, h, s] tok'[h, s, :]         (input of d W_out = dy^T out_x)
@@ -124,8 +124,9 @@ __global__ __launch_bounds__(256) void backward_tables_kernel(const float *__res
 }
 
 // ------------------------------------------------------------------------------------------------
-// slice_softmax_backward_mfma_kernel: grid (G, B), H waves; wave h owns head h (its tok' / d num fragments stay in
-// registers), the W_slice fragments are shared through LDS.  Per 32-point tile and head:
+// slice_softmax_backward_mfma_kernel: grid (G, B), H waves; wave h owns head h; its tok' / d num fragments stay in
+// registers (S <= 64) or in LDS (S = 128, where the registers are needed for d w), the W_slice fragments are shared
+// through LDS.  Per 32-point tile and head:
 //   z^T  (S x pts) = W_slice . x_mid^T + b_slice                       B = x_mid rows, 16-byte natural loads
 //   dw^T (S x pts) = tok' . g^T + d num . fx_mid^T + d nrm             B = g / fx_mid rows
 //   w: unpacked from w_pack; dot = sum_s w dw; dz = (w / T) (dw - dot); dT -= sum dz z / T
@@ -134,35 +135,43 @@ __global__ __launch_bounds__(256) void backward_tables_kernel(const float *__res
 // the last valid row and their stores are masked.
 // ------------------------------------------------------------------------------------------------
 template <int S>
-__global__ __launch_bounds__(512) void slice_softmax_backward_mfma_kernel(
+__global__ __launch_bounds__(S > 64 ? 256 : 512) void slice_softmax_backward_mfma_kernel(
     const uint16_t *__restrict__ x_mid, const uint16_t *__restrict__ fx_mid, const uint16_t *__restrict__ d_out_x,
     const u32x4 *__restrict__ w_pack, const u32x4 *__restrict__ tabs, const float *__restrict__ d_norm,
     const float *__restrict__ b_slice, const float *__restrict__ temperature, uint16_t *__restrict__ d_proj,
     uint16_t *__restrict__ d_z, float *__restrict__ dT_part, int64_t N, int tpb, int H) {
   constexpr int ST = (S + 31) / 32, NCH = S / 16, ST2 = 2 * ST;
+  constexpr bool LDSTAB = S > 64;  // tok' / d num fragments of d w in LDS instead of registers
   __shared__ u32x4 wsh[(ST2 + NCH) * 64];
   __shared__ float bsl[ST * 32];
-  __shared__ float dnl[16 * ST * 32];  // d nrm of every head of this batch (H <= 16)
+  __shared__ float dnl[8 * ST * 32];  // d nrm of every head of this batch (H <= 8)
+  extern __shared__ u32x4 tabl[];     // LDSTAB: [H][2 * ST2][64]
   const BwdTablePlan tp = bwd_table_plan(S);
   const int tid = threadIdx.x, lane = tid & 63, i = lane & 31, g = lane >> 5;
-  const int h = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int h = blockIdx.z * (blockDim.x >> 6) + wave;  // grid.z walks groups of heads (S = 128: 4 waves per workgroup)
   const int b = blockIdx.y;
   const int HD = H * 32;
   const int64_t bh = (int64_t)b * H + h;
 
   for (int u = tid; u < (ST2 + NCH) * 64; u += blockDim.x) wsh[u] = tabs[u];
   for (int s = tid; s < ST * 32; s += blockDim.x) bsl[s] = s < S ? b_slice[s] : 0.f;
-  u32x4 tokA[ST2], dnA[ST2], dnT[NCH];
+  u32x4 tokA[LDSTAB ? 1 : ST2], dnA[LDSTAB ? 1 : ST2], dnT[NCH];
   {
     const u32x4 *mine = tabs + tp.shared_units + bh * tp.per_head_units + lane;
+    if constexpr (LDSTAB) {
+      for (int f = 0; f < 2 * ST2; ++f) tabl[(wave * 2 * ST2 + f) * 64 + lane] = mine[f * 64];
+    } else {
 #pragma unroll
-    for (int f = 0; f < ST2; ++f) {
-      tokA[f] = mine[f * 64];
-      dnA[f] = mine[(ST2 + f) * 64];
+      for (int f = 0; f < ST2; ++f) {
+        tokA[f] = mine[f * 64];
+        dnA[f] = mine[(ST2 + f) * 64];
+      }
     }
 #pragma unroll
     for (int cq = 0; cq < NCH; ++cq) dnT[cq] = mine[(2 * ST2 + cq) * 64];
   }
+  const u32x4 *mytab = tabl + (wave * 2 * ST2) * 64 + lane;  // LDSTAB: this head's tok' fragments, then its d num fragments
   for (int e = tid; e < H * ST * 32; e += blockDim.x) {
     const int hh = e / (ST * 32), sl = e - hh * ST * 32;
     dnl[e] = sl < S ? d_norm[((int64_t)b * H + hh) * S + sl] : 0.f;
@@ -188,22 +197,6 @@ __global__ __launch_bounds__(512) void slice_softmax_backward_mfma_kernel(
 #pragma unroll
       for (int cq = 0; cq < NCH; ++cq) wq[cq] = wsrc[cq * 64];
     }
-    f32x16 z[ST], dw[ST];
-#pragma unroll
-    for (int st = 0; st < ST; ++st) {
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        z[st][r] = bsl[32 * st + rowmap(r, g)];
-        dw[st][r] = dnl[(h * ST + st) * 32 + rowmap(r, g)];
-      }
-#pragma unroll
-      for (int kk = 0; kk < 2; ++kk) {
-        z[st] = mma(wsh[(st * 2 + kk) * 64 + lane], xm[kk], z[st]);
-        dw[st] = mma(tokA[st * 2 + kk], gg[kk], dw[st]);
-        dw[st] = mma(dnA[st * 2 + kk], fm[kk], dw[st]);
-      }
-    }
-    __builtin_amdgcn_sched_barrier(0);
     // w of this lane's (point, slices): chunk cq = 2st + half holds registers 8 half .. 8 half + 7 as bf16
     auto w_of = [&](int st, int r) {
       const int cq = 2 * st + (r >> 3), j = r & 7;
@@ -211,18 +204,39 @@ __global__ __launch_bounds__(512) void slice_softmax_backward_mfma_kernel(
       const uint32_t pair = wq[cq][j >> 1];
       return __uint_as_float((j & 1) ? (pair & 0xffff0000u) : (pair << 16));
     };
-    // per point: dot = sum_s w dw;  sum_s dz z = (sum_s w dw z - dot sum_s w z) / T  (the logits are not needed again)
+    // per point: dot = sum_s w dw;  sum_s dz z = (sum_s w dw z - dot sum_s w z) / T: the logits of a slice tile are
+    // consumed as soon as they exist, only d w stays live across the tiles
+    f32x16 dw[ST];
     float dot = 0.f, a1 = 0.f, a2 = 0.f;
 #pragma unroll
-    for (int st = 0; st < ST; ++st)
+    for (int st = 0; st < ST; ++st) {
+      f32x16 z;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        z[r] = bsl[32 * st + rowmap(r, g)];
+        dw[st][r] = dnl[(h * ST + st) * 32 + rowmap(r, g)];
+      }
+#pragma unroll
+      for (int kk = 0; kk < 2; ++kk) {
+        z = mma(wsh[(st * 2 + kk) * 64 + lane], xm[kk], z);
+        if constexpr (LDSTAB) {
+          dw[st] = mma(mytab[(st * 2 + kk) * 64], gg[kk], dw[st]);
+          dw[st] = mma(mytab[(ST2 + st * 2 + kk) * 64], fm[kk], dw[st]);
+        } else {
+          dw[st] = mma(tokA[st * 2 + kk], gg[kk], dw[st]);
+          dw[st] = mma(dnA[st * 2 + kk], fm[kk], dw[st]);
+        }
+      }
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const float w = w_of(st, r);
         const float wd = w * dw[st][r];
         dot += wd;
-        a1 = fmaf(wd, z[st][r], a1);
-        a2 = fmaf(w, z[st][r], a2);
+        a1 = fmaf(wd, z[r], a1);
+        a2 = fmaf(w, z[r], a2);
       }
+      __builtin_amdgcn_sched_barrier(0);
+    }
     dot = half_sum(dot);
     tsum += (a1 - dot * a2) * inv_t;  // a1, a2 are this lane's halves; the halves add up in the final wave sum
     f32x16(&dz)[ST] = dw;  // d z replaces d w in place
@@ -250,13 +264,13 @@ __global__ __launch_bounds__(512) void slice_softmax_backward_mfma_kernel(
   }
   // d T of this (workgroup, head): every lane holds part of the sum over its points and slices
   tsum = wave_sum(tsum);
-  if (lane == 0) dT_part[((int64_t)blockIdx.y * gridDim.x + blockIdx.x) * H + h] = -tsum * inv_t;
+  if (lane == 0) dT_part[((int64_t)blockIdx.y * gridDim.x + blockIdx.x) * H + h] = -tsum * inv_t;  // heads: disjoint
 }
 
 // ================================================================================================
 // host side
 // ================================================================================================
-bool backward_supported(const pa_shape &s) { return supported(PA_BF16, s) && s.S <= 64; }
+bool backward_supported(const pa_shape &s) { return supported(PA_BF16, s); }
 
 int64_t backward_groups(const pa_shape &s, int num_cu) {
   int64_t g = (2 * (int64_t)num_cu + s.B - 1) / s.B;
@@ -300,10 +314,15 @@ int slice_softmax_backward(const pa_shape &s, const pa_params &p, const void *x_
                      (int)(s.B * s.H), (int)s.S);
   int rc = launch_status();
   if (rc) return rc;
-  const dim3 grid((unsigned)backward_groups(s, num_cu), (unsigned)s.B), block((unsigned)(s.H * 64));
+  // S = 128: 4 waves (heads) per workgroup, one wave per SIMD, their tok' / d num fragments in (dynamic) LDS
+  const int waves = (int)(s.S > 64 ? 4 : s.H);
+  const int groups = (int)(s.H / waves);
+  const dim3 grid((unsigned)backward_groups(s, num_cu), (unsigned)s.B, (unsigned)groups), block((unsigned)(waves * 64));
   const int tpb = (int)tiles_per_batch(s);
+  const size_t lds = s.S > 64 ? (size_t)waves * 2 * 2 * ((s.S + 31) / 32) * 64 * 16 : 0;
+  if ((rc = allow_dynamic_lds(slice_softmax_backward_mfma_kernel<128>, lds))) return rc;
 #define PA_LAUNCH_BWD(SS)                                                                                              \
-  hipLaunchKernelGGL((slice_softmax_backward_mfma_kernel<SS>), grid, block, 0, st, static_cast<const uint16_t *>(x_mid), \
+  hipLaunchKernelGGL((slice_softmax_backward_mfma_kernel<SS>), grid, block, lds, st, static_cast<const uint16_t *>(x_mid), \
                      static_cast<const uint16_t *>(fx_mid), static_cast<const uint16_t *>(d_out_x),                     \
                      static_cast<const u32x4 *>(w_pack), tabs, d_norm, p.in_project_slice_bias, p.temperature,          \
                      static_cast<uint16_t *>(d_proj), static_cast<uint16_t *>(d_z), dT_part, s.N, tpb, (int)s.H)
@@ -311,6 +330,7 @@ int slice_softmax_backward(const pa_shape &s, const pa_params &p, const void *x_
     case 16: PA_LAUNCH_BWD(16); break;
     case 32: PA_LAUNCH_BWD(32); break;
     case 64: PA_LAUNCH_BWD(64); break;
+    case 128: PA_LAUNCH_BWD(128); break;
     default: return PA_ERR_UNSUPPORTED;
   }
 #undef PA_LAUNCH_BWD

@@ -134,7 +134,8 @@ def test_gradients_reach_the_input_only_when_asked():
     assert all(p.grad is None for p in hip.parameters())
 
 
-@pytest.mark.parametrize("B,N,C,S", [(2, 2048, 256, 64), (3, 1000, 128, 32), (1, 77, 128, 16), (2, 333, 256, 32)])
+@pytest.mark.parametrize("B,N,C,S", [(2, 2048, 256, 64), (3, 1000, 128, 32), (1, 77, 128, 16), (2, 333, 256, 32),
+                                     (2, 1500, 256, 128), (1, 999, 128, 128)])
 def test_bf16_mfma_backward_matches_oracle_and_general_path(B, N, C, S):
     """Shapes the bf16 MFMA backward serves (ragged N, B > 1, every S <= 64): gradients against the fp32 oracle and
     against the general-kernel backward run on the same bf16 inputs."""
