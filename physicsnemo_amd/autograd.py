@@ -45,6 +45,10 @@ def _conv_weight_grad(d_out: torch.Tensor, x: torch.Tensor, grid: tuple, k: int)
 
     d_out (B, N, O), x (B, N, C) channels-last over `grid`; returns (O, C, k, ..., k) in d_out's dtype."""
     B, O, C, nd, pad = x.shape[0], d_out.shape[-1], x.shape[-1], len(grid), k // 2
+    if nd == 2:
+        # one product against the unfolded (im2col) input: its columns are ordered (c, u, v) like the weight
+        cols = torch.nn.functional.unfold(x.reshape(B, *grid, C).permute(0, 3, 1, 2), k, padding=pad)  # (B, C k k, N)
+        return (_rows(d_out).t() @ cols.transpose(1, 2).reshape(-1, C * k * k)).reshape(O, C, k, k)
     dg, xg = d_out.reshape(B, *grid, O), x.reshape(B, *grid, C)
     dW = torch.zeros((O, C) + (k,) * nd, dtype=d_out.dtype, device=x.device)
     for tap in itertools.product(range(k), repeat=nd):
