@@ -144,3 +144,20 @@ def test_product_package_never_imports_the_oracle():
             if f.endswith((".py", ".hip", ".h", ".cpp")):
                 text = open(os.path.join(dirpath, f)).read()
                 assert "oracle" not in text.lower(), f
+
+
+def test_integration_stub_structs_match_the_binding():
+    """The ctypes stub printed in INTEGRATION.md must lay out pa_shape / pa_params / pa_block_tail like the header."""
+    import re
+    text = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+
+    def fields(cls):
+        body = text[text.index(f"class {cls}(Structure):"):]
+        body = body[:body.index("\nclass ", 1) if "\nclass " in body[1:] else None]
+        body = body[:body.index("\n\n")] if "\n\n" in body else body
+        return re.findall(r'"([a-z_A-Z0-9]+)"', body)
+
+    assert fields("pa_shape") == [n for n, _ in _lib.PaShape._fields_]
+    assert fields("pa_params") == [n for n, _ in _lib.PaParams._fields_]
+    assert fields("pa_block_tail") == [n for n, _ in _lib.PaBlockTail._fields_]
+    assert fields("pa_mlp_params") == [n for n, _ in _lib.PaMlpParams._fields_]
