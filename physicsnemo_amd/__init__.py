@@ -1,4 +1,4 @@
-"""MI355X-native forward path of Transolver's PhysicsAttention layer (hand-written HIP kernels behind a C ABI)."""
+"""MI355X-native PhysicsAttention layer of Transolver and its callers (hand-written HIP kernels behind a C ABI)."""
 from .physics_attention import (  # noqa: F401
     PhysicsAttentionBase,
     PhysicsAttentionIrregularMesh,

@@ -18,6 +18,7 @@ import numpy as np
 import torch
 import torch.nn as nn
 
+from . import checkpoint as _ckpt
 from . import functional as PF
 from .physics_attention import (PhysicsAttentionIrregularMesh, PhysicsAttentionStructuredMesh2D,
                                 PhysicsAttentionStructuredMesh3D)
@@ -151,6 +152,12 @@ class Transolver(nn.Module):
                  structured_shape: None | tuple[int, ...] = None, use_te: bool = True, time_input: bool = False,
                  plus: bool = False) -> None:
         super().__init__()
+        # constructor arguments as the reference records them for its checkpoints (core/module.py:196-223)
+        self._args = dict(functional_dim=functional_dim, out_dim=out_dim, embedding_dim=embedding_dim, n_layers=n_layers,
+                          n_hidden=n_hidden, dropout=dropout, n_head=n_head, act=act, mlp_ratio=mlp_ratio,
+                          slice_num=slice_num, unified_pos=unified_pos, ref=ref,
+                          structured_shape=list(structured_shape) if structured_shape is not None else None,
+                          use_te=use_te, time_input=time_input, plus=plus)
         if time_input:
             raise NotImplementedError("time_input=True is not built")
         self.use_te = use_te
@@ -185,6 +192,36 @@ class Transolver(nn.Module):
             for i in range(n_layers)
         ])
         self.initialize_weights()
+
+    # ---------------------------------------------------------------- .mdlus checkpoints (core/module.py:446-1070)
+    def save(self, file_name: str | None = None) -> None:
+        """Writes a ``.mdlus`` checkpoint the reference's ``Module.from_checkpoint`` / ``load`` accept."""
+        _ckpt.write_mdlus(file_name or "Transolver.mdlus", "Transolver", "physicsnemo.models.transolver.transolver",
+                          self._args, self.state_dict())
+
+    def load(self, file_name: str, map_location=None, strict: bool = True) -> None:
+        """Loads the weights of a ``.mdlus`` checkpoint (zip or legacy tar) into this model."""
+        device = map_location if map_location is not None else next(self.parameters()).device
+        _, _, state = _ckpt.read_mdlus(file_name, map_location=device)
+        self.load_state_dict(state, strict=strict)
+
+    @classmethod
+    def from_checkpoint(cls, file_name: str, override_args: dict | None = None, strict: bool = True) -> "Transolver":
+        """Builds the model from the constructor arguments stored in a ``.mdlus`` checkpoint and loads its weights.
+        ``use_te`` is the one argument the reference lets a caller override (transolver.py ``_overridable_args``)."""
+        args, _, state = _ckpt.read_mdlus(file_name)
+        if args.get("__name__") != "Transolver":
+            raise IOError(f"checkpoint holds a {args.get('__name__')!r}, not a Transolver")
+        ctor = dict(args["__args__"])
+        for key, value in (override_args or {}).items():
+            if key != "use_te":
+                raise ValueError(f"Argument '{key}' cannot be overridden for Transolver.")
+            ctor[key] = value
+        if ctor.get("structured_shape") is not None:
+            ctor["structured_shape"] = tuple(ctor["structured_shape"])
+        model = cls(**ctor)
+        model.load_state_dict(state, strict=strict)
+        return model
 
     # ---------------------------------------------------------------- glue layers on the library kernels
     def _glue_on_library(self, fx: torch.Tensor) -> bool:
