@@ -332,8 +332,22 @@ def _trunc_normal_by_rejection_(t: torch.Tensor, std: float, a: float = -2.0, b:
     return t
 
 
+class OraclePositionalEmbedding(nn.Module):
+    """physicsnemo/nn/module/embedding_layers.py:67-152 as Transolver builds it (transolver.py:532-538): not learnable,
+    embed_fn 'cos_sin', endpoint False: freqs_k = max_positions^(-k / (C/2)), output [cos(t freqs) | sin(t freqs)]."""
+
+    def __init__(self, num_channels, max_positions=10000):
+        super().__init__()
+        freqs = torch.arange(start=0, end=num_channels // 2, dtype=torch.float32) / (num_channels // 2)
+        self.register_buffer("freqs", (1 / max_positions) ** freqs)
+
+    def forward(self, x):
+        x = torch.outer(x, self.freqs)
+        return torch.cat([x.cos(), x.sin()], dim=1)
+
+
 class OracleTransolver(nn.Module):
-    """transolver.py:447-736 (use_te=False, time_input=False, plus=False).
+    """transolver.py:447-736 (use_te=False, plus=False); time_input adds the timestep embedding of :531-543, :721-725.
 
     ``init="rejection"`` draws trunc_normal_ the torch>=2.12 way (see above); ``init="native"`` calls
     this interpreter's ``nn.init.trunc_normal_``.
@@ -341,7 +355,7 @@ class OracleTransolver(nn.Module):
 
     def __init__(self, functional_dim, out_dim, embedding_dim=None, n_layers=4, n_hidden=256, dropout=0.0,
                  n_head=8, mlp_ratio=4, slice_num=32, unified_pos=False, ref=8, structured_shape=None,
-                 init="native"):
+                 init="native", time_input=False):
         super().__init__()
         if n_hidden % n_head != 0:
             raise ValueError(f"Transolver requires n_hidden % n_head == 0, but got n_hidden={n_hidden}, n_head={n_head}")
@@ -357,6 +371,10 @@ class OracleTransolver(nn.Module):
             self.embedding_dim = embedding_dim
         self.preprocess = OracleMlp(functional_dim + self.embedding_dim, n_hidden * 2, n_hidden)
         self.n_hidden = n_hidden
+        self.time_input = time_input
+        if time_input:  # transolver.py:531-543
+            self.time_embed = OraclePositionalEmbedding(n_hidden)
+            self.time_fc = nn.Sequential(nn.Linear(n_hidden, n_hidden), nn.SiLU(), nn.Linear(n_hidden, n_hidden))
         self.blocks = nn.ModuleList([
             OracleTransolverBlock(n_head, n_hidden, dropout, mlp_ratio=mlp_ratio, out_dim=out_dim,
                                   slice_num=slice_num, spatial_shape=structured_shape,
@@ -378,7 +396,7 @@ class OracleTransolver(nn.Module):
             nn.init.constant_(m.bias, 0)
             nn.init.constant_(m.weight, 1.0)
 
-    def forward(self, fx, embedding=None):
+    def forward(self, fx, embedding=None, time=None):
         if fx.ndim < 2:
             raise ValueError(f"Expected input tensor with at least 2 dimensions, got {fx.ndim}D tensor with shape {tuple(fx.shape)}")
         if not self.unified_pos and embedding is None:
@@ -394,6 +412,9 @@ class OracleTransolver(nn.Module):
                 embedding = embedding.reshape(embedding.shape[0], -1, embedding.shape[-1])
         fx = torch.cat((embedding, fx), -1)  # embedding FIRST (:716)
         fx = self.preprocess(fx)
+        if time is not None:  # :721-725: the (B, C) embedding is repeated over the tokens, then goes through time_fc
+            time_emb = self.time_embed(time).unsqueeze(1).repeat(1, fx.shape[1], 1)
+            fx = fx + self.time_fc(time_emb)
         for blk in self.blocks:
             fx = blk(fx)
         if unflatten:

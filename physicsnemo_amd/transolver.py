@@ -1,5 +1,5 @@
 """Host-side mirror of the caller of the hot path: TransolverBlock and Transolver
-(physicsnemo/models/transolver/transolver.py:137-309 and :447-736, use_te=False, time_input=False, plus=False).
+(physicsnemo/models/transolver/transolver.py:137-309 and :447-736, use_te=False).
 
 Inference (no gradients required): the PhysicsAttention layer, its residual add and the LayerNorm that follows it
 run in the HIP library, and so does
@@ -54,6 +54,26 @@ class Mlp(nn.Module):
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         return self.layers(x)
+
+
+class PositionalEmbedding(nn.Module):
+    """Timestep features [cos(t f_k) | sin(t f_k)], f_k = max_positions^(-k / (C/2)) (reference
+    physicsnemo/nn/module/embedding_layers.py:67-152 with the arguments Transolver passes, transolver.py:532-538)."""
+
+    def __init__(self, num_channels: int, max_positions: int = 10000):
+        super().__init__()
+        freqs = torch.arange(start=0, end=num_channels // 2, dtype=torch.float32) / (num_channels // 2)
+        self.register_buffer("freqs", (1 / max_positions) ** freqs)
+        self.register_load_state_dict_pre_hook(self._fill_missing_freqs)
+
+    @staticmethod
+    def _fill_missing_freqs(module, state_dict, prefix, *_args, **_kwargs):
+        if prefix + "freqs" not in state_dict:  # older checkpoints kept freqs out of the state dict (:135-140)
+            state_dict[prefix + "freqs"] = module.freqs.clone()
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        x = torch.outer(x, self.freqs)
+        return torch.cat([x.cos(), x.sin()], dim=1)
 
 
 class TransolverBlock(nn.Module):
@@ -158,8 +178,6 @@ class Transolver(nn.Module):
                           slice_num=slice_num, unified_pos=unified_pos, ref=ref,
                           structured_shape=list(structured_shape) if structured_shape is not None else None,
                           use_te=use_te, time_input=time_input, plus=plus)
-        if time_input:
-            raise NotImplementedError("time_input=True is not built")
         self.use_te = use_te
         if not n_hidden % n_head == 0:
             raise ValueError(
@@ -185,6 +203,9 @@ class Transolver(nn.Module):
         self.preprocess = Mlp(functional_dim + self.embedding_dim, n_hidden * 2, n_hidden, act)
         self.time_input = time_input
         self.n_hidden = n_hidden
+        if time_input:  # timestep embedding and its projection (reference :531-543)
+            self.time_embed = PositionalEmbedding(n_hidden)
+            self.time_fc = nn.Sequential(nn.Linear(n_hidden, n_hidden), nn.SiLU(), nn.Linear(n_hidden, n_hidden))
         self.blocks = nn.ModuleList([
             TransolverBlock(num_heads=n_head, hidden_dim=n_hidden, dropout=dropout, act=act, mlp_ratio=mlp_ratio,
                             out_dim=out_dim, slice_num=slice_num, spatial_shape=structured_shape,
@@ -227,8 +248,8 @@ class Transolver(nn.Module):
     def _glue_on_library(self, fx: torch.Tensor) -> bool:
         """Inference on a GPU with a GELU preprocess Mlp: the preprocess Mlp, the first LayerNorm and the output Linear
         run on the library's row kernels; otherwise (training, other activations) they are PyTorch-ROCm tensor ops."""
-        if not fx.is_cuda or self.blocks[0]._needs_grad(fx) or any(p.requires_grad for p in self.preprocess.parameters()) \
-                and torch.is_grad_enabled():
+        if not fx.is_cuda or (torch.is_grad_enabled() and (fx.requires_grad or any(p.requires_grad
+                                                                                   for p in self.parameters()))):
             return False
         act = self.preprocess.layers[1]
         if not (isinstance(act, nn.GELU) and act.approximate == "none"):
@@ -280,8 +301,8 @@ class Transolver(nn.Module):
                 f"Expected input tensor with at least 2 dimensions, got {fx.ndim}D tensor with shape {tuple(fx.shape)}")
         if not self.unified_pos and embedding is None:
             raise ValueError("Embedding is required when unified_pos=False")
-        if time is not None:
-            raise NotImplementedError("time input is not built")
+        if time is not None and not self.time_input:
+            raise ValueError("time was given but the model was built with time_input=False")
         unflatten_output = False
         if self.unified_pos:
             embedding = self.embedding.repeat(fx.shape[0], 1, 1)
@@ -303,11 +324,17 @@ class Transolver(nn.Module):
                 fx = self._library_linear(self._library_linear(fx.contiguous(), lin1, gelu=True), lin2)
             else:
                 fx = self.preprocess(fx).contiguous()
+        else:
+            fx = self.preprocess(fx)
+        if time is not None:
+            # every token of a batch gets the same vector, so time_fc runs on (B, C) and is broadcast (reference
+            # :721-725 repeats first; the arithmetic per token is the same)
+            time_emb = self.time_fc(self.time_embed(time.to(torch.float32)))
+            fx = (fx + time_emb.to(fx.dtype).unsqueeze(1)).contiguous()
+        if on_library:
             ln = self.blocks[0].ln_1
             fx, normed = PF.residual_layernorm(fx, ln_weight=ln.weight.detach().float().contiguous(),
                                                ln_bias=ln.bias.detach().float().contiguous(), ln_eps=ln.eps)
-        else:
-            fx = self.preprocess(fx)
         # each block hands the next one its residual stream and, when the fused MLP kernel ran, LayerNorm_1 of it
         for k, block in enumerate(self.blocks):
             if block.last_layer:

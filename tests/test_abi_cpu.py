@@ -204,3 +204,36 @@ def test_mdlus_checkpoints_round_trip_and_legacy_tar(tmp_path):
     bad.write_bytes(b"not an archive")
     with pytest.raises(IOError):
         ck.read_mdlus(str(bad))
+
+
+def test_time_input_model_matches_oracle_layout_and_embedding_closed_forms():
+    from oracle import torch_oracle as to
+    kw = dict(functional_dim=2, out_dim=1, embedding_dim=2, n_layers=2, n_hidden=32, n_head=4, slice_num=8, mlp_ratio=2)
+    torch.manual_seed(5)
+    m = pn.Transolver(time_input=True, use_te=False, **kw)
+    torch.manual_seed(5)
+    o = to.OracleTransolver(time_input=True, **kw)
+    assert list(m.state_dict()) == list(o.state_dict())
+    assert all(torch.equal(m.state_dict()[k], o.state_dict()[k]) for k in m.state_dict())
+    assert "time_embed.freqs" in m.state_dict() and "time_fc.2.bias" in m.state_dict()
+    # the embedding: f_k = 10000^(-k/16) for 32 channels; t = 0 gives [1..1 | 0..0]; cos first, then sin
+    emb = o.time_embed
+    k = torch.arange(16, dtype=torch.float64)
+    assert torch.allclose(emb.freqs.double(), 10000.0 ** (-k / 16), rtol=1e-6)
+    e0 = emb(torch.zeros(3))
+    assert torch.equal(e0[:, :16], torch.ones(3, 16)) and torch.equal(e0[:, 16:], torch.zeros(3, 16))
+    t = torch.tensor([0.3, 7.0])
+    e = emb(t).double()
+    assert torch.allclose(e[:, 0], torch.cos(t.double()), atol=1e-6) and torch.allclose(e[:, 16], torch.sin(t.double()), atol=1e-6)
+    assert torch.allclose(e[:, :16] ** 2 + e[:, 16:] ** 2, torch.ones(2, 16, dtype=torch.float64), atol=1e-6)
+    # a time_fc whose last Linear is zero leaves the model equal to the one evaluated without time
+    fx, pos = torch.randn(2, 20, 2), torch.randn(2, 20, 2)
+    with torch.no_grad():
+        o.time_fc[2].weight.zero_()
+        o.time_fc[2].bias.zero_()
+        assert torch.equal(o(fx, pos, time=t), o(fx, pos))
+    # old checkpoints without the freqs buffer still load (reference embedding_layers.py:135-140)
+    sd = {k: v for k, v in o.state_dict().items() if k != "time_embed.freqs"}
+    m.load_state_dict(sd)
+    with pytest.raises(ValueError, match="time_input=False"):
+        pn.Transolver(use_te=False, **kw)(fx, pos, time=t)

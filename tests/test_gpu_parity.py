@@ -268,3 +268,21 @@ def test_rows_gemm_entry_point(dtype, B, N, cin, cout, grid, k):
         assert_fp32_close(got, want, "rows gemm")
     else:
         assert_rel_l2(got, want, "rows gemm", tol=5e-3)
+
+
+def test_time_input_model_forward():
+    announce("Transolver with time_input")
+    torch.manual_seed(0)
+    kw = dict(functional_dim=2, out_dim=3, embedding_dim=3, n_layers=2, n_hidden=64, n_head=4, slice_num=8, mlp_ratio=2)
+    m = pn.Transolver(time_input=True, use_te=False, **kw).eval().cuda()
+    ref = to.OracleTransolver(time_input=True, **kw).eval()
+    ref.load_state_dict(m.state_dict())
+    fx, emb, t = torch.randn(3, 150, 2), torch.randn(3, 150, 3), torch.tensor([0.0, 12.5, 400.0])
+    with torch.no_grad():
+        want = ref(fx, emb, time=t)
+        got = m(fx.cuda(), emb.cuda(), time=t.cuda())
+        assert_fp32_close(got, want, "model with time")
+        assert not torch.allclose(got.cpu(), ref(fx, emb), atol=1e-3)  # the time input matters
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            got16 = m(fx.cuda(), emb.cuda(), time=t.cuda())
+        assert_rel_l2(got16, want, "model with time, bf16 autocast", tol=3e-2)
