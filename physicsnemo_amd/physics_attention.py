@@ -137,7 +137,7 @@ class PhysicsAttentionBase(nn.Module):
         if torch.is_autocast_enabled("cuda"):
             ac = torch.get_autocast_dtype("cuda")
             if ac != torch.bfloat16:
-                raise TypeError(f"autocast dtype {ac} is not supported (bfloat16 only)")
+                raise TypeError(f"autocast dtype {ac} is not supported (bfloat16, or float16 served in float32)")
             x = x.to(torch.bfloat16)
         if x.dtype not in (torch.float32, torch.bfloat16):
             raise TypeError(f"expected float32 or bfloat16 input, got {x.dtype}")
@@ -160,9 +160,20 @@ class PhysicsAttentionBase(nn.Module):
             self.in_project_slice.bias, self.temperature, self.qkv_project.weight, self.out_linear.weight,
             self.out_linear.bias)
 
+    @staticmethod
+    def _wants_fp16(x: torch.Tensor) -> bool:
+        """float16 inputs / float16 autocast (the reference's AMP smoke tests): there are no float16 kernels; the layer
+        then computes in float32 with autocast off and hands back float16, i.e. at least the precision asked for."""
+        if x.dtype == torch.float16:
+            return True
+        return torch.is_autocast_enabled("cuda") and torch.get_autocast_dtype("cuda") == torch.float16
+
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         """(B, N, C) -> (B, N, C); replaces reference forward :501-558.  With gradients enabled on tensors that
         require them the differentiable path runs (stage-level kernels + backward kernels)."""
+        if x.is_cuda and self._wants_fp16(x):
+            with torch.autocast("cuda", enabled=False):
+                return self.forward(x.float()).to(torch.float16)
         self._validate(x)
         needs_grad = self._needs_grad(x)
         x = self._prepare_input(x)
@@ -199,6 +210,9 @@ class PhysicsAttentionBase(nn.Module):
     def forward_block(self, x: torch.Tensor, residual: torch.Tensor, ln: nn.LayerNorm):
         """Layer + the caller block's ``+ residual`` and following LayerNorm in one pass
         (physicsnemo/models/transolver/transolver.py:300-303).  Returns (fx_new, LayerNorm(fx_new))."""
+        if x.is_cuda and self._wants_fp16(x):
+            with torch.autocast("cuda", enabled=False):  # float32 inside, as the residual stream of the caller is
+                return self.forward_block(x.float(), residual.float(), ln)
         self._validate(x)
         if self.plus:
             y = self.forward_with_noise(x, None)

@@ -286,3 +286,38 @@ def test_time_input_model_forward():
         with torch.autocast("cuda", dtype=torch.bfloat16):
             got16 = m(fx.cuda(), emb.cuda(), time=t.cuda())
         assert_rel_l2(got16, want, "model with time, bf16 autocast", tol=3e-2)
+
+
+def test_fp16_autocast_is_served_and_memory_does_not_grow():
+    """The reference's optimisation smoke tests run AMP with float16 on GPUs, and its layer tests bound the memory
+    growth over repeated forwards (test_physics_attention.py:745-781): both must hold for the drop-in."""
+    announce("fp16 autocast + memory growth")
+    ref, hip = make_pair("irregular", 64, 4, 16, 8)
+    x = torch.randn(2, 300, 64)
+    with torch.no_grad():
+        want = ref(x)
+        with torch.autocast("cuda", dtype=torch.float16):
+            y = hip(x.cuda())
+        assert y.dtype == torch.float16
+        assert_rel_l2(y, want, "fp16 autocast y", tol=2e-3)
+        assert hip(x.cuda().half()).dtype == torch.float16
+    torch.manual_seed(0)
+    m = pn.Transolver(functional_dim=2, out_dim=1, embedding_dim=2, n_layers=2, n_hidden=64, n_head=4, slice_num=8,
+                      mlp_ratio=2, use_te=False).eval().cuda()
+    o = to.OracleTransolver(functional_dim=2, out_dim=1, embedding_dim=2, n_layers=2, n_hidden=64, n_head=4, slice_num=8,
+                            mlp_ratio=2).eval()
+    o.load_state_dict(m.state_dict())
+    fx, emb = torch.randn(2, 300, 2), torch.randn(2, 300, 2)
+    with torch.no_grad():
+        with torch.autocast("cuda", dtype=torch.float16):
+            out = m(fx.cuda(), emb.cuda())
+        assert_rel_l2(out, o(fx, emb), "fp16 autocast model", tol=1e-2)
+        xb = x.cuda()
+        for _ in range(3):
+            hip(xb)
+        torch.cuda.synchronize()
+        before = torch.cuda.memory_allocated()
+        for _ in range(10):
+            hip(xb)
+        torch.cuda.synchronize()
+        assert torch.cuda.memory_allocated() - before < 1 << 20
