@@ -255,10 +255,10 @@ int pa_mfma_backward_query(const pa_shape *shape);
 /* Weight-gradient product over the row axis (d W = d out^T . in, the adjoint of a Linear): for bf16 matrices a
  * (rows, lda) and b (rows, ldb) in natural layout,  P[i][j] = sum_m a[m][i] * b[m][j]  for i < cols_a, j < cols_b.
  * cols_a, cols_b multiples of 32 (cols_b in {32, 64, 128, 256}; cols_a <= 256 or a multiple of 256); lda, ldb multiples
- * of 8.  The kernel leaves pa_cols_gemm_chunks(rows) partial results, partials (chunks, cols_a, cols_b) float32; the
+ * of 8.  The kernel leaves pa_cols_gemm_chunks(rows, cols_a) partial results, partials (chunks, cols_a, cols_b) float32; the
  * caller adds them up over the first index (fixed order: deterministic).  col_sum_partials (chunks, cols_a) float32,
  * optional (NULL to skip): the column sums of a, i.e. the bias gradient that goes with the weight gradient. */
-int64_t pa_cols_gemm_chunks(int64_t rows);
+int64_t pa_cols_gemm_chunks(int64_t rows, int64_t cols_a);
 int pa_cols_gemm(int64_t rows, const void *a, int64_t lda, int64_t cols_a, const void *b, int64_t ldb, int64_t cols_b,
                  float *partials, float *col_sum_partials, void *stream);
 /* bf16 Linear over the rows of `in` (B, N, c_in) -> H*32 columns, weight (H*32, c_in) bf16, bias float32 or NULL:
@@ -305,6 +305,14 @@ int pa_mlp_forward(int dtype, int64_t rows, int64_t C, int64_t F, const pa_mlp_p
 /* The block tail on its own (TR.py:300-303, :305-307): y (rows, C) <- y + tail->residual (if given), then
  * tail->ln_out = LayerNorm(y) (if given).  For callers whose producer of y is not one of the fused kernels. */
 int pa_residual_layernorm(int dtype, int64_t rows, int64_t C, void *y, const pa_block_tail *tail, void *stream);
+
+/* Backward of LayerNorm over the last axis (TR.py:210, :300-307; the reference relies on autograd): x, dy, dx (rows, C)
+ * in the activation dtype, C a multiple of 4 (float32) / 8 (bf16) and <= 1024; the statistics are recomputed from x.
+ * partials: float32 (pa_layernorm_backward_groups(rows), 2, C): [g][0][:] = that group's share of d gamma,
+ * [g][1][:] of d beta; the caller adds them up over g. */
+int64_t pa_layernorm_backward_groups(int64_t rows);
+int pa_layernorm_backward(int dtype, int64_t rows, int64_t C, const void *x, const void *dy, const float *gamma,
+                          float eps, void *dx, float *partials, void *stream);
 
 /* ---- whole layer ------------------------------------------------------------------------------ */
 

@@ -26,7 +26,7 @@ EXPORTED = [
     "pa_mfma_backward_query", "pa_rows_gemm_packed", "pa_mfma_slice_weighted_sum", "pa_mfma_deslice",
     "pa_mfma_backward_tables_bytes", "pa_mfma_backward_groups", "pa_mfma_slice_softmax_backward",
     "pa_cols_gemm_chunks", "pa_cols_gemm", "pa_residual_layernorm",
-    "pa_mfma_layer_forward", "pa_rows_gemm_act",
+    "pa_mfma_layer_forward", "pa_rows_gemm_act", "pa_layernorm_backward_groups", "pa_layernorm_backward",
 ]
 
 PA_BUF_BLOB, PA_BUF_FX_PACK, PA_BUF_W_PACK, PA_BUF_PARTIALS, PA_BUF_TOKP = range(5)
@@ -145,7 +145,7 @@ def load() -> ctypes.CDLL:
     lib.pa_mfma_slice_softmax_backward.restype = c_int
     lib.pa_mfma_slice_softmax_backward.argtypes = [ps, pp] + [c_void_p] * 12
     lib.pa_cols_gemm_chunks.restype = c_int64
-    lib.pa_cols_gemm_chunks.argtypes = [c_int64]
+    lib.pa_cols_gemm_chunks.argtypes = [c_int64, c_int64]
     lib.pa_cols_gemm.restype = c_int
     lib.pa_cols_gemm.argtypes = [c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_void_p]
     lib.pa_residual_layernorm.restype = c_int
@@ -154,6 +154,11 @@ def load() -> ctypes.CDLL:
     lib.pa_mfma_layer_forward.argtypes = [ps, pp, c_void_p, c_void_p, c_void_p, pt, c_void_p, c_void_p, c_int64, c_void_p]
     lib.pa_rows_gemm_act.restype = c_int
     lib.pa_rows_gemm_act.argtypes = [c_int, ps, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p]
+    lib.pa_layernorm_backward_groups.restype = c_int64
+    lib.pa_layernorm_backward_groups.argtypes = [c_int64]
+    lib.pa_layernorm_backward.restype = c_int
+    lib.pa_layernorm_backward.argtypes = [c_int, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p,
+                                          c_void_p]
     _lib = lib
     return lib
 

@@ -166,3 +166,69 @@ class PhysicsAttentionMfmaFunction(torch.autograd.Function):
         out_x = st.deslice()
         d_proj, d_z, d_temp = st.slice_softmax_backward(x_mid, fx_mid, g, d_num, d_norm)
         return _finish_backward(ctx, x, dy, out_x, d_wqkv, d_proj, d_z, d_temp, x_mid, temperature)
+
+
+class LinearFunction(torch.autograd.Function):
+    """torch.nn.functional.linear for the block MLP in bf16 training: the two row GEMMs (forward, input gradient) go to
+    the GEMM library, the weight and bias gradients -- products over the huge row axis, where the library's kernels
+    leave most of the machine idle -- to `cols_gemm_kernel`, which also returns them in float32."""
+
+    @staticmethod
+    def forward(ctx, x, weight, bias):
+        w16 = weight.to(x.dtype)
+        ctx.save_for_backward(x, w16)
+        ctx.param_dtypes = (weight.dtype, bias.dtype if bias is not None else None)
+        return torch.nn.functional.linear(x, w16, bias.to(x.dtype) if bias is not None else None)
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, w16 = ctx.saved_tensors
+        dy = dy.contiguous()
+        dx = (dy @ w16) if ctx.needs_input_grad[0] else None
+        dw = db = None
+        if ctx.needs_input_grad[1] or ctx.needs_input_grad[2]:
+            dy2, x2 = _rows(dy), _rows(x).contiguous()
+            if PF.cols_gemm_supported(dy2, x2):
+                dw, db = PF.cols_gemm(dy2, x2, col_sums=True)
+            elif PF.cols_gemm_supported(x2, dy2):  # wide output, narrow input: form (x^T dy) and transpose
+                dw = PF.cols_gemm(x2, dy2).t()
+                db = dy2.sum(0, dtype=torch.float32)
+            else:
+                dw, db = dy2.t() @ x2, dy2.sum(0, dtype=torch.float32)
+            dw = dw.to(ctx.param_dtypes[0])
+            db = db.to(ctx.param_dtypes[1]) if ctx.param_dtypes[1] is not None else None
+        return dx, dw, db
+
+
+def linear(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None) -> torch.Tensor:
+    """Differentiable linear layer; on bf16 GPU tensors the weight gradient runs on the library's kernel."""
+    if x.is_cuda and x.dtype == torch.bfloat16:
+        return LinearFunction.apply(x.contiguous(), weight, bias)
+    return torch.nn.functional.linear(x, weight, bias)
+
+
+class LayerNormFunction(torch.autograd.Function):
+    """LayerNorm over the last axis on the library's kernels, forward and backward, in the input's dtype (fp32 or bf16;
+    statistics in fp32).  The backward recomputes the statistics from the saved input."""
+
+    @staticmethod
+    def forward(ctx, x, weight, bias, eps):
+        x = x.contiguous()
+        w32, b32 = weight.detach().float().contiguous(), bias.detach().float().contiguous()
+        _, out = PF.residual_layernorm(x, ln_weight=w32, ln_bias=b32, ln_eps=eps)
+        ctx.save_for_backward(x, w32)
+        ctx.eps, ctx.param_dtypes = eps, (weight.dtype, bias.dtype)
+        return out
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, w32 = ctx.saved_tensors
+        dx, dg, db = PF.layernorm_backward(x, dy.to(x.dtype).contiguous(), w32, ctx.eps)
+        return dx, dg.to(ctx.param_dtypes[0]), db.to(ctx.param_dtypes[1]), None
+
+
+def layer_norm(x: torch.Tensor, ln: torch.nn.LayerNorm) -> torch.Tensor:
+    """Differentiable LayerNorm: the library's kernels where they serve the rows, the module itself otherwise."""
+    if len(ln.normalized_shape) == 1 and ln.elementwise_affine and ln.bias is not None and PF.layernorm_supported(x):
+        return LayerNormFunction.apply(x, ln.weight, ln.bias, ln.eps)
+    return ln(x)

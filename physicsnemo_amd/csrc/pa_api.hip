@@ -421,9 +421,24 @@ int pa_residual_layernorm(int dtype, int64_t rows, int64_t C, void *y, const pa_
   return pa::general::residual_ln(dtype, s, y, *tail, static_cast<hipStream_t>(stream));
 }
 
-int64_t pa_cols_gemm_chunks(int64_t rows) {
+int64_t pa_layernorm_backward_groups(int64_t rows) {
   if (rows <= 0) return PA_ERR_DIMS;
-  return pa::gemm::cols_gemm_chunks(rows, compute_units());
+  return pa::general::layernorm_backward_groups(rows);
+}
+
+int pa_layernorm_backward(int dtype, int64_t rows, int64_t C, const void *x, const void *dy, const float *gamma, float eps,
+                          void *dx, float *partials, void *stream) {
+  if (dtype != PA_F32 && dtype != PA_BF16) return PA_ERR_UNSUPPORTED;
+  if (rows <= 0 || C <= 0 || C > 1024) return PA_ERR_DIMS;
+  if (!x || !dy || !gamma || !dx || !partials) return PA_ERR_NULL;
+  if (!aligned16(x) || !aligned16(dy) || !aligned16(dx)) return PA_ERR_ALIGN;
+  return pa::general::layernorm_backward(dtype, rows, C, x, dy, gamma, eps, dx, partials,
+                                         static_cast<hipStream_t>(stream));
+}
+
+int64_t pa_cols_gemm_chunks(int64_t rows, int64_t cols_a) {
+  if (rows <= 0 || cols_a <= 0) return PA_ERR_DIMS;
+  return pa::gemm::cols_gemm_chunks(rows, cols_a, compute_units());
 }
 
 int pa_cols_gemm(int64_t rows, const void *a, int64_t lda, int64_t cols_a, const void *b, int64_t ldb, int64_t cols_b,

@@ -427,10 +427,12 @@ __global__ __launch_bounds__(512) void cols_gemm_kernel(const uint16_t *__restri
   }
 }
 
-int64_t cols_gemm_chunks(int64_t M, int num_cu) {
-  const int64_t nblk = (M + 31) / 32;
-  int64_t g = 2 * (int64_t)num_cu;
-  if (g > nblk) g = nblk;
+// row chunks: about two workgroups per CU over all column groups, and at least 32 blocks of 32 rows per chunk so that
+// the partial results stay small next to the rows a chunk reads
+int64_t cols_gemm_chunks(int64_t M, int64_t OA, int num_cu) {
+  const int64_t nblk = (M + 31) / 32, gy = (OA + 255) / 256;
+  int64_t g = 2 * (int64_t)num_cu / gy;
+  if (g > nblk / 32) g = nblk / 32;
   return g < 1 ? 1 : g;
 }
 
@@ -438,7 +440,7 @@ int cols_gemm(const void *A, int64_t lda, int64_t OA, const void *B, int64_t ldb
               float *partials, float *col_sums, int num_cu, hipStream_t st) {
   if (OA % 32 != 0 || OB % 32 != 0 || OA <= 0 || OB <= 0 || lda % 8 != 0 || ldb % 8 != 0) return PA_ERR_UNSUPPORTED;
   if (OA > 256 && OA % 256 != 0) return PA_ERR_UNSUPPORTED;
-  const int64_t G = cols_gemm_chunks(M, num_cu);
+  const int64_t G = cols_gemm_chunks(M, OA, num_cu);
   const int64_t nblk = (M + 31) / 32;
   const int64_t per = (nblk + G - 1) / G;
   const dim3 grid((unsigned)G, (unsigned)((OA + 255) / 256)), block((unsigned)((OA < 256 ? OA : 256) * 2));

@@ -591,6 +591,107 @@ __global__ __launch_bounds__(256) void residual_ln_vec_kernel(T *__restrict__ y,
   }
 }
 
+// layernorm_backward_kernel: backward of y = (x - mean) * rstd * gamma + beta over rows of whole 16-byte units.
+//   xh = (x - mean) rstd;  g = dy gamma;  dx = rstd (g - mean_c(g) - xh mean_c(g xh));  d gamma = sum_rows dy xh;
+//   d beta = sum_rows dy.   One wave per row at a time (statistics recomputed from x), lane l owns units l, l + 64, ...;
+// every wave accumulates d gamma / d beta of its columns over the rows it walks, the four waves of a workgroup add up
+// through LDS and each workgroup leaves one partial [2][C] (the caller adds the partials in index order).
+template <typename T, int UPL>
+__global__ __launch_bounds__(256) void layernorm_backward_kernel(const T *__restrict__ x, const T *__restrict__ dy,
+                                                                 const float *__restrict__ gamma, float eps,
+                                                                 T *__restrict__ dx, float *__restrict__ partials,
+                                                                 int64_t M, int C) {
+  constexpr int UE = 16 / sizeof(T);
+  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+  extern __shared__ float red[];  // [4 waves][2][C]
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int units = C / UE;
+  float gam[UPL][UE], dg[UPL][UE], db[UPL][UE];
+#pragma unroll
+  for (int k = 0; k < UPL; ++k)
+#pragma unroll
+    for (int e = 0; e < UE; ++e) {
+      const int c = (lane + 64 * k) * UE + e;
+      gam[k][e] = c < C ? gamma[c] : 0.f;
+      dg[k][e] = db[k][e] = 0.f;
+    }
+  const float inv_c = 1.f / (float)C;
+  for (int64_t m = (int64_t)blockIdx.x * 4 + wave; m < M; m += (int64_t)gridDim.x * 4) {
+    float xv[UPL][UE], gv[UPL][UE];
+    float sum = 0.f;
+#pragma unroll
+    for (int k = 0; k < UPL; ++k) {
+      const int u = lane + 64 * k;
+#pragma unroll
+      for (int e = 0; e < UE; ++e) xv[k][e] = gv[k][e] = 0.f;
+      if (u < units) {
+        u32x4 a = *reinterpret_cast<const u32x4 *>(x + m * C + u * UE);
+        u32x4 d = *reinterpret_cast<const u32x4 *>(dy + m * C + u * UE);
+        const T *ae = reinterpret_cast<const T *>(&a), *de = reinterpret_cast<const T *>(&d);
+#pragma unroll
+        for (int e = 0; e < UE; ++e) {
+          xv[k][e] = load_as_f32(ae + e);
+          gv[k][e] = load_as_f32(de + e);  // dy for now
+          sum += xv[k][e];
+        }
+      }
+    }
+    const float mean = wave_sum(sum) * inv_c;
+    float sq = 0.f;
+#pragma unroll
+    for (int k = 0; k < UPL; ++k)
+      if (lane + 64 * k < units) {
+#pragma unroll
+        for (int e = 0; e < UE; ++e) {
+          const float dlt = xv[k][e] - mean;
+          sq = fmaf(dlt, dlt, sq);
+        }
+      }
+    const float rstd = rsqrtf(wave_sum(sq) * inv_c + eps);
+    float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+    for (int k = 0; k < UPL; ++k)
+      if (lane + 64 * k < units) {
+#pragma unroll
+        for (int e = 0; e < UE; ++e) {
+          const float xh = (xv[k][e] - mean) * rstd, dyv = gv[k][e];
+          dg[k][e] = fmaf(dyv, xh, dg[k][e]);
+          db[k][e] += dyv;
+          const float g = dyv * gam[k][e];
+          xv[k][e] = xh;
+          gv[k][e] = g;
+          s1 += g;
+          s2 = fmaf(g, xh, s2);
+        }
+      }
+    s1 = wave_sum(s1) * inv_c;
+    s2 = wave_sum(s2) * inv_c;
+#pragma unroll
+    for (int k = 0; k < UPL; ++k) {
+      const int u = lane + 64 * k;
+      if (u < units) {
+        alignas(16) T o[UE];
+#pragma unroll
+        for (int e = 0; e < UE; ++e) store_from_f32(o + e, rstd * (gv[k][e] - s1 - xv[k][e] * s2));
+        *reinterpret_cast<u32x4 *>(dx + m * C + u * UE) = *reinterpret_cast<const u32x4 *>(o);
+      }
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < UPL; ++k)
+#pragma unroll
+    for (int e = 0; e < UE; ++e) {
+      const int c = (lane + 64 * k) * UE + e;
+      if (c < C) {
+        red[(wave * 2 + 0) * C + c] = dg[k][e];
+        red[(wave * 2 + 1) * C + c] = db[k][e];
+      }
+    }
+  __syncthreads();
+  for (int i = threadIdx.x; i < 2 * C; i += 256)
+    partials[(int64_t)blockIdx.x * 2 * C + i] = ((red[i] + red[2 * C + i]) + red[4 * C + i]) + red[6 * C + i];
+}
+
 // ------------------------------------------------------------------------------------------------
 // dequant_e4m3_kernel: out[o, k] = bf16(scale[o] * decode_e4m3fn(in[o, k])).  e4m3fn: 1 sign, 4 exponent (bias 7),
 // 3 mantissa bits; exponent 0 is subnormal (2^-6 * m/8); 0x7f / 0xff are NaN; there are no infinities.
@@ -862,6 +963,35 @@ static int residual_ln_t(const pa_shape &s, void *y, const pa_block_tail &tail, 
     hipLaunchKernelGGL((residual_ln_kernel<T>), grid, dim3(256), 0, st, yp, res, tail.ln_gamma, tail.ln_beta,
                        tail.ln_eps, lo, M, C);
   return launch_status();
+}
+
+int64_t layernorm_backward_groups(int64_t rows) { return std::min<int64_t>((rows + 3) / 4, 256 * 8); }
+
+template <typename T>
+static int layernorm_backward_t(int64_t rows, int C, const void *x, const void *dy, const float *gamma, float eps, void *dx,
+                                float *partials, hipStream_t st) {
+  constexpr int UE = 16 / sizeof(T);
+  if (C % UE != 0) return PA_ERR_UNSUPPORTED;
+  const int upl = (C / UE + 63) / 64;
+  const dim3 grid((unsigned)layernorm_backward_groups(rows));
+  const size_t lds = (size_t)8 * C * 4;
+  const T *xp = static_cast<const T *>(x), *dp = static_cast<const T *>(dy);
+  T *op = static_cast<T *>(dx);
+  if (upl <= 1)
+    hipLaunchKernelGGL((layernorm_backward_kernel<T, 1>), grid, dim3(256), lds, st, xp, dp, gamma, eps, op, partials, rows, C);
+  else if (upl <= 2)
+    hipLaunchKernelGGL((layernorm_backward_kernel<T, 2>), grid, dim3(256), lds, st, xp, dp, gamma, eps, op, partials, rows, C);
+  else if (upl <= 4)
+    hipLaunchKernelGGL((layernorm_backward_kernel<T, 4>), grid, dim3(256), lds, st, xp, dp, gamma, eps, op, partials, rows, C);
+  else
+    return PA_ERR_UNSUPPORTED;
+  return launch_status();
+}
+
+int layernorm_backward(int dtype, int64_t rows, int64_t C, const void *x, const void *dy, const float *gamma, float eps,
+                       void *dx, float *partials, hipStream_t st) {
+  return dtype == PA_F32 ? layernorm_backward_t<float>(rows, (int)C, x, dy, gamma, eps, dx, partials, st)
+                         : layernorm_backward_t<bf16>(rows, (int)C, x, dy, gamma, eps, dx, partials, st);
 }
 
 int residual_ln(int dtype, const pa_shape &s, void *y, const pa_block_tail &tail, hipStream_t st) {

@@ -58,7 +58,7 @@ namespace gemm {
 bool serves(const GemmArgs &a, int nsets, size_t elem_bytes);
 int launch(const GemmArgs &a, int nsets, int dtype, hipStream_t st);
 // weight-gradient products over the row axis: partials[g][oa][ob] = sum over chunk g of A[m][oa] * B[m][ob] (bf16 in)
-int64_t cols_gemm_chunks(int64_t M, int num_cu);
+int64_t cols_gemm_chunks(int64_t M, int64_t OA, int num_cu);
 int cols_gemm(const void *A, int64_t lda, int64_t OA, const void *B, int64_t ldb, int64_t OB, int64_t M,
               float *partials, float *col_sums, int num_cu, hipStream_t st);
 }  // namespace gemm
@@ -83,6 +83,9 @@ int combine_attention(const pa_shape &s, const pa_params &p, const float *partia
                       float *slice_norm, float *out_token, hipStream_t st);
 int deslice(int dtype, const pa_shape &s, const void *w, const float *out_token, void *out_x, hipStream_t st);
 int residual_ln(int dtype, const pa_shape &s, void *y, const pa_block_tail &tail, hipStream_t st);
+int64_t layernorm_backward_groups(int64_t rows);
+int layernorm_backward(int dtype, int64_t rows, int64_t C, const void *x, const void *dy, const float *gamma, float eps,
+                       void *dx, float *partials, hipStream_t st);
 }  // namespace general
 
 namespace backward {

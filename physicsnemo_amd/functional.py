@@ -202,6 +202,30 @@ def residual_layernorm(y, residual=None, ln_weight=None, ln_bias=None, ln_eps=1e
     return y if ln_out is None else (y, ln_out)
 
 
+def layernorm_supported(x: torch.Tensor) -> bool:
+    """True if the LayerNorm forward / backward kernels serve rows like x's (GPU, fp32 or bf16, whole 16-byte units)."""
+    if not x.is_cuda or x.dtype not in (torch.float32, torch.bfloat16):
+        return False
+    unit = 4 if x.dtype == torch.float32 else 8
+    return x.shape[-1] % unit == 0 and x.shape[-1] <= 1024
+
+
+def layernorm_backward(x, dy, ln_weight, ln_eps=1e-5):
+    """(dx, d gamma, d beta) of LayerNorm over the last axis; x, dy in the activation dtype, gamma float32."""
+    _need_cuda(x, dy, ln_weight)
+    lib = _lib.load()
+    C = x.shape[-1]
+    rows = x.numel() // C
+    groups = lib.pa_layernorm_backward_groups(rows)
+    partials = torch.empty(int(groups), 2, C, dtype=torch.float32, device=x.device)
+    dx = torch.empty_like(x)
+    _lib.check(lib.pa_layernorm_backward(_lib.dtype_code(x.dtype), rows, C, x.data_ptr(), dy.data_ptr(),
+                                         ln_weight.data_ptr(), float(ln_eps), dx.data_ptr(), partials.data_ptr(),
+                                         _lib.current_stream_ptr(x.device)), "pa_layernorm_backward")
+    sums = partials.sum(0)
+    return dx, sums[0], sums[1]
+
+
 def mlp_supported(dtype: torch.dtype, rows: int, C: int, F: int) -> bool:
     """True if `mlp_forward` serves this shape with the MFMA kernel (bf16, C in {128, 256}, F a multiple of 64)."""
     if dtype != torch.bfloat16:
@@ -382,7 +406,7 @@ def cols_gemm(a: torch.Tensor, b: torch.Tensor, col_sums: bool = False):
     rows = a.numel() // ca
     if b.numel() // cb != rows:
         raise ValueError("cols_gemm needs the same number of rows on both sides")
-    chunks = lib.pa_cols_gemm_chunks(rows)
+    chunks = lib.pa_cols_gemm_chunks(rows, ca)
     partials = torch.empty(int(chunks), ca, cb, dtype=torch.float32, device=a.device)
     sums = torch.empty(int(chunks), ca, dtype=torch.float32, device=a.device) if col_sums else None
     _lib.check(lib.pa_cols_gemm(rows, a.data_ptr(), ca, ca, b.data_ptr(), cb, cb, partials.data_ptr(), _lib.ptr(sums),

@@ -18,6 +18,7 @@ import numpy as np
 import torch
 import torch.nn as nn
 
+from . import autograd as PA
 from . import checkpoint as _ckpt
 from . import functional as PF
 from .physics_attention import (PhysicsAttentionIrregularMesh, PhysicsAttentionStructuredMesh2D,
@@ -127,14 +128,25 @@ class TransolverBlock(nn.Module):
     def _needs_grad(self, fx: torch.Tensor) -> bool:
         return torch.is_grad_enabled() and (fx.requires_grad or any(p.requires_grad for p in self.parameters()))
 
+    def _mlp_with_grad(self, normed: torch.Tensor) -> torch.Tensor:
+        """ln_mlp1[1] in training; under bf16 autocast its Linears use `autograd.linear` (weight gradients on the
+        library's row-axis kernel), otherwise the module as it is."""
+        mlp = self.ln_mlp1[1]
+        if normed.is_cuda and torch.is_autocast_enabled("cuda") and torch.get_autocast_dtype("cuda") == torch.bfloat16:
+            lin1, act, lin2 = mlp.layers[0], mlp.layers[1], mlp.layers[2]
+            with torch.autocast("cuda", enabled=False):
+                h = PA.linear(normed.to(torch.bfloat16), lin1.weight, lin1.bias)
+                return PA.linear(act(h), lin2.weight, lin2.bias)
+        return mlp(normed)
+
     def forward_chain(self, fx: torch.Tensor, normed_in: torch.Tensor | None, next_ln: nn.LayerNorm | None):
         """One block inside a chain of blocks: takes LayerNorm_1(fx) if the previous stage already produced it and
         returns (fx_out, next_ln(fx_out) or None).  Same arithmetic as `forward` (reference :300-303)."""
         if self._needs_grad(fx):
             # training: the layer's autograd path, LayerNorms / MLP as differentiable tensor ops (reference :300-303)
-            x_in = normed_in if normed_in is not None else self.ln_1(fx)
+            x_in = normed_in if normed_in is not None else PA.layer_norm(fx, self.ln_1)
             fx1 = self.Attn(x_in) + fx
-            return self.ln_mlp1(fx1) + fx1, None
+            return self._mlp_with_grad(PA.layer_norm(fx1, self.ln_mlp1[0])) + fx1, None
         x_in = normed_in if normed_in is not None else self.ln_1(fx)
         # fx1 = Attn(ln_1(fx)) + fx and LayerNorm(fx1) come out of one fused library call (reference :300, :303)
         fx1, normed = self.Attn.forward_block(x_in, fx, self.ln_mlp1[0])

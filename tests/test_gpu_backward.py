@@ -265,3 +265,47 @@ def test_mfma_backward_at_scale_agrees_with_general_path():
     for name in res[0]:
         if name != "temperature":
             assert_rel_l2(res[0][name], res[1][name], f"grad {name}", tol=3e-2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rows,C", [(1000, 256), (37, 48), (4096, 512), (300, 1024)])
+def test_layernorm_and_linear_autograd_functions(dtype, rows, C):
+    announce("LayerNormFunction / LinearFunction", dtype, rows, C)
+    from physicsnemo_amd import autograd as PA
+    torch.manual_seed(rows)
+    ln = torch.nn.LayerNorm(C)
+    with torch.no_grad():
+        ln.weight.uniform_(0.5, 1.5)
+        ln.bias.uniform_(-0.5, 0.5)
+    x, probe = torch.randn(2, rows, C), torch.randn(2, rows, C)
+    xr = x.to(dtype).float().clone().requires_grad_(True)  # reference: fp32 arithmetic on the same (rounded) input
+    (ln(xr) * probe).sum().backward()
+    want = (xr.grad, ln.weight.grad.clone(), ln.bias.grad.clone())
+    ln.zero_grad()
+    lng = ln.cuda()
+    xg = x.detach().to(dtype).cuda().requires_grad_(True)
+    y = PA.layer_norm(xg, lng)
+    assert y.dtype == dtype and y.grad_fn is not None
+    (y.float() * probe.cuda()).sum().backward()
+    got = (xg.grad, lng.weight.grad, lng.bias.grad)
+    for name, g, w in zip(("dx", "d gamma", "d beta"), got, want):
+        if dtype == torch.float32:
+            assert_fp32_close(g, w, name, rtol=2e-4)
+        else:
+            assert_rel_l2(g, w, name, tol=1e-2)
+    if dtype == torch.bfloat16:
+        lin = torch.nn.Linear(C, 256)
+        xr = x.detach().bfloat16().float().requires_grad_(True)
+        p2 = torch.randn(2, rows, 256)
+        (torch.nn.functional.linear(xr, lin.weight.bfloat16().float(), lin.bias) * p2).sum().backward()
+        wx = xr.grad
+        lin.zero_grad(set_to_none=True)  # the reference pass above left gradients on the parameters
+        lin = lin.cuda()
+        xg = x.detach().bfloat16().cuda().requires_grad_(True)
+        out = PA.linear(xg, lin.weight, lin.bias)
+        (out.float() * p2.cuda()).sum().backward()
+        assert lin.weight.grad.dtype == torch.float32
+        assert_rel_l2(xg.grad, wx, "linear dx", tol=1e-2)
+        ref_dw = (p2.bfloat16().float().reshape(-1, 256).t() @ x.bfloat16().float().reshape(-1, C))
+        assert_rel_l2(lin.weight.grad, ref_dw, "linear dW", tol=1e-2)
+        assert_rel_l2(lin.bias.grad, p2.bfloat16().float().reshape(-1, 256).sum(0), "linear db", tol=1e-2)
