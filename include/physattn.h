@@ -211,6 +211,20 @@ int pa_slice_softmax_backward(int dtype, const pa_shape *shape, const pa_params 
                               const float *d_num, const float *d_norm, void *d_proj, void *d_z,
                               float *d_temperature_partials, void *stream);
 
+/* The same for Transolver++ (plus = True; PA.py:166-170, :530-532, gumbel_softmax.py:49-57): one projection
+ * (fx_mid is x_mid), `uniform` the samples given to pa_slice_softmax_plus, w its output.  Outputs:
+ *   d_x_mid (B,N,H*D): the whole gradient of the projection (slice logits, aggregation and proj_temperature paths);
+ *   d_z (B,N,H,S) as above;  d_a1 (B,N,H,S), activation dtype: gradient of the proj_temperature[0] output;
+ *   d_a2 (B,N,H) float32: gradient of the proj_temperature[2] output;
+ *   d_temperature_partials: pa_backward_point_tiles_plus(shape) * H float32; d temperature[h] is the sum over the
+ *   first index (the lower clamp at 0.01 is already applied per point). */
+int64_t pa_backward_point_tiles_plus(const pa_shape *shape);
+int pa_slice_softmax_plus_backward(int dtype, const pa_shape *shape, const pa_params *p, const pa_plus_params *plus,
+                                   const void *x_mid, const void *uniform, const void *w, const void *d_out_x,
+                                   const float *out_slice_token, const float *d_num, const float *d_norm,
+                                   void *d_x_mid, void *d_z, void *d_a1, float *d_a2, float *d_temperature_partials,
+                                   void *stream);
+
 /* ---- stage-level entry points of the bf16 MFMA kernels (shapes with pa_query_path() == 1) ------
  * Intermediates use an internal register-order ("packed") layout; buffers are opaque to the caller and
  * sized by pa_mfma_buffer_bytes(shape, which):

@@ -23,6 +23,7 @@ EXPORTED = [
      "pa_mfma_combine_attention", "pa_mfma_deslice_project", "pa_mlp_query", "pa_mlp_workspace_bytes", "pa_mlp_forward",
     "pa_rows_gemm", "pa_slice_weighted_sum", "pa_backward_query", "pa_backward_point_tiles",
     "pa_slice_attention_backward", "pa_slice_softmax_backward", "pa_slice_softmax_plus",
+    "pa_backward_point_tiles_plus", "pa_slice_softmax_plus_backward",
     "pa_mfma_backward_query", "pa_rows_gemm_packed", "pa_mfma_slice_weighted_sum", "pa_mfma_deslice",
     "pa_mfma_backward_tables_bytes", "pa_mfma_backward_groups", "pa_mfma_slice_softmax_backward",
     "pa_cols_gemm_chunks", "pa_cols_gemm", "pa_residual_layernorm",
@@ -130,6 +131,10 @@ def load() -> ctypes.CDLL:
     lib.pa_slice_softmax_backward.argtypes = [c_int, ps, pp] + [c_void_p] * 11
     lib.pa_slice_softmax_plus.restype = c_int
     lib.pa_slice_softmax_plus.argtypes = [c_int, ps, pp, POINTER(PaPlusParams)] + [c_void_p] * 4
+    lib.pa_backward_point_tiles_plus.restype = c_int64
+    lib.pa_backward_point_tiles_plus.argtypes = [ps]
+    lib.pa_slice_softmax_plus_backward.restype = c_int
+    lib.pa_slice_softmax_plus_backward.argtypes = [c_int, ps, pp, POINTER(PaPlusParams)] + [c_void_p] * 13
     lib.pa_mfma_backward_query.restype = c_int
     lib.pa_mfma_backward_query.argtypes = [ps]
     lib.pa_rows_gemm_packed.restype = c_int

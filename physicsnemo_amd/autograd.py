@@ -182,6 +182,65 @@ class PhysicsAttentionMfmaFunction(torch.autograd.Function):
         return _finish_backward(ctx, x, dy, out_x, d_wqkv, d_proj, d_z, d_temp, x_mid, temperature)
 
 
+class PhysicsAttentionPlusFunction(torch.autograd.Function):
+    """Transolver++ (plus=True) layer, differentiable w.r.t. x and its twelve parameters; general kernels.  ``uniform``
+    (B, N, H, S) holds the samples behind the Gumbel noise and gets no gradient (the reference draws them with
+    ``torch.rand_like``, gumbel_softmax.py:50)."""
+
+    @staticmethod
+    def forward(ctx, x, uniform, dims, kparams, wx, bx, ws, bs, temperature, pt_w1, pt_b1, pt_w2, pt_b2, wqkv, wo, bo):
+        x_mid, _ = PF.project_inputs(x, kparams, dims)
+        w = PF.slice_softmax_plus(x_mid, uniform, kparams, dims)
+        tok, norm = PF.slice_reduce(w, x_mid, dims)
+        tok_out = PF.slice_attention(tok, kparams, dims)
+        y, out_x = PF.deslice_project(w, tok_out, kparams, dims, return_out_x=True)
+        ctx.save_for_backward(x, uniform, x_mid, w, tok, norm, tok_out, out_x)
+        ctx.dims, ctx.kparams = dims, kparams
+        ctx.param_like = (wx, bx, ws, bs, temperature, pt_w1, pt_b1, pt_w2, pt_b2, wqkv, wo, bo)
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, uniform, x_mid, w, tok, norm, tok_out, out_x = ctx.saved_tensors
+        dims, kp = ctx.dims, ctx.kparams
+        B, N, C, H, D, S = dims.B, dims.N, dims.C, dims.H, dims.D, dims.S
+        HD = H * D
+        dy = dy.to(x.dtype).contiguous()
+        linear = PF.LayerDims(B, N, C, H, D, S)
+        g = PF.rows_gemm(dy, kp["out_linear_weight"].view(C, HD).t().contiguous(), None, linear, C, HD)
+        d_tok_out = PF.slice_weighted_sum(w, g, dims)[..., :D].contiguous()
+        d_num, d_norm, d_wqkv = PF.slice_attention_backward(tok, norm, d_tok_out, kp, dims)
+        d_xm, d_z, d_a1, d_a2, d_temp = PF.slice_softmax_plus_backward(x_mid, uniform, w, g, tok_out, d_num, d_norm,
+                                                                       kp, dims)
+        d_wo, d_bo = _wgrad(dy, out_x)
+        xm_rows = x_mid.reshape(-1, D)
+        d_ws, d_bs = _wgrad(d_z.reshape(-1, S), xm_rows)
+        # proj_temperature = Linear(D, S) -> GELU -> Linear(S, 1) -> GELU: the kernel returns the gradients of the two
+        # Linear outputs; the second weight gradient needs the hidden activation again
+        d_w1, d_b1 = _wgrad(d_a1.reshape(-1, S), xm_rows)
+        hidden = torch.nn.functional.gelu(torch.addmm(kp["proj_temperature_0_bias"], xm_rows.float(),
+                                                      kp["proj_temperature_0_weight"].view(S, D).t()))
+        d_w2 = d_a2.reshape(1, -1) @ hidden
+        d_b2 = d_a2.sum().reshape(1)
+
+        k = dims.conv_k
+        wx = kp["in_project_x_weight"]
+        if k == 0:
+            dx = PF.rows_gemm(d_xm, wx.view(HD, C).t().contiguous(), None, linear, HD, C) if ctx.needs_input_grad[0] else None
+            d_wx, d_bx = _wgrad(d_xm, x)
+        else:
+            grid = (dims.grid_h, dims.grid_w) + ((dims.grid_d,) if dims.grid_d > 0 else ())
+            w_t = wx.view(HD, C, *((k,) * len(grid))).flip(dims=tuple(range(2, 2 + len(grid)))).transpose(0, 1).contiguous()
+            dx = PF.rows_gemm(d_xm, w_t, None, dims, HD, C) if ctx.needs_input_grad[0] else None
+            d_wx = _conv_weight_grad(d_xm, x, grid, k)
+            d_bx = _rows(d_xm).sum(0, dtype=torch.float32)
+
+        grads = (d_wx, d_bx, d_ws, d_bs, d_temp, d_w1, d_b1, d_w2, d_b2, d_wqkv, d_wo, d_bo)
+        grads = tuple(gr.reshape(p.shape).to(p.dtype) if ctx.needs_input_grad[4 + i] else None
+                      for i, (gr, p) in enumerate(zip(grads, ctx.param_like)))
+        return (dx, None, None, None) + grads
+
+
 class LinearFunction(torch.autograd.Function):
     """torch.nn.functional.linear for the block MLP in bf16 training: the two row GEMMs (forward, input gradient) go to
     the GEMM library, the weight and bias gradients -- products over the huge row axis, where the library's kernels

@@ -408,6 +408,36 @@ int pa_slice_softmax_backward(int dtype, const pa_shape *shape, const pa_params 
                                      d_proj, d_z, d_temperature_partials, static_cast<hipStream_t>(stream));
 }
 
+int64_t pa_backward_point_tiles_plus(const pa_shape *shape) {
+  int rc = check_backward_shape(PA_F32, shape);
+  if (rc) return rc;
+  const int64_t tiles = pa::backward::point_tiles(*shape, true);
+  return tiles == 0 ? (int64_t)PA_ERR_UNSUPPORTED : tiles;
+}
+
+int pa_slice_softmax_plus_backward(int dtype, const pa_shape *shape, const pa_params *p, const pa_plus_params *plus,
+                                   const void *x_mid, const void *uniform, const void *w, const void *d_out_x,
+                                   const float *out_slice_token, const float *d_num, const float *d_norm,
+                                   void *d_x_mid, void *d_z, void *d_a1, float *d_a2, float *d_temperature_partials,
+                                   void *stream) {
+  int rc = check_backward_shape(dtype, shape);
+  if (rc) return rc;
+  if (pa::backward::point_tile_rows(*shape, true) == 0) return PA_ERR_UNSUPPORTED;
+  if (!p || !p->in_project_slice_weight || !p->in_project_slice_bias || !p->temperature) return PA_ERR_NULL;
+  if (!plus || !plus->proj_temperature_0_weight || !plus->proj_temperature_0_bias || !plus->proj_temperature_2_weight ||
+      !plus->proj_temperature_2_bias)
+    return PA_ERR_NULL;
+  if (!x_mid || !uniform || !w || !d_out_x || !out_slice_token || !d_num || !d_norm || !d_x_mid || !d_z || !d_a1 ||
+      !d_a2 || !d_temperature_partials)
+    return PA_ERR_NULL;
+  if (!aligned16(x_mid) || !aligned16(uniform) || !aligned16(w) || !aligned16(d_out_x) || !aligned16(d_x_mid) ||
+      !aligned16(d_z) || !aligned16(d_a1))
+    return PA_ERR_ALIGN;
+  return pa::backward::slice_softmax_plus(dtype, *shape, *p, *plus, x_mid, uniform, w, d_out_x, out_slice_token, d_num,
+                                          d_norm, d_x_mid, d_z, d_a1, d_a2, d_temperature_partials,
+                                          static_cast<hipStream_t>(stream));
+}
+
 int pa_residual_layernorm(int dtype, int64_t rows, int64_t C, void *y, const pa_block_tail *tail, void *stream) {
   if (dtype != PA_F32 && dtype != PA_BF16) return PA_ERR_UNSUPPORTED;
   if (rows <= 0 || C <= 0 || C > (1 << 16)) return PA_ERR_DIMS;

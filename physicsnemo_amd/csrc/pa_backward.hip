@@ -172,14 +172,28 @@ __global__ __launch_bounds__(kAttnBwdThreads) void slice_attention_backward_kern
 // D+1) and three R x (S+1) arrays (w, d w -> d z, logits).  R is a power of two <= 32, 256 / R threads share a row
 // in the row reductions.
 // Outputs: d_proj (B, N, 2*H*D) = [d x_mid | d fx_mid], d_z (B, N, H, S), dT_part[tile, h] (summed by the caller).
+//
+// PLUS (Transolver++, PA.py:166-170, :530-532): one projection (fx_mid is x_mid; d_proj is (B, N, H*D) and holds the
+// sum of both gradients), the softmax argument is (logits + Gumbel noise) / temp with the per-point
+//   temp = max(temperature[h] + gelu(a2), 0.01),  a2 = b2 + sum_s w2[s] gelu(a1[s]),  a1 = b1 + W1 x_mid[n,h,:]
+// so  d temp = -sum_s d l[s] (logits + noise)[s] / temp^2, which flows (where temp was not clamped) into temperature[h]
+// (dT_part, no mask left for the caller) and through the small MLP:  d a2 = d temp gelu'(a2)  (d_a2 (B, N, H) float32),
+// d a1[s] = d a2 w2[s] gelu'(a1[s])  (d_a1 (B, N, H, S)),  d x_mid += d a1 . W1.
 // ------------------------------------------------------------------------------------------------
-template <typename T>
+struct PlusArgs {
+  const void *uniform;   // (B, N, H, S) activation type
+  const float *w1, *b1, *w2, *b2;
+  void *d_a1;            // (B, N, H, S) activation type
+  float *d_a2;           // (B, N, H)
+};
+
+template <typename T, bool PLUS>
 __global__ __launch_bounds__(256) void slice_softmax_backward_kernel(
     const T *__restrict__ x_mid, const T *__restrict__ fx_mid, const T *__restrict__ w, const T *__restrict__ d_out_x,
     const float *__restrict__ out_token, const float *__restrict__ d_num, const float *__restrict__ d_norm,
     const float *__restrict__ w_slice, const float *__restrict__ b_slice, const float *__restrict__ temperature,
     T *__restrict__ d_proj, T *__restrict__ d_z, float *__restrict__ dT_part, int64_t N, int H, int D, int S, int R,
-    int tiles_per_batch) {
+    int tiles_per_batch, PlusArgs plus) {
   extern __shared__ float lds[];
   const int D1 = D + 1, S1 = S + 1;
   float *to = lds;               // S * D1
@@ -193,6 +207,10 @@ __global__ __launch_bounds__(256) void slice_softmax_backward_kernel(
   float *wl = go + R * D1;       // R * S1
   float *dwl = wl + R * S1;      // R * S1
   float *lgl = dwl + R * S1;     // R * S1
+  float *w1 = lgl + R * S1;      // PLUS only: S * D1
+  float *b1 = w1 + S * D1;       // S
+  float *w2 = b1 + S;            // S
+  float *a1l = w2 + S;           // R * S1
   __shared__ float red[4];
   const int t = threadIdx.x;
   const int h = blockIdx.y;
@@ -201,8 +219,8 @@ __global__ __launch_bounds__(256) void slice_softmax_backward_kernel(
   const int rows = (int)min((int64_t)R, N - n0);
   const int64_t m0 = (int64_t)b * N + n0;
   const int HD = H * D, HS = H * S;
-  const float temp = clamp_temperature(temperature[h]);
-  const float inv_temp = 1.f / temp;
+  const float temp_h = PLUS ? temperature[h] : clamp_temperature(temperature[h]);
+  const float inv_temp_h = 1.f / temp_h;
 
   const int64_t bh = (int64_t)b * H + h;
   for (int i = t; i < S * D; i += 256) {
@@ -210,10 +228,15 @@ __global__ __launch_bounds__(256) void slice_softmax_backward_kernel(
     to[s * D1 + d] = out_token[bh * S * D + i];
     dn[s * D1 + d] = d_num[bh * S * D + i];
     ws[s * D1 + d] = w_slice[i];
+    if constexpr (PLUS) w1[s * D1 + d] = plus.w1[i];
   }
   for (int i = t; i < S; i += 256) {
     dnr[i] = d_norm[bh * S + i];
     bs[i] = b_slice[i];
+    if constexpr (PLUS) {
+      b1[i] = plus.b1[i];
+      w2[i] = plus.w2[i];
+    }
   }
   for (int i = t; i < R * D; i += 256) {
     const int r = i / D, d = i - r * D;
@@ -240,31 +263,74 @@ __global__ __launch_bounds__(256) void slice_softmax_backward_kernel(
       dw = fmaf(gr[d], tr[d], dw);
       dw = fmaf(fr[d], nr[d], dw);
     }
-    lgl[r * S1 + s] = round_to(x_mid, z + bs[s]) * inv_temp;  // the forward divides the stored Linear output
     dwl[r * S1 + s] = dw + dnr[s];
+    if constexpr (PLUS) {
+      const float *vr = w1 + s * D1;
+      float a = b1[s];
+      for (int d = 0; d < D; ++d) a = fmaf(xr[d], vr[d], a);
+      a1l[r * S1 + s] = a;
+      const float u = r < rows ? load_as_f32(static_cast<const T *>(plus.uniform) + (m0 + r) * HS + h * S + s) : 0.5f;
+      lgl[r * S1 + s] = round_to(x_mid, z + bs[s]) - logf(-logf(u + 1e-8f) + 1e-8f);  // divided by temp below
+    } else {
+      lgl[r * S1 + s] = round_to(x_mid, z + bs[s]) * inv_temp_h;  // the forward divides the stored Linear output
+    }
   }
   __syncthreads();
 
   // softmax backward per row; 256 / R threads per row
   const int tpr = 256 / R;
   const int r_own = t / tpr, j_own = t - r_own * tpr;
+  float inv_temp = inv_temp_h, traw = 0.f, a2 = 0.f;
+  if constexpr (PLUS) {
+    a2 = 0.f;
+    for (int s = j_own; s < S; s += tpr) a2 = fmaf(w2[s], gelu_erf(a1l[r_own * S1 + s]), a2);
+    for (int off = tpr >> 1; off > 0; off >>= 1) a2 += __shfl_xor(a2, off, 64);
+    a2 += plus.b2[0];
+    traw = temp_h + gelu_erf(a2);
+    inv_temp = 1.f / round_to(x_mid, fmaxf(traw, 0.01f));
+  }
+  // The softmax is formed again in float32 for its own backward: its rows then sum to one, which the identity
+  // sum_s d l[s] = 0 behind d temperature needs (with weights rounded to bf16 the defect, times the common offset of
+  // the logits, would swamp it).  The stored weights still serve the aggregation and deslice terms.
+  const float yscale = PLUS ? inv_temp : 1.f;  // lgl holds the softmax argument itself when not PLUS
+  float mx = -INFINITY;
+  for (int s = j_own; s < S; s += tpr) mx = fmaxf(mx, lgl[r_own * S1 + s] * yscale);
+  for (int off = tpr >> 1; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+  float sum = 0.f;
+  for (int s = j_own; s < S; s += tpr) sum += expf(lgl[r_own * S1 + s] * yscale - mx);
+  for (int off = tpr >> 1; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+  const float inv_sum = 1.f / sum;
+  auto weight = [&](int s) { return r_own < rows ? expf(lgl[r_own * S1 + s] * yscale - mx) * inv_sum : 0.f; };
   float dot = 0.f;
-  for (int s = j_own; s < S; s += tpr) dot = fmaf(wl[r_own * S1 + s], dwl[r_own * S1 + s], dot);
+  for (int s = j_own; s < S; s += tpr) dot = fmaf(weight(s), dwl[r_own * S1 + s], dot);
   for (int off = tpr >> 1; off > 0; off >>= 1) dot += __shfl_xor(dot, off, 64);
   float tsum = 0.f;
   for (int s = j_own; s < S; s += tpr) {
-    const float dl = wl[r_own * S1 + s] * (dwl[r_own * S1 + s] - dot);
+    const float dl = weight(s) * (dwl[r_own * S1 + s] - dot);
     tsum = fmaf(dl, lgl[r_own * S1 + s], tsum);
     dwl[r_own * S1 + s] = dl * inv_temp;
+  }
+  if constexpr (PLUS) {
+    for (int off = tpr >> 1; off > 0; off >>= 1) tsum += __shfl_xor(tsum, off, 64);
+    const float d_temp = traw >= 0.01f ? -tsum * inv_temp * inv_temp : 0.f;  // clamp(min): gradient where not clamped
+    const float d_a2 = d_temp * gelu_erf_grad(a2);
+    for (int s = j_own; s < S; s += tpr) a1l[r_own * S1 + s] = d_a2 * w2[s] * gelu_erf_grad(a1l[r_own * S1 + s]);
+    if (j_own == 0 && r_own < rows) plus.d_a2[(m0 + r_own) * H + h] = d_a2;
+    tsum = j_own == 0 ? d_temp : 0.f;  // summed over the tile's rows below
   }
   tsum = wave_sum(tsum);
   if ((t & 63) == 0) red[t >> 6] = tsum;
   __syncthreads();
-  if (t == 0) dT_part[(int64_t)blockIdx.x * H + h] = -(((red[0] + red[1]) + red[2]) + red[3]) * inv_temp;
+  if (t == 0) {
+    const float total = ((red[0] + red[1]) + red[2]) + red[3];
+    dT_part[(int64_t)blockIdx.x * H + h] = PLUS ? total : -total * inv_temp_h;
+  }
 
   for (int i = t; i < rows * S; i += 256) {
     const int r = i / S, s = i - r * S;
     store_from_f32(d_z + (m0 + r) * HS + h * S + s, dwl[r * S1 + s]);
+    if constexpr (PLUS)
+      store_from_f32(static_cast<T *>(plus.d_a1) + (m0 + r) * HS + h * S + s, a1l[r * S1 + s]);
   }
   for (int i = t; i < rows * D; i += 256) {
     const int r = i / D, d = i - r * D;
@@ -274,8 +340,14 @@ __global__ __launch_bounds__(256) void slice_softmax_backward_kernel(
       dx = fmaf(zr[s], ws[s * D1 + d], dx);
       df = fmaf(wr[s], dn[s * D1 + d], df);
     }
-    store_from_f32(d_proj + (m0 + r) * 2 * HD + h * D + d, dx);
-    store_from_f32(d_proj + (m0 + r) * 2 * HD + HD + h * D + d, df);
+    if constexpr (PLUS) {
+      const float *ar = a1l + r * S1;
+      for (int s = 0; s < S; ++s) dx = fmaf(ar[s], w1[s * D1 + d], dx);
+      store_from_f32(d_proj + (m0 + r) * HD + h * D + d, dx + df);
+    } else {
+      store_from_f32(d_proj + (m0 + r) * 2 * HD + h * D + d, dx);
+      store_from_f32(d_proj + (m0 + r) * 2 * HD + HD + h * D + d, df);
+    }
   }
 }
 
@@ -299,46 +371,62 @@ int slice_attention(const pa_shape &s, const pa_params &p, const float *slice_to
 }
 
 // Rows per tile of slice_softmax_backward_kernel: the largest power of two <= 32 whose LDS footprint fits; 0 = none.
-int point_tile_rows(const pa_shape &s) {
-  const size_t fixed = (size_t)(3 * s.S * (s.D + 1) + 2 * s.S) * 4;
-  for (int R = 32; R >= 4; R >>= 1) {
-    const size_t per = (size_t)R * (3 * (s.D + 1) + 3 * (s.S + 1)) * 4;
-    if (fixed + per <= 120 * 1024) return R;
-  }
+static size_t point_tile_lds(const pa_shape &s, int R, bool plus) {
+  size_t words = (size_t)(3 * s.S * (s.D + 1) + 2 * s.S) + (size_t)R * (3 * (s.D + 1) + 3 * (s.S + 1));
+  if (plus) words += (size_t)(s.S * (s.D + 1) + 2 * s.S) + (size_t)R * (s.S + 1);
+  return words * 4;
+}
+
+int point_tile_rows(const pa_shape &s, bool plus) {
+  for (int R = 32; R >= 4; R >>= 1)
+    if (point_tile_lds(s, R, plus) <= 120 * 1024) return R;
   return 0;
 }
 
-int64_t point_tiles(const pa_shape &s) {
-  const int R = point_tile_rows(s);
+int64_t point_tiles(const pa_shape &s, bool plus) {
+  const int R = point_tile_rows(s, plus);
   return R == 0 ? 0 : s.B * ((s.N + R - 1) / R);
 }
 
-template <typename T>
+template <typename T, bool PLUS>
 static int slice_softmax_t(const pa_shape &s, const pa_params &p, const void *x_mid, const void *fx_mid, const void *w,
                            const void *d_out_x, const float *out_token, const float *d_num, const float *d_norm,
-                           void *d_proj, void *d_z, float *dT_part, hipStream_t st) {
-  const int R = point_tile_rows(s);
+                           void *d_proj, void *d_z, float *dT_part, const PlusArgs &plus, hipStream_t st) {
+  const int R = point_tile_rows(s, PLUS);
   if (R == 0) return PA_ERR_UNSUPPORTED;
-  const size_t lds =
-      (size_t)(3 * s.S * (s.D + 1) + 2 * s.S + (size_t)R * (3 * (s.D + 1) + 3 * (s.S + 1))) * 4;
-  int rc = allow_dynamic_lds(slice_softmax_backward_kernel<T>, lds);
+  const size_t lds = point_tile_lds(s, R, PLUS);
+  int rc = allow_dynamic_lds(slice_softmax_backward_kernel<T, PLUS>, lds);
   if (rc) return rc;
   const int tiles = (int)((s.N + R - 1) / R);
   dim3 grid((unsigned)(tiles * s.B), (unsigned)s.H);
-  hipLaunchKernelGGL((slice_softmax_backward_kernel<T>), grid, dim3(256), lds, st, static_cast<const T *>(x_mid),
+  hipLaunchKernelGGL((slice_softmax_backward_kernel<T, PLUS>), grid, dim3(256), lds, st, static_cast<const T *>(x_mid),
                      static_cast<const T *>(fx_mid), static_cast<const T *>(w), static_cast<const T *>(d_out_x),
                      out_token, d_num, d_norm, p.in_project_slice_weight, p.in_project_slice_bias, p.temperature,
                      static_cast<T *>(d_proj), static_cast<T *>(d_z), dT_part, s.N, (int)s.H, (int)s.D, (int)s.S, R,
-                     tiles);
+                     tiles, plus);
   return launch_status();
 }
 
 int slice_softmax(int dtype, const pa_shape &s, const pa_params &p, const void *x_mid, const void *fx_mid,
                   const void *w, const void *d_out_x, const float *out_token, const float *d_num, const float *d_norm,
                   void *d_proj, void *d_z, float *dT_part, hipStream_t st) {
-  return dtype == PA_F32
-             ? slice_softmax_t<float>(s, p, x_mid, fx_mid, w, d_out_x, out_token, d_num, d_norm, d_proj, d_z, dT_part, st)
-             : slice_softmax_t<bf16>(s, p, x_mid, fx_mid, w, d_out_x, out_token, d_num, d_norm, d_proj, d_z, dT_part, st);
+  const PlusArgs none{};
+  return dtype == PA_F32 ? slice_softmax_t<float, false>(s, p, x_mid, fx_mid, w, d_out_x, out_token, d_num, d_norm,
+                                                         d_proj, d_z, dT_part, none, st)
+                         : slice_softmax_t<bf16, false>(s, p, x_mid, fx_mid, w, d_out_x, out_token, d_num, d_norm,
+                                                        d_proj, d_z, dT_part, none, st);
+}
+
+int slice_softmax_plus(int dtype, const pa_shape &s, const pa_params &p, const pa_plus_params &pp, const void *x_mid,
+                       const void *uniform, const void *w, const void *d_out_x, const float *out_token,
+                       const float *d_num, const float *d_norm, void *d_x_mid, void *d_z, void *d_a1, float *d_a2,
+                       float *dT_part, hipStream_t st) {
+  const PlusArgs plus{uniform, pp.proj_temperature_0_weight, pp.proj_temperature_0_bias, pp.proj_temperature_2_weight,
+                      pp.proj_temperature_2_bias, d_a1, d_a2};
+  return dtype == PA_F32 ? slice_softmax_t<float, true>(s, p, x_mid, x_mid, w, d_out_x, out_token, d_num, d_norm,
+                                                        d_x_mid, d_z, dT_part, plus, st)
+                         : slice_softmax_t<bf16, true>(s, p, x_mid, x_mid, w, d_out_x, out_token, d_num, d_norm,
+                                                       d_x_mid, d_z, dT_part, plus, st);
 }
 
 }  // namespace backward

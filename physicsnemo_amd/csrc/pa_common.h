@@ -39,6 +39,11 @@ __device__ __forceinline__ float round_to(const bf16 *, float v) { return bf16_b
 // GELU in its erf form (torch.nn.GELU default, activations.py:198)
 __device__ __forceinline__ float gelu_erf(float v) { return 0.5f * v * (1.f + erff(v * 0.70710678118654752f)); }
 
+// its derivative: Phi(v) + v phi(v)
+__device__ __forceinline__ float gelu_erf_grad(float v) {
+  return 0.5f * (1.f + erff(v * 0.70710678118654752f)) + v * 0.3989422804014327f * expf(-0.5f * v * v);
+}
+
 __device__ __forceinline__ float clamp_temperature(float t) { return fminf(fmaxf(t, kTempMin), kTempMax); }
 
 // wave64 butterfly reductions

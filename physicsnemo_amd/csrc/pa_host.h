@@ -93,11 +93,15 @@ size_t attention_lds_bytes(const pa_shape &s);
 int slice_attention(const pa_shape &s, const pa_params &p, const float *slice_token, const float *slice_norm,
                     const float *d_out_token, float *scratch, float *d_num, float *d_norm, float *d_wqkv_part,
                     hipStream_t st);
-int point_tile_rows(const pa_shape &s);
-int64_t point_tiles(const pa_shape &s);
+int point_tile_rows(const pa_shape &s, bool plus = false);  // plus: the Transolver++ form of the per-point kernel
+int64_t point_tiles(const pa_shape &s, bool plus = false);
 int slice_softmax(int dtype, const pa_shape &s, const pa_params &p, const void *x_mid, const void *fx_mid,
                   const void *w, const void *d_out_x, const float *out_token, const float *d_num, const float *d_norm,
                   void *d_proj, void *d_z, float *dT_part, hipStream_t st);
+int slice_softmax_plus(int dtype, const pa_shape &s, const pa_params &p, const pa_plus_params &pp, const void *x_mid,
+                       const void *uniform, const void *w, const void *d_out_x, const float *out_token,
+                       const float *d_num, const float *d_norm, void *d_x_mid, void *d_z, void *d_a1, float *d_a2,
+                       float *dT_part, hipStream_t st);
 }  // namespace backward
 
 namespace mfma {

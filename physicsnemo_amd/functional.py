@@ -484,3 +484,31 @@ def slice_softmax_backward(x_mid, fx_mid, w, d_out_x, tok_out, d_num, d_norm, pa
                                              d_proj.data_ptr(), d_z.data_ptr(), dT.data_ptr(),
                                              _lib.current_stream_ptr(w.device)), "pa_slice_softmax_backward")
     return d_proj, d_z, dT.sum(0)
+
+
+def plus_backward_supported(dtype: torch.dtype, dims: LayerDims) -> bool:
+    return backward_supported(dtype, dims) and _lib.load().pa_backward_point_tiles_plus(byref(dims.c())) > 0
+
+
+def slice_softmax_plus_backward(x_mid, uniform, w, d_out_x, tok_out, d_num, d_norm, params, dims: LayerDims):
+    """Transolver++ form of `slice_softmax_backward`.  Returns (d x_mid (B,N,HD), d_z (B,N,H,S), d_a1 (B,N,H,S),
+    d_a2 (B,N,H) float32, d temperature (H) float32); d_a1 / d_a2 are the gradients of the two proj_temperature Linear
+    outputs."""
+    _need_cuda(x_mid, uniform, w, d_out_x, tok_out, d_num, d_norm)
+    lib = _lib.load()
+    shape = dims.c()
+    tiles = lib.pa_backward_point_tiles_plus(byref(shape))
+    if tiles < 0:
+        _lib.check(int(tiles), "pa_backward_point_tiles_plus")
+    d_x_mid = torch.empty(dims.B, dims.N, dims.H * dims.D, dtype=w.dtype, device=w.device)
+    d_z = torch.empty(dims.B, dims.N, dims.H, dims.S, dtype=w.dtype, device=w.device)
+    d_a1 = torch.empty_like(d_z)
+    d_a2 = torch.empty(dims.B, dims.N, dims.H, dtype=torch.float32, device=w.device)
+    dT = torch.empty(int(tiles), dims.H, dtype=torch.float32, device=w.device)
+    plus = _lib.PaPlusParams(*[_lib.ptr(params[k]) for k, _ in _lib.PaPlusParams._fields_])
+    _lib.check(lib.pa_slice_softmax_plus_backward(
+        _lib.dtype_code(w.dtype), byref(shape), byref(_c_params(params)), byref(plus), x_mid.data_ptr(),
+        uniform.data_ptr(), w.data_ptr(), d_out_x.data_ptr(), tok_out.data_ptr(), d_num.data_ptr(), d_norm.data_ptr(),
+        d_x_mid.data_ptr(), d_z.data_ptr(), d_a1.data_ptr(), d_a2.data_ptr(), dT.data_ptr(),
+        _lib.current_stream_ptr(w.device)), "pa_slice_softmax_plus_backward")
+    return d_x_mid, d_z, d_a1, d_a2, dT.sum(0)

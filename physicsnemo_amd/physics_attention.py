@@ -8,8 +8,8 @@ reference classes in physicsnemo/nn/module/physics_attention.py:
   PhysicsAttentionStructuredMesh3D:786-907
 so that a reference ``state_dict`` loads unchanged and seeded construction consumes the RNG identically.
 
-``plus=True`` (Transolver++) runs through the stage-level kernels, forward only.  ``use_te`` is accepted for signature compatibility and ignored: the HIP kernels are the
-only backend and there is no CPU path.  Under ``torch.no_grad()`` the fused inference kernels run; with gradients
+``plus=True`` (Transolver++) runs through the stage-level kernels, forward and backward.  ``use_te`` is accepted for
+signature compatibility and ignored: the HIP kernels are the only backend and there is no CPU path.  Under ``torch.no_grad()`` the fused inference kernels run; with gradients
 enabled on tensors that require them the stage-level kernels run and the backward pass is served by the library's
 backward kernels (see ``autograd.py``).
 """
@@ -19,7 +19,7 @@ import torch
 import torch.nn as nn
 
 from . import functional as PF
-from .autograd import PhysicsAttentionFunction, PhysicsAttentionMfmaFunction
+from .autograd import PhysicsAttentionFunction, PhysicsAttentionMfmaFunction, PhysicsAttentionPlusFunction
 
 __all__ = ["PhysicsAttentionBase", "PhysicsAttentionIrregularMesh", "PhysicsAttentionStructuredMesh2D",
            "PhysicsAttentionStructuredMesh3D"]
@@ -149,7 +149,7 @@ class PhysicsAttentionBase(nn.Module):
         if self.fp8_weights:
             raise RuntimeError("fp8 weights are an inference format: no gradients flow through them")
         if self.plus:
-            raise NotImplementedError("the backward kernels do not cover Transolver++ (plus=True)")
+            return self._forward_plus_with_grad(x, None)
         dims = self.layer_dims(x)
         if not PF.backward_supported(x.dtype, dims):
             raise RuntimeError(f"the backward kernels do not serve this shape: {dims}")
@@ -159,6 +159,20 @@ class PhysicsAttentionBase(nn.Module):
             self.in_project_fx.weight, self.in_project_fx.bias, self.in_project_slice.weight,
             self.in_project_slice.bias, self.temperature, self.qkv_project.weight, self.out_linear.weight,
             self.out_linear.bias)
+
+    def _forward_plus_with_grad(self, x: torch.Tensor, noise_u: torch.Tensor | None) -> torch.Tensor:
+        """Training path of Transolver++: `autograd.PhysicsAttentionPlusFunction` on the general kernels."""
+        dims = self.layer_dims(x)
+        if not PF.plus_backward_supported(x.dtype, dims):
+            raise RuntimeError(f"the backward kernels do not serve this shape: {dims}")
+        if noise_u is None:
+            noise_u = torch.rand((dims.B, dims.N, dims.H, dims.S), dtype=x.dtype, device=x.device)
+        pt = self.proj_temperature
+        return PhysicsAttentionPlusFunction.apply(
+            x, noise_u.detach().to(x.dtype).contiguous(), dims, self.kernel_params(x.dtype, x.device),
+            self.in_project_x.weight, self.in_project_x.bias, self.in_project_slice.weight, self.in_project_slice.bias,
+            self.temperature, pt[0].weight, pt[0].bias, pt[2].weight, pt[2].bias, self.qkv_project.weight,
+            self.out_linear.weight, self.out_linear.bias)
 
     @staticmethod
     def _wants_fp16(x: torch.Tensor) -> bool:
@@ -190,8 +204,8 @@ class PhysicsAttentionBase(nn.Module):
         if not self.plus:
             raise RuntimeError("forward_with_noise is the plus=True path")
         self._validate(x)
-        if self._needs_grad(x):
-            raise NotImplementedError("the backward kernels do not cover Transolver++ (plus=True)")
+        if self._needs_grad(x) and not stages:
+            return self._forward_plus_with_grad(self._prepare_input(x), noise_u)
         x = self._prepare_input(x)
         dims = self.layer_dims(x)
         p = self.kernel_params(x.dtype, x.device)

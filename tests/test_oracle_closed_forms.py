@@ -157,6 +157,35 @@ def test_oracle_gradient_matches_finite_differences(variant):
     assert torch.autograd.gradcheck(fn, (x, *params), eps=1e-6, atol=1e-6, rtol=1e-5)
 
 
+def test_oracle_plus_gradient_matches_finite_differences():
+    """Gradient of the Transolver++ branch of the oracle (given the uniform samples), pinned the same way; the
+    per-point temperatures are kept away from the clamp at 0.01, where the function has a kink."""
+    torch.manual_seed(12)
+    m = to.OraclePhysicsAttentionIrregularMesh(6, heads=2, dim_head=3, slice_num=4, plus=True).double()
+    with torch.no_grad():
+        m.temperature.copy_(torch.tensor([0.8, 1.5], dtype=torch.float64).view(1, 1, 2, 1))
+    u = torch.rand(2, 7, 2, 4, dtype=torch.float64)
+
+    class GivenNoise(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.m = m
+
+        def forward(self, x):
+            return self.m.forward_with_noise(x, u)
+
+    wrapped = GivenNoise()
+    names = [k for k, _ in wrapped.named_parameters()]
+    params = [p.detach().clone().requires_grad_(True) for _, p in wrapped.named_parameters()]
+    x = torch.randn(2, 7, 6, dtype=torch.float64, requires_grad=True)
+
+    def fn(x, *ps):
+        return torch.func.functional_call(wrapped, dict(zip(names, ps)), (x,))
+
+    assert "m.proj_temperature.2.weight" in names
+    assert torch.autograd.gradcheck(fn, (x, *params), eps=1e-6, atol=1e-6, rtol=1e-5)
+
+
 def test_plus_branch_numpy_vs_torch_and_special_cases():
     torch.manual_seed(21)
     B, N, C, H, D, S = 2, 9, 6, 2, 4, 5
