@@ -129,7 +129,7 @@ __global__ __launch_bounds__(256) void backward_tables_kernel(const float *__res
 // through LDS.  Per 32-point tile and head:
 //   z^T  (S x pts) = W_slice . x_mid^T + b_slice                       B = x_mid rows, 16-byte natural loads
 //   dw^T (S x pts) = tok' . g^T + d num . fx_mid^T + d nrm             B = g / fx_mid rows
-//   w: unpacked from w_pack; dot = sum_s w dw; dz = (w / T) (dw - dot); dT -= sum dz z / T
+//   w: unpacked from w_pack; dot = sum_s w dw / sum_s w; dz = (w / T) (dw - dot); dT -= sum dz z / T
 //   d x_mid^T (32 x pts) = W_slice^T . dz^T (B = bf16(dz^T) straight from registers); d fx_mid^T = d num^T . w (B = w_pack)
 // Rows beyond N have w = 0 in w_pack (the forward writes zeros), so they contribute nothing; their loads are clamped to
 // the last valid row and their stores are masked.
@@ -207,7 +207,7 @@ __global__ __launch_bounds__(S > 64 ? 256 : 512) void slice_softmax_backward_mfm
     // per point: dot = sum_s w dw;  sum_s dz z = (sum_s w dw z - dot sum_s w z) / T: the logits of a slice tile are
     // consumed as soon as they exist, only d w stays live across the tiles
     f32x16 dw[ST];
-    float dot = 0.f, a1 = 0.f, a2 = 0.f;
+    float dot = 0.f, a1 = 0.f, a2 = 0.f, wsum = 0.f;
 #pragma unroll
     for (int st = 0; st < ST; ++st) {
       f32x16 z;
@@ -232,12 +232,16 @@ __global__ __launch_bounds__(S > 64 ? 256 : 512) void slice_softmax_backward_mfm
         const float w = w_of(st, r);
         const float wd = w * dw[st][r];
         dot += wd;
+        wsum += w;
         a1 = fmaf(wd, z[r], a1);
         a2 = fmaf(w, z[r], a2);
       }
       __builtin_amdgcn_sched_barrier(0);
     }
-    dot = half_sum(dot);
+    // the bf16 weights of a point do not sum to one exactly: dividing by their sum keeps sum_s d z = 0, without which
+    // the defect times the common offset of the logits leaks into d temperature and d bias
+    wsum = half_sum(wsum);
+    dot = wsum > 0.f ? half_sum(dot) / wsum : 0.f;
     tsum += (a1 - dot * a2) * inv_t;  // a1, a2 are this lane's halves; the halves add up in the final wave sum
     f32x16(&dz)[ST] = dw;  // d z replaces d w in place
 #pragma unroll

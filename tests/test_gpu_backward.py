@@ -167,12 +167,11 @@ def test_bf16_mfma_backward_matches_oracle_and_general_path(B, N, C, S):
     general = run(PA.PhysicsAttentionFunction)
     for name in want:
         assert torch.isfinite(got[name]).all(), name
-        # d temperature is H scalars, each a sum of cancelling terms d l * logit over all points and slices formed
-        # from bf16 activations: its relative error is several times that of the tensor-valued gradients
-        tol = 1e-1 if name == "temperature" else 3e-2
-        assert_rel_l2(got[name], want[name], f"MFMA bf16 grad {name} vs fp32 oracle", tol=tol)
-        if name != "temperature":  # the general path rounds the logits to bf16 first: its d temperature is noisier still
-            assert_rel_l2(got[name], general[name], f"MFMA vs general bf16 grad {name}", tol=tol)
+        # d temperature is H scalars, each a sum of cancelling terms d l * logit over all points and slices; both
+        # kernels keep sum_s d l = 0 per point (weights renormalised / softmax re-formed in float32), which holds it
+        # to the bar of the tensor-valued gradients
+        assert_rel_l2(got[name], want[name], f"MFMA bf16 grad {name} vs fp32 oracle", tol=3e-2)
+        assert_rel_l2(got[name], general[name], f"MFMA vs general bf16 grad {name}", tol=3e-2)
     t = got["temperature"].flatten().cpu()
     assert t[0] == 0.0  # 0.3 is below the clamp: no gradient
 
