@@ -225,6 +225,33 @@ int pa_slice_softmax_plus_backward(int dtype, const pa_shape *shape, const pa_pa
                                    void *d_x_mid, void *d_z, void *d_a1, float *d_a2, float *d_temperature_partials,
                                    void *stream);
 
+/* ---- GALE: cross-attention of the slice tokens to a context (physicsnemo/nn/module/gale.py) ------
+ * A GALE layer (gale.py:242-478) is a PhysicsAttention layer whose slice-token stage also attends to a context
+ * (B,H,Sc,Dc) and blends the two results (gale.py:87-145 _gale_compute_slice_attention_cross, :43-84
+ * _mix_self_and_cross); every other stage is the entry points above.  All tensors float32. */
+typedef struct pa_gale_params {
+  const float *cross_q_weight; /* (D, D)  */
+  const float *cross_q_bias;   /* (D)     */
+  const float *cross_k_weight; /* (D, Dc) */
+  const float *cross_k_bias;   /* (D)     */
+  const float *cross_v_weight; /* (D, Dc) */
+  const float *cross_v_bias;   /* (D)     */
+  const float *state_mixing;   /* scalar; state_mixing_mode "weighted": out = sigmoid(m) self + (1 - sigmoid(m)) cross */
+  const float *concat_project_weight; /* (D, 2D) concat_project[0]; mode "concat_project":                          */
+  const float *concat_project_bias;   /* (D)      out = gelu([self | cross] W^T + b).  Exactly one mode is non-NULL. */
+} pa_gale_params;
+/* out_slice_token (B,H,S,D) = blend(self_out_slice_token, softmax(q k^T / sqrt(D)) v) with q from slice_token and
+ * k, v from context (B,H,context_slices,context_dim).  tokp: NULL, or the PA_BUF_TOKP buffer of the MFMA kernels,
+ * which then receives the result as operands of pa_mfma_deslice_project (shapes with pa_query_path() == 1 only). */
+int pa_slice_cross_attention_mix(const pa_shape *shape, const pa_gale_params *gale, int64_t context_slices,
+                                 int64_t context_dim, const float *slice_token, const float *self_out_slice_token,
+                                 const float *context, float *out_slice_token, void *tokp, void *stream);
+
+/* Attended slice tokens (B,H,S,32) float32 computed by the caller (e.g. a GALE token stage under autograd) -> the
+ * PA_BUF_TOKP operands of pa_mfma_deslice_project, which pa_mfma_combine_attention otherwise writes
+ * (shapes with pa_query_path() == 1). */
+int pa_mfma_pack_tokens(const pa_shape *shape, const float *out_slice_token, void *tokp, void *stream);
+
 /* ---- stage-level entry points of the bf16 MFMA kernels (shapes with pa_query_path() == 1) ------
  * Intermediates use an internal register-order ("packed") layout; buffers are opaque to the caller and
  * sized by pa_mfma_buffer_bytes(shape, which):

@@ -80,7 +80,7 @@ def conv3d_projection(x, weight, bias, grid_h, grid_w, grid_d):
     return out.reshape(b, n, o) + _f64(bias)
 
 
-def layer_forward(p, x, heads, dim_head, variant="irregular", spatial_shape=None, noise_u=None):
+def layer_forward(p, x, heads, dim_head, variant="irregular", spatial_shape=None, noise_u=None, context=None):
     """All intermediates of one layer in float64 (steps 1-9 below follow physics_attention.py:529-558).
 
     p: in_project_x.{weight,bias}, in_project_fx.{weight,bias}, in_project_slice.{weight,bias},
@@ -88,6 +88,8 @@ def layer_forward(p, x, heads, dim_head, variant="irregular", spatial_shape=None
     Transolver++ (plus=True) is selected by the absence of in_project_fx.weight: then fx_mid = x_mid (:530-532),
     p also holds proj_temperature.{0,2}.{weight,bias} and noise_u (B, N, H, S) holds the uniform samples behind
     the Gumbel noise (gumbel_softmax.py:50).
+    GALE (gale.py:148-239): with `context` (B, H, Sc, Dc) and cross_{q,k,v}.{weight,bias} plus either state_mixing or
+    concat_project.0.{weight,bias} in p, the attended slice tokens are blended with their cross-attention to the context.
     """
     plus = "in_project_fx.weight" not in p
     if plus:
@@ -146,11 +148,32 @@ def layer_forward(p, x, heads, dim_head, variant="irregular", spatial_shape=None
     a = np.exp(sc)
     a = a / a.sum(axis=-1, keepdims=True)
     tok_out = np.einsum("bhst,bhte->bhse", a, v)
+    if context is not None:
+        tok_out = gale_blend(p, tok, tok_out, context)
     # 8. deslice with the un-normalised w, merge heads (:492-495)
     o = np.einsum("bnhs,bhsd->bnhd", w, tok_out).reshape(B, N, H * D)
     # 9. output projection (:498)
     y = np.einsum("bnk,ok->bno", o, _f64(p["out_linear.weight"])) + _f64(p["out_linear.bias"])
     return dict(x_mid=xm, fx_mid=fm, logits=logits, w=w, norm=norm, tok=tok, tok_out=tok_out, y=y)
+
+
+def gale_blend(p, tok, self_out, context):
+    """GALE slice-token stage: cross-attention to the context (gale.py:112-144) and the blend (gale.py:76-84)."""
+    ctx = _f64(context)
+    D = tok.shape[-1]
+    q = np.einsum("bhsd,ed->bhse", tok, _f64(p["cross_q.weight"])) + _f64(p["cross_q.bias"])
+    k = np.einsum("bhuc,ec->bhue", ctx, _f64(p["cross_k.weight"])) + _f64(p["cross_k.bias"])
+    v = np.einsum("bhuc,ec->bhue", ctx, _f64(p["cross_v.weight"])) + _f64(p["cross_v.bias"])
+    sc = np.einsum("bhse,bhue->bhsu", q, k) / math.sqrt(D)
+    sc = sc - sc.max(axis=-1, keepdims=True)
+    a = np.exp(sc)
+    a = a / a.sum(axis=-1, keepdims=True)
+    cross = np.einsum("bhsu,bhue->bhse", a, v)
+    if "state_mixing" in p:
+        m = 1.0 / (1.0 + np.exp(-float(np.asarray(p["state_mixing"]).reshape(-1)[0])))
+        return m * self_out + (1.0 - m) * cross
+    cat = np.concatenate([self_out, cross], axis=-1)
+    return gelu_erf(np.einsum("bhsk,ek->bhse", cat, _f64(p["concat_project.0.weight"])) + _f64(p["concat_project.0.bias"]))
 
 
 def layer_norm(x, gamma, beta, eps=1e-5):

@@ -174,9 +174,10 @@ class _AttentionCore(nn.Module):
     def _project(self, x):  # pragma: no cover - abstract
         raise NotImplementedError
 
-    def stages(self, x, noise_u=None):
+    def stages(self, x, noise_u=None, context=None):
         """Forward returning every intermediate (used by the parity tests).  ``noise_u`` (plus=True only): the
-        uniform samples behind the Gumbel noise; drawn with ``torch.rand_like`` when not given, as the reference does."""
+        uniform samples behind the Gumbel noise; drawn with ``torch.rand_like`` when not given, as the reference does.
+        ``context``: GALE subclasses only."""
         x_mid, fx_mid = self._project(x)
         logits = slice_logits(x_mid, self.in_project_slice.weight, self.in_project_slice.bias)
         if self.plus:
@@ -184,10 +185,14 @@ class _AttentionCore(nn.Module):
             w, tok, norm, _ = slice_weights_and_tokens_plus(logits, x_mid, self.temperature, self.proj_temperature, u)
         else:
             w, tok, norm = slice_weights_and_tokens(logits, fx_mid, self.temperature)
-        tok_out = slice_attention(tok, self.qkv_project.weight, self.dim_head)
+        tok_out = self._token_stage(tok, context)
         y = deslice_and_project(w, tok_out, self.out_linear.weight, self.out_linear.bias)
         return dict(x_mid=x_mid, fx_mid=fx_mid, logits=logits, w=w, tok=tok, norm=norm,
                     tok_out=tok_out, y=self.out_dropout(y))
+
+    def _token_stage(self, tok, context):
+        """Slice tokens -> attended slice tokens; the GALE subclasses add the cross-attention to a context."""
+        return slice_attention(tok, self.qkv_project.weight, self.dim_head)
 
     def forward(self, x):
         # Validation and messages: physics_attention.py:516-526
@@ -256,6 +261,75 @@ class OraclePhysicsAttentionStructuredMesh3D(_AttentionCore):
         return project_conv3d(x, self.in_project_x.weight, self.in_project_x.bias,
                               self.in_project_fx.weight, self.in_project_fx.bias,
                               self.heads, self.dim_head, self.H, self.W, self.D)
+
+
+
+# --------------------------------------------------------------------------- GALE (physicsnemo/nn/module/gale.py)
+def gale_cross_attention(tok, context, cross_q, cross_k, cross_v):
+    """Cross-attention of slice tokens (B,H,S,D) to a context (B,H,Sc,Dc) (gale.py:87-145, use_te=False branch):
+    q from the tokens, k and v from the context, SDPA with its default 1/sqrt(D) scale and no mask."""
+    return F.scaled_dot_product_attention(cross_q(tok), cross_k(context), cross_v(context), is_causal=False)
+
+
+def gale_mix(self_out, cross_out, mode, state_mixing=None, concat_project=None):
+    """Blend of the two attention results (gale.py:43-84)."""
+    if mode == "weighted":
+        m = torch.sigmoid(state_mixing)
+        return m * self_out + (1 - m) * cross_out
+    if mode == "concat_project":
+        return concat_project(torch.cat([self_out, cross_out], dim=-1))
+    raise ValueError(f"Invalid state_mixing_mode: {mode!r}")
+
+
+class _GALECore:
+    """Cross-attention parameters (gale.py:401-429) and the GALE forward (gale.py:148-239) on top of a layer class."""
+
+    def _init_cross(self, dim_head, context_dim, state_mixing_mode):
+        self.cross_q = nn.Linear(dim_head, dim_head)
+        self.cross_k = nn.Linear(context_dim, dim_head)
+        self.cross_v = nn.Linear(context_dim, dim_head)
+        self.state_mixing_mode = state_mixing_mode
+        if state_mixing_mode == "weighted":
+            self.state_mixing = nn.Parameter(torch.tensor(0.0))
+        elif state_mixing_mode == "concat_project":
+            self.concat_project = nn.Sequential(nn.Linear(2 * dim_head, dim_head), nn.GELU())
+        else:
+            raise ValueError(f"Invalid state_mixing_mode: {state_mixing_mode!r}")
+
+    def _token_stage(self, tok, context):
+        self_out = slice_attention(tok, self.qkv_project.weight, self.dim_head)
+        if context is None:  # gale.py:226-228
+            return self_out
+        cross = gale_cross_attention(tok, context, self.cross_q, self.cross_k, self.cross_v)
+        return gale_mix(self_out, cross, self.state_mixing_mode, getattr(self, "state_mixing", None),
+                        getattr(self, "concat_project", None))
+
+    def forward(self, x, context=None):
+        if len(x) == 0:
+            raise ValueError("Expected non-empty tuple of input tensors")
+        for i, t in enumerate(x):
+            if t.ndim != 3:
+                raise ValueError(f"Expected 3D input tensor (B, N, C) at index {i}, "
+                                 f"got {t.ndim}D tensor with shape {tuple(t.shape)}")
+        return [self.stages(t, context=context)["y"] for t in x]
+
+
+class OracleGALE(_GALECore, OraclePhysicsAttentionIrregularMesh):
+    """gale.py:242-398 with use_te=False, concrete_dropout=False."""
+
+    def __init__(self, dim, heads=8, dim_head=64, dropout=0.0, slice_num=64, plus=False, context_dim=0,
+                 state_mixing_mode="weighted"):
+        super().__init__(dim, heads, dim_head, dropout, slice_num, plus)
+        self._init_cross(dim_head, context_dim, state_mixing_mode)
+
+
+class OracleGALEStructuredMesh2D(_GALECore, OraclePhysicsAttentionStructuredMesh2D):
+    """gale.py:447-478 with use_te=False."""
+
+    def __init__(self, dim, spatial_shape, heads=8, dim_head=64, dropout=0.0, slice_num=64, kernel=3, plus=False,
+                 context_dim=0, state_mixing_mode="weighted"):
+        super().__init__(dim, spatial_shape, heads, dim_head, dropout, slice_num, kernel, plus)
+        self._init_cross(dim_head, context_dim, state_mixing_mode)
 
 
 class OracleMlp(nn.Module):

@@ -23,7 +23,8 @@ EXPORTED = [
      "pa_mfma_combine_attention", "pa_mfma_deslice_project", "pa_mlp_query", "pa_mlp_workspace_bytes", "pa_mlp_forward",
     "pa_rows_gemm", "pa_slice_weighted_sum", "pa_backward_query", "pa_backward_point_tiles",
     "pa_slice_attention_backward", "pa_slice_softmax_backward", "pa_slice_softmax_plus",
-    "pa_backward_point_tiles_plus", "pa_slice_softmax_plus_backward",
+    "pa_backward_point_tiles_plus", "pa_slice_softmax_plus_backward", "pa_slice_cross_attention_mix",
+    "pa_mfma_pack_tokens",
     "pa_mfma_backward_query", "pa_rows_gemm_packed", "pa_mfma_slice_weighted_sum", "pa_mfma_deslice",
     "pa_mfma_backward_tables_bytes", "pa_mfma_backward_groups", "pa_mfma_slice_softmax_backward",
     "pa_cols_gemm_chunks", "pa_cols_gemm", "pa_residual_layernorm",
@@ -51,6 +52,12 @@ class PaMlpParams(Structure):
 class PaPlusParams(Structure):
     _fields_ = [(n, c_void_p) for n in ("proj_temperature_0_weight", "proj_temperature_0_bias",
                                         "proj_temperature_2_weight", "proj_temperature_2_bias")]
+
+
+class PaGaleParams(Structure):
+    _fields_ = [(n, c_void_p) for n in ("cross_q_weight", "cross_q_bias", "cross_k_weight", "cross_k_bias",
+                                        "cross_v_weight", "cross_v_bias", "state_mixing", "concat_project_weight",
+                                        "concat_project_bias")]
 
 
 class PaBlockTail(Structure):
@@ -135,6 +142,10 @@ def load() -> ctypes.CDLL:
     lib.pa_backward_point_tiles_plus.argtypes = [ps]
     lib.pa_slice_softmax_plus_backward.restype = c_int
     lib.pa_slice_softmax_plus_backward.argtypes = [c_int, ps, pp, POINTER(PaPlusParams)] + [c_void_p] * 13
+    lib.pa_slice_cross_attention_mix.restype = c_int
+    lib.pa_slice_cross_attention_mix.argtypes = [ps, POINTER(PaGaleParams), c_int64, c_int64] + [c_void_p] * 6
+    lib.pa_mfma_pack_tokens.restype = c_int
+    lib.pa_mfma_pack_tokens.argtypes = [ps] + [c_void_p] * 3
     lib.pa_mfma_backward_query.restype = c_int
     lib.pa_mfma_backward_query.argtypes = [ps]
     lib.pa_rows_gemm_packed.restype = c_int

@@ -76,9 +76,10 @@ def _slice_weight_grad(d_z: torch.Tensor, x_mid: torch.Tensor, H: int, S: int, D
     return _wgrad(d_z.reshape(-1, S), x_mid.reshape(-1, D))
 
 
-def _finish_backward(ctx, x, dy, out_x, d_wqkv, d_proj, d_z, d_temp, x_mid, temperature):
+def _finish_backward(ctx, x, dy, out_x, d_wqkv, d_proj, d_z, d_temp, x_mid, temperature, param_offset=3):
     """Everything after the layer-specific kernels: d x (input-gradient GEMM / transposed convolution) and the weight
-    and bias gradients, which are plain GEMMs / column sums over the point axis."""
+    and bias gradients, which are plain GEMMs / column sums over the point axis.  Returns (d x, None, None, the ten
+    parameter gradients); `param_offset`: position of the first parameter among the Function's inputs."""
     dims, kp = ctx.dims, ctx.kparams
     B, N, C, H, D, S = dims.B, dims.N, dims.C, dims.H, dims.D, dims.S
     HD = H * D
@@ -105,7 +106,7 @@ def _finish_backward(ctx, x, dy, out_x, d_wqkv, d_proj, d_z, d_temp, x_mid, temp
         d_b_in = _rows(d_proj).sum(0, dtype=torch.float32)
 
     grads = (d_w_in[:HD], d_b_in[:HD], d_w_in[HD:], d_b_in[HD:], d_ws, d_bs, d_temp, d_wqkv, d_wo, d_bo)
-    grads = tuple(gr.reshape(p.shape).to(p.dtype) if ctx.needs_input_grad[3 + i] else None
+    grads = tuple(gr.reshape(p.shape).to(p.dtype) if gr is not None and ctx.needs_input_grad[param_offset + i] else None
                   for i, (gr, p) in enumerate(zip(grads, ctx.param_like)))
     return (dx, None, None) + grads
 
@@ -239,6 +240,91 @@ class PhysicsAttentionPlusFunction(torch.autograd.Function):
         grads = tuple(gr.reshape(p.shape).to(p.dtype) if ctx.needs_input_grad[4 + i] else None
                       for i, (gr, p) in enumerate(zip(grads, ctx.param_like)))
         return (dx, None, None, None) + grads
+
+
+class GALEFunction(torch.autograd.Function):
+    """GALE layer with a context (gale.py:148-239), differentiable w.r.t. x, the context, the ten PhysicsAttention
+    parameters and the cross-attention / blend parameters.
+
+    The per-point stages are the layer's kernels, forward and backward, as in the two Functions above.  The slice-token
+    stage in between (self-attention, cross-attention to the context, blend: S x D work per (batch, head), independent
+    of the number of points) is evaluated by `token_stage(tok, context)` with PyTorch ops under autograd in the
+    forward; the backward asks that small graph for d tok, d context and the gradients of `stage_params`."""
+
+    @staticmethod
+    def forward(ctx, x, context, dims, kparams, token_stage, n_stage, *params):
+        layer_params, stage_params = params[:len(params) - n_stage], params[len(params) - n_stage:]
+        mfma = PF.mfma_backward_supported(x.dtype, dims)
+        if mfma:
+            st = PF.MfmaStages(kparams, dims, x.device)
+            st.pack_params()
+            if st.fused_groups > 0:
+                st.project_softmax_reduce(x)
+            else:
+                st.project_softmax(x)
+                st.slice_reduce()
+            st.combine_attention()  # for the normalised slice tokens; its self-attention result is replaced below
+            tok, norm = st.tok, st.norm
+        else:
+            x_mid, fx_mid = PF.project_inputs(x, kparams, dims)
+            w = PF.slice_softmax(x_mid, kparams, dims)
+            tok, norm = PF.slice_reduce(w, fx_mid, dims)
+        with torch.enable_grad():
+            tok_leaf = tok.detach().requires_grad_(True)
+            ctx_leaf = context.detach().requires_grad_(ctx.needs_input_grad[1])
+            out_graph = token_stage(tok_leaf, ctx_leaf)
+        out_tok = out_graph.detach().float().contiguous()
+        if mfma:
+            st.set_out_tokens(out_tok)
+            y = torch.empty_like(x)
+            st.deslice_project(y)
+            ctx.save_for_backward(x, layer_params[6])
+            ctx.stages = st
+        else:
+            y, out_x = PF.deslice_project(w, out_tok, kparams, dims, return_out_x=True)
+            ctx.save_for_backward(x, layer_params[6], x_mid, fx_mid, w, out_x)
+        ctx.mfma, ctx.dims, ctx.kparams = mfma, dims, kparams
+        ctx.tok, ctx.norm, ctx.out_tok = tok, norm, out_tok
+        ctx.graph = (out_graph, tok_leaf, ctx_leaf, stage_params)
+        ctx.param_like = layer_params
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        dims, kp = ctx.dims, ctx.kparams
+        C, HD, D = dims.C, dims.H * dims.D, dims.D
+        x, temperature = ctx.saved_tensors[:2]
+        dy = dy.to(x.dtype).contiguous()
+        linear = PF.LayerDims(dims.B, dims.N, C, dims.H, D, dims.S)
+        w_out_t = kp["out_linear_weight"].view(C, HD).t().contiguous()
+        if ctx.mfma:
+            st = ctx.stages
+            g, g_pack = st.rows_gemm_packed(dy, w_out_t, None)
+            x_mid, fx_mid = PF.project_inputs(x, kp, dims)
+            d_out_tok = st.slice_weighted_sum(g_pack)[..., :D].contiguous()
+        else:
+            x_mid, fx_mid, w, out_x = ctx.saved_tensors[2:]
+            g = PF.rows_gemm(dy, w_out_t, None, linear, C, HD)
+            d_out_tok = PF.slice_weighted_sum(w, g, dims)[..., :D].contiguous()
+        # slice-token stage: PyTorch's graph of the forward
+        out_graph, tok_leaf, ctx_leaf, stage_params = ctx.graph
+        wanted = [tok_leaf] + ([ctx_leaf] if ctx_leaf.requires_grad else []) + \
+                 [p for p in stage_params if p.requires_grad]
+        got = list(torch.autograd.grad(out_graph, wanted, d_out_tok.to(out_graph.dtype), allow_unused=True))
+        d_tok = got.pop(0).float()
+        d_context = got.pop(0) if ctx_leaf.requires_grad else None
+        d_stage = [got.pop(0) if p.requires_grad else None for p in stage_params]
+        # tok = num / nrm
+        d_num = (d_tok / ctx.norm[..., None]).contiguous()
+        d_norm = (-(d_tok * ctx.tok).sum(-1) / ctx.norm).contiguous()
+        if ctx.mfma:
+            out_x = st.deslice()
+            d_proj, d_z, d_temp = st.slice_softmax_backward(x_mid, fx_mid, g, d_num, d_norm)
+        else:
+            d_proj, d_z, d_temp = PF.slice_softmax_backward(x_mid, fx_mid, w, g, ctx.out_tok, d_num, d_norm, kp, dims)
+        # qkv_project.weight takes part in the token stage only: its gradient comes with `d_stage`
+        base = _finish_backward(ctx, x, dy, out_x, None, d_proj, d_z, d_temp, x_mid, temperature, param_offset=6)
+        return (base[0], d_context, None, None, None, None) + base[3:] + tuple(d_stage)
 
 
 class LinearFunction(torch.autograd.Function):

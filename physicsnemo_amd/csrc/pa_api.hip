@@ -438,6 +438,34 @@ int pa_slice_softmax_plus_backward(int dtype, const pa_shape *shape, const pa_pa
                                           static_cast<hipStream_t>(stream));
 }
 
+int pa_slice_cross_attention_mix(const pa_shape *shape, const pa_gale_params *gale, int64_t context_slices,
+                                 int64_t context_dim, const float *slice_token, const float *self_out_slice_token,
+                                 const float *context, float *out_slice_token, void *tokp, void *stream) {
+  int rc = check_shape(PA_F32, shape);
+  if (rc) return rc;
+  if (context_slices <= 0 || context_dim <= 0 || context_slices > (1 << 16) || context_dim > (1 << 16))
+    return PA_ERR_DIMS;
+  if (!gale || !gale->cross_q_weight || !gale->cross_q_bias || !gale->cross_k_weight || !gale->cross_k_bias ||
+      !gale->cross_v_weight || !gale->cross_v_bias)
+    return PA_ERR_NULL;
+  const bool weighted = gale->state_mixing != nullptr;
+  const bool concat = gale->concat_project_weight != nullptr && gale->concat_project_bias != nullptr;
+  if (weighted == concat) return PA_ERR_NULL;  // exactly one blend mode
+  if (!slice_token || !self_out_slice_token || !context || !out_slice_token) return PA_ERR_NULL;
+  if (tokp && !pa::mfma::supported(PA_BF16, *shape)) return PA_ERR_UNSUPPORTED;
+  if (pa::gale::lds_bytes(*shape, context_slices, context_dim) > pa::kMaxLdsBytes) return PA_ERR_UNSUPPORTED;
+  return pa::gale::slice_cross_mix(*shape, *gale, context_slices, context_dim, slice_token, self_out_slice_token,
+                                   context, out_slice_token, tokp, static_cast<hipStream_t>(stream));
+}
+
+int pa_mfma_pack_tokens(const pa_shape *shape, const float *out_slice_token, void *tokp, void *stream) {
+  int rc = check_shape(PA_BF16, shape);
+  if (rc) return rc;
+  if (!pa::mfma::supported(PA_BF16, *shape)) return PA_ERR_UNSUPPORTED;
+  if (!out_slice_token || !tokp) return PA_ERR_NULL;
+  return pa::gale::pack_tokens(*shape, out_slice_token, tokp, static_cast<hipStream_t>(stream));
+}
+
 int pa_residual_layernorm(int dtype, int64_t rows, int64_t C, void *y, const pa_block_tail *tail, void *stream) {
   if (dtype != PA_F32 && dtype != PA_BF16) return PA_ERR_UNSUPPORTED;
   if (rows <= 0 || C <= 0 || C > (1 << 16)) return PA_ERR_DIMS;

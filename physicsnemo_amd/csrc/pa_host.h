@@ -104,6 +104,13 @@ int slice_softmax_plus(int dtype, const pa_shape &s, const pa_params &p, const p
                        float *dT_part, hipStream_t st);
 }  // namespace backward
 
+namespace gale {
+size_t lds_bytes(const pa_shape &s, int64_t Sc, int64_t Dc);
+int pack_tokens(const pa_shape &s, const float *out_token, void *tokp, hipStream_t st);
+int slice_cross_mix(const pa_shape &s, const pa_gale_params &gp, int64_t Sc, int64_t Dc, const float *slice_token,
+                    const float *self_token, const float *context, float *out_token, void *tokp, hipStream_t st);
+}  // namespace gale
+
 namespace mfma {
 bool staged_supported(int dtype, const pa_shape &s);
 int slice_softmax_pack(const pa_shape &s, const pa_params &p, const void *x_mid, void *w_pack, int num_cu,

@@ -315,6 +315,13 @@ class MfmaStages:
                                                       self._producer_groups, self.tok.data_ptr(), self.norm.data_ptr(), self.tok_out.data_ptr(),
                                                       self.tokp.data_ptr(), self._stream()), "pa_mfma_combine_attention")
 
+    def set_out_tokens(self, out_tok):
+        """Attended slice tokens computed by the caller (B,H,S,32 float32) in place of `combine_attention`'s."""
+        _need_cuda(out_tok)
+        self.tok_out.copy_(out_tok)
+        _lib.check(self.lib.pa_mfma_pack_tokens(byref(self.shape), self.tok_out.data_ptr(), self.tokp.data_ptr(),
+                                                self._stream()), "pa_mfma_pack_tokens")
+
     # ---- backward-pass stages (pa_mfma_backward_query() == 1) ----
     def rows_gemm_packed(self, inp, weight, bias, natural=True, packed=True):
         """bf16 Linear (B, N, c_in) -> H*32 columns; returns (natural (B, N, H*32) or None, packed buffer or None)."""
@@ -512,3 +519,19 @@ def slice_softmax_plus_backward(x_mid, uniform, w, d_out_x, tok_out, d_num, d_no
         d_x_mid.data_ptr(), d_z.data_ptr(), d_a1.data_ptr(), d_a2.data_ptr(), dT.data_ptr(),
         _lib.current_stream_ptr(w.device)), "pa_slice_softmax_plus_backward")
     return d_x_mid, d_z, d_a1, d_a2, dT.sum(0)
+
+
+def slice_cross_attention_mix(tok, self_out, context, gale_params: dict, dims: LayerDims, tokp=None):
+    """GALE slice-token stage: cross-attention of the slice tokens (B,H,S,D) to `context` (B,H,Sc,Dc) blended with the
+    self-attention output; all float32.  `gale_params`: the cross_q/k/v weights and biases plus either ``state_mixing``
+    or ``concat_project_weight`` / ``concat_project_bias``.  `tokp`: the MFMA deslice operand buffer to fill as well."""
+    _need_cuda(tok, self_out, context)
+    if context.dtype != torch.float32 or context.ndim != 4 or context.shape[:2] != (dims.B, dims.H):
+        raise ValueError(f"context must be float32 (B, H, Sc, Dc) = ({dims.B}, {dims.H}, ., .), got {tuple(context.shape)}")
+    gp = _lib.PaGaleParams(*[_lib.ptr(gale_params.get(k)) for k, _ in _lib.PaGaleParams._fields_])
+    out = torch.empty_like(tok)
+    _lib.check(_lib.load().pa_slice_cross_attention_mix(
+        byref(dims.c()), byref(gp), context.shape[2], context.shape[3], tok.data_ptr(), self_out.data_ptr(),
+        context.data_ptr(), out.data_ptr(), _lib.ptr(tokp), _lib.current_stream_ptr(tok.device)),
+        "pa_slice_cross_attention_mix")
+    return out

@@ -1,0 +1,193 @@
+"""GALE (Geometry-Aware Latent Embeddings) attention layers on the PhysicsAttention HIP kernels.
+
+Mirrors ``physicsnemo/nn/module/gale.py``:
+  GALE:242-398 (irregular), GALEStructuredMesh2D:447-478, GALEStructuredMesh3D:480-512, ``_gale_cross_init``:401-429,
+  ``_gale_forward_impl``:148-239, ``_gale_compute_slice_attention_cross``:87-145, ``_mix_self_and_cross``:43-84.
+
+A GALE layer is a PhysicsAttention layer whose slice tokens, besides attending to each other, attend to a context
+``(B, H, S_c, D_c)``; the two results are blended (learned sigmoid gate, or concatenation + Linear + GELU) before the
+deslice.  Same constructor arguments, parameter names and ``forward(x: tuple, context=None) -> list`` as the
+reference, so a reference ``state_dict`` loads unchanged.  Every per-point stage runs on the layer's own kernels (the
+fused bf16 MFMA kernels where they serve the shape); the cross-attention + blend is one small kernel per (batch, head).
+With gradients required the per-point stages run on the layer's forward / backward kernels and the slice-token stage
+(S x D work per (batch, head)) is evaluated with PyTorch ops under autograd (``autograd.GALEFunction``).
+"""
+from __future__ import annotations
+
+import torch
+import torch.nn as nn
+
+from . import functional as PF
+from .autograd import GALEFunction
+from .physics_attention import (
+    PhysicsAttentionIrregularMesh,
+    PhysicsAttentionStructuredMesh2D,
+    PhysicsAttentionStructuredMesh3D,
+)
+
+_MODES = ("weighted", "concat_project")
+
+
+def _gale_cross_init(self: nn.Module, dim_head: int, context_dim: int, state_mixing_mode: str) -> None:
+    """Cross-attention parameters in the reference's registration order (gale.py:401-429)."""
+    self.cross_q = nn.Linear(dim_head, dim_head)
+    self.cross_k = nn.Linear(context_dim, dim_head)
+    self.cross_v = nn.Linear(context_dim, dim_head)
+    self.state_mixing_mode = state_mixing_mode
+    if state_mixing_mode == "weighted":
+        self.state_mixing = nn.Parameter(torch.tensor(0.0))
+    elif state_mixing_mode == "concat_project":
+        self.concat_project = nn.Sequential(nn.Linear(2 * dim_head, dim_head), nn.GELU())
+    else:
+        raise ValueError(f"Invalid state_mixing_mode: {state_mixing_mode!r}. Expected 'weighted' or 'concat_project'.")
+    self.context_dim = context_dim
+
+
+class _GALEForwardMixin:
+    """``forward`` shared by the three variants (reference ``_gale_forward_impl``)."""
+
+    def gale_params(self, device: torch.device) -> dict:
+        """The cross-attention / blend parameters as float32 contiguous tensors on `device`."""
+        def f32(t):
+            return t.detach().to(device=device, dtype=torch.float32).contiguous()
+
+        p = {f"cross_{n}_{kind}": f32(getattr(getattr(self, f"cross_{n}"), kind))
+             for n in "qkv" for kind in ("weight", "bias")}
+        if self.state_mixing_mode == "weighted":
+            p["state_mixing"] = f32(self.state_mixing).reshape(1)
+        else:
+            p["concat_project_weight"] = f32(self.concat_project[0].weight)
+            p["concat_project_bias"] = f32(self.concat_project[0].bias)
+        return p
+
+    def _check_context(self, context: torch.Tensor, batch: int) -> None:
+        if context.ndim != 4 or context.shape[0] != batch or context.shape[1] != self.heads or \
+                context.shape[3] != self.context_dim:
+            raise ValueError(f"Expected context of shape (B, H, S_c, D_c) = ({batch}, {self.heads}, S_c, "
+                             f"{self.context_dim}), got {tuple(context.shape)}")
+
+    def _stage_params(self) -> list:
+        p = [self.qkv_project.weight, self.cross_q.weight, self.cross_q.bias, self.cross_k.weight, self.cross_k.bias,
+             self.cross_v.weight, self.cross_v.bias]
+        if self.state_mixing_mode == "weighted":
+            return p + [self.state_mixing]
+        return p + [self.concat_project[0].weight, self.concat_project[0].bias]
+
+    def _token_stage(self, tok: torch.Tensor, context: torch.Tensor) -> torch.Tensor:
+        """Slice tokens (B,H,S,D) -> blended attended tokens with PyTorch ops in float32 (reference :207-229)."""
+        sdpa = torch.nn.functional.scaled_dot_product_attention
+        with torch.autocast("cuda", enabled=False):
+            tok, context = tok.float(), context.float()
+            B, H, S, D = tok.shape
+            q, k, v = torch.nn.functional.linear(tok, self.qkv_project.weight.float()).reshape(B, H, S, 3, D).unbind(3)
+            self_out = sdpa(q, k, v, is_causal=False)
+            cross = sdpa(self.cross_q(tok), self.cross_k(context), self.cross_v(context), is_causal=False)
+            if self.state_mixing_mode == "weighted":
+                m = torch.sigmoid(self.state_mixing)
+                return m * self_out + (1 - m) * cross
+            return self.concat_project(torch.cat([self_out, cross], dim=-1))
+
+    def _forward_one_with_grad(self, x: torch.Tensor, context: torch.Tensor) -> torch.Tensor:
+        if self.plus or self.fp8_weights:
+            raise NotImplementedError("GALE training with a context is served for plus=False without fp8 weights")
+        if x.is_cuda and self._wants_fp16(x):
+            with torch.autocast("cuda", enabled=False):
+                return self._forward_one_with_grad(x.float(), context).to(torch.float16)
+        x = self._prepare_input(x)
+        dims = self.layer_dims(x)
+        if not PF.backward_supported(x.dtype, dims):
+            raise RuntimeError(f"the backward kernels do not serve this shape: {dims}")
+        stage = self._stage_params()
+        return GALEFunction.apply(
+            x, context, dims, self.kernel_params(x.dtype, x.device), self._token_stage, len(stage),
+            self.in_project_x.weight, self.in_project_x.bias, self.in_project_fx.weight, self.in_project_fx.bias,
+            self.in_project_slice.weight, self.in_project_slice.bias, self.temperature, self.qkv_project.weight,
+            self.out_linear.weight, self.out_linear.bias, *stage)
+
+    def _forward_one(self, x: torch.Tensor, context: torch.Tensor | None, gp: dict | None) -> torch.Tensor:
+        if context is None:  # self-attention only: the plain layer (reference :226-228)
+            return super().forward(x)
+        if x.is_cuda and self._wants_fp16(x):
+            with torch.autocast("cuda", enabled=False):
+                return self._forward_one(x.float(), context, gp).to(torch.float16)
+        x = self._prepare_input(x)
+        dims = self.layer_dims(x)
+        p = self.kernel_params(x.dtype, x.device)
+        if not self.plus and not self.fp8_weights and PF.query_path(x.dtype, dims) == 1:
+            st = PF.MfmaStages(p, dims, x.device)
+            st.pack_params()
+            if st.fused_groups > 0:
+                st.project_softmax_reduce(x)
+            else:
+                st.project_softmax(x)
+                st.slice_reduce()
+            st.combine_attention()
+            PF.slice_cross_attention_mix(st.tok, st.tok_out, context, gp, dims, tokp=st.tokp)
+            y = torch.empty_like(x)
+            st.deslice_project(y)
+            return y
+        if self.fp8_weights:
+            raise NotImplementedError("fp8 weights are served by the plain layer only")
+        x_mid, fx_mid = PF.project_inputs(x, p, dims)
+        if self.plus:
+            u = torch.rand((dims.B, dims.N, dims.H, dims.S), dtype=x.dtype, device=x.device)
+            w = PF.slice_softmax_plus(x_mid, u, p, dims)
+        else:
+            w = PF.slice_softmax(x_mid, p, dims)
+        tok, _ = PF.slice_reduce(w, fx_mid, dims)
+        self_out = PF.slice_attention(tok, p, dims)
+        out_tok = PF.slice_cross_attention_mix(tok, self_out, context, gp, dims)
+        return PF.deslice_project(w, out_tok, p, dims)
+
+    def forward(self, x: tuple, context: torch.Tensor | None = None) -> list:
+        """x: tuple of (B, N, C) tensors; context (B, H, S_c, D_c) or None -> list of (B, N, C) tensors."""
+        if isinstance(x, torch.Tensor):
+            raise TypeError("GALE takes a tuple of input tensors (reference gale.py:352-356)")
+        if len(x) == 0:
+            raise ValueError("Expected non-empty tuple of input tensors")
+        for i, t in enumerate(x):
+            if t.ndim != 3:
+                raise ValueError(f"Expected 3D input tensor (B, N, C) at index {i}, "
+                                 f"got {t.ndim}D tensor with shape {tuple(t.shape)}")
+        gp = None
+        if context is not None:
+            for t in x:
+                self._validate(t)
+            self._check_context(context, x[0].shape[0])
+            if torch.is_grad_enabled() and (context.requires_grad or any(self._needs_grad(t) for t in x)):
+                return [self._forward_one_with_grad(t, context) for t in x]
+            context = context.detach().float().contiguous()
+            gp = self.gale_params(context.device)
+        return [self._forward_one(t, context, gp) for t in x]
+
+
+class GALE(_GALEForwardMixin, PhysicsAttentionIrregularMesh):
+    """Irregular-mesh GALE layer (reference gale.py:242-398)."""
+
+    def __init__(self, dim: int, heads: int = 8, dim_head: int = 64, dropout: float = 0.0, slice_num: int = 64,
+                 use_te: bool = False, plus: bool = False, context_dim: int = 0, concrete_dropout: bool = False,
+                 state_mixing_mode: str = "weighted"):
+        super().__init__(dim, heads, dim_head, dropout, slice_num, use_te, plus)
+        _gale_cross_init(self, dim_head, context_dim, state_mixing_mode)
+        if concrete_dropout:
+            raise NotImplementedError("ConcreteDropout is a training-time regulariser; the HIP layer has none")
+
+
+class GALEStructuredMesh2D(_GALEForwardMixin, PhysicsAttentionStructuredMesh2D):
+    """GALE with Conv2d projections on a 2-D grid (reference gale.py:447-478)."""
+
+    def __init__(self, dim: int, spatial_shape: tuple[int, int], heads: int = 8, dim_head: int = 64,
+                 dropout: float = 0.0, slice_num: int = 64, kernel: int = 3, use_te: bool = False, plus: bool = False,
+                 context_dim: int = 0, state_mixing_mode: str = "weighted"):
+        super().__init__(dim, spatial_shape, heads, dim_head, dropout, slice_num, kernel, use_te, plus)
+        _gale_cross_init(self, dim_head, context_dim, state_mixing_mode)
+
+
+class GALEStructuredMesh3D(_GALEForwardMixin, PhysicsAttentionStructuredMesh3D):
+    """GALE with Conv3d projections on a 3-D grid (reference gale.py:480-512)."""
+
+    def __init__(self, dim: int, spatial_shape: tuple[int, int, int], heads: int = 8, dim_head: int = 64,
+                 dropout: float = 0.0, slice_num: int = 64, kernel: int = 3, use_te: bool = False, plus: bool = False,
+                 context_dim: int = 0, state_mixing_mode: str = "weighted"):
+        super().__init__(dim, spatial_shape, heads, dim_head, dropout, slice_num, kernel, use_te, plus)
+        _gale_cross_init(self, dim_head, context_dim, state_mixing_mode)

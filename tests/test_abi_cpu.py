@@ -237,3 +237,27 @@ def test_time_input_model_matches_oracle_layout_and_embedding_closed_forms():
     m.load_state_dict(sd)
     with pytest.raises(ValueError, match="time_input=False"):
         pn.Transolver(use_te=False, **kw)(fx, pos, time=t)
+
+
+def test_gale_modules_share_the_reference_state_dict_contract():
+    """GALE variants: constructor arguments, parameter names / order / shapes as in gale.py:242-512 (the oracle holds
+    the same contract, pinned against the reference's registration order in test_oracle_gale.py)."""
+    from oracle import torch_oracle as to
+    for mode in ("weighted", "concat_project"):
+        torch.manual_seed(0)
+        ref = to.OracleGALE(16, heads=2, dim_head=8, slice_num=4, context_dim=5, state_mixing_mode=mode)
+        torch.manual_seed(0)
+        hip = pn.GALE(16, heads=2, dim_head=8, slice_num=4, context_dim=5, state_mixing_mode=mode, use_te=False)
+        assert list(hip.state_dict()) == list(ref.state_dict())
+        for k, v in ref.state_dict().items():  # same seed, same construction order: same initial values
+            assert torch.equal(hip.state_dict()[k], v), k
+        hip.load_state_dict(ref.state_dict())
+    g2 = pn.GALEStructuredMesh2D(16, (3, 4), heads=2, dim_head=8, slice_num=4, kernel=3, context_dim=5)
+    assert g2.in_project_x.weight.shape == (16, 16, 3, 3) and g2.cross_k.weight.shape == (8, 5)
+    g3 = pn.GALEStructuredMesh3D(16, (2, 3, 4), heads=2, dim_head=8, slice_num=4, kernel=3, context_dim=5,
+                                 state_mixing_mode="concat_project")
+    assert g3.in_project_x.weight.ndim == 5 and g3.concat_project[0].weight.shape == (8, 16)
+    with pytest.raises(ValueError, match="Invalid state_mixing_mode"):
+        pn.GALE(16, heads=2, dim_head=8, slice_num=4, context_dim=5, state_mixing_mode="sum")
+    with pytest.raises(RuntimeError, match="GPU"), torch.no_grad():
+        pn.GALE(16, heads=2, dim_head=8, slice_num=4, context_dim=5)((torch.randn(1, 7, 16),), torch.randn(1, 2, 3, 5))

@@ -1,0 +1,167 @@
+"""GALE layers (PhysicsAttention + cross-attention of the slice tokens to a context) on the HIP kernels against the
+oracle.  Bars: fp32 rtol 1e-4 (gradients 2e-4) with atol = rtol * max|ref|; bf16 output rel-L2 <= 1e-2 and bf16
+gradients rel-L2 <= 5e-2 (d temperature 6e-2; measured: 3.3e-2 for the gradients through the slice softmax, under 1e-2
+for the rest) against the fp32 oracle."""
+import pytest
+import torch
+
+from oracle import torch_oracle as to
+import physicsnemo_amd as pn
+from physicsnemo_amd import functional as PF
+from gpu_util import announce, assert_fp32_close, assert_rel_l2
+
+pytestmark = pytest.mark.gpu
+
+
+def _pair(variant, mode, dim, heads, dim_head, S, context_dim, grid=None, plus=False, seed=0):
+    torch.manual_seed(seed)
+    kw = dict(heads=heads, dim_head=dim_head, slice_num=S, context_dim=context_dim, state_mixing_mode=mode, plus=plus)
+    if variant == "irregular":
+        ref, hip = to.OracleGALE(dim, **kw), pn.GALE(dim, use_te=False, **kw)
+    elif variant == "structured2d":
+        ref = to.OracleGALEStructuredMesh2D(dim, grid, kernel=3, **kw)
+        hip = pn.GALEStructuredMesh2D(dim, grid, kernel=3, use_te=False, **kw)
+    else:
+        raise ValueError(variant)
+    with torch.no_grad():
+        ref.in_project_slice.weight.mul_(2.0)
+        if mode == "weighted":
+            ref.state_mixing.fill_(0.6)
+    hip.load_state_dict(ref.state_dict())
+    return ref.eval(), hip.eval().cuda()
+
+
+@pytest.mark.parametrize("variant,mode,dim,heads,dim_head,S,B,N,Sc,Dc,grid", [
+    ("irregular", "weighted", 32, 4, 8, 8, 2, 300, 5, 7, None),
+    ("irregular", "concat_project", 32, 4, 8, 8, 2, 300, 5, 7, None),
+    ("irregular", "weighted", 64, 2, 32, 64, 1, 1000, 1, 16, None),
+    ("irregular", "concat_project", 48, 3, 16, 20, 3, 77, 130, 3, None),
+    ("structured2d", "weighted", 32, 4, 8, 16, 2, 63, 9, 12, (7, 9)),
+])
+def test_fp32_gale_matches_oracle(variant, mode, dim, heads, dim_head, S, B, N, Sc, Dc, grid):
+    announce("fp32 GALE", variant, mode, dim, heads, dim_head, S, B, N, Sc, Dc, grid)
+    ref, hip = _pair(variant, mode, dim, heads, dim_head, S, Dc, grid)
+    x1, x2 = torch.randn(B, N, dim), torch.randn(B, N, dim)
+    ctx = torch.randn(B, heads, Sc, Dc)
+    with torch.no_grad():
+        want = ref((x1, x2), ctx)
+        got = hip((x1.cuda(), x2.cuda()), ctx.cuda())
+        assert isinstance(got, list) and len(got) == 2
+        for g, w in zip(got, want):
+            assert_fp32_close(g, w, "GALE y")
+        # no context: the plain layer (fused path)
+        assert_fp32_close(hip((x1.cuda(),))[0], ref((x1,))[0], "GALE y without context")
+
+
+def test_cross_mix_stage_against_oracle_functions():
+    announce("GALE cross-attention + blend stage")
+    B, H, S, D, Sc, Dc = 2, 3, 24, 16, 11, 5
+    for mode in ("weighted", "concat_project"):
+        torch.manual_seed(4)
+        ref = to.OracleGALE(H * D, heads=H, dim_head=D, slice_num=S, context_dim=Dc, state_mixing_mode=mode)
+        hip = pn.GALE(H * D, heads=H, dim_head=D, slice_num=S, context_dim=Dc, state_mixing_mode=mode, use_te=False)
+        hip.load_state_dict(ref.state_dict())
+        tok, self_out, ctx = torch.randn(B, H, S, D), torch.randn(B, H, S, D), torch.randn(B, H, Sc, Dc)
+        with torch.no_grad():
+            cross = to.gale_cross_attention(tok, ctx, ref.cross_q, ref.cross_k, ref.cross_v)
+            want = to.gale_mix(self_out, cross, mode, getattr(ref, "state_mixing", None),
+                               getattr(ref, "concat_project", None))
+        dims = PF.LayerDims(B, 100, H * D, H, D, S)
+        got = PF.slice_cross_attention_mix(tok.cuda(), self_out.cuda(), ctx.cuda(), hip.gale_params(torch.device("cuda")),
+                                           dims)
+        assert_fp32_close(got, want, f"blend {mode}")
+
+
+@pytest.mark.parametrize("mode,S,N", [("weighted", 64, 4096), ("concat_project", 32, 5000), ("weighted", 128, 3000)])
+def test_bf16_gale_on_the_mfma_kernels(mode, S, N):
+    announce("bf16 GALE MFMA", mode, S, N)
+    ref, hip = _pair("irregular", mode, 256, 8, 32, S, 32)
+    x = torch.randn(2, N, 256)
+    ctx = torch.randn(2, 8, 48, 32)
+    xb = x.cuda().bfloat16()
+    assert PF.query_path(torch.bfloat16, hip.layer_dims(xb)) == 1
+    with torch.no_grad():
+        want = ref((x,), ctx)[0]
+        got = hip((xb,), ctx.cuda())[0]
+        plain = hip((xb,))[0]
+    assert got.dtype == torch.bfloat16
+    assert_rel_l2(got, want, "bf16 GALE y", tol=1e-2)
+    assert to.rel_l2(plain.float().cpu(), want) > 5e-2  # the context matters in this case
+
+
+def test_gale_plus_and_errors():
+    announce("GALE plus / errors")
+    ref, hip = _pair("irregular", "weighted", 32, 4, 8, 8, 7, plus=True)
+    x = torch.randn(2, 200, 32, device="cuda")
+    ctx = torch.randn(2, 4, 5, 7, device="cuda")
+    with torch.no_grad():
+        torch.manual_seed(5)
+        a = hip((x,), ctx)[0]
+        torch.manual_seed(5)
+        b = hip((x,), ctx)[0]
+    assert torch.equal(a, b) and torch.isfinite(a).all()
+    with pytest.raises(ValueError, match="non-empty"):
+        hip(())
+    with pytest.raises(ValueError, match="Expected 3D input tensor"):
+        hip((x[0],), ctx)
+    with pytest.raises(ValueError, match="Expected context"):
+        hip((x,), ctx[:, :2])
+    with pytest.raises(TypeError):
+        hip(x, ctx)
+    with pytest.raises(NotImplementedError):  # training with a context: plus=False only
+        hip((x.requires_grad_(True),), ctx)
+
+
+def _gale_grads(module, x, ctx, probe):
+    module.zero_grad(set_to_none=True)
+    x = x.clone().requires_grad_(True)
+    ctx = ctx.clone().requires_grad_(True)
+    y = module((x,), ctx)[0]
+    (y.float() * probe.to(y.device)).sum().backward()
+    out = {"x": x.grad, "context": ctx.grad}
+    out.update({name: p.grad for name, p in module.named_parameters()})
+    return y, out
+
+
+@pytest.mark.parametrize("variant,mode,dim,heads,dim_head,S,B,N,Sc,Dc,grid", [
+    ("irregular", "weighted", 32, 4, 8, 8, 2, 300, 5, 7, None),
+    ("irregular", "concat_project", 64, 2, 32, 64, 1, 1000, 9, 16, None),
+    ("structured2d", "weighted", 32, 4, 8, 16, 2, 63, 9, 12, (7, 9)),
+])
+def test_fp32_gale_gradients(variant, mode, dim, heads, dim_head, S, B, N, Sc, Dc, grid):
+    announce("fp32 GALE backward", variant, mode, dim, heads, dim_head, S, B, N, Sc, Dc, grid)
+    ref, hip = _pair(variant, mode, dim, heads, dim_head, S, Dc, grid)
+    ref.train(), hip.train()
+    x, probe, ctx = torch.randn(B, N, dim), torch.randn(B, N, dim), torch.randn(B, heads, Sc, Dc)
+    y_ref, want = _gale_grads(ref, x, ctx, probe)
+    y_hip, got = _gale_grads(hip, x.cuda(), ctx.cuda(), probe)
+    assert_fp32_close(y_hip, y_ref, "forward y (training path)")
+    assert set(got) == set(want)
+    for name in want:
+        assert got[name] is not None and got[name].shape == want[name].shape, name
+        if name == "cross_k.bias":  # shifts every score of a query alike: the gradient is zero in exact arithmetic
+            assert got[name].abs().max() < 1e-5 and want[name].abs().max() < 1e-5
+            continue
+        assert_fp32_close(got[name], want[name], f"grad {name}", rtol=2e-4)
+
+
+def test_bf16_gale_gradients_on_the_mfma_kernels():
+    announce("bf16 GALE backward (autocast, MFMA)")
+    ref, hip = _pair("irregular", "weighted", 256, 8, 32, 64, 32)
+    ref.train(), hip.train()
+    torch.manual_seed(5)
+    x, probe, ctx = torch.randn(2, 2048, 256), torch.randn(2, 2048, 256), torch.randn(2, 8, 48, 32)
+    _, want = _gale_grads(ref, x, ctx, probe)
+    hip.zero_grad(set_to_none=True)
+    xc, cc = x.cuda().requires_grad_(True), ctx.cuda().requires_grad_(True)
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        y = hip((xc,), cc)[0]
+    assert y.dtype == torch.bfloat16
+    (y.float() * probe.cuda()).sum().backward()
+    got = {"x": xc.grad, "context": cc.grad}
+    got.update({name: p.grad for name, p in hip.named_parameters()})
+    for name in want:
+        assert got[name] is not None and torch.isfinite(got[name]).all(), name
+        if name != "cross_k.bias":
+            # d temperature: 8 scalars, each a sum of cancelling terms over 4096 points of bf16 activations
+            assert_rel_l2(got[name], want[name], f"bf16 GALE grad {name}", tol=6e-2 if name == "temperature" else 5e-2)
