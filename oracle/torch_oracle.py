@@ -332,6 +332,71 @@ class OracleGALEStructuredMesh2D(_GALECore, OraclePhysicsAttentionStructuredMesh
         self._init_cross(dim_head, context_dim, state_mixing_mode)
 
 
+class _ProjectorCore(nn.Module):
+    """Slice components and forward of the GeoTransolver context projectors
+    (physicsnemo/models/geotransolver/context_projector.py:108-187, :338-378): the encoding half of the layer; returns
+    the slice tokens (B, H, S, D).  in_project_slice keeps nn.Linear's default init here (no orthogonal_)."""
+
+    def _init_slice_components(self, dim_head, slice_num, heads, plus):
+        self.in_project_slice = nn.Linear(dim_head, slice_num)
+        self.temperature = nn.Parameter(torch.ones([1, 1, heads, 1]) * 0.5)
+        if plus:
+            self.proj_temperature = nn.Sequential(nn.Linear(dim_head, slice_num), nn.GELU(),
+                                                  nn.Linear(slice_num, 1), nn.GELU())
+
+    def forward(self, x, noise_u=None):
+        if x.ndim != 3:
+            raise ValueError(f"Expected 3D input tensor (B, N, C), got {x.ndim}D tensor with shape {tuple(x.shape)}")
+        x_mid, fx_mid = self._project(x)
+        logits = slice_logits(x_mid, self.in_project_slice.weight, self.in_project_slice.bias)
+        if self.plus:
+            u = torch.rand_like(logits) if noise_u is None else noise_u
+            return slice_weights_and_tokens_plus(logits, x_mid, self.temperature, self.proj_temperature, u)[1]
+        return slice_weights_and_tokens(logits, fx_mid, self.temperature)[1]
+
+
+class OracleContextProjector(_ProjectorCore):
+    """context_projector.py:190-378 with use_te=False, concrete_dropout=False."""
+
+    def __init__(self, dim, heads=8, dim_head=64, dropout=0.0, slice_num=64, plus=False):
+        super().__init__()
+        self.dim, self.heads, self.dim_head, self.plus = dim, heads, dim_head, plus
+        self.in_project_x = nn.Linear(dim, heads * dim_head)
+        if not plus:
+            self.in_project_fx = nn.Linear(dim, heads * dim_head)
+        self.softmax = nn.Softmax(dim=-1)
+        self._init_slice_components(dim_head, slice_num, heads, plus)
+
+    def _project(self, x):
+        if self.plus:
+            x_mid = split_heads(F.linear(x, self.in_project_x.weight, self.in_project_x.bias), self.heads, self.dim_head)
+            return x_mid, x_mid
+        return project_linear(x, self.in_project_x.weight, self.in_project_x.bias, self.in_project_fx.weight,
+                              self.in_project_fx.bias, self.heads, self.dim_head)
+
+
+class OracleStructuredContextProjector(_ProjectorCore):
+    """context_projector.py:380-486 with use_te=False, plus=False: Conv2d / Conv3d projections."""
+
+    def __init__(self, dim, spatial_shape, heads=8, dim_head=64, dropout=0.0, slice_num=64, kernel=3):
+        super().__init__()
+        if len(spatial_shape) not in (2, 3):
+            raise ValueError(f"StructuredContextProjector expects spatial_shape of length 2 or 3, got {spatial_shape!r}")
+        self.dim, self.heads, self.dim_head, self.plus = dim, heads, dim_head, False
+        self.spatial_shape = tuple(int(s) for s in spatial_shape)
+        conv = nn.Conv2d if len(spatial_shape) == 2 else nn.Conv3d
+        self.in_project_x = conv(dim, heads * dim_head, kernel, 1, kernel // 2)
+        self.in_project_fx = conv(dim, heads * dim_head, kernel, 1, kernel // 2)
+        self.softmax = nn.Softmax(dim=-1)
+        self.dropout = nn.Dropout(dropout)
+        self._init_slice_components(dim_head, slice_num, heads, False)
+
+    def _project(self, x):
+        fn = project_conv2d if len(self.spatial_shape) == 2 else project_conv3d
+        return fn(x, self.in_project_x.weight, self.in_project_x.bias, self.in_project_fx.weight,
+                  self.in_project_fx.bias, self.heads, self.dim_head, *self.spatial_shape)
+
+
 class OracleMlp(nn.Module):
     """Linear -> GELU(erf) -> Linear, keys ``layers.0`` / ``layers.2``
     (physicsnemo/nn/module/mlp_layers.py:139-173 with one hidden width; activations.py:198 'gelu' -> nn.GELU())."""

@@ -84,7 +84,7 @@ def _finish_backward(ctx, x, dy, out_x, d_wqkv, d_proj, d_z, d_temp, x_mid, temp
     B, N, C, H, D, S = dims.B, dims.N, dims.C, dims.H, dims.D, dims.S
     HD = H * D
     linear = PF.LayerDims(B, N, C, H, D, S)
-    d_wo, d_bo = _wgrad(dy, out_x)
+    d_wo, d_bo = _wgrad(dy, out_x) if out_x is not None else (None, None)  # None: no out_linear (context projector)
     d_ws, d_bs = _slice_weight_grad(d_z, x_mid, H, S, D)
     t = temperature.reshape(-1)
     d_temp = d_temp * ((t >= 0.5) & (t <= 5.0)).to(d_temp.dtype)
@@ -325,6 +325,56 @@ class GALEFunction(torch.autograd.Function):
         # qkv_project.weight takes part in the token stage only: its gradient comes with `d_stage`
         base = _finish_backward(ctx, x, dy, out_x, None, d_proj, d_z, d_temp, x_mid, temperature, param_offset=6)
         return (base[0], d_context, None, None, None, None) + base[3:] + tuple(d_stage)
+
+
+class SliceTokensFunction(torch.autograd.Function):
+    """x -> normalised slice tokens (B,H,S,D) float32: the projection, slice-softmax and aggregation stages of the
+    layer on their own (a GeoTransolver context projector, context_projector.py:338-378), differentiable w.r.t. x and
+    the seven parameters involved.  The backward is the per-point backward kernel with no deslice term (d out_x = 0)."""
+
+    @staticmethod
+    def forward(ctx, x, dims, kparams, wx, bx, wf, bf, ws, bs, temperature):
+        mfma = PF.mfma_backward_supported(x.dtype, dims)
+        if mfma:
+            st = PF.MfmaStages(kparams, dims, x.device)
+            st.pack_params()
+            if st.fused_groups > 0:
+                st.project_softmax_reduce(x)
+            else:
+                st.project_softmax(x)
+                st.slice_reduce()
+            st.combine_attention()
+            tok, norm = st.tok.clone(), st.norm
+            ctx.stages = st
+            ctx.save_for_backward(x, temperature, tok, norm)
+        else:
+            x_mid, fx_mid = PF.project_inputs(x, kparams, dims)
+            w = PF.slice_softmax(x_mid, kparams, dims)
+            tok, norm = PF.slice_reduce(w, fx_mid, dims)
+            ctx.save_for_backward(x, temperature, tok, norm, x_mid, fx_mid, w)
+        ctx.mfma, ctx.dims, ctx.kparams = mfma, dims, kparams
+        ctx.param_like = (wx, bx, wf, bf, ws, bs, temperature)
+        return tok
+
+    @staticmethod
+    def backward(ctx, d_tok):
+        dims, kp = ctx.dims, ctx.kparams
+        x, temperature, tok, norm = ctx.saved_tensors[:4]
+        d_tok = d_tok.float()
+        d_num = (d_tok / norm[..., None]).contiguous()
+        d_norm = (-(d_tok * tok).sum(-1) / norm).contiguous()
+        g = torch.zeros(dims.B, dims.N, dims.H * dims.D, dtype=x.dtype, device=x.device)
+        if ctx.mfma:
+            st = ctx.stages
+            st.tok_out.zero_()
+            x_mid, fx_mid = PF.project_inputs(x, kp, dims)
+            d_proj, d_z, d_temp = st.slice_softmax_backward(x_mid, fx_mid, g, d_num, d_norm)
+        else:
+            x_mid, fx_mid, w = ctx.saved_tensors[4:]
+            d_proj, d_z, d_temp = PF.slice_softmax_backward(x_mid, fx_mid, w, g, torch.zeros_like(tok), d_num, d_norm,
+                                                            kp, dims)
+        base = _finish_backward(ctx, x, None, None, None, d_proj, d_z, d_temp, x_mid, temperature)
+        return base[:3] + base[3:10]
 
 
 class LinearFunction(torch.autograd.Function):

@@ -1,0 +1,177 @@
+"""Context projectors of GeoTransolver on the PhysicsAttention HIP kernels.
+
+Mirrors ``physicsnemo/models/geotransolver/context_projector.py``: ContextProjector:190-378 (Linear projections),
+StructuredContextProjector:380-486 (Conv2d / Conv3d projections), ``_SliceToContextMixin``:108-187.
+
+A context projector is the encoding half of a PhysicsAttention layer -- projections, slice softmax, aggregation --
+and returns the slice tokens ``(B, H, S, D)`` that GALE layers cross-attend to; it never projects back to the points.
+It therefore runs on stages (a) and (b) of the layer: the fused bf16 MFMA kernel where it serves the shape (its slice
+self-attention and deslice operands are simply not used), the natural-layout kernels otherwise.  Same constructor
+arguments and parameter names as the reference; ``concrete_dropout=True`` is not served.
+"""
+from __future__ import annotations
+
+import torch
+import torch.nn as nn
+
+from . import functional as PF
+from .autograd import SliceTokensFunction
+
+
+class _SliceToContextMixin:
+    """Shared slice components and forward (reference :108-187, :338-378, :466-486)."""
+
+    def _init_slice_components(self, dim_head: int, slice_num: int, heads: int, plus: bool) -> None:
+        self.in_project_slice = nn.Linear(dim_head, slice_num)
+        self.temperature = nn.Parameter(torch.ones([1, 1, heads, 1]) * 0.5)
+        if plus:
+            self.proj_temperature = nn.Sequential(nn.Linear(dim_head, slice_num), nn.GELU(),
+                                                  nn.Linear(slice_num, 1), nn.GELU())
+        self.slice_num = slice_num
+        self._kernel_param_cache: dict = {}
+
+    def _conv_geometry(self):
+        return 0, 0, 0, 0
+
+    def layer_dims(self, x: torch.Tensor) -> PF.LayerDims:
+        gh, gw, k, gd = self._conv_geometry()
+        return PF.LayerDims(x.shape[0], x.shape[1], self.dim, self.heads, self.dim_head, self.slice_num, gh, gw, k, gd)
+
+    def kernel_params(self, dtype: torch.dtype, device: torch.device) -> dict:
+        """Parameters as the C ABI wants them (projection weights in `dtype`, the rest float32).  The layer's
+        qkv_project / out_linear, which a projector does not have, are zero tensors: the fused kernels' parameter pack
+        reads them, nothing a projector returns depends on them."""
+        named = [("in_project_x_weight", self.in_project_x.weight, True),
+                 ("in_project_x_bias", self.in_project_x.bias, False)]
+        if self.plus:
+            named += [(f"proj_temperature_{i}_{kind}", getattr(self.proj_temperature[i], kind), False)
+                      for i in (0, 2) for kind in ("weight", "bias")]
+        else:
+            named += [("in_project_fx_weight", self.in_project_fx.weight, True),
+                      ("in_project_fx_bias", self.in_project_fx.bias, False)]
+        named += [("in_project_slice_weight", self.in_project_slice.weight, False),
+                  ("in_project_slice_bias", self.in_project_slice.bias, False),
+                  ("temperature", self.temperature, False)]
+        stamp = (dtype, device) + tuple((p.data_ptr(), p._version, p.dtype) for _, p, _ in named)
+        if self._kernel_param_cache.get("stamp") == stamp:
+            return self._kernel_param_cache["params"]
+        with torch.no_grad():
+            params = {name: p.detach().to(device=device, dtype=dtype if big else torch.float32).contiguous().reshape(-1).clone()
+                      for name, p, big in named}
+            HD, D = self.heads * self.dim_head, self.dim_head
+            params["qkv_project_weight"] = torch.zeros(3 * D * D, dtype=torch.float32, device=device)
+            params["out_linear_weight"] = torch.zeros(self.dim * HD, dtype=dtype, device=device)
+            params["out_linear_bias"] = torch.zeros(self.dim, dtype=torch.float32, device=device)
+        self._kernel_param_cache = {"stamp": stamp, "params": params}
+        return params
+
+    def _check_spatial(self, x: torch.Tensor) -> None:
+        pass
+
+    def _prepare_input(self, x: torch.Tensor) -> torch.Tensor:
+        if not x.is_cuda:
+            raise RuntimeError("physicsnemo_amd context projectors run on GPU tensors only (no CPU fallback)")
+        if torch.is_autocast_enabled("cuda"):
+            ac = torch.get_autocast_dtype("cuda")
+            x = x.to(torch.float32 if ac == torch.float16 else ac)
+        elif x.dtype == torch.float16:
+            x = x.float()
+        if x.dtype not in (torch.float32, torch.bfloat16):
+            raise TypeError(f"expected float32 or bfloat16 input, got {x.dtype}")
+        self._check_spatial(x)
+        return x.contiguous()
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        """(B, N, C) -> slice tokens (B, H, S, D), float32."""
+        if x.ndim != 3:
+            raise ValueError(f"Expected 3D input tensor (B, N, C), got {x.ndim}D tensor with shape {tuple(x.shape)}")
+        if x.shape[-1] != self.dim:
+            raise ValueError(f"Expected input feature dimension {self.dim}, got {x.shape[-1]}")
+        needs_grad = torch.is_grad_enabled() and (x.requires_grad or any(p.requires_grad for p in self.parameters()))
+        x = self._prepare_input(x)
+        dims = self.layer_dims(x)
+        p = self.kernel_params(x.dtype, x.device)
+        if needs_grad:
+            if self.plus:
+                raise NotImplementedError("training a plus=True context projector is not served")
+            if not PF.backward_supported(x.dtype, dims):
+                raise RuntimeError(f"the backward kernels do not serve this shape: {dims}")
+            return SliceTokensFunction.apply(x, dims, p, self.in_project_x.weight, self.in_project_x.bias,
+                                             self.in_project_fx.weight, self.in_project_fx.bias,
+                                             self.in_project_slice.weight, self.in_project_slice.bias, self.temperature)
+        if not self.plus and PF.query_path(x.dtype, dims) == 1:
+            st = PF.MfmaStages(p, dims, x.device)
+            st.pack_params()
+            if st.fused_groups > 0:
+                st.project_softmax_reduce(x)
+            else:
+                st.project_softmax(x)
+                st.slice_reduce()
+            st.combine_attention()
+            return st.tok
+        x_mid, fx_mid = PF.project_inputs(x, p, dims)
+        if self.plus:
+            u = torch.rand((dims.B, dims.N, dims.H, dims.S), dtype=x.dtype, device=x.device)
+            w = PF.slice_softmax_plus(x_mid, u, p, dims)
+        else:
+            w = PF.slice_softmax(x_mid, p, dims)
+        return PF.slice_reduce(w, fx_mid, dims)[0]
+
+
+class ContextProjector(_SliceToContextMixin, nn.Module):
+    """Irregular point sets: nn.Linear projections (reference :190-378)."""
+
+    def __init__(self, dim: int, heads: int = 8, dim_head: int = 64, dropout: float = 0.0, slice_num: int = 64,
+                 use_te: bool = False, plus: bool = False, concrete_dropout: bool = False):
+        super().__init__()
+        if concrete_dropout:
+            raise NotImplementedError("ConcreteDropout is a training-time regulariser; the HIP projector has none")
+        inner_dim = dim_head * heads
+        self.dim, self.dim_head, self.heads, self.plus = dim, dim_head, heads, plus
+        self.scale = dim_head ** -0.5
+        self.use_te = use_te
+        # registration order follows the reference so state_dict order and RNG draws agree
+        self.in_project_x = nn.Linear(dim, inner_dim)
+        if not plus:
+            self.in_project_fx = nn.Linear(dim, inner_dim)
+        self.softmax = nn.Softmax(dim=-1)
+        self._init_slice_components(dim_head, slice_num, heads, plus)
+        self.output_dropout = None
+
+
+class StructuredContextProjector(_SliceToContextMixin, nn.Module):
+    """2-D / 3-D grids: Conv2d / Conv3d projections (reference :380-486)."""
+
+    def __init__(self, dim: int, spatial_shape: tuple, heads: int = 8, dim_head: int = 64, dropout: float = 0.0,
+                 slice_num: int = 64, kernel: int = 3, use_te: bool = False, plus: bool = False,
+                 concrete_dropout: bool = False):
+        super().__init__()
+        if len(spatial_shape) not in (2, 3):
+            raise ValueError(f"StructuredContextProjector expects spatial_shape of length 2 or 3, got {spatial_shape!r}")
+        if concrete_dropout:
+            raise NotImplementedError("ConcreteDropout is a training-time regulariser; the HIP projector has none")
+        inner_dim = dim_head * heads
+        self.dim, self.dim_head, self.heads, self.plus = dim, dim_head, heads, plus
+        self.use_te = use_te
+        self.spatial_shape = tuple(int(s) for s in spatial_shape)
+        self._nd = len(self.spatial_shape)
+        self.kernel = kernel
+        conv = nn.Conv2d if self._nd == 2 else nn.Conv3d
+        self.in_project_x = conv(dim, inner_dim, kernel, 1, kernel // 2)
+        if not plus:
+            self.in_project_fx = conv(dim, inner_dim, kernel, 1, kernel // 2)
+        self.softmax = nn.Softmax(dim=-1)
+        self.dropout = nn.Dropout(dropout)
+        self._init_slice_components(dim_head, slice_num, heads, plus)
+        self.output_dropout = None
+
+    def _conv_geometry(self):
+        s = self.spatial_shape
+        return s[0], s[1], self.kernel, (s[2] if self._nd == 3 else 0)
+
+    def _check_spatial(self, x: torch.Tensor) -> None:
+        n = 1
+        for s in self.spatial_shape:
+            n *= s
+        if x.shape[1] != n:
+            raise ValueError(f"Expected N={n} tokens for {self._nd}D grid, got N={x.shape[1]}")

@@ -165,3 +165,98 @@ def test_bf16_gale_gradients_on_the_mfma_kernels():
         if name != "cross_k.bias":
             # d temperature: 8 scalars, each a sum of cancelling terms over 4096 points of bf16 activations
             assert_rel_l2(got[name], want[name], f"bf16 GALE grad {name}", tol=6e-2 if name == "temperature" else 5e-2)
+
+
+# ---------------------------------------------------------------------------------------------------
+# context projectors (GeoTransolver): the encoding half of the layer, returning slice tokens
+# ---------------------------------------------------------------------------------------------------
+def _projector_pair(variant, dim, heads, dim_head, S, grid=None, plus=False, seed=0):
+    torch.manual_seed(seed)
+    if variant == "irregular":
+        ref = to.OracleContextProjector(dim, heads=heads, dim_head=dim_head, slice_num=S, plus=plus)
+        hip = pn.ContextProjector(dim, heads=heads, dim_head=dim_head, slice_num=S, plus=plus)
+    else:
+        ref = to.OracleStructuredContextProjector(dim, grid, heads=heads, dim_head=dim_head, slice_num=S, kernel=3)
+        hip = pn.StructuredContextProjector(dim, grid, heads=heads, dim_head=dim_head, slice_num=S, kernel=3)
+    with torch.no_grad():
+        ref.in_project_slice.weight.mul_(4.0)
+    hip.load_state_dict(ref.state_dict())
+    return ref.eval(), hip.eval().cuda()
+
+
+@pytest.mark.parametrize("variant,dim,heads,dim_head,S,B,N,grid", [
+    ("irregular", 6, 4, 8, 8, 2, 300, None),         # input width differs from heads * dim_head
+    ("irregular", 64, 2, 32, 64, 1, 1000, None),
+    ("structured2d", 5, 4, 8, 16, 2, 63, (7, 9)),
+    ("structured3d", 3, 2, 8, 8, 2, 60, (3, 4, 5)),
+])
+def test_fp32_context_projector_tokens_and_gradients(variant, dim, heads, dim_head, S, B, N, grid):
+    announce("fp32 context projector", variant, dim, heads, dim_head, S, B, N, grid)
+    ref, hip = _projector_pair("irregular" if variant == "irregular" else "structured", dim, heads, dim_head, S, grid)
+    x = torch.randn(B, N, dim)
+    with torch.no_grad():
+        want = ref(x)
+        got = hip(x.cuda())
+    assert got.shape == (B, heads, S, dim_head) and got.dtype == torch.float32
+    assert_fp32_close(got, want, "slice tokens")
+    probe = torch.randn(B, heads, S, dim_head)
+    ref.train(), hip.train()
+    xr = x.clone().requires_grad_(True)
+    (ref(xr) * probe).sum().backward()
+    xh = x.cuda().requires_grad_(True)
+    tok = hip(xh)
+    assert_fp32_close(tok, want, "slice tokens (training path)")
+    (tok * probe.cuda()).sum().backward()
+    assert_fp32_close(xh.grad, xr.grad, "grad x", rtol=2e-4)
+    grads = dict(hip.named_parameters())
+    for name, p in ref.named_parameters():
+        assert grads[name].grad is not None, name
+        assert_fp32_close(grads[name].grad, p.grad, f"grad {name}", rtol=2e-4)
+
+
+def test_bf16_context_projector_feeds_gale_on_the_mfma_kernels():
+    announce("bf16 context projector -> GALE")
+    ref_p, hip_p = _projector_pair("irregular", 256, 8, 32, 64)
+    ref_g, hip_g = _pair("irregular", "weighted", 256, 8, 32, 64, 32)
+    geom, x = torch.randn(2, 3000, 256), torch.randn(2, 4096, 256)
+    with torch.no_grad():
+        ctx_ref = ref_p(geom)
+        want = ref_g((x,), ctx_ref)[0]
+        gb = geom.cuda().bfloat16()
+        assert PF.query_path(torch.bfloat16, hip_p.layer_dims(gb)) == 1
+        ctx_hip = hip_p(gb)
+        got = hip_g((x.cuda().bfloat16(),), ctx_hip)[0]
+    assert_rel_l2(ctx_hip, ctx_ref, "bf16 context tokens", tol=1e-2)
+    assert_rel_l2(got, want, "bf16 GALE y from projected context", tol=1e-2)
+    # training through both, bf16 autocast
+    ref_p.train(), hip_p.train(), ref_g.train(), hip_g.train()
+    probe = torch.randn(2, 4096, 256)
+    (ref_g((x,), ref_p(geom))[0] * probe).sum().backward()
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        y = hip_g((x.cuda(),), hip_p(geom.cuda()))[0]
+    (y.float() * probe.cuda()).sum().backward()
+    for name, p in ref_p.named_parameters():
+        g = dict(hip_p.named_parameters())[name].grad
+        assert g is not None and torch.isfinite(g).all(), name
+        assert_rel_l2(g, p.grad, f"bf16 projector grad {name}", tol=1e-1 if name == "temperature" else 5e-2)
+
+
+def test_context_projector_plus_and_errors():
+    announce("context projector plus / errors")
+    ref, hip = _projector_pair("irregular", 16, 4, 8, 8, plus=True)
+    x = torch.randn(2, 200, 16, device="cuda")
+    with torch.no_grad():
+        torch.manual_seed(3)
+        a = hip(x)
+        torch.manual_seed(3)
+        b = hip(x)
+    assert a.shape == (2, 4, 8, 8) and torch.equal(a, b) and torch.isfinite(a).all()
+    with pytest.raises(ValueError, match="Expected 3D input tensor"):
+        hip(x[0])
+    with pytest.raises(NotImplementedError):
+        hip(x.requires_grad_(True))
+    with pytest.raises(ValueError, match="length 2 or 3"):
+        pn.StructuredContextProjector(4, (3,), heads=2, dim_head=8)
+    sp = pn.StructuredContextProjector(4, (3, 4), heads=2, dim_head=8, slice_num=4).cuda()
+    with pytest.raises(ValueError, match="Expected N=12 tokens"), torch.no_grad():
+        sp(torch.randn(1, 13, 4, device="cuda"))

@@ -138,3 +138,37 @@ def test_gale_state_dict_contract_and_validation():
         m(())
     with pytest.raises(ValueError, match="Expected 3D input tensor"):
         m((torch.randn(3, 16),))
+
+
+def test_context_projector_is_the_encoding_half_of_the_layer():
+    """context_projector.py:338-378 computes exactly the slice tokens of a PhysicsAttention layer with the same
+    projection / slice parameters (physics_attention.py:529-540); state_dict order as registered in :283-300."""
+    torch.manual_seed(2)
+    proj = to.OracleContextProjector(10, heads=2, dim_head=6, slice_num=5).double()
+    assert list(proj.state_dict()) == ["temperature", "in_project_x.weight", "in_project_x.bias", "in_project_fx.weight",
+                                       "in_project_fx.bias", "in_project_slice.weight", "in_project_slice.bias"]
+    layer = to.OraclePhysicsAttentionIrregularMesh(10, heads=2, dim_head=6, slice_num=5).double()
+    layer.load_state_dict(proj.state_dict(), strict=False)
+    x = torch.randn(2, 9, 10, dtype=torch.float64)
+    with torch.no_grad():
+        tok = proj(x)
+        assert tok.shape == (2, 2, 5, 6)
+        torch.testing.assert_close(tok, layer.stages(x)["tok"])
+    ref = no.layer_forward({**_sd_np(layer)}, x.numpy(), 2, 6)
+    np.testing.assert_allclose(tok.numpy(), ref["tok"], rtol=1e-10, atol=1e-12)
+    # structured: same statement with the convolutions
+    sp = to.OracleStructuredContextProjector(4, (3, 4), heads=2, dim_head=6, slice_num=5).double()
+    sl = to.OraclePhysicsAttentionStructuredMesh2D(4, (3, 4), heads=2, dim_head=6, slice_num=5, kernel=3).double()
+    sl.load_state_dict(sp.state_dict(), strict=False)
+    xs = torch.randn(2, 12, 4, dtype=torch.float64)
+    with torch.no_grad():
+        torch.testing.assert_close(sp(xs), sl.stages(xs)["tok"])
+    with pytest.raises(ValueError, match="length 2 or 3"):
+        to.OracleStructuredContextProjector(4, (3,), heads=2, dim_head=6)
+    # plus: one projection, given noise
+    pp = to.OracleContextProjector(10, heads=2, dim_head=6, slice_num=5, plus=True).double()
+    lp = to.OraclePhysicsAttentionIrregularMesh(10, heads=2, dim_head=6, slice_num=5, plus=True).double()
+    lp.load_state_dict(pp.state_dict(), strict=False)
+    u = torch.rand(2, 9, 2, 5, dtype=torch.float64)
+    with torch.no_grad():
+        torch.testing.assert_close(pp(x, u), lp.stages(x, u)["tok"])
