@@ -171,6 +171,77 @@ def time_training_step(points, C, S, reps=3):
                        "backward kernel, split-row MFMA weight-gradient kernel"}
 
 
+def time_variants(points, C, S, reps=5):
+    """The neighbouring layer variants at the layer workload's size where they fit, each forward (no_grad) and, where
+    served, forward + backward: Transolver++ (general kernels), the structured-3D layer (implicit-GEMM projections +
+    general stages), a GALE layer with a projected context (MFMA kernels + the cross-attention stage) and the context
+    projector itself."""
+    import torch
+
+    import physicsnemo_amd as pn
+
+    H = C // 32
+    out = []
+
+    def timed(fn, n=reps):
+        for _ in range(2):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(n):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / n * 1e3
+
+    def entry(name, pts, fwd_ms, train_ms=None):
+        e = {"workload": name, "points": pts, "ms_forward": round(fwd_ms, 3),
+             "mpoints_per_s": round(pts / (fwd_ms * 1e-3) / 1e6, 2)}
+        if train_ms is not None:
+            e["ms_forward_backward"] = round(train_ms, 3)
+        out.append(e)
+
+    def train_step(module, call, x):
+        def step():
+            module.zero_grad(set_to_none=True)
+            x.grad = None
+            with torch.autocast("cuda", dtype=torch.bfloat16):
+                y = call()
+            y.backward(torch.ones_like(y))
+        return step
+
+    torch.manual_seed(0)
+    # GALE + context projector, bf16, MFMA kernels
+    geom = torch.randn(1, points // 4, C, device="cuda").bfloat16()
+    proj = pn.ContextProjector(C, heads=H, dim_head=32, slice_num=S).cuda()
+    gale = pn.GALE(C, heads=H, dim_head=32, slice_num=S, context_dim=32, use_te=False).cuda()
+    x = torch.randn(1, points, C, device="cuda").bfloat16()
+    with torch.no_grad():
+        ctx = proj(geom)
+        entry(f"ContextProjector bf16, C={C}, S={S}", points // 4, timed(lambda: proj(geom)))
+        entry(f"GALE layer bf16 with context ({S} x 32), C={C}, S={S}", points, timed(lambda: gale((x,), ctx)))
+    xg = x.clone().requires_grad_(True)
+    out[-1]["ms_forward_backward"] = round(timed(train_step(gale, lambda: gale((xg,), ctx)[0], xg), 3), 3)
+    del geom, x, xg
+    # Transolver++ (general kernels, fp32 arithmetic): a quarter of the points
+    pts = points // 4
+    plus = pn.PhysicsAttentionIrregularMesh(C, heads=H, dim_head=32, slice_num=S, use_te=False, plus=True).cuda()
+    xp = torch.randn(1, pts, C, device="cuda").bfloat16()
+    with torch.no_grad():
+        fwd = timed(lambda: plus(xp), 3)
+    xpg = xp.clone().requires_grad_(True)
+    entry(f"Transolver++ layer bf16 (general kernels), C={C}, S={S}", pts, fwd,
+          timed(train_step(plus, lambda: plus(xpg), xpg), 2))
+    del xp, xpg
+    # structured 3-D, 64^3 grid, Conv3d k=3 projections
+    g = 64
+    s3 = pn.PhysicsAttentionStructuredMesh3D(C, (g, g, g), heads=H, dim_head=32, slice_num=S, kernel=3,
+                                             use_te=False).cuda()
+    x3 = torch.randn(1, g ** 3, C, device="cuda").bfloat16()
+    with torch.no_grad():
+        entry(f"structured-3D layer bf16, {g}^3 grid, Conv3d k=3, C={C}, S={S}", g ** 3, timed(lambda: s3(x3), 3))
+    return out
+
+
 def time_full_model(name, B, N, functional_dim, embedding_dim, slice_num, n_layers, steps=5, warmup=2, n_hidden=256,
                     fp8_weights=False, graph=True):
     """Forward of a whole Transolver (bf16 autocast, random-init weights, synthetic N(0,1) inputs) -> Mpoints/s.
@@ -381,6 +452,7 @@ def main():
     if not args.no_models:
         out["block_mlp"] = time_block_mlp(1 << 20, 256, 1024)
         out["training_step"] = time_training_step(N, C, S)
+        out["variants"] = time_variants(N, C, S)
         out["full_model"] = [
             time_structured_model(),
             time_full_model("cfg2: Transolver irregular 2D, 8 layers", 8, 32768, 3, 2, 64, 8),

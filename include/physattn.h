@@ -66,6 +66,10 @@ typedef struct pa_shape {
   int64_t B, N, C, H, D, S;
   int64_t grid_h, grid_w, conv_k;
   int64_t grid_d;
+  /* layout of convolution weights: 0 = as torch holds them, (c_out, c_in, k, k[, k]); 1 = tap-major,
+   * (c_out, k, k[, k], c_in) -- the order of the implicit GEMM's reduction index, which lets the kernels fetch
+   * weights with full-width loads (several times faster; the Python modules repack once per parameter set) */
+  int64_t conv_tap_major;
 } pa_shape;
 
 /* Parameters of one layer, named as the reference state_dict keys (PA.py:285-327, :625-627, :740-742). */

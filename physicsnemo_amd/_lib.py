@@ -35,7 +35,8 @@ PA_BUF_BLOB, PA_BUF_FX_PACK, PA_BUF_W_PACK, PA_BUF_PARTIALS, PA_BUF_TOKP = range
 
 
 class PaShape(Structure):
-    _fields_ = [(n, c_int64) for n in ("B", "N", "C", "H", "D", "S", "grid_h", "grid_w", "conv_k", "grid_d")]
+    _fields_ = [(n, c_int64) for n in ("B", "N", "C", "H", "D", "S", "grid_h", "grid_w", "conv_k", "grid_d",
+                                        "conv_tap_major")]
 
 
 class PaParams(Structure):

@@ -62,6 +62,13 @@ def _conv_weight_grad(d_out: torch.Tensor, x: torch.Tensor, grid: tuple, k: int)
     return dW
 
 
+def _torch_conv_layout(w_flat: torch.Tensor, O: int, C: int, taps: tuple, dims) -> torch.Tensor:
+    """The kernel-form convolution weight (flat; tap-major when `dims.conv_tap_major`) as torch's (O, C, k, ...)."""
+    if dims.conv_tap_major:
+        return w_flat.view(O, *taps, C).movedim(-1, 1)
+    return w_flat.view(O, C, *taps)
+
+
 def _slice_weight_grad(d_z: torch.Tensor, x_mid: torch.Tensor, H: int, S: int, D: int):
     """d W_slice[s, d] = sum over points and heads of d z[n, h, s] x_mid[n, h, d] (+ d b_slice).
 
@@ -98,9 +105,11 @@ def _finish_backward(ctx, x, dy, out_x, d_wqkv, d_proj, d_z, d_temp, x_mid, temp
     else:
         grid = (dims.grid_h, dims.grid_w) + ((dims.grid_d,) if dims.grid_d > 0 else ())
         taps = (k,) * len(grid)
-        w_both = torch.cat([wx.view(HD, C, *taps), wf.view(HD, C, *taps)], dim=0)  # (2HD, C, k, ...)
+        w_both = torch.cat([_torch_conv_layout(wx, HD, C, taps, dims), _torch_conv_layout(wf, HD, C, taps, dims)],
+                           dim=0)  # (2HD, C, k, ...)
         # transposed convolution = the same gather with flipped taps and swapped channel roles
-        w_t = w_both.flip(dims=tuple(range(2, 2 + len(grid)))).transpose(0, 1).contiguous()
+        w_t = w_both.flip(dims=tuple(range(2, 2 + len(grid)))).transpose(0, 1)  # (C, 2HD, k, ...)
+        w_t = (w_t.movedim(1, -1) if dims.conv_tap_major else w_t).contiguous()
         dx = PF.rows_gemm(d_proj, w_t, None, dims, 2 * HD, C) if ctx.needs_input_grad[0] else None
         d_w_in = _conv_weight_grad(d_proj, x, grid, k)
         d_b_in = _rows(d_proj).sum(0, dtype=torch.float32)
@@ -231,7 +240,8 @@ class PhysicsAttentionPlusFunction(torch.autograd.Function):
             d_wx, d_bx = _wgrad(d_xm, x)
         else:
             grid = (dims.grid_h, dims.grid_w) + ((dims.grid_d,) if dims.grid_d > 0 else ())
-            w_t = wx.view(HD, C, *((k,) * len(grid))).flip(dims=tuple(range(2, 2 + len(grid)))).transpose(0, 1).contiguous()
+            w_t = _torch_conv_layout(wx, HD, C, (k,) * len(grid), dims).flip(dims=tuple(range(2, 2 + len(grid)))).transpose(0, 1)
+            w_t = (w_t.movedim(1, -1) if dims.conv_tap_major else w_t).contiguous()
             dx = PF.rows_gemm(d_xm, w_t, None, dims, HD, C) if ctx.needs_input_grad[0] else None
             d_wx = _conv_weight_grad(d_xm, x, grid, k)
             d_bx = _rows(d_xm).sum(0, dtype=torch.float32)

@@ -16,6 +16,7 @@ import torch.nn as nn
 
 from . import functional as PF
 from .autograd import SliceTokensFunction
+from .physics_attention import _kernel_layout
 
 
 class _SliceToContextMixin:
@@ -35,7 +36,8 @@ class _SliceToContextMixin:
 
     def layer_dims(self, x: torch.Tensor) -> PF.LayerDims:
         gh, gw, k, gd = self._conv_geometry()
-        return PF.LayerDims(x.shape[0], x.shape[1], self.dim, self.heads, self.dim_head, self.slice_num, gh, gw, k, gd)
+        return PF.LayerDims(x.shape[0], x.shape[1], self.dim, self.heads, self.dim_head, self.slice_num, gh, gw, k, gd,
+                            1 if k > 0 else 0)
 
     def kernel_params(self, dtype: torch.dtype, device: torch.device) -> dict:
         """Parameters as the C ABI wants them (projection weights in `dtype`, the rest float32).  The layer's
@@ -56,8 +58,8 @@ class _SliceToContextMixin:
         if self._kernel_param_cache.get("stamp") == stamp:
             return self._kernel_param_cache["params"]
         with torch.no_grad():
-            params = {name: p.detach().to(device=device, dtype=dtype if big else torch.float32).contiguous().reshape(-1).clone()
-                      for name, p, big in named}
+            params = {name: _kernel_layout(p.detach()).to(device=device, dtype=dtype if big else torch.float32)
+                      .contiguous().reshape(-1).clone() for name, p, big in named}
             HD, D = self.heads * self.dim_head, self.dim_head
             params["qkv_project_weight"] = torch.zeros(3 * D * D, dtype=torch.float32, device=device)
             params["out_linear_weight"] = torch.zeros(self.dim * HD, dtype=dtype, device=device)

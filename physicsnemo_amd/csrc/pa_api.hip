@@ -12,6 +12,7 @@ int check_shape(int dtype, const pa_shape *s) {
   if (dtype == PA_BF16_W8 && s->conv_k != 0) return PA_ERR_UNSUPPORTED;
   if (s->B <= 0 || s->N <= 0 || s->C <= 0 || s->H <= 0 || s->D <= 0 || s->S <= 0) return PA_ERR_DIMS;
   if (s->conv_k < 0 || (s->conv_k == 0 && s->grid_d != 0)) return PA_ERR_DIMS;
+  if (s->conv_tap_major != 0 && s->conv_tap_major != 1) return PA_ERR_DIMS;
   if (s->conv_k > 0) {
     if (s->grid_h <= 0 || s->grid_w <= 0 || s->grid_d < 0) return PA_ERR_DIMS;
     if (s->grid_h * s->grid_w * (s->grid_d > 0 ? s->grid_d : 1) != s->N) return PA_ERR_DIMS;

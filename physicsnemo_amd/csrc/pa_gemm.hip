@@ -123,13 +123,18 @@ __global__ __launch_bounds__(256) void rows_gemm_mfma_kernel(GemmArgs a) {
 #pragma unroll
       for (int p = 0; p < NT; ++p) {
         const int o = o0 + r0 + 32 * p;
-        alignas(16) T e[UE];
+        if (a.w_tap_major) {  // W[o][tap][c]: the unit is contiguous, as for a Linear
+          pw[p] = u32x4{0, 0, 0, 0};
+          if (k_ok && o < a.O) pw[p] = *reinterpret_cast<const u32x4 *>(W + (int64_t)o * a.K + k);
+        } else {
+          alignas(16) T e[UE];
 #pragma unroll
-        for (int j = 0; j < UE; ++j) {
-          e[j] = T{};
-          if (k_ok && o < a.O) e[j] = W[(int64_t)o * a.K + (int64_t)(c + j) * taps + tap];
+          for (int j = 0; j < UE; ++j) {
+            e[j] = T{};
+            if (k_ok && o < a.O) e[j] = W[(int64_t)o * a.K + (int64_t)(c + j) * taps + tap];
+          }
+          pw[p] = *reinterpret_cast<const u32x4 *>(e);
         }
-        pw[p] = *reinterpret_cast<const u32x4 *>(e);
       }
     }
   };

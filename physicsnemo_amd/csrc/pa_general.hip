@@ -81,7 +81,8 @@ __global__ __launch_bounds__(256) void rows_gemm_kernel(GemmArgs a) {
           const int ii = i_ld + u - pad, jj = j_ld + v - pad, ll = l_ld + (a.gd > 0 ? z - pad : 0);
           if (m_ok && ii >= 0 && ii < a.gh && jj >= 0 && jj < a.gw && ll >= 0 && ll < gd)
             av = load_as_f32(in + ((b_ld * a.N + ((int64_t)ii * a.gw + jj) * gd + ll) * a.C + c));
-          if (o_ld < a.O) wv = load_as_f32(W + (int64_t)o_ld * a.K + (int64_t)c * taps + tap);
+          if (o_ld < a.O)
+            wv = load_as_f32(W + (int64_t)o_ld * a.K + (a.w_tap_major ? (int64_t)k : (int64_t)c * taps + tap));
         }
       }
       As[lk + q][lr] = av;
@@ -261,14 +262,14 @@ __global__ __launch_bounds__(256) void slice_softmax_plus_kernel(
 // ------------------------------------------------------------------------------------------------
 // slice_partial_kernel: grid (G chunks, B*H, output slabs).  For its chunk of points of one (b, h):
 //   partial[s, d] = sum_n w[n, s] * fx_mid[n, d]   (d < D),   partial[s, D] = sum_n w[n, s]
-// Each thread owns up to 16 outputs of a 4096-output slab and walks the chunk 32 points at a time
-// through LDS.  Sums run in a fixed order, so the result is bit-reproducible.
+// Each thread owns up to NS outputs (NS * 256 >= the outputs of the slab, at most 4096) and walks the chunk 32 points
+// at a time through LDS.  Sums run in a fixed order, so the result is bit-reproducible.
 // ------------------------------------------------------------------------------------------------
 constexpr int kAttnThreads = 1024;  // slice_combine_attn_kernel: 16 waves, one query row per wave at a time
 constexpr int kSlab = 4096;
 constexpr int kPartialTile = 32;
 
-template <typename T>
+template <typename T, int NS>
 __global__ __launch_bounds__(256) void slice_partial_kernel(const T *__restrict__ w, const T *__restrict__ fx_mid,
                                                             float *__restrict__ partials, int B, int64_t N, int H, int D,
                                                             int S, int64_t chunk) {
@@ -281,10 +282,10 @@ __global__ __launch_bounds__(256) void slice_partial_kernel(const T *__restrict_
   const int D1 = D + 1;
   const int n_out = S * D1;
   const int slab0 = blockIdx.z * kSlab;
-  int os[16], od[16];
-  float acc[16];
+  int os[NS], od[NS];
+  float acc[NS];
 #pragma unroll
-  for (int i = 0; i < 16; ++i) {
+  for (int i = 0; i < NS; ++i) {
     const int o = slab0 + t + 256 * i;
     const bool ok = o < n_out;
     os[i] = ok ? o / D1 : 0;
@@ -307,17 +308,18 @@ __global__ __launch_bounds__(256) void slice_partial_kernel(const T *__restrict_
       fl[i] = v;
     }
     __syncthreads();
+#pragma unroll(NS > 8 ? 1 : 2)  // a full unroll hoists every LDS read of the tile: 256 registers, one wave per SIMD
     for (int p = 0; p < kPartialTile; ++p) {
       const float *wp = wl + p * S;
       const float *fp = fl + p * D1;
 #pragma unroll
-      for (int i = 0; i < 16; ++i) acc[i] = fmaf(wp[os[i]], fp[od[i]], acc[i]);
+      for (int i = 0; i < NS; ++i) acc[i] = fmaf(wp[os[i]], fp[od[i]], acc[i]);
     }
     __syncthreads();
   }
   float *dst = partials + (((int64_t)g * B + b) * H + h) * n_out;
 #pragma unroll
-  for (int i = 0; i < 16; ++i) {
+  for (int i = 0; i < NS; ++i) {
     const int o = slab0 + t + 256 * i;
     if (o < n_out) dst[o] = acc[i];
   }
@@ -749,6 +751,7 @@ int project_inputs(int dtype, const pa_shape &s, const pa_params &p, const void 
   a.gw = (int)s.grid_w;
   a.ks = (int)s.conv_k;
   a.gd = (int)s.grid_d;
+  a.w_tap_major = (int)s.conv_tap_major;
   a.K = s.conv_k > 0 ? (int)(s.conv_k * s.conv_k * (s.grid_d > 0 ? s.conv_k : 1) * s.C) : (int)s.C;
   const int nsets = fx_mid ? 2 : 1;  // Transolver++ has a single projection
   return dtype == PA_F32 ? launch_gemm<float, float>(a, nsets, st) : launch_gemm<bf16, bf16>(a, nsets, st);
@@ -772,6 +775,7 @@ int rows_gemm(int dtype, const pa_shape &grid, int64_t c_in, int64_t c_out, cons
   a.gw = (int)grid.grid_w;
   a.ks = (int)grid.conv_k;
   a.gd = (int)grid.grid_d;
+  a.w_tap_major = (int)grid.conv_tap_major;
   a.K = grid.conv_k > 0 ? (int)(grid.conv_k * grid.conv_k * (grid.grid_d > 0 ? grid.conv_k : 1) * c_in) : (int)c_in;
   return dtype == PA_F32 ? launch_gemm<float, float>(a, 1, st) : launch_gemm<bf16, bf16>(a, 1, st);
 }
@@ -877,12 +881,19 @@ static int slice_partial_t(const pa_shape &s, const void *w, const void *fx_mid,
   const int64_t chunk = (s.N + G - 1) / G;
   const int n_out = (int)(s.S * (s.D + 1));
   const size_t lds = (size_t)(kPartialTile * s.S + kPartialTile * (s.D + 1)) * 4;
-  int rc = allow_dynamic_lds(slice_partial_kernel<T>, lds);
-  if (rc) return rc;
   dim3 grid((unsigned)G, (unsigned)(s.B * s.H), (unsigned)((n_out + kSlab - 1) / kSlab));
-  hipLaunchKernelGGL((slice_partial_kernel<T>), grid, dim3(256), lds, st, static_cast<const T *>(w),
-                     static_cast<const T *>(fx_mid), partials, (int)s.B, s.N, (int)s.H, (int)s.D, (int)s.S, chunk);
-  return launch_status();
+  const int per_thread = ((n_out < kSlab ? n_out : kSlab) + 255) / 256;
+  auto launch = [&](auto kernel) {
+    int rc = allow_dynamic_lds(kernel, lds);
+    if (rc) return rc;
+    hipLaunchKernelGGL(kernel, grid, dim3(256), lds, st, static_cast<const T *>(w), static_cast<const T *>(fx_mid),
+                       partials, (int)s.B, s.N, (int)s.H, (int)s.D, (int)s.S, chunk);
+    return launch_status();
+  };
+  if (per_thread <= 2) return launch(slice_partial_kernel<T, 2>);
+  if (per_thread <= 4) return launch(slice_partial_kernel<T, 4>);
+  if (per_thread <= 8) return launch(slice_partial_kernel<T, 8>);
+  return launch(slice_partial_kernel<T, 16>);
 }
 
 // `partials` holds G partial sums followed by one spare slot (index G) that receives their fixed-order total.

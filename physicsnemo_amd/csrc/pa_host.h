@@ -44,6 +44,7 @@ struct GemmArgs {
   int K, O;    // reduction length, output columns
   int C, N, gh, gw, ks;  // conv geometry (ks = 0: linear)
   int gd;                // depth of a 3-D grid (0: 2-D)
+  int w_tap_major;       // conv weights as (O, taps, C) (= the reduction order k = tap * C + c) instead of (O, C, taps)
   // MFMA kernel only, bf16, Linear, O = 32 * pack_heads: pack_tpb > 0 walks the rows batch by batch in tiles of 32
   // points (pack_tpb tiles per batch, the last one padded) and also writes each (tile, head) block of the result in
   // the packed operand layout of the MFMA slice kernels (fx_pack).  out[z] may then be NULL.

@@ -25,6 +25,7 @@ class LayerDims(NamedTuple):
     grid_w: int = 0
     conv_k: int = 0
     grid_d: int = 0
+    conv_tap_major: int = 0  # 1: convolution weights are laid out (c_out, k, k[, k], c_in) instead of torch's order
 
     def c(self) -> _lib.PaShape:
         return _lib.PaShape(*self)

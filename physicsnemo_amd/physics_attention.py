@@ -25,6 +25,12 @@ __all__ = ["PhysicsAttentionBase", "PhysicsAttentionIrregularMesh", "PhysicsAtte
            "PhysicsAttentionStructuredMesh3D"]
 
 
+def _kernel_layout(p: torch.Tensor) -> torch.Tensor:
+    """Convolution weights (O, C, k, k[, k]) -> tap-major (O, k, k[, k], C), the order in which the implicit GEMM
+    walks its reduction index (`conv_tap_major` of the shape); everything else unchanged."""
+    return p.movedim(1, -1) if p.ndim > 2 else p
+
+
 class PhysicsAttentionBase(nn.Module):
     """Parameters shared by the variants plus the HIP forward (reference base class: :262-327, :501-558)."""
 
@@ -70,7 +76,8 @@ class PhysicsAttentionBase(nn.Module):
 
     def layer_dims(self, x: torch.Tensor) -> PF.LayerDims:
         gh, gw, k, gd = self._conv_geometry()
-        return PF.LayerDims(x.shape[0], x.shape[1], self.dim, self.heads, self.dim_head, self.slice_num, gh, gw, k, gd)
+        return PF.LayerDims(x.shape[0], x.shape[1], self.dim, self.heads, self.dim_head, self.slice_num, gh, gw, k, gd,
+                            1 if k > 0 else 0)  # kernel_params() hands convolution weights over tap-major
 
     def kernel_params(self, dtype: torch.dtype, device: torch.device) -> dict:
         """Parameters as the C ABI wants them: the three large weights in ``dtype``, everything else float32,
@@ -102,7 +109,8 @@ class PhysicsAttentionBase(nn.Module):
             return self._kernel_param_cache["params"]
         with torch.no_grad():
             params = {
-                name: p.detach().to(device=device, dtype=dtype if big else torch.float32).contiguous().reshape(-1).clone()
+                name: _kernel_layout(p.detach()).to(device=device, dtype=dtype if big else torch.float32)
+                .contiguous().reshape(-1).clone()
                 for name, p, big in named
             }
             if fp8:
