@@ -174,8 +174,8 @@ def time_training_step(points, C, S, reps=3):
 def time_variants(points, C, S, reps=5):
     """The neighbouring layer variants at the layer workload's size where they fit, each forward (no_grad) and, where
     served, forward + backward: Transolver++ (general kernels), the structured-3D layer (implicit-GEMM projections +
-    general stages), a GALE layer with a projected context (MFMA kernels + the cross-attention stage) and the context
-    projector itself."""
+    general stages), a GALE layer with a projected context (MFMA kernels + the cross-attention stage), the context
+    projector itself and a FLARE layer."""
     import torch
 
     import physicsnemo_amd as pn
@@ -232,6 +232,12 @@ def time_variants(points, C, S, reps=5):
     entry(f"Transolver++ layer bf16 (general kernels), C={C}, S={S}", pts, fwd,
           timed(train_step(plus, lambda: plus(xpg), xpg), 2))
     del xp, xpg
+    # FLARE (general kernels + two composed row GEMMs), bf16
+    flare = pn.FLARE(C, heads=H, dim_head=32, n_global_queries=S).cuda()
+    xf = torch.randn(1, pts, C, device="cuda").bfloat16()
+    with torch.no_grad():
+        entry(f"FLARE layer bf16 (general kernels), C={C}, {S} global queries", pts, timed(lambda: flare(xf), 3))
+    del xf
     # structured 3-D, 64^3 grid, Conv3d k=3 projections
     g = 64
     s3 = pn.PhysicsAttentionStructuredMesh3D(C, (g, g, g), heads=H, dim_head=32, slice_num=S, kernel=3,

@@ -251,6 +251,20 @@ int pa_slice_cross_attention_mix(const pa_shape *shape, const pa_gale_params *ga
                                  int64_t context_dim, const float *slice_token, const float *self_out_slice_token,
                                  const float *context, float *out_slice_token, void *tokp, void *stream);
 
+/* ---- FLARE attention (physicsnemo/nn/module/flare_attention.py:38-72, :195-255) ------------------
+ * y = softmax_s(A) (softmax_n(A)^T v) with the scores A[b,n,h,s] = k[b,n,h,:] . q_global[h,s,:], S = number of global
+ * queries.  A (B,N,H,S) and v (B,N,H*D) come from pa_rows_gemm (the caller folds in_project_x, self_k / self_v and
+ * q_global into two weight matrices); then
+ *   pa_flare_column_weights  weights = exp(A - max_n A)          (column_max (B,H,S) float32 is an output as well;
+ *                            partials: pa_flare_column_max_chunks(shape) * B*H*S float32 of scratch)
+ *   pa_slice_reduce(weights, v)  ->  z = slice_token * slice_norm / (slice_norm - 1e-2)     (the first attention pass)
+ *   pa_flare_softmax_rows    A <- softmax_s(A) in place
+ *   pa_deslice_project(A, z) ->  out_linear(y)                                              (the second pass) */
+int64_t pa_flare_column_max_chunks(const pa_shape *shape);
+int pa_flare_column_weights(int dtype, const pa_shape *shape, const void *scores, float *partials, float *column_max,
+                            void *weights, void *stream);
+int pa_flare_softmax_rows(int dtype, const pa_shape *shape, void *scores, void *stream);
+
 /* Attended slice tokens (B,H,S,32) float32 computed by the caller (e.g. a GALE token stage under autograd) -> the
  * PA_BUF_TOKP operands of pa_mfma_deslice_project, which pa_mfma_combine_attention otherwise writes
  * (shapes with pa_query_path() == 1). */

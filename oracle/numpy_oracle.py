@@ -176,6 +176,26 @@ def gale_blend(p, tok, self_out, context):
     return gelu_erf(np.einsum("bhsk,ek->bhse", cat, _f64(p["concat_project.0.weight"])) + _f64(p["concat_project.0.bias"]))
 
 
+def flare_forward(p, x, heads, dim_head):
+    """FLARE layer in float64 (flare_attention.py:38-72, :222-255): scores A = k G^T with scale 1, softmax over the
+    points for the gather, softmax over the global queries for the hand-back."""
+    x = _f64(x)
+    B, N, C = x.shape
+    H, D = heads, dim_head
+    xm = (np.einsum("bnc,oc->bno", x, _f64(p["in_project_x.weight"])) + _f64(p["in_project_x.bias"])).reshape(B, N, H, D)
+    k = np.einsum("bnhd,ed->bnhe", xm, _f64(p["self_k.weight"])) + _f64(p["self_k.bias"])
+    v = np.einsum("bnhd,ed->bnhe", xm, _f64(p["self_v.weight"])) + _f64(p["self_v.bias"])
+    g = _f64(p["q_global"])[0]  # (H, S, D)
+    a = np.einsum("bnhe,hse->bnhs", k, g)
+    col = np.exp(a - a.max(axis=1, keepdims=True))
+    col = col / col.sum(axis=1, keepdims=True)          # softmax over the points, per (b, h, s)
+    z = np.einsum("bnhs,bnhe->bhse", col, v)
+    row = np.exp(a - a.max(axis=-1, keepdims=True))
+    row = row / row.sum(axis=-1, keepdims=True)         # softmax over the global queries, per (b, n, h)
+    y = np.einsum("bnhs,bhse->bnhe", row, z).reshape(B, N, H * D)
+    return np.einsum("bnk,ok->bno", y, _f64(p["out_linear.weight"])) + _f64(p["out_linear.bias"])
+
+
 def layer_norm(x, gamma, beta, eps=1e-5):
     """Biased-variance LayerNorm over the last axis (torch.nn.LayerNorm default eps; transolver.py:210)."""
     x = _f64(x)

@@ -332,6 +332,37 @@ class OracleGALEStructuredMesh2D(_GALECore, OraclePhysicsAttentionStructuredMesh
         self._init_cross(dim_head, context_dim, state_mixing_mode)
 
 
+# --------------------------------------------------------------------------- FLARE (flare_attention.py)
+def flare_self_attention(x_mid, q_global, self_k, self_v, scale=1.0):
+    """Two-pass attention through the learned global queries (flare_attention.py:38-72): x_mid (B,H,N,D),
+    q_global (1,H,S,D); z = SDPA(G, k, v) gathers from the points, SDPA(k, G, z) hands back to them; scale 1."""
+    g = q_global.to(dtype=x_mid.dtype).expand(x_mid.shape[0], -1, -1, -1)
+    k, v = self_k(x_mid), self_v(x_mid)
+    z = F.scaled_dot_product_attention(g, k, v, scale=scale)
+    return F.scaled_dot_product_attention(k, g, z, scale=scale)
+
+
+class OracleFLARE(nn.Module):
+    """flare_attention.py:118-255 with use_te=False."""
+
+    def __init__(self, dim, heads=8, dim_head=64, dropout=0.0, n_global_queries=64):
+        super().__init__()
+        self.dim, self.heads, self.dim_head = dim, heads, dim_head
+        self.scale = 1.0
+        self.q_global = nn.Parameter(torch.randn(1, heads, n_global_queries, dim_head))
+        self.in_project_x = nn.Linear(dim, heads * dim_head)
+        self.self_k = nn.Linear(dim_head, dim_head)
+        self.self_v = nn.Linear(dim_head, dim_head)
+        self.out_linear = nn.Linear(heads * dim_head, dim)
+        self.out_dropout = nn.Dropout(dropout)
+
+    def forward(self, x):
+        x_mid = split_heads(self.in_project_x(x), self.heads, self.dim_head).permute(0, 2, 1, 3)  # (B, H, N, D)
+        y = flare_self_attention(x_mid, self.q_global, self.self_k, self.self_v, self.scale)
+        out_x = y.permute(0, 2, 1, 3).reshape(x.shape[0], x.shape[1], self.heads * self.dim_head)
+        return self.out_dropout(self.out_linear(out_x))
+
+
 class _ProjectorCore(nn.Module):
     """Slice components and forward of the GeoTransolver context projectors
     (physicsnemo/models/geotransolver/context_projector.py:108-187, :338-378): the encoding half of the layer; returns

@@ -24,7 +24,7 @@ EXPORTED = [
     "pa_rows_gemm", "pa_slice_weighted_sum", "pa_backward_query", "pa_backward_point_tiles",
     "pa_slice_attention_backward", "pa_slice_softmax_backward", "pa_slice_softmax_plus",
     "pa_backward_point_tiles_plus", "pa_slice_softmax_plus_backward", "pa_slice_cross_attention_mix",
-    "pa_mfma_pack_tokens",
+    "pa_mfma_pack_tokens", "pa_flare_column_max_chunks", "pa_flare_column_weights", "pa_flare_softmax_rows",
     "pa_mfma_backward_query", "pa_rows_gemm_packed", "pa_mfma_slice_weighted_sum", "pa_mfma_deslice",
     "pa_mfma_backward_tables_bytes", "pa_mfma_backward_groups", "pa_mfma_slice_softmax_backward",
     "pa_cols_gemm_chunks", "pa_cols_gemm", "pa_residual_layernorm",
@@ -147,6 +147,12 @@ def load() -> ctypes.CDLL:
     lib.pa_slice_cross_attention_mix.argtypes = [ps, POINTER(PaGaleParams), c_int64, c_int64] + [c_void_p] * 6
     lib.pa_mfma_pack_tokens.restype = c_int
     lib.pa_mfma_pack_tokens.argtypes = [ps] + [c_void_p] * 3
+    lib.pa_flare_column_max_chunks.restype = c_int64
+    lib.pa_flare_column_max_chunks.argtypes = [ps]
+    lib.pa_flare_column_weights.restype = c_int
+    lib.pa_flare_column_weights.argtypes = [c_int, ps] + [c_void_p] * 5
+    lib.pa_flare_softmax_rows.restype = c_int
+    lib.pa_flare_softmax_rows.argtypes = [c_int, ps, c_void_p, c_void_p]
     lib.pa_mfma_backward_query.restype = c_int
     lib.pa_mfma_backward_query.argtypes = [ps]
     lib.pa_rows_gemm_packed.restype = c_int

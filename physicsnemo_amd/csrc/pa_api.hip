@@ -459,6 +459,31 @@ int pa_slice_cross_attention_mix(const pa_shape *shape, const pa_gale_params *ga
                                    context, out_slice_token, tokp, static_cast<hipStream_t>(stream));
 }
 
+int64_t pa_flare_column_max_chunks(const pa_shape *shape) {
+  int rc = check_shape(PA_F32, shape);
+  if (rc) return rc;
+  return pa::flare::column_max_chunks(*shape);
+}
+
+int pa_flare_column_weights(int dtype, const pa_shape *shape, const void *scores, float *partials, float *column_max,
+                            void *weights, void *stream) {
+  int rc = check_shape(dtype, shape);
+  if (rc) return rc;
+  if (dtype == PA_BF16_W8) return PA_ERR_UNSUPPORTED;
+  if (!scores || !partials || !column_max || !weights) return PA_ERR_NULL;
+  if (shape->B > 65535) return PA_ERR_UNSUPPORTED;
+  return pa::flare::column_weights(dtype, *shape, scores, partials, column_max, weights,
+                                   static_cast<hipStream_t>(stream));
+}
+
+int pa_flare_softmax_rows(int dtype, const pa_shape *shape, void *scores, void *stream) {
+  int rc = check_shape(dtype, shape);
+  if (rc) return rc;
+  if (dtype == PA_BF16_W8) return PA_ERR_UNSUPPORTED;
+  if (!scores) return PA_ERR_NULL;
+  return pa::flare::softmax_rows(dtype, *shape, scores, static_cast<hipStream_t>(stream));
+}
+
 int pa_mfma_pack_tokens(const pa_shape *shape, const float *out_slice_token, void *tokp, void *stream) {
   int rc = check_shape(PA_BF16, shape);
   if (rc) return rc;

@@ -1,0 +1,127 @@
+// FLARE attention (physicsnemo/nn/module/flare_attention.py:38-72, :195-255): low-rank attention through S learned global
+// queries per head.  With the scores A[b,n,h,s] = k[b,n,h,:] . q_global[h,s,:] (scale 1) the two passes are
+//   z[b,h,s,:] = sum_n softmax_n(A[b,:,h,s])[n] v[b,n,h,:]       (the queries gather from all points)
+//   y[b,n,h,:] = sum_s softmax_s(A[b,n,h,:])[s] z[b,h,s,:]       (every point reads the S summaries back)
+// which is the slice aggregation and the deslice of the PhysicsAttention layer with two different normalisations of
+// the same score matrix.  The scores and v come from the row GEMM kernels (the caller folds in_project_x, self_k /
+// self_v and q_global into two weight matrices); this file holds what is particular to FLARE:
+//   column_max_kernel(s)     m[b,h,s] = max_n A[b,n,h,s]                     two passes, like the slice aggregation
+//   column_weights_kernel    wc = exp(A - m)                                   -> pa_slice_reduce(wc, v) gives z
+//   softmax_rows_kernel      A <- softmax_s(A) in place                        -> pa_deslice_project(A, z) gives y
+// fp32 arithmetic, fp32 or bf16 storage, natural layouts.
+#include "pa_common.h"
+#include "pa_host.h"
+
+namespace pa {
+namespace flare {
+
+constexpr int kChunkRows = 256;  // points per workgroup of the first column-max pass
+
+// grid (chunks, B).  Workgroup (g, b): column maxima of rows [g*256, g*256+256) of batch b over all H*S columns.
+template <typename T>
+__global__ __launch_bounds__(256) void column_max_partial_kernel(const T *__restrict__ a, float *__restrict__ partial,
+                                                                 int64_t N, int HS) {
+  const int g = blockIdx.x, b = blockIdx.y;
+  const int64_t n0 = (int64_t)g * kChunkRows;
+  const int rows = (int)min((int64_t)kChunkRows, N - n0);
+  const T *src = a + ((int64_t)b * N + n0) * HS;
+  for (int c = threadIdx.x; c < HS; c += 256) {  // consecutive threads <-> consecutive columns: coalesced rows
+    float m = -INFINITY;
+    for (int r = 0; r < rows; ++r) m = fmaxf(m, load_as_f32(src + (int64_t)r * HS + c));
+    partial[((int64_t)g * gridDim.y + b) * HS + c] = m;
+  }
+}
+
+// grid (ceil(B*H*S / 256)): maximum over the G partials.
+__global__ __launch_bounds__(256) void column_max_combine_kernel(const float *__restrict__ partial, int G, int64_t BHS,
+                                                                 float *__restrict__ colmax) {
+  const int64_t o = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (o >= BHS) return;
+  float m = -INFINITY;
+  for (int g = 0; g < G; ++g) m = fmaxf(m, partial[(int64_t)g * BHS + o]);
+  colmax[o] = m;
+}
+
+// wc[b,n,c] = exp(A[b,n,c] - m[b,c]), c = h*S + s; element-wise over (B*N, H*S).
+template <typename T>
+__global__ __launch_bounds__(256) void column_weights_kernel(const T *__restrict__ a, const float *__restrict__ colmax,
+                                                             T *__restrict__ wc, int64_t N, int HS, int64_t total) {
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    const int64_t row = i / HS;
+    const int c = (int)(i - row * HS);
+    const int64_t b = row / N;
+    store_from_f32(wc + i, expf(load_as_f32(a + i) - colmax[b * HS + c]));
+  }
+}
+
+// In-place softmax over the S entries of every (point, head) row; L lanes share a row (L a power of two <= 64).
+template <typename T, int L>
+__global__ __launch_bounds__(256) void softmax_rows_kernel(T *__restrict__ a, int64_t rows, int S) {
+  const int per_wg = 256 / L;
+  const int sub = threadIdx.x / L, l = threadIdx.x % L;
+  for (int64_t row = (int64_t)blockIdx.x * per_wg + sub; row < rows; row += (int64_t)gridDim.x * per_wg) {
+    T *p = a + row * S;
+    float mx = -INFINITY;
+    for (int s = l; s < S; s += L) mx = fmaxf(mx, load_as_f32(p + s));
+#pragma unroll
+    for (int off = L >> 1; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+    float sum = 0.f;
+    for (int s = l; s < S; s += L) sum += expf(load_as_f32(p + s) - mx);
+#pragma unroll
+    for (int off = L >> 1; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+    const float inv = 1.f / sum;
+    for (int s = l; s < S; s += L) store_from_f32(p + s, expf(load_as_f32(p + s) - mx) * inv);
+  }
+}
+
+int64_t column_max_chunks(const pa_shape &s) { return (s.N + kChunkRows - 1) / kChunkRows; }
+
+template <typename T>
+static int column_weights_t(const pa_shape &s, const void *a, float *partial, float *colmax, void *wc, hipStream_t st) {
+  const int HS = (int)(s.H * s.S);
+  const int64_t G = column_max_chunks(s), BHS = s.B * HS, total = s.B * s.N * HS;
+  hipLaunchKernelGGL((column_max_partial_kernel<T>), dim3((unsigned)G, (unsigned)s.B), dim3(256), 0, st,
+                     static_cast<const T *>(a), partial, s.N, HS);
+  int rc = launch_status();
+  if (rc) return rc;
+  hipLaunchKernelGGL(column_max_combine_kernel, dim3((unsigned)((BHS + 255) / 256)), dim3(256), 0, st, partial, (int)G,
+                     BHS, colmax);
+  rc = launch_status();
+  if (rc) return rc;
+  int64_t blocks = (total + 255) / 256;
+  if (blocks > 8192) blocks = 8192;
+  hipLaunchKernelGGL((column_weights_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, st, static_cast<const T *>(a),
+                     colmax, static_cast<T *>(wc), s.N, HS, total);
+  return launch_status();
+}
+
+int column_weights(int dtype, const pa_shape &s, const void *a, float *partial, float *colmax, void *wc,
+                   hipStream_t st) {
+  return dtype == PA_F32 ? column_weights_t<float>(s, a, partial, colmax, wc, st)
+                         : column_weights_t<bf16>(s, a, partial, colmax, wc, st);
+}
+
+template <typename T, int L>
+static int softmax_rows_l(const pa_shape &s, void *a, hipStream_t st) {
+  const int64_t rows = s.B * s.N * s.H;
+  int64_t blocks = (rows + (256 / L) - 1) / (256 / L);
+  if (blocks > 16384) blocks = 16384;
+  hipLaunchKernelGGL((softmax_rows_kernel<T, L>), dim3((unsigned)blocks), dim3(256), 0, st, static_cast<T *>(a), rows,
+                     (int)s.S);
+  return launch_status();
+}
+
+template <typename T>
+static int softmax_rows_t(const pa_shape &s, void *a, hipStream_t st) {
+  if (s.S <= 8) return softmax_rows_l<T, 8>(s, a, st);
+  if (s.S <= 16) return softmax_rows_l<T, 16>(s, a, st);
+  if (s.S <= 32) return softmax_rows_l<T, 32>(s, a, st);
+  return softmax_rows_l<T, 64>(s, a, st);
+}
+
+int softmax_rows(int dtype, const pa_shape &s, void *a, hipStream_t st) {
+  return dtype == PA_F32 ? softmax_rows_t<float>(s, a, st) : softmax_rows_t<bf16>(s, a, st);
+}
+
+}  // namespace flare
+}  // namespace pa

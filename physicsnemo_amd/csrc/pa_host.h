@@ -105,6 +105,13 @@ int slice_softmax_plus(int dtype, const pa_shape &s, const pa_params &p, const p
                        float *dT_part, hipStream_t st);
 }  // namespace backward
 
+namespace flare {
+int64_t column_max_chunks(const pa_shape &s);
+int column_weights(int dtype, const pa_shape &s, const void *a, float *partial, float *colmax, void *wc,
+                   hipStream_t st);
+int softmax_rows(int dtype, const pa_shape &s, void *a, hipStream_t st);
+}  // namespace flare
+
 namespace gale {
 size_t lds_bytes(const pa_shape &s, int64_t Sc, int64_t Dc);
 int pack_tokens(const pa_shape &s, const float *out_token, void *tokp, hipStream_t st);

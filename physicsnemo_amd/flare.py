@@ -1,0 +1,103 @@
+"""FLARE (Fast Low-rank Attention Routing Engine) attention layer on the HIP kernels.
+
+Mirrors ``physicsnemo/nn/module/flare_attention.py``: FLARE:118-255, ``_flare_self_attention``:38-72.  Same constructor
+arguments, parameter names and ``forward(x) -> (B, N, C)``, so a reference ``state_dict`` loads unchanged.
+
+The layer is two attention passes through S learned global queries per head, with scores
+``A[b,n,h,s] = k[b,n,h,:] . q_global[h,s,:]`` (scale 1): the queries gather ``z = softmax_n(A)^T v`` from all points,
+then every point reads ``y = softmax_s(A) z`` back.  That is the slice aggregation and the deslice of the
+PhysicsAttention layer with two normalisations of one score matrix, so it runs on the same kernels:
+
+  A, v   two row GEMMs straight from x: in_project_x, self_k / self_v and q_global are linear maps applied one after
+         the other, composed once per parameter set into two weight matrices (H*S x C and H*D x C)
+  z      exp(A - max_n A) (``pa_flare_column_weights``), then the slice aggregation kernels
+  y      row softmax of A in place (``pa_flare_softmax_rows``), then deslice + out_linear
+
+Forward only: the backward kernels do not cover this layer.  ``use_te`` is accepted and ignored.
+"""
+from __future__ import annotations
+
+import torch
+import torch.nn as nn
+
+from . import functional as PF
+
+
+class FLARE(nn.Module):
+    def __init__(self, dim: int, heads: int = 8, dim_head: int = 64, dropout: float = 0.0,
+                 n_global_queries: int = 64, use_te: bool = False):
+        super().__init__()
+        self.use_te = use_te
+        self.dim, self.heads, self.dim_head, self.n_global_queries = dim, heads, dim_head, n_global_queries
+        self.scale = 1.0
+        inner_dim = dim_head * heads
+        # registration order follows the reference so state_dict order and RNG draws agree
+        self.q_global = nn.Parameter(torch.randn(1, heads, n_global_queries, dim_head))
+        self.in_project_x = nn.Linear(dim, inner_dim)
+        self.self_k = nn.Linear(dim_head, dim_head)
+        self.self_v = nn.Linear(dim_head, dim_head)
+        self.out_linear = nn.Linear(inner_dim, dim)
+        self.out_dropout = nn.Dropout(dropout)
+        self._cache: dict = {}
+
+    def kernel_params(self, dtype: torch.dtype, device: torch.device) -> dict:
+        """The composed GEMM weights (in `dtype`; biases float32) and out_linear, cached per parameter version."""
+        ps = [self.q_global, self.in_project_x.weight, self.in_project_x.bias, self.self_k.weight, self.self_k.bias,
+              self.self_v.weight, self.self_v.bias, self.out_linear.weight, self.out_linear.bias]
+        stamp = (dtype, device) + tuple((p.data_ptr(), p._version) for p in ps)
+        if self._cache.get("stamp") == stamp:
+            return self._cache["params"]
+        H, D, S, C = self.heads, self.dim_head, self.n_global_queries, self.dim
+        with torch.no_grad():
+            g, wx, bx, wk, bk, wv, bv, wo, bo = (p.detach().to(device=device, dtype=torch.float64) for p in ps)
+            wx_h, bx_h = wx.view(H, D, C), bx.view(H, D)
+            gk = g.view(H, S, D) @ wk                                     # (H, S, D): q_global . W_k
+            w_a = torch.einsum("hsd,hdc->hsc", gk, wx_h).reshape(H * S, C)
+            b_a = torch.einsum("hsd,hd->hs", gk, bx_h) + g.view(H, S, D) @ bk
+            w_v = torch.einsum("ed,hdc->hec", wv, wx_h).reshape(H * D, C)
+            b_v = torch.einsum("ed,hd->he", wv, bx_h) + bv
+            params = {
+                "scores_weight": w_a.to(dtype).contiguous(), "scores_bias": b_a.reshape(-1).float().contiguous(),
+                "values_weight": w_v.to(dtype).contiguous(), "values_bias": b_v.reshape(-1).float().contiguous(),
+                "out_linear_weight": wo.to(dtype).contiguous().reshape(-1),
+                "out_linear_bias": bo.float().contiguous(),
+            }
+        self._cache = {"stamp": stamp, "params": params}
+        return params
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        if x.ndim != 3:
+            raise ValueError(f"Expected 3D input tensor (B, N, C), got {x.ndim}D tensor with shape {tuple(x.shape)}")
+        if x.shape[-1] != self.dim:
+            raise ValueError(f"Expected input feature dimension {self.dim}, got {x.shape[-1]}")
+        if not x.is_cuda:
+            raise RuntimeError("physicsnemo_amd FLARE runs on GPU tensors only (no CPU fallback)")
+        if torch.is_grad_enabled() and (x.requires_grad or any(p.requires_grad for p in self.parameters())):
+            raise NotImplementedError("the backward kernels do not cover FLARE; run under torch.no_grad()")
+        if self.training and self.out_dropout.p > 0:
+            raise NotImplementedError("dropout > 0 in training mode is not served by the HIP layer")
+        out_dtype = None
+        if torch.is_autocast_enabled("cuda"):
+            ac = torch.get_autocast_dtype("cuda")
+            if ac == torch.float16:
+                out_dtype, ac = torch.float16, torch.float32
+            x = x.to(ac)
+        elif x.dtype == torch.float16:
+            out_dtype, x = torch.float16, x.float()
+        if x.dtype not in (torch.float32, torch.bfloat16):
+            raise TypeError(f"expected float32 or bfloat16 input, got {x.dtype}")
+        x = x.contiguous()
+        B, N, C = x.shape
+        H, D, S = self.heads, self.dim_head, self.n_global_queries
+        dims = PF.LayerDims(B, N, C, H, D, S)
+        p = self.kernel_params(x.dtype, x.device)
+        scores = PF.rows_gemm(x, p["scores_weight"], p["scores_bias"], dims, C, H * S).view(B, N, H, S)
+        values = PF.rows_gemm(x, p["values_weight"], p["values_bias"], dims, C, H * D)
+        weights, _ = PF.flare_column_weights(scores, dims)
+        tok, norm = PF.slice_reduce(weights, values, dims)
+        # the aggregation kernel divides by (sum + 1e-2), the slice norm of PhysicsAttention; FLARE's softmax has no such
+        # term (the sum is >= 1: the column maximum contributes exp(0))
+        z = (tok * (norm / (norm - 1e-2)).unsqueeze(-1)).contiguous()
+        PF.flare_softmax_rows_(scores, dims)
+        y = PF.deslice_project(scores, z, p, dims)
+        return y if out_dtype is None else y.to(out_dtype)

@@ -536,3 +536,30 @@ def slice_cross_attention_mix(tok, self_out, context, gale_params: dict, dims: L
         context.data_ptr(), out.data_ptr(), _lib.ptr(tokp), _lib.current_stream_ptr(tok.device)),
         "pa_slice_cross_attention_mix")
     return out
+
+
+def flare_column_weights(scores, dims: LayerDims):
+    """FLARE first pass weights: exp(A - max_n A) for the scores A (B,N,H,S); returns (weights like A, column max
+    (B,H,S) float32)."""
+    _need_cuda(scores)
+    lib = _lib.load()
+    shape = dims.c()
+    chunks = lib.pa_flare_column_max_chunks(byref(shape))
+    if chunks < 0:
+        _lib.check(int(chunks), "pa_flare_column_max_chunks")
+    f32 = dict(dtype=torch.float32, device=scores.device)
+    partials = torch.empty(int(chunks) * dims.B * dims.H * dims.S, **f32)
+    colmax = torch.empty(dims.B, dims.H, dims.S, **f32)
+    weights = torch.empty_like(scores)
+    _lib.check(lib.pa_flare_column_weights(_lib.dtype_code(scores.dtype), byref(shape), scores.data_ptr(),
+                                           partials.data_ptr(), colmax.data_ptr(), weights.data_ptr(),
+                                           _lib.current_stream_ptr(scores.device)), "pa_flare_column_weights")
+    return weights, colmax
+
+
+def flare_softmax_rows_(scores, dims: LayerDims):
+    """In-place softmax over the last axis of the scores (B,N,H,S)."""
+    _need_cuda(scores)
+    _lib.check(_lib.load().pa_flare_softmax_rows(_lib.dtype_code(scores.dtype), byref(dims.c()), scores.data_ptr(),
+                                                 _lib.current_stream_ptr(scores.device)), "pa_flare_softmax_rows")
+    return scores

@@ -1,0 +1,79 @@
+"""FLARE attention layer on the HIP kernels against the oracle.  Bars: fp32 rtol 1e-4 with atol = 1e-4 * max|ref|;
+bf16 rel-L2 <= 1e-2 against the fp32 oracle."""
+import pytest
+import torch
+
+from oracle import torch_oracle as to
+import physicsnemo_amd as pn
+from physicsnemo_amd import functional as PF
+from gpu_util import announce, assert_fp32_close, assert_rel_l2
+
+pytestmark = pytest.mark.gpu
+
+
+def _pair(dim, heads, dim_head, S, seed=0):
+    torch.manual_seed(seed)
+    ref = to.OracleFLARE(dim, heads=heads, dim_head=dim_head, n_global_queries=S)
+    hip = pn.FLARE(dim, heads=heads, dim_head=dim_head, n_global_queries=S)
+    hip.load_state_dict(ref.state_dict())
+    return ref.eval(), hip.eval().cuda()
+
+
+@pytest.mark.parametrize("dim,heads,dim_head,S,B,N", [
+    (32, 4, 8, 8, 2, 300),
+    (64, 2, 32, 64, 1, 1000),
+    (48, 3, 16, 20, 3, 77),
+    (24, 2, 8, 5, 2, 1),       # one point: both softmaxes degenerate on the point axis
+    (32, 4, 8, 1, 2, 515),     # one global query
+])
+def test_fp32_flare_matches_oracle(dim, heads, dim_head, S, B, N):
+    announce("fp32 FLARE", dim, heads, dim_head, S, B, N)
+    ref, hip = _pair(dim, heads, dim_head, S)
+    x = torch.randn(B, N, dim)
+    with torch.no_grad():
+        want = ref(x)
+        got = hip(x.cuda())
+    assert got.shape == want.shape
+    assert_fp32_close(got, want, "FLARE y")
+
+
+def test_flare_stages_against_closed_forms():
+    announce("FLARE stage kernels")
+    B, N, H, S = 2, 700, 3, 20
+    dims = PF.LayerDims(B, N, 48, H, 16, S)
+    a = torch.randn(B, N, H, S, device="cuda") * 3
+    w, colmax = PF.flare_column_weights(a, dims)
+    want_max = a.amax(dim=1)
+    assert torch.equal(colmax, want_max)
+    assert_fp32_close(w, torch.exp(a - want_max[:, None]), "exp(A - column max)")
+    rows = PF.flare_softmax_rows_(a.clone(), dims)
+    assert_fp32_close(rows, torch.softmax(a, dim=-1), "row softmax")
+
+
+@pytest.mark.parametrize("S,N", [(64, 8192), (32, 5000)])
+def test_bf16_flare(S, N):
+    announce("bf16 FLARE", S, N)
+    ref, hip = _pair(256, 8, 32, S)
+    x = torch.randn(2, N, 256)
+    with torch.no_grad():
+        want = ref(x)
+        got = hip(x.cuda().bfloat16())
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            got_ac = hip(x.cuda())
+    assert got.dtype == torch.bfloat16 and got_ac.dtype == torch.bfloat16
+    assert_rel_l2(got, want, "bf16 FLARE y", tol=1e-2)
+    assert torch.equal(got, got_ac)
+
+
+def test_flare_errors():
+    announce("FLARE errors")
+    _, hip = _pair(32, 4, 8, 8)
+    x = torch.randn(2, 50, 32, device="cuda")
+    with pytest.raises(ValueError, match="Expected 3D input tensor"), torch.no_grad():
+        hip(x[0])
+    with pytest.raises(ValueError, match="feature dimension"), torch.no_grad():
+        hip(x[..., :16])
+    with pytest.raises(NotImplementedError):
+        hip(x)  # parameters require grad and grad mode is on
+    with pytest.raises(RuntimeError, match="GPU"), torch.no_grad():
+        hip.cpu()(x.cpu())
