@@ -137,9 +137,11 @@ typedef struct pa_plus_params {
 
 /* Stage (a2) of Transolver++: replaces in_project_slice (PA.py:537) and the plus branch of
  * _compute_slices_from_projections (PA.py:166-170).  `uniform` (B,N,H,S), activation dtype: the U[0,1) samples the
- * reference draws with torch.rand_like(logits); the kernel forms the noise -log(-log(u + 1e-8) + 1e-8) itself. */
+ * reference draws with torch.rand_like(logits); the kernel forms the noise -log(-log(u + 1e-8) + 1e-8) itself.
+ * `scratch`: NULL, or B*N*H*S elements of the activation dtype; with it the two Linears over the (point, head) rows run
+ * on the row GEMM kernels (several times faster) and only the per-row part is left to a row kernel. */
 int pa_slice_softmax_plus(int dtype, const pa_shape *shape, const pa_params *p, const pa_plus_params *plus,
-                          const void *x_mid, const void *uniform, void *w, void *stream);
+                          const void *x_mid, const void *uniform, void *w, void *scratch, void *stream);
 
 /* Stage (b): slice-token aggregation, replaces PA.py:185-203.
  *   partials: float32 scratch of pa_reduce_partial_count(shape) * B*H*S*(D+1) elements (per-chunk sums

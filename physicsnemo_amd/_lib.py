@@ -138,7 +138,7 @@ def load() -> ctypes.CDLL:
     lib.pa_slice_softmax_backward.restype = c_int
     lib.pa_slice_softmax_backward.argtypes = [c_int, ps, pp] + [c_void_p] * 11
     lib.pa_slice_softmax_plus.restype = c_int
-    lib.pa_slice_softmax_plus.argtypes = [c_int, ps, pp, POINTER(PaPlusParams)] + [c_void_p] * 4
+    lib.pa_slice_softmax_plus.argtypes = [c_int, ps, pp, POINTER(PaPlusParams)] + [c_void_p] * 5
     lib.pa_backward_point_tiles_plus.restype = c_int64
     lib.pa_backward_point_tiles_plus.argtypes = [ps]
     lib.pa_slice_softmax_plus_backward.restype = c_int

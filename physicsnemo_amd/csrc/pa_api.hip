@@ -248,7 +248,7 @@ int pa_project_inputs(int dtype, const pa_shape *shape, const pa_params *p, cons
 }
 
 int pa_slice_softmax_plus(int dtype, const pa_shape *shape, const pa_params *p, const pa_plus_params *plus,
-                          const void *x_mid, const void *uniform, void *w, void *stream) {
+                          const void *x_mid, const void *uniform, void *w, void *scratch, void *stream) {
   int rc = check_shape(dtype, shape);
   if (rc) return rc;
   if (dtype == PA_BF16_W8) return PA_ERR_UNSUPPORTED;
@@ -257,8 +257,9 @@ int pa_slice_softmax_plus(int dtype, const pa_shape *shape, const pa_params *p, 
       !plus->proj_temperature_2_bias)
     return PA_ERR_NULL;
   if (!x_mid || !uniform || !w) return PA_ERR_NULL;
-  if (!aligned16(x_mid) || !aligned16(uniform) || !aligned16(w)) return PA_ERR_ALIGN;
-  return pa::general::slice_softmax_plus(dtype, *shape, *p, *plus, x_mid, uniform, w, static_cast<hipStream_t>(stream));
+  if (!aligned16(x_mid) || !aligned16(uniform) || !aligned16(w) || !aligned16(scratch)) return PA_ERR_ALIGN;
+  return pa::general::slice_softmax_plus(dtype, *shape, *p, *plus, x_mid, uniform, w, scratch,
+                                         static_cast<hipStream_t>(stream));
 }
 
 int pa_slice_softmax(int dtype, const pa_shape *shape, const pa_params *p, const void *x_mid, void *w, void *stream) {
@@ -481,7 +482,7 @@ int pa_flare_softmax_rows(int dtype, const pa_shape *shape, void *scores, void *
   if (rc) return rc;
   if (dtype == PA_BF16_W8) return PA_ERR_UNSUPPORTED;
   if (!scores) return PA_ERR_NULL;
-  return pa::flare::softmax_rows(dtype, *shape, scores, static_cast<hipStream_t>(stream));
+  return pa::flare::softmax_rows(dtype, *shape, scores, nullptr, static_cast<hipStream_t>(stream));
 }
 
 int pa_mfma_pack_tokens(const pa_shape *shape, const float *out_slice_token, void *tokp, void *stream) {

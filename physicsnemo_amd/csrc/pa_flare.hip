@@ -55,22 +55,26 @@ __global__ __launch_bounds__(256) void column_weights_kernel(const T *__restrict
 }
 
 // In-place softmax over the S entries of every (point, head) row; L lanes share a row (L a power of two <= 64).
+// temperature != nullptr: the entries are divided by clamp(temperature[head], 0.5, 5) first (row = point * H + head),
+// which makes this the softmax of the PhysicsAttention slice weights (PA.py:172-181).
 template <typename T, int L>
-__global__ __launch_bounds__(256) void softmax_rows_kernel(T *__restrict__ a, int64_t rows, int S) {
+__global__ __launch_bounds__(256) void softmax_rows_kernel(T *__restrict__ a, int64_t rows, int S,
+                                                           const float *__restrict__ temperature, int H) {
   const int per_wg = 256 / L;
   const int sub = threadIdx.x / L, l = threadIdx.x % L;
   for (int64_t row = (int64_t)blockIdx.x * per_wg + sub; row < rows; row += (int64_t)gridDim.x * per_wg) {
     T *p = a + row * S;
+    const float inv_t = temperature ? 1.f / clamp_temperature(temperature[row % H]) : 1.f;
     float mx = -INFINITY;
-    for (int s = l; s < S; s += L) mx = fmaxf(mx, load_as_f32(p + s));
+    for (int s = l; s < S; s += L) mx = fmaxf(mx, load_as_f32(p + s) * inv_t);
 #pragma unroll
     for (int off = L >> 1; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
     float sum = 0.f;
-    for (int s = l; s < S; s += L) sum += expf(load_as_f32(p + s) - mx);
+    for (int s = l; s < S; s += L) sum += expf(load_as_f32(p + s) * inv_t - mx);
 #pragma unroll
     for (int off = L >> 1; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
     const float inv = 1.f / sum;
-    for (int s = l; s < S; s += L) store_from_f32(p + s, expf(load_as_f32(p + s) - mx) * inv);
+    for (int s = l; s < S; s += L) store_from_f32(p + s, expf(load_as_f32(p + s) * inv_t - mx) * inv);
   }
 }
 
@@ -102,25 +106,25 @@ int column_weights(int dtype, const pa_shape &s, const void *a, float *partial, 
 }
 
 template <typename T, int L>
-static int softmax_rows_l(const pa_shape &s, void *a, hipStream_t st) {
+static int softmax_rows_l(const pa_shape &s, void *a, const float *temperature, hipStream_t st) {
   const int64_t rows = s.B * s.N * s.H;
   int64_t blocks = (rows + (256 / L) - 1) / (256 / L);
   if (blocks > 16384) blocks = 16384;
   hipLaunchKernelGGL((softmax_rows_kernel<T, L>), dim3((unsigned)blocks), dim3(256), 0, st, static_cast<T *>(a), rows,
-                     (int)s.S);
+                     (int)s.S, temperature, (int)s.H);
   return launch_status();
 }
 
 template <typename T>
-static int softmax_rows_t(const pa_shape &s, void *a, hipStream_t st) {
-  if (s.S <= 8) return softmax_rows_l<T, 8>(s, a, st);
-  if (s.S <= 16) return softmax_rows_l<T, 16>(s, a, st);
-  if (s.S <= 32) return softmax_rows_l<T, 32>(s, a, st);
-  return softmax_rows_l<T, 64>(s, a, st);
+static int softmax_rows_t(const pa_shape &s, void *a, const float *temperature, hipStream_t st) {
+  if (s.S <= 8) return softmax_rows_l<T, 8>(s, a, temperature, st);
+  if (s.S <= 16) return softmax_rows_l<T, 16>(s, a, temperature, st);
+  if (s.S <= 32) return softmax_rows_l<T, 32>(s, a, temperature, st);
+  return softmax_rows_l<T, 64>(s, a, temperature, st);
 }
 
-int softmax_rows(int dtype, const pa_shape &s, void *a, hipStream_t st) {
-  return dtype == PA_F32 ? softmax_rows_t<float>(s, a, st) : softmax_rows_t<bf16>(s, a, st);
+int softmax_rows(int dtype, const pa_shape &s, void *a, const float *temperature, hipStream_t st) {
+  return dtype == PA_F32 ? softmax_rows_t<float>(s, a, temperature, st) : softmax_rows_t<bf16>(s, a, temperature, st);
 }
 
 }  // namespace flare

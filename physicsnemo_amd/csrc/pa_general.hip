@@ -4,7 +4,7 @@
 //
 // Stage map (reference lines in include/physattn.h):
 //   rows_gemm_kernel          in_project_x / in_project_fx (Linear or k x k Conv2d as implicit GEMM), out_linear
-//   slice_softmax_kernel      in_project_slice + clamp(temperature) + softmax over S
+//   rows GEMM + softmax_rows  in_project_slice, then clamp(temperature) + softmax over S in place (pa_flare.hip)
 //   slice_partial_kernel      per-chunk sums  sum_n w[n,s] * [fx_mid[n,:], 1]
 //   slice_combine_attn_kernel fixed-order combine, / (norm + 1e-2), qkv, softmax(q k^T / sqrt D) v   (LDS resident)
 //   deslice_kernel            out_x[n,h,:] = sum_s w[n,h,s] * tok'[h,s,:]
@@ -119,66 +119,6 @@ __global__ __launch_bounds__(256) void rows_gemm_kernel(GemmArgs a) {
 }
 
 // ------------------------------------------------------------------------------------------------
-// slice_softmax_kernel: R consecutive rows (points) per workgroup.
-//   logits[r,h,s] = bias[s] + sum_d x_mid[r, h*D+d] * Wslice[s, d];  w = softmax_s(logits / clamp(T_h, .5, 5))
-// LDS: x rows (head stride D+1), Wslice, logits/weights (row stride S+1).  The finished block of
-// R*H*S weights is contiguous in global memory and is written with unit stride.
-// ------------------------------------------------------------------------------------------------
-template <typename T>
-__global__ __launch_bounds__(256) void slice_softmax_kernel(const T *__restrict__ x_mid, const float *__restrict__ w_slice,
-                                                            const float *__restrict__ b_slice,
-                                                            const float *__restrict__ temperature, T *__restrict__ w_out,
-                                                            int64_t M, int H, int D, int S, int R) {
-  extern __shared__ float lds[];
-  float *xs = lds;                       // R * H * (D+1)
-  float *wsl = xs + R * H * (D + 1);     // S * D
-  float *bsl = wsl + S * D;              // S
-  float *lg = bsl + S;                   // R * H * (S+1)
-  const int t = threadIdx.x;
-  const int64_t m0 = (int64_t)blockIdx.x * R;
-  const int rows = (int)min((int64_t)R, M - m0);
-  const int HD = H * D;
-  for (int i = t; i < rows * HD; i += 256) {
-    const int r = i / HD, c = i - r * HD;
-    const int h = c / D, d = c - h * D;
-    xs[(r * H + h) * (D + 1) + d] = load_as_f32(x_mid + (m0 + r) * HD + c);
-  }
-  for (int i = t; i < S * D; i += 256) wsl[i] = w_slice[i];
-  for (int i = t; i < S; i += 256) bsl[i] = b_slice[i];
-  __syncthreads();
-  for (int pair = t; pair < rows * H; pair += 256) {
-    const int h = pair % H;
-    const float temp = clamp_temperature(temperature[h]);
-    const float *xr = xs + pair * (D + 1);
-    float *lrow = lg + pair * (S + 1);
-    float mx = -INFINITY;
-    for (int s = 0; s < S; ++s) {
-      float acc = 0.f;
-      const float *wr = wsl + s * D;
-      for (int d = 0; d < D; ++d) acc = fmaf(xr[d], wr[d], acc);
-      // the Linear output is materialised in the storage type before the division (PA.py:537,177)
-      const float z = round_to(w_out, acc + bsl[s]) / temp;
-      lrow[s] = z;
-      mx = fmaxf(mx, z);
-    }
-    float sum = 0.f;
-    for (int s = 0; s < S; ++s) {
-      const float e = expf(lrow[s] - mx);
-      lrow[s] = e;
-      sum += e;
-    }
-    const float inv = 1.f / sum;
-    for (int s = 0; s < S; ++s) lrow[s] *= inv;
-  }
-  __syncthreads();
-  const int HS = H * S;
-  for (int i = t; i < rows * HS; i += 256) {
-    const int pair = i / S, s = i - pair * S;
-    store_from_f32(w_out + m0 * HS + i, lg[pair * (S + 1) + s]);
-  }
-}
-
-// ------------------------------------------------------------------------------------------------
 // slice_softmax_plus_kernel: the Transolver++ form of slice_softmax_kernel (PA.py:166-170, gumbel_softmax.py:49-57).
 //   temp[r,h]  = max(temperature[h] + gelu(b2 + sum_s w2[s] gelu(b1[s] + x_mid[r,h,:] . w1[s,:])), 0.01)
 //   w[r,h,:]   = softmax_s((logits[r,h,s] - log(-log(u[r,h,s] + 1e-8) + 1e-8)) / temp[r,h])
@@ -260,68 +200,127 @@ __global__ __launch_bounds__(256) void slice_softmax_plus_kernel(
 }
 
 // ------------------------------------------------------------------------------------------------
+// softmax_rows_plus_kernel: the row stage of the Transolver++ slice weights when the two Linears over the
+// (point, head) rows -- the slice logits and the hidden layer gelu(b1 + W1 x_mid) of proj_temperature -- were formed by
+// the row GEMM kernels (logits in `w`, hidden in `hidden`, both (rows, S)).  L lanes share a row:
+//   temp = max(temperature[h] + gelu(b2 + sum_s w2[s] hidden[s]), 0.01);  w <- softmax_s((w + noise(u)) / temp) in place
+// ------------------------------------------------------------------------------------------------
+template <typename T, int L>
+__global__ __launch_bounds__(256) void softmax_rows_plus_kernel(T *__restrict__ w, const T *__restrict__ hidden,
+                                                                const T *__restrict__ uniform,
+                                                                const float *__restrict__ temperature,
+                                                                const float *__restrict__ pt_w2,
+                                                                const float *__restrict__ pt_b2, int64_t rows, int S,
+                                                                int H) {
+  const int per_wg = 256 / L;
+  const int sub = threadIdx.x / L, l = threadIdx.x % L;
+  for (int64_t row = (int64_t)blockIdx.x * per_wg + sub; row < rows; row += (int64_t)gridDim.x * per_wg) {
+    T *p = w + row * S;
+    const T *hp = hidden + row * S, *up = uniform + row * S;
+    float tacc = 0.f;
+    for (int s = l; s < S; s += L) tacc = fmaf(pt_w2[s], load_as_f32(hp + s), tacc);
+#pragma unroll
+    for (int off = L >> 1; off > 0; off >>= 1) tacc += __shfl_xor(tacc, off, 64);
+    const float temp = round_to(w, fmaxf(temperature[row % H] + gelu_erf(tacc + pt_b2[0]), 0.01f));
+    const float inv_t = 1.f / temp;
+    auto arg = [&](int s) {
+      return (load_as_f32(p + s) - logf(-logf(load_as_f32(up + s) + 1e-8f) + 1e-8f)) * inv_t;
+    };
+    float mx = -INFINITY;
+    for (int s = l; s < S; s += L) mx = fmaxf(mx, arg(s));
+#pragma unroll
+    for (int off = L >> 1; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+    float sum = 0.f;
+    for (int s = l; s < S; s += L) sum += expf(arg(s) - mx);
+#pragma unroll
+    for (int off = L >> 1; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+    const float inv = 1.f / sum;
+    for (int s = l; s < S; s += L) store_from_f32(p + s, expf(arg(s) - mx) * inv);
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
 // slice_partial_kernel: grid (G chunks, B*H, output slabs).  For its chunk of points of one (b, h):
 //   partial[s, d] = sum_n w[n, s] * fx_mid[n, d]   (d < D),   partial[s, D] = sum_n w[n, s]
-// Each thread owns up to NS outputs (NS * 256 >= the outputs of the slab, at most 4096) and walks the chunk 32 points
-// at a time through LDS.  Sums run in a fixed order, so the result is bit-reproducible.
+// The (S x D+1) output is cut into 4 x 4 register tiles; a thread owns NS of them (tile t + 256 i of its slab of
+// 256 NS tiles) and walks the chunk 32 points at a time through LDS: per point and tile two 16-byte LDS reads
+// (4 slice weights, 4 features) feed 16 FMAs.  LDS rows are padded to multiples of four (zeros; column D of the
+// feature rows holds 1 for the count).  Sums run in a fixed order, so the result is bit-reproducible.
 // ------------------------------------------------------------------------------------------------
 constexpr int kAttnThreads = 1024;  // slice_combine_attn_kernel: 16 waves, one query row per wave at a time
-constexpr int kSlab = 4096;
 constexpr int kPartialTile = 32;
+constexpr int kPartialMaxNS = 4;
 
 template <typename T, int NS>
 __global__ __launch_bounds__(256) void slice_partial_kernel(const T *__restrict__ w, const T *__restrict__ fx_mid,
                                                             float *__restrict__ partials, int B, int64_t N, int H, int D,
                                                             int S, int64_t chunk) {
-  extern __shared__ float lds[];
-  float *wl = lds;                       // 32 * S
-  float *fl = wl + kPartialTile * S;     // 32 * (D+1)
+  extern __shared__ float4 lds4[];
+  const int D1 = D + 1, SB = (S + 3) / 4, DB = (D1 + 3) / 4;  // tiles along the slices / the features
+  float4 *wl = lds4;                      // 32 * SB
+  float4 *fl = wl + kPartialTile * SB;    // 32 * DB
+  float *wlf = reinterpret_cast<float *>(wl), *flf = reinterpret_cast<float *>(fl);
   const int t = threadIdx.x;
   const int g = blockIdx.x;
   const int b = blockIdx.y / H, h = blockIdx.y % H;
-  const int D1 = D + 1;
-  const int n_out = S * D1;
-  const int slab0 = blockIdx.z * kSlab;
-  int os[NS], od[NS];
-  float acc[NS];
+  const int n_tiles = SB * DB;
+  const int slab0 = blockIdx.z * 256 * NS;
+  int sb[NS], db[NS];
+  float acc[NS][4][4];
 #pragma unroll
   for (int i = 0; i < NS; ++i) {
-    const int o = slab0 + t + 256 * i;
-    const bool ok = o < n_out;
-    os[i] = ok ? o / D1 : 0;
-    od[i] = ok ? o % D1 : 0;
-    acc[i] = 0.f;
+    const int tile = slab0 + t + 256 * i;
+    const bool ok = tile < n_tiles;
+    sb[i] = ok ? tile % SB : 0;
+    db[i] = ok ? tile / SB : 0;
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) acc[i][u][v] = 0.f;
   }
   const int64_t n_begin = (int64_t)g * chunk;
   const int64_t n_end = min(N, n_begin + chunk);
   const int HS = H * S, HD = H * D;
   for (int64_t n0 = n_begin; n0 < n_end; n0 += kPartialTile) {
     const int pts = (int)min((int64_t)kPartialTile, n_end - n0);
-    for (int i = t; i < kPartialTile * S; i += 256) {
-      const int p = i / S, s = i - p * S;
-      wl[i] = p < pts ? load_as_f32(w + ((int64_t)b * N + n0 + p) * HS + h * S + s) : 0.f;
+    for (int i = t; i < kPartialTile * SB * 4; i += 256) {
+      const int p = i / (SB * 4), s = i - p * (SB * 4);
+      wlf[i] = (p < pts && s < S) ? load_as_f32(w + ((int64_t)b * N + n0 + p) * HS + h * S + s) : 0.f;
     }
-    for (int i = t; i < kPartialTile * D1; i += 256) {
-      const int p = i / D1, d = i - p * D1;
+    for (int i = t; i < kPartialTile * DB * 4; i += 256) {
+      const int p = i / (DB * 4), d = i - p * (DB * 4);
       float v = 0.f;
-      if (p < pts) v = d < D ? load_as_f32(fx_mid + ((int64_t)b * N + n0 + p) * HD + h * D + d) : 1.f;
-      fl[i] = v;
+      if (p < pts && d < D) v = load_as_f32(fx_mid + ((int64_t)b * N + n0 + p) * HD + h * D + d);
+      if (p < pts && d == D) v = 1.f;
+      flf[i] = v;
     }
     __syncthreads();
-#pragma unroll(NS > 8 ? 1 : 2)  // a full unroll hoists every LDS read of the tile: 256 registers, one wave per SIMD
+#pragma unroll 2
     for (int p = 0; p < kPartialTile; ++p) {
-      const float *wp = wl + p * S;
-      const float *fp = fl + p * D1;
 #pragma unroll
-      for (int i = 0; i < NS; ++i) acc[i] = fmaf(wp[os[i]], fp[od[i]], acc[i]);
+      for (int i = 0; i < NS; ++i) {
+        const float4 wv = wl[p * SB + sb[i]];
+        const float4 fv = fl[p * DB + db[i]];
+        const float ws[4] = {wv.x, wv.y, wv.z, wv.w}, fs[4] = {fv.x, fv.y, fv.z, fv.w};
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+#pragma unroll
+          for (int v = 0; v < 4; ++v) acc[i][u][v] = fmaf(ws[u], fs[v], acc[i][u][v]);
+      }
     }
     __syncthreads();
   }
-  float *dst = partials + (((int64_t)g * B + b) * H + h) * n_out;
+  float *dst = partials + (((int64_t)g * B + b) * H + h) * (S * D1);
 #pragma unroll
   for (int i = 0; i < NS; ++i) {
-    const int o = slab0 + t + 256 * i;
-    if (o < n_out) dst[o] = acc[i];
+    if (slab0 + t + 256 * i >= n_tiles) continue;
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        const int s = 4 * sb[i] + u, d = 4 * db[i] + v;
+        if (s < S && d < D1) dst[s * D1 + d] = acc[i][u][v];
+      }
   }
 }
 
@@ -719,7 +718,8 @@ __global__ __launch_bounds__(256) void dequant_e4m3_kernel(const uint8_t *__rest
 // ================================================================================================
 template <typename TA, typename TW>
 static int launch_gemm(const GemmArgs &a, int nsets, hipStream_t st) {
-  if (gemm::serves(a, nsets, sizeof(TA))) return gemm::launch(a, nsets, sizeof(TA) == 4 ? PA_F32 : PA_BF16, st);
+  if constexpr (sizeof(TA) == sizeof(TW))  // the MFMA kernels take both operands in one type
+    if (gemm::serves(a, nsets, sizeof(TA))) return gemm::launch(a, nsets, sizeof(TA) == 4 ? PA_F32 : PA_BF16, st);
   dim3 grid((unsigned)((a.M + 63) / 64), (unsigned)((a.O + 63) / 64), (unsigned)nsets);
   hipLaunchKernelGGL((rows_gemm_kernel<TA, TW>), grid, dim3(256), 0, st, a);
   return launch_status();
@@ -814,31 +814,71 @@ int out_linear(int dtype, const pa_shape &s, const pa_params &p, const void *out
   return dtype == PA_F32 ? launch_gemm<float, float>(a, 1, st) : launch_gemm<bf16, bf16>(a, 1, st);
 }
 
+// Slice weights (PA.py:537, :172-181): the logits are a Linear over the (point, head) rows -- D inputs, S outputs,
+// one weight for all heads -- so they come from the row GEMM kernels (MFMA for float32; the float32 weight against
+// bf16 rows takes the FMA kernel), written in the storage type as the reference's Linear output is; the softmax with
+// the head's clamped temperature then runs in place over each row of S.
 template <typename T>
 static int slice_softmax_t(const pa_shape &s, const pa_params &p, const void *x_mid, void *w, hipStream_t st) {
-  const int H = (int)s.H, D = (int)s.D, S = (int)s.S;
-  const size_t fixed = (size_t)(S * D + S) * 4;
-  const size_t per_row = (size_t)(H * (D + 1) + H * (S + 1)) * 4;
-  if (fixed + per_row > 60 * 1024) return PA_ERR_UNSUPPORTED;
-  int R = (int)((60 * 1024 - fixed) / per_row);
-  if (R > 8) R = 8;
-  const size_t lds = fixed + per_row * R;
-  int rc = allow_dynamic_lds(slice_softmax_kernel<T>, lds);
+  GemmArgs a{};
+  a.in = x_mid;
+  a.w[0] = p.in_project_slice_weight;
+  a.bias[0] = p.in_project_slice_bias;
+  a.out[0] = w;
+  a.M = s.B * s.N * s.H;
+  a.K = (int)s.D;
+  a.O = (int)s.S;
+  int rc = launch_gemm<T, float>(a, 1, st);
   if (rc) return rc;
-  const int64_t M = s.B * s.N;
-  hipLaunchKernelGGL((slice_softmax_kernel<T>), dim3((unsigned)((M + R - 1) / R)), dim3(256), lds, st,
-                     static_cast<const T *>(x_mid), p.in_project_slice_weight, p.in_project_slice_bias, p.temperature,
-                     static_cast<T *>(w), M, H, D, S, R);
-  return launch_status();
+  return flare::softmax_rows(sizeof(T) == 4 ? PA_F32 : PA_BF16, s, w, p.temperature, st);
 }
 
 int slice_softmax(int dtype, const pa_shape &s, const pa_params &p, const void *x_mid, void *w, hipStream_t st) {
   return dtype == PA_F32 ? slice_softmax_t<float>(s, p, x_mid, w, st) : slice_softmax_t<bf16>(s, p, x_mid, w, st);
 }
 
+template <typename T, int L>
+static int softmax_rows_plus_l(const pa_shape &s, const pa_params &p, const pa_plus_params &pp, void *w,
+                               const void *hidden, const void *uniform, hipStream_t st) {
+  const int64_t rows = s.B * s.N * s.H;
+  int64_t blocks = (rows + (256 / L) - 1) / (256 / L);
+  if (blocks > 16384) blocks = 16384;
+  hipLaunchKernelGGL((softmax_rows_plus_kernel<T, L>), dim3((unsigned)blocks), dim3(256), 0, st, static_cast<T *>(w),
+                     static_cast<const T *>(hidden), static_cast<const T *>(uniform), p.temperature,
+                     pp.proj_temperature_2_weight, pp.proj_temperature_2_bias, rows, (int)s.S, (int)s.H);
+  return launch_status();
+}
+
+// With a scratch buffer of B*N*H*S elements the two Linears run on the row GEMM kernels (several times faster than the
+// single kernel below, which forms them per point on the vector ALUs).
+template <typename T>
+static int slice_softmax_plus_staged(const pa_shape &s, const pa_params &p, const pa_plus_params &pp, const void *x_mid,
+                                     const void *uniform, void *w, void *scratch, hipStream_t st) {
+  GemmArgs a{};
+  a.in = x_mid;
+  a.M = s.B * s.N * s.H;
+  a.K = (int)s.D;
+  a.O = (int)s.S;
+  a.w[0] = p.in_project_slice_weight;
+  a.bias[0] = p.in_project_slice_bias;
+  a.out[0] = w;
+  int rc = launch_gemm<T, float>(a, 1, st);
+  if (rc) return rc;
+  a.w[0] = pp.proj_temperature_0_weight;
+  a.bias[0] = pp.proj_temperature_0_bias;
+  a.out[0] = scratch;
+  a.act = 1;
+  if ((rc = launch_gemm<T, float>(a, 1, st))) return rc;
+  if (s.S <= 8) return softmax_rows_plus_l<T, 8>(s, p, pp, w, scratch, uniform, st);
+  if (s.S <= 16) return softmax_rows_plus_l<T, 16>(s, p, pp, w, scratch, uniform, st);
+  if (s.S <= 32) return softmax_rows_plus_l<T, 32>(s, p, pp, w, scratch, uniform, st);
+  return softmax_rows_plus_l<T, 64>(s, p, pp, w, scratch, uniform, st);
+}
+
 template <typename T>
 static int slice_softmax_plus_t(const pa_shape &s, const pa_params &p, const pa_plus_params &pp, const void *x_mid,
-                                const void *uniform, void *w, hipStream_t st) {
+                                const void *uniform, void *w, void *scratch, hipStream_t st) {
+  if (scratch) return slice_softmax_plus_staged<T>(s, p, pp, x_mid, uniform, w, scratch, st);
   const int H = (int)s.H, D = (int)s.D, S = (int)s.S;
   const size_t fixed = (size_t)(2 * S * D + 3 * S) * 4;
   const size_t per_row = (size_t)(H * (D + 1) + H * (S + 1)) * 4;
@@ -857,9 +897,9 @@ static int slice_softmax_plus_t(const pa_shape &s, const pa_params &p, const pa_
 }
 
 int slice_softmax_plus(int dtype, const pa_shape &s, const pa_params &p, const pa_plus_params &pp, const void *x_mid,
-                       const void *uniform, void *w, hipStream_t st) {
-  return dtype == PA_F32 ? slice_softmax_plus_t<float>(s, p, pp, x_mid, uniform, w, st)
-                         : slice_softmax_plus_t<bf16>(s, p, pp, x_mid, uniform, w, st);
+                       const void *uniform, void *w, void *scratch, hipStream_t st) {
+  return dtype == PA_F32 ? slice_softmax_plus_t<float>(s, p, pp, x_mid, uniform, w, scratch, st)
+                         : slice_softmax_plus_t<bf16>(s, p, pp, x_mid, uniform, w, scratch, st);
 }
 
 // Number of point chunks of the first reduction pass: enough workgroups to fill 256 CUs several times
@@ -879,10 +919,12 @@ template <typename T>
 static int slice_partial_t(const pa_shape &s, const void *w, const void *fx_mid, float *partials, hipStream_t st) {
   const int64_t G = partial_count(s);
   const int64_t chunk = (s.N + G - 1) / G;
-  const int n_out = (int)(s.S * (s.D + 1));
-  const size_t lds = (size_t)(kPartialTile * s.S + kPartialTile * (s.D + 1)) * 4;
-  dim3 grid((unsigned)G, (unsigned)(s.B * s.H), (unsigned)((n_out + kSlab - 1) / kSlab));
-  const int per_thread = ((n_out < kSlab ? n_out : kSlab) + 255) / 256;
+  const int SB = (int)((s.S + 3) / 4), DB = (int)((s.D + 1 + 3) / 4);
+  const int n_tiles = SB * DB;
+  const size_t lds = (size_t)kPartialTile * (SB + DB) * 16;
+  const int per_thread = (n_tiles + 255) / 256;
+  const int ns = per_thread <= 1 ? 1 : (per_thread <= 2 ? 2 : kPartialMaxNS);
+  dim3 grid((unsigned)G, (unsigned)(s.B * s.H), (unsigned)((n_tiles + 256 * ns - 1) / (256 * ns)));
   auto launch = [&](auto kernel) {
     int rc = allow_dynamic_lds(kernel, lds);
     if (rc) return rc;
@@ -890,10 +932,9 @@ static int slice_partial_t(const pa_shape &s, const void *w, const void *fx_mid,
                        partials, (int)s.B, s.N, (int)s.H, (int)s.D, (int)s.S, chunk);
     return launch_status();
   };
-  if (per_thread <= 2) return launch(slice_partial_kernel<T, 2>);
-  if (per_thread <= 4) return launch(slice_partial_kernel<T, 4>);
-  if (per_thread <= 8) return launch(slice_partial_kernel<T, 8>);
-  return launch(slice_partial_kernel<T, 16>);
+  if (ns == 1) return launch(slice_partial_kernel<T, 1>);
+  if (ns == 2) return launch(slice_partial_kernel<T, 2>);
+  return launch(slice_partial_kernel<T, kPartialMaxNS>);
 }
 
 // `partials` holds G partial sums followed by one spare slot (index G) that receives their fixed-order total.

@@ -75,7 +75,7 @@ int rows_gemm_packed(const pa_shape &s, int64_t c_in, const void *in, const void
                      void *out_pack, hipStream_t st);
 int slice_softmax(int dtype, const pa_shape &s, const pa_params &p, const void *x_mid, void *w, hipStream_t st);
 int slice_softmax_plus(int dtype, const pa_shape &s, const pa_params &p, const pa_plus_params &pp, const void *x_mid,
-                       const void *uniform, void *w, hipStream_t st);
+                       const void *uniform, void *w, void *scratch, hipStream_t st);
 int64_t partial_count(const pa_shape &s);
 size_t combine_attn_lds_bytes(const pa_shape &s);
 int slice_partial(int dtype, const pa_shape &s, const void *w, const void *fx_mid, float *partials, hipStream_t st);
@@ -109,7 +109,8 @@ namespace flare {
 int64_t column_max_chunks(const pa_shape &s);
 int column_weights(int dtype, const pa_shape &s, const void *a, float *partial, float *colmax, void *wc,
                    hipStream_t st);
-int softmax_rows(int dtype, const pa_shape &s, void *a, hipStream_t st);
+// temperature: NULL, or (H) float32 -- the entries are then divided by clamp(temperature[head], 0.5, 5) first
+int softmax_rows(int dtype, const pa_shape &s, void *a, const float *temperature, hipStream_t st);
 }  // namespace flare
 
 namespace gale {

@@ -72,10 +72,11 @@ def slice_softmax_plus(x_mid, uniform, params, dims: LayerDims):
     if uniform.dtype != x_mid.dtype or uniform.shape != (dims.B, dims.N, dims.H, dims.S):
         raise ValueError("uniform samples must have the activation dtype and shape (B, N, H, S)")
     w = torch.empty(dims.B, dims.N, dims.H, dims.S, dtype=x_mid.dtype, device=x_mid.device)
+    scratch = torch.empty_like(w)  # hidden layer of proj_temperature: lets both Linears run on the row GEMM kernels
     plus = _lib.PaPlusParams(*[_lib.ptr(params[k]) for k, _ in _lib.PaPlusParams._fields_])
     _lib.check(_lib.load().pa_slice_softmax_plus(_lib.dtype_code(x_mid.dtype), byref(dims.c()),
                                                  byref(_c_params(params)), byref(plus), x_mid.data_ptr(),
-                                                 uniform.data_ptr(), w.data_ptr(),
+                                                 uniform.data_ptr(), w.data_ptr(), scratch.data_ptr(),
                                                  _lib.current_stream_ptr(x_mid.device)), "pa_slice_softmax_plus")
     return w
 
