@@ -474,6 +474,31 @@ class OracleTransolverBlock(nn.Module):
         return self.ln_mlp2(fx) if self.last_layer else fx  # :306-309
 
 
+class OracleGALEBlock(nn.Module):
+    """physicsnemo/nn/module/gale.py:764-1030 (use_te=False, attention_type="GALE", no concrete dropout): per input
+    tensor  fx = Attn(ln_1(fx), context) + fx;  fx = ln_mlp1(fx) + fx  (:1018-1028)."""
+
+    def __init__(self, num_heads, hidden_dim, dropout=0.0, mlp_ratio=4, slice_num=32, context_dim=0,
+                 spatial_shape=None, state_mixing_mode="weighted"):
+        super().__init__()
+        self.ln_1 = nn.LayerNorm(hidden_dim)
+        kw = dict(heads=num_heads, dim_head=hidden_dim // num_heads, dropout=dropout, slice_num=slice_num,
+                  context_dim=context_dim, state_mixing_mode=state_mixing_mode)
+        if spatial_shape is None:
+            self.Attn = OracleGALE(hidden_dim, **kw)
+        elif len(spatial_shape) == 2:
+            self.Attn = OracleGALEStructuredMesh2D(hidden_dim, spatial_shape, **kw)
+        else:
+            raise ValueError("oracle covers the irregular and structured-2D GALE blocks")
+        self.ln_mlp1 = nn.Sequential(nn.LayerNorm(hidden_dim),
+                                     OracleMlp(hidden_dim, hidden_dim * mlp_ratio, hidden_dim))
+
+    def forward(self, fx, global_context):
+        attn = self.Attn(tuple(self.ln_1(t) for t in fx), global_context)
+        out = [a + t for a, t in zip(attn, fx)]
+        return [self.ln_mlp1(t) + t for t in out]
+
+
 def unified_pos_grid(structured_shape, ref):
     """Distance of every grid point (i/(h-1), j/(w-1)) to a ref x ref lattice on [0,1]^2
     (transolver.py:617-645), shape (1, h*w, ref*ref), float32."""

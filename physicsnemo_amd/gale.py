@@ -2,7 +2,8 @@
 
 Mirrors ``physicsnemo/nn/module/gale.py``:
   GALE:242-398 (irregular), GALEStructuredMesh2D:447-478, GALEStructuredMesh3D:480-512, ``_gale_cross_init``:401-429,
-  ``_gale_forward_impl``:148-239, ``_gale_compute_slice_attention_cross``:87-145, ``_mix_self_and_cross``:43-84.
+  ``_gale_forward_impl``:148-239, ``_gale_compute_slice_attention_cross``:87-145, ``_mix_self_and_cross``:43-84,
+  GALEBlock:764-1030.
 
 A GALE layer is a PhysicsAttention layer whose slice tokens, besides attending to each other, attend to a context
 ``(B, H, S_c, D_c)``; the two results are blended (learned sigmoid gate, or concatenation + Linear + GELU) before the
@@ -191,3 +192,68 @@ class GALEStructuredMesh3D(_GALEForwardMixin, PhysicsAttentionStructuredMesh3D):
                  context_dim: int = 0, state_mixing_mode: str = "weighted"):
         super().__init__(dim, spatial_shape, heads, dim_head, dropout, slice_num, kernel, use_te, plus)
         _gale_cross_init(self, dim_head, context_dim, state_mixing_mode)
+
+
+class GALEBlock(nn.Module):
+    """LayerNorm -> GALE attention (with the shared context) -> +residual -> LayerNorm -> MLP -> +residual, for every
+    tensor of the input tuple (reference gale.py:764-1030).  ``attention_type="GALE_FA"`` and ``concrete_dropout`` are not
+    served.  The LayerNorms, the block MLP and its residual add run on the library kernels of the Transolver block."""
+
+    def __init__(self, num_heads: int, hidden_dim: int, dropout: float, act: str = "gelu", mlp_ratio: int = 4,
+                 last_layer: bool = False, out_dim: int = 1, slice_num: int = 32, use_te: bool = False,
+                 plus: bool = False, context_dim: int = 0, spatial_shape: tuple | None = None,
+                 attention_type: str = "GALE", concrete_dropout: bool = False, state_mixing_mode: str = "weighted"):
+        super().__init__()
+        from .transolver import Mlp  # the block MLP of the Transolver block (reference mlp_layers.py:101-173)
+
+        self.last_layer = last_layer
+        self.ln_1 = nn.LayerNorm(hidden_dim)
+        if attention_type == "GALE_FA":
+            raise NotImplementedError("attention_type='GALE_FA' (GALE with FLARE self-attention) is not served")
+        if attention_type != "GALE":
+            raise ValueError(f"Invalid attention type: {attention_type}. Expected 'GALE' or 'GALE_FA'.")
+        if concrete_dropout:
+            raise NotImplementedError("ConcreteDropout is a training-time regulariser; the HIP block has none")
+        common = dict(heads=num_heads, dim_head=hidden_dim // num_heads, dropout=dropout, slice_num=slice_num,
+                      use_te=use_te, plus=plus, context_dim=context_dim, state_mixing_mode=state_mixing_mode)
+        if spatial_shape is None:
+            self.Attn = GALE(hidden_dim, **common)
+        elif len(spatial_shape) == 2:
+            self.Attn = GALEStructuredMesh2D(hidden_dim, spatial_shape=tuple(int(v) for v in spatial_shape), **common)
+        elif len(spatial_shape) == 3:
+            self.Attn = GALEStructuredMesh3D(hidden_dim, spatial_shape=tuple(int(v) for v in spatial_shape), **common)
+        else:
+            raise ValueError(f"spatial_shape must be None, length-2, or length-3; got {spatial_shape!r}")
+        self.ln_mlp1 = nn.Sequential(nn.LayerNorm(hidden_dim), Mlp(hidden_dim, hidden_dim * mlp_ratio, hidden_dim, act))
+        self.attn_dropout = None
+        self.ffn_dropout = None
+        self._mlp_cache: dict = {}
+
+    def _one(self, fx: torch.Tensor, attn: torch.Tensor, needs_grad: bool) -> torch.Tensor:
+        from . import autograd as PA
+        from .transolver import TransolverBlock as TB
+
+        fx1 = attn + fx
+        normed = PA.layer_norm(fx1, self.ln_mlp1[0])
+        if not needs_grad and TB._mlp_kernel_serves(self, normed):
+            w1, b1, w2, b2 = TB._mlp_kernel_params(self, normed.device)
+            return PF.mlp_forward(normed, w1, b1, w2, b2, residual=fx1.to(normed.dtype).contiguous())
+        return TB._mlp_with_grad(self, normed) + fx1
+
+    def forward(self, fx: tuple, global_context: torch.Tensor | None) -> list:
+        from . import autograd as PA
+
+        if isinstance(fx, torch.Tensor):
+            raise TypeError("GALEBlock takes a tuple of input tensors")
+        if len(fx) == 0:
+            raise ValueError("Expected non-empty tuple of input tensors")
+        for i, t in enumerate(fx):
+            if t.ndim != 3:
+                raise ValueError(f"Expected 3D input tensor (B, N, C) at index {i}, "
+                                 f"got {t.ndim}D tensor with shape {tuple(t.shape)}")
+        needs_grad = torch.is_grad_enabled() and (any(t.requires_grad for t in fx) or
+                                                  any(p.requires_grad for p in self.parameters()))
+        if not needs_grad and torch.is_autocast_enabled("cuda") and torch.get_autocast_dtype("cuda") == torch.bfloat16:
+            fx = tuple(t.to(torch.bfloat16) for t in fx)  # inference: the residual stream in the compute type
+        attn = self.Attn(tuple(PA.layer_norm(t, self.ln_1) for t in fx), global_context)
+        return [self._one(t, a, needs_grad) for t, a in zip(fx, attn)]

@@ -260,3 +260,61 @@ def test_context_projector_plus_and_errors():
     sp = pn.StructuredContextProjector(4, (3, 4), heads=2, dim_head=8, slice_num=4).cuda()
     with pytest.raises(ValueError, match="Expected N=12 tokens"), torch.no_grad():
         sp(torch.randn(1, 13, 4, device="cuda"))
+
+
+# ---------------------------------------------------------------------------------------------------
+# GALE block
+# ---------------------------------------------------------------------------------------------------
+def _block_pair(hidden, heads, S, Dc, grid=None, mlp_ratio=2, seed=0):
+    torch.manual_seed(seed)
+    ref = to.OracleGALEBlock(heads, hidden, mlp_ratio=mlp_ratio, slice_num=S, context_dim=Dc, spatial_shape=grid)
+    hip = pn.GALEBlock(heads, hidden, 0.0, mlp_ratio=mlp_ratio, slice_num=S, context_dim=Dc, spatial_shape=grid)
+    with torch.no_grad():
+        ref.Attn.in_project_slice.weight.mul_(2.0)
+        ref.Attn.state_mixing.fill_(0.4)
+    hip.load_state_dict(ref.state_dict())
+    return ref.eval(), hip.eval().cuda()
+
+
+@pytest.mark.parametrize("hidden,heads,S,B,N,Sc,Dc,grid", [
+    (32, 4, 8, 2, 300, 5, 7, None),
+    (32, 4, 16, 2, 63, 9, 12, (7, 9)),
+])
+def test_fp32_gale_block_forward_and_gradients(hidden, heads, S, B, N, Sc, Dc, grid):
+    announce("fp32 GALE block", hidden, heads, S, B, N, Sc, Dc, grid)
+    ref, hip = _block_pair(hidden, heads, S, Dc, grid)
+    x1, x2, ctx = torch.randn(B, N, hidden), torch.randn(B, N, hidden), torch.randn(B, heads, Sc, Dc)
+    with torch.no_grad():
+        want = ref((x1, x2), ctx)
+        got = hip((x1.cuda(), x2.cuda()), ctx.cuda())
+    for g, w in zip(got, want):
+        assert_fp32_close(g, w, "GALE block y")
+    probe = torch.randn(B, N, hidden)
+    ref.train(), hip.train()
+    xr = x1.clone().requires_grad_(True)
+    (ref((xr,), ctx)[0] * probe).sum().backward()
+    xh = x1.cuda().requires_grad_(True)
+    (hip((xh,), ctx.cuda())[0] * probe.cuda()).sum().backward()
+    assert_fp32_close(xh.grad, xr.grad, "grad x", rtol=2e-4)
+    grads = dict(hip.named_parameters())
+    for name, p in ref.named_parameters():
+        if name == "Attn.cross_k.bias":
+            continue  # zero in exact arithmetic
+        assert grads[name].grad is not None, name
+        assert_fp32_close(grads[name].grad, p.grad, f"grad {name}", rtol=2e-4)
+
+
+def test_bf16_gale_block_on_the_fused_kernels():
+    announce("bf16 GALE block")
+    ref, hip = _block_pair(256, 8, 64, 32, mlp_ratio=4)
+    x, ctx = torch.randn(2, 4096, 256), torch.randn(2, 8, 48, 32)
+    with torch.no_grad():
+        want = ref((x,), ctx)[0]
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            got = hip((x.cuda(),), ctx.cuda())[0]
+    assert got.dtype == torch.bfloat16
+    assert_rel_l2(got, want, "bf16 GALE block y", tol=1e-2)
+    with pytest.raises(NotImplementedError):
+        pn.GALEBlock(8, 256, 0.0, attention_type="GALE_FA")
+    with pytest.raises(ValueError, match="Invalid attention type"):
+        pn.GALEBlock(8, 256, 0.0, attention_type="other")

@@ -172,3 +172,21 @@ def test_context_projector_is_the_encoding_half_of_the_layer():
     u = torch.rand(2, 9, 2, 5, dtype=torch.float64)
     with torch.no_grad():
         torch.testing.assert_close(pp(x, u), lp.stages(x, u)["tok"])
+
+
+def test_gale_block_against_numpy_pieces():
+    """OracleGALEBlock = LayerNorm, GALE layer, residual, LayerNorm, MLP, residual (gale.py:1018-1028), checked against
+    the NumPy restatements of each piece."""
+    torch.manual_seed(6)
+    blk = to.OracleGALEBlock(2, 12, mlp_ratio=2, slice_num=5, context_dim=7).double().eval()
+    x = torch.randn(2, 9, 12, dtype=torch.float64)
+    ctx = torch.randn(2, 2, 4, 7, dtype=torch.float64)
+    with torch.no_grad():
+        got = blk((x,), ctx)[0].numpy()
+    p = _sd_np(blk)
+    attn_p = {k[len("Attn."):]: v for k, v in p.items() if k.startswith("Attn.")}
+    h1 = no.layer_norm(x.numpy(), p["ln_1.weight"], p["ln_1.bias"])
+    fx = no.layer_forward(attn_p, h1, 2, 6, context=ctx.numpy())["y"] + x.numpy()
+    h2 = no.layer_norm(fx, p["ln_mlp1.0.weight"], p["ln_mlp1.0.bias"])
+    want = no.mlp(p, "ln_mlp1.1.", h2) + fx
+    np.testing.assert_allclose(got, want, rtol=1e-10, atol=1e-12)
