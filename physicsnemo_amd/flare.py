@@ -74,8 +74,6 @@ class FLARE(nn.Module):
             raise RuntimeError("physicsnemo_amd FLARE runs on GPU tensors only (no CPU fallback)")
         if torch.is_grad_enabled() and (x.requires_grad or any(p.requires_grad for p in self.parameters())):
             raise NotImplementedError("the backward kernels do not cover FLARE; run under torch.no_grad()")
-        if self.training and self.out_dropout.p > 0:
-            raise NotImplementedError("dropout > 0 in training mode is not served by the HIP layer")
         out_dtype = None
         if torch.is_autocast_enabled("cuda"):
             ac = torch.get_autocast_dtype("cuda")
@@ -100,4 +98,4 @@ class FLARE(nn.Module):
         z = (tok * (norm / (norm - 1e-2)).unsqueeze(-1)).contiguous()
         PF.flare_softmax_rows_(scores, dims)
         y = PF.deslice_project(scores, z, p, dims)
-        return y if out_dtype is None else y.to(out_dtype)
+        return self.out_dropout(y if out_dtype is None else y.to(out_dtype))

@@ -156,10 +156,11 @@ class _GALEForwardMixin:
                 self._validate(t)
             self._check_context(context, x[0].shape[0])
             if torch.is_grad_enabled() and (context.requires_grad or any(self._needs_grad(t) for t in x)):
-                return [self._forward_one_with_grad(t, context) for t in x]
+                return [self.out_dropout(self._forward_one_with_grad(t, context)) for t in x]
             context = context.detach().float().contiguous()
             gp = self.gale_params(context.device)
-        return [self._forward_one(t, context, gp) for t in x]
+        return [self.out_dropout(self._forward_one(t, context, gp)) if context is not None
+                else self._forward_one(t, None, None) for t in x]  # without a context the plain layer applies it
 
 
 class GALE(_GALEForwardMixin, PhysicsAttentionIrregularMesh):

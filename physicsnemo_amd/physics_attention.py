@@ -140,8 +140,6 @@ class PhysicsAttentionBase(nn.Module):
     def _prepare_input(self, x: torch.Tensor) -> torch.Tensor:
         if not x.is_cuda:
             raise RuntimeError("physicsnemo_amd PhysicsAttention runs on GPU tensors only (no CPU fallback)")
-        if self.training and self.out_dropout.p > 0:
-            raise RuntimeError("dropout > 0 in training mode is not served by the HIP kernels")
         if torch.is_autocast_enabled("cuda"):
             ac = torch.get_autocast_dtype("cuda")
             if ac != torch.bfloat16:
@@ -200,10 +198,12 @@ class PhysicsAttentionBase(nn.Module):
         needs_grad = self._needs_grad(x)
         x = self._prepare_input(x)
         if needs_grad:
-            return self._forward_with_grad(x)
-        if self.plus:
+            y = self._forward_with_grad(x)
+        elif self.plus:
             return self.forward_with_noise(x, None)
-        return PF.layer_forward(x, self.kernel_params(x.dtype, x.device), self.layer_dims(x))
+        else:
+            y = PF.layer_forward(x, self.kernel_params(x.dtype, x.device), self.layer_dims(x))
+        return self.out_dropout(y)  # identity unless training with dropout > 0 (reference :499)
 
     def forward_with_noise(self, x: torch.Tensor, noise_u: torch.Tensor | None, stages: bool = False):
         """Transolver++ forward (reference :166-170, :530-532) through the stage-level kernels.  ``noise_u``
@@ -213,7 +213,7 @@ class PhysicsAttentionBase(nn.Module):
             raise RuntimeError("forward_with_noise is the plus=True path")
         self._validate(x)
         if self._needs_grad(x) and not stages:
-            return self._forward_plus_with_grad(self._prepare_input(x), noise_u)
+            return self.out_dropout(self._forward_plus_with_grad(self._prepare_input(x), noise_u))
         x = self._prepare_input(x)
         dims = self.layer_dims(x)
         p = self.kernel_params(x.dtype, x.device)
@@ -227,7 +227,7 @@ class PhysicsAttentionBase(nn.Module):
         if stages:
             H, D = self.heads, self.dim_head
             return dict(x_mid=x_mid.view(dims.B, dims.N, H, D), w=w, tok=tok, norm=norm, tok_out=tok_out, y=y)
-        return y
+        return self.out_dropout(y)
 
     def forward_block(self, x: torch.Tensor, residual: torch.Tensor, ln: nn.LayerNorm):
         """Layer + the caller block's ``+ residual`` and following LayerNorm in one pass
@@ -236,8 +236,8 @@ class PhysicsAttentionBase(nn.Module):
             with torch.autocast("cuda", enabled=False):  # float32 inside, as the residual stream of the caller is
                 return self.forward_block(x.float(), residual.float(), ln)
         self._validate(x)
-        if self.plus:
-            y = self.forward_with_noise(x, None)
+        if self.plus or (self.training and self.out_dropout.p > 0):  # dropout sits between the layer and the residual add
+            y = self.forward(x)
             fx_new = y + residual.to(y.dtype)
             normed = torch.nn.functional.layer_norm(fx_new.float(), ln.normalized_shape, ln.weight, ln.bias, ln.eps)
             return fx_new, normed.to(y.dtype)

@@ -147,7 +147,7 @@ def test_product_package_never_imports_the_oracle():
 
 
 def test_integration_stub_structs_match_the_binding():
-    """The ctypes stub printed in INTEGRATION.md must lay out pa_shape / pa_params / pa_block_tail like the header."""
+    """The ctypes stub printed in the integration guide must lay out pa_shape / pa_params / pa_block_tail like the header."""
     import re
     text = open(os.path.join(ROOT, "INTEGRATION.md")).read()
 

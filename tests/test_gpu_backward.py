@@ -308,3 +308,27 @@ def test_layernorm_and_linear_autograd_functions(dtype, rows, C):
         ref_dw = (p2.bfloat16().float().reshape(-1, 256).t() @ x.bfloat16().float().reshape(-1, C))
         assert_rel_l2(lin.weight.grad, ref_dw, "linear dW", tol=1e-2)
         assert_rel_l2(lin.bias.grad, p2.bfloat16().float().reshape(-1, 256).sum(0), "linear db", tol=1e-2)
+
+
+def test_output_dropout_in_training_matches_the_reference_site():
+    """The reference applies nn.Dropout to the layer output in training mode (physics_attention.py:499): kept entries
+    are y / (1 - p), the rest zero, gradients flow through the kept entries only; eval mode is the identity."""
+    announce("output dropout in training")
+    torch.manual_seed(0)
+    layer = pn.PhysicsAttentionIrregularMesh(64, heads=2, dim_head=32, dropout=0.25, slice_num=16, use_te=False).cuda()
+    x = torch.randn(2, 2000, 64, device="cuda")
+    layer.eval()
+    with torch.no_grad():
+        y_eval = layer(x)
+    layer.train()
+    xg = x.clone().requires_grad_(True)
+    y = layer(xg)
+    kept = y != 0
+    frac = kept.float().mean().item()
+    assert abs(frac - 0.75) < 0.01, frac
+    assert_fp32_close(y[kept], (y_eval / 0.75)[kept], "kept entries")
+    y.sum().backward()
+    assert xg.grad is not None and torch.isfinite(xg.grad).all()
+    blk = pn.TransolverBlock(2, 64, 0.25, mlp_ratio=2, slice_num=16, use_te=False).cuda().train()
+    out = blk(x)
+    assert out.shape == x.shape and torch.isfinite(out).all()
