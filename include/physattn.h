@@ -266,6 +266,16 @@ int64_t pa_flare_column_max_chunks(const pa_shape *shape);
 int pa_flare_column_weights(int dtype, const pa_shape *shape, const void *scores, float *partials, float *column_max,
                             void *weights, void *stream);
 int pa_flare_softmax_rows(int dtype, const pa_shape *shape, void *scores, void *stream);
+/* Per-point part of the FLARE backward pass (the reference differentiates flare_attention.py:38-72 with autograd).
+ * row_weights = softmax_s(A), column_weights = exp(A - max_n A), values v, d_out_x = gradient of the hand-back result
+ * (B,N,H*D), z (B,H,S,D) float32, and d_num / d_den = gradients of the un-normalised gather sums (z = num / den):
+ *   d_scores (B,N,H,S) = row softmax backward of d_out_x . z^T  +  column_weights * (v . d_num^T + d_den)
+ *   d_values (B,N,H*D) = column_weights . d_num
+ * The rest of the backward is the entry points above: pa_rows_gemm (d out_x from d y; d x from d_scores | d_values),
+ * pa_slice_weighted_sum (d z), weight gradients as products over the point axis. */
+int pa_flare_backward_points(int dtype, const pa_shape *shape, const void *row_weights, const void *column_weights,
+                             const void *values, const void *d_out_x, const float *z, const float *d_num,
+                             const float *d_den, void *d_scores, void *d_values, void *stream);
 
 /* Attended slice tokens (B,H,S,32) float32 computed by the caller (e.g. a GALE token stage under autograd) -> the
  * PA_BUF_TOKP operands of pa_mfma_deslice_project, which pa_mfma_combine_attention otherwise writes

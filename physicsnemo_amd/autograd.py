@@ -387,6 +387,56 @@ class SliceTokensFunction(torch.autograd.Function):
         return base[:3] + base[3:10]
 
 
+class FlareFunction(torch.autograd.Function):
+    """FLARE layer core (flare_attention.py:38-72, :222-255) given the composed score / value weights: differentiable
+    w.r.t. x, the four composed tensors and out_linear.  The composition itself (q_global, self_k / self_v and
+    in_project_x folded into two matrices) is a handful of small tensor products done by the caller under autograd, so
+    the gradients reach the layer's own parameters through it."""
+
+    @staticmethod
+    def forward(ctx, x, dims, w_a, b_a, w_v, b_v, wo, bo):
+        B, N, C, H, D, S = dims.B, dims.N, dims.C, dims.H, dims.D, dims.S
+        wa_k, wv_k = w_a.detach().to(x.dtype).contiguous(), w_v.detach().to(x.dtype).contiguous()
+        scores = PF.rows_gemm(x, wa_k, b_a.detach().float().contiguous(), dims, C, H * S).view(B, N, H, S)
+        values = PF.rows_gemm(x, wv_k, b_v.detach().float().contiguous(), dims, C, H * D)
+        col_w, _ = PF.flare_column_weights(scores, dims)
+        tok, norm = PF.slice_reduce(col_w, values, dims)
+        den = norm - 1e-2  # the aggregation kernel adds the PhysicsAttention epsilon to the divisor; FLARE has none
+        z = (tok * (norm / den).unsqueeze(-1)).contiguous()
+        row_w = PF.flare_softmax_rows_(scores, dims)
+        kp = {"out_linear_weight": wo.detach().to(x.dtype).contiguous().reshape(-1),
+              "out_linear_bias": bo.detach().float().contiguous()}
+        y, out_x = PF.deslice_project(row_w, z, kp, dims, return_out_x=True)
+        ctx.save_for_backward(x, row_w, col_w, values, z, den, out_x, wa_k, wv_k, kp["out_linear_weight"])
+        ctx.dims = dims
+        ctx.dtypes = tuple(t.dtype for t in (w_a, b_a, w_v, b_v, wo, bo))
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, row_w, col_w, values, z, den, out_x, wa_k, wv_k, wo_k = ctx.saved_tensors
+        dims = ctx.dims
+        B, N, C, H, D, S = dims.B, dims.N, dims.C, dims.H, dims.D, dims.S
+        HD, HS = H * D, H * S
+        dy = dy.to(x.dtype).contiguous()
+        g = PF.rows_gemm(dy, wo_k.view(C, HD).t().contiguous(), None, dims, C, HD)
+        d_wo, d_bo = _wgrad(dy, out_x)
+        d_z = PF.slice_weighted_sum(row_w, g, dims)[..., :D]
+        d_num = (d_z / den.unsqueeze(-1)).contiguous()
+        d_den = (-(d_z * z).sum(-1) / den).contiguous()
+        d_a, d_v = PF.flare_backward_points(row_w, col_w, values, g, z, d_num, d_den, dims)
+        d_a = d_a.view(B, N, HS)
+        dx = None
+        if ctx.needs_input_grad[0]:
+            w_cat = torch.cat([wa_k, wv_k], dim=0).t().contiguous()  # (C, HS + HD)
+            dx = PF.rows_gemm(torch.cat([d_a, d_v], dim=-1), w_cat, None, dims, HS + HD, C)
+        d_wa, d_ba = _wgrad(d_a, x)
+        d_wv, d_bv = _wgrad(d_v, x)
+        grads = [gr.float().reshape(shape).to(dt) for gr, shape, dt in zip(
+            (d_wa, d_ba, d_wv, d_bv, d_wo, d_bo), ((HS, C), (HS,), (HD, C), (HD,), (C, HD), (C,)), ctx.dtypes)]
+        return (dx, None, *grads)
+
+
 class LinearFunction(torch.autograd.Function):
     """torch.nn.functional.linear for the block MLP in bf16 training: the two row GEMMs (forward, input gradient) go to
     the GEMM library, the weight and bias gradients -- products over the huge row axis, where the library's kernels

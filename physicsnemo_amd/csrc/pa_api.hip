@@ -485,6 +485,19 @@ int pa_flare_softmax_rows(int dtype, const pa_shape *shape, void *scores, void *
   return pa::flare::softmax_rows(dtype, *shape, scores, nullptr, static_cast<hipStream_t>(stream));
 }
 
+int pa_flare_backward_points(int dtype, const pa_shape *shape, const void *row_weights, const void *column_weights,
+                             const void *values, const void *d_out_x, const float *z, const float *d_num,
+                             const float *d_den, void *d_scores, void *d_values, void *stream) {
+  int rc = check_shape(dtype, shape);
+  if (rc) return rc;
+  if (dtype == PA_BF16_W8) return PA_ERR_UNSUPPORTED;
+  if (pa::flare::backward_tile_rows(*shape) == 0) return PA_ERR_UNSUPPORTED;
+  if (!row_weights || !column_weights || !values || !d_out_x || !z || !d_num || !d_den || !d_scores || !d_values)
+    return PA_ERR_NULL;
+  return pa::flare::backward_points(dtype, *shape, row_weights, column_weights, values, d_out_x, z, d_num, d_den,
+                                    d_scores, d_values, static_cast<hipStream_t>(stream));
+}
+
 int pa_mfma_pack_tokens(const pa_shape *shape, const float *out_slice_token, void *tokp, void *stream) {
   int rc = check_shape(PA_BF16, shape);
   if (rc) return rc;

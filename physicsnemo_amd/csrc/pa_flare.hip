@@ -8,6 +8,7 @@
 //   column_max_kernel(s)     m[b,h,s] = max_n A[b,n,h,s]                     two passes, like the slice aggregation
 //   column_weights_kernel    wc = exp(A - m)                                   -> pa_slice_reduce(wc, v) gives z
 //   softmax_rows_kernel      A <- softmax_s(A) in place                        -> pa_deslice_project(A, z) gives y
+//   flare_backward_kernel    per-point part of the backward pass: d A, d v
 // fp32 arithmetic, fp32 or bf16 storage, natural layouts.
 #include "pa_common.h"
 #include "pa_host.h"
@@ -78,7 +79,128 @@ __global__ __launch_bounds__(256) void softmax_rows_kernel(T *__restrict__ a, in
   }
 }
 
+// ------------------------------------------------------------------------------------------------
+// flare_backward_kernel: per-point part of the FLARE backward pass.  grid (row tiles of R points per batch, H).
+// With wr = softmax_s(A) (hand-back weights), wc = exp(A - max_n A) (gather weights), z the gathered summaries,
+// g = d y, and d num / d den the gradients of the un-normalised gather sums (z = num / den):
+//   d wr[n,s] = g[n,:] . z[s,:];        d A += wr (d wr - sum_s wr d wr)          (row softmax backward)
+//   d wc[n,s] = v[n,:] . d num[s,:] + d den[s];   d A += wc d wc                   (the column shift max_n A has no
+//                                                                                  gradient: z does not depend on it)
+//   d v[n,:]  = sum_s wc[n,s] d num[s,:]
+// LDS: the head's tables z, d num (row stride D+1), d den; the tile's rows of v, g (row stride D+1) and wr, wc, d wr,
+// wc d wc (row stride S+1).  R is a power of two <= 32; 256 / R threads share a row in the row reduction.
+// ------------------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void flare_backward_kernel(
+    const T *__restrict__ wr, const T *__restrict__ wc, const T *__restrict__ v, const T *__restrict__ g,
+    const float *__restrict__ z, const float *__restrict__ d_num, const float *__restrict__ d_den,
+    T *__restrict__ d_a, T *__restrict__ d_v, int64_t N, int H, int D, int S, int R, int tiles_per_batch) {
+  extern __shared__ float lds[];
+  const int D1 = D + 1, S1 = S + 1;
+  float *zt = lds;               // S * D1
+  float *dn = zt + S * D1;       // S * D1
+  float *dd = dn + S * D1;       // S
+  float *vl = dd + S;            // R * D1
+  float *gl = vl + R * D1;       // R * D1
+  float *wrl = gl + R * D1;      // R * S1
+  float *wcl = wrl + R * S1;     // R * S1
+  float *dwl = wcl + R * S1;     // R * S1: d wr, then d A
+  float *dcl = dwl + R * S1;     // R * S1: wc d wc
+  const int t = threadIdx.x;
+  const int h = blockIdx.y;
+  const int b = blockIdx.x / tiles_per_batch;
+  const int64_t n0 = (int64_t)(blockIdx.x % tiles_per_batch) * R;
+  const int rows = (int)min((int64_t)R, N - n0);
+  const int64_t m0 = (int64_t)b * N + n0;
+  const int HD = H * D, HS = H * S;
+  const int64_t bh = (int64_t)b * H + h;
+  for (int i = t; i < S * D; i += 256) {
+    const int s = i / D, d = i - s * D;
+    zt[s * D1 + d] = z[bh * S * D + i];
+    dn[s * D1 + d] = d_num[bh * S * D + i];
+  }
+  for (int i = t; i < S; i += 256) dd[i] = d_den[bh * S + i];
+  for (int i = t; i < R * D; i += 256) {
+    const int r = i / D, d = i - r * D;
+    const bool ok = r < rows;
+    const int64_t off = (m0 + r) * HD + h * D + d;
+    vl[r * D1 + d] = ok ? load_as_f32(v + off) : 0.f;
+    gl[r * D1 + d] = ok ? load_as_f32(g + off) : 0.f;
+  }
+  for (int i = t; i < R * S; i += 256) {
+    const int r = i / S, s = i - r * S;
+    const bool ok = r < rows;
+    const int64_t off = (m0 + r) * HS + h * S + s;
+    wrl[r * S1 + s] = ok ? load_as_f32(wr + off) : 0.f;
+    wcl[r * S1 + s] = ok ? load_as_f32(wc + off) : 0.f;
+  }
+  __syncthreads();
+  for (int i = t; i < R * S; i += 256) {
+    const int r = i / S, s = i - r * S;
+    const float *vr = vl + r * D1, *gr = gl + r * D1, *zr = zt + s * D1, *nr = dn + s * D1;
+    float dwr = 0.f, dwc = dd[s];
+    for (int d = 0; d < D; ++d) {
+      dwr = fmaf(gr[d], zr[d], dwr);
+      dwc = fmaf(vr[d], nr[d], dwc);
+    }
+    dwl[r * S1 + s] = dwr;
+    dcl[r * S1 + s] = wcl[r * S1 + s] * dwc;
+  }
+  __syncthreads();
+  const int tpr = 256 / R;
+  const int r_own = t / tpr, j_own = t - r_own * tpr;
+  float dot = 0.f;
+  for (int s = j_own; s < S; s += tpr) dot = fmaf(wrl[r_own * S1 + s], dwl[r_own * S1 + s], dot);
+  for (int off = tpr >> 1; off > 0; off >>= 1) dot += __shfl_xor(dot, off, 64);
+  for (int s = j_own; s < S; s += tpr)
+    dwl[r_own * S1 + s] = wrl[r_own * S1 + s] * (dwl[r_own * S1 + s] - dot) + dcl[r_own * S1 + s];
+  __syncthreads();
+  for (int i = t; i < rows * S; i += 256) {
+    const int r = i / S, s = i - r * S;
+    store_from_f32(d_a + (m0 + r) * HS + h * S + s, dwl[r * S1 + s]);
+  }
+  for (int i = t; i < rows * D; i += 256) {
+    const int r = i / D, d = i - r * D;
+    const float *wcr = wcl + r * S1;
+    float acc = 0.f;
+    for (int s = 0; s < S; ++s) acc = fmaf(wcr[s], dn[s * D1 + d], acc);
+    store_from_f32(d_v + (m0 + r) * HD + h * D + d, acc);
+  }
+}
+
 int64_t column_max_chunks(const pa_shape &s) { return (s.N + kChunkRows - 1) / kChunkRows; }
+
+int backward_tile_rows(const pa_shape &s) {
+  const size_t fixed = (size_t)(2 * s.S * (s.D + 1) + s.S) * 4;
+  for (int R = 32; R >= 4; R >>= 1) {
+    const size_t per = (size_t)R * (2 * (s.D + 1) + 4 * (s.S + 1)) * 4;
+    if (fixed + per <= 120 * 1024) return R;
+  }
+  return 0;
+}
+
+template <typename T>
+static int backward_points_t(const pa_shape &s, const void *wr, const void *wc, const void *v, const void *g,
+                             const float *z, const float *d_num, const float *d_den, void *d_a, void *d_v,
+                             hipStream_t st) {
+  const int R = backward_tile_rows(s);
+  if (R == 0) return PA_ERR_UNSUPPORTED;
+  const size_t lds = (size_t)(2 * s.S * (s.D + 1) + s.S + (size_t)R * (2 * (s.D + 1) + 4 * (s.S + 1))) * 4;
+  int rc = allow_dynamic_lds(flare_backward_kernel<T>, lds);
+  if (rc) return rc;
+  const int tiles = (int)((s.N + R - 1) / R);
+  hipLaunchKernelGGL((flare_backward_kernel<T>), dim3((unsigned)(tiles * s.B), (unsigned)s.H), dim3(256), lds, st,
+                     static_cast<const T *>(wr), static_cast<const T *>(wc), static_cast<const T *>(v),
+                     static_cast<const T *>(g), z, d_num, d_den, static_cast<T *>(d_a), static_cast<T *>(d_v), s.N,
+                     (int)s.H, (int)s.D, (int)s.S, R, tiles);
+  return launch_status();
+}
+
+int backward_points(int dtype, const pa_shape &s, const void *wr, const void *wc, const void *v, const void *g,
+                    const float *z, const float *d_num, const float *d_den, void *d_a, void *d_v, hipStream_t st) {
+  return dtype == PA_F32 ? backward_points_t<float>(s, wr, wc, v, g, z, d_num, d_den, d_a, d_v, st)
+                         : backward_points_t<bf16>(s, wr, wc, v, g, z, d_num, d_den, d_a, d_v, st);
+}
 
 template <typename T>
 static int column_weights_t(const pa_shape &s, const void *a, float *partial, float *colmax, void *wc, hipStream_t st) {

@@ -111,6 +111,9 @@ int column_weights(int dtype, const pa_shape &s, const void *a, float *partial, 
                    hipStream_t st);
 // temperature: NULL, or (H) float32 -- the entries are then divided by clamp(temperature[head], 0.5, 5) first
 int softmax_rows(int dtype, const pa_shape &s, void *a, const float *temperature, hipStream_t st);
+int backward_tile_rows(const pa_shape &s);
+int backward_points(int dtype, const pa_shape &s, const void *wr, const void *wc, const void *v, const void *g,
+                    const float *z, const float *d_num, const float *d_den, void *d_a, void *d_v, hipStream_t st);
 }  // namespace flare
 
 namespace gale {

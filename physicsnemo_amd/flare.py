@@ -13,7 +13,9 @@ PhysicsAttention layer with two normalisations of one score matrix, so it runs o
   z      exp(A - max_n A) (``pa_flare_column_weights``), then the slice aggregation kernels
   y      row softmax of A in place (``pa_flare_softmax_rows``), then deslice + out_linear
 
-Forward only: the backward kernels do not cover this layer.  ``use_te`` is accepted and ignored.
+With gradients required ``autograd.FlareFunction`` runs the same kernels forward and, backward, the per-point FLARE
+kernel plus the layer family's row / weight-gradient GEMMs; the weight composition is then done with tensor ops under
+autograd so the gradients reach q_global, self_k, self_v and in_project_x.  ``use_te`` is accepted and ignored.
 """
 from __future__ import annotations
 
@@ -21,6 +23,7 @@ import torch
 import torch.nn as nn
 
 from . import functional as PF
+from .autograd import FlareFunction
 
 
 class FLARE(nn.Module):
@@ -65,6 +68,20 @@ class FLARE(nn.Module):
         self._cache = {"stamp": stamp, "params": params}
         return params
 
+    def _composed(self, device: torch.device):
+        """(scores weight (H*S, C), scores bias, values weight (H*D, C), values bias) as differentiable float32
+        functions of the parameters."""
+        H, D, S, C = self.heads, self.dim_head, self.n_global_queries, self.dim
+        g = self.q_global.to(device=device, dtype=torch.float32).view(H, S, D)
+        wx_h = self.in_project_x.weight.float().view(H, D, C)
+        bx_h = self.in_project_x.bias.float().view(H, D)
+        gk = g @ self.self_k.weight.float()
+        w_a = torch.einsum("hsd,hdc->hsc", gk, wx_h).reshape(H * S, C)
+        b_a = (torch.einsum("hsd,hd->hs", gk, bx_h) + g @ self.self_k.bias.float()).reshape(-1)
+        w_v = torch.einsum("ed,hdc->hec", self.self_v.weight.float(), wx_h).reshape(H * D, C)
+        b_v = (torch.einsum("ed,hd->he", self.self_v.weight.float(), bx_h) + self.self_v.bias.float()).reshape(-1)
+        return w_a, b_a, w_v, b_v
+
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         if x.ndim != 3:
             raise ValueError(f"Expected 3D input tensor (B, N, C), got {x.ndim}D tensor with shape {tuple(x.shape)}")
@@ -72,8 +89,7 @@ class FLARE(nn.Module):
             raise ValueError(f"Expected input feature dimension {self.dim}, got {x.shape[-1]}")
         if not x.is_cuda:
             raise RuntimeError("physicsnemo_amd FLARE runs on GPU tensors only (no CPU fallback)")
-        if torch.is_grad_enabled() and (x.requires_grad or any(p.requires_grad for p in self.parameters())):
-            raise NotImplementedError("the backward kernels do not cover FLARE; run under torch.no_grad()")
+        needs_grad = torch.is_grad_enabled() and (x.requires_grad or any(p.requires_grad for p in self.parameters()))
         out_dtype = None
         if torch.is_autocast_enabled("cuda"):
             ac = torch.get_autocast_dtype("cuda")
@@ -88,6 +104,11 @@ class FLARE(nn.Module):
         B, N, C = x.shape
         H, D, S = self.heads, self.dim_head, self.n_global_queries
         dims = PF.LayerDims(B, N, C, H, D, S)
+        if needs_grad:
+            with torch.autocast("cuda", enabled=False):
+                w_a, b_a, w_v, b_v = self._composed(x.device)
+            y = FlareFunction.apply(x, dims, w_a, b_a, w_v, b_v, self.out_linear.weight, self.out_linear.bias)
+            return self.out_dropout(y if out_dtype is None else y.to(out_dtype))
         p = self.kernel_params(x.dtype, x.device)
         scores = PF.rows_gemm(x, p["scores_weight"], p["scores_bias"], dims, C, H * S).view(B, N, H, S)
         values = PF.rows_gemm(x, p["values_weight"], p["values_bias"], dims, C, H * D)

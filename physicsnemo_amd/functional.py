@@ -564,3 +564,15 @@ def flare_softmax_rows_(scores, dims: LayerDims):
     _lib.check(_lib.load().pa_flare_softmax_rows(_lib.dtype_code(scores.dtype), byref(dims.c()), scores.data_ptr(),
                                                  _lib.current_stream_ptr(scores.device)), "pa_flare_softmax_rows")
     return scores
+
+
+def flare_backward_points(row_w, col_w, values, d_out_x, z, d_num, d_den, dims: LayerDims):
+    """Per-point part of the FLARE backward pass: returns (d scores (B,N,H,S), d values (B,N,H*D))."""
+    _need_cuda(row_w, col_w, values, d_out_x, z, d_num, d_den)
+    d_scores = torch.empty_like(row_w)
+    d_values = torch.empty_like(values)
+    _lib.check(_lib.load().pa_flare_backward_points(
+        _lib.dtype_code(row_w.dtype), byref(dims.c()), row_w.data_ptr(), col_w.data_ptr(), values.data_ptr(),
+        d_out_x.data_ptr(), z.data_ptr(), d_num.data_ptr(), d_den.data_ptr(), d_scores.data_ptr(), d_values.data_ptr(),
+        _lib.current_stream_ptr(row_w.device)), "pa_flare_backward_points")
+    return d_scores, d_values

@@ -1,5 +1,5 @@
-"""FLARE attention layer on the HIP kernels against the oracle.  Bars: fp32 rtol 1e-4 with atol = 1e-4 * max|ref|;
-bf16 rel-L2 <= 1e-2 against the fp32 oracle."""
+"""FLARE attention layer on the HIP kernels against the oracle (and autograd over it).  Bars: fp32 rtol 1e-4 (gradients
+2e-4) with atol = rtol * max|ref|; bf16 output rel-L2 <= 1e-2, bf16 gradients <= 5e-2 against the fp32 oracle."""
 import pytest
 import torch
 
@@ -73,7 +73,50 @@ def test_flare_errors():
         hip(x[0])
     with pytest.raises(ValueError, match="feature dimension"), torch.no_grad():
         hip(x[..., :16])
-    with pytest.raises(NotImplementedError):
-        hip(x)  # parameters require grad and grad mode is on
     with pytest.raises(RuntimeError, match="GPU"), torch.no_grad():
         hip.cpu()(x.cpu())
+
+
+def _flare_grads(module, x, probe):
+    module.zero_grad(set_to_none=True)
+    x = x.clone().requires_grad_(True)
+    y = module(x)
+    (y.float() * probe.to(y.device)).sum().backward()
+    out = {"x": x.grad}
+    out.update({name: p.grad for name, p in module.named_parameters()})
+    return y, out
+
+
+@pytest.mark.parametrize("dim,heads,dim_head,S,B,N", [(32, 4, 8, 8, 2, 300), (64, 2, 32, 64, 1, 1000), (48, 3, 16, 20, 3, 77)])
+def test_fp32_flare_gradients(dim, heads, dim_head, S, B, N):
+    announce("fp32 FLARE backward", dim, heads, dim_head, S, B, N)
+    ref, hip = _pair(dim, heads, dim_head, S)
+    ref.train(), hip.train()
+    x, probe = torch.randn(B, N, dim), torch.randn(B, N, dim)
+    y_ref, want = _flare_grads(ref, x, probe)
+    y_hip, got = _flare_grads(hip, x.cuda(), probe)
+    assert_fp32_close(y_hip, y_ref, "forward y (training path)")
+    assert set(got) == set(want)
+    for name in want:
+        assert got[name] is not None and got[name].shape == want[name].shape, name
+        assert_fp32_close(got[name], want[name], f"grad {name}", rtol=2e-4)
+
+
+def test_bf16_flare_gradients():
+    announce("bf16 FLARE backward (autocast)")
+    ref, hip = _pair(256, 8, 32, 64)
+    ref.train(), hip.train()
+    torch.manual_seed(5)
+    x, probe = torch.randn(2, 2048, 256), torch.randn(2, 2048, 256)
+    _, want = _flare_grads(ref, x, probe)
+    hip.zero_grad(set_to_none=True)
+    xc = x.cuda().requires_grad_(True)
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        y = hip(xc)
+    assert y.dtype == torch.bfloat16
+    (y.float() * probe.cuda()).sum().backward()
+    got = {"x": xc.grad}
+    got.update({name: p.grad for name, p in hip.named_parameters()})
+    for name in want:
+        assert got[name] is not None and torch.isfinite(got[name]).all(), name
+        assert_rel_l2(got[name], want[name], f"bf16 FLARE grad {name}", tol=5e-2)

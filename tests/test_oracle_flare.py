@@ -66,3 +66,17 @@ def test_flare_is_equivariant_under_point_permutations_and_keeps_its_contract():
                                     "self_k.bias", "self_v.weight", "self_v.bias", "out_linear.weight",
                                     "out_linear.bias"]
     assert m.state_dict()["q_global"].shape == (1, 2, 5, 6) and m.scale == 1.0
+
+
+def test_oracle_flare_gradient_matches_finite_differences():
+    """The GPU backward test compares against autograd over the torch oracle; here that gradient is pinned by central
+    finite differences in float64."""
+    m = _flare(dim=6, heads=2, dim_head=3, S=4)
+    names = [k for k, _ in m.named_parameters()]
+    params = [p.detach().clone().requires_grad_(True) for _, p in m.named_parameters()]
+    x = torch.randn(2, 7, 6, dtype=torch.float64, requires_grad=True)
+
+    def fn(x, *ps):
+        return torch.func.functional_call(m, dict(zip(names, ps)), (x,))
+
+    assert torch.autograd.gradcheck(fn, (x, *params), eps=1e-6, atol=1e-6, rtol=1e-5)
