@@ -163,6 +163,10 @@ int pa_slice_attention(const pa_shape *shape, const pa_params *p, const float *s
 int pa_deslice_project(int dtype, const pa_shape *shape, const pa_params *p, const void *w,
                        const float *out_slice_token, void *scratch, void *y, const pa_block_tail *tail,
                        void *stream);
+/* The deslice alone (PA.py:492-495): out_x (B,N,H*D) = sum_s w[n,h,s] out_slice_token[h,s,:], heads merged; used where
+ * something other than out_linear follows (GALE_FA blends two such results first, gale.py:735-760). */
+int pa_deslice(int dtype, const pa_shape *shape, const void *w, const float *out_slice_token, void *out_x,
+               void *stream);
 
 /* ---- backward pass (general kernels; fp32 arithmetic, fp32 or bf16 storage) -------------------------
  * The reference has no backward code of its own: gradients come from autograd over PA.py:501-558

@@ -363,6 +363,39 @@ class OracleFLARE(nn.Module):
         return self.out_dropout(self.out_linear(out_x))
 
 
+class OracleGALE_FA(nn.Module):
+    """physicsnemo/nn/module/gale.py:513-762 with use_te=False, concrete_dropout=False: FLARE self-attention per point,
+    blended with a per-point cross-attention to the context (scale 1 in both), then out_linear."""
+
+    def __init__(self, dim, heads=8, dim_head=64, dropout=0.0, n_global_queries=64, context_dim=0,
+                 state_mixing_mode="weighted"):
+        super().__init__()
+        self.dim, self.heads, self.dim_head = dim, heads, dim_head
+        self.scale = 1.0
+        self.q_global = nn.Parameter(torch.randn(1, heads, n_global_queries, dim_head))
+        self.in_project_x = nn.Linear(dim, heads * dim_head)
+        self.self_k = nn.Linear(dim_head, dim_head)
+        self.self_v = nn.Linear(dim_head, dim_head)
+        if context_dim > 0:
+            _GALECore._init_cross(self, dim_head, context_dim, state_mixing_mode)
+        self.out_linear = nn.Linear(heads * dim_head, dim)
+        self.out_dropout = nn.Dropout(dropout)
+
+    def forward(self, x, context=None):
+        outs = []
+        for t in x:
+            x_mid = split_heads(self.in_project_x(t), self.heads, self.dim_head).permute(0, 2, 1, 3)  # (B, H, N, D)
+            y = flare_self_attention(x_mid, self.q_global, self.self_k, self.self_v, self.scale)
+            if context is not None:
+                cross = F.scaled_dot_product_attention(self.cross_q(x_mid), self.cross_k(context),
+                                                       self.cross_v(context), scale=self.scale)
+                y = gale_mix(y, cross, self.state_mixing_mode, getattr(self, "state_mixing", None),
+                             getattr(self, "concat_project", None))
+            y = y.permute(0, 2, 1, 3).reshape(t.shape[0], t.shape[1], self.heads * self.dim_head)
+            outs.append(self.out_dropout(self.out_linear(y)))
+        return outs
+
+
 class _ProjectorCore(nn.Module):
     """Slice components and forward of the GeoTransolver context projectors
     (physicsnemo/models/geotransolver/context_projector.py:108-187, :338-378): the encoding half of the layer; returns

@@ -319,6 +319,16 @@ int pa_deslice_project(int dtype, const pa_shape *shape, const pa_params *p, con
   return rc;
 }
 
+int pa_deslice(int dtype, const pa_shape *shape, const void *w, const float *out_slice_token, void *out_x,
+               void *stream) {
+  int rc = check_shape(dtype, shape);
+  if (rc) return rc;
+  if (dtype == PA_BF16_W8) return PA_ERR_UNSUPPORTED;
+  if (!w || !out_slice_token || !out_x) return PA_ERR_NULL;
+  if (!aligned16(w) || !aligned16(out_x)) return PA_ERR_ALIGN;
+  return pa::general::deslice(dtype, *shape, w, out_slice_token, out_x, static_cast<hipStream_t>(stream));
+}
+
 int pa_rows_gemm(int dtype, const pa_shape *grid, int64_t c_in, int64_t c_out, const void *in, const void *weight,
                  const float *bias, void *out, void *stream) {
   return pa_rows_gemm_act(dtype, grid, c_in, c_out, in, weight, bias, 0, out, stream);

@@ -120,3 +120,113 @@ class FLARE(nn.Module):
         PF.flare_softmax_rows_(scores, dims)
         y = PF.deslice_project(scores, z, p, dims)
         return self.out_dropout(y if out_dtype is None else y.to(out_dtype))
+
+
+class GALE_FA(nn.Module):
+    """GALE with FLARE self-attention (reference gale.py:513-762): the FLARE two-pass self-attention of every point,
+    optionally blended with a per-point cross-attention to a context (B, H, S_c, D_c), then out_linear.  Same
+    constructor arguments, parameter names and ``forward(x: tuple, context=None) -> list`` as the reference.
+
+    Every stage is a row GEMM or a slice-weight kernel of the layer family: the cross-attention of a point is
+    ``softmax_u(q_n . k_u) v_u`` with scale 1 -- scores from a row GEMM whose weight folds in_project_x, cross_q and the
+    context's keys (one weight per batch element), an in-place row softmax, and the deslice kernel with the context's
+    values as slice tokens.  Forward only."""
+
+    def __init__(self, dim: int, heads: int = 8, dim_head: int = 64, dropout: float = 0.0, n_global_queries: int = 64,
+                 use_te: bool = False, context_dim: int = 0, concrete_dropout: bool = False,
+                 state_mixing_mode: str = "weighted"):
+        super().__init__()
+        from .gale import _gale_cross_init
+
+        if concrete_dropout:
+            raise NotImplementedError("ConcreteDropout is a training-time regulariser; the HIP layer has none")
+        self.use_te = use_te
+        self.dim, self.heads, self.dim_head, self.n_global_queries = dim, heads, dim_head, n_global_queries
+        self.scale = 1.0
+        inner_dim = dim_head * heads
+        self.q_global = nn.Parameter(torch.randn(1, heads, n_global_queries, dim_head))
+        self.in_project_x = nn.Linear(dim, inner_dim)
+        self.self_k = nn.Linear(dim_head, dim_head)
+        self.self_v = nn.Linear(dim_head, dim_head)
+        if context_dim > 0:
+            _gale_cross_init(self, dim_head, context_dim, state_mixing_mode)
+        self.context_dim = context_dim
+        self.out_linear = nn.Linear(inner_dim, dim)
+        self.out_dropout = nn.Dropout(dropout)
+        self._cache: dict = {}
+
+    kernel_params = FLARE.kernel_params
+
+    def _self_attention(self, x: torch.Tensor, p: dict, dims: PF.LayerDims) -> torch.Tensor:
+        """FLARE two-pass attention -> (B, N, H*D), before out_linear."""
+        B, N, C, H, D, S = dims.B, dims.N, dims.C, dims.H, dims.D, dims.S
+        scores = PF.rows_gemm(x, p["scores_weight"], p["scores_bias"], dims, C, H * S).view(B, N, H, S)
+        values = PF.rows_gemm(x, p["values_weight"], p["values_bias"], dims, C, H * D)
+        weights, _ = PF.flare_column_weights(scores, dims)
+        tok, norm = PF.slice_reduce(weights, values, dims)
+        z = (tok * (norm / (norm - 1e-2)).unsqueeze(-1)).contiguous()
+        return PF.deslice(PF.flare_softmax_rows_(scores, dims), z, dims)
+
+    def _cross_attention(self, x: torch.Tensor, context: torch.Tensor, dims: PF.LayerDims) -> torch.Tensor:
+        """Per-point cross-attention to the context (reference :735-744) -> (B, N, H*D)."""
+        B, N, C, H, D = dims.B, dims.N, dims.C, dims.H, dims.D
+        Sc = context.shape[2]
+        with torch.no_grad():
+            ctx = context.double()
+            k = ctx @ self.cross_k.weight.double().t() + self.cross_k.bias.double()      # (B, H, Sc, D)
+            v = (ctx @ self.cross_v.weight.double().t() + self.cross_v.bias.double()).float().contiguous()
+            wx_h = self.in_project_x.weight.double().view(H, D, C)
+            bx_h = self.in_project_x.bias.double().view(H, D)
+            kq = k @ self.cross_q.weight.double()                                        # k_u . W_q: (B, H, Sc, D)
+            w_c = torch.einsum("bhud,hdc->bhuc", kq, wx_h).reshape(B, H * Sc, C)
+            b_c = (torch.einsum("bhud,hd->bhu", kq, bx_h) + k @ self.cross_q.bias.double()).reshape(B, H * Sc)
+        cdims = PF.LayerDims(B, N, C, H, D, Sc)
+        one = PF.LayerDims(1, N, C, H, D, Sc)
+        scores = torch.empty(B, N, H, Sc, dtype=x.dtype, device=x.device)
+        for b in range(B):  # the score weight holds the batch element's keys
+            scores[b] = PF.rows_gemm(x[b:b + 1], w_c[b].to(x.dtype).contiguous(), b_c[b].float().contiguous(), one, C,
+                                     H * Sc).view(N, H, Sc)
+        return PF.deslice(PF.flare_softmax_rows_(scores, cdims), v, cdims)
+
+    def _mix(self, self_x: torch.Tensor, cross_x: torch.Tensor, dims: PF.LayerDims) -> torch.Tensor:
+        if self.state_mixing_mode == "weighted":
+            m = torch.sigmoid(self.state_mixing.detach().float())
+            return (m * self_x.float() + (1 - m) * cross_x.float()).to(self_x.dtype)
+        B, N, H, D = dims.B, dims.N, dims.H, dims.D
+        cat = torch.cat([self_x.view(B, N, H, D), cross_x.view(B, N, H, D)], dim=-1).reshape(B, N * H, 2 * D).contiguous()
+        lin = self.concat_project[0]
+        out = PF.rows_gemm(cat, lin.weight.detach().to(cat.dtype).contiguous(), lin.bias.detach().float().contiguous(),
+                           PF.LayerDims(B, N * H, 2 * D, 1, 1, 1), 2 * D, D, gelu=True)
+        return out.view(B, N, H * D)
+
+    def forward(self, x: tuple, context: torch.Tensor | None = None) -> list:
+        if isinstance(x, torch.Tensor):
+            raise TypeError("GALE_FA takes a tuple of input tensors")
+        if len(x) == 0:
+            raise ValueError("Expected non-empty tuple of input tensors")
+        outs = []
+        for i, t in enumerate(x):
+            if t.ndim != 3:
+                raise ValueError(f"Expected 3D input tensor (B, N, C) at index {i}, "
+                                 f"got {t.ndim}D tensor with shape {tuple(t.shape)}")
+            if not t.is_cuda:
+                raise RuntimeError("physicsnemo_amd GALE_FA runs on GPU tensors only (no CPU fallback)")
+            if torch.is_grad_enabled() and (t.requires_grad or any(p.requires_grad for p in self.parameters())):
+                raise NotImplementedError("the backward kernels do not cover GALE_FA; run under torch.no_grad()")
+            if torch.is_autocast_enabled("cuda") and torch.get_autocast_dtype("cuda") == torch.bfloat16:
+                t = t.to(torch.bfloat16)
+            if t.dtype not in (torch.float32, torch.bfloat16):
+                t = t.float()
+            t = t.contiguous()
+            B, N, C = t.shape
+            dims = PF.LayerDims(B, N, C, self.heads, self.dim_head, self.n_global_queries)
+            p = self.kernel_params(t.dtype, t.device)
+            y = self._self_attention(t, p, dims)
+            if context is not None:
+                if self.context_dim <= 0:
+                    raise ValueError("this GALE_FA was built without cross-attention (context_dim = 0)")
+                y = self._mix(y, self._cross_attention(t, context.to(t.device), dims), dims)
+            out = PF.rows_gemm(y, p["out_linear_weight"].view(C, -1), p["out_linear_bias"],
+                               PF.LayerDims(B, N, y.shape[-1], 1, 1, 1), y.shape[-1], C)
+            outs.append(self.out_dropout(out))
+        return outs

@@ -576,3 +576,12 @@ def flare_backward_points(row_w, col_w, values, d_out_x, z, d_num, d_den, dims: 
         d_out_x.data_ptr(), z.data_ptr(), d_num.data_ptr(), d_den.data_ptr(), d_scores.data_ptr(), d_values.data_ptr(),
         _lib.current_stream_ptr(row_w.device)), "pa_flare_backward_points")
     return d_scores, d_values
+
+
+def deslice(w, tok_out, dims: LayerDims):
+    """out_x (B, N, H*D) = sum_s w[n,h,s] tok_out[h,s,:] (heads merged), without the output projection."""
+    _need_cuda(w, tok_out)
+    out_x = torch.empty(dims.B, dims.N, dims.H * dims.D, dtype=w.dtype, device=w.device)
+    _lib.check(_lib.load().pa_deslice(_lib.dtype_code(w.dtype), byref(dims.c()), w.data_ptr(), tok_out.data_ptr(),
+                                      out_x.data_ptr(), _lib.current_stream_ptr(w.device)), "pa_deslice")
+    return out_x

@@ -197,8 +197,8 @@ class GALEStructuredMesh3D(_GALEForwardMixin, PhysicsAttentionStructuredMesh3D):
 
 class GALEBlock(nn.Module):
     """LayerNorm -> GALE attention (with the shared context) -> +residual -> LayerNorm -> MLP -> +residual, for every
-    tensor of the input tuple (reference gale.py:764-1030).  ``attention_type="GALE_FA"`` and ``concrete_dropout`` are not
-    served.  The LayerNorms, the block MLP and its residual add run on the library kernels of the Transolver block."""
+    tensor of the input tuple (reference gale.py:764-1030).  ``attention_type="GALE_FA"`` builds the FLARE form of the
+    attention (inference only); ``concrete_dropout`` is not served.  The LayerNorms, the block MLP and its residual add run on the library kernels of the Transolver block."""
 
     def __init__(self, num_heads: int, hidden_dim: int, dropout: float, act: str = "gelu", mlp_ratio: int = 4,
                  last_layer: bool = False, out_dim: int = 1, slice_num: int = 32, use_te: bool = False,
@@ -209,15 +209,19 @@ class GALEBlock(nn.Module):
 
         self.last_layer = last_layer
         self.ln_1 = nn.LayerNorm(hidden_dim)
-        if attention_type == "GALE_FA":
-            raise NotImplementedError("attention_type='GALE_FA' (GALE with FLARE self-attention) is not served")
-        if attention_type != "GALE":
+        if attention_type not in ("GALE", "GALE_FA"):
             raise ValueError(f"Invalid attention type: {attention_type}. Expected 'GALE' or 'GALE_FA'.")
         if concrete_dropout:
             raise NotImplementedError("ConcreteDropout is a training-time regulariser; the HIP block has none")
         common = dict(heads=num_heads, dim_head=hidden_dim // num_heads, dropout=dropout, slice_num=slice_num,
                       use_te=use_te, plus=plus, context_dim=context_dim, state_mixing_mode=state_mixing_mode)
-        if spatial_shape is None:
+        if attention_type == "GALE_FA":  # FLARE self-attention; inference only (reference :932-943)
+            from .flare import GALE_FA
+
+            self.Attn = GALE_FA(hidden_dim, heads=num_heads, dim_head=hidden_dim // num_heads, dropout=dropout,
+                                n_global_queries=slice_num, use_te=use_te, context_dim=context_dim,
+                                state_mixing_mode=state_mixing_mode)
+        elif spatial_shape is None:
             self.Attn = GALE(hidden_dim, **common)
         elif len(spatial_shape) == 2:
             self.Attn = GALEStructuredMesh2D(hidden_dim, spatial_shape=tuple(int(v) for v in spatial_shape), **common)

@@ -120,3 +120,44 @@ def test_bf16_flare_gradients():
     for name in want:
         assert got[name] is not None and torch.isfinite(got[name]).all(), name
         assert_rel_l2(got[name], want[name], f"bf16 FLARE grad {name}", tol=5e-2)
+
+
+@pytest.mark.parametrize("mode,dim,heads,dim_head,S,B,N,Sc,Dc", [
+    ("weighted", 32, 4, 8, 8, 2, 300, 5, 7),
+    ("concat_project", 48, 3, 16, 20, 3, 77, 9, 4),
+    ("weighted", 64, 2, 32, 64, 1, 1000, 1, 16),
+])
+def test_fp32_gale_fa_matches_oracle(mode, dim, heads, dim_head, S, B, N, Sc, Dc):
+    announce("fp32 GALE_FA", mode, dim, heads, dim_head, S, B, N, Sc, Dc)
+    torch.manual_seed(0)
+    kw = dict(heads=heads, dim_head=dim_head, n_global_queries=S, context_dim=Dc, state_mixing_mode=mode)
+    ref, hip = to.OracleGALE_FA(dim, **kw).eval(), pn.GALE_FA(dim, **kw).eval()
+    if mode == "weighted":
+        with torch.no_grad():
+            ref.state_mixing.fill_(0.3)
+    hip.load_state_dict(ref.state_dict())
+    hip.cuda()
+    x1, x2, ctx = torch.randn(B, N, dim), torch.randn(B, N, dim), torch.randn(B, heads, Sc, Dc)
+    with torch.no_grad():
+        want = ref((x1, x2), ctx)
+        got = hip((x1.cuda(), x2.cuda()), ctx.cuda())
+        for g, w in zip(got, want):
+            assert_fp32_close(g, w, "GALE_FA y")
+        assert_fp32_close(hip((x1.cuda(),))[0], ref((x1,))[0], "GALE_FA y without context")
+
+
+def test_bf16_gale_fa():
+    announce("bf16 GALE_FA")
+    torch.manual_seed(0)
+    kw = dict(heads=8, dim_head=32, n_global_queries=64, context_dim=32)
+    ref, hip = to.OracleGALE_FA(256, **kw).eval(), pn.GALE_FA(256, **kw).eval()
+    hip.load_state_dict(ref.state_dict())
+    hip.cuda()
+    x, ctx = torch.randn(2, 4096, 256), torch.randn(2, 8, 48, 32)
+    with torch.no_grad():
+        want = ref((x,), ctx)[0]
+        got = hip((x.cuda().bfloat16(),), ctx.cuda())[0]
+    assert got.dtype == torch.bfloat16
+    assert_rel_l2(got, want, "bf16 GALE_FA y", tol=1e-2)
+    with pytest.raises(NotImplementedError):
+        hip((x.cuda(),), ctx.cuda())

@@ -314,7 +314,9 @@ def test_bf16_gale_block_on_the_fused_kernels():
             got = hip((x.cuda(),), ctx.cuda())[0]
     assert got.dtype == torch.bfloat16
     assert_rel_l2(got, want, "bf16 GALE block y", tol=1e-2)
-    with pytest.raises(NotImplementedError):
-        pn.GALEBlock(8, 256, 0.0, attention_type="GALE_FA")
+    fa = pn.GALEBlock(8, 256, 0.0, attention_type="GALE_FA", slice_num=32, context_dim=32).eval().cuda()
+    with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
+        out = fa((x.cuda(),), ctx.cuda())[0]
+    assert isinstance(fa.Attn, pn.GALE_FA) and out.shape == x.shape and torch.isfinite(out).all()
     with pytest.raises(ValueError, match="Invalid attention type"):
         pn.GALEBlock(8, 256, 0.0, attention_type="other")

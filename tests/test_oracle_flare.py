@@ -80,3 +80,32 @@ def test_oracle_flare_gradient_matches_finite_differences():
         return torch.func.functional_call(m, dict(zip(names, ps)), (x,))
 
     assert torch.autograd.gradcheck(fn, (x, *params), eps=1e-6, atol=1e-6, rtol=1e-5)
+
+
+def test_gale_fa_special_cases():
+    """GALE_FA (gale.py:654-762): no context = the FLARE layer; gate -> 1 / 0 = self only / cross only; with one
+    context token the per-point cross-attention returns cross_v(context) whatever the queries are (scale 1 plays no
+    role then), so the cross-only output is W_out . concat_h(cross_v(ctx_h)) + b_out at every point."""
+    torch.manual_seed(8)
+    m = to.OracleGALE_FA(12, heads=2, dim_head=6, n_global_queries=5, context_dim=7).double().eval()
+    flare = to.OracleFLARE(12, heads=2, dim_head=6, n_global_queries=5).double().eval()
+    flare.load_state_dict({k: v for k, v in m.state_dict().items() if k in flare.state_dict()})
+    assert list(m.state_dict())[:2] == ["q_global", "state_mixing"] and list(m.state_dict())[-2:] == [
+        "out_linear.weight", "out_linear.bias"]
+    x = torch.randn(2, 9, 12, dtype=torch.float64)
+    ctx = torch.randn(2, 2, 1, 7, dtype=torch.float64)
+    with torch.no_grad():
+        torch.testing.assert_close(m((x,))[0], flare(x))
+        m.state_mixing.fill_(40.0)
+        torch.testing.assert_close(m((x,), ctx)[0], flare(x))
+        m.state_mixing.fill_(-40.0)
+        v = ctx[:, :, 0, :] @ m.cross_v.weight.t() + m.cross_v.bias
+        want = v.reshape(2, 1, 12) @ m.out_linear.weight.t() + m.out_linear.bias
+        torch.testing.assert_close(m((x,), ctx)[0], want.expand(2, 9, 12))
+        # several context tokens: explicit softmax at scale 1 over the context axis
+        ctx4 = torch.randn(2, 2, 4, 7, dtype=torch.float64)
+        xm = m.in_project_x(x).reshape(2, 9, 2, 6).permute(0, 2, 1, 3)
+        q, k, vv = m.cross_q(xm), m.cross_k(ctx4), m.cross_v(ctx4)
+        cross = torch.softmax(q @ k.transpose(-1, -2), dim=-1) @ vv
+        want4 = cross.permute(0, 2, 1, 3).reshape(2, 9, 12) @ m.out_linear.weight.t() + m.out_linear.bias
+        torch.testing.assert_close(m((x,), ctx4)[0], want4)
