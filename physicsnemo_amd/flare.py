@@ -24,6 +24,7 @@ import torch.nn as nn
 
 from . import functional as PF
 from .autograd import FlareFunction
+from .transolver import Mlp, Transolver, TransolverBlock
 
 
 class FLARE(nn.Module):
@@ -67,6 +68,14 @@ class FLARE(nn.Module):
             }
         self._cache = {"stamp": stamp, "params": params}
         return params
+
+    def forward_block(self, x: torch.Tensor, residual: torch.Tensor, ln: nn.LayerNorm):
+        """Layer + the caller block's ``+ residual`` and following LayerNorm (flare.py:98-99): (fx_new, LayerNorm(fx_new))
+        with the add and the LayerNorm in one library kernel."""
+        y = self.forward(x).contiguous()
+        return PF.residual_layernorm(y, residual=residual.to(y.dtype).contiguous(),
+                                     ln_weight=ln.weight.detach().float().contiguous(),
+                                     ln_bias=ln.bias.detach().float().contiguous(), ln_eps=ln.eps)
 
     def _composed(self, device: torch.device):
         """(scores weight (H*S, C), scores bias, values weight (H*D, C), values bias) as differentiable float32
@@ -230,3 +239,48 @@ class GALE_FA(nn.Module):
                                PF.LayerDims(B, N, y.shape[-1], 1, 1, 1), y.shape[-1], C)
             outs.append(self.out_dropout(out))
         return outs
+
+
+# ---------------------------------------------------------------------------------------------------
+# the FLARE model (physicsnemo/models/flare/flare.py): Transolver with FLARE blocks
+# ---------------------------------------------------------------------------------------------------
+class FLAREBlock(TransolverBlock):
+    """LayerNorm -> FLARE attention -> +residual -> LayerNorm -> MLP -> +residual [-> LayerNorm -> Linear]
+    (reference flare.py:37-104); the chaining, LayerNorm and block-MLP kernels are the Transolver block's."""
+
+    def __init__(self, num_heads: int, hidden_dim: int, dropout: float, act: str = "gelu", mlp_ratio: int = 4,
+                 last_layer: bool = False, out_dim: int = 1, n_global_queries: int = 32, use_te: bool = False):
+        nn.Module.__init__(self)
+        self.last_layer = last_layer
+        self.ln_1 = nn.LayerNorm(hidden_dim)
+        self.Attn = FLARE(hidden_dim, heads=num_heads, dim_head=hidden_dim // num_heads, dropout=dropout,
+                          n_global_queries=n_global_queries, use_te=use_te)
+        self.ln_mlp1 = nn.Sequential(nn.LayerNorm(hidden_dim),
+                                     Mlp(hidden_dim, hidden_dim * mlp_ratio, hidden_dim, act))
+        if last_layer:
+            self.ln_mlp2 = nn.Sequential(nn.LayerNorm(hidden_dim), nn.Linear(hidden_dim, out_dim))
+        self._mlp_cache = {}
+
+class FLAREModel(Transolver):
+    """Transolver with FLARE attention (reference flare.py:107-213, class ``FLARE`` there): same constructor
+    (without ``plus``), inputs and outputs as `Transolver`.  As in the reference the Transolver is built first, then
+    its blocks are replaced and the weight init runs again, so seeded construction consumes the generator alike."""
+
+    _mdlus_class = ("FLARE", "physicsnemo.models.flare.flare")
+
+    def __init__(self, functional_dim: int, out_dim: int, embedding_dim: int | None = None, n_layers: int = 4,
+                 n_hidden: int = 256, dropout: float = 0.0, n_head: int = 8, act: str = "gelu", mlp_ratio: int = 4,
+                 slice_num: int = 32, unified_pos: bool = False, ref: int = 8,
+                 structured_shape: tuple | None = None, time_input: bool = False, use_te: bool = False):
+        super().__init__(functional_dim=functional_dim, out_dim=out_dim, embedding_dim=embedding_dim,
+                         n_layers=n_layers, n_hidden=n_hidden, dropout=dropout, n_head=n_head, act=act,
+                         mlp_ratio=mlp_ratio, slice_num=slice_num, unified_pos=unified_pos, ref=ref,
+                         structured_shape=structured_shape, use_te=use_te, time_input=time_input, plus=False)
+        self._args.pop("plus", None)
+        self.blocks = nn.ModuleList([
+            FLAREBlock(num_heads=n_head, hidden_dim=n_hidden, dropout=dropout, act=act, mlp_ratio=mlp_ratio,
+                       last_layer=(i == n_layers - 1), out_dim=out_dim, n_global_queries=slice_num, use_te=use_te)
+            for i in range(n_layers)
+        ])
+        self.initialize_weights()
+

@@ -227,10 +227,12 @@ class Transolver(nn.Module):
         self.initialize_weights()
 
     # ---------------------------------------------------------------- .mdlus checkpoints (core/module.py:446-1070)
+    _mdlus_class = ("Transolver", "physicsnemo.models.transolver.transolver")  # class name and module in args.json
+
     def save(self, file_name: str | None = None) -> None:
         """Writes a ``.mdlus`` checkpoint the reference's ``Module.from_checkpoint`` / ``load`` accept."""
-        _ckpt.write_mdlus(file_name or "Transolver.mdlus", "Transolver", "physicsnemo.models.transolver.transolver",
-                          self._args, self.state_dict())
+        name, module = self._mdlus_class
+        _ckpt.write_mdlus(file_name or f"{name}.mdlus", name, module, self._args, self.state_dict())
 
     def load(self, file_name: str, map_location=None, strict: bool = True) -> None:
         """Loads the weights of a ``.mdlus`` checkpoint (zip or legacy tar) into this model."""
@@ -243,8 +245,8 @@ class Transolver(nn.Module):
         """Builds the model from the constructor arguments stored in a ``.mdlus`` checkpoint and loads its weights.
         ``use_te`` is the one argument the reference lets a caller override (transolver.py ``_overridable_args``)."""
         args, _, state = _ckpt.read_mdlus(file_name)
-        if args.get("__name__") != "Transolver":
-            raise IOError(f"checkpoint holds a {args.get('__name__')!r}, not a Transolver")
+        if args.get("__name__") != cls._mdlus_class[0]:
+            raise IOError(f"checkpoint holds a {args.get('__name__')!r}, not a {cls._mdlus_class[0]}")
         ctor = dict(args["__args__"])
         for key, value in (override_args or {}).items():
             if key != "use_te":

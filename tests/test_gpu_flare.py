@@ -161,3 +161,62 @@ def test_bf16_gale_fa():
     assert_rel_l2(got, want, "bf16 GALE_FA y", tol=1e-2)
     with pytest.raises(NotImplementedError):
         hip((x.cuda(),), ctx.cuda())
+
+
+# ---------------------------------------------------------------------------------------------------
+# FLARE model (Transolver with FLARE blocks) against the reference's golden outputs
+# ---------------------------------------------------------------------------------------------------
+import os
+
+GOLD = os.path.join(os.path.dirname(__file__), "golden")
+
+
+@pytest.mark.parametrize("kind", ["structured2d", "irregular"])
+def test_flare_model_reproduces_reference_golden_output(kind):
+    """reference test/models/flare/test_flare.py:124-193: seed 0, the same inputs, its own atol; the weights come from
+    the oracle model (whose seeded construction reproduces the golden files on the CPU)."""
+    announce("FLARE model golden", kind)
+    torch.manual_seed(0)
+    if kind == "structured2d":
+        kw = dict(structured_shape=(85, 85), n_layers=8, n_hidden=64, n_head=4, mlp_ratio=1, functional_dim=1, out_dim=1,
+                  slice_num=32, ref=1, unified_pos=True)
+        ref = to.OracleFLAREModel(init="rejection", **kw)
+        a, b = torch.randn(4, 85 * 85, 1), torch.randn(4, 85, 85)
+        name, atol = "flare_2d_output.pth", 2e-3
+    else:
+        kw = dict(structured_shape=None, n_layers=8, n_hidden=64, n_head=4, mlp_ratio=1, functional_dim=2,
+                  embedding_dim=3, out_dim=1, slice_num=32, unified_pos=False)
+        ref = to.OracleFLAREModel(init="rejection", **kw)
+        a, b = torch.randn(4, 12345, 3), torch.randn(4, 12345, 2)
+        name, atol = "flare_irregular_output.pth", 1e-3
+    gold = torch.load(os.path.join(GOLD, name), weights_only=True)[0]
+    hip = pn.FLAREModel(use_te=False, **kw)
+    hip.load_state_dict(ref.state_dict())
+    hip = hip.eval().cuda()
+    with torch.no_grad():
+        out = hip(a.cuda(), b.cuda()).cpu()
+    assert out.shape == gold.shape
+    assert torch.allclose(out, gold, rtol=1e-3, atol=atol)
+    assert_fp32_close(out, gold, "FLARE model vs golden", rtol=2e-4)
+
+
+def test_flare_model_training_step_and_checkpoint(tmp_path):
+    announce("FLARE model training step")
+    torch.manual_seed(0)
+    kw = dict(functional_dim=2, out_dim=3, embedding_dim=3, n_layers=2, n_hidden=32, n_head=4, slice_num=8, mlp_ratio=2)
+    m = pn.FLAREModel(use_te=False, **kw).cuda().train()
+    ref = to.OracleFLAREModel(**kw).train()
+    ref.load_state_dict(m.state_dict())
+    fx, emb, target = torch.randn(2, 200, 2), torch.randn(2, 200, 3), torch.randn(2, 200, 3)
+    ((ref(fx, emb) - target) ** 2).mean().backward()
+    ((m(fx.cuda(), emb.cuda()) - target.cuda()) ** 2).mean().backward()
+    grads = dict(m.named_parameters())
+    for name, p in ref.named_parameters():
+        assert grads[name].grad is not None, name
+        assert_fp32_close(grads[name].grad, p.grad, f"grad {name}", rtol=5e-4)
+    path = str(tmp_path / "flare.mdlus")
+    m.save(path)
+    again = pn.FLAREModel.from_checkpoint(path).cuda().eval()
+    m.eval()
+    with torch.no_grad():
+        assert torch.equal(again(fx.cuda(), emb.cuda()), m(fx.cuda(), emb.cuda()))

@@ -43,3 +43,37 @@ def test_irregular_model_matches_reference_golden():
     assert out.shape == gold.shape == (4, 12345, 1)
     assert torch.allclose(out, gold, rtol=1e-3, atol=1e-3)
     assert (out - gold).abs().max().item() < 5e-6
+
+
+def test_flare_structured2d_model_matches_reference_golden():
+    # reference: test/models/flare/test_flare.py:124-158 (atol 2e-3)
+    from oracle.torch_oracle import OracleFLAREModel
+    torch.manual_seed(0)
+    model = OracleFLAREModel(structured_shape=(85, 85), n_layers=8, n_hidden=64, n_head=4, mlp_ratio=1,
+                             functional_dim=1, out_dim=1, slice_num=32, ref=1, unified_pos=True, init="rejection")
+    fx = torch.randn(4, 85 * 85, 1)
+    embedding = torch.randn(4, 85, 85)
+    with torch.no_grad():
+        out = model(fx, embedding)
+    gold = _load("flare_2d_output.pth")
+    assert out.shape == gold.shape == (4, 7225, 1)
+    print("flare 2d max abs diff", (out - gold).abs().max().item())
+    assert torch.allclose(out, gold, rtol=1e-3, atol=2e-3)
+    assert (out - gold).abs().max().item() < 5e-6
+
+
+def test_flare_irregular_model_matches_reference_golden():
+    # reference: test/models/flare/test_flare.py:161-193 (atol 1e-3)
+    from oracle.torch_oracle import OracleFLAREModel
+    torch.manual_seed(0)
+    model = OracleFLAREModel(structured_shape=None, n_layers=8, n_hidden=64, n_head=4, mlp_ratio=1, functional_dim=2,
+                             embedding_dim=3, out_dim=1, slice_num=32, unified_pos=False, init="rejection")
+    a = torch.randn(4, 12345, 3)
+    b = torch.randn(4, 12345, 2)
+    with torch.no_grad():
+        out = model(a, b)
+    gold = _load("flare_irregular_output.pth")
+    assert out.shape == gold.shape == (4, 12345, 1)
+    print("flare irregular max abs diff", (out - gold).abs().max().item())
+    assert torch.allclose(out, gold, rtol=1e-3, atol=1e-3)
+    assert (out - gold).abs().max().item() < 5e-6
