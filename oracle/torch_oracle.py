@@ -692,6 +692,82 @@ class OracleFLAREModel(OracleTransolver):
         self.apply(self._init_weights)
 
 
+class OracleGlobalContextBuilder(nn.Module):
+    """physicsnemo/models/geotransolver/context_projector.py:766-1069 without the ball-query local features
+    (include_local_features=False): the context is the geometry tokens and the global-embedding tokens, each from a
+    context projector, concatenated along the feature axis (:1047-1059)."""
+
+    def __init__(self, geometry_dim, global_dim, n_hidden, n_head, dropout=0.0, slice_num=32, plus=False,
+                 structured_shape=None):
+        super().__init__()
+        dim_head = n_hidden // n_head
+        self._context_dim = 0
+        self.local_extractors = None
+        if geometry_dim is not None:
+            if structured_shape is not None:
+                self.geometry_tokenizer = OracleStructuredContextProjector(geometry_dim, structured_shape, n_head,
+                                                                           dim_head, dropout, slice_num)
+            else:
+                self.geometry_tokenizer = OracleContextProjector(geometry_dim, n_head, dim_head, dropout, slice_num, plus)
+            self._context_dim += dim_head
+        else:
+            self.geometry_tokenizer = None
+        if global_dim is not None:
+            self.global_tokenizer = OracleContextProjector(global_dim, n_head, dim_head, dropout, slice_num, plus)
+            self._context_dim += dim_head
+        else:
+            self.global_tokenizer = None
+
+    def get_context_dim(self):
+        return self._context_dim
+
+    def build_context(self, geometry=None, global_embedding=None):
+        parts = []
+        if self.geometry_tokenizer is not None and geometry is not None:
+            parts.append(self.geometry_tokenizer(geometry))
+        if self.global_tokenizer is not None and global_embedding is not None:
+            parts.append(self.global_tokenizer(global_embedding))
+        return torch.cat(parts, dim=-1) if parts else None
+
+
+class OracleGeoTransolver(nn.Module):
+    """physicsnemo/models/geotransolver/geotransolver.py:390-766 with use_te=False, include_local_features=False,
+    attention_type="GALE", no time input: context from the builder, one preprocess Mlp per input stream, GALE blocks
+    sharing the context, one LayerNorm + Linear head per stream.  No weight re-initialisation: parameters keep the
+    default nn.Linear / orthogonal_ draws of their constructors, in construction order (:460-558)."""
+
+    def __init__(self, functional_dim, out_dim, geometry_dim=None, global_dim=None, n_layers=4, n_hidden=256,
+                 dropout=0.0, n_head=8, mlp_ratio=4, slice_num=32, plus=False, structured_shape=None,
+                 state_mixing_mode="weighted"):
+        super().__init__()
+        fdims = (functional_dim,) if isinstance(functional_dim, int) else tuple(functional_dim)
+        odims = (out_dim,) if isinstance(out_dim, int) else tuple(out_dim)
+        if len(fdims) != len(odims):
+            raise ValueError(f"functional_dim and out_dim must be the same length, but instead got {len(fdims)} and {len(odims)}")
+        self.structured_shape = structured_shape
+        self.context_builder = OracleGlobalContextBuilder(geometry_dim, global_dim, n_hidden, n_head, dropout, slice_num,
+                                                          plus, structured_shape)
+        context_dim = self.context_builder.get_context_dim()
+        self.preprocess = nn.ModuleList([OracleMlp(f, n_hidden * 2, n_hidden) for f in fdims])
+        self.n_hidden = n_hidden
+        self.blocks = nn.ModuleList([
+            OracleGALEBlock(n_head, n_hidden, dropout, mlp_ratio=mlp_ratio, slice_num=slice_num, context_dim=context_dim,
+                            spatial_shape=structured_shape, state_mixing_mode=state_mixing_mode)
+            for _ in range(n_layers)
+        ])
+        self.ln_mlp_out = nn.ModuleList([nn.Sequential(nn.LayerNorm(n_hidden), nn.Linear(n_hidden, o)) for o in odims])
+
+    def forward(self, local_embedding, local_positions=None, global_embedding=None, geometry=None):
+        single = isinstance(local_embedding, torch.Tensor)
+        streams = (local_embedding,) if single else tuple(local_embedding)
+        context = self.context_builder.build_context(geometry, global_embedding)
+        x = [self.preprocess[i](t) for i, t in enumerate(streams)]
+        for blk in self.blocks:
+            x = blk(tuple(x), context)
+        x = [self.ln_mlp_out[i](t) for i, t in enumerate(x)]
+        return x[0] if single else tuple(x)
+
+
 def rel_l2(a: torch.Tensor, b: torch.Tensor) -> float:
     """||a - b||_2 / ||b||_2 in float64."""
     a64, b64 = a.double().flatten(), b.double().flatten()

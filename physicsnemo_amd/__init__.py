@@ -8,6 +8,7 @@ from .physics_attention import (  # noqa: F401
 from .context_projector import ContextProjector, StructuredContextProjector  # noqa: F401
 from .flare import FLARE, FLAREBlock, FLAREModel, GALE_FA  # noqa: F401
 from .gale import GALE, GALEBlock, GALEStructuredMesh2D, GALEStructuredMesh3D  # noqa: F401
+from .geotransolver import GeoTransolver, GlobalContextBuilder  # noqa: F401
 from .graphs import GraphedForward  # noqa: F401
 from .transolver import Mlp, Transolver, TransolverBlock  # noqa: F401
 

@@ -77,3 +77,42 @@ def test_flare_irregular_model_matches_reference_golden():
     print("flare irregular max abs diff", (out - gold).abs().max().item())
     assert torch.allclose(out, gold, rtol=1e-3, atol=1e-3)
     assert (out - gold).abs().max().item() < 5e-6
+
+
+def test_geotransolver_basic_matches_reference_golden():
+    # reference: test/models/geotransolver/test_geotransolver.py:400-437 (seed 42, atol 1e-3)
+    from oracle.torch_oracle import OracleGeoTransolver
+    torch.manual_seed(42)
+    model = OracleGeoTransolver(functional_dim=32, out_dim=4, geometry_dim=3, global_dim=16, n_layers=2, n_hidden=64,
+                                n_head=4, mlp_ratio=2, slice_num=8)
+    local_emb = torch.randn(2, 100, 32)
+    geometry = torch.randn(2, 235, 3)
+    global_emb = torch.randn(2, 5, 16)
+    with torch.no_grad():
+        out = model(local_emb, local_emb[:, :, :3], global_emb, geometry)
+    gold = _load("geotransolver_basic_output.pth")
+    assert out.shape == gold.shape == (2, 100, 4)
+    print("geotransolver basic max abs diff", (out - gold).abs().max().item())
+    assert torch.allclose(out, gold, rtol=1e-3, atol=1e-3)
+    assert (out - gold).abs().max().item() < 5e-6
+
+
+def test_geotransolver_tuple_matches_reference_golden():
+    # reference: test_geotransolver.py:440-490 (seed 42, two input streams, atol 2e-3)
+    from oracle.torch_oracle import OracleGeoTransolver
+    torch.manual_seed(42)
+    model = OracleGeoTransolver(functional_dim=(32, 48), out_dim=(4, 6), geometry_dim=3, global_dim=16, n_layers=2,
+                                n_hidden=64, n_head=4, mlp_ratio=2, slice_num=8)
+    e1, e2 = torch.randn(2, 100, 32), torch.randn(2, 150, 48)
+    geometry = torch.randn(2, 235, 3)
+    global_emb = torch.randn(2, 5, 16)
+    with torch.no_grad():
+        out = model((e1, e2), (e1[:, :, :3], e2[:, :, :3]), global_emb, geometry)
+    gold = torch.load(os.path.join(GOLD, "geotransolver_tuple_output.pth"), weights_only=True)
+    print("golden keys", type(gold), list(gold.keys()) if isinstance(gold, dict) else None)
+    for i, o in enumerate(out):
+        g = gold[i]
+        assert o.shape == g.shape
+        print("geotransolver tuple", i, "max abs diff", (o - g).abs().max().item())
+        assert torch.allclose(o, g, rtol=1e-3, atol=2e-3)
+        assert (o - g).abs().max().item() < 5e-6
