@@ -238,6 +238,15 @@ def time_variants(points, C, S, reps=5):
     with torch.no_grad():
         entry(f"FLARE layer bf16 (general kernels), C={C}, {S} global queries", pts, timed(lambda: flare(xf), 3))
     del xf
+    # GeoTransolver: context projectors + 4 GALE blocks (fused attention kernels, block-MLP kernel), bf16 autocast
+    geo = pn.GeoTransolver(functional_dim=8, out_dim=4, geometry_dim=3, global_dim=16, n_layers=4, n_hidden=C,
+                           n_head=H, slice_num=S).cuda().eval()
+    ge, gg, gl = (torch.randn(1, pts, 8, device="cuda"), torch.randn(1, pts // 4, 3, device="cuda"),
+                  torch.randn(1, 8, 16, device="cuda"))
+    with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
+        entry(f"GeoTransolver bf16, 4 GALE blocks, hidden {C}, S={S}, geometry {pts // 4} points", pts,
+              timed(lambda: geo(ge, None, gl, gg), 3))
+    del ge, gg, gl, geo
     # structured 3-D, 64^3 grid, Conv3d k=3 projections
     g = 64
     s3 = pn.PhysicsAttentionStructuredMesh3D(C, (g, g, g), heads=H, dim_head=32, slice_num=S, kernel=3,
