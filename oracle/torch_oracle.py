@@ -16,7 +16,17 @@ Pinning status (what checks this file, see tests/test_oracle_*.py):
   * closed forms and invariants (softmax rows, clamp special cases, norm sum,
     N=1 eps case, zero slice weight => hand-computable layer output, k=1 conv == linear);
   * the reference's own golden outputs ``tests/golden/transolver2d_output.pth`` and
-    ``transolver_irregular_output.pth`` (whole model, rtol 1e-3 / atol 2e-3 and 1e-3).
+    ``transolver_irregular_output.pth`` (whole model, rtol 1e-3 / atol 2e-3 and 1e-3; matched to < 5e-6);
+  * the Transolver++ branch (``plus=True``): NumPy restatement, reductions to the plain layer, the 0.01 floor, the
+    Gumbel moments; its gradient and the plain layer's by float64 finite differences;
+  * GALE layers / block, the context projectors and ``OracleGeoTransolver``: the reference's golden outputs
+    ``geotransolver_basic_output.pth`` / ``geotransolver_tuple_output.pth`` (matched to < 1e-6), plus closed forms
+    (no context, gate at +-inf, a single context token, zero keys, concatenation order);
+  * FLARE layer / block / model: the reference's golden outputs ``flare_2d_output.pth`` / ``flare_irregular_output.pth``
+    (matched to < 1e-6), NumPy restatement, zero-query and one-query closed forms, finite-difference gradient;
+  * ``OracleGALE_FA`` has no golden file in the reference: it is pinned by its reductions to the FLARE layer (no context,
+    gate at +inf), the single-context-token closed form and the explicit scale-1 softmax over the context
+    (tests/test_oracle_flare.py); its ``concat_project`` blend shares ``gale_mix`` with the GALE layer.
 """
 
 from __future__ import annotations
