@@ -50,3 +50,33 @@ def test_graph_replay_of_a_model_equals_eager():
             want = fwd(fx, emb)
             torch.cuda.synchronize()
             assert torch.equal(got, want)
+
+
+def test_graph_replay_of_flare_and_geotransolver_models_equals_eager():
+    """The reference validates CUDA-graph capture of these models (test_flare.py, test_geotransolver.py
+    ``validate_cuda_graphs``); here every replay must equal the eager call bit for bit."""
+    announce("graph replay: FLARE model and GeoTransolver")
+    torch.manual_seed(2)
+    dev = torch.device("cuda:0")
+    flare = pn.FLAREModel(functional_dim=2, embedding_dim=3, out_dim=1, n_layers=2, n_hidden=64, n_head=4, mlp_ratio=1,
+                          slice_num=32, use_te=False).eval().to(dev)
+    geo = pn.GeoTransolver(functional_dim=6, out_dim=3, geometry_dim=3, global_dim=5, n_layers=2, n_hidden=64, n_head=4,
+                           mlp_ratio=2, slice_num=8).eval().to(dev)
+
+    def run_geo(e, glob, geom):
+        return geo(e, None, glob, geom)
+
+    cases = [
+        (flare, [(torch.randn(2, 1234, 2, device=dev), torch.randn(2, 1234, 3, device=dev)) for _ in range(3)]),
+        (run_geo, [(torch.randn(2, 700, 6, device=dev), torch.randn(2, 4, 5, device=dev),
+                    torch.randn(2, 300, 3, device=dev)) for _ in range(3)]),
+    ]
+    with torch.no_grad():
+        for fn, inputs in cases:
+            graphed = pn.GraphedForward(fn, *inputs[0])
+            for args in inputs + inputs[:1]:
+                got = graphed(*args).clone()
+                torch.cuda.synchronize()
+                want = fn(*args)
+                torch.cuda.synchronize()
+                assert torch.equal(got, want)
