@@ -72,6 +72,11 @@ class FLARE(nn.Module):
     def forward_block(self, x: torch.Tensor, residual: torch.Tensor, ln: nn.LayerNorm):
         """Layer + the caller block's ``+ residual`` and following LayerNorm (flare.py:98-99): (fx_new, LayerNorm(fx_new))
         with the add and the LayerNorm in one library kernel."""
+        fp16 = x.dtype == torch.float16 or (torch.is_autocast_enabled("cuda")
+                                            and torch.get_autocast_dtype("cuda") == torch.float16)
+        if fp16:  # float32 inside, as the residual stream of the caller is
+            with torch.autocast("cuda", enabled=False):
+                return self.forward_block(x.float(), residual.float(), ln)
         y = self.forward(x).contiguous()
         return PF.residual_layernorm(y, residual=residual.to(y.dtype).contiguous(),
                                      ln_weight=ln.weight.detach().float().contiguous(),

@@ -105,3 +105,23 @@ def test_bf16_geotransolver_on_the_fused_kernels():
         with torch.autocast("cuda", dtype=torch.bfloat16):
             got = hip(e.cuda(), None, glob.cuda(), geom.cuda())
     assert_rel_l2(got, want, "bf16 GeoTransolver", tol=1e-2)
+
+
+def test_float16_autocast_is_served_in_float32():
+    """The reference's AMP checks run these models under float16 autocast; there are no float16 kernels, the layers
+    then compute in float32 (at least the precision asked for)."""
+    announce("fp16 autocast: GeoTransolver, FLARE model")
+    torch.manual_seed(3)
+    geo = pn.GeoTransolver(functional_dim=6, out_dim=3, geometry_dim=3, global_dim=5, n_layers=2, n_hidden=32, n_head=4,
+                           mlp_ratio=2, slice_num=8).eval().cuda()
+    flare = pn.FLAREModel(functional_dim=2, embedding_dim=3, out_dim=1, n_layers=2, n_hidden=32, n_head=4, mlp_ratio=1,
+                          slice_num=8, use_te=False).eval().cuda()
+    e, glob, geom = torch.randn(2, 300, 6).cuda(), torch.randn(2, 4, 5).cuda(), torch.randn(2, 100, 3).cuda()
+    a, b = torch.randn(2, 300, 2).cuda(), torch.randn(2, 300, 3).cuda()
+    with torch.no_grad():
+        want_g, want_f = geo(e, None, glob, geom), flare(a, b)
+        with torch.autocast("cuda", dtype=torch.float16):
+            got_g, got_f = geo(e, None, glob, geom), flare(a, b)
+    assert torch.isfinite(got_g).all() and torch.isfinite(got_f).all()
+    assert_rel_l2(got_g, want_g, "GeoTransolver under fp16 autocast", tol=5e-3)
+    assert_rel_l2(got_f, want_f, "FLARE model under fp16 autocast", tol=5e-3)
