@@ -3,7 +3,7 @@
 // layer (projections, slice softmax, aggregation, slice self-attention, deslice + out_linear) is the PhysicsAttention
 // layer's own kernels; this stage sits between the slice self-attention and the deslice.
 //
-// One workgroup per (batch, head); fp32 arithmetic on the vector ALUs (the stage is S x D work, independent of the
+// One workgroup per (batch, head), operands and weights in LDS; fp32 arithmetic on the vector ALUs (the stage is S x D work, independent of the
 // number of points):
 //   q = tok Wq^T + bq (S x D);  k = ctx Wk^T + bk,  v = ctx Wv^T + bv (Sc x D)
 //   cross = softmax(q k^T / sqrt(D)) v
@@ -29,6 +29,10 @@ __global__ __launch_bounds__(kThreads) void slice_cross_mix_kernel(
   float *k = q + S * D1;          // Sc * D1
   float *v = k + Sc * D1;         // Sc * D1
   float *prow = v + Sc * D1;      // (kThreads / 64) * Sc
+  float *wq = prow + (kThreads / 64) * Sc;  // D * D1   cross_q weight rows
+  float *wk = wq + D * D1;                  // D * Dc1  cross_k weight rows
+  float *wv = wk + D * Dc1;                 // D * Dc1  cross_v weight rows
+  float *wc = wv + D * Dc1;                 // D * (2D + 1)  concat_project weight rows (that blend mode only)
   const int t = threadIdx.x, wave = t >> 6, lane = t & 63;
   const int64_t bh = blockIdx.x;
   const float *tk = slice_token + bh * S * D;
@@ -36,22 +40,29 @@ __global__ __launch_bounds__(kThreads) void slice_cross_mix_kernel(
 
   for (int i = t; i < S * D; i += kThreads) tok[(i / D) * D1 + (i % D)] = tk[i];
   for (int i = t; i < Sc * Dc; i += kThreads) ctx[(i / Dc) * Dc1 + (i % Dc)] = cx[i];
+  // the three weights go through LDS: read from global memory inside the dot products, every term waits for its load
+  for (int i = t; i < D * D; i += kThreads) wq[(i / D) * D1 + (i % D)] = gp.cross_q_weight[i];
+  for (int i = t; i < D * Dc; i += kThreads) {
+    wk[(i / Dc) * Dc1 + (i % Dc)] = gp.cross_k_weight[i];
+    wv[(i / Dc) * Dc1 + (i % Dc)] = gp.cross_v_weight[i];
+  }
+  if (!gp.state_mixing)
+    for (int i = t; i < D * 2 * D; i += kThreads) wc[(i / (2 * D)) * (2 * D + 1) + (i % (2 * D))] = gp.concat_project_weight[i];
   __syncthreads();
   for (int i = t; i < S * D; i += kThreads) {
     const int s = i / D, e = i - s * D;
-    const float *wr = gp.cross_q_weight + (int64_t)e * D;
+    const float *wr = wq + e * D1;
     float acc = gp.cross_q_bias[e];
     for (int d = 0; d < D; ++d) acc = fmaf(tok[s * D1 + d], wr[d], acc);
     q[s * D1 + e] = acc;
   }
   for (int i = t; i < Sc * D; i += kThreads) {
     const int u = i / D, e = i - u * D;
-    const float *wk = gp.cross_k_weight + (int64_t)e * Dc;
-    const float *wv = gp.cross_v_weight + (int64_t)e * Dc;
+    const float *wkr = wk + e * Dc1, *wvr = wv + e * Dc1;
     float ak = gp.cross_k_bias[e], av = gp.cross_v_bias[e];
     for (int c = 0; c < Dc; ++c) {
-      ak = fmaf(ctx[u * Dc1 + c], wk[c], ak);
-      av = fmaf(ctx[u * Dc1 + c], wv[c], av);
+      ak = fmaf(ctx[u * Dc1 + c], wkr[c], ak);
+      av = fmaf(ctx[u * Dc1 + c], wvr[c], av);
     }
     k[u * D1 + e] = ak;
     v[u * D1 + e] = av;
@@ -101,7 +112,7 @@ __global__ __launch_bounds__(kThreads) void slice_cross_mix_kernel(
     if (gp.state_mixing) {
       o = mixw * sf[i] + (1.f - mixw) * tok[s * D1 + e];
     } else {
-      const float *wr = gp.concat_project_weight + (int64_t)e * 2 * D;
+      const float *wr = wc + e * (2 * D + 1);
       float acc = gp.concat_project_bias[e];
       for (int d = 0; d < D; ++d) acc = fmaf(sf[s * D + d], wr[d], acc);
       for (int d = 0; d < D; ++d) acc = fmaf(tok[s * D1 + d], wr[D + d], acc);
@@ -134,7 +145,8 @@ int pack_tokens(const pa_shape &s, const float *out_token, void *tokp, hipStream
 }
 
 size_t lds_bytes(const pa_shape &s, int64_t Sc, int64_t Dc) {
-  return (size_t)(2 * s.S * (s.D + 1) + Sc * (Dc + 1) + 2 * Sc * (s.D + 1) + (kThreads / 64) * Sc) * 4;
+  return (size_t)(2 * s.S * (s.D + 1) + Sc * (Dc + 1) + 2 * Sc * (s.D + 1) + (kThreads / 64) * Sc +
+                  s.D * (s.D + 1) + 2 * s.D * (Dc + 1) + s.D * (2 * s.D + 1)) * 4;
 }
 
 int slice_cross_mix(const pa_shape &s, const pa_gale_params &gp, int64_t Sc, int64_t Dc, const float *slice_token,

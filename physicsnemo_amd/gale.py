@@ -19,7 +19,9 @@ import torch
 import torch.nn as nn
 
 from . import functional as PF
+from . import autograd as PA
 from .autograd import GALEFunction
+from .transolver import Mlp, TransolverBlock
 from .physics_attention import (
     PhysicsAttentionIrregularMesh,
     PhysicsAttentionStructuredMesh2D,
@@ -140,6 +142,39 @@ class _GALEForwardMixin:
         out_tok = PF.slice_cross_attention_mix(tok, self_out, context, gp, dims)
         return PF.deslice_project(w, out_tok, p, dims)
 
+    def forward_block(self, x: torch.Tensor, residual: torch.Tensor, ln: nn.LayerNorm,
+                      context: torch.Tensor | None = None, gp: dict | None = None):
+        """One input tensor: layer (with the context) + the caller block's ``+ residual`` and following LayerNorm
+        (reference gale.py:1019-1024) -> (fx_new, LayerNorm(fx_new)); inference only.  On the MFMA shapes the add and
+        the LayerNorm are the tail of the deslice kernel, as in the plain layer."""
+        if context is None:
+            return super().forward_block(x, residual, ln)
+        if x.is_cuda and self._wants_fp16(x):
+            with torch.autocast("cuda", enabled=False):
+                return self.forward_block(x.float(), residual.float(), ln, context, gp)
+        self._validate(x)
+        x = self._prepare_input(x)
+        residual = residual.to(x.dtype).contiguous()
+        ln_w, ln_b = ln.weight.detach().float().contiguous(), ln.bias.detach().float().contiguous()
+        dims = self.layer_dims(x)
+        fused = (not self.plus and not self.fp8_weights and not (self.training and self.out_dropout.p > 0)
+                 and PF.query_path(x.dtype, dims) == 1)
+        if not fused:
+            y = self.out_dropout(self._forward_one(x, context, gp)).contiguous()
+            return PF.residual_layernorm(y, residual=residual, ln_weight=ln_w, ln_bias=ln_b, ln_eps=ln.eps)
+        st = PF.MfmaStages(self.kernel_params(x.dtype, x.device), dims, x.device)
+        st.pack_params()
+        if st.fused_groups > 0:
+            st.project_softmax_reduce(x)
+        else:
+            st.project_softmax(x)
+            st.slice_reduce()
+        st.combine_attention()
+        PF.slice_cross_attention_mix(st.tok, st.tok_out, context, gp, dims, tokp=st.tokp)
+        fx_new, normed = torch.empty_like(x), torch.empty_like(x)
+        st.deslice_project(fx_new, residual=residual, ln_weight=ln_w, ln_bias=ln_b, ln_eps=ln.eps, ln_out=normed)
+        return fx_new, normed
+
     def forward(self, x: tuple, context: torch.Tensor | None = None) -> list:
         """x: tuple of (B, N, C) tensors; context (B, H, S_c, D_c) or None -> list of (B, N, C) tensors."""
         if isinstance(x, torch.Tensor):
@@ -205,8 +240,6 @@ class GALEBlock(nn.Module):
                  plus: bool = False, context_dim: int = 0, spatial_shape: tuple | None = None,
                  attention_type: str = "GALE", concrete_dropout: bool = False, state_mixing_mode: str = "weighted"):
         super().__init__()
-        from .transolver import Mlp  # the block MLP of the Transolver block (reference mlp_layers.py:101-173)
-
         self.last_layer = last_layer
         self.ln_1 = nn.LayerNorm(hidden_dim)
         if attention_type not in ("GALE", "GALE_FA"):
@@ -234,20 +267,40 @@ class GALEBlock(nn.Module):
         self.ffn_dropout = None
         self._mlp_cache: dict = {}
 
-    def _one(self, fx: torch.Tensor, attn: torch.Tensor, needs_grad: bool) -> torch.Tensor:
-        from . import autograd as PA
-        from .transolver import TransolverBlock as TB
+    # the block MLP (reference mlp_layers.py:101-173) and its kernels are the Transolver block's
+    _mlp_kernel_params = TransolverBlock._mlp_kernel_params
+    _mlp_kernel_serves = TransolverBlock._mlp_kernel_serves
+    _mlp_with_grad = TransolverBlock._mlp_with_grad
+    _mlp_residual = TransolverBlock._mlp_residual
 
+    def _one(self, fx: torch.Tensor, attn: torch.Tensor, needs_grad: bool) -> torch.Tensor:
         fx1 = attn + fx
         normed = PA.layer_norm(fx1, self.ln_mlp1[0])
-        if not needs_grad and TB._mlp_kernel_serves(self, normed):
-            w1, b1, w2, b2 = TB._mlp_kernel_params(self, normed.device)
+        if not needs_grad and self._mlp_kernel_serves(normed):
+            w1, b1, w2, b2 = self._mlp_kernel_params(normed.device)
             return PF.mlp_forward(normed, w1, b1, w2, b2, residual=fx1.to(normed.dtype).contiguous())
-        return TB._mlp_with_grad(self, normed) + fx1
+        return self._mlp_with_grad(normed) + fx1
+
+    def forward_chain(self, fx: tuple, normed_in, global_context: torch.Tensor | None, next_ln: nn.LayerNorm | None):
+        """Inference, one block inside a chain: takes LayerNorm_1 of every stream if the previous block produced it and
+        returns (outputs, next_ln(outputs) or None).  The residual adds and LayerNorms ride on the deslice and block-MLP
+        kernels (same arithmetic as `forward`)."""
+        attn = self.Attn
+        gp = None
+        if global_context is not None:
+            attn._check_context(global_context, fx[0].shape[0])
+            global_context = global_context.detach().float().contiguous()
+            gp = attn.gale_params(global_context.device)
+        outs, normed_out = [], []
+        for i, t in enumerate(fx):
+            x_in = normed_in[i] if normed_in is not None else PA.layer_norm(t, self.ln_1)
+            fx1, normed = attn.forward_block(x_in, t, self.ln_mlp1[0], global_context, gp)
+            out, nxt = self._mlp_residual(fx1, normed, next_ln)
+            outs.append(out)
+            normed_out.append(nxt)
+        return outs, (normed_out if next_ln is not None and all(n is not None for n in normed_out) else None)
 
     def forward(self, fx: tuple, global_context: torch.Tensor | None) -> list:
-        from . import autograd as PA
-
         if isinstance(fx, torch.Tensor):
             raise TypeError("GALEBlock takes a tuple of input tensors")
         if len(fx) == 0:

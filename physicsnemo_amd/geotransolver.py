@@ -187,8 +187,20 @@ class GeoTransolver(nn.Module):
                              f"with shape {tuple(global_embedding.shape)}")
         embedding_states, _, _ = self.context_builder.build_context(streams, local_positions, geometry, global_embedding)
         x = [self.preprocess[i](t) for i, t in enumerate(streams)]
-        for block in self.blocks:
-            x = block(tuple(x), embedding_states)
+        needs_grad = torch.is_grad_enabled() and (any(t.requires_grad for t in x)
+                                                  or any(p.requires_grad for p in self.parameters()))
+        chain = not needs_grad and all(t.is_cuda for t in x) and all(hasattr(b.Attn, "gale_params") for b in self.blocks)
+        if chain:
+            # inference: each block hands the next one LayerNorm_1 of its outputs (computed in its MLP kernel's tail)
+            if torch.is_autocast_enabled("cuda") and torch.get_autocast_dtype("cuda") == torch.bfloat16:
+                x = [t.to(torch.bfloat16) for t in x]
+            normed = None
+            for k, block in enumerate(self.blocks):
+                next_ln = self.blocks[k + 1].ln_1 if k + 1 < len(self.blocks) else None
+                x, normed = block.forward_chain(tuple(x), normed, embedding_states, next_ln)
+        else:
+            for block in self.blocks:
+                x = block(tuple(x), embedding_states)
         point_features = list(x)
         x = [self.ln_mlp_out[i](t) for i, t in enumerate(x)]
         if self.structured_shape is not None and unflatten_output:

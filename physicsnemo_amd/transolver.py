@@ -150,6 +150,11 @@ class TransolverBlock(nn.Module):
         x_in = normed_in if normed_in is not None else self.ln_1(fx)
         # fx1 = Attn(ln_1(fx)) + fx and LayerNorm(fx1) come out of one fused library call (reference :300, :303)
         fx1, normed = self.Attn.forward_block(x_in, fx, self.ln_mlp1[0])
+        return self._mlp_residual(fx1, normed, next_ln)
+
+    def _mlp_residual(self, fx1: torch.Tensor, normed: torch.Tensor, next_ln: nn.LayerNorm | None):
+        """fx1 + Mlp(normed) and, with `next_ln`, its LayerNorm (reference :303, and :300 of the next block): the fused
+        block-MLP kernel where it serves the shape, else the tensor-op MLP followed by one add (+ LayerNorm) kernel."""
         if self._mlp_kernel_serves(normed):
             w1, b1, w2, b2 = self._mlp_kernel_params(normed.device)
             if next_ln is None:
