@@ -3,7 +3,8 @@
 // layer (projections, slice softmax, aggregation, slice self-attention, deslice + out_linear) is the PhysicsAttention
 // layer's own kernels; this stage sits between the slice self-attention and the deslice.
 //
-// One workgroup per (batch, head), operands and weights in LDS; fp32 arithmetic on the vector ALUs (the stage is S x D work, independent of the
+// Workgroups (batch * head, blocks of 16 slice tokens), operands and weights in LDS (every workgroup forms k and v of
+// its (batch, head) itself); fp32 arithmetic on the vector ALUs (the stage is S x D work, independent of the
 // number of points):
 //   q = tok Wq^T + bq (S x D);  k = ctx Wk^T + bk,  v = ctx Wv^T + bv (Sc x D)
 //   cross = softmax(q k^T / sqrt(D)) v
@@ -17,6 +18,7 @@ namespace pa {
 namespace gale {
 
 constexpr int kThreads = 256;
+constexpr int kQueryBlock = 16;  // slice tokens per workgroup: grid.y = ceil(S / 16) workgroups share a (batch, head)
 
 __global__ __launch_bounds__(kThreads) void slice_cross_mix_kernel(
     const float *__restrict__ slice_token, const float *__restrict__ self_token, const float *__restrict__ context,
@@ -35,6 +37,7 @@ __global__ __launch_bounds__(kThreads) void slice_cross_mix_kernel(
   float *wc = wv + D * Dc1;                 // D * (2D + 1)  concat_project weight rows (that blend mode only)
   const int t = threadIdx.x, wave = t >> 6, lane = t & 63;
   const int64_t bh = blockIdx.x;
+  const int s0 = blockIdx.y * kQueryBlock, s1 = min(S, s0 + kQueryBlock);  // this workgroup's slice tokens
   const float *tk = slice_token + bh * S * D;
   const float *cx = context + bh * Sc * Dc;
 
@@ -49,7 +52,7 @@ __global__ __launch_bounds__(kThreads) void slice_cross_mix_kernel(
   if (!gp.state_mixing)
     for (int i = t; i < D * 2 * D; i += kThreads) wc[(i / (2 * D)) * (2 * D + 1) + (i % (2 * D))] = gp.concat_project_weight[i];
   __syncthreads();
-  for (int i = t; i < S * D; i += kThreads) {
+  for (int i = s0 * D + t; i < s1 * D; i += kThreads) {
     const int s = i / D, e = i - s * D;
     const float *wr = wq + e * D1;
     float acc = gp.cross_q_bias[e];
@@ -71,7 +74,7 @@ __global__ __launch_bounds__(kThreads) void slice_cross_mix_kernel(
 
   const float scale = rsqrtf((float)D);
   float *pr = prow + wave * Sc;
-  for (int s = wave; s < S; s += kThreads / 64) {
+  for (int s = s0 + wave; s < s1; s += kThreads / 64) {
     const float *qs = q + s * D1;
     float mx = -INFINITY;
     for (int u = lane; u < Sc; u += 64) {
@@ -106,7 +109,7 @@ __global__ __launch_bounds__(kThreads) void slice_cross_mix_kernel(
   float mixw = 0.f;
   if (gp.state_mixing) mixw = 1.f / (1.f + expf(-gp.state_mixing[0]));
   const int NCH = S / 16;
-  for (int i = t; i < S * D; i += kThreads) {
+  for (int i = s0 * D + t; i < s1 * D; i += kThreads) {
     const int s = i / D, e = i - s * D;
     float o;
     if (gp.state_mixing) {
@@ -154,7 +157,8 @@ int slice_cross_mix(const pa_shape &s, const pa_gale_params &gp, int64_t Sc, int
   const size_t lds = lds_bytes(s, Sc, Dc);
   int rc = allow_dynamic_lds(slice_cross_mix_kernel, lds);
   if (rc) return rc;
-  hipLaunchKernelGGL(slice_cross_mix_kernel, dim3((unsigned)(s.B * s.H)), dim3(kThreads), lds, st, slice_token,
+  hipLaunchKernelGGL(slice_cross_mix_kernel, dim3((unsigned)(s.B * s.H), (unsigned)((s.S + kQueryBlock - 1) / kQueryBlock)),
+                     dim3(kThreads), lds, st, slice_token,
                      self_token, context, gp, out_token, static_cast<uint16_t *>(tokp), (int)s.S, (int)s.D, (int)Sc,
                      (int)Dc);
   return launch_status();
