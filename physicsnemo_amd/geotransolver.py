@@ -16,6 +16,7 @@ from collections.abc import Sequence
 import torch
 import torch.nn as nn
 
+from . import autograd as PA
 from .context_projector import ContextProjector, StructuredContextProjector
 from .gale import GALEBlock
 from .transolver import Mlp, Transolver
@@ -202,7 +203,8 @@ class GeoTransolver(nn.Module):
             for block in self.blocks:
                 x = block(tuple(x), embedding_states)
         point_features = list(x)
-        x = [self.ln_mlp_out[i](t) for i, t in enumerate(x)]
+        # per-stream head: LayerNorm on the library kernel (forward and backward), then the output Linear
+        x = [self.ln_mlp_out[i][1](PA.layer_norm(t, self.ln_mlp_out[i][0])) for i, t in enumerate(x)]
         if self.structured_shape is not None and unflatten_output:
             x = [t.reshape(t.shape[0], *self.structured_shape, -1) for t in x]
         out = x[0] if single_input else tuple(x)
