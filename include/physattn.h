@@ -336,6 +336,12 @@ int pa_mfma_backward_query(const pa_shape *shape);
 int64_t pa_cols_gemm_chunks(int64_t rows, int64_t cols_a);
 int pa_cols_gemm(int64_t rows, const void *a, int64_t lda, int64_t cols_a, const void *b, int64_t ldb, int64_t cols_b,
                  float *partials, float *col_sum_partials, void *stream);
+/* The same for float32 operands (fp32 MFMA, natural row-major operands; cols_a, cols_b, lda, ldb multiples of 4):
+ * partials pa_cols_gemm_f32_chunks(rows, cols_a, cols_b) * cols_a * cols_b float32, col_sum_partials chunks * cols_a
+ * or NULL. */
+int64_t pa_cols_gemm_f32_chunks(int64_t rows, int64_t cols_a, int64_t cols_b);
+int pa_cols_gemm_f32(int64_t rows, const void *a, int64_t lda, int64_t cols_a, const void *b, int64_t ldb,
+                     int64_t cols_b, float *partials, float *col_sum_partials, void *stream);
 /* bf16 Linear over the rows of `in` (B, N, c_in) -> H*32 columns, weight (H*32, c_in) bf16, bias float32 or NULL:
  * `out` natural (B, N, H*32) and/or `out_pack` in the packed layout of PA_BUF_FX_PACK (either may be NULL). */
 int pa_rows_gemm_packed(const pa_shape *shape, int64_t c_in, const void *in, const void *weight, const float *bias,

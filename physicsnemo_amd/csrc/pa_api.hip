@@ -558,6 +558,20 @@ int pa_cols_gemm(int64_t rows, const void *a, int64_t lda, int64_t cols_a, const
                              static_cast<hipStream_t>(stream));
 }
 
+int64_t pa_cols_gemm_f32_chunks(int64_t rows, int64_t cols_a, int64_t cols_b) {
+  if (rows <= 0 || cols_a <= 0 || cols_b <= 0) return PA_ERR_DIMS;
+  return pa::gemm::cols_gemm_f32_chunks(rows, cols_a, cols_b, compute_units());
+}
+
+int pa_cols_gemm_f32(int64_t rows, const void *a, int64_t lda, int64_t cols_a, const void *b, int64_t ldb,
+                     int64_t cols_b, float *partials, float *col_sum_partials, void *stream) {
+  if (rows <= 0 || cols_a <= 0 || cols_b <= 0 || lda < cols_a || ldb < cols_b) return PA_ERR_DIMS;
+  if (!a || !b || !partials) return PA_ERR_NULL;
+  if (!aligned16(a) || !aligned16(b) || !aligned16(partials)) return PA_ERR_ALIGN;
+  return pa::gemm::cols_gemm_f32(a, lda, cols_a, b, ldb, cols_b, rows, partials, col_sum_partials, compute_units(),
+                                 static_cast<hipStream_t>(stream));
+}
+
 int pa_mfma_backward_query(const pa_shape *shape) {
   int rc = check_shape(PA_BF16, shape);
   if (rc) return rc;

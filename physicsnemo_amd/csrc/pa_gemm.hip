@@ -433,6 +433,122 @@ __global__ __launch_bounds__(512) void cols_gemm_kernel(const uint16_t *__restri
 }
 
 // row chunks: about two workgroups per CU over all column groups, and at least 32 blocks of 32 rows per chunk so that
+// ------------------------------------------------------------------------------------------------
+// cols_gemm_f32_kernel: the float32 form of the weight-gradient product  P[oa][ob] = sum_m A[m][oa] * B[m][ob].
+// v_mfma_f32_32x32x2_f32 reduces over two rows m per instruction with lane (i, g) supplying A[m0 + g][oa0 + i] and
+// B[m0 + g][ob0 + i]: consecutive lanes read consecutive columns of a row, so natural row-major operands need no
+// transposition.  A workgroup (4 waves) owns a 128 x 128 block of P for one chunk of rows: 32 rows of its 128 + 128
+// operand columns at a time go through LDS (coalesced 16-byte loads, double buffered), wave w multiplies the 64 x 64
+// sub-block (w & 1, w >> 1): per pair of rows 2 + 2 LDS words feed 4 MFMAs.  Row chunks come back as partials
+// P[g][oa][ob] (fixed-order sum by the caller); col_sums[g][oa] = sum_m A[m][oa] from the same pass (blockIdx.z == 0).
+// ------------------------------------------------------------------------------------------------
+constexpr int kF32Tile = 128, kF32Rows = 32;
+
+__global__ __launch_bounds__(256) void cols_gemm_f32_kernel(const float *__restrict__ A, int lda, int OA,
+                                                            const float *__restrict__ B, int ldb, int OB, int64_t M,
+                                                            int64_t rows_per_chunk, float *__restrict__ partials,
+                                                            float *__restrict__ col_sums) {
+  __shared__ float As[2][kF32Rows][kF32Tile];
+  __shared__ float Bs[2][kF32Rows][kF32Tile];
+  const int t = threadIdx.x, lane = t & 63, i = lane & 31, g = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+  const int oa0 = blockIdx.y * kF32Tile, ob0 = blockIdx.z * kF32Tile;
+  const int64_t m_begin = (int64_t)blockIdx.x * rows_per_chunk;
+  const int64_t m_end = min(M, m_begin + rows_per_chunk);
+  const int wa = (wave & 1) * 64, wb = (wave >> 1) * 64;  // this wave's sub-block of the tile
+
+  f32x16 acc[2][2];
+#pragma unroll
+  for (int u = 0; u < 2; ++u)
+#pragma unroll
+    for (int v = 0; v < 2; ++v)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[u][v][r] = 0.f;
+  float csum[2] = {0.f, 0.f};
+
+  // staging: 32 rows x 128 columns = 1024 float4 per operand, 4 per thread
+  const int sr = t >> 5, sc = (t & 31) * 4;  // row 0..7 (+8 k), column of the float4
+  float4 pa[4], pb[4];
+  auto fetch = [&](int64_t m0) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int64_t m = m0 + sr + 8 * k;
+      pa[k] = pb[k] = float4{0.f, 0.f, 0.f, 0.f};
+      if (m < m_end) {
+        if (oa0 + sc < OA) pa[k] = *reinterpret_cast<const float4 *>(A + m * lda + oa0 + sc);
+        if (ob0 + sc < OB) pb[k] = *reinterpret_cast<const float4 *>(B + m * ldb + ob0 + sc);
+      }
+    }
+  };
+  auto stage = [&](int buf) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      *reinterpret_cast<float4 *>(&As[buf][sr + 8 * k][sc]) = pa[k];
+      *reinterpret_cast<float4 *>(&Bs[buf][sr + 8 * k][sc]) = pb[k];
+    }
+  };
+  fetch(m_begin);
+  int buf = 0;
+  for (int64_t m0 = m_begin; m0 < m_end; m0 += kF32Rows) {
+    stage(buf);
+    __syncthreads();
+    fetch(m0 + kF32Rows < m_end ? m0 + kF32Rows : m0);  // the last block re-fetches itself: no branch around the loads
+#pragma unroll 4
+    for (int k = 0; k < kF32Rows; k += 2) {
+      const float a0 = As[buf][k + g][wa + i], a1 = As[buf][k + g][wa + 32 + i];
+      const float b0 = Bs[buf][k + g][wb + i], b1 = Bs[buf][k + g][wb + 32 + i];
+      acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b0, acc[0][0], 0, 0, 0);
+      acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b1, acc[0][1], 0, 0, 0);
+      acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b0, acc[1][0], 0, 0, 0);
+      acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1, acc[1][1], 0, 0, 0);
+      csum[0] += a0;
+      csum[1] += a1;
+    }
+    buf ^= 1;
+  }
+  // C/D layout: lane (i, g) holds column ob = i, register r holds row oa = rowmap(r, g)
+  float *dst = partials + (int64_t)blockIdx.x * OA * OB;
+#pragma unroll
+  for (int u = 0; u < 2; ++u)
+#pragma unroll
+    for (int v = 0; v < 2; ++v) {
+      const int ob = ob0 + wb + 32 * v + i;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int oa = oa0 + wa + 32 * u + mfma::rowmap(r, g);
+        if (oa < OA && ob < OB) dst[(int64_t)oa * OB + ob] = acc[u][v][r];
+      }
+    }
+  if (col_sums && blockIdx.z == 0 && (wave >> 1) == 0) {
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const float total = csum[u] + __shfl_xor(csum[u], 32, 64);  // the two row parities
+      const int oa = oa0 + wa + 32 * u + i;
+      if (g == 0 && oa < OA) col_sums[(int64_t)blockIdx.x * OA + oa] = total;
+    }
+  }
+}
+
+int64_t cols_gemm_f32_chunks(int64_t M, int64_t OA, int64_t OB, int num_cu) {
+  const int64_t tiles = ((OA + kF32Tile - 1) / kF32Tile) * ((OB + kF32Tile - 1) / kF32Tile);
+  int64_t g = (3 * (int64_t)num_cu + tiles - 1) / tiles;  // about three workgroups per compute unit in all
+  const int64_t cap = (M + 1023) / 1024;                  // at least 1024 rows per chunk
+  if (g > cap) g = cap;
+  return g < 1 ? 1 : g;
+}
+
+int cols_gemm_f32(const void *A, int64_t lda, int64_t OA, const void *B, int64_t ldb, int64_t OB, int64_t M,
+                  float *partials, float *col_sums, int num_cu, hipStream_t st) {
+  if (OA <= 0 || OB <= 0 || OA % 4 != 0 || OB % 4 != 0 || lda % 4 != 0 || ldb % 4 != 0) return PA_ERR_UNSUPPORTED;
+  const int64_t G = cols_gemm_f32_chunks(M, OA, OB, num_cu);
+  int64_t per = (M + G - 1) / G;
+  per = (per + kF32Rows - 1) / kF32Rows * kF32Rows;
+  const dim3 grid((unsigned)G, (unsigned)((OA + kF32Tile - 1) / kF32Tile), (unsigned)((OB + kF32Tile - 1) / kF32Tile));
+  hipLaunchKernelGGL(cols_gemm_f32_kernel, grid, dim3(256), 0, st, static_cast<const float *>(A), (int)lda, (int)OA,
+                     static_cast<const float *>(B), (int)ldb, (int)OB, M, per, partials, col_sums);
+  return launch_status();
+}
+
 // the partial results stay small next to the rows a chunk reads
 int64_t cols_gemm_chunks(int64_t M, int64_t OA, int num_cu) {
   const int64_t nblk = (M + 31) / 32, gy = (OA + 255) / 256;

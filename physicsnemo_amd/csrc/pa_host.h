@@ -62,6 +62,10 @@ int launch(const GemmArgs &a, int nsets, int dtype, hipStream_t st);
 int64_t cols_gemm_chunks(int64_t M, int64_t OA, int num_cu);
 int cols_gemm(const void *A, int64_t lda, int64_t OA, const void *B, int64_t ldb, int64_t OB, int64_t M,
               float *partials, float *col_sums, int num_cu, hipStream_t st);
+// the same for float32 operands (fp32 MFMA)
+int64_t cols_gemm_f32_chunks(int64_t M, int64_t OA, int64_t OB, int num_cu);
+int cols_gemm_f32(const void *A, int64_t lda, int64_t OA, const void *B, int64_t ldb, int64_t OB, int64_t M,
+                  float *partials, float *col_sums, int num_cu, hipStream_t st);
 }  // namespace gemm
 
 namespace general {

@@ -400,12 +400,15 @@ def mfma_backward_supported(dtype: torch.dtype, dims: LayerDims) -> bool:
 
 def cols_gemm_supported(a: torch.Tensor, b: torch.Tensor) -> bool:
     ca, cb = a.shape[-1], b.shape[-1]
+    if a.dtype == torch.float32 and b.dtype == torch.float32:  # fp32 MFMA kernel: worth it from a few thousand rows on
+        return a.is_cuda and ca % 4 == 0 and cb % 4 == 0 and a.numel() // ca >= 4096
     return (a.dtype == torch.bfloat16 and b.dtype == torch.bfloat16 and a.is_cuda and ca % 32 == 0
             and (ca <= 256 or ca % 256 == 0) and cb in (32, 64, 128, 256))
 
 
 def cols_gemm(a: torch.Tensor, b: torch.Tensor, col_sums: bool = False):
-    """a^T . b over the leading (row) axes: bf16 (..., ca) and (..., cb) with equal row counts -> float32 (ca, cb).
+    """a^T . b over the leading (row) axes: bf16 or float32 (..., ca) and (..., cb) with equal row counts -> float32
+    (ca, cb).
 
     The weight-gradient product d W = d out^T . in on the MFMA kernel `cols_gemm_kernel`; with `col_sums` the column
     sums of a (the matching bias gradient) come back as well, from the same pass."""
@@ -415,6 +418,14 @@ def cols_gemm(a: torch.Tensor, b: torch.Tensor, col_sums: bool = False):
     rows = a.numel() // ca
     if b.numel() // cb != rows:
         raise ValueError("cols_gemm needs the same number of rows on both sides")
+    a, b = a.contiguous(), b.contiguous()
+    if a.dtype == torch.float32:
+        chunks = lib.pa_cols_gemm_f32_chunks(rows, ca, cb)
+        partials = torch.empty(int(chunks), ca, cb, dtype=torch.float32, device=a.device)
+        sums = torch.empty(int(chunks), ca, dtype=torch.float32, device=a.device) if col_sums else None
+        _lib.check(lib.pa_cols_gemm_f32(rows, a.data_ptr(), ca, ca, b.data_ptr(), cb, cb, partials.data_ptr(),
+                                        _lib.ptr(sums), _lib.current_stream_ptr(a.device)), "pa_cols_gemm_f32")
+        return (partials.sum(0), sums.sum(0)) if col_sums else partials.sum(0)
     chunks = lib.pa_cols_gemm_chunks(rows, ca)
     partials = torch.empty(int(chunks), ca, cb, dtype=torch.float32, device=a.device)
     sums = torch.empty(int(chunks), ca, dtype=torch.float32, device=a.device) if col_sums else None

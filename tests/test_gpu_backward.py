@@ -216,6 +216,21 @@ def test_cols_gemm_weight_gradient_product(rows, ca, cb):
     assert torch.equal(got, PF.cols_gemm(a, b))  # fixed summation order
 
 
+@pytest.mark.parametrize("rows,ca,cb", [(5000, 64, 32), (4099, 256, 256), (8192, 512, 132), (70001, 4, 260), (300000, 128, 256)])
+def test_cols_gemm_float32(rows, ca, cb):
+    announce("cols_gemm float32", rows, ca, cb)
+    torch.manual_seed(rows)
+    a = torch.randn(rows, ca, device="cuda") + 0.25
+    b = torch.randn(rows, cb, device="cuda")
+    assert PF.cols_gemm_supported(a, b)
+    got, sums = PF.cols_gemm(a, b, col_sums=True)
+    assert_fp32_close(sums, a.double().sum(0).float(), "column sums of a", rtol=1e-4)
+    want = a.double().t() @ b.double()
+    assert got.shape == (ca, cb) and got.dtype == torch.float32
+    assert_fp32_close(got, want.float(), "a^T b", rtol=1e-4)
+    assert torch.equal(got, PF.cols_gemm(a, b))  # fixed summation order
+
+
 def test_bf16_model_training_step_runs_the_mfma_backward():
     announce("Transolver training step, bf16 autocast, MFMA backward inside the blocks")
     torch.manual_seed(1)
