@@ -257,6 +257,33 @@ int pa_slice_cross_attention_mix(const pa_shape *shape, const pa_gale_params *ga
                                  int64_t context_dim, const float *slice_token, const float *self_out_slice_token,
                                  const float *context, float *out_slice_token, void *tokp, void *stream);
 
+/* ---- Ball query (physicsnemo/nn/module/ball_query.py:32-140, BQWarp.forward with neighbors_in_radius set; the order
+ * of physicsnemo/nn/functional/neighbors/radius_search/_torch_impl.py:59-160) --------------------------------------
+ * For every query the up to max_neighbors (<= 64) nearest points with distance <= radius, ascending by distance (equal
+ * distances: lower index first).  points (batch, n_points, 3), queries (batch, n_queries, 3) float32;
+ * indices (batch, n_queries, max_neighbors) int64, 0 in unused slots; optional outputs (NULL to skip):
+ * neighbor_points (batch, n_queries, max_neighbors, 3) float32, zeros in unused slots; neighbor_dists
+ * (batch, n_queries, max_neighbors) float32; counts (batch, n_queries) int32 = used slots.  Used by the local
+ * features of GeoTransolver (physicsnemo/models/geotransolver/context_projector.py:491-606). */
+int pa_ball_query(int64_t batch, int64_t n_points, int64_t n_queries, int64_t max_neighbors, float radius,
+                  const float *points, const float *queries, int64_t *indices, float *neighbor_points,
+                  float *neighbor_dists, int32_t *counts, void *stream);
+
+/* The same search over a cell list the caller has built (for large clouds; pa_ball_query looks at every pair):
+ * the points of each batch binned into cells_per_axis^3 cells whose edge along every axis is >= radius * 1.0001,
+ *   grid (batch, 6) float32 = origin x, y, z and 1 / edge x, y, z;  cell of a point = floor((p - origin) / edge) per
+ *   axis clamped to the grid, cell index (ix * G + iy) * G + iz;
+ *   sorted_points (batch * n_points, 3): the points ordered by (batch, cell index); sorted_index (batch * n_points)
+ *   int32: each one's index within its batch; cell_start (batch * G^3 + 1) int32: offset of every cell's first point in
+ *   that order;  query_order (batch, n_queries) int32 or NULL: a processing order of each batch's queries (a
+ *   permutation; spatially sorted queries read the same cells in neighbouring lanes).
+ * Same outputs as pa_ball_query, identical results. */
+int pa_ball_query_cells(int64_t batch, int64_t n_points, int64_t n_queries, int64_t max_neighbors, float radius,
+                        int64_t cells_per_axis, const float *grid, const float *sorted_points,
+                        const int32_t *sorted_index, const int32_t *cell_start, const float *queries,
+                        const int32_t *query_order, int64_t *indices, float *neighbor_points, float *neighbor_dists,
+                        int32_t *counts, void *stream);
+
 /* ---- FLARE attention (physicsnemo/nn/module/flare_attention.py:38-72, :195-255) ------------------
  * y = softmax_s(A) (softmax_n(A)^T v) with the scores A[b,n,h,s] = k[b,n,h,:] . q_global[h,s,:], S = number of global
  * queries.  A (B,N,H,S) and v (B,N,H*D) come from pa_rows_gemm (the caller folds in_project_x, self_k / self_v and

@@ -26,7 +26,14 @@ Pinning status (what checks this file, see tests/test_oracle_*.py):
     (matched to < 1e-6), NumPy restatement, zero-query and one-query closed forms, finite-difference gradient;
   * ``OracleGALE_FA`` has no golden file in the reference: it is pinned by its reductions to the FLARE layer (no context,
     gate at +inf), the single-context-token closed form and the explicit scale-1 softmax over the context
-    (tests/test_oracle_flare.py); its ``concat_project`` blend shares ``gale_mix`` with the GALE layer.
+    (tests/test_oracle_flare.py); its ``concat_project`` blend shares ``gale_mix`` with the GALE layer;
+  * ``radius_search_nearest`` (ball query) and the local-feature modules on top of it: the lattice problem of the
+    reference's own radius-search test (test/nn/functional/neighbors/test_radius_search.py:28-47), whose construction
+    fixes every neighbour list, and brute-force loops on small random clouds (tests/test_oracle_ball_query.py).  The
+    reference holds no golden output for ``include_local_features=True`` (its tests check shapes and finiteness), so
+    the widened ``OracleGeoTransolver`` is pinned only through its parts and the shapes those tests state; where a query
+    has fewer candidate points than ``max_points`` the reference's torch backend fills the spare slots with point 0
+    while its Warp backend leaves zeros: zeros here.
 """
 
 from __future__ import annotations
@@ -702,17 +709,111 @@ class OracleFLAREModel(OracleTransolver):
         self.apply(self._init_weights)
 
 
+def radius_search_nearest(points: torch.Tensor, queries: torch.Tensor, radius: float, max_points: int):
+    """physicsnemo/nn/functional/neighbors/radius_search/_torch_impl.py:96-160 (the max_points form, batched):
+    Euclidean distances of all pairs, the max_points smallest per query, those beyond the radius dropped.
+    points (B, N, 3), queries (B, Q, 3) -> indices (B, Q, K) int64 (0 where unused), neighbour coordinates
+    (B, Q, K, 3) (zeros where unused), distances (B, Q, K) (0 where unused)."""
+    dists = torch.cdist(points, queries, p=2.0, compute_mode="donot_use_mm_for_euclid_dist")  # (B, N, Q)
+    k = min(max_points, dists.shape[1])
+    values, indices = torch.topk(dists, k=k, dim=1, largest=False)  # ascending along dim 1
+    if k < max_points:
+        values = torch.nn.functional.pad(values, (0, 0, 0, max_points - k), value=0.0)
+        indices = torch.nn.functional.pad(indices, (0, 0, 0, max_points - k), value=0)
+        inside = torch.nn.functional.pad(values[:, :k] <= radius, (0, 0, 0, max_points - k), value=False)
+    else:
+        inside = values <= radius
+    # (the reference tests `values <= radius` on the padded zeros as well, which marks the padding as selected and
+    #  makes it gather point 0; callers with fewer points than max_points are outside what its tests cover -- here the
+    #  padding stays unused)
+    idx = torch.where(inside, indices, 0).permute(0, 2, 1)
+    dist = torch.where(inside, values, 0).permute(0, 2, 1)
+    gathered = torch.gather(points, 1, idx.reshape(idx.shape[0], -1, 1).expand(-1, -1, 3)).reshape(*idx.shape, 3)
+    out = gathered * inside.permute(0, 2, 1)[..., None].to(points.dtype)
+    return idx, out, dist
+
+
+class OracleBQ(nn.Module):
+    """physicsnemo/nn/module/ball_query.py:32-140 (BQWarp) with reverse_mapping=True: neighbours of every p_grid point
+    among the points x."""
+
+    def __init__(self, radius, neighbors_in_radius):
+        super().__init__()
+        self.radius, self.neighbors_in_radius = radius, neighbors_in_radius
+
+    def forward(self, x, p_grid):
+        idx, out, _ = radius_search_nearest(x, p_grid, self.radius, self.neighbors_in_radius)
+        return idx, out
+
+
+class _OracleLayers(nn.Module):
+    """physicsnemo/nn/module/mlp_layers.py:32-120 (Mlp with a list of hidden widths): Linear, act, ..., Linear in a
+    Sequential called `layers`."""
+
+    def __init__(self, dims):
+        super().__init__()
+        mods = []
+        for i in range(len(dims) - 1):
+            mods.append(nn.Linear(dims[i], dims[i + 1]))
+            if i < len(dims) - 2:
+                mods.append(nn.GELU())
+        self.layers = nn.Sequential(*mods)
+
+    def forward(self, x):
+        return self.layers(x)
+
+
+class OracleGeometricFeatureProcessor(nn.Module):
+    """context_projector.py:491-606: ball query, neighbour coordinates flattened (B, N, K*3), Mlp
+    (K*3 -> hidden -> hidden/2 -> hidden, GELU), tanh."""
+
+    def __init__(self, radius, neighbors_in_radius, feature_dim, hidden_dim):
+        super().__init__()
+        self.bq_warp = OracleBQ(radius, neighbors_in_radius)
+        self.mlp = _OracleLayers([feature_dim * neighbors_in_radius, hidden_dim, hidden_dim // 2, hidden_dim])
+
+    def forward(self, query_points, key_features):
+        _, neighbors = self.bq_warp(query_points, key_features)
+        return torch.tanh(self.mlp(neighbors.flatten(2)))
+
+
+class OracleMultiScaleFeatureExtractor(nn.Module):
+    """context_projector.py:609-763: per radius a processor and a context projector; context features are
+    tokenizer(processor(coords, geometry)) (:722-741), local features cat(processor(geometry, coords)) (:743-763)."""
+
+    def __init__(self, geometry_dim, radii, neighbors_in_radius, hidden_dim, n_head, dim_head, dropout=0.0, slice_num=64,
+                 plus=False):
+        super().__init__()
+        self.processors = nn.ModuleList([OracleGeometricFeatureProcessor(r, k, geometry_dim, hidden_dim)
+                                         for r, k in zip(radii, neighbors_in_radius)])
+        self.tokenizers = nn.ModuleList([OracleContextProjector(hidden_dim, n_head, dim_head, dropout, slice_num, plus)
+                                         for _ in radii])
+
+    def extract_context_features(self, spatial_coords, geometry):
+        return [tok(proc(spatial_coords, geometry)) for proc, tok in zip(self.processors, self.tokenizers)]
+
+    def extract_local_features(self, spatial_coords, geometry):
+        return torch.cat([proc(geometry, spatial_coords) for proc in self.processors], dim=-1)
+
+
 class OracleGlobalContextBuilder(nn.Module):
-    """physicsnemo/models/geotransolver/context_projector.py:766-1069 without the ball-query local features
-    (include_local_features=False): the context is the geometry tokens and the global-embedding tokens, each from a
-    context projector, concatenated along the feature axis (:1047-1059)."""
+    """physicsnemo/models/geotransolver/context_projector.py:766-1069: the context is the multi-scale ball-query
+    tokens of every stream (include_local_features=True, :1020-1034), the geometry tokens and the global-embedding
+    tokens, each from a context projector, concatenated along the feature axis (:1036-1059)."""
 
     def __init__(self, geometry_dim, global_dim, n_hidden, n_head, dropout=0.0, slice_num=32, plus=False,
-                 structured_shape=None):
+                 structured_shape=None, functional_dims=(), include_local_features=False, radii=(0.05, 0.25),
+                 neighbors_in_radius=(8, 32), n_hidden_local=32):
         super().__init__()
         dim_head = n_hidden // n_head
         self._context_dim = 0
-        self.local_extractors = None
+        if geometry_dim is not None and include_local_features and structured_shape is None:
+            self.local_extractors = nn.ModuleList([
+                OracleMultiScaleFeatureExtractor(geometry_dim, radii, neighbors_in_radius, n_hidden_local, n_head,
+                                                 dim_head, dropout, slice_num, plus) for _ in functional_dims])
+            self._context_dim += dim_head * len(radii) * len(functional_dims)
+        else:
+            self.local_extractors = None
         if geometry_dim is not None:
             if structured_shape is not None:
                 self.geometry_tokenizer = OracleStructuredContextProjector(geometry_dim, structured_shape, n_head,
@@ -731,47 +832,69 @@ class OracleGlobalContextBuilder(nn.Module):
     def get_context_dim(self):
         return self._context_dim
 
-    def build_context(self, geometry=None, global_embedding=None):
-        parts = []
+    def build_context(self, geometry=None, global_embedding=None, local_positions=None):
+        """Returns the context, or (context, per-stream local features) when the local extractors exist."""
+        parts, local = [], None
+        if self.local_extractors is not None and geometry is not None:
+            local = []
+            for i, ext in enumerate(self.local_extractors):
+                parts.extend(ext.extract_context_features(local_positions[i], geometry))
+                local.append(ext.extract_local_features(local_positions[i], geometry))
         if self.geometry_tokenizer is not None and geometry is not None:
             parts.append(self.geometry_tokenizer(geometry))
         if self.global_tokenizer is not None and global_embedding is not None:
             parts.append(self.global_tokenizer(global_embedding))
-        return torch.cat(parts, dim=-1) if parts else None
+        context = torch.cat(parts, dim=-1) if parts else None
+        return context if self.local_extractors is None else (context, local)
 
 
 class OracleGeoTransolver(nn.Module):
-    """physicsnemo/models/geotransolver/geotransolver.py:390-766 with use_te=False, include_local_features=False,
-    attention_type="GALE", no time input: context from the builder, one preprocess Mlp per input stream, GALE blocks
-    sharing the context, one LayerNorm + Linear head per stream.  No weight re-initialisation: parameters keep the
-    default nn.Linear / orthogonal_ draws of their constructors, in construction order (:460-558)."""
+    """physicsnemo/models/geotransolver/geotransolver.py:390-766 with use_te=False, attention_type="GALE", no time
+    input: context from the builder, one preprocess Mlp per input stream, GALE blocks sharing the context, one
+    LayerNorm + Linear head per stream; with include_local_features the ball-query features of every stream are
+    appended to its hidden state (:725-729), which widens blocks and heads to n_hidden + n_hidden_local * len(radii)
+    (:502-506).  No weight re-initialisation: parameters keep the default nn.Linear / orthogonal_ draws of their
+    constructors, in construction order (:460-558)."""
 
     def __init__(self, functional_dim, out_dim, geometry_dim=None, global_dim=None, n_layers=4, n_hidden=256,
                  dropout=0.0, n_head=8, mlp_ratio=4, slice_num=32, plus=False, structured_shape=None,
-                 state_mixing_mode="weighted"):
+                 state_mixing_mode="weighted", include_local_features=False, radii=None, neighbors_in_radius=None,
+                 n_hidden_local=32):
         super().__init__()
+        radii = [0.05, 0.25] if radii is None else radii
+        neighbors_in_radius = [8, 32] if neighbors_in_radius is None else neighbors_in_radius
         fdims = (functional_dim,) if isinstance(functional_dim, int) else tuple(functional_dim)
         odims = (out_dim,) if isinstance(out_dim, int) else tuple(out_dim)
         if len(fdims) != len(odims):
             raise ValueError(f"functional_dim and out_dim must be the same length, but instead got {len(fdims)} and {len(odims)}")
         self.structured_shape = structured_shape
+        self.include_local_features = include_local_features
         self.context_builder = OracleGlobalContextBuilder(geometry_dim, global_dim, n_hidden, n_head, dropout, slice_num,
-                                                          plus, structured_shape)
+                                                          plus, structured_shape, fdims, include_local_features, radii,
+                                                          neighbors_in_radius, n_hidden_local)
         context_dim = self.context_builder.get_context_dim()
         self.preprocess = nn.ModuleList([OracleMlp(f, n_hidden * 2, n_hidden) for f in fdims])
         self.n_hidden = n_hidden
+        wide = n_hidden + n_hidden_local * len(radii) if include_local_features else n_hidden
         self.blocks = nn.ModuleList([
-            OracleGALEBlock(n_head, n_hidden, dropout, mlp_ratio=mlp_ratio, slice_num=slice_num, context_dim=context_dim,
+            OracleGALEBlock(n_head, wide, dropout, mlp_ratio=mlp_ratio, slice_num=slice_num, context_dim=context_dim,
                             spatial_shape=structured_shape, state_mixing_mode=state_mixing_mode)
             for _ in range(n_layers)
         ])
-        self.ln_mlp_out = nn.ModuleList([nn.Sequential(nn.LayerNorm(n_hidden), nn.Linear(n_hidden, o)) for o in odims])
+        self.ln_mlp_out = nn.ModuleList([nn.Sequential(nn.LayerNorm(wide), nn.Linear(wide, o)) for o in odims])
 
     def forward(self, local_embedding, local_positions=None, global_embedding=None, geometry=None):
         single = isinstance(local_embedding, torch.Tensor)
         streams = (local_embedding,) if single else tuple(local_embedding)
-        context = self.context_builder.build_context(geometry, global_embedding)
+        if isinstance(local_positions, torch.Tensor):
+            local_positions = (local_positions,)
+        context = self.context_builder.build_context(geometry, global_embedding, local_positions)
+        local = None
+        if self.context_builder.local_extractors is not None:
+            context, local = context
         x = [self.preprocess[i](t) for i, t in enumerate(streams)]
+        if local is not None:
+            x = [torch.cat([x[i], local[i]], dim=-1) for i in range(len(x))]
         for blk in self.blocks:
             x = blk(tuple(x), context)
         x = [self.ln_mlp_out[i](t) for i, t in enumerate(x)]

@@ -5,7 +5,8 @@ from .physics_attention import (  # noqa: F401
     PhysicsAttentionStructuredMesh2D,
     PhysicsAttentionStructuredMesh3D,
 )
-from .context_projector import ContextProjector, StructuredContextProjector  # noqa: F401
+from .context_projector import (BQWarp, ContextProjector, GeometricFeatureProcessor,  # noqa: F401
+                                MultiScaleFeatureExtractor, StructuredContextProjector)
 from .flare import FLARE, FLAREBlock, FLAREModel, GALE_FA  # noqa: F401
 from .gale import GALE, GALEBlock, GALEStructuredMesh2D, GALEStructuredMesh3D  # noqa: F401
 from .geotransolver import GeoTransolver, GlobalContextBuilder  # noqa: F401

@@ -1,7 +1,9 @@
 """Context projectors of GeoTransolver on the PhysicsAttention HIP kernels.
 
 Mirrors ``physicsnemo/models/geotransolver/context_projector.py``: ContextProjector:190-378 (Linear projections),
-StructuredContextProjector:380-486 (Conv2d / Conv3d projections), ``_SliceToContextMixin``:108-187.
+StructuredContextProjector:380-486 (Conv2d / Conv3d projections), ``_SliceToContextMixin``:108-187,
+GeometricFeatureProcessor:491-606 and MultiScaleFeatureExtractor:609-763 (ball-query local features; the ball query
+is ``BQWarp`` of ``physicsnemo/nn/module/ball_query.py:32-140`` on the library's HIP kernel).
 
 A context projector is the encoding half of a PhysicsAttention layer -- projections, slice softmax, aggregation --
 and returns the slice tokens ``(B, H, S, D)`` that GALE layers cross-attend to; it never projects back to the points.
@@ -177,3 +179,84 @@ class StructuredContextProjector(_SliceToContextMixin, nn.Module):
             n *= s
         if x.shape[1] != n:
             raise ValueError(f"Expected N={n} tokens for {self._nd}D grid, got N={x.shape[1]}")
+
+
+class BQWarp(nn.Module):
+    """Ball-query layer (reference physicsnemo/nn/module/ball_query.py:32-140; the name is the reference's, the search
+    runs on the library's HIP kernel).  With ``reverse_mapping`` (the default) it returns, for every point of ``p_grid``,
+    the up to ``neighbors_in_radius`` nearest points of ``x`` within ``radius``: (indices (B, Q, K), coordinates
+    (B, Q, K, 3)), nearest first, index 0 / zero coordinates in unused slots -- the order of the reference's torch
+    backend (radius_search/_torch_impl.py:96-160); its Warp backend keeps the first K it meets in hash-grid order, an
+    order that is not specified.  Gradients flow to the coordinates that were gathered, as in the reference."""
+
+    def __init__(self, radius: float = 0.25, neighbors_in_radius: int | None = 10):
+        super().__init__()
+        if neighbors_in_radius is None:
+            raise NotImplementedError("the variable-length form (neighbors_in_radius=None) is not served")
+        self.radius = radius
+        self.neighbors_in_radius = neighbors_in_radius
+
+    def forward(self, x: torch.Tensor, p_grid: torch.Tensor, reverse_mapping: bool = True):
+        if p_grid.shape[-1] != x.shape[-1] or x.shape[-1] != 3:
+            raise ValueError("The last dimension of p_grid and x must be 3")
+        if p_grid.ndim in (4, 5):
+            p_grid = p_grid.reshape(p_grid.shape[0], -1, 3)
+        elif p_grid.ndim != 3:
+            raise ValueError("p_grid must be 3D, 4D, 5D only")
+        points, queries = (x, p_grid) if reverse_mapping else (p_grid, x)
+        idx, out, counts = PF.ball_query(points, queries, self.radius, self.neighbors_in_radius)
+        if torch.is_grad_enabled() and points.requires_grad:
+            K = self.neighbors_in_radius
+            used = torch.arange(K, device=idx.device) < counts[..., None]
+            flat = idx.reshape(idx.shape[0], -1, 1).expand(-1, -1, 3)
+            out = points.gather(1, flat).reshape(*idx.shape, 3) * used[..., None].to(points.dtype)
+        else:
+            out = out.to(points.dtype)
+        return idx, out
+
+
+class GeometricFeatureProcessor(nn.Module):
+    """One radius of the local geometric features (reference :491-606): ball query, the neighbours' coordinates
+    flattened, a three-layer GELU Mlp (``mlp.layers.0/2/4``), tanh."""
+
+    def __init__(self, radius: float, neighbors_in_radius: int, feature_dim: int, hidden_dim: int):
+        super().__init__()
+        self.bq_warp = BQWarp(radius=radius, neighbors_in_radius=neighbors_in_radius)
+        self.mlp = nn.Module()
+        self.mlp.layers = nn.Sequential(nn.Linear(feature_dim * neighbors_in_radius, hidden_dim), nn.GELU(),
+                                        nn.Linear(hidden_dim, hidden_dim // 2), nn.GELU(),
+                                        nn.Linear(hidden_dim // 2, hidden_dim))
+
+    def forward(self, query_points: torch.Tensor, key_features: torch.Tensor) -> torch.Tensor:
+        if query_points.ndim != 3:
+            raise ValueError(f"Expected 3D query_points tensor (B, N, 3), got {query_points.ndim}D tensor with shape "
+                             f"{tuple(query_points.shape)}")
+        if key_features.ndim != 3:
+            raise ValueError(f"Expected 3D key_features tensor (B, N, C), got {key_features.ndim}D tensor with shape "
+                             f"{tuple(key_features.shape)}")
+        _, neighbors = self.bq_warp(query_points, key_features)
+        return torch.tanh(self.mlp.layers(neighbors.flatten(2)))
+
+
+class MultiScaleFeatureExtractor(nn.Module):
+    """Local geometric features at several radii (reference :609-763): per radius one processor and one context
+    projector that turns its features into slice tokens."""
+
+    def __init__(self, geometry_dim: int, radii: list, neighbors_in_radius: list, hidden_dim: int, n_head: int,
+                 dim_head: int, dropout: float = 0.0, slice_num: int = 64, use_te: bool = False, plus: bool = False,
+                 concrete_dropout: bool = False):
+        super().__init__()
+        self.num_scales = len(radii)
+        self.processors = nn.ModuleList([GeometricFeatureProcessor(radii[i], neighbors_in_radius[i], geometry_dim,
+                                                                   hidden_dim) for i in range(self.num_scales)])
+        self.tokenizers = nn.ModuleList([ContextProjector(hidden_dim, n_head, dim_head, dropout, slice_num, use_te, plus,
+                                                          concrete_dropout=concrete_dropout)
+                                         for _ in range(self.num_scales)])
+
+    def extract_context_features(self, spatial_coords: torch.Tensor, geometry: torch.Tensor) -> list:
+        """One (B, H, S, D) context per radius: the geometry points' neighbourhoods among the mesh points."""
+        return [tok(proc(spatial_coords, geometry)) for proc, tok in zip(self.processors, self.tokenizers)]
+
+    def extract_local_features(self, spatial_coords: torch.Tensor, geometry: torch.Tensor) -> torch.Tensor:
+        """(B, N, hidden_dim * num_scales): the mesh points' neighbourhoods among the geometry points."""
+        return torch.cat([proc(geometry, spatial_coords) for proc in self.processors], dim=-1)

@@ -558,6 +558,28 @@ int pa_cols_gemm(int64_t rows, const void *a, int64_t lda, int64_t cols_a, const
                              static_cast<hipStream_t>(stream));
 }
 
+int pa_ball_query(int64_t batch, int64_t n_points, int64_t n_queries, int64_t max_neighbors, float radius,
+                  const float *points, const float *queries, int64_t *indices, float *neighbor_points,
+                  float *neighbor_dists, int32_t *counts, void *stream) {
+  if (batch <= 0 || n_points <= 0 || n_queries <= 0 || max_neighbors <= 0 || !(radius >= 0.f)) return PA_ERR_DIMS;
+  if (!points || !queries || !indices) return PA_ERR_NULL;
+  return pa::ballquery::ball_query(batch, n_points, n_queries, max_neighbors, radius, points, queries, indices,
+                                   neighbor_points, neighbor_dists, counts, static_cast<hipStream_t>(stream));
+}
+
+int pa_ball_query_cells(int64_t batch, int64_t n_points, int64_t n_queries, int64_t max_neighbors, float radius,
+                        int64_t cells_per_axis, const float *grid, const float *sorted_points,
+                        const int32_t *sorted_index, const int32_t *cell_start, const float *queries,
+                        const int32_t *query_order, int64_t *indices, float *neighbor_points, float *neighbor_dists,
+                        int32_t *counts, void *stream) {
+  if (batch <= 0 || n_points <= 0 || n_queries <= 0 || max_neighbors <= 0 || cells_per_axis <= 0 || !(radius >= 0.f))
+    return PA_ERR_DIMS;
+  if (!grid || !sorted_points || !sorted_index || !cell_start || !queries || !indices) return PA_ERR_NULL;
+  return pa::ballquery::ball_query_cells(batch, n_points, n_queries, max_neighbors, radius, cells_per_axis, grid,
+                                         sorted_points, sorted_index, cell_start, queries, query_order, indices,
+                                         neighbor_points, neighbor_dists, counts, static_cast<hipStream_t>(stream));
+}
+
 int64_t pa_cols_gemm_f32_chunks(int64_t rows, int64_t cols_a, int64_t cols_b) {
   if (rows <= 0 || cols_a <= 0 || cols_b <= 0) return PA_ERR_DIMS;
   return pa::gemm::cols_gemm_f32_chunks(rows, cols_a, cols_b, compute_units());

@@ -127,6 +127,15 @@ int slice_cross_mix(const pa_shape &s, const pa_gale_params &gp, int64_t Sc, int
                     const float *self_token, const float *context, float *out_token, void *tokp, hipStream_t st);
 }  // namespace gale
 
+namespace ballquery {
+int ball_query(int64_t B, int64_t Np, int64_t Nq, int64_t K, float radius, const float *points, const float *queries,
+               int64_t *indices, float *out_points, float *out_dists, int32_t *counts, hipStream_t st);
+int ball_query_cells(int64_t B, int64_t Np, int64_t Nq, int64_t K, float radius, int64_t G, const float *grid,
+                     const float *sorted_points, const int32_t *sorted_index, const int32_t *cell_start,
+                     const float *queries, const int32_t *query_order, int64_t *indices, float *out_points,
+                     float *out_dists, int32_t *counts, hipStream_t st);
+}  // namespace ballquery
+
 namespace mfma {
 bool staged_supported(int dtype, const pa_shape &s);
 int slice_softmax_pack(const pa_shape &s, const pa_params &p, const void *x_mid, void *w_pack, int num_cu,

@@ -596,3 +596,67 @@ def deslice(w, tok_out, dims: LayerDims):
     _lib.check(_lib.load().pa_deslice(_lib.dtype_code(w.dtype), byref(dims.c()), w.data_ptr(), tok_out.data_ptr(),
                                       out_x.data_ptr(), _lib.current_stream_ptr(w.device)), "pa_deslice")
     return out_x
+
+
+def _cell_list(pts: torch.Tensor, radius: float, G: int):
+    """Bins (B, Np, 3) points into G^3 cells of edge >= radius * 1.0001 per batch: (grid (B, 6), points sorted by
+    (batch, cell), their indices within the batch, cell offsets) -- the cell list `pa_ball_query_cells` reads.  Device
+    ops only, no synchronisation."""
+    B, Np = pts.shape[0], pts.shape[1]
+    lo, hi = pts.amin(1), pts.amax(1)
+    edge = torch.clamp((hi - lo) / G, min=max(float(radius) * 1.0001, 1e-30))
+    grid = torch.cat([lo, 1.0 / edge], dim=1).contiguous()  # (B, 6)
+    return grid, *_bin(pts, grid, G, want_start=True)
+
+
+def _bin(p: torch.Tensor, grid: torch.Tensor, G: int, want_start: bool):
+    """Order of the points of `p` (B, N, 3) by (batch, cell of `grid`)."""
+    B, N = p.shape[0], p.shape[1]
+    c = torch.floor((p - grid[:, None, :3]) * grid[:, None, 3:]).clamp_(0, G - 1).to(torch.int64)
+    key = ((c[..., 0] * G + c[..., 1]) * G + c[..., 2]) + torch.arange(B, device=p.device)[:, None] * (G ** 3)
+    skey, perm = torch.sort(key.reshape(-1))
+    within = (perm - torch.div(perm, N, rounding_mode="floor") * N).to(torch.int32)
+    if not want_start:
+        return within
+    start = torch.searchsorted(skey, torch.arange(B * G ** 3 + 1, device=p.device)).to(torch.int32)
+    return p.reshape(-1, 3)[perm].contiguous(), within, start
+
+
+def ball_query(points: torch.Tensor, queries: torch.Tensor, radius: float, max_neighbors: int, return_dists: bool = False,
+               method: str | None = None):
+    """For every query the up to `max_neighbors` nearest points within `radius`, nearest first.
+
+    points (B, Np, 3), queries (B, Nq, 3) -> indices (B, Nq, K) int64 (0 in unused slots), neighbor coordinates
+    (B, Nq, K, 3) float32 (zeros in unused slots), counts (B, Nq) int32 [, distances (B, Nq, K)].  Not differentiable:
+    callers that need gradients w.r.t. `points` gather them again by the indices.  `method`: "pairs" looks at every
+    pair, "cells" bins the points into a uniform grid first (the default from 2048 points on); same results."""
+    if not (points.is_cuda and queries.is_cuda):
+        raise RuntimeError("physicsnemo_amd kernels need CUDA (ROCm) tensors")
+    if points.ndim != 3 or queries.ndim != 3 or points.shape[-1] != 3 or queries.shape[-1] != 3:
+        raise ValueError("ball_query needs (B, N, 3) points and queries")
+    if points.shape[0] != queries.shape[0]:
+        raise ValueError(f"Batch dimensions must match: points has {points.shape[0]}, queries has {queries.shape[0]}")
+    pts, qs = points.detach().float().contiguous(), queries.detach().float().contiguous()
+    B, Np, Nq, K = pts.shape[0], pts.shape[1], qs.shape[1], int(max_neighbors)
+    idx = torch.empty(B, Nq, K, dtype=torch.int64, device=pts.device)
+    out = torch.empty(B, Nq, K, 3, dtype=torch.float32, device=pts.device)
+    counts = torch.empty(B, Nq, dtype=torch.int32, device=pts.device)
+    dists = torch.empty(B, Nq, K, dtype=torch.float32, device=pts.device) if return_dists else None
+    method = method or ("cells" if Np >= 2048 else "pairs")
+    if method == "cells":
+        G = int(min(128, max(2, round((Np / 2.0) ** (1.0 / 3.0)))))  # about two points per cell of a filled box
+        while B * G ** 3 >= 2 ** 31:
+            G //= 2
+        grid, spts, sidx, start = _cell_list(pts, radius, G)
+        order = _bin(qs, grid, G, want_start=False) if Nq >= 256 else None
+        _lib.check(_lib.load().pa_ball_query_cells(B, Np, Nq, K, float(radius), G, grid.data_ptr(), spts.data_ptr(),
+                                                   sidx.data_ptr(), start.data_ptr(), qs.data_ptr(), _lib.ptr(order),
+                                                   idx.data_ptr(), out.data_ptr(), _lib.ptr(dists), counts.data_ptr(),
+                                                   _lib.current_stream_ptr(pts.device)), "pa_ball_query_cells")
+    elif method == "pairs":
+        _lib.check(_lib.load().pa_ball_query(B, Np, Nq, K, float(radius), pts.data_ptr(), qs.data_ptr(), idx.data_ptr(),
+                                             out.data_ptr(), _lib.ptr(dists), counts.data_ptr(),
+                                             _lib.current_stream_ptr(pts.device)), "pa_ball_query")
+    else:
+        raise ValueError(f"unknown ball_query method {method!r}")
+    return (idx, out, counts, dists) if return_dists else (idx, out, counts)

@@ -1,12 +1,12 @@
 """GeoTransolver on the PhysicsAttention / GALE HIP kernels.
 
 Mirrors ``physicsnemo/models/geotransolver/geotransolver.py`` (GeoTransolver:390-766) and the context builder of
-``context_projector.py`` (GlobalContextBuilder:766-1069) for ``include_local_features=False``: geometry and global
-embeddings are projected onto slice tokens by context projectors and concatenated into the context every GALE block
-cross-attends to; each input stream has its own preprocess Mlp and LayerNorm + Linear head.  Same constructor
-arguments, parameter names and forward signature as the reference, so its checkpoints load unchanged.  The ball-query
-local features (``include_local_features=True``) and the not-yet-implemented ``time`` input of the reference are not
-served.
+``context_projector.py`` (GlobalContextBuilder:766-1069): geometry and global embeddings are projected onto slice
+tokens by context projectors and concatenated into the context every GALE block cross-attends to; with
+``include_local_features=True`` ball-query neighbourhoods at several radii add further contexts and widen every
+point's hidden state; each input stream has its own preprocess Mlp and LayerNorm + Linear head.  Same constructor
+arguments, parameter names and forward signature as the reference, so its checkpoints load unchanged.  The
+not-yet-implemented ``time`` input of the reference is refused as it is there.
 """
 from __future__ import annotations
 
@@ -17,7 +17,7 @@ import torch
 import torch.nn as nn
 
 from . import autograd as PA
-from .context_projector import ContextProjector, StructuredContextProjector
+from .context_projector import ContextProjector, MultiScaleFeatureExtractor, StructuredContextProjector
 from .gale import GALEBlock
 from .transolver import Mlp, Transolver
 
@@ -31,8 +31,8 @@ def _normalize_dim(x) -> tuple:
 
 
 class GlobalContextBuilder(nn.Module):
-    """Context (B, H, S, D_c) from geometry and global embeddings (reference context_projector.py:766-1069 without the
-    local ball-query extractors): one context projector each, concatenated along the feature axis."""
+    """Context (B, H, S, D_c) from geometry and global embeddings and, optionally, the multi-scale ball-query features
+    (reference context_projector.py:766-1069): one context projector each, concatenated along the feature axis."""
 
     def __init__(self, functional_dims: tuple, geometry_dim: int | None = None, global_dim: int | None = None,
                  radii=None, neighbors_in_radius=None, n_hidden_local: int = 32, n_hidden: int = 256, n_head: int = 8,
@@ -40,13 +40,19 @@ class GlobalContextBuilder(nn.Module):
                  include_local_features: bool = False, structured_shape: tuple | None = None,
                  concrete_dropout: bool = False):
         super().__init__()
-        if include_local_features:
-            raise NotImplementedError("the ball-query local features (include_local_features=True) are not served")
+        radii = [0.05, 0.25] if radii is None else radii
+        neighbors_in_radius = [8, 32] if neighbors_in_radius is None else neighbors_in_radius
         dim_head = n_hidden // n_head
         self.structured_shape = structured_shape
-        self.local_extractors = None
         self._context_dim = 0
         kw = dict(use_te=use_te, plus=plus, concrete_dropout=concrete_dropout)
+        if geometry_dim is not None and include_local_features and structured_shape is None:
+            self.local_extractors = nn.ModuleList([
+                MultiScaleFeatureExtractor(geometry_dim, radii, neighbors_in_radius, n_hidden_local, n_head, dim_head,
+                                           dropout, slice_num, **kw) for _ in functional_dims])
+            self._context_dim += dim_head * len(radii) * len(functional_dims)
+        else:
+            self.local_extractors = None
         if geometry_dim is not None:
             if structured_shape is not None:
                 self.geometry_tokenizer = StructuredContextProjector(geometry_dim, structured_shape, n_head, dim_head,
@@ -66,15 +72,25 @@ class GlobalContextBuilder(nn.Module):
         return self._context_dim
 
     def build_context(self, local_embeddings, local_positions, geometry=None, global_embedding=None):
-        """Returns (context or None, None, detached geometry context or None), as the reference does."""
-        parts, geometry_context = [], None
+        """Returns (context or None, per-stream local features or None, detached geometry context or None), as the
+        reference does."""
+        if len(local_embeddings) == 0:
+            raise ValueError("Expected non-empty tuple of local embeddings")
+        parts, geometry_context, local_features = [], None, None
+        if local_positions is None and self.local_extractors is not None:
+            raise ValueError("Local positions are required if local features are enabled.")
+        if self.local_extractors is not None and geometry is not None:
+            local_features = []
+            for i in range(len(local_embeddings)):
+                parts.extend(self.local_extractors[i].extract_context_features(local_positions[i], geometry))
+                local_features.append(self.local_extractors[i].extract_local_features(local_positions[i], geometry))
         if self.geometry_tokenizer is not None and geometry is not None:
             geometry_context = self.geometry_tokenizer(geometry)
             parts.append(geometry_context)
         if self.global_tokenizer is not None and global_embedding is not None:
             parts.append(self.global_tokenizer(global_embedding))
         context = torch.cat(parts, dim=-1) if parts else None
-        return context, None, (geometry_context.detach() if geometry_context is not None else None)
+        return context, local_features, (geometry_context.detach() if geometry_context is not None else None)
 
 
 class GeoTransolver(nn.Module):
@@ -116,7 +132,9 @@ class GeoTransolver(nn.Module):
         if n_hidden % n_head != 0:
             raise ValueError(f"GeoTransolver requires n_hidden % n_head == 0, got n_hidden={n_hidden}, n_head={n_head}")
         functional_dims, out_dims = _normalize_dim(functional_dim), _normalize_dim(out_dim)
-        self.radii = []
+        radii = [0.05, 0.25] if radii is None else radii
+        neighbors_in_radius = [8, 32] if neighbors_in_radius is None else neighbors_in_radius
+        self.radii = radii if include_local_features else []
         self.context_builder = GlobalContextBuilder(
             functional_dims=functional_dims, geometry_dim=geometry_dim, global_dim=global_dim, radii=radii,
             neighbors_in_radius=neighbors_in_radius, n_hidden_local=n_hidden_local, n_hidden=n_hidden, n_head=n_head,
@@ -129,14 +147,16 @@ class GeoTransolver(nn.Module):
                              f"{len(functional_dims)} and {len(out_dims)}")
         self.preprocess = nn.ModuleList([Mlp(f, n_hidden * 2, n_hidden, act) for f in functional_dims])
         self.n_hidden = n_hidden
+        effective_hidden = n_hidden + n_hidden_local * len(self.radii) if include_local_features else n_hidden
         self.blocks = nn.ModuleList([
-            GALEBlock(num_heads=n_head, hidden_dim=n_hidden, dropout=dropout, act=act, mlp_ratio=mlp_ratio,
+            GALEBlock(num_heads=n_head, hidden_dim=effective_hidden, dropout=dropout, act=act, mlp_ratio=mlp_ratio,
                       slice_num=slice_num, last_layer=(i == n_layers - 1), use_te=use_te, plus=plus,
                       context_dim=context_dim, spatial_shape=structured_shape, attention_type=attention_type,
                       concrete_dropout=concrete_dropout, state_mixing_mode=state_mixing_mode)
             for i in range(n_layers)
         ])
-        self.ln_mlp_out = nn.ModuleList([nn.Sequential(nn.LayerNorm(n_hidden), nn.Linear(n_hidden, o)) for o in out_dims])
+        self.ln_mlp_out = nn.ModuleList([nn.Sequential(nn.LayerNorm(effective_hidden), nn.Linear(effective_hidden, o))
+                                         for o in out_dims])
         self.time_input = time_input
         if time_input:
             self.time_fc = nn.Sequential(nn.Linear(n_hidden, n_hidden), nn.SiLU(), nn.Linear(n_hidden, n_hidden))
@@ -186,8 +206,11 @@ class GeoTransolver(nn.Module):
         if global_embedding is not None and global_embedding.ndim != 3:
             raise ValueError(f"Expected 3D global_embedding tensor (B, N_g, C_g), got {global_embedding.ndim}D tensor "
                              f"with shape {tuple(global_embedding.shape)}")
-        embedding_states, _, _ = self.context_builder.build_context(streams, local_positions, geometry, global_embedding)
+        embedding_states, local_bq, _ = self.context_builder.build_context(streams, local_positions, geometry,
+                                                                           global_embedding)
         x = [self.preprocess[i](t) for i, t in enumerate(streams)]
+        if self.include_local_features and local_bq is not None:
+            x = [torch.cat([x[i], local_bq[i].to(x[i].dtype)], dim=-1) for i in range(len(x))]
         needs_grad = torch.is_grad_enabled() and (any(t.requires_grad for t in x)
                                                   or any(p.requires_grad for p in self.parameters()))
         chain = not needs_grad and all(t.is_cuda for t in x) and all(hasattr(b.Attn, "gale_params") for b in self.blocks)
