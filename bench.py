@@ -14,6 +14,7 @@ from __future__ import annotations
 
 import argparse
 import json
+import math
 import os
 import statistics
 import sys
@@ -247,6 +248,13 @@ def time_variants(points, C, S, reps=5):
         entry(f"GeoTransolver bf16, 4 GALE blocks, hidden {C}, S={S}, geometry {pts // 4} points", pts,
               timed(lambda: geo(ge, None, gl, gg), 3))
     del ge, gg, gl, geo
+    # ball query of the GeoTransolver local features: 8 nearest within a radius that holds about 8 points
+    from physicsnemo_amd import functional as PF
+    cloud, probes = torch.rand(1, pts, 3, device="cuda"), torch.rand(1, pts, 3, device="cuda")
+    radius = (8 / pts * 3 / (4 * math.pi)) ** (1 / 3)
+    entry(f"ball query (cell list), {pts} points, K=8, radius {radius:.4f}", pts,
+          timed(lambda: PF.ball_query(cloud, probes, radius, 8), 3))
+    del cloud, probes
     # structured 3-D, 64^3 grid, Conv3d k=3 projections
     g = 64
     s3 = pn.PhysicsAttentionStructuredMesh3D(C, (g, g, g), heads=H, dim_head=32, slice_num=S, kernel=3,
