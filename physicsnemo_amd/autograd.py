@@ -21,6 +21,12 @@ def _rows(t: torch.Tensor) -> torch.Tensor:
     return t.reshape(-1, t.shape[-1])
 
 
+def _aligned(t: torch.Tensor) -> torch.Tensor:
+    """`t` itself, or a copy when it is a view that starts off a 16-byte boundary (a batch element of odd size)."""
+    t = t.contiguous()
+    return t if t.data_ptr() % 16 == 0 else t.clone()
+
+
 def _wgrad(d_out: torch.Tensor, inp: torch.Tensor):
     """(d W, d b) = (d out^T . in, column sums of d out) over all rows: one pass of the library's MFMA kernel where it
     serves the shape, else the GEMM library and a reduction."""
@@ -391,7 +397,8 @@ class FlareFunction(torch.autograd.Function):
     """FLARE layer core (flare_attention.py:38-72, :222-255) given the composed score / value weights: differentiable
     w.r.t. x, the four composed tensors and out_linear.  The composition itself (q_global, self_k / self_v and
     in_project_x folded into two matrices) is a handful of small tensor products done by the caller under autograd, so
-    the gradients reach the layer's own parameters through it."""
+    the gradients reach the layer's own parameters through it.  Without out_linear (`wo` None) the result is the
+    attention output (B, N, H*D) itself, for callers that blend it with something else first (GALE_FA)."""
 
     @staticmethod
     def forward(ctx, x, dims, w_a, b_a, w_v, b_v, wo, bo):
@@ -404,23 +411,33 @@ class FlareFunction(torch.autograd.Function):
         den = norm - 1e-2  # the aggregation kernel adds the PhysicsAttention epsilon to the divisor; FLARE has none
         z = (tok * (norm / den).unsqueeze(-1)).contiguous()
         row_w = PF.flare_softmax_rows_(scores, dims)
+        ctx.dims = dims
+        ctx.projected = wo is not None
+        if not ctx.projected:
+            out_x = PF.deslice(row_w, z, dims)
+            ctx.save_for_backward(x, row_w, col_w, values, z, den, wa_k, wv_k)
+            ctx.dtypes = tuple(t.dtype for t in (w_a, b_a, w_v, b_v))
+            return out_x
         kp = {"out_linear_weight": wo.detach().to(x.dtype).contiguous().reshape(-1),
               "out_linear_bias": bo.detach().float().contiguous()}
         y, out_x = PF.deslice_project(row_w, z, kp, dims, return_out_x=True)
-        ctx.save_for_backward(x, row_w, col_w, values, z, den, out_x, wa_k, wv_k, kp["out_linear_weight"])
-        ctx.dims = dims
+        ctx.save_for_backward(x, row_w, col_w, values, z, den, wa_k, wv_k, out_x, kp["out_linear_weight"])
         ctx.dtypes = tuple(t.dtype for t in (w_a, b_a, w_v, b_v, wo, bo))
         return y
 
     @staticmethod
     def backward(ctx, dy):
-        x, row_w, col_w, values, z, den, out_x, wa_k, wv_k, wo_k = ctx.saved_tensors
+        x, row_w, col_w, values, z, den, wa_k, wv_k = ctx.saved_tensors[:8]
         dims = ctx.dims
         B, N, C, H, D, S = dims.B, dims.N, dims.C, dims.H, dims.D, dims.S
         HD, HS = H * D, H * S
         dy = dy.to(x.dtype).contiguous()
-        g = PF.rows_gemm(dy, wo_k.view(C, HD).t().contiguous(), None, dims, C, HD)
-        d_wo, d_bo = _wgrad(dy, out_x)
+        if ctx.projected:
+            out_x, wo_k = ctx.saved_tensors[8:]
+            g = PF.rows_gemm(dy, wo_k.view(C, HD).t().contiguous(), None, dims, C, HD)
+            d_wo, d_bo = _wgrad(dy, out_x)
+        else:
+            g, d_wo, d_bo = dy, None, None
         d_z = PF.slice_weighted_sum(row_w, g, dims)[..., :D]
         d_num = (d_z / den.unsqueeze(-1)).contiguous()
         d_den = (-(d_z * z).sum(-1) / den).contiguous()
@@ -434,7 +451,57 @@ class FlareFunction(torch.autograd.Function):
         d_wv, d_bv = _wgrad(d_v, x)
         grads = [gr.float().reshape(shape).to(dt) for gr, shape, dt in zip(
             (d_wa, d_ba, d_wv, d_bv, d_wo, d_bo), ((HS, C), (HS,), (HD, C), (HD,), (C, HD), (C,)), ctx.dtypes)]
+        if not ctx.projected:
+            grads += [None, None]
         return (dx, None, *grads)
+
+
+class PointCrossFunction(torch.autograd.Function):
+    """Cross-attention of every point to a small set of context tokens, scale 1 (GALE_FA, reference gale.py:735-744):
+    out[b,n,h,:] = sum_u softmax_u(x[b,n,:] . w_c[b,(h,u),:] + b_c[b,(h,u)]) v[b,h,u,:].  The caller folds in_project_x,
+    cross_q and the context's keys into the per-batch score weight `w_c` (B, H*Sc, C) / `b_c` (B, H*Sc) and projects
+    the context's values `v` (B, H, Sc, D), all under autograd.  Scores from the row GEMM, the in-place row softmax and
+    the deslice kernel; backward: the row-softmax part of the FLARE per-point kernel (gather weights zero), the
+    slice-weighted sum for d v, row / column GEMMs for d x and d w_c."""
+
+    @staticmethod
+    def forward(ctx, x, dims, w_c, b_c, v):
+        B, N, C, H, Sc = dims.B, dims.N, dims.C, dims.H, dims.S
+        one = PF.LayerDims(1, N, C, H, dims.D, Sc)
+        wk = w_c.detach().to(x.dtype).contiguous()
+        bk = b_c.detach().float().contiguous()
+        scores = torch.empty(B, N, H, Sc, dtype=x.dtype, device=x.device)
+        for b in range(B):  # the score weight holds the batch element's keys
+            scores[b] = PF.rows_gemm(_aligned(x[b:b + 1]), _aligned(wk[b]), _aligned(bk[b]), one, C, H * Sc).view(N, H, Sc)
+        p = PF.flare_softmax_rows_(scores, dims)
+        v32 = v.detach().float().contiguous()
+        ctx.save_for_backward(x, p, v32, wk)
+        ctx.dims = dims
+        ctx.dtypes = (w_c.dtype, b_c.dtype, v.dtype)
+        return PF.deslice(p, v32, dims)
+
+    @staticmethod
+    def backward(ctx, g):
+        x, p, v32, wk = ctx.saved_tensors
+        dims = ctx.dims
+        B, N, C, H, D, Sc = dims.B, dims.N, dims.C, dims.H, dims.D, dims.S
+        g = g.to(x.dtype).contiguous()
+        d_v = PF.slice_weighted_sum(p, g, dims)[..., :D]
+        zeros_w = torch.zeros_like(p)
+        d_s, _ = PF.flare_backward_points(p, zeros_w, g, g, v32, torch.zeros_like(v32),
+                                          torch.zeros(B, H, Sc, dtype=torch.float32, device=x.device), dims)
+        d_s = d_s.view(B, N, H * Sc)
+        one = PF.LayerDims(1, N, C, H, D, Sc)
+        dx = torch.empty_like(x) if ctx.needs_input_grad[0] else None
+        d_w, d_b = [], []
+        for b in range(B):
+            if dx is not None:
+                dx[b] = PF.rows_gemm(_aligned(d_s[b:b + 1]), _aligned(wk[b].t()), None, one, H * Sc, C)[0]
+            dw_b, db_b = _wgrad(_aligned(d_s[b]), _aligned(x[b]))
+            d_w.append(dw_b.float())
+            d_b.append(db_b.float())
+        return (dx, None, torch.stack(d_w).to(ctx.dtypes[0]), torch.stack(d_b).to(ctx.dtypes[1]),
+                d_v.to(ctx.dtypes[2]))
 
 
 class LinearFunction(torch.autograd.Function):

@@ -144,7 +144,8 @@ class GALE_FA(nn.Module):
     Every stage is a row GEMM or a slice-weight kernel of the layer family: the cross-attention of a point is
     ``softmax_u(q_n . k_u) v_u`` with scale 1 -- scores from a row GEMM whose weight folds in_project_x, cross_q and the
     context's keys (one weight per batch element), an in-place row softmax, and the deslice kernel with the context's
-    values as slice tokens.  Forward only."""
+    values as slice tokens.  With gradients required the same kernels run inside `FlareFunction` (self-attention) and
+    `PointCrossFunction` (cross-attention); the weight compositions and the blend are PyTorch ops under autograd."""
 
     def __init__(self, dim: int, heads: int = 8, dim_head: int = 64, dropout: float = 0.0, n_global_queries: int = 64,
                  use_te: bool = False, context_dim: int = 0, concrete_dropout: bool = False,
@@ -170,6 +171,41 @@ class GALE_FA(nn.Module):
         self._cache: dict = {}
 
     kernel_params = FLARE.kernel_params
+    _composed = FLARE._composed
+
+    def _cross_composed(self, context: torch.Tensor):
+        """(score weight (B, H*Sc, C), score bias (B, H*Sc), values (B, H, Sc, D)) as differentiable float32 functions of
+        the parameters and the context."""
+        H, D, C = self.heads, self.dim_head, self.dim
+        ctx = context.float()
+        B, Sc = ctx.shape[0], ctx.shape[2]
+        k = torch.nn.functional.linear(ctx, self.cross_k.weight.float(), self.cross_k.bias.float())  # (B, H, Sc, D)
+        v = torch.nn.functional.linear(ctx, self.cross_v.weight.float(), self.cross_v.bias.float())
+        wx_h, bx_h = self.in_project_x.weight.float().view(H, D, C), self.in_project_x.bias.float().view(H, D)
+        kq = k @ self.cross_q.weight.float()
+        w_c = torch.einsum("bhud,hdc->bhuc", kq, wx_h).reshape(B, H * Sc, C)
+        b_c = (torch.einsum("bhud,hd->bhu", kq, bx_h) + k @ self.cross_q.bias.float()).reshape(B, H * Sc)
+        return w_c, b_c, v
+
+    def _forward_one_with_grad(self, t: torch.Tensor, context: torch.Tensor | None, dims: PF.LayerDims) -> torch.Tensor:
+        from .autograd import FlareFunction, PointCrossFunction, linear
+
+        B, N, H, D = dims.B, dims.N, dims.H, dims.D
+        with torch.autocast("cuda", enabled=False):
+            w_a, b_a, w_v, b_v = self._composed(t.device)
+            y = FlareFunction.apply(t, dims, w_a, b_a, w_v, b_v, None, None)
+            if context is not None:
+                w_c, b_c, v = self._cross_composed(context.to(t.device))
+                cdims = PF.LayerDims(B, N, dims.C, H, D, context.shape[2])
+                cross = PointCrossFunction.apply(t, cdims, w_c, b_c, v)
+                if self.state_mixing_mode == "weighted":
+                    m = torch.sigmoid(self.state_mixing.float())
+                    y = (m * y.float() + (1 - m) * cross.float()).to(t.dtype)
+                else:
+                    lin = self.concat_project[0]
+                    cat = torch.cat([y.view(B, N, H, D), cross.view(B, N, H, D)], dim=-1)
+                    y = torch.nn.functional.gelu(linear(cat, lin.weight, lin.bias)).reshape(B, N, H * D)
+            return linear(y, self.out_linear.weight, self.out_linear.bias)
 
     def _self_attention(self, x: torch.Tensor, p: dict, dims: PF.LayerDims) -> torch.Tensor:
         """FLARE two-pass attention -> (B, N, H*D), before out_linear."""
@@ -198,7 +234,8 @@ class GALE_FA(nn.Module):
         one = PF.LayerDims(1, N, C, H, D, Sc)
         scores = torch.empty(B, N, H, Sc, dtype=x.dtype, device=x.device)
         for b in range(B):  # the score weight holds the batch element's keys
-            scores[b] = PF.rows_gemm(x[b:b + 1], w_c[b].to(x.dtype).contiguous(), b_c[b].float().contiguous(), one, C,
+            xb = x[b:b + 1] if x[b].data_ptr() % 16 == 0 else x[b:b + 1].clone()
+            scores[b] = PF.rows_gemm(xb, w_c[b].to(x.dtype).contiguous(), b_c[b].float().contiguous(), one, C,
                                      H * Sc).view(N, H, Sc)
         return PF.deslice(PF.flare_softmax_rows_(scores, cdims), v, cdims)
 
@@ -225,8 +262,8 @@ class GALE_FA(nn.Module):
                                  f"got {t.ndim}D tensor with shape {tuple(t.shape)}")
             if not t.is_cuda:
                 raise RuntimeError("physicsnemo_amd GALE_FA runs on GPU tensors only (no CPU fallback)")
-            if torch.is_grad_enabled() and (t.requires_grad or any(p.requires_grad for p in self.parameters())):
-                raise NotImplementedError("the backward kernels do not cover GALE_FA; run under torch.no_grad()")
+            needs_grad = torch.is_grad_enabled() and (t.requires_grad or (context is not None and context.requires_grad)
+                                                      or any(p.requires_grad for p in self.parameters()))
             if torch.is_autocast_enabled("cuda") and torch.get_autocast_dtype("cuda") == torch.bfloat16:
                 t = t.to(torch.bfloat16)
             if t.dtype not in (torch.float32, torch.bfloat16):
@@ -234,11 +271,14 @@ class GALE_FA(nn.Module):
             t = t.contiguous()
             B, N, C = t.shape
             dims = PF.LayerDims(B, N, C, self.heads, self.dim_head, self.n_global_queries)
+            if context is not None and self.context_dim <= 0:
+                raise ValueError("this GALE_FA was built without cross-attention (context_dim = 0)")
+            if needs_grad:
+                outs.append(self.out_dropout(self._forward_one_with_grad(t, context, dims)))
+                continue
             p = self.kernel_params(t.dtype, t.device)
             y = self._self_attention(t, p, dims)
             if context is not None:
-                if self.context_dim <= 0:
-                    raise ValueError("this GALE_FA was built without cross-attention (context_dim = 0)")
                 y = self._mix(y, self._cross_attention(t, context.to(t.device), dims), dims)
             out = PF.rows_gemm(y, p["out_linear_weight"].view(C, -1), p["out_linear_bias"],
                                PF.LayerDims(B, N, y.shape[-1], 1, 1, 1), y.shape[-1], C)

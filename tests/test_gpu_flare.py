@@ -159,8 +159,84 @@ def test_bf16_gale_fa():
         got = hip((x.cuda().bfloat16(),), ctx.cuda())[0]
     assert got.dtype == torch.bfloat16
     assert_rel_l2(got, want, "bf16 GALE_FA y", tol=1e-2)
-    with pytest.raises(NotImplementedError):
-        hip((x.cuda(),), ctx.cuda())
+
+
+@pytest.mark.parametrize("mode,dim,heads,dim_head,S,B,N,Sc,Dc,with_ctx", [
+    ("weighted", 32, 4, 8, 8, 2, 300, 5, 7, True),
+    ("concat_project", 48, 3, 16, 20, 3, 77, 9, 4, True),
+    ("weighted", 64, 2, 32, 64, 1, 1000, 1, 16, True),
+    ("weighted", 64, 2, 32, 16, 2, 500, 6, 16, False),
+])
+def test_fp32_gale_fa_gradients_match_autograd_over_the_oracle(mode, dim, heads, dim_head, S, B, N, Sc, Dc, with_ctx):
+    announce("fp32 GALE_FA gradients", mode, dim, heads, dim_head, S, B, N, Sc, Dc, with_ctx)
+    torch.manual_seed(1)
+    kw = dict(heads=heads, dim_head=dim_head, n_global_queries=S, context_dim=Dc, state_mixing_mode=mode)
+    ref, hip = to.OracleGALE_FA(dim, **kw).train(), pn.GALE_FA(dim, **kw).train()
+    if mode == "weighted":
+        with torch.no_grad():
+            ref.state_mixing.fill_(-0.4)
+    hip.load_state_dict(ref.state_dict())
+    hip.cuda()
+    x, ctx, dy = torch.randn(B, N, dim), torch.randn(B, heads, Sc, Dc), torch.randn(B, N, dim)
+    xr, cr = x.clone().requires_grad_(), ctx.clone().requires_grad_()
+    xh, ch = x.clone().cuda().requires_grad_(), ctx.clone().cuda().requires_grad_()
+    yr = ref((xr,), cr if with_ctx else None)[0]
+    yh = hip((xh,), ch if with_ctx else None)[0]
+    assert_fp32_close(yh, yr, "GALE_FA y (training path)")
+    yr.backward(dy)
+    yh.backward(dy.cuda())
+    assert_fp32_close(xh.grad, xr.grad, "d x", rtol=5e-4)
+    if with_ctx:
+        assert_fp32_close(ch.grad, cr.grad, "d context", rtol=5e-4)
+    grads = dict(hip.named_parameters())
+    for name, p in ref.named_parameters():
+        if p.grad is None:
+            assert grads[name].grad is None, name  # the cross-attention parameters without a context
+            continue
+        if name == "cross_k.bias":
+            continue  # zero in exact arithmetic: a shift of all keys leaves the softmax unchanged
+        if Sc == 1 and name.startswith(("cross_q", "cross_k")):
+            assert float(grads[name].grad.abs().max()) < 1e-4  # one context token: its softmax weight is 1 whatever q, k
+            continue
+        assert_fp32_close(grads[name].grad, p.grad, f"grad {name}", rtol=5e-4)
+
+
+def test_bf16_gale_fa_gradients_and_geotransolver_training_with_gale_fa():
+    announce("bf16 GALE_FA gradients")
+    torch.manual_seed(2)
+    kw = dict(heads=8, dim_head=32, n_global_queries=32, context_dim=32)
+    ref, hip = to.OracleGALE_FA(256, **kw).train(), pn.GALE_FA(256, **kw).train()
+    hip.load_state_dict(ref.state_dict())
+    hip.cuda()
+    x, ctx, dy = torch.randn(1, 6000, 256), torch.randn(1, 8, 16, 32), torch.randn(1, 6000, 256)
+    xr = x.clone().requires_grad_()
+    ref((xr,), ctx)[0].backward(dy)
+    xh = x.clone().cuda().requires_grad_()
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        yh = hip((xh,), ctx.cuda())[0]
+    assert yh.dtype == torch.bfloat16
+    yh.backward(dy.cuda().bfloat16())
+    assert_rel_l2(xh.grad, xr.grad, "bf16 d x", tol=5e-2)
+    grads = dict(hip.named_parameters())
+    for name, p in ref.named_parameters():
+        if name == "cross_k.bias":
+            continue
+        assert_rel_l2(grads[name].grad, p.grad, f"bf16 grad {name}", tol=6e-2)
+
+    announce("GeoTransolver with GALE_FA blocks: training step")
+    model = pn.GeoTransolver(functional_dim=6, out_dim=3, geometry_dim=3, global_dim=5, n_layers=2, n_hidden=32, n_head=4,
+                             mlp_ratio=2, slice_num=8, attention_type="GALE_FA", use_te=False).cuda().train()
+    e, geom, glob = torch.randn(2, 150, 6).cuda(), torch.randn(2, 90, 3).cuda(), torch.randn(2, 4, 5).cuda()
+    opt = torch.optim.SGD(model.parameters(), lr=1e-2)
+    losses = []
+    for _ in range(3):
+        opt.zero_grad()
+        loss = (model(e, None, glob, geom) ** 2).mean()
+        loss.backward()
+        opt.step()
+        losses.append(float(loss.detach()))
+    assert all(p.grad is not None and torch.isfinite(p.grad).all() for p in model.parameters())
+    assert losses[-1] < losses[0]
 
 
 # ---------------------------------------------------------------------------------------------------
