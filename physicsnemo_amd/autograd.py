@@ -198,6 +198,45 @@ class PhysicsAttentionMfmaFunction(torch.autograd.Function):
         return _finish_backward(ctx, x, dy, out_x, d_wqkv, d_proj, d_z, d_temp, x_mid, temperature)
 
 
+def _plus_backward_tail(ctx, x, uniform, x_mid, w, tok_out, out_x, dy, g, d_num, d_norm, d_wqkv, first_param):
+    """Everything of the Transolver++ backward after the slice-token stage: the per-point kernel, d x and the parameter
+    gradients (d_wqkv is passed through; None when the caller's token-stage graph provides it).  Returns (d x, the
+    twelve parameter gradients in the order of `ctx.param_like`)."""
+    dims, kp = ctx.dims, ctx.kparams
+    B, N, C, H, D, S = dims.B, dims.N, dims.C, dims.H, dims.D, dims.S
+    HD = H * D
+    linear = PF.LayerDims(B, N, C, H, D, S)
+    d_xm, d_z, d_a1, d_a2, d_temp = PF.slice_softmax_plus_backward(x_mid, uniform, w, g, tok_out, d_num, d_norm, kp, dims)
+    d_wo, d_bo = _wgrad(dy, out_x)
+    xm_rows = x_mid.reshape(-1, D)
+    d_ws, d_bs = _wgrad(d_z.reshape(-1, S), xm_rows)
+    # proj_temperature = Linear(D, S) -> GELU -> Linear(S, 1) -> GELU: the kernel returns the gradients of the two
+    # Linear outputs; the second weight gradient needs the hidden activation again
+    d_w1, d_b1 = _wgrad(d_a1.reshape(-1, S), xm_rows)
+    hidden = torch.nn.functional.gelu(torch.addmm(kp["proj_temperature_0_bias"], xm_rows.float(),
+                                                  kp["proj_temperature_0_weight"].view(S, D).t()))
+    d_w2 = d_a2.reshape(1, -1) @ hidden
+    d_b2 = d_a2.sum().reshape(1)
+
+    k = dims.conv_k
+    wx = kp["in_project_x_weight"]
+    if k == 0:
+        dx = PF.rows_gemm(d_xm, wx.view(HD, C).t().contiguous(), None, linear, HD, C) if ctx.needs_input_grad[0] else None
+        d_wx, d_bx = _wgrad(d_xm, x)
+    else:
+        grid = (dims.grid_h, dims.grid_w) + ((dims.grid_d,) if dims.grid_d > 0 else ())
+        w_t = _torch_conv_layout(wx, HD, C, (k,) * len(grid), dims).flip(dims=tuple(range(2, 2 + len(grid)))).transpose(0, 1)
+        w_t = (w_t.movedim(1, -1) if dims.conv_tap_major else w_t).contiguous()
+        dx = PF.rows_gemm(d_xm, w_t, None, dims, HD, C) if ctx.needs_input_grad[0] else None
+        d_wx = _conv_weight_grad(d_xm, x, grid, k)
+        d_bx = _rows(d_xm).sum(0, dtype=torch.float32)
+
+    grads = (d_wx, d_bx, d_ws, d_bs, d_temp, d_w1, d_b1, d_w2, d_b2, d_wqkv, d_wo, d_bo)
+    grads = tuple(gr.reshape(p.shape).to(p.dtype) if gr is not None and ctx.needs_input_grad[first_param + i] else None
+                  for i, (gr, p) in enumerate(zip(grads, ctx.param_like)))
+    return dx, grads
+
+
 class PhysicsAttentionPlusFunction(torch.autograd.Function):
     """Transolver++ (plus=True) layer, differentiable w.r.t. x and its twelve parameters; general kernels.  ``uniform``
     (B, N, H, S) holds the samples behind the Gumbel noise and gets no gradient (the reference draws them with
@@ -219,43 +258,60 @@ class PhysicsAttentionPlusFunction(torch.autograd.Function):
     def backward(ctx, dy):
         x, uniform, x_mid, w, tok, norm, tok_out, out_x = ctx.saved_tensors
         dims, kp = ctx.dims, ctx.kparams
-        B, N, C, H, D, S = dims.B, dims.N, dims.C, dims.H, dims.D, dims.S
-        HD = H * D
+        C, HD, D = dims.C, dims.H * dims.D, dims.D
         dy = dy.to(x.dtype).contiguous()
-        linear = PF.LayerDims(B, N, C, H, D, S)
+        linear = PF.LayerDims(dims.B, dims.N, C, dims.H, D, dims.S)
         g = PF.rows_gemm(dy, kp["out_linear_weight"].view(C, HD).t().contiguous(), None, linear, C, HD)
         d_tok_out = PF.slice_weighted_sum(w, g, dims)[..., :D].contiguous()
         d_num, d_norm, d_wqkv = PF.slice_attention_backward(tok, norm, d_tok_out, kp, dims)
-        d_xm, d_z, d_a1, d_a2, d_temp = PF.slice_softmax_plus_backward(x_mid, uniform, w, g, tok_out, d_num, d_norm,
-                                                                       kp, dims)
-        d_wo, d_bo = _wgrad(dy, out_x)
-        xm_rows = x_mid.reshape(-1, D)
-        d_ws, d_bs = _wgrad(d_z.reshape(-1, S), xm_rows)
-        # proj_temperature = Linear(D, S) -> GELU -> Linear(S, 1) -> GELU: the kernel returns the gradients of the two
-        # Linear outputs; the second weight gradient needs the hidden activation again
-        d_w1, d_b1 = _wgrad(d_a1.reshape(-1, S), xm_rows)
-        hidden = torch.nn.functional.gelu(torch.addmm(kp["proj_temperature_0_bias"], xm_rows.float(),
-                                                      kp["proj_temperature_0_weight"].view(S, D).t()))
-        d_w2 = d_a2.reshape(1, -1) @ hidden
-        d_b2 = d_a2.sum().reshape(1)
-
-        k = dims.conv_k
-        wx = kp["in_project_x_weight"]
-        if k == 0:
-            dx = PF.rows_gemm(d_xm, wx.view(HD, C).t().contiguous(), None, linear, HD, C) if ctx.needs_input_grad[0] else None
-            d_wx, d_bx = _wgrad(d_xm, x)
-        else:
-            grid = (dims.grid_h, dims.grid_w) + ((dims.grid_d,) if dims.grid_d > 0 else ())
-            w_t = _torch_conv_layout(wx, HD, C, (k,) * len(grid), dims).flip(dims=tuple(range(2, 2 + len(grid)))).transpose(0, 1)
-            w_t = (w_t.movedim(1, -1) if dims.conv_tap_major else w_t).contiguous()
-            dx = PF.rows_gemm(d_xm, w_t, None, dims, HD, C) if ctx.needs_input_grad[0] else None
-            d_wx = _conv_weight_grad(d_xm, x, grid, k)
-            d_bx = _rows(d_xm).sum(0, dtype=torch.float32)
-
-        grads = (d_wx, d_bx, d_ws, d_bs, d_temp, d_w1, d_b1, d_w2, d_b2, d_wqkv, d_wo, d_bo)
-        grads = tuple(gr.reshape(p.shape).to(p.dtype) if ctx.needs_input_grad[4 + i] else None
-                      for i, (gr, p) in enumerate(zip(grads, ctx.param_like)))
+        dx, grads = _plus_backward_tail(ctx, x, uniform, x_mid, w, tok_out, out_x, dy, g, d_num, d_norm, d_wqkv, 4)
         return (dx, None, None, None) + grads
+
+
+class GALEPlusFunction(torch.autograd.Function):
+    """Transolver++ form of the GALE layer with a context (gale.py:148-239 with plus=True): the per-point stages of
+    `PhysicsAttentionPlusFunction`, the slice-token stage (self-attention, cross-attention, blend) as a PyTorch graph
+    like in `GALEFunction`.  Differentiable w.r.t. x, the context, the twelve layer parameters and the stage's."""
+
+    @staticmethod
+    def forward(ctx, x, uniform, context, dims, kparams, token_stage, n_stage, *params):
+        layer_params, stage_params = params[:len(params) - n_stage], params[len(params) - n_stage:]
+        x_mid, _ = PF.project_inputs(x, kparams, dims)
+        w = PF.slice_softmax_plus(x_mid, uniform, kparams, dims)
+        tok, norm = PF.slice_reduce(w, x_mid, dims)
+        with torch.enable_grad():
+            tok_leaf = tok.detach().requires_grad_(True)
+            ctx_leaf = context.detach().requires_grad_(ctx.needs_input_grad[2])
+            out_graph = token_stage(tok_leaf, ctx_leaf)
+        tok_out = out_graph.detach().float().contiguous()
+        y, out_x = PF.deslice_project(w, tok_out, kparams, dims, return_out_x=True)
+        ctx.save_for_backward(x, uniform, x_mid, w, tok, norm, tok_out, out_x)
+        ctx.dims, ctx.kparams = dims, kparams
+        ctx.param_like = layer_params
+        ctx.graph = (out_graph, tok_leaf, ctx_leaf, stage_params)
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, uniform, x_mid, w, tok, norm, tok_out, out_x = ctx.saved_tensors
+        dims, kp = ctx.dims, ctx.kparams
+        C, HD, D = dims.C, dims.H * dims.D, dims.D
+        dy = dy.to(x.dtype).contiguous()
+        linear = PF.LayerDims(dims.B, dims.N, C, dims.H, D, dims.S)
+        g = PF.rows_gemm(dy, kp["out_linear_weight"].view(C, HD).t().contiguous(), None, linear, C, HD)
+        d_tok_out = PF.slice_weighted_sum(w, g, dims)[..., :D].contiguous()
+        out_graph, tok_leaf, ctx_leaf, stage_params = ctx.graph
+        wanted = [tok_leaf] + ([ctx_leaf] if ctx_leaf.requires_grad else []) + \
+                 [p for p in stage_params if p.requires_grad]
+        got = list(torch.autograd.grad(out_graph, wanted, d_tok_out.to(out_graph.dtype), allow_unused=True))
+        d_tok = got.pop(0).float()
+        d_context = got.pop(0) if ctx_leaf.requires_grad else None
+        d_stage = [got.pop(0) if p.requires_grad else None for p in stage_params]
+        d_num = (d_tok / norm[..., None]).contiguous()
+        d_norm = (-(d_tok * tok).sum(-1) / norm).contiguous()
+        # qkv_project.weight takes part in the token stage only: its gradient comes with `d_stage`
+        dx, grads = _plus_backward_tail(ctx, x, uniform, x_mid, w, tok_out, out_x, dy, g, d_num, d_norm, None, 7)
+        return (dx, None, d_context, None, None, None, None) + grads + tuple(d_stage)
 
 
 class GALEFunction(torch.autograd.Function):

@@ -20,7 +20,7 @@ import torch.nn as nn
 
 from . import functional as PF
 from . import autograd as PA
-from .autograd import GALEFunction
+from .autograd import GALEFunction, GALEPlusFunction
 from .transolver import Mlp, TransolverBlock
 from .physics_attention import (
     PhysicsAttentionIrregularMesh,
@@ -91,13 +91,23 @@ class _GALEForwardMixin:
             return self.concat_project(torch.cat([self_out, cross], dim=-1))
 
     def _forward_one_with_grad(self, x: torch.Tensor, context: torch.Tensor) -> torch.Tensor:
-        if self.plus or self.fp8_weights:
-            raise NotImplementedError("GALE training with a context is served for plus=False without fp8 weights")
+        if self.fp8_weights:
+            raise NotImplementedError("GALE training with a context is not served with fp8 weights")
         if x.is_cuda and self._wants_fp16(x):
             with torch.autocast("cuda", enabled=False):
                 return self._forward_one_with_grad(x.float(), context).to(torch.float16)
         x = self._prepare_input(x)
         dims = self.layer_dims(x)
+        if self.plus:
+            if not PF.plus_backward_supported(x.dtype, dims):
+                raise RuntimeError(f"the backward kernels do not serve this shape: {dims}")
+            stage, pt = self._stage_params(), self.proj_temperature
+            u = torch.rand((dims.B, dims.N, dims.H, dims.S), dtype=x.dtype, device=x.device)
+            return GALEPlusFunction.apply(
+                x, u, context, dims, self.kernel_params(x.dtype, x.device), self._token_stage, len(stage),
+                self.in_project_x.weight, self.in_project_x.bias, self.in_project_slice.weight,
+                self.in_project_slice.bias, self.temperature, pt[0].weight, pt[0].bias, pt[2].weight, pt[2].bias,
+                self.qkv_project.weight, self.out_linear.weight, self.out_linear.bias, *stage)
         if not PF.backward_supported(x.dtype, dims):
             raise RuntimeError(f"the backward kernels do not serve this shape: {dims}")
         stage = self._stage_params()

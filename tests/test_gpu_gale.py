@@ -108,8 +108,35 @@ def test_gale_plus_and_errors():
         hip((x,), ctx[:, :2])
     with pytest.raises(TypeError):
         hip(x, ctx)
-    with pytest.raises(NotImplementedError):  # training with a context: plus=False only
-        hip((x.requires_grad_(True),), ctx)
+
+
+@pytest.mark.parametrize("mode", ["weighted", "concat_project"])
+def test_gale_plus_gradients_with_context_match_autograd_over_the_oracle(mode):
+    """plus=True with a context, training: the layer draws its Gumbel samples on the device; the same seed and shape
+    give the test the same samples for the oracle."""
+    announce("GALE plus gradients with context", mode)
+    ref, hip = _pair("irregular", mode, 32, 4, 8, 8, 7, plus=True, seed=3)
+    ref.train(), hip.train()
+    B, N = 2, 300
+    x, ctx, probe = torch.randn(B, N, 32), torch.randn(B, 4, 5, 7), torch.randn(B, N, 32)
+    torch.manual_seed(11)
+    u = torch.rand((B, N, 4, 8), dtype=torch.float32, device="cuda")
+    xr, cr = x.clone().requires_grad_(), ctx.clone().requires_grad_()
+    yr = ref.stages(xr, noise_u=u.cpu(), context=cr)["y"]
+    (yr * probe).sum().backward()
+    xh, ch = x.clone().cuda().requires_grad_(), ctx.clone().cuda().requires_grad_()
+    torch.manual_seed(11)
+    yh = hip((xh,), ch)[0]
+    assert_fp32_close(yh, yr, "GALE plus y (training path)")
+    (yh * probe.cuda()).sum().backward()
+    assert_fp32_close(xh.grad, xr.grad, "d x", rtol=5e-4)
+    assert_fp32_close(ch.grad, cr.grad, "d context", rtol=5e-4)
+    grads = dict(hip.named_parameters())
+    for name, p in ref.named_parameters():
+        if name == "cross_k.bias" or p.grad is None:
+            continue  # zero in exact arithmetic / in_project_fx, which plus=True does not use
+        assert grads[name].grad is not None, name
+        assert_fp32_close(grads[name].grad, p.grad, f"grad {name}", rtol=5e-4)
 
 
 def _gale_grads(module, x, ctx, probe):
