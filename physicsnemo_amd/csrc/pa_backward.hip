@@ -252,27 +252,55 @@ __global__ __launch_bounds__(256) void slice_softmax_backward_kernel(
   }
   __syncthreads();
 
-  // d w and the logits
-  for (int i = t; i < R * S; i += 256) {
-    const int r = i / S, s = i - r * S;
-    const float *xr = xm + r * D1, *fr = fm + r * D1, *gr = go + r * D1;
-    const float *tr = to + s * D1, *nr = dn + s * D1, *wr = ws + s * D1;
-    float z = 0.f, dw = 0.f;
-    for (int d = 0; d < D; ++d) {
-      z = fmaf(xr[d], wr[d], z);
-      dw = fmaf(gr[d], tr[d], dw);
-      dw = fmaf(fr[d], nr[d], dw);
-    }
-    dwl[r * S1 + s] = dw + dnr[s];
-    if constexpr (PLUS) {
-      const float *vr = w1 + s * D1;
-      float a = b1[s];
-      for (int d = 0; d < D; ++d) a = fmaf(xr[d], vr[d], a);
-      a1l[r * S1 + s] = a;
-      const float u = r < rows ? load_as_f32(static_cast<const T *>(plus.uniform) + (m0 + r) * HS + h * S + s) : 0.5f;
-      lgl[r * S1 + s] = round_to(x_mid, z + bs[s]) - logf(-logf(u + 1e-8f) + 1e-8f);  // divided by temp below
-    } else {
-      lgl[r * S1 + s] = round_to(x_mid, z + bs[s]) * inv_temp_h;  // the forward divides the stored Linear output
+  // d w and the logits: a thread owns 2 rows x 4 slices (slices sq, sq + SQ, ...: neighbouring lanes read
+  // neighbouring table rows, whose odd stride spreads them over the banks; the row operands are wave-wide broadcasts),
+  // 18 LDS reads feed 24 multiply-adds
+  {
+    const int SQ = (S + 3) >> 2;
+    for (int tile = t; tile < (R >> 1) * SQ; tile += 256) {
+      const int rp = tile / SQ, sq = tile - rp * SQ, r0 = 2 * rp;
+      int so[4];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) so[k] = min(sq + k * SQ, S - 1) * D1;
+      const float *x0 = xm + r0 * D1, *f0 = fm + r0 * D1, *g0 = go + r0 * D1;
+      float z[2][4], dw[2][4], a[2][4];
+#pragma unroll
+      for (int jj = 0; jj < 2; ++jj)
+#pragma unroll
+        for (int k = 0; k < 4; ++k) z[jj][k] = dw[jj][k] = a[jj][k] = 0.f;
+      for (int d = 0; d < D; ++d) {
+        const float xa = x0[d], xb = x0[D1 + d], fa = f0[d], fb = f0[D1 + d], ga = g0[d], gb = g0[D1 + d];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          const float tv = to[so[k] + d], nv = dn[so[k] + d], wv = ws[so[k] + d];
+          z[0][k] = fmaf(xa, wv, z[0][k]);
+          z[1][k] = fmaf(xb, wv, z[1][k]);
+          dw[0][k] = fmaf(fa, nv, fmaf(ga, tv, dw[0][k]));
+          dw[1][k] = fmaf(fb, nv, fmaf(gb, tv, dw[1][k]));
+          if constexpr (PLUS) {
+            const float v1 = w1[so[k] + d];
+            a[0][k] = fmaf(xa, v1, a[0][k]);
+            a[1][k] = fmaf(xb, v1, a[1][k]);
+          }
+        }
+      }
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const int sl = sq + k * SQ;
+        if (sl >= S) continue;
+#pragma unroll
+        for (int jj = 0; jj < 2; ++jj) {
+          const int r = r0 + jj;
+          dwl[r * S1 + sl] = dw[jj][k] + dnr[sl];
+          if constexpr (PLUS) {
+            a1l[r * S1 + sl] = a[jj][k] + b1[sl];
+            const float u = r < rows ? load_as_f32(static_cast<const T *>(plus.uniform) + (m0 + r) * HS + h * S + sl) : 0.5f;
+            lgl[r * S1 + sl] = round_to(x_mid, z[jj][k] + bs[sl]) - logf(-logf(u + 1e-8f) + 1e-8f);  // divided by temp below
+          } else {
+            lgl[r * S1 + sl] = round_to(x_mid, z[jj][k] + bs[sl]) * inv_temp_h;  // the forward divides the stored Linear output
+          }
+        }
+      }
     }
   }
   __syncthreads();
@@ -332,21 +360,50 @@ __global__ __launch_bounds__(256) void slice_softmax_backward_kernel(
     if constexpr (PLUS)
       store_from_f32(static_cast<T *>(plus.d_a1) + (m0 + r) * HS + h * S + s, a1l[r * S1 + s]);
   }
-  for (int i = t; i < rows * D; i += 256) {
-    const int r = i / D, d = i - r * D;
-    const float *wr = wl + r * S1, *zr = dwl + r * S1;
-    float dx = 0.f, df = 0.f;
-    for (int s = 0; s < S; ++s) {
-      dx = fmaf(zr[s], ws[s * D1 + d], dx);
-      df = fmaf(wr[s], dn[s * D1 + d], df);
+  // d x_mid and d fx_mid: a thread owns 2 rows x 2 features (features dq and dq + DQ), 8 LDS reads per 8 multiply-adds
+  const int DQ = (D + 1) >> 1;
+  for (int tile = t; tile < (R >> 1) * DQ; tile += 256) {
+    const int rp = tile / DQ, dq = tile - rp * DQ, r0 = 2 * rp;
+    const int d0 = dq, d1 = min(dq + DQ, D - 1);
+    const float *wr = wl + r0 * S1, *zr = dwl + r0 * S1;
+    float dx[2][2] = {{0.f, 0.f}, {0.f, 0.f}}, df[2][2] = {{0.f, 0.f}, {0.f, 0.f}};
+    for (int sl = 0; sl < S; ++sl) {
+      const float za = zr[sl], zb = zr[S1 + sl], wa = wr[sl], wb = wr[S1 + sl];
+      const float w0 = ws[sl * D1 + d0], w1v = ws[sl * D1 + d1], n0 = dn[sl * D1 + d0], n1 = dn[sl * D1 + d1];
+      dx[0][0] = fmaf(za, w0, dx[0][0]);
+      dx[0][1] = fmaf(za, w1v, dx[0][1]);
+      dx[1][0] = fmaf(zb, w0, dx[1][0]);
+      dx[1][1] = fmaf(zb, w1v, dx[1][1]);
+      df[0][0] = fmaf(wa, n0, df[0][0]);
+      df[0][1] = fmaf(wa, n1, df[0][1]);
+      df[1][0] = fmaf(wb, n0, df[1][0]);
+      df[1][1] = fmaf(wb, n1, df[1][1]);
     }
     if constexpr (PLUS) {
-      const float *ar = a1l + r * S1;
-      for (int s = 0; s < S; ++s) dx = fmaf(ar[s], w1[s * D1 + d], dx);
-      store_from_f32(d_proj + (m0 + r) * HD + h * D + d, dx + df);
-    } else {
-      store_from_f32(d_proj + (m0 + r) * 2 * HD + h * D + d, dx);
-      store_from_f32(d_proj + (m0 + r) * 2 * HD + HD + h * D + d, df);
+      const float *ar = a1l + r0 * S1;
+      for (int sl = 0; sl < S; ++sl) {
+        const float aa = ar[sl], ab = ar[S1 + sl], v0 = w1[sl * D1 + d0], v1 = w1[sl * D1 + d1];
+        dx[0][0] = fmaf(aa, v0, dx[0][0]);
+        dx[0][1] = fmaf(aa, v1, dx[0][1]);
+        dx[1][0] = fmaf(ab, v0, dx[1][0]);
+        dx[1][1] = fmaf(ab, v1, dx[1][1]);
+      }
+    }
+#pragma unroll
+    for (int jj = 0; jj < 2; ++jj) {
+      const int r = r0 + jj;
+      if (r >= rows) continue;
+#pragma unroll
+      for (int k = 0; k < 2; ++k) {
+        const int d = dq + k * DQ;
+        if (d >= D) continue;
+        if constexpr (PLUS) {
+          store_from_f32(d_proj + (m0 + r) * HD + h * D + d, dx[jj][k] + df[jj][k]);
+        } else {
+          store_from_f32(d_proj + (m0 + r) * 2 * HD + h * D + d, dx[jj][k]);
+          store_from_f32(d_proj + (m0 + r) * 2 * HD + HD + h * D + d, df[jj][k]);
+        }
+      }
     }
   }
 }
