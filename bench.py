@@ -33,6 +33,9 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--settle-ms", type=float, default=150.0,
+                    help="untimed run-in of the same call before the warm-up steps: after an idle spell the engine clock "
+                         "overshoots, is throttled and takes some 20 ms of load to converge")
     ap.add_argument("--points", type=int, default=1 << 20)
     ap.add_argument("--batch", type=int, default=1)
     ap.add_argument("--hidden", type=int, default=256)
@@ -65,10 +68,25 @@ def mfma_flops_per_point(C, S):
     }
 
 
+SETTLE_MS = 150.0  # set from --settle-ms
+
+
+def run_in(fn):
+    """Untimed run-in before a timed region: keeps the GPU under the very load that is about to be timed until the
+    clock governor has converged (after an idle spell the engine clock overshoots, is throttled, and takes some 20 ms
+    of load to settle: the first twenty calls of the layer run up to 35 % longer than the rest)."""
+    import torch
+
+    t_end = time.perf_counter() + SETTLE_MS * 1e-3
+    while time.perf_counter() < t_end:
+        fn()
+        torch.cuda.synchronize()
+
+
 def time_kernel(fn, reps):
     import torch
 
-    fn()
+    run_in(fn)
     torch.cuda.synchronize()
     start = torch.cuda.Event(enable_timing=True)
     stop = torch.cuda.Event(enable_timing=True)
@@ -138,7 +156,7 @@ def time_block_mlp(rows, C, hidden, reps=10):
             "hbm_frac": round(4 * rows * C * 2 / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
 
 
-def time_training_step(points, C, S, reps=3):
+def time_training_step(points, C, S, reps=10):
     """Forward + backward of one layer under bf16 autocast at the layer workload's size (gradients w.r.t. the input
     and all ten parameters)."""
     import torch
@@ -157,6 +175,7 @@ def time_training_step(points, C, S, reps=3):
             y = layer(x)
         y.backward(dy)
 
+    run_in(step)
     for _ in range(2):
         step()
     torch.cuda.synchronize()
@@ -185,6 +204,7 @@ def time_variants(points, C, S, reps=5):
     out = []
 
     def timed(fn, n=reps):
+        run_in(fn)
         for _ in range(2):
             fn()
         torch.cuda.synchronize()
@@ -290,6 +310,7 @@ def time_full_model(name, B, N, functional_dim, embedding_dim, slice_num, n_laye
             return model(a, b)
 
     def timed(fn):
+        run_in(lambda: fn(fx, emb))
         for _ in range(warmup):
             o = fn(fx, emb)
         torch.cuda.synchronize()
@@ -331,6 +352,7 @@ def time_structured_model(steps=5, warmup=2):
     pos = torch.stack(torch.meshgrid(lin, lin, indexing="ij"), -1).reshape(1, 7225, 2).repeat(4, 1, 1).cuda()
     fx = torch.randn(4, 7225, 1, generator=g).cuda()
     def timed(fn):
+        run_in(fn)
         for _ in range(warmup):
             o = fn()
         torch.cuda.synchronize()
@@ -381,7 +403,10 @@ def main():
     dims = layer.layer_dims(x)
     path = PF.query_path(torch.bfloat16, dims)
 
+    global SETTLE_MS
+    SETTLE_MS = args.settle_ms
     with torch.no_grad():
+        run_in(lambda: layer(x))
         for _ in range(args.warmup):
             y = layer(x)
         torch.cuda.synchronize()
@@ -396,6 +421,7 @@ def main():
 
     # the same call recorded once into a HIP graph and replayed (same kernels, one submission per step)
     graphed = pn.GraphedForward(layer, x)  # its static input holds a copy of x
+    run_in(graphed.replay)
     for _ in range(args.warmup):
         graphed.replay()
     torch.cuda.synchronize()
@@ -464,7 +490,7 @@ def main():
     out = {
         "metric": "Mpoints/s per PhysicsAttention layer at 1M pts bf16; % HBM/MFMA roofline",
         "value": round(mpoints, 2), "unit": "Mpoints/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "settle_ms": args.settle_ms, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "cfg3: single PhysicsAttentionIrregularMesh layer forward", "batch": B, "points": N,
                    "hidden": C, "heads": H, "dim_head": 32, "slice_num": S,
