@@ -79,6 +79,53 @@ __global__ __launch_bounds__(256) void softmax_rows_kernel(T *__restrict__ a, in
   }
 }
 
+// The same with 16-byte accesses, for rows that are a whole number of 16-byte units (S a multiple of 8 in bf16, of 4
+// in float32): LR lanes share a row (a power of two >= S / unit), a lane keeps its unit in registers between the load
+// and the store, so every element is read once, exponentiated once and written once.
+template <typename T, int LR>
+__global__ __launch_bounds__(256) void softmax_rows_vec_kernel(T *__restrict__ a, int64_t rows, int S,
+                                                               const float *__restrict__ temperature, int H) {
+  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+  constexpr int UE = 16 / sizeof(T);
+  constexpr int per_wg = 256 / LR;
+  const int sub = threadIdx.x / LR, l = threadIdx.x % LR;
+  const bool mine = l * UE < S;
+  for (int64_t row = (int64_t)blockIdx.x * per_wg + sub; row < rows; row += (int64_t)gridDim.x * per_wg) {
+    T *p = a + row * S + l * UE;
+    const float inv_t = temperature ? 1.f / clamp_temperature(temperature[row % H]) : 1.f;
+    float v[UE];
+    float mx = -INFINITY;
+    if (mine) {
+      const u32x4 raw = *reinterpret_cast<const u32x4 *>(p);
+      const T *e = reinterpret_cast<const T *>(&raw);
+#pragma unroll
+      for (int j = 0; j < UE; ++j) {
+        v[j] = load_as_f32(e + j) * inv_t;
+        mx = fmaxf(mx, v[j]);
+      }
+    }
+#pragma unroll
+    for (int off = LR >> 1; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+    float sum = 0.f;
+    if (mine) {
+#pragma unroll
+      for (int j = 0; j < UE; ++j) {
+        v[j] = expf(v[j] - mx);
+        sum += v[j];
+      }
+    }
+#pragma unroll
+    for (int off = LR >> 1; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+    if (mine) {
+      const float inv = 1.f / sum;
+      alignas(16) T o[UE];
+#pragma unroll
+      for (int j = 0; j < UE; ++j) store_from_f32(o + j, v[j] * inv);
+      *reinterpret_cast<u32x4 *>(p) = *reinterpret_cast<const u32x4 *>(o);
+    }
+  }
+}
+
 // ------------------------------------------------------------------------------------------------
 // flare_backward_kernel: per-point part of the FLARE backward pass.  grid (row tiles of R points per batch, H).
 // With wr = softmax_s(A) (hand-back weights), wc = exp(A - max_n A) (gather weights), z the gathered summaries,
@@ -237,8 +284,29 @@ static int softmax_rows_l(const pa_shape &s, void *a, const float *temperature, 
   return launch_status();
 }
 
+template <typename T, int LR>
+static int softmax_rows_vec(const pa_shape &s, void *a, const float *temperature, hipStream_t st) {
+  const int64_t rows = s.B * s.N * s.H;
+  int64_t blocks = (rows + (256 / LR) - 1) / (256 / LR);
+  if (blocks > 16384) blocks = 16384;
+  hipLaunchKernelGGL((softmax_rows_vec_kernel<T, LR>), dim3((unsigned)blocks), dim3(256), 0, st, static_cast<T *>(a),
+                     rows, (int)s.S, temperature, (int)s.H);
+  return launch_status();
+}
+
 template <typename T>
 static int softmax_rows_t(const pa_shape &s, void *a, const float *temperature, hipStream_t st) {
+  constexpr int UE = 16 / sizeof(T);
+  if (s.S % UE == 0 && s.S / UE <= 64 && reinterpret_cast<uintptr_t>(a) % 16 == 0) {
+    const int64_t units = s.S / UE;
+    if (units <= 1) return softmax_rows_vec<T, 1>(s, a, temperature, st);
+    if (units <= 2) return softmax_rows_vec<T, 2>(s, a, temperature, st);
+    if (units <= 4) return softmax_rows_vec<T, 4>(s, a, temperature, st);
+    if (units <= 8) return softmax_rows_vec<T, 8>(s, a, temperature, st);
+    if (units <= 16) return softmax_rows_vec<T, 16>(s, a, temperature, st);
+    if (units <= 32) return softmax_rows_vec<T, 32>(s, a, temperature, st);
+    return softmax_rows_vec<T, 64>(s, a, temperature, st);
+  }
   if (s.S <= 8) return softmax_rows_l<T, 8>(s, a, temperature, st);
   if (s.S <= 16) return softmax_rows_l<T, 16>(s, a, temperature, st);
   if (s.S <= 32) return softmax_rows_l<T, 32>(s, a, temperature, st);

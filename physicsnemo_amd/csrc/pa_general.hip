@@ -239,6 +239,75 @@ __global__ __launch_bounds__(256) void softmax_rows_plus_kernel(T *__restrict__ 
   }
 }
 
+// The same with 16-byte accesses, for rows that are a whole number of 16-byte units: LR lanes share a row (a power of
+// two >= S / unit), a lane keeps its unit of softmax arguments in registers, so every element is read once and its
+// Gumbel noise (two logarithms) is formed once.
+template <typename T, int LR>
+__global__ __launch_bounds__(256) void softmax_rows_plus_vec_kernel(T *__restrict__ w, const T *__restrict__ hidden,
+                                                                    const T *__restrict__ uniform,
+                                                                    const float *__restrict__ temperature,
+                                                                    const float *__restrict__ pt_w2,
+                                                                    const float *__restrict__ pt_b2, int64_t rows, int S,
+                                                                    int H) {
+  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+  constexpr int UE = 16 / sizeof(T);
+  constexpr int per_wg = 256 / LR;
+  const int sub = threadIdx.x / LR, l = threadIdx.x % LR;
+  const bool mine = l * UE < S;
+  float w2[UE];
+#pragma unroll
+  for (int j = 0; j < UE; ++j) w2[j] = mine ? pt_w2[l * UE + j] : 0.f;
+  const float b2 = pt_b2[0];
+  for (int64_t row = (int64_t)blockIdx.x * per_wg + sub; row < rows; row += (int64_t)gridDim.x * per_wg) {
+    const int64_t off0 = row * S + l * UE;
+    float v[UE];
+    float tacc = 0.f;
+    if (mine) {
+      const u32x4 rw = *reinterpret_cast<const u32x4 *>(w + off0);
+      const u32x4 rh = *reinterpret_cast<const u32x4 *>(hidden + off0);
+      const u32x4 ru = *reinterpret_cast<const u32x4 *>(uniform + off0);
+      const T *ew = reinterpret_cast<const T *>(&rw), *eh = reinterpret_cast<const T *>(&rh),
+              *eu = reinterpret_cast<const T *>(&ru);
+#pragma unroll
+      for (int j = 0; j < UE; ++j) {
+        tacc = fmaf(w2[j], load_as_f32(eh + j), tacc);
+        v[j] = load_as_f32(ew + j) - logf(-logf(load_as_f32(eu + j) + 1e-8f) + 1e-8f);
+      }
+    }
+#pragma unroll
+    for (int off = LR >> 1; off > 0; off >>= 1) tacc += __shfl_xor(tacc, off, 64);
+    const float temp = round_to(w, fmaxf(temperature[row % H] + gelu_erf(tacc + b2), 0.01f));
+    const float inv_t = 1.f / temp;
+    float mx = -INFINITY;
+    if (mine) {
+#pragma unroll
+      for (int j = 0; j < UE; ++j) {
+        v[j] *= inv_t;
+        mx = fmaxf(mx, v[j]);
+      }
+    }
+#pragma unroll
+    for (int off = LR >> 1; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+    float sum = 0.f;
+    if (mine) {
+#pragma unroll
+      for (int j = 0; j < UE; ++j) {
+        v[j] = expf(v[j] - mx);
+        sum += v[j];
+      }
+    }
+#pragma unroll
+    for (int off = LR >> 1; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+    if (mine) {
+      const float inv = 1.f / sum;
+      alignas(16) T o[UE];
+#pragma unroll
+      for (int j = 0; j < UE; ++j) store_from_f32(o + j, v[j] * inv);
+      *reinterpret_cast<u32x4 *>(w + off0) = *reinterpret_cast<const u32x4 *>(o);
+    }
+  }
+}
+
 // ------------------------------------------------------------------------------------------------
 // slice_partial_kernel: grid (G chunks, B*H, output slabs).  For its chunk of points of one (b, h):
 //   partial[s, d] = sum_n w[n, s] * fx_mid[n, d]   (d < D),   partial[s, D] = sum_n w[n, s]
@@ -849,6 +918,18 @@ static int softmax_rows_plus_l(const pa_shape &s, const pa_params &p, const pa_p
   return launch_status();
 }
 
+template <typename T, int LR>
+static int softmax_rows_plus_vec(const pa_shape &s, const pa_params &p, const pa_plus_params &pp, void *w,
+                                 const void *hidden, const void *uniform, hipStream_t st) {
+  const int64_t rows = s.B * s.N * s.H;
+  int64_t blocks = (rows + (256 / LR) - 1) / (256 / LR);
+  if (blocks > 16384) blocks = 16384;
+  hipLaunchKernelGGL((softmax_rows_plus_vec_kernel<T, LR>), dim3((unsigned)blocks), dim3(256), 0, st,
+                     static_cast<T *>(w), static_cast<const T *>(hidden), static_cast<const T *>(uniform), p.temperature,
+                     pp.proj_temperature_2_weight, pp.proj_temperature_2_bias, rows, (int)s.S, (int)s.H);
+  return launch_status();
+}
+
 // With a scratch buffer of B*N*H*S elements the two Linears run on the row GEMM kernels (several times faster than the
 // single kernel below, which forms them per point on the vector ALUs).
 template <typename T>
@@ -869,6 +950,18 @@ static int slice_softmax_plus_staged(const pa_shape &s, const pa_params &p, cons
   a.out[0] = scratch;
   a.act = 1;
   if ((rc = launch_gemm<T, float>(a, 1, st))) return rc;
+  constexpr int UE = 16 / sizeof(T);
+  if (s.S % UE == 0 && s.S / UE <= 64 && (reinterpret_cast<uintptr_t>(w) | reinterpret_cast<uintptr_t>(scratch) |
+                                          reinterpret_cast<uintptr_t>(uniform)) % 16 == 0) {
+    const int64_t units = s.S / UE;
+    if (units <= 1) return softmax_rows_plus_vec<T, 1>(s, p, pp, w, scratch, uniform, st);
+    if (units <= 2) return softmax_rows_plus_vec<T, 2>(s, p, pp, w, scratch, uniform, st);
+    if (units <= 4) return softmax_rows_plus_vec<T, 4>(s, p, pp, w, scratch, uniform, st);
+    if (units <= 8) return softmax_rows_plus_vec<T, 8>(s, p, pp, w, scratch, uniform, st);
+    if (units <= 16) return softmax_rows_plus_vec<T, 16>(s, p, pp, w, scratch, uniform, st);
+    if (units <= 32) return softmax_rows_plus_vec<T, 32>(s, p, pp, w, scratch, uniform, st);
+    return softmax_rows_plus_vec<T, 64>(s, p, pp, w, scratch, uniform, st);
+  }
   if (s.S <= 8) return softmax_rows_plus_l<T, 8>(s, p, pp, w, scratch, uniform, st);
   if (s.S <= 16) return softmax_rows_plus_l<T, 16>(s, p, pp, w, scratch, uniform, st);
   if (s.S <= 32) return softmax_rows_plus_l<T, 32>(s, p, pp, w, scratch, uniform, st);
