@@ -536,17 +536,87 @@ __global__ __launch_bounds__(256) void deslice_kernel(const T *__restrict__ w, c
   const int rows = (int)min((int64_t)R, N - n0);
   const int64_t m0 = (int64_t)b * N + n0;
   for (int i = t; i < S * D; i += 256) tk[i] = out_token[((int64_t)b * H + h) * S * D + i];
-  for (int i = t; i < rows * S; i += 256) {
-    const int r = i / S, s = i - r * S;
-    wl[r * (S + 1) + s] = load_as_f32(w + (m0 + r) * H * S + h * S + s);
+  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+  typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+  constexpr int UE = 16 / sizeof(T);
+  if (S % UE == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0) {  // 16-byte loads of the slice weights
+    const int units = S / UE;
+    for (int i = t; i < R * units; i += 256) {  // rows past the end of the batch: zeros
+      const int r = i / units, u = i - r * units;
+      u32x4 raw = {0u, 0u, 0u, 0u};
+      if (r < rows) raw = *reinterpret_cast<const u32x4 *>(w + (m0 + r) * H * S + h * S + u * UE);
+      const T *e = reinterpret_cast<const T *>(&raw);
+#pragma unroll
+      for (int j = 0; j < UE; ++j) wl[r * (S + 1) + u * UE + j] = load_as_f32(e + j);
+    }
+  } else {
+    for (int i = t; i < R * S; i += 256) {
+      const int r = i / S, s = i - r * S;
+      wl[r * (S + 1) + s] = r < rows ? load_as_f32(w + (m0 + r) * H * S + h * S + s) : 0.f;
+    }
   }
   __syncthreads();
-  for (int i = t; i < rows * D; i += 256) {
-    const int r = i / D, d = i - r * D;
-    const float *wr = wl + r * (S + 1);
-    float acc = 0.f;
-    for (int s = 0; s < S; ++s) acc = fmaf(wr[s], tk[s * D + d], acc);
-    store_from_f32(out_x + (m0 + r) * H * D + h * D + d, acc);
+  if (D % 4 == 0 && reinterpret_cast<uintptr_t>(out_x) % 16 == 0) {
+    // a thread owns 4 rows x 4 adjacent features: one 16-byte and four 4-byte LDS reads per 16 multiply-adds, and the
+    // results leave as 8- or 16-byte stores
+    const int DQ4 = D >> 2, S1 = S + 1;
+    for (int tile = t; tile < (R >> 2) * DQ4; tile += 256) {
+      const int rq = tile / DQ4, dq = tile - rq * DQ4, r0 = 4 * rq;
+      if (r0 >= rows) continue;
+      const float *w0 = wl + r0 * S1;
+      float acc[4][4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int k = 0; k < 4; ++k) acc[j][k] = 0.f;
+      for (int sl = 0; sl < S; ++sl) {
+        const float4 tv = *reinterpret_cast<const float4 *>(tk + sl * D + 4 * dq);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float wv = w0[j * S1 + sl];
+          acc[j][0] = fmaf(wv, tv.x, acc[j][0]);
+          acc[j][1] = fmaf(wv, tv.y, acc[j][1]);
+          acc[j][2] = fmaf(wv, tv.z, acc[j][2]);
+          acc[j][3] = fmaf(wv, tv.w, acc[j][3]);
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        if (r0 + j >= rows) continue;
+        alignas(16) T o4[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) store_from_f32(o4 + k, acc[j][k]);
+        T *dst = out_x + (m0 + r0 + j) * H * D + h * D + 4 * dq;
+        if constexpr (sizeof(T) == 2) *reinterpret_cast<u32x2 *>(dst) = *reinterpret_cast<const u32x2 *>(o4);
+        else *reinterpret_cast<u32x4 *>(dst) = *reinterpret_cast<const u32x4 *>(o4);
+      }
+    }
+    return;
+  }
+  // a thread owns 4 rows x 2 features (features dq and dq + DQ): 6 LDS reads per 8 multiply-adds
+  const int DQ = (D + 1) >> 1, S1 = S + 1;
+  for (int tile = t; tile < (R >> 2) * DQ; tile += 256) {
+    const int rq = tile / DQ, dq = tile - rq * DQ, r0 = 4 * rq;
+    if (r0 >= rows) continue;
+    const int d1 = min(dq + DQ, D - 1);
+    const float *w0 = wl + r0 * S1;
+    float acc[4][2] = {{0.f, 0.f}, {0.f, 0.f}, {0.f, 0.f}, {0.f, 0.f}};
+    for (int sl = 0; sl < S; ++sl) {
+      const float t0 = tk[sl * D + dq], t1 = tk[sl * D + d1];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float wv = w0[j * S1 + sl];
+        acc[j][0] = fmaf(wv, t0, acc[j][0]);
+        acc[j][1] = fmaf(wv, t1, acc[j][1]);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      if (r0 + j >= rows) continue;
+      T *o = out_x + (m0 + r0 + j) * H * D + h * D;
+      store_from_f32(o + dq, acc[j][0]);
+      if (dq + DQ < D) store_from_f32(o + dq + DQ, acc[j][1]);
+    }
   }
 }
 
@@ -1069,7 +1139,8 @@ int slice_partial(int dtype, const pa_shape &s, const void *w, const void *fx_mi
 
 template <typename T>
 static int deslice_t(const pa_shape &s, const void *w, const float *out_token, void *out_x, hipStream_t st) {
-  int R = 32;
+  int R = 128;  // rows per workgroup: the head's token table (S x D floats) is loaded once per tile
+  while (R > 8 && (size_t)(s.S * s.D + R * (s.S + 1)) * 4 > 48 * 1024) R >>= 1;
   size_t lds = (size_t)(s.S * s.D + R * (s.S + 1)) * 4;
   int rc = allow_dynamic_lds(deslice_kernel<T>, lds);
   if (rc) return rc;
