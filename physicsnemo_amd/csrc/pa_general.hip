@@ -312,12 +312,12 @@ __global__ __launch_bounds__(256) void softmax_rows_plus_vec_kernel(T *__restric
 // slice_partial_kernel: grid (G chunks, B*H, output slabs).  For its chunk of points of one (b, h):
 //   partial[s, d] = sum_n w[n, s] * fx_mid[n, d]   (d < D),   partial[s, D] = sum_n w[n, s]
 // The (S x D+1) output is cut into 4 x 4 register tiles; a thread owns NS of them (tile t + 256 i of its slab of
-// 256 NS tiles) and walks the chunk 32 points at a time through LDS: per point and tile two 16-byte LDS reads
+// 256 NS tiles) and walks the chunk 64 points at a time through LDS: per point and tile two 16-byte LDS reads
 // (4 slice weights, 4 features) feed 16 FMAs.  LDS rows are padded to multiples of four (zeros; column D of the
 // feature rows holds 1 for the count).  Sums run in a fixed order, so the result is bit-reproducible.
 // ------------------------------------------------------------------------------------------------
 constexpr int kAttnThreads = 1024;  // slice_combine_attn_kernel: 16 waves, one query row per wave at a time
-constexpr int kPartialTile = 32;
+constexpr int kPartialTile = 64;
 constexpr int kPartialMaxNS = 4;
 
 template <typename T, int NS>
@@ -326,8 +326,8 @@ __global__ __launch_bounds__(256) void slice_partial_kernel(const T *__restrict_
                                                             int S, int64_t chunk) {
   extern __shared__ float4 lds4[];
   const int D1 = D + 1, SB = (S + 3) / 4, DB = (D1 + 3) / 4;  // tiles along the slices / the features
-  float4 *wl = lds4;                      // 32 * SB
-  float4 *fl = wl + kPartialTile * SB;    // 32 * DB
+  float4 *wl = lds4;                      // kPartialTile * SB
+  float4 *fl = wl + kPartialTile * SB;    // kPartialTile * DB
   float *wlf = reinterpret_cast<float *>(wl), *flf = reinterpret_cast<float *>(fl);
   const int t = threadIdx.x;
   const int g = blockIdx.x;
@@ -350,18 +350,50 @@ __global__ __launch_bounds__(256) void slice_partial_kernel(const T *__restrict_
   const int64_t n_begin = (int64_t)g * chunk;
   const int64_t n_end = min(N, n_begin + chunk);
   const int HS = H * S, HD = H * D;
+  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+  constexpr int UE = 16 / sizeof(T);
+  const bool vec_w = S % UE == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0;
+  const bool vec_f = D % UE == 0 && reinterpret_cast<uintptr_t>(fx_mid) % 16 == 0;
   for (int64_t n0 = n_begin; n0 < n_end; n0 += kPartialTile) {
     const int pts = (int)min((int64_t)kPartialTile, n_end - n0);
-    for (int i = t; i < kPartialTile * SB * 4; i += 256) {
-      const int p = i / (SB * 4), s = i - p * (SB * 4);
-      wlf[i] = (p < pts && s < S) ? load_as_f32(w + ((int64_t)b * N + n0 + p) * HS + h * S + s) : 0.f;
+    if (vec_w) {  // 16-byte loads: the rows are whole numbers of 16-byte units
+      const int units = S / UE;
+      for (int i = t; i < kPartialTile * units; i += 256) {
+        const int p = i / units, u = i - p * units;
+        u32x4 raw = {0u, 0u, 0u, 0u};
+        if (p < pts) raw = *reinterpret_cast<const u32x4 *>(w + ((int64_t)b * N + n0 + p) * HS + h * S + u * UE);
+        const T *e = reinterpret_cast<const T *>(&raw);
+#pragma unroll
+        for (int j = 0; j < UE; ++j) wlf[p * (SB * 4) + u * UE + j] = load_as_f32(e + j);
+      }
+    } else {
+      for (int i = t; i < kPartialTile * SB * 4; i += 256) {
+        const int p = i / (SB * 4), s = i - p * (SB * 4);
+        wlf[i] = (p < pts && s < S) ? load_as_f32(w + ((int64_t)b * N + n0 + p) * HS + h * S + s) : 0.f;
+      }
     }
-    for (int i = t; i < kPartialTile * DB * 4; i += 256) {
-      const int p = i / (DB * 4), d = i - p * (DB * 4);
-      float v = 0.f;
-      if (p < pts && d < D) v = load_as_f32(fx_mid + ((int64_t)b * N + n0 + p) * HD + h * D + d);
-      if (p < pts && d == D) v = 1.f;
-      flf[i] = v;
+    if (vec_f) {
+      const int units = D / UE;
+      for (int i = t; i < kPartialTile * units; i += 256) {
+        const int p = i / units, u = i - p * units;
+        u32x4 raw = {0u, 0u, 0u, 0u};
+        if (p < pts) raw = *reinterpret_cast<const u32x4 *>(fx_mid + ((int64_t)b * N + n0 + p) * HD + h * D + u * UE);
+        const T *e = reinterpret_cast<const T *>(&raw);
+#pragma unroll
+        for (int j = 0; j < UE; ++j) flf[p * (DB * 4) + u * UE + j] = load_as_f32(e + j);
+      }
+      for (int i = t; i < kPartialTile * (DB * 4 - D); i += 256) {  // the count column and the padding behind it
+        const int p = i / (DB * 4 - D), d = D + i - p * (DB * 4 - D);
+        flf[p * (DB * 4) + d] = (p < pts && d == D) ? 1.f : 0.f;
+      }
+    } else {
+      for (int i = t; i < kPartialTile * DB * 4; i += 256) {
+        const int p = i / (DB * 4), d = i - p * (DB * 4);
+        float v = 0.f;
+        if (p < pts && d < D) v = load_as_f32(fx_mid + ((int64_t)b * N + n0 + p) * HD + h * D + d);
+        if (p < pts && d == D) v = 1.f;
+        flf[i] = v;
+      }
     }
     __syncthreads();
 #pragma unroll 2
