@@ -238,17 +238,58 @@ __global__ __launch_bounds__(256) void slice_softmax_backward_kernel(
       w2[i] = plus.w2[i];
     }
   }
-  for (int i = t; i < R * D; i += 256) {
-    const int r = i / D, d = i - r * D;
-    const bool ok = r < rows;
-    const int64_t off = (m0 + r) * HD + h * D + d;
-    xm[r * D1 + d] = ok ? load_as_f32(x_mid + off) : 0.f;
-    fm[r * D1 + d] = ok ? load_as_f32(fx_mid + off) : 0.f;
-    go[r * D1 + d] = ok ? load_as_f32(d_out_x + off) : 0.f;
+  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+  constexpr int UE = 16 / sizeof(T);
+  // rows that are whole numbers of 16-byte units move with 16-byte accesses
+  const bool vec_d = D % UE == 0 && (reinterpret_cast<uintptr_t>(x_mid) | reinterpret_cast<uintptr_t>(fx_mid) |
+                                     reinterpret_cast<uintptr_t>(d_out_x) | reinterpret_cast<uintptr_t>(d_proj)) % 16 == 0;
+  const bool vec_s = S % UE == 0 && (reinterpret_cast<uintptr_t>(w) | reinterpret_cast<uintptr_t>(d_z) |
+                                     (PLUS ? reinterpret_cast<uintptr_t>(plus.d_a1) : 0)) % 16 == 0;
+  if (vec_d) {
+    const int units = D / UE;
+    for (int i = t; i < R * units; i += 256) {
+      const int r = i / units, u = i - r * units;
+      u32x4 rx = {0u, 0u, 0u, 0u}, rf = rx, rg = rx;
+      if (r < rows) {
+        const int64_t off = (m0 + r) * HD + h * D + u * UE;
+        rx = *reinterpret_cast<const u32x4 *>(x_mid + off);
+        rf = *reinterpret_cast<const u32x4 *>(fx_mid + off);
+        rg = *reinterpret_cast<const u32x4 *>(d_out_x + off);
+      }
+      const T *ex = reinterpret_cast<const T *>(&rx), *ef = reinterpret_cast<const T *>(&rf),
+              *eg = reinterpret_cast<const T *>(&rg);
+#pragma unroll
+      for (int j = 0; j < UE; ++j) {
+        xm[r * D1 + u * UE + j] = load_as_f32(ex + j);
+        fm[r * D1 + u * UE + j] = load_as_f32(ef + j);
+        go[r * D1 + u * UE + j] = load_as_f32(eg + j);
+      }
+    }
+  } else {
+    for (int i = t; i < R * D; i += 256) {
+      const int r = i / D, d = i - r * D;
+      const bool ok = r < rows;
+      const int64_t off = (m0 + r) * HD + h * D + d;
+      xm[r * D1 + d] = ok ? load_as_f32(x_mid + off) : 0.f;
+      fm[r * D1 + d] = ok ? load_as_f32(fx_mid + off) : 0.f;
+      go[r * D1 + d] = ok ? load_as_f32(d_out_x + off) : 0.f;
+    }
   }
-  for (int i = t; i < R * S; i += 256) {
-    const int r = i / S, s = i - r * S;
-    wl[r * S1 + s] = r < rows ? load_as_f32(w + (m0 + r) * HS + h * S + s) : 0.f;
+  if (vec_s) {
+    const int units = S / UE;
+    for (int i = t; i < R * units; i += 256) {
+      const int r = i / units, u = i - r * units;
+      u32x4 rw = {0u, 0u, 0u, 0u};
+      if (r < rows) rw = *reinterpret_cast<const u32x4 *>(w + (m0 + r) * HS + h * S + u * UE);
+      const T *ew = reinterpret_cast<const T *>(&rw);
+#pragma unroll
+      for (int j = 0; j < UE; ++j) wl[r * S1 + u * UE + j] = load_as_f32(ew + j);
+    }
+  } else {
+    for (int i = t; i < R * S; i += 256) {
+      const int r = i / S, s = i - r * S;
+      wl[r * S1 + s] = r < rows ? load_as_f32(w + (m0 + r) * HS + h * S + s) : 0.f;
+    }
   }
   __syncthreads();
 
@@ -354,11 +395,28 @@ __global__ __launch_bounds__(256) void slice_softmax_backward_kernel(
     dT_part[(int64_t)blockIdx.x * H + h] = PLUS ? total : -total * inv_temp_h;
   }
 
-  for (int i = t; i < rows * S; i += 256) {
-    const int r = i / S, s = i - r * S;
-    store_from_f32(d_z + (m0 + r) * HS + h * S + s, dwl[r * S1 + s]);
-    if constexpr (PLUS)
-      store_from_f32(static_cast<T *>(plus.d_a1) + (m0 + r) * HS + h * S + s, a1l[r * S1 + s]);
+  if (vec_s) {
+    const int units = S / UE;
+    for (int i = t; i < rows * units; i += 256) {
+      const int r = i / units, u = i - r * units;
+      alignas(16) T o[UE];
+#pragma unroll
+      for (int j = 0; j < UE; ++j) store_from_f32(o + j, dwl[r * S1 + u * UE + j]);
+      *reinterpret_cast<u32x4 *>(d_z + (m0 + r) * HS + h * S + u * UE) = *reinterpret_cast<const u32x4 *>(o);
+      if constexpr (PLUS) {
+#pragma unroll
+        for (int j = 0; j < UE; ++j) store_from_f32(o + j, a1l[r * S1 + u * UE + j]);
+        *reinterpret_cast<u32x4 *>(static_cast<T *>(plus.d_a1) + (m0 + r) * HS + h * S + u * UE) =
+            *reinterpret_cast<const u32x4 *>(o);
+      }
+    }
+  } else {
+    for (int i = t; i < rows * S; i += 256) {
+      const int r = i / S, s = i - r * S;
+      store_from_f32(d_z + (m0 + r) * HS + h * S + s, dwl[r * S1 + s]);
+      if constexpr (PLUS)
+        store_from_f32(static_cast<T *>(plus.d_a1) + (m0 + r) * HS + h * S + s, a1l[r * S1 + s]);
+    }
   }
   // d x_mid and d fx_mid: a thread owns 2 rows x 2 features (features dq and dq + DQ), 8 LDS reads per 8 multiply-adds
   const int DQ = (D + 1) >> 1;
@@ -397,12 +455,32 @@ __global__ __launch_bounds__(256) void slice_softmax_backward_kernel(
       for (int k = 0; k < 2; ++k) {
         const int d = dq + k * DQ;
         if (d >= D) continue;
-        if constexpr (PLUS) {
+        if (vec_d) {  // xm / fm are free since the first phase: the results leave through them as 16-byte stores
+          xm[r * D1 + d] = PLUS ? dx[jj][k] + df[jj][k] : dx[jj][k];
+          fm[r * D1 + d] = df[jj][k];
+        } else if constexpr (PLUS) {
           store_from_f32(d_proj + (m0 + r) * HD + h * D + d, dx[jj][k] + df[jj][k]);
         } else {
           store_from_f32(d_proj + (m0 + r) * 2 * HD + h * D + d, dx[jj][k]);
           store_from_f32(d_proj + (m0 + r) * 2 * HD + HD + h * D + d, df[jj][k]);
         }
+      }
+    }
+  }
+  if (vec_d) {
+    __syncthreads();
+    const int units = D / UE;
+    for (int i = t; i < rows * units; i += 256) {
+      const int r = i / units, u = i - r * units;
+      alignas(16) T o[UE];
+#pragma unroll
+      for (int j = 0; j < UE; ++j) store_from_f32(o + j, xm[r * D1 + u * UE + j]);
+      T *dst = d_proj + (m0 + r) * (PLUS ? HD : 2 * HD) + h * D + u * UE;
+      *reinterpret_cast<u32x4 *>(dst) = *reinterpret_cast<const u32x4 *>(o);
+      if constexpr (!PLUS) {
+#pragma unroll
+        for (int j = 0; j < UE; ++j) store_from_f32(o + j, fm[r * D1 + u * UE + j]);
+        *reinterpret_cast<u32x4 *>(dst + HD) = *reinterpret_cast<const u32x4 *>(o);
       }
     }
   }
