@@ -24,6 +24,31 @@ namespace general {
 // 64x64 output tile per 256-thread workgroup, 4x4 outputs per thread, K staged 16 at a time through LDS.
 // blockIdx.z selects one of two (W, bias, out) sets that share the same input (x_mid and fx_mid).
 // ------------------------------------------------------------------------------------------------
+// four consecutive elements with one 8- or 16-byte access
+template <typename T>
+__device__ __forceinline__ void load4(const T *p, float (&v)[4]) {
+  if constexpr (sizeof(T) == 2) {
+    const uint2 r = *reinterpret_cast<const uint2 *>(p);
+    const T *e = reinterpret_cast<const T *>(&r);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) v[j] = load_as_f32(e + j);
+  } else {
+    const float4 r = *reinterpret_cast<const float4 *>(p);
+    v[0] = r.x, v[1] = r.y, v[2] = r.z, v[3] = r.w;
+  }
+}
+template <typename T>
+__device__ __forceinline__ void store4(T *p, const float (&v)[4]) {
+  if constexpr (sizeof(T) == 2) {
+    alignas(8) T o[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) store_from_f32(o + j, v[j]);
+    *reinterpret_cast<uint2 *>(p) = *reinterpret_cast<const uint2 *>(o);
+  } else {
+    *reinterpret_cast<float4 *>(p) = float4{v[0], v[1], v[2], v[3]};
+  }
+}
+
 template <typename TA, typename TW>
 __global__ __launch_bounds__(256) void rows_gemm_kernel(GemmArgs a) {
   __shared__ float As[16][64 + 4];
@@ -65,7 +90,23 @@ __global__ __launch_bounds__(256) void rows_gemm_kernel(GemmArgs a) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
 
+  // a Linear whose rows are whole numbers of four elements is staged with 8- / 16-byte loads
+  const bool vec = a.ks == 0 && a.K % 4 == 0 && reinterpret_cast<uintptr_t>(in) % 16 == 0 &&
+                   reinterpret_cast<uintptr_t>(W) % 16 == 0;
+  const bool vec_out = a.O % 4 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0;
   for (int k0 = 0; k0 < a.K; k0 += 16) {
+    if (vec) {
+      float av4[4] = {0.f, 0.f, 0.f, 0.f}, wv4[4] = {0.f, 0.f, 0.f, 0.f};
+      if (k0 + lk < a.K) {
+        if (m_ok) load4(in + m_ld * a.K + k0 + lk, av4);
+        if (o_ld < a.O) load4(W + (int64_t)o_ld * a.K + k0 + lk, wv4);
+      }
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        As[lk + q][lr] = av4[q];
+        Ws[lk + q][lr] = wv4[q];
+      }
+    } else
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
       const int k = k0 + lk + q;
@@ -107,6 +148,16 @@ __global__ __launch_bounds__(256) void rows_gemm_kernel(GemmArgs a) {
   for (int i = 0; i < 4; ++i) {
     const int64_t m = m0 + ty * 4 + i;
     if (m >= a.M) continue;
+    if (vec_out && o0 + tx * 4 < a.O) {
+      float v4[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float v = acc[i][j] + (bias ? bias[o0 + tx * 4 + j] : 0.f);
+        v4[j] = a.act == 1 ? gelu_erf(v) : v;
+      }
+      store4(out + m * a.O + o0 + tx * 4, v4);
+      continue;
+    }
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int o = o0 + tx * 4 + j;
