@@ -215,7 +215,7 @@ def _plus_backward_tail(ctx, x, uniform, x_mid, w, tok_out, out_x, dy, g, d_num,
     d_w1, d_b1 = _wgrad(d_a1.reshape(-1, S), xm_rows)
     hidden = torch.nn.functional.gelu(torch.addmm(kp["proj_temperature_0_bias"], xm_rows.float(),
                                                   kp["proj_temperature_0_weight"].view(S, D).t()))
-    d_w2 = d_a2.reshape(1, -1) @ hidden
+    d_w2 = (d_a2.reshape(-1, 1) * hidden).sum(0, keepdim=True)  # (1, rows) x (rows, S): a reduction, not a GEMM shape
     d_b2 = d_a2.sum().reshape(1)
 
     k = dims.conv_k

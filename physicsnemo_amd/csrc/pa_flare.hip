@@ -33,14 +33,66 @@ __global__ __launch_bounds__(256) void column_max_partial_kernel(const T *__rest
   }
 }
 
-// grid (ceil(B*H*S / 256)): maximum over the G partials.
+// The same with 16-byte loads, for rows that are whole numbers of 16-byte units: a thread keeps the running maxima of
+// its unit of columns; when a row has fewer than 256 units several row groups share the chunk and meet in LDS.
+template <typename T>
+__global__ __launch_bounds__(256) void column_max_partial_vec_kernel(const T *__restrict__ a, float *__restrict__ partial,
+                                                                     int64_t N, int HS) {
+  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+  constexpr int UE = 16 / sizeof(T);
+  __shared__ float red[256 * UE];
+  const int g = blockIdx.x, b = blockIdx.y, t = threadIdx.x;
+  const int64_t n0 = (int64_t)g * kChunkRows;
+  const int rows = (int)min((int64_t)kChunkRows, N - n0);
+  const T *src = a + ((int64_t)b * N + n0) * HS;
+  const int units = HS / UE;
+  const int upb = units < 256 ? units : 256;  // units per pass
+  const int groups = 256 / upb;               // row groups per pass
+  const int rg = t / upb, u_in = t - rg * upb;
+  float *dst = partial + ((int64_t)g * gridDim.y + b) * HS;
+  for (int u0 = 0; u0 < units; u0 += upb) {
+    const int u = u0 + u_in;
+    float m[UE];
+#pragma unroll
+    for (int j = 0; j < UE; ++j) m[j] = -INFINITY;
+    if (rg < groups && u < units) {
+      for (int r = rg; r < rows; r += groups) {
+        const u32x4 raw = *reinterpret_cast<const u32x4 *>(src + (int64_t)r * HS + u * UE);
+        const T *e = reinterpret_cast<const T *>(&raw);
+#pragma unroll
+        for (int j = 0; j < UE; ++j) m[j] = fmaxf(m[j], load_as_f32(e + j));
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < UE; ++j) red[t * UE + j] = m[j];
+    __syncthreads();
+    // column c of this pass: the maximum over the row groups
+    for (int c = t; c < upb * UE && u0 * UE + c < HS; c += 256) {
+      float v = -INFINITY;
+      for (int q = 0; q < groups; ++q) v = fmaxf(v, red[(q * upb) * UE + c]);
+      dst[u0 * UE + c] = v;
+    }
+  }
+}
+
+// grid (ceil(B*H*S / 16)): maximum over the G partials; 16 outputs x 16 interleaved slices of the partials per
+// workgroup, the slices meet in LDS.
 __global__ __launch_bounds__(256) void column_max_combine_kernel(const float *__restrict__ partial, int G, int64_t BHS,
                                                                  float *__restrict__ colmax) {
-  const int64_t o = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (o >= BHS) return;
+  __shared__ float red[16][17];
+  const int oc = threadIdx.x & 15, q = threadIdx.x >> 4;
+  const int64_t o = (int64_t)blockIdx.x * 16 + oc;
   float m = -INFINITY;
-  for (int g = 0; g < G; ++g) m = fmaxf(m, partial[(int64_t)g * BHS + o]);
-  colmax[o] = m;
+  if (o < BHS)
+    for (int g = q; g < G; g += 16) m = fmaxf(m, partial[(int64_t)g * BHS + o]);
+  red[q][oc] = m;
+  __syncthreads();
+  if (q == 0 && o < BHS) {
+#pragma unroll
+    for (int k = 1; k < 16; ++k) m = fmaxf(m, red[k][oc]);
+    colmax[o] = m;
+  }
 }
 
 // wc[b,n,c] = exp(A[b,n,c] - m[b,c]), c = h*S + s; element-wise over (B*N, H*S).
@@ -52,6 +104,41 @@ __global__ __launch_bounds__(256) void column_weights_kernel(const T *__restrict
     const int c = (int)(i - row * HS);
     const int64_t b = row / N;
     store_from_f32(wc + i, expf(load_as_f32(a + i) - colmax[b * HS + c]));
+  }
+}
+
+// The same with 16-byte accesses (H*S a multiple of the 16-byte unit).
+template <typename T>
+__global__ __launch_bounds__(256) void column_weights_vec_kernel(const T *__restrict__ a,
+                                                                 const float *__restrict__ colmax, T *__restrict__ wc,
+                                                                 int64_t N, int HS, int64_t total_units) {
+  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+  constexpr int UE = 16 / sizeof(T);
+  const int units = HS / UE;
+  const bool narrow = total_units < (int64_t)1 << 32;  // 64-bit divisions cost more than the exponentials
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total_units; i += (int64_t)gridDim.x * 256) {
+    int64_t row, b;
+    if (narrow) {
+      const uint32_t r32 = (uint32_t)i / (uint32_t)units;
+      row = r32;
+      b = N < ((int64_t)1 << 32) ? (int64_t)(r32 / (uint32_t)N) : 0;
+    } else {
+      row = i / units;
+      b = row / N;
+    }
+    const int c = (int)(i - row * units) * UE;
+    const u32x4 raw = *reinterpret_cast<const u32x4 *>(a + i * UE);
+    const T *e = reinterpret_cast<const T *>(&raw);
+    float cm[UE];  // the unit's column maxima with 16-byte loads (c is a multiple of UE, UE a multiple of 4)
+#pragma unroll
+    for (int j = 0; j < UE; j += 4) {
+      const float4 q = *reinterpret_cast<const float4 *>(colmax + b * HS + c + j);
+      cm[j] = q.x, cm[j + 1] = q.y, cm[j + 2] = q.z, cm[j + 3] = q.w;
+    }
+    alignas(16) T o[UE];
+#pragma unroll
+    for (int j = 0; j < UE; ++j) store_from_f32(o + j, expf(load_as_f32(e + j) - cm[j]));
+    *reinterpret_cast<u32x4 *>(wc + i * UE) = *reinterpret_cast<const u32x4 *>(o);
   }
 }
 
@@ -253,14 +340,29 @@ template <typename T>
 static int column_weights_t(const pa_shape &s, const void *a, float *partial, float *colmax, void *wc, hipStream_t st) {
   const int HS = (int)(s.H * s.S);
   const int64_t G = column_max_chunks(s), BHS = s.B * HS, total = s.B * s.N * HS;
-  hipLaunchKernelGGL((column_max_partial_kernel<T>), dim3((unsigned)G, (unsigned)s.B), dim3(256), 0, st,
-                     static_cast<const T *>(a), partial, s.N, HS);
+  constexpr int UE = 16 / sizeof(T);
+  const bool vec = HS % UE == 0 && (reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(wc) |
+                                    reinterpret_cast<uintptr_t>(colmax)) % 16 == 0;
+  if (vec)
+    hipLaunchKernelGGL((column_max_partial_vec_kernel<T>), dim3((unsigned)G, (unsigned)s.B), dim3(256), 0, st,
+                       static_cast<const T *>(a), partial, s.N, HS);
+  else
+    hipLaunchKernelGGL((column_max_partial_kernel<T>), dim3((unsigned)G, (unsigned)s.B), dim3(256), 0, st,
+                       static_cast<const T *>(a), partial, s.N, HS);
   int rc = launch_status();
   if (rc) return rc;
-  hipLaunchKernelGGL(column_max_combine_kernel, dim3((unsigned)((BHS + 255) / 256)), dim3(256), 0, st, partial, (int)G,
+  hipLaunchKernelGGL(column_max_combine_kernel, dim3((unsigned)((BHS + 15) / 16)), dim3(256), 0, st, partial, (int)G,
                      BHS, colmax);
   rc = launch_status();
   if (rc) return rc;
+  if (vec) {
+    const int64_t total_units = total / UE;
+    int64_t blocks = (total_units + 255) / 256;
+    if (blocks > 16384) blocks = 16384;
+    hipLaunchKernelGGL((column_weights_vec_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, st,
+                       static_cast<const T *>(a), colmax, static_cast<T *>(wc), s.N, HS, total_units);
+    return launch_status();
+  }
   int64_t blocks = (total + 255) / 256;
   if (blocks > 8192) blocks = 8192;
   hipLaunchKernelGGL((column_weights_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, st, static_cast<const T *>(a),
