@@ -432,6 +432,16 @@ int pa_layer_forward(int dtype, const pa_shape *shape, const pa_params *p, const
                      const pa_block_tail *tail, float *slice_token_out, void *workspace,
                      int64_t workspace_bytes, void *stream);
 
+/* The Transolver++ layer (plus = True: PA.py:166-170, :530-537; one projection, per-point temperature, Gumbel noise
+ * from the caller's samples `uniform` (B,N,H,S) bf16) on the staged bf16 MFMA kernels: dtype PA_BF16, D = 32,
+ * C in {128, 256, 512}, S in {16, 32, 64, 128}, Linear projections (pa_layer_forward_plus_supported() == 1; other
+ * shapes run the stage sequence on the general kernels).  Workspace: pa_layer_forward_plus_workspace_bytes(). */
+int pa_layer_forward_plus_supported(int dtype, const pa_shape *shape);
+int64_t pa_layer_forward_plus_workspace_bytes(int dtype, const pa_shape *shape);
+int pa_layer_forward_plus(int dtype, const pa_shape *shape, const pa_params *p, const pa_plus_params *plus,
+                          const void *x, const void *uniform, void *y, const pa_block_tail *tail,
+                          float *slice_token_out, void *workspace, int64_t workspace_bytes, void *stream);
+
 /* pa_layer_forward for the fused MFMA shapes (pa_query_path() == 1, bf16 weights) with the parameters already
  * repacked by pa_mfma_pack_params into `blob` (PA_BUF_BLOB bytes): callers that run many forwards with unchanged
  * weights keep the blob and skip the repack.  Of `p` only qkv_project_weight is read.  Workspace as for

@@ -25,7 +25,8 @@ EXPORTED = [
     "pa_slice_attention_backward", "pa_slice_softmax_backward", "pa_slice_softmax_plus",
     "pa_backward_point_tiles_plus", "pa_slice_softmax_plus_backward", "pa_slice_cross_attention_mix",
     "pa_mfma_pack_tokens", "pa_flare_column_max_chunks", "pa_flare_column_weights", "pa_flare_softmax_rows",
-    "pa_flare_backward_points", "pa_deslice", "pa_cols_gemm_f32_chunks", "pa_cols_gemm_f32", "pa_ball_query", "pa_ball_query_cells",
+    "pa_flare_backward_points", "pa_deslice", "pa_cols_gemm_f32_chunks", "pa_cols_gemm_f32", "pa_ball_query", "pa_ball_query_cells", "pa_layer_forward_plus_supported",
+    "pa_layer_forward_plus_workspace_bytes", "pa_layer_forward_plus",
     "pa_mfma_backward_query", "pa_rows_gemm_packed", "pa_mfma_slice_weighted_sum", "pa_mfma_deslice",
     "pa_mfma_backward_tables_bytes", "pa_mfma_backward_groups", "pa_mfma_slice_softmax_backward",
     "pa_cols_gemm_chunks", "pa_cols_gemm", "pa_residual_layernorm",
@@ -158,6 +159,13 @@ def load() -> ctypes.CDLL:
     lib.pa_flare_backward_points.argtypes = [c_int, ps] + [c_void_p] * 10
     lib.pa_deslice.restype = c_int
     lib.pa_deslice.argtypes = [c_int, ps] + [c_void_p] * 4
+    lib.pa_layer_forward_plus_supported.restype = c_int
+    lib.pa_layer_forward_plus_supported.argtypes = [c_int, ps]
+    lib.pa_layer_forward_plus_workspace_bytes.restype = c_int64
+    lib.pa_layer_forward_plus_workspace_bytes.argtypes = [c_int, ps]
+    lib.pa_layer_forward_plus.restype = c_int
+    lib.pa_layer_forward_plus.argtypes = [c_int, ps, pp, POINTER(PaPlusParams), c_void_p, c_void_p, c_void_p,
+                                          POINTER(PaBlockTail), c_void_p, c_void_p, c_int64, c_void_p]
     lib.pa_ball_query.restype = c_int
     lib.pa_ball_query.argtypes = [c_int64, c_int64, c_int64, c_int64, c_float, c_void_p, c_void_p, c_void_p,
                                   c_void_p, c_void_p, c_void_p, c_void_p]

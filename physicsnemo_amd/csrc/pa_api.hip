@@ -886,4 +886,63 @@ int pa_layer_forward(int dtype, const pa_shape *shape, const pa_params *p, const
   return rc;
 }
 
+int pa_layer_forward_plus_supported(int dtype, const pa_shape *shape) {
+  if (check_shape(dtype, shape)) return 0;
+  return pa::mfma::staged_supported(dtype, *shape) ? 1 : 0;
+}
+
+int64_t pa_layer_forward_plus_workspace_bytes(int dtype, const pa_shape *shape) {
+  int rc = check_shape(dtype, shape);
+  if (rc) return rc;
+  if (!pa::mfma::staged_supported(dtype, *shape)) return PA_ERR_UNSUPPORTED;
+  return plan_staged(*shape).total;
+}
+
+int pa_layer_forward_plus(int dtype, const pa_shape *shape, const pa_params *p, const pa_plus_params *plus,
+                          const void *x, const void *uniform, void *y, const pa_block_tail *tail,
+                          float *slice_token_out, void *workspace, int64_t workspace_bytes, void *stream) {
+  int rc = check_shape(dtype, shape);
+  if (rc) return rc;
+  if (!p || !plus || !x || !uniform || !y || !workspace) return PA_ERR_NULL;
+  if (!p->in_project_x_weight || !p->in_project_slice_weight || !p->in_project_slice_bias || !p->temperature ||
+      !p->qkv_project_weight || !p->out_linear_weight || !plus->proj_temperature_0_weight ||
+      !plus->proj_temperature_0_bias || !plus->proj_temperature_2_weight || !plus->proj_temperature_2_bias)
+    return PA_ERR_NULL;
+  if (!aligned16(x) || !aligned16(uniform) || !aligned16(y) || !aligned16(workspace)) return PA_ERR_ALIGN;
+  if ((rc = check_tail(tail))) return rc;
+  const pa_shape &s = *shape;
+  if (!pa::mfma::staged_supported(dtype, s)) return PA_ERR_UNSUPPORTED;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const StagedPlan sp = plan_staged(s);
+  if (workspace_bytes < sp.total) return PA_ERR_WORKSPACE;
+  char *ws = static_cast<char *>(workspace);
+  void *x_mid = ws + sp.off_x_mid, *fxp = ws + sp.off_fx, *wp = ws + sp.off_w, *tokp = ws + sp.off_tokp;
+  float *partials = reinterpret_cast<float *>(ws + sp.off_partials);
+  float *tok = slice_token_out ? slice_token_out : reinterpret_cast<float *>(ws + sp.off_tok);
+  float *norm = reinterpret_cast<float *>(ws + sp.off_norm);
+  float *tok_out = reinterpret_cast<float *>(ws + sp.off_tok_out);
+  pa::GemmArgs a{};  // x -> x_mid, natural layout for the slice weights and packed for the aggregation (fx_mid is x_mid)
+  a.in = x;
+  a.w[0] = p->in_project_x_weight;
+  a.bias[0] = p->in_project_x_bias;
+  a.out[0] = x_mid;
+  a.out_pack[0] = fxp;
+  a.M = s.B * s.N;
+  a.N = (int)s.N;
+  a.K = a.C = (int)s.C;
+  a.O = (int)(s.H * 32);
+  a.pack_tpb = (int)pa::mfma::tiles_per_batch(s);
+  a.pack_heads = (int)s.H;
+  if (!pa::gemm::serves(a, 1, 2)) return PA_ERR_UNSUPPORTED;
+  if ((rc = pa::gemm::launch(a, 1, PA_BF16, st))) return rc;
+  if ((rc = pa::mfma::slice_softmax_pack_plus(s, *p, *plus, x_mid, uniform, wp, compute_units(), st))) return rc;
+  if ((rc = pa::mfma::slice_reduce(s, wp, fxp, partials, st))) return rc;
+  if ((rc = pa::mfma::combine_attention(s, *p, partials, sp.G, tok, norm, tok_out, tokp, st))) return rc;
+  void *out_x = x_mid;
+  if ((rc = pa::mfma::deslice_natural(s, wp, tokp, out_x, compute_units(), st))) return rc;
+  if ((rc = pa::general::out_linear(dtype, s, *p, out_x, y, st))) return rc;
+  if (tail_active(tail)) rc = pa::general::residual_ln(dtype, s, y, *tail, st);
+  return rc;
+}
+
 }  // extern "C"

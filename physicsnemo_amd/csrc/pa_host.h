@@ -138,6 +138,8 @@ int ball_query_cells(int64_t B, int64_t Np, int64_t Nq, int64_t K, float radius,
 
 namespace mfma {
 bool staged_supported(int dtype, const pa_shape &s);
+int slice_softmax_pack_plus(const pa_shape &s, const pa_params &p, const pa_plus_params &pp, const void *x_mid,
+                            const void *uniform, void *w_pack, int num_cu, hipStream_t st);
 int slice_softmax_pack(const pa_shape &s, const pa_params &p, const void *x_mid, void *w_pack, int num_cu,
                        hipStream_t st);
 bool backward_supported(const pa_shape &s);

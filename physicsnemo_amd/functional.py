@@ -193,6 +193,35 @@ def layer_forward(x, params, dims: LayerDims, residual=None, ln_weight=None, ln_
     return (out, tok) if return_slice_tokens else out
 
 
+def layer_forward_plus_supported(dtype: torch.dtype, dims: LayerDims) -> bool:
+    """True where the whole Transolver++ layer runs on the staged bf16 MFMA kernels."""
+    if dtype != torch.bfloat16:
+        return False
+    return bool(_lib.load().pa_layer_forward_plus_supported(_lib.PA_BF16, byref(dims.c())))
+
+
+def layer_forward_plus(x, uniform, params, dims: LayerDims, residual=None, ln_weight=None, ln_bias=None, ln_eps=1e-5):
+    """Whole Transolver++ layer (plus=True) on the staged bf16 MFMA kernels; `uniform` (B, N, H, S) bf16: the samples
+    behind the Gumbel noise.  Returns y, or (fx_new, ln_out) with a tail."""
+    _need_cuda(x, uniform, residual)
+    if uniform.dtype != x.dtype or uniform.shape != (dims.B, dims.N, dims.H, dims.S):
+        raise ValueError("uniform samples must have the activation dtype and shape (B, N, H, S)")
+    lib = _lib.load()
+    code, shape = _lib.dtype_code(x.dtype), dims.c()
+    nbytes = lib.pa_layer_forward_plus_workspace_bytes(code, byref(shape))
+    if nbytes < 0:
+        _lib.check(int(nbytes), "pa_layer_forward_plus_workspace_bytes")
+    workspace = torch.empty(int(nbytes), dtype=torch.uint8, device=x.device)
+    y = torch.empty(dims.B, dims.N, dims.C, dtype=x.dtype, device=x.device)
+    ln_out = torch.empty_like(y) if ln_weight is not None else None
+    tail = _c_tail(residual, ln_weight, ln_bias, ln_eps, ln_out)
+    plus = _lib.PaPlusParams(*[_lib.ptr(params[k]) for k, _ in _lib.PaPlusParams._fields_])
+    _lib.check(lib.pa_layer_forward_plus(code, byref(shape), byref(_c_params(params)), byref(plus), x.data_ptr(),
+                                         uniform.data_ptr(), y.data_ptr(), byref(tail), None, workspace.data_ptr(),
+                                         int(nbytes), _lib.current_stream_ptr(x.device)), "pa_layer_forward_plus")
+    return y if (residual is None and ln_out is None) else (y, ln_out)
+
+
 def residual_layernorm(y, residual=None, ln_weight=None, ln_bias=None, ln_eps=1e-5):
     """In place y <- y + residual (if given); returns (y, LayerNorm(y)) when ln_weight is given, else y."""
     _need_cuda(y, residual, ln_weight, ln_bias)

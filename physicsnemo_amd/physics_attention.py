@@ -217,10 +217,13 @@ class PhysicsAttentionBase(nn.Module):
         x = self._prepare_input(x)
         dims = self.layer_dims(x)
         p = self.kernel_params(x.dtype, x.device)
-        x_mid, fx_mid = PF.project_inputs(x, p, dims)
         if noise_u is None:
             noise_u = torch.rand((dims.B, dims.N, dims.H, dims.S), dtype=x.dtype, device=x.device)
-        w = PF.slice_softmax_plus(x_mid, noise_u.to(x.dtype).contiguous(), p, dims)
+        noise_u = noise_u.to(x.dtype).contiguous()
+        if not stages and not self.fp8_weights and PF.layer_forward_plus_supported(x.dtype, dims):
+            return self.out_dropout(PF.layer_forward_plus(x, noise_u, p, dims))  # staged bf16 MFMA kernels
+        x_mid, fx_mid = PF.project_inputs(x, p, dims)
+        w = PF.slice_softmax_plus(x_mid, noise_u, p, dims)
         tok, norm = PF.slice_reduce(w, fx_mid, dims)
         tok_out = PF.slice_attention(tok, p, dims)
         y = PF.deslice_project(w, tok_out, p, dims)
@@ -236,6 +239,15 @@ class PhysicsAttentionBase(nn.Module):
             with torch.autocast("cuda", enabled=False):  # float32 inside, as the residual stream of the caller is
                 return self.forward_block(x.float(), residual.float(), ln)
         self._validate(x)
+        if self.plus and not self._needs_grad(x) and not self.fp8_weights and not (self.training and self.out_dropout.p > 0):
+            xp = self._prepare_input(x)
+            dims = self.layer_dims(xp)
+            if PF.layer_forward_plus_supported(xp.dtype, dims):
+                u = torch.rand((dims.B, dims.N, dims.H, dims.S), dtype=xp.dtype, device=xp.device)
+                return PF.layer_forward_plus(
+                    xp, u, self.kernel_params(xp.dtype, xp.device), dims, residual=residual.to(xp.dtype).contiguous(),
+                    ln_weight=ln.weight.detach().float().contiguous(), ln_bias=ln.bias.detach().float().contiguous(),
+                    ln_eps=ln.eps)
         if self.plus or (self.training and self.out_dropout.p > 0):  # dropout sits between the layer and the residual add
             y = self.forward(x)
             fx_new = y + residual.to(y.dtype)

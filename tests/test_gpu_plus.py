@@ -61,6 +61,44 @@ def test_bf16_plus_layer():
     assert_rel_l2(got, want, "bf16 plus y", tol=2e-2)
 
 
+@pytest.mark.parametrize("dim,heads,S,B,N", [(256, 8, 64, 1, 5000), (128, 4, 16, 3, 1777), (256, 8, 32, 2, 4096),
+                                             (512, 16, 128, 1, 4100), (256, 8, 128, 1, 4097)])
+def test_bf16_plus_layer_on_the_mfma_kernels(dim, heads, S, B, N):
+    """The whole Transolver++ layer on the staged bf16 MFMA kernels: against the fp32 oracle with the same samples, and
+    against the stage-by-stage general kernels on the same bf16 inputs."""
+    from physicsnemo_amd import functional as PF
+
+    announce("bf16 plus MFMA", dim, heads, S, B, N)
+    ref, hip = _pair("irregular", dim, heads, 32, S, seed=S + B)
+    x = torch.randn(B, N, dim)
+    u = torch.rand(B, N, heads, S).bfloat16()
+    xb = x.cuda().bfloat16()
+    assert PF.layer_forward_plus_supported(torch.bfloat16, hip.layer_dims(xb))
+    with torch.no_grad():
+        want = ref.forward_with_noise(x, u.float())
+        got = hip.forward_with_noise(xb, u.cuda())
+        general = hip.forward_with_noise(xb, u.cuda(), stages=True)["y"]
+    assert got.dtype == torch.bfloat16 and torch.isfinite(got.float()).all()
+    assert_rel_l2(got, want, "bf16 plus y (MFMA) vs fp32 oracle", tol=2e-2)
+    assert_rel_l2(got, general, "bf16 plus y: MFMA vs general kernels", tol=1e-2)
+
+
+def test_bf16_plus_block_tail_on_the_mfma_kernels():
+    announce("bf16 plus forward_block")
+    ref, hip = _pair("irregular", 256, 8, 32, 64, seed=5)
+    ln = torch.nn.LayerNorm(256).cuda()
+    x, res = torch.randn(1, 4500, 256).cuda().bfloat16(), torch.randn(1, 4500, 256).cuda().bfloat16()
+    with torch.no_grad():
+        torch.manual_seed(3)
+        fx_new, normed = hip.forward_block(x, res, ln)
+        torch.manual_seed(3)
+        u = torch.rand(1, 4500, 8, 64, dtype=torch.bfloat16, device="cuda")
+        y = hip.forward_with_noise(x, u)
+    want = y.float() + res.float()
+    assert_rel_l2(fx_new, want, "fx_new", tol=1e-2)
+    assert_rel_l2(normed, torch.nn.functional.layer_norm(want, (256,), ln.weight, ln.bias, ln.eps), "LayerNorm", tol=1e-2)
+
+
 def test_plus_forward_draws_its_own_noise_reproducibly():
     announce("plus self-drawn noise")
     ref, hip = _pair("irregular", 32, 4, 8, 8)
