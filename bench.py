@@ -243,14 +243,14 @@ def time_variants(points, C, S, reps=5):
     xg = x.clone().requires_grad_(True)
     out[-1]["ms_forward_backward"] = round(timed(train_step(gale, lambda: gale((xg,), ctx)[0], xg), 3), 3)
     del geom, x, xg
-    # Transolver++ (general kernels, fp32 arithmetic): a quarter of the points
+    # Transolver++ (inference on the staged MFMA kernels, training on the general kernels): a quarter of the points
     pts = points // 4
     plus = pn.PhysicsAttentionIrregularMesh(C, heads=H, dim_head=32, slice_num=S, use_te=False, plus=True).cuda()
     xp = torch.randn(1, pts, C, device="cuda").bfloat16()
     with torch.no_grad():
         fwd = timed(lambda: plus(xp), 3)
     xpg = xp.clone().requires_grad_(True)
-    entry(f"Transolver++ layer bf16 (general kernels), C={C}, S={S}", pts, fwd,
+    entry(f"Transolver++ layer bf16 (staged MFMA forward; training on the general kernels), C={C}, S={S}", pts, fwd,
           timed(train_step(plus, lambda: plus(xpg), xpg), 2))
     del xp, xpg
     # FLARE (general kernels + two composed row GEMMs), bf16
