@@ -1,0 +1,73 @@
+"""Shapes that fall on and off the 16-byte fast paths of the general kernels (slice counts and head widths that are,
+or are not, whole numbers of 16-byte units in float32 and bf16), ragged point counts, batches: forward stages and all
+gradients against the oracle.  Bars: fp32 rtol 1e-4 (gradients 2e-4), bf16 rel-L2 1e-2 (gradients 3e-2; the scalar
+temperature sums 1e-1)."""
+import pytest
+import torch
+
+from gpu_util import announce, assert_fp32_close, assert_rel_l2, make_pair
+
+pytestmark = pytest.mark.gpu
+
+STAGES = ("x_mid", "fx_mid", "w", "tok", "norm", "tok_out", "y")
+#          dim heads dim_head  S    B   N
+SHAPES = [(40, 2, 20, 20, 2, 131),    # S = 20: units of four only;  D = 20
+          (36, 3, 12, 6, 1, 257),     # S = 6: no vector path at all; D = 12
+          (80, 2, 40, 24, 3, 65),     # D = 40, S = 24: whole 16-byte units in both types
+          (64, 8, 8, 40, 1, 1000),    # many heads, narrow
+          (64, 2, 32, 128, 2, 300),   # S = 128
+          (32, 1, 32, 10, 2, 33),     # one head, S = 10
+          (24, 2, 12, 4, 4, 7)]       # a handful of points
+
+
+@pytest.mark.parametrize("dim,heads,dim_head,S,B,N", SHAPES)
+def test_fp32_forward_stages_and_gradients(dim, heads, dim_head, S, B, N):
+    announce("shape sweep fp32", dim, heads, dim_head, S, B, N)
+    ref, hip = make_pair("irregular", dim, heads, dim_head, S, seed=S + N, sharpen=2.0)
+    x, probe = torch.randn(B, N, dim), torch.randn(B, N, dim)
+    with torch.no_grad():
+        want = ref.stages(x)
+        got = hip.forward_stages(x.cuda())
+    for k in STAGES:
+        assert_fp32_close(got[k], want[k], k)
+    ref.train(), hip.train()
+    xr, xh = x.clone().requires_grad_(), x.clone().cuda().requires_grad_()
+    (ref(xr) * probe).sum().backward()
+    (hip(xh) * probe.cuda()).sum().backward()
+    assert_fp32_close(xh.grad, xr.grad, "d x", rtol=2e-4)
+    grads = dict(hip.named_parameters())
+    for name, p in ref.named_parameters():
+        assert_fp32_close(grads[name].grad, p.grad, f"grad {name}", rtol=2e-4)
+
+
+@pytest.mark.parametrize("dim,heads,dim_head,S,B,N", SHAPES)
+def test_bf16_forward_and_gradients(dim, heads, dim_head, S, B, N):
+    announce("shape sweep bf16", dim, heads, dim_head, S, B, N)
+    ref, hip = make_pair("irregular", dim, heads, dim_head, S, seed=S + N)
+    x, probe = torch.randn(B, N, dim), torch.randn(B, N, dim)
+    ref.train(), hip.train()
+    xr = x.clone().requires_grad_()
+    yr = ref(xr)
+    (yr * probe).sum().backward()
+    xh = x.clone().cuda().bfloat16().requires_grad_()
+    yh = hip(xh)
+    assert yh.dtype == torch.bfloat16
+    assert_rel_l2(yh, yr, "bf16 y", tol=1e-2)
+    (yh.float() * probe.cuda()).sum().backward()
+    assert_rel_l2(xh.grad, xr.grad, "bf16 d x", tol=3e-2)
+    grads = dict(hip.named_parameters())
+    for name, p in ref.named_parameters():
+        tol = 1e-1 if name in ("temperature", "in_project_slice.bias") else 3e-2
+        assert_rel_l2(grads[name].grad, p.grad, f"bf16 grad {name}", tol=tol)
+
+
+def test_backward_refuses_slice_tables_beyond_lds_with_a_clear_error():
+    """The slice-attention backward keeps seven S x (D + 1) float32 tables in LDS: S = 128 with D = 48 does not fit.
+    The forward serves the shape; asking for gradients raises instead of computing something else."""
+    announce("backward LDS limit")
+    ref, hip = make_pair("irregular", 96, 2, 48, 128)
+    x = torch.randn(1, 200, 96)
+    with torch.no_grad():
+        assert_fp32_close(hip(x.cuda()), ref(x), "forward y")
+    with pytest.raises(RuntimeError, match="backward kernels do not serve this shape"):
+        hip(x.cuda().requires_grad_())
