@@ -253,11 +253,11 @@ def time_variants(points, C, S, reps=5):
     entry(f"Transolver++ layer bf16 (staged MFMA forward; training on the general kernels), C={C}, S={S}", pts, fwd,
           timed(train_step(plus, lambda: plus(xpg), xpg), 2))
     del xp, xpg
-    # FLARE (general kernels + two composed row GEMMs), bf16
+    # FLARE (two composed row GEMMs + the MFMA slice kernels), bf16
     flare = pn.FLARE(C, heads=H, dim_head=32, n_global_queries=S).cuda()
     xf = torch.randn(1, pts, C, device="cuda").bfloat16()
     with torch.no_grad():
-        entry(f"FLARE layer bf16 (general kernels), C={C}, {S} global queries", pts, timed(lambda: flare(xf), 3))
+        entry(f"FLARE layer bf16 (MFMA kernels), C={C}, {S} global queries", pts, timed(lambda: flare(xf), 3))
     del xf
     # GeoTransolver: context projectors + 4 GALE blocks (fused attention kernels, block-MLP kernel), bf16 autocast
     geo = pn.GeoTransolver(functional_dim=8, out_dim=4, geometry_dim=3, global_dim=16, n_layers=4, n_hidden=C,

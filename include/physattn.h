@@ -297,6 +297,18 @@ int64_t pa_flare_column_max_chunks(const pa_shape *shape);
 int pa_flare_column_weights(int dtype, const pa_shape *shape, const void *scores, float *partials, float *column_max,
                             void *weights, void *stream);
 int pa_flare_softmax_rows(int dtype, const pa_shape *shape, void *scores, void *stream);
+/* The whole FLARE layer forward on the bf16 MFMA kernels (flare_attention.py:222-255 with the weights composed as
+ * above): scores and values by the weights-stationary row GEMM (values straight into the packed operand layout),
+ * column maxima, one kernel that writes both normalisations of the scores as packed operands, the MFMA aggregation and
+ * deslice kernels of the PhysicsAttention layer, out_linear (+ optional residual / LayerNorm tail).  bf16, D = 32,
+ * C = H*32 in {128, 256}, S in {16, 32, 64, 128}, B*N >= 4096 (pa_flare_forward_mfma_supported() == 1).
+ * scores_weight (H*S, C) bf16, values_weight (H*32, C) bf16, out_linear_weight (C, H*32) bf16, biases float32. */
+int pa_flare_forward_mfma_supported(const pa_shape *shape);
+int64_t pa_flare_forward_mfma_workspace_bytes(const pa_shape *shape);
+int pa_flare_forward_mfma(const pa_shape *shape, const void *scores_weight, const float *scores_bias,
+                          const void *values_weight, const float *values_bias, const void *out_linear_weight,
+                          const float *out_linear_bias, const void *x, void *y, const pa_block_tail *tail,
+                          void *workspace, int64_t workspace_bytes, void *stream);
 /* Per-point part of the FLARE backward pass (the reference differentiates flare_attention.py:38-72 with autograd).
  * row_weights = softmax_s(A), column_weights = exp(A - max_n A), values v, d_out_x = gradient of the hand-back result
  * (B,N,H*D), z (B,H,S,D) float32, and d_num / d_den = gradients of the un-normalised gather sums (z = num / den):

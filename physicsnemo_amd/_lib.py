@@ -26,7 +26,8 @@ EXPORTED = [
     "pa_backward_point_tiles_plus", "pa_slice_softmax_plus_backward", "pa_slice_cross_attention_mix",
     "pa_mfma_pack_tokens", "pa_flare_column_max_chunks", "pa_flare_column_weights", "pa_flare_softmax_rows",
     "pa_flare_backward_points", "pa_deslice", "pa_cols_gemm_f32_chunks", "pa_cols_gemm_f32", "pa_ball_query", "pa_ball_query_cells", "pa_layer_forward_plus_supported",
-    "pa_layer_forward_plus_workspace_bytes", "pa_layer_forward_plus",
+    "pa_layer_forward_plus_workspace_bytes", "pa_layer_forward_plus", "pa_flare_forward_mfma_supported",
+    "pa_flare_forward_mfma_workspace_bytes", "pa_flare_forward_mfma",
     "pa_mfma_backward_query", "pa_rows_gemm_packed", "pa_mfma_slice_weighted_sum", "pa_mfma_deslice",
     "pa_mfma_backward_tables_bytes", "pa_mfma_backward_groups", "pa_mfma_slice_softmax_backward",
     "pa_cols_gemm_chunks", "pa_cols_gemm", "pa_residual_layernorm",
@@ -159,6 +160,12 @@ def load() -> ctypes.CDLL:
     lib.pa_flare_backward_points.argtypes = [c_int, ps] + [c_void_p] * 10
     lib.pa_deslice.restype = c_int
     lib.pa_deslice.argtypes = [c_int, ps] + [c_void_p] * 4
+    lib.pa_flare_forward_mfma_supported.restype = c_int
+    lib.pa_flare_forward_mfma_supported.argtypes = [ps]
+    lib.pa_flare_forward_mfma_workspace_bytes.restype = c_int64
+    lib.pa_flare_forward_mfma_workspace_bytes.argtypes = [ps]
+    lib.pa_flare_forward_mfma.restype = c_int
+    lib.pa_flare_forward_mfma.argtypes = [ps] + [c_void_p] * 8 + [POINTER(PaBlockTail), c_void_p, c_int64, c_void_p]
     lib.pa_layer_forward_plus_supported.restype = c_int
     lib.pa_layer_forward_plus_supported.argtypes = [c_int, ps]
     lib.pa_layer_forward_plus_workspace_bytes.restype = c_int64

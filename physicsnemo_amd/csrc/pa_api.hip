@@ -886,6 +886,117 @@ int pa_layer_forward(int dtype, const pa_shape *shape, const pa_params *p, const
   return rc;
 }
 
+// Workspace plan of the FLARE layer on the MFMA kernels.
+struct FlarePlan {
+  int64_t off_scores, off_v, off_wc, off_wr, off_partials, off_z, off_tokp, off_colmax, off_cmpart, off_out_x, total;
+  int64_t G;
+};
+
+static FlarePlan plan_flare(const pa_shape &s) {
+  FlarePlan p{};
+  p.G = mfma_groups(s, false);
+  const int64_t tiles = s.B * pa::mfma::tiles_per_batch(s);
+  int64_t off = 0;
+  p.off_scores = off;  // later the natural-layout attention output (B, N, H*32)
+  off += round_up(s.B * s.N * s.H * (s.S > 32 ? s.S : 32) * 2, 256);
+  p.off_v = off;
+  off += round_up(tiles * s.H * 2 * 1024, 256);
+  p.off_wc = off;
+  off += round_up(tiles * s.H * (s.S / 16) * 1024, 256);
+  p.off_wr = off;
+  off += round_up(tiles * s.H * (s.S / 16) * 1024, 256);
+  p.off_partials = off;
+  off += round_up((p.G + 1) * s.B * s.H * s.S * (s.D + 1) * 4, 256);
+  p.off_z = off;
+  off += round_up(s.B * s.H * s.S * s.D * 4, 256);
+  p.off_tokp = off;
+  off += round_up(pa::mfma::tokp_bytes(s), 256);
+  p.off_colmax = off;
+  off += round_up(s.B * s.H * s.S * 4, 256);
+  p.off_cmpart = off;
+  off += round_up(pa::flare::column_max_chunks(s) * s.B * s.H * s.S * 4, 256);
+  p.off_out_x = p.off_scores;  // the scores are dead once both weight packs exist
+  p.total = off;
+  return p;
+}
+
+static bool flare_mfma_supported(const pa_shape &s) {
+  return pa::mfma::supported(PA_BF16, s) && s.B * s.N >= 4096;
+}
+
+int pa_flare_forward_mfma_supported(const pa_shape *shape) {
+  if (check_shape(PA_BF16, shape)) return 0;
+  return flare_mfma_supported(*shape) ? 1 : 0;
+}
+
+int64_t pa_flare_forward_mfma_workspace_bytes(const pa_shape *shape) {
+  int rc = check_shape(PA_BF16, shape);
+  if (rc) return rc;
+  if (!flare_mfma_supported(*shape)) return PA_ERR_UNSUPPORTED;
+  return plan_flare(*shape).total;
+}
+
+int pa_flare_forward_mfma(const pa_shape *shape, const void *scores_weight, const float *scores_bias,
+                          const void *values_weight, const float *values_bias, const void *out_linear_weight,
+                          const float *out_linear_bias, const void *x, void *y, const pa_block_tail *tail,
+                          void *workspace, int64_t workspace_bytes, void *stream) {
+  int rc = check_shape(PA_BF16, shape);
+  if (rc) return rc;
+  if (!scores_weight || !values_weight || !out_linear_weight || !x || !y || !workspace) return PA_ERR_NULL;
+  if (!aligned16(scores_weight) || !aligned16(values_weight) || !aligned16(out_linear_weight) || !aligned16(x) ||
+      !aligned16(y) || !aligned16(workspace))
+    return PA_ERR_ALIGN;
+  if ((rc = check_tail(tail))) return rc;
+  const pa_shape &s = *shape;
+  if (!flare_mfma_supported(s)) return PA_ERR_UNSUPPORTED;
+  const FlarePlan fp = plan_flare(s);
+  if (workspace_bytes < fp.total) return PA_ERR_WORKSPACE;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  char *ws = static_cast<char *>(workspace);
+  void *scores = ws + fp.off_scores, *vp = ws + fp.off_v, *wc = ws + fp.off_wc, *wr = ws + fp.off_wr;
+  void *tokp = ws + fp.off_tokp, *out_x = ws + fp.off_out_x;
+  float *partials = reinterpret_cast<float *>(ws + fp.off_partials), *z = reinterpret_cast<float *>(ws + fp.off_z);
+  float *colmax = reinterpret_cast<float *>(ws + fp.off_colmax), *cmpart = reinterpret_cast<float *>(ws + fp.off_cmpart);
+  pa::GemmArgs a{};  // scores A = x . W_a^T + b_a, natural layout (B, N, H*S)
+  a.in = x;
+  a.w[0] = scores_weight;
+  a.bias[0] = scores_bias;
+  a.out[0] = scores;
+  a.M = s.B * s.N;
+  a.N = (int)s.N;
+  a.K = a.C = (int)s.C;
+  a.O = (int)(s.H * s.S);
+  if (!pa::gemm::serves(a, 1, 2)) return PA_ERR_UNSUPPORTED;
+  if ((rc = pa::gemm::launch(a, 1, PA_BF16, st))) return rc;
+  pa::GemmArgs v{};  // values, packed operand layout
+  v.in = x;
+  v.w[0] = values_weight;
+  v.bias[0] = values_bias;
+  v.out_pack[0] = vp;
+  v.M = s.B * s.N;
+  v.N = (int)s.N;
+  v.K = v.C = (int)s.C;
+  v.O = (int)(s.H * 32);
+  v.pack_tpb = (int)pa::mfma::tiles_per_batch(s);
+  v.pack_heads = (int)s.H;
+  if (!pa::gemm::serves(v, 1, 2)) return PA_ERR_UNSUPPORTED;
+  if ((rc = pa::gemm::launch(v, 1, PA_BF16, st))) return rc;
+  if ((rc = pa::flare::column_max(PA_BF16, s, scores, cmpart, colmax, st))) return rc;
+  if ((rc = pa::flare::pack_weights(s, scores, colmax, wc, wr, compute_units(), st))) return rc;
+  if ((rc = pa::mfma::slice_reduce(s, wc, vp, partials, st))) return rc;
+  const float *sums = nullptr;
+  if ((rc = pa::general::combine_partials(s, partials, fp.G, &sums, st))) return rc;
+  if ((rc = pa::flare::normalise(s, sums, z, st))) return rc;
+  if ((rc = pa::gale::pack_tokens(s, z, tokp, st))) return rc;
+  if ((rc = pa::mfma::deslice_natural(s, wr, tokp, out_x, compute_units(), st))) return rc;
+  pa_params po{};
+  po.out_linear_weight = out_linear_weight;
+  po.out_linear_bias = out_linear_bias;
+  if ((rc = pa::general::out_linear(PA_BF16, s, po, out_x, y, st))) return rc;
+  if (tail_active(tail)) rc = pa::general::residual_ln(PA_BF16, s, y, *tail, st);
+  return rc;
+}
+
 int pa_layer_forward_plus_supported(int dtype, const pa_shape *shape) {
   if (check_shape(dtype, shape)) return 0;
   return pa::mfma::staged_supported(dtype, *shape) ? 1 : 0;

@@ -12,6 +12,7 @@
 // fp32 arithmetic, fp32 or bf16 storage, natural layouts.
 #include "pa_common.h"
 #include "pa_host.h"
+#include "pa_mfma_ops.h"
 
 namespace pa {
 namespace flare {
@@ -334,6 +335,150 @@ int backward_points(int dtype, const pa_shape &s, const void *wr, const void *wc
                     const float *z, const float *d_num, const float *d_den, void *d_a, void *d_v, hipStream_t st) {
   return dtype == PA_F32 ? backward_points_t<float>(s, wr, wc, v, g, z, d_num, d_den, d_a, d_v, st)
                          : backward_points_t<bf16>(s, wr, wc, v, g, z, d_num, d_den, d_a, d_v, st);
+}
+
+// ------------------------------------------------------------------------------------------------
+// pack_weights_kernel: both normalisations of the scores in the packed operand layout of the bf16 MFMA slice kernels
+// (what their own softmax kernel writes: wave = head, lanes <-> the tile's points, registers <-> slices), read from
+// the natural-layout scores with 8-byte loads:
+//   wc_pack = exp(A - max_n A)    gather weights   -> slice_reduce_kernel with the packed values gives num | den
+//   wr_pack = softmax_s(A)        hand-back weights -> deslice_natural_kernel with the packed summaries gives y
+// grid (G, B, head groups), one wave per head of the group; rows beyond N get zero weights.
+// ------------------------------------------------------------------------------------------------
+template <int S>
+__global__ __launch_bounds__(512) void pack_weights_kernel(const uint16_t *__restrict__ scores,
+                                                           const float *__restrict__ colmax,
+                                                           mfma::u32x4 *__restrict__ wc_pack,
+                                                           mfma::u32x4 *__restrict__ wr_pack, int64_t N, int tpb, int H) {
+  using mfma::f32x16;
+  using mfma::rowmap;
+  constexpr int ST = (S + 31) / 32, NCH = S / 16;
+  const int tid = threadIdx.x, lane = tid & 63, i = lane & 31, g = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int h = blockIdx.z * (blockDim.x >> 6) + wave;
+  const int b = blockIdx.y;
+  const int HS = H * S;
+  float cm[ST][16];
+#pragma unroll
+  for (int st = 0; st < ST; ++st)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int sl = 32 * st + rowmap(r, g);
+      cm[st][r] = sl < S ? colmax[((int64_t)b * H + h) * S + sl] : 0.f;
+    }
+  for (int t = blockIdx.x; t < tpb; t += gridDim.x) {
+    const int64_t n = (int64_t)t * 32 + i;
+    const bool valid = n < N;
+    const uint16_t *srow = scores + ((int64_t)b * N + (valid ? n : N - 1)) * HS + h * S;
+    f32x16 a[ST];
+#pragma unroll
+    for (int st = 0; st < ST; ++st)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int s0 = 32 * st + 8 * q + 4 * g;  // slices rowmap(4 q .. 4 q + 3, g)
+        if (s0 < S) {
+          const uint2 raw = *reinterpret_cast<const uint2 *>(srow + s0);
+          a[st][4 * q + 0] = __uint_as_float(raw.x << 16);
+          a[st][4 * q + 1] = __uint_as_float(raw.x & 0xffff0000u);
+          a[st][4 * q + 2] = __uint_as_float(raw.y << 16);
+          a[st][4 * q + 3] = __uint_as_float(raw.y & 0xffff0000u);
+        } else {
+#pragma unroll
+          for (int j = 0; j < 4; ++j) a[st][4 * q + j] = -1e30f;  // slices beyond S: weight 0
+        }
+      }
+    const int64_t base = ((((int64_t)b * tpb + t) * H + h) * NCH) * 64 + lane;
+    const float keep = valid ? 1.f : 0.f;
+    float mx = -INFINITY;
+#pragma unroll
+    for (int st = 0; st < ST; ++st) {
+      f32x16 e;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        e[r] = __builtin_amdgcn_exp2f((a[st][r] - cm[st][r]) * kLog2e);
+        mx = fmaxf(mx, a[st][r]);
+      }
+      if (2 * st < NCH) wc_pack[base + (2 * st) * 64] = mfma::pack_half<0>(e, keep);
+      if (2 * st + 1 < NCH) wc_pack[base + (2 * st + 1) * 64] = mfma::pack_half<1>(e, keep);
+    }
+    mx = mfma::half_max(mx);
+    float sum = 0.f;
+#pragma unroll
+    for (int st = 0; st < ST; ++st)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        a[st][r] = __builtin_amdgcn_exp2f((a[st][r] - mx) * kLog2e);
+        sum += a[st][r];
+      }
+    sum = mfma::half_sum(sum);
+    const float inv = valid ? __builtin_amdgcn_rcpf(sum) : 0.f;
+#pragma unroll
+    for (int cq = 0; cq < NCH; ++cq)
+      wr_pack[base + cq * 64] = (cq & 1) ? mfma::pack_half<1>(a[cq >> 1], inv) : mfma::pack_half<0>(a[cq >> 1], inv);
+  }
+}
+
+int pack_weights(const pa_shape &s, const void *scores, const float *colmax, void *wc_pack, void *wr_pack, int num_cu,
+                 hipStream_t st) {
+  const int waves = (int)(s.H < 8 ? s.H : 8);
+  if (s.H % waves != 0 || s.S % 16 != 0) return PA_ERR_UNSUPPORTED;
+  const int groups = (int)(s.H / waves);
+  int64_t gx = (4 * (int64_t)num_cu + s.B * groups - 1) / (s.B * groups);
+  const int64_t tpb = (s.N + 31) / 32;
+  if (gx > tpb) gx = tpb;
+  if (gx < 1) gx = 1;
+  const dim3 grid((unsigned)gx, (unsigned)s.B, (unsigned)groups), block((unsigned)(waves * 64));
+#define PA_LAUNCH_PW(SS)                                                                                       \
+  hipLaunchKernelGGL((pack_weights_kernel<SS>), grid, block, 0, st, static_cast<const uint16_t *>(scores), colmax, \
+                     static_cast<mfma::u32x4 *>(wc_pack), static_cast<mfma::u32x4 *>(wr_pack), s.N, (int)tpb, (int)s.H)
+  switch (s.S) {
+    case 16: PA_LAUNCH_PW(16); break;
+    case 32: PA_LAUNCH_PW(32); break;
+    case 64: PA_LAUNCH_PW(64); break;
+    case 128: PA_LAUNCH_PW(128); break;
+    default: return PA_ERR_UNSUPPORTED;
+  }
+#undef PA_LAUNCH_PW
+  return launch_status();
+}
+
+// z[b,h,s,:] = num / den from the (D + 1)-wide sums of the aggregation (den = the count column)
+__global__ __launch_bounds__(256) void normalise_kernel(const float *__restrict__ sums, float *__restrict__ z,
+                                                        int64_t total, int D) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= total) return;
+  const int64_t row = idx / D;
+  const int d = (int)(idx - row * D);
+  z[idx] = sums[row * (D + 1) + d] / sums[row * (D + 1) + D];
+}
+
+int normalise(const pa_shape &s, const float *sums, float *z, hipStream_t st) {
+  const int64_t total = s.B * s.H * s.S * s.D;
+  hipLaunchKernelGGL(normalise_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, sums, z, total,
+                     (int)s.D);
+  return launch_status();
+}
+
+template <typename T>
+static int column_max_t(const pa_shape &s, const void *a, float *partial, float *colmax, hipStream_t st) {
+  const int HS = (int)(s.H * s.S);
+  const int64_t G = column_max_chunks(s), BHS = s.B * HS;
+  constexpr int UE = 16 / sizeof(T);
+  if (HS % UE == 0 && reinterpret_cast<uintptr_t>(a) % 16 == 0)
+    hipLaunchKernelGGL((column_max_partial_vec_kernel<T>), dim3((unsigned)G, (unsigned)s.B), dim3(256), 0, st,
+                       static_cast<const T *>(a), partial, s.N, HS);
+  else
+    hipLaunchKernelGGL((column_max_partial_kernel<T>), dim3((unsigned)G, (unsigned)s.B), dim3(256), 0, st,
+                       static_cast<const T *>(a), partial, s.N, HS);
+  int rc = launch_status();
+  if (rc) return rc;
+  hipLaunchKernelGGL(column_max_combine_kernel, dim3((unsigned)((BHS + 15) / 16)), dim3(256), 0, st, partial, (int)G,
+                     BHS, colmax);
+  return launch_status();
+}
+
+int column_max(int dtype, const pa_shape &s, const void *a, float *partial, float *colmax, hipStream_t st) {
+  return dtype == PA_F32 ? column_max_t<float>(s, a, partial, colmax, st) : column_max_t<bf16>(s, a, partial, colmax, st);
 }
 
 template <typename T>

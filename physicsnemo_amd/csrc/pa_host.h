@@ -115,6 +115,11 @@ int column_weights(int dtype, const pa_shape &s, const void *a, float *partial, 
                    hipStream_t st);
 // temperature: NULL, or (H) float32 -- the entries are then divided by clamp(temperature[head], 0.5, 5) first
 int softmax_rows(int dtype, const pa_shape &s, void *a, const float *temperature, hipStream_t st);
+int column_max(int dtype, const pa_shape &s, const void *a, float *partial, float *colmax, hipStream_t st);
+// bf16 scores (B,N,H,S) -> exp(A - column max) and softmax_s(A) in the packed layout of the MFMA slice kernels
+int pack_weights(const pa_shape &s, const void *scores, const float *colmax, void *wc_pack, void *wr_pack, int num_cu,
+                 hipStream_t st);
+int normalise(const pa_shape &s, const float *sums, float *z, hipStream_t st);
 int backward_tile_rows(const pa_shape &s);
 int backward_points(int dtype, const pa_shape &s, const void *wr, const void *wc, const void *v, const void *g,
                     const float *z, const float *d_num, const float *d_den, void *d_a, void *d_v, hipStream_t st);

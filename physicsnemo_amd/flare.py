@@ -43,6 +43,7 @@ class FLARE(nn.Module):
         self.out_linear = nn.Linear(inner_dim, dim)
         self.out_dropout = nn.Dropout(dropout)
         self._cache: dict = {}
+        self.use_mfma = True  # bf16 inference on the MFMA kernels where they serve the shape (False: general kernels)
 
     def kernel_params(self, dtype: torch.dtype, device: torch.device) -> dict:
         """The composed GEMM weights (in `dtype`; biases float32) and out_linear, cached per parameter version."""
@@ -77,10 +78,24 @@ class FLARE(nn.Module):
         if fp16:  # float32 inside, as the residual stream of the caller is
             with torch.autocast("cuda", enabled=False):
                 return self.forward_block(x.float(), residual.float(), ln)
+        if (not self._needs_grad(x) and x.is_cuda and self.use_mfma and x.ndim == 3
+                and not (self.training and self.out_dropout.p > 0)):
+            xb = x.to(torch.get_autocast_dtype("cuda")) if torch.is_autocast_enabled("cuda") else x
+            if xb.dtype == torch.bfloat16:
+                xb = xb.contiguous()
+                dims = PF.LayerDims(xb.shape[0], xb.shape[1], xb.shape[2], self.heads, self.dim_head, self.n_global_queries)
+                if xb.shape[2] == self.dim and PF.flare_forward_mfma_supported(xb.dtype, dims):
+                    return PF.flare_forward_mfma(
+                        xb, self.kernel_params(xb.dtype, xb.device), dims, residual=residual.to(xb.dtype).contiguous(),
+                        ln_weight=ln.weight.detach().float().contiguous(), ln_bias=ln.bias.detach().float().contiguous(),
+                        ln_eps=ln.eps)
         y = self.forward(x).contiguous()
         return PF.residual_layernorm(y, residual=residual.to(y.dtype).contiguous(),
                                      ln_weight=ln.weight.detach().float().contiguous(),
                                      ln_bias=ln.bias.detach().float().contiguous(), ln_eps=ln.eps)
+
+    def _needs_grad(self, x: torch.Tensor) -> bool:
+        return torch.is_grad_enabled() and (x.requires_grad or any(p.requires_grad for p in self.parameters()))
 
     def _composed(self, device: torch.device):
         """(scores weight (H*S, C), scores bias, values weight (H*D, C), values bias) as differentiable float32
@@ -124,6 +139,9 @@ class FLARE(nn.Module):
             y = FlareFunction.apply(x, dims, w_a, b_a, w_v, b_v, self.out_linear.weight, self.out_linear.bias)
             return self.out_dropout(y if out_dtype is None else y.to(out_dtype))
         p = self.kernel_params(x.dtype, x.device)
+        if self.use_mfma and PF.flare_forward_mfma_supported(x.dtype, dims):
+            y = PF.flare_forward_mfma(x, p, dims)
+            return self.out_dropout(y if out_dtype is None else y.to(out_dtype))
         scores = PF.rows_gemm(x, p["scores_weight"], p["scores_bias"], dims, C, H * S).view(B, N, H, S)
         values = PF.rows_gemm(x, p["values_weight"], p["values_bias"], dims, C, H * D)
         weights, _ = PF.flare_column_weights(scores, dims)

@@ -579,6 +579,31 @@ def slice_cross_attention_mix(tok, self_out, context, gale_params: dict, dims: L
     return out
 
 
+def flare_forward_mfma_supported(dtype: torch.dtype, dims: LayerDims) -> bool:
+    """True where the whole FLARE layer forward runs on the bf16 MFMA kernels."""
+    return dtype == torch.bfloat16 and bool(_lib.load().pa_flare_forward_mfma_supported(byref(dims.c())))
+
+
+def flare_forward_mfma(x, params, dims: LayerDims, residual=None, ln_weight=None, ln_bias=None, ln_eps=1e-5):
+    """FLARE layer forward on the bf16 MFMA kernels from the composed weights of `FLARE.kernel_params`.  Returns y, or
+    (fx_new, ln_out) with a tail."""
+    _need_cuda(x, residual)
+    lib, shape = _lib.load(), dims.c()
+    nbytes = lib.pa_flare_forward_mfma_workspace_bytes(byref(shape))
+    if nbytes < 0:
+        _lib.check(int(nbytes), "pa_flare_forward_mfma_workspace_bytes")
+    workspace = torch.empty(int(nbytes), dtype=torch.uint8, device=x.device)
+    y = torch.empty(dims.B, dims.N, dims.C, dtype=x.dtype, device=x.device)
+    ln_out = torch.empty_like(y) if ln_weight is not None else None
+    tail = _c_tail(residual, ln_weight, ln_bias, ln_eps, ln_out)
+    _lib.check(lib.pa_flare_forward_mfma(
+        byref(shape), params["scores_weight"].data_ptr(), params["scores_bias"].data_ptr(),
+        params["values_weight"].data_ptr(), params["values_bias"].data_ptr(), params["out_linear_weight"].data_ptr(),
+        params["out_linear_bias"].data_ptr(), x.data_ptr(), y.data_ptr(), byref(tail), workspace.data_ptr(), int(nbytes),
+        _lib.current_stream_ptr(x.device)), "pa_flare_forward_mfma")
+    return y if (residual is None and ln_out is None) else (y, ln_out)
+
+
 def flare_column_weights(scores, dims: LayerDims):
     """FLARE first pass weights: exp(A - max_n A) for the scores A (B,N,H,S); returns (weights like A, column max
     (B,H,S) float32)."""

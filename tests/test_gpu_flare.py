@@ -122,6 +122,39 @@ def test_bf16_flare_gradients():
         assert_rel_l2(got[name], want[name], f"bf16 FLARE grad {name}", tol=5e-2)
 
 
+@pytest.mark.parametrize("dim,heads,S,B,N", [(256, 8, 64, 1, 5000), (128, 4, 16, 3, 1777), (256, 8, 32, 2, 4096),
+                                             (256, 8, 128, 1, 4097), (128, 4, 64, 2, 2500)])
+def test_bf16_flare_on_the_mfma_kernels(dim, heads, S, B, N):
+    """The whole FLARE layer on the bf16 MFMA kernels: against the fp32 oracle and against the general kernels on the
+    same bf16 input; with the block tail."""
+    from physicsnemo_amd import functional as PF
+
+    announce("bf16 FLARE MFMA", dim, heads, S, B, N)
+    torch.manual_seed(S + B)
+    kw = dict(heads=heads, dim_head=32, n_global_queries=S)
+    ref, hip = to.OracleFLARE(dim, **kw).eval(), pn.FLARE(dim, **kw).eval()
+    hip.load_state_dict(ref.state_dict())
+    hip.cuda()
+    x = torch.randn(B, N, dim)
+    xb = x.cuda().bfloat16()
+    assert PF.flare_forward_mfma_supported(torch.bfloat16, PF.LayerDims(B, N, dim, heads, 32, S))
+    with torch.no_grad():
+        want = ref(x)
+        got = hip(xb)
+        hip.use_mfma = False
+        general = hip(xb)
+        hip.use_mfma = True
+        ln = torch.nn.LayerNorm(dim).cuda()
+        res = torch.randn(B, N, dim, device="cuda").bfloat16()
+        fx_new, normed = hip.forward_block(xb, res, ln)
+    assert got.dtype == torch.bfloat16 and torch.isfinite(got.float()).all()
+    assert_rel_l2(got, want, "bf16 FLARE y (MFMA) vs fp32 oracle", tol=1e-2)
+    assert_rel_l2(got, general, "bf16 FLARE y: MFMA vs general kernels", tol=1e-2)
+    tail = got.float() + res.float()
+    assert_rel_l2(fx_new, tail, "fx_new", tol=1e-2)
+    assert_rel_l2(normed, torch.nn.functional.layer_norm(tail, (dim,), ln.weight, ln.bias, ln.eps), "LayerNorm", tol=1e-2)
+
+
 @pytest.mark.parametrize("mode,dim,heads,dim_head,S,B,N,Sc,Dc", [
     ("weighted", 32, 4, 8, 8, 2, 300, 5, 7),
     ("concat_project", 48, 3, 16, 20, 3, 77, 9, 4),
