@@ -852,7 +852,13 @@ int pa_layer_forward(int dtype, const pa_shape *shape, const pa_params *p, const
     a.out_pack[1] = fxp;
     a.M = s.B * s.N;
     a.N = (int)s.N;
-    a.K = a.C = (int)s.C;
+    a.C = (int)s.C;
+    a.gh = (int)s.grid_h;
+    a.gw = (int)s.grid_w;
+    a.gd = (int)s.grid_d;
+    a.ks = (int)s.conv_k;
+    a.w_tap_major = (int)s.conv_tap_major;
+    a.K = s.conv_k > 0 ? (int)(s.conv_k * s.conv_k * (s.grid_d > 0 ? s.conv_k : 1) * s.C) : (int)s.C;
     a.O = (int)(s.H * 32);
     a.pack_tpb = (int)pa::mfma::tiles_per_batch(s);
     a.pack_heads = (int)s.H;
@@ -1040,7 +1046,13 @@ int pa_layer_forward_plus(int dtype, const pa_shape *shape, const pa_params *p, 
   a.out_pack[0] = fxp;
   a.M = s.B * s.N;
   a.N = (int)s.N;
-  a.K = a.C = (int)s.C;
+  a.C = (int)s.C;
+  a.gh = (int)s.grid_h;
+  a.gw = (int)s.grid_w;
+  a.gd = (int)s.grid_d;
+  a.ks = (int)s.conv_k;
+  a.w_tap_major = (int)s.conv_tap_major;
+  a.K = s.conv_k > 0 ? (int)(s.conv_k * s.conv_k * (s.grid_d > 0 ? s.conv_k : 1) * s.C) : (int)s.C;
   a.O = (int)(s.H * 32);
   a.pack_tpb = (int)pa::mfma::tiles_per_batch(s);
   a.pack_heads = (int)s.H;

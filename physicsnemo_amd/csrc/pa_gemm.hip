@@ -82,9 +82,9 @@ __global__ __launch_bounds__(256) void rows_gemm_mfma_kernel(GemmArgs a) {
     const int64_t m = m0 + r0 + 32 * p;
     arow[p] = real_row(m);
     ci[p] = cj[p] = cl[p] = 0;
-    if (a.ks > 0 && m < a.M) {  // convolutions never use the padded numbering
-      const int64_t b = m / a.N;
-      int n = (int)(m - b * a.N);
+    if (a.ks > 0 && arow[p] >= 0) {  // grid coordinates from the real row (the padded numbering skips rows)
+      const int64_t b = arow[p] / a.N;
+      int n = (int)(arow[p] - b * a.N);
       cl[p] = n % gd;
       n /= gd;
       ci[p] = n / a.gw;

@@ -208,7 +208,9 @@ __global__ __launch_bounds__(512) void slice_softmax_pack_plus_kernel(
 
 // shapes of the staged path: what the fused kernels serve plus C = 512, large enough for the row kernels to pay off
 bool staged_supported(int dtype, const pa_shape &s) {
-  if (dtype != PA_BF16 || s.conv_k != 0 || s.D != 32 || s.C != s.H * 32) return false;
+  // grid convolutions as projections: the implicit-GEMM kernel writes the same two layouts (tap-major weights)
+  if (s.conv_k != 0 && (s.conv_tap_major != 1 || s.C % 8 != 0)) return false;
+  if (dtype != PA_BF16 || s.D != 32 || s.C != s.H * 32) return false;
   if (s.C != 128 && s.C != 256 && s.C != 512) return false;
   if (s.S != 16 && s.S != 32 && s.S != 64 && s.S != 128) return false;
   if ((s.N + 31) / 32 * s.B > ((int64_t)1 << 31) / 16 || s.B > 65535) return false;

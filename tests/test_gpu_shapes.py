@@ -5,6 +5,9 @@ temperature sums 1e-1)."""
 import pytest
 import torch
 
+from oracle import torch_oracle as to
+import physicsnemo_amd as pn
+from physicsnemo_amd import functional as PF
 from gpu_util import announce, assert_fp32_close, assert_rel_l2, make_pair
 
 pytestmark = pytest.mark.gpu
@@ -71,3 +74,52 @@ def test_backward_refuses_slice_tables_beyond_lds_with_a_clear_error():
         assert_fp32_close(hip(x.cuda()), ref(x), "forward y")
     with pytest.raises(RuntimeError, match="backward kernels do not serve this shape"):
         hip(x.cuda().requires_grad_())
+
+
+@pytest.mark.parametrize("variant,grid,kernel,dim,heads,S,B", [
+    ("structured2d", (64, 64), 3, 128, 4, 32, 1),
+    ("structured2d", (48, 50), 5, 256, 8, 64, 2),
+    ("structured3d", (16, 16, 16), 3, 256, 8, 64, 1),
+    ("structured3d", (12, 10, 9), 3, 128, 4, 16, 4),
+])
+def test_bf16_structured_layers_on_the_staged_mfma_kernels(variant, grid, kernel, dim, heads, S, B):
+    """Grid-convolution projections feeding the staged bf16 MFMA kernels (the implicit-GEMM kernel writes x_mid in
+    natural layout and fx_mid in the packed operand layout), against the fp32 oracle; with the block tail."""
+    announce("bf16 structured staged MFMA", variant, grid, kernel, dim, heads, S, B)
+    ref, hip = make_pair(variant, dim, heads, 32, S, spatial=grid, kernel=kernel, seed=S)
+    n = 1
+    for g in grid:
+        n *= g
+    x = torch.randn(B, n, dim)
+    xb = x.cuda().bfloat16()
+    assert PF.query_path(torch.bfloat16, hip.layer_dims(xb)) == 2
+    with torch.no_grad():
+        want = ref(x)
+        got = hip(xb)
+        ln = torch.nn.LayerNorm(dim).cuda()
+        res = torch.randn(B, n, dim, device="cuda").bfloat16()
+        fx_new, normed = hip.forward_block(xb, res, ln)
+    assert got.dtype == torch.bfloat16
+    assert_rel_l2(got, want, "bf16 structured y vs fp32 oracle", tol=1e-2)
+    tail = got.float() + res.float()
+    assert_rel_l2(fx_new, tail, "fx_new", tol=1e-2)
+    assert_rel_l2(normed, torch.nn.functional.layer_norm(tail, (dim,), ln.weight, ln.bias, ln.eps), "LayerNorm", tol=1e-2)
+
+
+def test_bf16_structured_plus_layer_on_the_staged_mfma_kernels():
+    announce("bf16 structured plus staged MFMA")
+    torch.manual_seed(0)
+    grid, dim, heads, S = (64, 64), 128, 4, 32
+    ref = to.OraclePhysicsAttentionStructuredMesh2D(dim, grid, heads=heads, dim_head=32, slice_num=S, kernel=3, plus=True)
+    hip = pn.PhysicsAttentionStructuredMesh2D(dim, grid, heads=heads, dim_head=32, slice_num=S, kernel=3, plus=True,
+                                              use_te=False)
+    hip.load_state_dict(ref.state_dict())
+    ref.eval(), hip.eval().cuda()
+    x = torch.randn(1, 4096, dim)
+    u = torch.rand(1, 4096, heads, S).bfloat16()
+    xb = x.cuda().bfloat16()
+    assert PF.layer_forward_plus_supported(torch.bfloat16, hip.layer_dims(xb))
+    with torch.no_grad():
+        want = ref.forward_with_noise(x, u.float())
+        got = hip.forward_with_noise(xb, u.cuda())
+    assert_rel_l2(got, want, "bf16 structured plus y vs fp32 oracle", tol=2e-2)
