@@ -77,6 +77,8 @@ def run_in(fn):
     of load to settle: the first twenty calls of the layer run up to 35 % longer than the rest)."""
     import torch
 
+    fn()  # the first call may carry one-time set-up (parameter repacking, library initialisation): not part of the run-in
+    torch.cuda.synchronize()
     t_end = time.perf_counter() + SETTLE_MS * 1e-3
     while time.perf_counter() < t_end:
         fn()
