@@ -270,6 +270,17 @@ def time_variants(points, C, S, reps=5):
         entry(f"GeoTransolver bf16, 4 GALE blocks, hidden {C}, S={S}, geometry {pts // 4} points", pts,
               timed(lambda: geo(ge, None, gl, gg), 3))
     del ge, gg, gl, geo
+    # whole models of the two variants, 4 layers, bf16 autocast: blocks chained through the same kernels
+    for label, model in (("FLARE model", pn.FLAREModel(functional_dim=8, out_dim=4, embedding_dim=3, n_layers=4, n_hidden=C,
+                                                       n_head=H, slice_num=S, use_te=False)),
+                         ("Transolver++ model", pn.Transolver(functional_dim=8, out_dim=4, embedding_dim=3, n_layers=4,
+                                                              n_hidden=C, n_head=H, slice_num=S, plus=True,
+                                                              use_te=False))):
+        model = model.cuda().eval()
+        mf, me = torch.randn(1, pts, 8, device="cuda"), torch.randn(1, pts, 3, device="cuda")
+        with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
+            entry(f"{label} bf16, 4 layers, hidden {C}, S={S}", pts, timed(lambda: model(mf, me), 3))
+        del model, mf, me
     # ball query of the GeoTransolver local features: 8 nearest within a radius that holds about 8 points
     from physicsnemo_amd import functional as PF
     cloud, probes = torch.rand(1, pts, 3, device="cuda"), torch.rand(1, pts, 3, device="cuda")
