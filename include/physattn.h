@@ -302,7 +302,9 @@ int pa_flare_softmax_rows(int dtype, const pa_shape *shape, void *scores, void *
  * column maxima, one kernel that writes both normalisations of the scores as packed operands, the MFMA aggregation and
  * deslice kernels of the PhysicsAttention layer, out_linear (+ optional residual / LayerNorm tail).  bf16, D = 32,
  * C = H*32 in {128, 256}, S in {16, 32, 64, 128}, B*N >= 4096 (pa_flare_forward_mfma_supported() == 1).
- * scores_weight (H*S, C) bf16, values_weight (H*32, C) bf16, out_linear_weight (C, H*32) bf16, biases float32. */
+ * scores_weight (H*S, C) bf16, values_weight (H*32, C) bf16, out_linear_weight (C, H*32) bf16, biases float32.
+ * out_linear_weight NULL (tail NULL as well): y receives the attention output (B, N, H*32) itself, for callers that
+ * blend it with something else before the output projection (GALE_FA, gale.py:735-760). */
 int pa_flare_forward_mfma_supported(const pa_shape *shape);
 int64_t pa_flare_forward_mfma_workspace_bytes(const pa_shape *shape);
 int pa_flare_forward_mfma(const pa_shape *shape, const void *scores_weight, const float *scores_bias,

@@ -948,11 +948,12 @@ int pa_flare_forward_mfma(const pa_shape *shape, const void *scores_weight, cons
                           void *workspace, int64_t workspace_bytes, void *stream) {
   int rc = check_shape(PA_BF16, shape);
   if (rc) return rc;
-  if (!scores_weight || !values_weight || !out_linear_weight || !x || !y || !workspace) return PA_ERR_NULL;
+  if (!scores_weight || !values_weight || !x || !y || !workspace) return PA_ERR_NULL;
   if (!aligned16(scores_weight) || !aligned16(values_weight) || !aligned16(out_linear_weight) || !aligned16(x) ||
       !aligned16(y) || !aligned16(workspace))
     return PA_ERR_ALIGN;
   if ((rc = check_tail(tail))) return rc;
+  if (!out_linear_weight && tail_active(tail)) return PA_ERR_UNSUPPORTED;  // the tail follows out_linear
   const pa_shape &s = *shape;
   if (!flare_mfma_supported(s)) return PA_ERR_UNSUPPORTED;
   const FlarePlan fp = plan_flare(s);
@@ -960,7 +961,7 @@ int pa_flare_forward_mfma(const pa_shape *shape, const void *scores_weight, cons
   hipStream_t st = static_cast<hipStream_t>(stream);
   char *ws = static_cast<char *>(workspace);
   void *scores = ws + fp.off_scores, *vp = ws + fp.off_v, *wc = ws + fp.off_wc, *wr = ws + fp.off_wr;
-  void *tokp = ws + fp.off_tokp, *out_x = ws + fp.off_out_x;
+  void *tokp = ws + fp.off_tokp, *out_x = out_linear_weight ? ws + fp.off_out_x : y;  // no out_linear: y is out_x
   float *partials = reinterpret_cast<float *>(ws + fp.off_partials), *z = reinterpret_cast<float *>(ws + fp.off_z);
   float *colmax = reinterpret_cast<float *>(ws + fp.off_colmax), *cmpart = reinterpret_cast<float *>(ws + fp.off_cmpart);
   pa::GemmArgs a{};  // scores A = x . W_a^T + b_a, natural layout (B, N, H*S)
@@ -995,6 +996,7 @@ int pa_flare_forward_mfma(const pa_shape *shape, const void *scores_weight, cons
   if ((rc = pa::flare::normalise(s, sums, z, st))) return rc;
   if ((rc = pa::gale::pack_tokens(s, z, tokp, st))) return rc;
   if ((rc = pa::mfma::deslice_natural(s, wr, tokp, out_x, compute_units(), st))) return rc;
+  if (!out_linear_weight) return PA_OK;
   pa_params po{};
   po.out_linear_weight = out_linear_weight;
   po.out_linear_bias = out_linear_bias;

@@ -295,7 +295,10 @@ class GALE_FA(nn.Module):
                 outs.append(self.out_dropout(self._forward_one_with_grad(t, context, dims)))
                 continue
             p = self.kernel_params(t.dtype, t.device)
-            y = self._self_attention(t, p, dims)
+            if PF.flare_forward_mfma_supported(t.dtype, dims):
+                y = PF.flare_forward_mfma(t, p, dims, project=False)  # bf16: the self-attention on the MFMA kernels
+            else:
+                y = self._self_attention(t, p, dims)
             if context is not None:
                 y = self._mix(y, self._cross_attention(t, context.to(t.device), dims), dims)
             out = PF.rows_gemm(y, p["out_linear_weight"].view(C, -1), p["out_linear_bias"],

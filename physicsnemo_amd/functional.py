@@ -584,22 +584,25 @@ def flare_forward_mfma_supported(dtype: torch.dtype, dims: LayerDims) -> bool:
     return dtype == torch.bfloat16 and bool(_lib.load().pa_flare_forward_mfma_supported(byref(dims.c())))
 
 
-def flare_forward_mfma(x, params, dims: LayerDims, residual=None, ln_weight=None, ln_bias=None, ln_eps=1e-5):
+def flare_forward_mfma(x, params, dims: LayerDims, residual=None, ln_weight=None, ln_bias=None, ln_eps=1e-5,
+                       project: bool = True):
     """FLARE layer forward on the bf16 MFMA kernels from the composed weights of `FLARE.kernel_params`.  Returns y, or
-    (fx_new, ln_out) with a tail."""
+    (fx_new, ln_out) with a tail; `project=False`: the attention output (B, N, H*32) before out_linear."""
     _need_cuda(x, residual)
     lib, shape = _lib.load(), dims.c()
     nbytes = lib.pa_flare_forward_mfma_workspace_bytes(byref(shape))
     if nbytes < 0:
         _lib.check(int(nbytes), "pa_flare_forward_mfma_workspace_bytes")
     workspace = torch.empty(int(nbytes), dtype=torch.uint8, device=x.device)
-    y = torch.empty(dims.B, dims.N, dims.C, dtype=x.dtype, device=x.device)
+    y = torch.empty(dims.B, dims.N, dims.C if project else dims.H * 32, dtype=x.dtype, device=x.device)
     ln_out = torch.empty_like(y) if ln_weight is not None else None
     tail = _c_tail(residual, ln_weight, ln_bias, ln_eps, ln_out)
     _lib.check(lib.pa_flare_forward_mfma(
         byref(shape), params["scores_weight"].data_ptr(), params["scores_bias"].data_ptr(),
-        params["values_weight"].data_ptr(), params["values_bias"].data_ptr(), params["out_linear_weight"].data_ptr(),
-        params["out_linear_bias"].data_ptr(), x.data_ptr(), y.data_ptr(), byref(tail), workspace.data_ptr(), int(nbytes),
+        params["values_weight"].data_ptr(), params["values_bias"].data_ptr(),
+        params["out_linear_weight"].data_ptr() if project else None,
+        params["out_linear_bias"].data_ptr() if project else None, x.data_ptr(), y.data_ptr(), byref(tail),
+        workspace.data_ptr(), int(nbytes),
         _lib.current_stream_ptr(x.device)), "pa_flare_forward_mfma")
     return y if (residual is None and ln_out is None) else (y, ln_out)
 
