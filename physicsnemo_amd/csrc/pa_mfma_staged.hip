@@ -92,14 +92,6 @@ __global__ __launch_bounds__(512) void slice_softmax_pack_kernel(const uint16_t 
 //   w        = softmax_s((logits[s] - log(-log(u[s] + 1e-8) + 1e-8)) / temp)             u: the caller's U[0,1) samples
 // `uniform` (B, N, H, S) bf16 in natural layout: a lane reads its slices (runs of four) with 8-byte loads.
 // ------------------------------------------------------------------------------------------------
-__device__ __forceinline__ float gelu_logistic(float x) {
-  // x Phi(x), Phi in the logistic form 1 / (1 + exp(-2 x P(x^2))), P fitted to the erf form (max |error| 2.6e-5)
-  const float x2 = fminf(x * x, 81.f);
-  float p = fmaf(-3.51902394e-04f * -2.f * kLog2e, x2, 3.70080200e-02f * -2.f * kLog2e);
-  p = fmaf(p, x2, 7.97505275e-01f * -2.f * kLog2e);
-  return x * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(x * p));
-}
-
 template <int S>
 __global__ __launch_bounds__(512) void slice_softmax_pack_plus_kernel(
     const uint16_t *__restrict__ x_mid, const uint16_t *__restrict__ uniform, const float *__restrict__ w_slice,

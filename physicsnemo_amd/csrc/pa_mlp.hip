@@ -91,16 +91,7 @@ __device__ __forceinline__ void static_for(F &&f) {
   static_for_impl(f, std::make_integer_sequence<int, N>{});
 }
 
-// GELU(x) = x * Phi(x), Phi in the logistic form 1 / (1 + exp(-2 x P(x^2))) with P fitted to the exact erf form:
-// max |error| 2.6e-5 over all x (the plain tanh form has 4.7e-4); |x| is clamped where Phi is 0 or 1 in fp32.
-__device__ __forceinline__ float gelu(float x) {
-  const float x2 = fminf(x * x, 81.f);  // beyond |x| = 9 Phi is 0 or 1 in fp32; keeps x P(x^2) monotone
-  // -2 * log2(e) * (c0 + c1 x^2 + c2 x^4)
-  float p = fmaf(-3.51902394e-04f * -2.f * kLog2e, x2, 3.70080200e-02f * -2.f * kLog2e);
-  p = fmaf(p, x2, 7.97505275e-01f * -2.f * kLog2e);
-  const float e = __builtin_amdgcn_exp2f(x * p);
-  return x * __builtin_amdgcn_rcpf(1.f + e);
-}
+__device__ __forceinline__ float gelu(float x) { return gelu_logistic(x); }
 
 // 8 floats -> 8 bf16 (round to nearest even)
 __device__ __forceinline__ u32x4 pack8(const float (&v)[8]) {
