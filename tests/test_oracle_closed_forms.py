@@ -398,7 +398,7 @@ def test_state_dict_keys_and_shapes_match_reference_contract():
 
 def test_mlp_kernel_gelu_constants_against_exact_erf():
     """The fused MLP kernel evaluates GELU as x / (1 + exp2(x * P(min(x^2, 81)))) with the three constants found in
-    physicsnemo_amd/csrc/pa_mlp.hip.  Evaluate that form (float32, constants parsed from the source) against the
+    physicsnemo_amd/csrc/pa_common.h (gelu_logistic).  Evaluate that form (float32, constants parsed from the source) against the
     exact erf form on a dense grid: a wrong or mistyped constant moves the error far above the bound."""
     import math
     import os
@@ -406,8 +406,8 @@ def test_mlp_kernel_gelu_constants_against_exact_erf():
 
     import numpy as np
 
-    src = open(os.path.join(os.path.dirname(__file__), "..", "physicsnemo_amd", "csrc", "pa_mlp.hip")).read()
-    body = src[src.index("__device__ __forceinline__ float gelu(float x)"):]
+    src = open(os.path.join(os.path.dirname(__file__), "..", "physicsnemo_amd", "csrc", "pa_common.h")).read()
+    body = src[src.index("__device__ __forceinline__ float gelu_logistic(float x)"):]
     body = body[:body.index("}")]
     consts = [float(c) for c in re.findall(r"(-?\d\.\d+e-?\d+)f \* -2\.f \* kLog2e", body)]
     assert len(consts) == 3, consts
