@@ -136,8 +136,8 @@ __global__ __launch_bounds__(512) void slice_softmax_pack_plus_kernel(
     const u32x4 xm0 = *reinterpret_cast<const u32x4 *>(row), xm1 = *reinterpret_cast<const u32x4 *>(row + 16);
     // the point's temperature
     float a2 = 0.f;
-#pragma unroll
-    for (int st = 0; st < ST; ++st) {
+#pragma unroll 1
+    for (int st = 0; st < ST; ++st) {  // not unrolled: the tile's registers are free again before the logits are formed
       f32x16 hd;
 #pragma unroll
       for (int r = 0; r < 16; ++r) hd[r] = b1l[32 * st + rowmap(r, g)];
