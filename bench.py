@@ -118,7 +118,6 @@ def cpu_baseline(state_dict, x_cpu_f32, C, H, S, target_seconds):
         per_point = (time.perf_counter() - t0) / probe
         # 2 warm-ups + 5 timed runs within the budget
         n = int(min(n_total, max(probe, target_seconds / 7.0 / per_point)))
-        n = min(n, 262144)
         xs = x_cpu_f32[:, :n].contiguous()
         for _ in range(2):
             ref(xs)
