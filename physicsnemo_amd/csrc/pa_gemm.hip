@@ -549,6 +549,119 @@ int cols_gemm_f32(const void *A, int64_t lda, int64_t OA, const void *B, int64_t
   return launch_status();
 }
 
+// ------------------------------------------------------------------------------------------------
+// cols_gemm_lds_kernel: the same product with the transposition done by the LDS read pattern instead of on the
+// matrix cores.  A workgroup (8 waves, 4 along A's columns x 2 along B's) owns a 256 x 256 block of P for its chunk
+// of rows; 32 rows of both operands at a time are staged in LDS as they lie in memory (16-byte loads; row stride 260
+// elements, so that the two half-waves, eight rows apart, fall on different banks), and a lane gathers its operand
+// -- eight consecutive rows m of one column -- with eight 2-byte LDS reads.  Wave tile 64 x 128: 6 operand fragments
+// feed 8 MFMAs.  grid (G row chunks, ceil(OA / 256)); OB <= 256.
+// ------------------------------------------------------------------------------------------------
+constexpr int kColsLd = 260;
+
+__global__ __launch_bounds__(512) void cols_gemm_lds_kernel(const uint16_t *__restrict__ A, int lda, int OA,
+                                                            const uint16_t *__restrict__ B, int ldb, int OB, int64_t M,
+                                                            int64_t per, float *__restrict__ partials,
+                                                            float *__restrict__ col_sums) {
+  __shared__ uint16_t As[2][32 * kColsLd];
+  __shared__ uint16_t Bs[2][32 * kColsLd];
+  const int t = threadIdx.x, lane = t & 63, i = lane & 31, g = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+  const int wa = (wave & 3) * 64, wb = (wave >> 2) * 128;
+  const int oa0 = blockIdx.y * 256;
+  const int64_t blk0 = (int64_t)blockIdx.x * per, nblk = (M + 31) / 32;
+  const int64_t blk1 = blk0 + per < nblk ? blk0 + per : nblk;
+
+  f32x16 acc[2][4];
+#pragma unroll
+  for (int u = 0; u < 2; ++u)
+#pragma unroll
+    for (int v = 0; v < 4; ++v)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[u][v][r] = 0.f;
+  float csum[2] = {0.f, 0.f};
+
+  // staging: 32 rows x 32 units of 8 columns per operand = 1024 units, two per thread
+  const int sr = t >> 5, su = (t & 31) * 8;  // row (and row + 16), first column of the unit
+  u32x4 pa[2], pb[2];
+  auto fetch = [&](int64_t blk) {
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+      const int64_t m = blk * 32 + sr + 16 * k;
+      pa[k] = pb[k] = u32x4{0, 0, 0, 0};
+      if (m < M) {
+        if (oa0 + su < OA) pa[k] = *reinterpret_cast<const u32x4 *>(A + m * lda + oa0 + su);
+        if (su < OB) pb[k] = *reinterpret_cast<const u32x4 *>(B + m * ldb + su);
+      }
+    }
+  };
+  auto stage = [&](int buf) {
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+      // 8-byte aligned halves: the row stride is a multiple of four elements, not of eight
+      uint2 *da = reinterpret_cast<uint2 *>(&As[buf][(sr + 16 * k) * kColsLd + su]);
+      uint2 *db = reinterpret_cast<uint2 *>(&Bs[buf][(sr + 16 * k) * kColsLd + su]);
+      da[0] = uint2{pa[k][0], pa[k][1]};
+      da[1] = uint2{pa[k][2], pa[k][3]};
+      db[0] = uint2{pb[k][0], pb[k][1]};
+      db[1] = uint2{pb[k][2], pb[k][3]};
+    }
+  };
+  auto gather = [&](const uint16_t *base) {  // rows 0..7 of one column -> an MFMA operand
+    u32x4 f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      f[j] = (uint32_t)base[(2 * j) * kColsLd] | ((uint32_t)base[(2 * j + 1) * kColsLd] << 16);
+    return f;
+  };
+  if (blk0 < blk1) fetch(blk0);
+  int buf = 0;
+  for (int64_t blk = blk0; blk < blk1; ++blk) {
+    stage(buf);
+    __syncthreads();
+    if (blk + 1 < blk1) fetch(blk + 1);
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      const uint16_t *ar = &As[buf][(16 * ks + 8 * g) * kColsLd + wa + i];
+      const uint16_t *br = &Bs[buf][(16 * ks + 8 * g) * kColsLd + wb + i];
+      u32x4 af[2], bf[4];
+#pragma unroll
+      for (int u = 0; u < 2; ++u) af[u] = gather(ar + 32 * u);
+#pragma unroll
+      for (int v = 0; v < 4; ++v) bf[v] = gather(br + 32 * v);
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+#pragma unroll
+        for (int v = 0; v < 4; ++v) acc[u][v] = mfma::mma(af[u], bf[v], acc[u][v]);
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          csum[u] += __uint_as_float(af[u][j] << 16) + __uint_as_float(af[u][j] & 0xffff0000u);
+      }
+    }
+    buf ^= 1;
+  }
+  float *dst = partials + (int64_t)blockIdx.x * OA * OB;
+#pragma unroll
+  for (int u = 0; u < 2; ++u)
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      const int ob = wb + 32 * v + i;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int oa = oa0 + wa + 32 * u + mfma::rowmap(r, g);
+        if (oa < OA && ob < OB) dst[(int64_t)oa * OB + ob] = acc[u][v][r];
+      }
+    }
+  if (col_sums && (wave >> 2) == 0) {
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const float total = csum[u] + __shfl_xor(csum[u], 32, 64);
+      const int oa = oa0 + wa + 32 * u + i;
+      if (g == 0 && oa < OA) col_sums[(int64_t)blockIdx.x * OA + oa] = total;
+    }
+  }
+}
+
 // the partial results stay small next to the rows a chunk reads
 int64_t cols_gemm_chunks(int64_t M, int64_t OA, int num_cu) {
   const int64_t nblk = (M + 31) / 32, gy = (OA + 255) / 256;
@@ -566,6 +679,11 @@ int cols_gemm(const void *A, int64_t lda, int64_t OA, const void *B, int64_t ldb
   const int64_t per = (nblk + G - 1) / G;
   const dim3 grid((unsigned)G, (unsigned)((OA + 255) / 256)), block((unsigned)((OA < 256 ? OA : 256) * 2));
   const uint16_t *a = static_cast<const uint16_t *>(A), *b = static_cast<const uint16_t *>(B);
+  if (OA >= 128 && OB >= 128 && OB <= 256) {  // wide products: the LDS-gather kernel (its 256 x 256 tile would idle on narrow ones)
+    hipLaunchKernelGGL(cols_gemm_lds_kernel, dim3((unsigned)G, (unsigned)((OA + 255) / 256)), dim3(512), 0, st, a,
+                       (int)lda, (int)OA, b, (int)ldb, (int)OB, M, per, partials, col_sums);
+    return launch_status();
+  }
 #define PA_COLS(NBV) \
   hipLaunchKernelGGL((cols_gemm_kernel<NBV>), grid, block, 0, st, a, (int)lda, (int)OA, b, (int)ldb, M, per, partials, col_sums)
   switch (OB / 32) {
