@@ -46,6 +46,7 @@ extern "C" {
 #define PA_ERR_UNSUPPORTED (-3) /* shape/dtype outside what the kernels serve */
 #define PA_ERR_ALIGN (-4)       /* a pointer is not 16-byte aligned */
 #define PA_ERR_WORKSPACE (-5)   /* workspace too small */
+#define PA_ERR_SCRATCH (-6)     /* the problem needs more than PA_STATIC_SCRATCH_BYTES of the library's static scratch */
 
 /* Limits of the general kernels (PA_ERR_UNSUPPORTED beyond them). */
 #define PA_MAX_D 128
@@ -151,6 +152,18 @@ int pa_slice_softmax_plus(int dtype, const pa_shape *shape, const pa_params *p, 
 int64_t pa_reduce_partial_count(const pa_shape *shape);
 int pa_slice_reduce(int dtype, const pa_shape *shape, const void *w, const void *fx_mid, float *partials,
                     float *slice_token, float *slice_norm, void *stream);
+
+/* Stage (b) without any device allocation and without a workspace argument.  No counterpart in the reference: it is
+ * for callers that cannot allocate device memory -- code under HIP graph capture, tight serving loops, harnesses
+ * that forbid hipMalloc.  Same kernels, same arguments and bit-identical results as pa_slice_reduce; the per-chunk
+ * partial sums live in a static device array of PA_STATIC_SCRATCH_BYTES that every GPU the library runs on holds
+ * until the process ends.  PA_ERR_SCRATCH if pa_reduce_partial_count(shape) * B*H*S*(D+1) * 4 bytes exceed it.
+ * Calls on one GPU share that GPU's array: calls that overlap in time on the same GPU race on it (calls on one
+ * stream, or otherwise ordered, are safe).  Only `shape`'s B, N, H, D, S are read. */
+#define PA_STATIC_SCRATCH_BYTES (64ll << 20)
+int64_t pa_static_scratch_bytes(void);
+int pa_slice_reduce_static(int dtype, const pa_shape *shape, const void *w, const void *fx_mid, float *slice_token,
+                           float *slice_norm, void *stream);
 
 /* Stage (c): self-attention among the S slice tokens of each (batch, head), replaces
  * _compute_slice_attention_sdpa (PA.py:429-465): softmax(q k^T / sqrt(D)) v, float32, LDS resident. */

@@ -32,6 +32,7 @@ EXPORTED = [
     "pa_mfma_backward_tables_bytes", "pa_mfma_backward_groups", "pa_mfma_slice_softmax_backward",
     "pa_cols_gemm_chunks", "pa_cols_gemm", "pa_residual_layernorm",
     "pa_mfma_layer_forward", "pa_rows_gemm_act", "pa_layernorm_backward_groups", "pa_layernorm_backward",
+    "pa_static_scratch_bytes", "pa_slice_reduce_static",
 ]
 
 PA_BUF_BLOB, PA_BUF_FX_PACK, PA_BUF_W_PACK, PA_BUF_PARTIALS, PA_BUF_TOKP = range(5)
@@ -99,6 +100,10 @@ def load() -> ctypes.CDLL:
     lib.pa_reduce_partial_count.argtypes = [ps]
     lib.pa_slice_reduce.restype = c_int
     lib.pa_slice_reduce.argtypes = [c_int, ps, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]
+    lib.pa_static_scratch_bytes.restype = c_int64
+    lib.pa_static_scratch_bytes.argtypes = []
+    lib.pa_slice_reduce_static.restype = c_int
+    lib.pa_slice_reduce_static.argtypes = [c_int, ps, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]
     lib.pa_slice_attention.restype = c_int
     lib.pa_slice_attention.argtypes = [ps, pp, c_void_p, c_void_p, c_void_p]
     lib.pa_deslice_project.restype = c_int

@@ -157,9 +157,12 @@ int64_t body_bytes(int dtype, const pa_shape &s) {
 }
 
 int compute_units() {
+  static int cached[64];  // per device; 0 = not yet asked (racing first calls write the same value)
   int dev = 0, n = 0;
   if (hipGetDevice(&dev) != hipSuccess) return 256;
+  if (dev >= 0 && dev < 64 && cached[dev] > 0) return cached[dev];
   if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) return 256;
+  if (dev >= 0 && dev < 64) cached[dev] = n;
   return n;
 }
 
@@ -216,6 +219,7 @@ const char *pa_status_string(int code) {
     case PA_ERR_UNSUPPORTED: return "shape or dtype outside the supported range";
     case PA_ERR_ALIGN: return "a pointer is not 16-byte aligned";
     case PA_ERR_WORKSPACE: return "workspace too small";
+    case PA_ERR_SCRATCH: return "problem too large for the library's static scratch buffer";
     default: return code > 0 ? "hip error" : "unknown error";
   }
 }

@@ -107,6 +107,20 @@ def slice_reduce(w, fx_mid, dims: LayerDims):
     return tok, norm
 
 
+def slice_reduce_static(w, fx_mid, dims: LayerDims, out=None):
+    """`slice_reduce` through the entry point that allocates nothing: the partial sums live in the library's static
+    device scratch.  `out` = (slice_token, slice_norm) float32 tensors to fill (allocated here when omitted: the
+    library call itself never allocates).  Calls that overlap on one GPU race on the shared scratch."""
+    _need_cuda(w, fx_mid)
+    tok, norm = out if out is not None else (
+        torch.empty(dims.B, dims.H, dims.S, dims.D, dtype=torch.float32, device=w.device),
+        torch.empty(dims.B, dims.H, dims.S, dtype=torch.float32, device=w.device))
+    _lib.check(_lib.load().pa_slice_reduce_static(_lib.dtype_code(w.dtype), byref(dims.c()), w.data_ptr(),
+                                                  fx_mid.data_ptr(), tok.data_ptr(), norm.data_ptr(),
+                                                  _lib.current_stream_ptr(w.device)), "pa_slice_reduce_static")
+    return tok, norm
+
+
 def slice_attention(tok, params, dims: LayerDims):
     _need_cuda(tok)
     lib = _lib.load()
