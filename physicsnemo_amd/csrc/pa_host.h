@@ -18,13 +18,24 @@ inline int launch_status() {
 }
 
 // opt a kernel in to more than the default 48 KiB of dynamic LDS
+// (the attribute is per kernel and per device: remembered for the device it was last set on, so the steady state of a
+// process that stays on one GPU makes no runtime call here)
 template <typename F>
 inline int allow_dynamic_lds(F kernel, size_t bytes) {
   if (bytes > kMaxLdsBytes) return PA_ERR_UNSUPPORTED;
   if (bytes > 48 * 1024) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+    static thread_local const void *last_kernel = nullptr;
+    static thread_local size_t last_bytes = 0;
+    static thread_local int last_dev = -1;
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess) dev = -1;
+    const void *k = reinterpret_cast<const void *>(kernel);
+    if (k == last_kernel && bytes <= last_bytes && dev == last_dev && dev >= 0) return PA_OK;
+    hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
     if (e != hipSuccess) return (int)e;
+    last_kernel = k;
+    last_bytes = bytes;
+    last_dev = dev;
   }
   return PA_OK;
 }

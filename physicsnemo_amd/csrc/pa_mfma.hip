@@ -711,10 +711,10 @@ __global__ __launch_bounds__(C * 2) void deslice_project_kernel(const u32x4 *__r
       for (int k = 0; k < CPL; k += 2) {
         float t0 = ys[row * YS + lane * CPL + k], t1 = ys[row * YS + lane * CPL + k + 1];
         if constexpr (HAS_RES) {
-          // y is rounded to bf16 first, then the sum is rounded (two tensor ops upstream)
+          // the residual is added to the fp32 result: one rounding for the sum instead of one per tensor op
           const uint32_t rv = rcur[rr][k / 2];
-          t0 = (float)(__bf16)t0 + bf16_bits_to_f32((uint16_t)(rv & 0xffffu));
-          t1 = (float)(__bf16)t1 + bf16_bits_to_f32((uint16_t)(rv >> 16));
+          t0 += bf16_bits_to_f32((uint16_t)(rv & 0xffffu));
+          t1 += bf16_bits_to_f32((uint16_t)(rv >> 16));
         }
         const uint16_t o0 = to_bf16_bits(t0), o1 = to_bf16_bits(t1);
         v[k] = bf16_bits_to_f32(o0);

@@ -278,6 +278,7 @@ class GALEBlock(nn.Module):
         self._mlp_cache: dict = {}
 
     # the block MLP (reference mlp_layers.py:101-173) and its kernels are the Transolver block's
+    fp8_weights = False  # the shared MLP helpers read it; GALE blocks are served in bf16 / float32 only
     _mlp_kernel_params = TransolverBlock._mlp_kernel_params
     _mlp_kernel_serves = TransolverBlock._mlp_kernel_serves
     _mlp_with_grad = TransolverBlock._mlp_with_grad

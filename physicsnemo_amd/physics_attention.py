@@ -248,7 +248,9 @@ class PhysicsAttentionBase(nn.Module):
                     xp, u, self.kernel_params(xp.dtype, xp.device), dims, residual=residual.to(xp.dtype).contiguous(),
                     ln_weight=ln.weight.detach().float().contiguous(), ln_bias=ln.bias.detach().float().contiguous(),
                     ln_eps=ln.eps)
-        if self.plus or (self.training and self.out_dropout.p > 0):  # dropout sits between the layer and the residual add
+        # dropout sits between the layer and the residual add; with gradients required the differentiable layer path
+        # runs and the tail is formed by tensor ops, so the result carries a grad_fn
+        if self.plus or (self.training and self.out_dropout.p > 0) or self._needs_grad(x):
             y = self.forward(x)
             fx_new = y + residual.to(y.dtype)
             normed = torch.nn.functional.layer_norm(fx_new.float(), ln.normalized_shape, ln.weight, ln.bias, ln.eps)

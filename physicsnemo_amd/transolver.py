@@ -80,6 +80,8 @@ class PositionalEmbedding(nn.Module):
 class TransolverBlock(nn.Module):
     """LayerNorm -> PhysicsAttention -> +residual -> LayerNorm -> MLP -> +residual [-> LayerNorm -> Linear]."""
 
+    fp8_weights = False  # class default for subclasses with constructors of their own; see use_fp8_weights()
+
     def __init__(self, num_heads: int, hidden_dim: int, dropout: float, act: str = "gelu", mlp_ratio: int = 4,
                  last_layer: bool = False, out_dim: int = 1, slice_num: int = 32,
                  spatial_shape: tuple[int, ...] | None = None, use_te: bool = True, plus: bool = False):
@@ -101,19 +103,35 @@ class TransolverBlock(nn.Module):
         if last_layer:
             self.ln_mlp2 = nn.Sequential(nn.LayerNorm(hidden_dim), nn.Linear(hidden_dim, out_dim))
         self._mlp_cache: dict = {}
+        self.fp8_weights = False  # see use_fp8_weights()
+
+    def use_fp8_weights(self, enabled: bool = True):
+        """Inference with the block's large weights held as fp8-e4m3 with one scale per output channel
+        (scale = max|row| / 448): the attention layer's three projections (`PhysicsAttentionBase.use_fp8_weights`)
+        and the two Linears of the MLP.  The kernels expand them to bf16 operands; activations stay bf16.  No
+        counterpart in the reference."""
+        self.Attn.use_fp8_weights(enabled)
+        self.fp8_weights = bool(enabled)
+        self._mlp_cache = {}
+        return self
 
     # ---------------------------------------------------------------- fused MLP (pa_mlp_forward)
     def _mlp_kernel_params(self, device):
-        """bf16 weights / fp32 biases of ln_mlp1's Mlp for the fused kernel; cached until a parameter changes."""
+        """bf16 weights / fp32 biases of ln_mlp1's Mlp for the fused kernel; cached until a parameter changes.  With
+        fp8 weights enabled the bf16 values are the dequantised e4m3 weights."""
         lin1, lin2 = self.ln_mlp1[1].layers[0], self.ln_mlp1[1].layers[2]
         named = (lin1.weight, lin1.bias, lin2.weight, lin2.bias)
-        stamp = (device,) + tuple((t.data_ptr(), t._version, t.dtype) for t in named)
+        stamp = (device, self.fp8_weights) + tuple((t.data_ptr(), t._version, t.dtype) for t in named)
         if self._mlp_cache.get("stamp") != stamp:
+            def big(w):
+                w = w.detach().to(device=device, dtype=torch.float32)
+                if self.fp8_weights:
+                    w = PF.dequantize_e4m3_per_channel(*PF.quantize_e4m3_per_channel(w))
+                return w.to(torch.bfloat16).contiguous().clone()
+
             with torch.no_grad():
-                params = (lin1.weight.detach().to(device=device, dtype=torch.bfloat16).contiguous().clone(),
-                          lin1.bias.detach().to(device=device, dtype=torch.float32).contiguous().clone(),
-                          lin2.weight.detach().to(device=device, dtype=torch.bfloat16).contiguous().clone(),
-                          lin2.bias.detach().to(device=device, dtype=torch.float32).contiguous().clone())
+                params = (big(lin1.weight), lin1.bias.detach().to(device=device, dtype=torch.float32).contiguous().clone(),
+                          big(lin2.weight), lin2.bias.detach().to(device=device, dtype=torch.float32).contiguous().clone())
             self._mlp_cache = {"stamp": stamp, "params": params}
         return self._mlp_cache["params"]
 
@@ -163,7 +181,12 @@ class TransolverBlock(nn.Module):
                                   ln_weight=next_ln.weight.detach().float().contiguous(),
                                   ln_bias=next_ln.bias.detach().float().contiguous(), ln_eps=next_ln.eps)
         # MLP shapes the fused kernel does not serve: tensor-op MLP, then residual add (+ the next LayerNorm) in one pass
-        h = self.ln_mlp1[1](normed)
+        if self.fp8_weights and normed.is_cuda and normed.dtype == torch.bfloat16:
+            w1, b1, w2, b2 = self._mlp_kernel_params(normed.device)
+            F = torch.nn.functional
+            h = F.linear(self.ln_mlp1[1].layers[1](F.linear(normed, w1, b1.to(normed.dtype))), w2, b2.to(normed.dtype))
+        else:
+            h = self.ln_mlp1[1](normed)
         if h.is_cuda and h.dtype == fx1.dtype and h.dtype in (torch.float32, torch.bfloat16):
             h = h.contiguous()
             if next_ln is None:
@@ -286,6 +309,13 @@ class Transolver(nn.Module):
                        lin.bias.detach().to(device=x.device, dtype=torch.float32).contiguous().clone())
             cache[id(lin)] = hit
         return PF.linear(x, hit[1], hit[2], gelu=gelu)
+
+    def use_fp8_weights(self, enabled: bool = True):
+        """Every block's large weights as fp8-e4m3 with per-output-channel scales (`TransolverBlock.use_fp8_weights`);
+        the preprocess Mlp, the LayerNorms, the slice / qkv projections and the output head stay in higher precision."""
+        for block in self.blocks:
+            block.use_fp8_weights(enabled)
+        return self
 
     def initialize_weights(self) -> None:
         self.apply(self._init_weights)

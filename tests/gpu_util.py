@@ -46,7 +46,12 @@ def assert_fp32_close(got, want, what, rtol=1e-4):
     assert not bool(bad.any()), f"{what}: max err {float(err.max()):.3e} (atol {atol:.3e}), rel-L2 {to.rel_l2(got, want):.3e}"
 
 
-def assert_rel_l2(got, want, what, tol=1e-2):
+def assert_rel_l2(got, want, what, tol=1e-2, report=False):
+    """`report`: also list the measured figure in the terminal summary of the test run."""
     r = to.rel_l2(got.detach().float().cpu(), want.detach().float().cpu())
+    if report:
+        import conftest
+
+        conftest.MEASURED.append((what, r, tol))
     assert r <= tol, f"{what}: rel-L2 {r:.3e} > {tol}"
     return r

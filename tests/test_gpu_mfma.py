@@ -146,10 +146,12 @@ def test_mfma_determinism_and_point_permutation():
     assert_rel_l2(y3, y[:, perm], "outputs follow the permutation", tol=2e-3)
 
 
-def test_mfma_full_size_properties():
-    # headline shape (1,048,576 points, C=256, S=64): size-independent properties instead of an oracle run
-    announce("mfma full size")
-    B, N, C, S = 1, 1 << 20, 256, 64
+@pytest.mark.parametrize("S", [16, 32, 64, 128])
+def test_mfma_full_size_properties(S):
+    # headline shape (1,048,576 points, C=256) over the slice sweep, through the layer call the benchmark times:
+    # size-independent properties instead of an oracle run
+    announce("mfma full size", S)
+    B, N, C = 1, 1 << 20, 256
     H = C // 32
     torch.manual_seed(0)
     hip = pn.PhysicsAttentionIrregularMesh(C, heads=H, dim_head=32, slice_num=S, use_te=False).eval().cuda()
@@ -157,28 +159,62 @@ def test_mfma_full_size_properties():
     xb = torch.randn(B, N, C, generator=g).bfloat16().cuda()
     p = hip.kernel_params(torch.bfloat16, xb.device)
     dims = hip.layer_dims(xb)
+    assert PF.query_path(torch.bfloat16, dims) == 1
+    with torch.no_grad():
+        y, tok = PF.layer_forward(xb, p, dims, return_slice_tokens=True)
+    assert torch.isfinite(y.float()).all()
+    # the same kernels launched one by one (fused (a)+(b) where the layer call fuses them) give the identical result
+    # and expose the slice norms and the attended tokens
     st = PF.MfmaStages(p, dims, xb.device)
-    y = torch.empty_like(xb)
-    st.pack_params(); st.project_softmax(xb); st.slice_reduce(); st.combine_attention(); st.deslice_project(y)
+    y2 = torch.empty_like(xb)
+    st.pack_params()
+    if st.fused_groups > 0:
+        st.project_softmax_reduce(xb)
+    else:
+        st.project_softmax(xb)
+        st.slice_reduce()
+    st.combine_attention()
+    st.deslice_project(y2)
+    assert torch.equal(y2, y) and torch.equal(st.tok, tok)
+    del y2
+    # every point spreads a total weight of one over the slices
     total = (st.norm - 0.01).sum(-1)
     assert torch.allclose(total, torch.full_like(total, float(N)), rtol=2e-3)
-    assert torch.isfinite(y.float()).all()
-    # a 4096-point prefix run through the oracle with the full run's slice tokens: y = deslice(w, tok') for those points
-    sub = xb[:, :4096].float().cpu()
     ref = to.OraclePhysicsAttentionIrregularMesh(C, heads=H, dim_head=32, slice_num=S).eval()
     ref.load_state_dict({k: v.cpu() for k, v in hip.state_dict().items()})
     with torch.no_grad():
+        # slice attention of the oracle on the full run's slice tokens
+        want_tok_out = to.slice_attention(tok.cpu(), ref.qkv_project.weight, 32)
+        assert_rel_l2(st.tok_out, want_tok_out, f"S={S}: attended tokens of the full-size run", tol=1e-4)
+        # a 4096-point prefix through the oracle with the full run's attended tokens: y = deslice(w, tok') there
+        sub = xb[:, :4096].float().cpu()
         xm, _ = ref._project(sub)
         w, _, _ = to.slice_weights_and_tokens(to.slice_logits(xm, ref.in_project_slice.weight, ref.in_project_slice.bias),
                                               torch.zeros(1, 4096, H, 32), ref.temperature)
         want = to.deslice_and_project(w, st.tok_out.cpu(), ref.out_linear.weight, ref.out_linear.bias)
-    assert_rel_l2(y[:, :4096], want, "prefix of the full-size output")
+    assert_rel_l2(y[:, :4096], want, f"S={S}: prefix of the full-size layer output", report=True)
+    # a slice token is a convex combination of fx_mid rows shrunk by (norm - 0.01) / norm, so it lies inside the
+    # per-channel range of fx_mid over all points (widened to contain zero)
+    with torch.no_grad():
+        fx_mid = torch.nn.functional.linear(xb.float(), hip.in_project_fx.weight.float(), hip.in_project_fx.bias.float())
+        lo = fx_mid.amin(1).clamp_max(0).view(B, H, 1, 32).cpu()
+        hi = fx_mid.amax(1).clamp_min(0).view(B, H, 1, 32).cpu()
+        del fx_mid
+    tk = tok.cpu()
+    assert bool(((tk >= lo - 1e-2) & (tk <= hi + 1e-2)).all())
 
 
-@pytest.mark.parametrize("B,N,C,S", [(2, 3000, 256, 64), (1, 2000, 128, 32), (1, 700, 512, 128), (1, 6000, 512, 128)])
-def test_fp8_e4m3_weight_variant(B, N, C, S):
-    # bf16 activations, fp8-e4m3 per-output-channel-scaled projection weights.  The reference for the 1e-2 bar is
-    # the fp32 oracle holding the SAME (dequantised) weights; the error against the unquantised weights is printed.
+# bound = what the number format allows for the shape: e4m3 keeps 3 mantissa bits, and the rounding of the weights
+# ALONE (fp32 oracle with dequantised weights against fp32 oracle with the original ones, listed in the test summary)
+# already costs 0.65e-2 .. 1.2e-2 depending on the shape; the 512-wide layers exceed 1e-2 before any kernel runs.
+@pytest.mark.parametrize("B,N,C,S,bound", [(2, 3000, 256, 64, 1e-2), (1, 2000, 128, 32, 1e-2),
+                                           (1, 700, 512, 128, 1.4e-2), (1, 6000, 512, 128, 1.4e-2)])
+def test_fp8_e4m3_weight_variant(B, N, C, S, bound):
+    # bf16 activations, fp8-e4m3 per-output-channel-scaled projection weights.  Checks: (1) rel-L2 against the fp32
+    # oracle holding the ORIGINAL (unquantised) weights: within `bound`, and never more than the quantisation error of
+    # the weights and the bf16 error of the kernels (4e-3) combined; (2) rel-L2 <= 1e-2 (measured: 2e-3) against the
+    # fp32 oracle holding the dequantised weights, which isolates the kernels from the quantisation error, and
+    # bit-equality with the bf16 path fed those dequantised weights.
     announce("fp8 weights", B, N, C, S)
     H = C // 32
     ref, hip = make_pair("irregular", C, H, 32, S)
@@ -200,6 +236,12 @@ def test_fp8_e4m3_weight_variant(B, N, C, S):
             getattr(hip, name).weight.copy_(deq[name].cuda())
         y16 = hip(xb)
     assert y8.dtype == torch.bfloat16
+    q_err = to.rel_l2(want_q, want_full)
+    import conftest
+
+    conftest.MEASURED.append((f"(oracle only) e4m3 weight rounding alone, C={C} S={S} N={N}", q_err, bound))
+    err = assert_rel_l2(y8, want_full, f"fp8-weight layer C={C} S={S} N={N} vs the fp32 oracle with the ORIGINAL weights",
+                        tol=bound, report=True)
+    assert err <= (q_err ** 2 + 4e-3 ** 2) ** 0.5, (err, q_err)
     assert_rel_l2(y8, want_q, "fp8-weight layer vs fp32 oracle with the dequantised weights")
     assert torch.equal(y8, y16)
-    print("rel-L2 against the unquantised fp32 layer:", to.rel_l2(y8.float().cpu(), want_full), flush=True)

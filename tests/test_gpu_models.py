@@ -6,6 +6,7 @@ import torch
 
 from oracle import torch_oracle as to
 import physicsnemo_amd as pn
+from physicsnemo_amd import functional as PF
 from gpu_util import announce, assert_fp32_close, assert_rel_l2
 
 pytestmark = pytest.mark.gpu
@@ -50,8 +51,19 @@ def test_cfg2_irregular_bf16_autocast():
         with torch.autocast("cuda", dtype=torch.bfloat16):
             got = hip(fx.cuda(), pos.cuda())
     assert got.shape == (B, N, 4)
-    # eight bf16 layers deep: the north-star bar (rel-L2 1e-2 vs fp32) is stated per layer; the model gets 2e-2
-    assert_rel_l2(got, want, "cfg2 model output", tol=2e-2)
+    # for scale: the oracle itself under bf16 autocast on the CPU (the reference's own mixed-precision recipe: fp32
+    # parameters, bf16 matrix products, fp32 softmax / LayerNorm / residual stream) against its fp32 run
+    with torch.no_grad(), torch.autocast("cpu", dtype=torch.bfloat16):
+        ref_bf16 = ref(fx[:1, :8192], pos[:1, :8192]).float()
+    with torch.no_grad():
+        want_sub = ref(fx[:1, :8192], pos[:1, :8192])
+    import conftest
+
+    conftest.MEASURED.append(("(oracle only) cfg2 model under CPU bf16 autocast vs its fp32 run, 8192 points",
+                              to.rel_l2(ref_bf16, want_sub), 1.0))
+    # eight bf16 blocks deep with a bf16 residual stream: measured 1.0e-2 .. 1.1e-2 (the single-layer bar is 1e-2); the
+    # measured figure is listed in the test summary
+    assert_rel_l2(got, want, "cfg2 model output (8 blocks, bf16 autocast)", tol=1.2e-2, report=True)
 
 
 def test_cfg4_surface_bf16_layer_stack_reduced():
@@ -73,4 +85,43 @@ def test_cfg4_surface_bf16_layer_stack_reduced():
         want = ref(fx, emb)
         with torch.autocast("cuda", dtype=torch.bfloat16):
             got = hip(fx.cuda(), emb.cuda())
-    assert_rel_l2(got, want, "cfg4-class model output", tol=2e-2)
+    assert_rel_l2(got, want, "cfg4-class model output (8 blocks, bf16 autocast)", tol=1.2e-2, report=True)
+
+
+@pytest.mark.parametrize("fp8", [False, True])
+def test_cfg5_volume_model_reduced_points(fp8):
+    # cfg5 as configured -- 12 layers, n_hidden 512, 16 heads (D = 32), 128 slices, 3 coordinates + 4 fields -> 4
+    # channels, bf16 activations, optionally fp8-e4m3 per-channel-scaled projection and MLP weights -- at 8192 points
+    # (the oracle's budget) against the fp32 oracle holding the ORIGINAL weights
+    announce("cfg5 volume model", "fp8" if fp8 else "bf16")
+    ref, hip = _pair(functional_dim=4, embedding_dim=3, out_dim=4, n_layers=12, n_hidden=512, n_head=16, slice_num=128)
+    g = torch.Generator().manual_seed(1234)
+    N = 8192
+    pos = torch.rand(1, N, 3, generator=g)
+    fx = torch.randn(1, N, 4, generator=g)
+    with torch.no_grad():
+        want = ref(fx, pos)
+        if fp8:
+            hip.use_fp8_weights(True)
+            # the same rounding applied to the oracle's weights: isolates the kernels from the number format
+            for blk in ref.blocks:
+                for lin in (blk.Attn.in_project_x, blk.Attn.in_project_fx, blk.Attn.out_linear, blk.ln_mlp1[1].layers[0],
+                            blk.ln_mlp1[1].layers[2]):
+                    lin.weight.copy_(PF.dequantize_e4m3_per_channel(*PF.quantize_e4m3_per_channel(lin.weight)))
+            want_q = ref(fx, pos)
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            got = hip(fx.cuda(), pos.cuda())
+    assert got.shape == (1, N, 4)
+    if not fp8:
+        # twelve bf16 blocks deep (the residual stream is rounded to bf16 twice per block): measured 1.2e-2
+        assert_rel_l2(got, want, "cfg5 model output (12 blocks, bf16) vs the fp32 oracle", tol=1.5e-2, report=True)
+        return
+    # e4m3 keeps 3 mantissa bits: rounding the 60 large weight matrices of the model ALONE moves the fp32 oracle's
+    # output by the first figure below; the kernels are held to the bf16 bar against the oracle with the same weights
+    import conftest
+
+    conftest.MEASURED.append(("(oracle only) e4m3 rounding of the cfg5 model's weights alone", to.rel_l2(want_q, want), 1.0))
+    assert_rel_l2(got, want_q, "cfg5 model output (12 blocks, fp8 weights) vs the fp32 oracle with the dequantised weights",
+                  tol=1.5e-2, report=True)
+    assert_rel_l2(got, want, "cfg5 model output (12 blocks, fp8 weights) vs the fp32 oracle with the ORIGINAL weights",
+                  tol=9e-2, report=True)
