@@ -354,7 +354,9 @@ int pa_mfma_pack_tokens(const pa_shape *shape, const float *out_slice_token, voi
 int64_t pa_mfma_buffer_bytes(const pa_shape *shape, int which);
 /* Repack the layer parameters (bf16 large weights) for the MFMA kernels; run once per parameter set. */
 int pa_mfma_pack_params(const pa_shape *shape, const pa_params *p, void *blob, void *stream);
-/* Kernel (a): projections + slice logits + temperature softmax (PA.py:529-537, :172-181). x is bf16 (B,N,C). */
+/* Kernel (a): projections + slice logits + temperature softmax (PA.py:529-537, :172-181). x is bf16 (B,N,C).
+ * fx_pack receives fx_mid WITHOUT the in_project_fx bias: pa_mfma_combine_attention adds bias * (sum of the weights)
+ * to the summed values, which is the same sum. */
 int pa_mfma_project_softmax(const pa_shape *shape, const void *blob, const void *x, void *fx_pack, void *w_pack,
                             void *stream);
 /* Kernel (b): first pass of the slice aggregation (PA.py:185-203) -> partials. */
@@ -369,7 +371,8 @@ int pa_mfma_project_softmax_reduce(const pa_shape *shape, const void *blob, cons
  * PA_ERR_UNSUPPORTED where it does not apply), 0 for pa_mfma_slice_reduce. Pass it to pa_mfma_combine_attention. */
 int64_t pa_mfma_partial_groups(const pa_shape *shape, int fused);
 /* Second pass + kernel (c): fixed-order combine, normalisation, slice attention (PA.py:185-203, :429-465).
- * groups = pa_mfma_partial_groups() of the producer. slice_token / slice_norm may be NULL. Writes out_slice_token (B,H,S,D) float32 and its packed copy tokp. */
+ * groups = pa_mfma_partial_groups() of the producer. slice_token / slice_norm may be NULL. Writes out_slice_token (B,H,S,D) float32 and its packed copy tokp.
+ * Reads p->qkv_project_weight and p->in_project_fx_bias (the bias the producers above leave out of their sums). */
 int pa_mfma_combine_attention(const pa_shape *shape, const pa_params *p, const float *partials, int64_t groups,
                               float *slice_token, float *slice_norm, float *out_slice_token, void *tokp,
                               void *stream);

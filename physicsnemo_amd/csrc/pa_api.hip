@@ -201,7 +201,7 @@ int mfma_layer(const pa_shape &s, const pa_params &p, const void *blob, const vo
     if ((rc = pa::mfma::project_softmax(s, blob, x, fxp, wp, nullptr, compute_units(), st))) return rc;
     if ((rc = pa::mfma::slice_reduce(s, wp, fxp, partials, st))) return rc;
   }
-  if ((rc = pa::mfma::combine_attention(s, p, partials, mp.G, tok, norm, tok_out, tokp, st))) return rc;
+  if ((rc = pa::mfma::combine_attention(s, p, p.in_project_fx_bias, partials, mp.G, tok, norm, tok_out, tokp, st))) return rc;
   return pa::mfma::deslice_project(s, blob, wp, tokp, y, tail_active(tail) ? tail : nullptr, compute_units(), st);
 }
 
@@ -744,10 +744,11 @@ int pa_mfma_combine_attention(const pa_shape *shape, const pa_params *p, const f
   if (rc) return rc;
   if (groups < 1 || (groups + 1) * shape->B * shape->H * shape->S * (shape->D + 1) * 4 > mfma_partials_bytes(*shape))
     return PA_ERR_DIMS;
-  if (!p || !p->qkv_project_weight || !partials || !out_slice_token || !tokp) return PA_ERR_NULL;
+  if (!p || !p->qkv_project_weight || !p->in_project_fx_bias || !partials || !out_slice_token || !tokp) return PA_ERR_NULL;
   if (!aligned16(partials) || !aligned16(tokp)) return PA_ERR_ALIGN;
   hipStream_t st = static_cast<hipStream_t>(stream);
-  return pa::mfma::combine_attention(*shape, *p, partials, groups, slice_token, slice_norm, out_slice_token, tokp, st);
+  return pa::mfma::combine_attention(*shape, *p, p->in_project_fx_bias, partials, groups, slice_token, slice_norm,
+                                     out_slice_token, tokp, st);
 }
 
 int pa_mfma_deslice_project(const pa_shape *shape, const void *blob, const void *w_pack, const void *tokp, void *y,
@@ -870,7 +871,7 @@ int pa_layer_forward(int dtype, const pa_shape *shape, const pa_params *p, const
     if ((rc = pa::gemm::launch(a, 2, PA_BF16, st))) return rc;
     if ((rc = pa::mfma::slice_softmax_pack(s, *p, x_mid, wp, compute_units(), st))) return rc;
     if ((rc = pa::mfma::slice_reduce(s, wp, fxp, partials, st))) return rc;
-    if ((rc = pa::mfma::combine_attention(s, *p, partials, sp.G, tok, norm, tok_out, tokp, st))) return rc;
+    if ((rc = pa::mfma::combine_attention(s, *p, nullptr, partials, sp.G, tok, norm, tok_out, tokp, st))) return rc;
     void *out_x = x_mid;
     if ((rc = pa::mfma::deslice_natural(s, wp, tokp, out_x, compute_units(), st))) return rc;
     if ((rc = pa::general::out_linear(dtype, s, *p, out_x, y, st))) return rc;
@@ -1066,7 +1067,7 @@ int pa_layer_forward_plus(int dtype, const pa_shape *shape, const pa_params *p, 
   if ((rc = pa::gemm::launch(a, 1, PA_BF16, st))) return rc;
   if ((rc = pa::mfma::slice_softmax_pack_plus(s, *p, *plus, x_mid, uniform, wp, compute_units(), st))) return rc;
   if ((rc = pa::mfma::slice_reduce(s, wp, fxp, partials, st))) return rc;
-  if ((rc = pa::mfma::combine_attention(s, *p, partials, sp.G, tok, norm, tok_out, tokp, st))) return rc;
+  if ((rc = pa::mfma::combine_attention(s, *p, nullptr, partials, sp.G, tok, norm, tok_out, tokp, st))) return rc;
   void *out_x = x_mid;
   if ((rc = pa::mfma::deslice_natural(s, wp, tokp, out_x, compute_units(), st))) return rc;
   if ((rc = pa::general::out_linear(dtype, s, *p, out_x, y, st))) return rc;

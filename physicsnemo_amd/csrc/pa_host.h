@@ -179,8 +179,8 @@ bool fuse_reduce(const pa_shape &s);
 int project_softmax(const pa_shape &s, const void *blob, const void *x, void *fx_pack, void *w_pack, float *partials,
                     int num_cu, hipStream_t st);
 int slice_reduce(const pa_shape &s, const void *w_pack, const void *fx_pack, float *partials, hipStream_t st);
-int combine_attention(const pa_shape &s, const pa_params &p, const float *partials, int64_t G, float *slice_token,
-                      float *slice_norm, float *out_token, void *tokp, hipStream_t st);
+int combine_attention(const pa_shape &s, const pa_params &p, const float *fx_bias, const float *partials, int64_t G,
+                      float *slice_token, float *slice_norm, float *out_token, void *tokp, hipStream_t st);
 int deslice_project(const pa_shape &s, const void *blob, const void *w_pack, const void *tokp, void *y,
                     const pa_block_tail *tail, int num_cu, hipStream_t st);
 }  // namespace mfma

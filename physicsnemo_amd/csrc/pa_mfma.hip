@@ -26,14 +26,20 @@ namespace pa {
 namespace mfma {
 
 // ------------------------------------------------------------------------------------------------
-// Packed parameter blob (built once per call by pack_params_kernel).  Offsets in 16-byte units.
+// Packed parameter blob (built once per parameter set by pack_params_kernel).  Offsets in 16-byte units.
 //   win [h][m][ks][lane]  m = 0: in_project_x, 1: in_project_fx; W_m[h*32 + i][16ks + 8g + j]
 //   wsl [st][kk][lane]    in_project_slice[32st + i][kperm(kk, g, j)]   (0 beyond S)
 //   wout[ct][h][kk][lane] out_linear[32ct + i][h*32 + kperm(kk, g, j)],  ct < C/32
-//   then float vectors: bias_x[C], bias_fx[C], bias_slice[ST*32] (-1e30 beyond S), bias_out[C], tscale[H]
+//   then float vectors (offsets in floats from fvec): bias_fx[C]; bias_logit[H][ST*32] = the slice bias with the bias
+//   of in_project_x folded in, b_slice[s] + sum_d W_slice[s][d] * b_x[h*32 + d] (-1e30 beyond S); bias_out[C];
+//   tscale[H] = log2(e) / clamp(temperature)
+// The projection kernel therefore forms x_mid and fx_mid WITHOUT their biases: the one of x_mid reaches the slice
+// logits through bias_logit, the one of fx_mid is added to the slice tokens after the aggregation
+// (sum_n w (fx + b) = sum_n w fx + b sum_n w).
 // ------------------------------------------------------------------------------------------------
 struct BlobPlan {
   int64_t win, wsl, wout, fvec, total_units;  // 16-byte units
+  int f_bias_fx, f_bias_logit, f_bias_out, f_tscale, nfloat;  // float offsets from fvec
 };
 
 __host__ __device__ inline BlobPlan blob_plan(int C, int S) {
@@ -43,8 +49,12 @@ __host__ __device__ inline BlobPlan blob_plan(int C, int S) {
   p.wsl = p.win + (int64_t)H * 2 * KS * 64;
   p.wout = p.wsl + (int64_t)ST * 2 * 64;
   p.fvec = p.wout + (int64_t)CT * H * 2 * 64;
-  const int64_t nfloat = 3 * C + ST * 32 + H;
-  p.total_units = p.fvec + (nfloat + 3) / 4;
+  p.f_bias_fx = 0;
+  p.f_bias_logit = C;
+  p.f_bias_out = p.f_bias_logit + H * ST * 32;
+  p.f_tscale = p.f_bias_out + C;
+  p.nfloat = p.f_tscale + H;
+  p.total_units = p.fvec + (p.nfloat + 3) / 4;
   return p;
 }
 
@@ -88,14 +98,23 @@ __global__ __launch_bounds__(256) void pack_params_kernel(pa_params p, u32x4 *__
     blob[u] = v;
   }
   float *fv = reinterpret_cast<float *>(blob + bp.fvec);
-  const int nfloat = 3 * C + ST * 32 + H;
-  for (int k = blockIdx.x * 256 + threadIdx.x; k < nfloat; k += gridDim.x * 256) {
+  for (int k = blockIdx.x * 256 + threadIdx.x; k < bp.nfloat; k += gridDim.x * 256) {
     float v;
-    if (k < C) v = p.in_project_x_bias[k];
-    else if (k < 2 * C) v = p.in_project_fx_bias[k - C];
-    else if (k < 2 * C + ST * 32) v = (k - 2 * C) < S ? p.in_project_slice_bias[k - 2 * C] : -1e30f;
-    else if (k < 3 * C + ST * 32) v = p.out_linear_bias[k - 2 * C - ST * 32];
-    else v = kLog2e / clamp_temperature(p.temperature[k - 3 * C - ST * 32]);
+    if (k < bp.f_bias_logit) {
+      v = p.in_project_fx_bias[k];
+    } else if (k < bp.f_bias_out) {
+      const int q = k - bp.f_bias_logit, h = q / (ST * 32), sidx = q - h * (ST * 32);
+      if (sidx < S) {
+        v = p.in_project_slice_bias[sidx];
+        for (int d = 0; d < 32; ++d) v = fmaf(p.in_project_slice_weight[sidx * 32 + d], p.in_project_x_bias[h * 32 + d], v);
+      } else {
+        v = -1e30f;
+      }
+    } else if (k < bp.f_tscale) {
+      v = p.out_linear_bias[k - bp.f_bias_out];
+    } else {
+      v = kLog2e / clamp_temperature(p.temperature[k - bp.f_tscale]);
+    }
     fv[k] = v;
   }
 }
@@ -109,20 +128,36 @@ __global__ __launch_bounds__(256) void pack_params_kernel(pa_params p, u32x4 *__
 //   softmax over s: in-lane over the accumulator registers plus one exchange with lane^32               -> w_pack
 //   !FUSED: fx_mid -> fx_pack (kernel (b) aggregates later)
 //    FUSED: w^T (lanes <-> slices, registers <-> points) = w_chunk . SEL  (an exact MFMA "transpose"),
-//           tok^T_h (32 d x S) += bf16(fx_mid)^T . w^T, norm_h += sum_n w; accumulators live in LDS between tiles
-//           (a wave owns its head, so there is no cross-wave reduction) and leave as one partial per workgroup:
-//           partials[g][b][h][s][0..D-1] = sum_n w fx_mid, [..][D] = sum_n w   (layout of the combine kernel).
+//           tok^T_h (32 d x S) += bf16(fx_mid)^T . w^T, norm_h += sum_n w in per-head accumulators that stay in
+//           registers for the whole kernel (a wave owns its head, so there is no cross-wave reduction) and leave
+//           as one partial per workgroup: partials[g][b][h][s][0..D-1] = sum_n w fx_mid, [..][D] = sum_n w
+//           (layout of the combine kernel).
+// Both biases of the projections are applied elsewhere (see the parameter blob).
 // Grid (G workgroups per batch, B); workgroup (g, b) walks the tile sets g, g+G, ... of batch b, H waves (two per
 // SIMD for C = 256).  Wave h owns head h and keeps its Wx | Wfx fragments (2 * KS * 4 = 128 registers for C = 256)
-// in registers for the whole kernel: after the prologue there is no weight traffic at all.  The x rows of a SET of
-// TS tiles are staged in LDS by the whole workgroup with full-row coalesced loads; unit u (16 bytes) of row r is
-// stored at r*(UPR+1) + u: the one-unit stagger per row makes the 16 lanes of a 128-bit access (rows i..i+15, same
-// unit) cover all 64 banks, so both the row-wise writes and the fragment reads (row i, unit 2ks+g) are free of bank
-// conflicts, and every fragment address is one base register plus an immediate offset.  One fragment read (1 KiB) feeds two MFMAs.  The set buffers are double buffered; the next
-// set is fetched one tile at a time into registers at the start of a tile and written to LDS at its end; one
-// barrier per set.  The loop over sets is the only loop; its body has no branch around a global memory operation
-// (slots past the last tile of the batch recompute it and re-store identical values; they skip the aggregation).
+// in registers for the whole kernel: after the prologue there is no weight traffic at all.
+// The x rows of a SET of TS tiles are staged in LDS by direct global -> LDS loads (no registers, no LDS write
+// instructions): one wave load moves 64 x 16 bytes = RPC rows to 1 KiB of contiguous LDS.  A tile is NCK = 32 / RPC
+// such chunks, chunk c holding rows c, c + NCK, ...; chunks lie 65 units apart, so unit u of row r sits at
+// (r % NCK) * 65 + (r / NCK) * UPR + u.  For C = 256 (NCK = 16) the 16 lanes of a 128-bit access (rows i..i+15, same
+// unit) cover all 64 banks, and every fragment address is one base register plus an immediate offset.  One fragment
+// read (1 KiB) feeds two MFMAs.  The set buffers are double buffered; the loads of the next set are issued one tile
+// at a time at the start of a tile; one barrier per set.  The loop over sets is the only loop; its body has no
+// branch around a global memory operation (slots past the last tile of the batch recompute it and re-store
+// identical values; they add nothing to the aggregation).
 // ------------------------------------------------------------------------------------------------
+
+// One direct global -> LDS load of 64 x 16 bytes: lane l reads sbase + voff(l) and its data land at LDS byte address
+// lds + 16 l.  sbase and lds are wave-uniform.  Asynchronous, counted by vmcnt like any load.
+__device__ __forceinline__ void load_row_chunk_to_lds(const void *sbase, unsigned voff, unsigned lds) {
+  asm volatile(
+      "s_mov_b32 m0, %2\n\t"
+      "s_nop 0\n\t"
+      "global_load_lds_dwordx4 %1, %0" ::"s"(sbase),
+      "v"(voff), "s"(lds)
+      : "memory");
+}
+
 template <int C, int S, bool FUSED>
 __global__ __launch_bounds__((C / 32) * 64) void project_softmax_kernel(const u32x4 *__restrict__ blob,
                                                                         const uint16_t *__restrict__ x,
@@ -131,25 +166,26 @@ __global__ __launch_bounds__((C / 32) * 64) void project_softmax_kernel(const u3
                                                                         float *__restrict__ partials, int64_t N, int tpb) {
   constexpr int H = C / 32, KS = C / 16, ST = (S + 31) / 32, NCH = S / 16, D1 = 33;
   constexpr int WAVES = H, NT = WAVES * 64;
-  constexpr int TS = FUSED ? 2 : 4;     // tiles per set (the fused form needs LDS for the accumulators)
+  constexpr int TS = 4;                 // tiles per set
   constexpr int UPR = C / 8;            // 16-byte units per row
-  constexpr int ROWU = UPR + 1;         // LDS row stride in units: one unit of stagger per row (see above)
-  constexpr int SET_UNITS = TS * 32 * ROWU;
-  constexpr int CHUNK = 32 * UPR / NT;  // units per thread and tile when staging
-  constexpr int ACC_UNITS = ST * 4 * 64 + ST * 16;  // per head: tok^T accumulator (16-byte units) + norm row
-  static_assert((32 * UPR) % NT == 0, "a tile must split evenly over the workgroup");
+  constexpr int RPC = 64 / UPR;         // rows per chunk (one wave load)
+  constexpr int NCK = 32 / RPC;         // chunks per tile
+  constexpr int TILE_UNITS = NCK * 65;
+  constexpr int SET_UNITS = TS * TILE_UNITS;
+  constexpr int CPW = NCK / WAVES;      // chunks per wave and tile
+  constexpr int STORES_PER_TILE = NCH + (FUSED ? 0 : 2);
+  static_assert(NCK % WAVES == 0, "the chunks of a tile must split evenly over the waves");
   extern __shared__ u32x4 smem[];
   u32x4 *xs = smem;                     // 2 * SET_UNITS
   u32x4 *wsl = xs + 2 * SET_UNITS;      // ST * 2 * 64
-  u32x4 *sel = wsl + ST * 2 * 64;       // 2 * 64: the 0/1 selection matrices of the MFMA transpose
-  u32x4 *accs = sel + 2 * 64;           // FUSED: H * ACC_UNITS
-  float *fvec = reinterpret_cast<float *>(accs + (FUSED ? H * ACC_UNITS : 0));
-  float *bias_x = fvec, *bias_f = fvec + C, *bias_s = fvec + 2 * C, *tscale = fvec + 3 * C + ST * 32;
+  u32x4 *sel = wsl + ST * 2 * 64;       // 4 * 64: the 0/1 selection matrices of the MFMA transpose + two zero ones
+  float *fvec = reinterpret_cast<float *>(sel + 4 * 64);
   const BlobPlan bp = blob_plan(C, S);
   const int tid = threadIdx.x, lane = tid & 63, i = lane & 31, g = lane >> 5;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: addresses derived from it stay scalar
   const int h = wave;
   const int b = blockIdx.y;
+  const float *bias_s = fvec + bp.f_bias_logit + h * (ST * 32), *tscale = fvec + bp.f_tscale;
 
   u32x4 wx[KS], wf[KS];
 #pragma unroll
@@ -161,192 +197,268 @@ __global__ __launch_bounds__((C / 32) * 64) void project_softmax_kernel(const u3
   for (int u = tid; u < ST * 2 * 64; u += NT) wsl[u] = blob[bp.wsl + u];
   {
     const float *src = reinterpret_cast<const float *>(blob + bp.fvec);
-    for (int k = tid; k < 3 * C + ST * 32 + H; k += NT) fvec[k] = src[k];
+    for (int k = tid; k < bp.nfloat; k += NT) fvec[k] = src[k];
   }
-  u32x4 *acc_tok = accs + h * ACC_UNITS;                                        // [st][q][lane]: registers 4q..4q+3
-  float *acc_nrm = reinterpret_cast<float *>(accs + h * ACC_UNITS + ST * 4 * 64);  // [st][lane]
+  // per-head accumulators of the aggregation: tokacc[st][r] = sum_n w[n, 32st + i] fx_mid[n, rowmap(r, g)],
+  // nrmacc[st] = this half-wave's share of sum_n w[n, 32st + i]
+  f32x16 tokacc[ST];
+  float nrmacc[ST];
+#pragma unroll
+  for (int st = 0; st < ST; ++st) {
+    nrmacc[st] = 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) tokacc[st][r] = 0.f;
+  }
   if constexpr (FUSED) {
-    if (tid < 128) {
-      const int par = tid >> 6;
+    if (tid < 256) {  // the two 0/1 selection matrices of the MFMA transpose, then two all-zero ones
+      const int par = (tid >> 6) & 1;
       bf16x8 s8;
 #pragma unroll
-      for (int j = 0; j < 8; ++j) s8[j] = (__bf16)((i == kperm(par, g, j)) ? 1.f : 0.f);
+      for (int j = 0; j < 8; ++j) s8[j] = (__bf16)((tid < 128 && i == kperm(par, g, j)) ? 1.f : 0.f);
       sel[tid] = __builtin_bit_cast(u32x4, s8);
     }
-    for (int u = lane; u < ACC_UNITS; u += 64) acc_tok[u] = u32x4{0, 0, 0, 0};
   }
 
   const int nsets = (tpb + TS - 1) / TS;  // per batch
   const int nloc = (nsets - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x;
   const uint16_t *xbatch = x + (int64_t)b * N * C;
-  // staging: this thread's CHUNK units of tile `tile` of the batch: unit k*NT + tid -> row rc, position pos.  The
-  // load only issues (rows beyond N re-read row 0 of the tile); the values are first touched in stage_store, a whole
-  // tile of work later, where rows beyond N are replaced by zeros.
-  auto stage_load = [&](int tile, u32x4(&st)[CHUNK], int &rows_ok) {
-    const int t = tile < tpb ? tile : tpb - 1;
-    const uint16_t *xbase = xbatch + (int64_t)t * 32 * C;
-    rows_ok = (int)min((int64_t)32, N - (int64_t)t * 32);
+  const int rows_last = (int)(N - (int64_t)(tpb - 1) * 32);  // rows of the batch's last tile
+  // staging: this wave's CPW chunks of tile `tile` of the batch into slot t of buffer buf.  Lane l of chunk c fetches
+  // unit l % UPR of row c + NCK * (l / UPR); rows beyond N re-read row 0 of the tile (their weights are zeroed later).
+  const int srow = lane / UPR, sunit = lane % UPR;
+  auto stage = [&](int tile, int buf, int t) {
+    const int tl = tile < tpb ? tile : tpb - 1;
+    const uint16_t *xbase = xbatch + (int64_t)tl * 32 * C;
+    const int rows_ok = tl == tpb - 1 ? rows_last : 32;
 #pragma unroll
-    for (int k = 0; k < CHUNK; ++k) {
-      const int idx = k * NT + tid, rc = idx / UPR, pos = idx - rc * UPR;
-      st[k] = *reinterpret_cast<const u32x4 *>(xbase + (rc < rows_ok ? rc : 0) * C + pos * 8);
-    }
-  };
-  auto stage_store = [&](int buf, int t, const u32x4(&st)[CHUNK], int rows_ok) {
-#pragma unroll
-    for (int k = 0; k < CHUNK; ++k) {
-      const int idx = k * NT + tid, rc = idx / UPR, pos = idx - rc * UPR;
-      xs[buf * SET_UNITS + (t * 32 + rc) * ROWU + pos] = rc < rows_ok ? st[k] : u32x4{0, 0, 0, 0};
+    for (int k = 0; k < CPW; ++k) {
+      const int c = wave * CPW + k;
+      int row = c + NCK * srow;
+      row = row < rows_ok ? row : 0;
+      const unsigned lds = (unsigned)(uintptr_t)(xs + buf * SET_UNITS + t * TILE_UNITS + c * 65);
+      load_row_chunk_to_lds(xbase, (unsigned)(row * C + sunit * 8) * 2u, lds);
     }
   };
 #pragma unroll
-  for (int t = 0; t < TS; ++t) {  // first set
-    u32x4 st[CHUNK];
-    int rows_ok;
-    stage_load((int)blockIdx.x * TS + t, st, rows_ok);
-    stage_store(0, t, st, rows_ok);
-  }
+  for (int t = 0; t < TS; ++t) stage((int)blockIdx.x * TS + t, 0, t);  // first set
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
 
+  // A tile is worked on in two halves.
+  //   MFMA half:   aggregation products of the tile before (operands left by its vector half), then the two
+  //                projections of this tile, their results packed to bf16 operands.  Every MFMA here is independent
+  //                of vector work, so the matrix pipe is fed back to back; registers: accumulators + fragment ring.
+  //   vector half: slice logits (4 short MFMAs), softmax over the slices of each point in the base-2 domain,
+  //                w = exp2((l - max) * log2e / T) / sum, the store of w_pack, the MFMA "transpose" of the weights,
+  //                slice norms, and the transposed weights packed as operands of the next MFMA half.
+  struct Tile {  // left by the MFMA half
+    u32x4 xb0, xb1;    // x_mid^T as B operands of the logits
+    u32x4 fx0, fx1;    // fx_mid^T as A operands of the aggregation
+    int64_t tile;      // global tile index (b * tpb + tile in batch)
+    bool dup;          // a slot past the batch's last tile: recomputed, contributes nothing to the aggregation
+    bool valid;        // this lane's point exists
+  };
+  struct Agg {  // left by the vector half: operands of the aggregation products
+    u32x4 tp[ST][2];
+    u32x4 fx0, fx1;
+  };
+  auto aggregate = [&](const Agg &ag) {
+    if constexpr (FUSED) {
+#pragma unroll
+      for (int st = 0; st < ST; ++st) tokacc[st] = mma(ag.fx0, ag.tp[st][0], tokacc[st]);
+#pragma unroll
+      for (int st = 0; st < ST; ++st) tokacc[st] = mma(ag.fx1, ag.tp[st][1], tokacc[st]);
+    }
+  };
+  auto mfma_half = [&](int buf, int t, int slot, Tile &tl, const Agg &ag) {
+    __builtin_amdgcn_s_setprio(3);  // goes first: its issue slots are few and feed the matrix pipe
+    tl.dup = slot >= tpb;
+    const int tb = tl.dup ? tpb - 1 : slot;
+    tl.tile = (int64_t)b * tpb + tb;
+    tl.valid = (int64_t)tb * 32 + i < N;
+    const u32x4 *xb = xs + buf * SET_UNITS + t * TILE_UNITS + (i % NCK) * 65 + (i / NCK) * UPR + g;
+    // x fragments are read AHEAD k-steps before the MFMAs that use them
+    constexpr int RING = 4, AHEAD = RING - 1;
+    u32x4 xf[RING];
+#pragma unroll
+    for (int q = 0; q < AHEAD; ++q) xf[q] = xb[2 * q];
+    __builtin_amdgcn_sched_barrier(0);
+    aggregate(ag);
+    __builtin_amdgcn_sched_barrier(0);
+    f32x16 ax, af;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) ax[r] = af[r] = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      if (ks + AHEAD < KS) xf[(ks + AHEAD) % RING] = xb[2 * (ks + AHEAD)];
+      ax = mma(wx[ks], xf[ks % RING], ax);
+      af = mma(xf[ks % RING], wf[ks], af);
+      __builtin_amdgcn_sched_barrier(0);  // keeps the compiler from sinking the reads back next to their uses
+    }
+    tl.xb0 = pack_half<0>(ax);
+    tl.xb1 = pack_half<1>(ax);
+    tl.fx0 = pack_half<0>(af);
+    tl.fx1 = pack_half<1>(af);
+    if constexpr (!FUSED) {
+      u32x4 *fdst = fx_pack + ((tl.tile * H + h) * 2) * 64 + lane;
+      fdst[0] = tl.fx0;
+      fdst[64] = tl.fx1;
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  auto vector_half = [&](const Tile &tl, Agg &ag) {
+    __builtin_amdgcn_s_setprio(0);  // fills the issue slots the other wave of the SIMD leaves
+    f32x16 lg[ST];
+#pragma unroll
+    for (int st = 0; st < ST; ++st) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) lg[st][r] = bias_s[32 * st + rowmap(r, g)];
+    }
+#pragma unroll
+    for (int st = 0; st < ST; ++st) lg[st] = mma(wsl[(st * 2 + 0) * 64 + lane], tl.xb0, lg[st]);
+#pragma unroll
+    for (int st = 0; st < ST; ++st) lg[st] = mma(wsl[(st * 2 + 1) * 64 + lane], tl.xb1, lg[st]);
+    float mx = -INFINITY;
+#pragma unroll
+    for (int st = 0; st < ST; ++st)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) mx = fmaxf(mx, lg[st][r]);
+    mx = half_max(mx);
+    const float sc = tscale[h];
+    const float off = mx * sc;
+    float sum[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int st = 0; st < ST; ++st)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const float e = __builtin_amdgcn_exp2f(fmaf(lg[st][r], sc, -off));
+        lg[st][r] = e;
+        sum[r & 3] += e;
+      }
+    const float tot = half_sum((sum[0] + sum[1]) + (sum[2] + sum[3]));
+    const float inv = tl.valid ? __builtin_amdgcn_rcpf(tot) : 0.f;  // rows beyond N get zero weight
+    u32x4 wp[2 * ST];
+#pragma unroll
+    for (int st = 0; st < ST; ++st) {
+      wp[2 * st] = pack_half<0>(lg[st], inv);
+      wp[2 * st + 1] = pack_half<1>(lg[st], inv);
+    }
+    u32x4 *wdst = w_pack + ((tl.tile * H + h) * NCH) * 64 + lane;
+#pragma unroll
+    for (int cq = 0; cq < NCH; ++cq) wdst[cq * 64] = wp[cq];
+    if constexpr (FUSED) {
+      // transposed weights (lanes <-> slices, registers <-> points); a slot past the batch's last tile multiplies by
+      // the all-zero selection matrices instead and so adds nothing
+      const u32x4 *sl = sel + (tl.dup ? 2 * 64 : 0) + lane;
+      const u32x4 sel0 = sl[0], sel1 = sl[64];
+      f32x16 tr[ST];
+#pragma unroll
+      for (int st = 0; st < ST; ++st) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) tr[st][r] = 0.f;
+        tr[st] = mma(wp[2 * st], sel0, tr[st]);
+      }
+      if constexpr (NCH > 1) {
+#pragma unroll
+        for (int st = 0; st < ST; ++st) tr[st] = mma(wp[2 * st + 1], sel1, tr[st]);
+      }
+#pragma unroll
+      for (int st = 0; st < ST; ++st) {
+        float s0 = tr[st][0] + tr[st][1], s1 = tr[st][2] + tr[st][3];
+#pragma unroll
+        for (int r = 4; r < 16; r += 4) {
+          s0 += tr[st][r] + tr[st][r + 1];
+          s1 += tr[st][r + 2] + tr[st][r + 3];
+        }
+        nrmacc[st] += s0 + s1;
+        ag.tp[st][0] = pack_half<0>(tr[st]);
+        ag.tp[st][1] = pack_half<1>(tr[st]);
+      }
+      ag.fx0 = tl.fx0;
+      ag.fx1 = tl.fx1;
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+
+  auto wait_staged = [&]() {
+    // the loads of the next set have landed once at most the stores of the last tile are still in flight
+    if constexpr (STORES_PER_TILE == 1) asm volatile("s_waitcnt vmcnt(1)" ::: "memory");
+    else if constexpr (STORES_PER_TILE == 2) asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
+    else if constexpr (STORES_PER_TILE == 3) asm volatile("s_waitcnt vmcnt(3)" ::: "memory");
+    else if constexpr (STORES_PER_TILE == 4) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+    else if constexpr (STORES_PER_TILE == 6) asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
+    else if constexpr (STORES_PER_TILE == 8) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  };
+  // The two waves of a SIMD (waves w and w + 4 of an 8-wave workgroup) run the halves out of phase: the upper four
+  // go MFMA half, then vector half of the same tile; the lower four start with the vector half of the tile before.
+  // Between two barriers one wave of each SIMD is then feeding the matrix pipe while the other fills the issue slots
+  // it leaves (lower priority) with vector work.  Both orders stage the next set at the same places and meet at the
+  // same barriers.
+  const bool lower = WAVES == 8 && wave < 4;
+  // nothing to finish before the first tile: placeholders with zero operands; the w_pack store of the placeholder
+  // tile (lower waves) lands on this workgroup's first tile with zero weights and is overwritten there by the real
+  // one (same lanes, same addresses, later in program order); it is marked as a slot that adds nothing
+  Tile tl;
+  Agg ag;
+#pragma unroll
+  for (int st = 0; st < ST; ++st) ag.tp[st][0] = ag.tp[st][1] = u32x4{0, 0, 0, 0};
+  ag.fx0 = ag.fx1 = u32x4{0, 0, 0, 0};
+  tl.xb0 = tl.xb1 = tl.fx0 = tl.fx1 = u32x4{0, 0, 0, 0};
+  tl.tile = (int64_t)b * tpb + min((int)blockIdx.x * TS, tpb - 1);
+  tl.dup = true;
+  tl.valid = false;
   int set = blockIdx.x;
-  for (int sl = 0; sl < nloc; ++sl) {
-    const int buf = sl & 1;
-    const int set_next = set + (int)gridDim.x < nsets ? set + (int)gridDim.x : set;  // the last set re-fetches itself
+  if (!lower) {
+    for (int sl = 0; sl < nloc; ++sl) {
+      const int buf = sl & 1;
+      const int set_next = set + (int)gridDim.x < nsets ? set + (int)gridDim.x : set;  // the last set re-fetches itself
 #pragma unroll
-    for (int t = 0; t < TS; ++t) {
-      __builtin_amdgcn_sched_barrier(0);  // keep each tile's work (and its register live ranges) to itself
-      u32x4 stg[CHUNK];
-      int stg_rows;
-      stage_load(set_next * TS + t, stg, stg_rows);
-      __builtin_amdgcn_sched_barrier(0);
-      const int slot = set * TS + t;
-      const bool dup = slot >= tpb;  // past the batch's last tile: recompute it, contribute nothing
-      const int tb = dup ? tpb - 1 : slot;
-      const int64_t tile = (int64_t)b * tpb + tb;
-      const bool valid = (int64_t)tb * 32 + i < N;
-
-      // ---- products ----
-      const u32x4 *xb = xs + buf * SET_UNITS + (t * 32 + i) * ROWU + g;
-      f32x16 ax, af;
-      {
-        const float bf = bias_f[h * 32 + i];
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          ax[r] = bias_x[h * 32 + rowmap(r, g)];
-          af[r] = bf;
-        }
-      }
-      // x fragments are read AHEAD k-steps before the MFMAs that use them (S = 128 has no registers to spare)
-      constexpr int RING = ST > 2 ? 2 : 3, AHEAD = RING - 1;
-      u32x4 xf[RING];
-#pragma unroll
-      for (int q = 0; q < AHEAD; ++q) xf[q] = xb[2 * q];
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        if (ks + AHEAD < KS) xf[(ks + AHEAD) % RING] = xb[2 * (ks + AHEAD)];
-        ax = mma(wx[ks], xf[ks % RING], ax);
-        af = mma(xf[ks % RING], wf[ks], af);
-        __builtin_amdgcn_sched_barrier(0);  // keeps the compiler from sinking the reads back next to their uses
-      }
-      const u32x4 fxp0 = pack_half<0>(af), fxp1 = pack_half<1>(af);
-      if constexpr (!FUSED) {
-        u32x4 *fdst = fx_pack + ((tile * H + h) * 2) * 64 + lane;
-        fdst[0] = fxp0;
-        fdst[64] = fxp1;
-      }
-      const u32x4 xb0 = pack_half<0>(ax), xb1 = pack_half<1>(ax);
-      f32x16 lg[ST];
-#pragma unroll
-      for (int st = 0; st < ST; ++st) {
-#pragma unroll
-        for (int r = 0; r < 16; ++r) lg[st][r] = bias_s[32 * st + rowmap(r, g)];
-        lg[st] = mma(wsl[(st * 2 + 0) * 64 + lane], xb0, lg[st]);
-        lg[st] = mma(wsl[(st * 2 + 1) * 64 + lane], xb1, lg[st]);
-      }
-      __builtin_amdgcn_sched_barrier(0);
-
-      // ---- softmax over the slices of each point, in the base-2 domain: w = exp2((l - max) * log2e / T) / sum ----
-      float mx = -INFINITY;
-#pragma unroll
-      for (int st = 0; st < ST; ++st)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) mx = fmaxf(mx, lg[st][r]);
-      mx = half_max(mx);
-      const float sc = tscale[h];
-      const float off = mx * sc;
-      float sum = 0.f;
-#pragma unroll
-      for (int st = 0; st < ST; ++st)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const float e = __builtin_amdgcn_exp2f(fmaf(lg[st][r], sc, -off));
-          lg[st][r] = e;
-          sum += e;
-        }
-      sum = half_sum(sum);
-      const float inv = valid ? __builtin_amdgcn_rcpf(sum) : 0.f;  // rows beyond N get zero weight
-      u32x4 wp[2 * ST];
-#pragma unroll
-      for (int st = 0; st < ST; ++st) {
-        wp[2 * st] = pack_half<0>(lg[st], inv);
-        wp[2 * st + 1] = pack_half<1>(lg[st], inv);
-      }
-      u32x4 *wdst = w_pack + ((tile * H + h) * NCH) * 64 + lane;
-#pragma unroll
-      for (int cq = 0; cq < NCH; ++cq) wdst[cq * 64] = wp[cq];
-      __builtin_amdgcn_sched_barrier(0);
-
-      // ---- aggregation of this tile into the head's LDS accumulators ----
-      if constexpr (FUSED) {
-        if (!dup) {
-#pragma unroll
-          for (int st = 0; st < ST; ++st) {
-            f32x16 tr;
-#pragma unroll
-            for (int r = 0; r < 16; ++r) tr[r] = 0.f;
-            tr = mma(wp[2 * st], sel[lane], tr);
-            if (2 * st + 1 < NCH) tr = mma(wp[2 * st + 1], sel[64 + lane], tr);
-            float s16 = 0.f;
-#pragma unroll
-            for (int r = 0; r < 16; ++r) s16 += tr[r];
-            acc_nrm[st * 64 + lane] += s16;
-            f32x16 tok;
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-              const u32x4 v = acc_tok[(st * 4 + q) * 64 + lane];
-#pragma unroll
-              for (int k = 0; k < 4; ++k) tok[4 * q + k] = __uint_as_float(v[k]);
-            }
-            tok = mma(fxp0, pack_half<0>(tr), tok);
-            tok = mma(fxp1, pack_half<1>(tr), tok);
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-              u32x4 v;
-#pragma unroll
-              for (int k = 0; k < 4; ++k) v[k] = __float_as_uint(tok[4 * q + k]);
-              acc_tok[(st * 4 + q) * 64 + lane] = v;
-            }
-          }
-        }
+      for (int t = 0; t < TS; ++t) {
+        __builtin_amdgcn_sched_barrier(0);  // keep each tile's work (and its register live ranges) to itself
+        stage(set_next * TS + t, buf ^ 1, t);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma_half(buf, t, set * TS + t, tl, ag);
+        vector_half(tl, ag);
         __builtin_amdgcn_sched_barrier(0);
       }
-      stage_store(buf ^ 1, t, stg, stg_rows);
-      __builtin_amdgcn_sched_barrier(0);
+      set = set_next;
+      wait_staged();
+      __syncthreads();
     }
-    set = set_next;
-    __syncthreads();
+    aggregate(ag);
+  } else {
+    for (int sl = 0; sl < nloc; ++sl) {
+      const int buf = sl & 1;
+      const int set_next = set + (int)gridDim.x < nsets ? set + (int)gridDim.x : set;
+#pragma unroll
+      for (int t = 0; t < TS; ++t) {
+        __builtin_amdgcn_sched_barrier(0);
+        stage(set_next * TS + t, buf ^ 1, t);
+        __builtin_amdgcn_sched_barrier(0);
+        vector_half(tl, ag);
+        mfma_half(buf, t, set * TS + t, tl, ag);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      set = set_next;
+      wait_staged();
+      __syncthreads();
+    }
+    vector_half(tl, ag);
+    aggregate(ag);
   }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // nothing may still be landing in LDS when the workgroup ends
   if constexpr (FUSED) {
     // this wave's head: accumulators -> partials[g][b][h][s][d], [..][D] = count
     float *dst = partials + (((int64_t)blockIdx.x * gridDim.y + b) * H + h) * (S * D1);
-    const float *tokf = reinterpret_cast<const float *>(acc_tok);
 #pragma unroll
     for (int st = 0; st < ST; ++st) {
       const int s = 32 * st + i;
+      const float nrm = half_sum(nrmacc[st]);
       if (s < S) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) dst[s * D1 + rowmap(r, g)] = tokf[((st * 4 + (r >> 2)) * 64 + lane) * 4 + (r & 3)];
-        if (g == 0) dst[s * D1 + 32] = acc_nrm[st * 64 + lane] + acc_nrm[st * 64 + lane + 32];
+        for (int r = 0; r < 16; ++r) dst[s * D1 + rowmap(r, g)] = tokacc[st][r];
+        if (g == 0) dst[s * D1 + 32] = nrm;
       }
     }
   }
@@ -461,11 +573,12 @@ __device__ __forceinline__ f32x16 mma32(float a, float b, f32x16 c) {
 
 template <int S>
 __global__ __launch_bounds__(64 * ((S + 31) / 32)) void slice_attention_kernel(const float *__restrict__ combined,
+                                                                               const float *__restrict__ fx_bias,
                                                                                const float *__restrict__ w_qkv,
                                                                                float *__restrict__ slice_token,
                                                                                float *__restrict__ slice_norm,
                                                                                float *__restrict__ out_token,
-                                                                               uint16_t *__restrict__ tokp) {
+                                                                               uint16_t *__restrict__ tokp, int heads) {
   constexpr int NTILE = (S + 31) / 32, D = 32, D1 = 33, NCH = S / 16;
   __shared__ float ks[NTILE * 32 * D1], vs[NTILE * 32 * D1];
   const int bh = blockIdx.x, tid = threadIdx.x, lane = tid & 63, i = lane & 31, g = lane >> 5;
@@ -474,10 +587,15 @@ __global__ __launch_bounds__(64 * ((S + 31) / 32)) void slice_attention_kernel(c
   const bool live = s < S;
 
   const float *src = combined + ((int64_t)bh * S + (live ? s : 0)) * D1;
-  const float cnt = src[D] + kSliceNormEps;
+  const float wsum = src[D], cnt = wsum + kSliceNormEps;
+  // fx_bias (H*32, or NULL): bias of in_project_fx left out of the summed fx_mid: sum_n w (fx + b) = sum_n w fx + b sum_n w
+  const float *fb = fx_bias ? fx_bias + (bh % heads) * D : nullptr;
   float tk[16];  // tok[s][2kk + g]
 #pragma unroll
-  for (int kk = 0; kk < 16; ++kk) tk[kk] = live ? src[2 * kk + g] / cnt : 0.f;
+  for (int kk = 0; kk < 16; ++kk) {
+    const float num = fb ? fmaf(fb[2 * kk + g], wsum, src[2 * kk + g]) : src[2 * kk + g];
+    tk[kk] = live ? num / cnt : 0.f;
+  }
   if (live) {
     if (slice_token) {
 #pragma unroll
@@ -597,7 +715,7 @@ __global__ __launch_bounds__(C * 2) void deslice_project_kernel(const u32x4 *__r
     wout[h][0] = blob[bp.wout + ((wave * H + h) * 2 + 0) * 64 + lane];
     wout[h][1] = blob[bp.wout + ((wave * H + h) * 2 + 1) * 64 + lane];
   }
-  const float *fv = reinterpret_cast<const float *>(blob + bp.fvec) + 2 * C + ST * 32;
+  const float *fv = reinterpret_cast<const float *>(blob + bp.fvec) + bp.f_bias_out;
   const float bias = fv[wave * 32 + i];
   float gam[CPL], bet[CPL];
 #pragma unroll
@@ -790,7 +908,8 @@ int pack_params(const pa_shape &s, const pa_params &p, void *blob, hipStream_t s
 
 // workgroups per batch of kernel (a): about one resident workgroup per CU in total
 int64_t project_groups(const pa_shape &s, int num_cu, bool fused) {
-  const int64_t ts = fused ? 2 : 4;
+  const int64_t ts = 4;
+  (void)fused;
   const int64_t nsets = (tiles_per_batch(s) + ts - 1) / ts;
   int64_t g = num_cu / s.B;
   if (g < 1) g = 1;
@@ -803,10 +922,8 @@ bool fuse_reduce(const pa_shape &s) { return s.S <= 64; }  // the LDS accumulato
 template <int C, int S, bool FUSED>
 static int project_softmax_f(const pa_shape &s, const void *blob, const void *x, void *fx_pack, void *w_pack,
                              float *partials, int num_cu, hipStream_t st) {
-  constexpr int ST = (S + 31) / 32, H = C / 32, TS = FUSED ? 2 : 4, UPR = C / 8, WAVES = H;
-  constexpr int ACC_UNITS = ST * 4 * 64 + ST * 16;
-  const size_t lds = (size_t)(2 * TS * 32 * (UPR + 1) + ST * 2 * 64 + 2 * 64 + (FUSED ? H * ACC_UNITS : 0)) * 16 +
-                     (size_t)(3 * C + ST * 32 + H) * 4;
+  constexpr int ST = (S + 31) / 32, H = C / 32, TS = 4, UPR = C / 8, WAVES = H, NCK = 32 / (64 / UPR);
+  const size_t lds = (size_t)(2 * TS * NCK * 65 + ST * 2 * 64 + 4 * 64) * 16 + (size_t)blob_plan(C, S).nfloat * 4;
   int rc = allow_dynamic_lds(project_softmax_kernel<C, S, FUSED>, lds);
   if (rc) return rc;
   const int64_t tpb = tiles_per_batch(s);
@@ -915,24 +1032,27 @@ int slice_reduce(const pa_shape &s, const void *w_pack, const void *fx_pack, flo
 }
 
 template <int S>
-static int slice_attention_s(const pa_shape &s, const float *combined, const float *w_qkv, float *slice_token,
-                             float *slice_norm, float *out_token, void *tokp, hipStream_t st) {
+static int slice_attention_s(const pa_shape &s, const float *combined, const float *fx_bias, const float *w_qkv,
+                             float *slice_token, float *slice_norm, float *out_token, void *tokp, hipStream_t st) {
   hipLaunchKernelGGL((slice_attention_kernel<S>), dim3((unsigned)(s.B * s.H)), dim3(64 * ((S + 31) / 32)), 0, st, combined,
-                     w_qkv, slice_token, slice_norm, out_token, static_cast<uint16_t *>(tokp));
+                     fx_bias, w_qkv, slice_token, slice_norm, out_token, static_cast<uint16_t *>(tokp), (int)s.H);
   return launch_status();
 }
 
-// second pass of the reduction + kernel (c); also leaves the attended tokens as bf16 operands of kernel (d)
-int combine_attention(const pa_shape &s, const pa_params &p, const float *partials, int64_t G, float *slice_token,
-                      float *slice_norm, float *out_token, void *tokp, hipStream_t st) {
+// second pass of the reduction + kernel (c); also leaves the attended tokens as bf16 operands of kernel (d).
+// fx_bias: the in_project_fx bias when the partials come from project_softmax_kernel (which sums fx_mid without it),
+// NULL when the summed values already carry their bias.
+int combine_attention(const pa_shape &s, const pa_params &p, const float *fx_bias, const float *partials, int64_t G,
+                      float *slice_token, float *slice_norm, float *out_token, void *tokp, hipStream_t st) {
   const float *combined = nullptr;
   int rc = pa::general::combine_partials(s, partials, G, &combined, st);
   if (rc) return rc;
+  const float *wq = p.qkv_project_weight;
   switch (s.S) {
-    case 16: return slice_attention_s<16>(s, combined, p.qkv_project_weight, slice_token, slice_norm, out_token, tokp, st);
-    case 32: return slice_attention_s<32>(s, combined, p.qkv_project_weight, slice_token, slice_norm, out_token, tokp, st);
-    case 64: return slice_attention_s<64>(s, combined, p.qkv_project_weight, slice_token, slice_norm, out_token, tokp, st);
-    case 128: return slice_attention_s<128>(s, combined, p.qkv_project_weight, slice_token, slice_norm, out_token, tokp, st);
+    case 16: return slice_attention_s<16>(s, combined, fx_bias, wq, slice_token, slice_norm, out_token, tokp, st);
+    case 32: return slice_attention_s<32>(s, combined, fx_bias, wq, slice_token, slice_norm, out_token, tokp, st);
+    case 64: return slice_attention_s<64>(s, combined, fx_bias, wq, slice_token, slice_norm, out_token, tokp, st);
+    case 128: return slice_attention_s<128>(s, combined, fx_bias, wq, slice_token, slice_norm, out_token, tokp, st);
     default: return PA_ERR_UNSUPPORTED;
   }
 }

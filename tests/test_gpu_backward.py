@@ -171,7 +171,9 @@ def test_bf16_mfma_backward_matches_oracle_and_general_path(B, N, C, S):
         # kernels keep sum_s d l = 0 per point (weights renormalised / softmax re-formed in float32), which holds it
         # to the bar of the tensor-valued gradients
         assert_rel_l2(got[name], want[name], f"MFMA bf16 grad {name} vs fp32 oracle", tol=3e-2)
-        assert_rel_l2(got[name], general[name], f"MFMA vs general bf16 grad {name}", tol=3e-2)
+        # two bf16 paths, each within 3e-2 of the oracle: their mutual distance may reach the sum for the H scalars
+        assert_rel_l2(got[name], general[name], f"MFMA vs general bf16 grad {name}",
+                      tol=6e-2 if name == "temperature" else 3e-2)
     t = got["temperature"].flatten().cpu()
     assert t[0] == 0.0  # 0.3 is below the clamp: no gradient
 
