@@ -46,6 +46,10 @@ def parse_args():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy (known traffic) so FETCH_SIZE / WRITE_SIZE can be scaled")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="target CPU time of the baseline leg")
+    ap.add_argument("--no-sweep", action="store_true", help="skip the slice_num sweep of the layer workload")
+    ap.add_argument("--write-traffic", nargs=2, metavar=("FETCH_DIR", "WRITE_DIR"),
+                    help="no GPU work: read the counter files of two rocprofv3 --pmc runs of this script (FETCH_SIZE, "
+                         "WRITE_SIZE, both with --calibrate-copy) and write profiles/hbm_traffic.json")
     return ap.parse_args()
 
 
@@ -297,26 +301,52 @@ def time_variants(points, C, S, reps=5):
     return out
 
 
-def time_full_model(name, B, N, functional_dim, embedding_dim, slice_num, n_layers, steps=5, warmup=2, n_hidden=256,
-                    fp8_weights=False, graph=True):
-    """Forward of a whole Transolver (bf16 autocast, random-init weights, synthetic N(0,1) inputs) -> Mpoints/s.
+def synthetic_points(kind, B, N, gen):
+    """Point coordinates of the full-model workloads (CPU, float32): "annulus" -- uniform in the annulus 0.5 <= r <= 1
+    (2 coordinates); "surface" -- an ellipsoid (1, 0.6, 0.4) perturbed by two low-order harmonics, with unit normals
+    (3 + 3); "box" -- uniform in the unit cube (3)."""
+    import torch
 
-    The PhysicsAttention layers, the block MLPs, their residual adds and the LayerNorms between them run in the HIP
-    library; the remaining glue (preprocess MLP, first LayerNorm, output Linear) is PyTorch-ROCm.
+    if kind == "annulus":
+        r = torch.sqrt(torch.empty(B, N).uniform_(0.25, 1.0, generator=gen))
+        th = torch.empty(B, N).uniform_(0, 2 * math.pi, generator=gen)
+        return torch.stack((r * torch.cos(th), r * torch.sin(th)), -1)
+    if kind == "surface":
+        th = torch.acos(torch.empty(B, N).uniform_(-1, 1, generator=gen))
+        ph = torch.empty(B, N).uniform_(0, 2 * math.pi, generator=gen)
+        rad = 1 + 0.1 * (3 * torch.cos(th) ** 2 - 1) / 2 + 0.05 * torch.sin(th) ** 2 * torch.cos(th) * torch.cos(2 * ph)
+        xyz = torch.stack((1.0 * rad * torch.sin(th) * torch.cos(ph), 0.6 * rad * torch.sin(th) * torch.sin(ph),
+                           0.4 * rad * torch.cos(th)), -1)
+        nrm = torch.nn.functional.normalize(xyz / torch.tensor([1.0, 0.36, 0.16]), dim=-1)
+        return torch.cat((xyz, nrm), -1)
+    if kind == "box":
+        return torch.rand(B, N, 3, generator=gen)
+    raise ValueError(kind)
+
+
+def time_full_model(name, B, N, functional_dim, points, slice_num, n_layers, steps=5, warmup=2, n_hidden=256,
+                    fp8_weights=False, graph=True):
+    """Forward of a whole Transolver (bf16 autocast, random-init weights, synthetic inputs: coordinates from
+    `synthetic_points(points, ...)`, N(0,1) fields) -> Mpoints/s.
+
+    The PhysicsAttention layers, the block MLPs, their residual adds and the LayerNorms between them, the preprocess
+    MLP, the first LayerNorm and the output Linear run in the HIP library; PyTorch-ROCm only concatenates the inputs.
+    `fp8_weights`: every block's large weights (attention projections and MLP Linears) as fp8-e4m3 with
+    per-output-channel scales.
     """
     import torch
 
     import physicsnemo_amd as pn
 
     torch.manual_seed(0)
-    model = pn.Transolver(functional_dim=functional_dim, embedding_dim=embedding_dim, out_dim=4, n_layers=n_layers,
-                          n_hidden=n_hidden, n_head=n_hidden // 32, slice_num=slice_num, use_te=False).eval().cuda()
-    if fp8_weights:  # the layers' three large weights as fp8-e4m3 bytes with per-output-channel scales
-        for blk in model.blocks:
-            blk.Attn.use_fp8_weights(True)
     g = torch.Generator().manual_seed(1234)
-    fx = torch.randn(B, N, functional_dim, generator=g).cuda()
-    emb = torch.randn(B, N, embedding_dim, generator=g).cuda()
+    emb = synthetic_points(points, B, N, g)
+    fx = torch.randn(B, N, functional_dim, generator=g)
+    model = pn.Transolver(functional_dim=functional_dim, embedding_dim=emb.shape[-1], out_dim=4, n_layers=n_layers,
+                          n_hidden=n_hidden, n_head=n_hidden // 32, slice_num=slice_num, use_te=False).eval().cuda()
+    if fp8_weights:
+        model.use_fp8_weights(True)
+    fx, emb = fx.cuda(), emb.cuda()
     def fwd(a, b):
         with torch.autocast("cuda", dtype=torch.bfloat16):
             return model(a, b)
@@ -336,6 +366,8 @@ def time_full_model(name, B, N, functional_dim, embedding_dim, slice_num, n_laye
         dt, out = timed(fwd)
         assert torch.isfinite(out.float()).all()
         res = {"workload": name, "batch": B, "points": N, "layers": n_layers, "hidden": n_hidden, "slice_num": slice_num,
+               "inputs": f"{points} coordinates + {functional_dim} N(0,1) field(s)",
+               "weights": "fp8-e4m3 per-output-channel (attention projections + MLP Linears)" if fp8_weights else "bf16",
                "ms_per_forward": round(dt * 1e3, 3), "mpoints_per_s": round(B * N / dt / 1e6, 2)}
         if graph:
             graphed = pn.GraphedForward(fwd, fx, emb)  # the same forward replayed from a HIP graph
@@ -388,97 +420,147 @@ def time_structured_model(steps=5, warmup=2):
             "mpoints_per_s_graph": round(4 * 7225 / dt_graph / 1e6, 2)}
 
 
-def main():
-    args = parse_args()
-    if args.gpus != 1:
-        print(f"bench.py measures one GPU only (got --gpus {args.gpus}): this build has no multi-GPU path; "
-              "run with --gpus 1.", file=sys.stderr)
-        sys.exit(2)
+def source_stamp():
+    """Hash of the kernel sources the traffic figures were measured with (the snapshot on the GPU box has no git
+    metadata, so the stamp is taken from the files themselves)."""
+    import hashlib
+
+    h = hashlib.sha256()
+    for name in ("pa_mfma.hip", "pa_mfma_ops.h"):
+        with open(os.path.join(ROOT, "physicsnemo_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+
+
+def measured_traffic(kernel, B, N, C, S):
+    """HBM bytes per launch of `kernel` from the committed rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE summary, or None when
+    the summary was taken with other kernel sources or another workload than the ones running now."""
+    try:
+        with open(TRAFFIC_FILE) as f:
+            rec = json.load(f)
+    except (OSError, ValueError):
+        return None
+    if rec.get("source_stamp") != source_stamp():
+        return None
+    key = f"{kernel}:B{B}:N{N}:C{C}:S{S}"
+    ent = rec.get("kernels", {}).get(key)
+    return None if ent is None else int(ent["hbm_bytes"])
+
+
+def write_traffic(fetch_dir, write_dir, B, N, C, S):
+    """Turns two rocprofv3 --pmc runs of this script (FETCH_SIZE, then WRITE_SIZE; --calibrate-copy adds a plain 1 GiB
+    copy of known traffic that fixes the scale of each counter) into profiles/hbm_traffic.json."""
+    import csv
+    import glob
+
+    def per_kernel(d, counter):
+        acc = {}
+        for fn in glob.glob(os.path.join(d, "**", "*counter_collection.csv"), recursive=True):
+            with open(fn) as f:
+                for r in csv.DictReader(f):
+                    if r["Counter_Name"] == counter:
+                        acc.setdefault(r["Kernel_Name"], []).append(float(r["Counter_Value"]))
+        return {k: sum(v[-10:]) / len(v[-10:]) for k, v in acc.items()}
+
+    fetch, write = per_kernel(fetch_dir, "FETCH_SIZE"), per_kernel(write_dir, "WRITE_SIZE")
+    copy = [k for k in fetch if "copyBuffer" in k]
+    if not copy:
+        raise SystemExit("no calibration copy in the counter files: run the profiled command with --calibrate-copy")
+    f_scale = (1 << 20) / fetch[copy[0]]   # KiB the copy really read / KiB the counter reports
+    w_scale = (1 << 20) / write[copy[0]]
+    names = {"project_softmax_reduce": ("project_softmax_kernel", ", true>"), "project_softmax": ("project_softmax_kernel", ", false>"),
+             "slice_reduce": ("slice_reduce_kernel", ""), "deslice_project": ("deslice_project_kernel", "")}
+    out = {"source_stamp": source_stamp(), "fetch_scale": round(f_scale, 4), "write_scale": round(w_scale, 4),
+           "kernels": {}}
+    for short, (frag, tail) in names.items():
+        hits = [k for k in fetch if frag in k and tail in k]
+        if not hits:
+            continue
+        k = hits[0]
+        rd, wr = fetch[k] * f_scale * 1024, write.get(k, 0.0) * w_scale * 1024
+        out["kernels"][f"{short}:B{B}:N{N}:C{C}:S{S}"] = {"kernel": k, "hbm_read_bytes": int(rd), "hbm_write_bytes": int(wr),
+                                                          "hbm_bytes": int(rd + wr)}
+    with open(TRAFFIC_FILE, "w") as f:
+        json.dump(out, f, indent=1)
+    print(json.dumps(out, indent=1))
+
+
+def measure_layer(B, N, C, S, steps, warmup, kernel_reps, x_cpu=None, cold=False):
+    """One PhysicsAttentionIrregularMesh layer at (B, N, C, S), bf16: whole-layer time through the module and the C ABI,
+    the same call replayed from a HIP graph, and every kernel of the layer timed on its own."""
     import torch
 
     import physicsnemo_amd as pn
     from physicsnemo_amd import functional as PF
 
-    if not torch.cuda.is_available():
-        print("bench.py needs a GPU (no CPU path exists for the product)", file=sys.stderr)
-        sys.exit(2)
     dev = torch.device("cuda:0")
-    B, N, C, S = args.batch, args.points, args.hidden, args.slices
     H = C // 32
     torch.manual_seed(0)
     layer = pn.PhysicsAttentionIrregularMesh(C, heads=H, dim_head=32, slice_num=S, use_te=False).eval()
     state = {k: v.clone() for k, v in layer.state_dict().items()}
     layer = layer.to(dev)
-    gen = torch.Generator().manual_seed(1234)
-    x_cpu = torch.randn(B, N, C, generator=gen)
+    if x_cpu is None:
+        x_cpu = torch.randn(B, N, C, generator=torch.Generator().manual_seed(1234))
     x = x_cpu.to(dev).bfloat16().contiguous()
     dims = layer.layer_dims(x)
     path = PF.query_path(torch.bfloat16, dims)
+    res = {"state": state, "path": path}
 
-    global SETTLE_MS
-    SETTLE_MS = args.settle_ms
-    with torch.no_grad():
-        run_in(lambda: layer(x))
-        for _ in range(args.warmup):
+    def timed_steps():
+        for _ in range(warmup):
             y = layer(x)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        for _ in range(args.steps):
+        for _ in range(steps):
             y = layer(x)
         torch.cuda.synchronize()
-        elapsed = time.perf_counter() - t0
-    ms_per_step = elapsed / args.steps * 1e3
-    mpoints = B * N / (ms_per_step * 1e-3) / 1e6
+        return (time.perf_counter() - t0) / steps * 1e3, y
+
+    with torch.no_grad():
+        if cold:
+            # the plain procedure -- `warmup` untimed calls, then `steps` timed ones -- straight after an idle spell:
+            # it includes the clock governor's transient of the first ~20 ms of load
+            layer(x)
+            torch.cuda.synchronize()
+            time.sleep(0.5)
+            res["ms_per_step_cold"], _ = timed_steps()
+        run_in(lambda: layer(x))
+        res["ms_per_step"], y = timed_steps()
     assert torch.isfinite(y[:, :1024].float()).all()
 
-    # the same call recorded once into a HIP graph and replayed (same kernels, one submission per step)
-    graphed = pn.GraphedForward(layer, x)  # its static input holds a copy of x
+    graphed = pn.GraphedForward(layer, x)  # the same call recorded once into a HIP graph and replayed
     run_in(graphed.replay)
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         graphed.replay()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    for _ in range(steps):
         graphed.replay()
     torch.cuda.synchronize()
-    ms_graph = (time.perf_counter() - t0) / args.steps * 1e3
+    res["ms_graph"] = (time.perf_counter() - t0) / steps * 1e3
     del graphed
 
-    if args.calibrate_copy:
-        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
-        dst = torch.empty_like(src)
-        for _ in range(3):
-            dst.copy_(src)
-        torch.cuda.synchronize()
-        del src, dst
-
-    kernels = {}
-    roofline = None
+    kernels, roofline = {}, None
     if path == 1:
         params = layer.kernel_params(torch.bfloat16, dev)
         st = PF.MfmaStages(params, dims, dev)
         yk = torch.empty_like(x)
         st.pack_params()
         fused = st.fused_groups > 0  # the layer call runs kernels (a)+(b) as one launch
-        stage_fns = {}
+        stage_fns = {"project_softmax": lambda: st.project_softmax(x), "slice_reduce": st.slice_reduce}
         if fused:  # the separate kernels first, so that the later stages time on the layer path's partials
-            stage_fns["project_softmax"] = lambda: st.project_softmax(x)
-            stage_fns["slice_reduce"] = st.slice_reduce
             stage_fns["project_softmax_reduce"] = lambda: st.project_softmax_reduce(x)
-        else:
-            stage_fns["project_softmax"] = lambda: st.project_softmax(x)
-            stage_fns["slice_reduce"] = st.slice_reduce
-        stage_fns.update({
-            "combine_attention": st.combine_attention,
-            "deslice_project": lambda: st.deslice_project(yk),
-            "pack_params": st.pack_params,
-        })
+        stage_fns.update({"combine_attention": st.combine_attention, "deslice_project": lambda: st.deslice_project(yk),
+                          "pack_params": st.pack_params})
         on_path = ({"project_softmax_reduce", "deslice_project"} if fused else
                    {"project_softmax", "slice_reduce", "deslice_project"})
         bytes_pp = algorithmic_bytes_per_point(C, H, S)
         flops_pp = mfma_flops_per_point(C, S)
         for name, fn in stage_fns.items():
-            ms = time_kernel(fn, args.kernel_reps)
+            ms = time_kernel(fn, kernel_reps)
             entry = {"ms": round(ms, 4)}
             if name in bytes_pp:
                 gbs = bytes_pp[name] * B * N / (ms * 1e-3) / 1e9
@@ -490,39 +572,97 @@ def main():
             entry["on_layer_path"] = name in on_path or name == "combine_attention"
             kernels[name] = entry
         dominant = max(on_path, key=lambda k: kernels[k]["ms"])
-        # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a 1 GiB copy (x2.0 / x1.0);
-        # measured for the default workload only (profiles/layer_cfg3_s64_hbm_traffic.md)
-        measured_traffic = {"project_softmax_reduce": (517 + 1041) << 20, "project_softmax": (542 + 1536) << 20, "slice_reduce": (1536 + 8) << 20,
-                            "deslice_project": (1025 + 512) << 20}
-        default_workload = (B, N, C, S) == (1, 1 << 20, 256, 64)
         roofline = {"kernel": dominant, "bound": "hbm", "achieved": kernels[dominant]["hbm_gbs"], "peak": HBM_PEAK_GBS,
                     "unit": "GB/s", "frac": kernels[dominant]["hbm_frac"],
-                    "traffic": measured_traffic[dominant] if default_workload else None}
+                    "traffic": measured_traffic(dominant, B, N, C, S)}
+        del st, yk
+    res.update({"kernels": kernels, "roofline": roofline, "H": H})
+    del layer, x
+    torch.cuda.empty_cache()
+    return res
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU only (got --gpus {args.gpus}): this build has no multi-GPU path; "
+              "run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+    B, N, C, S = args.batch, args.points, args.hidden, args.slices
+    if args.write_traffic:
+        write_traffic(args.write_traffic[0], args.write_traffic[1], B, N, C, S)
+        return
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (no CPU path exists for the product)", file=sys.stderr)
+        sys.exit(2)
+    dev = torch.device("cuda:0")
+    H = C // 32
+    global SETTLE_MS
+    SETTLE_MS = args.settle_ms
+    gen = torch.Generator().manual_seed(1234)
+    x_cpu = torch.randn(B, N, C, generator=gen)
+    m = measure_layer(B, N, C, S, args.steps, args.warmup, args.kernel_reps, x_cpu=x_cpu, cold=True)
+    ms_per_step, path, kernels = m["ms_per_step"], m["path"], m["kernels"]
+    mpoints = B * N / (ms_per_step * 1e-3) / 1e6
+
+    if args.calibrate_copy:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+
+    def layer_fracs(bn, c, s, ms):
+        """Whole-layer HBM fractions: against the fused floor (x read twice, y written once: 3 C b bytes per point) and
+        against the four-kernel contract dataflow ((3 H S + 5 C) b bytes per point)."""
+        floor_b, contract_b = 3 * c * 2, (3 * (c // 32) * s + 5 * c) * 2
+        t = ms * 1e-3
+        return {"roofline_vs_floor": round(floor_b * bn / t / 1e9 / HBM_PEAK_GBS, 4),
+                "vs_contract": round(contract_b * bn / t / 1e9 / HBM_PEAK_GBS, 4),
+                "floor_bytes_per_point": floor_b, "contract_bytes_per_point": contract_b}
 
     out = {
         "metric": "Mpoints/s per PhysicsAttention layer at 1M pts bf16; % HBM/MFMA roofline",
         "value": round(mpoints, 2), "unit": "Mpoints/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "settle_ms": args.settle_ms, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "settle_ms": args.settle_ms, "ms_per_step": round(ms_per_step, 4),
+        "ms_per_step_cold": round(m["ms_per_step_cold"], 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "cfg3: single PhysicsAttentionIrregularMesh layer forward", "batch": B, "points": N,
                    "hidden": C, "heads": H, "dim_head": 32, "slice_num": S,
                    "kernel_path": {0: "general", 1: "mfma", 2: "mfma-staged"}[path]},
-        "roofline": roofline, "kernels": kernels,
-        "graph_replay": {"ms_per_step": round(ms_graph, 4), "mpoints_per_s": round(B * N / (ms_graph * 1e-3) / 1e6, 2)},
+        "roofline": m["roofline"], "kernels": kernels, "layer": layer_fracs(B * N, C, S, ms_per_step),
+        "graph_replay": {"ms_per_step": round(m["ms_graph"], 4),
+                         "mpoints_per_s": round(B * N / (m["ms_graph"] * 1e-3) / 1e6, 2)},
     }
+    if not args.no_sweep:
+        # cfg3's slice sweep: the same layer and points at every slice count (the headline count taken from above)
+        sweep = []
+        for s_k in (16, 32, 64, 128):
+            mk = m if s_k == S else measure_layer(B, N, C, s_k, args.steps, args.warmup, max(5, args.kernel_reps // 2))
+            e = {"slice_num": s_k, "ms_per_step": round(mk["ms_per_step"], 4),
+                 "mpoints_per_s": round(B * N / (mk["ms_per_step"] * 1e-3) / 1e6, 2),
+                 "kernels": {k: {f: v[f] for f in ("ms", "hbm_frac", "mfma_frac") if f in v}
+                             for k, v in mk["kernels"].items() if v.get("on_layer_path")}}
+            e.update(layer_fracs(B * N, C, s_k, mk["ms_per_step"]))
+            sweep.append(e)
+        out["slice_sweep"] = sweep
     if not args.no_models:
         out["block_mlp"] = time_block_mlp(1 << 20, 256, 1024)
         out["training_step"] = time_training_step(N, C, S)
         out["variants"] = time_variants(N, C, S)
         out["full_model"] = [
             time_structured_model(),
-            time_full_model("cfg2: Transolver irregular 2D, 8 layers", 8, 32768, 3, 2, 64, 8),
-            time_full_model("cfg4: Transolver 3D surface cloud, 8 layers", 1, 1000000, 1, 6, 32, 8),
-            time_full_model("cfg5: Transolver 3D volume, 12 layers, hidden 512, fp8-e4m3 projection weights", 1, 4194304,
-                            4, 3, 128, 12, steps=2, warmup=1, n_hidden=512, fp8_weights=True, graph=False),
+            time_full_model("cfg2: Transolver irregular 2D, 8 layers", 8, 32768, 3, "annulus", 64, 8),
+            time_full_model("cfg4: Transolver 3D surface cloud, 8 layers", 1, 1000000, 1, "surface", 32, 8),
+            time_full_model("cfg5: Transolver 3D volume, 12 layers, hidden 512, fp8-e4m3 weights", 1, 4194304,
+                            4, "box", 128, 12, steps=2, warmup=1, n_hidden=512, fp8_weights=True, graph=False),
         ]
     if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(state, x_cpu, C, H, S, args.cpu_seconds)
+        out["cpu_baseline"] = cpu_baseline(m["state"], x_cpu, C, H, S, args.cpu_seconds)
     print(json.dumps(out), flush=True)
 
 

@@ -768,11 +768,19 @@ __global__ __launch_bounds__(C * 2) void deslice_project_kernel(const u32x4 *__r
     }
     const int64_t n0 = t * 32;
     // deslice this wave's head (last use of wcur)
-    f32x16 ox;
+    // (two interleaved accumulation chains: a dependent MFMA would wait for its predecessor's last pass)
+    f32x16 ox, ox2;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) ox[r] = 0.f;
+    for (int r = 0; r < 16; ++r) ox[r] = ox2[r] = 0.f;
 #pragma unroll
-    for (int cq = 0; cq < NCH; ++cq) ox = mma(tps[(wave * NCH + cq) * 64 + lane], wcur[cq], ox);
+    for (int cq = 0; cq < NCH; cq += 2) {
+      ox = mma(tps[(wave * NCH + cq) * 64 + lane], wcur[cq], ox);
+      if (cq + 1 < NCH) ox2 = mma(tps[(wave * NCH + cq + 1) * 64 + lane], wcur[cq + 1], ox2);
+    }
+    if constexpr (NCH > 1) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) ox[r] += ox2[r];
+    }
     // fetch the next item's slice weights and residual rows (the last iteration re-fetches its own)
     const int64_t item_next = item + gridDim.x;
     const bool more = !MASKED && item_next < total_items;
@@ -795,9 +803,12 @@ __global__ __launch_bounds__(C * 2) void deslice_project_kernel(const u32x4 *__r
     oxs[(wave * 2 + 1) * 64 + lane] = pack_half<1>(ox);
     __syncthreads();
     // this wave's 32 output channels
-    f32x16 acc;
+    f32x16 acc, acc2;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) acc[r] = bias;
+    for (int r = 0; r < 16; ++r) {
+      acc[r] = bias;
+      acc2[r] = 0.f;
+    }
 #pragma unroll
     for (int hh = 0; hh < H; hh += 4) {
       u32x4 of[4][2];
@@ -810,11 +821,11 @@ __global__ __launch_bounds__(C * 2) void deslice_project_kernel(const u32x4 *__r
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         acc = mma(of[q][0], wout[hh + q][0], acc);
-        acc = mma(of[q][1], wout[hh + q][1], acc);
+        acc2 = mma(of[q][1], wout[hh + q][1], acc2);
       }
     }
 #pragma unroll
-    for (int r = 0; r < 16; ++r) ys[rowmap(r, g) * YS + wave * 32 + i] = acc[r];
+    for (int r = 0; r < 16; ++r) ys[rowmap(r, g) * YS + wave * 32 + i] = acc[r] + acc2[r];
     __syncthreads();
     // finish ROWS full rows per wave
 #pragma unroll
