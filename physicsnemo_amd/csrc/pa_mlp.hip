@@ -69,15 +69,19 @@ __global__ __launch_bounds__(256) void pack_kernel(const uint16_t *__restrict__ 
   }
 }
 
-// One direct global -> LDS load of 64 x 16 bytes (no registers): the wave's lanes read sbase + voff (voff = 16 * lane)
-// and the data land at LDS byte address lds + 16 * lane.  sbase and lds are wave-uniform.  The load is asynchronous
-// and counted by vmcnt; its data must not be read before a wait and a barrier.
-__device__ __forceinline__ void load_to_lds(const void *sbase, unsigned voff, unsigned lds) {
+// Four direct global -> LDS loads of 64 x 16 bytes each (no registers): the wave's lanes read sbase + 1024 q + 16 lane
+// (q = 0..3) and the data land at LDS byte address lds + 1024 q + 16 lane; the instruction offset advances the
+// global and the LDS address alike.  sbase and lds are wave-uniform.  The loads are asynchronous and counted by
+// vmcnt; their data must not be read before a wait and a barrier.
+__device__ __forceinline__ void load_4k_to_lds(const void *sbase, unsigned lane16, unsigned lds) {
   asm volatile(
       "s_mov_b32 m0, %2\n\t"
       "s_nop 0\n\t"
-      "global_load_lds_dwordx4 %1, %0" ::"s"(sbase),
-      "v"(voff), "s"(lds)
+      "global_load_lds_dwordx4 %1, %0\n\t"
+      "global_load_lds_dwordx4 %1, %0 offset:1024\n\t"
+      "global_load_lds_dwordx4 %1, %0 offset:2048\n\t"
+      "global_load_lds_dwordx4 %1, %0 offset:3072" ::"s"(sbase),
+      "v"(lane16), "s"(lds)
       : "memory");
 }
 
@@ -90,8 +94,6 @@ template <int N, class F>
 __device__ __forceinline__ void static_for(F &&f) {
   static_for_impl(f, std::make_integer_sequence<int, N>{});
 }
-
-__device__ __forceinline__ float gelu(float x) { return gelu_logistic(x); }
 
 // 8 floats -> 8 bf16 (round to nearest even)
 __device__ __forceinline__ u32x4 pack8(const float (&v)[8]) {
@@ -115,6 +117,18 @@ __device__ __forceinline__ float half_wave_sum(float v) {
   const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
   return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
+
+#ifdef PA_PROFILE
+__device__ unsigned long long pa_prof[256 * 4 * 12];  // [workgroup][wave][interval]
+#define PA_T(k)                                                   \
+  do {                                                            \
+    const unsigned long long now_ = __builtin_readcyclecounter(); \
+    pacc[k] += now_ - tlast;                                      \
+    tlast = now_;                                                 \
+  } while (0)
+#else
+#define PA_T(k) do { } while (0)
+#endif
 
 template <int C, int TAIL>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void mlp_kernel(
@@ -150,12 +164,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     bet[k] = HAS_LN ? ln_beta[i * CPH + k] : 0.f;
   }
 
-  static_assert(NDMA == KS, "one direct-to-LDS load per step of the first phase");
-  // piece q of this wave's share of slot c into buffer gs & 1
-  auto fetch_piece = [&](int64_t gs, int c, int q) {
-    const u32x4 *src = blob + (int64_t)c * SU + wave * WU + q * 64;
-    const unsigned dst = (unsigned)(uintptr_t)(wbuf + (gs & 1) * SU + wave * WU + q * 64);
-    load_to_lds(src, lane * 16, dst);
+  static_assert(NDMA % 4 == 0 && NDMA / 4 <= KS / 4, "the fetch of a slot is issued in groups of four loads");
+  // pieces 4k .. 4k+3 (1 KB each) of this wave's share of slot c into buffer gs & 1
+  auto fetch_quad = [&](int64_t gs, int c, int k) {
+    const u32x4 *src = blob + (int64_t)c * SU + wave * WU + k * 256;
+    const unsigned dst = (unsigned)(uintptr_t)(wbuf + (gs & 1) * SU + wave * WU + k * 256);
+    load_4k_to_lds(src, lane * 16, dst);
   };
   auto load_rows = [&](int64_t mb, u32x4(&ub)[2][KS]) {  // the pair's rows of block mb as B operands
     const int64_t row0 = mb * kRowsPerBlock + rg * 64;
@@ -170,9 +184,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   };
 
   int64_t gs = 0;  // slots processed so far by this workgroup (buffer parity)
+#ifdef PA_PROFILE
+  unsigned long long pacc[12] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+  unsigned long long tlast = __builtin_readcyclecounter();
+  const unsigned long long t_begin = tlast, w_begin = wall_clock64();
+#endif
   if ((int64_t)blockIdx.x < nblocks) {
 #pragma unroll
-    for (int q = 0; q < NDMA; ++q) fetch_piece(0, 0, q);
+    for (int k = 0; k < NDMA / 4; ++k) fetch_quad(0, 0, k);
   }
   // lane (i, g) holds row 32m + i, channels 16ks + 8g .. + 7
   u32x4 ub[2][KS];
@@ -189,20 +208,39 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     // gelu(h) of hidden chunk c-1 as B operands [m][kk]: this wave's tile and the partner's
     u32x4 hown[2][2], hpar[2][2];
     float hrest[2][8];  // second half (registers 8..15) of this wave's h tile of chunk c-1, before the activation
+    float fl[2][8];     // gelu of the first half (registers 0..7) of the tile of chunk c
+    // The 32 activations of a slot (evaluation e: e < 16 -> hrest[e / 8][e % 8], else the first half of hacc) are
+    // spread over its 32 / NE steps and software-pipelined over three half-steps, so that two independent
+    // dependency chains are in flight behind every MFMA (a wave is alone on its SIMD and issues in order: a single
+    // chain would leave its latencies exposed):
+    //   behind the first MFMA of step s:      end of evaluation s - 1 (1 + e, rcp, x *)  |  start of evaluation s
+    //   behind the second MFMA of step s:     polynomial and exp2 of evaluation s; one piece of the next slot's fetch
+    // The last evaluation of a slot ends in the first step of the next one.
+    constexpr int NE = 16 / KS > 0 ? 16 / KS : 1;  // evaluations per step
+    constexpr int NS1 = KS, NS2 = 4 * CTH;
+    static_assert(NS1 * NE == 16 && NS2 * NE == 16, "both phases must cover 16 evaluations");
+    float px[NE], pe[NE];           // evaluation in its last part: argument, exp2 term
+    float cx[NE], cx2[NE], cq[NE];  // evaluation in its first parts: argument, min(x^2, 81), polynomial so far
+    // nothing of the block before may reach this one (its last slot evaluates what the zero weights of the padding
+    // slot produce from its rows: finite only if those rows are)
+#pragma unroll
+    for (int q = 0; q < NE; ++q) px[q] = pe[q] = 0.f;
 #pragma unroll
     for (int m = 0; m < 2; ++m) {
       hown[m][0] = u32x4{0, 0, 0, 0};
 #pragma unroll
-      for (int j = 0; j < 8; ++j) hrest[m][j] = 0.f;
+      for (int j = 0; j < 8; ++j) hrest[m][j] = fl[m][j] = 0.f;
     }
 
     for (int c = 0; c <= NC; ++c, ++gs) {
       // slot gs has landed (every wave waits for its own share, then all meet) and the other buffer is free.  The
       // first slot of a later block was waited for before the epilogue of the block before it, whose stores may
       // still be in flight here.
+      PA_T(0);
       if (c > 0 || gs == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      PA_T(1);
       __syncthreads();
-      const bool has_next = c < NC || mb + gridDim.x < nblocks;
+      PA_T(2);
       const int c_next = c < NC ? c + 1 : 0;
       const u32x4 *wb = wbuf + (gs & 1) * SU + lane;
       // this wave's fragments of the slot: W1 of hidden tile p; W2 of its channel half, hidden tile p ("own") first
@@ -210,7 +248,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
       const u32x4 *w2own = wb + (NF1 + p * CTH * 4 + 2 * p) * 64, *w2par = wb + (NF1 + p * CTH * 4 + 2 * (1 - p)) * 64;
 
       // One slot = 2 phases of KS resp. 4 * CTH steps; a step = one weight fragment (read from LDS AHEAD steps
-      // early), two MFMAs and, behind them, one or two gelu evaluations:
+      // early) and two MFMAs with the vector work of the activations behind each:
       //   phase 1   h^T tile p of hidden chunk c += W1 fragment . u^T (both row halves);
       //             gelu of the second half of the tile of chunk c-1 -> the tile is complete, goes to the partner
       //   phase 2   y^T += W2 fragment(ct, k4) of hidden chunk c-1 . gelu(h)^T (own tile, then the partner's);
@@ -219,79 +257,105 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
       f32x16 hacc[2];
 #pragma unroll
       for (int r = 0; r < 16; ++r) hacc[0][r] = hacc[1][r] = b1s[(c < NC ? 64 * c : 0) + 32 * p + rowmap(r, g)];
-      {
-        constexpr int EV = 16 / KS > 0 ? 16 / KS : 1;  // evaluations per step (16 over KS steps)
-        static_assert(KS * EV == 16 || KS == 16, "phase 1 must cover 16 evaluations");
-        u32x4 fr[RING];
-        static_for<AHEAD>([&](auto q) { fr[decltype(q)::value] = w1f[decltype(q)::value * 64]; });
-        // the first fragments and the bias are on their way: now the next slot's fetch, whose issue keeps the wave
-        // busy for a while (its buffer was last read in phase 2 of the slot before this one)
-        if (has_next) {
-#pragma unroll
-          for (int q = 0; q < NDMA; ++q) fetch_piece(gs + 1, c_next, q);
-        }
-        static_for<KS>([&](auto st) {
-          constexpr int step = decltype(st)::value;
-          if constexpr (step + AHEAD < KS) fr[(step + AHEAD) % RING] = w1f[(step + AHEAD) * 64];
-          const u32x4 a = fr[step % RING];
-          hacc[0] = mma(a, ub[0][step], hacc[0]);
-          hacc[1] = mma(a, ub[1][step], hacc[1]);
-          static_for<(KS == 16 ? 1 : 16 / KS)>([&](auto q) {
-            constexpr int E = step * (KS == 16 ? 1 : 16 / KS) + decltype(q)::value, m = E / 8, j = E % 8;
-            hrest[m][j] = gelu(hrest[m][j]);
+      // vector work behind the first MFMA of step S (0 .. NS1 + NS2 - 1 over both phases)
+      auto behind_first = [&](auto S_) {
+        constexpr int S = decltype(S_)::value;
+        static_for<NE>([&](auto q_) {
+          constexpr int q = decltype(q_)::value, e = S * NE + q, ep = (e + 32 - NE) % 32, m = (ep % 16) / 8, j = ep % 8;
+          const float done = px[q] * __builtin_amdgcn_rcpf(1.f + pe[q]);
+          if constexpr (ep < 16) {
+            hrest[m][j] = done;
             if constexpr (j == 7) hown[m][1] = pack8(hrest[m]);
-          });
-          __builtin_amdgcn_sched_barrier(0);  // keeps the issue order as written
+          } else {
+            fl[m][j] = done;
+            if constexpr (j == 7) hown[m][0] = pack8(fl[m]);
+          }
+          if constexpr (e < 16) cx[q] = hrest[e / 8][e % 8];
+          else cx[q] = hacc[(e - 16) / 8][e % 8];
+          cx2[q] = fminf(cx[q] * cx[q], 81.f);
+          cq[q] = fmaf(-3.51902394e-04f * -2.f * kLog2e, cx2[q], 3.70080200e-02f * -2.f * kLog2e);
         });
-      }
-      // the tile of chunk c-1 is complete: hand it to the partner, take the partner's
+      };
+      auto behind_second = [&]() {
 #pragma unroll
-      for (int m = 0; m < 2; ++m)
-#pragma unroll
-        for (int kk = 0; kk < 2; ++kk) xch[((wave * 2 + m) * 2 + kk) * 64 + lane] = hown[m][kk];
+        for (int q = 0; q < NE; ++q) {
+          const float t2 = fmaf(cq[q], cx2[q], 7.97505275e-01f * -2.f * kLog2e);
+          px[q] = cx[q];
+          pe[q] = __builtin_amdgcn_exp2f(cx[q] * t2);
+        }
+      };
       {
-        constexpr int NS2 = 4 * CTH, EV = 16 / NS2 > 0 ? 16 / NS2 : 1;
-        static_assert(NS2 * EV == 16, "phase 2 must cover 16 evaluations");
-        float fl[2][8];
-        u32x4 hfirst[2];
-        auto frag2 = [&](auto st) {  // step -> (k4' = step / CTH, ct = step % CTH); k4' < 2: own tile, kk = k4' % 2
-          constexpr int t = decltype(st)::value, k4 = t / CTH, ct = t % CTH;
-          return (k4 < 2 ? w2own : w2par)[(ct * 4 + (k4 & 1)) * 64];
+        // fragment of step S of the slot: W1 (tile p, k-step S) in phase 1, then W2 with (k4' = t / CTH, ct = t % CTH),
+        // k4' < 2: own tile, kk = k4' % 2
+        auto frag = [&](auto S_) {
+          constexpr int S = decltype(S_)::value;
+          if constexpr (S < NS1) {
+            return w1f[S * 64];
+          } else {
+            constexpr int t = S - NS1, k4 = t / CTH, ct = t % CTH;
+            return (k4 < 2 ? w2own : w2par)[(ct * 4 + (k4 & 1)) * 64];
+          }
         };
-        u32x4 fr[RING];
-        static_for<AHEAD>([&](auto q) { fr[decltype(q)::value] = frag2(q); });
-        static_for<NS2>([&](auto st) {
-          constexpr int t = decltype(st)::value, k4 = t / CTH, ct = t % CTH, kk = k4 & 1;
-          if constexpr (t == 2 * CTH - 2) {  // two steps before the partner's tile (written before phase 2) is needed
+        u32x4 fr[RING];  // one ring over both phases: the first fragments of phase 2 are on their way before phase 1 ends
+        static_for<AHEAD>([&](auto q) { fr[decltype(q)::value] = frag(q); });
+        static_for<NS1 + NS2>([&](auto S_) {
+          constexpr int S = decltype(S_)::value;
+          if constexpr (S == NS1) PA_T(3);
+          if constexpr (S == NS1 + 2 * CTH - 2) {  // two steps before the partner's tile (written in step NS1) is needed
             __syncthreads();
 #pragma unroll
             for (int m = 0; m < 2; ++m)
 #pragma unroll
               for (int k = 0; k < 2; ++k) hpar[m][k] = xch[(((wave ^ 1) * 2 + m) * 2 + k) * 64 + lane];
           }
-          if constexpr (t + AHEAD < NS2) fr[(t + AHEAD) % RING] = frag2(std::integral_constant<int, t + AHEAD>{});
-          const u32x4 a = fr[t % RING];
-          yacc[0][ct] = mma(a, k4 < 2 ? hown[0][kk] : hpar[0][kk], yacc[0][ct]);
-          yacc[1][ct] = mma(a, k4 < 2 ? hown[1][kk] : hpar[1][kk], yacc[1][ct]);
-          static_for<EV>([&](auto q) {
-            constexpr int E = t * EV + decltype(q)::value, m = E / 8, j = E % 8;
-            fl[m][j] = gelu(hacc[m][j]);
-            if constexpr (j == 7) hfirst[m] = pack8(fl[m]);
-          });
-          __builtin_amdgcn_sched_barrier(0);
-        });
+          if constexpr (S + AHEAD < NS1 + NS2) fr[(S + AHEAD) % RING] = frag(std::integral_constant<int, S + AHEAD>{});
+          const u32x4 a = fr[S % RING];
+          if constexpr (S < NS1) {
+            hacc[0] = mma(a, ub[0][S], hacc[0]);
+            __builtin_amdgcn_sched_barrier(0);  // keeps the issue order as written
+            behind_first(S_);
+            __builtin_amdgcn_sched_barrier(0);
+            hacc[1] = mma(a, ub[1][S], hacc[1]);
+            __builtin_amdgcn_sched_barrier(0);
+            behind_second();
+            // the other buffer was last read in phase 2 of the slot before this one
+            if constexpr (S % 4 == 3 && S / 4 < NDMA / 4) fetch_quad(gs + 1, c_next, S / 4);
+            __builtin_amdgcn_sched_barrier(0);
+          } else {
+            constexpr int t = S - NS1, k4 = t / CTH, ct = t % CTH, kk = k4 & 1;
+            // own tile: hown[m][0] (first half of chunk c-1) is read in steps 0 .. CTH-1 and rewritten (chunk c) from
+            // step 8 / NE on; hown[m][1] is complete after the first half-step of step 0 and read from step CTH on
+            yacc[0][ct] = mma(a, k4 < 2 ? hown[0][kk] : hpar[0][kk], yacc[0][ct]);
+            __builtin_amdgcn_sched_barrier(0);
+            behind_first(S_);
+            __builtin_amdgcn_sched_barrier(0);
+            yacc[1][ct] = mma(a, k4 < 2 ? hown[1][kk] : hpar[1][kk], yacc[1][ct]);
+            __builtin_amdgcn_sched_barrier(0);
+            behind_second();
+            if constexpr (t == 0) {
+              // the tile of chunk c-1 is complete: hand it to the partner (who reads it after the barrier above;
+              // the one at the start of the next slot separates that read from the next write)
 #pragma unroll
-        for (int m = 0; m < 2; ++m) {
-          hown[m][0] = hfirst[m];
+              for (int m = 0; m < 2; ++m)
+#pragma unroll
+                for (int k = 0; k < 2; ++k) xch[((wave * 2 + m) * 2 + k) * 64 + lane] = hown[m][k];
+            }
+            __builtin_amdgcn_sched_barrier(0);
+          }
+        });
+        PA_T(4);
+#pragma unroll
+        for (int m = 0; m < 2; ++m)
 #pragma unroll
           for (int j = 0; j < 8; ++j) hrest[m][j] = hacc[m][8 + j];
-        }
       }
     }
 
     // ---- epilogue: the buffer of the last slot is idle once every wave is past its last MFMA ----
+    PA_T(0);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's share of the next block's first slot has landed
     __syncthreads();
+    PA_T(8);
     // the rows of this workgroup's next block travel while the epilogue runs (past the end: this block again)
     load_rows(mb + gridDim.x < nblocks ? mb + gridDim.x : mb, ub);
     uint32_t *stg = reinterpret_cast<uint32_t *>(wbuf + ((gs - 1) & 1) * SU) + rg * 64 * (C / 2);  // [64 rows][C/2 words]
@@ -311,7 +375,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
           pk[1] = (uint32_t)to_bf16_bits(v2) | ((uint32_t)to_bf16_bits(v3) << 16);
           *reinterpret_cast<u32x2 *>(stg + rw * (C / 2) + gr * 2) = pk;
         }
+    PA_T(9);
     __syncthreads();  // both waves of a pair have staged their channel halves
+    PA_T(10);
     // wave p finishes rows 32p .. 32p+31 of the pair, two per step: lanes 0-31 one row, lanes 32-63 the next, CPH
     // consecutive channels per lane (16-byte accesses for C = 256)
     typedef uint32_t rowv __attribute__((ext_vector_type(WPH)));
@@ -369,26 +435,413 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         if (ok) *reinterpret_cast<rowv *>(ln_out + r * C + i * CPH) = lb;
       }
     }
+    PA_T(5);
   }
+#ifdef PA_PROFILE
+  if (lane == 0) {
+    unsigned long long *dstp = pa_prof + ((int)blockIdx.x * 4 + wave) * 12;
+    for (int k = 0; k < 6; ++k) dstp[k] = pacc[k];
+    for (int k = 8; k < 12; ++k) dstp[k] = pacc[k];
+    dstp[6] = __builtin_readcyclecounter() - t_begin;
+    dstp[7] = wall_clock64() - w_begin;
+  }
+#endif
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // nothing may still be landing in LDS when the workgroup ends
 }
 
 // ---------------------------------------------------------------------------------------------------------------
-bool supported(int dtype, int64_t rows, int64_t C, int64_t F) {
-  return dtype == PA_BF16 && rows > 0 && (C == 128 || C == 256) && F >= 64 && F % 64 == 0 && F <= 8192;
+// The same MLP for C = 512 (and, for comparison, 256): every wave owns 32 rows of the block outright.
+//
+// One workgroup of 4 waves per CU, one wave per SIMD; a block is 128 rows.  A wave keeps its rows' inputs (B operands,
+// C/4 registers) and all C output channels of y^T (C/2 accumulation registers) for the whole block and shares nothing
+// but the weight stream with the other waves: no tile exchange, one barrier per slot.  The price is that a weight
+// fragment read from LDS feeds one MFMA only (32 B per cycle and SIMD, half of what LDS delivers).
+//
+// Weights stream through LDS in slots of HS hidden units (HS = 16384 / C: 64 KB of W1 and W2 fragments per slot, two
+// buffers).  The MFMAs of the two products alternate, so that no accumulator is used twice in a row and the vector
+// work of the activation finds an MFMA to hide behind everywhere; the products therefore run two slots apart:
+//   slot c:   h(c)^T = W1[chunk c] . u^T + b1           (first MFMA of every pair)
+//             g(c-1) = gelu(h(c-1)), rounded to bf16: B operands of the second product (vector work, in two or three
+//             parts behind consecutive MFMAs)
+//             y^T   += W2[:, chunk c-2] . g(c-2)^T      (second MFMA of every pair)
+// Slot c of the packed weights holds the fragments in the order they are consumed: pair P = 0..31 -> W1 fragment
+// (tile P % NT, k-step P / NT) of chunk c, then W2 fragment (ct = P % CT, tile and k-half from P / CT) of chunk c-2.
+// ---------------------------------------------------------------------------------------------------------------
+namespace rows {
+
+template <int C>
+struct Cfg {
+  static constexpr int KS = C / 16, CT = C / 32;
+  static constexpr int HS = 16384 / C;  // hidden units per slot
+  static constexpr int NT = HS / 32;    // hidden tiles per slot
+  static constexpr int NP = 32;         // MFMA pairs per slot
+  static constexpr int SU = 2 * NP * 64;  // 16-byte units per slot
+  static_assert(NT * KS == NP && CT * NT * 2 == NP, "both products take 32 MFMAs per slot");
+};
+
+__global__ __launch_bounds__(256) void pack_kernel(const uint16_t *__restrict__ w1, const uint16_t *__restrict__ w2,
+                                                   u32x4 *__restrict__ blob, int C, int F) {
+  const int KS = C / 16, CT = C / 32, HS = 16384 / C, NT = HS / 32, NCH = F / HS;
+  (void)KS;
+  const int64_t total = (int64_t)(NCH + 2) * 4096;
+  for (int64_t u = (int64_t)blockIdx.x * 256 + threadIdx.x; u < total; u += (int64_t)gridDim.x * 256) {
+    const int c = (int)(u >> 12), r = (int)(u & 4095), frag = r >> 6, lane = r & 63, i = lane & 31, g = lane >> 5;
+    const int P = frag >> 1;
+    uint16_t e[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) e[j] = 0;
+    if ((frag & 1) == 0) {
+      if (c < NCH) {
+        const int n = P % NT, ks = P / NT;
+        const uint16_t *src = w1 + (int64_t)(HS * c + 32 * n + i) * C + 16 * ks + 8 * g;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) e[j] = src[j];
+      }
+    } else if (c >= 2) {
+      const int ct = P % CT, nk = P / CT, n = nk >> 1, kk = nk & 1;
+      const uint16_t *src = w2 + (int64_t)(32 * ct + i) * F + HS * (c - 2) + 32 * n;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) e[j] = src[kperm(kk, g, j)];
+    }
+    u32x4 v;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) v[j] = (uint32_t)e[2 * j] | ((uint32_t)e[2 * j + 1] << 16);
+    blob[u] = v;
+  }
 }
 
-int64_t blob_bytes(int64_t C, int64_t F) { return (F / 64 + 1) * (int64_t)slot_units((int)C) * 16; }
+// acc += A . B with the accumulator in ordinary vector registers.  The compiler places every MFMA accumulator of a
+// kernel with more than 256 registers in the accumulation half of the register file; the 256 registers of y^T fill
+// that half, so the h^T tile is kept out of it by issuing its MFMAs this way.  The compiler does not see an MFMA here:
+// the caller keeps vector reads and writes of acc well away from it (an MFMA on another accumulator in between).
+__device__ __forceinline__ void mma_in_vgprs(u32x4 a, u32x4 b, f32x16 &acc) {
+  asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(acc) : "v"(a), "v"(b));
+}
+
+template <int C, int TAIL>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void mlp_rows_kernel(
+    const u32x4 *__restrict__ blob, const float *__restrict__ b1, const float *__restrict__ b2,
+    const uint16_t *__restrict__ u, uint16_t *__restrict__ y, const uint16_t *__restrict__ residual,
+    const float *__restrict__ ln_gamma, const float *__restrict__ ln_beta, float ln_eps, uint16_t *__restrict__ ln_out,
+    int64_t M, int F, int64_t nblocks) {
+  using K = Cfg<C>;
+  constexpr bool HAS_RES = TAIL == 1 || TAIL == 2, HAS_LN = TAIL == 1 || TAIL == 3;
+  constexpr int KS = K::KS, CT = K::CT, HS = K::HS, NT = K::NT, NP = K::NP, SU = K::SU;
+  constexpr int WU = SU / 4;    // units of a slot fetched by each wave (16 KB: four groups of four loads)
+  constexpr int CPH = C / 32;   // consecutive channels per lane in the row-major epilogue (half a wave per row)
+  constexpr int WPH = CPH / 2;  // 32-bit words per lane and row
+  constexpr int G4 = C / 4;     // 8-byte granules (4 channels) per staged row
+  constexpr int RPR = 16384 / (2 * C);  // rows a wave stages per round of the epilogue (its 16 KB of the idle buffer)
+  constexpr int NROUND = 32 / RPR;
+  extern __shared__ u32x4 smem[];
+  u32x4 *wbuf = smem;  // 2 * SU
+  float *b1s = reinterpret_cast<float *>(wbuf + 2 * SU);
+  float *b2s = b1s + F;
+  float *gams = b2s + C, *bets = gams + C;  // LayerNorm weight and bias
+  const int tid = threadIdx.x, lane = tid & 63, i = lane & 31, g = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: addresses derived from it stay scalar
+  const int NCH = F / HS;
+
+  for (int k = tid; k < F; k += 256) b1s[k] = b1[k];
+  for (int k = tid; k < C; k += 256) {
+    b2s[k] = b2[k];
+    gams[k] = HAS_LN ? ln_gamma[k] : 1.f;
+    bets[k] = HAS_LN ? ln_beta[k] : 0.f;
+  }
+  __syncthreads();  // the biases are read before the first barrier of the slot loop
+  const int half = lane >> 5;  // in the epilogue each half of the wave finishes one row per step
+
+  // 4 KB group k of this wave's share of slot c into buffer gs & 1
+  auto fetch_group = [&](int64_t gs, int c, int k) {
+    const u32x4 *src = blob + (int64_t)c * SU + wave * WU + k * 256;
+    const unsigned dst = (unsigned)(uintptr_t)(wbuf + (gs & 1) * SU + wave * WU + k * 256);
+    load_4k_to_lds(src, lane * 16, dst);
+  };
+  // lane (i, g) holds row i of the wave's 32, channels 16 ks + 8 g .. + 7
+  auto load_rows = [&](int64_t mb, u32x4(&ub)[KS]) {
+    int64_t r = mb * kRowsPerBlock + wave * 32 + i;
+    if (r >= M) r = M - 1;
+    const uint16_t *src = u + r * C + 8 * g;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) ub[ks] = *reinterpret_cast<const u32x4 *>(src + 16 * ks);
+  };
+
+  int64_t gs = 0;  // slots processed so far by this workgroup (buffer parity)
+  if ((int64_t)blockIdx.x < nblocks) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) fetch_group(0, 0, k);
+  }
+  u32x4 ub[KS];
+  if ((int64_t)blockIdx.x < nblocks) load_rows(blockIdx.x, ub);
+  for (int64_t mb = blockIdx.x; mb < nblocks; mb += gridDim.x) {
+    const int64_t row0 = mb * kRowsPerBlock + wave * 32;
+    f32x16 yacc[CT];  // channel 32 ct + rowmap(r, g) of row i
+    f32x16 hacc[NT];  // hidden unit 32 n + rowmap(r, g) of the slot's chunk, row i
+    // the output bias is where the sum starts; nothing of the block before may reach this one (the padding slots
+    // multiply what the rows produce by zero weights, which is zero only for finite rows)
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) yacc[ct][r] = b2s[32 * ct + rowmap(r, g)];
+#pragma unroll
+    for (int n = 0; n < NT; ++n)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) hacc[n][r] = 0.f;
+    // gelu(h) of chunk c-2 as B operands [tile][k half].  The operands of chunk c-1 replace them one by one as soon
+    // as the last MFMA that reads the old one is issued: operand q = 2 n + kk is read by pairs q CT .. (q+1) CT - 1 and
+    // complete (eight evaluations, packed two by two into gnew) with evaluation 8 q + 7.
+    u32x4 gprev[NT][2], gnew = u32x4{0, 0, 0, 0};
+#pragma unroll
+    for (int n = 0; n < NT; ++n) gprev[n][0] = gprev[n][1] = u32x4{0, 0, 0, 0};
+
+    for (int c = 0; c < NCH + 2; ++c, ++gs) {
+      // slot gs has landed (every wave waits for its own share, then all meet) and the other buffer is free.  The
+      // first slot of a later block was waited for before the epilogue of the block before it, whose stores may
+      // still be in flight here.
+      if (c > 0 || gs == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      __syncthreads();
+      const int c_next = c < NCH + 1 ? c + 1 : 0;
+      const u32x4 *wb = wbuf + (gs & 1) * SU + lane;
+      float hprev[NT][16];  // h(c-1), to be activated in this slot
+#pragma unroll
+      for (int n = 0; n < NT; ++n)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          hprev[n][r] = hacc[n][r];
+          hacc[n][r] = b1s[(c < NCH ? HS * c : 0) + 32 * n + rowmap(r, g)];
+        }
+      // evaluation e = 0 .. 16 NT - 1 of the slot is register e % 16 of tile e / 16; eight results in a row make one
+      // B operand.  NT = 2: one evaluation per pair, its end behind the first MFMA of the next pair; NT = 1: one
+      // evaluation per two pairs.
+      float ex = 0.f, ex2 = 0.f, eq = 0.f, ee = 0.f;  // evaluation in flight: argument, min(x^2, 81), polynomial, exp2 term
+      float feven = 0.f;                              // result of the even evaluation of a pair of results
+      auto begin1 = [&](auto e_) {
+        constexpr int e = decltype(e_)::value;
+        ex = hprev[e / 16][e % 16];
+        ex2 = fminf(ex * ex, 81.f);
+        eq = fmaf(-3.51902394e-04f * -2.f * kLog2e, ex2, 3.70080200e-02f * -2.f * kLog2e);
+      };
+      auto begin2 = [&]() {
+        const float t2 = fmaf(eq, ex2, 7.97505275e-01f * -2.f * kLog2e);
+        ee = __builtin_amdgcn_exp2f(ex * t2);
+      };
+      // end of evaluation e with argument x and exp2 term t
+      auto finish = [&](auto e_, float x, float t) {
+        constexpr int e = decltype(e_)::value, j = e % 8;
+        const float v = x * __builtin_amdgcn_rcpf(1.f + t);
+        if constexpr (j % 2 == 0) feven = v;
+        else gnew[j / 2] = (uint32_t)to_bf16_bits(feven) | ((uint32_t)to_bf16_bits(v) << 16);
+      };
+      // operand q of chunk c-1 replaces the one of chunk c-2
+      auto publish = [&](auto q_) {
+        constexpr int q = decltype(q_)::value;
+        gprev[q / 2][q % 2] = gnew;
+      };
+
+      constexpr int RING = 4, AHEAD = 3;  // in fragments; a pair consumes two
+      u32x4 fr[RING];
+      static_for<AHEAD>([&](auto q) { fr[decltype(q)::value] = wb[decltype(q)::value * 64]; });
+      static_for<NP>([&](auto P_) {
+        constexpr int P = decltype(P_)::value;
+        constexpr int n1 = P % NT, ks1 = P / NT;
+        constexpr int ct = P % CT, nk = P / CT, n2 = nk >> 1, kk = nk & 1;
+        if constexpr (2 * P + AHEAD < 2 * NP) fr[(2 * P + AHEAD) % RING] = wb[(2 * P + AHEAD) * 64];
+        if constexpr (P == 0) asm volatile("s_nop 7" ::: "memory");  // hacc was just written by vector instructions
+        mma_in_vgprs(fr[(2 * P) % RING], ub[ks1], hacc[n1]);
+        __builtin_amdgcn_sched_barrier(0);  // keeps the issue order as written
+        // Evaluation e ends behind the first MFMA of pair PF(e) = e EPV + EPV (EPV = pairs per evaluation), operand q
+        // is complete at PF(8 q + 7) = (q + 1) CT and last read by the second MFMA of pair (q + 1) CT - 1: it is
+        // published behind the second MFMA of pair (q + 1) CT (operand 2 NT - 1: of the last pair, where its last
+        // evaluation ends too).
+        constexpr int EPV = 2 / NT;
+        if constexpr (EPV == 1) {
+          // the end of the evaluation before and the start of this one: two independent chains
+          const float done_x = ex, done_e = ee;
+          begin1(P_);
+          if constexpr (P > 0) finish(std::integral_constant<int, P - 1>{}, done_x, done_e);
+        } else {
+          if constexpr (P % 2 == 0) {
+            const float done_x = ex, done_e = ee;
+            begin1(std::integral_constant<int, P / 2>{});
+            if constexpr (P > 0) finish(std::integral_constant<int, P / 2 - 1>{}, done_x, done_e);
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        if constexpr (2 * P + 1 + AHEAD < 2 * NP) fr[(2 * P + 1 + AHEAD) % RING] = wb[(2 * P + 1 + AHEAD) * 64];
+        yacc[ct] = mma(fr[(2 * P + 1) % RING], gprev[n2][kk], yacc[ct]);
+        __builtin_amdgcn_sched_barrier(0);
+        if constexpr (EPV == 1 || P % 2 == 0) begin2();
+        if constexpr (P > 0 && P % CT == 0) publish(std::integral_constant<int, P / CT - 1>{});
+        if constexpr (P == NP - 1) {
+          finish(std::integral_constant<int, 16 * NT - 1>{}, ex, ee);
+          publish(std::integral_constant<int, 2 * NT - 1>{});
+        }
+        // the other buffer was last read in the slot before this one
+        if constexpr (P % 8 == 3) fetch_group(gs + 1, c_next, P / 8);
+        __builtin_amdgcn_sched_barrier(0);
+      });
+    }
+
+    // ---- epilogue: the buffer of the last slot is idle once every wave is past its last MFMA; each wave stages
+    // ---- its own rows in its own quarter of it, RPR rows at a time ----
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's share of the next block's first slot has landed
+    __syncthreads();
+    uint32_t *stg = reinterpret_cast<uint32_t *>(wbuf + ((gs - 1) & 1) * SU + wave * WU);  // [RPR rows][C/2 words]
+    typedef uint32_t rowv __attribute__((ext_vector_type(4)));
+    constexpr int NV = WPH / 4;  // 16-byte pieces per lane and row
+    static_assert(WPH % 4 == 0, "a lane handles whole 16-byte pieces of a row");
+#pragma unroll
+    for (int rd = 0; rd < NROUND; ++rd) {
+      // the round's residual rows first: they travel while the rows are staged
+      rowv rsd[RPR / 2][NV];
+      if constexpr (HAS_RES) {
+#pragma unroll
+        for (int rr = 0; rr < RPR / 2; ++rr) {
+          int64_t r = row0 + rd * RPR + 2 * rr + half;
+          if (r >= M) r = M - 1;
+#pragma unroll
+          for (int v = 0; v < NV; ++v) rsd[rr][v] = *reinterpret_cast<const rowv *>(residual + r * C + i * CPH + 8 * v);
+        }
+      }
+      // y^T -> bf16 -> staged rows; granule gr (4 channels) of row rw sits at gr ^ ((2 rw) % G4)
+      if (NROUND == 1 || (i / RPR) == rd) {
+        const int rw = i % RPR;
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const int ch = 32 * ct + 8 * q + 4 * g;
+            const int gr = (ch >> 2) ^ ((2 * rw) & (G4 - 1));
+            u32x2 pk;
+            pk[0] = (uint32_t)to_bf16_bits(yacc[ct][4 * q + 0]) | ((uint32_t)to_bf16_bits(yacc[ct][4 * q + 1]) << 16);
+            pk[1] = (uint32_t)to_bf16_bits(yacc[ct][4 * q + 2]) | ((uint32_t)to_bf16_bits(yacc[ct][4 * q + 3]) << 16);
+            *reinterpret_cast<u32x2 *>(stg + rw * (C / 2) + gr * 2) = pk;
+          }
+      }
+      // the wave's LDS operations complete in order: its reads below see the writes above.  Once the last round is
+      // staged the accumulators are free: the rows of this workgroup's next block travel while the epilogue runs
+      // (past the end: this block again)
+      if (rd == NROUND - 1) load_rows(mb + gridDim.x < nblocks ? mb + gridDim.x : mb, ub);
+      // two rows per step: lanes 0-31 one row, lanes 32-63 the next, CPH consecutive channels per lane
+#pragma unroll
+      for (int rr = 0; rr < RPR / 2; ++rr) {
+        const int rw = 2 * rr + half;
+        const int64_t r = row0 + rd * RPR + rw;
+        const bool ok = r < M;
+        rowv sv[NV];
+        // granules (4 channels) i*CPH/4 .. of row rw; the swizzle flips an even number, so pairs stay adjacent
+#pragma unroll
+        for (int v = 0; v < NV; ++v)
+          sv[v] = *reinterpret_cast<const rowv *>(stg + rw * (C / 2) + ((((i * CPH + 8 * v) / 4) ^ ((2 * rw) & (G4 - 1))) << 1));
+        float val[CPH];
+        rowv ob[NV];
+#pragma unroll
+        for (int w = 0; w < WPH; ++w) {
+          float t0 = bf16_bits_to_f32((uint16_t)(sv[w / 4][w % 4] & 0xffffu)), t1 = bf16_bits_to_f32((uint16_t)(sv[w / 4][w % 4] >> 16));
+          if constexpr (HAS_RES) {  // the MLP output is a bf16 tensor; the sum is rounded again
+            t0 += bf16_bits_to_f32((uint16_t)(rsd[rr][w / 4][w % 4] & 0xffffu));
+            t1 += bf16_bits_to_f32((uint16_t)(rsd[rr][w / 4][w % 4] >> 16));
+          }
+          const uint16_t o0 = to_bf16_bits(t0), o1 = to_bf16_bits(t1);
+          val[2 * w] = bf16_bits_to_f32(o0);
+          val[2 * w + 1] = bf16_bits_to_f32(o1);
+          ob[w / 4][w % 4] = (uint32_t)o0 | ((uint32_t)o1 << 16);
+        }
+        if (ok) {
+#pragma unroll
+          for (int v = 0; v < NV; ++v) *reinterpret_cast<rowv *>(y + r * C + i * CPH + 8 * v) = ob[v];
+        }
+        if constexpr (HAS_LN) {
+          float s1 = 0.f;
+#pragma unroll
+          for (int k = 0; k < CPH; ++k) s1 += val[k];
+          const float mean = half_wave_sum(s1) * (1.f / C);
+          float s2 = 0.f;
+#pragma unroll
+          for (int k = 0; k < CPH; ++k) {
+            const float dl = val[k] - mean;
+            s2 = fmaf(dl, dl, s2);
+          }
+          const float rstd = rsqrtf(half_wave_sum(s2) * (1.f / C) + ln_eps);
+          rowv lb[NV];
+#pragma unroll
+          for (int w = 0; w < WPH; ++w) {
+            const int ch = i * CPH + 2 * w;
+            const uint16_t l0 = to_bf16_bits((val[2 * w] - mean) * rstd * gams[ch] + bets[ch]);
+            const uint16_t l1 = to_bf16_bits((val[2 * w + 1] - mean) * rstd * gams[ch + 1] + bets[ch + 1]);
+            lb[w / 4][w % 4] = (uint32_t)l0 | ((uint32_t)l1 << 16);
+          }
+          if (ok) {
+#pragma unroll
+            for (int v = 0; v < NV; ++v) *reinterpret_cast<rowv *>(ln_out + r * C + i * CPH + 8 * v) = lb[v];
+          }
+        }
+      }
+    }
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // nothing may still be landing in LDS when the workgroup ends
+}
+
+}  // namespace rows
+
+// ---------------------------------------------------------------------------------------------------------------
+// C = 512 runs the row-owning kernel; C in {128, 256} the paired one
+static bool use_rows_kernel(int64_t C) { return C == 512; }
+
+bool supported(int dtype, int64_t rows, int64_t C, int64_t F) {
+  if (dtype != PA_BF16 || rows <= 0 || F < 64 || F % 64 != 0 || F > 8192) return false;
+  if (use_rows_kernel(C)) return F <= 4096;
+  return C == 128 || C == 256;
+}
+
+int64_t blob_bytes(int64_t C, int64_t F) {
+  if (use_rows_kernel(C)) return (F / (16384 / C) + 2) * (int64_t)4096 * 16;
+  return (F / 64 + 1) * (int64_t)slot_units((int)C) * 16;
+}
 
 static size_t lds_bytes(int C, int F) { return (size_t)(2 * slot_units(C) + 4 * 4 * 64) * 16 + (size_t)(F + C) * 4; }
 
 int pack(int64_t C, int64_t F, const void *w1, const void *w2, void *blob, hipStream_t st) {
-  const int64_t total = (F / 64 + 1) * (int64_t)slot_units((int)C);
+  const bool by_rows = use_rows_kernel(C);
+  const int64_t total = by_rows ? (F / (16384 / C) + 2) * (int64_t)4096 : (F / 64 + 1) * (int64_t)slot_units((int)C);
   const int grid = (int)((total + 255) / 256 < 1024 ? (total + 255) / 256 : 1024);
-  hipLaunchKernelGGL(pack_kernel, dim3(grid), dim3(256), 0, st, static_cast<const uint16_t *>(w1),
-                     static_cast<const uint16_t *>(w2), static_cast<u32x4 *>(blob), (int)C, (int)F);
+  if (by_rows)
+    hipLaunchKernelGGL(rows::pack_kernel, dim3(grid), dim3(256), 0, st, static_cast<const uint16_t *>(w1),
+                       static_cast<const uint16_t *>(w2), static_cast<u32x4 *>(blob), (int)C, (int)F);
+  else
+    hipLaunchKernelGGL(pack_kernel, dim3(grid), dim3(256), 0, st, static_cast<const uint16_t *>(w1),
+                       static_cast<const uint16_t *>(w2), static_cast<u32x4 *>(blob), (int)C, (int)F);
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? PA_OK : (int)e;
+}
+
+template <int C, int TAIL>
+static int launch_rows(int64_t rows, int F, const void *blob, const float *b1, const float *b2, const void *u, void *y,
+                       const pa_block_tail *tail, int num_cu, hipStream_t st) {
+  const size_t lds = (size_t)2 * rows::Cfg<C>::SU * 16 + (size_t)(F + 3 * C) * 4;
+  if (lds > kMaxLdsBytes) return PA_ERR_UNSUPPORTED;
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(rows::mlp_rows_kernel<C, TAIL>),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  if (e != hipSuccess) return (int)e;
+  const int64_t nblocks = (rows + kRowsPerBlock - 1) / kRowsPerBlock;
+  const int64_t grid = nblocks < num_cu ? nblocks : num_cu;
+  hipLaunchKernelGGL((rows::mlp_rows_kernel<C, TAIL>), dim3((unsigned)grid), dim3(256), lds, st,
+                     static_cast<const u32x4 *>(blob), b1, b2, static_cast<const uint16_t *>(u),
+                     static_cast<uint16_t *>(y), tail ? static_cast<const uint16_t *>(tail->residual) : nullptr,
+                     tail ? tail->ln_gamma : nullptr, tail ? tail->ln_beta : nullptr, tail ? tail->ln_eps : 0.f,
+                     tail ? static_cast<uint16_t *>(tail->ln_out) : nullptr, rows, F, nblocks);
+  e = hipGetLastError();
+  return e == hipSuccess ? PA_OK : (int)e;
+}
+
+template <int C>
+static int launch_rows_c(int64_t rows, int F, const void *blob, const float *b1, const float *b2, const void *u, void *y,
+                         const pa_block_tail *tail, int num_cu, hipStream_t st) {
+  const bool res = tail && tail->residual, ln = tail && tail->ln_out;
+  if (res && ln) return launch_rows<C, 1>(rows, F, blob, b1, b2, u, y, tail, num_cu, st);
+  if (res) return launch_rows<C, 2>(rows, F, blob, b1, b2, u, y, tail, num_cu, st);
+  if (ln) return launch_rows<C, 3>(rows, F, blob, b1, b2, u, y, tail, num_cu, st);
+  return launch_rows<C, 0>(rows, F, blob, b1, b2, u, y, nullptr, num_cu, st);
 }
 
 template <int C, int TAIL>
@@ -422,6 +875,7 @@ static int launch_c(int64_t rows, int F, const void *blob, const float *b1, cons
 
 int forward(int64_t rows, int64_t C, int64_t F, const void *blob, const float *b1, const float *b2, const void *u,
             void *y, const pa_block_tail *tail, int num_cu, hipStream_t st) {
+  if (C == 512) return launch_rows_c<512>(rows, (int)F, blob, b1, b2, u, y, tail, num_cu, st);
   if (C == 256) return launch_c<256>(rows, (int)F, blob, b1, b2, u, y, tail, num_cu, st);
   if (C == 128) return launch_c<128>(rows, (int)F, blob, b1, b2, u, y, tail, num_cu, st);
   return PA_ERR_UNSUPPORTED;

@@ -35,6 +35,7 @@ def _case(rows_shape, C, Fh, seed=0, scale=1.0):
 @pytest.mark.parametrize("rows_shape,C,Fh", [
     ((1, 4096), 256, 1024), ((2, 1000), 256, 1024), ((1, 257), 256, 256), ((3, 77), 128, 512), ((1, 1), 256, 1024),
     ((1, 5000), 128, 128), ((1, 20000), 256, 512),
+    ((1, 4096), 512, 2048), ((2, 777), 512, 2048), ((1, 1), 512, 64), ((1, 33000), 512, 512),
 ])
 def test_mlp_matches_fp32_oracle(rows_shape, C, Fh):
     announce("mlp", rows_shape, C, Fh)
@@ -78,5 +79,6 @@ def test_mlp_gelu_tails_and_determinism():
 
 def test_mlp_rejects_unsupported():
     assert not PF.mlp_supported(torch.float32, 100, 256, 1024)
-    assert not PF.mlp_supported(torch.bfloat16, 100, 512, 2048)
+    assert not PF.mlp_supported(torch.bfloat16, 100, 384, 1536)
+    assert not PF.mlp_supported(torch.bfloat16, 100, 512, 8192)
     assert not PF.mlp_supported(torch.bfloat16, 100, 256, 1000)
