@@ -103,6 +103,15 @@ __device__ __forceinline__ u32x4 pack8(const float (&v)[8]) {
   return __builtin_bit_cast(u32x4, o);
 }
 
+// 2 floats -> 2 bf16 (round to nearest even), the first in the low half
+__device__ __forceinline__ uint32_t pack2(float a, float b) {
+  typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+  bf16x2 o;
+  o[0] = (__bf16)a;
+  o[1] = (__bf16)b;
+  return __builtin_bit_cast(uint32_t, o);
+}
+
 // sum over the 32 lanes of this lane's half of the wave, returned in every lane of the half: DPP steps inside each
 // row of 16 lanes, then v_permlane16_swap pairs the two rows of the half
 __device__ __forceinline__ float half_wave_sum(float v) {
@@ -118,17 +127,6 @@ __device__ __forceinline__ float half_wave_sum(float v) {
   return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
-#ifdef PA_PROFILE
-__device__ unsigned long long pa_prof[256 * 4 * 12];  // [workgroup][wave][interval]
-#define PA_T(k)                                                   \
-  do {                                                            \
-    const unsigned long long now_ = __builtin_readcyclecounter(); \
-    pacc[k] += now_ - tlast;                                      \
-    tlast = now_;                                                 \
-  } while (0)
-#else
-#define PA_T(k) do { } while (0)
-#endif
 
 template <int C, int TAIL>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void mlp_kernel(
@@ -184,11 +182,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   };
 
   int64_t gs = 0;  // slots processed so far by this workgroup (buffer parity)
-#ifdef PA_PROFILE
-  unsigned long long pacc[12] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-  unsigned long long tlast = __builtin_readcyclecounter();
-  const unsigned long long t_begin = tlast, w_begin = wall_clock64();
-#endif
   if ((int64_t)blockIdx.x < nblocks) {
 #pragma unroll
     for (int k = 0; k < NDMA / 4; ++k) fetch_quad(0, 0, k);
@@ -236,11 +229,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
       // slot gs has landed (every wave waits for its own share, then all meet) and the other buffer is free.  The
       // first slot of a later block was waited for before the epilogue of the block before it, whose stores may
       // still be in flight here.
-      PA_T(0);
       if (c > 0 || gs == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-      PA_T(1);
       __syncthreads();
-      PA_T(2);
       const int c_next = c < NC ? c + 1 : 0;
       const u32x4 *wb = wbuf + (gs & 1) * SU + lane;
       // this wave's fragments of the slot: W1 of hidden tile p; W2 of its channel half, hidden tile p ("own") first
@@ -300,7 +290,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         static_for<AHEAD>([&](auto q) { fr[decltype(q)::value] = frag(q); });
         static_for<NS1 + NS2>([&](auto S_) {
           constexpr int S = decltype(S_)::value;
-          if constexpr (S == NS1) PA_T(3);
           if constexpr (S == NS1 + 2 * CTH - 2) {  // two steps before the partner's tile (written in step NS1) is needed
             __syncthreads();
 #pragma unroll
@@ -343,7 +332,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
             __builtin_amdgcn_sched_barrier(0);
           }
         });
-        PA_T(4);
 #pragma unroll
         for (int m = 0; m < 2; ++m)
 #pragma unroll
@@ -352,10 +340,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     }
 
     // ---- epilogue: the buffer of the last slot is idle once every wave is past its last MFMA ----
-    PA_T(0);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's share of the next block's first slot has landed
     __syncthreads();
-    PA_T(8);
     // the rows of this workgroup's next block travel while the epilogue runs (past the end: this block again)
     load_rows(mb + gridDim.x < nblocks ? mb + gridDim.x : mb, ub);
     uint32_t *stg = reinterpret_cast<uint32_t *>(wbuf + ((gs - 1) & 1) * SU) + rg * 64 * (C / 2);  // [64 rows][C/2 words]
@@ -375,9 +361,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
           pk[1] = (uint32_t)to_bf16_bits(v2) | ((uint32_t)to_bf16_bits(v3) << 16);
           *reinterpret_cast<u32x2 *>(stg + rw * (C / 2) + gr * 2) = pk;
         }
-    PA_T(9);
     __syncthreads();  // both waves of a pair have staged their channel halves
-    PA_T(10);
     // wave p finishes rows 32p .. 32p+31 of the pair, two per step: lanes 0-31 one row, lanes 32-63 the next, CPH
     // consecutive channels per lane (16-byte accesses for C = 256)
     typedef uint32_t rowv __attribute__((ext_vector_type(WPH)));
@@ -435,17 +419,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         if (ok) *reinterpret_cast<rowv *>(ln_out + r * C + i * CPH) = lb;
       }
     }
-    PA_T(5);
   }
-#ifdef PA_PROFILE
-  if (lane == 0) {
-    unsigned long long *dstp = pa_prof + ((int)blockIdx.x * 4 + wave) * 12;
-    for (int k = 0; k < 6; ++k) dstp[k] = pacc[k];
-    for (int k = 8; k < 12; ++k) dstp[k] = pacc[k];
-    dstp[6] = __builtin_readcyclecounter() - t_begin;
-    dstp[7] = wall_clock64() - w_begin;
-  }
-#endif
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // nothing may still be landing in LDS when the workgroup ends
 }
 
@@ -528,8 +502,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   constexpr bool HAS_RES = TAIL == 1 || TAIL == 2, HAS_LN = TAIL == 1 || TAIL == 3;
   constexpr int KS = K::KS, CT = K::CT, HS = K::HS, NT = K::NT, NP = K::NP, SU = K::SU;
   constexpr int WU = SU / 4;    // units of a slot fetched by each wave (16 KB: four groups of four loads)
-  constexpr int CPH = C / 32;   // consecutive channels per lane in the row-major epilogue (half a wave per row)
-  constexpr int WPH = CPH / 2;  // 32-bit words per lane and row
   constexpr int G4 = C / 4;     // 8-byte granules (4 channels) per staged row
   constexpr int RPR = 16384 / (2 * C);  // rows a wave stages per round of the epilogue (its 16 KB of the idle buffer)
   constexpr int NROUND = 32 / RPR;
@@ -549,7 +521,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     bets[k] = HAS_LN ? ln_beta[k] : 0.f;
   }
   __syncthreads();  // the biases are read before the first barrier of the slot loop
-  const int half = lane >> 5;  // in the epilogue each half of the wave finishes one row per step
 
   // 4 KB group k of this wave's share of slot c into buffer gs & 1
   auto fetch_group = [&](int64_t gs, int c, int k) {
@@ -630,7 +601,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         constexpr int e = decltype(e_)::value, j = e % 8;
         const float v = x * __builtin_amdgcn_rcpf(1.f + t);
         if constexpr (j % 2 == 0) feven = v;
-        else gnew[j / 2] = (uint32_t)to_bf16_bits(feven) | ((uint32_t)to_bf16_bits(v) << 16);
+        else gnew[j / 2] = pack2(feven, v);
       };
       // operand q of chunk c-1 replaces the one of chunk c-2
       auto publish = [&](auto q_) {
@@ -638,7 +609,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         gprev[q / 2][q % 2] = gnew;
       };
 
-      constexpr int RING = 4, AHEAD = 3;  // in fragments; a pair consumes two
+      constexpr int RING = 8, AHEAD = 6;  // in fragments; a pair consumes two
       u32x4 fr[RING];
       static_for<AHEAD>([&](auto q) { fr[decltype(q)::value] = wb[decltype(q)::value * 64]; });
       static_for<NP>([&](auto P_) {
@@ -686,97 +657,108 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     // ---- its own rows in its own quarter of it, RPR rows at a time ----
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's share of the next block's first slot has landed
     __syncthreads();
+    // lane indices taken afresh, so that nothing derived from them for the epilogue is kept across the slot loop
+    int il = i, gl = g;
+    asm volatile("" : "+v"(il), "+v"(gl));
+    const int hl = gl;  // each half of the wave finishes one row per step
     uint32_t *stg = reinterpret_cast<uint32_t *>(wbuf + ((gs - 1) & 1) * SU + wave * WU);  // [RPR rows][C/2 words]
     typedef uint32_t rowv __attribute__((ext_vector_type(4)));
-    constexpr int NV = WPH / 4;  // 16-byte pieces per lane and row
-    static_assert(WPH % 4 == 0, "a lane handles whole 16-byte pieces of a row");
+    typedef float f32x4 __attribute__((ext_vector_type(4)));
+    constexpr int NV = C / 256;  // 16-byte pieces per lane and row: piece v = channels 256 v + 8 il .. + 7
+    static_assert(C % 256 == 0, "half a wave covers 256 consecutive channels per access");
+    // y^T -> bf16 once: yp[ct][q] = channels 32 ct + 8 q + 4 g .. + 3 of row i; the accumulators are free after this
+    u32x2 yp[CT][4];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        yp[ct][q][0] = pack2(yacc[ct][4 * q + 0], yacc[ct][4 * q + 1]);
+        yp[ct][q][1] = pack2(yacc[ct][4 * q + 2], yacc[ct][4 * q + 3]);
+      }
+    constexpr int NIT = RPR / 2;             // steps per round: two rows each
+    constexpr int PF = NIT < 4 ? NIT : 4;    // residual rows are fetched this many steps ahead
 #pragma unroll
     for (int rd = 0; rd < NROUND; ++rd) {
-      // the round's residual rows first: they travel while the rows are staged
-      rowv rsd[RPR / 2][NV];
-      if constexpr (HAS_RES) {
-#pragma unroll
-        for (int rr = 0; rr < RPR / 2; ++rr) {
-          int64_t r = row0 + rd * RPR + 2 * rr + half;
+      rowv rsd[NIT][NV];
+      auto load_residual = [&](auto rr_) {
+        constexpr int rr = decltype(rr_)::value;
+        if constexpr (HAS_RES) {
+          int64_t r = row0 + rd * RPR + 2 * rr + hl;
           if (r >= M) r = M - 1;
 #pragma unroll
-          for (int v = 0; v < NV; ++v) rsd[rr][v] = *reinterpret_cast<const rowv *>(residual + r * C + i * CPH + 8 * v);
+          for (int v = 0; v < NV; ++v) rsd[rr][v] = *reinterpret_cast<const rowv *>(residual + r * C + 256 * v + 8 * il);
         }
-      }
-      // y^T -> bf16 -> staged rows; granule gr (4 channels) of row rw sits at gr ^ ((2 rw) % G4)
-      if (NROUND == 1 || (i / RPR) == rd) {
-        const int rw = i % RPR;
+      };
+      static_for<PF>(load_residual);
+      // staged rows: granule gr (4 channels) of row rw sits at gr ^ ((2 rw) % G4)
+      if (NROUND == 1 || (il / RPR) == rd) {
+        const int rw = il % RPR;
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct)
 #pragma unroll
           for (int q = 0; q < 4; ++q) {
-            const int ch = 32 * ct + 8 * q + 4 * g;
-            const int gr = (ch >> 2) ^ ((2 * rw) & (G4 - 1));
-            u32x2 pk;
-            pk[0] = (uint32_t)to_bf16_bits(yacc[ct][4 * q + 0]) | ((uint32_t)to_bf16_bits(yacc[ct][4 * q + 1]) << 16);
-            pk[1] = (uint32_t)to_bf16_bits(yacc[ct][4 * q + 2]) | ((uint32_t)to_bf16_bits(yacc[ct][4 * q + 3]) << 16);
-            *reinterpret_cast<u32x2 *>(stg + rw * (C / 2) + gr * 2) = pk;
+            const int gr = (8 * ct + 2 * q + gl) ^ ((2 * rw) & (G4 - 1));
+            *reinterpret_cast<u32x2 *>(stg + rw * (C / 2) + gr * 2) = yp[ct][q];
           }
       }
       // the wave's LDS operations complete in order: its reads below see the writes above.  Once the last round is
-      // staged the accumulators are free: the rows of this workgroup's next block travel while the epilogue runs
-      // (past the end: this block again)
+      // staged the rows of this workgroup's next block can travel (past the end: this block again)
       if (rd == NROUND - 1) load_rows(mb + gridDim.x < nblocks ? mb + gridDim.x : mb, ub);
-      // two rows per step: lanes 0-31 one row, lanes 32-63 the next, CPH consecutive channels per lane
-#pragma unroll
-      for (int rr = 0; rr < RPR / 2; ++rr) {
-        const int rw = 2 * rr + half;
+      // two rows per step: lanes 0-31 one row, lanes 32-63 the next
+      static_for<NIT>([&](auto rr_) {
+        constexpr int rr = decltype(rr_)::value;
+        if constexpr (rr + PF < NIT) load_residual(std::integral_constant<int, rr + PF>{});
+        const int rw = 2 * rr + hl;
         const int64_t r = row0 + rd * RPR + rw;
         const bool ok = r < M;
-        rowv sv[NV];
-        // granules (4 channels) i*CPH/4 .. of row rw; the swizzle flips an even number, so pairs stay adjacent
+        float val[8 * NV];
 #pragma unroll
-        for (int v = 0; v < NV; ++v)
-          sv[v] = *reinterpret_cast<const rowv *>(stg + rw * (C / 2) + ((((i * CPH + 8 * v) / 4) ^ ((2 * rw) & (G4 - 1))) << 1));
-        float val[CPH];
-        rowv ob[NV];
+        for (int v = 0; v < NV; ++v) {
+          // granules 64 v + 2 il, + 1 of row rw; the swizzle flips an even number, so the pair stays adjacent
+          const rowv sv = *reinterpret_cast<const rowv *>(stg + rw * (C / 2) + (((64 * v + 2 * il) ^ ((2 * rw) & (G4 - 1))) << 1));
+          rowv ob;
 #pragma unroll
-        for (int w = 0; w < WPH; ++w) {
-          float t0 = bf16_bits_to_f32((uint16_t)(sv[w / 4][w % 4] & 0xffffu)), t1 = bf16_bits_to_f32((uint16_t)(sv[w / 4][w % 4] >> 16));
-          if constexpr (HAS_RES) {  // the MLP output is a bf16 tensor; the sum is rounded again
-            t0 += bf16_bits_to_f32((uint16_t)(rsd[rr][w / 4][w % 4] & 0xffffu));
-            t1 += bf16_bits_to_f32((uint16_t)(rsd[rr][w / 4][w % 4] >> 16));
+          for (int w = 0; w < 4; ++w) {
+            float t0 = __uint_as_float(sv[w] << 16), t1 = __uint_as_float(sv[w] & 0xffff0000u);
+            if constexpr (HAS_RES) {  // the MLP output is a bf16 tensor; the sum is rounded again
+              t0 += __uint_as_float(rsd[rr][v][w] << 16);
+              t1 += __uint_as_float(rsd[rr][v][w] & 0xffff0000u);
+            }
+            ob[w] = pack2(t0, t1);
+            val[8 * v + 2 * w] = __uint_as_float(ob[w] << 16);
+            val[8 * v + 2 * w + 1] = __uint_as_float(ob[w] & 0xffff0000u);
           }
-          const uint16_t o0 = to_bf16_bits(t0), o1 = to_bf16_bits(t1);
-          val[2 * w] = bf16_bits_to_f32(o0);
-          val[2 * w + 1] = bf16_bits_to_f32(o1);
-          ob[w / 4][w % 4] = (uint32_t)o0 | ((uint32_t)o1 << 16);
-        }
-        if (ok) {
-#pragma unroll
-          for (int v = 0; v < NV; ++v) *reinterpret_cast<rowv *>(y + r * C + i * CPH + 8 * v) = ob[v];
+          if (ok) *reinterpret_cast<rowv *>(y + r * C + 256 * v + 8 * il) = ob;
         }
         if constexpr (HAS_LN) {
           float s1 = 0.f;
 #pragma unroll
-          for (int k = 0; k < CPH; ++k) s1 += val[k];
+          for (int k = 0; k < 8 * NV; ++k) s1 += val[k];
           const float mean = half_wave_sum(s1) * (1.f / C);
           float s2 = 0.f;
 #pragma unroll
-          for (int k = 0; k < CPH; ++k) {
+          for (int k = 0; k < 8 * NV; ++k) {
             const float dl = val[k] - mean;
             s2 = fmaf(dl, dl, s2);
           }
           const float rstd = rsqrtf(half_wave_sum(s2) * (1.f / C) + ln_eps);
-          rowv lb[NV];
+          const float shift = -mean * rstd;
 #pragma unroll
-          for (int w = 0; w < WPH; ++w) {
-            const int ch = i * CPH + 2 * w;
-            const uint16_t l0 = to_bf16_bits((val[2 * w] - mean) * rstd * gams[ch] + bets[ch]);
-            const uint16_t l1 = to_bf16_bits((val[2 * w + 1] - mean) * rstd * gams[ch + 1] + bets[ch + 1]);
-            lb[w / 4][w % 4] = (uint32_t)l0 | ((uint32_t)l1 << 16);
-          }
-          if (ok) {
+          for (int v = 0; v < NV; ++v) {
+            const f32x4 ga = *reinterpret_cast<const f32x4 *>(gams + 256 * v + 8 * il), gb = *reinterpret_cast<const f32x4 *>(gams + 256 * v + 8 * il + 4);
+            const f32x4 ba = *reinterpret_cast<const f32x4 *>(bets + 256 * v + 8 * il), bb = *reinterpret_cast<const f32x4 *>(bets + 256 * v + 8 * il + 4);
+            rowv lb;
 #pragma unroll
-            for (int v = 0; v < NV; ++v) *reinterpret_cast<rowv *>(ln_out + r * C + i * CPH + 8 * v) = lb[v];
+            for (int w = 0; w < 4; ++w) {
+              const float g0 = w < 2 ? ga[2 * w] : gb[2 * w - 4], g1 = w < 2 ? ga[2 * w + 1] : gb[2 * w - 3];
+              const float c0 = w < 2 ? ba[2 * w] : bb[2 * w - 4], c1 = w < 2 ? ba[2 * w + 1] : bb[2 * w - 3];
+              lb[w] = pack2(fmaf(fmaf(val[8 * v + 2 * w], rstd, shift), g0, c0), fmaf(fmaf(val[8 * v + 2 * w + 1], rstd, shift), g1, c1));
+            }
+            if (ok) *reinterpret_cast<rowv *>(ln_out + r * C + 256 * v + 8 * il) = lb;
           }
         }
-      }
+        __builtin_amdgcn_sched_barrier(0);
+      });
     }
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // nothing may still be landing in LDS when the workgroup ends
