@@ -110,14 +110,45 @@ MfmaPlan plan_mfma(const pa_shape &s) {
   return p;
 }
 
-// Workspace plan of the staged MFMA path.
+// Workspace plan of the staged MFMA path.  The slice weights are never stored: the token sums and the hand-back to
+// the points each recompute them from x_mid.
 struct StagedPlan {
-  int64_t off_x_mid, off_fx, off_w, off_partials, off_tok, off_norm, off_tok_out, off_tokp, total;
+  int64_t off_x_mid, off_fx, off_partials, off_tok, off_norm, off_tok_out, off_tokp, total;
   int64_t G;
 };
 
 StagedPlan plan_staged(const pa_shape &s) {
   StagedPlan p{};
+  p.G = pa::mfma::softmax_reduce_groups(s, compute_units());
+  const int64_t tiles = s.B * pa::mfma::tiles_per_batch(s);
+  int64_t off = 0;
+  p.off_x_mid = off;  // natural (B, N, H*32); overwritten by out_x, 64 bytes at a time, as the weights are recomputed
+  off += round_up(s.B * s.N * s.H * 32 * 2, 256);
+  p.off_fx = off;
+  off += round_up(tiles * s.H * 2 * 1024, 256);
+  p.off_partials = off;
+  off += round_up((p.G + 1) * s.B * s.H * s.S * (s.D + 1) * 4, 256);
+  p.off_tok = off;
+  off += round_up(s.B * s.H * s.S * s.D * 4, 256);
+  p.off_norm = off;
+  off += round_up(s.B * s.H * s.S * 4, 256);
+  p.off_tok_out = off;
+  off += round_up(s.B * s.H * s.S * s.D * 4, 256);
+  p.off_tokp = off;
+  off += round_up(s.B * s.H * (s.S / 16) * 1024, 256);
+  p.total = off;
+  return p;
+}
+
+// Workspace plan of the Transolver++ layer: the staged kernels with the slice weights stored (their Gumbel noise
+// comes from the caller's samples, which are read once).
+struct PlusPlan {
+  int64_t off_x_mid, off_fx, off_w, off_partials, off_tok, off_norm, off_tok_out, off_tokp, total;
+  int64_t G;
+};
+
+PlusPlan plan_plus(const pa_shape &s) {
+  PlusPlan p{};
   p.G = mfma_groups(s, false);
   const int64_t tiles = s.B * pa::mfma::tiles_per_batch(s);
   int64_t off = 0;
@@ -842,7 +873,7 @@ int pa_layer_forward(int dtype, const pa_shape *shape, const pa_params *p, const
   if (pa::mfma::staged_supported(dtype, s)) {
     const StagedPlan sp = plan_staged(s);
     if (workspace_bytes < sp.total) return PA_ERR_WORKSPACE;
-    void *x_mid = ws + sp.off_x_mid, *fxp = ws + sp.off_fx, *wp = ws + sp.off_w, *tokp = ws + sp.off_tokp;
+    void *x_mid = ws + sp.off_x_mid, *fxp = ws + sp.off_fx, *tokp = ws + sp.off_tokp;
     float *partials = reinterpret_cast<float *>(ws + sp.off_partials);
     float *tok = slice_token_out ? slice_token_out : reinterpret_cast<float *>(ws + sp.off_tok);
     float *norm = reinterpret_cast<float *>(ws + sp.off_norm);
@@ -869,11 +900,10 @@ int pa_layer_forward(int dtype, const pa_shape *shape, const pa_params *p, const
     a.pack_heads = (int)s.H;
     if (!pa::gemm::serves(a, 2, 2)) return PA_ERR_UNSUPPORTED;
     if ((rc = pa::gemm::launch(a, 2, PA_BF16, st))) return rc;
-    if ((rc = pa::mfma::slice_softmax_pack(s, *p, x_mid, wp, compute_units(), st))) return rc;
-    if ((rc = pa::mfma::slice_reduce(s, wp, fxp, partials, st))) return rc;
+    if ((rc = pa::mfma::slice_softmax_reduce(s, *p, x_mid, fxp, partials, compute_units(), st))) return rc;
     if ((rc = pa::mfma::combine_attention(s, *p, nullptr, partials, sp.G, tok, norm, tok_out, tokp, st))) return rc;
     void *out_x = x_mid;
-    if ((rc = pa::mfma::deslice_natural(s, wp, tokp, out_x, compute_units(), st))) return rc;
+    if ((rc = pa::mfma::deslice_recompute(s, *p, x_mid, tokp, out_x, compute_units(), st))) return rc;
     if ((rc = pa::general::out_linear(dtype, s, *p, out_x, y, st))) return rc;
     if (tail_active(tail)) rc = pa::general::residual_ln(dtype, s, y, *tail, st);
     return rc;
@@ -1019,7 +1049,7 @@ int64_t pa_layer_forward_plus_workspace_bytes(int dtype, const pa_shape *shape) 
   int rc = check_shape(dtype, shape);
   if (rc) return rc;
   if (!pa::mfma::staged_supported(dtype, *shape)) return PA_ERR_UNSUPPORTED;
-  return plan_staged(*shape).total;
+  return plan_plus(*shape).total;
 }
 
 int pa_layer_forward_plus(int dtype, const pa_shape *shape, const pa_params *p, const pa_plus_params *plus,
@@ -1037,7 +1067,7 @@ int pa_layer_forward_plus(int dtype, const pa_shape *shape, const pa_params *p, 
   const pa_shape &s = *shape;
   if (!pa::mfma::staged_supported(dtype, s)) return PA_ERR_UNSUPPORTED;
   hipStream_t st = static_cast<hipStream_t>(stream);
-  const StagedPlan sp = plan_staged(s);
+  const PlusPlan sp = plan_plus(s);
   if (workspace_bytes < sp.total) return PA_ERR_WORKSPACE;
   char *ws = static_cast<char *>(workspace);
   void *x_mid = ws + sp.off_x_mid, *fxp = ws + sp.off_fx, *wp = ws + sp.off_w, *tokp = ws + sp.off_tokp;

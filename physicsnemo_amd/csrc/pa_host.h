@@ -158,6 +158,13 @@ int slice_softmax_pack_plus(const pa_shape &s, const pa_params &p, const pa_plus
                             const void *uniform, void *w_pack, int num_cu, hipStream_t st);
 int slice_softmax_pack(const pa_shape &s, const pa_params &p, const void *x_mid, void *w_pack, int num_cu,
                        hipStream_t st);
+// the same weights recomputed where they are used, never stored: token sums (softmax_reduce_groups partials) and
+// the hand-back to the points (out_x may be x_mid)
+int64_t softmax_reduce_groups(const pa_shape &s, int num_cu);
+int slice_softmax_reduce(const pa_shape &s, const pa_params &p, const void *x_mid, const void *fx_pack,
+                         float *partials, int num_cu, hipStream_t st);
+int deslice_recompute(const pa_shape &s, const pa_params &p, const void *x_mid, const void *tokp, void *out_x,
+                      int num_cu, hipStream_t st);
 bool backward_supported(const pa_shape &s);
 int64_t backward_groups(const pa_shape &s, int num_cu);
 int64_t backward_tables_bytes(const pa_shape &s);

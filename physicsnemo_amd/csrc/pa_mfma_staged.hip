@@ -198,6 +198,189 @@ __global__ __launch_bounds__(512) void slice_softmax_pack_plus_kernel(
   }
 }
 
+// ------------------------------------------------------------------------------------------------
+// The slice weights of one head for one tile of 32 points, formed in registers: logits, temperature softmax, bf16
+// operand chunks.  chunk[cq] (cq = 0 .. S/16 - 1) is what slice_softmax_pack_kernel stores: as an A operand its rows
+// are the points and its reduction index the slices 16 cq + kperm order; the same registers serve as a B operand
+// whose columns are the points.  Both kernels below recompute the weights from x_mid instead of passing them through
+// memory (S/16 KB per point and head group written once and read twice otherwise); the arithmetic is identical in
+// both, so the weights that aggregate the tokens and the ones that hand them back are the same numbers.
+// ------------------------------------------------------------------------------------------------
+template <int S>
+__device__ __forceinline__ void slice_weights_of_tile(const u32x4 *__restrict__ wsl, const float *__restrict__ bsl,
+                                                      u32x4 xm0, u32x4 xm1, float sc, bool valid, int lane, int g,
+                                                      u32x4 (&chunk)[S / 16]) {
+  constexpr int ST = (S + 31) / 32, NCH = S / 16;
+  f32x16 lg[ST];
+#pragma unroll
+  for (int st = 0; st < ST; ++st) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) lg[st][r] = bsl[32 * st + rowmap(r, g)];
+    lg[st] = mma(wsl[(st * 2 + 0) * 64 + lane], xm0, lg[st]);
+    lg[st] = mma(wsl[(st * 2 + 1) * 64 + lane], xm1, lg[st]);
+  }
+  float mx = -INFINITY;
+#pragma unroll
+  for (int st = 0; st < ST; ++st)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) mx = fmaxf(mx, lg[st][r]);
+  mx = half_max(mx);
+  const float off = mx * sc;
+  float sum = 0.f;
+#pragma unroll
+  for (int st = 0; st < ST; ++st)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const float e = __builtin_amdgcn_exp2f(fmaf(lg[st][r], sc, -off));
+      lg[st][r] = e;
+      sum += e;
+    }
+  sum = half_sum(sum);
+  const float inv = valid ? __builtin_amdgcn_rcpf(sum) : 0.f;
+#pragma unroll
+  for (int cq = 0; cq < NCH; ++cq) chunk[cq] = (cq & 1) ? pack_half<1>(lg[cq >> 1], inv) : pack_half<0>(lg[cq >> 1], inv);
+}
+
+// W_slice as A operands (k = d in natural order) and the slice bias, as slice_softmax_pack_kernel stages them
+template <int S>
+__device__ __forceinline__ void stage_slice_projection(const float *__restrict__ w_slice, const float *__restrict__ b_slice,
+                                                       u32x4 *wsl, float *bsl) {
+  constexpr int ST = (S + 31) / 32;
+  for (int u = threadIdx.x; u < ST * 2 * 64; u += blockDim.x) {
+    const int ul = u & 63, ui = ul & 31, ug = ul >> 5, f = u >> 6, st = f >> 1, kk = f & 1;
+    const int s = 32 * st + ui;
+    bf16x8 e;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) e[j] = (__bf16)(s < S ? w_slice[s * 32 + 16 * kk + 8 * ug + j] : 0.f);
+    wsl[u] = __builtin_bit_cast(u32x4, e);
+  }
+  for (int s = threadIdx.x; s < ST * 32; s += blockDim.x) bsl[s] = s < S ? b_slice[s] : -1e30f;  // slices beyond S: weight 0
+}
+
+// ------------------------------------------------------------------------------------------------
+// slice_softmax_reduce_kernel: slice weights and the first pass of the slice-token sums in one kernel.
+// grid (G, B, head groups), one wave per head of the group; wave h walks the batch's 32-point tiles g, g + G, ...
+// and keeps the sums of its (batch, head) in registers:
+//   w^T (32 s x 32 pts, lane <-> slice) = chunk . SEL          (an exact MFMA transpose, as in slice_reduce_kernel)
+//   norm[s] += sum over the tile's points;   tok^T (32 d x 32 s) += fx_chunk (A: rows d, k = points) . bf16(w^T)
+// One partial per workgroup row: partials[g][b][h][s][0..D-1] = sum_n w fx, [..][D] = sum_n w.
+// ------------------------------------------------------------------------------------------------
+template <int S>
+__global__ __launch_bounds__(512) void slice_softmax_reduce_kernel(const uint16_t *__restrict__ x_mid,
+                                                                   const u32x4 *__restrict__ fx_pack,
+                                                                   const float *__restrict__ w_slice,
+                                                                   const float *__restrict__ b_slice,
+                                                                   const float *__restrict__ temperature,
+                                                                   float *__restrict__ partials, int64_t N, int tpb,
+                                                                   int H) {
+  constexpr int ST = (S + 31) / 32, NCH = S / 16, D1 = 33;
+  __shared__ u32x4 wsl[ST * 2 * 64];
+  __shared__ float bsl[ST * 32];
+  const int tid = threadIdx.x, lane = tid & 63, i = lane & 31, g = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int h = blockIdx.z * (blockDim.x >> 6) + wave;
+  const int b = blockIdx.y;
+  const int HD = H * 32;
+  stage_slice_projection<S>(w_slice, b_slice, wsl, bsl);
+  __syncthreads();
+  const float sc = kLog2e / clamp_temperature(temperature[h]);
+  u32x4 sel[2];
+#pragma unroll
+  for (int par = 0; par < 2; ++par) {
+    bf16x8 s8;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) s8[j] = (__bf16)((i == kperm(par, g, j)) ? 1.f : 0.f);
+    sel[par] = __builtin_bit_cast(u32x4, s8);
+  }
+  f32x16 tok[ST];
+  float nrm[ST];
+#pragma unroll
+  for (int st = 0; st < ST; ++st) {
+    nrm[st] = 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) tok[st][r] = 0.f;
+  }
+  for (int t = blockIdx.x; t < tpb; t += gridDim.x) {
+    const int64_t n = (int64_t)t * 32 + i;
+    const bool valid = n < N;
+    const uint16_t *row = x_mid + ((int64_t)b * N + (valid ? n : N - 1)) * HD + h * 32 + 8 * g;
+    const u32x4 xm0 = *reinterpret_cast<const u32x4 *>(row), xm1 = *reinterpret_cast<const u32x4 *>(row + 16);
+    const u32x4 *fsrc = fx_pack + ((((int64_t)b * tpb + t) * H + h) * 2) * 64 + lane;
+    const u32x4 f0 = fsrc[0], f1 = fsrc[64];
+    u32x4 chunk[NCH];
+    slice_weights_of_tile<S>(wsl, bsl, xm0, xm1, sc, valid, lane, g, chunk);
+#pragma unroll
+    for (int st = 0; st < ST; ++st) {
+      f32x16 tr;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) tr[r] = 0.f;
+      tr = mma(chunk[2 * st], sel[0], tr);
+      if (2 * st + 1 < NCH) tr = mma(chunk[2 * st + 1 < NCH ? 2 * st + 1 : 0], sel[1], tr);
+      float s16 = 0.f;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) s16 += tr[r];
+      nrm[st] += s16;
+      tok[st] = mma(f0, pack_half<0>(tr), tok[st]);
+      tok[st] = mma(f1, pack_half<1>(tr), tok[st]);
+    }
+  }
+  float *dst = partials + (((int64_t)blockIdx.x * gridDim.y + b) * H + h) * (S * D1);
+#pragma unroll
+  for (int st = 0; st < ST; ++st) {
+    const int s = 32 * st + i;
+    const float total = half_sum(nrm[st]);
+    if (s < S) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) dst[s * D1 + rowmap(r, g)] = tok[st][r];
+      if (g == 0) dst[s * D1 + 32] = total;
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// deslice_recompute_kernel: the attended tokens back to the points, slice weights recomputed from x_mid.
+// grid (G, B, head groups), one wave per head of the group;
+//   out_x^T_h (32 d x 32 pts) = tok'^T_h (A: tokp fragments, registers) . w_h (B: the chunks)
+// out_x may be x_mid itself: a wave reads the 64 bytes of its (point, head) before it writes them, and nobody else
+// touches them.
+// ------------------------------------------------------------------------------------------------
+template <int S>
+__global__ __launch_bounds__(512) void deslice_recompute_kernel(const uint16_t *x_mid, const u32x4 *__restrict__ tokp,
+                                                                const float *__restrict__ w_slice,
+                                                                const float *__restrict__ b_slice,
+                                                                const float *__restrict__ temperature, uint16_t *out_x,
+                                                                int64_t N, int tpb, int H) {
+  constexpr int ST = (S + 31) / 32, NCH = S / 16;
+  __shared__ u32x4 wsl[ST * 2 * 64];
+  __shared__ float bsl[ST * 32];
+  const int tid = threadIdx.x, lane = tid & 63, i = lane & 31, g = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int h = blockIdx.z * (blockDim.x >> 6) + wave;
+  const int b = blockIdx.y;
+  const int HD = H * 32;
+  stage_slice_projection<S>(w_slice, b_slice, wsl, bsl);
+  __syncthreads();
+  const float sc = kLog2e / clamp_temperature(temperature[h]);
+  u32x4 tp[NCH];
+#pragma unroll
+  for (int cq = 0; cq < NCH; ++cq) tp[cq] = tokp[(((int64_t)b * H + h) * NCH + cq) * 64 + lane];
+  for (int t = blockIdx.x; t < tpb; t += gridDim.x) {
+    const int64_t n = (int64_t)t * 32 + i;
+    const bool valid = n < N;
+    const int64_t m = (int64_t)b * N + (valid ? n : N - 1);
+    const uint16_t *row = x_mid + m * HD + h * 32 + 8 * g;
+    const u32x4 xm0 = *reinterpret_cast<const u32x4 *>(row), xm1 = *reinterpret_cast<const u32x4 *>(row + 16);
+    u32x4 chunk[NCH];
+    slice_weights_of_tile<S>(wsl, bsl, xm0, xm1, sc, valid, lane, g, chunk);
+    f32x16 ox;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) ox[r] = 0.f;
+#pragma unroll
+    for (int cq = 0; cq < NCH; ++cq) ox = mma(tp[cq], chunk[cq], ox);
+    store_tile_natural(ox, out_x + m * HD + h * 32, g, valid);
+  }
+}
+
 // shapes of the staged path: what the fused kernels serve plus C = 512, large enough for the row kernels to pay off
 bool staged_supported(int dtype, const pa_shape &s) {
   // grid convolutions as projections: the implicit-GEMM kernel writes the same two layouts (tap-major weights)
@@ -258,6 +441,66 @@ int slice_softmax_pack_plus(const pa_shape &s, const pa_params &p, const pa_plus
     default: return PA_ERR_UNSUPPORTED;
   }
 #undef PA_LAUNCH_SSPP
+  return launch_status();
+}
+
+// grid of the two recomputing kernels: waves = heads per workgroup, about two workgroups per CU
+static void recompute_grid(const pa_shape &s, int num_cu, dim3 *grid, dim3 *block) {
+  const int waves = (int)(s.H < 8 ? s.H : 8);
+  const int groups = (int)(s.H / waves);
+  int64_t gx = (2 * (int64_t)num_cu + s.B * groups - 1) / (s.B * groups);
+  const int64_t tpb = tiles_per_batch(s);
+  if (gx > tpb) gx = tpb;
+  if (gx < 1) gx = 1;
+  *grid = dim3((unsigned)gx, (unsigned)s.B, (unsigned)groups);
+  *block = dim3((unsigned)(waves * 64));
+}
+
+int64_t softmax_reduce_groups(const pa_shape &s, int num_cu) {
+  dim3 grid, block;
+  recompute_grid(s, num_cu, &grid, &block);
+  return grid.x;
+}
+
+int slice_softmax_reduce(const pa_shape &s, const pa_params &p, const void *x_mid, const void *fx_pack,
+                         float *partials, int num_cu, hipStream_t st) {
+  if (s.H % (s.H < 8 ? s.H : 8) != 0) return PA_ERR_UNSUPPORTED;
+  dim3 grid, block;
+  recompute_grid(s, num_cu, &grid, &block);
+  const int tpb = (int)tiles_per_batch(s);
+#define PA_LAUNCH_SSR(SS)                                                                                            \
+  hipLaunchKernelGGL((slice_softmax_reduce_kernel<SS>), grid, block, 0, st, static_cast<const uint16_t *>(x_mid),    \
+                     static_cast<const u32x4 *>(fx_pack), p.in_project_slice_weight, p.in_project_slice_bias,        \
+                     p.temperature, partials, s.N, tpb, (int)s.H)
+  switch (s.S) {
+    case 16: PA_LAUNCH_SSR(16); break;
+    case 32: PA_LAUNCH_SSR(32); break;
+    case 64: PA_LAUNCH_SSR(64); break;
+    case 128: PA_LAUNCH_SSR(128); break;
+    default: return PA_ERR_UNSUPPORTED;
+  }
+#undef PA_LAUNCH_SSR
+  return launch_status();
+}
+
+int deslice_recompute(const pa_shape &s, const pa_params &p, const void *x_mid, const void *tokp, void *out_x,
+                      int num_cu, hipStream_t st) {
+  if (s.H % (s.H < 8 ? s.H : 8) != 0) return PA_ERR_UNSUPPORTED;
+  dim3 grid, block;
+  recompute_grid(s, num_cu, &grid, &block);
+  const int tpb = (int)tiles_per_batch(s);
+#define PA_LAUNCH_DR(SS)                                                                                          \
+  hipLaunchKernelGGL((deslice_recompute_kernel<SS>), grid, block, 0, st, static_cast<const uint16_t *>(x_mid),    \
+                     static_cast<const u32x4 *>(tokp), p.in_project_slice_weight, p.in_project_slice_bias,        \
+                     p.temperature, static_cast<uint16_t *>(out_x), s.N, tpb, (int)s.H)
+  switch (s.S) {
+    case 16: PA_LAUNCH_DR(16); break;
+    case 32: PA_LAUNCH_DR(32); break;
+    case 64: PA_LAUNCH_DR(64); break;
+    case 128: PA_LAUNCH_DR(128); break;
+    default: return PA_ERR_UNSUPPORTED;
+  }
+#undef PA_LAUNCH_DR
   return launch_status();
 }
 
