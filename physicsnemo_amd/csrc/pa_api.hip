@@ -113,7 +113,7 @@ MfmaPlan plan_mfma(const pa_shape &s) {
 // Workspace plan of the staged MFMA path.  The slice weights are never stored: the token sums and the hand-back to
 // the points each recompute them from x_mid.
 struct StagedPlan {
-  int64_t off_x_mid, off_fx, off_partials, off_tok, off_norm, off_tok_out, off_tokp, total;
+  int64_t off_x_mid, off_fx, off_partials, off_tok, off_norm, off_tok_out, off_tokp, off_wout, total;
   int64_t G;
 };
 
@@ -122,8 +122,10 @@ StagedPlan plan_staged(const pa_shape &s) {
   p.G = pa::mfma::softmax_reduce_groups(s, compute_units());
   const int64_t tiles = s.B * pa::mfma::tiles_per_batch(s);
   int64_t off = 0;
-  p.off_x_mid = off;  // natural (B, N, H*32); overwritten by out_x, 64 bytes at a time, as the weights are recomputed
-  off += round_up(s.B * s.N * s.H * 32 * 2, 256);
+  // x_mid as rows (B, N, H*32) or as packed tiles (whole tiles per batch); overwritten by out_x, one point and head
+  // at a time, as the weights are recomputed
+  p.off_x_mid = off;
+  off += round_up(tiles * 32 * s.H * 32 * 2, 256);
   p.off_fx = off;
   off += round_up(tiles * s.H * 2 * 1024, 256);
   p.off_partials = off;
@@ -136,6 +138,8 @@ StagedPlan plan_staged(const pa_shape &s) {
   off += round_up(s.B * s.H * s.S * s.D * 4, 256);
   p.off_tokp = off;
   off += round_up(s.B * s.H * (s.S / 16) * 1024, 256);
+  p.off_wout = off;  // the three projections' weights in fragment order, where the row-owning kernels serve them
+  if (pa::mlp::linear_supported(PA_BF16, s.B * s.N, s.C)) off += round_up(3 * pa::mlp::linear_blob_bytes(s.C), 256);
   p.total = off;
   return p;
 }
@@ -878,6 +882,20 @@ int pa_layer_forward(int dtype, const pa_shape *shape, const pa_params *p, const
     float *tok = slice_token_out ? slice_token_out : reinterpret_cast<float *>(ws + sp.off_tok);
     float *norm = reinterpret_cast<float *>(ws + sp.off_norm);
     float *tok_out = reinterpret_cast<float *>(ws + sp.off_tok_out);
+    if (s.conv_k == 0 && pa::mlp::linear_supported(dtype, s.B * s.N, s.C)) {
+      // every stage on packed tiles of 32 points: projections, token sums, hand-back, out_linear with the tail
+      char *blob = ws + sp.off_wout;
+      if ((rc = pa::mlp::project_packed(s.B, s.N, s.C, p->in_project_x_weight, p->in_project_x_bias,
+                                        p->in_project_fx_weight, p->in_project_fx_bias, x, x_mid, fxp, blob,
+                                        compute_units(), st)))
+        return rc;
+      if ((rc = pa::mfma::slice_softmax_reduce(s, *p, x_mid, true, fxp, partials, compute_units(), st))) return rc;
+      if ((rc = pa::mfma::combine_attention(s, *p, nullptr, partials, sp.G, tok, norm, tok_out, tokp, st))) return rc;
+      if ((rc = pa::mfma::deslice_recompute(s, *p, x_mid, true, tokp, x_mid, compute_units(), st))) return rc;
+      return pa::mlp::linear_packed(s.B, s.N, s.C, p->out_linear_weight, p->out_linear_bias, x_mid, y,
+                                    tail_active(tail) ? tail : nullptr, blob + 2 * pa::mlp::linear_blob_bytes(s.C),
+                                    compute_units(), st);
+    }
     pa::GemmArgs a{};  // x -> x_mid (natural) and fx_mid (packed): two weight sets over the same rows
     a.in = x;
     a.w[0] = p->in_project_x_weight;
@@ -900,10 +918,13 @@ int pa_layer_forward(int dtype, const pa_shape *shape, const pa_params *p, const
     a.pack_heads = (int)s.H;
     if (!pa::gemm::serves(a, 2, 2)) return PA_ERR_UNSUPPORTED;
     if ((rc = pa::gemm::launch(a, 2, PA_BF16, st))) return rc;
-    if ((rc = pa::mfma::slice_softmax_reduce(s, *p, x_mid, fxp, partials, compute_units(), st))) return rc;
+    if ((rc = pa::mfma::slice_softmax_reduce(s, *p, x_mid, false, fxp, partials, compute_units(), st))) return rc;
     if ((rc = pa::mfma::combine_attention(s, *p, nullptr, partials, sp.G, tok, norm, tok_out, tokp, st))) return rc;
     void *out_x = x_mid;
-    if ((rc = pa::mfma::deslice_recompute(s, *p, x_mid, tokp, out_x, compute_units(), st))) return rc;
+    if ((rc = pa::mfma::deslice_recompute(s, *p, x_mid, false, tokp, out_x, compute_units(), st))) return rc;
+    if (pa::mlp::linear_supported(dtype, s.B * s.N, s.C))  // out_linear, the residual and the LayerNorm in one pass
+      return pa::mlp::linear(s.B * s.N, s.C, p->out_linear_weight, p->out_linear_bias, out_x, y,
+                             tail_active(tail) ? tail : nullptr, ws + sp.off_wout, compute_units(), st);
     if ((rc = pa::general::out_linear(dtype, s, *p, out_x, y, st))) return rc;
     if (tail_active(tail)) rc = pa::general::residual_ln(dtype, s, y, *tail, st);
     return rc;

@@ -161,10 +161,11 @@ int slice_softmax_pack(const pa_shape &s, const pa_params &p, const void *x_mid,
 // the same weights recomputed where they are used, never stored: token sums (softmax_reduce_groups partials) and
 // the hand-back to the points (out_x may be x_mid)
 int64_t softmax_reduce_groups(const pa_shape &s, int num_cu);
-int slice_softmax_reduce(const pa_shape &s, const pa_params &p, const void *x_mid, const void *fx_pack,
+// packed_x: x_mid (and out_x) are packed operand tiles [tile][head][2][64 lanes] of 16 bytes instead of rows
+int slice_softmax_reduce(const pa_shape &s, const pa_params &p, const void *x_mid, bool packed_x, const void *fx_pack,
                          float *partials, int num_cu, hipStream_t st);
-int deslice_recompute(const pa_shape &s, const pa_params &p, const void *x_mid, const void *tokp, void *out_x,
-                      int num_cu, hipStream_t st);
+int deslice_recompute(const pa_shape &s, const pa_params &p, const void *x_mid, bool packed_x, const void *tokp,
+                      void *out_x, int num_cu, hipStream_t st);
 bool backward_supported(const pa_shape &s);
 int64_t backward_groups(const pa_shape &s, int num_cu);
 int64_t backward_tables_bytes(const pa_shape &s);
@@ -198,6 +199,18 @@ int64_t blob_bytes(int64_t C, int64_t F);
 int pack(int64_t C, int64_t F, const void *w1, const void *w2, void *blob, hipStream_t st);
 int forward(int64_t rows, int64_t C, int64_t F, const void *blob, const float *b1, const float *b2, const void *u,
             void *y, const pa_block_tail *tail, int num_cu, hipStream_t st);
+// y = W x + bias [+ residual] [-> LayerNorm] for bf16 rows, W (C x C) bf16 row-major; blob: linear_blob_bytes(C) of scratch
+bool linear_supported(int dtype, int64_t rows, int64_t C);
+int64_t linear_blob_bytes(int64_t C);
+int linear(int64_t rows, int64_t C, const void *w, const float *bias, const void *x, void *y, const pa_block_tail *tail,
+           void *blob, int num_cu, hipStream_t st);
+// the same with x as packed operand tiles [B tpb][C / 32][2][64 lanes] (k order kperm within a head)
+int linear_packed(int64_t B, int64_t N, int64_t C, const void *w, const float *bias, const void *x_pack, void *y,
+                  const pa_block_tail *tail, void *blob, int num_cu, hipStream_t st);
+// the layer's two Linear input projections as packed operand tiles; blob: 2 linear_blob_bytes(C) of scratch
+int project_packed(int64_t B, int64_t N, int64_t C, const void *w_x, const float *b_x, const void *w_fx,
+                   const float *b_fx, const void *x, void *xm_pack, void *fx_pack, void *blob, int num_cu,
+                   hipStream_t st);
 }  // namespace mlp
 
 }  // namespace pa

@@ -241,8 +241,9 @@ __device__ __forceinline__ void slice_weights_of_tile(const u32x4 *__restrict__ 
   for (int cq = 0; cq < NCH; ++cq) chunk[cq] = (cq & 1) ? pack_half<1>(lg[cq >> 1], inv) : pack_half<0>(lg[cq >> 1], inv);
 }
 
-// W_slice as A operands (k = d in natural order) and the slice bias, as slice_softmax_pack_kernel stages them
-template <int S>
+// W_slice as A operands and the slice bias, as slice_softmax_pack_kernel stages them; the reduction index runs over
+// d in natural order (x_mid read from its rows) or in kperm order (PACKED_X: x_mid read as packed operand tiles)
+template <int S, bool PACKED_X>
 __device__ __forceinline__ void stage_slice_projection(const float *__restrict__ w_slice, const float *__restrict__ b_slice,
                                                        u32x4 *wsl, float *bsl) {
   constexpr int ST = (S + 31) / 32;
@@ -251,7 +252,8 @@ __device__ __forceinline__ void stage_slice_projection(const float *__restrict__
     const int s = 32 * st + ui;
     bf16x8 e;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) e[j] = (__bf16)(s < S ? w_slice[s * 32 + 16 * kk + 8 * ug + j] : 0.f);
+    for (int j = 0; j < 8; ++j)
+      e[j] = (__bf16)(s < S ? w_slice[s * 32 + (PACKED_X ? kperm(kk, ug, j) : 16 * kk + 8 * ug + j)] : 0.f);
     wsl[u] = __builtin_bit_cast(u32x4, e);
   }
   for (int s = threadIdx.x; s < ST * 32; s += blockDim.x) bsl[s] = s < S ? b_slice[s] : -1e30f;  // slices beyond S: weight 0
@@ -265,7 +267,8 @@ __device__ __forceinline__ void stage_slice_projection(const float *__restrict__
 //   norm[s] += sum over the tile's points;   tok^T (32 d x 32 s) += fx_chunk (A: rows d, k = points) . bf16(w^T)
 // One partial per workgroup row: partials[g][b][h][s][0..D-1] = sum_n w fx, [..][D] = sum_n w.
 // ------------------------------------------------------------------------------------------------
-template <int S>
+// PACKED_X: x_mid is [tile][head][2][lane] (the B operands themselves) instead of (B, N, H*32) rows.
+template <int S, bool PACKED_X>
 __global__ __launch_bounds__(512) void slice_softmax_reduce_kernel(const uint16_t *__restrict__ x_mid,
                                                                    const u32x4 *__restrict__ fx_pack,
                                                                    const float *__restrict__ w_slice,
@@ -281,7 +284,7 @@ __global__ __launch_bounds__(512) void slice_softmax_reduce_kernel(const uint16_
   const int h = blockIdx.z * (blockDim.x >> 6) + wave;
   const int b = blockIdx.y;
   const int HD = H * 32;
-  stage_slice_projection<S>(w_slice, b_slice, wsl, bsl);
+  stage_slice_projection<S, PACKED_X>(w_slice, b_slice, wsl, bsl);
   __syncthreads();
   const float sc = kLog2e / clamp_temperature(temperature[h]);
   u32x4 sel[2];
@@ -303,8 +306,16 @@ __global__ __launch_bounds__(512) void slice_softmax_reduce_kernel(const uint16_
   for (int t = blockIdx.x; t < tpb; t += gridDim.x) {
     const int64_t n = (int64_t)t * 32 + i;
     const bool valid = n < N;
-    const uint16_t *row = x_mid + ((int64_t)b * N + (valid ? n : N - 1)) * HD + h * 32 + 8 * g;
-    const u32x4 xm0 = *reinterpret_cast<const u32x4 *>(row), xm1 = *reinterpret_cast<const u32x4 *>(row + 16);
+    u32x4 xm0, xm1;
+    if constexpr (PACKED_X) {
+      const u32x4 *xsrc = reinterpret_cast<const u32x4 *>(x_mid) + ((((int64_t)b * tpb + t) * H + h) * 2) * 64 + lane;
+      xm0 = xsrc[0];
+      xm1 = xsrc[64];
+    } else {
+      const uint16_t *row = x_mid + ((int64_t)b * N + (valid ? n : N - 1)) * HD + h * 32 + 8 * g;
+      xm0 = *reinterpret_cast<const u32x4 *>(row);
+      xm1 = *reinterpret_cast<const u32x4 *>(row + 16);
+    }
     const u32x4 *fsrc = fx_pack + ((((int64_t)b * tpb + t) * H + h) * 2) * 64 + lane;
     const u32x4 f0 = fsrc[0], f1 = fsrc[64];
     u32x4 chunk[NCH];
@@ -344,7 +355,9 @@ __global__ __launch_bounds__(512) void slice_softmax_reduce_kernel(const uint16_
 // out_x may be x_mid itself: a wave reads the 64 bytes of its (point, head) before it writes them, and nobody else
 // touches them.
 // ------------------------------------------------------------------------------------------------
-template <int S>
+// PACKED_X: x_mid and out_x are [tile][head][2][lane] operand tiles (out_x: lanes <-> points, k = the head's channels in
+// kperm order, what linear_rows_kernel reads as its rows).
+template <int S, bool PACKED_X>
 __global__ __launch_bounds__(512) void deslice_recompute_kernel(const uint16_t *x_mid, const u32x4 *__restrict__ tokp,
                                                                 const float *__restrict__ w_slice,
                                                                 const float *__restrict__ b_slice,
@@ -358,7 +371,7 @@ __global__ __launch_bounds__(512) void deslice_recompute_kernel(const uint16_t *
   const int h = blockIdx.z * (blockDim.x >> 6) + wave;
   const int b = blockIdx.y;
   const int HD = H * 32;
-  stage_slice_projection<S>(w_slice, b_slice, wsl, bsl);
+  stage_slice_projection<S, PACKED_X>(w_slice, b_slice, wsl, bsl);
   __syncthreads();
   const float sc = kLog2e / clamp_temperature(temperature[h]);
   u32x4 tp[NCH];
@@ -368,8 +381,17 @@ __global__ __launch_bounds__(512) void deslice_recompute_kernel(const uint16_t *
     const int64_t n = (int64_t)t * 32 + i;
     const bool valid = n < N;
     const int64_t m = (int64_t)b * N + (valid ? n : N - 1);
-    const uint16_t *row = x_mid + m * HD + h * 32 + 8 * g;
-    const u32x4 xm0 = *reinterpret_cast<const u32x4 *>(row), xm1 = *reinterpret_cast<const u32x4 *>(row + 16);
+    const int64_t pk = ((((int64_t)b * tpb + t) * H + h) * 2) * 64 + lane;
+    u32x4 xm0, xm1;
+    if constexpr (PACKED_X) {
+      const u32x4 *xsrc = reinterpret_cast<const u32x4 *>(x_mid) + pk;
+      xm0 = xsrc[0];
+      xm1 = xsrc[64];
+    } else {
+      const uint16_t *row = x_mid + m * HD + h * 32 + 8 * g;
+      xm0 = *reinterpret_cast<const u32x4 *>(row);
+      xm1 = *reinterpret_cast<const u32x4 *>(row + 16);
+    }
     u32x4 chunk[NCH];
     slice_weights_of_tile<S>(wsl, bsl, xm0, xm1, sc, valid, lane, g, chunk);
     f32x16 ox;
@@ -377,7 +399,13 @@ __global__ __launch_bounds__(512) void deslice_recompute_kernel(const uint16_t *
     for (int r = 0; r < 16; ++r) ox[r] = 0.f;
 #pragma unroll
     for (int cq = 0; cq < NCH; ++cq) ox = mma(tp[cq], chunk[cq], ox);
-    store_tile_natural(ox, out_x + m * HD + h * 32, g, valid);
+    if constexpr (PACKED_X) {
+      u32x4 *odst = reinterpret_cast<u32x4 *>(out_x) + pk;
+      odst[0] = pack_half<0>(ox);
+      odst[64] = pack_half<1>(ox);
+    } else {
+      store_tile_natural(ox, out_x + m * HD + h * 32, g, valid);
+    }
   }
 }
 
@@ -462,16 +490,18 @@ int64_t softmax_reduce_groups(const pa_shape &s, int num_cu) {
   return grid.x;
 }
 
-int slice_softmax_reduce(const pa_shape &s, const pa_params &p, const void *x_mid, const void *fx_pack,
+int slice_softmax_reduce(const pa_shape &s, const pa_params &p, const void *x_mid, bool packed_x, const void *fx_pack,
                          float *partials, int num_cu, hipStream_t st) {
   if (s.H % (s.H < 8 ? s.H : 8) != 0) return PA_ERR_UNSUPPORTED;
   dim3 grid, block;
   recompute_grid(s, num_cu, &grid, &block);
   const int tpb = (int)tiles_per_batch(s);
-#define PA_LAUNCH_SSR(SS)                                                                                            \
-  hipLaunchKernelGGL((slice_softmax_reduce_kernel<SS>), grid, block, 0, st, static_cast<const uint16_t *>(x_mid),    \
-                     static_cast<const u32x4 *>(fx_pack), p.in_project_slice_weight, p.in_project_slice_bias,        \
+#define PA_LAUNCH_SSR1(SS, PK)                                                                                         \
+  hipLaunchKernelGGL((slice_softmax_reduce_kernel<SS, PK>), grid, block, 0, st, static_cast<const uint16_t *>(x_mid), \
+                     static_cast<const u32x4 *>(fx_pack), p.in_project_slice_weight, p.in_project_slice_bias,          \
                      p.temperature, partials, s.N, tpb, (int)s.H)
+#define PA_LAUNCH_SSR(SS) \
+  if (packed_x) PA_LAUNCH_SSR1(SS, true); else PA_LAUNCH_SSR1(SS, false)
   switch (s.S) {
     case 16: PA_LAUNCH_SSR(16); break;
     case 32: PA_LAUNCH_SSR(32); break;
@@ -480,19 +510,22 @@ int slice_softmax_reduce(const pa_shape &s, const pa_params &p, const void *x_mi
     default: return PA_ERR_UNSUPPORTED;
   }
 #undef PA_LAUNCH_SSR
+#undef PA_LAUNCH_SSR1
   return launch_status();
 }
 
-int deslice_recompute(const pa_shape &s, const pa_params &p, const void *x_mid, const void *tokp, void *out_x,
-                      int num_cu, hipStream_t st) {
+int deslice_recompute(const pa_shape &s, const pa_params &p, const void *x_mid, bool packed_x, const void *tokp,
+                      void *out_x, int num_cu, hipStream_t st) {
   if (s.H % (s.H < 8 ? s.H : 8) != 0) return PA_ERR_UNSUPPORTED;
   dim3 grid, block;
   recompute_grid(s, num_cu, &grid, &block);
   const int tpb = (int)tiles_per_batch(s);
-#define PA_LAUNCH_DR(SS)                                                                                          \
-  hipLaunchKernelGGL((deslice_recompute_kernel<SS>), grid, block, 0, st, static_cast<const uint16_t *>(x_mid),    \
-                     static_cast<const u32x4 *>(tokp), p.in_project_slice_weight, p.in_project_slice_bias,        \
+#define PA_LAUNCH_DR1(SS, PK)                                                                                      \
+  hipLaunchKernelGGL((deslice_recompute_kernel<SS, PK>), grid, block, 0, st, static_cast<const uint16_t *>(x_mid), \
+                     static_cast<const u32x4 *>(tokp), p.in_project_slice_weight, p.in_project_slice_bias,          \
                      p.temperature, static_cast<uint16_t *>(out_x), s.N, tpb, (int)s.H)
+#define PA_LAUNCH_DR(SS) \
+  if (packed_x) PA_LAUNCH_DR1(SS, true); else PA_LAUNCH_DR1(SS, false)
   switch (s.S) {
     case 16: PA_LAUNCH_DR(16); break;
     case 32: PA_LAUNCH_DR(32); break;
@@ -501,6 +534,7 @@ int deslice_recompute(const pa_shape &s, const pa_params &p, const void *x_mid, 
     default: return PA_ERR_UNSUPPORTED;
   }
 #undef PA_LAUNCH_DR
+#undef PA_LAUNCH_DR1
   return launch_status();
 }
 

@@ -492,6 +492,123 @@ __device__ __forceinline__ void mma_in_vgprs(u32x4 a, u32x4 b, f32x16 &acc) {
   asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(acc) : "v"(a), "v"(b));
 }
 
+// Epilogue of the row-owning kernels: a wave's y^T (channel 32 ct + rowmap(r, g) of row i, C channels x 32 rows) to
+// row-major bf16 rows, + residual, LayerNorm, full-row stores.  The rows pass through `stg`, the wave's own 16 KB of
+// LDS, RPR = 8192 / C rows at a time; after_staging() is called once the last round is staged (the accumulators are
+// free from then on).  gams / bets: LayerNorm weight and bias in LDS.
+template <int C, bool HAS_RES, bool HAS_LN, class AfterStaging>
+__device__ __forceinline__ void finish_rows(const f32x16 (&yacc)[C / 32], uint32_t *stg, int i, int g, int64_t row0,
+                                            int64_t M, const uint16_t *__restrict__ residual, uint16_t *__restrict__ y,
+                                            uint16_t *__restrict__ ln_out, const float *gams, const float *bets,
+                                            float ln_eps, AfterStaging &&after_staging) {
+  constexpr int CT = C / 32;
+  constexpr int G4 = C / 4;             // 8-byte granules (4 channels) per staged row
+  constexpr int RPR = 16384 / (2 * C);  // rows staged per round
+  constexpr int NROUND = 32 / RPR;
+  // lane indices taken afresh, so that nothing derived from them for the epilogue is kept across the slot loop
+  int il = i, gl = g;
+  asm volatile("" : "+v"(il), "+v"(gl));
+  const int hl = gl;  // each half of the wave finishes one row per step
+  typedef uint32_t rowv __attribute__((ext_vector_type(4)));
+  typedef float f32x4 __attribute__((ext_vector_type(4)));
+  constexpr int NV = C / 256;  // 16-byte pieces per lane and row: piece v = channels 256 v + 8 il .. + 7
+  static_assert(C % 256 == 0, "half a wave covers 256 consecutive channels per access");
+  // y^T -> bf16 once: yp[ct][q] = channels 32 ct + 8 q + 4 g .. + 3 of row i; the accumulators are free after this
+  u32x2 yp[CT][4];
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      yp[ct][q][0] = pack2(yacc[ct][4 * q + 0], yacc[ct][4 * q + 1]);
+      yp[ct][q][1] = pack2(yacc[ct][4 * q + 2], yacc[ct][4 * q + 3]);
+    }
+  constexpr int NIT = RPR / 2;             // steps per round: two rows each
+  constexpr int PF = NIT < 4 ? NIT : 4;    // residual rows are fetched this many steps ahead
+#pragma unroll
+  for (int rd = 0; rd < NROUND; ++rd) {
+    rowv rsd[NIT][NV];
+    auto load_residual = [&](auto rr_) {
+      constexpr int rr = decltype(rr_)::value;
+      if constexpr (HAS_RES) {
+        int64_t r = row0 + rd * RPR + 2 * rr + hl;
+        if (r >= M) r = M > 0 ? M - 1 : 0;  // M = 0: a wave without rows (nothing is stored)
+#pragma unroll
+        for (int v = 0; v < NV; ++v) rsd[rr][v] = *reinterpret_cast<const rowv *>(residual + r * C + 256 * v + 8 * il);
+      }
+    };
+    static_for<PF>(load_residual);
+    // staged rows: granule gr (4 channels) of row rw sits at gr ^ ((2 rw) % G4)
+    if (NROUND == 1 || (il / RPR) == rd) {
+      const int rw = il % RPR;
+#pragma unroll
+      for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int gr = (8 * ct + 2 * q + gl) ^ ((2 * rw) & (G4 - 1));
+          *reinterpret_cast<u32x2 *>(stg + rw * (C / 2) + gr * 2) = yp[ct][q];
+        }
+    }
+    // the wave's LDS operations complete in order: its reads below see the writes above.  Once the last round is
+    // staged the rows of this workgroup's next block can travel (past the end: this block again)
+    if (rd == NROUND - 1) after_staging();
+    // two rows per step: lanes 0-31 one row, lanes 32-63 the next
+    static_for<NIT>([&](auto rr_) {
+      constexpr int rr = decltype(rr_)::value;
+      if constexpr (rr + PF < NIT) load_residual(std::integral_constant<int, rr + PF>{});
+      const int rw = 2 * rr + hl;
+      const int64_t r = row0 + rd * RPR + rw;
+      const bool ok = r < M;
+      float val[8 * NV];
+#pragma unroll
+      for (int v = 0; v < NV; ++v) {
+        // granules 64 v + 2 il, + 1 of row rw; the swizzle flips an even number, so the pair stays adjacent
+        const rowv sv = *reinterpret_cast<const rowv *>(stg + rw * (C / 2) + (((64 * v + 2 * il) ^ ((2 * rw) & (G4 - 1))) << 1));
+        rowv ob;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+          float t0 = __uint_as_float(sv[w] << 16), t1 = __uint_as_float(sv[w] & 0xffff0000u);
+          if constexpr (HAS_RES) {  // the MLP output is a bf16 tensor; the sum is rounded again
+            t0 += __uint_as_float(rsd[rr][v][w] << 16);
+            t1 += __uint_as_float(rsd[rr][v][w] & 0xffff0000u);
+          }
+          ob[w] = pack2(t0, t1);
+          val[8 * v + 2 * w] = __uint_as_float(ob[w] << 16);
+          val[8 * v + 2 * w + 1] = __uint_as_float(ob[w] & 0xffff0000u);
+        }
+        if (ok) *reinterpret_cast<rowv *>(y + r * C + 256 * v + 8 * il) = ob;
+      }
+      if constexpr (HAS_LN) {
+        float s1 = 0.f;
+#pragma unroll
+        for (int k = 0; k < 8 * NV; ++k) s1 += val[k];
+        const float mean = half_wave_sum(s1) * (1.f / C);
+        float s2 = 0.f;
+#pragma unroll
+        for (int k = 0; k < 8 * NV; ++k) {
+          const float dl = val[k] - mean;
+          s2 = fmaf(dl, dl, s2);
+        }
+        const float rstd = rsqrtf(half_wave_sum(s2) * (1.f / C) + ln_eps);
+        const float shift = -mean * rstd;
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+          const f32x4 ga = *reinterpret_cast<const f32x4 *>(gams + 256 * v + 8 * il), gb = *reinterpret_cast<const f32x4 *>(gams + 256 * v + 8 * il + 4);
+          const f32x4 ba = *reinterpret_cast<const f32x4 *>(bets + 256 * v + 8 * il), bb = *reinterpret_cast<const f32x4 *>(bets + 256 * v + 8 * il + 4);
+          rowv lb;
+#pragma unroll
+          for (int w = 0; w < 4; ++w) {
+            const float g0 = w < 2 ? ga[2 * w] : gb[2 * w - 4], g1 = w < 2 ? ga[2 * w + 1] : gb[2 * w - 3];
+            const float c0 = w < 2 ? ba[2 * w] : bb[2 * w - 4], c1 = w < 2 ? ba[2 * w + 1] : bb[2 * w - 3];
+            lb[w] = pack2(fmaf(fmaf(val[8 * v + 2 * w], rstd, shift), g0, c0), fmaf(fmaf(val[8 * v + 2 * w + 1], rstd, shift), g1, c1));
+          }
+          if (ok) *reinterpret_cast<rowv *>(ln_out + r * C + 256 * v + 8 * il) = lb;
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    });
+  }
+}
+
 template <int C, int TAIL>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void mlp_rows_kernel(
     const u32x4 *__restrict__ blob, const float *__restrict__ b1, const float *__restrict__ b2,
@@ -502,9 +619,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   constexpr bool HAS_RES = TAIL == 1 || TAIL == 2, HAS_LN = TAIL == 1 || TAIL == 3;
   constexpr int KS = K::KS, CT = K::CT, HS = K::HS, NT = K::NT, NP = K::NP, SU = K::SU;
   constexpr int WU = SU / 4;    // units of a slot fetched by each wave (16 KB: four groups of four loads)
-  constexpr int G4 = C / 4;     // 8-byte granules (4 channels) per staged row
-  constexpr int RPR = 16384 / (2 * C);  // rows a wave stages per round of the epilogue (its 16 KB of the idle buffer)
-  constexpr int NROUND = 32 / RPR;
   extern __shared__ u32x4 smem[];
   u32x4 *wbuf = smem;  // 2 * SU
   float *b1s = reinterpret_cast<float *>(wbuf + 2 * SU);
@@ -657,109 +771,233 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     // ---- its own rows in its own quarter of it, RPR rows at a time ----
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's share of the next block's first slot has landed
     __syncthreads();
-    // lane indices taken afresh, so that nothing derived from them for the epilogue is kept across the slot loop
-    int il = i, gl = g;
-    asm volatile("" : "+v"(il), "+v"(gl));
-    const int hl = gl;  // each half of the wave finishes one row per step
-    uint32_t *stg = reinterpret_cast<uint32_t *>(wbuf + ((gs - 1) & 1) * SU + wave * WU);  // [RPR rows][C/2 words]
-    typedef uint32_t rowv __attribute__((ext_vector_type(4)));
-    typedef float f32x4 __attribute__((ext_vector_type(4)));
-    constexpr int NV = C / 256;  // 16-byte pieces per lane and row: piece v = channels 256 v + 8 il .. + 7
-    static_assert(C % 256 == 0, "half a wave covers 256 consecutive channels per access");
-    // y^T -> bf16 once: yp[ct][q] = channels 32 ct + 8 q + 4 g .. + 3 of row i; the accumulators are free after this
-    u32x2 yp[CT][4];
+    uint32_t *stg = reinterpret_cast<uint32_t *>(wbuf + ((gs - 1) & 1) * SU + wave * WU);  // this wave's 16 KB
+    // once the last rows are staged the rows of this workgroup's next block can travel (past the end: this block again)
+    finish_rows<C, HAS_RES, HAS_LN>(yacc, stg, i, g, row0, M, residual, y, ln_out, gams, bets, ln_eps,
+                                    [&]() { load_rows(mb + gridDim.x < nblocks ? mb + gridDim.x : mb, ub); });
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // nothing may still be landing in LDS when the workgroup ends
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// linear_rows_kernel: y = W x + b [+ residual] [-> LayerNorm(y)] for bf16 rows with C inputs and C outputs (the
+// layer's out_linear with the block's residual and the following LayerNorm, transolver.py:296-300), on the skeleton
+// of mlp_rows_kernel: a wave owns 32 rows (inputs as B operands, all C outputs of y^T in accumulation registers), W
+// streams through LDS in slots of 64 fragments in consumption order (fragment j of slot c: output tile j % CT,
+// k-step c (64 / CT) + j / CT), one barrier per slot, the epilogue above.
+// ---------------------------------------------------------------------------------------------------------------
+// head_order = 0: the reduction index of k-step ks runs over input channels 16 ks + 8 g + j (rows read in natural
+// layout); 1: over 32 (ks / 2) + kperm(ks % 2, g, j) (rows read as the packed operand tiles the slice kernels write)
+__global__ __launch_bounds__(256) void linear_pack_kernel(const uint16_t *__restrict__ w, u32x4 *__restrict__ blob, int C,
+                                                          int head_order) {
+  const int CT = C / 32, KPS = 64 / CT;
+  const int64_t total = (int64_t)C * C / 8;
+  for (int64_t u = (int64_t)blockIdx.x * 256 + threadIdx.x; u < total; u += (int64_t)gridDim.x * 256) {
+    const int c = (int)(u >> 12), j = (int)(u & 4095) >> 6, lane = (int)(u & 63), i = lane & 31, g = lane >> 5;
+    const int ct = j % CT, ks = c * KPS + j / CT;
+    const uint16_t *row = w + (int64_t)(32 * ct + i) * C;
+    if (!head_order) {
+      blob[u] = *reinterpret_cast<const u32x4 *>(row + 16 * ks + 8 * g);
+    } else {
+      uint16_t e[8];
+#pragma unroll
+      for (int q = 0; q < 8; ++q) e[q] = row[32 * (ks >> 1) + kperm(ks & 1, g, q)];
+      u32x4 v;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) v[q] = (uint32_t)e[2 * q] | ((uint32_t)e[2 * q + 1] << 16);
+      blob[u] = v;
+    }
+  }
+}
+
+// PACKED_IN: the rows arrive as packed operand tiles, x = [tile][head][2][lane] of 16 bytes with tile = b tpb + t
+// covering points 32 t .. 32 t + 31 of batch b (N points per batch, tpb tiles); a wave then owns one tile and a block
+// four consecutive ones.  Otherwise x is (M, C) row-major and a block 128 consecutive rows (N, tpb unused).
+template <int C, int TAIL, bool PACKED_IN>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void linear_rows_kernel(
+    const u32x4 *__restrict__ blob, const float *__restrict__ bias, const uint16_t *__restrict__ x,
+    uint16_t *__restrict__ y, const uint16_t *__restrict__ residual, const float *__restrict__ ln_gamma,
+    const float *__restrict__ ln_beta, float ln_eps, uint16_t *__restrict__ ln_out, int64_t M, int64_t nblocks,
+    int64_t N, int tpb) {
+  constexpr bool HAS_RES = TAIL == 1 || TAIL == 2, HAS_LN = TAIL == 1 || TAIL == 3;
+  constexpr int KS = C / 16, CT = C / 32, SU = 4096, WU = SU / 4;
+  constexpr int NSLOT = CT * KS / 64, KPS = 64 / CT;
+  static_assert(64 % CT == 0 && CT * KS % 64 == 0, "whole k-steps per slot");
+  extern __shared__ u32x4 smem[];
+  u32x4 *wbuf = smem;  // 2 * SU
+  float *bs = reinterpret_cast<float *>(wbuf + 2 * SU);
+  float *gams = bs + C, *bets = gams + C;
+  const int tid = threadIdx.x, lane = tid & 63, i = lane & 31, g = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: addresses derived from it stay scalar
+  for (int k = tid; k < C; k += 256) {
+    bs[k] = bias ? bias[k] : 0.f;
+    gams[k] = HAS_LN ? ln_gamma[k] : 1.f;
+    bets[k] = HAS_LN ? ln_beta[k] : 0.f;
+  }
+  __syncthreads();
+  auto fetch_group = [&](int64_t gs, int c, int k) {
+    const u32x4 *src = blob + (int64_t)c * SU + wave * WU + k * 256;
+    const unsigned dst = (unsigned)(uintptr_t)(wbuf + (gs & 1) * SU + wave * WU + k * 256);
+    load_4k_to_lds(src, lane * 16, dst);
+  };
+  const int64_t ntiles = PACKED_IN ? M : 0;  // PACKED_IN: M counts tiles
+  auto load_rows = [&](int64_t mb, u32x4(&ub)[KS]) {
+    if constexpr (PACKED_IN) {
+      int64_t gt = mb * 4 + wave;
+      if (gt >= ntiles) gt = ntiles - 1;
+      const u32x4 *src = reinterpret_cast<const u32x4 *>(x) + gt * (KS * 64) + lane;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) ub[ks] = src[ks * 64];
+    } else {
+      int64_t r = mb * kRowsPerBlock + wave * 32 + i;
+      if (r >= M) r = M - 1;
+      const uint16_t *src = x + r * C + 8 * g;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) ub[ks] = *reinterpret_cast<const u32x4 *>(src + 16 * ks);
+    }
+  };
+  int64_t gs = 0;
+  if ((int64_t)blockIdx.x < nblocks) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) fetch_group(0, 0, k);
+  }
+  u32x4 ub[KS];
+  if ((int64_t)blockIdx.x < nblocks) load_rows(blockIdx.x, ub);
+  for (int64_t mb = blockIdx.x; mb < nblocks; mb += gridDim.x) {
+    // first row of this wave and the end of its valid rows
+    int64_t row0 = mb * kRowsPerBlock + wave * 32, row_end = M;
+    if constexpr (PACKED_IN) {
+      const int64_t gt = mb * 4 + wave, bb = gt / tpb, t = gt - bb * tpb;
+      row0 = bb * N + t * 32;
+      row_end = gt < ntiles ? (bb + 1) * N : 0;  // tiles past the end own no rows
+      if (gt >= ntiles) row0 = 0;
+    }
+    f32x16 yacc[CT];
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct)
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        yp[ct][q][0] = pack2(yacc[ct][4 * q + 0], yacc[ct][4 * q + 1]);
-        yp[ct][q][1] = pack2(yacc[ct][4 * q + 2], yacc[ct][4 * q + 3]);
-      }
-    constexpr int NIT = RPR / 2;             // steps per round: two rows each
-    constexpr int PF = NIT < 4 ? NIT : 4;    // residual rows are fetched this many steps ahead
-#pragma unroll
-    for (int rd = 0; rd < NROUND; ++rd) {
-      rowv rsd[NIT][NV];
-      auto load_residual = [&](auto rr_) {
-        constexpr int rr = decltype(rr_)::value;
-        if constexpr (HAS_RES) {
-          int64_t r = row0 + rd * RPR + 2 * rr + hl;
-          if (r >= M) r = M - 1;
-#pragma unroll
-          for (int v = 0; v < NV; ++v) rsd[rr][v] = *reinterpret_cast<const rowv *>(residual + r * C + 256 * v + 8 * il);
-        }
-      };
-      static_for<PF>(load_residual);
-      // staged rows: granule gr (4 channels) of row rw sits at gr ^ ((2 rw) % G4)
-      if (NROUND == 1 || (il / RPR) == rd) {
-        const int rw = il % RPR;
-#pragma unroll
-        for (int ct = 0; ct < CT; ++ct)
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            const int gr = (8 * ct + 2 * q + gl) ^ ((2 * rw) & (G4 - 1));
-            *reinterpret_cast<u32x2 *>(stg + rw * (C / 2) + gr * 2) = yp[ct][q];
-          }
-      }
-      // the wave's LDS operations complete in order: its reads below see the writes above.  Once the last round is
-      // staged the rows of this workgroup's next block can travel (past the end: this block again)
-      if (rd == NROUND - 1) load_rows(mb + gridDim.x < nblocks ? mb + gridDim.x : mb, ub);
-      // two rows per step: lanes 0-31 one row, lanes 32-63 the next
-      static_for<NIT>([&](auto rr_) {
-        constexpr int rr = decltype(rr_)::value;
-        if constexpr (rr + PF < NIT) load_residual(std::integral_constant<int, rr + PF>{});
-        const int rw = 2 * rr + hl;
-        const int64_t r = row0 + rd * RPR + rw;
-        const bool ok = r < M;
-        float val[8 * NV];
-#pragma unroll
-        for (int v = 0; v < NV; ++v) {
-          // granules 64 v + 2 il, + 1 of row rw; the swizzle flips an even number, so the pair stays adjacent
-          const rowv sv = *reinterpret_cast<const rowv *>(stg + rw * (C / 2) + (((64 * v + 2 * il) ^ ((2 * rw) & (G4 - 1))) << 1));
-          rowv ob;
-#pragma unroll
-          for (int w = 0; w < 4; ++w) {
-            float t0 = __uint_as_float(sv[w] << 16), t1 = __uint_as_float(sv[w] & 0xffff0000u);
-            if constexpr (HAS_RES) {  // the MLP output is a bf16 tensor; the sum is rounded again
-              t0 += __uint_as_float(rsd[rr][v][w] << 16);
-              t1 += __uint_as_float(rsd[rr][v][w] & 0xffff0000u);
-            }
-            ob[w] = pack2(t0, t1);
-            val[8 * v + 2 * w] = __uint_as_float(ob[w] << 16);
-            val[8 * v + 2 * w + 1] = __uint_as_float(ob[w] & 0xffff0000u);
-          }
-          if (ok) *reinterpret_cast<rowv *>(y + r * C + 256 * v + 8 * il) = ob;
-        }
-        if constexpr (HAS_LN) {
-          float s1 = 0.f;
-#pragma unroll
-          for (int k = 0; k < 8 * NV; ++k) s1 += val[k];
-          const float mean = half_wave_sum(s1) * (1.f / C);
-          float s2 = 0.f;
-#pragma unroll
-          for (int k = 0; k < 8 * NV; ++k) {
-            const float dl = val[k] - mean;
-            s2 = fmaf(dl, dl, s2);
-          }
-          const float rstd = rsqrtf(half_wave_sum(s2) * (1.f / C) + ln_eps);
-          const float shift = -mean * rstd;
-#pragma unroll
-          for (int v = 0; v < NV; ++v) {
-            const f32x4 ga = *reinterpret_cast<const f32x4 *>(gams + 256 * v + 8 * il), gb = *reinterpret_cast<const f32x4 *>(gams + 256 * v + 8 * il + 4);
-            const f32x4 ba = *reinterpret_cast<const f32x4 *>(bets + 256 * v + 8 * il), bb = *reinterpret_cast<const f32x4 *>(bets + 256 * v + 8 * il + 4);
-            rowv lb;
-#pragma unroll
-            for (int w = 0; w < 4; ++w) {
-              const float g0 = w < 2 ? ga[2 * w] : gb[2 * w - 4], g1 = w < 2 ? ga[2 * w + 1] : gb[2 * w - 3];
-              const float c0 = w < 2 ? ba[2 * w] : bb[2 * w - 4], c1 = w < 2 ? ba[2 * w + 1] : bb[2 * w - 3];
-              lb[w] = pack2(fmaf(fmaf(val[8 * v + 2 * w], rstd, shift), g0, c0), fmaf(fmaf(val[8 * v + 2 * w + 1], rstd, shift), g1, c1));
-            }
-            if (ok) *reinterpret_cast<rowv *>(ln_out + r * C + 256 * v + 8 * il) = lb;
-          }
-        }
+      for (int r = 0; r < 16; ++r) yacc[ct][r] = bs[32 * ct + rowmap(r, g)];
+    static_for<NSLOT>([&](auto c_) {
+      constexpr int c = decltype(c_)::value;
+      // slot gs has landed and the other buffer is free (the first slot of a later block was waited for before the
+      // epilogue of the block before it, whose stores may still be in flight here)
+      if (c > 0 || gs == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      __syncthreads();
+      const u32x4 *wb = wbuf + (gs & 1) * SU + lane;
+      constexpr int RING = 8, AHEAD = 6;
+      u32x4 fr[RING];
+      static_for<AHEAD>([&](auto q) { fr[decltype(q)::value] = wb[decltype(q)::value * 64]; });
+      static_for<64>([&](auto j_) {
+        constexpr int j = decltype(j_)::value, ct = j % CT, ks = c * KPS + j / CT;
+        if constexpr (j + AHEAD < 64) fr[(j + AHEAD) % RING] = wb[(j + AHEAD) * 64];
+        yacc[ct] = mma(fr[j % RING], ub[ks], yacc[ct]);
+        if constexpr (j % 16 == 7) fetch_group(gs + 1, (c + 1) % NSLOT, j / 16);
         __builtin_amdgcn_sched_barrier(0);
       });
-    }
+      ++gs;
+    });
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's share of the next block's first slot has landed
+    __syncthreads();
+    uint32_t *stg = reinterpret_cast<uint32_t *>(wbuf + ((gs - 1) & 1) * SU + wave * WU);  // this wave's 16 KB
+    finish_rows<C, HAS_RES, HAS_LN>(yacc, stg, i, g, row0, row_end, residual, y, ln_out, gams, bets, ln_eps,
+                                    [&]() { load_rows(mb + gridDim.x < nblocks ? mb + gridDim.x : mb, ub); });
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // nothing may still be landing in LDS when the workgroup ends
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// project_rows_kernel: the layer's two input projections (PA.py:501-514 for the irregular mesh) on the same skeleton,
+// written as the packed operand tiles the slice kernels read: a wave owns one tile of 32 points (tile = b tpb + t),
+// keeps its rows as MFMA operands and runs two products over them, one after the other:
+//   x_mid^T = W_x . x^T + b_x    weights as A, rows as B: lanes <-> points, registers <-> channels; two packed halves
+//                                per head are B operands (columns = points, k = the head's channels in kperm order)
+//   fx_mid  = x . W_fx^T + b_fx  rows as A, weights as B: lanes <-> channels, registers <-> points; two packed halves
+//                                per head are A operands (rows = channels, k = points in kperm order)
+// Both leave as 1 KB stores of 16 bytes per lane: out[((tile H + head) 2 + half) 64 + lane].
+// blob: W_x then W_fx, each in the fragment order of linear_pack_kernel (natural k order).
+// ---------------------------------------------------------------------------------------------------------------
+template <int C>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void project_rows_kernel(
+    const u32x4 *__restrict__ blob, const float *__restrict__ bias_x, const float *__restrict__ bias_fx,
+    const uint16_t *__restrict__ x, u32x4 *__restrict__ xm_pack, u32x4 *__restrict__ fx_pack, int64_t N, int tpb,
+    int64_t ntiles, int64_t nblocks) {
+  constexpr int KS = C / 16, CT = C / 32, SU = 4096, WU = SU / 4;
+  constexpr int NSLOT = CT * KS / 64, KPS = 64 / CT;
+  extern __shared__ u32x4 smem[];
+  u32x4 *wbuf = smem;  // 2 * SU
+  float *bxs = reinterpret_cast<float *>(wbuf + 2 * SU);
+  float *bfs = bxs + C;
+  const int tid = threadIdx.x, lane = tid & 63, i = lane & 31, g = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: addresses derived from it stay scalar
+  for (int k = tid; k < C; k += 256) {
+    bxs[k] = bias_x ? bias_x[k] : 0.f;
+    bfs[k] = bias_fx ? bias_fx[k] : 0.f;
+  }
+  __syncthreads();
+  auto fetch_group = [&](int64_t gs, int c, int k) {
+    const u32x4 *src = blob + (int64_t)c * SU + wave * WU + k * 256;
+    const unsigned dst = (unsigned)(uintptr_t)(wbuf + (gs & 1) * SU + wave * WU + k * 256);
+    load_4k_to_lds(src, lane * 16, dst);
+  };
+  // lane (i, g) holds point i of the wave's tile, channels 16 ks + 8 g .. + 7; points past the batch's end repeat
+  // its last one (the slice kernels give them zero weight)
+  auto load_rows = [&](int64_t mb, u32x4(&ub)[KS]) {
+    int64_t gt = mb * 4 + wave;
+    if (gt >= ntiles) gt = ntiles - 1;
+    const int64_t bb = gt / tpb, t = gt - bb * tpb;
+    int64_t n = t * 32 + i;
+    if (n >= N) n = N - 1;
+    const uint16_t *src = x + (bb * N + n) * C + 8 * g;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) ub[ks] = *reinterpret_cast<const u32x4 *>(src + 16 * ks);
+  };
+  int64_t gs = 0;
+  if ((int64_t)blockIdx.x < nblocks) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) fetch_group(0, 0, k);
+  }
+  u32x4 ub[KS];
+  if ((int64_t)blockIdx.x < nblocks) load_rows(blockIdx.x, ub);
+  for (int64_t mb = blockIdx.x; mb < nblocks; mb += gridDim.x) {
+    const int64_t gt = mb * 4 + wave;
+    const bool live = gt < ntiles;
+    f32x16 yacc[CT];
+    static_for<2>([&](auto pass_) {
+      constexpr int pass = decltype(pass_)::value;
+#pragma unroll
+      for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) yacc[ct][r] = pass == 0 ? bxs[32 * ct + rowmap(r, g)] : bfs[32 * ct + i];
+      static_for<NSLOT>([&](auto c_) {
+        constexpr int c = decltype(c_)::value;
+        // slot gs has landed and the other buffer is free
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        const u32x4 *wb = wbuf + (gs & 1) * SU + lane;
+        constexpr int RING = 8, AHEAD = 6;
+        u32x4 fr[RING];
+        static_for<AHEAD>([&](auto q) { fr[decltype(q)::value] = wb[decltype(q)::value * 64]; });
+        static_for<64>([&](auto j_) {
+          constexpr int j = decltype(j_)::value, ct = j % CT, ks = c * KPS + j / CT;
+          if constexpr (j + AHEAD < 64) fr[(j + AHEAD) % RING] = wb[(j + AHEAD) * 64];
+          if constexpr (pass == 0) yacc[ct] = mma(fr[j % RING], ub[ks], yacc[ct]);
+          else yacc[ct] = mma(ub[ks], fr[j % RING], yacc[ct]);
+          if constexpr (j % 16 == 7) fetch_group(gs + 1, (pass * NSLOT + c + 1) % (2 * NSLOT), j / 16);
+          __builtin_amdgcn_sched_barrier(0);
+        });
+        ++gs;
+      });
+      // the rows of this workgroup's next block travel while the second product's tiles are stored
+      if constexpr (pass == 1) load_rows(mb + gridDim.x < nblocks ? mb + gridDim.x : mb, ub);
+      u32x4 *dst = (pass == 0 ? xm_pack : fx_pack) + (live ? gt : 0) * (CT * 2 * 64) + lane;
+      if (live) {
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) {
+          dst[(2 * ct + 0) * 64] = pack_half<0>(yacc[ct]);
+          dst[(2 * ct + 1) * 64] = pack_half<1>(yacc[ct]);
+        }
+      }
+    });
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // nothing may still be landing in LDS when the workgroup ends
 }
@@ -853,6 +1091,88 @@ static int launch_c(int64_t rows, int F, const void *blob, const float *b1, cons
   if (res) return launch<C, 2>(rows, F, blob, b1, b2, u, y, tail, num_cu, st);
   if (ln) return launch<C, 3>(rows, F, blob, b1, b2, u, y, tail, num_cu, st);
   return launch<C, 0>(rows, F, blob, b1, b2, u, y, nullptr, num_cu, st);
+}
+
+// ---- out_linear with the block's tail on the row-owning kernel --------------------------------------------------
+bool linear_supported(int dtype, int64_t rows, int64_t C) { return dtype == PA_BF16 && rows > 0 && C == 512; }
+
+int64_t linear_blob_bytes(int64_t C) { return C * C * 2; }
+
+template <int C, int TAIL, bool PACKED_IN>
+static int launch_linear(int64_t rows, const void *blob, const float *bias, const void *x, void *y,
+                         const pa_block_tail *tail, int64_t N, int tpb, int num_cu, hipStream_t st) {
+  const size_t lds = (size_t)2 * 4096 * 16 + (size_t)3 * C * 4;
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(rows::linear_rows_kernel<C, TAIL, PACKED_IN>),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  if (e != hipSuccess) return (int)e;
+  // PACKED_IN: `rows` counts tiles of 32 points, four to a block
+  const int64_t nblocks = PACKED_IN ? (rows + 3) / 4 : (rows + kRowsPerBlock - 1) / kRowsPerBlock;
+  const int64_t grid = nblocks < num_cu ? nblocks : num_cu;
+  hipLaunchKernelGGL((rows::linear_rows_kernel<C, TAIL, PACKED_IN>), dim3((unsigned)grid), dim3(256), lds, st,
+                     static_cast<const u32x4 *>(blob), bias, static_cast<const uint16_t *>(x),
+                     static_cast<uint16_t *>(y), tail ? static_cast<const uint16_t *>(tail->residual) : nullptr,
+                     tail ? tail->ln_gamma : nullptr, tail ? tail->ln_beta : nullptr, tail ? tail->ln_eps : 0.f,
+                     tail ? static_cast<uint16_t *>(tail->ln_out) : nullptr, rows, nblocks, N, tpb);
+  e = hipGetLastError();
+  return e == hipSuccess ? PA_OK : (int)e;
+}
+
+template <bool PACKED_IN>
+static int linear_any(int64_t rows, int64_t C, const void *w, const float *bias, const void *x, void *y,
+                      const pa_block_tail *tail, void *blob, int64_t N, int tpb, int num_cu, hipStream_t st) {
+  if (C != 512) return PA_ERR_UNSUPPORTED;
+  const int64_t total = C * C / 8;
+  hipLaunchKernelGGL(rows::linear_pack_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st,
+                     static_cast<const uint16_t *>(w), static_cast<u32x4 *>(blob), (int)C, PACKED_IN ? 1 : 0);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return (int)e;
+  const bool res = tail && tail->residual, ln = tail && tail->ln_out;
+  if (res && ln) return launch_linear<512, 1, PACKED_IN>(rows, blob, bias, x, y, tail, N, tpb, num_cu, st);
+  if (res) return launch_linear<512, 2, PACKED_IN>(rows, blob, bias, x, y, tail, N, tpb, num_cu, st);
+  if (ln) return launch_linear<512, 3, PACKED_IN>(rows, blob, bias, x, y, tail, N, tpb, num_cu, st);
+  return launch_linear<512, 0, PACKED_IN>(rows, blob, bias, x, y, nullptr, N, tpb, num_cu, st);
+}
+
+// y = W x + bias (+ tail) for (rows, C) row-major x; `blob` = linear_blob_bytes(C) bytes of scratch for the
+// fragment-ordered weights
+int linear(int64_t rows, int64_t C, const void *w, const float *bias, const void *x, void *y, const pa_block_tail *tail,
+           void *blob, int num_cu, hipStream_t st) {
+  return linear_any<false>(rows, C, w, bias, x, y, tail, blob, 0, 1, num_cu, st);
+}
+
+// the same with x as packed operand tiles [B tpb][C / 32][2][64 lanes] of 16 bytes (tile b tpb + t = points
+// 32 t .. 32 t + 31 of batch b, k order kperm within a head); y and the tail tensors stay (B, N, C) row-major
+int linear_packed(int64_t B, int64_t N, int64_t C, const void *w, const float *bias, const void *x_pack, void *y,
+                  const pa_block_tail *tail, void *blob, int num_cu, hipStream_t st) {
+  const int64_t tpb = (N + 31) / 32;
+  return linear_any<true>(B * tpb, C, w, bias, x_pack, y, tail, blob, N, (int)tpb, num_cu, st);
+}
+
+// the layer's two input projections as packed operand tiles (x_mid: B operands, fx_mid: A operands); `blob` =
+// 2 linear_blob_bytes(C) bytes of scratch
+int project_packed(int64_t B, int64_t N, int64_t C, const void *w_x, const float *b_x, const void *w_fx,
+                   const float *b_fx, const void *x, void *xm_pack, void *fx_pack, void *blob, int num_cu,
+                   hipStream_t st) {
+  if (C != 512) return PA_ERR_UNSUPPORTED;
+  const int64_t total = C * C / 8;
+  u32x4 *bl = static_cast<u32x4 *>(blob);
+  hipLaunchKernelGGL(rows::linear_pack_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st,
+                     static_cast<const uint16_t *>(w_x), bl, (int)C, 0);
+  hipLaunchKernelGGL(rows::linear_pack_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st,
+                     static_cast<const uint16_t *>(w_fx), bl + total, (int)C, 0);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return (int)e;
+  const size_t lds = (size_t)2 * 4096 * 16 + (size_t)2 * C * 4;
+  e = hipFuncSetAttribute(reinterpret_cast<const void *>(rows::project_rows_kernel<512>),
+                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  if (e != hipSuccess) return (int)e;
+  const int64_t tpb = (N + 31) / 32, ntiles = B * tpb, nblocks = (ntiles + 3) / 4;
+  const int64_t grid = nblocks < num_cu ? nblocks : num_cu;
+  hipLaunchKernelGGL((rows::project_rows_kernel<512>), dim3((unsigned)grid), dim3(256), lds, st, bl, b_x, b_fx,
+                     static_cast<const uint16_t *>(x), static_cast<u32x4 *>(xm_pack), static_cast<u32x4 *>(fx_pack), N,
+                     (int)tpb, ntiles, nblocks);
+  e = hipGetLastError();
+  return e == hipSuccess ? PA_OK : (int)e;
 }
 
 int forward(int64_t rows, int64_t C, int64_t F, const void *blob, const float *b1, const float *b2, const void *u,
