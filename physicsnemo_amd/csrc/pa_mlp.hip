@@ -906,34 +906,48 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 }
 
 // ---------------------------------------------------------------------------------------------------------------
-// project_rows_kernel: the layer's two input projections (PA.py:501-514 for the irregular mesh) on the same skeleton,
-// written as the packed operand tiles the slice kernels read: a wave owns one tile of 32 points (tile = b tpb + t),
-// keeps its rows as MFMA operands and runs two products over them, one after the other:
-//   x_mid^T = W_x . x^T + b_x    weights as A, rows as B: lanes <-> points, registers <-> channels; two packed halves
-//                                per head are B operands (columns = points, k = the head's channels in kperm order)
-//   fx_mid  = x . W_fx^T + b_fx  rows as A, weights as B: lanes <-> channels, registers <-> points; two packed halves
-//                                per head are A operands (rows = channels, k = points in kperm order)
-// Both leave as 1 KB stores of 16 bytes per lane: out[((tile H + head) 2 + half) 64 + lane].
-// blob: W_x then W_fx, each in the fragment order of linear_pack_kernel (natural k order).
+// project_rows_kernel: the layer's two input projections (PA.py:501-514 for the irregular mesh), written as the packed
+// operand tiles the slice kernels read.  Workgroup = 8 waves (two per SIMD), a block = 8 tiles of 32 points; a wave
+// owns one tile (tile = b tpb + t), keeps its rows as MFMA operands (C/4 registers) and runs two products over them:
+//   x_mid^T = W_x . x^T + b_x    weights as A, rows as B: lanes <-> points, registers <-> channels; the two packed
+//                                halves of a head are B operands (columns = points, k = the head's channels, kperm order)
+//   fx_mid  = x . W_fx^T + b_fx  rows as A, weights as B: lanes <-> channels, registers <-> points; the two packed
+//                                halves of a head are A operands (rows = channels, k = points, kperm order)
+// Output tiles are the outer loop: a slot of the weight stream (64 fragments, 64 KB) holds all C/16 k-steps of two
+// heads, interleaved so that the two accumulators alternate; when the slot is done the two heads leave as four 1 KB
+// stores per wave: out[((tile H + head) 2 + half) 64 + lane].  Only two accumulators are live, which is what lets two
+// waves share a SIMD, and the stores are spread evenly over the kernel.
+// blob: W_x then W_fx, each H/2 slots in that order (project_pack_kernel).
 // ---------------------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void project_pack_kernel(const uint16_t *__restrict__ w, u32x4 *__restrict__ blob, int C) {
+  const int64_t total = (int64_t)C * C / 8;
+  for (int64_t u = (int64_t)blockIdx.x * 256 + threadIdx.x; u < total; u += (int64_t)gridDim.x * 256) {
+    const int c = (int)(u >> 12), j = (int)(u & 4095) >> 6, lane = (int)(u & 63), i = lane & 31, g = lane >> 5;
+    const int ct = 2 * c + (j & 1), ks = j >> 1;
+    blob[u] = *reinterpret_cast<const u32x4 *>(w + (int64_t)(32 * ct + i) * C + 16 * ks + 8 * g);
+  }
+}
+
 template <int C>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void project_rows_kernel(
+__global__ __launch_bounds__(512) void project_rows_kernel(
     const u32x4 *__restrict__ blob, const float *__restrict__ bias_x, const float *__restrict__ bias_fx,
     const uint16_t *__restrict__ x, u32x4 *__restrict__ xm_pack, u32x4 *__restrict__ fx_pack, int64_t N, int tpb,
     int64_t ntiles, int64_t nblocks) {
-  constexpr int KS = C / 16, CT = C / 32, SU = 4096, WU = SU / 4;
-  constexpr int NSLOT = CT * KS / 64, KPS = 64 / CT;
+  constexpr int KS = C / 16, CT = C / 32, SU = 4096, WU = SU / 8;
+  constexpr int NSLOT = CT / 2;  // slots per product
+  static_assert(KS == 32, "a slot holds the k-steps of two heads");
   extern __shared__ u32x4 smem[];
   u32x4 *wbuf = smem;  // 2 * SU
   float *bxs = reinterpret_cast<float *>(wbuf + 2 * SU);
   float *bfs = bxs + C;
   const int tid = threadIdx.x, lane = tid & 63, i = lane & 31, g = lane >> 5;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: addresses derived from it stay scalar
-  for (int k = tid; k < C; k += 256) {
+  for (int k = tid; k < C; k += 512) {
     bxs[k] = bias_x ? bias_x[k] : 0.f;
     bfs[k] = bias_fx ? bias_fx[k] : 0.f;
   }
   __syncthreads();
+  // 4 KB group k (0, 1) of this wave's eighth of slot c (0 .. 2 NSLOT - 1 over both products) into buffer gs & 1
   auto fetch_group = [&](int64_t gs, int c, int k) {
     const u32x4 *src = blob + (int64_t)c * SU + wave * WU + k * 256;
     const unsigned dst = (unsigned)(uintptr_t)(wbuf + (gs & 1) * SU + wave * WU + k * 256);
@@ -942,7 +956,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   // lane (i, g) holds point i of the wave's tile, channels 16 ks + 8 g .. + 7; points past the batch's end repeat
   // its last one (the slice kernels give them zero weight)
   auto load_rows = [&](int64_t mb, u32x4(&ub)[KS]) {
-    int64_t gt = mb * 4 + wave;
+    int64_t gt = mb * 8 + wave;
     if (gt >= ntiles) gt = ntiles - 1;
     const int64_t bb = gt / tpb, t = gt - bb * tpb;
     int64_t n = t * 32 + i;
@@ -953,51 +967,56 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   };
   int64_t gs = 0;
   if ((int64_t)blockIdx.x < nblocks) {
-#pragma unroll
-    for (int k = 0; k < 4; ++k) fetch_group(0, 0, k);
+    fetch_group(0, 0, 0);
+    fetch_group(0, 0, 1);
   }
   u32x4 ub[KS];
-  if ((int64_t)blockIdx.x < nblocks) load_rows(blockIdx.x, ub);
   for (int64_t mb = blockIdx.x; mb < nblocks; mb += gridDim.x) {
-    const int64_t gt = mb * 4 + wave;
+    const int64_t gt = mb * 8 + wave;
     const bool live = gt < ntiles;
-    f32x16 yacc[CT];
-    static_for<2>([&](auto pass_) {
-      constexpr int pass = decltype(pass_)::value;
+    load_rows(mb, ub);
+    for (int c = 0; c < 2 * NSLOT; ++c, ++gs) {
+      const bool second = c >= NSLOT;          // the fx product
+      const int ct0 = 2 * (c - (second ? NSLOT : 0));  // heads ct0, ct0 + 1
+      // Slot gs has landed (every wave waits for its own share, then all meet) and the other buffer is free.  The
+      // share was requested before the four stores of the slot before: those may still be in flight.
+      if (c == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      else asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+      __syncthreads();
+      const u32x4 *wb = wbuf + (gs & 1) * SU + lane;
+      f32x16 acc[2];
 #pragma unroll
-      for (int ct = 0; ct < CT; ++ct)
+      for (int q = 0; q < 2; ++q)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) yacc[ct][r] = pass == 0 ? bxs[32 * ct + rowmap(r, g)] : bfs[32 * ct + i];
-      static_for<NSLOT>([&](auto c_) {
-        constexpr int c = decltype(c_)::value;
-        // slot gs has landed and the other buffer is free
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();
-        const u32x4 *wb = wbuf + (gs & 1) * SU + lane;
-        constexpr int RING = 8, AHEAD = 6;
-        u32x4 fr[RING];
-        static_for<AHEAD>([&](auto q) { fr[decltype(q)::value] = wb[decltype(q)::value * 64]; });
+        for (int r = 0; r < 16; ++r) acc[q][r] = second ? bfs[32 * (ct0 + q) + i] : bxs[32 * (ct0 + q) + rowmap(r, g)];
+      constexpr int RING = 6, AHEAD = 4;
+      u32x4 fr[RING];
+      static_for<AHEAD>([&](auto q) { fr[decltype(q)::value] = wb[decltype(q)::value * 64]; });
+      const int c_next = c + 1 < 2 * NSLOT ? c + 1 : 0;
+      if (!second) {
         static_for<64>([&](auto j_) {
-          constexpr int j = decltype(j_)::value, ct = j % CT, ks = c * KPS + j / CT;
+          constexpr int j = decltype(j_)::value;
           if constexpr (j + AHEAD < 64) fr[(j + AHEAD) % RING] = wb[(j + AHEAD) * 64];
-          if constexpr (pass == 0) yacc[ct] = mma(fr[j % RING], ub[ks], yacc[ct]);
-          else yacc[ct] = mma(ub[ks], fr[j % RING], yacc[ct]);
-          if constexpr (j % 16 == 7) fetch_group(gs + 1, (pass * NSLOT + c + 1) % (2 * NSLOT), j / 16);
+          acc[j & 1] = mma(fr[j % RING], ub[j >> 1], acc[j & 1]);
+          if constexpr (j == 1 || j == 9) fetch_group(gs + 1, c_next, j / 8);
           __builtin_amdgcn_sched_barrier(0);
         });
-        ++gs;
-      });
-      // the rows of this workgroup's next block travel while the second product's tiles are stored
-      if constexpr (pass == 1) load_rows(mb + gridDim.x < nblocks ? mb + gridDim.x : mb, ub);
-      u32x4 *dst = (pass == 0 ? xm_pack : fx_pack) + (live ? gt : 0) * (CT * 2 * 64) + lane;
-      if (live) {
-#pragma unroll
-        for (int ct = 0; ct < CT; ++ct) {
-          dst[(2 * ct + 0) * 64] = pack_half<0>(yacc[ct]);
-          dst[(2 * ct + 1) * 64] = pack_half<1>(yacc[ct]);
-        }
+      } else {
+        static_for<64>([&](auto j_) {
+          constexpr int j = decltype(j_)::value;
+          if constexpr (j + AHEAD < 64) fr[(j + AHEAD) % RING] = wb[(j + AHEAD) * 64];
+          acc[j & 1] = mma(ub[j >> 1], fr[j % RING], acc[j & 1]);
+          if constexpr (j == 1 || j == 9) fetch_group(gs + 1, c_next, j / 8);
+          __builtin_amdgcn_sched_barrier(0);
+        });
       }
-    });
+      // exactly four stores per slot and wave (see the wait above): tiles past the end rewrite the last one's
+      u32x4 *dst = (second ? fx_pack : xm_pack) + ((live ? gt : ntiles - 1) * CT + ct0) * (2 * 64) + lane;
+      dst[0] = pack_half<0>(acc[0]);
+      dst[64] = pack_half<1>(acc[0]);
+      dst[128] = pack_half<0>(acc[1]);
+      dst[192] = pack_half<1>(acc[1]);
+    }
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // nothing may still be landing in LDS when the workgroup ends
 }
@@ -1156,19 +1175,19 @@ int project_packed(int64_t B, int64_t N, int64_t C, const void *w_x, const float
   if (C != 512) return PA_ERR_UNSUPPORTED;
   const int64_t total = C * C / 8;
   u32x4 *bl = static_cast<u32x4 *>(blob);
-  hipLaunchKernelGGL(rows::linear_pack_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st,
-                     static_cast<const uint16_t *>(w_x), bl, (int)C, 0);
-  hipLaunchKernelGGL(rows::linear_pack_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st,
-                     static_cast<const uint16_t *>(w_fx), bl + total, (int)C, 0);
+  hipLaunchKernelGGL(rows::project_pack_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st,
+                     static_cast<const uint16_t *>(w_x), bl, (int)C);
+  hipLaunchKernelGGL(rows::project_pack_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st,
+                     static_cast<const uint16_t *>(w_fx), bl + total, (int)C);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return (int)e;
   const size_t lds = (size_t)2 * 4096 * 16 + (size_t)2 * C * 4;
   e = hipFuncSetAttribute(reinterpret_cast<const void *>(rows::project_rows_kernel<512>),
                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (e != hipSuccess) return (int)e;
-  const int64_t tpb = (N + 31) / 32, ntiles = B * tpb, nblocks = (ntiles + 3) / 4;
+  const int64_t tpb = (N + 31) / 32, ntiles = B * tpb, nblocks = (ntiles + 7) / 8;
   const int64_t grid = nblocks < num_cu ? nblocks : num_cu;
-  hipLaunchKernelGGL((rows::project_rows_kernel<512>), dim3((unsigned)grid), dim3(256), lds, st, bl, b_x, b_fx,
+  hipLaunchKernelGGL((rows::project_rows_kernel<512>), dim3((unsigned)grid), dim3(512), lds, st, bl, b_x, b_fx,
                      static_cast<const uint16_t *>(x), static_cast<u32x4 *>(xm_pack), static_cast<u32x4 *>(fx_pack), N,
                      (int)tpb, ntiles, nblocks);
   e = hipGetLastError();
