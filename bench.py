@@ -463,11 +463,12 @@ def write_traffic(fetch_dir, write_dir, B, N, C, S):
                 for r in csv.DictReader(f):
                     if r["Counter_Name"] == counter:
                         acc.setdefault(r["Kernel_Name"], []).append(float(r["Counter_Value"]))
-        return {k: sum(v[-10:]) / len(v[-10:]) for k, v in acc.items()}
+        # the runtime's copy kernel also serves small transfers: the 1 GiB calibration copy is its largest dispatch
+        return {k: (max(v) if "copyBuffer" in k else sum(v[-10:]) / len(v[-10:])) for k, v in acc.items()}
 
     fetch, write = per_kernel(fetch_dir, "FETCH_SIZE"), per_kernel(write_dir, "WRITE_SIZE")
     copy = [k for k in fetch if "copyBuffer" in k]
-    if not copy:
+    if not copy or fetch[copy[0]] < (1 << 18) or write.get(copy[0], 0) < (1 << 18):
         raise SystemExit("no calibration copy in the counter files: run the profiled command with --calibrate-copy")
     f_scale = (1 << 20) / fetch[copy[0]]   # KiB the copy really read / KiB the counter reports
     w_scale = (1 << 20) / write[copy[0]]
