@@ -440,6 +440,14 @@ int64_t pa_mlp_workspace_bytes(int dtype, int64_t rows, int64_t C, int64_t F);
 int pa_mlp_forward(int dtype, int64_t rows, int64_t C, int64_t F, const pa_mlp_params *p, const void *u, void *y,
                    const pa_block_tail *tail, void *workspace, int64_t workspace_bytes, void *stream);
 
+/* The same in two steps, for callers that keep the repacked weights between calls (one pa_mlp_pack per parameter set):
+ * pa_mlp_pack writes pa_mlp_workspace_bytes() bytes into `packed`; pa_mlp_forward_packed is pa_mlp_forward with
+ * p->w1 / p->w2 replaced by that buffer (p->b1, p->b2 are still read).  No reference counterpart (the reference's
+ * Linear layers keep their weights in the layout the GEMM library wants). */
+int pa_mlp_pack(int dtype, int64_t C, int64_t F, const pa_mlp_params *p, void *packed, int64_t packed_bytes, void *stream);
+int pa_mlp_forward_packed(int dtype, int64_t rows, int64_t C, int64_t F, const void *packed, const float *b1,
+                          const float *b2, const void *u, void *y, const pa_block_tail *tail, void *stream);
+
 /* The block tail on its own (TR.py:300-303, :305-307): y (rows, C) <- y + tail->residual (if given), then
  * tail->ln_out = LayerNorm(y) (if given).  For callers whose producer of y is not one of the fused kernels. */
 int pa_residual_layernorm(int dtype, int64_t rows, int64_t C, void *y, const pa_block_tail *tail, void *stream);

@@ -805,6 +805,28 @@ int64_t pa_mlp_workspace_bytes(int dtype, int64_t rows, int64_t C, int64_t F) {
   return round_up(pa::mlp::blob_bytes(C, F), 256);
 }
 
+int pa_mlp_pack(int dtype, int64_t C, int64_t F, const pa_mlp_params *p, void *packed, int64_t packed_bytes,
+                void *stream) {
+  if (C <= 0 || F <= 0) return PA_ERR_DIMS;
+  if (!pa::mlp::supported(dtype, 1, C, F)) return PA_ERR_UNSUPPORTED;
+  if (!p || !p->w1 || !p->w2 || !packed) return PA_ERR_NULL;
+  if (!aligned16(p->w1) || !aligned16(p->w2) || !aligned16(packed)) return PA_ERR_ALIGN;
+  if (packed_bytes < pa::mlp::blob_bytes(C, F)) return PA_ERR_WORKSPACE;
+  return pa::mlp::pack(C, F, p->w1, p->w2, packed, static_cast<hipStream_t>(stream));
+}
+
+int pa_mlp_forward_packed(int dtype, int64_t rows, int64_t C, int64_t F, const void *packed, const float *b1,
+                          const float *b2, const void *u, void *y, const pa_block_tail *tail, void *stream) {
+  if (rows <= 0 || C <= 0 || F <= 0) return PA_ERR_DIMS;
+  if (!pa::mlp::supported(dtype, rows, C, F)) return PA_ERR_UNSUPPORTED;
+  if (!packed || !b1 || !b2 || !u || !y) return PA_ERR_NULL;
+  if (!aligned16(packed) || !aligned16(u) || !aligned16(y)) return PA_ERR_ALIGN;
+  int rc = check_tail(tail);
+  if (rc) return rc;
+  return pa::mlp::forward(rows, C, F, packed, b1, b2, u, y, tail_active(tail) ? tail : nullptr, compute_units(),
+                          static_cast<hipStream_t>(stream));
+}
+
 int pa_mlp_forward(int dtype, int64_t rows, int64_t C, int64_t F, const pa_mlp_params *p, const void *u, void *y,
                    const pa_block_tail *tail, void *workspace, int64_t workspace_bytes, void *stream) {
   if (rows <= 0 || C <= 0 || F <= 0) return PA_ERR_DIMS;

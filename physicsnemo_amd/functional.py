@@ -301,6 +301,38 @@ def mlp_forward(u, w1, b1, w2, b2, residual=None, ln_weight=None, ln_bias=None, 
     return y if ln_out is None else (y, ln_out)
 
 
+def mlp_pack(w1, w2):
+    """The two weights of the MLP in the fused kernel's operand order: one call per parameter set; the result is the
+    `packed` argument of mlp_forward_packed.  w1 (F, C), w2 (C, F) bfloat16."""
+    _need_cuda(w1, w2)
+    lib = _lib.load()
+    C, F = w1.shape[1], w1.shape[0]
+    code = _lib.dtype_code(w1.dtype)
+    nbytes = lib.pa_mlp_workspace_bytes(code, 1, C, F)
+    if nbytes < 0:
+        _lib.check(int(nbytes), "pa_mlp_workspace_bytes")
+    packed = torch.empty(int(nbytes), dtype=torch.uint8, device=w1.device)
+    params = _lib.PaMlpParams(_lib.ptr(w1), None, _lib.ptr(w2), None)
+    _lib.check(lib.pa_mlp_pack(code, C, F, byref(params), packed.data_ptr(), int(nbytes),
+                               _lib.current_stream_ptr(w1.device)), "pa_mlp_pack")
+    return packed
+
+
+def mlp_forward_packed(u, packed, b1, b2, residual=None, ln_weight=None, ln_bias=None, ln_eps=1e-5):
+    """mlp_forward with the weights already in operand order (mlp_pack); b1 (F), b2 (C) float32."""
+    _need_cuda(u, packed, b1, b2, residual, ln_weight, ln_bias)
+    lib = _lib.load()
+    C, F = b2.numel(), b1.numel()
+    rows = u.numel() // C
+    y = torch.empty_like(u)
+    ln_out = torch.empty_like(u) if ln_weight is not None else None
+    tail = _c_tail(residual, ln_weight, ln_bias, ln_eps, ln_out)
+    _lib.check(lib.pa_mlp_forward_packed(_lib.dtype_code(u.dtype), rows, C, F, packed.data_ptr(), b1.data_ptr(),
+                                         b2.data_ptr(), u.data_ptr(), y.data_ptr(), byref(tail),
+                                         _lib.current_stream_ptr(u.device)), "pa_mlp_forward_packed")
+    return y if ln_out is None else (y, ln_out)
+
+
 class MfmaStages:
     """The bf16 MFMA kernels one by one (pa_mfma_* entry points) with their opaque buffers held as torch tensors.
 

@@ -280,6 +280,7 @@ class GALEBlock(nn.Module):
     # the block MLP (reference mlp_layers.py:101-173) and its kernels are the Transolver block's
     fp8_weights = False  # the shared MLP helpers read it; GALE blocks are served in bf16 / float32 only
     _mlp_kernel_params = TransolverBlock._mlp_kernel_params
+    _mlp_kernel_packed = TransolverBlock._mlp_kernel_packed
     _mlp_kernel_serves = TransolverBlock._mlp_kernel_serves
     _mlp_with_grad = TransolverBlock._mlp_with_grad
     _mlp_residual = TransolverBlock._mlp_residual
@@ -288,8 +289,8 @@ class GALEBlock(nn.Module):
         fx1 = attn + fx
         normed = PA.layer_norm(fx1, self.ln_mlp1[0])
         if not needs_grad and self._mlp_kernel_serves(normed):
-            w1, b1, w2, b2 = self._mlp_kernel_params(normed.device)
-            return PF.mlp_forward(normed, w1, b1, w2, b2, residual=fx1.to(normed.dtype).contiguous())
+            packed, b1, b2 = self._mlp_kernel_packed(normed.device)
+            return PF.mlp_forward_packed(normed, packed, b1, b2, residual=fx1.to(normed.dtype).contiguous())
         return self._mlp_with_grad(normed) + fx1
 
     def forward_chain(self, fx: tuple, normed_in, global_context: torch.Tensor | None, next_ln: nn.LayerNorm | None):

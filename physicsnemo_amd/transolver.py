@@ -135,6 +135,13 @@ class TransolverBlock(nn.Module):
             self._mlp_cache = {"stamp": stamp, "params": params}
         return self._mlp_cache["params"]
 
+    def _mlp_kernel_packed(self, device):
+        """(packed weights, b1, b2) for pa_mlp_forward_packed: the weights repacked once per parameter set."""
+        w1, b1, w2, b2 = self._mlp_kernel_params(device)
+        if "packed" not in self._mlp_cache:
+            self._mlp_cache["packed"] = PF.mlp_pack(w1, w2)
+        return self._mlp_cache["packed"], b1, b2
+
     def _mlp_kernel_serves(self, normed: torch.Tensor) -> bool:
         mlp = self.ln_mlp1[1]
         if not (normed.is_cuda and normed.dtype == torch.bfloat16 and isinstance(mlp.layers[1], nn.GELU)
@@ -174,12 +181,12 @@ class TransolverBlock(nn.Module):
         """fx1 + Mlp(normed) and, with `next_ln`, its LayerNorm (reference :303, and :300 of the next block): the fused
         block-MLP kernel where it serves the shape, else the tensor-op MLP followed by one add (+ LayerNorm) kernel."""
         if self._mlp_kernel_serves(normed):
-            w1, b1, w2, b2 = self._mlp_kernel_params(normed.device)
+            packed, b1, b2 = self._mlp_kernel_packed(normed.device)
             if next_ln is None:
-                return PF.mlp_forward(normed, w1, b1, w2, b2, residual=fx1), None
-            return PF.mlp_forward(normed, w1, b1, w2, b2, residual=fx1,
-                                  ln_weight=next_ln.weight.detach().float().contiguous(),
-                                  ln_bias=next_ln.bias.detach().float().contiguous(), ln_eps=next_ln.eps)
+                return PF.mlp_forward_packed(normed, packed, b1, b2, residual=fx1), None
+            return PF.mlp_forward_packed(normed, packed, b1, b2, residual=fx1,
+                                         ln_weight=next_ln.weight.detach().float().contiguous(),
+                                         ln_bias=next_ln.bias.detach().float().contiguous(), ln_eps=next_ln.eps)
         # MLP shapes the fused kernel does not serve: tensor-op MLP, then residual add (+ the next LayerNorm) in one pass
         if self.fp8_weights and normed.is_cuda and normed.dtype == torch.bfloat16:
             w1, b1, w2, b2 = self._mlp_kernel_params(normed.device)

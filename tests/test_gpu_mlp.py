@@ -77,6 +77,20 @@ def test_mlp_gelu_tails_and_determinism():
     assert torch.equal(y_prefix, y[:, :777])
 
 
+def test_mlp_packed_weights_give_the_same_bits():
+    announce("mlp, weights packed once")
+    for C, Fh in ((256, 1024), (512, 2048), (128, 256)):
+        ref, u, res, gamma, beta, args = _case((1, 1500), C, Fh, seed=5)
+        dev = args["u"].device
+        with torch.no_grad():
+            y, ln = PF.mlp_forward(**args, residual=res.to(dev), ln_weight=gamma.to(dev), ln_bias=beta.to(dev))
+            packed = PF.mlp_pack(args["w1"], args["w2"])
+            for _ in range(2):  # the packed buffer is read only
+                y2, ln2 = PF.mlp_forward_packed(args["u"], packed, args["b1"], args["b2"], residual=res.to(dev),
+                                                ln_weight=gamma.to(dev), ln_bias=beta.to(dev))
+                assert torch.equal(y, y2) and torch.equal(ln, ln2)
+
+
 def test_mlp_rejects_unsupported():
     assert not PF.mlp_supported(torch.float32, 100, 256, 1024)
     assert not PF.mlp_supported(torch.bfloat16, 100, 384, 1536)
