@@ -653,6 +653,14 @@ def main():
         out["slice_sweep"] = sweep
     if not args.no_models:
         out["block_mlp"] = time_block_mlp(1 << 20, 256, 1024)
+        out["block_mlp_c512"] = time_block_mlp(1 << 20, 512, 2048)
+        # the cfg5 layer shape at the layer workload's point count (staged MFMA kernels on packed tiles)
+        m5 = measure_layer(1, N, 512, 128, 5, 2, 5)
+        out["layer_c512_s128"] = dict({"points": N, "hidden": 512, "heads": 16, "slice_num": 128,
+                                       "ms_per_step": round(m5["ms_per_step"], 4),
+                                       "mpoints_per_s": round(N / (m5["ms_per_step"] * 1e-3) / 1e6, 2),
+                                       "kernel_path": {0: "general", 1: "mfma", 2: "mfma-staged"}[m5["path"]]},
+                                      **layer_fracs(N, 512, 128, m5["ms_per_step"]))
         out["training_step"] = time_training_step(N, C, S)
         out["variants"] = time_variants(N, C, S)
         out["full_model"] = [
