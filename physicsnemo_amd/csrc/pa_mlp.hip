@@ -23,6 +23,7 @@
 #include "pa_host.h"
 #include "pa_mfma_ops.h"
 
+#include <cstdlib>
 #include <type_traits>
 #include <utility>
 
@@ -493,17 +494,17 @@ __device__ __forceinline__ void mma_in_vgprs(u32x4 a, u32x4 b, f32x16 &acc) {
 }
 
 // Epilogue of the row-owning kernels: a wave's y^T (channel 32 ct + rowmap(r, g) of row i, C channels x 32 rows) to
-// row-major bf16 rows, + residual, LayerNorm, full-row stores.  The rows pass through `stg`, the wave's own 16 KB of
-// LDS, RPR = 8192 / C rows at a time; after_staging() is called once the last round is staged (the accumulators are
-// free from then on).  gams / bets: LayerNorm weight and bias in LDS.
-template <int C, bool HAS_RES, bool HAS_LN, class AfterStaging>
+// row-major bf16 rows, + residual, LayerNorm, full-row stores.  The rows pass through `stg`, the wave's own STG bytes
+// of LDS, RPR = STG / (2 C) rows at a time; after_staging() is called once the last round is staged (the accumulators
+// are free from then on).  gams / bets: LayerNorm weight and bias in LDS.
+template <int C, bool HAS_RES, bool HAS_LN, int STG = 16384, class AfterStaging>
 __device__ __forceinline__ void finish_rows(const f32x16 (&yacc)[C / 32], uint32_t *stg, int i, int g, int64_t row0,
                                             int64_t M, const uint16_t *__restrict__ residual, uint16_t *__restrict__ y,
                                             uint16_t *__restrict__ ln_out, const float *gams, const float *bets,
                                             float ln_eps, AfterStaging &&after_staging) {
   constexpr int CT = C / 32;
   constexpr int G4 = C / 4;             // 8-byte granules (4 channels) per staged row
-  constexpr int RPR = 16384 / (2 * C);  // rows staged per round
+  constexpr int RPR = STG / (2 * C);  // rows staged per round
   constexpr int NROUND = 32 / RPR;
   // lane indices taken afresh, so that nothing derived from them for the epilogue is kept across the slot loop
   int il = i, gl = g;
@@ -780,6 +781,164 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 }
 
 // ---------------------------------------------------------------------------------------------------------------
+// mlp_rows2_kernel: the row-owning MLP for C = 256 with two waves per SIMD.  Workgroup = 8 waves, a block = 256 rows, a
+// wave owns 32 rows: inputs as B operands (64 registers), y^T for all 256 channels (128 registers), everything else
+// small enough for 256 registers per wave, so that the second wave of a SIMD covers the first one's vector work and
+// LDS waits.  Weights stream in slots of 32 hidden units (32 KB: 16 W1 fragments of chunk c, then 16 W2 fragments of
+// chunk c-1 ordered k-half major), two buffers, one barrier per slot; per slot a wave runs
+//   phase 1   h(c)^T = W1[chunk c] . u^T + b1                       16 MFMAs on one accumulator
+//   phase 2   y^T += W2[:, chunk c-1] . g(c-1)^T                    16 MFMAs (k half 0 for all channel tiles, then 1)
+//             with g(c) = gelu(h(c)) evaluated behind them, one value per MFMA, straight from the accumulator of
+//             phase 1; the first B operand of g(c) replaces that of g(c-1) once its last reader is issued.
+// The epilogue stages through 8 KB per wave of a separate 64 KB region.
+// ---------------------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void pack2_kernel(const uint16_t *__restrict__ w1, const uint16_t *__restrict__ w2,
+                                                    u32x4 *__restrict__ blob, int C, int F) {
+  const int KS = C / 16, CT = C / 32, NCH = F / 32, SU = (KS + 2 * CT) * 64;
+  const int64_t total = (int64_t)(NCH + 1) * SU;
+  for (int64_t u = (int64_t)blockIdx.x * 256 + threadIdx.x; u < total; u += (int64_t)gridDim.x * 256) {
+    const int c = (int)(u / SU), r = (int)(u - (int64_t)c * SU), frag = r >> 6, lane = r & 63, i = lane & 31, g = lane >> 5;
+    uint16_t e[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) e[j] = 0;
+    if (frag < KS) {
+      if (c < NCH) {
+        const uint16_t *src = w1 + (int64_t)(32 * c + i) * C + 16 * frag + 8 * g;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) e[j] = src[j];
+      }
+    } else if (c > 0) {
+      const int t = frag - KS, kk = t / CT, ct = t % CT;
+      const uint16_t *src = w2 + (int64_t)(32 * ct + i) * F + 32 * (c - 1);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) e[j] = src[kperm(kk, g, j)];
+    }
+    u32x4 v;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) v[j] = (uint32_t)e[2 * j] | ((uint32_t)e[2 * j + 1] << 16);
+    blob[u] = v;
+  }
+}
+
+template <int C, int TAIL>
+__global__ __launch_bounds__(512) void mlp_rows2_kernel(
+    const u32x4 *__restrict__ blob, const float *__restrict__ b1, const float *__restrict__ b2,
+    const uint16_t *__restrict__ u, uint16_t *__restrict__ y, const uint16_t *__restrict__ residual,
+    const float *__restrict__ ln_gamma, const float *__restrict__ ln_beta, float ln_eps, uint16_t *__restrict__ ln_out,
+    int64_t M, int F, int64_t nblocks) {
+  constexpr bool HAS_RES = TAIL == 1 || TAIL == 2, HAS_LN = TAIL == 1 || TAIL == 3;
+  constexpr int KS = C / 16, CT = C / 32, NF = KS + 2 * CT, SU = NF * 64;
+  constexpr int WU = SU / 8;       // units of a slot fetched by each wave
+  static_assert(WU == 256, "one group of four loads per wave and slot");
+  constexpr int STG = 8192;        // bytes of epilogue staging per wave
+  constexpr int kRows = 256;       // rows per block
+  extern __shared__ u32x4 smem[];
+  u32x4 *wbuf = smem;                                             // 2 * SU
+  uint32_t *stage = reinterpret_cast<uint32_t *>(wbuf + 2 * SU);  // 8 waves x STG bytes
+  float *b1s = reinterpret_cast<float *>(stage + 8 * STG / 4);
+  float *b2s = b1s + F;
+  float *gams = b2s + C, *bets = gams + C;
+  const int tid = threadIdx.x, lane = tid & 63, i = lane & 31, g = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: addresses derived from it stay scalar
+  const int NCH = F / 32;
+  for (int k = tid; k < F; k += 512) b1s[k] = b1[k];
+  for (int k = tid; k < C; k += 512) {
+    b2s[k] = b2[k];
+    gams[k] = HAS_LN ? ln_gamma[k] : 1.f;
+    bets[k] = HAS_LN ? ln_beta[k] : 0.f;
+  }
+  __syncthreads();
+  auto fetch = [&](int64_t gs, int c) {  // this wave's 4 KB of slot c into buffer gs & 1
+    const u32x4 *src = blob + (int64_t)c * SU + wave * WU;
+    const unsigned dst = (unsigned)(uintptr_t)(wbuf + (gs & 1) * SU + wave * WU);
+    load_4k_to_lds(src, lane * 16, dst);
+  };
+  auto load_rows = [&](int64_t mb, u32x4(&ub)[KS]) {
+    int64_t r = mb * kRows + wave * 32 + i;
+    if (r >= M) r = M - 1;
+    const uint16_t *src = u + r * C + 8 * g;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) ub[ks] = *reinterpret_cast<const u32x4 *>(src + 16 * ks);
+  };
+  int64_t gs = 0;
+  if ((int64_t)blockIdx.x < nblocks) fetch(0, 0);
+  u32x4 ub[KS];
+  if ((int64_t)blockIdx.x < nblocks) load_rows(blockIdx.x, ub);
+  for (int64_t mb = blockIdx.x; mb < nblocks; mb += gridDim.x) {
+    const int64_t row0 = mb * kRows + wave * 32;
+    f32x16 yacc[CT];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) yacc[ct][r] = b2s[32 * ct + rowmap(r, g)];
+    // gelu(h) of the chunk before as the two B operands of phase 2; nothing of the block before may reach this one.
+    // The 16 activations of a chunk are spread over the 32 MFMAs that follow its first product, one per two MFMAs:
+    // the first eight (k half 0) behind phase 2 of the same slot, straight from the accumulator, the other eight
+    // (copied to hrest at the end of the slot) behind phase 1 of the next one.
+    u32x4 gop[2] = {u32x4{0, 0, 0, 0}, u32x4{0, 0, 0, 0}}, gnew = u32x4{0, 0, 0, 0};
+    float hrest[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) hrest[j] = 0.f;
+    float ex = 0.f, ee = 0.f, feven = 0.f;  // evaluation in flight: argument and exp2 term; even result of a pair
+    auto begin = [&](float x) {
+      ex = x;
+      const float x2 = fminf(x * x, 81.f);
+      float q = fmaf(-3.51902394e-04f * -2.f * kLog2e, x2, 3.70080200e-02f * -2.f * kLog2e);
+      q = fmaf(q, x2, 7.97505275e-01f * -2.f * kLog2e);
+      ee = __builtin_amdgcn_exp2f(x * q);
+    };
+    auto finish = [&](auto j_) {  // result j (0 .. 7) of the operand being formed
+      constexpr int j = decltype(j_)::value;
+      const float v = ex * __builtin_amdgcn_rcpf(1.f + ee);
+      if constexpr (j % 2 == 0) feven = v;
+      else gnew[j / 2] = pack2(feven, v);
+    };
+    for (int c = 0; c <= NCH; ++c, ++gs) {
+      // slot gs has landed (every wave waits for its own share, then all meet) and the other buffer is free.  The
+      // first slot of a later block was waited for before the epilogue of the block before it.
+      if (c > 0 || gs == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      __syncthreads();
+      const u32x4 *wb = wbuf + (gs & 1) * SU + lane;
+      f32x16 hacc;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) hacc[r] = b1s[(c < NCH ? 32 * c : 0) + rowmap(r, g)];
+      constexpr int RING = 3, AHEAD = 2;
+      u32x4 fr[RING];
+      static_for<AHEAD>([&](auto q) { fr[decltype(q)::value] = wb[decltype(q)::value * 64]; });
+      static_for<KS>([&](auto S_) {
+        constexpr int S = decltype(S_)::value;
+        if constexpr (S + AHEAD < NF) fr[(S + AHEAD) % RING] = wb[(S + AHEAD) * 64];
+        hacc = mma(fr[S % RING], ub[S], hacc);
+        __builtin_amdgcn_sched_barrier(0);
+        // second half of the activations of the chunk before: value S / 2 starts behind even steps, ends behind odd ones
+        if constexpr (S % 2 == 0) begin(hrest[S / 2]);
+        else finish(std::integral_constant<int, S / 2>{});
+        if constexpr (S == 1) fetch(gs + 1, c < NCH ? c + 1 : 0);  // the other buffer was last read in the slot before
+        __builtin_amdgcn_sched_barrier(0);
+      });
+      static_assert(KS == 16 && 2 * CT == 16, "eight activations per phase");
+      gop[1] = gnew;  // k half 1 of the chunk before: its last reader was the last step of the slot before
+      static_for<2 * CT>([&](auto t_) {
+        constexpr int t = decltype(t_)::value, S = KS + t, kk = t / CT, ct = t % CT;
+        if constexpr (S + AHEAD < NF) fr[(S + AHEAD) % RING] = wb[(S + AHEAD) * 64];
+        yacc[ct] = mma(fr[S % RING], gop[kk], yacc[ct]);
+        __builtin_amdgcn_sched_barrier(0);
+        if constexpr (t % 2 == 0) begin(hacc[t / 2]);
+        else finish(std::integral_constant<int, t / 2>{});
+        __builtin_amdgcn_sched_barrier(0);
+      });
+      gop[0] = gnew;  // k half 0 of this chunk; that of the chunk before was last read by step CT - 1
+#pragma unroll
+      for (int j = 0; j < 8; ++j) hrest[j] = hacc[8 + j];
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's share of the next block's first slot has landed
+    finish_rows<C, HAS_RES, HAS_LN, STG>(yacc, stage + wave * (STG / 4), i, g, row0, M, residual, y, ln_out, gams, bets,
+                                         ln_eps, [&]() { load_rows(mb + gridDim.x < nblocks ? mb + gridDim.x : mb, ub); });
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // nothing may still be landing in LDS when the workgroup ends
+}
+
+// ---------------------------------------------------------------------------------------------------------------
 // linear_rows_kernel: y = W x + b [+ residual] [-> LayerNorm(y)] for bf16 rows with C inputs and C outputs (the
 // layer's out_linear with the block's residual and the following LayerNorm, transolver.py:296-300), on the skeleton
 // of mlp_rows_kernel: a wave owns 32 rows (inputs as B operands, all C outputs of y^T in accumulation registers), W
@@ -1024,8 +1183,9 @@ __global__ __launch_bounds__(512) void project_rows_kernel(
 }  // namespace rows
 
 // ---------------------------------------------------------------------------------------------------------------
-// C = 512 runs the row-owning kernel; C in {128, 256} the paired one
+// C = 512 runs the row-owning kernel with one wave per SIMD, C = 256 the one with two, C = 128 the paired kernel
 static bool use_rows_kernel(int64_t C) { return C == 512; }
+static bool use_rows2_kernel(int64_t C) { return C == 256 && !getenv("PA_MLP_PAIRED"); }
 
 bool supported(int dtype, int64_t rows, int64_t C, int64_t F) {
   if (dtype != PA_BF16 || rows <= 0 || F < 64 || F % 64 != 0 || F > 8192) return false;
@@ -1035,16 +1195,22 @@ bool supported(int dtype, int64_t rows, int64_t C, int64_t F) {
 
 int64_t blob_bytes(int64_t C, int64_t F) {
   if (use_rows_kernel(C)) return (F / (16384 / C) + 2) * (int64_t)4096 * 16;
+  if (use_rows2_kernel(C)) return (F / 32 + 1) * (int64_t)(C / 16 + 2 * (C / 32)) * 64 * 16;
   return (F / 64 + 1) * (int64_t)slot_units((int)C) * 16;
 }
 
 static size_t lds_bytes(int C, int F) { return (size_t)(2 * slot_units(C) + 4 * 4 * 64) * 16 + (size_t)(F + C) * 4; }
 
 int pack(int64_t C, int64_t F, const void *w1, const void *w2, void *blob, hipStream_t st) {
-  const bool by_rows = use_rows_kernel(C);
-  const int64_t total = by_rows ? (F / (16384 / C) + 2) * (int64_t)4096 : (F / 64 + 1) * (int64_t)slot_units((int)C);
+  const bool by_rows = use_rows_kernel(C), by_rows2 = use_rows2_kernel(C);
+  const int64_t total = by_rows    ? (F / (16384 / C) + 2) * (int64_t)4096
+                        : by_rows2 ? (F / 32 + 1) * (int64_t)(C / 16 + 2 * (C / 32)) * 64
+                                   : (F / 64 + 1) * (int64_t)slot_units((int)C);
   const int grid = (int)((total + 255) / 256 < 1024 ? (total + 255) / 256 : 1024);
-  if (by_rows)
+  if (by_rows2)
+    hipLaunchKernelGGL(rows::pack2_kernel, dim3(grid), dim3(256), 0, st, static_cast<const uint16_t *>(w1),
+                       static_cast<const uint16_t *>(w2), static_cast<u32x4 *>(blob), (int)C, (int)F);
+  else if (by_rows)
     hipLaunchKernelGGL(rows::pack_kernel, dim3(grid), dim3(256), 0, st, static_cast<const uint16_t *>(w1),
                        static_cast<const uint16_t *>(w2), static_cast<u32x4 *>(blob), (int)C, (int)F);
   else
@@ -1071,6 +1237,35 @@ static int launch_rows(int64_t rows, int F, const void *blob, const float *b1, c
                      tail ? static_cast<uint16_t *>(tail->ln_out) : nullptr, rows, F, nblocks);
   e = hipGetLastError();
   return e == hipSuccess ? PA_OK : (int)e;
+}
+
+template <int C, int TAIL>
+static int launch_rows2(int64_t rows, int F, const void *blob, const float *b1, const float *b2, const void *u, void *y,
+                        const pa_block_tail *tail, int num_cu, hipStream_t st) {
+  const size_t lds = (size_t)2 * (C / 16 + 2 * (C / 32)) * 64 * 16 + 8 * 8192 + (size_t)(F + 3 * C) * 4;
+  if (lds > kMaxLdsBytes) return PA_ERR_UNSUPPORTED;
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(rows::mlp_rows2_kernel<C, TAIL>),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  if (e != hipSuccess) return (int)e;
+  const int64_t nblocks = (rows + 255) / 256;
+  const int64_t grid = nblocks < num_cu ? nblocks : num_cu;
+  hipLaunchKernelGGL((rows::mlp_rows2_kernel<C, TAIL>), dim3((unsigned)grid), dim3(512), lds, st,
+                     static_cast<const u32x4 *>(blob), b1, b2, static_cast<const uint16_t *>(u),
+                     static_cast<uint16_t *>(y), tail ? static_cast<const uint16_t *>(tail->residual) : nullptr,
+                     tail ? tail->ln_gamma : nullptr, tail ? tail->ln_beta : nullptr, tail ? tail->ln_eps : 0.f,
+                     tail ? static_cast<uint16_t *>(tail->ln_out) : nullptr, rows, F, nblocks);
+  e = hipGetLastError();
+  return e == hipSuccess ? PA_OK : (int)e;
+}
+
+template <int C>
+static int launch_rows2_c(int64_t rows, int F, const void *blob, const float *b1, const float *b2, const void *u, void *y,
+                          const pa_block_tail *tail, int num_cu, hipStream_t st) {
+  const bool res = tail && tail->residual, ln = tail && tail->ln_out;
+  if (res && ln) return launch_rows2<C, 1>(rows, F, blob, b1, b2, u, y, tail, num_cu, st);
+  if (res) return launch_rows2<C, 2>(rows, F, blob, b1, b2, u, y, tail, num_cu, st);
+  if (ln) return launch_rows2<C, 3>(rows, F, blob, b1, b2, u, y, tail, num_cu, st);
+  return launch_rows2<C, 0>(rows, F, blob, b1, b2, u, y, nullptr, num_cu, st);
 }
 
 template <int C>
@@ -1197,6 +1392,7 @@ int project_packed(int64_t B, int64_t N, int64_t C, const void *w_x, const float
 int forward(int64_t rows, int64_t C, int64_t F, const void *blob, const float *b1, const float *b2, const void *u,
             void *y, const pa_block_tail *tail, int num_cu, hipStream_t st) {
   if (C == 512) return launch_rows_c<512>(rows, (int)F, blob, b1, b2, u, y, tail, num_cu, st);
+  if (C == 256 && use_rows2_kernel(C)) return launch_rows2_c<256>(rows, (int)F, blob, b1, b2, u, y, tail, num_cu, st);
   if (C == 256) return launch_c<256>(rows, (int)F, blob, b1, b2, u, y, tail, num_cu, st);
   if (C == 128) return launch_c<128>(rows, (int)F, blob, b1, b2, u, y, tail, num_cu, st);
   return PA_ERR_UNSUPPORTED;
