@@ -820,38 +820,47 @@ __global__ __launch_bounds__(256) void pack2_kernel(const uint16_t *__restrict__
   }
 }
 
-template <int C, int TAIL>
-__global__ __launch_bounds__(512) void mlp_rows2_kernel(
+// WAVES = 8: one workgroup per CU (two waves per SIMD from the same workgroup), epilogue staged in a region of its
+// own.  WAVES = 4: two workgroups per CU, each with one wave per SIMD and its own weight stream; the epilogue of one
+// (bound by the CU's store rate) then overlaps with the matrix work of the other; it stages through the idle weight
+// buffer.
+template <int C, int TAIL, int WAVES>
+__global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void mlp_rows2_kernel(
     const u32x4 *__restrict__ blob, const float *__restrict__ b1, const float *__restrict__ b2,
     const uint16_t *__restrict__ u, uint16_t *__restrict__ y, const uint16_t *__restrict__ residual,
     const float *__restrict__ ln_gamma, const float *__restrict__ ln_beta, float ln_eps, uint16_t *__restrict__ ln_out,
     int64_t M, int F, int64_t nblocks) {
   constexpr bool HAS_RES = TAIL == 1 || TAIL == 2, HAS_LN = TAIL == 1 || TAIL == 3;
   constexpr int KS = C / 16, CT = C / 32, NF = KS + 2 * CT, SU = NF * 64;
-  constexpr int WU = SU / 8;       // units of a slot fetched by each wave
-  static_assert(WU == 256, "one group of four loads per wave and slot");
+  constexpr int WU = SU / WAVES;   // units of a slot fetched by each wave
+  constexpr int NGRP = WU / 256;   // groups of four loads per wave and slot
+  static_assert(WU % 256 == 0, "whole groups of four loads per wave and slot");
   constexpr int STG = 8192;        // bytes of epilogue staging per wave
-  constexpr int kRows = 256;       // rows per block
+  constexpr int kRows = 32 * WAVES;  // rows per block
+  constexpr bool OWN_STAGE = WAVES == 8;
   extern __shared__ u32x4 smem[];
   u32x4 *wbuf = smem;                                             // 2 * SU
-  uint32_t *stage = reinterpret_cast<uint32_t *>(wbuf + 2 * SU);  // 8 waves x STG bytes
-  float *b1s = reinterpret_cast<float *>(stage + 8 * STG / 4);
+  uint32_t *stage = reinterpret_cast<uint32_t *>(wbuf + 2 * SU);  // OWN_STAGE: 8 waves x STG bytes
+  float *b1s = reinterpret_cast<float *>(stage + (OWN_STAGE ? 8 * STG / 4 : 0));
   float *b2s = b1s + F;
   float *gams = b2s + C, *bets = gams + C;
   const int tid = threadIdx.x, lane = tid & 63, i = lane & 31, g = lane >> 5;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: addresses derived from it stay scalar
   const int NCH = F / 32;
-  for (int k = tid; k < F; k += 512) b1s[k] = b1[k];
-  for (int k = tid; k < C; k += 512) {
+  for (int k = tid; k < F; k += 64 * WAVES) b1s[k] = b1[k];
+  for (int k = tid; k < C; k += 64 * WAVES) {
     b2s[k] = b2[k];
     gams[k] = HAS_LN ? ln_gamma[k] : 1.f;
     bets[k] = HAS_LN ? ln_beta[k] : 0.f;
   }
   __syncthreads();
-  auto fetch = [&](int64_t gs, int c) {  // this wave's 4 KB of slot c into buffer gs & 1
-    const u32x4 *src = blob + (int64_t)c * SU + wave * WU;
-    const unsigned dst = (unsigned)(uintptr_t)(wbuf + (gs & 1) * SU + wave * WU);
-    load_4k_to_lds(src, lane * 16, dst);
+  auto fetch = [&](int64_t gs, int c) {  // this wave's share of slot c into buffer gs & 1
+#pragma unroll
+    for (int k = 0; k < NGRP; ++k) {
+      const u32x4 *src = blob + (int64_t)c * SU + wave * WU + k * 256;
+      const unsigned dst = (unsigned)(uintptr_t)(wbuf + (gs & 1) * SU + wave * WU + k * 256);
+      load_4k_to_lds(src, lane * 16, dst);
+    }
   };
   auto load_rows = [&](int64_t mb, u32x4(&ub)[KS]) {
     int64_t r = mb * kRows + wave * 32 + i;
@@ -932,7 +941,12 @@ __global__ __launch_bounds__(512) void mlp_rows2_kernel(
       for (int j = 0; j < 8; ++j) hrest[j] = hacc[8 + j];
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's share of the next block's first slot has landed
-    finish_rows<C, HAS_RES, HAS_LN, STG>(yacc, stage + wave * (STG / 4), i, g, row0, M, residual, y, ln_out, gams, bets,
+    uint32_t *stg = stage + wave * (STG / 4);
+    if constexpr (!OWN_STAGE) {  // the buffer of the last slot is idle once every wave is past its last MFMA
+      __syncthreads();
+      stg = reinterpret_cast<uint32_t *>(wbuf + ((gs - 1) & 1) * SU) + wave * (STG / 4);
+    }
+    finish_rows<C, HAS_RES, HAS_LN, STG>(yacc, stg, i, g, row0, M, residual, y, ln_out, gams, bets,
                                          ln_eps, [&]() { load_rows(mb + gridDim.x < nblocks ? mb + gridDim.x : mb, ub); });
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // nothing may still be landing in LDS when the workgroup ends
@@ -1242,14 +1256,16 @@ static int launch_rows(int64_t rows, int F, const void *blob, const float *b1, c
 template <int C, int TAIL>
 static int launch_rows2(int64_t rows, int F, const void *blob, const float *b1, const float *b2, const void *u, void *y,
                         const pa_block_tail *tail, int num_cu, hipStream_t st) {
-  const size_t lds = (size_t)2 * (C / 16 + 2 * (C / 32)) * 64 * 16 + 8 * 8192 + (size_t)(F + 3 * C) * 4;
+  constexpr int WAVES = 8;  // one workgroup per CU; 4 (two per CU, own weight streams) measured 2 % slower
+  const size_t lds = (size_t)2 * (C / 16 + 2 * (C / 32)) * 64 * 16 + (WAVES == 8 ? 8 * 8192 : 0) + (size_t)(F + 3 * C) * 4;
   if (lds > kMaxLdsBytes) return PA_ERR_UNSUPPORTED;
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(rows::mlp_rows2_kernel<C, TAIL>),
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(rows::mlp_rows2_kernel<C, TAIL, WAVES>),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (e != hipSuccess) return (int)e;
-  const int64_t nblocks = (rows + 255) / 256;
-  const int64_t grid = nblocks < num_cu ? nblocks : num_cu;
-  hipLaunchKernelGGL((rows::mlp_rows2_kernel<C, TAIL>), dim3((unsigned)grid), dim3(512), lds, st,
+  const int64_t nblocks = (rows + 32 * WAVES - 1) / (32 * WAVES);
+  const int64_t resident = (int64_t)num_cu * (8 / WAVES);
+  const int64_t grid = nblocks < resident ? nblocks : resident;
+  hipLaunchKernelGGL((rows::mlp_rows2_kernel<C, TAIL, WAVES>), dim3((unsigned)grid), dim3(64 * WAVES), lds, st,
                      static_cast<const u32x4 *>(blob), b1, b2, static_cast<const uint16_t *>(u),
                      static_cast<uint16_t *>(y), tail ? static_cast<const uint16_t *>(tail->residual) : nullptr,
                      tail ? tail->ln_gamma : nullptr, tail ? tail->ln_beta : nullptr, tail ? tail->ln_eps : 0.f,
