@@ -1,9 +1,16 @@
 // Fused block MLP on gfx950 MFMA:  y = W2 . gelu(W1 . u + b1) + b2  [+ residual]  [-> LayerNorm(y)]
-// for bf16 rows u (M x C), hidden width F, C in {128, 256}, F a multiple of 64.
+// for bf16 rows u (M x C), hidden width F (a multiple of 64).
 // Replaces the reference's `ln_mlp1[1](ln) + fx` (physicsnemo/models/transolver/transolver.py:301-303; Mlp:
 // physicsnemo/nn/module/mlp_layers.py:139-173, GELU = erf form, activations.py:188-243) and hands the
 // LayerNorm of the result to the next consumer (next block's ln_1 or the output head's LayerNorm).
 //
+// Three tilings, chosen by C (namespace rows holds the two in which a wave owns its rows outright, together with the
+// row GEMMs of the 512-wide layer built on the same skeleton):
+//   C = 128   mlp_kernel        pairs of waves share 64 rows and split hidden tiles and output channels (below)
+//   C = 256   mlp_rows2_kernel  32 rows per wave, two waves per SIMD
+//   C = 512   mlp_rows_kernel   32 rows per wave, one wave per SIMD, the two products interleaved
+//
+// mlp_kernel:
 // One workgroup of 4 waves per CU, one wave per SIMD (256 vector + 256 accumulation registers per lane).  A block
 // of 128 rows is shared by two pairs of waves; the waves (rg, p = 0 / 1) of a pair own the same 64 rows:
 //   * the rows of u stay in registers as B operands for the whole block (lane <-> row, k <-> channel);
@@ -23,7 +30,6 @@
 #include "pa_host.h"
 #include "pa_mfma_ops.h"
 
-#include <cstdlib>
 #include <type_traits>
 #include <utility>
 
@@ -1199,7 +1205,7 @@ __global__ __launch_bounds__(512) void project_rows_kernel(
 // ---------------------------------------------------------------------------------------------------------------
 // C = 512 runs the row-owning kernel with one wave per SIMD, C = 256 the one with two, C = 128 the paired kernel
 static bool use_rows_kernel(int64_t C) { return C == 512; }
-static bool use_rows2_kernel(int64_t C) { return C == 256 && !getenv("PA_MLP_PAIRED"); }
+static bool use_rows2_kernel(int64_t C) { return C == 256; }
 
 bool supported(int dtype, int64_t rows, int64_t C, int64_t F) {
   if (dtype != PA_BF16 || rows <= 0 || F < 64 || F % 64 != 0 || F > 8192) return false;
@@ -1408,8 +1414,7 @@ int project_packed(int64_t B, int64_t N, int64_t C, const void *w_x, const float
 int forward(int64_t rows, int64_t C, int64_t F, const void *blob, const float *b1, const float *b2, const void *u,
             void *y, const pa_block_tail *tail, int num_cu, hipStream_t st) {
   if (C == 512) return launch_rows_c<512>(rows, (int)F, blob, b1, b2, u, y, tail, num_cu, st);
-  if (C == 256 && use_rows2_kernel(C)) return launch_rows2_c<256>(rows, (int)F, blob, b1, b2, u, y, tail, num_cu, st);
-  if (C == 256) return launch_c<256>(rows, (int)F, blob, b1, b2, u, y, tail, num_cu, st);
+  if (C == 256) return launch_rows2_c<256>(rows, (int)F, blob, b1, b2, u, y, tail, num_cu, st);
   if (C == 128) return launch_c<128>(rows, (int)F, blob, b1, b2, u, y, tail, num_cu, st);
   return PA_ERR_UNSUPPORTED;
 }
