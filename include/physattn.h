@@ -430,7 +430,8 @@ typedef struct pa_mlp_params {
   const float *b2;
 } pa_mlp_params;
 
-/* 1 if pa_mlp_forward serves (dtype, rows, C, F) [bf16, C in {128, 256, 512}, F a multiple of 64 (C = 512: up to 4096)], else 0. */
+/* 1 if pa_mlp_forward serves (dtype, rows, C, F) [bf16, C in {128, 256, 512}, F a multiple of 64 up to 8192 / 7424 /
+ * 6656 for the three widths (what the kernel's LDS holds)], else 0. */
 int pa_mlp_query(int dtype, int64_t rows, int64_t C, int64_t F);
 /* Bytes of workspace pa_mlp_forward needs (the repacked weights), or a negative error code. */
 int64_t pa_mlp_workspace_bytes(int dtype, int64_t rows, int64_t C, int64_t F);

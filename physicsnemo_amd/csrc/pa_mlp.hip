@@ -1207,10 +1207,17 @@ __global__ __launch_bounds__(512) void project_rows_kernel(
 static bool use_rows_kernel(int64_t C) { return C == 512; }
 static bool use_rows2_kernel(int64_t C) { return C == 256; }
 
+// dynamic LDS of the kernel that serves (C, F): two weight buffers, staging / exchange areas, biases and LayerNorm vectors
+static size_t lds_need(int64_t C, int64_t F) {
+  if (use_rows_kernel(C)) return (size_t)2 * 4096 * 16 + (size_t)(F + 3 * C) * 4;
+  if (use_rows2_kernel(C)) return (size_t)2 * (C / 16 + 2 * (C / 32)) * 64 * 16 + 8 * 8192 + (size_t)(F + 3 * C) * 4;
+  return (size_t)(2 * slot_units((int)C) + 4 * 4 * 64) * 16 + (size_t)(F + C) * 4;
+}
+
 bool supported(int dtype, int64_t rows, int64_t C, int64_t F) {
   if (dtype != PA_BF16 || rows <= 0 || F < 64 || F % 64 != 0 || F > 8192) return false;
-  if (use_rows_kernel(C)) return F <= 4096;
-  return C == 128 || C == 256;
+  if (C != 128 && C != 256 && C != 512) return false;
+  return lds_need(C, F) <= (size_t)kMaxLdsBytes;
 }
 
 int64_t blob_bytes(int64_t C, int64_t F) {
@@ -1219,7 +1226,6 @@ int64_t blob_bytes(int64_t C, int64_t F) {
   return (F / 64 + 1) * (int64_t)slot_units((int)C) * 16;
 }
 
-static size_t lds_bytes(int C, int F) { return (size_t)(2 * slot_units(C) + 4 * 4 * 64) * 16 + (size_t)(F + C) * 4; }
 
 int pack(int64_t C, int64_t F, const void *w1, const void *w2, void *blob, hipStream_t st) {
   const bool by_rows = use_rows_kernel(C), by_rows2 = use_rows2_kernel(C);
@@ -1243,7 +1249,7 @@ int pack(int64_t C, int64_t F, const void *w1, const void *w2, void *blob, hipSt
 template <int C, int TAIL>
 static int launch_rows(int64_t rows, int F, const void *blob, const float *b1, const float *b2, const void *u, void *y,
                        const pa_block_tail *tail, int num_cu, hipStream_t st) {
-  const size_t lds = (size_t)2 * rows::Cfg<C>::SU * 16 + (size_t)(F + 3 * C) * 4;
+  const size_t lds = lds_need(C, F);
   if (lds > kMaxLdsBytes) return PA_ERR_UNSUPPORTED;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(rows::mlp_rows_kernel<C, TAIL>),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -1263,7 +1269,7 @@ template <int C, int TAIL>
 static int launch_rows2(int64_t rows, int F, const void *blob, const float *b1, const float *b2, const void *u, void *y,
                         const pa_block_tail *tail, int num_cu, hipStream_t st) {
   constexpr int WAVES = 8;  // one workgroup per CU; 4 (two per CU, own weight streams) measured 2 % slower
-  const size_t lds = (size_t)2 * (C / 16 + 2 * (C / 32)) * 64 * 16 + (WAVES == 8 ? 8 * 8192 : 0) + (size_t)(F + 3 * C) * 4;
+  const size_t lds = lds_need(C, F);  // sized for WAVES = 8 (own staging region)
   if (lds > kMaxLdsBytes) return PA_ERR_UNSUPPORTED;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(rows::mlp_rows2_kernel<C, TAIL, WAVES>),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -1303,7 +1309,7 @@ static int launch_rows_c(int64_t rows, int F, const void *blob, const float *b1,
 template <int C, int TAIL>
 static int launch(int64_t rows, int F, const void *blob, const float *b1, const float *b2, const void *u, void *y,
                   const pa_block_tail *tail, int num_cu, hipStream_t st) {
-  const size_t lds = lds_bytes(C, F);
+  const size_t lds = lds_need(C, F);
   if (lds > kMaxLdsBytes) return PA_ERR_UNSUPPORTED;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(mlp_kernel<C, TAIL>),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);

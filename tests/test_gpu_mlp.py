@@ -36,6 +36,7 @@ def _case(rows_shape, C, Fh, seed=0, scale=1.0):
     ((1, 4096), 256, 1024), ((2, 1000), 256, 1024), ((1, 257), 256, 256), ((3, 77), 128, 512), ((1, 1), 256, 1024),
     ((1, 5000), 128, 128), ((1, 20000), 256, 512),
     ((1, 4096), 512, 2048), ((2, 777), 512, 2048), ((1, 1), 512, 64), ((1, 33000), 512, 512),
+    ((1, 300), 512, 6656), ((1, 300), 256, 7424), ((1, 300), 128, 8192),  # the widest hidden layers that fit LDS
 ])
 def test_mlp_matches_fp32_oracle(rows_shape, C, Fh):
     announce("mlp", rows_shape, C, Fh)
@@ -95,4 +96,5 @@ def test_mlp_rejects_unsupported():
     assert not PF.mlp_supported(torch.float32, 100, 256, 1024)
     assert not PF.mlp_supported(torch.bfloat16, 100, 384, 1536)
     assert not PF.mlp_supported(torch.bfloat16, 100, 512, 8192)
+    assert not PF.mlp_supported(torch.bfloat16, 100, 256, 8192)
     assert not PF.mlp_supported(torch.bfloat16, 100, 256, 1000)
