@@ -483,8 +483,9 @@ int pa_layer_forward_plus(int dtype, const pa_shape *shape, const pa_params *p, 
 
 /* pa_layer_forward for the fused MFMA shapes (pa_query_path() == 1, bf16 weights) with the parameters already
  * repacked by pa_mfma_pack_params into `blob` (PA_BUF_BLOB bytes): callers that run many forwards with unchanged
- * weights keep the blob and skip the repack.  Of `p` only qkv_project_weight is read.  Workspace as for
- * pa_layer_forward.  No reference counterpart. */
+ * weights keep the blob and skip the repack.  For S <= 64 only qkv_project_weight and in_project_fx_bias of `p` are
+ * read; for S = 128 the call runs the packed-tile kernels of the staged family, which take every parameter from `p`
+ * (bf16 weights) and leave `blob` unused.  Workspace as for pa_layer_forward.  No reference counterpart. */
 int pa_mfma_layer_forward(const pa_shape *shape, const pa_params *p, const void *blob, const void *x, void *y,
                           const pa_block_tail *tail, float *slice_token_out, void *workspace,
                           int64_t workspace_bytes, void *stream);

@@ -80,9 +80,16 @@ int64_t mfma_groups(const pa_shape &s, bool fused) {
   return fused ? pa::mfma::project_groups(s, compute_units(), true) : pa::mfma::reduce_groups(s);
 }
 
+// S = 128 (the slice-token sums do not fit beside the weights of the fused kernel): the layer call runs the packed-tile
+// sequence of the staged path instead of kernels (a), (b), (d), where its row kernels serve the width
+bool mfma_layer_on_tiles(const pa_shape &s) {
+  return !pa::mfma::fuse_reduce(s) && pa::mlp::linear_supported(PA_BF16, s.B * s.N, s.C);
+}
+
 int64_t mfma_partials_bytes(const pa_shape &s) {
   int64_t g = mfma_groups(s, false);
   if (pa::mfma::fuse_reduce(s)) g = std::max(g, mfma_groups(s, true));
+  if (mfma_layer_on_tiles(s)) g = std::max(g, pa::mfma::softmax_reduce_groups(s, compute_units()));
   return (g + 1) * s.B * s.H * s.S * (s.D + 1) * 4;  // G partials + their total
 }
 
@@ -90,8 +97,8 @@ MfmaPlan plan_mfma(const pa_shape &s) {
   MfmaPlan p{};
   p.G = mfma_groups(s, pa::mfma::fuse_reduce(s));
   int64_t off = 0;
-  p.off_blob = off;
-  off += round_up(pa::mfma::blob_bytes(s), 256);
+  p.off_blob = off;  // the repacked parameters; on the packed-tile sequence the three projections in fragment order
+  off += round_up(std::max(pa::mfma::blob_bytes(s), 3 * pa::mlp::linear_blob_bytes(s.C)), 256);
   p.off_fx = off;
   off += round_up(pa::mfma::fx_pack_bytes(s), 256);
   p.off_w = off;
@@ -230,6 +237,21 @@ int mfma_layer(const pa_shape &s, const pa_params &p, const void *blob, const vo
   float *norm = reinterpret_cast<float *>(ws + mp.off_norm);
   float *tok_out = reinterpret_cast<float *>(ws + mp.off_tok_out);
   int rc;
+  if (mfma_layer_on_tiles(s)) {
+    // slice weights recomputed where they are used, never stored; every intermediate a packed tile of 32 points.
+    // x_mid / out_x take the room of the slice weights, the projections' fragments that of the parameter blob.
+    char *wts = ws + mp.off_blob;
+    const int64_t G = pa::mfma::softmax_reduce_groups(s, compute_units());
+    if ((rc = pa::mlp::project_packed(s.B, s.N, s.C, p.in_project_x_weight, p.in_project_x_bias, p.in_project_fx_weight,
+                                      p.in_project_fx_bias, x, wp, fxp, wts, compute_units(), st)))
+      return rc;
+    if ((rc = pa::mfma::slice_softmax_reduce(s, p, wp, true, fxp, partials, compute_units(), st))) return rc;
+    if ((rc = pa::mfma::combine_attention(s, p, nullptr, partials, G, tok, norm, tok_out, tokp, st))) return rc;
+    if ((rc = pa::mfma::deslice_recompute(s, p, wp, true, tokp, wp, compute_units(), st))) return rc;
+    return pa::mlp::linear_packed(s.B, s.N, s.C, p.out_linear_weight, p.out_linear_bias, wp, y,
+                                  tail_active(tail) ? tail : nullptr, wts + 2 * pa::mlp::linear_blob_bytes(s.C),
+                                  compute_units(), st);
+  }
   if (pa::mfma::fuse_reduce(s)) {  // kernel (a) also leaves the partial slice-token sums
     if ((rc = pa::mfma::project_softmax(s, blob, x, nullptr, wp, partials, compute_units(), st))) return rc;
   } else {
@@ -851,6 +873,13 @@ int pa_mfma_layer_forward(const pa_shape *shape, const pa_params *p, const void 
   if (!p || !p->qkv_project_weight || !blob || !x || !y || !workspace) return PA_ERR_NULL;
   if (!aligned16(blob) || !aligned16(x) || !aligned16(y) || !aligned16(workspace)) return PA_ERR_ALIGN;
   if ((rc = check_tail(tail))) return rc;
+  if (mfma_layer_on_tiles(*shape)) {  // this sequence reads the parameters themselves, not the blob
+    if (!p->in_project_x_weight || !p->in_project_fx_weight || !p->in_project_slice_weight ||
+        !p->in_project_slice_bias || !p->temperature || !p->out_linear_weight)
+      return PA_ERR_NULL;
+    if (!aligned16(p->in_project_x_weight) || !aligned16(p->in_project_fx_weight) || !aligned16(p->out_linear_weight))
+      return PA_ERR_ALIGN;
+  }
   const MfmaPlan mp = plan_mfma(*shape);
   if (workspace_bytes < mp.total) return PA_ERR_WORKSPACE;
   return mfma_layer(*shape, *p, blob, x, y, tail, slice_token_out, static_cast<char *>(workspace), mp,

@@ -472,11 +472,13 @@ int slice_softmax_pack_plus(const pa_shape &s, const pa_params &p, const pa_plus
   return launch_status();
 }
 
-// grid of the two recomputing kernels: waves = heads per workgroup, about two workgroups per CU
+// grid of the two recomputing kernels: waves = heads per workgroup; a workgroup of 8 waves fills a CU (two waves per
+// SIMD at their register count), so one workgroup per CU: fewer partial sums to combine
 static void recompute_grid(const pa_shape &s, int num_cu, dim3 *grid, dim3 *block) {
   const int waves = (int)(s.H < 8 ? s.H : 8);
   const int groups = (int)(s.H / waves);
-  int64_t gx = (2 * (int64_t)num_cu + s.B * groups - 1) / (s.B * groups);
+  const int per_cu = waves >= 8 ? 1 : 2;
+  int64_t gx = (per_cu * (int64_t)num_cu + s.B * groups - 1) / (s.B * groups);
   const int64_t tpb = tiles_per_batch(s);
   if (gx > tpb) gx = tpb;
   if (gx < 1) gx = 1;

@@ -1092,17 +1092,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 //                                halves of a head are B operands (columns = points, k = the head's channels, kperm order)
 //   fx_mid  = x . W_fx^T + b_fx  rows as A, weights as B: lanes <-> channels, registers <-> points; the two packed
 //                                halves of a head are A operands (rows = channels, k = points, kperm order)
-// Output tiles are the outer loop: a slot of the weight stream (64 fragments, 64 KB) holds all C/16 k-steps of two
-// heads, interleaved so that the two accumulators alternate; when the slot is done the two heads leave as four 1 KB
-// stores per wave: out[((tile H + head) 2 + half) 64 + lane].  Only two accumulators are live, which is what lets two
-// waves share a SIMD, and the stores are spread evenly over the kernel.
-// blob: W_x then W_fx, each H/2 slots in that order (project_pack_kernel).
+// Output tiles are the outer loop: a slot of the weight stream (64 fragments, 64 KB) holds all C/16 k-steps of
+// HPS = 1024 / C heads, interleaved so that the HPS accumulators take turns; when the slot is done the heads leave as
+// 2 HPS stores of 1 KB per wave: out[((tile H + head) 2 + half) 64 + lane].  Only HPS accumulators are live, which is
+// what lets two waves share a SIMD, and the stores are spread evenly over the kernel.
+// blob: W_x then W_fx, each H / HPS slots in that order (project_pack_kernel).
 // ---------------------------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void project_pack_kernel(const uint16_t *__restrict__ w, u32x4 *__restrict__ blob, int C) {
+  const int KS = C / 16, HPS = 64 / KS;  // heads per slot
   const int64_t total = (int64_t)C * C / 8;
   for (int64_t u = (int64_t)blockIdx.x * 256 + threadIdx.x; u < total; u += (int64_t)gridDim.x * 256) {
     const int c = (int)(u >> 12), j = (int)(u & 4095) >> 6, lane = (int)(u & 63), i = lane & 31, g = lane >> 5;
-    const int ct = 2 * c + (j & 1), ks = j >> 1;
+    const int ct = HPS * c + j % HPS, ks = j / HPS;
     blob[u] = *reinterpret_cast<const u32x4 *>(w + (int64_t)(32 * ct + i) * C + 16 * ks + 8 * g);
   }
 }
@@ -1113,8 +1114,9 @@ __global__ __launch_bounds__(512) void project_rows_kernel(
     const uint16_t *__restrict__ x, u32x4 *__restrict__ xm_pack, u32x4 *__restrict__ fx_pack, int64_t N, int tpb,
     int64_t ntiles, int64_t nblocks) {
   constexpr int KS = C / 16, CT = C / 32, SU = 4096, WU = SU / 8;
-  constexpr int NSLOT = CT / 2;  // slots per product
-  static_assert(KS == 32, "a slot holds the k-steps of two heads");
+  constexpr int HPS = 64 / KS;       // heads per slot (2 at C = 512, 4 at C = 256)
+  constexpr int NSLOT = CT / HPS;    // slots per product
+  static_assert(KS * HPS == 64 && CT % HPS == 0, "a slot holds all k-steps of HPS heads");
   extern __shared__ u32x4 smem[];
   u32x4 *wbuf = smem;  // 2 * SU
   float *bxs = reinterpret_cast<float *>(wbuf + 2 * SU);
@@ -1156,16 +1158,17 @@ __global__ __launch_bounds__(512) void project_rows_kernel(
     load_rows(mb, ub);
     for (int c = 0; c < 2 * NSLOT; ++c, ++gs) {
       const bool second = c >= NSLOT;          // the fx product
-      const int ct0 = 2 * (c - (second ? NSLOT : 0));  // heads ct0, ct0 + 1
+      const int ct0 = HPS * (c - (second ? NSLOT : 0));  // heads ct0 .. ct0 + HPS - 1
       // Slot gs has landed (every wave waits for its own share, then all meet) and the other buffer is free.  The
-      // share was requested before the four stores of the slot before: those may still be in flight.
+      // share was requested before the 2 HPS stores of the slot before: those may still be in flight.
       if (c == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-      else asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+      else if constexpr (HPS == 2) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+      else asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
       __syncthreads();
       const u32x4 *wb = wbuf + (gs & 1) * SU + lane;
-      f32x16 acc[2];
+      f32x16 acc[HPS];
 #pragma unroll
-      for (int q = 0; q < 2; ++q)
+      for (int q = 0; q < HPS; ++q)
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[q][r] = second ? bfs[32 * (ct0 + q) + i] : bxs[32 * (ct0 + q) + rowmap(r, g)];
       constexpr int RING = 6, AHEAD = 4;
@@ -1176,7 +1179,7 @@ __global__ __launch_bounds__(512) void project_rows_kernel(
         static_for<64>([&](auto j_) {
           constexpr int j = decltype(j_)::value;
           if constexpr (j + AHEAD < 64) fr[(j + AHEAD) % RING] = wb[(j + AHEAD) * 64];
-          acc[j & 1] = mma(fr[j % RING], ub[j >> 1], acc[j & 1]);
+          acc[j % HPS] = mma(fr[j % RING], ub[j / HPS], acc[j % HPS]);
           if constexpr (j == 1 || j == 9) fetch_group(gs + 1, c_next, j / 8);
           __builtin_amdgcn_sched_barrier(0);
         });
@@ -1184,17 +1187,18 @@ __global__ __launch_bounds__(512) void project_rows_kernel(
         static_for<64>([&](auto j_) {
           constexpr int j = decltype(j_)::value;
           if constexpr (j + AHEAD < 64) fr[(j + AHEAD) % RING] = wb[(j + AHEAD) * 64];
-          acc[j & 1] = mma(ub[j >> 1], fr[j % RING], acc[j & 1]);
+          acc[j % HPS] = mma(ub[j / HPS], fr[j % RING], acc[j % HPS]);
           if constexpr (j == 1 || j == 9) fetch_group(gs + 1, c_next, j / 8);
           __builtin_amdgcn_sched_barrier(0);
         });
       }
-      // exactly four stores per slot and wave (see the wait above): tiles past the end rewrite the last one's
+      // exactly 2 HPS stores per slot and wave (see the wait above): tiles past the end rewrite the last one's
       u32x4 *dst = (second ? fx_pack : xm_pack) + ((live ? gt : ntiles - 1) * CT + ct0) * (2 * 64) + lane;
-      dst[0] = pack_half<0>(acc[0]);
-      dst[64] = pack_half<1>(acc[0]);
-      dst[128] = pack_half<0>(acc[1]);
-      dst[192] = pack_half<1>(acc[1]);
+#pragma unroll
+      for (int q = 0; q < HPS; ++q) {
+        dst[(2 * q) * 64] = pack_half<0>(acc[q]);
+        dst[(2 * q + 1) * 64] = pack_half<1>(acc[q]);
+      }
     }
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // nothing may still be landing in LDS when the workgroup ends
@@ -1336,7 +1340,9 @@ static int launch_c(int64_t rows, int F, const void *blob, const float *b1, cons
 }
 
 // ---- out_linear with the block's tail on the row-owning kernel --------------------------------------------------
-bool linear_supported(int dtype, int64_t rows, int64_t C) { return dtype == PA_BF16 && rows > 0 && C == 512; }
+bool linear_supported(int dtype, int64_t rows, int64_t C) {
+  return dtype == PA_BF16 && rows > 0 && (C == 512 || C == 256);
+}
 
 int64_t linear_blob_bytes(int64_t C) { return C * C * 2; }
 
@@ -1359,20 +1365,27 @@ static int launch_linear(int64_t rows, const void *blob, const float *bias, cons
   return e == hipSuccess ? PA_OK : (int)e;
 }
 
+template <int C, bool PACKED_IN>
+static int linear_c(int64_t rows, const void *blob, const float *bias, const void *x, void *y, const pa_block_tail *tail,
+                    int64_t N, int tpb, int num_cu, hipStream_t st) {
+  const bool res = tail && tail->residual, ln = tail && tail->ln_out;
+  if (res && ln) return launch_linear<C, 1, PACKED_IN>(rows, blob, bias, x, y, tail, N, tpb, num_cu, st);
+  if (res) return launch_linear<C, 2, PACKED_IN>(rows, blob, bias, x, y, tail, N, tpb, num_cu, st);
+  if (ln) return launch_linear<C, 3, PACKED_IN>(rows, blob, bias, x, y, tail, N, tpb, num_cu, st);
+  return launch_linear<C, 0, PACKED_IN>(rows, blob, bias, x, y, nullptr, N, tpb, num_cu, st);
+}
+
 template <bool PACKED_IN>
 static int linear_any(int64_t rows, int64_t C, const void *w, const float *bias, const void *x, void *y,
                       const pa_block_tail *tail, void *blob, int64_t N, int tpb, int num_cu, hipStream_t st) {
-  if (C != 512) return PA_ERR_UNSUPPORTED;
+  if (C != 512 && C != 256) return PA_ERR_UNSUPPORTED;
   const int64_t total = C * C / 8;
   hipLaunchKernelGGL(rows::linear_pack_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st,
                      static_cast<const uint16_t *>(w), static_cast<u32x4 *>(blob), (int)C, PACKED_IN ? 1 : 0);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return (int)e;
-  const bool res = tail && tail->residual, ln = tail && tail->ln_out;
-  if (res && ln) return launch_linear<512, 1, PACKED_IN>(rows, blob, bias, x, y, tail, N, tpb, num_cu, st);
-  if (res) return launch_linear<512, 2, PACKED_IN>(rows, blob, bias, x, y, tail, N, tpb, num_cu, st);
-  if (ln) return launch_linear<512, 3, PACKED_IN>(rows, blob, bias, x, y, tail, N, tpb, num_cu, st);
-  return launch_linear<512, 0, PACKED_IN>(rows, blob, bias, x, y, nullptr, N, tpb, num_cu, st);
+  if (C == 512) return linear_c<512, PACKED_IN>(rows, blob, bias, x, y, tail, N, tpb, num_cu, st);
+  return linear_c<256, PACKED_IN>(rows, blob, bias, x, y, tail, N, tpb, num_cu, st);
 }
 
 // y = W x + bias (+ tail) for (rows, C) row-major x; `blob` = linear_blob_bytes(C) bytes of scratch for the
@@ -1395,7 +1408,7 @@ int linear_packed(int64_t B, int64_t N, int64_t C, const void *w, const float *b
 int project_packed(int64_t B, int64_t N, int64_t C, const void *w_x, const float *b_x, const void *w_fx,
                    const float *b_fx, const void *x, void *xm_pack, void *fx_pack, void *blob, int num_cu,
                    hipStream_t st) {
-  if (C != 512) return PA_ERR_UNSUPPORTED;
+  if (C != 512 && C != 256) return PA_ERR_UNSUPPORTED;
   const int64_t total = C * C / 8;
   u32x4 *bl = static_cast<u32x4 *>(blob);
   hipLaunchKernelGGL(rows::project_pack_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st,
@@ -1405,14 +1418,20 @@ int project_packed(int64_t B, int64_t N, int64_t C, const void *w_x, const float
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return (int)e;
   const size_t lds = (size_t)2 * 4096 * 16 + (size_t)2 * C * 4;
-  e = hipFuncSetAttribute(reinterpret_cast<const void *>(rows::project_rows_kernel<512>),
-                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  const void *kernel = C == 512 ? reinterpret_cast<const void *>(rows::project_rows_kernel<512>)
+                                : reinterpret_cast<const void *>(rows::project_rows_kernel<256>);
+  e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (e != hipSuccess) return (int)e;
   const int64_t tpb = (N + 31) / 32, ntiles = B * tpb, nblocks = (ntiles + 7) / 8;
   const int64_t grid = nblocks < num_cu ? nblocks : num_cu;
-  hipLaunchKernelGGL((rows::project_rows_kernel<512>), dim3((unsigned)grid), dim3(512), lds, st, bl, b_x, b_fx,
-                     static_cast<const uint16_t *>(x), static_cast<u32x4 *>(xm_pack), static_cast<u32x4 *>(fx_pack), N,
-                     (int)tpb, ntiles, nblocks);
+  if (C == 512)
+    hipLaunchKernelGGL((rows::project_rows_kernel<512>), dim3((unsigned)grid), dim3(512), lds, st, bl, b_x, b_fx,
+                       static_cast<const uint16_t *>(x), static_cast<u32x4 *>(xm_pack), static_cast<u32x4 *>(fx_pack),
+                       N, (int)tpb, ntiles, nblocks);
+  else
+    hipLaunchKernelGGL((rows::project_rows_kernel<256>), dim3((unsigned)grid), dim3(512), lds, st, bl, b_x, b_fx,
+                       static_cast<const uint16_t *>(x), static_cast<u32x4 *>(xm_pack), static_cast<u32x4 *>(fx_pack),
+                       N, (int)tpb, ntiles, nblocks);
   e = hipGetLastError();
   return e == hipSuccess ? PA_OK : (int)e;
 }

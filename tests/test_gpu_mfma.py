@@ -102,8 +102,10 @@ def test_mfma_stage_entry_points_agree_with_layer_call(B, N, C, S):
         assert_rel_l2(st.norm, norm_ab, "fused vs separate slice norm", tol=1e-5)
         assert_rel_l2(y_f, y_ab, "fused vs separate output", tol=2e-3)
     else:
-        assert torch.equal(y_ab, y)
-        assert torch.equal(tok_ab, tok)
+        # S = 128: the layer call runs the packed-tile sequence (slice weights recomputed, not stored), the stage entry
+        # points kernels (a), (b), (d): the same function, bf16 roundings in a different order
+        assert_rel_l2(y, y_ab, "layer call vs stage kernels: output", tol=4e-3)
+        assert_rel_l2(tok, tok_ab, "layer call vs stage kernels: slice tokens", tol=4e-3)
     # norm invariant: sum_s (norm - 0.01) = number of points, up to bf16 rounding of the weights
     total = (st.norm - 0.01).sum(-1)
     assert torch.allclose(total, torch.full_like(total, float(N)), rtol=2e-3)
@@ -175,7 +177,13 @@ def test_mfma_full_size_properties(S):
         st.slice_reduce()
     st.combine_attention()
     st.deslice_project(y2)
-    assert torch.equal(y2, y) and torch.equal(st.tok, tok)
+    if st.fused_groups > 0:
+        assert torch.equal(y2, y) and torch.equal(st.tok, tok)
+    else:
+        # S = 128: the layer call runs the packed-tile sequence (slice weights recomputed, not stored); the stage
+        # kernels compute the same function with a different rounding order
+        assert_rel_l2(y, y2, f"S={S}: layer call vs stage kernels", tol=4e-3)
+        assert_rel_l2(tok, st.tok, f"S={S}: slice tokens, layer call vs stage kernels", tol=4e-3)
     del y2
     # every point spreads a total weight of one over the slices
     total = (st.norm - 0.01).sum(-1)
