@@ -203,10 +203,13 @@ __global__ __launch_bounds__(512) void slice_softmax_pack_plus_kernel(
 // operand chunks.  chunk[cq] (cq = 0 .. S/16 - 1) is what slice_softmax_pack_kernel stores: as an A operand its rows
 // are the points and its reduction index the slices 16 cq + kperm order; the same registers serve as a B operand
 // whose columns are the points.  Both kernels below recompute the weights from x_mid instead of passing them through
-// memory (S/16 KB per point and head group written once and read twice otherwise); the arithmetic is identical in
-// both, so the weights that aggregate the tokens and the ones that hand them back are the same numbers.
+// memory (S/16 KB per point and head group written once and read twice otherwise).  The token sums use
+// bf16(e_s / sum e), the hand-back bf16(e_s) divided by the sum of those rounded values: the same softmax, each rounded
+// once.
 // ------------------------------------------------------------------------------------------------
-template <int S>
+// DEFER: the chunks hold bf16(exp2(..)) without the division by their sum; the caller divides what it forms from them
+// by the sum of the same rounded values (one more MFMA column), which saves a pass over the S values per point.
+template <int S, bool DEFER = false>
 __device__ __forceinline__ void slice_weights_of_tile(const u32x4 *__restrict__ wsl, const float *__restrict__ bsl,
                                                       u32x4 xm0, u32x4 xm1, float sc, bool valid, int lane, int g,
                                                       u32x4 (&chunk)[S / 16]) {
@@ -226,19 +229,28 @@ __device__ __forceinline__ void slice_weights_of_tile(const u32x4 *__restrict__ 
     for (int r = 0; r < 16; ++r) mx = fmaxf(mx, lg[st][r]);
   mx = half_max(mx);
   const float off = mx * sc;
-  float sum = 0.f;
+  if constexpr (DEFER) {
 #pragma unroll
-  for (int st = 0; st < ST; ++st)
+    for (int st = 0; st < ST; ++st)
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const float e = __builtin_amdgcn_exp2f(fmaf(lg[st][r], sc, -off));
-      lg[st][r] = e;
-      sum += e;
-    }
-  sum = half_sum(sum);
-  const float inv = valid ? __builtin_amdgcn_rcpf(sum) : 0.f;
+      for (int r = 0; r < 16; ++r) lg[st][r] = __builtin_amdgcn_exp2f(fmaf(lg[st][r], sc, -off));
 #pragma unroll
-  for (int cq = 0; cq < NCH; ++cq) chunk[cq] = (cq & 1) ? pack_half<1>(lg[cq >> 1], inv) : pack_half<0>(lg[cq >> 1], inv);
+    for (int cq = 0; cq < NCH; ++cq) chunk[cq] = (cq & 1) ? pack_half<1>(lg[cq >> 1]) : pack_half<0>(lg[cq >> 1]);
+  } else {
+    float sum = 0.f;
+#pragma unroll
+    for (int st = 0; st < ST; ++st)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const float e = __builtin_amdgcn_exp2f(fmaf(lg[st][r], sc, -off));
+        lg[st][r] = e;
+        sum += e;
+      }
+    sum = half_sum(sum);
+    const float inv = valid ? __builtin_amdgcn_rcpf(sum) : 0.f;
+#pragma unroll
+    for (int cq = 0; cq < NCH; ++cq) chunk[cq] = (cq & 1) ? pack_half<1>(lg[cq >> 1], inv) : pack_half<0>(lg[cq >> 1], inv);
+  }
 }
 
 // W_slice as A operands and the slice bias, as slice_softmax_pack_kernel stages them; the reduction index runs over
@@ -392,13 +404,22 @@ __global__ __launch_bounds__(512) void deslice_recompute_kernel(const uint16_t *
       xm0 = *reinterpret_cast<const u32x4 *>(row);
       xm1 = *reinterpret_cast<const u32x4 *>(row + 16);
     }
+    // un-normalised weights e_s (bf16); out = (sum_s e_s tok'_s) / (sum_s e_s), the denominator from an MFMA whose A
+    // operand is all ones: every row of that product is the column sum of the same rounded values
     u32x4 chunk[NCH];
-    slice_weights_of_tile<S>(wsl, bsl, xm0, xm1, sc, valid, lane, g, chunk);
-    f32x16 ox;
+    slice_weights_of_tile<S, true>(wsl, bsl, xm0, xm1, sc, valid, lane, g, chunk);
+    f32x16 ox, den;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) ox[r] = 0.f;
+    for (int r = 0; r < 16; ++r) ox[r] = den[r] = 0.f;
+    const u32x4 ones = u32x4{0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u};
 #pragma unroll
-    for (int cq = 0; cq < NCH; ++cq) ox = mma(tp[cq], chunk[cq], ox);
+    for (int cq = 0; cq < NCH; ++cq) {
+      ox = mma(tp[cq], chunk[cq], ox);
+      den = mma(ones, chunk[cq], den);
+    }
+    const float inv = __builtin_amdgcn_rcpf(den[0]);
+#pragma unroll
+    for (int r = 0; r < 16; ++r) ox[r] *= inv;
     if constexpr (PACKED_X) {
       u32x4 *odst = reinterpret_cast<u32x4 *>(out_x) + pk;
       odst[0] = pack_half<0>(ox);
