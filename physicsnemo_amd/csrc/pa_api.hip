@@ -39,14 +39,16 @@ int64_t dequant_bytes(int dtype, const pa_shape &s) {
 
 // Workspace plan of the general path.
 struct GeneralPlan {
-  int64_t off_x_mid, off_fx_mid, off_w, off_partials, off_tok, off_norm, off_tok_out, total;
+  int64_t off_x_mid, off_fx_mid, off_w, off_partials, off_tok, off_norm, off_tok_out, off_blob, total;
   int64_t G;
+  bool conv_front;  // float32 structured 2-D layer of the fused front end's shape class
 };
 
 GeneralPlan plan_general(int dtype, const pa_shape &s) {
   GeneralPlan p{};
   const int64_t e = elem_bytes(dtype), M = s.B * s.N, HD = s.H * s.D;
-  p.G = pa::general::partial_count(s);
+  p.conv_front = pa::conv::supported(dtype, s);
+  p.G = p.conv_front ? pa::conv::groups(s) : pa::general::partial_count(s);
   int64_t off = 0;
   p.off_x_mid = off;  // reused for out_x once the slice weights exist
   off += round_up(M * HD * e, 256);
@@ -62,6 +64,8 @@ GeneralPlan plan_general(int dtype, const pa_shape &s) {
   off += round_up(s.B * s.H * s.S * 4, 256);
   p.off_tok_out = off;
   off += round_up(s.B * s.H * s.S * s.D * 4, 256);
+  p.off_blob = off;  // the convolution weights cut into bf16 pieces, in fragment order
+  if (p.conv_front) off += round_up(pa::conv::blob_bytes(s), 256);
   p.total = off;
   return p;
 }
@@ -988,9 +992,13 @@ int pa_layer_forward(int dtype, const pa_shape *shape, const pa_params *p, const
   float *norm = reinterpret_cast<float *>(ws + plan.off_norm);
   float *tok_out = reinterpret_cast<float *>(ws + plan.off_tok_out);
 
-  if ((rc = pa::general::project_inputs(dtype, s, *p, x, x_mid, fx_mid, st))) return rc;
-  if ((rc = pa::general::slice_softmax(dtype, s, *p, x_mid, w, st))) return rc;
-  if ((rc = pa::general::slice_partial(dtype, s, w, fx_mid, partials, st))) return rc;
+  if (plan.conv_front) {  // both convolutions, the slice softmax and the partial token sums in one launch
+    if ((rc = pa::conv::front(s, *p, x, ws + plan.off_blob, w, partials, st))) return rc;
+  } else {
+    if ((rc = pa::general::project_inputs(dtype, s, *p, x, x_mid, fx_mid, st))) return rc;
+    if ((rc = pa::general::slice_softmax(dtype, s, *p, x_mid, w, st))) return rc;
+    if ((rc = pa::general::slice_partial(dtype, s, w, fx_mid, partials, st))) return rc;
+  }
   if ((rc = pa::general::combine_attention(s, *p, partials, plan.G, tok, norm, tok_out, st))) return rc;
   void *out_x = x_mid;
   if ((rc = pa::general::deslice(dtype, s, w, tok_out, out_x, st))) return rc;

@@ -1,0 +1,370 @@
+// Float32 front end of the structured-grid layer (PhysicsAttentionStructuredMesh2D, PA.py:744-783 with the shared
+// slice weights of PA.py:172-203): the two k x k convolutions of the input, the slice logits, the temperature
+// softmax and the partial slice-token sums in one launch.
+//
+// Shape class: C = 128 channels, 8 heads of 16, 32 slices, 2-D grid, odd k.
+//
+// The convolutions are one implicit GEMM, M = points, N = 256 (x_mid | fx_mid), K = k k 128 (tap-major), computed
+// with float32 accuracy on the bf16 matrix cores: every float32 operand is cut into three bf16 pieces
+// a = a1 + a2 + a3 (8 significant bits each, exact), and a . b is taken as the six bf16 products
+// a1 b1 + a1 b2 + a2 b1 + a2 b2 + a1 b3 + a3 b1 accumulated in float32 (the dropped products are below 2^-23 |a b|).
+// Six v_mfma_f32_32x32x16_bf16 cost 48 passes where the sixteen-times narrower v_mfma_f32_32x32x2_f32 needs 128.
+// The weights are cut once per call by split_pack_kernel into the fragment order the waves read; the activations
+// are cut in registers, once per k-step for all eight column tiles of a wave.
+//
+// Workgroup = 8 waves = 4 tiles of 32 points of one batch, two waves per tile and per SIMD: the x_mid wave owns the
+// tile's 32 x 128 x_mid outputs, the fx_mid wave its 32 x 128 fx_mid outputs (64 accumulator registers each).  Weights
+// (24 KB per k-step) and input rows (the x_mid wave fetches them for both) go from L2 into four-slot LDS rings with
+// global_load_lds, three k-steps ahead; one barrier per k-step, and the waits on the in-order counter vmcnt leave the
+// two newest groups in flight.  The x_mid tiles are computed with the weights as the A operand (lanes <-> points), the
+// fx_mid tiles with the rows as the A operand (lanes <-> channels, registers <-> points), which is the form each is
+// needed in afterwards:
+//   logits^T = W_slice x_mid^T   (float32 MFMA, lanes <-> points)   -> per-point maximum and sum in registers
+//   logits   = x_mid W_slice^T   (the same operands swapped, lanes <-> slices) -> w = exp(l / T - max) / sum
+//   tokens  += w^T fx_mid        (float32 MFMA over the 32 points, by the fx_mid wave; w crosses through LDS in the
+//                                 register layout of the A operand, one head behind the x_mid wave)
+// w leaves in natural layout (B, N, H, S) for the hand-back to the points; the token sums of the four tiles are added
+// through LDS in a fixed order and leave as one partial per workgroup, [g][b][h][S][D + 1] with the slice norm in the
+// last column (the layout slice_combine_attn_kernel sums).
+#include "pa_host.h"
+#include "pa_mfma_ops.h"
+
+namespace pa {
+namespace conv {
+
+using mfma::f32x16;
+using mfma::half_max;
+using mfma::half_sum;
+using mfma::mma;
+using mfma::rowmap;
+using mfma::u32x4;
+
+constexpr int kC = 128, kH = 8, kD = 16, kS = 32, kD1 = kD + 1;
+constexpr int kColTiles = 8;                       // 4 of x_mid, 4 of fx_mid
+constexpr int kStepsPerTap = kC / 16;              // k-steps of 16 channels
+constexpr int kStepUnits = kColTiles * 3 * 64;     // 16-byte units per k-step: 8 tiles x 3 pieces x 1 KB
+constexpr int kRing = 4;
+constexpr int kTokFloats = kH * kS * kD1;          // one partial
+// the ring, reused after the convolution for 4 token sums, 4 x 2 weight tiles in transit and the softmax statistics
+constexpr size_t kEpilogueBytes = (size_t)4 * kTokFloats * 4 + 4 * 2 * 4096 + 4 * 64 * 4;
+constexpr size_t kRingBytes = (size_t)kRing * kStepUnits * 16 + (size_t)kRing * 4 * 2048;  // weights + input rows
+constexpr size_t kLdsBytes = kRingBytes > kEpilogueBytes ? kRingBytes : kEpilogueBytes;
+
+// v = f1 + f2 + f3, each with at most 8 significant bits (exact: every difference below is representable)
+__device__ __forceinline__ void split3(float v, uint32_t (&h)[3]) {
+  const uint32_t u = __float_as_uint(v);
+  const float r1 = v - __uint_as_float(u & 0xffff0000u);
+  const uint32_t u1 = __float_as_uint(r1);
+  const float r2 = r1 - __uint_as_float(u1 & 0xffff0000u);
+  h[0] = u >> 16;
+  h[1] = u1 >> 16;
+  h[2] = __float_as_uint(r2) >> 16;
+}
+
+// blob unit ((step 8 + ct) 3 + piece) 64 + lane: the B operand (lane (i, g): output channel 32 (ct % 4) + i of weight
+// set ct / 4, k = 8 g .. 8 g + 7 of the step) of one bf16 piece.  step = tap 8 + channel block.
+__global__ __launch_bounds__(256) void split_pack_kernel(const float *__restrict__ wx, const float *__restrict__ wfx,
+                                                         u32x4 *__restrict__ blob, int taps, int tap_major) {
+  const int64_t total = (int64_t)taps * kStepsPerTap * kColTiles * 64;
+  for (int64_t u = (int64_t)blockIdx.x * 256 + threadIdx.x; u < total; u += (int64_t)gridDim.x * 256) {
+    const int lane = (int)(u & 63), ct = (int)(u >> 6) & 7, step = (int)(u >> 9);
+    const int tap = step / kStepsPerTap, c0 = (step % kStepsPerTap) * 16 + 8 * (lane >> 5);
+    const int o = 32 * (ct & 3) + (lane & 31);
+    const float *w = ct < 4 ? wx : wfx;
+    uint32_t h[8][3];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int c = c0 + e;
+      const int64_t idx = tap_major ? ((int64_t)o * taps + tap) * kC + c : ((int64_t)o * kC + c) * taps + tap;
+      split3(w[idx], h[e]);
+    }
+#pragma unroll
+    for (int pl = 0; pl < 3; ++pl) {
+      u32x4 v;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) v[q] = h[2 * q][pl] | (h[2 * q + 1][pl] << 16);
+      blob[((int64_t)step * kColTiles + ct) * 192 + pl * 64 + lane] = v;
+    }
+  }
+  if (blockIdx.x == 0 && threadIdx.x < 4) blob[total * 3 + threadIdx.x] = u32x4{0u, 0u, 0u, 0u};  // the zero page
+}
+
+// NKB KB (1 KB per instruction) from src + 16 lane to LDS byte address lds + 16 lane; the instruction offset advances
+// both addresses.  Asynchronous, counted by vmcnt.
+__device__ __forceinline__ void load_3k_to_lds(const void *sbase, unsigned lane16, unsigned lds) {
+  asm volatile(
+      "s_mov_b32 m0, %2\n\t"
+      "s_nop 0\n\t"
+      "global_load_lds_dwordx4 %1, %0\n\t"
+      "global_load_lds_dwordx4 %1, %0 offset:1024\n\t"
+      "global_load_lds_dwordx4 %1, %0 offset:2048" ::"s"(sbase),
+      "v"(lane16), "s"(lds)
+      : "memory");
+}
+
+template <class F, int... I>
+__device__ __forceinline__ void static_for_impl(F &&f, std::integer_sequence<int, I...>) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void static_for(F &&f) {
+  static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+
+__device__ __forceinline__ f32x16 mma32(float a, float b, f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
+}
+
+__global__ __launch_bounds__(512) void conv_slice_kernel(
+    const u32x4 *__restrict__ blob, const float *__restrict__ bias_x, const float *__restrict__ bias_fx,
+    const float *__restrict__ w_slice, const float *__restrict__ b_slice, const float *__restrict__ temperature,
+    const float *__restrict__ x, float *__restrict__ w_out, float *__restrict__ partials, int B, int N, int gh, int gw,
+    int ks, int bpb) {
+  extern __shared__ u32x4 smem[];
+  const int tid = threadIdx.x, lane = tid & 63, i = lane & 31, g = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int t = wave & 3;        // the wave's tile of the workgroup's four
+  const int role = wave >> 2;    // 0: the x_mid half of the columns and the slice weights, 1: fx_mid and the token sums
+  const int b = blockIdx.x / bpb, gblk = blockIdx.x - b * bpb;
+  const int n0 = (gblk * 4 + t) * 32;                    // first point of the tile (may lie past the end)
+  const int valid = min(max(N - n0, 0), 32);             // its points that exist
+  const int n = min(n0 + i, N - 1);                      // lanes past the end repeat the last point (weight 0 below)
+  const int ci = n / gw, cj = n - ci * gw;
+  const float *xb = x + (int64_t)b * N * kC + 8 * g;
+  const int pad = ks >> 1, steps = ks * ks * kStepsPerTap;
+
+  // this lane's 8 channels of the input row k-step `k` reads: the tap's neighbour, or 32 zero bytes outside the grid
+  const float *zero_page = reinterpret_cast<const float *>(blob + (int64_t)steps * kStepUnits);
+  auto row_ptr = [&](int k) -> const float * {
+    const int tap = k >> 3, c0 = (k & 7) * 16;
+    const int u = tap / ks, v = tap - u * ks;
+    const int ii = ci + u - pad, jj = cj + v - pad;
+    const bool ok = ii >= 0 && ii < gh && jj >= 0 && jj < gw;
+    return ok ? xb + (int64_t)(ii * gw + jj) * kC + c0 : zero_page;
+  };
+  // the row as three bf16 A / B operands (lane (i, g): point i, k = 8 g .. 8 g + 7)
+  auto split_row = [&](const u32x4 (&raw)[2], u32x4 (&pl)[3]) {
+    uint32_t h[8][3];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) split3(__uint_as_float(raw[e >> 2][e & 3]), h[e]);
+#pragma unroll
+    for (int p = 0; p < 3; ++p)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) pl[p][q] = h[2 * q][p] | (h[2 * q + 1][p] << 16);
+  };
+  // Group k of the memory stream: the x_mid wave's rows of k-step k (lane (i, g): point i, two 16-byte halves of its
+  // 8 channels) into the row ring, then every wave's eighth (3 KB) of the step's weights into the weight ring; both
+  // with global_load_lds, slot k % 4.  Five (x_mid wave) or three operations on the in-order counter vmcnt.
+  u32x4 *rowbuf = smem + kRing * kStepUnits + t * 128;  // + slot * 512: [half][lane]
+  auto issue_group = [&](int k, auto role_) {
+    if constexpr (decltype(role_)::value == 0) {
+      const float *p = row_ptr(k);
+      const unsigned dst = (unsigned)(uintptr_t)(rowbuf + (k % kRing) * 512);
+      asm volatile(
+          "s_mov_b32 m0, %1\n\t"
+          "s_nop 0\n\t"
+          "global_load_lds_dwordx4 %0, off" ::"v"(p), "s"(dst)
+          : "memory");
+      asm volatile(
+          "s_mov_b32 m0, %1\n\t"
+          "s_nop 0\n\t"
+          "global_load_lds_dwordx4 %0, off offset:16" ::"v"(p), "s"(dst + 1024 - 16)  // the offset moves both addresses
+          : "memory");
+    }
+    const u32x4 *src = blob + (int64_t)k * kStepUnits + wave * 192;
+    const unsigned dst = (unsigned)(uintptr_t)(smem + (k % kRing) * kStepUnits + wave * 192);
+    load_3k_to_lds(src, lane * 16, dst);
+  };
+
+  // role 0, x_mid tiles: lane (i, g) <-> point i, register r <-> channel 32 ct + rowmap(r, g)
+  // role 1, fx_mid tiles: lane (i, g) <-> channel 32 ct + i, register r <-> point rowmap(r, g)
+  f32x16 acc[4];
+  // the k-steps, compiled once per role so that neither carries the other's operand order
+  auto convolve = [&](auto role_) {
+    constexpr int ROLE = decltype(role_)::value;
+#pragma unroll
+    for (int ct = 0; ct < 4; ++ct)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        if constexpr (ROLE == 0) acc[ct][r] = bias_x ? bias_x[32 * ct + rowmap(r, g)] : 0.f;
+        else acc[ct][r] = bias_fx ? bias_fx[32 * ct + i] : 0.f;
+      }
+    u32x4 raw[2], cur[3], nxt[3];
+    issue_group(0, role_);
+    issue_group(1, role_);
+    issue_group(2, role_);
+    // vmcnt(0), as the builtin so that the compiler too knows the bias loads above are complete (it would otherwise
+    // wait for them, and with them for everything in flight, at their first use inside the loop)
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    __syncthreads();
+    raw[0] = rowbuf[lane];
+    raw[1] = rowbuf[64 + lane];
+    split_row(raw, cur);
+    for (int s = 0; s < steps; ++s) {
+      // Groups up to s + 2 are issued.  Step s needs the weights of group s and, for the split below, the rows of
+      // group s + 1: the rest of group s + 1 and group s + 2 may stay in flight (3 + 5 operations of an x_mid wave,
+      // 3 + 3 of an fx_mid wave).  Each wave waits for its own share, then all meet; the slots of step s - 1 are free
+      // once every wave is here.
+      if (s + 2 < steps) {
+        if constexpr (ROLE == 0) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+        else asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
+      } else {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      }
+      __syncthreads();
+      if (s + 1 < steps) {
+        const u32x4 *rb = rowbuf + ((s + 1) % kRing) * 512 + lane;
+        raw[0] = rb[0];
+        raw[1] = rb[64];
+      }
+      if (s + 3 < steps) issue_group(s + 3, role_);
+      const u32x4 *wb = smem + (s % kRing) * kStepUnits + ROLE * (4 * 192) + lane;
+      u32x4 fr[4][3];
+#pragma unroll
+      for (int ct = 0; ct < 4; ++ct)
+#pragma unroll
+        for (int p = 0; p < 3; ++p) fr[ct][p] = wb[(ct * 3 + p) * 64];
+      // the six products, the four column tiles taking turns
+      auto product = [&](int pw, int pa) {
+#pragma unroll
+        for (int ct = 0; ct < 4; ++ct) {
+          if constexpr (ROLE == 0) acc[ct] = mma(fr[ct][pw], cur[pa], acc[ct]);
+          else acc[ct] = mma(cur[pa], fr[ct][pw], acc[ct]);
+        }
+      };
+      product(0, 0);
+      product(1, 0);
+      if (s + 1 < steps) split_row(raw, nxt);
+      product(0, 1);
+      product(1, 1);
+      product(2, 0);
+      product(0, 2);
+#pragma unroll
+      for (int p = 0; p < 3; ++p) cur[p] = nxt[p];
+    }
+  };
+  if (role == 0) convolve(std::integral_constant<int, 0>{});
+  else convolve(std::integral_constant<int, 1>{});
+  __syncthreads();  // the ring is free: it now holds the token sums, the weights in transit and the softmax statistics
+
+  float *red = reinterpret_cast<float *>(smem);                     // [tile][h][s][D + 1]
+  float *mine = red + t * kTokFloats;
+  u32x4 *xchg = smem + (4 * kTokFloats) / 4 + t * (2 * 256);        // [tile][buffer][q][lane]: one head's weights
+  float *stat = reinterpret_cast<float *>(smem + (4 * kTokFloats) / 4 + 4 * 2 * 256) + t * 64;  // [max | 1 / sum][point]
+  // W_slice[s][d] for MFMA m of a head: this lane's channel of the pair (k = g) is d = 8 (m / 4) + 4 g + m % 4, the
+  // channel the x_mid registers hold in that position
+  float ws[8], bs_r[16];
+#pragma unroll
+  for (int m = 0; m < 8; ++m) ws[m] = w_slice[i * kD + rowmap(m, g)];
+#pragma unroll
+  for (int r = 0; r < 16; ++r) bs_r[r] = b_slice ? b_slice[rowmap(r, g)] : 0.f;
+  const float bs_i = b_slice ? b_slice[i] : 0.f;
+  float *wrow = w_out + ((int64_t)b * N + n0) * (kH * kS) + i;
+
+  // round h: the x_mid wave makes head h's weights and leaves them in LDS; the fx_mid wave sums head h - 1's tokens
+  static_for<kH + 1>([&](auto h_) {
+    constexpr int hh = decltype(h_)::value;
+    if (role == 0 && hh < kH) {
+      constexpr int h = hh < kH ? hh : 0, ct = h / 2, half = h % 2;
+      const float inv_t = temperature ? kLog2e / clamp_temperature(temperature[h]) : kLog2e;
+      // lanes <-> points: the head's softmax statistics
+      f32x16 lt;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) lt[r] = bs_r[r];
+#pragma unroll
+      for (int m = 0; m < 8; ++m) lt = mma32(ws[m], acc[ct][8 * half + m], lt);
+      float mx = lt[0] * inv_t;
+#pragma unroll
+      for (int r = 1; r < 16; ++r) mx = fmaxf(mx, lt[r] * inv_t);
+      mx = half_max(mx);
+      float sum = 0.f;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) sum += __builtin_amdgcn_exp2f(lt[r] * inv_t - mx);
+      sum = half_sum(sum);
+      if (g == 0) {
+        stat[i] = mx;
+        stat[32 + i] = 1.f / sum;
+      }
+      __builtin_amdgcn_wave_barrier();
+      // lanes <-> slices, register r <-> point rowmap(r, g): the weights, as the A operand of the token sums
+      f32x16 ln;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) ln[r] = bs_i;
+#pragma unroll
+      for (int m = 0; m < 8; ++m) ln = mma32(acc[ct][8 * half + m], ws[m], ln);
+      float nrm = 0.f;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const float4 mq = *reinterpret_cast<const float4 *>(stat + 8 * q + 4 * g);
+        const float4 iq = *reinterpret_cast<const float4 *>(stat + 32 + 8 * q + 4 * g);
+        const float mqa[4] = {mq.x, mq.y, mq.z, mq.w}, iqa[4] = {iq.x, iq.y, iq.z, iq.w};
+        u32x4 out;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int r = 4 * q + e, pt = 8 * q + 4 * g + e;
+          float wv = __builtin_amdgcn_exp2f(ln[r] * inv_t - mqa[e]) * iqa[e];
+          if (pt >= valid) wv = 0.f;
+          else wrow[(int64_t)pt * (kH * kS) + h * kS] = wv;
+          out[e] = __float_as_uint(wv);
+          nrm += wv;
+        }
+        xchg[(h & 1) * 256 + q * 64 + lane] = out;
+      }
+      __builtin_amdgcn_wave_barrier();
+      nrm = half_sum(nrm);
+      if (g == 0) mine[h * (kS * kD1) + i * kD1 + kD] = nrm;
+    }
+    if (role == 1 && hh > 0) {
+      constexpr int h = hh > 0 ? hh - 1 : 0, ct = h / 2, half = h % 2;
+      f32x16 tk;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) tk[r] = 0.f;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const u32x4 wq = xchg[(h & 1) * 256 + q * 64 + lane];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) tk = mma32(__uint_as_float(wq[e]), acc[ct][4 * q + e], tk);
+      }
+      // lane (i, g): channel 32 ct + i of fx_mid, register r <-> slice rowmap(r, g); the head's 16 channels are kept
+      if ((i >> 4) == half) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) mine[h * (kS * kD1) + rowmap(r, g) * kD1 + (i & 15)] = tk[r];
+      }
+    }
+    __syncthreads();
+  });
+  float *dst = partials + ((int64_t)gblk * B + b) * kTokFloats;
+  for (int idx = tid; idx < kTokFloats; idx += 512)
+    dst[idx] = ((red[idx] + red[kTokFloats + idx]) + red[2 * kTokFloats + idx]) + red[3 * kTokFloats + idx];
+}
+
+bool supported(int dtype, const pa_shape &s) {
+  return dtype == PA_F32 && s.conv_k > 0 && s.conv_k % 2 == 1 && s.grid_d == 0 && s.C == kC && s.H == kH && s.D == kD &&
+         s.S == kS && s.grid_h * s.grid_w == s.N && s.N * kC < (int64_t)1 << 29;
+}
+
+int64_t groups(const pa_shape &s) { return ((s.N + 31) / 32 + 3) / 4; }
+
+int64_t blob_bytes(const pa_shape &s) { return s.conv_k * s.conv_k * kStepsPerTap * (int64_t)kStepUnits * 16 + 64; }
+
+int front(const pa_shape &s, const pa_params &p, const void *x, void *blob, void *w, float *partials, hipStream_t st) {
+  if (!supported(PA_F32, s)) return PA_ERR_UNSUPPORTED;
+  const int taps = (int)(s.conv_k * s.conv_k);
+  const int64_t units = (int64_t)taps * kStepsPerTap * kColTiles * 64;
+  hipLaunchKernelGGL(split_pack_kernel, dim3((unsigned)((units + 255) / 256)), dim3(256), 0, st,
+                     static_cast<const float *>(p.in_project_x_weight), static_cast<const float *>(p.in_project_fx_weight),
+                     static_cast<u32x4 *>(blob), taps, (int)s.conv_tap_major);
+  int rc = launch_status();
+  if (rc) return rc;
+  if ((rc = allow_dynamic_lds(conv_slice_kernel, kLdsBytes))) return rc;
+  const int bpb = (int)groups(s);
+  hipLaunchKernelGGL(conv_slice_kernel, dim3((unsigned)(s.B * bpb)), dim3(512), kLdsBytes, st,
+                     static_cast<const u32x4 *>(blob), p.in_project_x_bias, p.in_project_fx_bias,
+                     static_cast<const float *>(p.in_project_slice_weight), p.in_project_slice_bias, p.temperature,
+                     static_cast<const float *>(x), static_cast<float *>(w), partials, (int)s.B, (int)s.N,
+                     (int)s.grid_h, (int)s.grid_w, (int)s.conv_k, bpb);
+  return launch_status();
+}
+
+}  // namespace conv
+}  // namespace pa

@@ -104,6 +104,16 @@ int layernorm_backward(int dtype, int64_t rows, int64_t C, const void *x, const 
                        void *dx, float *partials, hipStream_t st);
 }  // namespace general
 
+namespace conv {
+// float32 structured 2-D front end (C = 128, 8 heads of 16, 32 slices): both convolutions on split-bf16 MFMA products,
+// slice softmax and partial token sums in one launch.  `w`: (B, N, H, S) float32; `partials`: groups(s) partials of
+// B * H * S * (D + 1) floats each, in the layout the general combine kernels read.
+bool supported(int dtype, const pa_shape &s);
+int64_t groups(const pa_shape &s);
+int64_t blob_bytes(const pa_shape &s);
+int front(const pa_shape &s, const pa_params &p, const void *x, void *blob, void *w, float *partials, hipStream_t st);
+}  // namespace conv
+
 namespace backward {
 size_t attention_lds_bytes(const pa_shape &s);
 int slice_attention(const pa_shape &s, const pa_params &p, const float *slice_token, const float *slice_norm,

@@ -51,6 +51,32 @@ def test_fp32_structured2d_stages_and_layer(kernel, grid):
     assert_fp32_close(y, want["y"], "layer y")
 
 
+@pytest.mark.parametrize("kernel,grid,B", [(1, (9, 14), 2), (3, (13, 11), 3), (3, (40, 37), 2), (5, (16, 23), 1),
+                                           (3, (85, 85), 1)])
+def test_fp32_structured2d_fused_front_end(kernel, grid, B):
+    # C = 128, 8 heads of 16, 32 slices: the layer call runs the fused front end (both convolutions as split-bf16 MFMA
+    # products, slice softmax and partial token sums in one launch); the stage API runs the float32-MFMA kernels.
+    # Grids with ragged last tiles (126, 143 points), workgroups with idle waves (143 points: 5 tiles) and cfg1's grid.
+    announce("fp32 structured2d fused front end", kernel, grid, B)
+    dim, heads, dim_head, S = 128, 8, 16, 32
+    ref, hip = make_pair("structured2d", dim, heads, dim_head, S, spatial=grid, kernel=kernel, sharpen=2.0,
+                         temps=[0.3 + 5.7 * i / 7 for i in range(8)])
+    x = torch.randn(B, grid[0] * grid[1], dim)
+    with torch.no_grad():
+        want = ref.stages(x)
+        want64 = ref.double().stages(x.double())["y"]
+        staged = hip.forward_stages(x.cuda())["y"]
+        y = hip(x.cuda())
+    assert_fp32_close(y, want["y"], "layer y")
+    # against the float64 run of the oracle the split products are as close as the float32 matrix instructions
+    e_fused, e_staged = to.rel_l2(y.double().cpu(), want64), to.rel_l2(staged.double().cpu(), want64)
+    import conftest
+
+    conftest.MEASURED.append((f"structured 2D fp32 layer vs float64 oracle, k={kernel} grid={grid}: fused front end "
+                              f"(split-bf16 products); stage kernels (fp32 MFMA) {e_staged:.2e}", e_fused, 2e-6))
+    assert e_fused < 2e-6 and e_fused < 4 * e_staged + 2e-7
+
+
 @pytest.mark.parametrize("kernel,grid", [(3, (4, 4, 4)), (3, (8, 8, 8)), (5, (8, 8, 8)), (3, (3, 5, 7)), (1, (4, 6, 5))])
 def test_fp32_structured3d_stages_and_layer(kernel, grid):
     announce("fp32 structured3d", kernel, grid)
