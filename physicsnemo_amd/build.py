@@ -15,7 +15,7 @@ CSRC = os.path.join(PKG_DIR, "csrc")
 OBJ_DIR = os.path.join(CSRC, "build")
 LIB_PATH = os.path.join(PKG_DIR, "libphysattn.so")
 SOURCES = ["pa_api.hip", "pa_general.hip", "pa_mfma.hip", "pa_mlp.hip", "pa_backward.hip", "pa_gemm.hip", "pa_mfma_bwd.hip",
-           "pa_mfma_staged.hip", "pa_gale.hip", "pa_flare.hip", "pa_ball_query.hip", "pa_noalloc.hip", "pa_conv.hip"]
+           "pa_mfma_staged.hip", "pa_gale.hip", "pa_flare.hip", "pa_ball_query.hip", "pa_noalloc.hip", "pa_conv.hip", "pa_rows_f32.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",

@@ -42,6 +42,8 @@ struct GeneralPlan {
   int64_t off_x_mid, off_fx_mid, off_w, off_partials, off_tok, off_norm, off_tok_out, off_blob, total;
   int64_t G;
   bool conv_front;  // float32 structured 2-D layer of the fused front end's shape class
+  bool rows_back;   // float32 layer whose hand-back, out_linear and tail run in the row kernel
+  int64_t off_blob_out;
 };
 
 GeneralPlan plan_general(int dtype, const pa_shape &s) {
@@ -66,6 +68,9 @@ GeneralPlan plan_general(int dtype, const pa_shape &s) {
   off += round_up(s.B * s.H * s.S * s.D * 4, 256);
   p.off_blob = off;  // the convolution weights cut into bf16 pieces, in fragment order
   if (p.conv_front) off += round_up(pa::conv::blob_bytes(s), 256);
+  p.rows_back = pa::f32rows::backend_supported(dtype, s);
+  p.off_blob_out = off;  // out_linear's weight in the same form
+  if (p.rows_back) off += round_up(pa::f32rows::backend_blob_bytes(), 256);
   p.total = off;
   return p;
 }
@@ -823,32 +828,44 @@ int pa_mfma_deslice_project(const pa_shape *shape, const void *blob, const void 
                                    static_cast<hipStream_t>(stream));
 }
 
-int pa_mlp_query(int dtype, int64_t rows, int64_t C, int64_t F) { return pa::mlp::supported(dtype, rows, C, F) ? 1 : 0; }
+// float32 at C = 128 runs the split-bf16 row kernel, bf16 the MFMA kernels of pa_mlp.hip
+static bool mlp_served(int dtype, int64_t rows, int64_t C, int64_t F) {
+  return pa::mlp::supported(dtype, rows, C, F) || pa::f32rows::mlp_supported(dtype, rows, C, F);
+}
+static int64_t mlp_blob_bytes(int dtype, int64_t C, int64_t F) {
+  return dtype == PA_F32 ? pa::f32rows::mlp_blob_bytes(F) : pa::mlp::blob_bytes(C, F);
+}
+
+int pa_mlp_query(int dtype, int64_t rows, int64_t C, int64_t F) { return mlp_served(dtype, rows, C, F) ? 1 : 0; }
 
 int64_t pa_mlp_workspace_bytes(int dtype, int64_t rows, int64_t C, int64_t F) {
   if (rows <= 0 || C <= 0 || F <= 0) return PA_ERR_DIMS;
-  if (!pa::mlp::supported(dtype, rows, C, F)) return PA_ERR_UNSUPPORTED;
-  return round_up(pa::mlp::blob_bytes(C, F), 256);
+  if (!mlp_served(dtype, rows, C, F)) return PA_ERR_UNSUPPORTED;
+  return round_up(mlp_blob_bytes(dtype, C, F), 256);
 }
 
 int pa_mlp_pack(int dtype, int64_t C, int64_t F, const pa_mlp_params *p, void *packed, int64_t packed_bytes,
                 void *stream) {
   if (C <= 0 || F <= 0) return PA_ERR_DIMS;
-  if (!pa::mlp::supported(dtype, 1, C, F)) return PA_ERR_UNSUPPORTED;
+  if (!mlp_served(dtype, 1, C, F)) return PA_ERR_UNSUPPORTED;
   if (!p || !p->w1 || !p->w2 || !packed) return PA_ERR_NULL;
   if (!aligned16(p->w1) || !aligned16(p->w2) || !aligned16(packed)) return PA_ERR_ALIGN;
-  if (packed_bytes < pa::mlp::blob_bytes(C, F)) return PA_ERR_WORKSPACE;
+  if (packed_bytes < mlp_blob_bytes(dtype, C, F)) return PA_ERR_WORKSPACE;
+  if (dtype == PA_F32) return pa::f32rows::mlp_pack(F, p->w1, p->w2, packed, static_cast<hipStream_t>(stream));
   return pa::mlp::pack(C, F, p->w1, p->w2, packed, static_cast<hipStream_t>(stream));
 }
 
 int pa_mlp_forward_packed(int dtype, int64_t rows, int64_t C, int64_t F, const void *packed, const float *b1,
                           const float *b2, const void *u, void *y, const pa_block_tail *tail, void *stream) {
   if (rows <= 0 || C <= 0 || F <= 0) return PA_ERR_DIMS;
-  if (!pa::mlp::supported(dtype, rows, C, F)) return PA_ERR_UNSUPPORTED;
+  if (!mlp_served(dtype, rows, C, F)) return PA_ERR_UNSUPPORTED;
   if (!packed || !b1 || !b2 || !u || !y) return PA_ERR_NULL;
   if (!aligned16(packed) || !aligned16(u) || !aligned16(y)) return PA_ERR_ALIGN;
   int rc = check_tail(tail);
   if (rc) return rc;
+  if (dtype == PA_F32)
+    return pa::f32rows::mlp_forward(rows, F, packed, b1, b2, u, y, tail_active(tail) ? tail : nullptr,
+                                    static_cast<hipStream_t>(stream));
   return pa::mlp::forward(rows, C, F, packed, b1, b2, u, y, tail_active(tail) ? tail : nullptr, compute_units(),
                           static_cast<hipStream_t>(stream));
 }
@@ -856,14 +873,18 @@ int pa_mlp_forward_packed(int dtype, int64_t rows, int64_t C, int64_t F, const v
 int pa_mlp_forward(int dtype, int64_t rows, int64_t C, int64_t F, const pa_mlp_params *p, const void *u, void *y,
                    const pa_block_tail *tail, void *workspace, int64_t workspace_bytes, void *stream) {
   if (rows <= 0 || C <= 0 || F <= 0) return PA_ERR_DIMS;
-  if (!pa::mlp::supported(dtype, rows, C, F)) return PA_ERR_UNSUPPORTED;
+  if (!mlp_served(dtype, rows, C, F)) return PA_ERR_UNSUPPORTED;
   if (!p || !p->w1 || !p->b1 || !p->w2 || !p->b2 || !u || !y || !workspace) return PA_ERR_NULL;
   if (!aligned16(p->w1) || !aligned16(p->w2) || !aligned16(u) || !aligned16(y) || !aligned16(workspace))
     return PA_ERR_ALIGN;
   int rc = check_tail(tail);
   if (rc) return rc;
-  if (workspace_bytes < pa::mlp::blob_bytes(C, F)) return PA_ERR_WORKSPACE;
+  if (workspace_bytes < mlp_blob_bytes(dtype, C, F)) return PA_ERR_WORKSPACE;
   hipStream_t st = static_cast<hipStream_t>(stream);
+  if (dtype == PA_F32) {
+    if ((rc = pa::f32rows::mlp_pack(F, p->w1, p->w2, workspace, st))) return rc;
+    return pa::f32rows::mlp_forward(rows, F, workspace, p->b1, p->b2, u, y, tail_active(tail) ? tail : nullptr, st);
+  }
   if ((rc = pa::mlp::pack(C, F, p->w1, p->w2, workspace, st))) return rc;
   return pa::mlp::forward(rows, C, F, workspace, p->b1, p->b2, u, y, tail_active(tail) ? tail : nullptr, compute_units(),
                           st);
@@ -1000,6 +1021,8 @@ int pa_layer_forward(int dtype, const pa_shape *shape, const pa_params *p, const
     if ((rc = pa::general::slice_partial(dtype, s, w, fx_mid, partials, st))) return rc;
   }
   if ((rc = pa::general::combine_attention(s, *p, partials, plan.G, tok, norm, tok_out, st))) return rc;
+  if (plan.rows_back)  // hand-back, out_linear, residual and LayerNorm in one launch
+    return pa::f32rows::backend(s, *p, w, tok_out, y, tail_active(tail) ? tail : nullptr, ws + plan.off_blob_out, st);
   void *out_x = x_mid;
   if ((rc = pa::general::deslice(dtype, s, w, tok_out, out_x, st))) return rc;
   if ((rc = pa::general::out_linear(dtype, s, *p, out_x, y, st))) return rc;

@@ -28,6 +28,7 @@
 // last column (the layout slice_combine_attn_kernel sums).
 #include "pa_host.h"
 #include "pa_mfma_ops.h"
+#include "pa_split_ops.h"
 
 namespace pa {
 namespace conv {
@@ -38,6 +39,7 @@ using mfma::half_sum;
 using mfma::mma;
 using mfma::rowmap;
 using mfma::u32x4;
+using namespace split;
 
 constexpr int kC = 128, kH = 8, kD = 16, kS = 32, kD1 = kD + 1;
 constexpr int kColTiles = 8;                       // 4 of x_mid, 4 of fx_mid
@@ -49,17 +51,6 @@ constexpr int kTokFloats = kH * kS * kD1;          // one partial
 constexpr size_t kEpilogueBytes = (size_t)4 * kTokFloats * 4 + 4 * 2 * 4096 + 4 * 64 * 4;
 constexpr size_t kRingBytes = (size_t)kRing * kStepUnits * 16 + (size_t)kRing * 4 * 2048;  // weights + input rows
 constexpr size_t kLdsBytes = kRingBytes > kEpilogueBytes ? kRingBytes : kEpilogueBytes;
-
-// v = f1 + f2 + f3, each with at most 8 significant bits (exact: every difference below is representable)
-__device__ __forceinline__ void split3(float v, uint32_t (&h)[3]) {
-  const uint32_t u = __float_as_uint(v);
-  const float r1 = v - __uint_as_float(u & 0xffff0000u);
-  const uint32_t u1 = __float_as_uint(r1);
-  const float r2 = r1 - __uint_as_float(u1 & 0xffff0000u);
-  h[0] = u >> 16;
-  h[1] = u1 >> 16;
-  h[2] = __float_as_uint(r2) >> 16;
-}
 
 // blob unit ((step 8 + ct) 3 + piece) 64 + lane: the B operand (lane (i, g): output channel 32 (ct % 4) + i of weight
 // set ct / 4, k = 8 g .. 8 g + 7 of the step) of one bf16 piece.  step = tap 8 + channel block.
@@ -87,32 +78,6 @@ __global__ __launch_bounds__(256) void split_pack_kernel(const float *__restrict
     }
   }
   if (blockIdx.x == 0 && threadIdx.x < 4) blob[total * 3 + threadIdx.x] = u32x4{0u, 0u, 0u, 0u};  // the zero page
-}
-
-// NKB KB (1 KB per instruction) from src + 16 lane to LDS byte address lds + 16 lane; the instruction offset advances
-// both addresses.  Asynchronous, counted by vmcnt.
-__device__ __forceinline__ void load_3k_to_lds(const void *sbase, unsigned lane16, unsigned lds) {
-  asm volatile(
-      "s_mov_b32 m0, %2\n\t"
-      "s_nop 0\n\t"
-      "global_load_lds_dwordx4 %1, %0\n\t"
-      "global_load_lds_dwordx4 %1, %0 offset:1024\n\t"
-      "global_load_lds_dwordx4 %1, %0 offset:2048" ::"s"(sbase),
-      "v"(lane16), "s"(lds)
-      : "memory");
-}
-
-template <class F, int... I>
-__device__ __forceinline__ void static_for_impl(F &&f, std::integer_sequence<int, I...>) {
-  (f(std::integral_constant<int, I>{}), ...);
-}
-template <int N, class F>
-__device__ __forceinline__ void static_for(F &&f) {
-  static_for_impl(f, std::make_integer_sequence<int, N>{});
-}
-
-__device__ __forceinline__ f32x16 mma32(float a, float b, f32x16 c) {
-  return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
 }
 
 __global__ __launch_bounds__(512) void conv_slice_kernel(
@@ -190,57 +155,77 @@ __global__ __launch_bounds__(512) void conv_slice_kernel(
         else acc[ct][r] = bias_fx ? bias_fx[32 * ct + i] : 0.f;
       }
     u32x4 raw[2], cur[3], nxt[3];
+    u32x4 fr[2][4][3];  // the weight fragments of the even / the odd k-steps
+    auto read_rows = [&](int k) {
+      const u32x4 *rb = rowbuf + (k % kRing) * 512 + lane;
+      raw[0] = rb[0];
+      raw[1] = rb[64];
+    };
+    auto read_fragments = [&](int k, u32x4 (&f)[4][3]) {
+      const u32x4 *wb = smem + (k % kRing) * kStepUnits + ROLE * (4 * 192) + lane;
+#pragma unroll
+      for (int ct = 0; ct < 4; ++ct)
+#pragma unroll
+        for (int p = 0; p < 3; ++p) f[ct][p] = wb[(ct * 3 + p) * 64];
+    };
     issue_group(0, role_);
     issue_group(1, role_);
     issue_group(2, role_);
+    issue_group(3, role_);
     // vmcnt(0), as the builtin so that the compiler too knows the bias loads above are complete (it would otherwise
     // wait for them, and with them for everything in flight, at their first use inside the loop)
     __builtin_amdgcn_s_waitcnt(0x0F70);
     __syncthreads();
-    raw[0] = rowbuf[lane];
-    raw[1] = rowbuf[64 + lane];
+    read_rows(0);
+    read_fragments(0, fr[0]);
     split_row(raw, cur);
-    for (int s = 0; s < steps; ++s) {
-      // Groups up to s + 2 are issued.  Step s needs the weights of group s and, for the split below, the rows of
-      // group s + 1: the rest of group s + 1 and group s + 2 may stay in flight (3 + 5 operations of an x_mid wave,
-      // 3 + 3 of an fx_mid wave).  Each wave waits for its own share, then all meet; the slots of step s - 1 are free
-      // once every wave is here.
-      if (s + 2 < steps) {
-        if constexpr (ROLE == 0) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
-        else asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
-      } else {
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-      }
-      __syncthreads();
-      if (s + 1 < steps) {
-        const u32x4 *rb = rowbuf + ((s + 1) % kRing) * 512 + lane;
-        raw[0] = rb[0];
-        raw[1] = rb[64];
-      }
-      if (s + 3 < steps) issue_group(s + 3, role_);
-      const u32x4 *wb = smem + (s % kRing) * kStepUnits + ROLE * (4 * 192) + lane;
-      u32x4 fr[4][3];
-#pragma unroll
-      for (int ct = 0; ct < 4; ++ct)
-#pragma unroll
-        for (int p = 0; p < 3; ++p) fr[ct][p] = wb[(ct * 3 + p) * 64];
-      // the six products, the four column tiles taking turns
-      auto product = [&](int pw, int pa) {
-#pragma unroll
-        for (int ct = 0; ct < 4; ++ct) {
-          if constexpr (ROLE == 0) acc[ct] = mma(fr[ct][pw], cur[pa], acc[ct]);
-          else acc[ct] = mma(cur[pa], fr[ct][pw], acc[ct]);
+    for (int s2 = 0; s2 < steps; s2 += 2) {
+      static_for<2>([&](auto par_) {
+        constexpr int par = decltype(par_)::value;
+        const int s = s2 + par;
+        // Groups up to s + 3 are issued.  This step multiplies the fragments and rows of step s, read from LDS one
+        // step ago, and reads those of step s + 1: group s + 1 must have landed, groups s + 2 and s + 3 may stay in
+        // flight (5 operations each for an x_mid wave, 3 for an fx_mid wave).  Each wave waits for its own share, then
+        // all meet; the slots of step s, read one step ago, are free once every wave is here.
+        constexpr int G = ROLE == 0 ? 5 : 3;
+        if (s + 3 < steps) {
+          if constexpr (G == 5) asm volatile("s_waitcnt vmcnt(10)" ::: "memory");
+          else asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
+        } else if (s + 2 < steps) {
+          if constexpr (G == 5) asm volatile("s_waitcnt vmcnt(5)" ::: "memory");
+          else asm volatile("s_waitcnt vmcnt(3)" ::: "memory");
+        } else {
+          asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         }
-      };
-      product(0, 0);
-      product(1, 0);
-      if (s + 1 < steps) split_row(raw, nxt);
-      product(0, 1);
-      product(1, 1);
-      product(2, 0);
-      product(0, 2);
+        __syncthreads();
+        // the six products, the four column tiles taking turns; the step's other work (the next group's loads, the
+        // next step's LDS reads and split) is spread between them so that it issues while the matrix core is busy
+        auto product = [&](int pw, int pa) {
 #pragma unroll
-      for (int p = 0; p < 3; ++p) cur[p] = nxt[p];
+          for (int ct = 0; ct < 4; ++ct) {
+            if constexpr (ROLE == 0) acc[ct] = mma(fr[par][ct][pw], cur[pa], acc[ct]);
+            else acc[ct] = mma(cur[pa], fr[par][ct][pw], acc[ct]);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        };
+        product(0, 0);
+        if (s + 4 < steps) issue_group(s + 4, role_);
+        __builtin_amdgcn_sched_barrier(0);
+        product(1, 0);
+        if (s + 1 < steps) {
+          read_rows(s + 1);
+          read_fragments(s + 1, fr[1 - par]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        product(0, 1);
+        if (s + 1 < steps) split_row(raw, nxt);
+        __builtin_amdgcn_sched_barrier(0);
+        product(1, 1);
+        product(2, 0);
+        product(0, 2);
+#pragma unroll
+        for (int p = 0; p < 3; ++p) cur[p] = nxt[p];
+      });
     }
   };
   if (role == 0) convolve(std::integral_constant<int, 0>{});

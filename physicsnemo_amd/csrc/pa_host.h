@@ -114,6 +114,22 @@ int64_t blob_bytes(const pa_shape &s);
 int front(const pa_shape &s, const pa_params &p, const void *x, void *blob, void *w, float *partials, hipStream_t st);
 }  // namespace conv
 
+namespace f32rows {
+// float32 per-point kernels of a 128-wide block on split-bf16 products.  backend: out_x = w . out_token per head
+// (8 heads of 16, 32 slices; w (B, N, H, S), out_token (B, H, S, D)), y = out_x W_out^T + b_out and the tail, one
+// launch; blob: backend_blob_bytes() of scratch for the repacked W_out.  mlp_*: Mlp(128 -> F -> 128), F a multiple of
+// 128, with the same tail; blob: mlp_blob_bytes(F) written by mlp_pack.
+bool backend_supported(int dtype, const pa_shape &s);
+int64_t backend_blob_bytes();
+int backend(const pa_shape &s, const pa_params &p, const void *w, const float *out_token, void *y,
+            const pa_block_tail *tail, void *blob, hipStream_t st);
+bool mlp_supported(int dtype, int64_t rows, int64_t C, int64_t F);
+int64_t mlp_blob_bytes(int64_t F);
+int mlp_pack(int64_t F, const void *w1, const void *w2, void *blob, hipStream_t st);
+int mlp_forward(int64_t rows, int64_t F, const void *blob, const float *b1, const float *b2, const void *u, void *y,
+                const pa_block_tail *tail, hipStream_t st);
+}  // namespace f32rows
+
 namespace backward {
 size_t attention_lds_bytes(const pa_shape &s);
 int slice_attention(const pa_shape &s, const pa_params &p, const float *slice_token, const float *slice_norm,

@@ -1,0 +1,373 @@
+// Float32 per-point kernels of a 128-wide block, on split-bf16 products (pa_split_ops.h):
+//   deslice_linear_kernel  the layer's way back to the points (PA.py:467-499): out_x = w . out_token per head,
+//                          y = out_x W_out^T + b_out, then the caller's residual and LayerNorm (TR.py:300-303)
+//   mlp_kernel             the block's MLP (mlp_layers.py:139-173, TR.py:301-307): y = W2 gelu(W1 u + b1) + b2 with the
+//                          same tail
+// Shape class: C = 128 channels (8 heads of 16, 32 slices for the hand-back), F a multiple of 128.
+//
+// Workgroup = 4 waves, a wave owns a tile of 32 rows and keeps every intermediate transposed: lane (i, g) <-> row i,
+// accumulator register r of column tile t <-> channel 32 t + rowmap(r, g).  A product Y^T = W X^T takes the weight as
+// the A operand and the rows as the B operand; the result, cut into bf16 pieces, is the B operand of the next product
+// provided that product's weight is packed with its reduction index in the order the registers hold the channels
+// (kperm).  So deslice -> out_linear and Linear -> GELU -> Linear run without the rows leaving the registers, and the
+// residual + LayerNorm tail is a sum over a lane's 64 registers and its partner lane.
+//
+// Weights are cut into pieces once (pack kernels) as units of 12 KB = one k-step (16 reduction indices) of 128 output
+// rows: [tile 0..3][piece 0..2][lane], and reach LDS with global_load_lds.
+#include "pa_host.h"
+#include "pa_mfma_ops.h"
+#include "pa_split_ops.h"
+
+namespace pa {
+namespace f32rows {
+
+using mfma::f32x16;
+using mfma::half_sum;
+using mfma::kperm;
+using mfma::mma;
+using mfma::rowmap;
+using mfma::u32x4;
+using namespace split;
+
+constexpr int kC = 128, kH = 8, kD = 16, kS = 32;
+constexpr int kUnit = 4 * 3 * 64;  // 16-byte elements of a weight unit (12 KB)
+
+// One unit of a 128-row block of a float32 weight: thread `v` (0 .. 255) packs tile v / 64, lane v % 64 = (i, g):
+// row 32 tile + i, reduction indices k0 + 8 g + j (natural) or k0 rounded down to 32 + kperm((k0 / 16) % 2, g, j).
+__device__ __forceinline__ void pack_unit(const float *w, int64_t ld, int k0, bool permuted, u32x4 *unit, int v) {
+  const int ot = v >> 6, lane = v & 63, i = lane & 31, g = lane >> 5;
+  const float *row = w + (int64_t)(32 * ot + i) * ld;
+  float e[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) e[j] = row[permuted ? (k0 & ~31) + kperm((k0 >> 4) & 1, g, j) : k0 + 8 * g + j];
+  u32x4 pl[3];
+  split8(e, pl);
+#pragma unroll
+  for (int p = 0; p < 3; ++p) unit[(ot * 3 + p) * 64 + lane] = pl[p];
+}
+
+// W (128, K) -> K / 16 units
+__global__ __launch_bounds__(256) void pack_linear_kernel(const float *__restrict__ w, int K, int permuted,
+                                                          u32x4 *__restrict__ blob) {
+  pack_unit(w, K, 16 * blockIdx.x, permuted != 0, blob + (int64_t)blockIdx.x * kUnit, threadIdx.x);
+}
+
+// Mlp weights W1 (F, 128), W2 (128, F) -> per chunk of 128 hidden features 8 units of W1's rows (natural order) and
+// 8 units of W2's columns (permuted: the hidden features arrive as accumulator registers)
+__global__ __launch_bounds__(256) void pack_mlp_kernel(const float *__restrict__ w1, const float *__restrict__ w2, int F,
+                                                       u32x4 *__restrict__ blob) {
+  const int c = blockIdx.x >> 4, u = blockIdx.x & 15;
+  u32x4 *unit = blob + (int64_t)blockIdx.x * kUnit;
+  if (u < 8) pack_unit(w1 + (int64_t)c * 128 * kC, kC, 16 * u, false, unit, threadIdx.x);
+  else pack_unit(w2 + c * 128, F, 16 * (u - 8), true, unit, threadIdx.x);
+}
+
+// acc[t] += unit's tile t (A operand) . rows (B operand bp): the six products, the four tiles taking turns
+__device__ __forceinline__ void kstep(f32x16 (&acc)[4], const u32x4 *unit_lane, const u32x4 (&bp)[3]) {
+  u32x4 fr[4][3];
+#pragma unroll
+  for (int t = 0; t < 4; ++t)
+#pragma unroll
+    for (int p = 0; p < 3; ++p) fr[t][p] = unit_lane[(t * 3 + p) * 64];
+  constexpr int pw[6] = {0, 1, 0, 1, 2, 0}, pa[6] = {0, 0, 1, 1, 0, 2};
+#pragma unroll
+  for (int q = 0; q < 6; ++q)
+#pragma unroll
+    for (int t = 0; t < 4; ++t) acc[t] = mma(fr[t][pw[q]], bp[pa[q]], acc[t]);
+}
+
+// registers 8 kk .. 8 kk + 7 of an accumulator tile as the B operand of the next product's k-step
+__device__ __forceinline__ void split_half(const f32x16 &v, int kk, u32x4 (&pl)[3]) {
+  float e[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) e[j] = kk ? v[8 + j] : v[j];
+  split8(e, pl);
+}
+
+// The tail on a wave's transposed tile: y = yT (+ residual) leaves, then LayerNorm(y) if asked for.  A lane holds 64
+// of its row's 128 channels (4 consecutive ones per register quad), its partner lane the others.  gb: gamma | beta.
+__device__ __forceinline__ void finish_rows(f32x16 (&yT)[4], int64_t row, bool ok, int g, const float *residual, float *y,
+                                            float *ln_out, const float *gb, float eps) {
+#pragma unroll
+  for (int t = 0; t < 4; ++t)
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int64_t at = row * kC + 32 * t + 8 * q + 4 * g;
+      float4 v = {yT[t][4 * q], yT[t][4 * q + 1], yT[t][4 * q + 2], yT[t][4 * q + 3]};
+      if (residual) {
+        const float4 r = *reinterpret_cast<const float4 *>(residual + at);
+        v.x += r.x, v.y += r.y, v.z += r.z, v.w += r.w;
+      }
+      if (ok) *reinterpret_cast<float4 *>(y + at) = v;
+      yT[t][4 * q] = v.x, yT[t][4 * q + 1] = v.y, yT[t][4 * q + 2] = v.z, yT[t][4 * q + 3] = v.w;
+    }
+  if (!ln_out) return;
+  float sum = 0.f;
+#pragma unroll
+  for (int t = 0; t < 4; ++t)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) sum += yT[t][r];
+  const float mean = half_sum(sum) * (1.f / kC);
+  float sq = 0.f;
+#pragma unroll
+  for (int t = 0; t < 4; ++t)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const float d = yT[t][r] - mean;
+      sq = fmaf(d, d, sq);
+    }
+  const float rstd = 1.f / sqrtf(half_sum(sq) * (1.f / kC) + eps);
+#pragma unroll
+  for (int t = 0; t < 4; ++t)
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int c0 = 32 * t + 8 * q + 4 * g;
+      const float4 ga = *reinterpret_cast<const float4 *>(gb + c0), be = *reinterpret_cast<const float4 *>(gb + kC + c0);
+      float4 o;
+      o.x = (yT[t][4 * q] - mean) * rstd * ga.x + be.x;
+      o.y = (yT[t][4 * q + 1] - mean) * rstd * ga.y + be.y;
+      o.z = (yT[t][4 * q + 2] - mean) * rstd * ga.z + be.z;
+      o.w = (yT[t][4 * q + 3] - mean) * rstd * ga.w + be.w;
+      if (ok) *reinterpret_cast<float4 *>(ln_out + row * kC + c0) = o;
+    }
+}
+
+struct Tail {
+  const float *residual, *gamma, *beta;
+  float *ln_out;
+  float eps;
+};
+
+__device__ __forceinline__ void stage_gamma_beta(float *gb, const Tail &tail, int tid) {
+  if (tid < kC) {
+    gb[tid] = tail.gamma ? tail.gamma[tid] : 1.f;
+    gb[kC + tid] = tail.beta ? tail.beta[tid] : 0.f;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// deslice_linear_kernel.  A workgroup's four tiles belong to one batch.  LDS: W_out as 8 units (96 KB), the batch's
+// attended slice tokens as A operands (48 KB), gamma | beta.
+//   out_x^T (head pair P: 32 channels x 32 points) = T_P w_P^T, reduction index k = 0 .. 63 over (head of the pair,
+//   slice): T_P[(hh, d)][k] = out_token[2 P + hh][k % 32][d] where k / 32 == hh, else 0;  w_P[point][k] is the point's
+//   64 consecutive weights of the two heads.
+// ---------------------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void deslice_linear_kernel(const u32x4 *__restrict__ blob,
+                                                             const float *__restrict__ b_out,
+                                                             const float *__restrict__ w,
+                                                             const float *__restrict__ out_token, float *__restrict__ y,
+                                                             Tail tail, int N, int bpb) {
+  extern __shared__ u32x4 smem[];
+  u32x4 *wout = smem;                   // 8 units
+  u32x4 *tokp = smem + 8 * kUnit;       // [pair][kk][piece][lane]
+  float *gb = reinterpret_cast<float *>(tokp + 16 * 192);
+  const int tid = threadIdx.x, lane = tid & 63, i = lane & 31, g = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int b = blockIdx.x / bpb, gblk = blockIdx.x - b * bpb;
+  const int n0 = (gblk * 4 + wave) * 32;
+  const int n = min(n0 + i, N - 1);
+  const bool ok = n0 + i < N;
+#pragma unroll
+  for (int u = 0; u < 8; ++u)
+    load_3k_to_lds(blob + u * kUnit + wave * 192, lane * 16, (unsigned)(uintptr_t)(wout + u * kUnit + wave * 192));
+  stage_gamma_beta(gb, tail, tid);
+  // the batch's tokens as block-diagonal A operands
+  const float *tok = out_token + (int64_t)b * kH * kS * kD;
+  for (int item = tid; item < 16 * 64; item += 256) {
+    const int pk = item >> 6, l = item & 63, li = l & 31, lg = l >> 5;
+    const int pair = pk >> 2, kk = pk & 3, hh = li >> 4, d = li & 15;
+    float e[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int k = 16 * kk + 8 * lg + j;
+      e[j] = (k >> 5) == hh ? tok[((2 * pair + hh) * kS + (k & 31)) * kD + d] : 0.f;
+    }
+    u32x4 pl[3];
+    split8(e, pl);
+#pragma unroll
+    for (int p = 0; p < 3; ++p) tokp[(pk * 3 + p) * 64 + l] = pl[p];
+  }
+  __syncthreads();
+  // out_x^T: the four head pairs take turns
+  f32x16 ox[4];
+#pragma unroll
+  for (int t = 0; t < 4; ++t)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) ox[t][r] = 0.f;
+  const float *wrow = w + ((int64_t)b * N + n) * (kH * kS) + 8 * g;
+#pragma unroll
+  for (int kk = 0; kk < 4; ++kk) {
+    u32x4 bp[4][3];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      const float4 *src = reinterpret_cast<const float4 *>(wrow + 64 * t + 16 * kk);
+      const float4 lo = src[0], hi = src[1];
+      const float e[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+      split8(e, bp[t]);
+    }
+    constexpr int pw[6] = {0, 1, 0, 1, 2, 0}, pa[6] = {0, 0, 1, 1, 0, 2};
+#pragma unroll
+    for (int q = 0; q < 6; ++q)
+#pragma unroll
+      for (int t = 0; t < 4; ++t)
+        ox[t] = mma(tokp[((t * 4 + kk) * 3 + pw[q]) * 64 + lane], bp[t][pa[q]], ox[t]);
+  }
+  // y^T = W_out out_x^T + b_out
+  f32x16 yT[4];
+#pragma unroll
+  for (int t = 0; t < 4; ++t)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) yT[t][r] = b_out ? b_out[32 * t + rowmap(r, g)] : 0.f;
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's share of W_out has landed
+  __syncthreads();
+#pragma unroll
+  for (int ks = 0; ks < 8; ++ks) {
+    u32x4 bp[3];
+    split_half(ox[ks >> 1], ks & 1, bp);
+    kstep(yT, wout + ks * kUnit + lane, bp);
+  }
+  finish_rows(yT, (int64_t)b * N + n, ok, g, tail.residual, y, tail.ln_out, gb, tail.eps);
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// mlp_kernel.  LDS: a ring of 12 weight units (144 KB), gamma | beta.  Chunk c of 128 hidden features uses units
+// 16 c .. 16 c + 7 (W1 rows) and 16 c + 8 .. 16 c + 15 (W2 columns); units are requested up to 12 ahead, 8 at a time
+// after the product that frees their slots.
+// ---------------------------------------------------------------------------------------------------------------
+constexpr int kMlpRing = 12;
+
+__global__ __launch_bounds__(256) void mlp_kernel(const u32x4 *__restrict__ blob, const float *__restrict__ b1,
+                                                  const float *__restrict__ b2, const float *__restrict__ u,
+                                                  float *__restrict__ y, Tail tail, int64_t M, int F) {
+  extern __shared__ u32x4 smem[];
+  float *gb = reinterpret_cast<float *>(smem + kMlpRing * kUnit);
+  const int tid = threadIdx.x, lane = tid & 63, i = lane & 31, g = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int64_t row0 = ((int64_t)blockIdx.x * 4 + wave) * 32;
+  const int64_t row = min(row0 + i, M - 1);
+  const bool ok = row0 + i < M;
+  const int total = (F / 128) * 16;
+  int issued = 0;
+  auto issue_upto = [&](int upto) {  // this wave's quarter (3 KB) of units issued .. upto - 1
+    for (; issued < upto && issued < total; ++issued)
+      load_3k_to_lds(blob + (int64_t)issued * kUnit + wave * 192, lane * 16,
+                     (unsigned)(uintptr_t)(smem + (issued % kMlpRing) * kUnit + wave * 192));
+  };
+  // units below `upto` have landed for every wave: at most the 4 newest units (3 operations each) stay in flight
+  auto wait_landed = [&](int upto) {
+    if (issued - upto >= 4) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+  };
+  issue_upto(kMlpRing);
+  stage_gamma_beta(gb, tail, tid);
+  // the wave's rows: lane (i, g) holds channels 16 ks + 8 g .. + 7 of row i
+  float xr[8][8];
+  {
+    const float *src = u + row * kC + 8 * g;
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) {
+      const float4 lo = *reinterpret_cast<const float4 *>(src + 16 * ks), hi = *reinterpret_cast<const float4 *>(src + 16 * ks + 4);
+      xr[ks][0] = lo.x, xr[ks][1] = lo.y, xr[ks][2] = lo.z, xr[ks][3] = lo.w;
+      xr[ks][4] = hi.x, xr[ks][5] = hi.y, xr[ks][6] = hi.z, xr[ks][7] = hi.w;
+    }
+  }
+  f32x16 yT[4];
+#pragma unroll
+  for (int t = 0; t < 4; ++t)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) yT[t][r] = b2 ? b2[32 * t + rowmap(r, g)] : 0.f;
+  // the compiler too must know these loads are complete before the loop (it cannot see the asynchronous ones)
+  __builtin_amdgcn_s_waitcnt(0x0F70);
+  for (int c = 0; c < F / 128; ++c) {
+    const int base = 16 * c;
+    f32x16 hT[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) hT[t][r] = b1 ? b1[128 * c + 32 * t + rowmap(r, g)] : 0.f;
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    wait_landed(base + 8);
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) {
+      u32x4 bp[3];
+      split8(xr[ks], bp);
+      kstep(hT, smem + ((base + ks) % kMlpRing) * kUnit + lane, bp);
+    }
+    __syncthreads();  // the slots of W1's units are free
+    issue_upto(base + 8 + kMlpRing);
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) hT[t][r] = gelu_erf(hT[t][r]);
+    wait_landed(base + 16);
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) {
+      u32x4 bp[3];
+      split_half(hT[ks >> 1], ks & 1, bp);
+      kstep(yT, smem + ((base + 8 + ks) % kMlpRing) * kUnit + lane, bp);
+    }
+    __syncthreads();  // the slots of W2's units are free
+    issue_upto(base + 16 + kMlpRing);
+  }
+  finish_rows(yT, row, ok, g, tail.residual, y, tail.ln_out, gb, tail.eps);
+}
+
+static Tail make_tail(const pa_block_tail *t) {
+  Tail r{};
+  if (!t) return r;
+  r.residual = static_cast<const float *>(t->residual);
+  r.ln_out = static_cast<float *>(t->ln_out);
+  r.gamma = t->ln_gamma;
+  r.beta = t->ln_beta;
+  r.eps = t->ln_eps;
+  return r;
+}
+
+bool backend_supported(int dtype, const pa_shape &s) {
+  return dtype == PA_F32 && s.C == kC && s.H == kH && s.D == kD && s.S == kS;
+}
+
+int64_t backend_blob_bytes() { return 8 * (int64_t)kUnit * 16; }
+
+int backend(const pa_shape &s, const pa_params &p, const void *w, const float *out_token, void *y,
+            const pa_block_tail *tail, void *blob, hipStream_t st) {
+  if (!backend_supported(PA_F32, s)) return PA_ERR_UNSUPPORTED;
+  hipLaunchKernelGGL(pack_linear_kernel, dim3(8), dim3(256), 0, st, static_cast<const float *>(p.out_linear_weight),
+                     kC, 1, static_cast<u32x4 *>(blob));
+  int rc = launch_status();
+  if (rc) return rc;
+  const size_t lds = (size_t)(8 * kUnit + 16 * 192) * 16 + 2 * kC * 4;
+  if ((rc = allow_dynamic_lds(deslice_linear_kernel, lds))) return rc;
+  const int bpb = (int)(((s.N + 31) / 32 + 3) / 4);
+  hipLaunchKernelGGL(deslice_linear_kernel, dim3((unsigned)(s.B * bpb)), dim3(256), lds, st,
+                     static_cast<const u32x4 *>(blob), p.out_linear_bias, static_cast<const float *>(w), out_token,
+                     static_cast<float *>(y), make_tail(tail), (int)s.N, bpb);
+  return launch_status();
+}
+
+bool mlp_supported(int dtype, int64_t M, int64_t C, int64_t F) {
+  return dtype == PA_F32 && M > 0 && C == kC && F >= 128 && F % 128 == 0 && F <= 8192;
+}
+
+int64_t mlp_blob_bytes(int64_t F) { return (F / 128) * 16 * (int64_t)kUnit * 16; }
+
+int mlp_pack(int64_t F, const void *w1, const void *w2, void *blob, hipStream_t st) {
+  hipLaunchKernelGGL(pack_mlp_kernel, dim3((unsigned)((F / 128) * 16)), dim3(256), 0, st, static_cast<const float *>(w1),
+                     static_cast<const float *>(w2), (int)F, static_cast<u32x4 *>(blob));
+  return launch_status();
+}
+
+int mlp_forward(int64_t M, int64_t F, const void *blob, const float *b1, const float *b2, const void *u, void *y,
+                const pa_block_tail *tail, hipStream_t st) {
+  const size_t lds = (size_t)kMlpRing * kUnit * 16 + 2 * kC * 4;
+  int rc = allow_dynamic_lds(mlp_kernel, lds);
+  if (rc) return rc;
+  const int64_t blocks = ((M + 31) / 32 + 3) / 4;
+  hipLaunchKernelGGL(mlp_kernel, dim3((unsigned)blocks), dim3(256), lds, st, static_cast<const u32x4 *>(blob), b1, b2,
+                     static_cast<const float *>(u), static_cast<float *>(y), make_tail(tail), M, (int)F);
+  return launch_status();
+}
+
+}  // namespace f32rows
+}  // namespace pa

@@ -272,16 +272,17 @@ def layernorm_backward(x, dy, ln_weight, ln_eps=1e-5):
 
 
 def mlp_supported(dtype: torch.dtype, rows: int, C: int, F: int) -> bool:
-    """True if `mlp_forward` serves this shape with the MFMA kernel (bf16, C in {128, 256}, F a multiple of 64)."""
-    if dtype != torch.bfloat16:
+    """True if `mlp_forward` serves this shape: bf16 with C in {128, 256, 512} and F a multiple of 64 (MFMA kernels), or
+    float32 with C = 128 and F a multiple of 128 (row kernel on split-bf16 products)."""
+    if dtype not in (torch.bfloat16, torch.float32):
         return False
-    return bool(_lib.load().pa_mlp_query(_lib.PA_BF16, rows, C, F))
+    return bool(_lib.load().pa_mlp_query(_lib.dtype_code(dtype), rows, C, F))
 
 
 def mlp_forward(u, w1, b1, w2, b2, residual=None, ln_weight=None, ln_bias=None, ln_eps=1e-5):
     """y = w2 . gelu(w1 . u + b1) + b2 [+ residual]; returns y, or (y, LayerNorm(y)) when ln_weight is given.
 
-    u (..., C) bfloat16; w1 (F, C), w2 (C, F) bfloat16; b1, b2, ln_weight, ln_bias float32."""
+    u (..., C) bfloat16 or float32; w1 (F, C), w2 (C, F) in the same dtype; b1, b2, ln_weight, ln_bias float32."""
     _need_cuda(u, w1, b1, w2, b2, residual, ln_weight, ln_bias)
     lib = _lib.load()
     C, F = w1.shape[1], w1.shape[0]
@@ -303,7 +304,7 @@ def mlp_forward(u, w1, b1, w2, b2, residual=None, ln_weight=None, ln_bias=None, 
 
 def mlp_pack(w1, w2):
     """The two weights of the MLP in the fused kernel's operand order: one call per parameter set; the result is the
-    `packed` argument of mlp_forward_packed.  w1 (F, C), w2 (C, F) bfloat16."""
+    `packed` argument of mlp_forward_packed.  w1 (F, C), w2 (C, F) bfloat16 or float32."""
     _need_cuda(w1, w2)
     lib = _lib.load()
     C, F = w1.shape[1], w1.shape[0]

@@ -289,7 +289,7 @@ class GALEBlock(nn.Module):
         fx1 = attn + fx
         normed = PA.layer_norm(fx1, self.ln_mlp1[0])
         if not needs_grad and self._mlp_kernel_serves(normed):
-            packed, b1, b2 = self._mlp_kernel_packed(normed.device)
+            packed, b1, b2 = self._mlp_kernel_packed(normed.device, normed.dtype)
             return PF.mlp_forward_packed(normed, packed, b1, b2, residual=fx1.to(normed.dtype).contiguous())
         return self._mlp_with_grad(normed) + fx1
 

@@ -116,18 +116,18 @@ class TransolverBlock(nn.Module):
         return self
 
     # ---------------------------------------------------------------- fused MLP (pa_mlp_forward)
-    def _mlp_kernel_params(self, device):
-        """bf16 weights / fp32 biases of ln_mlp1's Mlp for the fused kernel; cached until a parameter changes.  With
-        fp8 weights enabled the bf16 values are the dequantised e4m3 weights."""
+    def _mlp_kernel_params(self, device, dtype=torch.bfloat16):
+        """Weights (in the activation dtype: bf16, or float32) / fp32 biases of ln_mlp1's Mlp for the fused kernel;
+        cached until a parameter changes.  With fp8 weights enabled the bf16 values are the dequantised e4m3 weights."""
         lin1, lin2 = self.ln_mlp1[1].layers[0], self.ln_mlp1[1].layers[2]
         named = (lin1.weight, lin1.bias, lin2.weight, lin2.bias)
-        stamp = (device, self.fp8_weights) + tuple((t.data_ptr(), t._version, t.dtype) for t in named)
+        stamp = (device, dtype, self.fp8_weights) + tuple((t.data_ptr(), t._version, t.dtype) for t in named)
         if self._mlp_cache.get("stamp") != stamp:
             def big(w):
                 w = w.detach().to(device=device, dtype=torch.float32)
                 if self.fp8_weights:
                     w = PF.dequantize_e4m3_per_channel(*PF.quantize_e4m3_per_channel(w))
-                return w.to(torch.bfloat16).contiguous().clone()
+                return w.to(dtype).contiguous().clone()
 
             with torch.no_grad():
                 params = (big(lin1.weight), lin1.bias.detach().to(device=device, dtype=torch.float32).contiguous().clone(),
@@ -135,17 +135,19 @@ class TransolverBlock(nn.Module):
             self._mlp_cache = {"stamp": stamp, "params": params}
         return self._mlp_cache["params"]
 
-    def _mlp_kernel_packed(self, device):
+    def _mlp_kernel_packed(self, device, dtype=torch.bfloat16):
         """(packed weights, b1, b2) for pa_mlp_forward_packed: the weights repacked once per parameter set."""
-        w1, b1, w2, b2 = self._mlp_kernel_params(device)
+        w1, b1, w2, b2 = self._mlp_kernel_params(device, dtype)
         if "packed" not in self._mlp_cache:
             self._mlp_cache["packed"] = PF.mlp_pack(w1, w2)
         return self._mlp_cache["packed"], b1, b2
 
     def _mlp_kernel_serves(self, normed: torch.Tensor) -> bool:
         mlp = self.ln_mlp1[1]
-        if not (normed.is_cuda and normed.dtype == torch.bfloat16 and isinstance(mlp.layers[1], nn.GELU)
+        if not (normed.is_cuda and normed.dtype in (torch.bfloat16, torch.float32) and isinstance(mlp.layers[1], nn.GELU)
                 and mlp.layers[1].approximate == "none"):
+            return False
+        if normed.dtype == torch.float32 and self.fp8_weights:
             return False
         hidden = mlp.layers[0].out_features
         return PF.mlp_supported(normed.dtype, normed.numel() // normed.shape[-1], normed.shape[-1], hidden)
@@ -181,7 +183,7 @@ class TransolverBlock(nn.Module):
         """fx1 + Mlp(normed) and, with `next_ln`, its LayerNorm (reference :303, and :300 of the next block): the fused
         block-MLP kernel where it serves the shape, else the tensor-op MLP followed by one add (+ LayerNorm) kernel."""
         if self._mlp_kernel_serves(normed):
-            packed, b1, b2 = self._mlp_kernel_packed(normed.device)
+            packed, b1, b2 = self._mlp_kernel_packed(normed.device, normed.dtype)
             if next_ln is None:
                 return PF.mlp_forward_packed(normed, packed, b1, b2, residual=fx1), None
             return PF.mlp_forward_packed(normed, packed, b1, b2, residual=fx1,

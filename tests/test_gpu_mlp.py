@@ -8,7 +8,7 @@ import torch.nn.functional as F
 
 from oracle import torch_oracle as to
 from physicsnemo_amd import functional as PF
-from gpu_util import announce, assert_rel_l2
+from gpu_util import announce, assert_fp32_close, assert_rel_l2
 
 pytestmark = pytest.mark.gpu
 
@@ -98,3 +98,45 @@ def test_mlp_rejects_unsupported():
     assert not PF.mlp_supported(torch.bfloat16, 100, 512, 8192)
     assert not PF.mlp_supported(torch.bfloat16, 100, 256, 8192)
     assert not PF.mlp_supported(torch.bfloat16, 100, 256, 1000)
+
+
+@pytest.mark.parametrize("rows_shape,Fh", [((1, 4096), 128), ((2, 1000), 512), ((1, 1), 128), ((3, 77), 256),
+                                           ((4, 7225), 128), ((1, 300), 1024)])
+def test_mlp_fp32_matches_oracle(rows_shape, Fh):
+    # float32 at C = 128: the row kernel on split-bf16 products; ragged row counts, idle waves (77 rows: 3 tiles),
+    # several chunks of 128 hidden features, cfg1's shape (4 x 7225 rows, mlp_ratio 1)
+    announce("mlp fp32", rows_shape, Fh)
+    C = 128
+    torch.manual_seed(1)
+    ref = to.OracleMlp(C, Fh, C).eval()
+    u, res = torch.randn(*rows_shape, C), torch.randn(*rows_shape, C)
+    gamma, beta = torch.rand(C) + 0.5, torch.randn(C) * 0.1
+    dev = torch.device("cuda:0")
+    args = dict(u=u.to(dev), w1=ref.layers[0].weight.detach().to(dev).contiguous(), b1=ref.layers[0].bias.detach().to(dev),
+                w2=ref.layers[2].weight.detach().to(dev).contiguous(), b2=ref.layers[2].bias.detach().to(dev))
+    assert PF.mlp_supported(torch.float32, u.numel() // C, C, Fh)
+    with torch.no_grad():
+        want = ref(u)
+        want_sum = want + res
+        want_ln = F.layer_norm(want_sum, (C,), gamma, beta, 1e-5)
+        want64 = ref.double()(u.double())
+        y = PF.mlp_forward(**args)
+        y2, ln2 = PF.mlp_forward(**args, residual=res.to(dev), ln_weight=gamma.to(dev), ln_bias=beta.to(dev))
+        y3 = PF.mlp_forward(**args, residual=res.to(dev))
+        y4, ln4 = PF.mlp_forward(**args, ln_weight=gamma.to(dev), ln_bias=beta.to(dev))
+        packed = PF.mlp_pack(args["w1"], args["w2"])
+        y5 = PF.mlp_forward_packed(args["u"], packed, args["b1"], args["b2"])
+    assert y.dtype == torch.float32 and y.shape == u.shape
+    assert_fp32_close(y, want, "mlp output")
+    assert_fp32_close(y2, want_sum, "mlp + residual")
+    assert_fp32_close(ln2, want_ln, "LayerNorm(mlp + residual)")
+    assert_fp32_close(ln4, F.layer_norm(want, (C,), gamma, beta, 1e-5), "LayerNorm(mlp)")
+    assert torch.equal(y3, y2) and torch.equal(y4, y) and torch.equal(y5, y)
+    # float32 accuracy of the split products: as close to the float64 result as float32 tensor ops are
+    e_hip, e_f32 = to.rel_l2(y.double().cpu(), want64), to.rel_l2(want.double(), want64)
+    assert e_hip < 4 * e_f32 + 2e-7, (e_hip, e_f32)
+
+
+def test_mlp_fp32_unsupported_shapes():
+    assert not PF.mlp_supported(torch.float32, 100, 256, 1024)  # float32 is served at C = 128 only
+    assert not PF.mlp_supported(torch.float32, 100, 128, 192)   # hidden features in chunks of 128

@@ -77,6 +77,29 @@ def test_fp32_structured2d_fused_front_end(kernel, grid, B):
     assert e_fused < 2e-6 and e_fused < 4 * e_staged + 2e-7
 
 
+@pytest.mark.parametrize("B,N", [(2, 500), (1, 33), (3, 4100)])
+def test_fp32_irregular_row_kernel_back_end(B, N):
+    # C = 128, 8 heads of 16, 32 slices, irregular mesh: the layer call hands back to the points, applies out_linear
+    # and the block tail in the float32 row kernel (split-bf16 products); the front end runs the general kernels
+    announce("fp32 irregular, row-kernel back end", B, N)
+    dim, heads, dim_head, S = 128, 8, 16, 32
+    ref, hip = make_pair("irregular", dim, heads, dim_head, S, sharpen=2.0, temps=[0.3 + 5.7 * i / 7 for i in range(8)])
+    ln = torch.nn.LayerNorm(dim)
+    with torch.no_grad():
+        ln.weight.add_(0.2 * torch.randn(dim))
+        ln.bias.add_(0.2 * torch.randn(dim))
+    x, res = torch.randn(B, N, dim), torch.randn(B, N, dim)
+    with torch.no_grad():
+        want = ref(x)
+        want_fx = want + res
+        want_ln = ln(want_fx)
+        y = hip(x.cuda())
+        fx, normed = hip.forward_block(x.cuda(), res.cuda(), ln.cuda())
+    assert_fp32_close(y, want, "layer y")
+    assert_fp32_close(fx, want_fx, "fx_new")
+    assert_fp32_close(normed, want_ln, "LayerNorm(fx_new)")
+
+
 @pytest.mark.parametrize("kernel,grid", [(3, (4, 4, 4)), (3, (8, 8, 8)), (5, (8, 8, 8)), (3, (3, 5, 7)), (1, (4, 6, 5))])
 def test_fp32_structured3d_stages_and_layer(kernel, grid):
     announce("fp32 structured3d", kernel, grid)
