@@ -1014,7 +1014,9 @@ int pa_layer_forward(int dtype, const pa_shape *shape, const pa_params *p, const
   float *tok_out = reinterpret_cast<float *>(ws + plan.off_tok_out);
 
   if (plan.conv_front) {  // both convolutions, the slice softmax and the partial token sums in one launch
-    if ((rc = pa::conv::front(s, *p, x, ws + plan.off_blob, w, partials, st))) return rc;
+    if ((rc = pa::conv::front(s, *p, x, ws + plan.off_blob, w, partials,
+                              plan.rows_back ? ws + plan.off_blob_out : nullptr, st)))
+      return rc;
   } else {
     if ((rc = pa::general::project_inputs(dtype, s, *p, x, x_mid, fx_mid, st))) return rc;
     if ((rc = pa::general::slice_softmax(dtype, s, *p, x_mid, w, st))) return rc;
@@ -1022,7 +1024,8 @@ int pa_layer_forward(int dtype, const pa_shape *shape, const pa_params *p, const
   }
   if ((rc = pa::general::combine_attention(s, *p, partials, plan.G, tok, norm, tok_out, st))) return rc;
   if (plan.rows_back)  // hand-back, out_linear, residual and LayerNorm in one launch
-    return pa::f32rows::backend(s, *p, w, tok_out, y, tail_active(tail) ? tail : nullptr, ws + plan.off_blob_out, st);
+    return pa::f32rows::backend(s, *p, w, tok_out, y, tail_active(tail) ? tail : nullptr, ws + plan.off_blob_out,
+                                plan.conv_front, st);
   void *out_x = x_mid;
   if ((rc = pa::general::deslice(dtype, s, w, tok_out, out_x, st))) return rc;
   if ((rc = pa::general::out_linear(dtype, s, *p, out_x, y, st))) return rc;

@@ -47,17 +47,25 @@ constexpr int kStepsPerTap = kC / 16;              // k-steps of 16 channels
 constexpr int kStepUnits = kColTiles * 3 * 64;     // 16-byte units per k-step: 8 tiles x 3 pieces x 1 KB
 constexpr int kRing = 4;
 constexpr int kTokFloats = kH * kS * kD1;          // one partial
-// the ring, reused after the convolution for 4 token sums, 4 x 2 weight tiles in transit and the softmax statistics
-constexpr size_t kEpilogueBytes = (size_t)4 * kTokFloats * 4 + 4 * 2 * 4096 + 4 * 64 * 4;
+// the ring, reused after the convolution for 4 token sums, 4 x 4 weight tiles in transit and the softmax statistics
+constexpr size_t kEpilogueBytes = (size_t)4 * kTokFloats * 4 + 4 * 4 * 4096 + 4 * 128 * 4;
 constexpr size_t kRingBytes = (size_t)kRing * kStepUnits * 16 + (size_t)kRing * 4 * 2048;  // weights + input rows
 constexpr size_t kLdsBytes = kRingBytes > kEpilogueBytes ? kRingBytes : kEpilogueBytes;
 
 // blob unit ((step 8 + ct) 3 + piece) 64 + lane: the B operand (lane (i, g): output channel 32 (ct % 4) + i of weight
 // set ct / 4, k = 8 g .. 8 g + 7 of the step) of one bf16 piece.  step = tap 8 + channel block.
+// The last 8 workgroups (when w_out is given) cut out_linear's weight for the hand-back kernel of the same layer call.
 __global__ __launch_bounds__(256) void split_pack_kernel(const float *__restrict__ wx, const float *__restrict__ wfx,
-                                                         u32x4 *__restrict__ blob, int taps, int tap_major) {
+                                                         u32x4 *__restrict__ blob, int taps, int tap_major,
+                                                         int conv_blocks, const float *__restrict__ w_out,
+                                                         u32x4 *__restrict__ blob_out) {
+  if ((int)blockIdx.x >= conv_blocks) {
+    const int u = blockIdx.x - conv_blocks;
+    pack_unit(w_out, kC, 16 * u, true, blob_out + (int64_t)u * kUnit, threadIdx.x);
+    return;
+  }
   const int64_t total = (int64_t)taps * kStepsPerTap * kColTiles * 64;
-  for (int64_t u = (int64_t)blockIdx.x * 256 + threadIdx.x; u < total; u += (int64_t)gridDim.x * 256) {
+  for (int64_t u = (int64_t)blockIdx.x * 256 + threadIdx.x; u < total; u += (int64_t)conv_blocks * 256) {
     const int lane = (int)(u & 63), ct = (int)(u >> 6) & 7, step = (int)(u >> 9);
     const int tap = step / kStepsPerTap, c0 = (step % kStepsPerTap) * 16 + 8 * (lane >> 5);
     const int o = 32 * (ct & 3) + (lane & 31);
@@ -179,53 +187,67 @@ __global__ __launch_bounds__(512) void conv_slice_kernel(
     read_rows(0);
     read_fragments(0, fr[0]);
     split_row(raw, cur);
-    for (int s2 = 0; s2 < steps; s2 += 2) {
-      static_for<2>([&](auto par_) {
-        constexpr int par = decltype(par_)::value;
-        const int s = s2 + par;
-        // Groups up to s + 3 are issued.  This step multiplies the fragments and rows of step s, read from LDS one
-        // step ago, and reads those of step s + 1: group s + 1 must have landed, groups s + 2 and s + 3 may stay in
-        // flight (5 operations each for an x_mid wave, 3 for an fx_mid wave).  Each wave waits for its own share, then
-        // all meet; the slots of step s, read one step ago, are free once every wave is here.
-        constexpr int G = ROLE == 0 ? 5 : 3;
-        if (s + 3 < steps) {
-          if constexpr (G == 5) asm volatile("s_waitcnt vmcnt(10)" ::: "memory");
-          else asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
-        } else if (s + 2 < steps) {
-          if constexpr (G == 5) asm volatile("s_waitcnt vmcnt(5)" ::: "memory");
-          else asm volatile("s_waitcnt vmcnt(3)" ::: "memory");
-        } else {
-          asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        }
-        __syncthreads();
-        // the six products, the four column tiles taking turns; the step's other work (the next group's loads, the
-        // next step's LDS reads and split) is spread between them so that it issues while the matrix core is busy
-        auto product = [&](int pw, int pa) {
+    // One k-step.  Groups up to s + 3 are issued.  The step multiplies the fragments and rows of step s, read from LDS
+    // one step ago, and reads those of step s + 1: group s + 1 must have landed, groups s + 2 and s + 3 may stay in
+    // flight (5 operations each for an x_mid wave, 3 for an fx_mid wave).  Each wave waits for its own share, then all
+    // meet; the slots of step s, read one step ago, are free once every wave is here.  TAIL: one of the last four
+    // steps, where there is less to wait for, to read or to request.
+    auto step = [&](int s, auto par_, auto tail_) {
+      constexpr int par = decltype(par_)::value;
+      constexpr bool TAIL = decltype(tail_)::value;
+      if (!TAIL || s + 3 < steps) {
+        if constexpr (ROLE == 0) asm volatile("s_waitcnt vmcnt(10)" ::: "memory");
+        else asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
+      } else if (s + 2 < steps) {
+        if constexpr (ROLE == 0) asm volatile("s_waitcnt vmcnt(5)" ::: "memory");
+        else asm volatile("s_waitcnt vmcnt(3)" ::: "memory");
+      } else {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      }
+      __syncthreads();
+      if (!TAIL || s + 4 < steps) issue_group(s + 4, role_);
+      if (!TAIL || s + 1 < steps) {
+        read_rows(s + 1);
+        read_fragments(s + 1, fr[1 - par]);
+      }
+      // the six products, the four column tiles taking turns
+      auto product = [&](int pw, int pa) {
 #pragma unroll
-          for (int ct = 0; ct < 4; ++ct) {
-            if constexpr (ROLE == 0) acc[ct] = mma(fr[par][ct][pw], cur[pa], acc[ct]);
-            else acc[ct] = mma(cur[pa], fr[par][ct][pw], acc[ct]);
-          }
-          __builtin_amdgcn_sched_barrier(0);
-        };
-        product(0, 0);
-        if (s + 4 < steps) issue_group(s + 4, role_);
-        __builtin_amdgcn_sched_barrier(0);
-        product(1, 0);
-        if (s + 1 < steps) {
-          read_rows(s + 1);
-          read_fragments(s + 1, fr[1 - par]);
+        for (int ct = 0; ct < 4; ++ct) {
+          if constexpr (ROLE == 0) acc[ct] = mma(fr[par][ct][pw], cur[pa], acc[ct]);
+          else acc[ct] = mma(cur[pa], fr[par][ct][pw], acc[ct]);
         }
-        __builtin_amdgcn_sched_barrier(0);
-        product(0, 1);
-        if (s + 1 < steps) split_row(raw, nxt);
-        __builtin_amdgcn_sched_barrier(0);
-        product(1, 1);
-        product(2, 0);
-        product(0, 2);
+      };
+      product(0, 0);
+      product(1, 0);
+      product(0, 1);
+      product(1, 1);
+      product(2, 0);
+      product(0, 2);
+      if (!TAIL || s + 1 < steps) split_row(raw, nxt);
 #pragma unroll
-        for (int p = 0; p < 3; ++p) cur[p] = nxt[p];
-      });
+      for (int p = 0; p < 3; ++p) cur[p] = nxt[p];
+      if constexpr (!TAIL) {
+        // issue order: after every matrix instruction one LDS read (while there are any) and a few vector instructions,
+        // so that the step's other work runs while the matrix core is busy instead of ahead of it
+#pragma unroll
+        for (int k = 0; k < 24; ++k) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
+        }
+      }
+    };
+    constexpr std::integral_constant<int, 0> even{};
+    constexpr std::integral_constant<int, 1> odd{};
+    int s2 = 0;
+    for (; s2 + 5 < steps; s2 += 2) {
+      step(s2, even, std::false_type{});
+      step(s2 + 1, odd, std::false_type{});
+    }
+    for (; s2 < steps; s2 += 2) {
+      step(s2, even, std::true_type{});
+      step(s2 + 1, odd, std::true_type{});
     }
   };
   if (role == 0) convolve(std::integral_constant<int, 0>{});
@@ -234,8 +256,8 @@ __global__ __launch_bounds__(512) void conv_slice_kernel(
 
   float *red = reinterpret_cast<float *>(smem);                     // [tile][h][s][D + 1]
   float *mine = red + t * kTokFloats;
-  u32x4 *xchg = smem + (4 * kTokFloats) / 4 + t * (2 * 256);        // [tile][buffer][q][lane]: one head's weights
-  float *stat = reinterpret_cast<float *>(smem + (4 * kTokFloats) / 4 + 4 * 2 * 256) + t * 64;  // [max | 1 / sum][point]
+  u32x4 *xchg = smem + (4 * kTokFloats) / 4 + t * (4 * 256);        // [tile][round parity][head of the pair][q][lane]
+  float *stat = reinterpret_cast<float *>(smem + (4 * kTokFloats) / 4 + 4 * 4 * 256) + t * 128;  // [head][max | 1 / sum][point]
   // W_slice[s][d] for MFMA m of a head: this lane's channel of the pair (k = g) is d = 8 (m / 4) + 4 g + m % 4, the
   // channel the x_mid registers hold in that position
   float ws[8], bs_r[16];
@@ -244,77 +266,108 @@ __global__ __launch_bounds__(512) void conv_slice_kernel(
 #pragma unroll
   for (int r = 0; r < 16; ++r) bs_r[r] = b_slice ? b_slice[rowmap(r, g)] : 0.f;
   const float bs_i = b_slice ? b_slice[i] : 0.f;
-  float *wrow = w_out + ((int64_t)b * N + n0) * (kH * kS) + i;
+  float *wpoint = w_out + ((int64_t)b * N + n0 + i) * (kH * kS);  // this lane's point (when it exists)
 
-  // round h: the x_mid wave makes head h's weights and leaves them in LDS; the fx_mid wave sums head h - 1's tokens
-  static_for<kH + 1>([&](auto h_) {
-    constexpr int hh = decltype(h_)::value;
-    if (role == 0 && hh < kH) {
-      constexpr int h = hh < kH ? hh : 0, ct = h / 2, half = h % 2;
-      const float inv_t = temperature ? kLog2e / clamp_temperature(temperature[h]) : kLog2e;
-      // lanes <-> points: the head's softmax statistics
-      f32x16 lt;
+  // round r: the x_mid wave makes the weights of heads 2 r and 2 r + 1 (the halves of its column tile r) and leaves them
+  // in LDS; the fx_mid wave sums the tokens of the two heads of round r - 1.  The two heads' dependent MFMA chains
+  // take turns.
+  static_for<kH / 2 + 1>([&](auto r_) {
+    constexpr int rr = decltype(r_)::value;
+    if (role == 0 && rr < kH / 2) {
+      constexpr int ct = rr < kH / 2 ? rr : 0;
+      float inv_t[2];
 #pragma unroll
-      for (int r = 0; r < 16; ++r) lt[r] = bs_r[r];
+      for (int hf = 0; hf < 2; ++hf)
+        inv_t[hf] = temperature ? kLog2e / clamp_temperature(temperature[2 * ct + hf]) : kLog2e;
+      // lanes <-> points: the heads' softmax statistics
+      f32x16 lt[2];
 #pragma unroll
-      for (int m = 0; m < 8; ++m) lt = mma32(ws[m], acc[ct][8 * half + m], lt);
-      float mx = lt[0] * inv_t;
+      for (int r = 0; r < 16; ++r) lt[0][r] = lt[1][r] = bs_r[r];
 #pragma unroll
-      for (int r = 1; r < 16; ++r) mx = fmaxf(mx, lt[r] * inv_t);
-      mx = half_max(mx);
-      float sum = 0.f;
+      for (int m = 0; m < 8; ++m)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) sum += __builtin_amdgcn_exp2f(lt[r] * inv_t - mx);
-      sum = half_sum(sum);
-      if (g == 0) {
-        stat[i] = mx;
-        stat[32 + i] = 1.f / sum;
+        for (int hf = 0; hf < 2; ++hf) lt[hf] = mma32(ws[m], acc[ct][8 * hf + m], lt[hf]);
+#pragma unroll
+      for (int hf = 0; hf < 2; ++hf) {
+        float mx = lt[hf][0] * inv_t[hf];
+#pragma unroll
+        for (int r = 1; r < 16; ++r) mx = fmaxf(mx, lt[hf][r] * inv_t[hf]);
+        mx = half_max(mx);
+        float sum = 0.f;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          lt[hf][r] = __builtin_amdgcn_exp2f(lt[hf][r] * inv_t[hf] - mx);
+          sum += lt[hf][r];
+        }
+        sum = half_sum(sum);
+        const float inv = 1.f / sum;
+        if (g == 0) {
+          stat[64 * hf + i] = mx;
+          stat[64 * hf + 32 + i] = inv;
+        }
+        // the weights leave from this orientation: a lane holds 4 consecutive slices of its point per register quad
+        if (i < valid) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const float4 o = {lt[hf][4 * q] * inv, lt[hf][4 * q + 1] * inv, lt[hf][4 * q + 2] * inv, lt[hf][4 * q + 3] * inv};
+            *reinterpret_cast<float4 *>(wpoint + (2 * ct + hf) * kS + 8 * q + 4 * g) = o;
+          }
+        }
       }
       __builtin_amdgcn_wave_barrier();
       // lanes <-> slices, register r <-> point rowmap(r, g): the weights, as the A operand of the token sums
-      f32x16 ln;
+      f32x16 ln[2];
 #pragma unroll
-      for (int r = 0; r < 16; ++r) ln[r] = bs_i;
+      for (int r = 0; r < 16; ++r) ln[0][r] = ln[1][r] = bs_i;
 #pragma unroll
-      for (int m = 0; m < 8; ++m) ln = mma32(acc[ct][8 * half + m], ws[m], ln);
-      float nrm = 0.f;
+      for (int m = 0; m < 8; ++m)
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const float4 mq = *reinterpret_cast<const float4 *>(stat + 8 * q + 4 * g);
-        const float4 iq = *reinterpret_cast<const float4 *>(stat + 32 + 8 * q + 4 * g);
-        const float mqa[4] = {mq.x, mq.y, mq.z, mq.w}, iqa[4] = {iq.x, iq.y, iq.z, iq.w};
-        u32x4 out;
+        for (int hf = 0; hf < 2; ++hf) ln[hf] = mma32(acc[ct][8 * hf + m], ws[m], ln[hf]);
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int r = 4 * q + e, pt = 8 * q + 4 * g + e;
-          float wv = __builtin_amdgcn_exp2f(ln[r] * inv_t - mqa[e]) * iqa[e];
-          if (pt >= valid) wv = 0.f;
-          else wrow[(int64_t)pt * (kH * kS) + h * kS] = wv;
-          out[e] = __float_as_uint(wv);
-          nrm += wv;
+      for (int hf = 0; hf < 2; ++hf) {
+        const int h = 2 * ct + hf;
+        float nrm = 0.f;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const float4 mq = *reinterpret_cast<const float4 *>(stat + 64 * hf + 8 * q + 4 * g);
+          const float4 iq = *reinterpret_cast<const float4 *>(stat + 64 * hf + 32 + 8 * q + 4 * g);
+          const float mqa[4] = {mq.x, mq.y, mq.z, mq.w}, iqa[4] = {iq.x, iq.y, iq.z, iq.w};
+          u32x4 out;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const int r = 4 * q + e, pt = 8 * q + 4 * g + e;
+            float wv = __builtin_amdgcn_exp2f(ln[hf][r] * inv_t[hf] - mqa[e]) * iqa[e];
+            if (pt >= valid) wv = 0.f;
+            out[e] = __float_as_uint(wv);
+            nrm += wv;
+          }
+          xchg[((rr & 1) * 2 + hf) * 256 + q * 64 + lane] = out;
         }
-        xchg[(h & 1) * 256 + q * 64 + lane] = out;
+        nrm = half_sum(nrm);
+        if (g == 0) mine[h * (kS * kD1) + i * kD1 + kD] = nrm;
       }
-      __builtin_amdgcn_wave_barrier();
-      nrm = half_sum(nrm);
-      if (g == 0) mine[h * (kS * kD1) + i * kD1 + kD] = nrm;
     }
-    if (role == 1 && hh > 0) {
-      constexpr int h = hh > 0 ? hh - 1 : 0, ct = h / 2, half = h % 2;
-      f32x16 tk;
+    if (role == 1 && rr > 0) {
+      constexpr int ct = rr > 0 ? rr - 1 : 0;
+      f32x16 tk[2];
 #pragma unroll
-      for (int r = 0; r < 16; ++r) tk[r] = 0.f;
+      for (int r = 0; r < 16; ++r) tk[0][r] = tk[1][r] = 0.f;
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
-        const u32x4 wq = xchg[(h & 1) * 256 + q * 64 + lane];
+        u32x4 wq[2];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) tk = mma32(__uint_as_float(wq[e]), acc[ct][4 * q + e], tk);
-      }
-      // lane (i, g): channel 32 ct + i of fx_mid, register r <-> slice rowmap(r, g); the head's 16 channels are kept
-      if ((i >> 4) == half) {
+        for (int hf = 0; hf < 2; ++hf) wq[hf] = xchg[(((rr - 1) & 1) * 2 + hf) * 256 + q * 64 + lane];
 #pragma unroll
-        for (int r = 0; r < 16; ++r) mine[h * (kS * kD1) + rowmap(r, g) * kD1 + (i & 15)] = tk[r];
+        for (int e = 0; e < 4; ++e)
+#pragma unroll
+          for (int hf = 0; hf < 2; ++hf) tk[hf] = mma32(__uint_as_float(wq[hf][e]), acc[ct][4 * q + e], tk[hf]);
       }
+      // lane (i, g): channel 32 ct + i of fx_mid = channel i % 16 of head 2 ct + i / 16, register r <-> slice
+      // rowmap(r, g); each lane keeps the sums taken with its own head's weights
+      const int hf = i >> 4;
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        mine[(2 * ct + hf) * (kS * kD1) + rowmap(r, g) * kD1 + (i & 15)] = hf ? tk[1][r] : tk[0][r];
     }
     __syncthreads();
   });
@@ -332,13 +385,16 @@ int64_t groups(const pa_shape &s) { return ((s.N + 31) / 32 + 3) / 4; }
 
 int64_t blob_bytes(const pa_shape &s) { return s.conv_k * s.conv_k * kStepsPerTap * (int64_t)kStepUnits * 16 + 64; }
 
-int front(const pa_shape &s, const pa_params &p, const void *x, void *blob, void *w, float *partials, hipStream_t st) {
+int front(const pa_shape &s, const pa_params &p, const void *x, void *blob, void *w, float *partials, void *blob_out,
+          hipStream_t st) {
   if (!supported(PA_F32, s)) return PA_ERR_UNSUPPORTED;
   const int taps = (int)(s.conv_k * s.conv_k);
   const int64_t units = (int64_t)taps * kStepsPerTap * kColTiles * 64;
-  hipLaunchKernelGGL(split_pack_kernel, dim3((unsigned)((units + 255) / 256)), dim3(256), 0, st,
+  const int conv_blocks = (int)((units + 255) / 256);
+  hipLaunchKernelGGL(split_pack_kernel, dim3((unsigned)(conv_blocks + (blob_out ? 8 : 0))), dim3(256), 0, st,
                      static_cast<const float *>(p.in_project_x_weight), static_cast<const float *>(p.in_project_fx_weight),
-                     static_cast<u32x4 *>(blob), taps, (int)s.conv_tap_major);
+                     static_cast<u32x4 *>(blob), taps, (int)s.conv_tap_major, conv_blocks,
+                     static_cast<const float *>(p.out_linear_weight), static_cast<u32x4 *>(blob_out));
   int rc = launch_status();
   if (rc) return rc;
   if ((rc = allow_dynamic_lds(conv_slice_kernel, kLdsBytes))) return rc;

@@ -1209,8 +1209,12 @@ int combine_attention(const pa_shape &s, const pa_params &p, const float *partia
   if (rc) return rc;
   const int64_t stride = s.B * s.H * s.S * (s.D + 1);
   const float *src = partials;
-  if ((rc = combine_partials(s, partials, G, &src, st))) return rc;
-  hipLaunchKernelGGL(slice_combine_attn_kernel, dim3((unsigned)(s.B * s.H)), dim3(kAttnThreads), lds, st, src, G == 0 ? 0 : 1, stride,
+  int g_in = (int)G;  // a few partials are summed by the attention kernel itself, in index order
+  if (G > 8) {
+    if ((rc = combine_partials(s, partials, G, &src, st))) return rc;
+    g_in = 1;
+  }
+  hipLaunchKernelGGL(slice_combine_attn_kernel, dim3((unsigned)(s.B * s.H)), dim3(kAttnThreads), lds, st, src, g_in, stride,
                      p.qkv_project_weight, slice_token, slice_norm, out_token, (int)s.D, (int)s.S, stage_w);
   return launch_status();
 }

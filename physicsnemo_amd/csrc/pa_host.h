@@ -111,7 +111,10 @@ namespace conv {
 bool supported(int dtype, const pa_shape &s);
 int64_t groups(const pa_shape &s);
 int64_t blob_bytes(const pa_shape &s);
-int front(const pa_shape &s, const pa_params &p, const void *x, void *blob, void *w, float *partials, hipStream_t st);
+// blob_out (may be NULL): f32rows::backend_blob_bytes() that receive out_linear's weight in the form f32rows::backend
+// reads, cut by the same launch that cuts the convolution weights
+int front(const pa_shape &s, const pa_params &p, const void *x, void *blob, void *w, float *partials, void *blob_out,
+          hipStream_t st);
 }  // namespace conv
 
 namespace f32rows {
@@ -122,7 +125,7 @@ namespace f32rows {
 bool backend_supported(int dtype, const pa_shape &s);
 int64_t backend_blob_bytes();
 int backend(const pa_shape &s, const pa_params &p, const void *w, const float *out_token, void *y,
-            const pa_block_tail *tail, void *blob, hipStream_t st);
+            const pa_block_tail *tail, void *blob, bool blob_ready, hipStream_t st);
 bool mlp_supported(int dtype, int64_t rows, int64_t C, int64_t F);
 int64_t mlp_blob_bytes(int64_t F);
 int mlp_pack(int64_t F, const void *w1, const void *w2, void *blob, hipStream_t st);

@@ -30,21 +30,7 @@ using mfma::u32x4;
 using namespace split;
 
 constexpr int kC = 128, kH = 8, kD = 16, kS = 32;
-constexpr int kUnit = 4 * 3 * 64;  // 16-byte elements of a weight unit (12 KB)
-
-// One unit of a 128-row block of a float32 weight: thread `v` (0 .. 255) packs tile v / 64, lane v % 64 = (i, g):
-// row 32 tile + i, reduction indices k0 + 8 g + j (natural) or k0 rounded down to 32 + kperm((k0 / 16) % 2, g, j).
-__device__ __forceinline__ void pack_unit(const float *w, int64_t ld, int k0, bool permuted, u32x4 *unit, int v) {
-  const int ot = v >> 6, lane = v & 63, i = lane & 31, g = lane >> 5;
-  const float *row = w + (int64_t)(32 * ot + i) * ld;
-  float e[8];
-#pragma unroll
-  for (int j = 0; j < 8; ++j) e[j] = row[permuted ? (k0 & ~31) + kperm((k0 >> 4) & 1, g, j) : k0 + 8 * g + j];
-  u32x4 pl[3];
-  split8(e, pl);
-#pragma unroll
-  for (int p = 0; p < 3; ++p) unit[(ot * 3 + p) * 64 + lane] = pl[p];
-}
+using split::kUnit;
 
 // W (128, K) -> K / 16 units
 __global__ __launch_bounds__(256) void pack_linear_kernel(const float *__restrict__ w, int K, int permuted,
@@ -331,12 +317,14 @@ bool backend_supported(int dtype, const pa_shape &s) {
 int64_t backend_blob_bytes() { return 8 * (int64_t)kUnit * 16; }
 
 int backend(const pa_shape &s, const pa_params &p, const void *w, const float *out_token, void *y,
-            const pa_block_tail *tail, void *blob, hipStream_t st) {
+            const pa_block_tail *tail, void *blob, bool blob_ready, hipStream_t st) {
   if (!backend_supported(PA_F32, s)) return PA_ERR_UNSUPPORTED;
-  hipLaunchKernelGGL(pack_linear_kernel, dim3(8), dim3(256), 0, st, static_cast<const float *>(p.out_linear_weight),
-                     kC, 1, static_cast<u32x4 *>(blob));
-  int rc = launch_status();
-  if (rc) return rc;
+  int rc = PA_OK;
+  if (!blob_ready) {
+    hipLaunchKernelGGL(pack_linear_kernel, dim3(8), dim3(256), 0, st, static_cast<const float *>(p.out_linear_weight),
+                       kC, 1, static_cast<u32x4 *>(blob));
+    if ((rc = launch_status())) return rc;
+  }
   const size_t lds = (size_t)(8 * kUnit + 16 * 192) * 16 + 2 * kC * 4;
   if ((rc = allow_dynamic_lds(deslice_linear_kernel, lds))) return rc;
   const int bpb = (int)(((s.N + 31) / 32 + 3) / 4);

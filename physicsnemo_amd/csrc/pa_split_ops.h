@@ -50,6 +50,24 @@ __device__ __forceinline__ void load_3k_to_lds(const void *sbase, unsigned lane1
       : "memory");
 }
 
+// A float32 weight as A-operand fragments: units of 12 KB = one k-step (16 reduction indices) of 128 output rows,
+// [tile 0..3][piece 0..2][lane].
+constexpr int kUnit = 4 * 3 * 64;  // 16-byte elements of a unit
+
+// One unit of a 128-row block of a float32 weight: thread `v` (0 .. 255) packs tile v / 64, lane v % 64 = (i, g):
+// row 32 tile + i, reduction indices k0 + 8 g + j (natural) or k0 rounded down to 32 + mfma::kperm((k0 / 16) % 2, g, j).
+__device__ __forceinline__ void pack_unit(const float *w, int64_t ld, int k0, bool permuted, u32x4 *unit, int v) {
+  const int ot = v >> 6, lane = v & 63, i = lane & 31, g = lane >> 5;
+  const float *row = w + (int64_t)(32 * ot + i) * ld;
+  float e[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) e[j] = row[permuted ? (k0 & ~31) + mfma::kperm((k0 >> 4) & 1, g, j) : k0 + 8 * g + j];
+  u32x4 pl[3];
+  split8(e, pl);
+#pragma unroll
+  for (int p = 0; p < 3; ++p) unit[(ot * 3 + p) * 64 + lane] = pl[p];
+}
+
 template <class F, int... I>
 __device__ __forceinline__ void static_for_impl(F &&f, std::integer_sequence<int, I...>) {
   (f(std::integral_constant<int, I>{}), ...);
