@@ -449,6 +449,16 @@ int pa_mlp_pack(int dtype, int64_t C, int64_t F, const pa_mlp_params *p, void *p
 int pa_mlp_forward_packed(int dtype, int64_t rows, int64_t C, int64_t F, const void *packed, const float *b1,
                           const float *b2, const void *u, void *y, const pa_block_tail *tail, void *stream);
 
+/* The model's preprocess Mlp (TR.py:519-525 with mlp_layers.py:139-173): Linear(c_in -> F) -> GELU(erf) -> Linear(F -> C)
+ * over `rows` rows of u (rows, c_in), c_in = coordinates + fields per point; with a tail, tail->ln_out is the first
+ * block's LayerNorm of the result (TR.py:300).  Served for float32, C = 128, c_in <= 8, F a multiple of 128
+ * (pa_preprocess_query); p: w1 (F, c_in), w2 (C, F) float32.  workspace: pa_preprocess_workspace_bytes(). */
+int pa_preprocess_query(int dtype, int64_t rows, int64_t c_in, int64_t F, int64_t C);
+int64_t pa_preprocess_workspace_bytes(int dtype, int64_t rows, int64_t c_in, int64_t F, int64_t C);
+int pa_preprocess_forward(int dtype, int64_t rows, int64_t c_in, int64_t F, int64_t C, const pa_mlp_params *p,
+                          const void *u, void *y, const pa_block_tail *tail, void *workspace, int64_t workspace_bytes,
+                          void *stream);
+
 /* The block tail on its own (TR.py:300-303, :305-307): y (rows, C) <- y + tail->residual (if given), then
  * tail->ln_out = LayerNorm(y) (if given).  For callers whose producer of y is not one of the fused kernels. */
 int pa_residual_layernorm(int dtype, int64_t rows, int64_t C, void *y, const pa_block_tail *tail, void *stream);

@@ -34,6 +34,7 @@ EXPORTED = [
     "pa_cols_gemm_chunks", "pa_cols_gemm", "pa_residual_layernorm",
     "pa_mfma_layer_forward", "pa_rows_gemm_act", "pa_layernorm_backward_groups", "pa_layernorm_backward",
     "pa_static_scratch_bytes", "pa_slice_reduce_static",
+    "pa_preprocess_query", "pa_preprocess_workspace_bytes", "pa_preprocess_forward",
 ]
 
 PA_BUF_BLOB, PA_BUF_FX_PACK, PA_BUF_W_PACK, PA_BUF_PARTIALS, PA_BUF_TOKP = range(5)
@@ -139,6 +140,13 @@ def load() -> ctypes.CDLL:
     lib.pa_mlp_forward.restype = c_int
     lib.pa_mlp_forward.argtypes = [c_int, c_int64, c_int64, c_int64, POINTER(PaMlpParams), c_void_p, c_void_p, pt, c_void_p,
                                    c_int64, c_void_p]
+    lib.pa_preprocess_query.restype = c_int
+    lib.pa_preprocess_query.argtypes = [c_int, c_int64, c_int64, c_int64, c_int64]
+    lib.pa_preprocess_workspace_bytes.restype = c_int64
+    lib.pa_preprocess_workspace_bytes.argtypes = [c_int, c_int64, c_int64, c_int64, c_int64]
+    lib.pa_preprocess_forward.restype = c_int
+    lib.pa_preprocess_forward.argtypes = [c_int, c_int64, c_int64, c_int64, c_int64, POINTER(PaMlpParams), c_void_p,
+                                          c_void_p, pt, c_void_p, c_int64, c_void_p]
     lib.pa_rows_gemm.restype = c_int
     lib.pa_rows_gemm.argtypes = [c_int, ps, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]
     lib.pa_slice_weighted_sum.restype = c_int

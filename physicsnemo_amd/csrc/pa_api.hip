@@ -890,6 +890,30 @@ int pa_mlp_forward(int dtype, int64_t rows, int64_t C, int64_t F, const pa_mlp_p
                           st);
 }
 
+int pa_preprocess_query(int dtype, int64_t rows, int64_t c_in, int64_t F, int64_t C) {
+  return pa::f32rows::premlp_supported(dtype, rows, c_in, F, C) ? 1 : 0;
+}
+
+int64_t pa_preprocess_workspace_bytes(int dtype, int64_t rows, int64_t c_in, int64_t F, int64_t C) {
+  if (rows <= 0 || c_in <= 0 || F <= 0 || C <= 0) return PA_ERR_DIMS;
+  if (!pa::f32rows::premlp_supported(dtype, rows, c_in, F, C)) return PA_ERR_UNSUPPORTED;
+  return round_up(pa::f32rows::premlp_blob_bytes(F), 256);
+}
+
+int pa_preprocess_forward(int dtype, int64_t rows, int64_t c_in, int64_t F, int64_t C, const pa_mlp_params *p,
+                          const void *u, void *y, const pa_block_tail *tail, void *workspace, int64_t workspace_bytes,
+                          void *stream) {
+  if (rows <= 0 || c_in <= 0 || F <= 0 || C <= 0) return PA_ERR_DIMS;
+  if (!pa::f32rows::premlp_supported(dtype, rows, c_in, F, C)) return PA_ERR_UNSUPPORTED;
+  if (!p || !p->w1 || !p->b1 || !p->w2 || !p->b2 || !u || !y || !workspace) return PA_ERR_NULL;
+  if (!aligned16(p->w2) || !aligned16(y) || !aligned16(workspace)) return PA_ERR_ALIGN;
+  int rc = check_tail(tail);
+  if (rc) return rc;
+  if (workspace_bytes < pa::f32rows::premlp_blob_bytes(F)) return PA_ERR_WORKSPACE;
+  return pa::f32rows::premlp_forward(rows, c_in, F, p->w1, p->b1, p->w2, p->b2, u, y, tail_active(tail) ? tail : nullptr,
+                                     workspace, static_cast<hipStream_t>(stream));
+}
+
 int pa_mfma_layer_forward(const pa_shape *shape, const pa_params *p, const void *blob, const void *x, void *y,
                           const pa_block_tail *tail, float *slice_token_out, void *workspace, int64_t workspace_bytes,
                           void *stream) {

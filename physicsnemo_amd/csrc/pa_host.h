@@ -131,6 +131,12 @@ int64_t mlp_blob_bytes(int64_t F);
 int mlp_pack(int64_t F, const void *w1, const void *w2, void *blob, hipStream_t st);
 int mlp_forward(int64_t rows, int64_t F, const void *blob, const float *b1, const float *b2, const void *u, void *y,
                 const pa_block_tail *tail, hipStream_t st);
+// the model's preprocess Mlp, Linear(c_in -> F) -> GELU -> Linear(F -> 128), c_in <= 8, with the tail (the first
+// LayerNorm); blob: premlp_blob_bytes(F) of scratch
+bool premlp_supported(int dtype, int64_t rows, int64_t c_in, int64_t F, int64_t C);
+int64_t premlp_blob_bytes(int64_t F);
+int premlp_forward(int64_t rows, int64_t c_in, int64_t F, const void *w1, const float *b1, const void *w2,
+                   const float *b2, const void *u, void *y, const pa_block_tail *tail, void *blob, hipStream_t st);
 }  // namespace f32rows
 
 namespace backward {

@@ -153,9 +153,6 @@ __global__ __launch_bounds__(256) void deslice_linear_kernel(const u32x4 *__rest
   const int n0 = (gblk * 4 + wave) * 32;
   const int n = min(n0 + i, N - 1);
   const bool ok = n0 + i < N;
-#pragma unroll
-  for (int u = 0; u < 8; ++u)
-    load_3k_to_lds(blob + u * kUnit + wave * 192, lane * 16, (unsigned)(uintptr_t)(wout + u * kUnit + wave * 192));
   stage_gamma_beta(gb, tail, tid);
   // the batch's tokens as block-diagonal A operands
   const float *tok = out_token + (int64_t)b * kH * kS * kD;
@@ -173,6 +170,31 @@ __global__ __launch_bounds__(256) void deslice_linear_kernel(const u32x4 *__rest
 #pragma unroll
     for (int p = 0; p < 3; ++p) tokp[(pk * 3 + p) * 64 + l] = pl[p];
   }
+  // this lane's half of its point's weights (two runs of 8 per head), and the output bias
+  float wr[4][4][8];  // [head pair][kk][j]
+  {
+    const float *wrow = w + ((int64_t)b * N + n) * (kH * kS) + 8 * g;
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int kk = 0; kk < 4; ++kk) {
+        const float4 *src = reinterpret_cast<const float4 *>(wrow + 64 * t + 16 * kk);
+        const float4 lo = src[0], hi = src[1];
+        wr[t][kk][0] = lo.x, wr[t][kk][1] = lo.y, wr[t][kk][2] = lo.z, wr[t][kk][3] = lo.w;
+        wr[t][kk][4] = hi.x, wr[t][kk][5] = hi.y, wr[t][kk][6] = hi.z, wr[t][kk][7] = hi.w;
+      }
+  }
+  f32x16 yT[4];
+#pragma unroll
+  for (int t = 0; t < 4; ++t)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) yT[t][r] = b_out ? b_out[32 * t + rowmap(r, g)] : 0.f;
+  // Every load above is complete (the builtin, so that the compiler knows it too) before W_out is requested: from here
+  // on vmcnt counts this wave's 24 requests only, and the first product runs while they land.
+  __builtin_amdgcn_s_waitcnt(0x0F70);
+#pragma unroll
+  for (int u = 0; u < 8; ++u)
+    load_3k_to_lds(blob + u * kUnit + wave * 192, lane * 16, (unsigned)(uintptr_t)(wout + u * kUnit + wave * 192));
   __syncthreads();
   // out_x^T: the four head pairs take turns
   f32x16 ox[4];
@@ -180,17 +202,11 @@ __global__ __launch_bounds__(256) void deslice_linear_kernel(const u32x4 *__rest
   for (int t = 0; t < 4; ++t)
 #pragma unroll
     for (int r = 0; r < 16; ++r) ox[t][r] = 0.f;
-  const float *wrow = w + ((int64_t)b * N + n) * (kH * kS) + 8 * g;
 #pragma unroll
   for (int kk = 0; kk < 4; ++kk) {
     u32x4 bp[4][3];
 #pragma unroll
-    for (int t = 0; t < 4; ++t) {
-      const float4 *src = reinterpret_cast<const float4 *>(wrow + 64 * t + 16 * kk);
-      const float4 lo = src[0], hi = src[1];
-      const float e[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-      split8(e, bp[t]);
-    }
+    for (int t = 0; t < 4; ++t) split8(wr[t][kk], bp[t]);
     constexpr int pw[6] = {0, 1, 0, 1, 2, 0}, pa[6] = {0, 0, 1, 1, 0, 2};
 #pragma unroll
     for (int q = 0; q < 6; ++q)
@@ -198,20 +214,22 @@ __global__ __launch_bounds__(256) void deslice_linear_kernel(const u32x4 *__rest
       for (int t = 0; t < 4; ++t)
         ox[t] = mma(tokp[((t * 4 + kk) * 3 + pw[q]) * 64 + lane], bp[t][pa[q]], ox[t]);
   }
-  // y^T = W_out out_x^T + b_out
-  f32x16 yT[4];
-#pragma unroll
-  for (int t = 0; t < 4; ++t)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) yT[t][r] = b_out ? b_out[32 * t + rowmap(r, g)] : 0.f;
-  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's share of W_out has landed
-  __syncthreads();
-#pragma unroll
-  for (int ks = 0; ks < 8; ++ks) {
+  // y^T = W_out out_x^T + b_out; unit ks is needed at step ks: the 3 (7 - ks) younger requests may still be in flight
+  static_for<8>([&](auto ks_) {
+    constexpr int ks = decltype(ks_)::value;
+    if constexpr (ks == 0) asm volatile("s_waitcnt vmcnt(21)" ::: "memory");
+    if constexpr (ks == 1) asm volatile("s_waitcnt vmcnt(18)" ::: "memory");
+    if constexpr (ks == 2) asm volatile("s_waitcnt vmcnt(15)" ::: "memory");
+    if constexpr (ks == 3) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
+    if constexpr (ks == 4) asm volatile("s_waitcnt vmcnt(9)" ::: "memory");
+    if constexpr (ks == 5) asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
+    if constexpr (ks == 6) asm volatile("s_waitcnt vmcnt(3)" ::: "memory");
+    if constexpr (ks == 7) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
     u32x4 bp[3];
     split_half(ox[ks >> 1], ks & 1, bp);
     kstep(yT, wout + ks * kUnit + lane, bp);
-  }
+  });
   finish_rows(yT, (int64_t)b * N + n, ok, g, tail.residual, y, tail.ln_out, gb, tail.eps);
 }
 
@@ -245,7 +263,6 @@ __global__ __launch_bounds__(256) void mlp_kernel(const u32x4 *__restrict__ blob
     else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
   };
-  issue_upto(kMlpRing);
   stage_gamma_beta(gb, tail, tid);
   // the wave's rows: lane (i, g) holds channels 16 ks + 8 g .. + 7 of row i
   float xr[8][8];
@@ -258,43 +275,160 @@ __global__ __launch_bounds__(256) void mlp_kernel(const u32x4 *__restrict__ blob
       xr[ks][4] = hi.x, xr[ks][5] = hi.y, xr[ks][6] = hi.z, xr[ks][7] = hi.w;
     }
   }
-  f32x16 yT[4];
+  f32x16 yT[4], hT[4];
 #pragma unroll
   for (int t = 0; t < 4; ++t)
 #pragma unroll
-    for (int r = 0; r < 16; ++r) yT[t][r] = b2 ? b2[32 * t + rowmap(r, g)] : 0.f;
-  // the compiler too must know these loads are complete before the loop (it cannot see the asynchronous ones)
+    for (int r = 0; r < 16; ++r) {
+      yT[t][r] = b2 ? b2[32 * t + rowmap(r, g)] : 0.f;
+      hT[t][r] = b1 ? b1[32 * t + rowmap(r, g)] : 0.f;
+    }
+  // Every load above is complete (the builtin, so that the compiler knows it too) before the weights are requested:
+  // in the first chunk vmcnt counts this wave's requests only, and the products start while they land.
   __builtin_amdgcn_s_waitcnt(0x0F70);
+  issue_upto(kMlpRing);
+  __syncthreads();
+  // Step j (0 .. 15) of the first chunk needs unit j.  Units 0 .. 11 are requested up front, 12 .. 15 (and, with more
+  // chunks, 16 .. 19) after the first product: with one chunk the younger requests that may stay in flight are units
+  // j + 1 .. 11 during the first product and j + 1 .. 15 during the second.
+  auto wait_first_chunk = [&](auto j_) {
+    constexpr int j = decltype(j_)::value;
+    if (total > kMlpRing + 4) {  // more chunks follow: wait once per product, for all but the 4 youngest units
+      if constexpr (j == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      if constexpr (j == 8) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
+    } else {
+      constexpr int younger = j < 8 ? 3 * (11 - j) : 3 * (15 - j);
+      if constexpr (younger == 33) asm volatile("s_waitcnt vmcnt(33)" ::: "memory");
+      if constexpr (younger == 30) asm volatile("s_waitcnt vmcnt(30)" ::: "memory");
+      if constexpr (younger == 27) asm volatile("s_waitcnt vmcnt(27)" ::: "memory");
+      if constexpr (younger == 24) asm volatile("s_waitcnt vmcnt(24)" ::: "memory");
+      if constexpr (younger == 21) asm volatile("s_waitcnt vmcnt(21)" ::: "memory");
+      if constexpr (younger == 18) asm volatile("s_waitcnt vmcnt(18)" ::: "memory");
+      if constexpr (younger == 15) asm volatile("s_waitcnt vmcnt(15)" ::: "memory");
+      if constexpr (younger == 12) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
+      if constexpr (younger == 9) asm volatile("s_waitcnt vmcnt(9)" ::: "memory");
+      if constexpr (younger == 6) asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
+      if constexpr (younger == 3) asm volatile("s_waitcnt vmcnt(3)" ::: "memory");
+      if constexpr (younger == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
+    __syncthreads();
+  };
   for (int c = 0; c < F / 128; ++c) {
     const int base = 16 * c;
-    f32x16 hT[4];
+    if (c > 0) {
 #pragma unroll
-    for (int t = 0; t < 4; ++t)
+      for (int t = 0; t < 4; ++t)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) hT[t][r] = b1 ? b1[128 * c + 32 * t + rowmap(r, g)] : 0.f;
-    __builtin_amdgcn_s_waitcnt(0x0F70);
-    wait_landed(base + 8);
-#pragma unroll
-    for (int ks = 0; ks < 8; ++ks) {
+        for (int r = 0; r < 16; ++r) hT[t][r] = b1 ? b1[128 * c + 32 * t + rowmap(r, g)] : 0.f;
+      __builtin_amdgcn_s_waitcnt(0x0F70);
+      wait_landed(base + 8);
+    }
+    static_for<8>([&](auto ks_) {
+      constexpr int ks = decltype(ks_)::value;
+      if (c == 0) wait_first_chunk(ks_);
       u32x4 bp[3];
       split8(xr[ks], bp);
       kstep(hT, smem + ((base + ks) % kMlpRing) * kUnit + lane, bp);
-    }
+    });
     __syncthreads();  // the slots of W1's units are free
     issue_upto(base + 8 + kMlpRing);
 #pragma unroll
     for (int t = 0; t < 4; ++t)
 #pragma unroll
       for (int r = 0; r < 16; ++r) hT[t][r] = gelu_erf(hT[t][r]);
-    wait_landed(base + 16);
+    if (c > 0) wait_landed(base + 16);
+    static_for<8>([&](auto ks_) {
+      constexpr int ks = decltype(ks_)::value;
+      if (c == 0) wait_first_chunk(std::integral_constant<int, 8 + ks>{});
+      u32x4 bp[3];
+      split_half(hT[ks >> 1], ks & 1, bp);
+      kstep(yT, smem + ((base + 8 + ks) % kMlpRing) * kUnit + lane, bp);
+    });
+    __syncthreads();  // the slots of W2's units are free
+    issue_upto(base + 16 + kMlpRing);
+  }
+  finish_rows(yT, row, ok, g, tail.residual, y, tail.ln_out, gb, tail.eps);
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// premlp_kernel: the model's preprocess Mlp (TR.py:519-525), Linear(c_in -> F) -> GELU -> Linear(F -> 128) with a few
+// input features per point (coordinates and fields, c_in <= 8), and the first block's LayerNorm as the tail.  The first
+// Linear is c_in multiply-adds per hidden feature on the vector units (its weights sit in LDS, every lane of a half
+// wave reads the same feature's row); the second is mlp_kernel's second product over W2's units, 8 per chunk of 128
+// hidden features.
+// ---------------------------------------------------------------------------------------------------------------
+constexpr int kPreMaxIn = 8;
+
+__global__ __launch_bounds__(256) void pack_premlp_kernel(const float *__restrict__ w2, int F, u32x4 *__restrict__ blob) {
+  const int c = blockIdx.x >> 3, u = blockIdx.x & 7;
+  pack_unit(w2 + c * 128, F, 16 * u, true, blob + (int64_t)blockIdx.x * kUnit, threadIdx.x);
+}
+
+template <int C_IN>
+__global__ __launch_bounds__(256) void premlp_kernel(const u32x4 *__restrict__ blob, const float *__restrict__ w1,
+                                                     const float *__restrict__ b1, const float *__restrict__ b2,
+                                                     const float *__restrict__ u, float *__restrict__ y, Tail tail,
+                                                     int64_t M, int F) {
+  extern __shared__ u32x4 smem[];
+  float *gb = reinterpret_cast<float *>(smem + kMlpRing * kUnit);
+  float *w1s = gb + 2 * kC;  // [input feature 0 .. C_IN - 1 | bias][hidden feature]: (C_IN + 1) * F floats
+  const int tid = threadIdx.x, lane = tid & 63, i = lane & 31, g = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int64_t row0 = ((int64_t)blockIdx.x * 4 + wave) * 32;
+  const int64_t row = min(row0 + i, M - 1);
+  const bool ok = row0 + i < M;
+  const int total = (F / 128) * 8;
+  int issued = 0;
+  auto issue_upto = [&](int upto) {
+    for (; issued < upto && issued < total; ++issued)
+      load_3k_to_lds(blob + (int64_t)issued * kUnit + wave * 192, lane * 16,
+                     (unsigned)(uintptr_t)(smem + (issued % kMlpRing) * kUnit + wave * 192));
+  };
+  stage_gamma_beta(gb, tail, tid);
+  for (int k = tid; k < F * (C_IN + 1); k += 256) {
+    const int j = k / F, f = k - j * F;
+    w1s[k] = j < C_IN ? w1[f * C_IN + j] : (b1 ? b1[f] : 0.f);
+  }
+  float xin[C_IN];
+#pragma unroll
+  for (int j = 0; j < C_IN; ++j) xin[j] = u[row * C_IN + j];
+  f32x16 yT[4];
+#pragma unroll
+  for (int t = 0; t < 4; ++t)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) yT[t][r] = b2 ? b2[32 * t + rowmap(r, g)] : 0.f;
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // the loads above are complete before the weights are requested
+  issue_upto(kMlpRing);
+  __syncthreads();
+  for (int c = 0; c < F / 128; ++c) {
+    f32x16 hT[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {  // the quad's 4 consecutive hidden features
+        const float *wf = w1s + 128 * c + 32 * t + 8 * q + 4 * g;
+        float4 a = *reinterpret_cast<const float4 *>(wf + C_IN * F);
+#pragma unroll
+        for (int j = 0; j < C_IN; ++j) {
+          const float4 wj = *reinterpret_cast<const float4 *>(wf + j * F);
+          a.x = fmaf(xin[j], wj.x, a.x), a.y = fmaf(xin[j], wj.y, a.y);
+          a.z = fmaf(xin[j], wj.z, a.z), a.w = fmaf(xin[j], wj.w, a.w);
+        }
+        hT[t][4 * q] = gelu_erf(a.x), hT[t][4 * q + 1] = gelu_erf(a.y);
+        hT[t][4 * q + 2] = gelu_erf(a.z), hT[t][4 * q + 3] = gelu_erf(a.w);
+      }
+    // units 8 c .. 8 c + 7 have landed for every wave: at most the 4 youngest units stay in flight
+    if (issued - (8 * c + 8) >= 4) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) {
       u32x4 bp[3];
       split_half(hT[ks >> 1], ks & 1, bp);
-      kstep(yT, smem + ((base + 8 + ks) % kMlpRing) * kUnit + lane, bp);
+      kstep(yT, smem + ((8 * c + ks) % kMlpRing) * kUnit + lane, bp);
     }
-    __syncthreads();  // the slots of W2's units are free
-    issue_upto(base + 16 + kMlpRing);
+    __syncthreads();  // the slots of this chunk's units are free
+    issue_upto(8 * c + 8 + kMlpRing);
   }
   finish_rows(yT, row, ok, g, tail.residual, y, tail.ln_out, gb, tail.eps);
 }
@@ -355,6 +489,46 @@ int mlp_forward(int64_t M, int64_t F, const void *blob, const float *b1, const f
   hipLaunchKernelGGL(mlp_kernel, dim3((unsigned)blocks), dim3(256), lds, st, static_cast<const u32x4 *>(blob), b1, b2,
                      static_cast<const float *>(u), static_cast<float *>(y), make_tail(tail), M, (int)F);
   return launch_status();
+}
+
+static size_t premlp_lds(int64_t c_in, int64_t F) {
+  return (size_t)kMlpRing * kUnit * 16 + 2 * kC * 4 + (size_t)F * (c_in + 1) * 4;
+}
+
+bool premlp_supported(int dtype, int64_t M, int64_t c_in, int64_t F, int64_t C) {
+  return dtype == PA_F32 && M > 0 && C == kC && c_in >= 1 && c_in <= kPreMaxIn && F >= 128 && F % 128 == 0 &&
+         premlp_lds(c_in, F) <= 160 * 1024;
+}
+
+int64_t premlp_blob_bytes(int64_t F) { return (F / 128) * 8 * (int64_t)kUnit * 16; }
+
+int premlp_forward(int64_t M, int64_t c_in, int64_t F, const void *w1, const float *b1, const void *w2, const float *b2,
+                   const void *u, void *y, const pa_block_tail *tail, void *blob, hipStream_t st) {
+  hipLaunchKernelGGL(pack_premlp_kernel, dim3((unsigned)((F / 128) * 8)), dim3(256), 0, st,
+                     static_cast<const float *>(w2), (int)F, static_cast<u32x4 *>(blob));
+  int rc = launch_status();
+  if (rc) return rc;
+  const size_t lds = premlp_lds(c_in, F);
+  const int64_t blocks = ((M + 31) / 32 + 3) / 4;
+  auto launch = [&](auto kernel) {
+    int rc2 = allow_dynamic_lds(kernel, lds);
+    if (rc2) return rc2;
+    hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(256), lds, st, static_cast<const u32x4 *>(blob),
+                       static_cast<const float *>(w1), b1, b2, static_cast<const float *>(u), static_cast<float *>(y),
+                       make_tail(tail), M, (int)F);
+    return launch_status();
+  };
+  switch (c_in) {
+    case 1: return launch(premlp_kernel<1>);
+    case 2: return launch(premlp_kernel<2>);
+    case 3: return launch(premlp_kernel<3>);
+    case 4: return launch(premlp_kernel<4>);
+    case 5: return launch(premlp_kernel<5>);
+    case 6: return launch(premlp_kernel<6>);
+    case 7: return launch(premlp_kernel<7>);
+    case 8: return launch(premlp_kernel<8>);
+    default: return PA_ERR_UNSUPPORTED;
+  }
 }
 
 }  // namespace f32rows

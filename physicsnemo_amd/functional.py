@@ -302,6 +302,35 @@ def mlp_forward(u, w1, b1, w2, b2, residual=None, ln_weight=None, ln_bias=None, 
     return y if ln_out is None else (y, ln_out)
 
 
+def preprocess_supported(dtype: torch.dtype, rows: int, c_in: int, F: int, C: int) -> bool:
+    """True if `preprocess_forward` serves the shape (float32, C = 128, up to 8 input features, F a multiple of 128)."""
+    if dtype != torch.float32:
+        return False
+    return bool(_lib.load().pa_preprocess_query(_lib.PA_F32, rows, c_in, F, C))
+
+
+def preprocess_forward(u, w1, b1, w2, b2, ln_weight=None, ln_bias=None, ln_eps=1e-5):
+    """The model's preprocess Mlp in one launch: y = w2 . gelu(w1 . u + b1) + b2 for u (..., c_in) with a few input
+    features per point; returns y, or (y, LayerNorm(y)) when ln_weight is given."""
+    _need_cuda(u, w1, b1, w2, b2, ln_weight, ln_bias)
+    lib = _lib.load()
+    c_in, F, C = w1.shape[1], w1.shape[0], w2.shape[0]
+    rows = u.numel() // c_in
+    code = _lib.dtype_code(u.dtype)
+    nbytes = lib.pa_preprocess_workspace_bytes(code, rows, c_in, F, C)
+    if nbytes < 0:
+        _lib.check(int(nbytes), "pa_preprocess_workspace_bytes")
+    workspace = torch.empty(int(nbytes), dtype=torch.uint8, device=u.device)
+    y = torch.empty(*u.shape[:-1], C, dtype=u.dtype, device=u.device)
+    ln_out = torch.empty_like(y) if ln_weight is not None else None
+    params = _lib.PaMlpParams(_lib.ptr(w1), _lib.ptr(b1), _lib.ptr(w2), _lib.ptr(b2))
+    tail = _c_tail(None, ln_weight, ln_bias, ln_eps, ln_out)
+    _lib.check(lib.pa_preprocess_forward(code, rows, c_in, F, C, byref(params), u.data_ptr(), y.data_ptr(), byref(tail),
+                                         workspace.data_ptr(), int(nbytes), _lib.current_stream_ptr(u.device)),
+               "pa_preprocess_forward")
+    return y if ln_out is None else (y, ln_out)
+
+
 def mlp_pack(w1, w2):
     """The two weights of the MLP in the fused kernel's operand order: one call per parameter set; the result is the
     `packed` argument of mlp_forward_packed.  w1 (F, C), w2 (C, F) bfloat16 or float32."""

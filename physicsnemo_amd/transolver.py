@@ -373,12 +373,25 @@ class Transolver(nn.Module):
         fx = torch.cat((embedding.to(fx.dtype), fx), -1)  # embedding first, then the functional input (:716)
         on_library = self._glue_on_library(fx)
         normed = None
+        first_ln_done = False
         if on_library:
             # preprocess Mlp (Linear -> GELU -> Linear, :519-525) and the first block's LayerNorm on the library kernels
             if torch.is_autocast_enabled("cuda"):
                 fx = fx.to(torch.get_autocast_dtype("cuda"))
             lin1, lin2 = self.preprocess.layers[0], self.preprocess.layers[2]
-            if lin2.in_features <= 512:  # the weights-stationary row kernel holds up to 512 input features
+            rows = fx.numel() // fx.shape[-1]
+            if (time is None and len(self.preprocess.layers) == 3 and fx.dtype == torch.float32 and
+                    PF.preprocess_supported(fx.dtype, rows, lin1.in_features, lin1.out_features, lin2.out_features)):
+                # float32 at hidden 128: both Linears, the GELU and the first block's LayerNorm in one launch
+                ln = self.blocks[0].ln_1
+                f32 = dict(device=fx.device, dtype=torch.float32)
+                fx, normed = PF.preprocess_forward(
+                    fx.contiguous(), lin1.weight.detach().to(**f32).contiguous(), lin1.bias.detach().to(**f32).contiguous(),
+                    lin2.weight.detach().to(**f32).contiguous(), lin2.bias.detach().to(**f32).contiguous(),
+                    ln_weight=ln.weight.detach().float().contiguous(), ln_bias=ln.bias.detach().float().contiguous(),
+                    ln_eps=ln.eps)
+                first_ln_done = True
+            elif lin2.in_features <= 512:  # the weights-stationary row kernel holds up to 512 input features
                 fx = self._library_linear(self._library_linear(fx.contiguous(), lin1, gelu=True), lin2)
             else:
                 fx = self.preprocess(fx).contiguous()
@@ -389,7 +402,7 @@ class Transolver(nn.Module):
             # :721-725 repeats first; the arithmetic per token is the same)
             time_emb = self.time_fc(self.time_embed(time.to(torch.float32)))
             fx = (fx + time_emb.to(fx.dtype).unsqueeze(1)).contiguous()
-        if on_library:
+        if on_library and not first_ln_done:
             ln = self.blocks[0].ln_1
             fx, normed = PF.residual_layernorm(fx, ln_weight=ln.weight.detach().float().contiguous(),
                                                ln_bias=ln.bias.detach().float().contiguous(), ln_eps=ln.eps)

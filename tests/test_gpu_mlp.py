@@ -140,3 +140,30 @@ def test_mlp_fp32_matches_oracle(rows_shape, Fh):
 def test_mlp_fp32_unsupported_shapes():
     assert not PF.mlp_supported(torch.float32, 100, 256, 1024)  # float32 is served at C = 128 only
     assert not PF.mlp_supported(torch.float32, 100, 128, 192)   # hidden features in chunks of 128
+
+
+@pytest.mark.parametrize("rows_shape,c_in,Fh", [((4, 7225), 3, 256), ((1, 100), 1, 128), ((2, 333), 7, 256), ((1, 5000), 8, 384)])
+def test_preprocess_mlp_fp32_matches_oracle(rows_shape, c_in, Fh):
+    # the model's preprocess Mlp (a few input features per point -> F -> 128) and the first LayerNorm in one launch
+    announce("preprocess mlp fp32", rows_shape, c_in, Fh)
+    C = 128
+    torch.manual_seed(2)
+    ref = to.OracleMlp(c_in, Fh, C).eval()
+    u = torch.randn(*rows_shape, c_in)
+    gamma, beta = torch.rand(C) + 0.5, torch.randn(C) * 0.1
+    dev = torch.device("cuda:0")
+    args = dict(u=u.to(dev), w1=ref.layers[0].weight.detach().to(dev).contiguous(), b1=ref.layers[0].bias.detach().to(dev),
+                w2=ref.layers[2].weight.detach().to(dev).contiguous(), b2=ref.layers[2].bias.detach().to(dev))
+    assert PF.preprocess_supported(torch.float32, u.numel() // c_in, c_in, Fh, C)
+    with torch.no_grad():
+        want = ref(u)
+        want_ln = F.layer_norm(want, (C,), gamma, beta, 1e-5)
+        y = PF.preprocess_forward(**args)
+        y2, ln2 = PF.preprocess_forward(**args, ln_weight=gamma.to(dev), ln_bias=beta.to(dev))
+    assert y.shape == (*rows_shape, C) and y.dtype == torch.float32
+    assert_fp32_close(y, want, "preprocess mlp output")
+    assert_fp32_close(ln2, want_ln, "LayerNorm(preprocess mlp)")
+    assert torch.equal(y2, y)
+    assert not PF.preprocess_supported(torch.float32, 100, 9, 256, C)
+    assert not PF.preprocess_supported(torch.float32, 100, 8, 512, C)  # the first Linear no longer fits beside the ring
+    assert not PF.preprocess_supported(torch.float32, 100, 3, 256, 256)
