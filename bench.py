@@ -383,7 +383,9 @@ def time_full_model(name, B, N, functional_dim, points, slice_num, n_layers, ste
 
 def time_structured_model(steps=5, warmup=2):
     """cfg1: Transolver on a structured 85 x 85 grid (Conv2d k = 3 projections), fp32, 4 layers, hidden 128, 8 heads,
-    32 slices, mlp_ratio 1, batch 4 -> Mpoints/s.  Served by the general (fp32) kernels."""
+    32 slices, mlp_ratio 1, batch 4 -> Mpoints/s.  Served by the float32 kernels of this shape class: the structured
+    front end, the row kernels (hand-back + out_linear + tail, block MLP, preprocess MLP) and the general combine /
+    slice-attention kernels."""
     import torch
 
     import physicsnemo_amd as pn
@@ -409,13 +411,15 @@ def time_structured_model(steps=5, warmup=2):
     with torch.no_grad():
         dt, out = timed(lambda: model(fx, pos))
         assert torch.isfinite(out).all()
-        # 28 900 points per forward: the eager call is bound by its ~50 kernel submissions; the same forward replayed
-        # from a HIP graph is one submission
+        # 28 900 points per forward in 24 kernel submissions; the same forward replayed from a HIP graph is one
         graphed = pn.GraphedForward(model, fx, pos)
         dt_graph, out = timed(graphed.replay)
         assert torch.isfinite(out).all()
     return {"workload": "cfg1: Transolver structured 2D 85x85 (conv k=3), fp32, 4 layers", "batch": 4, "points": 7225,
-            "layers": 4, "slice_num": 32, "ms_per_forward": round(dt * 1e3, 3),
+            "layers": 4, "slice_num": 32,
+            "arithmetic": "float32 storage and accumulation; matrix products as six bf16 MFMA products of three-way "
+                          "split operands (error vs float64 as small as with float32 matrix instructions)",
+            "ms_per_forward": round(dt * 1e3, 3),
             "mpoints_per_s": round(4 * 7225 / dt / 1e6, 2), "ms_per_forward_graph": round(dt_graph * 1e3, 3),
             "mpoints_per_s_graph": round(4 * 7225 / dt_graph / 1e6, 2)}
 
