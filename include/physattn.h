@@ -449,6 +449,35 @@ int pa_mlp_pack(int dtype, int64_t C, int64_t F, const pa_mlp_params *p, void *p
 int pa_mlp_forward_packed(int dtype, int64_t rows, int64_t C, int64_t F, const void *packed, const float *b1,
                           const float *b2, const void *u, void *y, const pa_block_tail *tail, void *stream);
 
+/* ---- whole block ------------------------------------------------------------------------------ */
+
+/* The rest of TransolverBlock.forward behind the attention layer (TR.py:300-303): LayerNorm ln_mlp1[0] and
+ * Mlp ln_mlp1[1] (C -> F -> C, GELU erf); torch layouts, weights in the activation dtype. */
+typedef struct pa_block_mlp {
+  const float *ln_gamma; /* (C) */
+  const float *ln_beta;  /* (C) */
+  float ln_eps;
+  const void *w1;        /* (F, C) */
+  const float *b1;       /* (F) */
+  const void *w2;        /* (C, F) */
+  const float *b2;       /* (C) */
+  int64_t F;
+} pa_block_mlp;
+
+/* Replaces TransolverBlock.forward (TR.py:296-303) for a block that is not the last one, and the part of the last
+ * block before its output head:
+ *   fx1 = Attn(x) + fx_in;  fx_out = Mlp(LayerNorm(fx1)) + fx1;  next->ln_out = LayerNorm_next(fx_out)
+ * x (B,N,C) is LayerNorm_1(fx_in), which the caller has from the block before (or pa_preprocess_forward);
+ * next: ln_gamma / ln_beta / ln_eps / ln_out of the LayerNorm that follows (ln_1 of the next block, or ln_mlp2[0]),
+ * residual must be NULL; next may be NULL.  fx1 and its LayerNorm are never stored.
+ * Served where pa_block_query() is 1: float32, C = 128, 8 heads of 16, 32 slices, F a multiple of 128 (up to 1024).
+ * workspace: pa_block_workspace_bytes(). */
+int pa_block_query(int dtype, const pa_shape *shape, int64_t F);
+int64_t pa_block_workspace_bytes(int dtype, const pa_shape *shape, int64_t F);
+int pa_block_forward(int dtype, const pa_shape *shape, const pa_params *p, const pa_block_mlp *mlp, const void *x,
+                     const void *fx_in, void *fx_out, const pa_block_tail *next, void *workspace,
+                     int64_t workspace_bytes, void *stream);
+
 /* The model's preprocess Mlp (TR.py:519-525 with mlp_layers.py:139-173): Linear(c_in -> F) -> GELU(erf) -> Linear(F -> C)
  * over `rows` rows of u (rows, c_in), c_in = coordinates + fields per point; with a tail, tail->ln_out is the first
  * block's LayerNorm of the result (TR.py:300).  Served for float32, C = 128, c_in <= 8, F a multiple of 128

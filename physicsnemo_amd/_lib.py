@@ -35,6 +35,7 @@ EXPORTED = [
     "pa_mfma_layer_forward", "pa_rows_gemm_act", "pa_layernorm_backward_groups", "pa_layernorm_backward",
     "pa_static_scratch_bytes", "pa_slice_reduce_static",
     "pa_preprocess_query", "pa_preprocess_workspace_bytes", "pa_preprocess_forward",
+    "pa_block_query", "pa_block_workspace_bytes", "pa_block_forward",
 ]
 
 PA_BUF_BLOB, PA_BUF_FX_PACK, PA_BUF_W_PACK, PA_BUF_PARTIALS, PA_BUF_TOKP = range(5)
@@ -54,6 +55,11 @@ class PaParams(Structure):
 
 class PaMlpParams(Structure):
     _fields_ = [(n, c_void_p) for n in ("w1", "b1", "w2", "b2")]
+
+
+class PaBlockMlp(Structure):
+    _fields_ = [("ln_gamma", c_void_p), ("ln_beta", c_void_p), ("ln_eps", c_float), ("w1", c_void_p), ("b1", c_void_p),
+                ("w2", c_void_p), ("b2", c_void_p), ("F", c_int64)]
 
 
 class PaPlusParams(Structure):
@@ -140,6 +146,13 @@ def load() -> ctypes.CDLL:
     lib.pa_mlp_forward.restype = c_int
     lib.pa_mlp_forward.argtypes = [c_int, c_int64, c_int64, c_int64, POINTER(PaMlpParams), c_void_p, c_void_p, pt, c_void_p,
                                    c_int64, c_void_p]
+    lib.pa_block_query.restype = c_int
+    lib.pa_block_query.argtypes = [c_int, ps, c_int64]
+    lib.pa_block_workspace_bytes.restype = c_int64
+    lib.pa_block_workspace_bytes.argtypes = [c_int, ps, c_int64]
+    lib.pa_block_forward.restype = c_int
+    lib.pa_block_forward.argtypes = [c_int, ps, POINTER(PaParams), POINTER(PaBlockMlp), c_void_p, c_void_p, c_void_p, pt,
+                                     c_void_p, c_int64, c_void_p]
     lib.pa_preprocess_query.restype = c_int
     lib.pa_preprocess_query.argtypes = [c_int, c_int64, c_int64, c_int64, c_int64]
     lib.pa_preprocess_workspace_bytes.restype = c_int64

@@ -1057,6 +1057,52 @@ int pa_layer_forward(int dtype, const pa_shape *shape, const pa_params *p, const
   return rc;
 }
 
+int pa_block_query(int dtype, const pa_shape *shape, int64_t F) {
+  if (check_shape(dtype, shape)) return 0;
+  return pa::f32rows::block_supported(dtype, *shape, F) ? 1 : 0;
+}
+
+int64_t pa_block_workspace_bytes(int dtype, const pa_shape *shape, int64_t F) {
+  int rc = check_shape(dtype, shape);
+  if (rc) return rc;
+  if (!pa::f32rows::block_supported(dtype, *shape, F)) return PA_ERR_UNSUPPORTED;
+  return plan_general(dtype, *shape).total + round_up(pa::f32rows::block_blob_bytes(F), 256);
+}
+
+int pa_block_forward(int dtype, const pa_shape *shape, const pa_params *p, const pa_block_mlp *mlp, const void *x,
+                     const void *fx_in, void *fx_out, const pa_block_tail *next, void *workspace,
+                     int64_t workspace_bytes, void *stream) {
+  int rc = check_shape(dtype, shape);
+  if (rc) return rc;
+  if ((rc = check_params(p))) return rc;
+  if (!mlp || !mlp->ln_gamma || !mlp->ln_beta || !mlp->w1 || !mlp->b1 || !mlp->w2 || !mlp->b2) return PA_ERR_NULL;
+  if (!x || !fx_in || !fx_out || !workspace) return PA_ERR_NULL;
+  if (!aligned16(x) || !aligned16(fx_in) || !aligned16(fx_out) || !aligned16(workspace) || !aligned16(mlp->w1) ||
+      !aligned16(mlp->w2))
+    return PA_ERR_ALIGN;
+  if ((rc = check_tail(next))) return rc;
+  if (next && next->residual) return PA_ERR_UNSUPPORTED;  // the block's own residual is fx1
+  const pa_shape &s = *shape;
+  if (!pa::f32rows::block_supported(dtype, s, mlp->F)) return PA_ERR_UNSUPPORTED;
+  const GeneralPlan plan = plan_general(dtype, s);
+  if (workspace_bytes < plan.total + pa::f32rows::block_blob_bytes(mlp->F)) return PA_ERR_WORKSPACE;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  char *ws = static_cast<char *>(workspace);
+  void *x_mid = ws + plan.off_x_mid, *fx_mid = ws + plan.off_fx_mid, *w = ws + plan.off_w;
+  float *partials = reinterpret_cast<float *>(ws + plan.off_partials);
+  float *tok = reinterpret_cast<float *>(ws + plan.off_tok), *norm = reinterpret_cast<float *>(ws + plan.off_norm);
+  float *tok_out = reinterpret_cast<float *>(ws + plan.off_tok_out);
+  if (plan.conv_front) {
+    if ((rc = pa::conv::front(s, *p, x, ws + plan.off_blob, w, partials, nullptr, st))) return rc;
+  } else {
+    if ((rc = pa::general::project_inputs(dtype, s, *p, x, x_mid, fx_mid, st))) return rc;
+    if ((rc = pa::general::slice_softmax(dtype, s, *p, x_mid, w, st))) return rc;
+    if ((rc = pa::general::slice_partial(dtype, s, w, fx_mid, partials, st))) return rc;
+  }
+  if ((rc = pa::general::combine_attention(s, *p, partials, plan.G, tok, norm, tok_out, st))) return rc;
+  return pa::f32rows::block_tail(s, *p, *mlp, w, tok_out, fx_in, fx_out, next, ws + plan.total, st);
+}
+
 // Workspace plan of the FLARE layer on the MFMA kernels.
 struct FlarePlan {
   int64_t off_scores, off_v, off_wc, off_wr, off_partials, off_z, off_tokp, off_colmax, off_cmpart, off_out_x, total;

@@ -351,6 +351,211 @@ __global__ __launch_bounds__(256) void mlp_kernel(const u32x4 *__restrict__ blob
 }
 
 // ---------------------------------------------------------------------------------------------------------------
+// block_tail_kernel: everything of a block that is local to a point, after the slice attention (TR.py:300-303):
+//   out_x = w . out_token;  fx1 = out_x W_out^T + b_out + fx_in;  n = LayerNorm_2(fx1);
+//   fx_out = W2 gelu(W1 n + b1) + b2 + fx1;  next_ln_out = LayerNorm_next(fx_out)
+// = deslice_linear_kernel followed by mlp_kernel with the rows staying in registers in between (fx1 and its
+// LayerNorm are never stored).  Weight stream: W_out (units 0 .. 7), then per chunk of 128 hidden features W1's rows
+// and W2's columns (8 units each, both with the reduction index in register order); ring of 12 units whose last four
+// slots first hold the batch's slice tokens as A operands.  LDS behind the ring: gamma | beta of both LayerNorms and
+// the three biases.
+// ---------------------------------------------------------------------------------------------------------------
+struct BlockArgs {
+  const float *b_out, *w, *out_token, *fx_in;
+  const float *ln2_gamma, *ln2_beta;
+  float ln2_eps;
+  const float *b1, *b2;
+  float *fx_out;
+  Tail next;  // residual unused
+};
+
+__global__ __launch_bounds__(256) void pack_block_kernel(const float *__restrict__ w_out, const float *__restrict__ w1,
+                                                         const float *__restrict__ w2, int F, u32x4 *__restrict__ blob) {
+  u32x4 *unit = blob + (int64_t)blockIdx.x * kUnit;
+  if (blockIdx.x < 8) {
+    pack_unit(w_out, kC, 16 * blockIdx.x, true, unit, threadIdx.x);
+    return;
+  }
+  const int q = blockIdx.x - 8, c = q >> 4, u = q & 15;
+  if (u < 8) pack_unit(w1 + (int64_t)c * 128 * kC, kC, 16 * u, true, unit, threadIdx.x);
+  else pack_unit(w2 + c * 128, F, 16 * (u - 8), true, unit, threadIdx.x);
+}
+
+__global__ __launch_bounds__(256) void block_tail_kernel(const u32x4 *__restrict__ blob, BlockArgs a, int N, int bpb, int F) {
+  extern __shared__ u32x4 smem[];
+  u32x4 *tokp = smem + 8 * kUnit;  // [pair][kk][piece][lane], in ring slots 8 .. 11 until the hand-back is done
+  float *gb2 = reinterpret_cast<float *>(smem + kMlpRing * kUnit);  // gamma | beta of LayerNorm_2
+  float *gbn = gb2 + 2 * kC;                                        // gamma | beta of the next LayerNorm
+  float *bo = gbn + 2 * kC, *bb2 = bo + kC, *bb1 = bb2 + kC;        // b_out, b2, b1 (F)
+  const int tid = threadIdx.x, lane = tid & 63, i = lane & 31, g = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int b = blockIdx.x / bpb, gblk = blockIdx.x - b * bpb;
+  const int n0 = (gblk * 4 + wave) * 32;
+  const int n = min(n0 + i, N - 1);
+  const bool ok = n0 + i < N;
+  const int64_t row = (int64_t)b * N + n;
+  const int total = 8 + (F / 128) * 16;
+  int issued = 0;
+  auto issue_upto = [&](int upto) {
+    for (; issued < upto && issued < total; ++issued)
+      load_3k_to_lds(blob + (int64_t)issued * kUnit + wave * 192, lane * 16,
+                     (unsigned)(uintptr_t)(smem + (issued % kMlpRing) * kUnit + wave * 192));
+  };
+  auto wait_landed = [&](int upto) {  // units below `upto` have landed for every wave (4 younger units may be in flight)
+    if (issued - upto >= 4) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+  };
+  if (tid < kC) {
+    gb2[tid] = a.ln2_gamma[tid];
+    gb2[kC + tid] = a.ln2_beta[tid];
+    gbn[tid] = a.next.gamma ? a.next.gamma[tid] : 1.f;
+    gbn[kC + tid] = a.next.beta ? a.next.beta[tid] : 0.f;
+    bo[tid] = a.b_out ? a.b_out[tid] : 0.f;
+    bb2[tid] = a.b2 ? a.b2[tid] : 0.f;
+  }
+  for (int k = tid; k < F; k += 256) bb1[k] = a.b1 ? a.b1[k] : 0.f;
+  // the batch's tokens as block-diagonal A operands (deslice_linear_kernel)
+  const float *tok = a.out_token + (int64_t)b * kH * kS * kD;
+  for (int item = tid; item < 16 * 64; item += 256) {
+    const int pk = item >> 6, l = item & 63, li = l & 31, lg = l >> 5;
+    const int pair = pk >> 2, kk = pk & 3, hh = li >> 4, d = li & 15;
+    float e[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int k = 16 * kk + 8 * lg + j;
+      e[j] = (k >> 5) == hh ? tok[((2 * pair + hh) * kS + (k & 31)) * kD + d] : 0.f;
+    }
+    u32x4 pl[3];
+    split8(e, pl);
+#pragma unroll
+    for (int p = 0; p < 3; ++p) tokp[(pk * 3 + p) * 64 + l] = pl[p];
+  }
+  // this lane's half of its point's weights and of its residual row
+  float wr[4][4][8];
+  {
+    const float *wrow = a.w + row * (kH * kS) + 8 * g;
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int kk = 0; kk < 4; ++kk) {
+        const float4 *src = reinterpret_cast<const float4 *>(wrow + 64 * t + 16 * kk);
+        const float4 lo = src[0], hi = src[1];
+        wr[t][kk][0] = lo.x, wr[t][kk][1] = lo.y, wr[t][kk][2] = lo.z, wr[t][kk][3] = lo.w;
+        wr[t][kk][4] = hi.x, wr[t][kk][5] = hi.y, wr[t][kk][6] = hi.z, wr[t][kk][7] = hi.w;
+      }
+  }
+  f32x16 fx1[4];  // first the residual, then fx1
+#pragma unroll
+  for (int t = 0; t < 4; ++t)
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const float4 r = *reinterpret_cast<const float4 *>(a.fx_in + row * kC + 32 * t + 8 * q + 4 * g);
+      fx1[t][4 * q] = r.x, fx1[t][4 * q + 1] = r.y, fx1[t][4 * q + 2] = r.z, fx1[t][4 * q + 3] = r.w;
+    }
+  // every load above is complete (the builtin, so that the compiler knows it too) before the weights are requested
+  __builtin_amdgcn_s_waitcnt(0x0F70);
+  issue_upto(8);
+  __syncthreads();
+  // out_x^T: the four head pairs take turns
+  f32x16 ox[4];
+#pragma unroll
+  for (int t = 0; t < 4; ++t)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) ox[t][r] = 0.f;
+#pragma unroll
+  for (int kk = 0; kk < 4; ++kk) {
+    u32x4 bp[4][3];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) split8(wr[t][kk], bp[t]);
+    constexpr int pw[6] = {0, 1, 0, 1, 2, 0}, pa[6] = {0, 0, 1, 1, 0, 2};
+#pragma unroll
+    for (int q = 0; q < 6; ++q)
+#pragma unroll
+      for (int t = 0; t < 4; ++t)
+        ox[t] = mma(tokp[((t * 4 + kk) * 3 + pw[q]) * 64 + lane], bp[t][pa[q]], ox[t]);
+  }
+  __syncthreads();  // the tokens are used up: their slots join the ring
+  issue_upto(kMlpRing);
+  // fx1 = W_out out_x^T + b_out + fx_in
+#pragma unroll
+  for (int t = 0; t < 4; ++t)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) fx1[t][r] += bo[32 * t + rowmap(r, g)];
+  wait_landed(8);
+#pragma unroll
+  for (int ks = 0; ks < 8; ++ks) {
+    u32x4 bp[3];
+    split_half(ox[ks >> 1], ks & 1, bp);
+    kstep(fx1, smem + ks * kUnit + lane, bp);
+  }
+  __syncthreads();  // W_out's slots are free
+  issue_upto(8 + kMlpRing);
+  // n = LayerNorm_2(fx1), in registers
+  f32x16 nT[4];
+  {
+    float sum = 0.f;
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) sum += fx1[t][r];
+    const float mean = half_sum(sum) * (1.f / kC);
+    float sq = 0.f;
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const float d = fx1[t][r] - mean;
+        sq = fmaf(d, d, sq);
+      }
+    const float rstd = 1.f / sqrtf(half_sum(sq) * (1.f / kC) + a.ln2_eps);
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int c = 32 * t + rowmap(r, g);
+        nT[t][r] = (fx1[t][r] - mean) * rstd * gb2[c] + gb2[kC + c];
+      }
+  }
+  // the MLP; its second product accumulates on top of fx1 + b2
+#pragma unroll
+  for (int t = 0; t < 4; ++t)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) fx1[t][r] += bb2[32 * t + rowmap(r, g)];
+  for (int c = 0; c < F / 128; ++c) {
+    const int base = 8 + 16 * c;
+    f32x16 hT[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) hT[t][r] = bb1[128 * c + 32 * t + rowmap(r, g)];
+    wait_landed(base + 8);
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) {
+      u32x4 bp[3];
+      split_half(nT[ks >> 1], ks & 1, bp);
+      kstep(hT, smem + ((base + ks) % kMlpRing) * kUnit + lane, bp);
+    }
+    __syncthreads();  // the slots of W1's units are free
+    issue_upto(base + 8 + kMlpRing);
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) hT[t][r] = gelu_erf(hT[t][r]);
+    wait_landed(base + 16);
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) {
+      u32x4 bp[3];
+      split_half(hT[ks >> 1], ks & 1, bp);
+      kstep(fx1, smem + ((base + 8 + ks) % kMlpRing) * kUnit + lane, bp);
+    }
+    __syncthreads();  // the slots of W2's units are free
+    issue_upto(base + 16 + kMlpRing);
+  }
+  finish_rows(fx1, row, ok, g, nullptr, a.fx_out, a.next.ln_out, gbn, a.next.eps);
+}
+
+// ---------------------------------------------------------------------------------------------------------------
 // premlp_kernel: the model's preprocess Mlp (TR.py:519-525), Linear(c_in -> F) -> GELU -> Linear(F -> 128) with a few
 // input features per point (coordinates and fields, c_in <= 8), and the first block's LayerNorm as the tail.  The first
 // Linear is c_in multiply-adds per hidden feature on the vector units (its weights sit in LDS, every lane of a half
@@ -488,6 +693,42 @@ int mlp_forward(int64_t M, int64_t F, const void *blob, const float *b1, const f
   const int64_t blocks = ((M + 31) / 32 + 3) / 4;
   hipLaunchKernelGGL(mlp_kernel, dim3((unsigned)blocks), dim3(256), lds, st, static_cast<const u32x4 *>(blob), b1, b2,
                      static_cast<const float *>(u), static_cast<float *>(y), make_tail(tail), M, (int)F);
+  return launch_status();
+}
+
+static size_t block_lds(int64_t F) { return (size_t)kMlpRing * kUnit * 16 + (size_t)(4 * kC + 2 * kC + F) * 4; }
+
+bool block_supported(int dtype, const pa_shape &s, int64_t F) {
+  return backend_supported(dtype, s) && F >= 128 && F % 128 == 0 && block_lds(F) <= 160 * 1024;
+}
+
+int64_t block_blob_bytes(int64_t F) { return (8 + (F / 128) * 16) * (int64_t)kUnit * 16; }
+
+int block_tail(const pa_shape &s, const pa_params &p, const pa_block_mlp &m, const void *w, const float *out_token,
+               const void *fx_in, void *fx_out, const pa_block_tail *next, void *blob, hipStream_t st) {
+  if (!block_supported(PA_F32, s, m.F)) return PA_ERR_UNSUPPORTED;
+  hipLaunchKernelGGL(pack_block_kernel, dim3((unsigned)(8 + (m.F / 128) * 16)), dim3(256), 0, st,
+                     static_cast<const float *>(p.out_linear_weight), static_cast<const float *>(m.w1),
+                     static_cast<const float *>(m.w2), (int)m.F, static_cast<u32x4 *>(blob));
+  int rc = launch_status();
+  if (rc) return rc;
+  const size_t lds = block_lds(m.F);
+  if ((rc = allow_dynamic_lds(block_tail_kernel, lds))) return rc;
+  BlockArgs a{};
+  a.b_out = p.out_linear_bias;
+  a.w = static_cast<const float *>(w);
+  a.out_token = out_token;
+  a.fx_in = static_cast<const float *>(fx_in);
+  a.ln2_gamma = m.ln_gamma;
+  a.ln2_beta = m.ln_beta;
+  a.ln2_eps = m.ln_eps;
+  a.b1 = m.b1;
+  a.b2 = m.b2;
+  a.fx_out = static_cast<float *>(fx_out);
+  a.next = make_tail(next);
+  const int bpb = (int)(((s.N + 31) / 32 + 3) / 4);
+  hipLaunchKernelGGL(block_tail_kernel, dim3((unsigned)(s.B * bpb)), dim3(256), lds, st,
+                     static_cast<const u32x4 *>(blob), a, (int)s.N, bpb, (int)m.F);
   return launch_status();
 }
 

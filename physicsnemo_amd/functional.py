@@ -302,6 +302,36 @@ def mlp_forward(u, w1, b1, w2, b2, residual=None, ln_weight=None, ln_bias=None, 
     return y if ln_out is None else (y, ln_out)
 
 
+def block_supported(dtype: torch.dtype, dims: LayerDims, F: int) -> bool:
+    """True if `block_forward` serves the shape (float32, C = 128, 8 heads of 16, 32 slices, F a multiple of 128)."""
+    if dtype != torch.float32:
+        return False
+    return bool(_lib.load().pa_block_query(_lib.PA_F32, byref(dims.c()), F))
+
+
+def block_forward(x, fx_in, params, dims: LayerDims, ln2_weight, ln2_bias, ln2_eps, w1, b1, w2, b2,
+                  next_ln_weight=None, next_ln_bias=None, next_ln_eps=1e-5):
+    """One Transolver block behind its first LayerNorm in one library call: fx1 = Attn(x) + fx_in,
+    fx_out = Mlp(LayerNorm_2(fx1)) + fx1; returns fx_out, or (fx_out, LayerNorm_next(fx_out)) when next_ln_weight is
+    given.  x = LayerNorm_1(fx_in)."""
+    _need_cuda(x, fx_in, ln2_weight, ln2_bias, w1, b1, w2, b2, next_ln_weight, next_ln_bias)
+    lib = _lib.load()
+    code, shape, F = _lib.dtype_code(x.dtype), dims.c(), w1.shape[0]
+    nbytes = lib.pa_block_workspace_bytes(code, byref(shape), F)
+    if nbytes < 0:
+        _lib.check(int(nbytes), "pa_block_workspace_bytes")
+    workspace = torch.empty(int(nbytes), dtype=torch.uint8, device=x.device)
+    fx_out = torch.empty_like(fx_in)
+    ln_out = torch.empty_like(fx_in) if next_ln_weight is not None else None
+    mlp = _lib.PaBlockMlp(_lib.ptr(ln2_weight), _lib.ptr(ln2_bias), float(ln2_eps), _lib.ptr(w1), _lib.ptr(b1),
+                          _lib.ptr(w2), _lib.ptr(b2), F)
+    tail = _c_tail(None, next_ln_weight, next_ln_bias, next_ln_eps, ln_out)
+    _lib.check(lib.pa_block_forward(code, byref(shape), byref(_c_params(params)), byref(mlp), x.data_ptr(),
+                                    fx_in.data_ptr(), fx_out.data_ptr(), byref(tail), workspace.data_ptr(), int(nbytes),
+                                    _lib.current_stream_ptr(x.device)), "pa_block_forward")
+    return fx_out if ln_out is None else (fx_out, ln_out)
+
+
 def preprocess_supported(dtype: torch.dtype, rows: int, c_in: int, F: int, C: int) -> bool:
     """True if `preprocess_forward` serves the shape (float32, C = 128, up to 8 input features, F a multiple of 128)."""
     if dtype != torch.float32:

@@ -175,9 +175,36 @@ class TransolverBlock(nn.Module):
             fx1 = self.Attn(x_in) + fx
             return self._mlp_with_grad(PA.layer_norm(fx1, self.ln_mlp1[0])) + fx1, None
         x_in = normed_in if normed_in is not None else self.ln_1(fx)
+        whole = self._whole_block(x_in, fx, next_ln)
+        if whole is not None:
+            return whole
         # fx1 = Attn(ln_1(fx)) + fx and LayerNorm(fx1) come out of one fused library call (reference :300, :303)
         fx1, normed = self.Attn.forward_block(x_in, fx, self.ln_mlp1[0])
         return self._mlp_residual(fx1, normed, next_ln)
+
+    def _whole_block(self, x_in: torch.Tensor, fx: torch.Tensor, next_ln: nn.LayerNorm | None):
+        """The block behind ln_1 in one library call (pa_block_forward) where the shape is served (float32, hidden 128,
+        8 heads of 16, 32 slices), else None."""
+        attn, mlp = self.Attn, self.ln_mlp1[1]
+        if not (x_in.is_cuda and x_in.dtype == torch.float32 and fx.dtype == torch.float32 and not self.fp8_weights
+                and not getattr(attn, "plus", False) and isinstance(mlp.layers[1], nn.GELU)
+                and mlp.layers[1].approximate == "none" and hasattr(attn, "layer_dims")):
+            return None
+        if (attn.training and attn.out_dropout.p > 0) or torch.is_autocast_enabled("cuda"):
+            return None  # autocast runs the layer in its own dtype: the separate calls handle that
+        x = attn._prepare_input(x_in)
+        attn._validate(x_in)
+        dims = attn.layer_dims(x)
+        if not PF.block_supported(x.dtype, dims, mlp.layers[0].out_features):
+            return None
+        w1, b1, w2, b2 = self._mlp_kernel_params(x.device, torch.float32)
+        ln2 = self.ln_mlp1[0]
+        f32 = lambda t: t.detach().float().contiguous()
+        nxt = {} if next_ln is None else dict(next_ln_weight=f32(next_ln.weight), next_ln_bias=f32(next_ln.bias),
+                                              next_ln_eps=next_ln.eps)
+        out = PF.block_forward(x, fx.contiguous(), attn.kernel_params(x.dtype, x.device), dims, f32(ln2.weight),
+                               f32(ln2.bias), ln2.eps, w1, b1, w2, b2, **nxt)
+        return (out, None) if next_ln is None else out
 
     def _mlp_residual(self, fx1: torch.Tensor, normed: torch.Tensor, next_ln: nn.LayerNorm | None):
         """fx1 + Mlp(normed) and, with `next_ln`, its LayerNorm (reference :303, and :300 of the next block): the fused

@@ -9,6 +9,7 @@ import torch
 
 from oracle import torch_oracle as to
 import physicsnemo_amd as pn
+from physicsnemo_amd import functional as PF
 from gpu_util import announce, assert_fp32_close, assert_rel_l2, make_pair
 
 pytestmark = pytest.mark.gpu
@@ -98,6 +99,39 @@ def test_fp32_irregular_row_kernel_back_end(B, N):
     assert_fp32_close(y, want, "layer y")
     assert_fp32_close(fx, want_fx, "fx_new")
     assert_fp32_close(normed, want_ln, "LayerNorm(fx_new)")
+
+
+@pytest.mark.parametrize("spatial,B,mlp_ratio,last", [(None, 2, 1, False), ((13, 11), 3, 4, False), ((85, 85), 1, 1, True),
+                                                      (None, 1, 2, True)])
+def test_fp32_whole_block_in_one_call(spatial, B, mlp_ratio, last):
+    # hidden 128, 8 heads of 16, 32 slices: TransolverBlock.forward runs pa_block_forward (front end, combine + slice
+    # attention, then hand-back, out_linear, both residuals, the MLP and the LayerNorms in one launch); irregular and
+    # structured layers, ragged tiles, several chunks of hidden features, the last block with its output head
+    announce("fp32 whole block", spatial, B, mlp_ratio, last)
+    torch.manual_seed(3)
+    kw = dict(mlp_ratio=mlp_ratio, last_layer=last, out_dim=3, slice_num=32, spatial_shape=spatial)
+    ref = to.OracleTransolverBlock(8, 128, **kw).eval()
+    hip = pn.TransolverBlock(8, 128, 0.0, use_te=False, **kw).eval()
+    with torch.no_grad():
+        for ln in (ref.ln_1, ref.ln_mlp1[0]):
+            ln.weight.add_(0.2 * torch.randn(128))
+            ln.bias.add_(0.2 * torch.randn(128))
+        ref.Attn.in_project_slice.weight.mul_(2.0)
+    hip.load_state_dict(ref.state_dict())
+    hip = hip.cuda()
+    N = 333 if spatial is None else spatial[0] * spatial[1]
+    fx = torch.randn(B, N, 128)
+    calls = []
+    orig = PF.block_forward
+    PF.block_forward = lambda *a, **k: (calls.append(1), orig(*a, **k))[1]
+    try:
+        with torch.no_grad():
+            want = ref(fx)
+            got = hip(fx.cuda())
+    finally:
+        PF.block_forward = orig
+    assert calls, "the whole-block entry point did not run"
+    assert_fp32_close(got, want, "block output")
 
 
 @pytest.mark.parametrize("kernel,grid", [(3, (4, 4, 4)), (3, (8, 8, 8)), (5, (8, 8, 8)), (3, (3, 5, 7)), (1, (4, 6, 5))])
