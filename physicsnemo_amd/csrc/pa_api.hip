@@ -1039,7 +1039,7 @@ int pa_layer_forward(int dtype, const pa_shape *shape, const pa_params *p, const
 
   if (plan.conv_front) {  // both convolutions, the slice softmax and the partial token sums in one launch
     if ((rc = pa::conv::front(s, *p, x, ws + plan.off_blob, w, partials,
-                              plan.rows_back ? ws + plan.off_blob_out : nullptr, st)))
+                              plan.rows_back ? ws + plan.off_blob_out : nullptr, nullptr, st)))
       return rc;
   } else {
     if ((rc = pa::general::project_inputs(dtype, s, *p, x, x_mid, fx_mid, st))) return rc;
@@ -1093,14 +1093,14 @@ int pa_block_forward(int dtype, const pa_shape *shape, const pa_params *p, const
   float *tok = reinterpret_cast<float *>(ws + plan.off_tok), *norm = reinterpret_cast<float *>(ws + plan.off_norm);
   float *tok_out = reinterpret_cast<float *>(ws + plan.off_tok_out);
   if (plan.conv_front) {
-    if ((rc = pa::conv::front(s, *p, x, ws + plan.off_blob, w, partials, nullptr, st))) return rc;
+    if ((rc = pa::conv::front(s, *p, x, ws + plan.off_blob, w, partials, ws + plan.total, mlp, st))) return rc;
   } else {
     if ((rc = pa::general::project_inputs(dtype, s, *p, x, x_mid, fx_mid, st))) return rc;
     if ((rc = pa::general::slice_softmax(dtype, s, *p, x_mid, w, st))) return rc;
     if ((rc = pa::general::slice_partial(dtype, s, w, fx_mid, partials, st))) return rc;
   }
   if ((rc = pa::general::combine_attention(s, *p, partials, plan.G, tok, norm, tok_out, st))) return rc;
-  return pa::f32rows::block_tail(s, *p, *mlp, w, tok_out, fx_in, fx_out, next, ws + plan.total, st);
+  return pa::f32rows::block_tail(s, *p, *mlp, w, tok_out, fx_in, fx_out, next, ws + plan.total, plan.conv_front, st);
 }
 
 // Workspace plan of the FLARE layer on the MFMA kernels.

@@ -54,14 +54,24 @@ constexpr size_t kLdsBytes = kRingBytes > kEpilogueBytes ? kRingBytes : kEpilogu
 
 // blob unit ((step 8 + ct) 3 + piece) 64 + lane: the B operand (lane (i, g): output channel 32 (ct % 4) + i of weight
 // set ct / 4, k = 8 g .. 8 g + 7 of the step) of one bf16 piece.  step = tap 8 + channel block.
-// The last 8 workgroups (when w_out is given) cut out_linear's weight for the hand-back kernel of the same layer call.
+// The workgroups behind the first conv_blocks cut the weights of the same call's row kernel: out_linear's (8 units),
+// then, with w1 given, the block MLP's per chunk of 128 hidden features (8 units of W1's rows, 8 of W2's columns) --
+// all with the reduction index in register order (the layout f32rows::backend / block_tail read).
 __global__ __launch_bounds__(256) void split_pack_kernel(const float *__restrict__ wx, const float *__restrict__ wfx,
                                                          u32x4 *__restrict__ blob, int taps, int tap_major,
                                                          int conv_blocks, const float *__restrict__ w_out,
-                                                         u32x4 *__restrict__ blob_out) {
+                                                         const float *__restrict__ w1, const float *__restrict__ w2,
+                                                         int F, u32x4 *__restrict__ blob_out) {
   if ((int)blockIdx.x >= conv_blocks) {
     const int u = blockIdx.x - conv_blocks;
-    pack_unit(w_out, kC, 16 * u, true, blob_out + (int64_t)u * kUnit, threadIdx.x);
+    u32x4 *unit = blob_out + (int64_t)u * kUnit;
+    if (u < 8) {
+      pack_unit(w_out, kC, 16 * u, true, unit, threadIdx.x);
+    } else {
+      const int q = u - 8, c = q >> 4, v = q & 15;
+      if (v < 8) pack_unit(w1 + (int64_t)c * 128 * kC, kC, 16 * v, true, unit, threadIdx.x);
+      else pack_unit(w2 + c * 128, F, 16 * (v - 8), true, unit, threadIdx.x);
+    }
     return;
   }
   const int64_t total = (int64_t)taps * kStepsPerTap * kColTiles * 64;
@@ -386,15 +396,18 @@ int64_t groups(const pa_shape &s) { return ((s.N + 31) / 32 + 3) / 4; }
 int64_t blob_bytes(const pa_shape &s) { return s.conv_k * s.conv_k * kStepsPerTap * (int64_t)kStepUnits * 16 + 64; }
 
 int front(const pa_shape &s, const pa_params &p, const void *x, void *blob, void *w, float *partials, void *blob_out,
-          hipStream_t st) {
+          const pa_block_mlp *mlp, hipStream_t st) {
   if (!supported(PA_F32, s)) return PA_ERR_UNSUPPORTED;
   const int taps = (int)(s.conv_k * s.conv_k);
   const int64_t units = (int64_t)taps * kStepsPerTap * kColTiles * 64;
   const int conv_blocks = (int)((units + 255) / 256);
-  hipLaunchKernelGGL(split_pack_kernel, dim3((unsigned)(conv_blocks + (blob_out ? 8 : 0))), dim3(256), 0, st,
+  const int extra = !blob_out ? 0 : 8 + (mlp ? (int)(mlp->F / 128) * 16 : 0);
+  hipLaunchKernelGGL(split_pack_kernel, dim3((unsigned)(conv_blocks + extra)), dim3(256), 0, st,
                      static_cast<const float *>(p.in_project_x_weight), static_cast<const float *>(p.in_project_fx_weight),
                      static_cast<u32x4 *>(blob), taps, (int)s.conv_tap_major, conv_blocks,
-                     static_cast<const float *>(p.out_linear_weight), static_cast<u32x4 *>(blob_out));
+                     static_cast<const float *>(p.out_linear_weight), mlp ? static_cast<const float *>(mlp->w1) : nullptr,
+                     mlp ? static_cast<const float *>(mlp->w2) : nullptr, mlp ? (int)mlp->F : 0,
+                     static_cast<u32x4 *>(blob_out));
   int rc = launch_status();
   if (rc) return rc;
   if ((rc = allow_dynamic_lds(conv_slice_kernel, kLdsBytes))) return rc;

@@ -705,13 +705,15 @@ bool block_supported(int dtype, const pa_shape &s, int64_t F) {
 int64_t block_blob_bytes(int64_t F) { return (8 + (F / 128) * 16) * (int64_t)kUnit * 16; }
 
 int block_tail(const pa_shape &s, const pa_params &p, const pa_block_mlp &m, const void *w, const float *out_token,
-               const void *fx_in, void *fx_out, const pa_block_tail *next, void *blob, hipStream_t st) {
+               const void *fx_in, void *fx_out, const pa_block_tail *next, void *blob, bool blob_ready, hipStream_t st) {
   if (!block_supported(PA_F32, s, m.F)) return PA_ERR_UNSUPPORTED;
-  hipLaunchKernelGGL(pack_block_kernel, dim3((unsigned)(8 + (m.F / 128) * 16)), dim3(256), 0, st,
-                     static_cast<const float *>(p.out_linear_weight), static_cast<const float *>(m.w1),
-                     static_cast<const float *>(m.w2), (int)m.F, static_cast<u32x4 *>(blob));
-  int rc = launch_status();
-  if (rc) return rc;
+  int rc = PA_OK;
+  if (!blob_ready) {
+    hipLaunchKernelGGL(pack_block_kernel, dim3((unsigned)(8 + (m.F / 128) * 16)), dim3(256), 0, st,
+                       static_cast<const float *>(p.out_linear_weight), static_cast<const float *>(m.w1),
+                       static_cast<const float *>(m.w2), (int)m.F, static_cast<u32x4 *>(blob));
+    if ((rc = launch_status())) return rc;
+  }
   const size_t lds = block_lds(m.F);
   if ((rc = allow_dynamic_lds(block_tail_kernel, lds))) return rc;
   BlockArgs a{};
