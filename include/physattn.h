@@ -464,8 +464,16 @@ typedef struct pa_block_mlp {
   int64_t F;
 } pa_block_mlp;
 
-/* Replaces TransolverBlock.forward (TR.py:296-303) for a block that is not the last one, and the part of the last
- * block before its output head:
+/* The last block's output head ln_mlp2[1] (TR.py:305-307), a Linear(C -> O) over next->ln_out with O <= 4 outputs. */
+typedef struct pa_block_head {
+  const void *weight; /* (O, C), activation dtype */
+  const float *bias;  /* (O) or NULL */
+  int64_t O;
+  void *out;          /* (B, N, O), activation dtype */
+} pa_block_head;
+
+/* Replaces TransolverBlock.forward (TR.py:296-307): for a block that is not the last one head is NULL; for the last
+ * block next is ln_mlp2[0] and head its Linear (next->ln_out may then be NULL: the LayerNorm is not stored):
  *   fx1 = Attn(x) + fx_in;  fx_out = Mlp(LayerNorm(fx1)) + fx1;  next->ln_out = LayerNorm_next(fx_out)
  * x (B,N,C) is LayerNorm_1(fx_in), which the caller has from the block before (or pa_preprocess_forward);
  * next: ln_gamma / ln_beta / ln_eps / ln_out of the LayerNorm that follows (ln_1 of the next block, or ln_mlp2[0]),
@@ -475,8 +483,8 @@ typedef struct pa_block_mlp {
 int pa_block_query(int dtype, const pa_shape *shape, int64_t F);
 int64_t pa_block_workspace_bytes(int dtype, const pa_shape *shape, int64_t F);
 int pa_block_forward(int dtype, const pa_shape *shape, const pa_params *p, const pa_block_mlp *mlp, const void *x,
-                     const void *fx_in, void *fx_out, const pa_block_tail *next, void *workspace,
-                     int64_t workspace_bytes, void *stream);
+                     const void *fx_in, void *fx_out, const pa_block_tail *next, const pa_block_head *head,
+                     void *workspace, int64_t workspace_bytes, void *stream);
 
 /* The model's preprocess Mlp (TR.py:519-525 with mlp_layers.py:139-173): Linear(c_in -> F) -> GELU(erf) -> Linear(F -> C)
  * over `rows` rows of u (rows, c_in), c_in = coordinates + fields per point; with a tail, tail->ln_out is the first

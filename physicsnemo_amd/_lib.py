@@ -62,6 +62,10 @@ class PaBlockMlp(Structure):
                 ("w2", c_void_p), ("b2", c_void_p), ("F", c_int64)]
 
 
+class PaBlockHead(Structure):
+    _fields_ = [("weight", c_void_p), ("bias", c_void_p), ("O", c_int64), ("out", c_void_p)]
+
+
 class PaPlusParams(Structure):
     _fields_ = [(n, c_void_p) for n in ("proj_temperature_0_weight", "proj_temperature_0_bias",
                                         "proj_temperature_2_weight", "proj_temperature_2_bias")]
@@ -152,7 +156,7 @@ def load() -> ctypes.CDLL:
     lib.pa_block_workspace_bytes.argtypes = [c_int, ps, c_int64]
     lib.pa_block_forward.restype = c_int
     lib.pa_block_forward.argtypes = [c_int, ps, POINTER(PaParams), POINTER(PaBlockMlp), c_void_p, c_void_p, c_void_p, pt,
-                                     c_void_p, c_int64, c_void_p]
+                                     POINTER(PaBlockHead), c_void_p, c_int64, c_void_p]
     lib.pa_preprocess_query.restype = c_int
     lib.pa_preprocess_query.argtypes = [c_int, c_int64, c_int64, c_int64, c_int64]
     lib.pa_preprocess_workspace_bytes.restype = c_int64

@@ -1070,8 +1070,8 @@ int64_t pa_block_workspace_bytes(int dtype, const pa_shape *shape, int64_t F) {
 }
 
 int pa_block_forward(int dtype, const pa_shape *shape, const pa_params *p, const pa_block_mlp *mlp, const void *x,
-                     const void *fx_in, void *fx_out, const pa_block_tail *next, void *workspace,
-                     int64_t workspace_bytes, void *stream) {
+                     const void *fx_in, void *fx_out, const pa_block_tail *next, const pa_block_head *head,
+                     void *workspace, int64_t workspace_bytes, void *stream) {
   int rc = check_shape(dtype, shape);
   if (rc) return rc;
   if ((rc = check_params(p))) return rc;
@@ -1082,6 +1082,11 @@ int pa_block_forward(int dtype, const pa_shape *shape, const pa_params *p, const
     return PA_ERR_ALIGN;
   if ((rc = check_tail(next))) return rc;
   if (next && next->residual) return PA_ERR_UNSUPPORTED;  // the block's own residual is fx1
+  if (head) {  // behind the next LayerNorm, whose parameters must then be given (its output need not be stored)
+    if (!head->weight || !head->out || !next || !next->ln_gamma || !next->ln_beta) return PA_ERR_NULL;
+    if (head->O < 1 || head->O > 4) return PA_ERR_UNSUPPORTED;
+    if (!aligned16(head->weight)) return PA_ERR_ALIGN;
+  }
   const pa_shape &s = *shape;
   if (!pa::f32rows::block_supported(dtype, s, mlp->F)) return PA_ERR_UNSUPPORTED;
   const GeneralPlan plan = plan_general(dtype, s);
@@ -1100,7 +1105,8 @@ int pa_block_forward(int dtype, const pa_shape *shape, const pa_params *p, const
     if ((rc = pa::general::slice_partial(dtype, s, w, fx_mid, partials, st))) return rc;
   }
   if ((rc = pa::general::combine_attention(s, *p, partials, plan.G, tok, norm, tok_out, st))) return rc;
-  return pa::f32rows::block_tail(s, *p, *mlp, w, tok_out, fx_in, fx_out, next, ws + plan.total, plan.conv_front, st);
+  return pa::f32rows::block_tail(s, *p, *mlp, w, tok_out, fx_in, fx_out, next, head, ws + plan.total, plan.conv_front,
+                                 st);
 }
 
 // Workspace plan of the FLARE layer on the MFMA kernels.

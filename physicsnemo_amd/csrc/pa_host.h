@@ -137,7 +137,8 @@ int mlp_forward(int64_t rows, int64_t F, const void *blob, const float *b1, cons
 bool block_supported(int dtype, const pa_shape &s, int64_t F);
 int64_t block_blob_bytes(int64_t F);
 int block_tail(const pa_shape &s, const pa_params &p, const pa_block_mlp &m, const void *w, const float *out_token,
-               const void *fx_in, void *fx_out, const pa_block_tail *next, void *blob, bool blob_ready, hipStream_t st);
+               const void *fx_in, void *fx_out, const pa_block_tail *next, const pa_block_head *head, void *blob,
+               bool blob_ready, hipStream_t st);
 // the model's preprocess Mlp, Linear(c_in -> F) -> GELU -> Linear(F -> 128), c_in <= 8, with the tail (the first
 // LayerNorm); blob: premlp_blob_bytes(F) of scratch
 bool premlp_supported(int dtype, int64_t rows, int64_t c_in, int64_t F, int64_t C);

@@ -72,8 +72,15 @@ __device__ __forceinline__ void split_half(const f32x16 &v, int kk, u32x4 (&pl)[
 
 // The tail on a wave's transposed tile: y = yT (+ residual) leaves, then LayerNorm(y) if asked for.  A lane holds 64
 // of its row's 128 channels (4 consecutive ones per register quad), its partner lane the others.  gb: gamma | beta.
+struct Head {  // output head behind the LayerNorm: out (rows, O) = LayerNorm(y) W^T + b, O <= 4; w points into LDS
+  const float *w, *b;
+  float *out;
+  int O;
+};
+
 __device__ __forceinline__ void finish_rows(f32x16 (&yT)[4], int64_t row, bool ok, int g, const float *residual, float *y,
-                                            float *ln_out, const float *gb, float eps) {
+                                            float *ln_out, const float *gb, float eps, bool want_ln = false,
+                                            Head head = Head{nullptr, nullptr, nullptr, 0}) {
 #pragma unroll
   for (int t = 0; t < 4; ++t)
 #pragma unroll
@@ -87,7 +94,7 @@ __device__ __forceinline__ void finish_rows(f32x16 (&yT)[4], int64_t row, bool o
       if (ok) *reinterpret_cast<float4 *>(y + at) = v;
       yT[t][4 * q] = v.x, yT[t][4 * q + 1] = v.y, yT[t][4 * q + 2] = v.z, yT[t][4 * q + 3] = v.w;
     }
-  if (!ln_out) return;
+  if (!ln_out && !want_ln) return;
   float sum = 0.f;
 #pragma unroll
   for (int t = 0; t < 4; ++t)
@@ -114,8 +121,22 @@ __device__ __forceinline__ void finish_rows(f32x16 (&yT)[4], int64_t row, bool o
       o.y = (yT[t][4 * q + 1] - mean) * rstd * ga.y + be.y;
       o.z = (yT[t][4 * q + 2] - mean) * rstd * ga.z + be.z;
       o.w = (yT[t][4 * q + 3] - mean) * rstd * ga.w + be.w;
-      if (ok) *reinterpret_cast<float4 *>(ln_out + row * kC + c0) = o;
+      if (ok && ln_out) *reinterpret_cast<float4 *>(ln_out + row * kC + c0) = o;
+      yT[t][4 * q] = o.x, yT[t][4 * q + 1] = o.y, yT[t][4 * q + 2] = o.z, yT[t][4 * q + 3] = o.w;
     }
+  for (int o = 0; o < head.O; ++o) {  // a lane sums its 64 channels, its partner lane the others
+    float acc = 0.f;
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const float4 wq = *reinterpret_cast<const float4 *>(head.w + o * kC + 32 * t + 8 * q + 4 * g);
+        acc = fmaf(yT[t][4 * q], wq.x, acc), acc = fmaf(yT[t][4 * q + 1], wq.y, acc);
+        acc = fmaf(yT[t][4 * q + 2], wq.z, acc), acc = fmaf(yT[t][4 * q + 3], wq.w, acc);
+      }
+    acc = half_sum(acc) + (head.b ? head.b[o] : 0.f);
+    if (ok && g == 0) head.out[row * head.O + o] = acc;
+  }
 }
 
 struct Tail {
@@ -367,6 +388,9 @@ struct BlockArgs {
   const float *b1, *b2;
   float *fx_out;
   Tail next;  // residual unused
+  const float *head_w, *head_b;  // output head behind the next LayerNorm (O <= 4 outputs), or NULL
+  float *head_out;
+  int head_O;
 };
 
 __global__ __launch_bounds__(256) void pack_block_kernel(const float *__restrict__ w_out, const float *__restrict__ w1,
@@ -386,7 +410,7 @@ __global__ __launch_bounds__(256) void block_tail_kernel(const u32x4 *__restrict
   u32x4 *tokp = smem + 8 * kUnit;  // [pair][kk][piece][lane], in ring slots 8 .. 11 until the hand-back is done
   float *gb2 = reinterpret_cast<float *>(smem + kMlpRing * kUnit);  // gamma | beta of LayerNorm_2
   float *gbn = gb2 + 2 * kC;                                        // gamma | beta of the next LayerNorm
-  float *bo = gbn + 2 * kC, *bb2 = bo + kC, *bb1 = bb2 + kC;        // b_out, b2, b1 (F)
+  float *bo = gbn + 2 * kC, *bb2 = bo + kC, *hw = bb2 + kC, *bb1 = hw + 4 * kC;  // b_out, b2, head weight, b1 (F)
   const int tid = threadIdx.x, lane = tid & 63, i = lane & 31, g = lane >> 5;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int b = blockIdx.x / bpb, gblk = blockIdx.x - b * bpb;
@@ -415,6 +439,7 @@ __global__ __launch_bounds__(256) void block_tail_kernel(const u32x4 *__restrict
     bb2[tid] = a.b2 ? a.b2[tid] : 0.f;
   }
   for (int k = tid; k < F; k += 256) bb1[k] = a.b1 ? a.b1[k] : 0.f;
+  for (int k = tid; k < a.head_O * kC; k += 256) hw[k] = a.head_w[k];
   // the batch's tokens as block-diagonal A operands (deslice_linear_kernel)
   const float *tok = a.out_token + (int64_t)b * kH * kS * kD;
   for (int item = tid; item < 16 * 64; item += 256) {
@@ -552,7 +577,8 @@ __global__ __launch_bounds__(256) void block_tail_kernel(const u32x4 *__restrict
     __syncthreads();  // the slots of W2's units are free
     issue_upto(base + 16 + kMlpRing);
   }
-  finish_rows(fx1, row, ok, g, nullptr, a.fx_out, a.next.ln_out, gbn, a.next.eps);
+  finish_rows(fx1, row, ok, g, nullptr, a.fx_out, a.next.ln_out, gbn, a.next.eps, a.head_O > 0,
+              Head{hw, a.head_b, a.head_out, a.head_O});
 }
 
 // ---------------------------------------------------------------------------------------------------------------
@@ -696,7 +722,7 @@ int mlp_forward(int64_t M, int64_t F, const void *blob, const float *b1, const f
   return launch_status();
 }
 
-static size_t block_lds(int64_t F) { return (size_t)kMlpRing * kUnit * 16 + (size_t)(4 * kC + 2 * kC + F) * 4; }
+static size_t block_lds(int64_t F) { return (size_t)kMlpRing * kUnit * 16 + (size_t)(4 * kC + 2 * kC + 4 * kC + F) * 4; }
 
 bool block_supported(int dtype, const pa_shape &s, int64_t F) {
   return backend_supported(dtype, s) && F >= 128 && F % 128 == 0 && block_lds(F) <= 160 * 1024;
@@ -705,7 +731,8 @@ bool block_supported(int dtype, const pa_shape &s, int64_t F) {
 int64_t block_blob_bytes(int64_t F) { return (8 + (F / 128) * 16) * (int64_t)kUnit * 16; }
 
 int block_tail(const pa_shape &s, const pa_params &p, const pa_block_mlp &m, const void *w, const float *out_token,
-               const void *fx_in, void *fx_out, const pa_block_tail *next, void *blob, bool blob_ready, hipStream_t st) {
+               const void *fx_in, void *fx_out, const pa_block_tail *next, const pa_block_head *head, void *blob,
+               bool blob_ready, hipStream_t st) {
   if (!block_supported(PA_F32, s, m.F)) return PA_ERR_UNSUPPORTED;
   int rc = PA_OK;
   if (!blob_ready) {
@@ -728,6 +755,12 @@ int block_tail(const pa_shape &s, const pa_params &p, const pa_block_mlp &m, con
   a.b2 = m.b2;
   a.fx_out = static_cast<float *>(fx_out);
   a.next = make_tail(next);
+  if (head) {
+    a.head_w = static_cast<const float *>(head->weight);
+    a.head_b = head->bias;
+    a.head_out = static_cast<float *>(head->out);
+    a.head_O = (int)head->O;
+  }
   const int bpb = (int)(((s.N + 31) / 32 + 3) / 4);
   hipLaunchKernelGGL(block_tail_kernel, dim3((unsigned)(s.B * bpb)), dim3(256), lds, st,
                      static_cast<const u32x4 *>(blob), a, (int)s.N, bpb, (int)m.F);

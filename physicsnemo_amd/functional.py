@@ -310,11 +310,12 @@ def block_supported(dtype: torch.dtype, dims: LayerDims, F: int) -> bool:
 
 
 def block_forward(x, fx_in, params, dims: LayerDims, ln2_weight, ln2_bias, ln2_eps, w1, b1, w2, b2,
-                  next_ln_weight=None, next_ln_bias=None, next_ln_eps=1e-5):
+                  next_ln_weight=None, next_ln_bias=None, next_ln_eps=1e-5, head_weight=None, head_bias=None):
     """One Transolver block behind its first LayerNorm in one library call: fx1 = Attn(x) + fx_in,
     fx_out = Mlp(LayerNorm_2(fx1)) + fx1; returns fx_out, or (fx_out, LayerNorm_next(fx_out)) when next_ln_weight is
-    given.  x = LayerNorm_1(fx_in)."""
-    _need_cuda(x, fx_in, ln2_weight, ln2_bias, w1, b1, w2, b2, next_ln_weight, next_ln_bias)
+    given, or (fx_out, LayerNorm_next(fx_out) head_weight^T + head_bias) when the output head (up to 4 outputs) is given
+    as well.  x = LayerNorm_1(fx_in)."""
+    _need_cuda(x, fx_in, ln2_weight, ln2_bias, w1, b1, w2, b2, next_ln_weight, next_ln_bias, head_weight, head_bias)
     lib = _lib.load()
     code, shape, F = _lib.dtype_code(x.dtype), dims.c(), w1.shape[0]
     nbytes = lib.pa_block_workspace_bytes(code, byref(shape), F)
@@ -322,13 +323,19 @@ def block_forward(x, fx_in, params, dims: LayerDims, ln2_weight, ln2_bias, ln2_e
         _lib.check(int(nbytes), "pa_block_workspace_bytes")
     workspace = torch.empty(int(nbytes), dtype=torch.uint8, device=x.device)
     fx_out = torch.empty_like(fx_in)
-    ln_out = torch.empty_like(fx_in) if next_ln_weight is not None else None
+    ln_out = torch.empty_like(fx_in) if (next_ln_weight is not None and head_weight is None) else None
+    head, head_out = None, None
+    if head_weight is not None:
+        head_out = torch.empty(*fx_in.shape[:-1], head_weight.shape[0], dtype=fx_in.dtype, device=fx_in.device)
+        head = byref(_lib.PaBlockHead(_lib.ptr(head_weight), _lib.ptr(head_bias), head_weight.shape[0], head_out.data_ptr()))
     mlp = _lib.PaBlockMlp(_lib.ptr(ln2_weight), _lib.ptr(ln2_bias), float(ln2_eps), _lib.ptr(w1), _lib.ptr(b1),
                           _lib.ptr(w2), _lib.ptr(b2), F)
     tail = _c_tail(None, next_ln_weight, next_ln_bias, next_ln_eps, ln_out)
     _lib.check(lib.pa_block_forward(code, byref(shape), byref(_c_params(params)), byref(mlp), x.data_ptr(),
-                                    fx_in.data_ptr(), fx_out.data_ptr(), byref(tail), workspace.data_ptr(), int(nbytes),
-                                    _lib.current_stream_ptr(x.device)), "pa_block_forward")
+                                    fx_in.data_ptr(), fx_out.data_ptr(), byref(tail), head, workspace.data_ptr(),
+                                    int(nbytes), _lib.current_stream_ptr(x.device)), "pa_block_forward")
+    if head_out is not None:
+        return fx_out, head_out
     return fx_out if ln_out is None else (fx_out, ln_out)
 
 

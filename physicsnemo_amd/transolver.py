@@ -182,9 +182,11 @@ class TransolverBlock(nn.Module):
         fx1, normed = self.Attn.forward_block(x_in, fx, self.ln_mlp1[0])
         return self._mlp_residual(fx1, normed, next_ln)
 
-    def _whole_block(self, x_in: torch.Tensor, fx: torch.Tensor, next_ln: nn.LayerNorm | None):
+    def _whole_block(self, x_in: torch.Tensor, fx: torch.Tensor, next_ln: nn.LayerNorm | None,
+                     head: nn.Linear | None = None):
         """The block behind ln_1 in one library call (pa_block_forward) where the shape is served (float32, hidden 128,
-        8 heads of 16, 32 slices), else None."""
+        8 heads of 16, 32 slices), else None.  With `head` (the last block's ln_mlp2[1], up to 4 outputs) the second
+        element of the result is the head's output instead of the LayerNorm."""
         attn, mlp = self.Attn, self.ln_mlp1[1]
         if not (x_in.is_cuda and x_in.dtype == torch.float32 and fx.dtype == torch.float32 and not self.fp8_weights
                 and not getattr(attn, "plus", False) and isinstance(mlp.layers[1], nn.GELU)
@@ -202,6 +204,10 @@ class TransolverBlock(nn.Module):
         f32 = lambda t: t.detach().float().contiguous()
         nxt = {} if next_ln is None else dict(next_ln_weight=f32(next_ln.weight), next_ln_bias=f32(next_ln.bias),
                                               next_ln_eps=next_ln.eps)
+        if head is not None:
+            if next_ln is None or head.out_features > 4:
+                return None
+            nxt.update(head_weight=f32(head.weight), head_bias=None if head.bias is None else f32(head.bias))
         out = PF.block_forward(x, fx.contiguous(), attn.kernel_params(x.dtype, x.device), dims, f32(ln2.weight),
                                f32(ln2.bias), ln2.eps, w1, b1, w2, b2, **nxt)
         return (out, None) if next_ln is None else out
@@ -436,6 +442,13 @@ class Transolver(nn.Module):
         # each block hands the next one its residual stream and, when the fused MLP kernel ran, LayerNorm_1 of it
         for k, block in enumerate(self.blocks):
             if block.last_layer:
+                if not block._needs_grad(fx):
+                    x_in = normed if normed is not None else block.ln_1(fx)
+                    whole = block._whole_block(x_in, fx, block.ln_mlp2[0], head=block.ln_mlp2[1])
+                    if whole is not None:  # the block and its output head in one library call
+                        fx = whole[1]
+                        continue
+                    normed = x_in
                 fx, normed = block.forward_chain(fx, normed, block.ln_mlp2[0])
                 if normed is not None and on_library:
                     fx = self._library_linear(normed, block.ln_mlp2[1])  # output head (:305-307)

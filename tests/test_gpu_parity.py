@@ -132,6 +132,12 @@ def test_fp32_whole_block_in_one_call(spatial, B, mlp_ratio, last):
         PF.block_forward = orig
     assert calls, "the whole-block entry point did not run"
     assert_fp32_close(got, want, "block output")
+    if last:  # the output head inside the same call (what the model's last block runs)
+        with torch.no_grad():
+            xc = fx.cuda()
+            whole = hip._whole_block(hip.ln_1(xc), xc, hip.ln_mlp2[0], head=hip.ln_mlp2[1])
+        assert whole is not None
+        assert_fp32_close(whole[1], want, "block output, head in the call")
 
 
 @pytest.mark.parametrize("kernel,grid", [(3, (4, 4, 4)), (3, (8, 8, 8)), (5, (8, 8, 8)), (3, (3, 5, 7)), (1, (4, 6, 5))])
