@@ -415,13 +415,26 @@ def time_structured_model(steps=5, warmup=2):
         graphed = pn.GraphedForward(model, fx, pos)
         dt_graph, out = timed(graphed.replay)
         assert torch.isfinite(out).all()
+        # one block of the model on its own (pa_block_forward: front end, combine + slice attention, per-point tail)
+        block = model.blocks[1]
+        hx = torch.randn(4, 7225, 128, generator=g).cuda()
+        dt_block, o = timed(lambda: block(hx))
+        assert torch.isfinite(o).all()
+    # float32 FLOPs of a block: both 3 x 3 convolutions, slice logits, token sums, hand-back, out_linear, two MLP Linears
+    pts, C, H, D, S = 4 * 7225, 128, 8, 16, 32
+    block_flop = 2.0 * pts * (2 * 9 * C * C + H * D * S + 2 * H * S * D + C * C + 2 * C * C)
+    structured_block = {"ms": round(dt_block * 1e3, 4), "gflop": round(block_flop / 1e9, 2),
+                        "tflops": round(block_flop / dt_block / 1e12, 1),
+                        "frac_of_fp32_mfma_peak": round(block_flop / dt_block / 157.3e12, 3),
+                        "note": "float32-accurate FLOPs per second; the products run as bf16 MFMA pieces, so the float32 "
+                                "MFMA peak (157.3 TFLOP/s) is a yardstick here, not a bound"}
     return {"workload": "cfg1: Transolver structured 2D 85x85 (conv k=3), fp32, 4 layers", "batch": 4, "points": 7225,
             "layers": 4, "slice_num": 32,
             "arithmetic": "float32 storage and accumulation; matrix products as six bf16 MFMA products of three-way "
                           "split operands (error vs float64 as small as with float32 matrix instructions)",
             "ms_per_forward": round(dt * 1e3, 3),
             "mpoints_per_s": round(4 * 7225 / dt / 1e6, 2), "ms_per_forward_graph": round(dt_graph * 1e3, 3),
-            "mpoints_per_s_graph": round(4 * 7225 / dt_graph / 1e6, 2)}
+            "mpoints_per_s_graph": round(4 * 7225 / dt_graph / 1e6, 2), "block": structured_block}
 
 
 def source_stamp():
