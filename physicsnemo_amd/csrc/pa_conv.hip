@@ -47,8 +47,9 @@ constexpr int kStepsPerTap = kC / 16;              // k-steps of 16 channels
 constexpr int kStepUnits = kColTiles * 3 * 64;     // 16-byte units per k-step: 8 tiles x 3 pieces x 1 KB
 constexpr int kRing = 4;
 constexpr int kTokFloats = kH * kS * kD1;          // one partial
-// the ring, reused after the convolution for 4 token sums, 4 x 4 weight tiles in transit and the softmax statistics
-constexpr size_t kEpilogueBytes = (size_t)4 * kTokFloats * 4 + 4 * 4 * 4096 + 4 * 128 * 4;
+// the ring, reused after the convolution for 4 token sums, 4 x 4 accumulator tiles in transit between the two waves of
+// a tile, and every wave's softmax statistics
+constexpr size_t kEpilogueBytes = (size_t)4 * kTokFloats * 4 + 4 * 4 * 4096 + 8 * 128 * 4;
 constexpr size_t kRingBytes = (size_t)kRing * kStepUnits * 16 + (size_t)kRing * 4 * 2048;  // weights + input rows
 constexpr size_t kLdsBytes = kRingBytes > kEpilogueBytes ? kRingBytes : kEpilogueBytes;
 
@@ -266,8 +267,22 @@ __global__ __launch_bounds__(512) void conv_slice_kernel(
 
   float *red = reinterpret_cast<float *>(smem);                     // [tile][h][s][D + 1]
   float *mine = red + t * kTokFloats;
-  u32x4 *xchg = smem + (4 * kTokFloats) / 4 + t * (4 * 256);        // [tile][round parity][head of the pair][q][lane]
-  float *stat = reinterpret_cast<float *>(smem + (4 * kTokFloats) / 4 + 4 * 4 * 256) + t * 128;  // [head][max | 1 / sum][point]
+  u32x4 *xchg = smem + (4 * kTokFloats) / 4 + t * (4 * 256);        // [tile][role of the writer][tile of the pair][q][lane]
+  float *stat = reinterpret_cast<float *>(smem + (4 * kTokFloats) / 4 + 4 * 4 * 256) + wave * 128;  // [head][max | 1 / sum][point]
+  // The two waves of a tile share the eight heads: the x_mid wave takes heads 0 .. 3 and needs the fx_mid tiles 0, 1,
+  // the fx_mid wave takes heads 4 .. 7 and needs the x_mid tiles 2, 3.  One exchange of 32 registers each way through
+  // LDS, then every wave runs its heads from the logits to the token sums on its own.
+#pragma unroll
+  for (int c = 0; c < 2; ++c) {
+    f32x16 give;  // element by element: a select between the two arrays as wholes would keep them in memory
+#pragma unroll
+    for (int r = 0; r < 16; ++r) give[r] = role == 0 ? acc[2 + c][r] : acc[c][r];
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+      xchg[(role * 2 + c) * 256 + q * 64 + lane] =
+          u32x4{__float_as_uint(give[4 * q]), __float_as_uint(give[4 * q + 1]), __float_as_uint(give[4 * q + 2]),
+                __float_as_uint(give[4 * q + 3])};
+  }
   // W_slice[s][d] for MFMA m of a head: this lane's channel of the pair (k = g) is d = 8 (m / 4) + 4 g + m % 4, the
   // channel the x_mid registers hold in that position
   float ws[8], bs_r[16];
@@ -277,110 +292,110 @@ __global__ __launch_bounds__(512) void conv_slice_kernel(
   for (int r = 0; r < 16; ++r) bs_r[r] = b_slice ? b_slice[rowmap(r, g)] : 0.f;
   const float bs_i = b_slice ? b_slice[i] : 0.f;
   float *wpoint = w_out + ((int64_t)b * N + n0 + i) * (kH * kS);  // this lane's point (when it exists)
-
-  // round r: the x_mid wave makes the weights of heads 2 r and 2 r + 1 (the halves of its column tile r) and leaves them
-  // in LDS; the fx_mid wave sums the tokens of the two heads of round r - 1.  The two heads' dependent MFMA chains
-  // take turns.
-  static_for<kH / 2 + 1>([&](auto r_) {
-    constexpr int rr = decltype(r_)::value;
-    if (role == 0 && rr < kH / 2) {
-      constexpr int ct = rr < kH / 2 ? rr : 0;
-      float inv_t[2];
+  __syncthreads();
+  f32x16 xs[2], fs[2];  // this wave's two x_mid tiles (lanes <-> points) and fx_mid tiles (lanes <-> channels)
 #pragma unroll
-      for (int hf = 0; hf < 2; ++hf)
-        inv_t[hf] = temperature ? kLog2e / clamp_temperature(temperature[2 * ct + hf]) : kLog2e;
-      // lanes <-> points: the heads' softmax statistics
-      f32x16 lt[2];
+  for (int c = 0; c < 2; ++c) {
+    f32x16 got;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) lt[0][r] = lt[1][r] = bs_r[r];
+    for (int q = 0; q < 4; ++q) {
+      const u32x4 v = xchg[((1 - role) * 2 + c) * 256 + q * 64 + lane];
+      got[4 * q] = __uint_as_float(v[0]), got[4 * q + 1] = __uint_as_float(v[1]);
+      got[4 * q + 2] = __uint_as_float(v[2]), got[4 * q + 3] = __uint_as_float(v[3]);
+    }
 #pragma unroll
-      for (int m = 0; m < 8; ++m)
+    for (int r = 0; r < 16; ++r) {
+      xs[c][r] = role == 0 ? acc[c][r] : got[r];
+      fs[c][r] = role == 0 ? got[r] : acc[2 + c][r];
+    }
+  }
+  // heads 4 role + 2 c + {0, 1} are the halves of tile c; the two heads' dependent MFMA chains take turns
+  static_for<2>([&](auto c_) {
+    constexpr int c = decltype(c_)::value;
+    const int h0 = 4 * role + 2 * c;
+    float inv_t[2];
 #pragma unroll
-        for (int hf = 0; hf < 2; ++hf) lt[hf] = mma32(ws[m], acc[ct][8 * hf + m], lt[hf]);
+    for (int hf = 0; hf < 2; ++hf) inv_t[hf] = temperature ? kLog2e / clamp_temperature(temperature[h0 + hf]) : kLog2e;
+    // lanes <-> points: the heads' softmax statistics, and the weights as they leave (a lane holds 4 consecutive slices
+    // of its point per register quad)
+    f32x16 lt[2];
 #pragma unroll
-      for (int hf = 0; hf < 2; ++hf) {
-        float mx = lt[hf][0] * inv_t[hf];
+    for (int r = 0; r < 16; ++r) lt[0][r] = lt[1][r] = bs_r[r];
 #pragma unroll
-        for (int r = 1; r < 16; ++r) mx = fmaxf(mx, lt[hf][r] * inv_t[hf]);
-        mx = half_max(mx);
-        float sum = 0.f;
+    for (int m = 0; m < 8; ++m)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          lt[hf][r] = __builtin_amdgcn_exp2f(lt[hf][r] * inv_t[hf] - mx);
-          sum += lt[hf][r];
-        }
-        sum = half_sum(sum);
-        const float inv = 1.f / sum;
-        if (g == 0) {
-          stat[64 * hf + i] = mx;
-          stat[64 * hf + 32 + i] = inv;
-        }
-        // the weights leave from this orientation: a lane holds 4 consecutive slices of its point per register quad
-        if (i < valid) {
+      for (int hf = 0; hf < 2; ++hf) lt[hf] = mma32(ws[m], xs[c][8 * hf + m], lt[hf]);
 #pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            const float4 o = {lt[hf][4 * q] * inv, lt[hf][4 * q + 1] * inv, lt[hf][4 * q + 2] * inv, lt[hf][4 * q + 3] * inv};
-            *reinterpret_cast<float4 *>(wpoint + (2 * ct + hf) * kS + 8 * q + 4 * g) = o;
-          }
-        }
+    for (int hf = 0; hf < 2; ++hf) {
+      float mx = lt[hf][0] * inv_t[hf];
+#pragma unroll
+      for (int r = 1; r < 16; ++r) mx = fmaxf(mx, lt[hf][r] * inv_t[hf]);
+      mx = half_max(mx);
+      float sum = 0.f;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        lt[hf][r] = __builtin_amdgcn_exp2f(lt[hf][r] * inv_t[hf] - mx);
+        sum += lt[hf][r];
       }
-      __builtin_amdgcn_wave_barrier();
-      // lanes <-> slices, register r <-> point rowmap(r, g): the weights, as the A operand of the token sums
-      f32x16 ln[2];
-#pragma unroll
-      for (int r = 0; r < 16; ++r) ln[0][r] = ln[1][r] = bs_i;
-#pragma unroll
-      for (int m = 0; m < 8; ++m)
-#pragma unroll
-        for (int hf = 0; hf < 2; ++hf) ln[hf] = mma32(acc[ct][8 * hf + m], ws[m], ln[hf]);
-#pragma unroll
-      for (int hf = 0; hf < 2; ++hf) {
-        const int h = 2 * ct + hf;
-        float nrm = 0.f;
+      sum = half_sum(sum);
+      const float inv = 1.f / sum;
+      if (g == 0) {
+        stat[64 * hf + i] = mx;
+        stat[64 * hf + 32 + i] = inv;
+      }
+      if (i < valid) {
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-          const float4 mq = *reinterpret_cast<const float4 *>(stat + 64 * hf + 8 * q + 4 * g);
-          const float4 iq = *reinterpret_cast<const float4 *>(stat + 64 * hf + 32 + 8 * q + 4 * g);
-          const float mqa[4] = {mq.x, mq.y, mq.z, mq.w}, iqa[4] = {iq.x, iq.y, iq.z, iq.w};
-          u32x4 out;
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const int r = 4 * q + e, pt = 8 * q + 4 * g + e;
-            float wv = __builtin_amdgcn_exp2f(ln[hf][r] * inv_t[hf] - mqa[e]) * iqa[e];
-            if (pt >= valid) wv = 0.f;
-            out[e] = __float_as_uint(wv);
-            nrm += wv;
-          }
-          xchg[((rr & 1) * 2 + hf) * 256 + q * 64 + lane] = out;
+          const float4 o = {lt[hf][4 * q] * inv, lt[hf][4 * q + 1] * inv, lt[hf][4 * q + 2] * inv, lt[hf][4 * q + 3] * inv};
+          *reinterpret_cast<float4 *>(wpoint + (h0 + hf) * kS + 8 * q + 4 * g) = o;
         }
-        nrm = half_sum(nrm);
-        if (g == 0) mine[h * (kS * kD1) + i * kD1 + kD] = nrm;
       }
     }
-    if (role == 1 && rr > 0) {
-      constexpr int ct = rr > 0 ? rr - 1 : 0;
-      f32x16 tk[2];
+    __builtin_amdgcn_wave_barrier();
+    // lanes <-> slices, register r <-> point rowmap(r, g): the weights as the A operand of the token sums
+    f32x16 ln[2];
 #pragma unroll
-      for (int r = 0; r < 16; ++r) tk[0][r] = tk[1][r] = 0.f;
+    for (int r = 0; r < 16; ++r) ln[0][r] = ln[1][r] = bs_i;
+#pragma unroll
+    for (int m = 0; m < 8; ++m)
+#pragma unroll
+      for (int hf = 0; hf < 2; ++hf) ln[hf] = mma32(xs[c][8 * hf + m], ws[m], ln[hf]);
+#pragma unroll
+    for (int hf = 0; hf < 2; ++hf) {
+      float nrm = 0.f;
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
-        u32x4 wq[2];
+        const float4 mq = *reinterpret_cast<const float4 *>(stat + 64 * hf + 8 * q + 4 * g);
+        const float4 iq = *reinterpret_cast<const float4 *>(stat + 64 * hf + 32 + 8 * q + 4 * g);
+        const float mqa[4] = {mq.x, mq.y, mq.z, mq.w}, iqa[4] = {iq.x, iq.y, iq.z, iq.w};
 #pragma unroll
-        for (int hf = 0; hf < 2; ++hf) wq[hf] = xchg[(((rr - 1) & 1) * 2 + hf) * 256 + q * 64 + lane];
-#pragma unroll
-        for (int e = 0; e < 4; ++e)
-#pragma unroll
-          for (int hf = 0; hf < 2; ++hf) tk[hf] = mma32(__uint_as_float(wq[hf][e]), acc[ct][4 * q + e], tk[hf]);
+        for (int e = 0; e < 4; ++e) {
+          const int r = 4 * q + e, pt = 8 * q + 4 * g + e;
+          float wv = __builtin_amdgcn_exp2f(ln[hf][r] * inv_t[hf] - mqa[e]) * iqa[e];
+          if (pt >= valid) wv = 0.f;
+          ln[hf][r] = wv;
+          nrm += wv;
+        }
       }
-      // lane (i, g): channel 32 ct + i of fx_mid = channel i % 16 of head 2 ct + i / 16, register r <-> slice
-      // rowmap(r, g); each lane keeps the sums taken with its own head's weights
-      const int hf = i >> 4;
-#pragma unroll
-      for (int r = 0; r < 16; ++r)
-        mine[(2 * ct + hf) * (kS * kD1) + rowmap(r, g) * kD1 + (i & 15)] = hf ? tk[1][r] : tk[0][r];
+      nrm = half_sum(nrm);
+      if (g == 0) mine[(h0 + hf) * (kS * kD1) + i * kD1 + kD] = nrm;
     }
-    __syncthreads();
+    __builtin_amdgcn_wave_barrier();  // the statistics are read before the next pair overwrites them
+    f32x16 tk[2];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) tk[0][r] = tk[1][r] = 0.f;
+#pragma unroll
+    for (int m = 0; m < 16; ++m)
+#pragma unroll
+      for (int hf = 0; hf < 2; ++hf) tk[hf] = mma32(ln[hf][m], fs[c][m], tk[hf]);
+    // lane (i, g): channel i of the fx_mid tile = channel i % 16 of head h0 + i / 16, register r <-> slice
+    // rowmap(r, g); each lane keeps the sums taken with its own head's weights
+    const int hf = i >> 4;
+#pragma unroll
+    for (int r = 0; r < 16; ++r)
+      mine[(h0 + hf) * (kS * kD1) + rowmap(r, g) * kD1 + (i & 15)] = hf ? tk[1][r] : tk[0][r];
   });
+  __syncthreads();
   float *dst = partials + ((int64_t)gblk * B + b) * kTokFloats;
   for (int idx = tid; idx < kTokFloats; idx += 512)
     dst[idx] = ((red[idx] + red[kTokFloats + idx]) + red[2 * kTokFloats + idx]) + red[3 * kTokFloats + idx];
