@@ -2,7 +2,8 @@
 // slice weights of PA.py:172-203): the two k x k convolutions of the input, the slice logits, the temperature
 // softmax and the partial slice-token sums in one launch.
 //
-// Shape class: C = 128 channels, 8 heads of 16, 32 slices, 2-D grid, odd k.
+// Shape class: C = 128 channels, 8 heads of 16, 32 slices; 2-D grid with odd k, or Linear projections (the irregular
+// mesh, PA.py:501-514) as the 1 x 1 case.
 //
 // The convolutions are one implicit GEMM, M = points, N = 256 (x_mid | fx_mid), K = k k 128 (tap-major), computed
 // with float32 accuracy on the bf16 matrix cores: every float32 operand is cut into three bf16 pieces
@@ -401,19 +402,25 @@ __global__ __launch_bounds__(512) void conv_slice_kernel(
     dst[idx] = ((red[idx] + red[kTokFloats + idx]) + red[2 * kTokFloats + idx]) + red[3 * kTokFloats + idx];
 }
 
+// Linear projections (conv_k == 0: the irregular mesh) are the 1 x 1 case on an N x 1 grid
 bool supported(int dtype, const pa_shape &s) {
-  return dtype == PA_F32 && s.conv_k > 0 && s.conv_k % 2 == 1 && s.grid_d == 0 && s.C == kC && s.H == kH && s.D == kD &&
-         s.S == kS && s.grid_h * s.grid_w == s.N && s.N * kC < (int64_t)1 << 29;
+  if (dtype != PA_F32 || s.C != kC || s.H != kH || s.D != kD || s.S != kS || s.N * kC >= (int64_t)1 << 29) return false;
+  if (s.conv_k == 0) return s.grid_d == 0;
+  return s.conv_k % 2 == 1 && s.grid_d == 0 && s.grid_h * s.grid_w == s.N;
 }
 
 int64_t groups(const pa_shape &s) { return ((s.N + 31) / 32 + 3) / 4; }
 
-int64_t blob_bytes(const pa_shape &s) { return s.conv_k * s.conv_k * kStepsPerTap * (int64_t)kStepUnits * 16 + 64; }
+int64_t blob_bytes(const pa_shape &s) {
+  const int64_t k = s.conv_k > 0 ? s.conv_k : 1;
+  return k * k * kStepsPerTap * (int64_t)kStepUnits * 16 + 64;
+}
 
 int front(const pa_shape &s, const pa_params &p, const void *x, void *blob, void *w, float *partials, void *blob_out,
           const pa_block_mlp *mlp, hipStream_t st) {
   if (!supported(PA_F32, s)) return PA_ERR_UNSUPPORTED;
-  const int taps = (int)(s.conv_k * s.conv_k);
+  const int ks = s.conv_k > 0 ? (int)s.conv_k : 1, taps = ks * ks;
+  const int gh = s.conv_k > 0 ? (int)s.grid_h : (int)s.N, gw = s.conv_k > 0 ? (int)s.grid_w : 1;
   const int64_t units = (int64_t)taps * kStepsPerTap * kColTiles * 64;
   const int conv_blocks = (int)((units + 255) / 256);
   const int extra = !blob_out ? 0 : 8 + (mlp ? (int)(mlp->F / 128) * 16 : 0);
@@ -431,7 +438,7 @@ int front(const pa_shape &s, const pa_params &p, const void *x, void *blob, void
                      static_cast<const u32x4 *>(blob), p.in_project_x_bias, p.in_project_fx_bias,
                      static_cast<const float *>(p.in_project_slice_weight), p.in_project_slice_bias, p.temperature,
                      static_cast<const float *>(x), static_cast<float *>(w), partials, (int)s.B, (int)s.N,
-                     (int)s.grid_h, (int)s.grid_w, (int)s.conv_k, bpb);
+                     gh, gw, ks, bpb);
   return launch_status();
 }
 

@@ -80,8 +80,8 @@ def test_fp32_structured2d_fused_front_end(kernel, grid, B):
 
 @pytest.mark.parametrize("B,N", [(2, 500), (1, 33), (3, 4100)])
 def test_fp32_irregular_row_kernel_back_end(B, N):
-    # C = 128, 8 heads of 16, 32 slices, irregular mesh: the layer call hands back to the points, applies out_linear
-    # and the block tail in the float32 row kernel (split-bf16 products); the front end runs the general kernels
+    # C = 128, 8 heads of 16, 32 slices, irregular mesh: the layer call runs the fused front end (Linear projections as
+    # its 1 x 1 case) and hands back to the points, applies out_linear and the block tail in the float32 row kernel
     announce("fp32 irregular, row-kernel back end", B, N)
     dim, heads, dim_head, S = 128, 8, 16, 32
     ref, hip = make_pair("irregular", dim, heads, dim_head, S, sharpen=2.0, temps=[0.3 + 5.7 * i / 7 for i in range(8)])
