@@ -152,6 +152,47 @@ __device__ __forceinline__ void stage_gamma_beta(float *gb, const Tail &tail, in
   }
 }
 
+// The batch's attended slice tokens (H, S, D float32, 16 KB) as the block-diagonal A operands of the hand-back:
+// tokp[(pair 4 + kk) 3 + piece][lane], lane (i, g): row (hh, d) = (i / 16, i % 16), reduction index k = 16 kk + 8 g + j
+// over (head of the pair, slice) -- out_token[2 pair + hh][k % 32][d] where k / 32 == hh, else 0.  The tokens are read
+// once, coalesced (4 float4 per thread, fetched by the caller ahead of its other loads), put into `raw` (4096 floats
+// of LDS scratch) and cut from there.  Ends with a barrier.
+__device__ __forceinline__ void fetch_tokens(const float *tok, float4 (&t4)[4], int tid) {
+#pragma unroll
+  for (int q = 0; q < 4; ++q) t4[q] = reinterpret_cast<const float4 *>(tok)[tid + 256 * q];
+}
+__device__ __forceinline__ void build_token_operands(const float4 (&t4)[4], float *raw, u32x4 *tokp, int tid) {
+#pragma unroll
+  for (int q = 0; q < 4; ++q) reinterpret_cast<float4 *>(raw)[tid + 256 * q] = t4[q];
+  __syncthreads();
+  for (int item = tid; item < 16 * 64; item += 256) {
+    const int pk = item >> 6, l = item & 63, li = l & 31, lg = l >> 5;
+    const int pair = pk >> 2, kk = pk & 3, hh = li >> 4, d = li & 15;
+    float e[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int k = 16 * kk + 8 * lg + j;
+      e[j] = (k >> 5) == hh ? raw[((2 * pair + hh) * kS + (k & 31)) * kD + d] : 0.f;
+    }
+    u32x4 pl[3];
+    split8(e, pl);
+#pragma unroll
+    for (int p = 0; p < 3; ++p) tokp[(pk * 3 + p) * 64 + l] = pl[p];
+  }
+  __syncthreads();
+}
+
+// acc[t][r] += v[32 t + rowmap(r, g)] for a vector v of 128 floats in LDS (4 consecutive channels per register quad)
+__device__ __forceinline__ void add_channel_vector(f32x16 (&acc)[4], const float *v, int g) {
+#pragma unroll
+  for (int t = 0; t < 4; ++t)
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const float4 b = *reinterpret_cast<const float4 *>(v + 32 * t + 8 * q + 4 * g);
+      acc[t][4 * q] += b.x, acc[t][4 * q + 1] += b.y, acc[t][4 * q + 2] += b.z, acc[t][4 * q + 3] += b.w;
+    }
+}
+
 // ---------------------------------------------------------------------------------------------------------------
 // deslice_linear_kernel.  A workgroup's four tiles belong to one batch.  LDS: W_out as 8 units (96 KB), the batch's
 // attended slice tokens as A operands (48 KB), gamma | beta.
@@ -175,22 +216,8 @@ __global__ __launch_bounds__(256) void deslice_linear_kernel(const u32x4 *__rest
   const int n = min(n0 + i, N - 1);
   const bool ok = n0 + i < N;
   stage_gamma_beta(gb, tail, tid);
-  // the batch's tokens as block-diagonal A operands
-  const float *tok = out_token + (int64_t)b * kH * kS * kD;
-  for (int item = tid; item < 16 * 64; item += 256) {
-    const int pk = item >> 6, l = item & 63, li = l & 31, lg = l >> 5;
-    const int pair = pk >> 2, kk = pk & 3, hh = li >> 4, d = li & 15;
-    float e[8];
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const int k = 16 * kk + 8 * lg + j;
-      e[j] = (k >> 5) == hh ? tok[((2 * pair + hh) * kS + (k & 31)) * kD + d] : 0.f;
-    }
-    u32x4 pl[3];
-    split8(e, pl);
-#pragma unroll
-    for (int p = 0; p < 3; ++p) tokp[(pk * 3 + p) * 64 + l] = pl[p];
-  }
+  float4 tok4[4];
+  fetch_tokens(out_token + (int64_t)b * kH * kS * kD, tok4, tid);
   // this lane's half of its point's weights (two runs of 8 per head), and the output bias
   float wr[4][4][8];  // [head pair][kk][j]
   {
@@ -210,6 +237,8 @@ __global__ __launch_bounds__(256) void deslice_linear_kernel(const u32x4 *__rest
   for (int t = 0; t < 4; ++t)
 #pragma unroll
     for (int r = 0; r < 16; ++r) yT[t][r] = b_out ? b_out[32 * t + rowmap(r, g)] : 0.f;
+  // the batch's tokens as block-diagonal A operands (W_out's slots are still empty: their first 16 KB are the scratch)
+  build_token_operands(tok4, reinterpret_cast<float *>(smem), tokp, tid);
   // Every load above is complete (the builtin, so that the compiler knows it too) before W_out is requested: from here
   // on vmcnt counts this wave's 24 requests only, and the first product runs while they land.
   __builtin_amdgcn_s_waitcnt(0x0F70);
@@ -430,32 +459,18 @@ __global__ __launch_bounds__(256) void block_tail_kernel(const u32x4 *__restrict
     else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
   };
+  // every global load of the prologue is issued before the first of them is used: one round trip to memory
+  float sv[6] = {1.f, 0.f, 1.f, 0.f, 0.f, 0.f};
   if (tid < kC) {
-    gb2[tid] = a.ln2_gamma[tid];
-    gb2[kC + tid] = a.ln2_beta[tid];
-    gbn[tid] = a.next.gamma ? a.next.gamma[tid] : 1.f;
-    gbn[kC + tid] = a.next.beta ? a.next.beta[tid] : 0.f;
-    bo[tid] = a.b_out ? a.b_out[tid] : 0.f;
-    bb2[tid] = a.b2 ? a.b2[tid] : 0.f;
+    sv[0] = a.ln2_gamma[tid];
+    sv[1] = a.ln2_beta[tid];
+    if (a.next.gamma) sv[2] = a.next.gamma[tid];
+    if (a.next.beta) sv[3] = a.next.beta[tid];
+    if (a.b_out) sv[4] = a.b_out[tid];
+    if (a.b2) sv[5] = a.b2[tid];
   }
-  for (int k = tid; k < F; k += 256) bb1[k] = a.b1 ? a.b1[k] : 0.f;
-  for (int k = tid; k < a.head_O * kC; k += 256) hw[k] = a.head_w[k];
-  // the batch's tokens as block-diagonal A operands (deslice_linear_kernel)
-  const float *tok = a.out_token + (int64_t)b * kH * kS * kD;
-  for (int item = tid; item < 16 * 64; item += 256) {
-    const int pk = item >> 6, l = item & 63, li = l & 31, lg = l >> 5;
-    const int pair = pk >> 2, kk = pk & 3, hh = li >> 4, d = li & 15;
-    float e[8];
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const int k = 16 * kk + 8 * lg + j;
-      e[j] = (k >> 5) == hh ? tok[((2 * pair + hh) * kS + (k & 31)) * kD + d] : 0.f;
-    }
-    u32x4 pl[3];
-    split8(e, pl);
-#pragma unroll
-    for (int p = 0; p < 3; ++p) tokp[(pk * 3 + p) * 64 + l] = pl[p];
-  }
+  float4 tok4[4];
+  fetch_tokens(a.out_token + (int64_t)b * kH * kS * kD, tok4, tid);
   // this lane's half of its point's weights and of its residual row
   float wr[4][4][8];
   {
@@ -478,6 +493,16 @@ __global__ __launch_bounds__(256) void block_tail_kernel(const u32x4 *__restrict
       const float4 r = *reinterpret_cast<const float4 *>(a.fx_in + row * kC + 32 * t + 8 * q + 4 * g);
       fx1[t][4 * q] = r.x, fx1[t][4 * q + 1] = r.y, fx1[t][4 * q + 2] = r.z, fx1[t][4 * q + 3] = r.w;
     }
+  if (tid < kC) {
+    gb2[tid] = sv[0], gb2[kC + tid] = sv[1];
+    gbn[tid] = sv[2], gbn[kC + tid] = sv[3];
+    bo[tid] = sv[4], bb2[tid] = sv[5];
+  }
+  for (int k = tid; k < F; k += 256) bb1[k] = a.b1 ? a.b1[k] : 0.f;
+  for (int k = tid; k < a.head_O * kC; k += 256) hw[k] = a.head_w[k];
+  // the batch's tokens as block-diagonal A operands (the ring's first slots are still empty: 16 KB of them are the
+  // scratch)
+  build_token_operands(tok4, reinterpret_cast<float *>(smem), tokp, tid);
   // every load above is complete (the builtin, so that the compiler knows it too) before the weights are requested
   __builtin_amdgcn_s_waitcnt(0x0F70);
   issue_upto(8);
@@ -503,10 +528,7 @@ __global__ __launch_bounds__(256) void block_tail_kernel(const u32x4 *__restrict
   __syncthreads();  // the tokens are used up: their slots join the ring
   issue_upto(kMlpRing);
   // fx1 = W_out out_x^T + b_out + fx_in
-#pragma unroll
-  for (int t = 0; t < 4; ++t)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) fx1[t][r] += bo[32 * t + rowmap(r, g)];
+  add_channel_vector(fx1, bo, g);
   wait_landed(8);
 #pragma unroll
   for (int ks = 0; ks < 8; ++ks) {
@@ -537,23 +559,25 @@ __global__ __launch_bounds__(256) void block_tail_kernel(const u32x4 *__restrict
 #pragma unroll
     for (int t = 0; t < 4; ++t)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int c = 32 * t + rowmap(r, g);
-        nT[t][r] = (fx1[t][r] - mean) * rstd * gb2[c] + gb2[kC + c];
+      for (int q = 0; q < 4; ++q) {
+        const int c0 = 32 * t + 8 * q + 4 * g;
+        const float4 ga = *reinterpret_cast<const float4 *>(gb2 + c0), be = *reinterpret_cast<const float4 *>(gb2 + kC + c0);
+        nT[t][4 * q] = (fx1[t][4 * q] - mean) * rstd * ga.x + be.x;
+        nT[t][4 * q + 1] = (fx1[t][4 * q + 1] - mean) * rstd * ga.y + be.y;
+        nT[t][4 * q + 2] = (fx1[t][4 * q + 2] - mean) * rstd * ga.z + be.z;
+        nT[t][4 * q + 3] = (fx1[t][4 * q + 3] - mean) * rstd * ga.w + be.w;
       }
   }
   // the MLP; its second product accumulates on top of fx1 + b2
-#pragma unroll
-  for (int t = 0; t < 4; ++t)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) fx1[t][r] += bb2[32 * t + rowmap(r, g)];
+  add_channel_vector(fx1, bb2, g);
   for (int c = 0; c < F / 128; ++c) {
     const int base = 8 + 16 * c;
     f32x16 hT[4];
 #pragma unroll
     for (int t = 0; t < 4; ++t)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) hT[t][r] = bb1[128 * c + 32 * t + rowmap(r, g)];
+      for (int r = 0; r < 16; ++r) hT[t][r] = 0.f;
+    add_channel_vector(hT, bb1 + 128 * c, g);
     wait_landed(base + 8);
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) {
