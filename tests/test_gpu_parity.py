@@ -140,6 +140,26 @@ def test_fp32_whole_block_in_one_call(spatial, B, mlp_ratio, last):
         assert_fp32_close(whole[1], want, "block output, head in the call")
 
 
+def test_fp32_fused_path_is_bit_reproducible():
+    # the float32 kernels stream weights and rows through LDS rings with asynchronous loads and reduce the token sums
+    # in a fixed order: repeated calls on the same inputs must agree to the bit (a race would show up here first);
+    # model, block and layer level, cfg1's shape
+    announce("fp32 fused path: run-to-run bit equality")
+    torch.manual_seed(5)
+    m = pn.Transolver(functional_dim=1, embedding_dim=2, out_dim=1, n_layers=4, n_hidden=128, n_head=8, mlp_ratio=1,
+                      slice_num=32, structured_shape=(85, 85), unified_pos=False, use_te=False).eval().cuda()
+    lin = torch.linspace(0, 1, 85)
+    pos = torch.stack(torch.meshgrid(lin, lin, indexing="ij"), -1).reshape(1, 7225, 2).repeat(4, 1, 1).cuda()
+    fx = torch.randn(4, 7225, 1).cuda()
+    x = torch.randn(4, 7225, 128).cuda()
+    with torch.no_grad():
+        first = (m(fx, pos), m.blocks[1](x), m.blocks[1].Attn(x))
+        for _ in range(5):
+            again = (m(fx, pos), m.blocks[1](x), m.blocks[1].Attn(x))
+            for a, b in zip(first, again):
+                assert torch.equal(a, b)
+
+
 @pytest.mark.parametrize("kernel,grid", [(3, (4, 4, 4)), (3, (8, 8, 8)), (5, (8, 8, 8)), (3, (3, 5, 7)), (1, (4, 6, 5))])
 def test_fp32_structured3d_stages_and_layer(kernel, grid):
     announce("fp32 structured3d", kernel, grid)
