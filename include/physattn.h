@@ -55,6 +55,14 @@ extern "C" {
 /* Library version (major*10000 + minor*100 + patch). No reference counterpart. */
 int pa_version(void);
 
+/* 1 when marker ranges are on: the process environment held PA_ROCTX=1 when the library first looked and a roctx
+ * library (librocprofiler-sdk-roctx / libroctx64) could be opened at run time; 0 otherwise.  With ranges on, the
+ * layer-, block- and MLP-level entry points push a range named after themselves, and the fused layer brackets its
+ * three stages with "_compute_slices_from_projections", "_compute_slice_attention_sdpa" and
+ * "_project_attention_outputs" — the names of the reference's stages and of its record_function ranges
+ * (physicsnemo/nn/module/physics_attention.py:358,445,490) — for `rocprofv3 --marker-trace`. */
+int pa_markers_enabled(void);
+
 /* Static text for a PA_ERR_* code (or "hip error" for positive codes). No reference counterpart. */
 const char *pa_status_string(int code);
 

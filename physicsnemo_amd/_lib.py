@@ -35,7 +35,7 @@ EXPORTED = [
     "pa_mfma_layer_forward", "pa_rows_gemm_act", "pa_layernorm_backward_groups", "pa_layernorm_backward",
     "pa_static_scratch_bytes", "pa_slice_reduce_static",
     "pa_preprocess_query", "pa_preprocess_workspace_bytes", "pa_preprocess_forward",
-    "pa_block_query", "pa_block_workspace_bytes", "pa_block_forward",
+    "pa_block_query", "pa_block_workspace_bytes", "pa_block_forward", "pa_markers_enabled",
 ]
 
 PA_BUF_BLOB, PA_BUF_FX_PACK, PA_BUF_W_PACK, PA_BUF_PARTIALS, PA_BUF_TOKP = range(5)
@@ -98,6 +98,8 @@ def load() -> ctypes.CDLL:
     ps, pp, pt = POINTER(PaShape), POINTER(PaParams), POINTER(PaBlockTail)
     lib.pa_version.restype = c_int
     lib.pa_version.argtypes = []
+    lib.pa_markers_enabled.restype = c_int
+    lib.pa_markers_enabled.argtypes = []
     lib.pa_status_string.restype = c_char_p
     lib.pa_status_string.argtypes = [c_int]
     lib.pa_workspace_bytes.restype = c_int64

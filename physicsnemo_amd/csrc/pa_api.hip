@@ -1,10 +1,55 @@
 // C ABI of libphysattn.so: argument validation, workspace carving and dispatch.  No kernels here.
+#include <dlfcn.h>
+#include <stdlib.h>
+
 #include "pa_common.h"
 #include "pa_host.h"
 
 namespace {
 
 using pa::aligned16;
+
+// Optional marker ranges for rocprofv3 --marker-trace, in place of the reference's record_function brackets around its
+// stages ("_compute_slice_attention_sdpa", "_project_attention_outputs": physics_attention.py:445,490).  Off unless
+// the environment holds PA_ROCTX=1 when the first entry point runs; the marker library is looked up at run time, so
+// the library has no link-time dependency on it and runs without it.  A range covers the host-side enqueue of its
+// stage (the kernels themselves are asynchronous), as the reference's ranges do.
+struct Markers {
+  int (*push)(const char *);
+  int (*pop)();
+};
+
+const Markers &markers() {
+  static const Markers m = [] {
+    Markers r{nullptr, nullptr};
+    const char *e = getenv("PA_ROCTX");
+    if (!e || e[0] == '\0' || e[0] == '0') return r;
+    const char *names[] = {"librocprofiler-sdk-roctx.so.1", "librocprofiler-sdk-roctx.so", "libroctx64.so.4", "libroctx64.so",
+                           "/opt/rocm/lib/librocprofiler-sdk-roctx.so", "/opt/rocm/lib/libroctx64.so"};
+    for (const char *n : names) {
+      void *h = dlopen(n, RTLD_NOW | RTLD_GLOBAL);
+      if (!h) continue;
+      r.push = reinterpret_cast<int (*)(const char *)>(dlsym(h, "roctxRangePushA"));
+      r.pop = reinterpret_cast<int (*)()>(dlsym(h, "roctxRangePop"));
+      if (r.push && r.pop) return r;
+      r = Markers{nullptr, nullptr};
+    }
+    return r;
+  }();
+  return m;
+}
+
+struct Range {
+  bool on;
+  explicit Range(const char *name) : on(markers().push != nullptr) {
+    if (on) markers().push(name);
+  }
+  ~Range() {
+    if (on) markers().pop();
+  }
+  Range(const Range &) = delete;
+  Range &operator=(const Range &) = delete;
+};
 
 int check_shape(int dtype, const pa_shape *s) {
   if (!s) return PA_ERR_NULL;
@@ -261,13 +306,21 @@ int mfma_layer(const pa_shape &s, const pa_params &p, const void *blob, const vo
                                   tail_active(tail) ? tail : nullptr, wts + 2 * pa::mlp::linear_blob_bytes(s.C),
                                   compute_units(), st);
   }
-  if (pa::mfma::fuse_reduce(s)) {  // kernel (a) also leaves the partial slice-token sums
-    if ((rc = pa::mfma::project_softmax(s, blob, x, nullptr, wp, partials, compute_units(), st))) return rc;
-  } else {
-    if ((rc = pa::mfma::project_softmax(s, blob, x, fxp, wp, nullptr, compute_units(), st))) return rc;
-    if ((rc = pa::mfma::slice_reduce(s, wp, fxp, partials, st))) return rc;
+  {
+    Range r("_compute_slices_from_projections");
+    if (pa::mfma::fuse_reduce(s)) {  // kernel (a) also leaves the partial slice-token sums
+      if ((rc = pa::mfma::project_softmax(s, blob, x, nullptr, wp, partials, compute_units(), st))) return rc;
+    } else {
+      if ((rc = pa::mfma::project_softmax(s, blob, x, fxp, wp, nullptr, compute_units(), st))) return rc;
+      if ((rc = pa::mfma::slice_reduce(s, wp, fxp, partials, st))) return rc;
+    }
   }
-  if ((rc = pa::mfma::combine_attention(s, p, p.in_project_fx_bias, partials, mp.G, tok, norm, tok_out, tokp, st))) return rc;
+  {
+    Range r("_compute_slice_attention_sdpa");
+    if ((rc = pa::mfma::combine_attention(s, p, p.in_project_fx_bias, partials, mp.G, tok, norm, tok_out, tokp, st)))
+      return rc;
+  }
+  Range r("_project_attention_outputs");
   return pa::mfma::deslice_project(s, blob, wp, tokp, y, tail_active(tail) ? tail : nullptr, compute_units(), st);
 }
 
@@ -276,6 +329,8 @@ int mfma_layer(const pa_shape &s, const pa_params &p, const void *blob, const vo
 extern "C" {
 
 int pa_version(void) { return 100; }
+
+int pa_markers_enabled(void) { return markers().push != nullptr ? 1 : 0; }
 
 const char *pa_status_string(int code) {
   switch (code) {
@@ -857,6 +912,7 @@ int pa_mlp_pack(int dtype, int64_t C, int64_t F, const pa_mlp_params *p, void *p
 
 int pa_mlp_forward_packed(int dtype, int64_t rows, int64_t C, int64_t F, const void *packed, const float *b1,
                           const float *b2, const void *u, void *y, const pa_block_tail *tail, void *stream) {
+  Range entry("pa_mlp_forward_packed");
   if (rows <= 0 || C <= 0 || F <= 0) return PA_ERR_DIMS;
   if (!mlp_served(dtype, rows, C, F)) return PA_ERR_UNSUPPORTED;
   if (!packed || !b1 || !b2 || !u || !y) return PA_ERR_NULL;
@@ -872,6 +928,7 @@ int pa_mlp_forward_packed(int dtype, int64_t rows, int64_t C, int64_t F, const v
 
 int pa_mlp_forward(int dtype, int64_t rows, int64_t C, int64_t F, const pa_mlp_params *p, const void *u, void *y,
                    const pa_block_tail *tail, void *workspace, int64_t workspace_bytes, void *stream) {
+  Range entry("pa_mlp_forward");
   if (rows <= 0 || C <= 0 || F <= 0) return PA_ERR_DIMS;
   if (!mlp_served(dtype, rows, C, F)) return PA_ERR_UNSUPPORTED;
   if (!p || !p->w1 || !p->b1 || !p->w2 || !p->b2 || !u || !y || !workspace) return PA_ERR_NULL;
@@ -903,6 +960,7 @@ int64_t pa_preprocess_workspace_bytes(int dtype, int64_t rows, int64_t c_in, int
 int pa_preprocess_forward(int dtype, int64_t rows, int64_t c_in, int64_t F, int64_t C, const pa_mlp_params *p,
                           const void *u, void *y, const pa_block_tail *tail, void *workspace, int64_t workspace_bytes,
                           void *stream) {
+  Range entry("pa_preprocess_forward");
   if (rows <= 0 || c_in <= 0 || F <= 0 || C <= 0) return PA_ERR_DIMS;
   if (!pa::f32rows::premlp_supported(dtype, rows, c_in, F, C)) return PA_ERR_UNSUPPORTED;
   if (!p || !p->w1 || !p->b1 || !p->w2 || !p->b2 || !u || !y || !workspace) return PA_ERR_NULL;
@@ -917,6 +975,7 @@ int pa_preprocess_forward(int dtype, int64_t rows, int64_t c_in, int64_t F, int6
 int pa_mfma_layer_forward(const pa_shape *shape, const pa_params *p, const void *blob, const void *x, void *y,
                           const pa_block_tail *tail, float *slice_token_out, void *workspace, int64_t workspace_bytes,
                           void *stream) {
+  Range entry("pa_mfma_layer_forward");
   int rc = check_mfma(shape);
   if (rc) return rc;
   if (!p || !p->qkv_project_weight || !blob || !x || !y || !workspace) return PA_ERR_NULL;
@@ -938,6 +997,7 @@ int pa_mfma_layer_forward(const pa_shape *shape, const pa_params *p, const void 
 int pa_layer_forward(int dtype, const pa_shape *shape, const pa_params *p, const void *x, void *y,
                      const pa_block_tail *tail, float *slice_token_out, void *workspace, int64_t workspace_bytes,
                      void *stream) {
+  Range entry("pa_layer_forward");
   int rc = check_shape(dtype, shape);
   if (rc) return rc;
   if ((rc = check_params(p))) return rc;
@@ -1072,6 +1132,7 @@ int64_t pa_block_workspace_bytes(int dtype, const pa_shape *shape, int64_t F) {
 int pa_block_forward(int dtype, const pa_shape *shape, const pa_params *p, const pa_block_mlp *mlp, const void *x,
                      const void *fx_in, void *fx_out, const pa_block_tail *next, const pa_block_head *head,
                      void *workspace, int64_t workspace_bytes, void *stream) {
+  Range entry("pa_block_forward");
   int rc = check_shape(dtype, shape);
   if (rc) return rc;
   if ((rc = check_params(p))) return rc;
@@ -1237,6 +1298,7 @@ int64_t pa_layer_forward_plus_workspace_bytes(int dtype, const pa_shape *shape) 
 int pa_layer_forward_plus(int dtype, const pa_shape *shape, const pa_params *p, const pa_plus_params *plus,
                           const void *x, const void *uniform, void *y, const pa_block_tail *tail,
                           float *slice_token_out, void *workspace, int64_t workspace_bytes, void *stream) {
+  Range entry("pa_layer_forward_plus");
   int rc = check_shape(dtype, shape);
   if (rc) return rc;
   if (!p || !plus || !x || !uniform || !y || !workspace) return PA_ERR_NULL;

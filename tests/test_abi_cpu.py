@@ -25,6 +25,20 @@ def test_library_loads_and_exports_every_declared_symbol():
     assert lib.pa_status_string(0) == b"ok"
 
 
+def test_marker_ranges_follow_the_environment():
+    """PA_ROCTX=1 turns the roctx ranges on (the marker library is opened at run time); without it they are off."""
+    import subprocess
+    import sys
+    code = "from physicsnemo_amd import _lib; print(_lib.load().pa_markers_enabled())"
+    for value, expected in ((None, "0"), ("0", "0"), ("1", "1")):
+        env = {k: v for k, v in os.environ.items() if k != "PA_ROCTX"}
+        if value is not None:
+            env["PA_ROCTX"] = value
+        out = subprocess.run([sys.executable, "-c", code], cwd=ROOT, env=env, capture_output=True, text=True, timeout=120)
+        assert out.returncode == 0, out.stderr
+        assert out.stdout.strip().splitlines()[-1] == expected, (value, out.stdout, out.stderr)
+
+
 def _shape(**kw):
     base = dict(B=1, N=64, C=64, H=2, D=32, S=16, grid_h=0, grid_w=0, conv_k=0)
     base.update(kw)
