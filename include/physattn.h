@@ -51,6 +51,10 @@ extern "C" {
 /* Limits of the general kernels (PA_ERR_UNSUPPORTED beyond them). */
 #define PA_MAX_D 128
 #define PA_MAX_S 256
+/* Limits of the entry points that take plain row / column counts instead of a shape struct, the column GEMMs
+ * (PA_ERR_UNSUPPORTED beyond them): sizes are refused before any product of them is formed. */
+#define PA_MAX_ROWS (1ll << 40)
+#define PA_MAX_COLS (1ll << 24)
 
 /* Library version (major*10000 + minor*100 + patch). No reference counterpart. */
 int pa_version(void);

@@ -58,22 +58,32 @@ int check_shape(int dtype, const pa_shape *s) {
   if (s->B <= 0 || s->N <= 0 || s->C <= 0 || s->H <= 0 || s->D <= 0 || s->S <= 0) return PA_ERR_DIMS;
   if (s->conv_k < 0 || (s->conv_k == 0 && s->grid_d != 0)) return PA_ERR_DIMS;
   if (s->conv_tap_major != 0 && s->conv_tap_major != 1) return PA_ERR_DIMS;
-  if (s->conv_k > 0) {
-    if (s->grid_h <= 0 || s->grid_w <= 0 || s->grid_d < 0) return PA_ERR_DIMS;
-    if (s->grid_h * s->grid_w * (s->grid_d > 0 ? s->grid_d : 1) != s->N) return PA_ERR_DIMS;
-    const int64_t taps = s->conv_k * s->conv_k * (s->grid_d > 0 ? s->conv_k : 1);
-    if (taps * s->C > (int64_t)1 << 30) return PA_ERR_UNSUPPORTED;
-    if (s->conv_k % 2 == 0) return PA_ERR_UNSUPPORTED;  // even kernels change the output size in the reference
-  }
+  // the range of every single field first: none of the products below, here or in the workspace plans, can overflow
   if (s->D > PA_MAX_D || s->S > PA_MAX_S) return PA_ERR_UNSUPPORTED;
   if (s->C > (1 << 16) || s->H > 1024) return PA_ERR_UNSUPPORTED;
   if (s->N > (int64_t)1 << 31 || s->B > (1 << 20)) return PA_ERR_UNSUPPORTED;
   if (s->B * s->H > 65535) return PA_ERR_UNSUPPORTED;  // grid.y of the reduction
+  if (s->conv_k > 0) {
+    if (s->grid_h <= 0 || s->grid_w <= 0 || s->grid_d < 0) return PA_ERR_DIMS;
+    if (s->grid_h > s->N || s->grid_w > s->N || s->grid_d > s->N) return PA_ERR_DIMS;
+    const int64_t plane = s->grid_h * s->grid_w;  // at most 2^62
+    if (plane > s->N || plane * (s->grid_d > 0 ? s->grid_d : 1) != s->N) return PA_ERR_DIMS;
+    if (s->conv_k > 1024) return PA_ERR_UNSUPPORTED;
+    const int64_t taps = s->conv_k * s->conv_k * (s->grid_d > 0 ? s->conv_k : 1);
+    if (taps * s->C > (int64_t)1 << 30) return PA_ERR_UNSUPPORTED;
+    if (s->conv_k % 2 == 0) return PA_ERR_UNSUPPORTED;  // even kernels change the output size in the reference
+  }
   if (pa::general::combine_attn_lds_bytes(*s) > pa::kMaxLdsBytes) return PA_ERR_UNSUPPORTED;
   return PA_OK;
 }
 
 int64_t round_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
+
+// Limits of the row-count / column-count entry points (those without a pa_shape): sizes beyond them are refused
+// before any product of them is formed.
+constexpr int64_t kMaxRows = PA_MAX_ROWS, kMaxCols = PA_MAX_COLS;
+bool rows_ok(int64_t rows) { return rows <= kMaxRows; }
+bool cols_ok(int64_t cols) { return cols <= kMaxCols; }
 
 int64_t elem_bytes(int dtype) { return dtype == PA_F32 ? 4 : 2; }
 
@@ -671,12 +681,14 @@ int pa_layernorm_backward(int dtype, int64_t rows, int64_t C, const void *x, con
 
 int64_t pa_cols_gemm_chunks(int64_t rows, int64_t cols_a) {
   if (rows <= 0 || cols_a <= 0) return PA_ERR_DIMS;
+  if (!rows_ok(rows) || !cols_ok(cols_a)) return PA_ERR_UNSUPPORTED;
   return pa::gemm::cols_gemm_chunks(rows, cols_a, compute_units());
 }
 
 int pa_cols_gemm(int64_t rows, const void *a, int64_t lda, int64_t cols_a, const void *b, int64_t ldb, int64_t cols_b,
                  float *partials, float *col_sum_partials, void *stream) {
   if (rows <= 0 || cols_a <= 0 || cols_b <= 0 || lda < cols_a || ldb < cols_b) return PA_ERR_DIMS;
+  if (!rows_ok(rows) || !cols_ok(lda) || !cols_ok(ldb)) return PA_ERR_UNSUPPORTED;
   if (!a || !b || !partials) return PA_ERR_NULL;
   if (!aligned16(a) || !aligned16(b) || !aligned16(partials)) return PA_ERR_ALIGN;
   return pa::gemm::cols_gemm(a, lda, cols_a, b, ldb, cols_b, rows, partials, col_sum_partials, compute_units(),
@@ -707,12 +719,14 @@ int pa_ball_query_cells(int64_t batch, int64_t n_points, int64_t n_queries, int6
 
 int64_t pa_cols_gemm_f32_chunks(int64_t rows, int64_t cols_a, int64_t cols_b) {
   if (rows <= 0 || cols_a <= 0 || cols_b <= 0) return PA_ERR_DIMS;
+  if (!rows_ok(rows) || !cols_ok(cols_a) || !cols_ok(cols_b)) return PA_ERR_UNSUPPORTED;
   return pa::gemm::cols_gemm_f32_chunks(rows, cols_a, cols_b, compute_units());
 }
 
 int pa_cols_gemm_f32(int64_t rows, const void *a, int64_t lda, int64_t cols_a, const void *b, int64_t ldb,
                      int64_t cols_b, float *partials, float *col_sum_partials, void *stream) {
   if (rows <= 0 || cols_a <= 0 || cols_b <= 0 || lda < cols_a || ldb < cols_b) return PA_ERR_DIMS;
+  if (!rows_ok(rows) || !cols_ok(lda) || !cols_ok(ldb)) return PA_ERR_UNSUPPORTED;
   if (!a || !b || !partials) return PA_ERR_NULL;
   if (!aligned16(a) || !aligned16(b) || !aligned16(partials)) return PA_ERR_ALIGN;
   return pa::gemm::cols_gemm_f32(a, lda, cols_a, b, ldb, cols_b, rows, partials, col_sum_partials, compute_units(),
