@@ -51,6 +51,7 @@ extern "C" {
 /* Limits of the general kernels (PA_ERR_UNSUPPORTED beyond them). */
 #define PA_MAX_D 128
 #define PA_MAX_S 256
+#define PA_MAX_N 2147483647ll /* points per batch element */
 /* Limits of the entry points that take plain row / column counts instead of a shape struct, the column GEMMs
  * (PA_ERR_UNSUPPORTED beyond them): sizes are refused before any product of them is formed. */
 #define PA_MAX_ROWS (1ll << 40)

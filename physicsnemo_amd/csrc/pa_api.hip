@@ -61,7 +61,7 @@ int check_shape(int dtype, const pa_shape *s) {
   // the range of every single field first: none of the products below, here or in the workspace plans, can overflow
   if (s->D > PA_MAX_D || s->S > PA_MAX_S) return PA_ERR_UNSUPPORTED;
   if (s->C > (1 << 16) || s->H > 1024) return PA_ERR_UNSUPPORTED;
-  if (s->N > (int64_t)1 << 31 || s->B > (1 << 20)) return PA_ERR_UNSUPPORTED;
+  if (s->N > PA_MAX_N || s->B > (1 << 20)) return PA_ERR_UNSUPPORTED;  // kernels hold N in an int
   if (s->B * s->H > 65535) return PA_ERR_UNSUPPORTED;  // grid.y of the reduction
   if (s->conv_k > 0) {
     if (s->grid_h <= 0 || s->grid_w <= 0 || s->grid_d < 0) return PA_ERR_DIMS;
@@ -475,7 +475,7 @@ int pa_rows_gemm_act(int dtype, const pa_shape *grid, int64_t c_in, int64_t c_ou
   if (act != 0 && act != 1) return PA_ERR_UNSUPPORTED;
   if (dtype != PA_F32 && dtype != PA_BF16) return PA_ERR_UNSUPPORTED;
   if (grid->B <= 0 || grid->N <= 0 || c_in <= 0 || c_out <= 0 || grid->conv_k < 0) return PA_ERR_DIMS;
-  if (c_in > (1 << 16) || c_out > (1 << 16) || grid->N > (int64_t)1 << 31) return PA_ERR_UNSUPPORTED;
+  if (c_in > (1 << 16) || c_out > (1 << 16) || grid->N > PA_MAX_N) return PA_ERR_UNSUPPORTED;
   if (grid->conv_k > 0) {
     if (grid->grid_h <= 0 || grid->grid_w <= 0 || grid->grid_d < 0) return PA_ERR_DIMS;
     if (grid->grid_h * grid->grid_w * (grid->grid_d > 0 ? grid->grid_d : 1) != grid->N) return PA_ERR_DIMS;

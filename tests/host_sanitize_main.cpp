@@ -38,7 +38,7 @@ int main() {
 
   // ---- queries and workspace sizes over a grid of shapes, extremes included ----
   const int64_t Bs[] = {-1, 0, 1, 2, 7, 1 << 20, (int64_t)1 << 40};
-  const int64_t Ns[] = {-5, 0, 1, 31, 32, 33, 700, 4096, 28900, 1 << 20, (int64_t)1 << 31, ((int64_t)1 << 31) + 1,
+  const int64_t Ns[] = {-5, 0, 1, 31, 32, 33, 700, 4096, 28900, 1 << 20, PA_MAX_N, (int64_t)1 << 31, ((int64_t)1 << 31) + 1,
                         (int64_t)1 << 62};
   const int64_t Cs[] = {0, 1, 64, 128, 256, 512, 1 << 16, (1 << 16) + 1};
   const int64_t Hs[] = {0, 1, 4, 8, 16, 1024, 1025};
@@ -58,6 +58,7 @@ int main() {
                 CHECK(path <= 2);
                 CHECK((path < 0) == (ws < 0));  // a shape is either served with a size or refused by both
                 if (path >= 0) CHECK(ws >= 0);
+                if (N > PA_MAX_N) CHECK(path < 0);
                 const int64_t pc = pa_reduce_partial_count(&s);
                 CHECK(pc != 0);
                 (void)pa_backward_query(dtype, &s);
