@@ -44,11 +44,12 @@ def test_block_mlp_rows_beyond_2_32_elements():
     assert torch.isfinite(y0.float()).all()
 
 
-@pytest.mark.parametrize("S", [64, 128])
-def test_layer_points_beyond_2_32_elements(S):
-    # S = 64: the fused kernels of the headline path; S = 128: the packed-tile sequence with recomputed slice weights
-    announce("large layer", S, COPIES * N0)
-    C, H = 256, 8
+@pytest.mark.parametrize("C,S,COPIES", [(256, 64, 17), (256, 128, 17), (512, 128, 9)])
+def test_layer_points_beyond_2_32_elements(C, S, COPIES):
+    # C = 256, S = 64: the fused kernels of the headline path; S = 128: the packed-tile sequence with recomputed slice
+    # weights; C = 512: the staged kernels of the 512-wide layers
+    announce("large layer", C, S, COPIES * N0)
+    H = C // 32
     dev = torch.device("cuda:0")
     torch.manual_seed(3)
     layer = pn.PhysicsAttentionIrregularMesh(C, heads=H, dim_head=32, slice_num=S, use_te=False).eval().to(dev)
