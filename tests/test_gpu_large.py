@@ -90,3 +90,29 @@ def test_general_fp32_layer_beyond_2_32_elements():
     assert_rel_l2(tok, tok0, f"fp32: slice tokens of {copies} copies vs one copy", tol=1e-5)
     for k in (0, copies // 2, copies - 1):
         assert_rel_l2(y[:, k * n0:(k + 1) * n0], y0, f"fp32: outputs of copy {k}", tol=1e-5)
+
+
+@pytest.mark.parametrize("dtype,C,H,D,S,grid,B", [
+    (torch.bfloat16, 256, 8, 32, 64, (512, 513), 70),   # staged MFMA kernels behind the implicit-GEMM projections
+    (torch.float32, 128, 8, 16, 32, (256, 257), 515),   # fused float32 front end and row kernels
+])
+def test_structured2d_batches_beyond_2_32_elements(dtype, C, H, D, S, grid, B):
+    # batch elements are independent: a batch of B copies of one grid gives B copies of its output
+    n = grid[0] * grid[1]
+    announce("large structured2d", dtype, C, grid, B)
+    assert B * n * C > 1 << 32
+    dev = torch.device("cuda:0")
+    torch.manual_seed(9)
+    layer = pn.PhysicsAttentionStructuredMesh2D(C, grid, heads=H, dim_head=D, slice_num=S, kernel=3,
+                                                use_te=False).eval().to(dev)
+    g = torch.Generator().manual_seed(17)
+    x0 = torch.randn(1, n, C, generator=g).to(dtype).to(dev)
+    with torch.no_grad():
+        y0 = layer(x0)
+        x = x0.repeat(B, 1, 1)
+        y = layer(x)
+    del x
+    assert y.shape == (B, n, C) and torch.isfinite(y.float()).all()
+    tol = 2e-3 if dtype == torch.bfloat16 else 1e-5
+    for b in (0, 1, B // 2, B - 1):
+        assert_rel_l2(y[b:b + 1], y0, f"{dtype}: batch element {b} of {B}", tol=tol)
