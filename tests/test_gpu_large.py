@@ -116,3 +116,34 @@ def test_structured2d_batches_beyond_2_32_elements(dtype, C, H, D, S, grid, B):
     tol = 2e-3 if dtype == torch.bfloat16 else 1e-5
     for b in (0, 1, B // 2, B - 1):
         assert_rel_l2(y[b:b + 1], y0, f"{dtype}: batch element {b} of {B}", tol=tol)
+
+
+def test_layer_training_step_beyond_2_32_elements():
+    # forward + backward of the bf16 layer on 17 copies of a point set, probed with 17 copies of one cotangent: the slice
+    # tokens are those of one copy, so every parameter gradient is 17 times that of one copy and every copy of a point
+    # gets the input gradient of the original
+    announce("large training step", COPIES * N0)
+    C, H, S = 256, 8, 64
+    dev = torch.device("cuda:0")
+    torch.manual_seed(21)
+    layer = pn.PhysicsAttentionIrregularMesh(C, heads=H, dim_head=32, slice_num=S, use_te=False).to(dev)
+    g = torch.Generator().manual_seed(23)
+    x0 = torch.randn(1, N0, C, generator=g).bfloat16().to(dev)
+    probe0 = torch.randn(1, N0, C, generator=g).bfloat16().to(dev)
+
+    def step(x, probe):
+        layer.zero_grad(set_to_none=True)
+        xc = x.clone().requires_grad_(True)
+        y = layer(xc)
+        assert y.dtype == torch.bfloat16
+        (y.float() * probe.float()).sum().backward()
+        return xc.grad, {name: p.grad.clone() for name, p in layer.named_parameters()}
+
+    dx0, grads0 = step(x0, probe0)
+    dx, grads = step(x0.repeat(1, COPIES, 1), probe0.repeat(1, COPIES, 1))
+    assert dx.numel() > 1 << 32
+    for name, g0 in grads0.items():
+        assert torch.isfinite(grads[name]).all(), name
+        assert_rel_l2(grads[name], COPIES * g0, f"grad {name}: {COPIES} copies vs {COPIES} x one copy", tol=1e-2)
+    for k in (0, COPIES // 2, COPIES - 1):
+        assert_rel_l2(dx[:, k * N0:(k + 1) * N0], dx0, f"input gradient of copy {k}", tol=1e-2)
