@@ -195,6 +195,10 @@ class PhysicsAttentionBase(nn.Module):
             with torch.autocast("cuda", enabled=False):
                 return self.forward(x.float()).to(torch.float16)
         self._validate(x)
+        if x.numel() == 0:
+            # no points (or an empty batch): the reference's tensor ops return the empty (B, N, C) result
+            self._check_spatial(x)
+            return self._prepare_input(x).clone()
         needs_grad = self._needs_grad(x)
         x = self._prepare_input(x)
         if needs_grad:
@@ -239,6 +243,9 @@ class PhysicsAttentionBase(nn.Module):
             with torch.autocast("cuda", enabled=False):  # float32 inside, as the residual stream of the caller is
                 return self.forward_block(x.float(), residual.float(), ln)
         self._validate(x)
+        if x.numel() == 0:
+            y = self.forward(x)
+            return y + residual.to(y.dtype), y.clone()
         if self.plus and not self._needs_grad(x) and not self.fp8_weights and not (self.training and self.out_dropout.p > 0):
             xp = self._prepare_input(x)
             dims = self.layer_dims(xp)

@@ -123,3 +123,25 @@ def test_bf16_structured_plus_layer_on_the_staged_mfma_kernels():
         want = ref.forward_with_noise(x, u.float())
         got = hip.forward_with_noise(xb, u.cuda())
     assert_rel_l2(got, want, "bf16 structured plus y vs fp32 oracle", tol=2e-2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_empty_inputs_give_empty_outputs(dtype):
+    """No points, or an empty batch: the reference's tensor ops return the empty (B, N, C) tensor; so do the modules
+    (nothing is launched)."""
+    announce("empty inputs", dtype)
+    layer = pn.PhysicsAttentionIrregularMesh(128, heads=4, dim_head=32, slice_num=16, use_te=False).eval().cuda()
+    grid = pn.PhysicsAttentionStructuredMesh2D(128, (6, 5), heads=4, dim_head=32, slice_num=16, kernel=3,
+                                               use_te=False).eval().cuda()
+    ln = torch.nn.LayerNorm(128).cuda()
+    with torch.no_grad():
+        for shape in ((2, 0, 128), (0, 7, 128)):
+            x = torch.empty(shape, dtype=dtype, device="cuda")
+            y = layer(x)
+            assert y.shape == shape and y.dtype == dtype
+            fx, normed = layer.forward_block(x, torch.empty(shape, dtype=dtype, device="cuda"), ln)
+            assert fx.shape == shape and normed.shape == shape
+        y = grid(torch.empty((0, 30, 128), dtype=dtype, device="cuda"))
+        assert y.shape == (0, 30, 128)
+        with pytest.raises(RuntimeError):  # a token count that is not the grid's: the reference's view() fails too
+            grid(torch.empty((2, 0, 128), dtype=dtype, device="cuda"))
