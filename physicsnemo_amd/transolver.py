@@ -404,6 +404,9 @@ class Transolver(nn.Module):
             if embedding is not None and embedding.ndim != 3:
                 embedding = embedding.reshape(embedding.shape[0], -1, embedding.shape[-1])
         fx = torch.cat((embedding.to(fx.dtype), fx), -1)  # embedding first, then the functional input (:716)
+        if fx.numel() == 0 and self.structured_shape is None:
+            # no points or an empty batch: the reference's tensor ops return the empty (B, N, out_dim) result
+            return fx.new_zeros(fx.shape[:-1] + (self.blocks[-1].ln_mlp2[1].out_features,))
         on_library = self._glue_on_library(fx)
         normed = None
         first_ln_done = False

@@ -145,3 +145,9 @@ def test_empty_inputs_give_empty_outputs(dtype):
         assert y.shape == (0, 30, 128)
         with pytest.raises(RuntimeError):  # a token count that is not the grid's: the reference's view() fails too
             grid(torch.empty((2, 0, 128), dtype=dtype, device="cuda"))
+        model = pn.Transolver(functional_dim=2, out_dim=3, embedding_dim=2, n_layers=2, n_hidden=64, n_head=2,
+                              slice_num=8, use_te=False).eval().cuda().to(dtype)
+        for shape in ((2, 0), (0, 9)):
+            out = model(torch.empty(shape + (2,), dtype=dtype, device="cuda"),
+                        torch.empty(shape + (2,), dtype=dtype, device="cuda"))
+            assert out.shape == shape + (3,)
