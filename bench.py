@@ -24,6 +24,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
+TOP_CLOCK_GHZ = 2.4  # the clock the published peaks are quoted at
 HBM_PEAK_GBS = 8000.0       # MI355X HBM3E, published
 MFMA_BF16_PEAK_TF = 2500.0  # MI355X dense bf16, published
 
@@ -595,6 +596,17 @@ def measure_layer(B, N, C, S, steps, warmup, kernel_reps, x_cpu=None, cold=False
             roofline = {"kernel": dominant, "bound": "hbm", "achieved": kernels[dominant]["hbm_gbs"], "peak": HBM_PEAK_GBS,
                         "unit": "GB/s", "frac": kernels[dominant]["hbm_frac"],
                         "traffic": measured_traffic(dominant, B, N, C, S)}
+            if dominant == "project_softmax_reduce" and C == 256:
+                # the shader clock the chip holds under this kernel, read inside the kernel's clock-reporting twin
+                # (shader cycles against the 100 MHz wall clock over one workgroup's run) after the same run-in
+                run_in(lambda: st.project_softmax_reduce(x))
+                ghz = []
+                for _ in range(5):
+                    for _ in range(kernel_reps):  # the clocked launch queues behind these: no idle gap before it
+                        st.project_softmax_reduce(x)
+                    ghz.append(st.project_softmax_reduce_clocked(x)[0])
+                roofline["shader_clock_ghz"] = round(sorted(ghz)[2], 3)
+                roofline["top_clock_ghz"] = TOP_CLOCK_GHZ
         del st, yk
     res.update({"kernels": kernels, "roofline": roofline, "H": H})
     del layer, x

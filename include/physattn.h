@@ -380,6 +380,14 @@ int pa_mfma_slice_reduce(const pa_shape *shape, const void *w_pack, const void *
  * pa_layer_forward runs when it applies; PA_ERR_UNSUPPORTED otherwise. */
 int pa_mfma_project_softmax_reduce(const pa_shape *shape, const void *blob, const void *x, void *w_pack,
                                    float *partials, void *stream);
+/* pa_mfma_project_softmax_reduce with a clock reading: the same kernel (bit-identical w_pack and partials) whose
+ * workgroup in the middle of the grid also stores how long it ran -- clock_out[0] in shader cycles, clock_out[1] in
+ * ticks of the 100 MHz wall clock (device memory, 16 bytes, 16-byte aligned).  cycles / (10 * ticks) GHz is the shader
+ * clock the chip held under this kernel, which is what its roofline fractions should be read against (the published
+ * peaks assume the top clock).  Served for C = 256, S <= 64; PA_ERR_UNSUPPORTED otherwise.  No reference counterpart
+ * (a measurement aid for bench.py). */
+int pa_mfma_project_softmax_reduce_clocked(const pa_shape *shape, const void *blob, const void *x, void *w_pack,
+                                           float *partials, uint64_t *clock_out, void *stream);
 /* Number of partial sums a first pass leaves in `partials`: fused = 1 for pa_mfma_project_softmax_reduce (or
  * PA_ERR_UNSUPPORTED where it does not apply), 0 for pa_mfma_slice_reduce. Pass it to pa_mfma_combine_attention. */
 int64_t pa_mfma_partial_groups(const pa_shape *shape, int fused);

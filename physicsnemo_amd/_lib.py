@@ -36,6 +36,7 @@ EXPORTED = [
     "pa_static_scratch_bytes", "pa_slice_reduce_static",
     "pa_preprocess_query", "pa_preprocess_workspace_bytes", "pa_preprocess_forward",
     "pa_block_query", "pa_block_workspace_bytes", "pa_block_forward", "pa_markers_enabled",
+    "pa_mfma_project_softmax_reduce_clocked",
 ]
 
 PA_BUF_BLOB, PA_BUF_FX_PACK, PA_BUF_W_PACK, PA_BUF_PARTIALS, PA_BUF_TOKP = range(5)
@@ -136,6 +137,8 @@ def load() -> ctypes.CDLL:
     lib.pa_mfma_combine_attention.argtypes = [ps, pp, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]
     lib.pa_mfma_project_softmax_reduce.restype = c_int
     lib.pa_mfma_project_softmax_reduce.argtypes = [ps, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]
+    lib.pa_mfma_project_softmax_reduce_clocked.restype = c_int
+    lib.pa_mfma_project_softmax_reduce_clocked.argtypes = [ps, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]
     lib.pa_mfma_partial_groups.restype = c_int64
     lib.pa_mfma_partial_groups.argtypes = [ps, c_int]
     lib.pa_mfma_deslice_project.restype = c_int

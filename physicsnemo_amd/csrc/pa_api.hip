@@ -865,6 +865,18 @@ int pa_mfma_project_softmax_reduce(const pa_shape *shape, const void *blob, cons
                                    static_cast<hipStream_t>(stream));
 }
 
+int pa_mfma_project_softmax_reduce_clocked(const pa_shape *shape, const void *blob, const void *x, void *w_pack,
+                                           float *partials, uint64_t *clock_out, void *stream) {
+  int rc = check_mfma(shape);
+  if (rc) return rc;
+  if (!pa::mfma::fuse_reduce(*shape) || shape->C != 256) return PA_ERR_UNSUPPORTED;
+  if (!blob || !x || !w_pack || !partials || !clock_out) return PA_ERR_NULL;
+  if (!aligned16(blob) || !aligned16(x) || !aligned16(w_pack) || !aligned16(partials) || !aligned16(clock_out))
+    return PA_ERR_ALIGN;
+  return pa::mfma::project_softmax_clocked(*shape, blob, x, w_pack, partials, clock_out, compute_units(),
+                                           static_cast<hipStream_t>(stream));
+}
+
 int pa_mfma_slice_reduce(const pa_shape *shape, const void *w_pack, const void *fx_pack, float *partials, void *stream) {
   int rc = check_mfma(shape);
   if (rc) return rc;

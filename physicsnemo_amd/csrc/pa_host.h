@@ -229,6 +229,10 @@ int64_t project_groups(const pa_shape &s, int num_cu, bool fused);
 bool fuse_reduce(const pa_shape &s);
 int project_softmax(const pa_shape &s, const void *blob, const void *x, void *fx_pack, void *w_pack, float *partials,
                     int num_cu, hipStream_t st);
+// the fused form with the shader clock of one of its workgroups reported (C = 256, S <= 64): clock_out[0] = shader
+// cycles, clock_out[1] = ticks of the 100 MHz wall clock
+int project_softmax_clocked(const pa_shape &s, const void *blob, const void *x, void *w_pack, float *partials,
+                            uint64_t *clock_out, int num_cu, hipStream_t st);
 int slice_reduce(const pa_shape &s, const void *w_pack, const void *fx_pack, float *partials, hipStream_t st);
 int combine_attention(const pa_shape &s, const pa_params &p, const float *fx_bias, const float *partials, int64_t G,
                       float *slice_token, float *slice_norm, float *out_token, void *tokp, hipStream_t st);

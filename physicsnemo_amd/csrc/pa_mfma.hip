@@ -158,12 +158,14 @@ __device__ __forceinline__ void load_row_chunk_to_lds(const void *sbase, unsigne
       : "memory");
 }
 
-template <int C, int S, bool FUSED>
-__global__ __launch_bounds__((C / 32) * 64) void project_softmax_kernel(const u32x4 *__restrict__ blob,
-                                                                        const uint16_t *__restrict__ x,
-                                                                        u32x4 *__restrict__ fx_pack,
-                                                                        u32x4 *__restrict__ w_pack,
-                                                                        float *__restrict__ partials, int64_t N, int tpb) {
+// CLOCKED: the workgroup in the middle of the grid also reports how long it ran, in shader cycles (s_memtime) and in
+// ticks of the 100 MHz wall clock: clock_out[0], clock_out[1].  Their ratio is the shader clock the chip held under
+// this very kernel; everything else is the same code (two scalar reads at the start, one store at the end).
+template <int C, int S, bool FUSED, bool CLOCKED>
+__device__ __forceinline__ void project_softmax_body(const u32x4 *__restrict__ blob, const uint16_t *__restrict__ x,
+                                                     u32x4 *__restrict__ fx_pack, u32x4 *__restrict__ w_pack,
+                                                     float *__restrict__ partials, int64_t N, int tpb,
+                                                     uint64_t *__restrict__ clock_out) {
   constexpr int H = C / 32, KS = C / 16, ST = (S + 31) / 32, NCH = S / 16, D1 = 33;
   constexpr int WAVES = H, NT = WAVES * 64;
   constexpr int TS = 4;                 // tiles per set
@@ -185,6 +187,11 @@ __global__ __launch_bounds__((C / 32) * 64) void project_softmax_kernel(const u3
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: addresses derived from it stay scalar
   const int h = wave;
   const int b = blockIdx.y;
+  uint64_t cycles0 = 0, ticks0 = 0;
+  if constexpr (CLOCKED) {
+    cycles0 = __builtin_readcyclecounter();
+    ticks0 = wall_clock64();
+  }
   const float *bias_s = fvec + bp.f_bias_logit + h * (ST * 32), *tscale = fvec + bp.f_tscale;
 
   u32x4 wx[KS], wf[KS];
@@ -448,6 +455,12 @@ __global__ __launch_bounds__((C / 32) * 64) void project_softmax_kernel(const u3
     aggregate(ag);
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // nothing may still be landing in LDS when the workgroup ends
+  if constexpr (CLOCKED) {
+    if (blockIdx.x == gridDim.x / 2 && blockIdx.y == 0 && tid == 0) {
+      clock_out[0] = __builtin_readcyclecounter() - cycles0;
+      clock_out[1] = wall_clock64() - ticks0;
+    }
+  }
   if constexpr (FUSED) {
     // this wave's head: accumulators -> partials[g][b][h][s][d], [..][D] = count
     float *dst = partials + (((int64_t)blockIdx.x * gridDim.y + b) * H + h) * (S * D1);
@@ -462,6 +475,25 @@ __global__ __launch_bounds__((C / 32) * 64) void project_softmax_kernel(const u3
       }
     }
   }
+}
+
+template <int C, int S, bool FUSED>
+__global__ __launch_bounds__((C / 32) * 64) void project_softmax_kernel(const u32x4 *__restrict__ blob,
+                                                                        const uint16_t *__restrict__ x,
+                                                                        u32x4 *__restrict__ fx_pack,
+                                                                        u32x4 *__restrict__ w_pack,
+                                                                        float *__restrict__ partials, int64_t N, int tpb) {
+  project_softmax_body<C, S, FUSED, false>(blob, x, fx_pack, w_pack, partials, N, tpb, nullptr);
+}
+
+// the fused form with the clock reading
+template <int C, int S>
+__global__ __launch_bounds__((C / 32) * 64) void project_softmax_clocked_kernel(const u32x4 *__restrict__ blob,
+                                                                                const uint16_t *__restrict__ x,
+                                                                                u32x4 *__restrict__ w_pack,
+                                                                                float *__restrict__ partials, int64_t N,
+                                                                                int tpb, uint64_t *__restrict__ clock_out) {
+  project_softmax_body<C, S, true, true>(blob, x, nullptr, w_pack, partials, N, tpb, clock_out);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -930,28 +962,42 @@ int64_t project_groups(const pa_shape &s, int num_cu, bool fused) {
 
 bool fuse_reduce(const pa_shape &s) { return s.S <= 64; }  // the LDS accumulators of the fused form fit up to S = 64
 
-template <int C, int S, bool FUSED>
+template <int C, int S, bool FUSED, bool CLOCKED = false>
 static int project_softmax_f(const pa_shape &s, const void *blob, const void *x, void *fx_pack, void *w_pack,
-                             float *partials, int num_cu, hipStream_t st) {
+                             float *partials, uint64_t *clock_out, int num_cu, hipStream_t st) {
   constexpr int ST = (S + 31) / 32, H = C / 32, TS = 4, UPR = C / 8, WAVES = H, NCK = 32 / (64 / UPR);
   const size_t lds = (size_t)(2 * TS * NCK * 65 + ST * 2 * 64 + 4 * 64) * 16 + (size_t)blob_plan(C, S).nfloat * 4;
-  int rc = allow_dynamic_lds(project_softmax_kernel<C, S, FUSED>, lds);
-  if (rc) return rc;
   const int64_t tpb = tiles_per_batch(s);
   const int64_t G = project_groups(s, num_cu, FUSED);
-  hipLaunchKernelGGL((project_softmax_kernel<C, S, FUSED>), dim3((unsigned)G, (unsigned)s.B), dim3(WAVES * 64), lds, st,
-                     static_cast<const u32x4 *>(blob), static_cast<const uint16_t *>(x), static_cast<u32x4 *>(fx_pack),
-                     static_cast<u32x4 *>(w_pack), partials, s.N, (int)tpb);
+  if constexpr (CLOCKED) {
+    int rc = allow_dynamic_lds(project_softmax_clocked_kernel<C, S>, lds);
+    if (rc) return rc;
+    hipLaunchKernelGGL((project_softmax_clocked_kernel<C, S>), dim3((unsigned)G, (unsigned)s.B), dim3(WAVES * 64), lds, st,
+                       static_cast<const u32x4 *>(blob), static_cast<const uint16_t *>(x), static_cast<u32x4 *>(w_pack),
+                       partials, s.N, (int)tpb, clock_out);
+  } else {
+    int rc = allow_dynamic_lds(project_softmax_kernel<C, S, FUSED>, lds);
+    if (rc) return rc;
+    hipLaunchKernelGGL((project_softmax_kernel<C, S, FUSED>), dim3((unsigned)G, (unsigned)s.B), dim3(WAVES * 64), lds, st,
+                       static_cast<const u32x4 *>(blob), static_cast<const uint16_t *>(x), static_cast<u32x4 *>(fx_pack),
+                       static_cast<u32x4 *>(w_pack), partials, s.N, (int)tpb);
+  }
   return launch_status();
 }
 
 template <int C, int S>
 static int project_softmax_cs(const pa_shape &s, const void *blob, const void *x, void *fx_pack, void *w_pack,
-                              float *partials, int num_cu, hipStream_t st) {
+                              float *partials, uint64_t *clock_out, int num_cu, hipStream_t st) {
   if constexpr (S <= 64) {
-    if (partials) return project_softmax_f<C, S, true>(s, blob, x, fx_pack, w_pack, partials, num_cu, st);
+    if constexpr (C == 256) {  // the clocked twin exists for the width of the benchmark workload
+      if (partials && clock_out)
+        return project_softmax_f<C, S, true, true>(s, blob, x, fx_pack, w_pack, partials, clock_out, num_cu, st);
+    }
+    if (clock_out) return PA_ERR_UNSUPPORTED;
+    if (partials) return project_softmax_f<C, S, true>(s, blob, x, fx_pack, w_pack, partials, nullptr, num_cu, st);
   }
-  return project_softmax_f<C, S, false>(s, blob, x, fx_pack, w_pack, nullptr, num_cu, st);
+  if (clock_out) return PA_ERR_UNSUPPORTED;
+  return project_softmax_f<C, S, false>(s, blob, x, fx_pack, w_pack, nullptr, nullptr, num_cu, st);
 }
 
 template <int S>
@@ -1032,7 +1078,12 @@ static int deslice_project_cs(const pa_shape &s, const void *blob, const void *w
 // partials != nullptr (and S <= 64): fused with the first reduction pass; fx_pack is then not written
 int project_softmax(const pa_shape &s, const void *blob, const void *x, void *fx_pack, void *w_pack, float *partials,
                     int num_cu, hipStream_t st) {
-  PA_DISPATCH_CS(project_softmax_cs, s, blob, x, fx_pack, w_pack, partials, num_cu, st);
+  PA_DISPATCH_CS(project_softmax_cs, s, blob, x, fx_pack, w_pack, partials, nullptr, num_cu, st);
+}
+
+int project_softmax_clocked(const pa_shape &s, const void *blob, const void *x, void *w_pack, float *partials,
+                            uint64_t *clock_out, int num_cu, hipStream_t st) {
+  PA_DISPATCH_CS(project_softmax_cs, s, blob, x, nullptr, w_pack, partials, clock_out, num_cu, st);
 }
 
 int slice_reduce(const pa_shape &s, const void *w_pack, const void *fx_pack, float *partials, hipStream_t st) {

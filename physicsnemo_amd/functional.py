@@ -454,6 +454,19 @@ class MfmaStages:
                                                            self._stream()), "pa_mfma_project_softmax_reduce")
         self._producer_groups = self.fused_groups
 
+    def project_softmax_reduce_clocked(self, x):
+        """`project_softmax_reduce` with the shader clock one of its workgroups ran at: returns (GHz, cycles, ns).
+        Hidden width 256, slice_num <= 64."""
+        _need_cuda(x)
+        clock = torch.zeros(2, dtype=torch.int64, device=self.device)
+        _lib.check(self.lib.pa_mfma_project_softmax_reduce_clocked(byref(self.shape), self.blob.data_ptr(), x.data_ptr(),
+                                                                   self.w_pack.data_ptr(), self.partials.data_ptr(),
+                                                                   clock.data_ptr(), self._stream()),
+                   "pa_mfma_project_softmax_reduce_clocked")
+        self._producer_groups = self.fused_groups
+        cycles, ticks = (int(v) for v in clock.tolist())
+        return cycles / (10.0 * ticks), cycles, 10 * ticks
+
     def combine_attention(self):
         _lib.check(self.lib.pa_mfma_combine_attention(byref(self.shape), byref(self.cparams), self.partials.data_ptr(),
                                                       self._producer_groups, self.tok.data_ptr(), self.norm.data_ptr(), self.tok_out.data_ptr(),

@@ -253,3 +253,31 @@ def test_fp8_e4m3_weight_variant(B, N, C, S, bound):
     assert err <= (q_err ** 2 + 4e-3 ** 2) ** 0.5, (err, q_err)
     assert_rel_l2(y8, want_q, "fp8-weight layer vs fp32 oracle with the dequantised weights")
     assert torch.equal(y8, y16)
+
+
+@pytest.mark.parametrize("S", [16, 64])
+def test_clocked_twin_of_the_fused_kernel(S):
+    """The fused kernel's clock-reporting twin writes the same w_pack and partial sums, and a plausible shader clock."""
+    announce("clocked twin", S)
+    torch.manual_seed(S)
+    hip = pn.PhysicsAttentionIrregularMesh(256, heads=8, dim_head=32, slice_num=S, use_te=False).eval().cuda()
+    xb = torch.randn(2, 40000 + 5, 256).bfloat16().cuda()
+    st = PF.MfmaStages(hip.kernel_params(torch.bfloat16, xb.device), hip.layer_dims(xb), xb.device)
+    st.pack_params()
+    st.project_softmax_reduce(xb)
+    torch.cuda.synchronize()
+    w_ref, p_ref = st.w_pack.clone(), st.partials.clone()
+    st.w_pack.zero_()
+    st.partials.zero_()
+    ghz, cycles, ns = st.project_softmax_reduce_clocked(xb)
+    groups = st.fused_groups * 2 * 8 * S * 33 * 4  # bytes of the partial sums the kernel writes (the rest is spare)
+    assert torch.equal(st.w_pack, w_ref)
+    assert torch.equal(st.partials[:groups], p_ref[:groups])
+    assert cycles > 0 and ns > 0 and 0.3 < ghz < 2.6, (ghz, cycles, ns)
+    # other widths have no twin
+    small = pn.PhysicsAttentionIrregularMesh(128, heads=4, dim_head=32, slice_num=S, use_te=False).eval().cuda()
+    xs = torch.randn(1, 4096, 128).bfloat16().cuda()
+    st2 = PF.MfmaStages(small.kernel_params(torch.bfloat16, xs.device), small.layer_dims(xs), xs.device)
+    st2.pack_params()
+    with pytest.raises(RuntimeError):
+        st2.project_softmax_reduce_clocked(xs)
