@@ -56,6 +56,18 @@ __device__ __forceinline__ float gelu_erf_grad(float v) {
   return 0.5f * (1.f + erff(v * 0.70710678118654752f)) + v * 0.3989422804014327f * expf(-0.5f * v * v);
 }
 
+// Accesses to tensors that a kernel streams through once (activations in, activations out, the packed slice
+// weights): the non-temporal hint keeps them from displacing what the L2 is for -- weights, tables, partial sums --
+// and measured 9 % off kernel (d) and 5 % off the layer.  Any trivially copyable vector type.
+template <class T>
+__device__ __forceinline__ T load_streaming(const T *p) {
+  return __builtin_nontemporal_load(p);
+}
+template <class T>
+__device__ __forceinline__ void store_streaming(T *p, T v) {
+  __builtin_nontemporal_store(v, p);
+}
+
 __device__ __forceinline__ float clamp_temperature(float t) { return fminf(fmaxf(t, kTempMin), kTempMax); }
 
 // wave64 butterfly reductions

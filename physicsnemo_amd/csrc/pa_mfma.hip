@@ -352,7 +352,7 @@ __device__ __forceinline__ void project_softmax_body(const u32x4 *__restrict__ b
     }
     u32x4 *wdst = w_pack + ((tl.tile * H + h) * NCH) * 64 + lane;
 #pragma unroll
-    for (int cq = 0; cq < NCH; ++cq) wdst[cq * 64] = wp[cq];
+    for (int cq = 0; cq < NCH; ++cq) store_streaming(wdst + cq * 64, wp[cq]);
     if constexpr (FUSED) {
       // transposed weights (lanes <-> slices, registers <-> points); a slot past the batch's last tile multiplies by
       // the all-zero selection matrices instead and so adds nothing
@@ -765,13 +765,13 @@ __global__ __launch_bounds__(C * 2) void deslice_project_kernel(const u32x4 *__r
   {
     const u32x4 *wsrc = w_pack + (((b * tpb + t) * H + wave) * NCH) * 64 + lane;
 #pragma unroll
-    for (int cq = 0; cq < NCH; ++cq) wcur[cq] = wsrc[cq * 64];
+    for (int cq = 0; cq < NCH; ++cq) wcur[cq] = load_streaming(wsrc + cq * 64);
     if constexpr (HAS_RES) {
 #pragma unroll
       for (int rr = 0; rr < ROWS; ++rr) {
         int64_t n = t * 32 + wave * ROWS + rr;
         if (MASKED && n >= N) n = N - 1;
-        rcur[rr] = *reinterpret_cast<const rowvec *>(residual + (b * N + n) * C + lane * CPL);
+        rcur[rr] = load_streaming(reinterpret_cast<const rowvec *>(residual + (b * N + n) * C + lane * CPL));
       }
     }
   }
@@ -824,11 +824,11 @@ __global__ __launch_bounds__(C * 2) void deslice_project_kernel(const u32x4 *__r
     {
       const u32x4 *wsrc = w_pack + (((bn * tpb + tn) * H + wave) * NCH) * 64 + lane;
 #pragma unroll
-      for (int cq = 0; cq < NCH; ++cq) wnext[cq] = wsrc[cq * 64];
+      for (int cq = 0; cq < NCH; ++cq) wnext[cq] = load_streaming(wsrc + cq * 64);
       if constexpr (HAS_RES && !MASKED) {
 #pragma unroll
         for (int rr = 0; rr < ROWS; ++rr)
-          rnext[rr] = *reinterpret_cast<const rowvec *>(residual + (bn * N + tn * 32 + wave * ROWS + rr) * C + lane * CPL);
+          rnext[rr] = load_streaming(reinterpret_cast<const rowvec *>(residual + (bn * N + tn * 32 + wave * ROWS + rr) * C + lane * CPL));
       }
     }
     oxs[(wave * 2 + 0) * 64 + lane] = pack_half<0>(ox);
@@ -882,7 +882,7 @@ __global__ __launch_bounds__(C * 2) void deslice_project_kernel(const u32x4 *__r
         v[k + 1] = bf16_bits_to_f32(o1);
         ob[k / 2] = (uint32_t)o0 | ((uint32_t)o1 << 16);
       }
-      if (ok) *reinterpret_cast<rowvec *>(y + off) = ob;
+      if (ok) store_streaming(reinterpret_cast<rowvec *>(y + off), ob);
       if constexpr (HAS_LN) {
         float s1 = 0.f;
 #pragma unroll
@@ -902,7 +902,7 @@ __global__ __launch_bounds__(C * 2) void deslice_project_kernel(const u32x4 *__r
           const uint16_t l1 = to_bf16_bits((v[k + 1] - mean) * rstd * gam[k + 1] + bet[k + 1]);
           lb[k / 2] = (uint32_t)l0 | ((uint32_t)l1 << 16);
         }
-        if (ok) *reinterpret_cast<rowvec *>(ln_out + off) = lb;
+        if (ok) store_streaming(reinterpret_cast<rowvec *>(ln_out + off), lb);
       }
     }
     if (!more) break;

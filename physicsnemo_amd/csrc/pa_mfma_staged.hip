@@ -321,15 +321,15 @@ __global__ __launch_bounds__(512) void slice_softmax_reduce_kernel(const uint16_
     u32x4 xm0, xm1;
     if constexpr (PACKED_X) {
       const u32x4 *xsrc = reinterpret_cast<const u32x4 *>(x_mid) + ((((int64_t)b * tpb + t) * H + h) * 2) * 64 + lane;
-      xm0 = xsrc[0];
-      xm1 = xsrc[64];
+      xm0 = load_streaming(xsrc);
+      xm1 = load_streaming(xsrc + 64);
     } else {
       const uint16_t *row = x_mid + ((int64_t)b * N + (valid ? n : N - 1)) * HD + h * 32 + 8 * g;
       xm0 = *reinterpret_cast<const u32x4 *>(row);
       xm1 = *reinterpret_cast<const u32x4 *>(row + 16);
     }
     const u32x4 *fsrc = fx_pack + ((((int64_t)b * tpb + t) * H + h) * 2) * 64 + lane;
-    const u32x4 f0 = fsrc[0], f1 = fsrc[64];
+    const u32x4 f0 = load_streaming(fsrc), f1 = load_streaming(fsrc + 64);
     u32x4 chunk[NCH];
     slice_weights_of_tile<S>(wsl, bsl, xm0, xm1, sc, valid, lane, g, chunk);
 #pragma unroll
@@ -397,8 +397,8 @@ __global__ __launch_bounds__(512) void deslice_recompute_kernel(const uint16_t *
     u32x4 xm0, xm1;
     if constexpr (PACKED_X) {
       const u32x4 *xsrc = reinterpret_cast<const u32x4 *>(x_mid) + pk;
-      xm0 = xsrc[0];
-      xm1 = xsrc[64];
+      xm0 = load_streaming(xsrc);
+      xm1 = load_streaming(xsrc + 64);
     } else {
       const uint16_t *row = x_mid + m * HD + h * 32 + 8 * g;
       xm0 = *reinterpret_cast<const u32x4 *>(row);
@@ -422,8 +422,8 @@ __global__ __launch_bounds__(512) void deslice_recompute_kernel(const uint16_t *
     for (int r = 0; r < 16; ++r) ox[r] *= inv;
     if constexpr (PACKED_X) {
       u32x4 *odst = reinterpret_cast<u32x4 *>(out_x) + pk;
-      odst[0] = pack_half<0>(ox);
-      odst[64] = pack_half<1>(ox);
+      store_streaming(odst, pack_half<0>(ox));
+      store_streaming(odst + 64, pack_half<1>(ox));
     } else {
       store_tile_natural(ox, out_x + m * HD + h * 32, g, valid);
     }

@@ -379,7 +379,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
       for (int rr = 0; rr < NRS; ++rr) {
         int64_t r = row0 + 32 * p + 2 * rr + half;
         if (r >= M) r = M - 1;
-        rsd[rr] = *reinterpret_cast<const rowv *>(residual + r * C + i * CPH);
+        rsd[rr] = load_streaming(reinterpret_cast<const rowv *>(residual + r * C + i * CPH));
       }
     }
 #pragma unroll
@@ -403,7 +403,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         v[2 * w + 1] = bf16_bits_to_f32(o1);
         ob[w] = (uint32_t)o0 | ((uint32_t)o1 << 16);
       }
-      if (ok) *reinterpret_cast<rowv *>(y + r * C + i * CPH) = ob;
+      if (ok) store_streaming(reinterpret_cast<rowv *>(y + r * C + i * CPH), ob);
       if constexpr (HAS_LN) {
         float s1 = 0.f;
 #pragma unroll
@@ -423,7 +423,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
           const uint16_t l1 = to_bf16_bits((v[2 * w + 1] - mean) * rstd * gam[2 * w + 1] + bet[2 * w + 1]);
           lb[w] = (uint32_t)l0 | ((uint32_t)l1 << 16);
         }
-        if (ok) *reinterpret_cast<rowv *>(ln_out + r * C + i * CPH) = lb;
+        if (ok) store_streaming(reinterpret_cast<rowv *>(ln_out + r * C + i * CPH), lb);
       }
     }
   }
@@ -540,7 +540,7 @@ __device__ __forceinline__ void finish_rows(const f32x16 (&yacc)[C / 32], uint32
         int64_t r = row0 + rd * RPR + 2 * rr + hl;
         if (r >= M) r = M > 0 ? M - 1 : 0;  // M = 0: a wave without rows (nothing is stored)
 #pragma unroll
-        for (int v = 0; v < NV; ++v) rsd[rr][v] = *reinterpret_cast<const rowv *>(residual + r * C + 256 * v + 8 * il);
+        for (int v = 0; v < NV; ++v) rsd[rr][v] = load_streaming(reinterpret_cast<const rowv *>(residual + r * C + 256 * v + 8 * il));
       }
     };
     static_for<PF>(load_residual);
@@ -582,7 +582,7 @@ __device__ __forceinline__ void finish_rows(const f32x16 (&yacc)[C / 32], uint32
           val[8 * v + 2 * w] = __uint_as_float(ob[w] << 16);
           val[8 * v + 2 * w + 1] = __uint_as_float(ob[w] & 0xffff0000u);
         }
-        if (ok) *reinterpret_cast<rowv *>(y + r * C + 256 * v + 8 * il) = ob;
+        if (ok) store_streaming(reinterpret_cast<rowv *>(y + r * C + 256 * v + 8 * il), ob);
       }
       if constexpr (HAS_LN) {
         float s1 = 0.f;
@@ -608,7 +608,7 @@ __device__ __forceinline__ void finish_rows(const f32x16 (&yacc)[C / 32], uint32
             const float c0 = w < 2 ? ba[2 * w] : bb[2 * w - 4], c1 = w < 2 ? ba[2 * w + 1] : bb[2 * w - 3];
             lb[w] = pack2(fmaf(fmaf(val[8 * v + 2 * w], rstd, shift), g0, c0), fmaf(fmaf(val[8 * v + 2 * w + 1], rstd, shift), g1, c1));
           }
-          if (ok) *reinterpret_cast<rowv *>(ln_out + r * C + 256 * v + 8 * il) = lb;
+          if (ok) store_streaming(reinterpret_cast<rowv *>(ln_out + r * C + 256 * v + 8 * il), lb);
         }
       }
       __builtin_amdgcn_sched_barrier(0);
@@ -1026,7 +1026,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
       if (gt >= ntiles) gt = ntiles - 1;
       const u32x4 *src = reinterpret_cast<const u32x4 *>(x) + gt * (KS * 64) + lane;
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) ub[ks] = src[ks * 64];
+      for (int ks = 0; ks < KS; ++ks) ub[ks] = load_streaming(src + ks * 64);
     } else {
       int64_t r = mb * kRowsPerBlock + wave * 32 + i;
       if (r >= M) r = M - 1;
@@ -1196,8 +1196,8 @@ __global__ __launch_bounds__(512) void project_rows_kernel(
       u32x4 *dst = (second ? fx_pack : xm_pack) + ((live ? gt : ntiles - 1) * CT + ct0) * (2 * 64) + lane;
 #pragma unroll
       for (int q = 0; q < HPS; ++q) {
-        dst[(2 * q) * 64] = pack_half<0>(acc[q]);
-        dst[(2 * q + 1) * 64] = pack_half<1>(acc[q]);
+        store_streaming(dst + (2 * q) * 64, pack_half<0>(acc[q]));
+        store_streaming(dst + (2 * q + 1) * 64, pack_half<1>(acc[q]));
       }
     }
   }
