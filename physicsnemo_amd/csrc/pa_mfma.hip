@@ -308,8 +308,8 @@ __device__ __forceinline__ void project_softmax_body(const u32x4 *__restrict__ b
     tl.fx1 = pack_half<1>(af);
     if constexpr (!FUSED) {
       u32x4 *fdst = fx_pack + ((tl.tile * H + h) * 2) * 64 + lane;
-      fdst[0] = tl.fx0;
-      fdst[64] = tl.fx1;
+      store_streaming(fdst, tl.fx0);
+      store_streaming(fdst + 64, tl.fx1);
     }
     __builtin_amdgcn_sched_barrier(0);
   };
@@ -539,8 +539,8 @@ __global__ __launch_bounds__(256) void slice_reduce_kernel(const u32x4 *__restri
     const u32x4 *fsrc = fx_pack + ((gt * H + h) * 2) * 64 + lane;
     u32x4 wf[NCH];
 #pragma unroll
-    for (int cq = 0; cq < NCH; ++cq) wf[cq] = wsrc[cq * 64];
-    const u32x4 f0 = fsrc[0], f1 = fsrc[64];
+    for (int cq = 0; cq < NCH; ++cq) wf[cq] = load_streaming(wsrc + cq * 64);
+    const u32x4 f0 = load_streaming(fsrc), f1 = load_streaming(fsrc + 64);
 #pragma unroll
     for (int st = 0; st < ST; ++st) {
       f32x16 tr;

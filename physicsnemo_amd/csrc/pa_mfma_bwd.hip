@@ -40,7 +40,7 @@ __global__ __launch_bounds__(512) void deslice_natural_kernel(const u32x4 *__res
 #pragma unroll
     for (int r = 0; r < 16; ++r) ox[r] = 0.f;
 #pragma unroll
-    for (int cq = 0; cq < NCH; ++cq) ox = mma(tp[cq], wsrc[cq * 64], ox);
+    for (int cq = 0; cq < NCH; ++cq) ox = mma(tp[cq], load_streaming(wsrc + cq * 64), ox);
     const int64_t n = (int64_t)t * 32 + i;
     const bool ok = n < N;
     store_tile_natural(ox, out_x + ((int64_t)b * N + (ok ? n : 0)) * (H * 32) + h * 32, g, ok);
@@ -195,7 +195,7 @@ __global__ __launch_bounds__(S > 64 ? 256 : 512) void slice_softmax_backward_mfm
     {
       const u32x4 *wsrc = w_pack + ((((int64_t)b * tpb + t) * H + h) * NCH) * 64 + lane;
 #pragma unroll
-      for (int cq = 0; cq < NCH; ++cq) wq[cq] = wsrc[cq * 64];
+      for (int cq = 0; cq < NCH; ++cq) wq[cq] = load_streaming(wsrc + cq * 64);
     }
     // w of this lane's (point, slices): chunk cq = 2st + half holds registers 8 half .. 8 half + 7 as bf16
     auto w_of = [&](int st, int r) {
