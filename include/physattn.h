@@ -37,6 +37,9 @@ extern "C" {
 #define PA_BF16 1
 /* bf16 activations; the three large weights are fp8 e4m3 (OCP "fn": bias 7, no infinities, 0x7f/0xff = NaN) bytes
  * with one float32 scale per OUTPUT channel: W[o, :] = scale[o] * decode(byte[o, :]).  Irregular variant only.
+ * On the MFMA paths the kernels that repack the weights into operand fragments read the e4m3 bytes themselves
+ * (pa_mfma_pack_params, pa_mlp_pack_e4m3, the per-call repack of the 512-wide layers), so a call does the same
+ * launches as with bf16 weights; other shapes expand the weights to bf16 in the workspace first.
  * No reference counterpart (the reference's only fp8 is Transformer Engine delayed scaling). */
 #define PA_BF16_W8 2
 
@@ -365,7 +368,10 @@ int pa_mfma_pack_tokens(const pa_shape *shape, const float *out_slice_token, voi
 #define PA_BUF_PARTIALS 3
 #define PA_BUF_TOKP 4
 int64_t pa_mfma_buffer_bytes(const pa_shape *shape, int which);
-/* Repack the layer parameters (bf16 large weights) for the MFMA kernels; run once per parameter set. */
+/* Repack the layer parameters for the MFMA kernels; run once per parameter set.  The three large weights are bf16
+ * (all three p->*_scale NULL) or fp8-e4m3 bytes with per-output-channel scales (all three non-NULL, as PA_BF16_W8):
+ * the repacking kernel reads the e4m3 bytes itself, so a parameter set kept in fp8 is expanded once, here, and
+ * pa_mfma_layer_forward then runs exactly the bf16 launches. */
 int pa_mfma_pack_params(const pa_shape *shape, const pa_params *p, void *blob, void *stream);
 /* Kernel (a): projections + slice logits + temperature softmax (PA.py:529-537, :172-181). x is bf16 (B,N,C).
  * fx_pack receives fx_mid WITHOUT the in_project_fx bias: pa_mfma_combine_attention adds bias * (sum of the weights)
@@ -469,6 +475,12 @@ int pa_mlp_forward(int dtype, int64_t rows, int64_t C, int64_t F, const pa_mlp_p
 int pa_mlp_pack(int dtype, int64_t C, int64_t F, const pa_mlp_params *p, void *packed, int64_t packed_bytes, void *stream);
 int pa_mlp_forward_packed(int dtype, int64_t rows, int64_t C, int64_t F, const void *packed, const float *b1,
                           const float *b2, const void *u, void *y, const pa_block_tail *tail, void *stream);
+/* pa_mlp_pack for weights held as fp8-e4m3 bytes (layout as PA_BF16_W8: w1 (F,C), w2 (C,F) row-major bytes, 8-byte
+ * aligned, one float32 scale per output row): the repacking kernel reads the bytes and scales itself and writes the
+ * bf16 operand fragments pa_mlp_forward_packed(PA_BF16, ...) takes, bit-identical to pa_mlp_pack over the weights
+ * bf16(scale * e4m3).  No reference counterpart (the reference's only fp8 is Transformer Engine autocast). */
+int pa_mlp_pack_e4m3(int64_t C, int64_t F, const void *w1, const float *w1_scale, const void *w2, const float *w2_scale,
+                     void *packed, int64_t packed_bytes, void *stream);
 
 /* ---- whole block ------------------------------------------------------------------------------ */
 
@@ -549,11 +561,13 @@ int pa_layer_forward_plus(int dtype, const pa_shape *shape, const pa_params *p, 
                           const void *x, const void *uniform, void *y, const pa_block_tail *tail,
                           float *slice_token_out, void *workspace, int64_t workspace_bytes, void *stream);
 
-/* pa_layer_forward for the fused MFMA shapes (pa_query_path() == 1, bf16 weights) with the parameters already
- * repacked by pa_mfma_pack_params into `blob` (PA_BUF_BLOB bytes): callers that run many forwards with unchanged
- * weights keep the blob and skip the repack.  For S <= 64 only qkv_project_weight and in_project_fx_bias of `p` are
- * read; for S = 128 the call runs the packed-tile kernels of the staged family, which take every parameter from `p`
- * (bf16 weights) and leave `blob` unused.  Workspace as for pa_layer_forward.  No reference counterpart. */
+/* pa_layer_forward for the fused MFMA shapes (pa_query_path() == 1) with the parameters already repacked by
+ * pa_mfma_pack_params into `blob` (PA_BUF_BLOB bytes): callers that run many forwards with unchanged weights keep
+ * the blob and skip the repack.  For S <= 64 only qkv_project_weight and in_project_fx_bias of `p` are read (both
+ * required: PA_ERR_NULL otherwise -- the kernels sum fx_mid without its bias and the combine step adds it); for
+ * S = 128 the call runs the packed-tile kernels of the staged family, which take every parameter from `p` (bf16
+ * weights, or e4m3 bytes when the three scales are set) and leave `blob` unused.  Workspace as for
+ * pa_layer_forward.  No reference counterpart. */
 int pa_mfma_layer_forward(const pa_shape *shape, const pa_params *p, const void *blob, const void *x, void *y,
                           const pa_block_tail *tail, float *slice_token_out, void *workspace,
                           int64_t workspace_bytes, void *stream);

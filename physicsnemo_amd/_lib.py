@@ -20,7 +20,7 @@ EXPORTED = [
     "pa_slice_softmax", "pa_reduce_partial_count", "pa_slice_reduce", "pa_slice_attention",
     "pa_deslice_project", "pa_layer_forward", "pa_mfma_buffer_bytes", "pa_mfma_pack_params",
     "pa_mfma_project_softmax", "pa_mfma_slice_reduce", "pa_mfma_project_softmax_reduce", "pa_mfma_partial_groups",
-     "pa_mfma_combine_attention", "pa_mfma_deslice_project", "pa_mlp_query", "pa_mlp_workspace_bytes", "pa_mlp_forward", "pa_mlp_pack",
+     "pa_mfma_combine_attention", "pa_mfma_deslice_project", "pa_mlp_query", "pa_mlp_workspace_bytes", "pa_mlp_forward", "pa_mlp_pack", "pa_mlp_pack_e4m3",
      "pa_mlp_forward_packed",
     "pa_rows_gemm", "pa_slice_weighted_sum", "pa_backward_query", "pa_backward_point_tiles",
     "pa_slice_attention_backward", "pa_slice_softmax_backward", "pa_slice_softmax_plus",
@@ -149,6 +149,8 @@ def load() -> ctypes.CDLL:
     lib.pa_mlp_workspace_bytes.argtypes = [c_int, c_int64, c_int64, c_int64]
     lib.pa_mlp_pack.restype = c_int
     lib.pa_mlp_pack.argtypes = [c_int, c_int64, c_int64, POINTER(PaMlpParams), c_void_p, c_int64, c_void_p]
+    lib.pa_mlp_pack_e4m3.restype = c_int
+    lib.pa_mlp_pack_e4m3.argtypes = [c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p]
     lib.pa_mlp_forward_packed.restype = c_int
     lib.pa_mlp_forward_packed.argtypes = [c_int, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_void_p,
                                           c_void_p, pt, c_void_p]

@@ -306,13 +306,14 @@ int mfma_layer(const pa_shape &s, const pa_params &p, const void *blob, const vo
     // x_mid / out_x take the room of the slice weights, the projections' fragments that of the parameter blob.
     char *wts = ws + mp.off_blob;
     const int64_t G = pa::mfma::softmax_reduce_groups(s, compute_units());
-    if ((rc = pa::mlp::project_packed(s.B, s.N, s.C, p.in_project_x_weight, p.in_project_x_bias, p.in_project_fx_weight,
-                                      p.in_project_fx_bias, x, wp, fxp, wts, compute_units(), st)))
+    if ((rc = pa::mlp::project_packed(s.B, s.N, s.C, p.in_project_x_weight, p.in_project_x_scale, p.in_project_x_bias,
+                                      p.in_project_fx_weight, p.in_project_fx_scale, p.in_project_fx_bias, x, wp, fxp,
+                                      wts, compute_units(), st)))
       return rc;
     if ((rc = pa::mfma::slice_softmax_reduce(s, p, wp, true, fxp, partials, compute_units(), st))) return rc;
     if ((rc = pa::mfma::combine_attention(s, p, nullptr, partials, G, tok, norm, tok_out, tokp, st))) return rc;
     if ((rc = pa::mfma::deslice_recompute(s, p, wp, true, tokp, wp, compute_units(), st))) return rc;
-    return pa::mlp::linear_packed(s.B, s.N, s.C, p.out_linear_weight, p.out_linear_bias, wp, y,
+    return pa::mlp::linear_packed(s.B, s.N, s.C, p.out_linear_weight, p.out_linear_scale, p.out_linear_bias, wp, y,
                                   tail_active(tail) ? tail : nullptr, wts + 2 * pa::mlp::linear_blob_bytes(s.C),
                                   compute_units(), st);
   }
@@ -338,7 +339,7 @@ int mfma_layer(const pa_shape &s, const pa_params &p, const void *blob, const vo
 
 extern "C" {
 
-int pa_version(void) { return 100; }
+int pa_version(void) { return 110; }
 
 int pa_markers_enabled(void) { return markers().push != nullptr ? 1 : 0; }
 
@@ -834,6 +835,9 @@ int pa_mfma_pack_params(const pa_shape *shape, const pa_params *p, void *blob, v
   if ((rc = check_params(p))) return rc;
   if (!blob) return PA_ERR_NULL;
   if (!aligned16(blob)) return PA_ERR_ALIGN;
+  // all three scales (fp8-e4m3 large weights) or none (bf16)
+  const int scales = (p->in_project_x_scale != nullptr) + (p->in_project_fx_scale != nullptr) + (p->out_linear_scale != nullptr);
+  if (scales != 0 && scales != 3) return PA_ERR_NULL;
   return pa::mfma::pack_params(*shape, *p, blob, static_cast<hipStream_t>(stream));
 }
 
@@ -933,7 +937,18 @@ int pa_mlp_pack(int dtype, int64_t C, int64_t F, const pa_mlp_params *p, void *p
   if (!aligned16(p->w1) || !aligned16(p->w2) || !aligned16(packed)) return PA_ERR_ALIGN;
   if (packed_bytes < mlp_blob_bytes(dtype, C, F)) return PA_ERR_WORKSPACE;
   if (dtype == PA_F32) return pa::f32rows::mlp_pack(F, p->w1, p->w2, packed, static_cast<hipStream_t>(stream));
-  return pa::mlp::pack(C, F, p->w1, p->w2, packed, static_cast<hipStream_t>(stream));
+  return pa::mlp::pack(C, F, p->w1, nullptr, p->w2, nullptr, packed, static_cast<hipStream_t>(stream));
+}
+
+int pa_mlp_pack_e4m3(int64_t C, int64_t F, const void *w1, const float *w1_scale, const void *w2, const float *w2_scale,
+                     void *packed, int64_t packed_bytes, void *stream) {
+  if (C <= 0 || F <= 0) return PA_ERR_DIMS;
+  if (!mlp_served(PA_BF16, 1, C, F)) return PA_ERR_UNSUPPORTED;
+  if (!w1 || !w1_scale || !w2 || !w2_scale || !packed) return PA_ERR_NULL;
+  if ((reinterpret_cast<uintptr_t>(w1) & 7u) || (reinterpret_cast<uintptr_t>(w2) & 7u) || !aligned16(packed))
+    return PA_ERR_ALIGN;
+  if (packed_bytes < mlp_blob_bytes(PA_BF16, C, F)) return PA_ERR_WORKSPACE;
+  return pa::mlp::pack(C, F, w1, w1_scale, w2, w2_scale, packed, static_cast<hipStream_t>(stream));
 }
 
 int pa_mlp_forward_packed(int dtype, int64_t rows, int64_t C, int64_t F, const void *packed, const float *b1,
@@ -968,7 +983,7 @@ int pa_mlp_forward(int dtype, int64_t rows, int64_t C, int64_t F, const pa_mlp_p
     if ((rc = pa::f32rows::mlp_pack(F, p->w1, p->w2, workspace, st))) return rc;
     return pa::f32rows::mlp_forward(rows, F, workspace, p->b1, p->b2, u, y, tail_active(tail) ? tail : nullptr, st);
   }
-  if ((rc = pa::mlp::pack(C, F, p->w1, p->w2, workspace, st))) return rc;
+  if ((rc = pa::mlp::pack(C, F, p->w1, nullptr, p->w2, nullptr, workspace, st))) return rc;
   return pa::mlp::forward(rows, C, F, workspace, p->b1, p->b2, u, y, tail_active(tail) ? tail : nullptr, compute_units(),
                           st);
 }
@@ -1004,12 +1019,13 @@ int pa_mfma_layer_forward(const pa_shape *shape, const pa_params *p, const void 
   Range entry("pa_mfma_layer_forward");
   int rc = check_mfma(shape);
   if (rc) return rc;
-  if (!p || !p->qkv_project_weight || !blob || !x || !y || !workspace) return PA_ERR_NULL;
+  // the kernels sum fx_mid without its bias; the combine step adds bias * (sum of the weights) from p
+  if (!p || !p->qkv_project_weight || !p->in_project_fx_bias || !blob || !x || !y || !workspace) return PA_ERR_NULL;
   if (!aligned16(blob) || !aligned16(x) || !aligned16(y) || !aligned16(workspace)) return PA_ERR_ALIGN;
   if ((rc = check_tail(tail))) return rc;
   if (mfma_layer_on_tiles(*shape)) {  // this sequence reads the parameters themselves, not the blob
-    if (!p->in_project_x_weight || !p->in_project_fx_weight || !p->in_project_slice_weight ||
-        !p->in_project_slice_bias || !p->temperature || !p->out_linear_weight)
+    if (!p->in_project_x_weight || !p->in_project_x_bias || !p->in_project_fx_weight || !p->in_project_slice_weight ||
+        !p->in_project_slice_bias || !p->temperature || !p->out_linear_weight || !p->out_linear_bias)
       return PA_ERR_NULL;
     if (!aligned16(p->in_project_x_weight) || !aligned16(p->in_project_fx_weight) || !aligned16(p->out_linear_weight))
       return PA_ERR_ALIGN;
@@ -1034,24 +1050,37 @@ int pa_layer_forward(int dtype, const pa_shape *shape, const pa_params *p, const
   hipStream_t st = static_cast<hipStream_t>(stream);
 
   char *ws = static_cast<char *>(workspace);
-  pa_params deq;  // PA_BF16_W8: parameters with the fp8 weights expanded to bf16 in the workspace tail
-  if (dtype == PA_BF16_W8) {
+  pa_params local = *p;  // bf16 / float32: no scales, whatever the caller left in those fields
+  if (dtype != PA_BF16_W8) {
+    local.in_project_x_scale = local.in_project_fx_scale = local.out_linear_scale = nullptr;
+    p = &local;
+  } else {
+    // fp8-e4m3 large weights.  Where the shape runs on kernels that take their weights as repacked operand fragments
+    // (the fused MFMA kernels; the packed-tile sequence of the staged family) the repacking kernels read the e4m3
+    // bytes and scales themselves, so the call does the same launches as with bf16 weights.  The remaining shapes
+    // read weights in natural layout: for those the three matrices are first expanded to bf16 in the workspace tail.
     if (!p->in_project_x_scale || !p->in_project_fx_scale || !p->out_linear_scale) return PA_ERR_NULL;
     const int64_t body = body_bytes(PA_BF16, s);
     const int64_t one = round_up(s.H * s.D * s.C * 2, 256);
     if (workspace_bytes < body + 3 * one) return PA_ERR_WORKSPACE;
-    char *w0 = ws + body;
-    deq = *p;
-    if ((rc = pa::general::dequant_e4m3(p->in_project_x_weight, p->in_project_x_scale, w0, s.H * s.D, s.C, st))) return rc;
-    if ((rc = pa::general::dequant_e4m3(p->in_project_fx_weight, p->in_project_fx_scale, w0 + one, s.H * s.D, s.C, st)))
-      return rc;
-    if ((rc = pa::general::dequant_e4m3(p->out_linear_weight, p->out_linear_scale, w0 + 2 * one, s.C, s.H * s.D, st)))
-      return rc;
-    deq.in_project_x_weight = w0;
-    deq.in_project_fx_weight = w0 + one;
-    deq.out_linear_weight = w0 + 2 * one;
-    p = &deq;
     dtype = PA_BF16;
+    const bool packers_read_e4m3 =
+        pa::mfma::supported(dtype, s) ||
+        (pa::mfma::staged_supported(dtype, s) && s.conv_k == 0 && pa::mlp::linear_supported(dtype, s.B * s.N, s.C));
+    if (!packers_read_e4m3) {
+      char *w0 = ws + body;
+      if ((rc = pa::general::dequant_e4m3(p->in_project_x_weight, p->in_project_x_scale, w0, s.H * s.D, s.C, st)))
+        return rc;
+      if ((rc = pa::general::dequant_e4m3(p->in_project_fx_weight, p->in_project_fx_scale, w0 + one, s.H * s.D, s.C, st)))
+        return rc;
+      if ((rc = pa::general::dequant_e4m3(p->out_linear_weight, p->out_linear_scale, w0 + 2 * one, s.C, s.H * s.D, st)))
+        return rc;
+      local.in_project_x_weight = w0;
+      local.in_project_fx_weight = w0 + one;
+      local.out_linear_weight = w0 + 2 * one;
+      local.in_project_x_scale = local.in_project_fx_scale = local.out_linear_scale = nullptr;
+      p = &local;
+    }
   }
   if (pa::mfma::supported(dtype, s)) {
     const MfmaPlan mp = plan_mfma(s);
@@ -1071,14 +1100,14 @@ int pa_layer_forward(int dtype, const pa_shape *shape, const pa_params *p, const
     if (s.conv_k == 0 && pa::mlp::linear_supported(dtype, s.B * s.N, s.C)) {
       // every stage on packed tiles of 32 points: projections, token sums, hand-back, out_linear with the tail
       char *blob = ws + sp.off_wout;
-      if ((rc = pa::mlp::project_packed(s.B, s.N, s.C, p->in_project_x_weight, p->in_project_x_bias,
-                                        p->in_project_fx_weight, p->in_project_fx_bias, x, x_mid, fxp, blob,
-                                        compute_units(), st)))
+      if ((rc = pa::mlp::project_packed(s.B, s.N, s.C, p->in_project_x_weight, p->in_project_x_scale,
+                                        p->in_project_x_bias, p->in_project_fx_weight, p->in_project_fx_scale,
+                                        p->in_project_fx_bias, x, x_mid, fxp, blob, compute_units(), st)))
         return rc;
       if ((rc = pa::mfma::slice_softmax_reduce(s, *p, x_mid, true, fxp, partials, compute_units(), st))) return rc;
       if ((rc = pa::mfma::combine_attention(s, *p, nullptr, partials, sp.G, tok, norm, tok_out, tokp, st))) return rc;
       if ((rc = pa::mfma::deslice_recompute(s, *p, x_mid, true, tokp, x_mid, compute_units(), st))) return rc;
-      return pa::mlp::linear_packed(s.B, s.N, s.C, p->out_linear_weight, p->out_linear_bias, x_mid, y,
+      return pa::mlp::linear_packed(s.B, s.N, s.C, p->out_linear_weight, p->out_linear_scale, p->out_linear_bias, x_mid, y,
                                     tail_active(tail) ? tail : nullptr, blob + 2 * pa::mlp::linear_blob_bytes(s.C),
                                     compute_units(), st);
     }
@@ -1109,7 +1138,7 @@ int pa_layer_forward(int dtype, const pa_shape *shape, const pa_params *p, const
     void *out_x = x_mid;
     if ((rc = pa::mfma::deslice_recompute(s, *p, x_mid, false, tokp, out_x, compute_units(), st))) return rc;
     if (pa::mlp::linear_supported(dtype, s.B * s.N, s.C))  // out_linear, the residual and the LayerNorm in one pass
-      return pa::mlp::linear(s.B * s.N, s.C, p->out_linear_weight, p->out_linear_bias, out_x, y,
+      return pa::mlp::linear(s.B * s.N, s.C, p->out_linear_weight, nullptr, p->out_linear_bias, out_x, y,
                              tail_active(tail) ? tail : nullptr, ws + sp.off_wout, compute_units(), st);
     if ((rc = pa::general::out_linear(dtype, s, *p, out_x, y, st))) return rc;
     if (tail_active(tail)) rc = pa::general::residual_ln(dtype, s, y, *tail, st);

@@ -68,6 +68,49 @@ __device__ __forceinline__ void store_streaming(T *p, T v) {
   __builtin_nontemporal_store(v, p);
 }
 
+// e4m3fn (OCP): 1 sign, 4 exponent (bias 7), 3 mantissa bits; exponent 0 is subnormal (2^-6 * m/8); 0x7f / 0xff are
+// NaN; there are no infinities.
+__device__ __forceinline__ float decode_e4m3fn(uint8_t v) {
+  const int e = (v >> 3) & 15, m = v & 7;
+  float mag;
+  if (e == 15 && m == 7) mag = __uint_as_float(0x7fc00000u);
+  else if (e == 0) mag = (float)m * 0.001953125f;                             // m/8 * 2^-6
+  else mag = __uint_as_float((uint32_t)(e + 120) << 23 | (uint32_t)m << 20);  // 2^(e-7) * (1 + m/8)
+  return (v & 0x80) ? -mag : mag;
+}
+
+// A large weight matrix as the repacking kernels read it: bf16 bits (scale == nullptr), or fp8-e4m3 bytes with one
+// float32 scale per output row.  Element (row, col) as bf16 bits: the stored bits, or bf16(scale[row] * e4m3) rounded
+// to nearest even -- the value an expansion to bf16 followed by an ordinary bf16 repack would have produced.
+struct WeightView {
+  const void *w;
+  const float *scale;
+  int64_t ld;  // elements per row
+};
+__device__ __forceinline__ uint16_t weight_bits(const WeightView &v, int64_t row, int64_t col) {
+  const int64_t at = row * v.ld + col;
+  if (!v.scale) return static_cast<const uint16_t *>(v.w)[at];
+  return f32_to_bf16_bits(v.scale[row] * decode_e4m3fn(static_cast<const uint8_t *>(v.w)[at]));
+}
+// eight consecutive elements of a row (col a multiple of 8) as four packed pairs
+__device__ __forceinline__ void weight_bits8(const WeightView &v, int64_t row, int64_t col, uint32_t out[4]) {
+  const int64_t at = row * v.ld + col;
+  if (!v.scale) {
+    const uint4 q = *reinterpret_cast<const uint4 *>(static_cast<const uint16_t *>(v.w) + at);
+    out[0] = q.x; out[1] = q.y; out[2] = q.z; out[3] = q.w;
+    return;
+  }
+  const uint2 q = *reinterpret_cast<const uint2 *>(static_cast<const uint8_t *>(v.w) + at);
+  const float sc = v.scale[row];
+  const uint32_t b[2] = {q.x, q.y};
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const uint32_t lo = (b[k >> 1] >> (16 * (k & 1))) & 0xffu, hi = (b[k >> 1] >> (16 * (k & 1) + 8)) & 0xffu;
+    out[k] = (uint32_t)f32_to_bf16_bits(sc * decode_e4m3fn((uint8_t)lo)) |
+             ((uint32_t)f32_to_bf16_bits(sc * decode_e4m3fn((uint8_t)hi)) << 16);
+  }
+}
+
 __device__ __forceinline__ float clamp_temperature(float t) { return fminf(fmaxf(t, kTempMin), kTempMax); }
 
 // wave64 butterfly reductions

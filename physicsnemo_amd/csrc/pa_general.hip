@@ -916,18 +916,9 @@ __global__ __launch_bounds__(256) void layernorm_backward_kernel(const T *__rest
 }
 
 // ------------------------------------------------------------------------------------------------
-// dequant_e4m3_kernel: out[o, k] = bf16(scale[o] * decode_e4m3fn(in[o, k])).  e4m3fn: 1 sign, 4 exponent (bias 7),
-// 3 mantissa bits; exponent 0 is subnormal (2^-6 * m/8); 0x7f / 0xff are NaN; there are no infinities.
+// dequant_e4m3_kernel: out[o, k] = bf16(scale[o] * decode_e4m3fn(in[o, k])), for the shapes whose kernels read the
+// large weights in natural layout (the repacking kernels of the MFMA paths read the e4m3 bytes themselves).
 // ------------------------------------------------------------------------------------------------
-__device__ __forceinline__ float decode_e4m3fn(uint8_t v) {
-  const int e = (v >> 3) & 15, m = v & 7;
-  float mag;
-  if (e == 15 && m == 7) mag = __uint_as_float(0x7fc00000u);
-  else if (e == 0) mag = (float)m * 0.001953125f;                      // m/8 * 2^-6
-  else mag = __uint_as_float((uint32_t)(e + 120) << 23 | (uint32_t)m << 20);  // 2^(e-7) * (1 + m/8)
-  return (v & 0x80) ? -mag : mag;
-}
-
 __global__ __launch_bounds__(256) void dequant_e4m3_kernel(const uint8_t *__restrict__ in, const float *__restrict__ scale,
                                                            bf16 *__restrict__ out, int64_t rows, int64_t cols) {
   const int64_t n = rows * cols;

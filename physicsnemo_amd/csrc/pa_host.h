@@ -243,21 +243,23 @@ int deslice_project(const pa_shape &s, const void *blob, const void *w_pack, con
 namespace mlp {
 bool supported(int dtype, int64_t rows, int64_t C, int64_t F);
 int64_t blob_bytes(int64_t C, int64_t F);
-int pack(int64_t C, int64_t F, const void *w1, const void *w2, void *blob, hipStream_t st);
+// w*_scale: nullptr for bf16 weights; else the weight is fp8-e4m3 bytes with one float32 scale per output row
+int pack(int64_t C, int64_t F, const void *w1, const float *w1_scale, const void *w2, const float *w2_scale, void *blob,
+         hipStream_t st);
 int forward(int64_t rows, int64_t C, int64_t F, const void *blob, const float *b1, const float *b2, const void *u,
             void *y, const pa_block_tail *tail, int num_cu, hipStream_t st);
 // y = W x + bias [+ residual] [-> LayerNorm] for bf16 rows, W (C x C) bf16 row-major; blob: linear_blob_bytes(C) of scratch
 bool linear_supported(int dtype, int64_t rows, int64_t C);
 int64_t linear_blob_bytes(int64_t C);
-int linear(int64_t rows, int64_t C, const void *w, const float *bias, const void *x, void *y, const pa_block_tail *tail,
-           void *blob, int num_cu, hipStream_t st);
+int linear(int64_t rows, int64_t C, const void *w, const float *w_scale, const float *bias, const void *x, void *y,
+           const pa_block_tail *tail, void *blob, int num_cu, hipStream_t st);
 // the same with x as packed operand tiles [B tpb][C / 32][2][64 lanes] (k order kperm within a head)
-int linear_packed(int64_t B, int64_t N, int64_t C, const void *w, const float *bias, const void *x_pack, void *y,
-                  const pa_block_tail *tail, void *blob, int num_cu, hipStream_t st);
+int linear_packed(int64_t B, int64_t N, int64_t C, const void *w, const float *w_scale, const float *bias,
+                  const void *x_pack, void *y, const pa_block_tail *tail, void *blob, int num_cu, hipStream_t st);
 // the layer's two Linear input projections as packed operand tiles; blob: 2 linear_blob_bytes(C) of scratch
-int project_packed(int64_t B, int64_t N, int64_t C, const void *w_x, const float *b_x, const void *w_fx,
-                   const float *b_fx, const void *x, void *xm_pack, void *fx_pack, void *blob, int num_cu,
-                   hipStream_t st);
+int project_packed(int64_t B, int64_t N, int64_t C, const void *w_x, const float *s_x, const float *b_x, const void *w_fx,
+                   const float *s_fx, const float *b_fx, const void *x, void *xm_pack, void *fx_pack, void *blob,
+                   int num_cu, hipStream_t st);
 }  // namespace mlp
 
 }  // namespace pa

@@ -61,41 +61,40 @@ __host__ __device__ inline BlobPlan blob_plan(int C, int S) {
 __global__ __launch_bounds__(256) void pack_params_kernel(pa_params p, u32x4 *__restrict__ blob, int C, int S) {
   const int H = C / 32, KS = C / 16, ST = (S + 31) / 32;
   const BlobPlan bp = blob_plan(C, S);
-  const uint16_t *wx = static_cast<const uint16_t *>(p.in_project_x_weight);
-  const uint16_t *wfx = static_cast<const uint16_t *>(p.in_project_fx_weight);
-  const uint16_t *wo = static_cast<const uint16_t *>(p.out_linear_weight);
+  // the three large weights: bf16 bits, or fp8-e4m3 bytes with per-row scales when the parameter set carries scales
+  const WeightView wx{p.in_project_x_weight, p.in_project_x_scale, C}, wfx{p.in_project_fx_weight, p.in_project_fx_scale, C},
+      wo{p.out_linear_weight, p.out_linear_scale, C};
   const int64_t n_units = bp.fvec;
   for (int64_t u = (int64_t)blockIdx.x * 256 + threadIdx.x; u < n_units; u += (int64_t)gridDim.x * 256) {
     const int lane = (int)(u & 63), i = lane & 31, g = lane >> 5;
-    uint16_t e[8];
+    uint32_t e[4];
     if (u < bp.wsl) {
       int64_t q = u >> 6;
       const int ks = (int)(q % KS);
       q /= KS;
       const int m = (int)(q & 1), h = (int)(q >> 1);
-      const uint16_t *src = (m ? wfx : wx) + (int64_t)(h * 32 + i) * C + 16 * ks + 8 * g;
-#pragma unroll
-      for (int j = 0; j < 8; ++j) e[j] = src[j];
+      weight_bits8(m ? wfx : wx, h * 32 + i, 16 * ks + 8 * g, e);
     } else if (u < bp.wout) {
       const int q = (int)((u - bp.wsl) >> 6);
       const int kk = q & 1, st = q >> 1;
       const int s = 32 * st + i;
 #pragma unroll
-      for (int j = 0; j < 8; ++j)
-        e[j] = s < S ? to_bf16_bits(p.in_project_slice_weight[(int64_t)s * 32 + kperm(kk, g, j)]) : (uint16_t)0;
+      for (int j = 0; j < 4; ++j) {
+        const uint16_t lo = s < S ? to_bf16_bits(p.in_project_slice_weight[(int64_t)s * 32 + kperm(kk, g, 2 * j)]) : (uint16_t)0;
+        const uint16_t hi = s < S ? to_bf16_bits(p.in_project_slice_weight[(int64_t)s * 32 + kperm(kk, g, 2 * j + 1)]) : (uint16_t)0;
+        e[j] = (uint32_t)lo | ((uint32_t)hi << 16);
+      }
     } else {
       int q = (int)((u - bp.wout) >> 6);
       const int kk = q & 1;
       q >>= 1;
       const int h = q % H, ct = q / H;
-      const uint16_t *src = wo + (int64_t)(ct * 32 + i) * C + h * 32;
 #pragma unroll
-      for (int j = 0; j < 8; ++j) e[j] = src[kperm(kk, g, j)];
+      for (int j = 0; j < 4; ++j)
+        e[j] = (uint32_t)weight_bits(wo, ct * 32 + i, h * 32 + kperm(kk, g, 2 * j)) |
+               ((uint32_t)weight_bits(wo, ct * 32 + i, h * 32 + kperm(kk, g, 2 * j + 1)) << 16);
     }
-    u32x4 v;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) v[j] = (uint32_t)e[2 * j] | ((uint32_t)e[2 * j + 1] << 16);
-    blob[u] = v;
+    blob[u] = u32x4{e[0], e[1], e[2], e[3]};
   }
   float *fv = reinterpret_cast<float *>(blob + bp.fvec);
   for (int k = blockIdx.x * 256 + threadIdx.x; k < bp.nfloat; k += gridDim.x * 256) {
@@ -325,11 +324,18 @@ __device__ __forceinline__ void project_softmax_body(const u32x4 *__restrict__ b
     for (int st = 0; st < ST; ++st) lg[st] = mma(wsl[(st * 2 + 0) * 64 + lane], tl.xb0, lg[st]);
 #pragma unroll
     for (int st = 0; st < ST; ++st) lg[st] = mma(wsl[(st * 2 + 1) * 64 + lane], tl.xb1, lg[st]);
+    // one maximum chain per slice tile: the chain of the first tile runs while the MFMAs of the second complete
     float mx = -INFINITY;
 #pragma unroll
-    for (int st = 0; st < ST; ++st)
+    for (int r = 0; r < 16; ++r) mx = fmaxf(mx, lg[0][r]);
+    if constexpr (ST > 1) {
+      float mx2 = -INFINITY;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) mx = fmaxf(mx, lg[st][r]);
+      for (int st = 1; st < ST; ++st)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) mx2 = fmaxf(mx2, lg[st][r]);
+      mx = fmaxf(mx, mx2);
+    }
     mx = half_max(mx);
     const float sc = tscale[h];
     const float off = mx * sc;

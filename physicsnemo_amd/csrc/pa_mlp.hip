@@ -47,32 +47,26 @@ __host__ __device__ constexpr int slot_units(int C) { return (2 * (C / 16) + (C 
 // (zeros in the last slot) and W2 of hidden chunk c - 1 (zeros in the first).
 //   W1 fragment (n, ks): lane (i, g) holds W1[64c + 32n + i][16ks + 8g + j]
 //   W2 fragment (ct, k4 = 2n + kk): lane (i, g) holds W2[32ct + i][64(c-1) + 32n + kperm(kk, g, j)]
-__global__ __launch_bounds__(256) void pack_kernel(const uint16_t *__restrict__ w1, const uint16_t *__restrict__ w2,
-                                                   u32x4 *__restrict__ blob, int C, int F) {
+__global__ __launch_bounds__(256) void pack_kernel(WeightView w1, WeightView w2, u32x4 *__restrict__ blob, int C, int F) {
   const int KS = C / 16, NF1 = 2 * KS, SU = slot_units(C), NC = F / 64;
   const int64_t total = (int64_t)(NC + 1) * SU;
   for (int64_t u = (int64_t)blockIdx.x * 256 + threadIdx.x; u < total; u += (int64_t)gridDim.x * 256) {
     const int c = (int)(u / SU), r = (int)(u - (int64_t)c * SU), frag = r >> 6, lane = r & 63, i = lane & 31, g = lane >> 5;
-    uint16_t e[8];
-#pragma unroll
-    for (int j = 0; j < 8; ++j) e[j] = 0;
+    uint32_t e[4] = {0, 0, 0, 0};
     if (frag < NF1) {
       if (c < NC) {
         const int n = frag / KS, ks = frag - n * KS;
-        const uint16_t *src = w1 + (int64_t)(64 * c + 32 * n + i) * C + 16 * ks + 8 * g;
-#pragma unroll
-        for (int j = 0; j < 8; ++j) e[j] = src[j];
+        weight_bits8(w1, 64 * c + 32 * n + i, 16 * ks + 8 * g, e);
       }
     } else if (c > 0) {
       const int q = frag - NF1, ct = q >> 2, k4 = q & 3, n = k4 >> 1, kk = k4 & 1;
-      const uint16_t *src = w2 + (int64_t)(32 * ct + i) * F + 64 * (c - 1) + 32 * n;
+      const int64_t row2 = 32 * ct + i, col2 = 64 * (c - 1) + 32 * n;
 #pragma unroll
-      for (int j = 0; j < 8; ++j) e[j] = src[kperm(kk, g, j)];
+      for (int j = 0; j < 4; ++j)
+        e[j] = (uint32_t)weight_bits(w2, row2, col2 + kperm(kk, g, 2 * j)) |
+               ((uint32_t)weight_bits(w2, row2, col2 + kperm(kk, g, 2 * j + 1)) << 16);
     }
-    u32x4 v;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) v[j] = (uint32_t)e[2 * j] | ((uint32_t)e[2 * j + 1] << 16);
-    blob[u] = v;
+    blob[u] = u32x4{e[0], e[1], e[2], e[3]};
   }
 }
 
@@ -460,34 +454,28 @@ struct Cfg {
   static_assert(NT * KS == NP && CT * NT * 2 == NP, "both products take 32 MFMAs per slot");
 };
 
-__global__ __launch_bounds__(256) void pack_kernel(const uint16_t *__restrict__ w1, const uint16_t *__restrict__ w2,
-                                                   u32x4 *__restrict__ blob, int C, int F) {
+__global__ __launch_bounds__(256) void pack_kernel(WeightView w1, WeightView w2, u32x4 *__restrict__ blob, int C, int F) {
   const int KS = C / 16, CT = C / 32, HS = 16384 / C, NT = HS / 32, NCH = F / HS;
   (void)KS;
   const int64_t total = (int64_t)(NCH + 2) * 4096;
   for (int64_t u = (int64_t)blockIdx.x * 256 + threadIdx.x; u < total; u += (int64_t)gridDim.x * 256) {
     const int c = (int)(u >> 12), r = (int)(u & 4095), frag = r >> 6, lane = r & 63, i = lane & 31, g = lane >> 5;
     const int P = frag >> 1;
-    uint16_t e[8];
-#pragma unroll
-    for (int j = 0; j < 8; ++j) e[j] = 0;
+    uint32_t e[4] = {0, 0, 0, 0};
     if ((frag & 1) == 0) {
       if (c < NCH) {
         const int n = P % NT, ks = P / NT;
-        const uint16_t *src = w1 + (int64_t)(HS * c + 32 * n + i) * C + 16 * ks + 8 * g;
-#pragma unroll
-        for (int j = 0; j < 8; ++j) e[j] = src[j];
+        weight_bits8(w1, HS * c + 32 * n + i, 16 * ks + 8 * g, e);
       }
     } else if (c >= 2) {
       const int ct = P % CT, nk = P / CT, n = nk >> 1, kk = nk & 1;
-      const uint16_t *src = w2 + (int64_t)(32 * ct + i) * F + HS * (c - 2) + 32 * n;
+      const int64_t row2 = 32 * ct + i, col2 = HS * (c - 2) + 32 * n;
 #pragma unroll
-      for (int j = 0; j < 8; ++j) e[j] = src[kperm(kk, g, j)];
+      for (int j = 0; j < 4; ++j)
+        e[j] = (uint32_t)weight_bits(w2, row2, col2 + kperm(kk, g, 2 * j)) |
+               ((uint32_t)weight_bits(w2, row2, col2 + kperm(kk, g, 2 * j + 1)) << 16);
     }
-    u32x4 v;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) v[j] = (uint32_t)e[2 * j] | ((uint32_t)e[2 * j + 1] << 16);
-    blob[u] = v;
+    blob[u] = u32x4{e[0], e[1], e[2], e[3]};
   }
 }
 
@@ -798,31 +786,25 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 //             phase 1; the first B operand of g(c) replaces that of g(c-1) once its last reader is issued.
 // The epilogue stages through 8 KB per wave of a separate 64 KB region.
 // ---------------------------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void pack2_kernel(const uint16_t *__restrict__ w1, const uint16_t *__restrict__ w2,
-                                                    u32x4 *__restrict__ blob, int C, int F) {
+__global__ __launch_bounds__(256) void pack2_kernel(WeightView w1, WeightView w2, u32x4 *__restrict__ blob, int C, int F) {
   const int KS = C / 16, CT = C / 32, NCH = F / 32, SU = (KS + 2 * CT) * 64;
   const int64_t total = (int64_t)(NCH + 1) * SU;
   for (int64_t u = (int64_t)blockIdx.x * 256 + threadIdx.x; u < total; u += (int64_t)gridDim.x * 256) {
     const int c = (int)(u / SU), r = (int)(u - (int64_t)c * SU), frag = r >> 6, lane = r & 63, i = lane & 31, g = lane >> 5;
-    uint16_t e[8];
-#pragma unroll
-    for (int j = 0; j < 8; ++j) e[j] = 0;
+    uint32_t e[4] = {0, 0, 0, 0};
     if (frag < KS) {
       if (c < NCH) {
-        const uint16_t *src = w1 + (int64_t)(32 * c + i) * C + 16 * frag + 8 * g;
-#pragma unroll
-        for (int j = 0; j < 8; ++j) e[j] = src[j];
+        weight_bits8(w1, 32 * c + i, 16 * frag + 8 * g, e);
       }
     } else if (c > 0) {
       const int t = frag - KS, kk = t / CT, ct = t % CT;
-      const uint16_t *src = w2 + (int64_t)(32 * ct + i) * F + 32 * (c - 1);
+      const int64_t row2 = 32 * ct + i, col2 = 32 * (c - 1);
 #pragma unroll
-      for (int j = 0; j < 8; ++j) e[j] = src[kperm(kk, g, j)];
+      for (int j = 0; j < 4; ++j)
+        e[j] = (uint32_t)weight_bits(w2, row2, col2 + kperm(kk, g, 2 * j)) |
+               ((uint32_t)weight_bits(w2, row2, col2 + kperm(kk, g, 2 * j + 1)) << 16);
     }
-    u32x4 v;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) v[j] = (uint32_t)e[2 * j] | ((uint32_t)e[2 * j + 1] << 16);
-    blob[u] = v;
+    blob[u] = u32x4{e[0], e[1], e[2], e[3]};
   }
 }
 
@@ -967,25 +949,23 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void mlp_rows2_kernel(
 // ---------------------------------------------------------------------------------------------------------------
 // head_order = 0: the reduction index of k-step ks runs over input channels 16 ks + 8 g + j (rows read in natural
 // layout); 1: over 32 (ks / 2) + kperm(ks % 2, g, j) (rows read as the packed operand tiles the slice kernels write)
-__global__ __launch_bounds__(256) void linear_pack_kernel(const uint16_t *__restrict__ w, u32x4 *__restrict__ blob, int C,
-                                                          int head_order) {
+__global__ __launch_bounds__(256) void linear_pack_kernel(WeightView w, u32x4 *__restrict__ blob, int C, int head_order) {
   const int CT = C / 32, KPS = 64 / CT;
   const int64_t total = (int64_t)C * C / 8;
   for (int64_t u = (int64_t)blockIdx.x * 256 + threadIdx.x; u < total; u += (int64_t)gridDim.x * 256) {
     const int c = (int)(u >> 12), j = (int)(u & 4095) >> 6, lane = (int)(u & 63), i = lane & 31, g = lane >> 5;
     const int ct = j % CT, ks = c * KPS + j / CT;
-    const uint16_t *row = w + (int64_t)(32 * ct + i) * C;
+    const int64_t row = 32 * ct + i;
+    uint32_t e[4];
     if (!head_order) {
-      blob[u] = *reinterpret_cast<const u32x4 *>(row + 16 * ks + 8 * g);
+      weight_bits8(w, row, 16 * ks + 8 * g, e);
     } else {
-      uint16_t e[8];
 #pragma unroll
-      for (int q = 0; q < 8; ++q) e[q] = row[32 * (ks >> 1) + kperm(ks & 1, g, q)];
-      u32x4 v;
-#pragma unroll
-      for (int q = 0; q < 4; ++q) v[q] = (uint32_t)e[2 * q] | ((uint32_t)e[2 * q + 1] << 16);
-      blob[u] = v;
+      for (int q = 0; q < 4; ++q)
+        e[q] = (uint32_t)weight_bits(w, row, 32 * (ks >> 1) + kperm(ks & 1, g, 2 * q)) |
+               ((uint32_t)weight_bits(w, row, 32 * (ks >> 1) + kperm(ks & 1, g, 2 * q + 1)) << 16);
     }
+    blob[u] = u32x4{e[0], e[1], e[2], e[3]};
   }
 }
 
@@ -1098,13 +1078,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 // what lets two waves share a SIMD, and the stores are spread evenly over the kernel.
 // blob: W_x then W_fx, each H / HPS slots in that order (project_pack_kernel).
 // ---------------------------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void project_pack_kernel(const uint16_t *__restrict__ w, u32x4 *__restrict__ blob, int C) {
+__global__ __launch_bounds__(256) void project_pack_kernel(WeightView w, u32x4 *__restrict__ blob, int C) {
   const int KS = C / 16, HPS = 64 / KS;  // heads per slot
   const int64_t total = (int64_t)C * C / 8;
   for (int64_t u = (int64_t)blockIdx.x * 256 + threadIdx.x; u < total; u += (int64_t)gridDim.x * 256) {
     const int c = (int)(u >> 12), j = (int)(u & 4095) >> 6, lane = (int)(u & 63), i = lane & 31, g = lane >> 5;
     const int ct = HPS * c + j % HPS, ks = j / HPS;
-    blob[u] = *reinterpret_cast<const u32x4 *>(w + (int64_t)(32 * ct + i) * C + 16 * ks + 8 * g);
+    uint32_t e[4];
+    weight_bits8(w, 32 * ct + i, 16 * ks + 8 * g, e);
+    blob[u] = u32x4{e[0], e[1], e[2], e[3]};
   }
 }
 
@@ -1231,21 +1213,21 @@ int64_t blob_bytes(int64_t C, int64_t F) {
 }
 
 
-int pack(int64_t C, int64_t F, const void *w1, const void *w2, void *blob, hipStream_t st) {
+// w1_scale / w2_scale: nullptr for bf16 weights; else w1 / w2 are fp8-e4m3 bytes with one scale per output row
+int pack(int64_t C, int64_t F, const void *w1, const float *w1_scale, const void *w2, const float *w2_scale, void *blob,
+         hipStream_t st) {
+  const WeightView v1{w1, w1_scale, C}, v2{w2, w2_scale, F};
   const bool by_rows = use_rows_kernel(C), by_rows2 = use_rows2_kernel(C);
   const int64_t total = by_rows    ? (F / (16384 / C) + 2) * (int64_t)4096
                         : by_rows2 ? (F / 32 + 1) * (int64_t)(C / 16 + 2 * (C / 32)) * 64
                                    : (F / 64 + 1) * (int64_t)slot_units((int)C);
   const int grid = (int)((total + 255) / 256 < 1024 ? (total + 255) / 256 : 1024);
   if (by_rows2)
-    hipLaunchKernelGGL(rows::pack2_kernel, dim3(grid), dim3(256), 0, st, static_cast<const uint16_t *>(w1),
-                       static_cast<const uint16_t *>(w2), static_cast<u32x4 *>(blob), (int)C, (int)F);
+    hipLaunchKernelGGL(rows::pack2_kernel, dim3(grid), dim3(256), 0, st, v1, v2, static_cast<u32x4 *>(blob), (int)C, (int)F);
   else if (by_rows)
-    hipLaunchKernelGGL(rows::pack_kernel, dim3(grid), dim3(256), 0, st, static_cast<const uint16_t *>(w1),
-                       static_cast<const uint16_t *>(w2), static_cast<u32x4 *>(blob), (int)C, (int)F);
+    hipLaunchKernelGGL(rows::pack_kernel, dim3(grid), dim3(256), 0, st, v1, v2, static_cast<u32x4 *>(blob), (int)C, (int)F);
   else
-    hipLaunchKernelGGL(pack_kernel, dim3(grid), dim3(256), 0, st, static_cast<const uint16_t *>(w1),
-                       static_cast<const uint16_t *>(w2), static_cast<u32x4 *>(blob), (int)C, (int)F);
+    hipLaunchKernelGGL(pack_kernel, dim3(grid), dim3(256), 0, st, v1, v2, static_cast<u32x4 *>(blob), (int)C, (int)F);
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? PA_OK : (int)e;
 }
@@ -1376,12 +1358,12 @@ static int linear_c(int64_t rows, const void *blob, const float *bias, const voi
 }
 
 template <bool PACKED_IN>
-static int linear_any(int64_t rows, int64_t C, const void *w, const float *bias, const void *x, void *y,
-                      const pa_block_tail *tail, void *blob, int64_t N, int tpb, int num_cu, hipStream_t st) {
+static int linear_any(int64_t rows, int64_t C, const void *w, const float *w_scale, const float *bias, const void *x,
+                      void *y, const pa_block_tail *tail, void *blob, int64_t N, int tpb, int num_cu, hipStream_t st) {
   if (C != 512 && C != 256) return PA_ERR_UNSUPPORTED;
   const int64_t total = C * C / 8;
   hipLaunchKernelGGL(rows::linear_pack_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st,
-                     static_cast<const uint16_t *>(w), static_cast<u32x4 *>(blob), (int)C, PACKED_IN ? 1 : 0);
+                     WeightView{w, w_scale, C}, static_cast<u32x4 *>(blob), (int)C, PACKED_IN ? 1 : 0);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return (int)e;
   if (C == 512) return linear_c<512, PACKED_IN>(rows, blob, bias, x, y, tail, N, tpb, num_cu, st);
@@ -1389,32 +1371,32 @@ static int linear_any(int64_t rows, int64_t C, const void *w, const float *bias,
 }
 
 // y = W x + bias (+ tail) for (rows, C) row-major x; `blob` = linear_blob_bytes(C) bytes of scratch for the
-// fragment-ordered weights
-int linear(int64_t rows, int64_t C, const void *w, const float *bias, const void *x, void *y, const pa_block_tail *tail,
-           void *blob, int num_cu, hipStream_t st) {
-  return linear_any<false>(rows, C, w, bias, x, y, tail, blob, 0, 1, num_cu, st);
+// fragment-ordered weights.  w_scale: nullptr for a bf16 W, else W is fp8-e4m3 bytes with one scale per output row.
+int linear(int64_t rows, int64_t C, const void *w, const float *w_scale, const float *bias, const void *x, void *y,
+           const pa_block_tail *tail, void *blob, int num_cu, hipStream_t st) {
+  return linear_any<false>(rows, C, w, w_scale, bias, x, y, tail, blob, 0, 1, num_cu, st);
 }
 
 // the same with x as packed operand tiles [B tpb][C / 32][2][64 lanes] of 16 bytes (tile b tpb + t = points
 // 32 t .. 32 t + 31 of batch b, k order kperm within a head); y and the tail tensors stay (B, N, C) row-major
-int linear_packed(int64_t B, int64_t N, int64_t C, const void *w, const float *bias, const void *x_pack, void *y,
-                  const pa_block_tail *tail, void *blob, int num_cu, hipStream_t st) {
+int linear_packed(int64_t B, int64_t N, int64_t C, const void *w, const float *w_scale, const float *bias,
+                  const void *x_pack, void *y, const pa_block_tail *tail, void *blob, int num_cu, hipStream_t st) {
   const int64_t tpb = (N + 31) / 32;
-  return linear_any<true>(B * tpb, C, w, bias, x_pack, y, tail, blob, N, (int)tpb, num_cu, st);
+  return linear_any<true>(B * tpb, C, w, w_scale, bias, x_pack, y, tail, blob, N, (int)tpb, num_cu, st);
 }
 
 // the layer's two input projections as packed operand tiles (x_mid: B operands, fx_mid: A operands); `blob` =
-// 2 linear_blob_bytes(C) bytes of scratch
-int project_packed(int64_t B, int64_t N, int64_t C, const void *w_x, const float *b_x, const void *w_fx,
-                   const float *b_fx, const void *x, void *xm_pack, void *fx_pack, void *blob, int num_cu,
-                   hipStream_t st) {
+// 2 linear_blob_bytes(C) bytes of scratch.  s_x / s_fx: nullptr for bf16 weights, else per-row scales of e4m3 weights.
+int project_packed(int64_t B, int64_t N, int64_t C, const void *w_x, const float *s_x, const float *b_x, const void *w_fx,
+                   const float *s_fx, const float *b_fx, const void *x, void *xm_pack, void *fx_pack, void *blob,
+                   int num_cu, hipStream_t st) {
   if (C != 512 && C != 256) return PA_ERR_UNSUPPORTED;
   const int64_t total = C * C / 8;
   u32x4 *bl = static_cast<u32x4 *>(blob);
   hipLaunchKernelGGL(rows::project_pack_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st,
-                     static_cast<const uint16_t *>(w_x), bl, (int)C);
+                     WeightView{w_x, s_x, C}, bl, (int)C);
   hipLaunchKernelGGL(rows::project_pack_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st,
-                     static_cast<const uint16_t *>(w_fx), bl + total, (int)C);
+                     WeightView{w_fx, s_fx, C}, bl + total, (int)C);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return (int)e;
   const size_t lds = (size_t)2 * 4096 * 16 + (size_t)2 * C * 4;

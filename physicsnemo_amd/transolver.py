@@ -139,7 +139,15 @@ class TransolverBlock(nn.Module):
         """(packed weights, b1, b2) for pa_mlp_forward_packed: the weights repacked once per parameter set."""
         w1, b1, w2, b2 = self._mlp_kernel_params(device, dtype)
         if "packed" not in self._mlp_cache:
-            self._mlp_cache["packed"] = PF.mlp_pack(w1, w2)
+            if self.fp8_weights and dtype == torch.bfloat16:
+                # the e4m3 bytes and scales go to the repacking kernel as they are: expanded once per parameter set
+                lin1, lin2 = self.ln_mlp1[1].layers[0], self.ln_mlp1[1].layers[2]
+                with torch.no_grad():
+                    q1, s1 = PF.quantize_e4m3_per_channel(lin1.weight.detach().to(device))
+                    q2, s2 = PF.quantize_e4m3_per_channel(lin2.weight.detach().to(device))
+                self._mlp_cache["packed"] = PF.mlp_pack_e4m3(q1, s1, q2, s2)
+            else:
+                self._mlp_cache["packed"] = PF.mlp_pack(w1, w2)
         return self._mlp_cache["packed"], b1, b2
 
     def _mlp_kernel_serves(self, normed: torch.Tensor) -> bool:

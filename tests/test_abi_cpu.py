@@ -66,6 +66,44 @@ def test_argument_errors_are_codes_not_crashes():
     assert lib.pa_status_string(-5) == b"workspace too small"
 
 
+def test_mfma_layer_forward_rejects_missing_biases_and_mixed_scales():
+    """The fused kernels sum fx_mid without its bias and the combine step adds it from `p`: a parameter set without
+    in_project_fx_bias is an error, not a silently bias-free result.  Scales are all set (e4m3 weights) or all NULL."""
+    lib = _lib.load()
+    assert lib.pa_version() >= 110
+    s = _shape(B=1, N=4096, C=256, H=8, D=32, S=64)
+    names = [n for n, _ in _lib.PaParams._fields_]
+
+    def params(**null):
+        vals = {n: (256 if not n.endswith("_scale") else None) for n in names}
+        vals.update(null)
+        return _lib.PaParams(*[vals[n] for n in names])
+
+    big = 1 << 40
+    ok_args = (256, 256, 256, None, None, 256, big, None)  # blob, x, y, tail, tokens, workspace, bytes, stream
+    p = params(in_project_fx_bias=None)
+    assert lib.pa_mfma_layer_forward(ctypes.byref(s), ctypes.byref(p), *ok_args) == -1
+    p = params(qkv_project_weight=None)
+    assert lib.pa_mfma_layer_forward(ctypes.byref(s), ctypes.byref(p), *ok_args) == -1
+    # S = 128 runs the packed-tile sequence, which reads every parameter itself
+    s128 = _shape(B=1, N=4096, C=256, H=8, D=32, S=128)
+    for missing in ("in_project_x_bias", "in_project_fx_bias", "out_linear_bias", "in_project_x_weight"):
+        p = params(**{missing: None})
+        assert lib.pa_mfma_layer_forward(ctypes.byref(s128), ctypes.byref(p), *ok_args) == -1, missing
+    # repacking: one or two of the three scales is a malformed parameter set
+    p = params(in_project_x_scale=256)
+    assert lib.pa_mfma_pack_params(ctypes.byref(s), ctypes.byref(p), 256, None) == -1
+    p = params(in_project_x_scale=256, in_project_fx_scale=256)
+    assert lib.pa_mfma_pack_params(ctypes.byref(s), ctypes.byref(p), 256, None) == -1
+    # the e4m3 repack of the MLP weights: argument errors are codes
+    assert lib.pa_mlp_pack_e4m3(256, 1024, None, 256, 256, 256, 256, big, None) == -1
+    assert lib.pa_mlp_pack_e4m3(256, 1024, 256, None, 256, 256, 256, big, None) == -1
+    assert lib.pa_mlp_pack_e4m3(256, 1024, 260, 256, 256, 256, 256, big, None) == -4   # bytes must be 8-byte aligned
+    assert lib.pa_mlp_pack_e4m3(256, 1024, 256, 256, 256, 256, 256, 16, None) == -5
+    assert lib.pa_mlp_pack_e4m3(200, 1024, 256, 256, 256, 256, 256, big, None) == -3
+    assert lib.pa_mlp_pack_e4m3(0, 1024, 256, 256, 256, 256, 256, big, None) == -2
+
+
 def test_module_signatures_state_dict_and_seeded_init_match_oracle():
     from oracle import torch_oracle as to
     torch.manual_seed(7)

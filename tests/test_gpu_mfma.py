@@ -212,11 +212,16 @@ def test_mfma_full_size_properties(S):
     assert bool(((tk >= lo - 1e-2) & (tk <= hi + 1e-2)).all())
 
 
-# bound = what the number format allows for the shape: e4m3 keeps 3 mantissa bits, and the rounding of the weights
-# ALONE (fp32 oracle with dequantised weights against fp32 oracle with the original ones, listed in the test summary)
-# already costs 0.65e-2 .. 1.2e-2 depending on the shape; the 512-wide layers exceed 1e-2 before any kernel runs.
+# bound = what the number format allows for the shape: e4m3 keeps 3 mantissa bits, so every weight carries a relative
+# rounding error of 2.3 % rms whatever the scale (2.55 % with scale = max|row| / 448, 2.27 % with the per-row scale
+# search of quantize_e4m3_per_channel), and the rounding of the weights ALONE (fp32 oracle with dequantised weights
+# against fp32 oracle with the original ones, listed in the test summary) costs 0.6e-2 .. 1.1e-2 of the layer output
+# depending on the shape.  At 512 channels and 128 slices the 6000-point case stays within 1e-2 (7.6e-3; 7.9e-3 with
+# scale = max|row| / 448); the 700-point case sits at it (1.02e-2 from the rounding of the weights alone, 1.22e-2 with
+# max|row| / 448): few points per slice leave the slice tokens, and with them the inputs of out_linear, less
+# averaged, and no choice of one scale per channel changes the mantissa width.  Its bound is 1.1e-2.
 @pytest.mark.parametrize("B,N,C,S,bound", [(2, 3000, 256, 64, 1e-2), (1, 2000, 128, 32, 1e-2),
-                                           (1, 700, 512, 128, 1.4e-2), (1, 6000, 512, 128, 1.4e-2)])
+                                           (1, 700, 512, 128, 1.1e-2), (1, 6000, 512, 128, 1e-2)])
 def test_fp8_e4m3_weight_variant(B, N, C, S, bound):
     # bf16 activations, fp8-e4m3 per-output-channel-scaled projection weights.  Checks: (1) rel-L2 against the fp32
     # oracle holding the ORIGINAL (unquantised) weights: within `bound`, and never more than the quantisation error of
@@ -230,10 +235,11 @@ def test_fp8_e4m3_weight_variant(B, N, C, S, bound):
     xb = x.cuda().bfloat16()
     with torch.no_grad():
         want_full = ref(xb.float().cpu())
-        deq = {}
+        deq, quant = {}, {}
         for name in ("in_project_x", "in_project_fx", "out_linear"):
             w = getattr(ref, name).weight
             q, s = PF.quantize_e4m3_per_channel(w)
+            quant[name] = (q, s)
             deq[name] = PF.dequantize_e4m3_per_channel(q, s)
             getattr(ref, name).weight.copy_(deq[name])
         want_q = ref(xb.float().cpu())
@@ -253,6 +259,21 @@ def test_fp8_e4m3_weight_variant(B, N, C, S, bound):
     assert err <= (q_err ** 2 + 4e-3 ** 2) ** 0.5, (err, q_err)
     assert_rel_l2(y8, want_q, "fp8-weight layer vs fp32 oracle with the dequantised weights")
     assert torch.equal(y8, y16)
+    # the repacked parameter blob of the fused kernels is built from the e4m3 bytes by the repacking kernel itself:
+    # it equals the blob of the dequantised weights served as bf16 (what `hip` holds now)
+    dims = hip.layer_dims(xb)
+    if PF.query_path(torch.bfloat16, dims) == 1:
+        p16 = hip.kernel_params(torch.bfloat16, xb.device)
+        st16 = PF.MfmaStages(p16, dims, xb.device)
+        st16.pack_params()
+        p8 = {k: v for k, v in p16.items() if not k.startswith("_")}
+        for name in deq:
+            p8[name + "_weight"] = quant[name][0].cuda().reshape(-1)
+            p8[name + "_scale"] = quant[name][1].cuda()
+        st8 = PF.MfmaStages(p8, dims, xb.device)
+        st8.pack_params()
+        torch.cuda.synchronize()
+        assert torch.equal(st8.blob, st16.blob)
 
 
 @pytest.mark.parametrize("S", [16, 64])

@@ -167,3 +167,30 @@ def test_preprocess_mlp_fp32_matches_oracle(rows_shape, c_in, Fh):
     assert not PF.preprocess_supported(torch.float32, 100, 9, 256, C)
     assert not PF.preprocess_supported(torch.float32, 100, 8, 512, C)  # the first Linear no longer fits beside the ring
     assert not PF.preprocess_supported(torch.float32, 100, 3, 256, 256)
+
+
+@pytest.mark.parametrize("C,Fh", [(128, 512), (256, 1024), (512, 2048)])
+def test_mlp_repack_reads_e4m3_weights(C, Fh):
+    """pa_mlp_pack_e4m3 (the repacking kernel fed e4m3 bytes + per-row scales) writes the very fragments pa_mlp_pack
+    writes for the dequantised weights rounded to bf16: fp8 weights cost one expansion per parameter set, in the repack."""
+    announce("mlp e4m3 repack", C, Fh)
+    torch.manual_seed(C)
+    dev = torch.device("cuda:0")
+    w1, w2 = (torch.randn(Fh, C) / C ** 0.5).to(dev), (torch.randn(C, Fh) / Fh ** 0.5).to(dev)
+    w1[3] = 0  # an all-zero row: scale floor, zero bytes
+    q1, s1 = PF.quantize_e4m3_per_channel(w1)
+    q2, s2 = PF.quantize_e4m3_per_channel(w2)
+    d1, d2 = PF.dequantize_e4m3_per_channel(q1, s1), PF.dequantize_e4m3_per_channel(q2, s2)
+    # the searched scale never does worse than max|row| / 448
+    q1p, s1p = PF.quantize_e4m3_per_channel(w1, search=0)
+    err = lambda d, w: float((d - w).norm() / w.norm())
+    assert err(d1, w1) <= err(PF.dequantize_e4m3_per_channel(q1p, s1p), w1) + 1e-9
+    assert err(d1, w1) < 2.5e-2 and err(d2, w2) < 2.5e-2  # max|row| / 448: 2.55e-2
+    want = PF.mlp_pack(d1.bfloat16().contiguous(), d2.bfloat16().contiguous())
+    got = PF.mlp_pack_e4m3(q1, s1, q2, s2)
+    assert torch.equal(got, want)
+    u = torch.randn(1, 999, C).bfloat16().to(dev)
+    b1, b2 = torch.randn(Fh).to(dev) * 0.1, torch.randn(C).to(dev) * 0.1
+    y8 = PF.mlp_forward_packed(u, got, b1, b2)
+    y16 = PF.mlp_forward(u, d1.bfloat16().contiguous(), b1, d2.bfloat16().contiguous(), b2)
+    assert torch.equal(y8, y16)
