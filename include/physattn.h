@@ -173,7 +173,8 @@ int pa_slice_reduce(int dtype, const pa_shape *shape, const void *w, const void 
  * for callers that cannot allocate device memory -- code under HIP graph capture, tight serving loops, harnesses
  * that forbid hipMalloc.  Same kernels, same arguments and bit-identical results as pa_slice_reduce; the per-chunk
  * partial sums live in a static device array of PA_STATIC_SCRATCH_BYTES that every GPU the library runs on holds
- * until the process ends.  PA_ERR_SCRATCH if pa_reduce_partial_count(shape) * B*H*S*(D+1) * 4 bytes exceed it.
+ * until the process ends.  PA_ERR_SCRATCH if (pa_reduce_partial_count(shape) + 1) * B*H*S*(D+1) * 4 bytes exceed it
+ * (one slot per chunk and one for their fixed-order total).
  * Calls on one GPU share that GPU's array: calls that overlap in time on the same GPU race on it (calls on one
  * stream, or otherwise ordered, are safe).  Only `shape`'s B, N, H, D, S are read. */
 #define PA_STATIC_SCRATCH_BYTES (64ll << 20)

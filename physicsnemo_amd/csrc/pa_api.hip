@@ -479,8 +479,11 @@ int pa_rows_gemm_act(int dtype, const pa_shape *grid, int64_t c_in, int64_t c_ou
   if (c_in > (1 << 16) || c_out > (1 << 16) || grid->N > PA_MAX_N) return PA_ERR_UNSUPPORTED;
   if (grid->conv_k > 0) {
     if (grid->grid_h <= 0 || grid->grid_w <= 0 || grid->grid_d < 0) return PA_ERR_DIMS;
+    // every extent is at most N (itself at most PA_MAX_N) before any product is formed: no product can overflow
+    if (grid->grid_h > grid->N || grid->grid_w > grid->N || grid->grid_d > grid->N) return PA_ERR_DIMS;
+    if (grid->grid_h * grid->grid_w > grid->N) return PA_ERR_DIMS;
     if (grid->grid_h * grid->grid_w * (grid->grid_d > 0 ? grid->grid_d : 1) != grid->N) return PA_ERR_DIMS;
-    if (grid->conv_k % 2 == 0) return PA_ERR_UNSUPPORTED;
+    if (grid->conv_k % 2 == 0 || grid->conv_k > 1024) return PA_ERR_UNSUPPORTED;
     const int64_t taps = grid->conv_k * grid->conv_k * (grid->grid_d > 0 ? grid->conv_k : 1);
     if (taps * c_in > (int64_t)1 << 30) return PA_ERR_UNSUPPORTED;
   } else if (grid->grid_d != 0) {

@@ -402,9 +402,14 @@ __global__ __launch_bounds__(512) void conv_slice_kernel(
     dst[idx] = ((red[idx] + red[kTokFloats + idx]) + red[2 * kTokFloats + idx]) + red[3 * kTokFloats + idx];
 }
 
-// Linear projections (conv_k == 0: the irregular mesh) are the 1 x 1 case on an N x 1 grid
+int64_t groups(const pa_shape &s);
+
+// Linear projections (conv_k == 0: the irregular mesh) are the 1 x 1 case on an N x 1 grid.  One workgroup per 128
+// points leaves one partial token sum each (17 KB): beyond 4096 of them per call the workspace and the combine pass
+// outgrow what the front end saves, and the shape goes to the general kernels (whose partial count is capped).
 bool supported(int dtype, const pa_shape &s) {
   if (dtype != PA_F32 || s.C != kC || s.H != kH || s.D != kD || s.S != kS || s.N * kC >= (int64_t)1 << 29) return false;
+  if (groups(s) * s.B > 4096) return false;
   if (s.conv_k == 0) return s.grid_d == 0;
   return s.conv_k % 2 == 1 && s.grid_d == 0 && s.grid_h * s.grid_w == s.N;
 }

@@ -52,7 +52,7 @@ int pa_slice_reduce_static(int dtype, const pa_shape *shape, const void *w, cons
   if (dtype != PA_F32 && dtype != PA_BF16) return PA_ERR_UNSUPPORTED;
   const pa_shape &s = *shape;
   if (s.B <= 0 || s.N <= 0 || s.H <= 0 || s.D <= 0 || s.S <= 0) return PA_ERR_DIMS;
-  if (s.D > PA_MAX_D || s.S > PA_MAX_S || s.N > (int64_t)1 << 31 || s.B * s.H > 65535) return PA_ERR_UNSUPPORTED;
+  if (s.D > PA_MAX_D || s.S > PA_MAX_S || s.N > PA_MAX_N || s.B * s.H > 65535) return PA_ERR_UNSUPPORTED;
   if (pa::general::combine_attn_lds_bytes(s) > pa::kMaxLdsBytes) return PA_ERR_UNSUPPORTED;
   if (!w || !fx_mid || !slice_token || !slice_norm) return PA_ERR_NULL;
   if (!pa::aligned16(w) || !pa::aligned16(fx_mid)) return PA_ERR_ALIGN;

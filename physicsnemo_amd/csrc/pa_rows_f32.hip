@@ -748,8 +748,9 @@ int mlp_forward(int64_t M, int64_t F, const void *blob, const float *b1, const f
 
 static size_t block_lds(int64_t F) { return (size_t)kMlpRing * kUnit * 16 + (size_t)(4 * kC + 2 * kC + 4 * kC + F) * 4; }
 
+// F up to 1024 (mlp_ratio 8): what the interface documents and the parity tests cover
 bool block_supported(int dtype, const pa_shape &s, int64_t F) {
-  return backend_supported(dtype, s) && F >= 128 && F % 128 == 0 && block_lds(F) <= 160 * 1024;
+  return backend_supported(dtype, s) && F >= 128 && F % 128 == 0 && F <= 1024 && block_lds(F) <= 160 * 1024;
 }
 
 int64_t block_blob_bytes(int64_t F) { return (8 + (F / 128) * 16) * (int64_t)kUnit * 16; }

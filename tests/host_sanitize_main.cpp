@@ -164,6 +164,28 @@ int main() {
   CHECK(pa_slice_reduce_static(PA_BF16, &big, buf, buf, reinterpret_cast<float *>(buf), reinterpret_cast<float *>(buf),
                                nullptr) < 0);  // partial sums beyond the static array
 
+  // the row GEMM entry point forms its grid products itself: extreme extents must be refused before any product
+  for (int64_t gh : {(int64_t)1, (int64_t)85, (int64_t)1 << 31, (int64_t)1 << 40, (int64_t)1 << 62})
+    for (int64_t gw : {(int64_t)1, (int64_t)85, (int64_t)1 << 31, (int64_t)1 << 62})
+      for (int64_t gd : {(int64_t)0, (int64_t)7, (int64_t)1 << 31, (int64_t)1 << 62})
+        for (int64_t k : {(int64_t)1, (int64_t)3, (int64_t)1 << 20, (int64_t)1 << 40}) {
+          const pa_shape g = make(1, 85 * 85, 128, 8, 16, 32, gh, gw, k, gd, 0);
+          const int rc = pa_rows_gemm_act(PA_F32, &g, 128, 128, nullptr, nullptr, nullptr, 0, nullptr, nullptr);
+          CHECK(rc < 0);  // a bad grid, or (85 x 85, k = 1 / 3, no depth) the null tensors
+        }
+  // the fused layer needs in_project_fx_bias even with the parameters already repacked
+  {
+    pa_params q = p;
+    q.in_project_fx_bias = nullptr;
+    CHECK(pa_mfma_layer_forward(&ok, &q, buf, buf, buf, nullptr, nullptr, buf, (int64_t)1 << 40, nullptr) == PA_ERR_NULL);
+    q = p;
+    q.in_project_x_scale = reinterpret_cast<const float *>(buf);  // one scale of three
+    CHECK(pa_mfma_pack_params(&ok, &q, buf, nullptr) == PA_ERR_NULL);
+    CHECK(pa_mlp_pack_e4m3(256, 1024, buf, nullptr, buf, nullptr, buf, (int64_t)1 << 40, nullptr) == PA_ERR_NULL);
+    CHECK(pa_mlp_pack_e4m3(256, (int64_t)1 << 40, buf, reinterpret_cast<const float *>(buf), buf,
+                           reinterpret_cast<const float *>(buf), buf, (int64_t)1 << 40, nullptr) < 0);
+  }
+
   printf("host sanitize: %lld shapes answered, %d failures\n", answered, failures);
   return failures == 0 ? 0 : 1;
 }

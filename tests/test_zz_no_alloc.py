@@ -52,7 +52,7 @@ def test_static_scratch_rejects_oversized_problems():
     assert limit == 64 << 20
     B, N, H, D, S = 1, 1 << 20, 8, 32, 128  # (512 chunks + 1) x 8 heads x 128 x 33 floats = 69.3 MB > 64 MiB
     dims = PF.LayerDims(B, N, H * D, H, D, S)
-    need = int(lib.pa_reduce_partial_count(byref(dims.c()))) * B * H * S * (D + 1) * 4
+    need = (int(lib.pa_reduce_partial_count(byref(dims.c()))) + 1) * B * H * S * (D + 1) * 4  # chunks + their total
     assert need > limit
     dummy = torch.zeros(64, device="cuda")
     with pytest.raises(RuntimeError, match="static scratch"):
