@@ -125,3 +125,66 @@ def test_cfg5_volume_model_reduced_points(fp8):
                   tol=1.5e-2, report=True)
     assert_rel_l2(got, want, "cfg5 model output (12 blocks, fp8 weights) vs the fp32 oracle with the ORIGINAL weights",
                   tol=9e-2, report=True)
+
+
+def _surface_points(n, g):
+    th = torch.acos(torch.empty(n).uniform_(-1, 1, generator=g))
+    ph = torch.empty(n).uniform_(0, 2 * math.pi, generator=g)
+    rad = 1 + 0.1 * (3 * torch.cos(th) ** 2 - 1) / 2 + 0.05 * torch.sin(th) ** 2 * torch.cos(th) * torch.cos(2 * ph)
+    xyz = torch.stack((1.0 * rad * torch.sin(th) * torch.cos(ph), 0.6 * rad * torch.sin(th) * torch.sin(ph),
+                       0.4 * rad * torch.cos(th)), -1)
+    nrm = torch.nn.functional.normalize(xyz / torch.tensor([1.0, 0.36, 0.16]), dim=-1)
+    return torch.cat((xyz, nrm), -1)[None]
+
+
+# The full-size multi-block paths, pinned to the oracle in two steps.  (1) One copy of a point set goes through the
+# HIP model and through the fp32 oracle: the usual bound.  (2) The full-size input is COPIES copies of that point set:
+# every slice token is a weighted mean over the points, so the copies leave the tokens unchanged (up to the 1e-2 the
+# reference adds to the slice norms -- 1e-6 relative at these sizes -- and the order of the float32 partial sums), the
+# row-local stages (LayerNorms, MLPs, projections) see each copy as they saw the original, and every copy of a point
+# must come out as the original did, to within the bf16 rounding that a changed summation order can flip.
+@pytest.mark.parametrize("name", ["cfg4", "cfg5-fp8"])
+def test_full_size_models_by_replication(name):
+    g = torch.Generator().manual_seed(1234)
+    if name == "cfg4":
+        # cfg4: 1 000 000 surface points, n_hidden 256, 8 heads, 32 slices, 8 layers = 32 copies of 31 250 points
+        n0, copies, tol = 31250, 32, 1.3e-2  # 8 bf16 blocks deep: measured 1.17e-2 for one copy
+        kw = dict(functional_dim=1, embedding_dim=6, out_dim=4, n_layers=8, n_hidden=256, n_head=8, slice_num=32)
+        emb0, fx0 = _surface_points(n0, g), torch.randn(1, n0, 1, generator=g)
+    else:
+        # cfg5: 4 194 304 box points, n_hidden 512, 16 heads, 128 slices, 12 layers, fp8-e4m3 weights = 64 x 65 536
+        n0, copies, tol = 65536, 64, 1.5e-2
+        kw = dict(functional_dim=4, embedding_dim=3, out_dim=4, n_layers=12, n_hidden=512, n_head=16, slice_num=128)
+        emb0, fx0 = torch.rand(1, n0, 3, generator=g), torch.randn(1, n0, 4, generator=g)
+    announce("full-size model by replication", name, copies * n0)
+    ref, hip = _pair(**kw)
+    with torch.no_grad():
+        if name != "cfg4":
+            hip.use_fp8_weights(True)
+            for blk in ref.blocks:  # the oracle holds the dequantised weights: the kernels, not the format, are tested
+                for lin in (blk.Attn.in_project_x, blk.Attn.in_project_fx, blk.Attn.out_linear, blk.ln_mlp1[1].layers[0],
+                            blk.ln_mlp1[1].layers[2]):
+                    lin.weight.copy_(PF.dequantize_e4m3_per_channel(*PF.quantize_e4m3_per_channel(lin.weight)))
+        want0 = ref(fx0, emb0)
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            got0 = hip(fx0.cuda(), emb0.cuda())
+            full = hip(fx0.cuda().repeat(1, copies, 1), emb0.cuda().repeat(1, copies, 1))
+    assert full.shape == (1, copies * n0, 4) and torch.isfinite(full.float()).all()
+    assert_rel_l2(got0, want0, f"{name}: one copy ({n0} points) vs the fp32 oracle", tol=tol, report=True)
+    # every copy of the full-size output against the ORACLE's output for the point set (the bar itself), and against
+    # the HIP model's output for one copy: two bf16 evaluations whose slice tokens were summed in different orders
+    # differ by about as much as each differs from the fp32 result, so that second figure is reported, bounded loosely
+    want_gpu, got_gpu = want0.cuda(), got0.float()
+    worst_oracle = worst_copy = 0.0
+    for k in range(copies):
+        part = full[:, k * n0:(k + 1) * n0].float()
+        worst_oracle = max(worst_oracle, float((part - want_gpu).norm() / want_gpu.norm()))
+        worst_copy = max(worst_copy, float((part - got_gpu).norm() / got_gpu.norm()))
+    import conftest
+
+    conftest.MEASURED.append((f"{name}: worst copy of the full-size output ({copies * n0} points) vs the fp32 oracle",
+                              worst_oracle, tol))
+    conftest.MEASURED.append((f"{name}: worst copy of the full-size output vs the HIP output for one copy", worst_copy,
+                              1.5 * tol))
+    assert worst_oracle <= tol, worst_oracle
+    assert worst_copy <= 1.5 * tol, worst_copy
