@@ -507,7 +507,81 @@ def write_traffic(fetch_dir, write_dir, B, N, C, S):
     print(json.dumps(out, indent=1))
 
 
-def measure_layer(B, N, C, S, steps, warmup, kernel_reps, x_cpu=None, cold=False):
+# kernels of the packed-tile sequence (S = 128, and every 512-wide layer): algorithmic bytes and MFMA flops per point
+def staged_kernel_model(C, H, S, b=2):
+    return {
+        "project_rows_kernel": {"bytes": 3 * C * b, "flops": 4 * C * C},                  # x -> x_mid, fx_mid tiles
+        "slice_softmax_reduce_kernel": {"bytes": 2 * C * b, "flops": 4 * C * S},          # logits + token sums
+        "deslice_recompute_kernel": {"bytes": 2 * C * b, "flops": 4 * C * S},             # logits again + deslice
+        "linear_rows_kernel": {"bytes": 2 * C * b, "flops": 2 * C * C},                   # out_linear
+    }
+
+
+def trace_layer_kernels(layer, x, B, N, C, S, reps=10):
+    """Per-kernel GPU time of one layer call, from the profiler's kernel records (for the kernel sequences that have no
+    stage entry points of their own).  Averages over `reps` calls behind a run-in."""
+    import collections
+
+    import torch
+    from torch.profiler import ProfilerActivity, profile
+
+    H = C // 32
+    run_in(lambda: layer(x))
+    with torch.no_grad(), profile(activities=[ProfilerActivity.CUDA]) as prof:
+        for _ in range(reps):
+            layer(x)
+        torch.cuda.synchronize()
+    acc = collections.defaultdict(float)
+    for ev in prof.events():
+        if ev.device_type == torch.autograd.DeviceType.CUDA:
+            acc[ev.name] += ev.device_time  # microseconds
+    model, out = staged_kernel_model(C, H, S), {}
+    for name, us in sorted(acc.items(), key=lambda kv: -kv[1]):
+        ms = us / reps * 1e-3
+        short = name.split("(")[0].split("::")[-1].split("<")[0]
+        e = {"ms": round(ms, 4)}
+        if short in model and ms > 0:
+            gbs = model[short]["bytes"] * B * N / (ms * 1e-3) / 1e9
+            tf = model[short]["flops"] * B * N / (ms * 1e-3) / 1e12
+            e.update({"hbm_frac": round(gbs / HBM_PEAK_GBS, 4), "mfma_frac": round(tf / MFMA_BF16_PEAK_TF, 4)})
+        out[short] = e
+    return out
+
+
+def occupancy_sweep(x, layer, counts=(256, 192, 128, 64)):
+    """Kernel (a+b) restricted to n workgroups (= n compute units busy, the rest of the chip idle): time of the launch
+    and the shader clock the chip holds under it (the kernel's clock-reporting twin).  The cycles the kernel needs per
+    tile do not depend on n; the clock does."""
+    import torch
+
+    from physicsnemo_amd import _lib
+    from physicsnemo_amd import functional as PF
+
+    lib, out = _lib.load(), []
+    dev = x.device
+    try:
+        for n in counts:
+            _lib.check(lib.pa_set_compute_units(int(n)), "pa_set_compute_units")
+            st = PF.MfmaStages(layer.kernel_params(torch.bfloat16, dev), layer.layer_dims(x), dev)
+            st.pack_params()
+            run_in(lambda: st.project_softmax_reduce(x))
+            ms = time_kernel(lambda: st.project_softmax_reduce(x), 20)
+            ghz = []
+            for _ in range(5):
+                for _ in range(10):
+                    st.project_softmax_reduce(x)
+                ghz.append(st.project_softmax_reduce_clocked(x))
+            g = sorted(ghz)[2]
+            tiles = (x.shape[1] + 31) // 32 * x.shape[0]
+            out.append({"compute_units": int(n), "ms": round(ms, 4), "shader_clock_ghz": round(g[0], 3),
+                        "cycles_per_tile": round(g[1] / (tiles / n), 1)})
+            del st
+    finally:
+        lib.pa_set_compute_units(0)
+    return out
+
+
+def measure_layer(B, N, C, S, steps, warmup, kernel_reps, x_cpu=None, cold=False, occupancy=False):
     """One PhysicsAttentionIrregularMesh layer at (B, N, C, S), bf16: whole-layer time through the module and the C ABI,
     the same call replayed from a HIP graph, and every kernel of the layer timed on its own."""
     import torch
@@ -607,7 +681,15 @@ def measure_layer(B, N, C, S, steps, warmup, kernel_reps, x_cpu=None, cold=False
                     ghz.append(st.project_softmax_reduce_clocked(x)[0])
                 roofline["shader_clock_ghz"] = round(sorted(ghz)[2], 3)
                 roofline["top_clock_ghz"] = TOP_CLOCK_GHZ
+                # the MFMA fraction priced at the clock the chip actually holds under this kernel
+                roofline["mfma_frac_at_held_clock"] = round(
+                    kernels[dominant]["mfma_frac"] * TOP_CLOCK_GHZ / roofline["shader_clock_ghz"], 4)
         del st, yk
+        if occupancy and fused and C == 256:
+            res["occupancy_sweep"] = occupancy_sweep(x, layer)
+    if not any(k.get("on_layer_path") for k in kernels.values()):
+        # no stage entry points on this layer's path (packed-tile sequence): per-kernel times from the profiler
+        res["traced_kernels"] = trace_layer_kernels(layer, x, B, N, C, S)
     res.update({"kernels": kernels, "roofline": roofline, "H": H})
     del layer, x
     torch.cuda.empty_cache()
@@ -635,7 +717,8 @@ def main():
     SETTLE_MS = args.settle_ms
     gen = torch.Generator().manual_seed(1234)
     x_cpu = torch.randn(B, N, C, generator=gen)
-    m = measure_layer(B, N, C, S, args.steps, args.warmup, args.kernel_reps, x_cpu=x_cpu, cold=True)
+    m = measure_layer(B, N, C, S, args.steps, args.warmup, args.kernel_reps, x_cpu=x_cpu, cold=True,
+                      occupancy=not args.no_sweep)
     ms_per_step, path, kernels = m["ms_per_step"], m["path"], m["kernels"]
     mpoints = B * N / (ms_per_step * 1e-3) / 1e6
 
@@ -670,6 +753,8 @@ def main():
         "graph_replay": {"ms_per_step": round(m["ms_graph"], 4),
                          "mpoints_per_s": round(B * N / (m["ms_graph"] * 1e-3) / 1e6, 2)},
     }
+    if "occupancy_sweep" in m:
+        out["occupancy_sweep"] = {"kernel": "project_softmax_reduce", "points": B * N, "rows": m["occupancy_sweep"]}
     if not args.no_sweep:
         # cfg3's slice sweep: the same layer and points at every slice count (the headline count taken from above)
         sweep = []
@@ -681,8 +766,8 @@ def main():
                              for k, v in mk["kernels"].items() if v.get("on_layer_path")}}
             e.update(layer_fracs(B * N, C, s_k, mk["ms_per_step"]))
             if not e["kernels"]:
-                e["layer_kernels"] = ("packed-tile sequence: project_rows, slice_softmax_reduce, combine + slice attention, "
-                                      "deslice_recompute, linear_rows (slice weights recomputed, never stored)")
+                # packed-tile sequence (slice weights recomputed, never stored): per-kernel times from the profiler
+                e["kernels"] = mk.get("traced_kernels", {})
             sweep.append(e)
         out["slice_sweep"] = sweep
     if not args.no_models:
@@ -693,7 +778,8 @@ def main():
         out["layer_c512_s128"] = dict({"points": N, "hidden": 512, "heads": 16, "slice_num": 128,
                                        "ms_per_step": round(m5["ms_per_step"], 4),
                                        "mpoints_per_s": round(N / (m5["ms_per_step"] * 1e-3) / 1e6, 2),
-                                       "kernel_path": {0: "general", 1: "mfma", 2: "mfma-staged"}[m5["path"]]},
+                                       "kernel_path": {0: "general", 1: "mfma", 2: "mfma-staged"}[m5["path"]],
+                                       "kernels": m5.get("traced_kernels", {})},
                                       **layer_fracs(N, 512, 128, m5["ms_per_step"]))
         out["training_step"] = time_training_step(N, C, S)
         out["variants"] = time_variants(N, C, S)

@@ -63,6 +63,13 @@ extern "C" {
 /* Library version (major*10000 + minor*100 + patch). No reference counterpart. */
 int pa_version(void);
 
+/* Measurement knob, no reference counterpart: the persistent kernels (one workgroup per compute unit walking the
+ * tiles) size their grids by the device's compute-unit count; n > 0 makes them use n workgroups' worth instead, i.e.
+ * run on n compute units with the rest of the chip idle; 0 restores the device's count.  Process-wide; set it before
+ * sizing any workspace (partial-sum counts follow it).  bench.py uses it to show how the shader clock the chip holds
+ * under a kernel depends on how much of the chip that kernel keeps busy. */
+int pa_set_compute_units(int n);
+
 /* 1 when marker ranges are on: the process environment held PA_ROCTX=1 when the library first looked and a roctx
  * library (librocprofiler-sdk-roctx / libroctx64) could be opened at run time; 0 otherwise.  With ranges on, the
  * layer-, block- and MLP-level entry points push a range named after themselves, and the fused layer brackets its

@@ -16,7 +16,7 @@ LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libphysattn
 PA_F32, PA_BF16, PA_BF16_W8 = 0, 1, 2
 
 EXPORTED = [
-    "pa_version", "pa_status_string", "pa_workspace_bytes", "pa_query_path", "pa_project_inputs",
+    "pa_version", "pa_set_compute_units", "pa_status_string", "pa_workspace_bytes", "pa_query_path", "pa_project_inputs",
     "pa_slice_softmax", "pa_reduce_partial_count", "pa_slice_reduce", "pa_slice_attention",
     "pa_deslice_project", "pa_layer_forward", "pa_mfma_buffer_bytes", "pa_mfma_pack_params",
     "pa_mfma_project_softmax", "pa_mfma_slice_reduce", "pa_mfma_project_softmax_reduce", "pa_mfma_partial_groups",
@@ -99,6 +99,8 @@ def load() -> ctypes.CDLL:
     ps, pp, pt = POINTER(PaShape), POINTER(PaParams), POINTER(PaBlockTail)
     lib.pa_version.restype = c_int
     lib.pa_version.argtypes = []
+    lib.pa_set_compute_units.restype = c_int
+    lib.pa_set_compute_units.argtypes = [c_int]
     lib.pa_markers_enabled.restype = c_int
     lib.pa_markers_enabled.argtypes = []
     lib.pa_status_string.restype = c_char_p

@@ -5,6 +5,8 @@
 #include "pa_common.h"
 #include "pa_host.h"
 
+#include <atomic>
+
 namespace {
 
 using pa::aligned16;
@@ -262,7 +264,11 @@ int64_t body_bytes(int dtype, const pa_shape &s) {
   }
 }
 
+static std::atomic<int> g_compute_units_limit{0};
+
 int compute_units() {
+  const int limit = g_compute_units_limit.load(std::memory_order_relaxed);
+  if (limit > 0) return limit;
   static int cached[64];  // per device; 0 = not yet asked (racing first calls write the same value)
   int dev = 0, n = 0;
   if (hipGetDevice(&dev) != hipSuccess) return 256;
@@ -340,6 +346,12 @@ int mfma_layer(const pa_shape &s, const pa_params &p, const void *blob, const vo
 extern "C" {
 
 int pa_version(void) { return 110; }
+
+int pa_set_compute_units(int n) {
+  if (n < 0 || n > 4096) return PA_ERR_DIMS;
+  g_compute_units_limit.store(n, std::memory_order_relaxed);
+  return PA_OK;
+}
 
 int pa_markers_enabled(void) { return markers().push != nullptr ? 1 : 0; }
 
