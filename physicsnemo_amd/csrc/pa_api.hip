@@ -1004,11 +1004,14 @@ int pa_mlp_forward(int dtype, int64_t rows, int64_t C, int64_t F, const pa_mlp_p
 }
 
 int pa_preprocess_query(int dtype, int64_t rows, int64_t c_in, int64_t F, int64_t C) {
-  return pa::f32rows::premlp_supported(dtype, rows, c_in, F, C) ? 1 : 0;
+  if (rows <= 0 || rows > PA_MAX_ROWS || c_in <= 0 || F <= 0 || C <= 0) return 0;
+  return pa::f32rows::premlp_supported(dtype, rows, c_in, F, C) || pa::mlp::premlp_supported(dtype, rows, c_in, F, C) ? 1 : 0;
 }
 
 int64_t pa_preprocess_workspace_bytes(int dtype, int64_t rows, int64_t c_in, int64_t F, int64_t C) {
   if (rows <= 0 || c_in <= 0 || F <= 0 || C <= 0) return PA_ERR_DIMS;
+  if (rows > PA_MAX_ROWS) return PA_ERR_UNSUPPORTED;
+  if (pa::mlp::premlp_supported(dtype, rows, c_in, F, C)) return round_up(pa::mlp::premlp_blob_bytes(F, C), 256);
   if (!pa::f32rows::premlp_supported(dtype, rows, c_in, F, C)) return PA_ERR_UNSUPPORTED;
   return round_up(pa::f32rows::premlp_blob_bytes(F), 256);
 }
@@ -1018,6 +1021,29 @@ int pa_preprocess_forward(int dtype, int64_t rows, int64_t c_in, int64_t F, int6
                           void *stream) {
   Range entry("pa_preprocess_forward");
   if (rows <= 0 || c_in <= 0 || F <= 0 || C <= 0) return PA_ERR_DIMS;
+  if (rows > PA_MAX_ROWS) return PA_ERR_UNSUPPORTED;
+  if (pa::mlp::premlp_supported(dtype, rows, c_in, F, C)) {  // bf16: hidden layer on chip, MFMA row kernel
+    if (!p || !p->w1 || !p->b1 || !p->w2 || !p->b2 || !u || !y || !workspace) return PA_ERR_NULL;
+    if (!aligned16(p->w2) || !aligned16(y) || !aligned16(workspace)) return PA_ERR_ALIGN;
+    int rc = check_tail(tail);
+    if (rc) return rc;
+    if (workspace_bytes < pa::mlp::premlp_blob_bytes(F, C)) return PA_ERR_WORKSPACE;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    // the LayerNorm rides in the kernel's epilogue when a wave holds whole rows (C = 256) and nothing is added first
+    const bool ln_inside = tail && tail->ln_out && !tail->residual && C == 256;
+    rc = pa::mlp::premlp(rows, c_in, F, C, p->w1, p->b1, p->w2, p->b2, u, y, ln_inside ? tail->ln_gamma : nullptr,
+                         ln_inside ? tail->ln_beta : nullptr, ln_inside ? tail->ln_eps : 0.f,
+                         ln_inside ? tail->ln_out : nullptr, workspace, compute_units(), st);
+    if (rc || ln_inside || !tail_active(tail)) return rc;
+    pa_shape s{};
+    s.B = 1;
+    s.N = rows;
+    s.C = C;
+    s.H = 1;
+    s.D = 1;
+    s.S = 1;
+    return pa::general::residual_ln(dtype, s, y, *tail, st);
+  }
   if (!pa::f32rows::premlp_supported(dtype, rows, c_in, F, C)) return PA_ERR_UNSUPPORTED;
   if (!p || !p->w1 || !p->b1 || !p->w2 || !p->b2 || !u || !y || !workspace) return PA_ERR_NULL;
   if (!aligned16(p->w2) || !aligned16(y) || !aligned16(workspace)) return PA_ERR_ALIGN;

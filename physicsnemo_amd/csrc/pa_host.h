@@ -248,6 +248,12 @@ int pack(int64_t C, int64_t F, const void *w1, const float *w1_scale, const void
          hipStream_t st);
 int forward(int64_t rows, int64_t C, int64_t F, const void *blob, const float *b1, const float *b2, const void *u,
             void *y, const pa_block_tail *tail, int num_cu, hipStream_t st);
+// the preprocess MLP (c_in <= 16 inputs -> F -> C in {256, 512}) with the hidden layer kept on chip; bf16 rows and weights
+bool premlp_supported(int dtype, int64_t rows, int64_t c_in, int64_t F, int64_t C);
+int64_t premlp_blob_bytes(int64_t F, int64_t C);
+int premlp(int64_t rows, int64_t c_in, int64_t F, int64_t C, const void *w1, const float *b1, const void *w2,
+           const float *b2, const void *u, void *y, const float *ln_gamma, const float *ln_beta, float ln_eps,
+           void *ln_out, void *blob, int num_cu, hipStream_t st);
 // y = W x + bias [+ residual] [-> LayerNorm] for bf16 rows, W (C x C) bf16 row-major; blob: linear_blob_bytes(C) of scratch
 bool linear_supported(int dtype, int64_t rows, int64_t C);
 int64_t linear_blob_bytes(int64_t C);

@@ -495,7 +495,7 @@ template <int C, bool HAS_RES, bool HAS_LN, int STG = 16384, class AfterStaging>
 __device__ __forceinline__ void finish_rows(const f32x16 (&yacc)[C / 32], uint32_t *stg, int i, int g, int64_t row0,
                                             int64_t M, const uint16_t *__restrict__ residual, uint16_t *__restrict__ y,
                                             uint16_t *__restrict__ ln_out, const float *gams, const float *bets,
-                                            float ln_eps, AfterStaging &&after_staging) {
+                                            float ln_eps, AfterStaging &&after_staging, int64_t ld = C) {
   constexpr int CT = C / 32;
   constexpr int G4 = C / 4;             // 8-byte granules (4 channels) per staged row
   constexpr int RPR = STG / (2 * C);  // rows staged per round
@@ -528,7 +528,7 @@ __device__ __forceinline__ void finish_rows(const f32x16 (&yacc)[C / 32], uint32
         int64_t r = row0 + rd * RPR + 2 * rr + hl;
         if (r >= M) r = M > 0 ? M - 1 : 0;  // M = 0: a wave without rows (nothing is stored)
 #pragma unroll
-        for (int v = 0; v < NV; ++v) rsd[rr][v] = load_streaming(reinterpret_cast<const rowv *>(residual + r * C + 256 * v + 8 * il));
+        for (int v = 0; v < NV; ++v) rsd[rr][v] = load_streaming(reinterpret_cast<const rowv *>(residual + r * ld + 256 * v + 8 * il));
       }
     };
     static_for<PF>(load_residual);
@@ -570,7 +570,7 @@ __device__ __forceinline__ void finish_rows(const f32x16 (&yacc)[C / 32], uint32
           val[8 * v + 2 * w] = __uint_as_float(ob[w] << 16);
           val[8 * v + 2 * w + 1] = __uint_as_float(ob[w] & 0xffff0000u);
         }
-        if (ok) store_streaming(reinterpret_cast<rowv *>(y + r * C + 256 * v + 8 * il), ob);
+        if (ok) store_streaming(reinterpret_cast<rowv *>(y + r * ld + 256 * v + 8 * il), ob);
       }
       if constexpr (HAS_LN) {
         float s1 = 0.f;
@@ -596,7 +596,7 @@ __device__ __forceinline__ void finish_rows(const f32x16 (&yacc)[C / 32], uint32
             const float c0 = w < 2 ? ba[2 * w] : bb[2 * w - 4], c1 = w < 2 ? ba[2 * w + 1] : bb[2 * w - 3];
             lb[w] = pack2(fmaf(fmaf(val[8 * v + 2 * w], rstd, shift), g0, c0), fmaf(fmaf(val[8 * v + 2 * w + 1], rstd, shift), g1, c1));
           }
-          if (ok) store_streaming(reinterpret_cast<rowv *>(ln_out + r * C + 256 * v + 8 * il), lb);
+          if (ok) store_streaming(reinterpret_cast<rowv *>(ln_out + r * ld + 256 * v + 8 * il), lb);
         }
       }
       __builtin_amdgcn_sched_barrier(0);
@@ -936,6 +936,179 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void mlp_rows2_kernel(
     }
     finish_rows<C, HAS_RES, HAS_LN, STG>(yacc, stg, i, g, row0, M, residual, y, ln_out, gams, bets,
                                          ln_eps, [&]() { load_rows(mb + gridDim.x < nblocks ? mb + gridDim.x : mb, ub); });
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // nothing may still be landing in LDS when the workgroup ends
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// premlp_rows_kernel: the model's preprocess MLP, y = W2 . gelu(W1 . u + b1) + b2 [-> LayerNorm(y)], for rows with a
+// handful of input features (c_in <= 16: coordinates, normals, fields) and 256 output channels per launch
+// (transolver.py:518-525, and the first block's ln_1 at :300).  The hidden layer never reaches memory.
+// Workgroup = 8 waves, two per SIMD, a block = 256 rows; a wave owns 32 rows:
+//   u^T as ONE B operand (k = the c_in inputs, zero beyond), W1 whole in LDS as F / 32 A fragments, so a hidden chunk of
+//   32 units costs one MFMA: h(c)^T = W1[chunk c] . u^T + b1;
+//   y^T (256 channels x 32 rows, 128 registers) += W2[:, chunk c] . gelu(h(c))^T: 16 MFMAs per chunk, W2 streaming
+//   through LDS in slots of 16 fragments (16 KB), two buffers, one barrier per slot.
+// Software pipeline over the chunks, per iteration c: the first product of chunk c + 1 (its result is read an
+// iteration later), the 16 MFMAs of the second product of chunk c - 1, and behind each of them one of the 16
+// activations of chunk c (erf-accurate GELU, two evaluations in flight), which become the two B operands of the next
+// iteration.  The activations (16 per 17 MFMAs) make the loop vector-bound; it still runs several times faster than
+// two GEMM launches with the hidden layer in memory between them.
+// blob (premlp_pack_kernel): W1 fragments [F / 32][lane]: W1[32 n + i][8 g + j] (zero beyond c_in); then per column
+// block of 256 outputs the slots [F / 32][t = kk 8 + ct][lane]: W2[col0 + 32 ct + i][32 c + kperm(kk, g, j)].
+// ---------------------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void premlp_pack_kernel(const uint16_t *__restrict__ w1, const uint16_t *__restrict__ w2,
+                                                          u32x4 *__restrict__ blob, int c_in, int F, int C) {
+  const int NCH = F / 32;
+  const int64_t n1 = (int64_t)NCH * 64, total = n1 + (int64_t)(C / 256) * NCH * 16 * 64;
+  for (int64_t u = (int64_t)blockIdx.x * 256 + threadIdx.x; u < total; u += (int64_t)gridDim.x * 256) {
+    const int lane = (int)(u & 63), i = lane & 31, g = lane >> 5;
+    uint16_t e[8];
+    if (u < n1) {
+      const int n = (int)(u >> 6);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) e[j] = 8 * g + j < c_in ? w1[(int64_t)(32 * n + i) * c_in + 8 * g + j] : (uint16_t)0;
+    } else {
+      int64_t q = (u - n1) >> 6;
+      const int t = (int)(q & 15);
+      q >>= 4;
+      const int c = (int)(q % NCH), blk = (int)(q / NCH), kk = t >> 3, ct = t & 7;
+      const uint16_t *src = w2 + (int64_t)(256 * blk + 32 * ct + i) * F + 32 * c;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) e[j] = src[kperm(kk, g, j)];
+    }
+    u32x4 v;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) v[j] = (uint32_t)e[2 * j] | ((uint32_t)e[2 * j + 1] << 16);
+    blob[u] = v;
+  }
+}
+
+// two direct global -> LDS loads of 64 x 16 bytes each (2 KB), as load_4k_to_lds
+__device__ __forceinline__ void load_2k_to_lds(const void *sbase, unsigned lane16, unsigned lds) {
+  asm volatile(
+      "s_mov_b32 m0, %2\n\t"
+      "s_nop 0\n\t"
+      "global_load_lds_dwordx4 %1, %0\n\t"
+      "global_load_lds_dwordx4 %1, %0 offset:1024" ::"s"(sbase),
+      "v"(lane16), "s"(lds)
+      : "memory");
+}
+
+template <bool HAS_LN>
+__global__ __launch_bounds__(512, 1) void premlp_rows_kernel(
+    const u32x4 *__restrict__ blob, const float *__restrict__ b1, const float *__restrict__ b2,
+    const uint16_t *__restrict__ u, int c_in, uint16_t *__restrict__ y, int64_t ld, const float *__restrict__ ln_gamma,
+    const float *__restrict__ ln_beta, float ln_eps, uint16_t *__restrict__ ln_out, int64_t M, int F, int col_block,
+    int64_t nblocks) {
+  constexpr int C = 256, CT = 8, NF = 2 * CT, SU = NF * 64;  // a slot: 16 fragments
+  constexpr int WU = SU / 8;                                  // units of a slot fetched by each wave (2 KB)
+  constexpr int STG = 8192, kRows = 256;
+  extern __shared__ u32x4 smem[];
+  const int NCH = F / 32;
+  u32x4 *w1s = smem;                    // NCH * 64
+  u32x4 *wbuf = w1s + NCH * 64;         // 2 * SU
+  uint32_t *stage = reinterpret_cast<uint32_t *>(wbuf + 2 * SU);  // 8 waves x STG bytes
+  float *b1s = reinterpret_cast<float *>(stage + 8 * STG / 4);
+  float *b2s = b1s + F;
+  float *gams = b2s + C, *bets = gams + C;
+  const int tid = threadIdx.x, lane = tid & 63, i = lane & 31, g = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const u32x4 *w2blob = blob + (int64_t)NCH * 64 + (int64_t)col_block * NCH * SU;
+  for (int k = tid; k < NCH * 64; k += 512) w1s[k] = blob[k];
+  for (int k = tid; k < F; k += 512) b1s[k] = b1[k];
+  for (int k = tid; k < C; k += 512) {
+    b2s[k] = b2[256 * col_block + k];
+    gams[k] = HAS_LN ? ln_gamma[k] : 1.f;
+    bets[k] = HAS_LN ? ln_beta[k] : 0.f;
+  }
+  auto fetch = [&](int64_t gs, int c) {  // this wave's share of slot c into buffer gs & 1
+    const u32x4 *src = w2blob + (int64_t)c * SU + wave * WU;
+    const unsigned dst = (unsigned)(uintptr_t)(wbuf + (gs & 1) * SU + wave * WU);
+    load_2k_to_lds(src, lane * 16, dst);
+  };
+  // the wave's 32 rows as one B operand: lane (i, g) holds inputs 8 g .. 8 g + 7 of row i (zero beyond c_in)
+  auto load_rows = [&](int64_t mb) {
+    int64_t r = mb * kRows + wave * 32 + i;
+    if (r >= M) r = M - 1;
+    const uint16_t *src = u + r * c_in + 8 * g;
+    uint16_t e[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) e[j] = 8 * g + j < c_in ? src[j] : (uint16_t)0;
+    u32x4 v;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) v[j] = (uint32_t)e[2 * j] | ((uint32_t)e[2 * j + 1] << 16);
+    return v;
+  };
+  int64_t gs = 0;
+  if ((int64_t)blockIdx.x < nblocks) fetch(0, 0);
+  __syncthreads();  // W1 and the biases are in LDS
+  for (int64_t mb = blockIdx.x; mb < nblocks; mb += gridDim.x) {
+    const int64_t row0 = mb * kRows + wave * 32;
+    const u32x4 ub = load_rows(mb);
+    f32x16 yacc[CT];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) yacc[ct][r] = b2s[32 * ct + rowmap(r, g)];
+    // h of the chunk being activated; the operands of the chunk before (zero before the first: its slot adds nothing)
+    f32x16 hcur;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) hcur[r] = b1s[rowmap(r, g)];
+    hcur = mma(w1s[lane], ub, hcur);
+    u32x4 gop[2] = {u32x4{0, 0, 0, 0}, u32x4{0, 0, 0, 0}};
+    for (int c = 0; c <= NCH; ++c, ++gs) {
+      // slot gs has landed (every wave waits for its own share, then all meet) and the other buffer is free.  The
+      // first slot of a later block was waited for before the epilogue of the block before it.
+      if (c > 0 || gs == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      __syncthreads();
+      // iteration c + 1 reads chunk c; the last iteration fetches the first slot of the next block (chunk 0, twice:
+      // iteration 0 multiplies it by the zero operands)
+      fetch(gs + 1, c < NCH ? c : 0);
+      const u32x4 *wb = wbuf + (gs & 1) * SU + lane;
+      // first product of chunk c + 1 (clamped past the end: computed, never used)
+      const int cn = c + 1 < NCH ? c + 1 : NCH - 1;
+      f32x16 hnext;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) hnext[r] = b1s[32 * cn + rowmap(r, g)];
+      hnext = mma(w1s[cn * 64 + lane], ub, hnext);
+      u32x4 gnew[2];
+      float ex = 0.f, ee = 0.f, feven = 0.f;  // evaluation in flight: argument and exp2 term; even result of a pair
+      constexpr int RING = 3, AHEAD = 2;
+      u32x4 fr[RING];
+      static_for<AHEAD>([&](auto q) { fr[decltype(q)::value] = wb[decltype(q)::value * 64]; });
+      __builtin_amdgcn_sched_barrier(0);
+      static_for<NF>([&](auto t_) {
+        constexpr int t = decltype(t_)::value, kk = t / CT, ct = t % CT;
+        if constexpr (t + AHEAD < NF) fr[(t + AHEAD) % RING] = wb[(t + AHEAD) * 64];
+        yacc[ct] = mma(fr[t % RING], gop[kk], yacc[ct]);
+        __builtin_amdgcn_sched_barrier(0);
+        // the end of activation t - 1 and the start of activation t: two independent chains behind the MFMA
+        const float dx = ex, de = ee;
+        {
+          const float x = hcur[t];
+          ex = x;
+          const float x2 = fminf(x * x, 81.f);
+          float q = fmaf(-3.51902394e-04f * -2.f * kLog2e, x2, 3.70080200e-02f * -2.f * kLog2e);
+          q = fmaf(q, x2, 7.97505275e-01f * -2.f * kLog2e);
+          ee = __builtin_amdgcn_exp2f(x * q);
+        }
+        if constexpr (t > 0) {
+          constexpr int e = t - 1, j = e % 8;
+          const float v = dx * __builtin_amdgcn_rcpf(1.f + de);
+          if constexpr (j % 2 == 0) feven = v;
+          else gnew[e / 8][j / 2] = pack2(feven, v);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      });
+      gnew[1][3] = pack2(feven, ex * __builtin_amdgcn_rcpf(1.f + ee));
+      gop[0] = gnew[0];
+      gop[1] = gnew[1];
+      hcur = hnext;
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's share of the next block's first slot has landed
+    uint32_t *stg = stage + wave * (STG / 4);
+    finish_rows<C, false, HAS_LN, STG>(yacc, stg, i, g, row0, M, nullptr, y, ln_out, gams, bets, ln_eps, [] {}, ld);
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // nothing may still be landing in LDS when the workgroup ends
 }
@@ -1416,6 +1589,55 @@ int project_packed(int64_t B, int64_t N, int64_t C, const void *w_x, const float
                        N, (int)tpb, ntiles, nblocks);
   e = hipGetLastError();
   return e == hipSuccess ? PA_OK : (int)e;
+}
+
+// ---- the preprocess MLP (few inputs -> F -> C) on premlp_rows_kernel ---------------------------------------------
+static size_t premlp_lds(int64_t F) {
+  return (size_t)((F / 32) * 64 + 2 * 16 * 64) * 16 + (size_t)8 * 8192 + (size_t)(F + 3 * 256) * 4;
+}
+
+bool premlp_supported(int dtype, int64_t rows, int64_t c_in, int64_t F, int64_t C) {
+  if (dtype != PA_BF16 || rows <= 0 || c_in < 1 || c_in > 16 || F < 32 || F % 32 != 0 || F > 4096) return false;
+  if (C != 256 && C != 512) return false;
+  return premlp_lds(F) <= (size_t)kMaxLdsBytes;
+}
+
+int64_t premlp_blob_bytes(int64_t F, int64_t C) { return ((F / 32) * 64 + (C / 256) * (F / 32) * 16 * 64) * (int64_t)16; }
+
+// y (rows, C) = W2 gelu(W1 u + b1) + b2 for u (rows, c_in); with ln_out (C = 256 only): ln_out = LayerNorm(y) too.
+// C = 512 runs as two column blocks of 256 outputs (the hidden layer is evaluated once per block).
+int premlp(int64_t rows, int64_t c_in, int64_t F, int64_t C, const void *w1, const float *b1, const void *w2,
+           const float *b2, const void *u, void *y, const float *ln_gamma, const float *ln_beta, float ln_eps,
+           void *ln_out, void *blob, int num_cu, hipStream_t st) {
+  if (!premlp_supported(PA_BF16, rows, c_in, F, C)) return PA_ERR_UNSUPPORTED;
+  if (ln_out && C != 256) return PA_ERR_UNSUPPORTED;
+  const int64_t total = premlp_blob_bytes(F, C) / 16;
+  hipLaunchKernelGGL(rows::premlp_pack_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st,
+                     static_cast<const uint16_t *>(w1), static_cast<const uint16_t *>(w2), static_cast<u32x4 *>(blob),
+                     (int)c_in, (int)F, (int)C);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return (int)e;
+  const size_t lds = premlp_lds(F);
+  const void *kernel = ln_out ? reinterpret_cast<const void *>(rows::premlp_rows_kernel<true>)
+                              : reinterpret_cast<const void *>(rows::premlp_rows_kernel<false>);
+  e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  if (e != hipSuccess) return (int)e;
+  const int64_t nblocks = (rows + 255) / 256;
+  const int64_t grid = nblocks < num_cu ? nblocks : num_cu;
+  for (int blk = 0; blk < (int)(C / 256); ++blk) {
+    uint16_t *yb = static_cast<uint16_t *>(y) + 256 * blk;
+    if (ln_out)
+      hipLaunchKernelGGL(rows::premlp_rows_kernel<true>, dim3((unsigned)grid), dim3(512), lds, st,
+                         static_cast<const u32x4 *>(blob), b1, b2, static_cast<const uint16_t *>(u), (int)c_in, yb, C,
+                         ln_gamma, ln_beta, ln_eps, static_cast<uint16_t *>(ln_out), rows, (int)F, blk, nblocks);
+    else
+      hipLaunchKernelGGL(rows::premlp_rows_kernel<false>, dim3((unsigned)grid), dim3(512), lds, st,
+                         static_cast<const u32x4 *>(blob), b1, b2, static_cast<const uint16_t *>(u), (int)c_in, yb, C,
+                         nullptr, nullptr, 0.f, nullptr, rows, (int)F, blk, nblocks);
+    e = hipGetLastError();
+    if (e != hipSuccess) return (int)e;
+  }
+  return PA_OK;
 }
 
 int forward(int64_t rows, int64_t C, int64_t F, const void *blob, const float *b1, const float *b2, const void *u,

@@ -364,10 +364,11 @@ def block_forward(x, fx_in, params, dims: LayerDims, ln2_weight, ln2_bias, ln2_e
 
 
 def preprocess_supported(dtype: torch.dtype, rows: int, c_in: int, F: int, C: int) -> bool:
-    """True if `preprocess_forward` serves the shape (float32, C = 128, up to 8 input features, F a multiple of 128)."""
-    if dtype != torch.float32:
+    """True if `preprocess_forward` serves the shape: float32 with C = 128, up to 8 input features and F a multiple of
+    128, or bfloat16 with C in {256, 512}, up to 16 input features and F a multiple of 32."""
+    if dtype not in (torch.float32, torch.bfloat16):
         return False
-    return bool(_lib.load().pa_preprocess_query(_lib.PA_F32, rows, c_in, F, C))
+    return bool(_lib.load().pa_preprocess_query(_lib.dtype_code(dtype), rows, c_in, F, C))
 
 
 def preprocess_forward(u, w1, b1, w2, b2, ln_weight=None, ln_bias=None, ln_eps=1e-5):

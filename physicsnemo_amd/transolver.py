@@ -360,6 +360,21 @@ class Transolver(nn.Module):
             cache[id(lin)] = hit
         return PF.linear(x, hit[1], hit[2], gelu=gelu)
 
+    def _preprocess_params(self, dtype, device):
+        """The preprocess Mlp's weights in the activation dtype and its biases in float32, cached until one changes."""
+        lin1, lin2 = self.preprocess.layers[0], self.preprocess.layers[2]
+        named = (lin1.weight, lin1.bias, lin2.weight, lin2.bias)
+        stamp = (dtype, device) + tuple((t.data_ptr(), t._version, t.dtype) for t in named)
+        cache = self.__dict__.setdefault("_preprocess_cache", {})
+        if cache.get("stamp") != stamp:
+            with torch.no_grad():
+                cache["params"] = (lin1.weight.detach().to(device=device, dtype=dtype).contiguous().clone(),
+                                   lin1.bias.detach().to(device=device, dtype=torch.float32).contiguous().clone(),
+                                   lin2.weight.detach().to(device=device, dtype=dtype).contiguous().clone(),
+                                   lin2.bias.detach().to(device=device, dtype=torch.float32).contiguous().clone())
+            cache["stamp"] = stamp
+        return cache["params"]
+
     def use_fp8_weights(self, enabled: bool = True):
         """Every block's large weights as fp8-e4m3 with per-output-channel scales (`TransolverBlock.use_fp8_weights`);
         the preprocess Mlp, the LayerNorms, the slice / qkv projections and the output head stay in higher precision."""
@@ -424,16 +439,15 @@ class Transolver(nn.Module):
                 fx = fx.to(torch.get_autocast_dtype("cuda"))
             lin1, lin2 = self.preprocess.layers[0], self.preprocess.layers[2]
             rows = fx.numel() // fx.shape[-1]
-            if (time is None and len(self.preprocess.layers) == 3 and fx.dtype == torch.float32 and
+            if (time is None and len(self.preprocess.layers) == 3 and
                     PF.preprocess_supported(fx.dtype, rows, lin1.in_features, lin1.out_features, lin2.out_features)):
-                # float32 at hidden 128: both Linears, the GELU and the first block's LayerNorm in one launch
+                # both Linears, the GELU and the first block's LayerNorm in one library call with the hidden layer kept
+                # on chip (float32 at hidden 128; bfloat16 at hidden 256 / 512)
                 ln = self.blocks[0].ln_1
-                f32 = dict(device=fx.device, dtype=torch.float32)
+                w1, b1, w2, b2 = self._preprocess_params(fx.dtype, fx.device)
                 fx, normed = PF.preprocess_forward(
-                    fx.contiguous(), lin1.weight.detach().to(**f32).contiguous(), lin1.bias.detach().to(**f32).contiguous(),
-                    lin2.weight.detach().to(**f32).contiguous(), lin2.bias.detach().to(**f32).contiguous(),
-                    ln_weight=ln.weight.detach().float().contiguous(), ln_bias=ln.bias.detach().float().contiguous(),
-                    ln_eps=ln.eps)
+                    fx.contiguous(), w1, b1, w2, b2, ln_weight=ln.weight.detach().float().contiguous(),
+                    ln_bias=ln.bias.detach().float().contiguous(), ln_eps=ln.eps)
                 first_ln_done = True
             elif lin2.in_features <= 512:  # the weights-stationary row kernel holds up to 512 input features
                 fx = self._library_linear(self._library_linear(fx.contiguous(), lin1, gelu=True), lin2)

@@ -169,6 +169,42 @@ def test_preprocess_mlp_fp32_matches_oracle(rows_shape, c_in, Fh):
     assert not PF.preprocess_supported(torch.float32, 100, 3, 256, 256)
 
 
+@pytest.mark.parametrize("rows_shape,c_in,Fh,C", [
+    ((8, 32768), 5, 512, 256), ((1, 20000), 7, 512, 256), ((1, 8192), 7, 1024, 512), ((2, 333), 1, 32, 256),
+    ((1, 1), 16, 64, 512), ((1, 70001), 9, 1024, 512), ((3, 257), 3, 1728, 256),  # the widest hidden layer whose first Linear fits LDS
+])
+def test_preprocess_mlp_bf16_matches_oracle(rows_shape, c_in, Fh, C):
+    # the model's preprocess Mlp at the bf16 configurations (cfg2 / cfg4: 5 or 7 inputs -> 512 -> 256; cfg5: 7 -> 1024
+    # -> 512) with the hidden layer kept on chip, and the first LayerNorm (in the kernel's epilogue at 256 channels)
+    announce("preprocess mlp bf16", rows_shape, c_in, Fh, C)
+    torch.manual_seed(5)
+    ref = to.OracleMlp(c_in, Fh, C).eval()
+    with torch.no_grad():
+        for lin in (ref.layers[0], ref.layers[2]):  # bf16-representable weights: both sides compute with the same numbers
+            lin.weight.copy_(lin.weight.bfloat16().float())
+    u = torch.randn(*rows_shape, c_in).bfloat16()
+    gamma, beta = torch.rand(C) + 0.5, torch.randn(C) * 0.1
+    dev = torch.device("cuda:0")
+    args = dict(u=u.to(dev), w1=ref.layers[0].weight.detach().bfloat16().to(dev).contiguous(),
+                b1=ref.layers[0].bias.detach().to(dev), w2=ref.layers[2].weight.detach().bfloat16().to(dev).contiguous(),
+                b2=ref.layers[2].bias.detach().to(dev))
+    assert PF.preprocess_supported(torch.bfloat16, u.numel() // c_in, c_in, Fh, C)
+    with torch.no_grad():
+        want = ref(u.float())
+        want_ln = F.layer_norm(want, (C,), gamma, beta, 1e-5)
+        y = PF.preprocess_forward(**args)
+        y2, ln2 = PF.preprocess_forward(**args, ln_weight=gamma.to(dev), ln_bias=beta.to(dev))
+    assert y.shape == (*rows_shape, C) and y.dtype == torch.bfloat16
+    assert torch.isfinite(y.float()).all()
+    assert_rel_l2(y, want, "bf16 preprocess mlp output", report=True)
+    assert_rel_l2(ln2, want_ln, "LayerNorm(bf16 preprocess mlp)")
+    assert torch.equal(y2, y)
+    assert not PF.preprocess_supported(torch.bfloat16, 100, 17, 512, 256)
+    assert not PF.preprocess_supported(torch.bfloat16, 100, 7, 500, 256)
+    assert not PF.preprocess_supported(torch.bfloat16, 100, 7, 1760, 256)  # W1 no longer fits beside the stream
+    assert not PF.preprocess_supported(torch.bfloat16, 100, 7, 512, 128)
+
+
 @pytest.mark.parametrize("C,Fh", [(128, 512), (256, 1024), (512, 2048)])
 def test_mlp_repack_reads_e4m3_weights(C, Fh):
     """pa_mlp_pack_e4m3 (the repacking kernel fed e4m3 bytes + per-row scales) writes the very fragments pa_mlp_pack
