@@ -221,7 +221,7 @@ def test_mlp_repack_reads_e4m3_weights(C, Fh):
     q1p, s1p = PF.quantize_e4m3_per_channel(w1, search=0)
     err = lambda d, w: float((d - w).norm() / w.norm())
     assert err(d1, w1) <= err(PF.dequantize_e4m3_per_channel(q1p, s1p), w1) + 1e-9
-    assert err(d1, w1) < 2.5e-2 and err(d2, w2) < 2.5e-2  # max|row| / 448: 2.55e-2
+    assert err(d1, w1) < 2.6e-2 and err(d2, w2) < 2.6e-2  # 3 mantissa bits: 2.2e-2 .. 2.55e-2 whatever the scale
     want = PF.mlp_pack(d1.bfloat16().contiguous(), d2.bfloat16().contiguous())
     got = PF.mlp_pack_e4m3(q1, s1, q2, s2)
     assert torch.equal(got, want)
