@@ -465,8 +465,8 @@ typedef struct pa_mlp_params {
   const float *b2;
 } pa_mlp_params;
 
-/* 1 if pa_mlp_forward serves (dtype, rows, C, F) [bf16, C in {128, 256, 512}, F a multiple of 64 up to 8192 / 7424 /
- * 6656 for the three widths (what the kernel's LDS holds)], else 0. */
+/* 1 if pa_mlp_forward serves (dtype, rows, C, F) [bf16, C in {128, 256, 512}, F a multiple of 64 up to 8192 / 6912 /
+ * 5632 for the three widths (what the kernel's LDS holds)], else 0. */
 int pa_mlp_query(int dtype, int64_t rows, int64_t C, int64_t F);
 /* Bytes of workspace pa_mlp_forward needs (the repacked weights), or a negative error code. */
 int64_t pa_mlp_workspace_bytes(int dtype, int64_t rows, int64_t C, int64_t F);
@@ -483,6 +483,20 @@ int pa_mlp_forward(int dtype, int64_t rows, int64_t C, int64_t F, const pa_mlp_p
 int pa_mlp_pack(int dtype, int64_t C, int64_t F, const pa_mlp_params *p, void *packed, int64_t packed_bytes, void *stream);
 int pa_mlp_forward_packed(int dtype, int64_t rows, int64_t C, int64_t F, const void *packed, const float *b1,
                           const float *b2, const void *u, void *y, const pa_block_tail *tail, void *stream);
+/* pa_mlp_forward_packed for rows that still lack the LayerNorm in front of the Mlp: the kernel applies
+ * LayerNorm(in_ln) to the rows of u as it turns them into operands, so `ln_mlp1[0]` of TransolverBlock (TR.py:303) costs
+ * no pass over memory and its producer (the attention layer's tail) need not write a normalised copy.  With
+ * tail->residual == u this is TR.py:303 whole: y = u + Mlp(LayerNorm(u)).  bf16, C in {256, 512}
+ * (pa_mlp_input_ln_query() == 1). */
+typedef struct pa_input_ln {
+  const float *gamma; /* (C) */
+  const float *beta;  /* (C) */
+  float eps;
+} pa_input_ln;
+int pa_mlp_input_ln_query(int dtype, int64_t rows, int64_t C, int64_t F);
+int pa_mlp_forward_packed_ln(int dtype, int64_t rows, int64_t C, int64_t F, const void *packed, const float *b1,
+                             const float *b2, const pa_input_ln *in_ln, const void *u, void *y, const pa_block_tail *tail,
+                             void *stream);
 /* pa_mlp_pack for weights held as fp8-e4m3 bytes (layout as PA_BF16_W8: w1 (F,C), w2 (C,F) row-major bytes, 8-byte
  * aligned, one float32 scale per output row): the repacking kernel reads the bytes and scales itself and writes the
  * bf16 operand fragments pa_mlp_forward_packed(PA_BF16, ...) takes, bit-identical to pa_mlp_pack over the weights

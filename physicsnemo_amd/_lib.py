@@ -20,7 +20,7 @@ EXPORTED = [
     "pa_slice_softmax", "pa_reduce_partial_count", "pa_slice_reduce", "pa_slice_attention",
     "pa_deslice_project", "pa_layer_forward", "pa_mfma_buffer_bytes", "pa_mfma_pack_params",
     "pa_mfma_project_softmax", "pa_mfma_slice_reduce", "pa_mfma_project_softmax_reduce", "pa_mfma_partial_groups",
-     "pa_mfma_combine_attention", "pa_mfma_deslice_project", "pa_mlp_query", "pa_mlp_workspace_bytes", "pa_mlp_forward", "pa_mlp_pack", "pa_mlp_pack_e4m3",
+     "pa_mfma_combine_attention", "pa_mfma_deslice_project", "pa_mlp_query", "pa_mlp_workspace_bytes", "pa_mlp_forward", "pa_mlp_pack", "pa_mlp_pack_e4m3", "pa_mlp_input_ln_query", "pa_mlp_forward_packed_ln",
      "pa_mlp_forward_packed",
     "pa_rows_gemm", "pa_slice_weighted_sum", "pa_backward_query", "pa_backward_point_tiles",
     "pa_slice_attention_backward", "pa_slice_softmax_backward", "pa_slice_softmax_plus",
@@ -56,6 +56,10 @@ class PaParams(Structure):
 
 class PaMlpParams(Structure):
     _fields_ = [(n, c_void_p) for n in ("w1", "b1", "w2", "b2")]
+
+
+class PaInputLn(Structure):
+    _fields_ = [("gamma", c_void_p), ("beta", c_void_p), ("eps", c_float)]
 
 
 class PaBlockMlp(Structure):
@@ -151,6 +155,11 @@ def load() -> ctypes.CDLL:
     lib.pa_mlp_workspace_bytes.argtypes = [c_int, c_int64, c_int64, c_int64]
     lib.pa_mlp_pack.restype = c_int
     lib.pa_mlp_pack.argtypes = [c_int, c_int64, c_int64, POINTER(PaMlpParams), c_void_p, c_int64, c_void_p]
+    lib.pa_mlp_input_ln_query.restype = c_int
+    lib.pa_mlp_input_ln_query.argtypes = [c_int, c_int64, c_int64, c_int64]
+    lib.pa_mlp_forward_packed_ln.restype = c_int
+    lib.pa_mlp_forward_packed_ln.argtypes = [c_int, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_void_p,
+                                             POINTER(PaInputLn), c_void_p, c_void_p, POINTER(PaBlockTail), c_void_p]
     lib.pa_mlp_pack_e4m3.restype = c_int
     lib.pa_mlp_pack_e4m3.argtypes = [c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p]
     lib.pa_mlp_forward_packed.restype = c_int

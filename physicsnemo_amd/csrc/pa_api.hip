@@ -978,7 +978,30 @@ int pa_mlp_forward_packed(int dtype, int64_t rows, int64_t C, int64_t F, const v
   if (dtype == PA_F32)
     return pa::f32rows::mlp_forward(rows, F, packed, b1, b2, u, y, tail_active(tail) ? tail : nullptr,
                                     static_cast<hipStream_t>(stream));
-  return pa::mlp::forward(rows, C, F, packed, b1, b2, u, y, tail_active(tail) ? tail : nullptr, compute_units(),
+  return pa::mlp::forward(rows, C, F, packed, b1, b2, u, y, tail_active(tail) ? tail : nullptr, pa::mlp::InputLn{},
+                          compute_units(), static_cast<hipStream_t>(stream));
+}
+
+int pa_mlp_input_ln_query(int dtype, int64_t rows, int64_t C, int64_t F) {
+  if (rows <= 0 || rows > PA_MAX_ROWS || C <= 0 || F <= 0) return 0;
+  return pa::mlp::input_ln_supported(dtype, rows, C, F) ? 1 : 0;
+}
+
+int pa_mlp_forward_packed_ln(int dtype, int64_t rows, int64_t C, int64_t F, const void *packed, const float *b1,
+                             const float *b2, const pa_input_ln *in_ln, const void *u, void *y, const pa_block_tail *tail,
+                             void *stream) {
+  Range entry("pa_mlp_forward_packed_ln");
+  if (rows <= 0 || C <= 0 || F <= 0) return PA_ERR_DIMS;
+  if (rows > PA_MAX_ROWS || !pa::mlp::input_ln_supported(dtype, rows, C, F)) return PA_ERR_UNSUPPORTED;
+  if (!packed || !b1 || !b2 || !in_ln || !in_ln->gamma || !in_ln->beta || !u || !y) return PA_ERR_NULL;
+  if (!aligned16(packed) || !aligned16(u) || !aligned16(y)) return PA_ERR_ALIGN;
+  int rc = check_tail(tail);
+  if (rc) return rc;
+  pa::mlp::InputLn in;
+  in.gamma = in_ln->gamma;
+  in.beta = in_ln->beta;
+  in.eps = in_ln->eps;
+  return pa::mlp::forward(rows, C, F, packed, b1, b2, u, y, tail_active(tail) ? tail : nullptr, in, compute_units(),
                           static_cast<hipStream_t>(stream));
 }
 
@@ -999,8 +1022,8 @@ int pa_mlp_forward(int dtype, int64_t rows, int64_t C, int64_t F, const pa_mlp_p
     return pa::f32rows::mlp_forward(rows, F, workspace, p->b1, p->b2, u, y, tail_active(tail) ? tail : nullptr, st);
   }
   if ((rc = pa::mlp::pack(C, F, p->w1, nullptr, p->w2, nullptr, workspace, st))) return rc;
-  return pa::mlp::forward(rows, C, F, workspace, p->b1, p->b2, u, y, tail_active(tail) ? tail : nullptr, compute_units(),
-                          st);
+  return pa::mlp::forward(rows, C, F, workspace, p->b1, p->b2, u, y, tail_active(tail) ? tail : nullptr,
+                          pa::mlp::InputLn{}, compute_units(), st);
 }
 
 int pa_preprocess_query(int dtype, int64_t rows, int64_t c_in, int64_t F, int64_t C) {

@@ -246,8 +246,14 @@ int64_t blob_bytes(int64_t C, int64_t F);
 // w*_scale: nullptr for bf16 weights; else the weight is fp8-e4m3 bytes with one float32 scale per output row
 int pack(int64_t C, int64_t F, const void *w1, const float *w1_scale, const void *w2, const float *w2_scale, void *blob,
          hipStream_t st);
+// LayerNorm applied to the input rows on their way into the first product (gamma == nullptr: none)
+struct InputLn {
+  const float *gamma = nullptr, *beta = nullptr;
+  float eps = 0.f;
+};
+bool input_ln_supported(int dtype, int64_t rows, int64_t C, int64_t F);
 int forward(int64_t rows, int64_t C, int64_t F, const void *blob, const float *b1, const float *b2, const void *u,
-            void *y, const pa_block_tail *tail, int num_cu, hipStream_t st);
+            void *y, const pa_block_tail *tail, const InputLn &in, int num_cu, hipStream_t st);
 // the preprocess MLP (c_in <= 16 inputs -> F -> C in {256, 512}) with the hidden layer kept on chip; bf16 rows and weights
 bool premlp_supported(int dtype, int64_t rows, int64_t c_in, int64_t F, int64_t C);
 int64_t premlp_blob_bytes(int64_t F, int64_t C);

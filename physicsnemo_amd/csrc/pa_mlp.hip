@@ -487,6 +487,48 @@ __device__ __forceinline__ void mma_in_vgprs(u32x4 a, u32x4 b, f32x16 &acc) {
   asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(acc) : "v"(a), "v"(b));
 }
 
+// LayerNorm of a wave's 32 rows held as B operands (lane (i, g): channels 16 ks + 8 g .. + 7 of row i for every k-step,
+// i.e. half a row; lane ^ 32 holds the other half), in place: the rows a producer left un-normalised become the
+// operands of the first product.  Mean and variance in two passes over the registers, float32, as torch's LayerNorm;
+// gams / bets: weight and bias in LDS.
+template <int C>
+__device__ __forceinline__ void normalize_operand_rows(u32x4 (&ub)[C / 16], const float *gams, const float *bets, float eps,
+                                                       int g) {
+  constexpr int KS = C / 16;
+  typedef float f32x4 __attribute__((ext_vector_type(4)));
+  float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      s0 += __uint_as_float(ub[ks][w] << 16);
+      s1 += __uint_as_float(ub[ks][w] & 0xffff0000u);
+    }
+  const float mean = half_sum(s0 + s1) * (1.f / C);
+  float q0 = 0.f, q1 = 0.f;
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const float d0 = __uint_as_float(ub[ks][w] << 16) - mean, d1 = __uint_as_float(ub[ks][w] & 0xffff0000u) - mean;
+      q0 = fmaf(d0, d0, q0);
+      q1 = fmaf(d1, d1, q1);
+    }
+  const float rstd = rsqrtf(half_sum(q0 + q1) * (1.f / C) + eps), shift = -mean * rstd;
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    const f32x4 ga = *reinterpret_cast<const f32x4 *>(gams + 16 * ks + 8 * g), gb = *reinterpret_cast<const f32x4 *>(gams + 16 * ks + 8 * g + 4);
+    const f32x4 ba = *reinterpret_cast<const f32x4 *>(bets + 16 * ks + 8 * g), bb = *reinterpret_cast<const f32x4 *>(bets + 16 * ks + 8 * g + 4);
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const float g0 = w < 2 ? ga[2 * w] : gb[2 * w - 4], g1 = w < 2 ? ga[2 * w + 1] : gb[2 * w - 3];
+      const float c0 = w < 2 ? ba[2 * w] : bb[2 * w - 4], c1 = w < 2 ? ba[2 * w + 1] : bb[2 * w - 3];
+      const float v0 = __uint_as_float(ub[ks][w] << 16), v1 = __uint_as_float(ub[ks][w] & 0xffff0000u);
+      ub[ks][w] = pack2(fmaf(fmaf(v0, rstd, shift), g0, c0), fmaf(fmaf(v1, rstd, shift), g1, c1));
+    }
+  }
+}
+
 // Epilogue of the row-owning kernels: a wave's y^T (channel 32 ct + rowmap(r, g) of row i, C channels x 32 rows) to
 // row-major bf16 rows, + residual, LayerNorm, full-row stores.  The rows pass through `stg`, the wave's own STG bytes
 // of LDS, RPR = STG / (2 C) rows at a time; after_staging() is called once the last round is staged (the accumulators
@@ -604,12 +646,15 @@ __device__ __forceinline__ void finish_rows(const f32x16 (&yacc)[C / 32], uint32
   }
 }
 
+// in_gamma != nullptr: the rows of u are un-normalised; the kernel applies LayerNorm(in_gamma, in_beta, in_eps) to them
+// as it turns them into operands (the block's ln_mlp1[0], transolver.py:303, without a trip through memory).
 template <int C, int TAIL>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void mlp_rows_kernel(
     const u32x4 *__restrict__ blob, const float *__restrict__ b1, const float *__restrict__ b2,
     const uint16_t *__restrict__ u, uint16_t *__restrict__ y, const uint16_t *__restrict__ residual,
     const float *__restrict__ ln_gamma, const float *__restrict__ ln_beta, float ln_eps, uint16_t *__restrict__ ln_out,
-    int64_t M, int F, int64_t nblocks) {
+    int64_t M, int F, int64_t nblocks, const float *__restrict__ in_gamma, const float *__restrict__ in_beta,
+    float in_eps) {
   using K = Cfg<C>;
   constexpr bool HAS_RES = TAIL == 1 || TAIL == 2, HAS_LN = TAIL == 1 || TAIL == 3;
   constexpr int KS = K::KS, CT = K::CT, HS = K::HS, NT = K::NT, NP = K::NP, SU = K::SU;
@@ -619,6 +664,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   float *b1s = reinterpret_cast<float *>(wbuf + 2 * SU);
   float *b2s = b1s + F;
   float *gams = b2s + C, *bets = gams + C;  // LayerNorm weight and bias
+  float *igams = bets + C, *ibets = igams + C;  // weight and bias of the LayerNorm applied to the input rows
   const int tid = threadIdx.x, lane = tid & 63, i = lane & 31, g = lane >> 5;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: addresses derived from it stay scalar
   const int NCH = F / HS;
@@ -628,6 +674,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     b2s[k] = b2[k];
     gams[k] = HAS_LN ? ln_gamma[k] : 1.f;
     bets[k] = HAS_LN ? ln_beta[k] : 0.f;
+    igams[k] = in_gamma ? in_gamma[k] : 1.f;
+    ibets[k] = in_gamma ? in_beta[k] : 0.f;
   }
   __syncthreads();  // the biases are read before the first barrier of the slot loop
 
@@ -655,6 +703,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   if ((int64_t)blockIdx.x < nblocks) load_rows(blockIdx.x, ub);
   for (int64_t mb = blockIdx.x; mb < nblocks; mb += gridDim.x) {
     const int64_t row0 = mb * kRowsPerBlock + wave * 32;
+    if (in_gamma) normalize_operand_rows<C>(ub, igams, ibets, in_eps, g);
     f32x16 yacc[CT];  // channel 32 ct + rowmap(r, g) of row i
     f32x16 hacc[NT];  // hidden unit 32 n + rowmap(r, g) of the slot's chunk, row i
     // the output bias is where the sum starts; nothing of the block before may reach this one (the padding slots
@@ -817,7 +866,8 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void mlp_rows2_kernel(
     const u32x4 *__restrict__ blob, const float *__restrict__ b1, const float *__restrict__ b2,
     const uint16_t *__restrict__ u, uint16_t *__restrict__ y, const uint16_t *__restrict__ residual,
     const float *__restrict__ ln_gamma, const float *__restrict__ ln_beta, float ln_eps, uint16_t *__restrict__ ln_out,
-    int64_t M, int F, int64_t nblocks) {
+    int64_t M, int F, int64_t nblocks, const float *__restrict__ in_gamma, const float *__restrict__ in_beta,
+    float in_eps) {
   constexpr bool HAS_RES = TAIL == 1 || TAIL == 2, HAS_LN = TAIL == 1 || TAIL == 3;
   constexpr int KS = C / 16, CT = C / 32, NF = KS + 2 * CT, SU = NF * 64;
   constexpr int WU = SU / WAVES;   // units of a slot fetched by each wave
@@ -832,6 +882,7 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void mlp_rows2_kernel(
   float *b1s = reinterpret_cast<float *>(stage + (OWN_STAGE ? 8 * STG / 4 : 0));
   float *b2s = b1s + F;
   float *gams = b2s + C, *bets = gams + C;
+  float *igams = bets + C, *ibets = igams + C;  // weight and bias of the LayerNorm applied to the input rows
   const int tid = threadIdx.x, lane = tid & 63, i = lane & 31, g = lane >> 5;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: addresses derived from it stay scalar
   const int NCH = F / 32;
@@ -840,6 +891,8 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void mlp_rows2_kernel(
     b2s[k] = b2[k];
     gams[k] = HAS_LN ? ln_gamma[k] : 1.f;
     bets[k] = HAS_LN ? ln_beta[k] : 0.f;
+    igams[k] = in_gamma ? in_gamma[k] : 1.f;
+    ibets[k] = in_gamma ? in_beta[k] : 0.f;
   }
   __syncthreads();
   auto fetch = [&](int64_t gs, int c) {  // this wave's share of slot c into buffer gs & 1
@@ -863,6 +916,7 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void mlp_rows2_kernel(
   if ((int64_t)blockIdx.x < nblocks) load_rows(blockIdx.x, ub);
   for (int64_t mb = blockIdx.x; mb < nblocks; mb += gridDim.x) {
     const int64_t row0 = mb * kRows + wave * 32;
+    if (in_gamma) normalize_operand_rows<C>(ub, igams, ibets, in_eps, g);
     f32x16 yacc[CT];
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct)
@@ -1368,8 +1422,8 @@ static bool use_rows2_kernel(int64_t C) { return C == 256; }
 
 // dynamic LDS of the kernel that serves (C, F): two weight buffers, staging / exchange areas, biases and LayerNorm vectors
 static size_t lds_need(int64_t C, int64_t F) {
-  if (use_rows_kernel(C)) return (size_t)2 * 4096 * 16 + (size_t)(F + 3 * C) * 4;
-  if (use_rows2_kernel(C)) return (size_t)2 * (C / 16 + 2 * (C / 32)) * 64 * 16 + 8 * 8192 + (size_t)(F + 3 * C) * 4;
+  if (use_rows_kernel(C)) return (size_t)2 * 4096 * 16 + (size_t)(F + 5 * C) * 4;
+  if (use_rows2_kernel(C)) return (size_t)2 * (C / 16 + 2 * (C / 32)) * 64 * 16 + 8 * 8192 + (size_t)(F + 5 * C) * 4;
   return (size_t)(2 * slot_units((int)C) + 4 * 4 * 64) * 16 + (size_t)(F + C) * 4;
 }
 
@@ -1407,7 +1461,7 @@ int pack(int64_t C, int64_t F, const void *w1, const float *w1_scale, const void
 
 template <int C, int TAIL>
 static int launch_rows(int64_t rows, int F, const void *blob, const float *b1, const float *b2, const void *u, void *y,
-                       const pa_block_tail *tail, int num_cu, hipStream_t st) {
+                       const pa_block_tail *tail, const InputLn &in, int num_cu, hipStream_t st) {
   const size_t lds = lds_need(C, F);
   if (lds > kMaxLdsBytes) return PA_ERR_UNSUPPORTED;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(rows::mlp_rows_kernel<C, TAIL>),
@@ -1419,14 +1473,14 @@ static int launch_rows(int64_t rows, int F, const void *blob, const float *b1, c
                      static_cast<const u32x4 *>(blob), b1, b2, static_cast<const uint16_t *>(u),
                      static_cast<uint16_t *>(y), tail ? static_cast<const uint16_t *>(tail->residual) : nullptr,
                      tail ? tail->ln_gamma : nullptr, tail ? tail->ln_beta : nullptr, tail ? tail->ln_eps : 0.f,
-                     tail ? static_cast<uint16_t *>(tail->ln_out) : nullptr, rows, F, nblocks);
+                     tail ? static_cast<uint16_t *>(tail->ln_out) : nullptr, rows, F, nblocks, in.gamma, in.beta, in.eps);
   e = hipGetLastError();
   return e == hipSuccess ? PA_OK : (int)e;
 }
 
 template <int C, int TAIL>
 static int launch_rows2(int64_t rows, int F, const void *blob, const float *b1, const float *b2, const void *u, void *y,
-                        const pa_block_tail *tail, int num_cu, hipStream_t st) {
+                        const pa_block_tail *tail, const InputLn &in, int num_cu, hipStream_t st) {
   constexpr int WAVES = 8;  // one workgroup per CU; 4 (two per CU, own weight streams) measured 2 % slower
   const size_t lds = lds_need(C, F);  // sized for WAVES = 8 (own staging region)
   if (lds > kMaxLdsBytes) return PA_ERR_UNSUPPORTED;
@@ -1440,29 +1494,29 @@ static int launch_rows2(int64_t rows, int F, const void *blob, const float *b1, 
                      static_cast<const u32x4 *>(blob), b1, b2, static_cast<const uint16_t *>(u),
                      static_cast<uint16_t *>(y), tail ? static_cast<const uint16_t *>(tail->residual) : nullptr,
                      tail ? tail->ln_gamma : nullptr, tail ? tail->ln_beta : nullptr, tail ? tail->ln_eps : 0.f,
-                     tail ? static_cast<uint16_t *>(tail->ln_out) : nullptr, rows, F, nblocks);
+                     tail ? static_cast<uint16_t *>(tail->ln_out) : nullptr, rows, F, nblocks, in.gamma, in.beta, in.eps);
   e = hipGetLastError();
   return e == hipSuccess ? PA_OK : (int)e;
 }
 
 template <int C>
 static int launch_rows2_c(int64_t rows, int F, const void *blob, const float *b1, const float *b2, const void *u, void *y,
-                          const pa_block_tail *tail, int num_cu, hipStream_t st) {
+                          const pa_block_tail *tail, const InputLn &in, int num_cu, hipStream_t st) {
   const bool res = tail && tail->residual, ln = tail && tail->ln_out;
-  if (res && ln) return launch_rows2<C, 1>(rows, F, blob, b1, b2, u, y, tail, num_cu, st);
-  if (res) return launch_rows2<C, 2>(rows, F, blob, b1, b2, u, y, tail, num_cu, st);
-  if (ln) return launch_rows2<C, 3>(rows, F, blob, b1, b2, u, y, tail, num_cu, st);
-  return launch_rows2<C, 0>(rows, F, blob, b1, b2, u, y, nullptr, num_cu, st);
+  if (res && ln) return launch_rows2<C, 1>(rows, F, blob, b1, b2, u, y, tail, in, num_cu, st);
+  if (res) return launch_rows2<C, 2>(rows, F, blob, b1, b2, u, y, tail, in, num_cu, st);
+  if (ln) return launch_rows2<C, 3>(rows, F, blob, b1, b2, u, y, tail, in, num_cu, st);
+  return launch_rows2<C, 0>(rows, F, blob, b1, b2, u, y, nullptr, in, num_cu, st);
 }
 
 template <int C>
 static int launch_rows_c(int64_t rows, int F, const void *blob, const float *b1, const float *b2, const void *u, void *y,
-                         const pa_block_tail *tail, int num_cu, hipStream_t st) {
+                         const pa_block_tail *tail, const InputLn &in, int num_cu, hipStream_t st) {
   const bool res = tail && tail->residual, ln = tail && tail->ln_out;
-  if (res && ln) return launch_rows<C, 1>(rows, F, blob, b1, b2, u, y, tail, num_cu, st);
-  if (res) return launch_rows<C, 2>(rows, F, blob, b1, b2, u, y, tail, num_cu, st);
-  if (ln) return launch_rows<C, 3>(rows, F, blob, b1, b2, u, y, tail, num_cu, st);
-  return launch_rows<C, 0>(rows, F, blob, b1, b2, u, y, nullptr, num_cu, st);
+  if (res && ln) return launch_rows<C, 1>(rows, F, blob, b1, b2, u, y, tail, in, num_cu, st);
+  if (res) return launch_rows<C, 2>(rows, F, blob, b1, b2, u, y, tail, in, num_cu, st);
+  if (ln) return launch_rows<C, 3>(rows, F, blob, b1, b2, u, y, tail, in, num_cu, st);
+  return launch_rows<C, 0>(rows, F, blob, b1, b2, u, y, nullptr, in, num_cu, st);
 }
 
 template <int C, int TAIL>
@@ -1640,10 +1694,16 @@ int premlp(int64_t rows, int64_t c_in, int64_t F, int64_t C, const void *w1, con
   return PA_OK;
 }
 
+// in.gamma != nullptr: LayerNorm(in) is applied to the rows of u on their way in (C = 256 and 512 only)
+bool input_ln_supported(int dtype, int64_t rows, int64_t C, int64_t F) {
+  return supported(dtype, rows, C, F) && (C == 256 || C == 512);
+}
+
 int forward(int64_t rows, int64_t C, int64_t F, const void *blob, const float *b1, const float *b2, const void *u,
-            void *y, const pa_block_tail *tail, int num_cu, hipStream_t st) {
-  if (C == 512) return launch_rows_c<512>(rows, (int)F, blob, b1, b2, u, y, tail, num_cu, st);
-  if (C == 256) return launch_rows2_c<256>(rows, (int)F, blob, b1, b2, u, y, tail, num_cu, st);
+            void *y, const pa_block_tail *tail, const InputLn &in, int num_cu, hipStream_t st) {
+  if (C == 512) return launch_rows_c<512>(rows, (int)F, blob, b1, b2, u, y, tail, in, num_cu, st);
+  if (C == 256) return launch_rows2_c<256>(rows, (int)F, blob, b1, b2, u, y, tail, in, num_cu, st);
+  if (in.gamma) return PA_ERR_UNSUPPORTED;
   if (C == 128) return launch_c<128>(rows, (int)F, blob, b1, b2, u, y, tail, num_cu, st);
   return PA_ERR_UNSUPPORTED;
 }

@@ -429,8 +429,18 @@ def mlp_pack_e4m3(q1, scale1, q2, scale2):
     return packed
 
 
-def mlp_forward_packed(u, packed, b1, b2, residual=None, ln_weight=None, ln_bias=None, ln_eps=1e-5):
-    """mlp_forward with the weights already in operand order (mlp_pack); b1 (F), b2 (C) float32."""
+def mlp_input_ln_supported(dtype: torch.dtype, rows: int, C: int, F: int) -> bool:
+    """True if mlp_forward_packed can apply a LayerNorm to its input rows itself (bfloat16, C in {256, 512})."""
+    if dtype != torch.bfloat16:
+        return False
+    return bool(_lib.load().pa_mlp_input_ln_query(_lib.PA_BF16, rows, C, F))
+
+
+def mlp_forward_packed(u, packed, b1, b2, residual=None, ln_weight=None, ln_bias=None, ln_eps=1e-5, in_ln=None):
+    """mlp_forward with the weights already in operand order (mlp_pack); b1 (F), b2 (C) float32.
+
+    in_ln = (weight, bias, eps), float32: the rows of u are normalised by the kernel on their way in, i.e. the result is
+    w2 . gelu(w1 . LayerNorm(u) + b1) + b2 [+ residual] (mlp_input_ln_supported)."""
     _need_cuda(u, packed, b1, b2, residual, ln_weight, ln_bias)
     lib = _lib.load()
     C, F = b2.numel(), b1.numel()
@@ -438,9 +448,16 @@ def mlp_forward_packed(u, packed, b1, b2, residual=None, ln_weight=None, ln_bias
     y = torch.empty_like(u)
     ln_out = torch.empty_like(u) if ln_weight is not None else None
     tail = _c_tail(residual, ln_weight, ln_bias, ln_eps, ln_out)
-    _lib.check(lib.pa_mlp_forward_packed(_lib.dtype_code(u.dtype), rows, C, F, packed.data_ptr(), b1.data_ptr(),
-                                         b2.data_ptr(), u.data_ptr(), y.data_ptr(), byref(tail),
-                                         _lib.current_stream_ptr(u.device)), "pa_mlp_forward_packed")
+    if in_ln is not None:
+        _need_cuda(in_ln[0], in_ln[1])
+        cin = _lib.PaInputLn(in_ln[0].data_ptr(), in_ln[1].data_ptr(), float(in_ln[2]))
+        _lib.check(lib.pa_mlp_forward_packed_ln(_lib.dtype_code(u.dtype), rows, C, F, packed.data_ptr(), b1.data_ptr(),
+                                                b2.data_ptr(), byref(cin), u.data_ptr(), y.data_ptr(), byref(tail),
+                                                _lib.current_stream_ptr(u.device)), "pa_mlp_forward_packed_ln")
+    else:
+        _lib.check(lib.pa_mlp_forward_packed(_lib.dtype_code(u.dtype), rows, C, F, packed.data_ptr(), b1.data_ptr(),
+                                             b2.data_ptr(), u.data_ptr(), y.data_ptr(), byref(tail),
+                                             _lib.current_stream_ptr(u.device)), "pa_mlp_forward_packed")
     return y if ln_out is None else (y, ln_out)
 
 

@@ -238,14 +238,17 @@ class PhysicsAttentionBase(nn.Module):
 
     def forward_block(self, x: torch.Tensor, residual: torch.Tensor, ln: nn.LayerNorm):
         """Layer + the caller block's ``+ residual`` and following LayerNorm in one pass
-        (physicsnemo/models/transolver/transolver.py:300-303).  Returns (fx_new, LayerNorm(fx_new))."""
+        (physicsnemo/models/transolver/transolver.py:300-303).  Returns (fx_new, LayerNorm(fx_new)); with ln = None
+        (inference on the library kernels only) just fx_new."""
         if x.is_cuda and self._wants_fp16(x):
             with torch.autocast("cuda", enabled=False):  # float32 inside, as the residual stream of the caller is
                 return self.forward_block(x.float(), residual.float(), ln)
         self._validate(x)
         if x.numel() == 0:
             y = self.forward(x)
-            return y + residual.to(y.dtype), y.clone()
+            return (y + residual.to(y.dtype), y.clone()) if ln is not None else y + residual.to(y.dtype)
+        if ln is None and (self.plus or (self.training and self.out_dropout.p > 0) or self._needs_grad(x)):
+            return self.forward(x) + residual
         if self.plus and not self._needs_grad(x) and not self.fp8_weights and not (self.training and self.out_dropout.p > 0):
             xp = self._prepare_input(x)
             dims = self.layer_dims(xp)
@@ -264,6 +267,8 @@ class PhysicsAttentionBase(nn.Module):
             return fx_new, normed.to(y.dtype)
         x = self._prepare_input(x)
         residual = residual.to(x.dtype).contiguous()
+        if ln is None:
+            return PF.layer_forward(x, self.kernel_params(x.dtype, x.device), self.layer_dims(x), residual=residual)[0]
         return PF.layer_forward(
             x, self.kernel_params(x.dtype, x.device), self.layer_dims(x), residual=residual,
             ln_weight=ln.weight.detach().float().contiguous(), ln_bias=ln.bias.detach().float().contiguous(),

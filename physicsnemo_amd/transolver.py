@@ -160,6 +160,27 @@ class TransolverBlock(nn.Module):
         hidden = mlp.layers[0].out_features
         return PF.mlp_supported(normed.dtype, normed.numel() // normed.shape[-1], normed.shape[-1], hidden)
 
+    def _mlp_normalises_its_input(self, x_in: torch.Tensor) -> bool:
+        """True where the block runs as layer call (+ residual) -> MLP kernel with ln_mlp1[0] applied on the way in:
+        bf16 rows of 256 / 512 channels on the plain attention layer's fused tail."""
+        attn = self.Attn
+        if not (x_in.is_cuda and hasattr(attn, "layer_dims") and not getattr(attn, "plus", False)):
+            return False
+        if attn.training and attn.out_dropout.p > 0:
+            return False
+        dtype = torch.get_autocast_dtype("cuda") if torch.is_autocast_enabled("cuda") else x_in.dtype
+        if dtype != torch.bfloat16:
+            return False
+        mlp = self.ln_mlp1[1]
+        if not (isinstance(mlp.layers[1], nn.GELU) and mlp.layers[1].approximate == "none"):
+            return False
+        rows, C = x_in.numel() // x_in.shape[-1], x_in.shape[-1]
+        if C != 256:
+            # at 512 channels the MLP kernel runs one wave per SIMD and nothing hides the normalisation of its rows:
+            # measured, it costs the kernel what the layer's tail saves by not writing the normalised copy
+            return False
+        return PF.mlp_input_ln_supported(torch.bfloat16, rows, C, mlp.layers[0].out_features)
+
     def _needs_grad(self, fx: torch.Tensor) -> bool:
         return torch.is_grad_enabled() and (fx.requires_grad or any(p.requires_grad for p in self.parameters()))
 
@@ -186,8 +207,20 @@ class TransolverBlock(nn.Module):
         whole = self._whole_block(x_in, fx, next_ln)
         if whole is not None:
             return whole
+        ln2 = self.ln_mlp1[0]
+        if self._mlp_normalises_its_input(x_in):
+            # fx1 = Attn(ln_1(fx)) + fx from the layer call; the MLP kernel applies ln_mlp1[0] to its rows itself, so
+            # no normalised copy of fx1 is written or read (reference :300, :303)
+            fx1 = self.Attn.forward_block(x_in, fx, None)
+            packed, b1, b2 = self._mlp_kernel_packed(fx1.device, fx1.dtype)
+            in_ln = (ln2.weight.detach().float().contiguous(), ln2.bias.detach().float().contiguous(), ln2.eps)
+            if next_ln is None:
+                return PF.mlp_forward_packed(fx1, packed, b1, b2, residual=fx1, in_ln=in_ln), None
+            return PF.mlp_forward_packed(fx1, packed, b1, b2, residual=fx1, in_ln=in_ln,
+                                         ln_weight=next_ln.weight.detach().float().contiguous(),
+                                         ln_bias=next_ln.bias.detach().float().contiguous(), ln_eps=next_ln.eps)
         # fx1 = Attn(ln_1(fx)) + fx and LayerNorm(fx1) come out of one fused library call (reference :300, :303)
-        fx1, normed = self.Attn.forward_block(x_in, fx, self.ln_mlp1[0])
+        fx1, normed = self.Attn.forward_block(x_in, fx, ln2)
         return self._mlp_residual(fx1, normed, next_ln)
 
     def _whole_block(self, x_in: torch.Tensor, fx: torch.Tensor, next_ln: nn.LayerNorm | None,

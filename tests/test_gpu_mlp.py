@@ -36,7 +36,7 @@ def _case(rows_shape, C, Fh, seed=0, scale=1.0):
     ((1, 4096), 256, 1024), ((2, 1000), 256, 1024), ((1, 257), 256, 256), ((3, 77), 128, 512), ((1, 1), 256, 1024),
     ((1, 5000), 128, 128), ((1, 20000), 256, 512),
     ((1, 4096), 512, 2048), ((2, 777), 512, 2048), ((1, 1), 512, 64), ((1, 33000), 512, 512),
-    ((1, 300), 512, 6656), ((1, 300), 256, 7424), ((1, 300), 128, 8192),  # the widest hidden layers that fit LDS
+    ((1, 300), 512, 5632), ((1, 300), 256, 6912), ((1, 300), 128, 8192),  # the widest hidden layers that fit LDS
 ])
 def test_mlp_matches_fp32_oracle(rows_shape, C, Fh):
     announce("mlp", rows_shape, C, Fh)
@@ -203,6 +203,38 @@ def test_preprocess_mlp_bf16_matches_oracle(rows_shape, c_in, Fh, C):
     assert not PF.preprocess_supported(torch.bfloat16, 100, 7, 500, 256)
     assert not PF.preprocess_supported(torch.bfloat16, 100, 7, 1760, 256)  # W1 no longer fits beside the stream
     assert not PF.preprocess_supported(torch.bfloat16, 100, 7, 512, 128)
+
+
+@pytest.mark.parametrize("rows_shape,C,Fh", [((1, 4096), 256, 1024), ((2, 1001), 256, 512), ((1, 1), 256, 1024),
+                                             ((1, 4097), 512, 2048), ((3, 300), 512, 512)])
+def test_mlp_normalises_its_input_rows(rows_shape, C, Fh):
+    """pa_mlp_forward_packed_ln: y = u + Mlp(LayerNorm(u)) with the LayerNorm applied inside the kernel, against the
+    oracle's op sequence (transolver.py:303) and against the two-call sequence (LayerNorm kernel, then the MLP kernel)."""
+    announce("mlp with input LayerNorm", rows_shape, C, Fh)
+    ref, _, _, gamma, beta, args = _case(rows_shape, C, Fh, seed=3)
+    dev = args["u"].device
+    torch.manual_seed(9)
+    u = (torch.randn(*rows_shape, C) * 1.7 + 0.4).bfloat16()  # a residual stream: not centred, not unit variance
+    g_in, b_in = torch.rand(C) + 0.5, torch.randn(C) * 0.2
+    assert PF.mlp_input_ln_supported(torch.bfloat16, u.numel() // C, C, Fh)
+    assert not PF.mlp_input_ln_supported(torch.bfloat16, 100, 128, 512)
+    with torch.no_grad():
+        normed = F.layer_norm(u.float(), (C,), g_in, b_in, 1e-5)
+        want = u.float() + ref(normed)
+        want_ln = F.layer_norm(want, (C,), gamma, beta, 1e-5)
+        packed = PF.mlp_pack(args["w1"], args["w2"])
+        ud = u.to(dev)
+        in_ln = (g_in.to(dev), b_in.to(dev), 1e-5)
+        y, ln = PF.mlp_forward_packed(ud, packed, args["b1"], args["b2"], residual=ud, in_ln=in_ln,
+                                      ln_weight=gamma.to(dev), ln_bias=beta.to(dev))
+        y_plain = PF.mlp_forward_packed(ud, packed, args["b1"], args["b2"], residual=ud, in_ln=in_ln)
+        # the two-call sequence the fused form replaces
+        _, normed_dev = PF.residual_layernorm(ud.clone(), ln_weight=in_ln[0], ln_bias=in_ln[1], ln_eps=1e-5)
+        y2 = PF.mlp_forward_packed(normed_dev, packed, args["b1"], args["b2"], residual=ud)
+    assert_rel_l2(y, want, "u + Mlp(LayerNorm(u)), LayerNorm inside the kernel", report=True)
+    assert_rel_l2(ln, want_ln, "next LayerNorm of the same")
+    assert torch.equal(y_plain, y)
+    assert_rel_l2(y, y2.float().cpu(), "against the LayerNorm kernel followed by the MLP kernel", tol=3e-3)
 
 
 @pytest.mark.parametrize("C,Fh", [(128, 512), (256, 1024), (512, 2048)])
