@@ -489,32 +489,30 @@ __device__ __forceinline__ void mma_in_vgprs(u32x4 a, u32x4 b, f32x16 &acc) {
 
 // LayerNorm of a wave's 32 rows held as B operands (lane (i, g): channels 16 ks + 8 g .. + 7 of row i for every k-step,
 // i.e. half a row; lane ^ 32 holds the other half), in place: the rows a producer left un-normalised become the
-// operands of the first product.  Mean and variance in two passes over the registers, float32, as torch's LayerNorm;
-// gams / bets: weight and bias in LDS.
+// operands of the first product.  The sums of x and x^2 come from the packed pairs themselves (v_dot2c_f32_bf16: two
+// exact bf16 products and a float32 accumulation per instruction, four chains each), the variance as
+// E[x^2] - mean^2 in float32 -- exact enough for a residual stream, whose mean is of the order of its spread; gams /
+// bets: weight and bias in LDS.
 template <int C>
 __device__ __forceinline__ void normalize_operand_rows(u32x4 (&ub)[C / 16], const float *gams, const float *bets, float eps,
                                                        int g) {
   constexpr int KS = C / 16;
   typedef float f32x4 __attribute__((ext_vector_type(4)));
-  float s0 = 0.f, s1 = 0.f;
+  typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+  const bf16x2 ones = {(__bf16)1.f, (__bf16)1.f};
+  float s[4] = {0.f, 0.f, 0.f, 0.f}, q[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
     for (int w = 0; w < 4; ++w) {
-      s0 += __uint_as_float(ub[ks][w] << 16);
-      s1 += __uint_as_float(ub[ks][w] & 0xffff0000u);
+      const uint32_t word = ub[ks][w];  // through a scalar: a bit cast straight off the vector element reads element 0
+      const bf16x2 pr = __builtin_bit_cast(bf16x2, word);
+      s[w] = __builtin_amdgcn_fdot2_f32_bf16(pr, ones, s[w], false);
+      q[w] = __builtin_amdgcn_fdot2_f32_bf16(pr, pr, q[w], false);
     }
-  const float mean = half_sum(s0 + s1) * (1.f / C);
-  float q0 = 0.f, q1 = 0.f;
-#pragma unroll
-  for (int ks = 0; ks < KS; ++ks)
-#pragma unroll
-    for (int w = 0; w < 4; ++w) {
-      const float d0 = __uint_as_float(ub[ks][w] << 16) - mean, d1 = __uint_as_float(ub[ks][w] & 0xffff0000u) - mean;
-      q0 = fmaf(d0, d0, q0);
-      q1 = fmaf(d1, d1, q1);
-    }
-  const float rstd = rsqrtf(half_sum(q0 + q1) * (1.f / C) + eps), shift = -mean * rstd;
+  const float mean = half_sum((s[0] + s[1]) + (s[2] + s[3])) * (1.f / C);
+  const float ex2 = half_sum((q[0] + q[1]) + (q[2] + q[3])) * (1.f / C);
+  const float rstd = rsqrtf(fmaxf(fmaf(-mean, mean, ex2), 0.f) + eps), shift = -mean * rstd;
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks) {
     const f32x4 ga = *reinterpret_cast<const f32x4 *>(gams + 16 * ks + 8 * g), gb = *reinterpret_cast<const f32x4 *>(gams + 16 * ks + 8 * g + 4);

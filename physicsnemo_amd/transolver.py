@@ -177,7 +177,7 @@ class TransolverBlock(nn.Module):
         rows, C = x_in.numel() // x_in.shape[-1], x_in.shape[-1]
         if C != 256:
             # at 512 channels the MLP kernel runs one wave per SIMD and nothing hides the normalisation of its rows:
-            # measured, it costs the kernel what the layer's tail saves by not writing the normalised copy
+            # measured on the 12-block model, it costs that kernel more than the layer's tail saves
             return False
         return PF.mlp_input_ln_supported(torch.bfloat16, rows, C, mlp.layers[0].out_features)
 
