@@ -29,6 +29,9 @@ HBM_PEAK_GBS = 8000.0       # MI355X HBM3E, published
 MFMA_BF16_PEAK_TF = 2500.0  # MI355X dense bf16, published
 
 
+TRACE_KERNELS = True
+
+
 def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -48,6 +51,11 @@ def parse_args():
                     help="also run a plain 1 GiB device copy (known traffic) so FETCH_SIZE / WRITE_SIZE can be scaled")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="target CPU time of the baseline leg")
     ap.add_argument("--no-sweep", action="store_true", help="skip the slice_num sweep of the layer workload")
+    ap.add_argument("--no-kernel-trace", action="store_true",
+                    help="skip the in-process kernel trace (torch.profiler) of the layer calls without stage entry "
+                         "points; use it when the script itself runs under rocprofv3 (one tracer at a time)")
+    ap.add_argument("--mlp-only", action="store_true",
+                    help="only the two stand-alone block-MLP legs (for counter runs of those kernels)")
     ap.add_argument("--write-traffic", nargs=2, metavar=("FETCH_DIR", "WRITE_DIR"),
                     help="no GPU work: read the counter files of two rocprofv3 --pmc runs of this script (FETCH_SIZE, "
                          "WRITE_SIZE, both with --calibrate-copy) and write profiles/hbm_traffic.json")
@@ -370,6 +378,8 @@ def time_full_model(name, B, N, functional_dim, points, slice_num, n_layers, ste
                "inputs": f"{points} coordinates + {functional_dim} N(0,1) field(s)",
                "weights": "fp8-e4m3 per-output-channel (attention projections + MLP Linears)" if fp8_weights else "bf16",
                "ms_per_forward": round(dt * 1e3, 3), "mpoints_per_s": round(B * N / dt / 1e6, 2)}
+        if TRACE_KERNELS:
+            res["kernels"] = trace_forward_kernels(lambda: fwd(fx, emb))
         if graph:
             graphed = pn.GraphedForward(fwd, fx, emb)  # the same forward replayed from a HIP graph
             dt_graph, out = timed(lambda a, b: graphed.replay())
@@ -548,6 +558,31 @@ def trace_layer_kernels(layer, x, B, N, C, S, reps=10):
     return out
 
 
+def trace_forward_kernels(fn, top=6):
+    """One call of `fn` under the in-process tracer: share of GPU time by kernel (the `top` largest), the share spent in
+    this library's kernels, and how many launches went to a GEMM library (hipBLASLt / rocBLAS tile kernels)."""
+    import collections
+
+    import torch
+    from torch.profiler import ProfilerActivity, profile
+
+    with torch.no_grad(), profile(activities=[ProfilerActivity.CUDA]) as prof:
+        fn()
+        torch.cuda.synchronize()
+    acc, calls = collections.defaultdict(float), collections.defaultdict(int)
+    for ev in prof.events():
+        if ev.device_type == torch.autograd.DeviceType.CUDA:
+            acc[ev.name] += ev.device_time
+            calls[ev.name] += 1
+    total = sum(acc.values()) or 1.0
+    short = lambda n: n.split("(")[0].replace("void ", "")
+    return {"gpu_ms": round(total * 1e-3, 3),
+            "library_share": round(sum(v for k, v in acc.items() if short(k).startswith("pa::")) / total, 4),
+            "gemm_library_launches": sum(c for k, c in calls.items() if k.startswith(("Cijk_", "rocblas", "void rocblas"))),
+            "top": [{"kernel": short(k), "calls": calls[k], "share": round(v / total, 4)}
+                    for k, v in sorted(acc.items(), key=lambda kv: -kv[1])[:top]]}
+
+
 def occupancy_sweep(x, layer, counts=(256, 192, 128, 64)):
     """Kernel (a+b) restricted to n workgroups (= n compute units busy, the rest of the chip idle): time of the launch
     and the shader clock the chip holds under it (the kernel's clock-reporting twin).  The cycles the kernel needs per
@@ -687,7 +722,7 @@ def measure_layer(B, N, C, S, steps, warmup, kernel_reps, x_cpu=None, cold=False
         del st, yk
         if occupancy and fused and C == 256:
             res["occupancy_sweep"] = occupancy_sweep(x, layer)
-    if not any(k.get("on_layer_path") for k in kernels.values()):
+    if TRACE_KERNELS and not any(k.get("on_layer_path") for k in kernels.values()):
         # no stage entry points on this layer's path (packed-tile sequence): per-kernel times from the profiler
         res["traced_kernels"] = trace_layer_kernels(layer, x, B, N, C, S)
     res.update({"kernels": kernels, "roofline": roofline, "H": H})
@@ -713,8 +748,13 @@ def main():
         sys.exit(2)
     dev = torch.device("cuda:0")
     H = C // 32
-    global SETTLE_MS
+    if args.mlp_only:
+        print(json.dumps({"block_mlp": time_block_mlp(1 << 20, 256, 1024, reps=3),
+                          "block_mlp_c512": time_block_mlp(1 << 20, 512, 2048, reps=3)}), flush=True)
+        return
+    global SETTLE_MS, TRACE_KERNELS
     SETTLE_MS = args.settle_ms
+    TRACE_KERNELS = not args.no_kernel_trace
     gen = torch.Generator().manual_seed(1234)
     x_cpu = torch.randn(B, N, C, generator=gen)
     m = measure_layer(B, N, C, S, args.steps, args.warmup, args.kernel_reps, x_cpu=x_cpu, cold=True,
