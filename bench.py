@@ -170,6 +170,35 @@ def time_block_mlp(rows, C, hidden, reps=10):
             "hbm_frac": round(4 * rows * C * 2 / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
 
 
+def time_yardsticks(reps=20):
+    """What this card sustains on two textbook kernels, timed like every other leg (run-in first): the GEMM library
+    behind torch.matmul on a large square bf16 product, and a device-to-device copy of 1 GiB.  They are not part of
+    the product; they put a practical ceiling next to the published peaks the fractions above are priced at."""
+    import torch
+
+    n = 8192
+    a = torch.randn(n, n, device="cuda").bfloat16()
+    b = torch.randn(n, n, device="cuda").bfloat16()
+    src = torch.empty(1 << 28, device="cuda", dtype=torch.float32).normal_()
+    dst = torch.empty_like(src)
+    out = {}
+    for name, fn, work, unit, peak in (
+            ("library_gemm_bf16_8192", lambda: torch.matmul(a, b), 2.0 * n ** 3 / 1e12, "TFLOP/s", MFMA_BF16_PEAK_TF),
+            ("device_copy_1gib", lambda: dst.copy_(src), 2.0 * src.numel() * 4 / 1e9, "GB/s", HBM_PEAK_GBS)):
+        run_in(fn)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            fn()
+        torch.cuda.synchronize()
+        sec = (time.perf_counter() - t0) / reps
+        out[name] = {"ms": round(sec * 1e3, 4), "achieved": round(work / sec, 1), "unit": unit,
+                     "frac_of_peak": round(work / sec / peak, 4)}
+    del a, b, src, dst
+    torch.cuda.empty_cache()
+    return out
+
+
 def time_training_step(points, C, S, reps=10):
     """Forward + backward of one layer under bf16 autocast at the layer workload's size (gradients w.r.t. the input
     and all ten parameters)."""
@@ -821,6 +850,7 @@ def main():
                                        "kernel_path": {0: "general", 1: "mfma", 2: "mfma-staged"}[m5["path"]],
                                        "kernels": m5.get("traced_kernels", {})},
                                       **layer_fracs(N, 512, 128, m5["ms_per_step"]))
+        out["yardsticks"] = time_yardsticks()
         out["training_step"] = time_training_step(N, C, S)
         out["variants"] = time_variants(N, C, S)
         out["full_model"] = [
