@@ -550,22 +550,30 @@ int cols_gemm_f32(const void *A, int64_t lda, int64_t OA, const void *B, int64_t
 }
 
 // ------------------------------------------------------------------------------------------------
-// cols_gemm_lds_kernel: the same product with the transposition done by the LDS read pattern instead of on the
-// matrix cores.  A workgroup (8 waves, 4 along A's columns x 2 along B's) owns a 256 x 256 block of P for its chunk
-// of rows; 32 rows of both operands at a time are staged in LDS as they lie in memory (16-byte loads; row stride 260
-// elements, so that the two half-waves, eight rows apart, fall on different banks), and a lane gathers its operand
-// -- eight consecutive rows m of one column -- with eight 2-byte LDS reads.  Wave tile 64 x 128: 6 operand fragments
-// feed 8 MFMAs.  grid (G row chunks, ceil(OA / 256)); OB <= 256.
+// cols_gemm_lds_kernel: the same product with the transposition done by the LDS read instead of on the matrix
+// cores.  A workgroup (8 waves, 4 along A's columns x 2 along B's) owns a 256 x 256 block of P for its chunk of rows;
+// 32 rows of both operands at a time are staged in LDS as they lie in memory (16-byte loads and writes; row stride 288
+// elements), and a lane receives its operand -- eight consecutive rows m of one column -- from two transposing reads
+// (ds_read_b64_tr_b16: within a group of 16 lanes, lane l receives element l % 4 of what lanes l / 4, 4 + l / 4,
+// 8 + l / 4, 12 + l / 4 address; lane L addresses row m0 + L / 4, columns c0 + 4 (L % 4) .. + 3, so lane l ends up with
+// column c0 + l of rows m0 .. m0 + 3).  With 144 words between rows the four rows a half-wave reads fall on four
+// different quarters of the banks.  Wave tile 64 x 128: 6 operand fragments (12 reads) feed 8 MFMAs.
+// grid (G row chunks, ceil(OA / 256)); OB <= 256.
 // ------------------------------------------------------------------------------------------------
-constexpr int kColsLd = 260;
+constexpr int kColsLd = 288;
 
 __global__ __launch_bounds__(512) void cols_gemm_lds_kernel(const uint16_t *__restrict__ A, int lda, int OA,
                                                             const uint16_t *__restrict__ B, int ldb, int OB, int64_t M,
                                                             int64_t per, float *__restrict__ partials,
                                                             float *__restrict__ col_sums) {
-  __shared__ uint16_t As[2][32 * kColsLd];
-  __shared__ uint16_t Bs[2][32 * kColsLd];
-  const int t = threadIdx.x, lane = t & 63, i = lane & 31, g = lane >> 5;
+  typedef short v4i16 __attribute__((ext_vector_type(4)));
+  typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+  typedef __attribute__((address_space(3))) v4i16 *lds_v4i16;
+  typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+  extern __shared__ u32x4 cols_smem[];
+  uint16_t *As = reinterpret_cast<uint16_t *>(cols_smem);  // [2][32 * kColsLd]
+  uint16_t *Bs = As + 2 * 32 * kColsLd;                     // [2][32 * kColsLd]
+  const int t = threadIdx.x, lane = t & 63, g = lane >> 5;
   const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
   const int wa = (wave & 3) * 64, wb = (wave >> 2) * 128;
   const int oa0 = blockIdx.y * 256;
@@ -598,48 +606,50 @@ __global__ __launch_bounds__(512) void cols_gemm_lds_kernel(const uint16_t *__re
   auto stage = [&](int buf) {
 #pragma unroll
     for (int k = 0; k < 2; ++k) {
-      // 8-byte aligned halves: the row stride is a multiple of four elements, not of eight
-      uint2 *da = reinterpret_cast<uint2 *>(&As[buf][(sr + 16 * k) * kColsLd + su]);
-      uint2 *db = reinterpret_cast<uint2 *>(&Bs[buf][(sr + 16 * k) * kColsLd + su]);
-      da[0] = uint2{pa[k][0], pa[k][1]};
-      da[1] = uint2{pa[k][2], pa[k][3]};
-      db[0] = uint2{pb[k][0], pb[k][1]};
-      db[1] = uint2{pb[k][2], pb[k][3]};
+      *reinterpret_cast<u32x4 *>(&As[(buf * 32 + sr + 16 * k) * kColsLd + su]) = pa[k];
+      *reinterpret_cast<u32x4 *>(&Bs[(buf * 32 + sr + 16 * k) * kColsLd + su]) = pb[k];
     }
   };
-  auto gather = [&](const uint16_t *base) {  // rows 0..7 of one column -> an MFMA operand
-    u32x4 f;
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-      f[j] = (uint32_t)base[(2 * j) * kColsLd] | ((uint32_t)base[(2 * j + 1) * kColsLd] << 16);
-    return f;
+  // this lane's address inside a 32-row tile for the rows 8 g .. 8 g + 3 of k-step 0 and the 16 columns its group
+  // of lanes stands for (see above); k-step, upper four rows and column tile are constant offsets
+  const int l16 = lane & 15, q1 = (lane >> 4) & 1;
+  const int lane_off = (8 * g + (l16 >> 2)) * kColsLd + 16 * q1 + 4 * (l16 & 3);
+  auto operand = [&](const uint16_t *tile, int ks, int col) {  // rows 16 ks + 8 g .. + 7 of column col + (lane & 31)
+    const uint16_t *p = tile + lane_off + 16 * ks * kColsLd + col;
+    const u32x2 lo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16)(uintptr_t)p));
+    const u32x2 hi =
+        __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16)(uintptr_t)(p + 4 * kColsLd)));
+    return u32x4{lo[0], lo[1], hi[0], hi[1]};
   };
+  const bf16x2 ones = {(__bf16)1.f, (__bf16)1.f};
   if (blk0 < blk1) fetch(blk0);
   int buf = 0;
   for (int64_t blk = blk0; blk < blk1; ++blk) {
     stage(buf);
     __syncthreads();
     if (blk + 1 < blk1) fetch(blk + 1);
+    const uint16_t *at = As + buf * 32 * kColsLd, *bt = Bs + buf * 32 * kColsLd;
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
-      const uint16_t *ar = &As[buf][(16 * ks + 8 * g) * kColsLd + wa + i];
-      const uint16_t *br = &Bs[buf][(16 * ks + 8 * g) * kColsLd + wb + i];
       u32x4 af[2], bf[4];
 #pragma unroll
-      for (int u = 0; u < 2; ++u) af[u] = gather(ar + 32 * u);
+      for (int u = 0; u < 2; ++u) af[u] = operand(at, ks, wa + 32 * u);
 #pragma unroll
-      for (int v = 0; v < 4; ++v) bf[v] = gather(br + 32 * v);
+      for (int v = 0; v < 4; ++v) bf[v] = operand(bt, ks, wb + 32 * v);
 #pragma unroll
       for (int u = 0; u < 2; ++u) {
 #pragma unroll
         for (int v = 0; v < 4; ++v) acc[u][v] = mfma::mma(af[u], bf[v], acc[u][v]);
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
-          csum[u] += __uint_as_float(af[u][j] << 16) + __uint_as_float(af[u][j] & 0xffff0000u);
+        for (int j = 0; j < 4; ++j) {
+          const uint32_t word = af[u][j];
+          csum[u] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, word), ones, csum[u], false);
+        }
       }
     }
     buf ^= 1;
   }
+  const int i = lane & 31;
   float *dst = partials + (int64_t)blockIdx.x * OA * OB;
 #pragma unroll
   for (int u = 0; u < 2; ++u)
@@ -680,7 +690,10 @@ int cols_gemm(const void *A, int64_t lda, int64_t OA, const void *B, int64_t ldb
   const dim3 grid((unsigned)G, (unsigned)((OA + 255) / 256)), block((unsigned)((OA < 256 ? OA : 256) * 2));
   const uint16_t *a = static_cast<const uint16_t *>(A), *b = static_cast<const uint16_t *>(B);
   if (OA >= 128 && OB >= 128 && OB <= 256) {  // wide products: the LDS-gather kernel (its 256 x 256 tile would idle on narrow ones)
-    hipLaunchKernelGGL(cols_gemm_lds_kernel, dim3((unsigned)G, (unsigned)((OA + 255) / 256)), dim3(512), 0, st, a,
+    const size_t lds = (size_t)4 * 32 * kColsLd * 2;
+    const int rc = allow_dynamic_lds(cols_gemm_lds_kernel, lds);
+    if (rc) return rc;
+    hipLaunchKernelGGL(cols_gemm_lds_kernel, dim3((unsigned)G, (unsigned)((OA + 255) / 256)), dim3(512), lds, st, a,
                        (int)lda, (int)OA, b, (int)ldb, (int)OB, M, per, partials, col_sums);
     return launch_status();
   }
