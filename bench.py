@@ -236,8 +236,8 @@ def time_training_step(points, C, S, reps=10):
 
 def time_variants(points, C, S, reps=5):
     """The neighbouring layer variants at the layer workload's size where they fit, each forward (no_grad) and, where
-    served, forward + backward: Transolver++ (general kernels), the structured-3D layer (implicit-GEMM projections +
-    general stages), a GALE layer with a projected context (MFMA kernels + the cross-attention stage), the context
+    served, forward + backward: Transolver++, the structured 3-D and 2-D layers (implicit-GEMM projections + the
+    packed-tile stages), a GALE layer with a projected context (MFMA kernels + the cross-attention stage), the context
     projector itself and a FLARE layer."""
     import torch
 
@@ -336,6 +336,13 @@ def time_variants(points, C, S, reps=5):
     x3 = torch.randn(1, g ** 3, C, device="cuda").bfloat16()
     with torch.no_grad():
         entry(f"structured-3D layer bf16, {g}^3 grid, Conv3d k=3, C={C}, S={S}", g ** 3, timed(lambda: s3(x3), 3))
+    del s3, x3
+    # structured 2-D at the layer workload's point count: 1024 x 1024 grid, Conv2d k=3 projections
+    g2 = 1024
+    s2 = pn.PhysicsAttentionStructuredMesh2D(C, (g2, g2), heads=H, dim_head=32, slice_num=S, kernel=3, use_te=False).cuda()
+    x2 = torch.randn(1, g2 * g2, C, device="cuda").bfloat16()
+    with torch.no_grad():
+        entry(f"structured-2D layer bf16, {g2}x{g2} grid, Conv2d k=3, C={C}, S={S}", g2 * g2, timed(lambda: s2(x2), 3))
     return out
 
 

@@ -190,6 +190,14 @@ struct StagedPlan {
   int64_t G;
 };
 
+int64_t conv_taps(const pa_shape &s) { return s.conv_k * s.conv_k * (s.grid_d > 0 ? s.conv_k : 1); }
+
+// grid convolutions whose projections run on the implicit-GEMM kernel that writes packed tiles
+bool staged_conv_on_tiles(const pa_shape &s) {
+  return s.conv_k > 0 && pa::mlp::conv_project_supported(PA_BF16, s.B, s.N, s.C) &&
+         pa::mlp::linear_supported(PA_BF16, s.B * s.N, s.C);
+}
+
 StagedPlan plan_staged(const pa_shape &s) {
   StagedPlan p{};
   p.G = pa::mfma::softmax_reduce_groups(s, compute_units());
@@ -212,7 +220,9 @@ StagedPlan plan_staged(const pa_shape &s) {
   p.off_tokp = off;
   off += round_up(s.B * s.H * (s.S / 16) * 1024, 256);
   p.off_wout = off;  // the three projections' weights in fragment order, where the row-owning kernels serve them
-  if (pa::mlp::linear_supported(PA_BF16, s.B * s.N, s.C)) off += round_up(3 * pa::mlp::linear_blob_bytes(s.C), 256);
+  if (staged_conv_on_tiles(s))
+    off += round_up(pa::mlp::conv_project_blob_bytes(s.C, conv_taps(s)), 256) + round_up(pa::mlp::linear_blob_bytes(s.C), 256);
+  else if (pa::mlp::linear_supported(PA_BF16, s.B * s.N, s.C)) off += round_up(3 * pa::mlp::linear_blob_bytes(s.C), 256);
   p.total = off;
   return p;
 }
@@ -1173,6 +1183,22 @@ int pa_layer_forward(int dtype, const pa_shape *shape, const pa_params *p, const
       if ((rc = pa::mfma::deslice_recompute(s, *p, x_mid, true, tokp, x_mid, compute_units(), st))) return rc;
       return pa::mlp::linear_packed(s.B, s.N, s.C, p->out_linear_weight, p->out_linear_scale, p->out_linear_bias, x_mid, y,
                                     tail_active(tail) ? tail : nullptr, blob + 2 * pa::mlp::linear_blob_bytes(s.C),
+                                    compute_units(), st);
+    }
+    if (staged_conv_on_tiles(s)) {
+      // the same sequence behind the implicit-GEMM convolution kernel
+      char *blob = ws + sp.off_wout;
+      if ((rc = pa::mlp::conv_project_packed(s.B, s.N, s.C, s.grid_h, s.grid_w, s.grid_d, s.conv_k,
+                                             (int)s.conv_tap_major, p->in_project_x_weight, p->in_project_x_bias,
+                                             p->in_project_fx_weight, p->in_project_fx_bias, x, x_mid, fxp, blob,
+                                             compute_units(), st)))
+        return rc;
+      if ((rc = pa::mfma::slice_softmax_reduce(s, *p, x_mid, true, fxp, partials, compute_units(), st))) return rc;
+      if ((rc = pa::mfma::combine_attention(s, *p, nullptr, partials, sp.G, tok, norm, tok_out, tokp, st))) return rc;
+      if ((rc = pa::mfma::deslice_recompute(s, *p, x_mid, true, tokp, x_mid, compute_units(), st))) return rc;
+      return pa::mlp::linear_packed(s.B, s.N, s.C, p->out_linear_weight, nullptr, p->out_linear_bias, x_mid, y,
+                                    tail_active(tail) ? tail : nullptr,
+                                    blob + round_up(pa::mlp::conv_project_blob_bytes(s.C, conv_taps(s)), 256),
                                     compute_units(), st);
     }
     pa::GemmArgs a{};  // x -> x_mid (natural) and fx_mid (packed): two weight sets over the same rows

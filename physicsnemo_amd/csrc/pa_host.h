@@ -272,6 +272,13 @@ int linear_packed(int64_t B, int64_t N, int64_t C, const void *w, const float *w
 int project_packed(int64_t B, int64_t N, int64_t C, const void *w_x, const float *s_x, const float *b_x, const void *w_fx,
                    const float *s_fx, const float *b_fx, const void *x, void *xm_pack, void *fx_pack, void *blob,
                    int num_cu, hipStream_t st);
+// the same for the k x k (x k) grid convolutions of the structured layers, as an implicit GEMM over taps x channels;
+// blob: conv_project_blob_bytes(C, taps) of scratch
+bool conv_project_supported(int dtype, int64_t B, int64_t N, int64_t C);
+int64_t conv_project_blob_bytes(int64_t C, int64_t taps);
+int conv_project_packed(int64_t B, int64_t N, int64_t C, int64_t gh, int64_t gw, int64_t gd, int64_t k, int tap_major,
+                        const void *w_x, const float *b_x, const void *w_fx, const float *b_fx, const void *x,
+                        void *xm_pack, void *fx_pack, void *blob, int num_cu, hipStream_t st);
 }  // namespace mlp
 
 }  // namespace pa
