@@ -230,7 +230,7 @@ StagedPlan plan_staged(const pa_shape &s) {
 // Workspace plan of the Transolver++ layer: the staged kernels with the slice weights stored (their Gumbel noise
 // comes from the caller's samples, which are read once).
 struct PlusPlan {
-  int64_t off_x_mid, off_fx, off_w, off_partials, off_tok, off_norm, off_tok_out, off_tokp, total;
+  int64_t off_x_mid, off_fx, off_w, off_partials, off_tok, off_norm, off_tok_out, off_tokp, off_blob, total;
   int64_t G;
 };
 
@@ -255,6 +255,8 @@ PlusPlan plan_plus(const pa_shape &s) {
   off += round_up(s.B * s.H * s.S * s.D * 4, 256);
   p.off_tokp = off;
   off += round_up(s.B * s.H * (s.S / 16) * 1024, 256);
+  p.off_blob = off;  // the parameter blob of kernel (d), where that kernel serves the shape
+  if (pa::mfma::supported(PA_BF16, s)) off += round_up(pa::mfma::blob_bytes(s), 256);
   p.total = off;
   return p;
 }
@@ -1487,6 +1489,17 @@ int pa_layer_forward_plus(int dtype, const pa_shape *shape, const pa_params *p, 
   if ((rc = pa::mfma::slice_softmax_pack_plus(s, *p, *plus, x_mid, uniform, wp, compute_units(), st))) return rc;
   if ((rc = pa::mfma::slice_reduce(s, wp, fxp, partials, st))) return rc;
   if ((rc = pa::mfma::combine_attention(s, *p, nullptr, partials, sp.G, tok, norm, tok_out, tokp, st))) return rc;
+  if (pa::mfma::supported(dtype, s) && p->out_linear_bias) {
+    // hand-back, out_linear and the block's tail in kernel (d); of its parameter blob only the out_linear part is read,
+    // the places of the two input projections are filled from the one projection this variant has
+    pa_params q = *p;
+    q.in_project_fx_weight = p->in_project_x_weight;
+    q.in_project_x_bias = q.in_project_fx_bias = p->out_linear_bias;
+    q.in_project_x_scale = q.in_project_fx_scale = q.out_linear_scale = nullptr;
+    void *blob = ws + sp.off_blob;
+    if ((rc = pa::mfma::pack_params(s, q, blob, st))) return rc;
+    return pa::mfma::deslice_project(s, blob, wp, tokp, y, tail_active(tail) ? tail : nullptr, compute_units(), st);
+  }
   void *out_x = x_mid;
   if ((rc = pa::mfma::deslice_natural(s, wp, tokp, out_x, compute_units(), st))) return rc;
   if ((rc = pa::general::out_linear(dtype, s, *p, out_x, y, st))) return rc;
