@@ -1319,7 +1319,7 @@ int pa_block_forward(int dtype, const pa_shape *shape, const pa_params *p, const
 
 // Workspace plan of the FLARE layer on the MFMA kernels.
 struct FlarePlan {
-  int64_t off_scores, off_v, off_wc, off_wr, off_partials, off_z, off_tokp, off_colmax, off_cmpart, off_out_x, total;
+  int64_t off_scores, off_v, off_wc, off_wr, off_partials, off_z, off_tokp, off_colmax, off_cmpart, off_out_x, off_blob, total;
   int64_t G;
 };
 
@@ -1347,6 +1347,8 @@ static FlarePlan plan_flare(const pa_shape &s) {
   p.off_cmpart = off;
   off += round_up(pa::flare::column_max_chunks(s) * s.B * s.H * s.S * 4, 256);
   p.off_out_x = p.off_scores;  // the scores are dead once both weight packs exist
+  p.off_blob = off;            // the parameter blob of kernel (d)
+  off += round_up(pa::mfma::blob_bytes(s), 256);
   p.total = off;
   return p;
 }
@@ -1420,6 +1422,12 @@ int pa_flare_forward_mfma(const pa_shape *shape, const void *scores_weight, cons
   if ((rc = pa::general::combine_partials(s, partials, fp.G, &sums, st))) return rc;
   if ((rc = pa::flare::normalise(s, sums, z, st))) return rc;
   if ((rc = pa::gale::pack_tokens(s, z, tokp, st))) return rc;
+  if (out_linear_weight && out_linear_bias && pa::mfma::supported(PA_BF16, s)) {
+    // hand-back, out_linear and the block's tail in kernel (d)
+    void *blob = ws + fp.off_blob;
+    if ((rc = pa::mfma::pack_out_linear(s, out_linear_weight, nullptr, out_linear_bias, blob, st))) return rc;
+    return pa::mfma::deslice_project(s, blob, wr, tokp, y, tail_active(tail) ? tail : nullptr, compute_units(), st);
+  }
   if ((rc = pa::mfma::deslice_natural(s, wr, tokp, out_x, compute_units(), st))) return rc;
   if (!out_linear_weight) return PA_OK;
   pa_params po{};
@@ -1490,14 +1498,9 @@ int pa_layer_forward_plus(int dtype, const pa_shape *shape, const pa_params *p, 
   if ((rc = pa::mfma::slice_reduce(s, wp, fxp, partials, st))) return rc;
   if ((rc = pa::mfma::combine_attention(s, *p, nullptr, partials, sp.G, tok, norm, tok_out, tokp, st))) return rc;
   if (pa::mfma::supported(dtype, s) && p->out_linear_bias) {
-    // hand-back, out_linear and the block's tail in kernel (d); of its parameter blob only the out_linear part is read,
-    // the places of the two input projections are filled from the one projection this variant has
-    pa_params q = *p;
-    q.in_project_fx_weight = p->in_project_x_weight;
-    q.in_project_x_bias = q.in_project_fx_bias = p->out_linear_bias;
-    q.in_project_x_scale = q.in_project_fx_scale = q.out_linear_scale = nullptr;
+    // hand-back, out_linear and the block's tail in kernel (d), which reads the out_linear part of the parameter blob
     void *blob = ws + sp.off_blob;
-    if ((rc = pa::mfma::pack_params(s, q, blob, st))) return rc;
+    if ((rc = pa::mfma::pack_out_linear(s, p->out_linear_weight, nullptr, p->out_linear_bias, blob, st))) return rc;
     return pa::mfma::deslice_project(s, blob, wp, tokp, y, tail_active(tail) ? tail : nullptr, compute_units(), st);
   }
   void *out_x = x_mid;

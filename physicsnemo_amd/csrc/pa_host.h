@@ -225,6 +225,8 @@ int64_t fx_pack_bytes(const pa_shape &s);
 int64_t w_pack_bytes(const pa_shape &s);
 int64_t tokp_bytes(const pa_shape &s);
 int pack_params(const pa_shape &s, const pa_params &p, void *blob, hipStream_t st);
+int pack_out_linear(const pa_shape &s, const void *w_out, const float *w_scale, const float *b_out, void *blob,
+                    hipStream_t st);
 int64_t project_groups(const pa_shape &s, int num_cu, bool fused);
 bool fuse_reduce(const pa_shape &s);
 int project_softmax(const pa_shape &s, const void *blob, const void *x, void *fx_pack, void *w_pack, float *partials,

@@ -58,14 +58,15 @@ __host__ __device__ inline BlobPlan blob_plan(int C, int S) {
   return p;
 }
 
-__global__ __launch_bounds__(256) void pack_params_kernel(pa_params p, u32x4 *__restrict__ blob, int C, int S) {
+// only_out: fill in the out_linear part alone (wout, bias_out), which is all kernel (d) reads; nothing else of p is touched
+__global__ __launch_bounds__(256) void pack_params_kernel(pa_params p, u32x4 *__restrict__ blob, int C, int S, int only_out) {
   const int H = C / 32, KS = C / 16, ST = (S + 31) / 32;
   const BlobPlan bp = blob_plan(C, S);
   // the three large weights: bf16 bits, or fp8-e4m3 bytes with per-row scales when the parameter set carries scales
   const WeightView wx{p.in_project_x_weight, p.in_project_x_scale, C}, wfx{p.in_project_fx_weight, p.in_project_fx_scale, C},
       wo{p.out_linear_weight, p.out_linear_scale, C};
   const int64_t n_units = bp.fvec;
-  for (int64_t u = (int64_t)blockIdx.x * 256 + threadIdx.x; u < n_units; u += (int64_t)gridDim.x * 256) {
+  for (int64_t u = (only_out ? bp.wout : 0) + (int64_t)blockIdx.x * 256 + threadIdx.x; u < n_units; u += (int64_t)gridDim.x * 256) {
     const int lane = (int)(u & 63), i = lane & 31, g = lane >> 5;
     uint32_t e[4];
     if (u < bp.wsl) {
@@ -97,7 +98,8 @@ __global__ __launch_bounds__(256) void pack_params_kernel(pa_params p, u32x4 *__
     blob[u] = u32x4{e[0], e[1], e[2], e[3]};
   }
   float *fv = reinterpret_cast<float *>(blob + bp.fvec);
-  for (int k = blockIdx.x * 256 + threadIdx.x; k < bp.nfloat; k += gridDim.x * 256) {
+  for (int k = (only_out ? bp.f_bias_out : 0) + blockIdx.x * 256 + threadIdx.x; k < (only_out ? bp.f_tscale : bp.nfloat);
+       k += gridDim.x * 256) {
     float v;
     if (k < bp.f_bias_logit) {
       v = p.in_project_fx_bias[k];
@@ -951,7 +953,18 @@ int64_t w_pack_bytes(const pa_shape &s) { return s.B * tiles_per_batch(s) * s.H 
 int64_t tokp_bytes(const pa_shape &s) { return s.B * s.H * (s.S / 16) * 1024; }
 
 int pack_params(const pa_shape &s, const pa_params &p, void *blob, hipStream_t st) {
-  hipLaunchKernelGGL(pack_params_kernel, dim3(64), dim3(256), 0, st, p, static_cast<u32x4 *>(blob), (int)s.C, (int)s.S);
+  hipLaunchKernelGGL(pack_params_kernel, dim3(64), dim3(256), 0, st, p, static_cast<u32x4 *>(blob), (int)s.C, (int)s.S, 0);
+  return launch_status();
+}
+
+// the blob of kernel (d) alone, for layer variants that share only their hand-back with this family
+int pack_out_linear(const pa_shape &s, const void *w_out, const float *w_scale, const float *b_out, void *blob,
+                    hipStream_t st) {
+  pa_params p{};
+  p.out_linear_weight = w_out;
+  p.out_linear_scale = w_scale;
+  p.out_linear_bias = b_out;
+  hipLaunchKernelGGL(pack_params_kernel, dim3(64), dim3(256), 0, st, p, static_cast<u32x4 *>(blob), (int)s.C, (int)s.S, 1);
   return launch_status();
 }
 
