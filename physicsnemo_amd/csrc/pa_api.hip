@@ -330,6 +330,11 @@ int mfma_layer(const pa_shape &s, const pa_params &p, const void *blob, const vo
       return rc;
     if ((rc = pa::mfma::slice_softmax_reduce(s, p, wp, true, fxp, partials, compute_units(), st))) return rc;
     if ((rc = pa::mfma::combine_attention(s, p, nullptr, partials, G, tok, norm, tok_out, tokp, st))) return rc;
+    // hand-back, out_linear and the tail in kernel (d) with the slice weights recomputed from the x_mid tiles (the
+    // out_linear part of the parameter blob lies behind the room the projections' fragments took)
+    if (pa::mfma::deslice_recompute_project_supported(s))
+      return pa::mfma::deslice_recompute_project(s, p, blob, wp, tokp, y, tail_active(tail) ? tail : nullptr,
+                                                 compute_units(), st);
     if ((rc = pa::mfma::deslice_recompute(s, p, wp, true, tokp, wp, compute_units(), st))) return rc;
     return pa::mlp::linear_packed(s.B, s.N, s.C, p.out_linear_weight, p.out_linear_scale, p.out_linear_bias, wp, y,
                                   tail_active(tail) ? tail : nullptr, wts + 2 * pa::mlp::linear_blob_bytes(s.C),

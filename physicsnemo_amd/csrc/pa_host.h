@@ -240,6 +240,10 @@ int combine_attention(const pa_shape &s, const pa_params &p, const float *fx_bia
                       float *slice_token, float *slice_norm, float *out_token, void *tokp, hipStream_t st);
 int deslice_project(const pa_shape &s, const void *blob, const void *w_pack, const void *tokp, void *y,
                     const pa_block_tail *tail, int num_cu, hipStream_t st);
+// kernel (d) fed with x_mid tiles: the slice weights are recomputed per tile and never stored (S = 128)
+bool deslice_recompute_project_supported(const pa_shape &s);
+int deslice_recompute_project(const pa_shape &s, const pa_params &p, const void *blob, const void *xm_pack,
+                              const void *tokp, void *y, const pa_block_tail *tail, int num_cu, hipStream_t st);
 }  // namespace mfma
 
 namespace mlp {

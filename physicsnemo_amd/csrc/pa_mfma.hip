@@ -728,16 +728,24 @@ __global__ __launch_bounds__(64 * ((S + 31) / 32)) void slice_attention_kernel(c
 // operation and issues the next tile's loads right after the last use of the current ones, so every wait
 // counts exactly the younger operations.  MASKED = true: the ragged last tile of each batch (one per workgroup).
 // ------------------------------------------------------------------------------------------------
-template <int C, int S, int TAIL, bool MASKED>
+// RECOMPUTE: w_pack holds x_mid as packed operand tiles ([tile][head][2][lane], what rows::project_rows_kernel writes)
+// instead of slice weights; wave h forms its head's slice weights from them (logits against W_slice, softmax in the
+// base-2 domain, un-normalised bf16 weights, the denominator from an all-ones MFMA: slice_weights_of_tile) and never
+// stores them.  For slice counts at which the weights weigh more than x_mid (S = 128: 2 KB against 512 bytes per point).
+template <int C, int S, int TAIL, bool MASKED, bool RECOMPUTE = false>
 __global__ __launch_bounds__(C * 2) void deslice_project_kernel(const u32x4 *__restrict__ blob, const u32x4 *__restrict__ w_pack,
                                                                 const u32x4 *__restrict__ tokp, uint16_t *__restrict__ y,
                                                                 const uint16_t *__restrict__ residual,
                                                                 const float *__restrict__ ln_gamma,
                                                                 const float *__restrict__ ln_beta, float ln_eps,
                                                                 uint16_t *__restrict__ ln_out, int64_t N, int tpb,
-                                                                int nfull, int64_t total_items) {
+                                                                int nfull, int64_t total_items,
+                                                                const float *__restrict__ w_slice,
+                                                                const float *__restrict__ b_slice,
+                                                                const float *__restrict__ temperature) {
   constexpr bool HAS_RES = TAIL == 1 || TAIL == 2, HAS_LN = TAIL == 1 || TAIL == 3;
   constexpr int H = C / 32, ST = (S + 31) / 32, NCH = S / 16, NT = C * 2;
+  constexpr int NLD = RECOMPUTE ? 2 : NCH;  // 16-byte units a wave fetches per tile
   constexpr int ROWS = 32 / H;        // rows of the tile finished by each wave
   constexpr int CPL = C / 64;         // consecutive channels per lane in the epilogue
   constexpr int YS = C + 8;           // row stride (floats): rows 4 apart land 32 banks apart
@@ -745,9 +753,17 @@ __global__ __launch_bounds__(C * 2) void deslice_project_kernel(const u32x4 *__r
   __shared__ u32x4 oxs[H * 2 * 64];
   __shared__ u32x4 tps[H * NCH * 64];
   __shared__ float ys[32 * YS];
+  __shared__ u32x4 wsl[RECOMPUTE ? ST * 2 * 64 : 1];
+  __shared__ float bsl[RECOMPUTE ? ST * 32 : 1];
   const BlobPlan bp = blob_plan(C, S);
   const int tid = threadIdx.x, lane = tid & 63, i = lane & 31, g = lane >> 5;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: addresses derived from it stay scalar
+  float sc = 0.f;
+  if constexpr (RECOMPUTE) {
+    stage_slice_projection<S, true>(w_slice, b_slice, wsl, bsl);
+    sc = kLog2e / clamp_temperature(temperature[wave]);
+    __syncthreads();
+  }
 
   u32x4 wout[H][2];
 #pragma unroll
@@ -768,12 +784,12 @@ __global__ __launch_bounds__(C * 2) void deslice_project_kernel(const u32x4 *__r
   int64_t item = blockIdx.x;
   int64_t b = MASKED ? item : item / nfull;
   int64_t t = MASKED ? (int64_t)tpb - 1 : item - b * nfull;
-  u32x4 wcur[NCH];
+  u32x4 wcur[NLD];
   rowvec rcur[ROWS];
   {
-    const u32x4 *wsrc = w_pack + (((b * tpb + t) * H + wave) * NCH) * 64 + lane;
+    const u32x4 *wsrc = w_pack + (((b * tpb + t) * H + wave) * NLD) * 64 + lane;
 #pragma unroll
-    for (int cq = 0; cq < NCH; ++cq) wcur[cq] = load_streaming(wsrc + cq * 64);
+    for (int cq = 0; cq < NLD; ++cq) wcur[cq] = load_streaming(wsrc + cq * 64);
     if constexpr (HAS_RES) {
 #pragma unroll
       for (int rr = 0; rr < ROWS; ++rr) {
@@ -812,14 +828,30 @@ __global__ __launch_bounds__(C * 2) void deslice_project_kernel(const u32x4 *__r
     f32x16 ox, ox2;
 #pragma unroll
     for (int r = 0; r < 16; ++r) ox[r] = ox2[r] = 0.f;
+    if constexpr (RECOMPUTE) {
+      // out_x = (sum_s e_s tok'_s) / (sum_s e_s) with e_s the un-normalised bf16 weights; every row of the all-ones
+      // product is the column sum of the same rounded values
+      u32x4 chunk[NCH];
+      slice_weights_of_tile<S, true>(wsl, bsl, wcur[0], wcur[1], sc, true, lane, g, chunk);
+      const u32x4 ones = u32x4{0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u};
 #pragma unroll
-    for (int cq = 0; cq < NCH; cq += 2) {
-      ox = mma(tps[(wave * NCH + cq) * 64 + lane], wcur[cq], ox);
-      if (cq + 1 < NCH) ox2 = mma(tps[(wave * NCH + cq + 1) * 64 + lane], wcur[cq + 1], ox2);
-    }
-    if constexpr (NCH > 1) {
+      for (int cq = 0; cq < NCH; ++cq) {
+        ox = mma(tps[(wave * NCH + cq) * 64 + lane], chunk[cq], ox);
+        ox2 = mma(ones, chunk[cq], ox2);
+      }
+      const float inv = __builtin_amdgcn_rcpf(ox2[0]);
 #pragma unroll
-      for (int r = 0; r < 16; ++r) ox[r] += ox2[r];
+      for (int r = 0; r < 16; ++r) ox[r] *= inv;
+    } else {
+#pragma unroll
+      for (int cq = 0; cq < NCH; cq += 2) {
+        ox = mma(tps[(wave * NCH + cq) * 64 + lane], wcur[cq], ox);
+        if (cq + 1 < NCH) ox2 = mma(tps[(wave * NCH + cq + 1) * 64 + lane], wcur[cq + 1 < NCH ? cq + 1 : 0], ox2);
+      }
+      if constexpr (NCH > 1) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) ox[r] += ox2[r];
+      }
     }
     // fetch the next item's slice weights and residual rows (the last iteration re-fetches its own)
     const int64_t item_next = item + gridDim.x;
@@ -827,12 +859,12 @@ __global__ __launch_bounds__(C * 2) void deslice_project_kernel(const u32x4 *__r
     const int64_t itn = more ? item_next : item;
     const int64_t bn = MASKED ? b : itn / nfull;
     const int64_t tn = MASKED ? t : itn - bn * nfull;
-    u32x4 wnext[NCH];
+    u32x4 wnext[NLD];
     rowvec rnext[ROWS];
     {
-      const u32x4 *wsrc = w_pack + (((bn * tpb + tn) * H + wave) * NCH) * 64 + lane;
+      const u32x4 *wsrc = w_pack + (((bn * tpb + tn) * H + wave) * NLD) * 64 + lane;
 #pragma unroll
-      for (int cq = 0; cq < NCH; ++cq) wnext[cq] = load_streaming(wsrc + cq * 64);
+      for (int cq = 0; cq < NLD; ++cq) wnext[cq] = load_streaming(wsrc + cq * 64);
       if constexpr (HAS_RES && !MASKED) {
 #pragma unroll
         for (int rr = 0; rr < ROWS; ++rr)
@@ -918,7 +950,7 @@ __global__ __launch_bounds__(C * 2) void deslice_project_kernel(const u32x4 *__r
     b = bn;
     t = tn;
 #pragma unroll
-    for (int cq = 0; cq < NCH; ++cq) wcur[cq] = wnext[cq];
+    for (int cq = 0; cq < NLD; ++cq) wcur[cq] = wnext[cq];
     if constexpr (HAS_RES) {
 #pragma unroll
       for (int rr = 0; rr < ROWS; ++rr) rcur[rr] = rnext[rr];
@@ -1033,9 +1065,10 @@ static int slice_reduce_s(const pa_shape &s, const void *w_pack, const void *fx_
   return launch_status();
 }
 
-template <int C, int S, int TAIL>
+// sp: nullptr, or the slice projection's parameters when `w_pack` holds x_mid tiles and the weights are recomputed
+template <int C, int S, int TAIL, bool RECOMPUTE = false>
 static int deslice_project_t(const pa_shape &s, const void *blob, const void *w_pack, const void *tokp, void *y,
-                             const pa_block_tail *tail, int num_cu, hipStream_t st) {
+                             const pa_block_tail *tail, const pa_params *sp, int num_cu, hipStream_t st) {
   const int64_t tpb = tiles_per_batch(s);
   const int nfull = (int)(s.N / 32);
   const u32x4 *bl = static_cast<const u32x4 *>(blob), *wp = static_cast<const u32x4 *>(w_pack),
@@ -1045,11 +1078,13 @@ static int deslice_project_t(const pa_shape &s, const void *blob, const void *w_
   const float *gm = tail ? tail->ln_gamma : nullptr, *bt = tail ? tail->ln_beta : nullptr;
   const float eps = tail ? tail->ln_eps : 0.f;
   uint16_t *lo = static_cast<uint16_t *>(tail ? tail->ln_out : nullptr);
+  const float *wsl = sp ? sp->in_project_slice_weight : nullptr, *bsl = sp ? sp->in_project_slice_bias : nullptr;
+  const float *tmp = sp ? sp->temperature : nullptr;
   if (nfull > 0) {
     static int per_cu = 0;  // resident workgroups per CU for this instantiation
     if (per_cu == 0) {
       int nb = 0;
-      if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, deslice_project_kernel<C, S, TAIL, false>, C * 2, 0) !=
+      if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, deslice_project_kernel<C, S, TAIL, false, RECOMPUTE>, C * 2, 0) !=
               hipSuccess || nb < 1)
         nb = 1;
       per_cu = nb;
@@ -1057,14 +1092,14 @@ static int deslice_project_t(const pa_shape &s, const void *blob, const void *w_
     const int64_t total = (int64_t)nfull * s.B;
     int64_t grid = (int64_t)num_cu * per_cu;
     if (grid > total) grid = total;
-    hipLaunchKernelGGL((deslice_project_kernel<C, S, TAIL, false>), dim3((unsigned)grid), dim3(C * 2), 0, st, bl, wp, tp,
-                       yo, res, gm, bt, eps, lo, s.N, (int)tpb, nfull, total);
+    hipLaunchKernelGGL((deslice_project_kernel<C, S, TAIL, false, RECOMPUTE>), dim3((unsigned)grid), dim3(C * 2), 0, st, bl,
+                       wp, tp, yo, res, gm, bt, eps, lo, s.N, (int)tpb, nfull, total, wsl, bsl, tmp);
     int rc = launch_status();
     if (rc) return rc;
   }
   if (s.N % 32 != 0) {
-    hipLaunchKernelGGL((deslice_project_kernel<C, S, TAIL, true>), dim3((unsigned)s.B), dim3(C * 2), 0, st, bl, wp, tp, yo,
-                       res, gm, bt, eps, lo, s.N, (int)tpb, nfull, s.B);
+    hipLaunchKernelGGL((deslice_project_kernel<C, S, TAIL, true, RECOMPUTE>), dim3((unsigned)s.B), dim3(C * 2), 0, st, bl, wp,
+                       tp, yo, res, gm, bt, eps, lo, s.N, (int)tpb, nfull, s.B, wsl, bsl, tmp);
     return launch_status();
   }
   return PA_OK;
@@ -1074,10 +1109,21 @@ template <int C, int S>
 static int deslice_project_cs(const pa_shape &s, const void *blob, const void *w_pack, const void *tokp, void *y,
                               const pa_block_tail *tail, int num_cu, hipStream_t st) {
   const bool has_res = tail && tail->residual, has_ln = tail && tail->ln_out;
-  if (has_res && has_ln) return deslice_project_t<C, S, 1>(s, blob, w_pack, tokp, y, tail, num_cu, st);
-  if (has_res) return deslice_project_t<C, S, 2>(s, blob, w_pack, tokp, y, tail, num_cu, st);
-  if (has_ln) return deslice_project_t<C, S, 3>(s, blob, w_pack, tokp, y, tail, num_cu, st);
-  return deslice_project_t<C, S, 0>(s, blob, w_pack, tokp, y, tail, num_cu, st);
+  if (has_res && has_ln) return deslice_project_t<C, S, 1>(s, blob, w_pack, tokp, y, tail, nullptr, num_cu, st);
+  if (has_res) return deslice_project_t<C, S, 2>(s, blob, w_pack, tokp, y, tail, nullptr, num_cu, st);
+  if (has_ln) return deslice_project_t<C, S, 3>(s, blob, w_pack, tokp, y, tail, nullptr, num_cu, st);
+  return deslice_project_t<C, S, 0>(s, blob, w_pack, tokp, y, tail, nullptr, num_cu, st);
+}
+
+// the recomputing form (x_mid tiles in, slice weights never stored): the slice count it is meant for
+template <int C>
+static int deslice_recompute_project_c(const pa_shape &s, const pa_params &p, const void *blob, const void *xm_pack,
+                                       const void *tokp, void *y, const pa_block_tail *tail, int num_cu, hipStream_t st) {
+  const bool has_res = tail && tail->residual, has_ln = tail && tail->ln_out;
+  if (has_res && has_ln) return deslice_project_t<C, 128, 1, true>(s, blob, xm_pack, tokp, y, tail, &p, num_cu, st);
+  if (has_res) return deslice_project_t<C, 128, 2, true>(s, blob, xm_pack, tokp, y, tail, &p, num_cu, st);
+  if (has_ln) return deslice_project_t<C, 128, 3, true>(s, blob, xm_pack, tokp, y, tail, &p, num_cu, st);
+  return deslice_project_t<C, 128, 0, true>(s, blob, xm_pack, tokp, y, tail, &p, num_cu, st);
 }
 
 #define PA_DISPATCH_CS(FN, ...)                                     \
@@ -1141,6 +1187,15 @@ int combine_attention(const pa_shape &s, const pa_params &p, const float *fx_bia
 int deslice_project(const pa_shape &s, const void *blob, const void *w_pack, const void *tokp, void *y,
                     const pa_block_tail *tail, int num_cu, hipStream_t st) {
   PA_DISPATCH_CS(deslice_project_cs, s, blob, w_pack, tokp, y, tail, num_cu, st);
+}
+
+bool deslice_recompute_project_supported(const pa_shape &s) { return s.S == 128 && (s.C == 256 || s.C == 128); }
+
+int deslice_recompute_project(const pa_shape &s, const pa_params &p, const void *blob, const void *xm_pack,
+                              const void *tokp, void *y, const pa_block_tail *tail, int num_cu, hipStream_t st) {
+  if (!deslice_recompute_project_supported(s)) return PA_ERR_UNSUPPORTED;
+  if (s.C == 256) return deslice_recompute_project_c<256>(s, p, blob, xm_pack, tokp, y, tail, num_cu, st);
+  return deslice_recompute_project_c<128>(s, p, blob, xm_pack, tokp, y, tail, num_cu, st);
 }
 
 }  // namespace mfma

@@ -199,79 +199,6 @@ __global__ __launch_bounds__(512) void slice_softmax_pack_plus_kernel(
 }
 
 // ------------------------------------------------------------------------------------------------
-// The slice weights of one head for one tile of 32 points, formed in registers: logits, temperature softmax, bf16
-// operand chunks.  chunk[cq] (cq = 0 .. S/16 - 1) is what slice_softmax_pack_kernel stores: as an A operand its rows
-// are the points and its reduction index the slices 16 cq + kperm order; the same registers serve as a B operand
-// whose columns are the points.  Both kernels below recompute the weights from x_mid instead of passing them through
-// memory (S/16 KB per point and head group written once and read twice otherwise).  The token sums use
-// bf16(e_s / sum e), the hand-back bf16(e_s) divided by the sum of those rounded values: the same softmax, each rounded
-// once.
-// ------------------------------------------------------------------------------------------------
-// DEFER: the chunks hold bf16(exp2(..)) without the division by their sum; the caller divides what it forms from them
-// by the sum of the same rounded values (one more MFMA column), which saves a pass over the S values per point.
-template <int S, bool DEFER = false>
-__device__ __forceinline__ void slice_weights_of_tile(const u32x4 *__restrict__ wsl, const float *__restrict__ bsl,
-                                                      u32x4 xm0, u32x4 xm1, float sc, bool valid, int lane, int g,
-                                                      u32x4 (&chunk)[S / 16]) {
-  constexpr int ST = (S + 31) / 32, NCH = S / 16;
-  f32x16 lg[ST];
-#pragma unroll
-  for (int st = 0; st < ST; ++st) {
-#pragma unroll
-    for (int r = 0; r < 16; ++r) lg[st][r] = bsl[32 * st + rowmap(r, g)];
-    lg[st] = mma(wsl[(st * 2 + 0) * 64 + lane], xm0, lg[st]);
-    lg[st] = mma(wsl[(st * 2 + 1) * 64 + lane], xm1, lg[st]);
-  }
-  float mx = -INFINITY;
-#pragma unroll
-  for (int st = 0; st < ST; ++st)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) mx = fmaxf(mx, lg[st][r]);
-  mx = half_max(mx);
-  const float off = mx * sc;
-  if constexpr (DEFER) {
-#pragma unroll
-    for (int st = 0; st < ST; ++st)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) lg[st][r] = __builtin_amdgcn_exp2f(fmaf(lg[st][r], sc, -off));
-#pragma unroll
-    for (int cq = 0; cq < NCH; ++cq) chunk[cq] = (cq & 1) ? pack_half<1>(lg[cq >> 1]) : pack_half<0>(lg[cq >> 1]);
-  } else {
-    float sum = 0.f;
-#pragma unroll
-    for (int st = 0; st < ST; ++st)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const float e = __builtin_amdgcn_exp2f(fmaf(lg[st][r], sc, -off));
-        lg[st][r] = e;
-        sum += e;
-      }
-    sum = half_sum(sum);
-    const float inv = valid ? __builtin_amdgcn_rcpf(sum) : 0.f;
-#pragma unroll
-    for (int cq = 0; cq < NCH; ++cq) chunk[cq] = (cq & 1) ? pack_half<1>(lg[cq >> 1], inv) : pack_half<0>(lg[cq >> 1], inv);
-  }
-}
-
-// W_slice as A operands and the slice bias, as slice_softmax_pack_kernel stages them; the reduction index runs over
-// d in natural order (x_mid read from its rows) or in kperm order (PACKED_X: x_mid read as packed operand tiles)
-template <int S, bool PACKED_X>
-__device__ __forceinline__ void stage_slice_projection(const float *__restrict__ w_slice, const float *__restrict__ b_slice,
-                                                       u32x4 *wsl, float *bsl) {
-  constexpr int ST = (S + 31) / 32;
-  for (int u = threadIdx.x; u < ST * 2 * 64; u += blockDim.x) {
-    const int ul = u & 63, ui = ul & 31, ug = ul >> 5, f = u >> 6, st = f >> 1, kk = f & 1;
-    const int s = 32 * st + ui;
-    bf16x8 e;
-#pragma unroll
-    for (int j = 0; j < 8; ++j)
-      e[j] = (__bf16)(s < S ? w_slice[s * 32 + (PACKED_X ? kperm(kk, ug, j) : 16 * kk + 8 * ug + j)] : 0.f);
-    wsl[u] = __builtin_bit_cast(u32x4, e);
-  }
-  for (int s = threadIdx.x; s < ST * 32; s += blockDim.x) bsl[s] = s < S ? b_slice[s] : -1e30f;  // slices beyond S: weight 0
-}
-
-// ------------------------------------------------------------------------------------------------
 // slice_softmax_reduce_kernel: slice weights and the first pass of the slice-token sums in one kernel.
 // grid (G, B, head groups), one wave per head of the group; wave h walks the batch's 32-point tiles g, g + G, ...
 // and keeps the sums of its (batch, head) in registers:
