@@ -362,7 +362,7 @@ int mfma_layer(const pa_shape &s, const pa_params &p, const void *blob, const vo
 
 extern "C" {
 
-int pa_version(void) { return 110; }
+int pa_version(void) { return 111; }
 
 int pa_set_compute_units(int n) {
   if (n < 0 || n > 4096) return PA_ERR_DIMS;
