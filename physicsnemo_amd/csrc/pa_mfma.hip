@@ -728,24 +728,16 @@ __global__ __launch_bounds__(64 * ((S + 31) / 32)) void slice_attention_kernel(c
 // operation and issues the next tile's loads right after the last use of the current ones, so every wait
 // counts exactly the younger operations.  MASKED = true: the ragged last tile of each batch (one per workgroup).
 // ------------------------------------------------------------------------------------------------
-// RECOMPUTE: w_pack holds x_mid as packed operand tiles ([tile][head][2][lane], what rows::project_rows_kernel writes)
-// instead of slice weights; wave h forms its head's slice weights from them (logits against W_slice, softmax in the
-// base-2 domain, un-normalised bf16 weights, the denominator from an all-ones MFMA: slice_weights_of_tile) and never
-// stores them.  For slice counts at which the weights weigh more than x_mid (S = 128: 2 KB against 512 bytes per point).
-template <int C, int S, int TAIL, bool MASKED, bool RECOMPUTE = false>
+template <int C, int S, int TAIL, bool MASKED>
 __global__ __launch_bounds__(C * 2) void deslice_project_kernel(const u32x4 *__restrict__ blob, const u32x4 *__restrict__ w_pack,
                                                                 const u32x4 *__restrict__ tokp, uint16_t *__restrict__ y,
                                                                 const uint16_t *__restrict__ residual,
                                                                 const float *__restrict__ ln_gamma,
                                                                 const float *__restrict__ ln_beta, float ln_eps,
                                                                 uint16_t *__restrict__ ln_out, int64_t N, int tpb,
-                                                                int nfull, int64_t total_items,
-                                                                const float *__restrict__ w_slice,
-                                                                const float *__restrict__ b_slice,
-                                                                const float *__restrict__ temperature) {
+                                                                int nfull, int64_t total_items) {
   constexpr bool HAS_RES = TAIL == 1 || TAIL == 2, HAS_LN = TAIL == 1 || TAIL == 3;
-  constexpr int H = C / 32, ST = (S + 31) / 32, NCH = S / 16, NT = C * 2;
-  constexpr int NLD = RECOMPUTE ? 2 : NCH;  // 16-byte units a wave fetches per tile
+  constexpr int H = C / 32, NCH = S / 16, NT = C * 2;
   constexpr int ROWS = 32 / H;        // rows of the tile finished by each wave
   constexpr int CPL = C / 64;         // consecutive channels per lane in the epilogue
   constexpr int YS = C + 8;           // row stride (floats): rows 4 apart land 32 banks apart
@@ -753,17 +745,9 @@ __global__ __launch_bounds__(C * 2) void deslice_project_kernel(const u32x4 *__r
   __shared__ u32x4 oxs[H * 2 * 64];
   __shared__ u32x4 tps[H * NCH * 64];
   __shared__ float ys[32 * YS];
-  __shared__ u32x4 wsl[RECOMPUTE ? ST * 2 * 64 : 1];
-  __shared__ float bsl[RECOMPUTE ? ST * 32 : 1];
   const BlobPlan bp = blob_plan(C, S);
   const int tid = threadIdx.x, lane = tid & 63, i = lane & 31, g = lane >> 5;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: addresses derived from it stay scalar
-  float sc = 0.f;
-  if constexpr (RECOMPUTE) {
-    stage_slice_projection<S, true>(w_slice, b_slice, wsl, bsl);
-    sc = kLog2e / clamp_temperature(temperature[wave]);
-    __syncthreads();
-  }
 
   u32x4 wout[H][2];
 #pragma unroll
@@ -784,12 +768,12 @@ __global__ __launch_bounds__(C * 2) void deslice_project_kernel(const u32x4 *__r
   int64_t item = blockIdx.x;
   int64_t b = MASKED ? item : item / nfull;
   int64_t t = MASKED ? (int64_t)tpb - 1 : item - b * nfull;
-  u32x4 wcur[NLD];
+  u32x4 wcur[NCH];
   rowvec rcur[ROWS];
   {
-    const u32x4 *wsrc = w_pack + (((b * tpb + t) * H + wave) * NLD) * 64 + lane;
+    const u32x4 *wsrc = w_pack + (((b * tpb + t) * H + wave) * NCH) * 64 + lane;
 #pragma unroll
-    for (int cq = 0; cq < NLD; ++cq) wcur[cq] = load_streaming(wsrc + cq * 64);
+    for (int cq = 0; cq < NCH; ++cq) wcur[cq] = load_streaming(wsrc + cq * 64);
     if constexpr (HAS_RES) {
 #pragma unroll
       for (int rr = 0; rr < ROWS; ++rr) {
@@ -828,30 +812,14 @@ __global__ __launch_bounds__(C * 2) void deslice_project_kernel(const u32x4 *__r
     f32x16 ox, ox2;
 #pragma unroll
     for (int r = 0; r < 16; ++r) ox[r] = ox2[r] = 0.f;
-    if constexpr (RECOMPUTE) {
-      // out_x = (sum_s e_s tok'_s) / (sum_s e_s) with e_s the un-normalised bf16 weights; every row of the all-ones
-      // product is the column sum of the same rounded values
-      u32x4 chunk[NCH];
-      slice_weights_of_tile<S, true>(wsl, bsl, wcur[0], wcur[1], sc, true, lane, g, chunk);
-      const u32x4 ones = u32x4{0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u};
 #pragma unroll
-      for (int cq = 0; cq < NCH; ++cq) {
-        ox = mma(tps[(wave * NCH + cq) * 64 + lane], chunk[cq], ox);
-        ox2 = mma(ones, chunk[cq], ox2);
-      }
-      const float inv = __builtin_amdgcn_rcpf(ox2[0]);
+    for (int cq = 0; cq < NCH; cq += 2) {
+      ox = mma(tps[(wave * NCH + cq) * 64 + lane], wcur[cq], ox);
+      if (cq + 1 < NCH) ox2 = mma(tps[(wave * NCH + cq + 1) * 64 + lane], wcur[cq + 1 < NCH ? cq + 1 : 0], ox2);
+    }
+    if constexpr (NCH > 1) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) ox[r] *= inv;
-    } else {
-#pragma unroll
-      for (int cq = 0; cq < NCH; cq += 2) {
-        ox = mma(tps[(wave * NCH + cq) * 64 + lane], wcur[cq], ox);
-        if (cq + 1 < NCH) ox2 = mma(tps[(wave * NCH + cq + 1) * 64 + lane], wcur[cq + 1 < NCH ? cq + 1 : 0], ox2);
-      }
-      if constexpr (NCH > 1) {
-#pragma unroll
-        for (int r = 0; r < 16; ++r) ox[r] += ox2[r];
-      }
+      for (int r = 0; r < 16; ++r) ox[r] += ox2[r];
     }
     // fetch the next item's slice weights and residual rows (the last iteration re-fetches its own)
     const int64_t item_next = item + gridDim.x;
@@ -859,12 +827,12 @@ __global__ __launch_bounds__(C * 2) void deslice_project_kernel(const u32x4 *__r
     const int64_t itn = more ? item_next : item;
     const int64_t bn = MASKED ? b : itn / nfull;
     const int64_t tn = MASKED ? t : itn - bn * nfull;
-    u32x4 wnext[NLD];
+    u32x4 wnext[NCH];
     rowvec rnext[ROWS];
     {
-      const u32x4 *wsrc = w_pack + (((bn * tpb + tn) * H + wave) * NLD) * 64 + lane;
+      const u32x4 *wsrc = w_pack + (((bn * tpb + tn) * H + wave) * NCH) * 64 + lane;
 #pragma unroll
-      for (int cq = 0; cq < NLD; ++cq) wnext[cq] = load_streaming(wsrc + cq * 64);
+      for (int cq = 0; cq < NCH; ++cq) wnext[cq] = load_streaming(wsrc + cq * 64);
       if constexpr (HAS_RES && !MASKED) {
 #pragma unroll
         for (int rr = 0; rr < ROWS; ++rr)
@@ -950,10 +918,236 @@ __global__ __launch_bounds__(C * 2) void deslice_project_kernel(const u32x4 *__r
     b = bn;
     t = tn;
 #pragma unroll
-    for (int cq = 0; cq < NLD; ++cq) wcur[cq] = wnext[cq];
+    for (int cq = 0; cq < NCH; ++cq) wcur[cq] = wnext[cq];
     if constexpr (HAS_RES) {
 #pragma unroll
       for (int rr = 0; rr < ROWS; ++rr) rcur[rr] = rnext[rr];
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Kernel (d) for S = 128, fed with x_mid as packed operand tiles ([tile][head][2][lane], what
+// rows::project_rows_kernel writes) instead of slice weights: at this slice count the weights weigh 2 KB per point
+// against 512 bytes of x_mid, so they are formed again here and never stored.  Forming them is vector work (128 exp2
+// per point and head), the rest of the kernel is matrix, LDS and store work, so the waves split into two roles that
+// share the SIMDs pairwise (wave w and wave w + H/2 sit on the same SIMD):
+//   producers (waves 0 .. H/2-1, two heads each), one tile AHEAD of the consumers: slice weights of their heads from the
+//              x_mid tile (logits against W_slice, softmax in the base-2 domain, un-normalised bf16 weights:
+//              slice_weights_of_tile), out_x^T_h = tok'^T_h . w_h divided by the weights' sum (an all-ones MFMA)
+//              -> bf16 A operands into the other half of a double-buffered LDS patch
+//   consumers (waves H/2 .. H-1, two output tiles each): y = out_x . Wout^T with their slices of out_linear register
+//              resident -> fp32 tile into LDS; then rows 64/H per wave: + residual, rounding, LayerNorm, full-row stores.
+// Two barriers per tile: one hands the out_x patch over, one separates the consumers' two phases (the producers meet
+// it between their two heads).  TAIL, MASKED: as in deslice_project_kernel.
+// ------------------------------------------------------------------------------------------------
+template <int C, int TAIL, bool MASKED>
+__global__ __launch_bounds__(C * 2) void deslice_recompute_project_kernel(
+    const u32x4 *__restrict__ blob, const u32x4 *__restrict__ xm_pack, const u32x4 *__restrict__ tokp,
+    uint16_t *__restrict__ y, const uint16_t *__restrict__ residual, const float *__restrict__ ln_gamma,
+    const float *__restrict__ ln_beta, float ln_eps, uint16_t *__restrict__ ln_out, int64_t N, int tpb, int nfull,
+    int64_t total_items, const float *__restrict__ w_slice, const float *__restrict__ b_slice,
+    const float *__restrict__ temperature) {
+  constexpr bool HAS_RES = TAIL == 1 || TAIL == 2, HAS_LN = TAIL == 1 || TAIL == 3;
+  constexpr int S = 128, H = C / 32, ST = S / 32, NCH = S / 16, CT = C / 32;
+  constexpr int NPW = H / 2;          // producer waves = consumer waves
+  constexpr int HPP = H / NPW;        // heads per producer (2)
+  constexpr int CPC = CT / NPW;       // output tiles per consumer (2)
+  constexpr int ROWS = 32 / NPW;      // rows of the tile finished by each consumer
+  constexpr int CPL = C / 64;         // consecutive channels per lane in the epilogue
+  constexpr int YS = C + 8;           // row stride (floats): rows 4 apart land 32 banks apart
+  typedef uint32_t rowvec __attribute__((ext_vector_type(CPL / 2)));  // CPL bf16
+  __shared__ u32x4 oxs[2][H * 2 * 64];
+  __shared__ float ys[32 * YS];
+  __shared__ u32x4 wsl[ST * 2 * 64];
+  __shared__ float bsl[ST * 32];
+  const BlobPlan bp = blob_plan(C, S);
+  const int tid = threadIdx.x, lane = tid & 63, i = lane & 31, g = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: addresses derived from it stay scalar
+  const bool producer = wave < NPW;
+  stage_slice_projection<S, true>(w_slice, b_slice, wsl, bsl);
+  __syncthreads();
+
+  auto locate = [&](int64_t item, int64_t &b, int64_t &t) {
+    b = MASKED ? item : item / nfull;
+    t = MASKED ? (int64_t)tpb - 1 : item - b * nfull;
+  };
+  int64_t item = blockIdx.x;
+
+  if (producer) {
+    // ---- producers --------------------------------------------------------------------------------
+    float sc[HPP];
+#pragma unroll
+    for (int hh = 0; hh < HPP; ++hh) sc[hh] = kLog2e / clamp_temperature(temperature[wave * HPP + hh]);
+    u32x4 tp[HPP][NCH];
+    int64_t b_loaded = -1;
+    const u32x4 ones = u32x4{0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u};
+    u32x4 xcur[HPP][2];
+    auto fetch_x = [&](int64_t it, int hh) {  // the x_mid tile of head wave * HPP + hh of item `it`
+      int64_t b, t;
+      locate(it, b, t);
+      const u32x4 *src = xm_pack + (((b * tpb + t) * H + wave * HPP + hh) * 2) * 64 + lane;
+      xcur[hh][0] = load_streaming(src);
+      xcur[hh][1] = load_streaming(src + 64);
+    };
+    // out_x of item `it` (its x_mid tiles in xcur) into patch `buf`; `mid`: meet the barrier between the two heads
+    auto produce = [&](int64_t it, int buf, int64_t it_next, bool mid) {
+      int64_t b, t;
+      locate(it, b, t);
+      if (b != b_loaded) {  // wave-uniform: this batch's attended tokens of the wave's heads
+#pragma unroll
+        for (int hh = 0; hh < HPP; ++hh)
+#pragma unroll
+          for (int cq = 0; cq < NCH; ++cq) tp[hh][cq] = tokp[((b * H + wave * HPP + hh) * NCH + cq) * 64 + lane];
+        b_loaded = b;
+      }
+#pragma unroll
+      for (int hh = 0; hh < HPP; ++hh) {
+        u32x4 chunk[NCH];
+        slice_weights_of_tile<S, true>(wsl, bsl, xcur[hh][0], xcur[hh][1], sc[hh], true, lane, g, chunk);
+        fetch_x(it_next, hh);  // refilled in place for the next item, right behind their last use
+        f32x16 ox, den;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) ox[r] = den[r] = 0.f;
+#pragma unroll
+        for (int cq = 0; cq < NCH; ++cq) {
+          ox = mma(tp[hh][cq], chunk[cq], ox);
+          den = mma(ones, chunk[cq], den);
+        }
+        const float inv = __builtin_amdgcn_rcpf(den[0]);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) ox[r] *= inv;
+        const int h = wave * HPP + hh;
+        oxs[buf][(h * 2 + 0) * 64 + lane] = pack_half<0>(ox);
+        oxs[buf][(h * 2 + 1) * 64 + lane] = pack_half<1>(ox);
+        if (hh == 0 && mid) __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);  // one head at a time: their registers are not live together
+      }
+    };
+#pragma unroll
+    for (int hh = 0; hh < HPP; ++hh) fetch_x(item, hh);
+    {
+      const int64_t nx = !MASKED && item + gridDim.x < total_items ? item + gridDim.x : item;
+      produce(item, 0, nx, false);
+    }
+    __syncthreads();
+    for (int k = 0;; ++k) {
+      const int64_t next = item + gridDim.x;
+      const bool more = !MASKED && next < total_items;
+      if (more) {
+        const int64_t nn = next + gridDim.x < total_items ? next + gridDim.x : next;
+        produce(next, (k + 1) & 1, nn, true);
+      } else {
+        __syncthreads();
+      }
+      __syncthreads();
+      if (!more) break;
+      item = next;
+    }
+  } else {
+    // ---- consumers --------------------------------------------------------------------------------
+    const int cw = wave - NPW;
+    u32x4 wout[CPC][H][2];
+#pragma unroll
+    for (int c = 0; c < CPC; ++c)
+#pragma unroll
+      for (int h = 0; h < H; ++h) {
+        wout[c][h][0] = blob[bp.wout + (((cw * CPC + c) * H + h) * 2 + 0) * 64 + lane];
+        wout[c][h][1] = blob[bp.wout + (((cw * CPC + c) * H + h) * 2 + 1) * 64 + lane];
+      }
+    const float *fv = reinterpret_cast<const float *>(blob + bp.fvec) + bp.f_bias_out;
+    float bias[CPC];
+#pragma unroll
+    for (int c = 0; c < CPC; ++c) bias[c] = fv[(cw * CPC + c) * 32 + i];
+    float gam[CPL], bet[CPL];
+#pragma unroll
+    for (int k = 0; k < CPL; ++k) {
+      gam[k] = HAS_LN ? ln_gamma[lane * CPL + k] : 1.f;
+      bet[k] = HAS_LN ? ln_beta[lane * CPL + k] : 0.f;
+    }
+    __syncthreads();  // the first patch is there
+    for (int k = 0;; ++k) {
+      int64_t b, t;
+      locate(item, b, t);
+      const int64_t n0 = t * 32;
+      rowvec rcur[ROWS];
+      if constexpr (HAS_RES) {
+#pragma unroll
+        for (int rr = 0; rr < ROWS; ++rr) {
+          int64_t n = n0 + cw * ROWS + rr;
+          if (MASKED && n >= N) n = N - 1;
+          rcur[rr] = load_streaming(reinterpret_cast<const rowvec *>(residual + (b * N + n) * C + lane * CPL));
+        }
+      }
+      const u32x4 *ob = oxs[k & 1];
+      f32x16 acc[CPC];  // the output tiles take turns: two independent accumulation chains
+#pragma unroll
+      for (int c = 0; c < CPC; ++c)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[c][r] = bias[c];
+#pragma unroll
+      for (int hh = 0; hh < H; ++hh) {
+        const u32x4 of0 = ob[(hh * 2 + 0) * 64 + lane], of1 = ob[(hh * 2 + 1) * 64 + lane];
+#pragma unroll
+        for (int c = 0; c < CPC; ++c) acc[c] = mma(of0, wout[c][hh][0], acc[c]);
+#pragma unroll
+        for (int c = 0; c < CPC; ++c) acc[c] = mma(of1, wout[c][hh][1], acc[c]);
+      }
+#pragma unroll
+      for (int c = 0; c < CPC; ++c)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) ys[rowmap(r, g) * YS + (cw * CPC + c) * 32 + i] = acc[c][r];
+      __syncthreads();
+      // finish ROWS full rows per consumer
+#pragma unroll
+      for (int rr = 0; rr < ROWS; ++rr) {
+        const int row = cw * ROWS + rr;
+        const int64_t n = n0 + row;
+        const bool ok = !MASKED || n < N;
+        const int64_t off = (b * N + n) * C + lane * CPL;
+        float v[CPL];
+        rowvec ov;
+#pragma unroll
+        for (int q = 0; q < CPL; q += 2) {
+          float t0 = ys[row * YS + lane * CPL + q], t1 = ys[row * YS + lane * CPL + q + 1];
+          if constexpr (HAS_RES) {
+            // the residual is added to the fp32 result: one rounding for the sum instead of one per tensor op
+            const uint32_t rv = rcur[rr][q / 2];
+            t0 += bf16_bits_to_f32((uint16_t)(rv & 0xffffu));
+            t1 += bf16_bits_to_f32((uint16_t)(rv >> 16));
+          }
+          const uint16_t o0 = to_bf16_bits(t0), o1 = to_bf16_bits(t1);
+          v[q] = bf16_bits_to_f32(o0);
+          v[q + 1] = bf16_bits_to_f32(o1);
+          ov[q / 2] = (uint32_t)o0 | ((uint32_t)o1 << 16);
+        }
+        if (ok) store_streaming(reinterpret_cast<rowvec *>(y + off), ov);
+        if constexpr (HAS_LN) {
+          float s1 = 0.f;
+#pragma unroll
+          for (int q = 0; q < CPL; ++q) s1 += v[q];
+          const float mean = wave_sum(s1) * (1.f / C);
+          float s2 = 0.f;
+#pragma unroll
+          for (int q = 0; q < CPL; ++q) {
+            const float dl = v[q] - mean;
+            s2 = fmaf(dl, dl, s2);
+          }
+          const float rstd = rsqrtf(wave_sum(s2) * (1.f / C) + ln_eps);
+          rowvec lb;
+#pragma unroll
+          for (int q = 0; q < CPL; q += 2) {
+            const uint16_t l0 = to_bf16_bits((v[q] - mean) * rstd * gam[q] + bet[q]);
+            const uint16_t l1 = to_bf16_bits((v[q + 1] - mean) * rstd * gam[q + 1] + bet[q + 1]);
+            lb[q / 2] = (uint32_t)l0 | ((uint32_t)l1 << 16);
+          }
+          if (ok) store_streaming(reinterpret_cast<rowvec *>(ln_out + off), lb);
+        }
+      }
+      __syncthreads();
+      const int64_t next = item + gridDim.x;
+      if (MASKED || next >= total_items) break;
+      item = next;
     }
   }
 }
@@ -1065,10 +1259,9 @@ static int slice_reduce_s(const pa_shape &s, const void *w_pack, const void *fx_
   return launch_status();
 }
 
-// sp: nullptr, or the slice projection's parameters when `w_pack` holds x_mid tiles and the weights are recomputed
-template <int C, int S, int TAIL, bool RECOMPUTE = false>
+template <int C, int S, int TAIL>
 static int deslice_project_t(const pa_shape &s, const void *blob, const void *w_pack, const void *tokp, void *y,
-                             const pa_block_tail *tail, const pa_params *sp, int num_cu, hipStream_t st) {
+                             const pa_block_tail *tail, int num_cu, hipStream_t st) {
   const int64_t tpb = tiles_per_batch(s);
   const int nfull = (int)(s.N / 32);
   const u32x4 *bl = static_cast<const u32x4 *>(blob), *wp = static_cast<const u32x4 *>(w_pack),
@@ -1078,13 +1271,11 @@ static int deslice_project_t(const pa_shape &s, const void *blob, const void *w_
   const float *gm = tail ? tail->ln_gamma : nullptr, *bt = tail ? tail->ln_beta : nullptr;
   const float eps = tail ? tail->ln_eps : 0.f;
   uint16_t *lo = static_cast<uint16_t *>(tail ? tail->ln_out : nullptr);
-  const float *wsl = sp ? sp->in_project_slice_weight : nullptr, *bsl = sp ? sp->in_project_slice_bias : nullptr;
-  const float *tmp = sp ? sp->temperature : nullptr;
   if (nfull > 0) {
     static int per_cu = 0;  // resident workgroups per CU for this instantiation
     if (per_cu == 0) {
       int nb = 0;
-      if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, deslice_project_kernel<C, S, TAIL, false, RECOMPUTE>, C * 2, 0) !=
+      if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, deslice_project_kernel<C, S, TAIL, false>, C * 2, 0) !=
               hipSuccess || nb < 1)
         nb = 1;
       per_cu = nb;
@@ -1092,14 +1283,45 @@ static int deslice_project_t(const pa_shape &s, const void *blob, const void *w_
     const int64_t total = (int64_t)nfull * s.B;
     int64_t grid = (int64_t)num_cu * per_cu;
     if (grid > total) grid = total;
-    hipLaunchKernelGGL((deslice_project_kernel<C, S, TAIL, false, RECOMPUTE>), dim3((unsigned)grid), dim3(C * 2), 0, st, bl,
-                       wp, tp, yo, res, gm, bt, eps, lo, s.N, (int)tpb, nfull, total, wsl, bsl, tmp);
+    hipLaunchKernelGGL((deslice_project_kernel<C, S, TAIL, false>), dim3((unsigned)grid), dim3(C * 2), 0, st, bl, wp, tp,
+                       yo, res, gm, bt, eps, lo, s.N, (int)tpb, nfull, total);
     int rc = launch_status();
     if (rc) return rc;
   }
   if (s.N % 32 != 0) {
-    hipLaunchKernelGGL((deslice_project_kernel<C, S, TAIL, true, RECOMPUTE>), dim3((unsigned)s.B), dim3(C * 2), 0, st, bl, wp,
-                       tp, yo, res, gm, bt, eps, lo, s.N, (int)tpb, nfull, s.B, wsl, bsl, tmp);
+    hipLaunchKernelGGL((deslice_project_kernel<C, S, TAIL, true>), dim3((unsigned)s.B), dim3(C * 2), 0, st, bl, wp, tp, yo,
+                       res, gm, bt, eps, lo, s.N, (int)tpb, nfull, s.B);
+    return launch_status();
+  }
+  return PA_OK;
+}
+
+// the recomputing form (x_mid tiles in, slice weights never stored)
+template <int C, int TAIL>
+static int deslice_recompute_project_t(const pa_shape &s, const pa_params &p, const void *blob, const void *xm_pack,
+                                       const void *tokp, void *y, const pa_block_tail *tail, int num_cu, hipStream_t st) {
+  const int64_t tpb = tiles_per_batch(s);
+  const int nfull = (int)(s.N / 32);
+  const u32x4 *bl = static_cast<const u32x4 *>(blob), *xp = static_cast<const u32x4 *>(xm_pack),
+              *tp = static_cast<const u32x4 *>(tokp);
+  uint16_t *yo = static_cast<uint16_t *>(y);
+  const uint16_t *res = static_cast<const uint16_t *>(tail ? tail->residual : nullptr);
+  const float *gm = tail ? tail->ln_gamma : nullptr, *bt = tail ? tail->ln_beta : nullptr;
+  const float eps = tail ? tail->ln_eps : 0.f;
+  uint16_t *lo = static_cast<uint16_t *>(tail ? tail->ln_out : nullptr);
+  if (nfull > 0) {
+    const int64_t total = (int64_t)nfull * s.B;
+    const int64_t grid = num_cu < total ? num_cu : total;  // its LDS leaves room for one workgroup per CU
+    hipLaunchKernelGGL((deslice_recompute_project_kernel<C, TAIL, false>), dim3((unsigned)grid), dim3(C * 2), 0, st, bl, xp,
+                       tp, yo, res, gm, bt, eps, lo, s.N, (int)tpb, nfull, total, p.in_project_slice_weight,
+                       p.in_project_slice_bias, p.temperature);
+    int rc = launch_status();
+    if (rc) return rc;
+  }
+  if (s.N % 32 != 0) {
+    hipLaunchKernelGGL((deslice_recompute_project_kernel<C, TAIL, true>), dim3((unsigned)s.B), dim3(C * 2), 0, st, bl, xp, tp,
+                       yo, res, gm, bt, eps, lo, s.N, (int)tpb, nfull, s.B, p.in_project_slice_weight,
+                       p.in_project_slice_bias, p.temperature);
     return launch_status();
   }
   return PA_OK;
@@ -1109,21 +1331,20 @@ template <int C, int S>
 static int deslice_project_cs(const pa_shape &s, const void *blob, const void *w_pack, const void *tokp, void *y,
                               const pa_block_tail *tail, int num_cu, hipStream_t st) {
   const bool has_res = tail && tail->residual, has_ln = tail && tail->ln_out;
-  if (has_res && has_ln) return deslice_project_t<C, S, 1>(s, blob, w_pack, tokp, y, tail, nullptr, num_cu, st);
-  if (has_res) return deslice_project_t<C, S, 2>(s, blob, w_pack, tokp, y, tail, nullptr, num_cu, st);
-  if (has_ln) return deslice_project_t<C, S, 3>(s, blob, w_pack, tokp, y, tail, nullptr, num_cu, st);
-  return deslice_project_t<C, S, 0>(s, blob, w_pack, tokp, y, tail, nullptr, num_cu, st);
+  if (has_res && has_ln) return deslice_project_t<C, S, 1>(s, blob, w_pack, tokp, y, tail, num_cu, st);
+  if (has_res) return deslice_project_t<C, S, 2>(s, blob, w_pack, tokp, y, tail, num_cu, st);
+  if (has_ln) return deslice_project_t<C, S, 3>(s, blob, w_pack, tokp, y, tail, num_cu, st);
+  return deslice_project_t<C, S, 0>(s, blob, w_pack, tokp, y, tail, num_cu, st);
 }
 
-// the recomputing form (x_mid tiles in, slice weights never stored): the slice count it is meant for
 template <int C>
 static int deslice_recompute_project_c(const pa_shape &s, const pa_params &p, const void *blob, const void *xm_pack,
                                        const void *tokp, void *y, const pa_block_tail *tail, int num_cu, hipStream_t st) {
   const bool has_res = tail && tail->residual, has_ln = tail && tail->ln_out;
-  if (has_res && has_ln) return deslice_project_t<C, 128, 1, true>(s, blob, xm_pack, tokp, y, tail, &p, num_cu, st);
-  if (has_res) return deslice_project_t<C, 128, 2, true>(s, blob, xm_pack, tokp, y, tail, &p, num_cu, st);
-  if (has_ln) return deslice_project_t<C, 128, 3, true>(s, blob, xm_pack, tokp, y, tail, &p, num_cu, st);
-  return deslice_project_t<C, 128, 0, true>(s, blob, xm_pack, tokp, y, tail, &p, num_cu, st);
+  if (has_res && has_ln) return deslice_recompute_project_t<C, 1>(s, p, blob, xm_pack, tokp, y, tail, num_cu, st);
+  if (has_res) return deslice_recompute_project_t<C, 2>(s, p, blob, xm_pack, tokp, y, tail, num_cu, st);
+  if (has_ln) return deslice_recompute_project_t<C, 3>(s, p, blob, xm_pack, tokp, y, tail, num_cu, st);
+  return deslice_recompute_project_t<C, 0>(s, p, blob, xm_pack, tokp, y, tail, num_cu, st);
 }
 
 #define PA_DISPATCH_CS(FN, ...)                                     \
