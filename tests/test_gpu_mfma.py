@@ -63,6 +63,28 @@ def test_staged_mfma_layer_for_512_wide_layers(B, N, C, S):
     assert PF.query_path(torch.bfloat16, hip.layer_dims(xs)) == 0
 
 
+@pytest.mark.parametrize("B,N,C", [(2, 1500, 256), (3, 777, 128), (1, 4096, 256)])
+def test_s128_hand_back_with_block_tails(B, N, C):
+    # 128 slices at 128 / 256 channels: the hand-back kernel recomputes the slice weights from the x_mid tiles and carries
+    # the block's tail (ragged last tiles, several batch elements, residual with and without the LayerNorm)
+    announce("S=128 hand-back with tails", B, N, C)
+    ref, hip, xb, want, y, tok = _run(B, N, C, 128, sharpen=2.0)
+    assert_rel_l2(y, want["y"], "layer output")
+    ln = torch.nn.LayerNorm(C)
+    with torch.no_grad():
+        ln.weight.uniform_(0.5, 1.5)
+        ln.bias.uniform_(-0.5, 0.5)
+        res = torch.randn(B, N, C)
+        want_fx = want["y"] + res.bfloat16().float()
+        fx_new, normed = hip.forward_block(xb, res.cuda().bfloat16(), ln.cuda())
+        assert_rel_l2(fx_new, want_fx, "fx_new (residual + LayerNorm tail)")
+        assert_rel_l2(normed, ln.cpu()(want_fx), "LayerNorm(fx_new)", tol=1.5e-2)
+        fx_only = hip.forward_block(xb, res.cuda().bfloat16(), None)
+        fx_only = fx_only[0] if isinstance(fx_only, tuple) else fx_only
+        assert_rel_l2(fx_only, want_fx, "fx_new (residual tail)")
+        assert torch.equal(fx_only, fx_new)
+
+
 def test_mfma_sharp_softmax_and_clamped_temperatures():
     announce("mfma sharp softmax")
     temps = [0.1, 0.5, 1.0, 2.0, 5.0, 10.0, 0.7, 3.0]  # 0.1 and 10 exercise both clamps
