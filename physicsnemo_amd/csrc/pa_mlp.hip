@@ -1415,30 +1415,32 @@ __global__ __launch_bounds__(512) void project_rows_kernel(
 // conv_project_rows_kernel: the two input projections of the structured-grid layers (k x k Conv2d / k x k x k Conv3d,
 // stride 1, zero padding k / 2; PA.py:721-742, :857-867) as an implicit GEMM, written as the packed operand tiles the
 // slice kernels read.  The skeleton is project_rows_kernel's: workgroup = 8 waves (two per SIMD), a block = 8 tiles of
-// 32 points, a wave owns one tile.  The reduction runs over taps x channels: for one tap the wave holds the rows of its
-// points' neighbours at that tap as MFMA operands (C / 4 registers; rows outside the grid are read from a row of
-// zeros) and multiplies them with the tap's weights for all C outputs of one projection (C / 32 accumulators stay live
-// over all taps), first x_mid^T = W_x . x^T (weights as A), then fx_mid = x . W_fx^T (weights as B).  A register of
-// the rows is reloaded for the next tap right behind the last MFMA that read it, so the neighbour loads ride under a
-// whole tap of MFMAs.  Weights stream through LDS in slots of 64 fragments: slot (p taps + tap) SPT + hk holds k-steps
-// hk 64 / CT .. of tap `tap` for all CT output tiles of projection p (fragment j: output tile j % CT, k-step j / CT).
-// blob: the slots in that order, then 2 C bytes of zeros (conv_pack_kernel).
+// 32 points, a wave owns one tile.  The reduction runs over taps x channels in steps of one tap and 256 channels: for
+// such a step the wave holds the rows of its points' neighbours at that tap as MFMA operands (64 registers; rows
+// outside the grid are read from a row of zeros) and multiplies them with the step's weights for 256 outputs of one
+// projection, whose 8 accumulators stay live over all steps: first x_mid^T = W_x . x^T (weights as A), then
+// fx_mid = x . W_fx^T (weights as B), at 512 channels each in two passes of 256 outputs.  A register of the rows is
+// reloaded for the next step right behind the last MFMA that read it, so the neighbour loads ride under a whole step
+// of MFMAs.  Weights stream through LDS in slots of 64 fragments: slot (pass steps + step) 2 + hk holds k-steps
+// 8 hk .. 8 hk + 7 of that step for the pass's 8 output tiles (fragment j: output tile j % 8, k-step j / 8).
+// blob: the slots in that order, then 512 bytes of zeros (conv_pack_kernel).
 // ---------------------------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void conv_pack_kernel(WeightView wx, WeightView wfx, u32x4 *__restrict__ blob, int C,
                                                         int taps, int tap_major) {
-  const int CT = C / 32, KS = C / 16, SPT = CT * KS / 64, KPS = 64 / CT;
-  const int64_t total = (int64_t)2 * taps * SPT * 4096;
-  for (int64_t u = (int64_t)blockIdx.x * 256 + threadIdx.x; u < total + C / 8; u += (int64_t)gridDim.x * 256) {
+  const int NCH = C / 256, steps = taps * NCH;  // reduction steps per pass; passes: 2 projections x NCH output halves
+  const int64_t total = (int64_t)2 * NCH * steps * 2 * 4096;
+  for (int64_t u = (int64_t)blockIdx.x * 256 + threadIdx.x; u < total + 32; u += (int64_t)gridDim.x * 256) {
     if (u >= total) {
       blob[u] = u32x4{0, 0, 0, 0};
       continue;
     }
     const int slot = (int)(u >> 12), j = (int)(u & 4095) >> 6, lane = (int)(u & 63), i = lane & 31, g = lane >> 5;
-    const int p = slot / (taps * SPT), r = slot - p * (taps * SPT), tap = r / SPT, hk = r - tap * SPT;
-    const int ct = j % CT, ks = hk * KPS + j / CT;
-    const WeightView w = p ? wfx : wx;
-    const int64_t row = 32 * ct + i;
-    const int c0 = 16 * ks + 8 * g;
+    const int pass = slot / (steps * 2), r = slot - pass * (steps * 2), step = r >> 1, hk = r & 1;
+    const int proj = pass / NCH, oh = pass - proj * NCH, tap = step / NCH, ch = step - tap * NCH;
+    const int ct = j % 8, ks = hk * 8 + j / 8;
+    const WeightView w = proj ? wfx : wx;
+    const int64_t row = 32 * (8 * oh + ct) + i;
+    const int c0 = 256 * ch + 16 * ks + 8 * g;
     uint32_t e[4];
     if (tap_major) {
       weight_bits8(w, row, (int64_t)tap * C + c0, e);
@@ -1457,10 +1459,10 @@ __global__ __launch_bounds__(512) void conv_project_rows_kernel(
     const u32x4 *__restrict__ blob, const float *__restrict__ bias_x, const float *__restrict__ bias_fx,
     const uint16_t *__restrict__ x, u32x4 *__restrict__ xm_pack, u32x4 *__restrict__ fx_pack, int64_t N, int tpb,
     int64_t ntiles, int64_t nblocks, int gh, int gw, int gd, int ksz) {
-  constexpr int KS = C / 16, CT = C / 32, SU = 4096, WU = SU / 8;
-  constexpr int SPT = CT * KS / 64;  // slots per tap and projection
-  constexpr int KPS = 64 / CT;       // k-steps per slot
-  static_assert(CT * KS % 64 == 0 && 64 % CT == 0, "whole k-steps per slot, whole slots per tap");
+  constexpr int KS = 16, CTB = 8, SU = 4096, WU = SU / 8;  // k-steps and output tiles of a step, slot and wave share
+  constexpr int NCH = C / 256;   // 256-channel chunks of the input = output halves of a projection
+  constexpr int CT = C / 32;     // output tiles of a projection
+  static_assert(C % 256 == 0, "steps of 256 channels");
   extern __shared__ u32x4 smem[];
   u32x4 *wbuf = smem;  // 2 * SU
   float *bxs = reinterpret_cast<float *>(wbuf + 2 * SU);
@@ -1473,8 +1475,8 @@ __global__ __launch_bounds__(512) void conv_project_rows_kernel(
   }
   __syncthreads();
   const int gdd = gd > 0 ? gd : 1, ksd = gd > 0 ? ksz : 1, pad = ksz / 2;
-  const int taps = ksz * ksz * ksd;
-  const int nslots = 2 * taps * SPT;  // per block
+  const int taps = ksz * ksz * ksd, steps = taps * NCH;
+  const int nslots = 2 * NCH * steps * 2;  // per block
   const uint16_t *zero_row = reinterpret_cast<const uint16_t *>(blob + (int64_t)nslots * SU) + 8 * g;
   auto fetch_group = [&](int64_t gs, int c, int k) {
     const u32x4 *src = blob + (int64_t)c * SU + wave * WU + k * 256;
@@ -1497,12 +1499,14 @@ __global__ __launch_bounds__(512) void conv_project_rows_kernel(
     ci = nn / gw;
     cj = nn - ci * gw;
   };
-  // where this lane's neighbour at `tap` starts (its 16-byte piece of k-step 0), or the row of zeros outside the grid
-  auto tap_row = [&](int tap) -> const uint16_t * {
+  // where this lane's operand rows of reduction step `step` start (its 16-byte piece of k-step 0 of the step's 256
+  // channels of the neighbour at the step's tap), or the row of zeros outside the grid
+  auto step_row = [&](int step) -> const uint16_t * {
+    const int tap = step / NCH, ch = step - tap * NCH;
     const int uv = tap / ksd, zz = tap - uv * ksd, u = uv / ksz, v = uv - u * ksz;
     const int ii = ci + u - pad, jj = cj + v - pad, ll = cl + (gd > 0 ? zz - pad : 0);
     const bool ok = ii >= 0 && ii < gh && jj >= 0 && jj < gw && ll >= 0 && ll < gdd;
-    return ok ? xb + (((int64_t)ii * gw + jj) * gdd + ll) * C : zero_row;
+    return ok ? xb + (((int64_t)ii * gw + jj) * gdd + ll) * C + 256 * ch : zero_row;
   };
   int64_t gs = 0;
   u32x4 ub[KS];
@@ -1510,39 +1514,42 @@ __global__ __launch_bounds__(512) void conv_project_rows_kernel(
     fetch_group(0, 0, 0);
     fetch_group(0, 0, 1);
     locate(blockIdx.x);
-    const uint16_t *r0 = tap_row(0);
+    const uint16_t *r0 = step_row(0);
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) ub[ks] = *reinterpret_cast<const u32x4 *>(r0 + 16 * ks);
   }
   for (int64_t mb = blockIdx.x; mb < nblocks; mb += gridDim.x) {
     const int64_t gt = mb * 8 + wave;
     const int64_t gto = gt < ntiles ? gt : ntiles - 1;  // tiles past the end rewrite the last one's results
-    static_for<2>([&](auto p_) {
-      constexpr int p = decltype(p_)::value;  // 0: x_mid^T (weights as A), 1: fx_mid (weights as B)
-      f32x16 acc[CT];
+    static_for<2 * NCH>([&](auto p_) {
+      constexpr int p = decltype(p_)::value;
+      constexpr int proj = p / NCH;  // 0: x_mid^T (weights as A), 1: fx_mid (weights as B)
+      constexpr int oh = p % NCH;    // which 256 outputs
+      f32x16 acc[CTB];
 #pragma unroll
-      for (int ct = 0; ct < CT; ++ct)
+      for (int ct = 0; ct < CTB; ++ct)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) acc[ct][r] = p ? bfs[32 * ct + i] : bxs[32 * ct + rowmap(r, g)];
-      for (int tap = 0; tap < taps; ++tap) {
-        // the rows the registers are refilled with while this tap is multiplied: the next tap's, the first tap's again
-        // for the second projection, the first tap of the wave's tile in the workgroup's next block after that
+        for (int r = 0; r < 16; ++r)
+          acc[ct][r] = proj ? bfs[32 * (CTB * oh + ct) + i] : bxs[32 * (CTB * oh + ct) + rowmap(r, g)];
+      for (int step = 0; step < steps; ++step) {
+        // the rows the registers are refilled with while this step is multiplied: the next step's, the first step's
+        // again for the next pass, the first step of the wave's tile in the workgroup's next block after the last pass
         const uint16_t *nxt;
-        if (tap + 1 < taps) {
-          nxt = tap_row(tap + 1);
+        if (step + 1 < steps) {
+          nxt = step_row(step + 1);
         } else {
-          if (p == 1) locate(mb + gridDim.x < nblocks ? mb + gridDim.x : mb);
-          nxt = tap_row(0);
+          if (p == 2 * NCH - 1) locate(mb + gridDim.x < nblocks ? mb + gridDim.x : mb);
+          nxt = step_row(0);
         }
-        static_for<SPT>([&](auto hk_) {
+        static_for<2>([&](auto hk_) {
           constexpr int hk = decltype(hk_)::value;
-          const int c = (p * taps + tap) * SPT + hk;
+          const int c = (p * steps + step) * 2 + hk;
           // Slot gs has landed (every wave waits for its own share, then all meet) and the other buffer is free.  Its
-          // share was requested before the KPS - 1 row reloads that closed the slot before (and, at a projection's
-          // start, before the 2 CT stores of the projection before): those may still be in flight.
+          // share was requested before the 7 row reloads that closed the slot before (and, at a pass's start, before
+          // the 2 x 8 stores of the pass before): those may still be in flight.
           if (gs == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-          else if (tap == 0 && hk == 0) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(KPS - 1 + 2 * CT) : "memory");
-          else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(KPS - 1) : "memory");
+          else if (step == 0 && hk == 0) asm volatile("s_waitcnt vmcnt(23)" ::: "memory");
+          else asm volatile("s_waitcnt vmcnt(7)" ::: "memory");
           __syncthreads();
           const u32x4 *wb = wbuf + (gs & 1) * SU + lane;
           constexpr int RING = 6, AHEAD = 4;
@@ -1550,20 +1557,20 @@ __global__ __launch_bounds__(512) void conv_project_rows_kernel(
           static_for<AHEAD>([&](auto q) { fr[decltype(q)::value] = wb[decltype(q)::value * 64]; });
           const int c_next = c + 1 < nslots ? c + 1 : 0;
           static_for<64>([&](auto j_) {
-            constexpr int j = decltype(j_)::value, ct = j % CT, ks = hk * KPS + j / CT;
+            constexpr int j = decltype(j_)::value, ct = j % CTB, ks = hk * 8 + j / CTB;
             if constexpr (j + AHEAD < 64) fr[(j + AHEAD) % RING] = wb[(j + AHEAD) * 64];
-            if constexpr (p == 0) acc[ct] = mma(fr[j % RING], ub[ks], acc[ct]);
+            if constexpr (proj == 0) acc[ct] = mma(fr[j % RING], ub[ks], acc[ct]);
             else acc[ct] = mma(ub[ks], fr[j % RING], acc[ct]);
             if constexpr (j == 1 || j == 9) fetch_group(gs + 1, c_next, j / 8);
-            if constexpr (ct == CT - 1) ub[ks] = *reinterpret_cast<const u32x4 *>(nxt + 16 * ks);
+            if constexpr (ct == CTB - 1) ub[ks] = *reinterpret_cast<const u32x4 *>(nxt + 16 * ks);
             __builtin_amdgcn_sched_barrier(0);
           });
           ++gs;
         });
       }
-      u32x4 *dst = (p ? fx_pack : xm_pack) + gto * CT * (2 * 64) + lane;
+      u32x4 *dst = (proj ? fx_pack : xm_pack) + (gto * CT + CTB * oh) * (2 * 64) + lane;
 #pragma unroll
-      for (int ct = 0; ct < CT; ++ct) {
+      for (int ct = 0; ct < CTB; ++ct) {
         store_streaming(dst + (2 * ct) * 64, pack_half<0>(acc[ct]));
         store_streaming(dst + (2 * ct + 1) * 64, pack_half<1>(acc[ct]));
       }
@@ -1807,18 +1814,18 @@ int project_packed(int64_t B, int64_t N, int64_t C, const void *w_x, const float
 // the same for the grid convolutions of the structured layers (conv_project_rows_kernel); weights (H*32, C, k, ..) in
 // torch's layout or tap-major (H*32, k, .., C); `blob` = conv_project_blob_bytes(C, taps) bytes of scratch
 bool conv_project_supported(int dtype, int64_t B, int64_t N, int64_t C) {
-  return dtype == PA_BF16 && C == 256 && B > 0 && N > 0 && N * C * 2 < ((int64_t)1 << 40);
+  return dtype == PA_BF16 && (C == 256 || C == 512) && B > 0 && N > 0 && N * C * 2 < ((int64_t)1 << 40);
 }
 
-int64_t conv_project_blob_bytes(int64_t C, int64_t taps) { return 2 * taps * C * C * 2 + 2 * C; }
+int64_t conv_project_blob_bytes(int64_t C, int64_t taps) { return 2 * taps * C * C * 2 + 512; }
 
 int conv_project_packed(int64_t B, int64_t N, int64_t C, int64_t gh, int64_t gw, int64_t gd, int64_t k, int tap_major,
                         const void *w_x, const float *b_x, const void *w_fx, const float *b_fx, const void *x,
                         void *xm_pack, void *fx_pack, void *blob, int num_cu, hipStream_t st) {
-  if (C != 256 || k <= 0 || k % 2 == 0 || gh <= 0 || gw <= 0 || gd < 0) return PA_ERR_UNSUPPORTED;
+  if ((C != 256 && C != 512) || k <= 0 || k % 2 == 0 || gh <= 0 || gw <= 0 || gd < 0) return PA_ERR_UNSUPPORTED;
   if (gh * gw * (gd > 0 ? gd : 1) != N) return PA_ERR_DIMS;
   const int64_t taps = k * k * (gd > 0 ? k : 1);
-  const int64_t units = 2 * taps * C * C / 8 + C / 8;
+  const int64_t units = 2 * taps * C * C / 8 + 32;
   u32x4 *bl = static_cast<u32x4 *>(blob);
   const int64_t pgrid = (units + 255) / 256 < 2048 ? (units + 255) / 256 : 2048;
   hipLaunchKernelGGL(rows::conv_pack_kernel, dim3((unsigned)pgrid), dim3(256), 0, st,
@@ -1827,14 +1834,20 @@ int conv_project_packed(int64_t B, int64_t N, int64_t C, int64_t gh, int64_t gw,
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return (int)e;
   const size_t lds = (size_t)2 * 4096 * 16 + (size_t)2 * C * 4;
-  e = hipFuncSetAttribute(reinterpret_cast<const void *>(rows::conv_project_rows_kernel<256>),
-                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  const void *kernel = C == 512 ? reinterpret_cast<const void *>(rows::conv_project_rows_kernel<512>)
+                                : reinterpret_cast<const void *>(rows::conv_project_rows_kernel<256>);
+  e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (e != hipSuccess) return (int)e;
   const int64_t tpb = (N + 31) / 32, ntiles = B * tpb, nblocks = (ntiles + 7) / 8;
   const int64_t grid = nblocks < num_cu ? nblocks : num_cu;
-  hipLaunchKernelGGL((rows::conv_project_rows_kernel<256>), dim3((unsigned)grid), dim3(512), lds, st, bl, b_x, b_fx,
-                     static_cast<const uint16_t *>(x), static_cast<u32x4 *>(xm_pack), static_cast<u32x4 *>(fx_pack), N,
-                     (int)tpb, ntiles, nblocks, (int)gh, (int)gw, (int)gd, (int)k);
+  if (C == 512)
+    hipLaunchKernelGGL((rows::conv_project_rows_kernel<512>), dim3((unsigned)grid), dim3(512), lds, st, bl, b_x, b_fx,
+                       static_cast<const uint16_t *>(x), static_cast<u32x4 *>(xm_pack), static_cast<u32x4 *>(fx_pack),
+                       N, (int)tpb, ntiles, nblocks, (int)gh, (int)gw, (int)gd, (int)k);
+  else
+    hipLaunchKernelGGL((rows::conv_project_rows_kernel<256>), dim3((unsigned)grid), dim3(512), lds, st, bl, b_x, b_fx,
+                       static_cast<const uint16_t *>(x), static_cast<u32x4 *>(xm_pack), static_cast<u32x4 *>(fx_pack),
+                       N, (int)tpb, ntiles, nblocks, (int)gh, (int)gw, (int)gd, (int)k);
   e = hipGetLastError();
   return e == hipSuccess ? PA_OK : (int)e;
 }

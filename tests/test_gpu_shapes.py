@@ -81,17 +81,20 @@ def test_backward_refuses_slice_tables_beyond_lds_with_a_clear_error():
     ("structured2d", (48, 50), 5, 256, 8, 64, 2),
     ("structured3d", (16, 16, 16), 3, 256, 8, 64, 1),
     ("structured3d", (12, 10, 9), 3, 128, 4, 16, 4),
-    # 256 channels: the implicit-GEMM kernel that writes packed tiles; grids whose rows straddle the 32-point tiles,
+    # 256 / 512 channels: the implicit-GEMM kernel that writes packed tiles; grids whose rows straddle the 32-point tiles,
     # ragged last tiles, a grid narrower than the kernel's reach, one slice tile and four
     ("structured2d", (37, 29), 3, 256, 8, 32, 4),
     ("structured2d", (2050, 2), 3, 256, 8, 16, 1),
     ("structured2d", (1, 4100), 5, 256, 8, 64, 1),
     ("structured3d", (11, 9, 13), 3, 256, 8, 128, 4),
     ("structured3d", (3, 70, 20), 5, 256, 8, 32, 1),
+    # 512 channels on the same kernel: reduction steps of 256 channels, two passes of 256 outputs per projection
+    ("structured2d", (40, 37), 3, 512, 16, 64, 3),
+    ("structured3d", (9, 8, 10), 3, 512, 16, 128, 6),
 ])
 def test_bf16_structured_layers_on_the_staged_mfma_kernels(variant, grid, kernel, dim, heads, S, B):
     """Grid-convolution projections feeding the staged bf16 MFMA kernels (the implicit-GEMM kernels write fx_mid in the
-    packed operand layout and x_mid either in natural layout or, at 256 channels, as packed tiles too), against the
+    packed operand layout and x_mid either in natural layout or, at 256 / 512 channels, as packed tiles too), against the
     fp32 oracle; with the block tail."""
     announce("bf16 structured staged MFMA", variant, grid, kernel, dim, heads, S, B)
     ref, hip = make_pair(variant, dim, heads, 32, S, spatial=grid, kernel=kernel, seed=S)
