@@ -85,6 +85,33 @@ def test_s128_hand_back_with_block_tails(B, N, C):
         assert torch.equal(fx_only, fx_new)
 
 
+@pytest.mark.parametrize("B,N,C,S", [(2, 1500, 256, 128), (1, 4096, 256, 64), (3, 777, 128, 128)])
+def test_layer_entry_point_that_packs_per_call_matches_the_cached_blob_path(B, N, C, S):
+    # pa_layer_forward repacks the parameters into its workspace on every call; the module path keeps the repacked blob
+    # and calls pa_mfma_layer_forward: the same kernels on the same operands, bit for bit
+    from ctypes import byref
+
+    from physicsnemo_amd import _lib
+
+    announce("pa_layer_forward == pa_mfma_layer_forward", B, N, C, S)
+    _, hip, xb, _, y, tok = _run(B, N, C, S)
+    lib = _lib.load()
+    params = hip.kernel_params(torch.bfloat16, xb.device)
+    shape = hip.layer_dims(xb).c()
+    nbytes = int(lib.pa_workspace_bytes(_lib.PA_BF16, byref(shape)))
+    assert nbytes > 0
+    workspace = torch.empty(nbytes, dtype=torch.uint8, device=xb.device)
+    y2 = torch.empty_like(xb)
+    tok2 = torch.empty_like(tok)
+    tail = PF._c_tail(None, None, None, 1e-5, None)
+    _lib.check(lib.pa_layer_forward(_lib.PA_BF16, byref(shape), byref(PF._c_params(params)), xb.data_ptr(), y2.data_ptr(),
+                                    byref(tail), tok2.data_ptr(), workspace.data_ptr(), nbytes,
+                                    _lib.current_stream_ptr(xb.device)), "pa_layer_forward")
+    torch.cuda.synchronize()
+    assert torch.equal(y2, y)
+    assert torch.equal(tok2, tok)
+
+
 def test_mfma_sharp_softmax_and_clamped_temperatures():
     announce("mfma sharp softmax")
     temps = [0.1, 0.5, 1.0, 2.0, 5.0, 10.0, 0.7, 3.0]  # 0.1 and 10 exercise both clamps
