@@ -56,6 +56,9 @@ def parse_args():
                          "points; use it when the script itself runs under rocprofv3 (one tracer at a time)")
     ap.add_argument("--mlp-only", action="store_true",
                     help="only the two stand-alone block-MLP legs (for counter runs of those kernels)")
+    ap.add_argument("--conv-only", action="store_true",
+                    help="only the structured-grid legs: bf16 layers with Conv2d (1024 x 1024) and Conv3d (64^3) "
+                         "projections (for counter runs of the convolution kernel)")
     ap.add_argument("--write-traffic", nargs=2, metavar=("FETCH_DIR", "WRITE_DIR"),
                     help="no GPU work: read the counter files of two rocprofv3 --pmc runs of this script (FETCH_SIZE, "
                          "WRITE_SIZE, both with --calibrate-copy) and write profiles/hbm_traffic.json")
@@ -196,6 +199,42 @@ def time_yardsticks(reps=20):
                      "frac_of_peak": round(work / sec / peak, 4)}
     del a, b, src, dst
     torch.cuda.empty_cache()
+    return out
+
+
+def time_structured_layers(C, S, reps=5):
+    """bf16 structured-grid layers at the layer workload's width: a 1024 x 1024 grid with 3 x 3 Conv2d projections and a
+    64^3 grid with 3 x 3 x 3 Conv3d projections; per leg the layer time and the convolutions' share of the MFMA peak
+    (FLOPs of both projections over the time of the whole layer call: a lower bound for the kernel itself)."""
+    import torch
+
+    import physicsnemo_amd as pn
+
+    out = []
+    H = C // 32
+    for name, grid, layer_cls in (("structured-2D", (1024, 1024), pn.PhysicsAttentionStructuredMesh2D),
+                                  ("structured-3D", (64, 64, 64), pn.PhysicsAttentionStructuredMesh3D)):
+        n = 1
+        for gdim in grid:
+            n *= gdim
+        layer = layer_cls(C, grid, heads=H, dim_head=32, slice_num=S, kernel=3, use_te=False).cuda().eval()
+        x = torch.randn(1, n, C, device="cuda").bfloat16()
+        with torch.no_grad():
+            run_in(lambda: layer(x))
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(reps):
+                layer(x)
+            torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) / reps * 1e3
+        taps = 3 ** len(grid)
+        conv_tflop = 2.0 * taps * C * 2 * C * n / 1e12
+        out.append({"workload": f"{name} layer bf16, grid {'x'.join(map(str, grid))}, kernel 3, C={C}, S={S}", "points": n,
+                    "ms_forward": round(ms, 3), "mpoints_per_s": round(n / (ms * 1e-3) / 1e6, 2),
+                    "conv_tflop": round(conv_tflop, 3),
+                    "conv_mfma_frac_lower_bound": round(conv_tflop / (ms * 1e-3) / MFMA_BF16_PEAK_TF, 4)})
+        del layer, x
+        torch.cuda.empty_cache()
     return out
 
 
@@ -787,6 +826,9 @@ def main():
     if args.mlp_only:
         print(json.dumps({"block_mlp": time_block_mlp(1 << 20, 256, 1024, reps=3),
                           "block_mlp_c512": time_block_mlp(1 << 20, 512, 2048, reps=3)}), flush=True)
+        return
+    if args.conv_only:
+        print(json.dumps({"structured_layers": time_structured_layers(C, S)}), flush=True)
         return
     global SETTLE_MS, TRACE_KERNELS
     SETTLE_MS = args.settle_ms
